@@ -1,0 +1,400 @@
+// Host side of the C ABI declared in include/incin_rocm.h: device table, buffers,
+// streams/events, descriptor validation and kernel dispatch.  No kernel lives
+// here and no CPU implementation of the operator exists in this library: a
+// request no GPU kernel covers is an error, never a host fallback.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/incin_rocm.h"
+#include "sdpa_params.h"
+
+namespace incin_rocm {
+hipError_t launch_sdpa_generic(const SdpaParams& p, int dtype, hipStream_t stream);
+hipError_t launch_sdpa_prefill_mfma(const SdpaParams& p, int dtype, hipStream_t stream);
+hipError_t launch_sdpa_decode(const SdpaParams& p, int dtype, hipStream_t stream);
+int decode_keys_per_tile(int dtype, int D, int R);
+}  // namespace incin_rocm
+
+using incin_rocm::SdpaParams;
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int hip_fail(hipError_t e, const char* what)
+{
+    int code = (e == hipErrorOutOfMemory) ? INCIN_ROCM_ENOMEM
+             : (e == hipErrorInvalidDevice || e == hipErrorNoDevice) ? INCIN_ROCM_EDEVICE
+                                                                     : INCIN_ROCM_ERUNTIME;
+    return fail(code, "ROCm %s failed: %s (%s)", what, hipGetErrorString(e), hipGetErrorName(e));
+}
+
+#define HIP_TRY(expr, what)                         \
+    do {                                            \
+        hipError_t _e = (expr);                     \
+        if (_e != hipSuccess) return hip_fail(_e, what); \
+    } while (0)
+
+int use_device(int32_t dev)
+{
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(INCIN_ROCM_EDEVICE, "ROCm device query failed: %s", hipGetErrorString(e));
+    }
+    if (dev < 0 || dev >= n) return fail(INCIN_ROCM_EDEVICE, "invalid ROCm device ordinal %d (%d device(s) present)", dev, n);
+    HIP_TRY(hipSetDevice(dev), "hipSetDevice");
+    return 0;
+}
+
+size_t dtype_size(int dtype) { return dtype == INCIN_ROCM_F32 ? 4 : 2; }
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// What the dispatcher decided for one descriptor.
+struct Plan {
+    int impl;
+    int splits;
+    int split_len;
+    size_t ws_bytes;
+    bool empty;      // nothing to compute
+};
+
+bool fast_layout_ok(const incin_rocm_sdpa_desc_t* d, int vec)
+{
+    // 16-byte vector loads of whole rows: row starts and strides must be multiples of the vector.
+    if (!aligned16(d->q) || !aligned16(d->k) || !aligned16(d->v) || !aligned16(d->o)) return false;
+    for (int a = 0; a < 3; ++a) {
+        if (d->q_stride[a] % vec || d->k_stride[a] % vec || d->v_stride[a] % vec || d->o_stride[a] % vec) return false;
+    }
+    return true;
+}
+
+int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
+{
+    if (!d) return fail(INCIN_ROCM_EINVAL, "scaled_dot_product_attention: null descriptor");
+    if (d->dtype != INCIN_ROCM_F32 && d->dtype != INCIN_ROCM_F16 && d->dtype != INCIN_ROCM_BF16)
+        return fail(INCIN_ROCM_EDTYPE, "scaled_dot_product_attention: unsupported dtype tag %d on backend Rocm (f32, f16, bf16 only)", d->dtype);
+    const int64_t lim = 0x7fffffffLL;
+    if (d->B < 0 || d->Hq < 0 || d->Hkv < 0 || d->Sq < 0 || d->Skv < 0 || d->D < 0 || d->Dv < 0)
+        return fail(INCIN_ROCM_ESHAPE, "scaled_dot_product_attention: negative extent");
+    if (d->B > lim || d->Hq > lim || d->Hkv > lim || d->Sq > lim || d->Skv > lim || d->D > lim || d->Dv > lim)
+        return fail(INCIN_ROCM_ESHAPE, "scaled_dot_product_attention: extent exceeds 2^31-1");
+    plan->impl = INCIN_ROCM_IMPL_GENERIC;
+    plan->splits = 1;
+    plan->split_len = (int)d->Skv;
+    plan->ws_bytes = 0;
+    plan->empty = (d->B == 0 || d->Hq == 0 || d->Sq == 0 || d->Dv == 0);
+    if (plan->empty) return 0;
+    if (d->Hkv <= 0 || d->Hq % d->Hkv != 0)
+        return fail(INCIN_ROCM_ESHAPE,
+                    "scaled_dot_product_attention: %lld query heads cannot share %lld key/value heads (batch axes do not broadcast)",
+                    (long long)d->Hq, (long long)d->Hkv);
+    if (d->B > 65535 || d->Hq > 65535)
+        return fail(INCIN_ROCM_ESHAPE, "scaled_dot_product_attention: batch and head counts are limited to 65535 per launch");
+    if (!d->q || !d->o || (d->Skv > 0 && (!d->k || !d->v)))
+        return fail(INCIN_ROCM_EINVAL, "scaled_dot_product_attention: null tensor pointer");
+    if (d->impl < INCIN_ROCM_IMPL_AUTO || d->impl > INCIN_ROCM_IMPL_SPLITKV)
+        return fail(INCIN_ROCM_EINVAL, "scaled_dot_product_attention: unknown impl %d", d->impl);
+    if (d->num_splits < 0) return fail(INCIN_ROCM_EINVAL, "scaled_dot_product_attention: negative num_splits");
+
+    const int vec = d->dtype == INCIN_ROCM_F32 ? 4 : 8;
+    const int64_t R = (d->Hq / d->Hkv) * d->Sq;
+    const bool head_ok = d->D == d->Dv && (d->D == 64 || d->D == 128);
+    const bool fast_ok = head_ok && !d->add_mask && fast_layout_ok(d, vec) && d->Skv > 0;
+    const bool mfma_ok = fast_ok && d->dtype != INCIN_ROCM_F32 && d->scale > 0.0f && std::isfinite(d->scale);
+    const bool split_ok = fast_ok && d->Sq <= 64;
+
+    int impl = d->impl;
+    if (impl == INCIN_ROCM_IMPL_AUTO) {
+        if (split_ok && R <= 8 && d->Skv >= 256) impl = INCIN_ROCM_IMPL_SPLITKV;
+        else if (mfma_ok) impl = INCIN_ROCM_IMPL_MFMA;
+        else if (split_ok && R <= 8) impl = INCIN_ROCM_IMPL_SPLITKV;
+        else impl = INCIN_ROCM_IMPL_GENERIC;
+    }
+    if (impl == INCIN_ROCM_IMPL_MFMA && !mfma_ok)
+        return fail(INCIN_ROCM_EUNSUPPORTED,
+                    "scaled_dot_product_attention: the MFMA kernel needs f16/bf16, D == Dv in {64,128}, scale > 0, no dense mask and 16-byte aligned rows");
+    if (impl == INCIN_ROCM_IMPL_SPLITKV && !split_ok)
+        return fail(INCIN_ROCM_EUNSUPPORTED,
+                    "scaled_dot_product_attention: the split-KV kernel needs D == Dv in {64,128}, Sq <= 64, no dense mask and 16-byte aligned rows");
+    if (impl == INCIN_ROCM_IMPL_GENERIC && (d->D > 256 || d->Dv > 256))
+        return fail(INCIN_ROCM_EUNSUPPORTED,
+                    "scaled_dot_product_attention: head dimension %lld/%lld exceeds 256, no Rocm kernel covers it",
+                    (long long)d->D, (long long)d->Dv);
+    plan->impl = impl;
+
+    if (impl == INCIN_ROCM_IMPL_SPLITKV) {
+        const int rmax = R <= 1 ? 1 : R <= 2 ? 2 : R <= 4 ? 4 : 8;
+        const int64_t nchunks = (R + rmax - 1) / rmax;
+        const int tile = 4 * incin_rocm::decode_keys_per_tile(d->dtype, (int)d->D, (int)(R > 8 ? 8 : R));
+        int64_t splits = d->num_splits;
+        if (splits == 0) {
+            // enough workgroups for ~8 per compute unit, each split at least 512 keys
+            const int64_t groups = d->B * d->Hkv * nchunks;
+            splits = (2048 + groups - 1) / groups;
+            const int64_t max_by_len = d->Skv / 512 > 0 ? d->Skv / 512 : 1;
+            if (splits > max_by_len) splits = max_by_len;
+            if (splits < 1) splits = 1;
+        }
+        int64_t split_len = (d->Skv + splits - 1) / splits;
+        split_len = (split_len + tile - 1) / tile * tile;
+        splits = (d->Skv + split_len - 1) / split_len;
+        if (splits > 65535) return fail(INCIN_ROCM_ESHAPE, "scaled_dot_product_attention: too many splits");
+        if (d->Hkv * nchunks > 65535) return fail(INCIN_ROCM_ESHAPE, "scaled_dot_product_attention: too many head groups for one launch");
+        plan->splits = (int)splits;
+        plan->split_len = (int)split_len;
+        plan->ws_bytes = splits > 1 ? (size_t)(d->B * d->Hq * d->Sq * splits) * (size_t)(d->Dv + 2) * sizeof(float) : 0;
+    }
+    return 0;
+}
+
+void fill_params(const incin_rocm_sdpa_desc_t* d, const Plan& plan, SdpaParams* p)
+{
+    memset(p, 0, sizeof(*p));
+    p->q = d->q; p->k = d->k; p->v = d->v; p->o = d->o;
+    p->mask = d->add_mask;
+    p->kv_lens = d->kv_lens;
+    p->q_sb = d->q_stride[0]; p->q_sh = d->q_stride[1]; p->q_ss = d->q_stride[2];
+    p->k_sb = d->k_stride[0]; p->k_sh = d->k_stride[1]; p->k_ss = d->k_stride[2];
+    p->v_sb = d->v_stride[0]; p->v_sh = d->v_stride[1]; p->v_ss = d->v_stride[2];
+    p->o_sb = d->o_stride[0]; p->o_sh = d->o_stride[1]; p->o_ss = d->o_stride[2];
+    p->m_sb = d->mask_stride[0]; p->m_sh = d->mask_stride[1]; p->m_si = d->mask_stride[2]; p->m_sj = d->mask_stride[3];
+    p->B = (int)d->B; p->Hq = (int)d->Hq; p->Hkv = (int)d->Hkv; p->G = (int)(d->Hq / d->Hkv);
+    p->Sq = (int)d->Sq; p->Skv = (int)d->Skv; p->D = (int)d->D; p->Dv = (int)d->Dv;
+    p->scale = d->scale;
+    p->causal = d->causal ? 1 : 0;
+    p->num_splits = plan.splits;
+    p->split_len = plan.split_len;
+    if (plan.splits > 1) {
+        const size_t rows = (size_t)(d->B * d->Hq * d->Sq * plan.splits);
+        p->ws_acc = (float*)d->workspace;
+        p->ws_ml = (float*)d->workspace + rows * (size_t)d->Dv;
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* incin_rocm_last_error(void) { return g_err; }
+int incin_rocm_abi_version(void) { return INCIN_ROCM_ABI_VERSION; }
+
+int incin_rocm_device_count(int32_t* out)
+{
+    if (!out) return fail(INCIN_ROCM_EINVAL, "device_count: null output");
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e == hipErrorNoDevice) {
+        (void)hipGetLastError();
+        n = 0;
+    } else if (e != hipSuccess) {
+        (void)hipGetLastError();
+        *out = 0;
+        return hip_fail(e, "hipGetDeviceCount");
+    }
+    *out = n;
+    return 0;
+}
+
+int incin_rocm_device_info(int32_t dev, incin_rocm_device_info_t* out)
+{
+    if (!out) return fail(INCIN_ROCM_EINVAL, "device_info: null output");
+    if (int rc = use_device(dev)) return rc;
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, dev), "hipGetDeviceProperties");
+    memset(out, 0, sizeof(*out));
+    snprintf(out->name, sizeof(out->name), "%s", prop.name);
+    snprintf(out->arch, sizeof(out->arch), "%s", prop.gcnArchName);
+    out->compute_units = prop.multiProcessorCount;
+    out->clock_khz = prop.clockRate;
+    out->memory_clock_khz = prop.memoryClockRate;
+    out->memory_bus_bits = prop.memoryBusWidth;
+    out->lds_bytes_per_block = (int32_t)prop.sharedMemPerBlock;
+    out->wavefront_size = prop.warpSize;
+    out->hbm_bytes = (uint64_t)prop.totalGlobalMem;
+    return 0;
+}
+
+int incin_rocm_alloc(int32_t dev, size_t bytes, void** out)
+{
+    if (!out) return fail(INCIN_ROCM_EINVAL, "alloc: null output");
+    *out = nullptr;
+    if (int rc = use_device(dev)) return rc;
+    if (bytes == 0) bytes = 256;                       // a zero-element tensor still owns a distinct, aligned buffer
+    hipError_t e = hipMalloc(out, bytes);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        *out = nullptr;
+        return fail(e == hipErrorOutOfMemory ? INCIN_ROCM_ENOMEM : INCIN_ROCM_ERUNTIME,
+                    "ROCm allocation of %zu bytes on device %d failed: %s", bytes, dev, hipGetErrorString(e));
+    }
+    return 0;
+}
+
+int incin_rocm_free(int32_t dev, void* ptr)
+{
+    if (!ptr) return 0;
+    if (int rc = use_device(dev)) return rc;
+    HIP_TRY(hipFree(ptr), "hipFree");
+    return 0;
+}
+
+int incin_rocm_memset(int32_t dev, void* dst, int value, size_t bytes)
+{
+    if (bytes == 0) return 0;
+    if (!dst) return fail(INCIN_ROCM_EINVAL, "memset: null pointer");
+    if (int rc = use_device(dev)) return rc;
+    HIP_TRY(hipMemset(dst, value, bytes), "hipMemset");
+    return 0;
+}
+
+static int copy(int32_t dev, void* dst, const void* src, size_t bytes, hipMemcpyKind kind, const char* what)
+{
+    if (bytes == 0) return 0;
+    if (!dst || !src) return fail(INCIN_ROCM_EINVAL, "%s: null pointer", what);
+    if (int rc = use_device(dev)) return rc;
+    HIP_TRY(hipMemcpy(dst, src, bytes, kind), what);
+    return 0;
+}
+
+int incin_rocm_memcpy_h2d(int32_t dev, void* dst, const void* src, size_t bytes)
+{
+    return copy(dev, dst, src, bytes, hipMemcpyHostToDevice, "hipMemcpy(host to device)");
+}
+int incin_rocm_memcpy_d2h(int32_t dev, void* dst, const void* src, size_t bytes)
+{
+    return copy(dev, dst, src, bytes, hipMemcpyDeviceToHost, "hipMemcpy(device to host)");
+}
+int incin_rocm_memcpy_d2d(int32_t dev, void* dst, const void* src, size_t bytes)
+{
+    return copy(dev, dst, src, bytes, hipMemcpyDeviceToDevice, "hipMemcpy(device to device)");
+}
+
+int incin_rocm_sync(int32_t dev)
+{
+    if (int rc = use_device(dev)) return rc;
+    HIP_TRY(hipDeviceSynchronize(), "hipDeviceSynchronize");
+    return 0;
+}
+
+int incin_rocm_stream_create(int32_t dev, void** out)
+{
+    if (!out) return fail(INCIN_ROCM_EINVAL, "stream_create: null output");
+    *out = nullptr;
+    if (int rc = use_device(dev)) return rc;
+    hipStream_t s;
+    HIP_TRY(hipStreamCreateWithFlags(&s, hipStreamNonBlocking), "hipStreamCreateWithFlags");   // default priority
+    *out = (void*)s;
+    return 0;
+}
+
+int incin_rocm_stream_destroy(int32_t dev, void* stream)
+{
+    if (!stream) return 0;
+    if (int rc = use_device(dev)) return rc;
+    HIP_TRY(hipStreamDestroy((hipStream_t)stream), "hipStreamDestroy");
+    return 0;
+}
+
+int incin_rocm_stream_sync(int32_t dev, void* stream)
+{
+    if (int rc = use_device(dev)) return rc;
+    HIP_TRY(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize");
+    return 0;
+}
+
+int incin_rocm_event_create(int32_t dev, void** out)
+{
+    if (!out) return fail(INCIN_ROCM_EINVAL, "event_create: null output");
+    *out = nullptr;
+    if (int rc = use_device(dev)) return rc;
+    hipEvent_t e;
+    HIP_TRY(hipEventCreate(&e), "hipEventCreate");
+    *out = (void*)e;
+    return 0;
+}
+
+int incin_rocm_event_destroy(int32_t dev, void* event)
+{
+    if (!event) return 0;
+    if (int rc = use_device(dev)) return rc;
+    HIP_TRY(hipEventDestroy((hipEvent_t)event), "hipEventDestroy");
+    return 0;
+}
+
+int incin_rocm_event_record(int32_t dev, void* event, void* stream)
+{
+    if (!event) return fail(INCIN_ROCM_EINVAL, "event_record: null event");
+    if (int rc = use_device(dev)) return rc;
+    HIP_TRY(hipEventRecord((hipEvent_t)event, (hipStream_t)stream), "hipEventRecord");
+    return 0;
+}
+
+int incin_rocm_event_sync(int32_t dev, void* event)
+{
+    if (!event) return fail(INCIN_ROCM_EINVAL, "event_sync: null event");
+    if (int rc = use_device(dev)) return rc;
+    HIP_TRY(hipEventSynchronize((hipEvent_t)event), "hipEventSynchronize");
+    return 0;
+}
+
+int incin_rocm_event_elapsed_ms(int32_t dev, void* start, void* stop, float* out_ms)
+{
+    if (!start || !stop || !out_ms) return fail(INCIN_ROCM_EINVAL, "event_elapsed_ms: null argument");
+    if (int rc = use_device(dev)) return rc;
+    HIP_TRY(hipEventElapsedTime(out_ms, (hipEvent_t)start, (hipEvent_t)stop), "hipEventElapsedTime");
+    return 0;
+}
+
+int incin_rocm_sdpa_workspace(const incin_rocm_sdpa_desc_t* desc, size_t* bytes, int32_t* splits, int32_t* impl_out)
+{
+    Plan plan;
+    if (int rc = make_plan(desc, &plan)) return rc;
+    if (bytes) *bytes = plan.ws_bytes;
+    if (splits) *splits = plan.splits;
+    if (impl_out) *impl_out = plan.impl;
+    return 0;
+}
+
+int incin_rocm_sdpa_fwd(const incin_rocm_sdpa_desc_t* desc, void* stream)
+{
+    Plan plan;
+    if (int rc = make_plan(desc, &plan)) return rc;
+    if (plan.empty) return 0;
+    if (plan.ws_bytes > 0) {
+        if (!desc->workspace || desc->workspace_bytes < plan.ws_bytes)
+            return fail(INCIN_ROCM_EWORKSPACE,
+                        "scaled_dot_product_attention: split-KV needs %zu workspace bytes, %zu given",
+                        plan.ws_bytes, desc->workspace ? desc->workspace_bytes : (size_t)0);
+        if (!aligned16(desc->workspace)) return fail(INCIN_ROCM_EWORKSPACE, "scaled_dot_product_attention: workspace must be 16-byte aligned");
+    }
+    if (int rc = use_device(desc->device)) return rc;
+    SdpaParams p;
+    fill_params(desc, plan, &p);
+    hipStream_t s = (hipStream_t)stream;
+    hipError_t e;
+    switch (plan.impl) {
+        case INCIN_ROCM_IMPL_MFMA: e = incin_rocm::launch_sdpa_prefill_mfma(p, desc->dtype, s); break;
+        case INCIN_ROCM_IMPL_SPLITKV: e = incin_rocm::launch_sdpa_decode(p, desc->dtype, s); break;
+        default: e = incin_rocm::launch_sdpa_generic(p, desc->dtype, s); break;
+    }
+    if (e != hipSuccess) return hip_fail(e, "attention kernel launch");
+    return 0;
+}
+
+}  // extern "C"

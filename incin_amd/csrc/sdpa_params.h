@@ -1,0 +1,44 @@
+// Kernel-side view of one attention launch (filled from incin_rocm_sdpa_desc_t by
+// the host dispatcher after validation).  Strides are in elements.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace incin_rocm {
+
+struct SdpaParams {
+    const void* q;
+    const void* k;
+    const void* v;
+    void* o;
+    const void* mask;          // nullable dense additive mask (same dtype as q)
+    const int32_t* kv_lens;    // nullable, B entries
+    int64_t q_sb, q_sh, q_ss;
+    int64_t k_sb, k_sh, k_ss;
+    int64_t v_sb, v_sh, v_ss;
+    int64_t o_sb, o_sh, o_ss;
+    int64_t m_sb, m_sh, m_si, m_sj;
+    int32_t B, Hq, Hkv, G;     // G = Hq / Hkv
+    int32_t Sq, Skv, D, Dv;
+    float scale;
+    int32_t causal;
+    // split-KV only
+    int32_t num_splits;
+    int32_t split_len;         // keys per split (multiple of the kernel's key tile)
+    float* ws_acc;             // [B, Hq, Sq, num_splits, Dv] f32 partial numerators
+    float* ws_ml;              // [B, Hq, Sq, num_splits, 2]  running max (natural-log domain) and denominator
+};
+
+typedef __bf16 bf16_t;
+typedef _Float16 f16_t;
+
+template <typename T> __device__ __forceinline__ float to_f32(T x) { return (float)x; }
+template <typename T> __device__ __forceinline__ T from_f32(float x) { return (T)x; }
+
+// Number of keys a query row may look at, before kv_lens: causal alignment puts
+// the last query on the last key (query i sees keys j <= i + Skv - Sq).
+__device__ __forceinline__ int causal_limit(int i, int Sq, int Skv) { return i + (Skv - Sq) + 1; }
+
+__device__ __forceinline__ int clampi(int x, int lo, int hi) { return x < lo ? lo : (x > hi ? hi : x); }
+
+}  // namespace incin_rocm

@@ -1,0 +1,169 @@
+/*
+ * incin_rocm.h -- C ABI of the MI355X (gfx950) attention library that backs an
+ * opt-in `rocm` backend of incin-backends.
+ *
+ * Every entry point returns 0 on success or one of the INCIN_ROCM_E* codes; the
+ * text of the last failure on the calling thread is returned by
+ * incin_rocm_last_error().  No C++ exception, torch type or HIP type crosses
+ * this boundary: plain pointers, sizes and fixed-width integers only.
+ *
+ * What each entry point stands in for in the reference (paths relative to the
+ * reference checkout) is cited on its declaration.  The reference's GPU backends
+ * reach their driver through the `cudarc` crate; the same call shapes are what a
+ * Rust `incin-rocm-sys` crate binds here (bindings shown in INTEGRATION.md).
+ */
+#ifndef INCIN_ROCM_H
+#define INCIN_ROCM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define INCIN_ROCM_ABI_VERSION 1
+
+/* ---- status codes (mapped to incin_core::Error variants by the Rust side;
+ *      crates/incin-core/src/err.rs:109-223) --------------------------------- */
+enum {
+    INCIN_ROCM_OK = 0,
+    INCIN_ROCM_EINVAL = 1,        /* null pointer / malformed descriptor  -> Error::Msg                    */
+    INCIN_ROCM_ESHAPE = 2,        /* shape or stride rule violated        -> Error::ShapeMismatch          */
+    INCIN_ROCM_EDTYPE = 3,        /* dtype outside {f32,f16,bf16}         -> Error::UnsupportedDType       */
+    INCIN_ROCM_EDEVICE = 4,       /* bad ordinal / no device              -> Error::InvalidDeviceOrdinal   */
+    INCIN_ROCM_ENOMEM = 5,        /* device allocation failed             -> Error::OutOfMemory            */
+    INCIN_ROCM_EWORKSPACE = 6,    /* workspace missing or too small       -> Error::Msg                    */
+    INCIN_ROCM_EUNSUPPORTED = 7,  /* valid request with no kernel         -> Error::UnsupportedBackendOperation */
+    INCIN_ROCM_ERUNTIME = 8       /* HIP call failed                      -> Error::Msg("ROCm ... failed")  */
+};
+
+/* dtype tags: the float subset of DTypeId (crates/incin-core/src/tensor/dtype.rs:10-101) */
+enum { INCIN_ROCM_F32 = 0, INCIN_ROCM_F16 = 1, INCIN_ROCM_BF16 = 2 };
+
+/* kernel selection for incin_rocm_sdpa_desc_t.impl */
+enum {
+    INCIN_ROCM_IMPL_AUTO = 0,
+    INCIN_ROCM_IMPL_GENERIC = 1,   /* fp32-FMA tiled kernel: any dtype, D and Dv <= 256, dense masks     */
+    INCIN_ROCM_IMPL_MFMA = 2,      /* bf16/f16 MFMA prefill kernel: D == Dv in {64,128}                    */
+    INCIN_ROCM_IMPL_SPLITKV = 3    /* split-KV decode kernel + combine: D == Dv in {64,128}, few query rows */
+};
+
+/* Thread-local message of the last failing call on this thread ("" if none).
+ * Replaces the `Display` text cudarc errors carry into Error::Msg
+ * (crates/incin-backends/src/cuda/ops/matmul.rs:89). */
+const char* incin_rocm_last_error(void);
+int incin_rocm_abi_version(void);
+
+/* ---- device table -----------------------------------------------------------
+ * Replaces the per-ordinal context cache of the CUDA backend
+ * (crates/incin-backends/src/cuda/gpu.rs:99-152: `CudaContext::new(ordinal)`
+ * behind a process-wide map) and `detect::probe`
+ * (crates/incin-backends/src/detect.rs:69-77). */
+typedef struct {
+    char name[64];
+    char arch[32];              /* gcnArchName, e.g. "gfx950:sramecc+:xnack-" */
+    int32_t compute_units;
+    int32_t clock_khz;          /* max engine clock */
+    int32_t memory_clock_khz;
+    int32_t memory_bus_bits;
+    int32_t lds_bytes_per_block;
+    int32_t wavefront_size;
+    uint64_t hbm_bytes;
+} incin_rocm_device_info_t;
+
+int incin_rocm_device_count(int32_t* out);
+int incin_rocm_device_info(int32_t dev, incin_rocm_device_info_t* out);
+
+/* ---- buffers ----------------------------------------------------------------
+ * Replace CudaBuffer allocation and the H2D / D2H copies behind
+ * Backend::from_bytes / Backend::to_bytes
+ * (crates/incin-backends/src/cuda/storage.rs:24-59,
+ *  crates/incin-backends/src/cuda/backend.rs:1905-1937, 2007-2045).
+ * Allocations are at least 256-byte aligned (cuda/storage.rs:18).  Copies are
+ * synchronous with respect to the host, as the reference's are. */
+int incin_rocm_alloc(int32_t dev, size_t bytes, void** out);
+int incin_rocm_free(int32_t dev, void* ptr);
+int incin_rocm_memset(int32_t dev, void* dst, int value, size_t bytes);
+int incin_rocm_memcpy_h2d(int32_t dev, void* dst, const void* src, size_t bytes);
+int incin_rocm_memcpy_d2h(int32_t dev, void* dst, const void* src, size_t bytes);
+int incin_rocm_memcpy_d2d(int32_t dev, void* dst, const void* src, size_t bytes);
+int incin_rocm_sync(int32_t dev);      /* waits for the device's default stream and any stream created here */
+
+/* ---- streams and events -------------------------------------------------------
+ * The reference launches on cudarc's per-context default stream
+ * (crates/incin-backends/src/cuda/ops/matmul.rs:57-90); a NULL stream here means
+ * the same.  Streams are created at default priority only.  Events exist so a
+ * caller can time launches on the stream they were issued to. */
+int incin_rocm_stream_create(int32_t dev, void** out);
+int incin_rocm_stream_destroy(int32_t dev, void* stream);
+int incin_rocm_stream_sync(int32_t dev, void* stream);
+int incin_rocm_event_create(int32_t dev, void** out);
+int incin_rocm_event_destroy(int32_t dev, void* event);
+int incin_rocm_event_record(int32_t dev, void* event, void* stream);
+int incin_rocm_event_sync(int32_t dev, void* event);
+int incin_rocm_event_elapsed_ms(int32_t dev, void* start, void* stop, float* out_ms);
+
+/* ---- attention forward --------------------------------------------------------
+ * Replaces CpuBackendImpl::scaled_dot_product_attention
+ * (crates/incin-backends/src/cpu/ops/shape_ops.rs:1245-1269), the only
+ * implementation of TensorOps::scaled_dot_product_attention
+ * (crates/incin-core/src/tensor/backend.rs:485-492):
+ *
+ *     o = softmax(q k^T * scale + mask) v        row-wise softmax over keys
+ *
+ * The caller has already collapsed the operator's leading axes into
+ * (B, Hkv, G) by the reference's batch-broadcast rule
+ * (crates/incin-backends/src/cpu/ops/matmul.rs:198-221): query head hq reads
+ * key/value head hq / (Hq / Hkv); a broadcast axis is a stride of 0.
+ *
+ * Masking.  The reference knows one mask form, an additive tensor broadcast
+ * against the scores (shape_ops.rs:1262-1266).  `add_mask` is that tensor.
+ * `causal` and `kv_lens` state, without materialising them, the two additive
+ * masks of 0 / -inf that callers build most: key j is masked (as if -inf were
+ * added) when  causal != 0 and j > i + (Skv - Sq),  or  kv_lens != NULL and
+ * j >= kv_lens[b].  All three may be combined.  A query row with every key
+ * masked yields NaN, as the reference's softmax does (-inf - -inf).
+ *
+ * Output dtype equals the input dtype; accumulation is f32
+ * (crates/incin-backends/src/dtype_policy.rs:64-104).
+ */
+typedef struct {
+    int32_t dtype;                 /* INCIN_ROCM_F32 / F16 / BF16: q, k, v, o and add_mask all share it */
+    int32_t device;
+    int64_t B, Hq, Hkv, Sq, Skv, D, Dv;
+    int64_t q_stride[3];           /* elements: batch, head, sequence; the last axis has stride 1 */
+    int64_t k_stride[3];
+    int64_t v_stride[3];
+    int64_t o_stride[3];
+    const void* q;
+    const void* k;
+    const void* v;
+    void* o;
+    float scale;                   /* resolved by the caller: (float) scale.unwrap_or(1/sqrt(D)), the f64 -> f32
+                                      cast of shape_ops.rs:1259-1261 + elementwise_kernel.rs:87 */
+    int32_t causal;                /* 0 / 1 */
+    const int32_t* kv_lens;        /* nullable device pointer, B entries */
+    const void* add_mask;          /* nullable device pointer, dtype `dtype` */
+    int64_t mask_stride[4];        /* elements: batch, query head, query row, key; 0 = broadcast */
+    void* workspace;               /* device scratch for split-KV partials; see incin_rocm_sdpa_workspace */
+    size_t workspace_bytes;
+    int32_t num_splits;            /* 0 = library chooses */
+    int32_t impl;                  /* INCIN_ROCM_IMPL_*; AUTO unless a test pins a kernel */
+} incin_rocm_sdpa_desc_t;
+
+/* Validates the descriptor and reports the scratch bytes and the split count the
+ * launch will use (0 bytes and 1 split when the chosen kernel needs none).
+ * `impl_out` (nullable) receives the INCIN_ROCM_IMPL_* the library will run. */
+int incin_rocm_sdpa_workspace(const incin_rocm_sdpa_desc_t* desc, size_t* bytes, int32_t* splits, int32_t* impl_out);
+
+/* Enqueues the kernels on `stream` (NULL = the device's default stream) and
+ * returns without waiting.  The library keeps no pointer after return except the
+ * stream-ordered use of the buffers named in the descriptor, which the caller
+ * keeps alive until the stream has been synchronised. */
+int incin_rocm_sdpa_fwd(const incin_rocm_sdpa_desc_t* desc, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* INCIN_ROCM_H */
