@@ -19,6 +19,7 @@ OK, EINVAL, ESHAPE, EDTYPE, EDEVICE, ENOMEM, EWORKSPACE, EUNSUPPORTED, ERUNTIME 
 
 EXPORTS = [
     "incin_rocm_last_error", "incin_rocm_abi_version",
+    "incin_rocm_sizeof_sdpa_desc", "incin_rocm_sizeof_device_info",
     "incin_rocm_device_count", "incin_rocm_device_info",
     "incin_rocm_alloc", "incin_rocm_free", "incin_rocm_memset",
     "incin_rocm_memcpy_h2d", "incin_rocm_memcpy_d2h", "incin_rocm_memcpy_d2d", "incin_rocm_sync",
@@ -89,6 +90,10 @@ def load():
     lib.incin_rocm_last_error.restype = C.c_char_p
     for name in EXPORTS[1:]:
         getattr(lib, name).restype = C.c_int
+    lib.incin_rocm_sizeof_sdpa_desc.restype = C.c_size_t
+    lib.incin_rocm_sizeof_device_info.restype = C.c_size_t
+    if lib.incin_rocm_sizeof_sdpa_desc() != C.sizeof(SdpaDesc) or lib.incin_rocm_sizeof_device_info() != C.sizeof(DeviceInfo):
+        raise RuntimeError("libincin_rocm.so was built from a different include/incin_rocm.h than this binding mirrors")
     lib.incin_rocm_alloc.argtypes = [C.c_int32, C.c_size_t, C.POINTER(C.c_void_p)]
     lib.incin_rocm_free.argtypes = [C.c_int32, C.c_void_p]
     lib.incin_rocm_memset.argtypes = [C.c_int32, C.c_void_p, C.c_int, C.c_size_t]

@@ -193,6 +193,8 @@ extern "C" {
 
 const char* incin_rocm_last_error(void) { return g_err; }
 int incin_rocm_abi_version(void) { return INCIN_ROCM_ABI_VERSION; }
+size_t incin_rocm_sizeof_sdpa_desc(void) { return sizeof(incin_rocm_sdpa_desc_t); }
+size_t incin_rocm_sizeof_device_info(void) { return sizeof(incin_rocm_device_info_t); }
 
 int incin_rocm_device_count(int32_t* out)
 {

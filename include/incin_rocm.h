@@ -54,6 +54,9 @@ enum {
  * (crates/incin-backends/src/cuda/ops/matmul.rs:89). */
 const char* incin_rocm_last_error(void);
 int incin_rocm_abi_version(void);
+/* sizeof the two structs below as this build sees them, so a binding can check its mirrors. */
+size_t incin_rocm_sizeof_sdpa_desc(void);
+size_t incin_rocm_sizeof_device_info(void);
 
 /* ---- device table -----------------------------------------------------------
  * Replaces the per-ordinal context cache of the CUDA backend

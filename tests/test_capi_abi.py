@@ -1,0 +1,100 @@
+"""CPU-side checks of the C ABI: the library loads, exports every symbol the header
+declares, the descriptor layout matches the ctypes mirror, and descriptor
+validation (which runs before any device call) reports the documented codes."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from incin_amd import capi
+
+HEADER = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include", "incin_rocm.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(incin_rocm_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = capi.load()
+    names = declared_functions()
+    assert len(names) >= 20
+    for n in names:
+        assert hasattr(lib, n), "missing export %s" % n
+    assert set(names) == set(capi.EXPORTS)
+    assert lib.incin_rocm_abi_version() == 1
+
+
+def test_descriptor_layout_matches():
+    lib = capi.load()
+    lib.incin_rocm_sizeof_sdpa_desc.restype = C.c_size_t
+    assert lib.incin_rocm_sizeof_sdpa_desc() == C.sizeof(capi.SdpaDesc)
+    lib.incin_rocm_sizeof_device_info.restype = C.c_size_t
+    assert lib.incin_rocm_sizeof_device_info() == C.sizeof(capi.DeviceInfo)
+
+
+def _desc(**kw):
+    d = capi.SdpaDesc()
+    d.dtype, d.device = capi.BF16, 0
+    d.B, d.Hq, d.Hkv, d.Sq, d.Skv, d.D, d.Dv = 2, 4, 4, 128, 128, 128, 128
+    for name in ("q_stride", "k_stride", "v_stride", "o_stride"):
+        st = getattr(d, name)
+        st[0], st[1], st[2] = 4 * 128 * 128, 128 * 128, 128
+    d.q = d.k = d.v = d.o = 0x10000          # never dereferenced by validation
+    d.scale = 0.088
+    for k, v in kw.items():
+        setattr(d, k, v)
+    return d
+
+
+def _plan(d):
+    return capi.sdpa_workspace(d)
+
+
+def test_dispatch_choices():
+    assert _plan(_desc())[2] == capi.IMPL_MFMA
+    assert _plan(_desc(dtype=capi.F32))[2] == capi.IMPL_GENERIC
+    assert _plan(_desc(D=80, Dv=80))[2] == capi.IMPL_GENERIC
+    assert _plan(_desc(add_mask=0x20000))[2] == capi.IMPL_GENERIC
+    nbytes, splits, impl = _plan(_desc(Sq=1, Skv=8192, B=32, Hq=32, Hkv=32))
+    assert impl == capi.IMPL_SPLITKV and splits >= 1
+    assert nbytes == (0 if splits == 1 else 32 * 32 * 1 * splits * (128 + 2) * 4)
+    nbytes, splits, impl = _plan(_desc(Sq=1, Skv=8192, B=1, Hq=8, Hkv=2, num_splits=4))
+    assert impl == capi.IMPL_SPLITKV and splits == 4 and nbytes == 8 * 4 * 130 * 4
+    assert _plan(_desc(Sq=1, Skv=64))[2] in (capi.IMPL_MFMA, capi.IMPL_SPLITKV)
+    # empty problems need nothing
+    assert _plan(_desc(Sq=0))[0] == 0
+
+
+@pytest.mark.parametrize("kw,code", [
+    (dict(dtype=7), capi.EDTYPE),
+    (dict(Sq=-1), capi.ESHAPE),
+    (dict(Hq=6, Hkv=4), capi.ESHAPE),
+    (dict(q=None), capi.EINVAL),
+    (dict(impl=9), capi.EINVAL),
+    (dict(num_splits=-2), capi.EINVAL),
+    (dict(impl=capi.IMPL_MFMA, dtype=capi.F32), capi.EUNSUPPORTED),
+    (dict(impl=capi.IMPL_MFMA, D=80, Dv=80), capi.EUNSUPPORTED),
+    (dict(impl=capi.IMPL_SPLITKV, Sq=4096), capi.EUNSUPPORTED),
+    (dict(D=512, Dv=512), capi.EUNSUPPORTED),
+    (dict(B=70000), capi.ESHAPE),
+])
+def test_validation_errors(kw, code):
+    with pytest.raises(capi.RocmError) as e:
+        _plan(_desc(**kw))
+    assert e.value.code == code
+    assert e.value.message and capi.load().incin_rocm_last_error().decode() == e.value.message
+
+
+def test_null_descriptor_and_missing_workspace():
+    lib = capi.load()
+    assert lib.incin_rocm_sdpa_workspace(None, None, None, None) == capi.EINVAL
+    assert lib.incin_rocm_sdpa_fwd(None, None) == capi.EINVAL
+    d = _desc(Sq=1, Skv=8192, B=1, Hq=8, Hkv=8, num_splits=4)
+    with pytest.raises(capi.RocmError) as e:      # rejected before any device is touched
+        capi.sdpa_fwd(d)
+    assert e.value.code == capi.EWORKSPACE
+    assert lib.incin_rocm_device_count(None) == capi.EINVAL

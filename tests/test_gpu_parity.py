@@ -1,0 +1,248 @@
+"""Parity of the HIP kernels (through the C ABI) with the CPU oracle.
+
+Tolerances (max-abs error against the f32 oracle run on the same inputs, which
+for f16/bf16 are first rounded to the storage dtype):
+    f32  1e-5        f16 / bf16  2e-2
+"""
+import sys
+
+import numpy as np
+import pytest
+
+from incin_amd import capi, dtypes, host
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+TOL = {capi.F32: 1e-5, capi.F16: 2e-2, capi.BF16: 2e-2}
+SEED0 = 20261125
+
+
+def say(msg):
+    print(msg, file=sys.stderr, flush=True)
+
+
+def rng(seed):
+    return np.random.Generator(np.random.PCG64(seed))
+
+
+def inputs(seed, B, Hq, Hkv, Sq, Skv, D, Dv, dtype):
+    r = rng(seed)
+    q = dtypes.round_to(r.standard_normal((B, Hq, Sq, D), dtype=np.float32), dtype)
+    k = dtypes.round_to(r.standard_normal((B, Hkv, Skv, D), dtype=np.float32), dtype)
+    v = dtypes.round_to(r.standard_normal((B, Hkv, Skv, Dv), dtype=np.float32), dtype)
+    return q, k, v
+
+
+def oracle_full(q, k, v, G=1, **kw):
+    """Oracle on [B,Hq,..] operands; GQA is expressed the way the reference expresses it:
+    q [B,Hkv,G,S,D] against k, v [B,Hkv,1,S,D]."""
+    B, Hq, Sq, D = q.shape
+    Hkv = k.shape[1]
+    q5 = q.reshape(B, Hkv, G, Sq, D)
+    k5, v5 = k[:, :, None], v[:, :, None]
+    if "kv_lens" in kw and kw["kv_lens"] is not None:
+        kw = dict(kw, kv_lens=np.asarray(kw["kv_lens"], np.int32).reshape(B, 1, 1))
+    if kw.get("mask") is not None:
+        m = np.asarray(kw["mask"], np.float32)
+        if m.ndim == 4:                                    # [B|1, Hq|1, Sq, Skv] -> [B|1, Hkv|1, G|1, Sq, Skv]
+            if m.shape[1] == 1:
+                m = m[:, :, None]
+            else:
+                m = m.reshape(m.shape[0], Hkv, G, m.shape[2], m.shape[3])
+        kw = dict(kw, mask=m)
+    out = O.sdpa(q5, k5, v5, **kw)
+    return out.reshape(B, Hq, Sq, -1)
+
+
+def check(got, ref, tol, what):
+    assert got.shape == ref.shape, what
+    nan_g, nan_r = np.isnan(got), np.isnan(ref)
+    assert np.array_equal(nan_g, nan_r), "%s: NaN pattern differs (%d vs %d)" % (what, nan_g.sum(), nan_r.sum())
+    err = np.abs(np.where(nan_r, 0, got) - np.where(nan_r, 0, ref)).max() if got.size else 0.0
+    say("%s: max-abs err %.3e (tol %.0e)" % (what, err, tol))
+    assert err <= tol, "%s: max-abs error %.3e > %.0e" % (what, err, tol)
+
+
+def test_device_is_gfx950(gpu):
+    info = gpu.device_info(0)
+    say("device: %s %s CUs=%d clk=%d kHz" % (info.name.decode(), info.arch.decode(), info.compute_units, info.clock_khz))
+    assert info.arch.decode().startswith("gfx950")
+    assert info.wavefront_size == 64
+    with pytest.raises(capi.RocmError) as e:
+        gpu.device_info(99)
+    assert e.value.code == capi.EDEVICE
+
+
+def test_buffer_round_trip(gpu):
+    x = rng(1).standard_normal(100003).astype(np.float32)
+    buf = capi.DeviceBuffer.from_numpy(x)
+    assert buf.ptr % 256 == 0
+    assert np.array_equal(buf.to_numpy(np.float32, x.shape), x)
+    buf.free()
+    raw = dtypes.encode(x, capi.BF16)
+    t = host.DeviceTensor.from_f32(x.reshape(1, 1, 1, -1), capi.BF16)
+    assert np.array_equal(dtypes.encode(t.to_f32(), capi.BF16).reshape(-1), raw)
+
+
+# ---- BASELINE configs 1 and 2 (f32) ------------------------------------------------
+
+def test_config1_f32_single_head_noncausal(gpu):
+    q, k, v = inputs(SEED0 + 0, 1, 1, 1, 128, 128, 64, 64, capi.F32)
+    got, info = host.sdpa(q, k, v, capi.F32, scale=0.125, return_info=True)
+    assert info["impl"] == capi.IMPL_GENERIC
+    ref = O.sdpa(q, k, v, scale=0.125)
+    check(got, ref, 1e-5, "C1 f32 B1 H1 S128 D64")
+    assert np.abs(ref - O.brute_f64(q, k, v, scale=0.125)).max() < 1e-6
+
+
+def test_config2_f32_multi_head_causal(gpu):
+    q, k, v = inputs(SEED0 + 1, 4, 8, 8, 1024, 1024, 64, 64, capi.F32)
+    got = host.sdpa(q, k, v, capi.F32, causal=True)
+    mask = O.causal_additive_mask(1024, 1024)                       # the explicit 0/-inf tensor the CPU op is given
+    ref = O.sdpa(q, k, v, mask=mask)
+    check(got, ref, 1e-5, "C2 f32 B4 H8 S1024 D64 causal")
+    # the same mask handed over as a dense additive tensor goes through the mask path of the kernel
+    got2 = host.sdpa(q[:1, :2], k[:1, :2], v[:1, :2], capi.F32, mask=mask)
+    check(got2, ref[:1, :2], 1e-5, "C2 slice, dense additive mask")
+
+
+# ---- generic kernel: shapes, masks, dtypes ----------------------------------------------
+
+@pytest.mark.parametrize("dtype", [capi.F32, capi.F16, capi.BF16])
+@pytest.mark.parametrize("shape", [
+    # B, Hq, Hkv, Sq, Skv, D, Dv
+    (1, 1, 1, 1, 1, 1, 1),
+    (2, 3, 3, 77, 131, 40, 72),
+    (1, 4, 2, 65, 64, 128, 128),
+    (2, 2, 1, 5, 300, 200, 256),
+    (1, 2, 2, 130, 7, 16, 8),
+])
+def test_generic_shapes(gpu, dtype, shape):
+    B, Hq, Hkv, Sq, Skv, D, Dv = shape
+    q, k, v = inputs(100 + sum(shape), B, Hq, Hkv, Sq, Skv, D, Dv, dtype)
+    for causal in (False, True):
+        got = host.sdpa(q, k, v, dtype, causal=causal, impl=capi.IMPL_GENERIC)
+        ref = oracle_full(q, k, v, G=Hq // Hkv, causal=causal)
+        check(got, ref, TOL[dtype], "generic %s %r causal=%d" % (dtypes.NAMES[dtype], shape, causal))
+
+
+@pytest.mark.parametrize("dtype", [capi.F32, capi.BF16])
+def test_generic_dense_masks_and_lengths(gpu, dtype):
+    B, Hq, Hkv, Sq, Skv, D = 2, 4, 2, 70, 90, 32
+    q, k, v = inputs(7, B, Hq, Hkv, Sq, Skv, D, D, dtype)
+    r = rng(8)
+    for mshape in [(Sq, Skv), (1, Skv), (B, 1, Sq, Skv), (B, Hq, Sq, Skv), (1, Hq, 1, Skv)]:
+        m = dtypes.round_to(r.standard_normal(mshape, dtype=np.float32), dtype)
+        m = np.where(r.random(mshape) < 0.25, -np.inf, m).astype(np.float32)
+        m[..., 0] = 0.0                                             # keep every row alive
+        got = host.sdpa(q, k, v, dtype, mask=m, scale=0.3)
+        ref = oracle_full(q, k, v, G=2, mask=m, scale=0.3)
+        check(got, ref, TOL[dtype], "generic %s mask %r" % (dtypes.NAMES[dtype], mshape))
+    lens = np.array([0, 37], np.int32)                              # batch 0 has no visible key: NaN rows, as the reference
+    got = host.sdpa(q, k, v, dtype, kv_lens=lens, causal=True, impl=capi.IMPL_GENERIC)
+    ref = oracle_full(q, k, v, G=2, kv_lens=lens, causal=True)
+    assert np.isnan(ref[0]).all() and np.isfinite(ref[1]).all()
+    check(got, ref, TOL[dtype], "generic %s kv_lens+causal" % dtypes.NAMES[dtype])
+    m = np.zeros((Sq, Skv), np.float32)
+    m[3, :] = -np.inf                                               # one fully masked row
+    got = host.sdpa(q, k, v, dtype, mask=m)
+    check(got, oracle_full(q, k, v, G=2, mask=m), TOL[dtype], "generic fully masked row")
+
+
+def test_reference_golden_vectors_on_gpu(gpu):
+    import json, os
+    gold = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_vectors.json")))
+    g = gold["attention_heads"]
+    q = np.array([c["q"] for c in g["cases"]], np.float32).reshape(1, 2, 2, 1)
+    k = np.array([c["k"] for c in g["cases"]], np.float32).reshape(1, 2, 2, 1)
+    v = np.array([c["v"] for c in g["cases"]], np.float32).reshape(1, 2, 2, 1)
+    got = host.sdpa(q, k, v, capi.F32, scale=g["scale"]).reshape(-1)
+    exp = np.array([c["expected"] for c in g["cases"]]).reshape(-1)
+    assert np.abs(got - exp).max() <= g["tol"]
+    ones = np.ones((1, 1, 2, 4), np.float32)
+    got = host.sdpa(ones, ones, ones, capi.F32)
+    assert got.shape == (1, 1, 2, 4) and np.abs(got - 1.0).max() <= gold["sdpa_ones"]["tol"]
+    for case in gold["softmax"]["cases"]:
+        x = np.array(case["x"], np.float32)
+        got = host.sdpa(np.ones((1, 1, 1, 1), np.float32), x.reshape(1, 1, -1, 1),
+                        np.eye(len(x), dtype=np.float32).reshape(1, 1, len(x), len(x)), capi.F32, scale=1.0)
+        assert np.abs(got.reshape(-1) - np.array(case["expected"])).max() <= case["tol"]
+
+
+# ---- MFMA prefill kernel --------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", [capi.BF16, capi.F16])
+@pytest.mark.parametrize("shape", [
+    # B, Hq, Hkv, Sq, Skv, D
+    (1, 1, 1, 128, 128, 128),
+    (2, 4, 4, 512, 512, 128),
+    (1, 2, 2, 200, 333, 128),
+    (2, 8, 2, 256, 256, 128),
+    (1, 4, 1, 100, 1000, 64),
+    (1, 2, 2, 384, 129, 64),
+    (1, 1, 1, 17, 64, 128),
+])
+def test_mfma_prefill(gpu, dtype, shape):
+    B, Hq, Hkv, Sq, Skv, D = shape
+    q, k, v = inputs(200 + sum(shape), B, Hq, Hkv, Sq, Skv, D, D, dtype)
+    for causal in (False, True):
+        got, info = host.sdpa(q, k, v, dtype, causal=causal, impl=capi.IMPL_MFMA, return_info=True)
+        assert info["impl"] == capi.IMPL_MFMA
+        ref = oracle_full(q, k, v, G=Hq // Hkv, causal=causal)
+        check(got, ref, TOL[dtype], "mfma %s %r causal=%d" % (dtypes.NAMES[dtype], shape, causal))
+        gen = host.sdpa(q, k, v, dtype, causal=causal, impl=capi.IMPL_GENERIC)
+        check(got, gen, TOL[dtype], "mfma vs generic kernel %r causal=%d" % (shape, causal))
+
+
+def test_mfma_prefill_ragged_lengths(gpu):
+    B, Hq, Hkv, S, D = 3, 8, 2, 640, 128
+    q, k, v = inputs(31, B, Hq, Hkv, S, S, D, D, capi.BF16)
+    lens = np.array([640, 129, 0], np.int32)
+    got = host.sdpa(q, k, v, capi.BF16, causal=True, kv_lens=lens, impl=capi.IMPL_MFMA)
+    ref = oracle_full(q, k, v, G=4, causal=True, kv_lens=lens)
+    check(got, ref, 2e-2, "mfma bf16 GQA causal + kv_lens")
+    # padded keys == truncated keys
+    trunc = host.sdpa(q[1:2, :, :, :], k[1:2, :, :129], v[1:2, :, :129], capi.BF16, impl=capi.IMPL_MFMA)
+    padded = host.sdpa(q[1:2], k[1:2], v[1:2], capi.BF16, kv_lens=lens[1:2], impl=capi.IMPL_MFMA)
+    check(padded, trunc, 1e-6, "mfma padded == truncated")
+
+
+# ---- split-KV decode -----------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", [capi.BF16, capi.F16, capi.F32])
+@pytest.mark.parametrize("shape", [
+    # B, Hq, Hkv, Sq, Skv, D
+    (2, 4, 4, 1, 4096, 128),
+    (1, 8, 2, 1, 3000, 128),
+    (2, 8, 1, 1, 2048, 64),
+    (1, 2, 2, 3, 1500, 128),
+    (1, 16, 1, 1, 700, 64),
+])
+def test_decode_splitkv(gpu, dtype, shape):
+    B, Hq, Hkv, Sq, Skv, D = shape
+    q, k, v = inputs(300 + sum(shape), B, Hq, Hkv, Sq, Skv, D, D, dtype)
+    ref = oracle_full(q, k, v, G=Hq // Hkv, causal=True)
+    outs = []
+    for splits in (0, 1, 3, 8):
+        got, info = host.sdpa(q, k, v, dtype, causal=True, num_splits=splits, impl=capi.IMPL_SPLITKV, return_info=True)
+        assert info["impl"] == capi.IMPL_SPLITKV
+        check(got, ref, TOL[dtype], "decode %s %r splits=%d->%d" % (dtypes.NAMES[dtype], shape, splits, info["splits"]))
+        outs.append(got)
+    for o in outs[1:]:                                              # split-KV + combine == unsplit
+        check(o, outs[1], 1e-5 if dtype == capi.F32 else 8e-3, "decode split-count invariance")
+
+
+def test_decode_lengths_and_prefill_consistency(gpu):
+    B, H, Skv, D = 3, 4, 2048, 128
+    q, k, v = inputs(41, B, H, H, 1, Skv, D, D, capi.BF16)
+    lens = np.array([2048, 5, 0], np.int32)
+    got = host.sdpa(q, k, v, capi.BF16, kv_lens=lens, num_splits=4)
+    ref = oracle_full(q, k, v, kv_lens=lens)
+    assert np.isnan(ref[2]).all()
+    check(got, ref, 2e-2, "decode kv_lens incl. empty")
+    # decode output == last row of causal prefill over the same cache
+    qf, kf, vf = inputs(42, 1, 2, 2, 512, 512, 128, 128, capi.BF16)
+    full = host.sdpa(qf, kf, vf, capi.BF16, causal=True, impl=capi.IMPL_MFMA)
+    last = host.sdpa(qf[:, :, -1:], kf, vf, capi.BF16, causal=True)
+    check(last, full[:, :, -1:], 8e-3, "decode == last row of causal prefill")
