@@ -1,0 +1,219 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+One "step" is one launch of `incin_rocm_sdpa_fwd` over one batch of synthetic
+input already resident in HBM.  The headline workload is BASELINE config 3
+(bf16 causal prefill, B=8 H=16 S=4096 D=128); BASELINE config 4 (bf16 decode,
+B=32 H=32 KV=8192 D=128, split-KV + combine) is measured in the same run and
+reported under "decode".  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+
+Timing: K steps between two device synchronisations (wall clock -> ms_per_step,
+value) and, for the roofline figure, HIP events recorded around every launch on
+the stream the kernels run on (the library's event entry points).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+from incin_amd import capi, dtypes, host  # noqa: E402
+
+SEED0 = 20261125
+PEAK_BF16_TFLOPS = 2516.6   # 256 CUs x 2.4 GHz x 4096 dense bf16 FLOP/clk/CU (vendor: 2.5 PFLOP/s)
+PEAK_HBM_GBS = 8000.0       # HBM3E, vendor figure
+METRIC = "attn fwd TFLOP/s + % bf16 MFMA peak; decode KV GB/s + % HBM peak (1 GPU)"
+
+
+def rng(seed):
+    return np.random.Generator(np.random.PCG64(seed))
+
+
+def make_inputs(seed, B, Hq, Hkv, Sq, Skv, D, dtype):
+    r = rng(seed)
+    q = r.standard_normal((B, Hq, Sq, D), dtype=np.float32)
+    k = r.standard_normal((B, Hkv, Skv, D), dtype=np.float32)
+    v = r.standard_normal((B, Hkv, Skv, D), dtype=np.float32)
+    return q, k, v
+
+
+def causal_flops(B, Hq, Sq, Skv, D):
+    pairs = sum(min(max(i + 1 + Skv - Sq, 0), Skv) for i in range(Sq)) if Sq != Skv else Sq * (Sq + 1) // 2
+    return 4.0 * D * B * Hq * pairs
+
+
+class Workload:
+    """Device-resident operands + descriptor for one configuration."""
+
+    def __init__(self, name, seed, B, Hq, Hkv, Sq, Skv, D, dtype, causal):
+        self.name, self.shape = name, (B, Hq, Hkv, Sq, Skv, D)
+        self.dtype, self.causal = dtype, causal
+        q, k, v = make_inputs(seed, B, Hq, Hkv, Sq, Skv, D, dtype)
+        self.host = (q, k, v)
+        self.tq, self.tk, self.tv = (host.DeviceTensor.from_f32(x, dtype) for x in (q, k, v))
+        self.to = host.DeviceTensor((B, Hq, Sq, D), dtype)
+        self.desc = host.make_desc(self.tq, self.tk, self.tv, self.to, causal=causal)
+        nbytes, self.splits, self.impl = capi.sdpa_workspace(self.desc)
+        self.ws = capi.DeviceBuffer(nbytes) if nbytes else None
+        if self.ws is not None:
+            self.desc.workspace, self.desc.workspace_bytes = self.ws.ptr, self.ws.nbytes
+
+    def launch(self):
+        capi.sdpa_fwd(self.desc)
+
+    def time(self, steps, warmup):
+        """(wall ms per step over `steps` back-to-back launches, mean / median / min event ms per launch)"""
+        for _ in range(warmup):
+            self.launch()
+        capi.sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            self.launch()
+        capi.sync()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+        starts = [capi.Event() for _ in range(steps)]
+        stops = [capi.Event() for _ in range(steps)]
+        for i in range(steps):
+            starts[i].record()
+            self.launch()
+            stops[i].record()
+        capi.sync()
+        ev = np.array([starts[i].elapsed_ms(stops[i]) for i in range(steps)])
+        for e in starts + stops:
+            e.destroy()
+        return wall_ms, float(ev.mean()), float(np.median(ev)), float(ev.min())
+
+    def parity(self, n_rows=48):
+        """max-abs error of sampled output rows against the CPU oracle (checker only)."""
+        from oracle import oracle as O
+        B, Hq, Hkv, Sq, Skv, D = self.shape
+        G = Hq // Hkv
+        q, k, v = (dtypes.round_to(x, self.dtype) for x in self.host)
+        out = self.to.to_f32()
+        r = rng(99)
+        rows = np.stack([r.integers(0, B * Hq, n_rows), r.integers(0, Sq, n_rows)], axis=1)
+        rows[0] = (0, 0)
+        rows[1] = (B * Hq - 1, Sq - 1)
+        ref = O.sdpa_rows(q.reshape(B, Hkv, G, Sq, D), k[:, :, None], v[:, :, None], rows, causal=self.causal)
+        got = out.reshape(B * Hq, Sq, D)[rows[:, 0], rows[:, 1]]
+        return float(np.abs(got - ref).max())
+
+    def free(self):
+        for t in (self.tq.buf, self.tk.buf, self.tv.buf, self.to.buf, self.ws):
+            if t is not None:
+                t.free()
+
+
+def cpu_baseline_prefill(D, S, slices, dtype):
+    """The oracle's materialising form (the reference's execution shape: serial matmuls and
+    reductions, threaded elementwise maps) on `slices` (b,h) slices of the causal-prefill workload."""
+    from oracle import oracle as O
+    q, k, v = make_inputs(SEED0 + 2, 1, slices, slices, S, S, D, dtype)
+    q, k, v = (dtypes.round_to(x, dtype) for x in (q, k, v))
+    mask = O.causal_additive_mask(S, S)
+    t0 = time.perf_counter()
+    O.sdpa_materialised(q, k, v, mask=mask)
+    dt = time.perf_counter() - t0
+    return causal_flops(1, slices, S, S, D) / dt / 1e12, dt
+
+
+def cpu_baseline_decode(D, Skv, B, H, dtype):
+    from oracle import oracle as O
+    q, k, v = make_inputs(SEED0 + 3, B, H, H, 1, Skv, D, dtype)
+    q, k, v = (dtypes.round_to(x, dtype) for x in (q, k, v))
+    t0 = time.perf_counter()
+    O.sdpa_materialised(q, k, v)
+    dt = time.perf_counter() - t0
+    return 2.0 * B * H * Skv * D * 2 / dt / 1e9, dt
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only", choices=["prefill", "decode"], default=None,
+                    help="run a single workload (profiling); the JSON line still has every key")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path shards over batch and kv-head groups "
+              "with no communication; no multi-GPU figure is produced). Re-run with --gpus 1.", file=sys.stderr)
+        return 2
+
+    capi.load()
+    info = capi.device_info(0)
+    try:
+        ncores = len(os.sched_getaffinity(0))
+    except AttributeError:
+        ncores = os.cpu_count()
+    threads = int(os.environ.get("OMP_NUM_THREADS", ncores))
+
+    result = {
+        "metric": METRIC, "value": None, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic: Q,K,V i.i.d. N(0,1) from numpy PCG64(seed 20261125+config), rounded to bf16",
+        "config": {"workload": "BASELINE config 3: bf16 causal prefill B=8 H=16 S_q=S_kv=4096 D=128, scale=1/sqrt(128), "
+                               "f32 accumulate, bf16 out", "step": "one incin_rocm_sdpa_fwd launch"},
+        "device": {"name": info.name.decode(), "arch": info.arch.decode(), "compute_units": info.compute_units,
+                   "clock_khz": info.clock_khz},
+    }
+
+    if args.only in (None, "prefill"):
+        B, H, S, D = 8, 16, 4096, 128
+        w = Workload("prefill_c3", SEED0 + 2, B, H, H, S, S, D, capi.BF16, True)
+        wall, ev_mean, ev_med, ev_min = w.time(args.steps, args.warmup)
+        flops = causal_flops(B, H, S, S, D)
+        result["value"] = flops / (wall * 1e-3) / 1e12
+        result["ms_per_step"] = wall
+        result["roofline"] = {"bound": "mfma", "achieved": flops / (ev_mean * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
+                              "unit": "TFLOP/s", "frac": flops / (ev_mean * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": None,
+                              "kernel": "sdpa_prefill_mfma_kernel<bf16,128>", "algorithmic_flops_per_launch": flops,
+                              "launch_ms_mean": ev_mean, "launch_ms_median": ev_med, "launch_ms_min": ev_min}
+        result["parity_max_abs_err"] = w.parity()
+        w.free()
+        if not args.no_cpu_baseline:
+            slices = 12
+            val, dt = cpu_baseline_prefill(D, S, slices, capi.BF16)
+            result["cpu_baseline"] = {
+                "value": val, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                "sample": "%d of 128 (b,h) slices of config 3 (S=4096, D=128, explicit 0/-inf causal mask), oracle's "
+                          "materialising restatement of the reference CPU op (not the Rust binary): matmuls and "
+                          "reductions on 1 thread, elementwise maps on %d OpenMP threads; %.1f s; same causal FLOP count"
+                          % (slices, threads, dt)}
+
+    if args.only in (None, "decode"):
+        B, H, Skv, D = 32, 32, 8192, 128
+        w = Workload("decode_c4", SEED0 + 3, B, H, H, 1, Skv, D, capi.BF16, False)
+        wall, ev_mean, ev_med, ev_min = w.time(args.steps, args.warmup)
+        kv_bytes = 2.0 * B * H * Skv * D * 2
+        dec = {"workload": "BASELINE config 4: bf16 decode MHA B=32 H=32 S_q=1 KV=8192 D=128, split-KV partials + combine",
+               "metric": "decode KV GB/s", "value": kv_bytes / (wall * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": wall,
+               "num_splits": w.splits,
+               "roofline": {"bound": "hbm", "achieved": kv_bytes / (ev_mean * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                            "frac": kv_bytes / (ev_mean * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None,
+                            "kernel": "sdpa_decode_split_kernel<bf16,128,1,8> + sdpa_combine_kernel",
+                            "algorithmic_bytes_per_launch": kv_bytes,
+                            "launch_ms_mean": ev_mean, "launch_ms_median": ev_med, "launch_ms_min": ev_min},
+               "parity_max_abs_err": w.parity()}
+        w.free()
+        if not args.no_cpu_baseline:
+            val, dt = cpu_baseline_decode(D, Skv, 32, 32, capi.BF16)
+            dec["cpu_baseline"] = {"value": val, "unit": "GB/s", "cores": threads, "kind": "port",
+                                   "sample": "all of config 4 (B=32, H=32, KV=8192, D=128), oracle's materialising restatement of "
+                                             "the reference CPU op (serial matmuls and reductions); %.1f s" % dt}
+        result["decode"] = dec
+
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
