@@ -140,8 +140,10 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["prefill", "decode"], default=None,
-                    help="run a single workload (profiling); the JSON line still has every key")
+    ap.add_argument("--only", choices=["prefill", "decode", "copy"], default=None,
+                    help="run a single workload (profiling). 'copy' runs --steps device-to-device copies of 1 GiB "
+                         "through the library's plain copy kernel: the known-size dispatch that hardware byte "
+                         "counters (FETCH_SIZE / WRITE_SIZE) are calibrated against")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path shards over batch and kv-head groups "
@@ -165,6 +167,18 @@ def main():
         "device": {"name": info.name.decode(), "arch": info.arch.decode(), "compute_units": info.compute_units,
                    "clock_khz": info.clock_khz},
     }
+
+    if args.only == "copy":
+        n = 1 << 30
+        a, b = capi.DeviceBuffer(n), capi.DeviceBuffer(n)
+        capi.check(capi.load().incin_rocm_memset(0, a.ptr, 1, n))
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            capi.check(capi.load().incin_rocm_memcpy_d2d(0, b.ptr, a.ptr, n))
+        dt = (time.perf_counter() - t0) / args.steps
+        print(json.dumps({"metric": "copy16_kernel 1 GiB device-to-device", "bytes_read": n, "bytes_written": n,
+                          "ms_per_copy": dt * 1e3, "GBps_read_plus_write": 2 * n / dt / 1e9}))
+        return 0
 
     if args.only in (None, "prefill"):
         B, H, S, D = 8, 16, 4096, 128

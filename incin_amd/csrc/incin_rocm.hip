@@ -17,6 +17,7 @@ hipError_t launch_sdpa_generic(const SdpaParams& p, int dtype, hipStream_t strea
 hipError_t launch_sdpa_prefill_mfma(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_sdpa_decode(const SdpaParams& p, int dtype, hipStream_t stream);
 int decode_keys_per_tile(int dtype, int D, int R);
+hipError_t launch_copy16(void* dst, const void* src, size_t bytes, hipStream_t stream);
 }  // namespace incin_rocm
 
 using incin_rocm::SdpaParams;
@@ -116,7 +117,9 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     const int64_t R = (d->Hq / d->Hkv) * d->Sq;
     const bool head_ok = d->D == d->Dv && (d->D == 64 || d->D == 128);
     const bool fast_ok = head_ok && !d->add_mask && fast_layout_ok(d, vec) && d->Skv > 0;
-    const bool mfma_ok = fast_ok && d->dtype != INCIN_ROCM_F32 && d->scale > 0.0f && std::isfinite(d->scale);
+    // the MFMA kernel addresses a K/V tile with 32-bit byte offsets from the tile's first row
+    const bool tile_off_ok = d->k_stride[2] >= 0 && d->v_stride[2] >= 0 && d->k_stride[2] < (1 << 24) && d->v_stride[2] < (1 << 24);
+    const bool mfma_ok = fast_ok && tile_off_ok && d->dtype != INCIN_ROCM_F32 && d->scale > 0.0f && std::isfinite(d->scale);
     const bool split_ok = fast_ok && d->Sq <= 64;
 
     int impl = d->impl;
@@ -284,6 +287,15 @@ int incin_rocm_memcpy_d2h(int32_t dev, void* dst, const void* src, size_t bytes)
 }
 int incin_rocm_memcpy_d2d(int32_t dev, void* dst, const void* src, size_t bytes)
 {
+    if (bytes == 0) return 0;
+    if (!dst || !src) return fail(INCIN_ROCM_EINVAL, "memcpy_d2d: null pointer");
+    if (aligned16(dst) && aligned16(src) && bytes % 16 == 0) {
+        // a plain copy kernel on the default stream, then wait: synchronous like the other copies
+        if (int rc = use_device(dev)) return rc;
+        HIP_TRY(incin_rocm::launch_copy16(dst, src, bytes, nullptr), "copy kernel launch");
+        HIP_TRY(hipStreamSynchronize(nullptr), "hipStreamSynchronize");
+        return 0;
+    }
     return copy(dev, dst, src, bytes, hipMemcpyDeviceToDevice, "hipMemcpy(device to device)");
 }
 

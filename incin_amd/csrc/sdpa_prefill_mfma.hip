@@ -22,9 +22,19 @@
 //   O^T += V^T P^T       A = V^T read from the row-major V tile in LDS with the
 //                        transposing LDS read (ds_read_b64_tr_b16).
 //
-// K and V tiles are fetched from global memory into registers one tile ahead
-// and stored to padded LDS rows (K: +16 B, V: +64 B per row, chosen so the two
-// read patterns above are bank-conflict free).
+// Data movement: K and V tiles go from global memory straight into LDS
+// (buffer_load ... lds, 16 bytes per lane, no register staging), one tile ahead
+// of the computation, into two alternating LDS stages; one barrier per tile.
+// Out-of-range rows are zero-filled by the buffer descriptor's bounds check.
+// LDS rows are unpadded; instead the 16-byte chunk c of row r is stored at
+// chunk slot c ^ f(r), with f chosen so that both read patterns (16 lanes x 16
+// bytes down a column of rows for K; 4 rows x 64 bytes for the transposing V
+// read) touch every bank once.
+//
+// The running maximum is only raised when a tile's maximum exceeds it by more
+// than 2^8 (the accumulator and the running sum are rescaled then); otherwise
+// probabilities are computed against the stale maximum, which is exact in
+// exact arithmetic and keeps every intermediate within f32 / storage range.
 #include "sdpa_params.h"
 
 namespace incin_rocm {
@@ -35,7 +45,6 @@ typedef short short8v __attribute__((ext_vector_type(8)));
 typedef bf16_t bf16x8 __attribute__((ext_vector_type(8)));
 typedef f16_t f16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
-typedef unsigned int uint2v __attribute__((ext_vector_type(2)));
 
 template <typename T> struct Mma;
 template <> struct Mma<bf16_t> {
@@ -55,32 +64,50 @@ template <> struct Mma<f16_t> {
 
 constexpr int PF_BM = 128;     // query rows per workgroup
 constexpr int PF_BN = 64;      // keys per tile
-constexpr int PF_WAVES = 4;
+constexpr float PF_RESCALE_THRESHOLD = 8.0f;   // log2 units
 
 template <int D> struct PfLayout {
-    static constexpr int KSTR = D + 8;     // elements per K row in LDS (+16 B)
-    static constexpr int VSTR = D + 32;    // elements per V row in LDS (+64 B)
-    static constexpr int K_ELEMS = PF_BN * KSTR;
-    static constexpr int V_ELEMS = PF_BN * VSTR;
-    static constexpr int LDS_BYTES = (K_ELEMS + V_ELEMS) * 2;
+    static constexpr int ROWB = D * 2;                 // bytes per K/V row in LDS (unpadded)
+    static constexpr int CPR = D / 8;                  // 16-byte chunks per row
+    static constexpr int TILE_BYTES = PF_BN * ROWB;    // one K or V tile
+    static constexpr int STAGE_BYTES = 2 * TILE_BYTES; // K then V
+    static constexpr int LOADS_PER_WAVE = TILE_BYTES / 1024 / 4;   // wavefront-wide 1 KiB loads per tensor per tile
+    // chunk-slot swizzle: depends on the low 4 bits of the row only
+    static __device__ __forceinline__ int f(int r)
+    {
+        if (D == 128) return ((r & 3) << 2) | ((r >> 2) & 3);
+        return (((r >> 1) & 1) << 2) | ((r >> 2) & 3);
+    }
 };
+
+__device__ __forceinline__ float xor32_max(float x)
+{
+    // lanes l and l^32 exchange; both end with the maximum
+    auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+}
+
+__device__ __forceinline__ float xor32_sum(float x)
+{
+    auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+}
 
 template <typename T, int D>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void sdpa_prefill_mfma_kernel(SdpaParams p)
 {
+#if defined(__HIP_DEVICE_COMPILE__)   // the body uses device-only types (buffer descriptors); the host pass needs only the stub
     typedef typename Mma<T>::vec8 vec8;
     typedef PfLayout<D> L;
     constexpr int NSTEP = D / 16;          // k-steps of the S^T product
     constexpr int NDB = D / 32;            // 32-wide blocks of the head dimension
-    constexpr int CHUNKS = PF_BN * D / 8;  // 16-byte chunks per tile
-    constexpr int CPT = CHUNKS / 256;      // chunks per thread
-    constexpr int CPR = D / 8;             // chunks per row
+    constexpr int LPW = L::LOADS_PER_WAVE;
 
-    __shared__ __attribute__((aligned(16))) T Ks[L::K_ELEMS];
-    __shared__ __attribute__((aligned(16))) T Vs[L::V_ELEMS];
+    __shared__ __attribute__((aligned(1024))) char smem[2 * L::STAGE_BYTES];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);     // wavefront-uniform by construction: keep it scalar
     const int ql = lane & 31, g = lane >> 5;
     const int Sq = p.Sq, Skv = p.Skv;
 
@@ -120,6 +147,62 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     }
     const int n_tiles = (j_end + PF_BN - 1) / PF_BN;
 
+    // ---- global -> LDS copy plan ---------------------------------------------------
+    // wavefront-wide load number ii = wave*LPW + c fills LDS bytes [ii*1024, ii*1024 + 1024)
+    // of a tile; lane -> position p = ii*64 + lane -> (row, slot) -> global chunk slot ^ f(row).
+    int k_voff[LPW], v_voff[LPW];
+#pragma unroll
+    for (int c = 0; c < LPW; ++c) {
+        const int pos = (wave * LPW + c) * 64 + lane;
+        const int row = pos / L::CPR, slot = pos % L::CPR;
+        const int chunk = slot ^ L::f(row);
+        k_voff[c] = row * (int)p.k_ss * 2 + chunk * 16;
+        v_voff[c] = row * (int)p.v_ss * 2 + chunk * 16;
+    }
+    const int64_t k_tile_bytes = (int64_t)PF_BN * p.k_ss * 2, v_tile_bytes = (int64_t)PF_BN * p.v_ss * 2;
+    auto issue_tile = [&](int t, int stage) {
+        const int j0 = t * PF_BN;
+        // bytes from the first row of the tile to the end of the last valid row: loads past that return 0
+        int64_t k_rem = (int64_t)(Skv - j0 - 1) * p.k_ss * 2 + D * 2;
+        int64_t v_rem = (int64_t)(Skv - j0 - 1) * p.v_ss * 2 + D * 2;
+        if (k_rem > 0x7fffffffLL) k_rem = 0x7fffffffLL;
+        if (v_rem > 0x7fffffffLL) v_rem = 0x7fffffffLL;
+        __amdgpu_buffer_rsrc_t kr = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)kp + t * k_tile_bytes), 0, (int)k_rem, 0x00020000);
+        __amdgpu_buffer_rsrc_t vr = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)vp + t * v_tile_bytes), 0, (int)v_rem, 0x00020000);
+        char* kdst = smem + stage * L::STAGE_BYTES + wave * LPW * 1024;
+        char* vdst = kdst + L::TILE_BYTES;
+#pragma unroll
+        for (int c = 0; c < LPW; ++c)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, (__attribute__((address_space(3))) void*)(kdst + c * 1024), 16, k_voff[c], 0, 0, 0);
+#pragma unroll
+        for (int c = 0; c < LPW; ++c)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, (__attribute__((address_space(3))) void*)(vdst + c * 1024), 16, v_voff[c], 0, 0, 0);
+    };
+
+    // ---- LDS read addresses (bytes, stage 0) --------------------------------------------
+    // K operand: lane (ql, g) reads row 32*kb + ql, logical chunk 2*s + g
+    int k_addr[NSTEP];
+    {
+        const int F = L::f(ql);
+#pragma unroll
+        for (int s = 0; s < NSTEP; ++s) k_addr[s] = ql * L::ROWB + (((2 * s + g) ^ F) << 4);
+    }
+    // V operand (transposing read): the 16 lanes of a group fetch a 4-key x 16-d patch
+    // (lane n: key n/4, d 4*(n%4)..+3) and receive (d = n, keys 0..3).  Row within a
+    // 16-row block: 8*h + 4*g + n/4; logical chunk 4*db + 2*dh + (n%4)/2.
+    int v_addr[NDB][2];
+    {
+        const int n = lane & 15, dh = (lane >> 4) & 1;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int r = 8 * h + 4 * g + (n >> 2);
+                const int chunk = 4 * db + 2 * dh + ((n & 3) >> 1);
+                v_addr[db][h] = L::TILE_BYTES + r * L::ROWB + ((chunk ^ L::f(r)) << 4) + (n & 1) * 8;
+            }
+    }
+
     // ---- Q^T operand, resident in registers ---------------------------------------
     vec8 qreg[NSTEP];
     {
@@ -134,43 +217,12 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     for (int db = 0; db < NDB; ++db)
 #pragma unroll
         for (int r = 0; r < 16; ++r) o_acc[db][r] = 0.0f;
-    float m_run = -INFINITY;      // running max of the scaled scores, log2 units
+    float m_run = -INFINITY;      // reference maximum of the scaled scores (log2 units); may lag the true maximum
     float l_run = 0.0f;           // this lane's share of the running denominator
     const float c2 = p.scale * 1.4426950408889634f;
 
-    // ---- tile prefetch registers -----------------------------------------------------
-    uint4v kpre[CPT], vpre[CPT];
-    auto fetch = [&](int j0) {
-#pragma unroll
-        for (int c = 0; c < CPT; ++c) {
-            const int chunk = tid + c * 256;
-            const int row = chunk / CPR, col = (chunk % CPR) * 8;
-            const int j = min(j0 + row, Skv - 1);
-            kpre[c] = *(const uint4v*)(kp + (int64_t)j * p.k_ss + col);
-            vpre[c] = *(const uint4v*)(vp + (int64_t)j * p.v_ss + col);
-        }
-    };
-    auto stash = [&]() {
-#pragma unroll
-        for (int c = 0; c < CPT; ++c) {
-            const int chunk = tid + c * 256;
-            const int row = chunk / CPR, col = (chunk % CPR) * 8;
-            *(uint4v*)(Ks + row * L::KSTR + col) = kpre[c];
-            *(uint4v*)(Vs + row * L::VSTR + col) = vpre[c];
-        }
-    };
-
-    if (n_tiles > 0) fetch(0);
-
-    for (int t = 0; t < n_tiles; ++t) {
+    auto compute_tile = [&](int t, const char* stage_base) {
         const int j0 = t * PF_BN;
-        __syncthreads();                       // every wavefront has finished reading the previous tile
-        stash();
-        __syncthreads();
-        if (t + 1 < n_tiles) fetch(j0 + PF_BN);
-
-        if (j0 >= lim_wave_max) continue;      // no query of this wavefront sees this tile (uniform per wavefront)
-
         // ---- S^T = K Q^T ----------------------------------------------------------
         floatx16 s_acc[2];
 #pragma unroll
@@ -181,7 +233,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
         for (int s = 0; s < NSTEP; ++s) {
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
-                const vec8 a = *(const vec8*)(Ks + (kb * 32 + ql) * L::KSTR + s * 16 + g * 8);
+                const vec8 a = *(const vec8*)(stage_base + k_addr[s] + kb * 32 * L::ROWB);
                 s_acc[kb] = Mma<T>::run(a, qreg[s], s_acc[kb]);
             }
         }
@@ -199,17 +251,24 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
                 }
         }
 
-        // ---- online softmax --------------------------------------------------------------
+        // ---- online softmax with lazy rescaling ------------------------------------------
         float tmax = s_acc[0][0];
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, s_acc[kb][r]);
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-        const float m_new = fmaxf(m_run, tmax * c2);
-        const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
-        m_run = m_new;
+        tmax = xor32_max(tmax) * c2;
+        if (__builtin_amdgcn_ballot_w64(tmax > m_run + PF_RESCALE_THRESHOLD) != 0) {
+            const float m_new = fmaxf(m_run, tmax);
+            const float alpha = __builtin_amdgcn_exp2f(m_run - ((m_new == -INFINITY) ? 0.0f : m_new));
+            m_run = m_new;
+            l_run *= alpha;
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) o_acc[db][r] *= alpha;
+        }
+        const float m_use = (m_run == -INFINITY) ? 0.0f : m_run;
         float rsum = 0.0f;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
@@ -219,41 +278,47 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
                 s_acc[kb][r] = e;
                 rsum += e;
             }
-        l_run = fmaf(l_run, alpha, rsum);
-#pragma unroll
-        for (int db = 0; db < NDB; ++db)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) o_acc[db][r] *= alpha;
+        l_run += rsum;
 
         // ---- O^T += V^T P^T ---------------------------------------------------------------
         // k-step ks covers registers 8*(ks%2)..+7 of key block ks/2; element e of
-        // a lane is key 32*(ks/2) + 16*(ks%2) + 8*(e/4) + 4*g + (e%4).
+        // a lane is key 16*ks + 8*(e/4) + 4*g + (e%4).
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
             vec8 pb;
 #pragma unroll
             for (int e = 0; e < 8; ++e) pb[e] = (T)s_acc[ks / 2][8 * (ks % 2) + e];
-            const int kbase = 32 * (ks / 2) + 16 * (ks % 2) + 4 * g;
-            // transposing read: the 16 lanes of a group fetch a 4-key x 16-d patch
-            // (lane n: key n/4, d 4*(n%4)..+3) and receive (d = n, keys 0..3).
-            const int n = lane & 15, dh = (lane >> 4) & 1;
 #pragma unroll
             for (int db = 0; db < NDB; ++db) {
-                const T* base = Vs + (kbase + (n >> 2)) * L::VSTR + db * 32 + dh * 16 + (n & 3) * 4;
                 const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (short4v __attribute__((address_space(3)))*)(base));
+                    (short4v __attribute__((address_space(3)))*)(stage_base + v_addr[db][0] + ks * 16 * L::ROWB));
                 const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (short4v __attribute__((address_space(3)))*)(base + 8 * L::VSTR));
+                    (short4v __attribute__((address_space(3)))*)(stage_base + v_addr[db][1] + ks * 16 * L::ROWB));
                 short8v av;
                 av.lo = lo;
                 av.hi = hi;
                 o_acc[db] = Mma<T>::run(__builtin_bit_cast(vec8, av), pb, o_acc[db]);
             }
         }
+    };
+
+    if (n_tiles > 0) issue_tile(0, 0);
+    for (int t = 0; t < n_tiles; t += 2) {
+        // stage 0
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();       // tile t is in LDS for everyone; everyone has finished tile t-1 (stage 1 is free)
+        if (t + 1 < n_tiles) issue_tile(t + 1, 1);
+        if (t * PF_BN < lim_wave_max) compute_tile(t, smem);
+        if (t + 1 >= n_tiles) break;
+        // stage 1
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (t + 2 < n_tiles) issue_tile(t + 2, 0);
+        if ((t + 1) * PF_BN < lim_wave_max) compute_tile(t + 1, smem + L::STAGE_BYTES);
     }
 
     // ---- normalise and store ------------------------------------------------------------------
-    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+    const float l_tot = xor32_sum(l_run);
     const float inv = (l_tot == 0.0f) ? __builtin_nanf("") : 1.0f / l_tot;   // no visible key: NaN, as the reference
     if (my_i < Sq) {
         T* orow = op + (int64_t)my_i * p.o_ss;
@@ -268,6 +333,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
                 *(vec4*)(orow + db * 32 + r4 * 8 + g * 4) = w;
             }
     }
+#endif
 }
 
 template <typename T, int D>
@@ -280,7 +346,8 @@ static hipError_t launch_prefill_t(const SdpaParams& p, hipStream_t stream)
 }
 
 // Host has validated: dtype f16/bf16, D == Dv in {64,128}, scale > 0, no dense
-// mask, rows 16-byte aligned with unit last-dim stride.
+// mask, rows 16-byte aligned with unit last-dim stride, row strides below 2^24
+// elements (tile offsets fit the 32-bit buffer offset).
 hipError_t launch_sdpa_prefill_mfma(const SdpaParams& p, int dtype, hipStream_t stream)
 {
     if (dtype == 1) return p.D == 128 ? launch_prefill_t<f16_t, 128>(p, stream) : launch_prefill_t<f16_t, 64>(p, stream);
