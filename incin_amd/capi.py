@@ -11,7 +11,8 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libincin_rocm.so")
+# INCIN_ROCM_LIBRARY overrides the in-tree location (e.g. to load an installed or experimental build)
+LIB_PATH = os.environ.get("INCIN_ROCM_LIBRARY") or os.path.join(_HERE, "lib", "libincin_rocm.so")
 
 F32, F16, BF16 = 0, 1, 2
 IMPL_AUTO, IMPL_GENERIC, IMPL_MFMA, IMPL_SPLITKV = 0, 1, 2, 3

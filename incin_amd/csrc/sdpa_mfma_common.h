@@ -1,0 +1,87 @@
+// Shared pieces of the two MFMA attention kernels: operand types, the matrix
+// instruction wrappers, the LDS tile layout (chunk-slot swizzle) and the
+// lane <-> lane^32 exchanges.
+#pragma once
+#include "sdpa_params.h"
+
+namespace incin_rocm {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef short short8v __attribute__((ext_vector_type(8)));
+typedef bf16_t bf16x8 __attribute__((ext_vector_type(8)));
+typedef f16_t f16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
+
+template <typename T> struct Mma;
+template <> struct Mma<bf16_t> {
+    typedef bf16x8 vec8;
+    typedef bf16_t vec2 __attribute__((ext_vector_type(2)));
+    static __device__ __forceinline__ floatx16 run(vec8 a, vec8 b, floatx16 c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+    // acc + x[0] + x[1] (f32 accumulate of the two storage-precision values)
+    static __device__ __forceinline__ float add2(vec2 x, float acc)
+    {
+        const vec2 ones = {(bf16_t)1.0f, (bf16_t)1.0f};
+        return __builtin_amdgcn_fdot2_f32_bf16(x, ones, acc, false);
+    }
+};
+template <> struct Mma<f16_t> {
+    typedef f16x8 vec8;
+    typedef f16_t vec2 __attribute__((ext_vector_type(2)));
+    static __device__ __forceinline__ floatx16 run(vec8 a, vec8 b, floatx16 c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float add2(vec2 x, float acc)
+    {
+        const vec2 ones = {(f16_t)1.0f, (f16_t)1.0f};
+        return __builtin_amdgcn_fdot2(x, ones, acc, false);
+    }
+};
+
+constexpr int PF_BM = 128;     // query rows per workgroup
+constexpr int PF_BN = 64;      // keys per tile
+constexpr float PF_RESCALE_THRESHOLD = 8.0f;   // log2 units
+
+template <int D> struct PfLayout {
+    static constexpr int ROWB = D * 2;                 // bytes per K/V row in LDS (unpadded)
+    static constexpr int CPR = D / 8;                  // 16-byte chunks per row
+    static constexpr int TILE_BYTES = PF_BN * ROWB;    // one K or V tile
+    static constexpr int STAGE_BYTES = 2 * TILE_BYTES; // K then V
+    static constexpr int LOADS_PER_WAVE = TILE_BYTES / 1024 / 4;   // wavefront-wide 1 KiB loads per tensor per tile
+    // Chunk-slot swizzles (functions of the low 4 bits of the row).
+    // K tile: read by 16 lanes x 16 bytes down 16 consecutive rows at one logical chunk, so fk must
+    // take 16 distinct values over 16 consecutive rows (D = 64: 8 distinct over rows of one parity,
+    // because two 128-byte rows already split the banks).
+    static __device__ __forceinline__ int fk(int r)
+    {
+        if (D == 128) return ((r & 3) << 2) | ((r >> 2) & 3);
+        return (((r >> 1) & 1) << 2) | ((r >> 2) & 3);
+    }
+    // V tile: the transposing read takes 4 consecutive rows x 64 bytes per half-wavefront, so fv only
+    // has to move those 4 rows to 4 different 64-byte column groups; keeping it a function of row
+    // bits 0-1 (D = 64: bit 1) makes the read address base ^ (d_block << 6) + immediate.
+    static __device__ __forceinline__ int fv(int r)
+    {
+        if (D == 128) return (r & 3) << 2;
+        return ((r >> 1) & 1) << 2;
+    }
+};
+
+__device__ __forceinline__ float xor32_max(float x)
+{
+    // lanes l and l^32 exchange; both end with the maximum
+    auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+}
+
+__device__ __forceinline__ float xor32_sum(float x)
+{
+    auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+}
+
+}  // namespace incin_rocm

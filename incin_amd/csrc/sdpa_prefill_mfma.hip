@@ -27,7 +27,7 @@
 // of the computation, into two alternating LDS stages; one barrier per tile.
 // Out-of-range rows are zero-filled by the buffer descriptor's bounds check.
 // LDS rows are unpadded; instead the 16-byte chunk c of row r is stored at
-// chunk slot c ^ f(r), with f chosen so that both read patterns (16 lanes x 16
+// chunk slot c ^ f(r), with f chosen per tile so that both read patterns (16 lanes x 16
 // bytes down a column of rows for K; 4 rows x 64 bytes for the transposing V
 // read) touch every bank once.
 //
@@ -35,63 +35,9 @@
 // than 2^8 (the accumulator and the running sum are rescaled then); otherwise
 // probabilities are computed against the stale maximum, which is exact in
 // exact arithmetic and keeps every intermediate within f32 / storage range.
-#include "sdpa_params.h"
+#include "sdpa_mfma_common.h"
 
 namespace incin_rocm {
-
-typedef float floatx16 __attribute__((ext_vector_type(16)));
-typedef short short4v __attribute__((ext_vector_type(4)));
-typedef short short8v __attribute__((ext_vector_type(8)));
-typedef bf16_t bf16x8 __attribute__((ext_vector_type(8)));
-typedef f16_t f16x8 __attribute__((ext_vector_type(8)));
-typedef unsigned int uint4v __attribute__((ext_vector_type(4)));
-
-template <typename T> struct Mma;
-template <> struct Mma<bf16_t> {
-    typedef bf16x8 vec8;
-    static __device__ __forceinline__ floatx16 run(vec8 a, vec8 b, floatx16 c)
-    {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-    }
-};
-template <> struct Mma<f16_t> {
-    typedef f16x8 vec8;
-    static __device__ __forceinline__ floatx16 run(vec8 a, vec8 b, floatx16 c)
-    {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-    }
-};
-
-constexpr int PF_BM = 128;     // query rows per workgroup
-constexpr int PF_BN = 64;      // keys per tile
-constexpr float PF_RESCALE_THRESHOLD = 8.0f;   // log2 units
-
-template <int D> struct PfLayout {
-    static constexpr int ROWB = D * 2;                 // bytes per K/V row in LDS (unpadded)
-    static constexpr int CPR = D / 8;                  // 16-byte chunks per row
-    static constexpr int TILE_BYTES = PF_BN * ROWB;    // one K or V tile
-    static constexpr int STAGE_BYTES = 2 * TILE_BYTES; // K then V
-    static constexpr int LOADS_PER_WAVE = TILE_BYTES / 1024 / 4;   // wavefront-wide 1 KiB loads per tensor per tile
-    // chunk-slot swizzle: depends on the low 4 bits of the row only
-    static __device__ __forceinline__ int f(int r)
-    {
-        if (D == 128) return ((r & 3) << 2) | ((r >> 2) & 3);
-        return (((r >> 1) & 1) << 2) | ((r >> 2) & 3);
-    }
-};
-
-__device__ __forceinline__ float xor32_max(float x)
-{
-    // lanes l and l^32 exchange; both end with the maximum
-    auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-    return fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
-}
-
-__device__ __forceinline__ float xor32_sum(float x)
-{
-    auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-    return __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
-}
 
 template <typename T, int D>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
@@ -155,9 +101,8 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     for (int c = 0; c < LPW; ++c) {
         const int pos = (wave * LPW + c) * 64 + lane;
         const int row = pos / L::CPR, slot = pos % L::CPR;
-        const int chunk = slot ^ L::f(row);
-        k_voff[c] = row * (int)p.k_ss * 2 + chunk * 16;
-        v_voff[c] = row * (int)p.v_ss * 2 + chunk * 16;
+        k_voff[c] = row * (int)p.k_ss * 2 + (slot ^ L::fk(row)) * 16;
+        v_voff[c] = row * (int)p.v_ss * 2 + (slot ^ L::fv(row)) * 16;
     }
     const int64_t k_tile_bytes = (int64_t)PF_BN * p.k_ss * 2, v_tile_bytes = (int64_t)PF_BN * p.v_ss * 2;
     auto issue_tile = [&](int t, int stage) {
@@ -183,7 +128,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     // K operand: lane (ql, g) reads row 32*kb + ql, logical chunk 2*s + g
     int k_addr[NSTEP];
     {
-        const int F = L::f(ql);
+        const int F = L::fk(ql);
 #pragma unroll
         for (int s = 0; s < NSTEP; ++s) k_addr[s] = ql * L::ROWB + (((2 * s + g) ^ F) << 4);
     }
@@ -199,7 +144,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
             for (int h = 0; h < 2; ++h) {
                 const int r = 8 * h + 4 * g + (n >> 2);
                 const int chunk = 4 * db + 2 * dh + ((n & 3) >> 1);
-                v_addr[db][h] = L::TILE_BYTES + r * L::ROWB + ((chunk ^ L::f(r)) << 4) + (n & 1) * 8;
+                v_addr[db][h] = L::TILE_BYTES + r * L::ROWB + ((chunk ^ L::fv(r)) << 4) + (n & 1) * 8;
             }
     }
 
@@ -269,25 +214,29 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
                 for (int r = 0; r < 16; ++r) o_acc[db][r] *= alpha;
         }
         const float m_use = (m_run == -INFINITY) ? 0.0f : m_run;
+        // P^T in storage precision; element e of k-step ks is register 8*(ks%2)+e of key block ks/2,
+        // i.e. key 16*ks + 8*(e/4) + 4*g + (e%4)
+        vec8 pb[4];
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                pb[ks][e] = (T)__builtin_amdgcn_exp2f(fmaf(s_acc[ks / 2][8 * (ks % 2) + e], c2, -m_use));
+        // denominator from the rounded probabilities (the same values the numerator uses),
+        // two per instruction (v_dot2 with a vector of ones, f32 accumulate)
         float rsum = 0.0f;
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+        for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float e = __builtin_amdgcn_exp2f(fmaf(s_acc[kb][r], c2, -m_use));
-                s_acc[kb][r] = e;
-                rsum += e;
+            for (int e = 0; e < 8; e += 2) {
+                typename Mma<T>::vec2 pr = {pb[ks][e], pb[ks][e + 1]};
+                rsum = Mma<T>::add2(pr, rsum);
             }
         l_run += rsum;
 
         // ---- O^T += V^T P^T ---------------------------------------------------------------
-        // k-step ks covers registers 8*(ks%2)..+7 of key block ks/2; element e of
-        // a lane is key 16*ks + 8*(e/4) + 4*g + (e%4).
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
-            vec8 pb;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) pb[e] = (T)s_acc[ks / 2][8 * (ks % 2) + e];
 #pragma unroll
             for (int db = 0; db < NDB; ++db) {
                 const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
@@ -297,7 +246,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
                 short8v av;
                 av.lo = lo;
                 av.hi = hi;
-                o_acc[db] = Mma<T>::run(__builtin_bit_cast(vec8, av), pb, o_acc[db]);
+                o_acc[db] = Mma<T>::run(__builtin_bit_cast(vec8, av), pb[ks], o_acc[db]);
             }
         }
     };

@@ -172,6 +172,10 @@ def test_reference_golden_vectors_on_gpu(gpu):
 
 # ---- MFMA prefill kernel --------------------------------------------------------------------
 
+MFMA_IMPLS = [capi.IMPL_MFMA]
+
+
+@pytest.mark.parametrize("impl", MFMA_IMPLS)
 @pytest.mark.parametrize("dtype", [capi.BF16, capi.F16])
 @pytest.mark.parametrize("shape", [
     # B, Hq, Hkv, Sq, Skv, D
@@ -182,29 +186,32 @@ def test_reference_golden_vectors_on_gpu(gpu):
     (1, 4, 1, 100, 1000, 64),
     (1, 2, 2, 384, 129, 64),
     (1, 1, 1, 17, 64, 128),
+    (1, 2, 1, 1000, 1000, 128),
+    (1, 1, 1, 300, 40, 64),
 ])
-def test_mfma_prefill(gpu, dtype, shape):
+def test_mfma_prefill(gpu, dtype, shape, impl):
     B, Hq, Hkv, Sq, Skv, D = shape
     q, k, v = inputs(200 + sum(shape), B, Hq, Hkv, Sq, Skv, D, D, dtype)
     for causal in (False, True):
-        got, info = host.sdpa(q, k, v, dtype, causal=causal, impl=capi.IMPL_MFMA, return_info=True)
-        assert info["impl"] == capi.IMPL_MFMA
+        got, info = host.sdpa(q, k, v, dtype, causal=causal, impl=impl, return_info=True)
+        assert info["impl"] == impl
         ref = oracle_full(q, k, v, G=Hq // Hkv, causal=causal)
         check(got, ref, TOL[dtype], "mfma %s %r causal=%d" % (dtypes.NAMES[dtype], shape, causal))
         gen = host.sdpa(q, k, v, dtype, causal=causal, impl=capi.IMPL_GENERIC)
         check(got, gen, TOL[dtype], "mfma vs generic kernel %r causal=%d" % (shape, causal))
 
 
-def test_mfma_prefill_ragged_lengths(gpu):
+@pytest.mark.parametrize("impl", MFMA_IMPLS)
+def test_mfma_prefill_ragged_lengths(gpu, impl):
     B, Hq, Hkv, S, D = 3, 8, 2, 640, 128
     q, k, v = inputs(31, B, Hq, Hkv, S, S, D, D, capi.BF16)
     lens = np.array([640, 129, 0], np.int32)
-    got = host.sdpa(q, k, v, capi.BF16, causal=True, kv_lens=lens, impl=capi.IMPL_MFMA)
+    got = host.sdpa(q, k, v, capi.BF16, causal=True, kv_lens=lens, impl=impl)
     ref = oracle_full(q, k, v, G=4, causal=True, kv_lens=lens)
     check(got, ref, 2e-2, "mfma bf16 GQA causal + kv_lens")
     # padded keys == truncated keys
-    trunc = host.sdpa(q[1:2, :, :, :], k[1:2, :, :129], v[1:2, :, :129], capi.BF16, impl=capi.IMPL_MFMA)
-    padded = host.sdpa(q[1:2], k[1:2], v[1:2], capi.BF16, kv_lens=lens[1:2], impl=capi.IMPL_MFMA)
+    trunc = host.sdpa(q[1:2, :, :, :], k[1:2, :, :129], v[1:2, :, :129], capi.BF16, impl=impl)
+    padded = host.sdpa(q[1:2], k[1:2], v[1:2], capi.BF16, kv_lens=lens[1:2], impl=impl)
     check(padded, trunc, 1e-6, "mfma padded == truncated")
 
 
