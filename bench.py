@@ -29,6 +29,10 @@ from incin_amd import capi, dtypes, host  # noqa: E402
 SEED0 = 20261125
 PEAK_BF16_TFLOPS = 2516.6   # 256 CUs x 2.4 GHz x 4096 dense bf16 FLOP/clk/CU (vendor: 2.5 PFLOP/s)
 PEAK_HBM_GBS = 8000.0       # HBM3E, vendor figure
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same command (KiB per dispatch,
+# FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0 after calibration against the 1 GiB copy kernel): profiles/*.txt
+PREFILL_TRAFFIC_BYTES = (197934 * 2.0 + 131073) * 1024     # 5.40e8: |Q|+|K|+|V| read once, |O| written once
+DECODE_TRAFFIC_BYTES = (2097470 * 2.0 + 1088 + 256) * 1024  # 4.297e9: K and V read once + split partials
 METRIC = "attn fwd TFLOP/s + % bf16 MFMA peak; decode KV GB/s + % HBM peak (1 GPU)"
 
 
@@ -68,8 +72,18 @@ class Workload:
     def launch(self):
         capi.sdpa_fwd(self.desc)
 
+    def ramp(self, seconds=0.15):
+        """Setup, not measurement: keep the GPU busy until its clocks have settled (the first ~30 launches
+        after idle run up to 40% slower), so that the W warm-up steps and the K timed steps see steady state."""
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(10):
+                self.launch()
+            capi.sync()
+
     def time(self, steps, warmup):
         """(wall ms per step over `steps` back-to-back launches, mean / median / min event ms per launch)"""
+        self.ramp()
         for _ in range(warmup):
             self.launch()
         capi.sync()
@@ -188,7 +202,7 @@ def main():
         result["value"] = flops / (wall * 1e-3) / 1e12
         result["ms_per_step"] = wall
         result["roofline"] = {"bound": "mfma", "achieved": flops / (ev_mean * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
-                              "unit": "TFLOP/s", "frac": flops / (ev_mean * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": None,
+                              "unit": "TFLOP/s", "frac": flops / (ev_mean * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": PREFILL_TRAFFIC_BYTES,
                               "kernel": "sdpa_prefill_mfma_kernel<bf16,128>", "algorithmic_flops_per_launch": flops,
                               "launch_ms_mean": ev_mean, "launch_ms_median": ev_med, "launch_ms_min": ev_min}
         result["parity_max_abs_err"] = w.parity()
@@ -212,7 +226,7 @@ def main():
                "metric": "decode KV GB/s", "value": kv_bytes / (wall * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": wall,
                "num_splits": w.splits,
                "roofline": {"bound": "hbm", "achieved": kv_bytes / (ev_mean * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                            "frac": kv_bytes / (ev_mean * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None,
+                            "frac": kv_bytes / (ev_mean * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": DECODE_TRAFFIC_BYTES,
                             "kernel": "sdpa_decode_split_kernel<bf16,128,1,8> + sdpa_combine_kernel",
                             "algorithmic_bytes_per_launch": kv_bytes,
                             "launch_ms_mean": ev_mean, "launch_ms_median": ev_med, "launch_ms_min": ev_min},
