@@ -8,36 +8,49 @@
 // Shape of the computation (one workgroup = 4 wavefronts = 128 query rows, one
 // wavefront = 32 query rows, key tile = 64 keys):
 //
-//   S^T = K_tile Q^T     v_mfma_f32_32x32x16: A = K rows from LDS (16-byte reads),
-//                        B = Q^T held in registers for the whole kernel.
-//                        In the 32x32 result a lane owns ONE query (column
-//                        lane%32) and 16 keys per 32-key block, so the row max
-//                        and row sum of the softmax are in-lane reductions plus
-//                        a single exchange with lane^32.
-//   P^T                  exp2 of the scaled scores, rounded to the storage type
-//                        in registers; the accumulator layout of S^T is already
-//                        the B-operand layout of the next product (the key
-//                        order inside a k-step is a fixed permutation, which
-//                        the V reads below follow).
+//   S^T = K_tile Q'^T    v_mfma_f32_32x32x16: A = K rows from LDS (16-byte reads),
+//                        B = Q^T held in registers for the whole kernel, already
+//                        multiplied by scale*log2(e).  In the 32x32 result a lane
+//                        owns ONE query (column lane%32) and 16 keys per 32-key
+//                        block, so the row max and row sum of the softmax are
+//                        in-lane reductions plus one exchange with lane^32.  The
+//                        accumulator starts from -m_ref (the lane's reference
+//                        maximum) instead of 0, so the product already is s - m.
+//   P^T                  a bare exp2 of that, rounded to the storage type in
+//                        registers; the accumulator layout of S^T is already the
+//                        B-operand layout of the next product (the key order inside
+//                        a k-step is a fixed permutation, which the V reads follow).
 //   O^T += V^T P^T       A = V^T read from the row-major V tile in LDS with the
 //                        transposing LDS read (ds_read_b64_tr_b16).
 //
 // Data movement: K and V tiles go from global memory straight into LDS
-// (buffer_load ... lds, 16 bytes per lane, no register staging), one tile ahead
-// of the computation, into two alternating LDS stages; one barrier per tile.
-// Out-of-range rows are zero-filled by the buffer descriptor's bounds check.
-// LDS rows are unpadded; instead the 16-byte chunk c of row r is stored at
-// chunk slot c ^ f(r), with f chosen per tile so that both read patterns (16 lanes x 16
-// bytes down a column of rows for K; 4 rows x 64 bytes for the transposing V
-// read) touch every bank once.
+// (buffer_load ... lds, 16 bytes per lane, no register staging) into two
+// alternating buffers each; out-of-range rows are zero-filled by the buffer
+// descriptor's bounds check.  LDS rows are unpadded; the 16-byte chunk c of row r
+// is stored at chunk slot c ^ f(r), with f chosen per tile kind so that both read
+// patterns (16 lanes x 16 bytes down a column of rows for K; 4 rows x 64 bytes
+// for the transposing V read) touch every bank once.
 //
-// The running maximum is only raised when a tile's maximum exceeds it by more
-// than 2^8 (the accumulator and the running sum are rescaled then); otherwise
-// probabilities are computed against the stale maximum, which is exact in
-// exact arithmetic and keeps every intermediate within f32 / storage range.
+// Latency: with two wavefronts per SIMD the kernel is bound by LDS read latency
+// unless many operand reads are in flight, so matrix operands are fetched far
+// ahead of the MFMAs that use them: K operands four k-steps (8 MFMAs) ahead, V
+// operands 8 MFMAs ahead.  The one barrier per tile sits between the S^T product
+// and the softmax of the same tile; right after it the wavefront starts the
+// global loads of K(t+2) and V(t+1), the V(t) operand reads (their latency hides
+// under the softmax arithmetic) and, during O^T += V^T P^T, the first K(t+1)
+// operand reads for the next tile.
+//
+// The reference maximum is set from the first tile that holds a visible key and
+// afterwards only raised when a tile's maximum exceeds it by more than 2^8 (the
+// accumulator and the running sum are rescaled then); otherwise probabilities
+// are taken against the stale maximum, which is exact in exact arithmetic and
+// keeps every intermediate within f32 / storage range.
+#include <type_traits>
+
 #include "sdpa_mfma_common.h"
 
 namespace incin_rocm {
+
 
 template <typename T, int D>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
@@ -50,7 +63,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     constexpr int NDB = D / 32;            // 32-wide blocks of the head dimension
     constexpr int LPW = L::LOADS_PER_WAVE;
 
-    __shared__ __attribute__((aligned(1024))) char smem[2 * L::STAGE_BYTES];
+    __shared__ __attribute__((aligned(1024))) char smem[4 * L::TILE_BYTES];   // K buffers 0, 1, V buffers 0, 1
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);     // wavefront-uniform by construction: keep it scalar
@@ -105,26 +118,27 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
         v_voff[c] = row * (int)p.v_ss * 2 + (slot ^ L::fv(row)) * 16;
     }
     const int64_t k_tile_bytes = (int64_t)PF_BN * p.k_ss * 2, v_tile_bytes = (int64_t)PF_BN * p.v_ss * 2;
-    auto issue_tile = [&](int t, int stage) {
-        const int j0 = t * PF_BN;
-        // bytes from the first row of the tile to the end of the last valid row: loads past that return 0
-        int64_t k_rem = (int64_t)(Skv - j0 - 1) * p.k_ss * 2 + D * 2;
-        int64_t v_rem = (int64_t)(Skv - j0 - 1) * p.v_ss * 2 + D * 2;
-        if (k_rem > 0x7fffffffLL) k_rem = 0x7fffffffLL;
-        if (v_rem > 0x7fffffffLL) v_rem = 0x7fffffffLL;
-        __amdgpu_buffer_rsrc_t kr = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)kp + t * k_tile_bytes), 0, (int)k_rem, 0x00020000);
-        __amdgpu_buffer_rsrc_t vr = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)vp + t * v_tile_bytes), 0, (int)v_rem, 0x00020000);
-        char* kdst = smem + stage * L::STAGE_BYTES + wave * LPW * 1024;
-        char* vdst = kdst + L::TILE_BYTES;
+    // K buffer b at smem + b*TILE, V buffer b at smem + (2+b)*TILE
+    auto issue_k = [&](int t, int buf) __attribute__((always_inline)) {
+        int64_t rem = (int64_t)(Skv - t * PF_BN - 1) * p.k_ss * 2 + D * 2;   // bytes to the end of the last valid row: loads past that return 0
+        if (rem > 0x7fffffffLL) rem = 0x7fffffffLL;
+        __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)kp + t * k_tile_bytes), 0, (int)rem, 0x00020000);
+        char* dst = smem + buf * L::TILE_BYTES + wave * LPW * 1024;
 #pragma unroll
         for (int c = 0; c < LPW; ++c)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, (__attribute__((address_space(3))) void*)(kdst + c * 1024), 16, k_voff[c], 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)(dst + c * 1024), 16, k_voff[c], 0, 0, 0);
+    };
+    auto issue_v = [&](int t, int buf) __attribute__((always_inline)) {
+        int64_t rem = (int64_t)(Skv - t * PF_BN - 1) * p.v_ss * 2 + D * 2;
+        if (rem > 0x7fffffffLL) rem = 0x7fffffffLL;
+        __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)vp + t * v_tile_bytes), 0, (int)rem, 0x00020000);
+        char* dst = smem + (2 + buf) * L::TILE_BYTES + wave * LPW * 1024;
 #pragma unroll
         for (int c = 0; c < LPW; ++c)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, (__attribute__((address_space(3))) void*)(vdst + c * 1024), 16, v_voff[c], 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)(dst + c * 1024), 16, v_voff[c], 0, 0, 0);
     };
 
-    // ---- LDS read addresses (bytes, stage 0) --------------------------------------------
+    // ---- LDS read addresses (bytes inside a tile buffer) ------------------------------------
     // K operand: lane (ql, g) reads row 32*kb + ql, logical chunk 2*s + g
     int k_addr[NSTEP];
     {
@@ -144,7 +158,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
             for (int h = 0; h < 2; ++h) {
                 const int r = 8 * h + 4 * g + (n >> 2);
                 const int chunk = 4 * db + 2 * dh + ((n & 3) >> 1);
-                v_addr[db][h] = L::TILE_BYTES + r * L::ROWB + ((chunk ^ L::fv(r)) << 4) + (n & 1) * 8;
+                v_addr[db][h] = r * L::ROWB + ((chunk ^ L::fv(r)) << 4) + (n & 1) * 8;
             }
     }
 
@@ -156,114 +170,170 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
 #pragma unroll
         for (int s = 0; s < NSTEP; ++s) qreg[s] = *(const vec8*)(qrow + s * 16);
     }
+    // Fold scale * log2(e) into Q once (rounded back to the storage type): the matrix product then
+    // yields the scores directly in the log2 units the softmax works in.
+    const float c2 = p.scale * 1.4426950408889634f;
+#pragma unroll
+    for (int s = 0; s < NSTEP; ++s)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qreg[s][e] = (T)((float)qreg[s][e] * c2);
 
     floatx16 o_acc[NDB];
 #pragma unroll
     for (int db = 0; db < NDB; ++db)
 #pragma unroll
         for (int r = 0; r < 16; ++r) o_acc[db][r] = 0.0f;
-    float m_run = -INFINITY;      // reference maximum of the scaled scores (log2 units); may lag the true maximum
+    // Reference maximum m_ref (log2 units) of this lane's query.  It is baked into the matrix product:
+    // the first MFMA of every score block starts from the accumulator neg_ref = -m_ref instead of 0, so
+    // the product delivers s - m_ref and the probabilities are a bare exp2 of it.  m_ref is set from the
+    // first tile that holds a visible key and afterwards only raised, when a tile maximum exceeds it by
+    // more than 2^8 (lazy rescaling: exact in exact arithmetic, probabilities stay <= 2^8).
+    float m_ref = 0.0f;
+    bool inited = false;
+    floatx16 neg_ref;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) neg_ref[r] = 0.0f;
     float l_run = 0.0f;           // this lane's share of the running denominator
-    const float c2 = p.scale * 1.4426950408889634f;
 
-    auto compute_tile = [&](int t, const char* stage_base) {
+    // ---- matrix operands in flight ---------------------------------------------------------------
+    constexpr int KD = NSTEP < 4 ? NSTEP : 4;      // K operands are fetched KD k-steps ahead
+    constexpr int NPV = 4 * NDB;                   // MFMAs of one O^T update (4 k-steps of 16 keys x NDB blocks)
+    constexpr int VD = 8;                          // V operands are fetched VD MFMAs ahead
+    vec8 kbuf[KD][2];
+    vec8 vbuf[VD];
+    auto read_k = [&](const char* kb, int s) __attribute__((always_inline)) {
+#pragma unroll
+        for (int b2 = 0; b2 < 2; ++b2) kbuf[s % KD][b2] = *(const vec8*)(kb + k_addr[s] + b2 * 32 * L::ROWB);
+    };
+    auto read_v = [&](const char* vb, int i) __attribute__((always_inline)) {      // i = ks * NDB + db
+        const int ks = i / NDB, db = i % NDB;
+        short8v av;
+        av.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (short4v __attribute__((address_space(3)))*)(vb + v_addr[db][0] + ks * 16 * L::ROWB));
+        av.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (short4v __attribute__((address_space(3)))*)(vb + v_addr[db][1] + ks * 16 * L::ROWB));
+        vbuf[i % VD] = __builtin_bit_cast(vec8, av);
+    };
+
+    // One tile.  On entry kbuf holds the K(t) operands of k-steps 0..KD-1.  `par` = t % 2.
+    auto tile = [&](int t, auto PAR_) __attribute__((always_inline)) {
+        constexpr int par = decltype(PAR_)::value;
+        const char* k_cur = smem + par * L::TILE_BYTES;              // K(t)
+        const char* k_nxt = smem + (1 - par) * L::TILE_BYTES;        // K(t+1)
+        const char* v_cur = smem + (2 + par) * L::TILE_BYTES;        // V(t)
         const int j0 = t * PF_BN;
-        // ---- S^T = K Q^T ----------------------------------------------------------
+        const bool active = j0 < lim_wave_max;                       // some query of this wavefront sees this tile
         floatx16 s_acc[2];
+        vec8 pb[4];
+        // ---- S^T = K Q'^T - m_ref ------------------------------------------------------------
+        if (active) {
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+            for (int s = 0; s < NSTEP; ++s) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) s_acc[kb][r] = 0.0f;
-#pragma unroll
-        for (int s = 0; s < NSTEP; ++s) {
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                const vec8 a = *(const vec8*)(stage_base + k_addr[s] + kb * 32 * L::ROWB);
-                s_acc[kb] = Mma<T>::run(a, qreg[s], s_acc[kb]);
+                for (int b2 = 0; b2 < 2; ++b2)
+                    s_acc[b2] = Mma<T>::run(kbuf[s % KD][b2], qreg[s], s == 0 ? neg_ref : s_acc[b2]);
+                if (s + KD < NSTEP) read_k(k_cur, s + KD);
             }
         }
+        // ---- the tile's barrier: K(t+1) and V(t) are in LDS for everyone, everyone is past
+        //      S^T(t) (K buffer `par` is free) and past O^T(t-1) (V buffer `1-par` is free) ----
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (t + 2 < n_tiles) issue_k(t + 2, par);
+        if (t + 1 < n_tiles) issue_v(t + 1, 1 - par);
+        if (active) {
+#pragma unroll
+            for (int i = 0; i < VD; ++i) read_v(v_cur, i);            // latency hides under the softmax arithmetic
+            __builtin_amdgcn_sched_barrier(0);
 
-        // ---- masking (only tiles that cross a limit) --------------------------------
-        // register r of block kb is key j0 + 32*kb + 8*(r/4) + 4*g + (r%4)
-        if (j0 + PF_BN > lim_wave_min) {
-            const int rel = lim_lane - (j0 + 4 * g);
+            // ---- masking (only tiles that cross a limit) --------------------------------
+            // register r of block kb is key j0 + 32*kb + 8*(r/4) + 4*g + (r%4)
+            if (j0 + PF_BN > lim_wave_min) {
+                const int rel = lim_lane - (j0 + 4 * g);
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int kofs = 32 * kb + 8 * (r / 4) + (r % 4);
+                        if (kofs >= rel) s_acc[kb][r] = -INFINITY;
+                    }
+            }
+
+            // ---- online softmax with lazy rescaling ------------------------------------------
+            float tmax = s_acc[0][0];
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int kofs = 32 * kb + 8 * (r / 4) + (r % 4);
-                    if (kofs >= rel) s_acc[kb][r] = -INFINITY;
-                }
-        }
-
-        // ---- online softmax with lazy rescaling ------------------------------------------
-        float tmax = s_acc[0][0];
+                for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, s_acc[kb][r]);
+            tmax = xor32_max(tmax);                       // this tile's maximum relative to m_ref
+            const bool need = inited ? (tmax > PF_RESCALE_THRESHOLD) : (tmax > -INFINITY);
+            if (__builtin_amdgcn_ballot_w64(need) != 0) {
+                // move the reference to this tile's maximum (lanes that do not need it move by 0)
+                const float delta = need ? tmax : 0.0f;
+                const float alpha = inited ? __builtin_amdgcn_exp2f(-delta) : 1.0f;   // nothing accumulated yet: nothing to rescale
+                m_ref += delta;
+                inited = inited || need;
+                l_run *= alpha;
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+                for (int db = 0; db < NDB; ++db)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, s_acc[kb][r]);
-        tmax = xor32_max(tmax) * c2;
-        if (__builtin_amdgcn_ballot_w64(tmax > m_run + PF_RESCALE_THRESHOLD) != 0) {
-            const float m_new = fmaxf(m_run, tmax);
-            const float alpha = __builtin_amdgcn_exp2f(m_run - ((m_new == -INFINITY) ? 0.0f : m_new));
-            m_run = m_new;
-            l_run *= alpha;
+                    for (int r = 0; r < 16; ++r) o_acc[db][r] *= alpha;
 #pragma unroll
-            for (int db = 0; db < NDB; ++db)
+                for (int r = 0; r < 16; ++r) neg_ref[r] = -m_ref;
 #pragma unroll
-                for (int r = 0; r < 16; ++r) o_acc[db][r] *= alpha;
-        }
-        const float m_use = (m_run == -INFINITY) ? 0.0f : m_run;
-        // P^T in storage precision; element e of k-step ks is register 8*(ks%2)+e of key block ks/2,
-        // i.e. key 16*ks + 8*(e/4) + 4*g + (e%4)
-        vec8 pb[4];
+                for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-                pb[ks][e] = (T)__builtin_amdgcn_exp2f(fmaf(s_acc[ks / 2][8 * (ks % 2) + e], c2, -m_use));
-        // denominator from the rounded probabilities (the same values the numerator uses),
-        // two per instruction (v_dot2 with a vector of ones, f32 accumulate)
-        float rsum = 0.0f;
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-            for (int e = 0; e < 8; e += 2) {
-                typename Mma<T>::vec2 pr = {pb[ks][e], pb[ks][e + 1]};
-                rsum = Mma<T>::add2(pr, rsum);
+                    for (int r = 0; r < 16; ++r) s_acc[kb][r] -= delta;
             }
-        l_run += rsum;
+            // P^T in storage precision; element e of k-step ks is register 8*(ks%2)+e of key block ks/2,
+            // i.e. key 16*ks + 8*(e/4) + 4*g + (e%4)
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    pb[ks][e] = (T)__builtin_amdgcn_exp2f(s_acc[ks / 2][8 * (ks % 2) + e]);
+            // denominator from the rounded probabilities (the same values the numerator uses),
+            // two per instruction (v_dot2 with a vector of ones, f32 accumulate)
+            float rsum = 0.0f;
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+                for (int e = 0; e < 8; e += 2) {
+                    typename Mma<T>::vec2 pr = {pb[ks][e], pb[ks][e + 1]};
+                    rsum = Mma<T>::add2(pr, rsum);
+                }
+            l_run += rsum;
+            __builtin_amdgcn_sched_barrier(0);
 
-        // ---- O^T += V^T P^T ---------------------------------------------------------------
+            // ---- O^T += V^T P^T; the next tile's first K operands are fetched underneath --------
+            const bool next_active = (t + 1 < n_tiles) && (j0 + PF_BN < lim_wave_max);
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
+            for (int i = 0; i < NPV; ++i) {
+                o_acc[i % NDB] = Mma<T>::run(vbuf[i % VD], pb[i / NDB], o_acc[i % NDB]);
+                if (i + VD < NPV) read_v(v_cur, i + VD);
+                if (i == 1 && next_active) {
 #pragma unroll
-            for (int db = 0; db < NDB; ++db) {
-                const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (short4v __attribute__((address_space(3)))*)(stage_base + v_addr[db][0] + ks * 16 * L::ROWB));
-                const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (short4v __attribute__((address_space(3)))*)(stage_base + v_addr[db][1] + ks * 16 * L::ROWB));
-                short8v av;
-                av.lo = lo;
-                av.hi = hi;
-                o_acc[db] = Mma<T>::run(__builtin_bit_cast(vec8, av), pb[ks], o_acc[db]);
+                    for (int s = 0; s < KD; ++s) read_k(k_nxt, s);
+                }
             }
         }
     };
 
-    if (n_tiles > 0) issue_tile(0, 0);
-    for (int t = 0; t < n_tiles; t += 2) {
-        // stage 0
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();       // tile t is in LDS for everyone; everyone has finished tile t-1 (stage 1 is free)
-        if (t + 1 < n_tiles) issue_tile(t + 1, 1);
-        if (t * PF_BN < lim_wave_max) compute_tile(t, smem);
-        if (t + 1 >= n_tiles) break;
-        // stage 1
+    // prologue: K(0), K(1), V(0) in flight; first K operands of tile 0
+    if (n_tiles > 0) {
+        issue_k(0, 0);
+        if (n_tiles > 1) issue_k(1, 1);
+        issue_v(0, 0);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if (t + 2 < n_tiles) issue_tile(t + 2, 0);
-        if ((t + 1) * PF_BN < lim_wave_max) compute_tile(t + 1, smem + L::STAGE_BYTES);
+        if (lim_wave_max > 0) {
+#pragma unroll
+            for (int s = 0; s < KD; ++s) read_k(smem, s);
+        }
+        for (int t = 0; t < n_tiles; t += 2) {
+            tile(t, std::integral_constant<int, 0>{});
+            if (t + 1 < n_tiles) tile(t + 1, std::integral_constant<int, 1>{});
+        }
     }
 
     // ---- normalise and store ------------------------------------------------------------------
