@@ -15,7 +15,6 @@
 namespace incin_rocm {
 hipError_t launch_sdpa_generic(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_sdpa_prefill_mfma(const SdpaParams& p, int dtype, hipStream_t stream);
-hipError_t launch_sdpa_prefill_pipe(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_sdpa_decode(const SdpaParams& p, int dtype, hipStream_t stream);
 int decode_keys_per_tile(int dtype, int D, int R);
 hipError_t launch_copy16(void* dst, const void* src, size_t bytes, hipStream_t stream);
@@ -110,7 +109,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         return fail(INCIN_ROCM_ESHAPE, "scaled_dot_product_attention: batch and head counts are limited to 65535 per launch");
     if (!d->q || !d->o || (d->Skv > 0 && (!d->k || !d->v)))
         return fail(INCIN_ROCM_EINVAL, "scaled_dot_product_attention: null tensor pointer");
-    if (d->impl < INCIN_ROCM_IMPL_AUTO || d->impl > INCIN_ROCM_IMPL_MFMA_PIPE)
+    if (d->impl < INCIN_ROCM_IMPL_AUTO || d->impl > INCIN_ROCM_IMPL_SPLITKV)
         return fail(INCIN_ROCM_EINVAL, "scaled_dot_product_attention: unknown impl %d", d->impl);
     if (d->num_splits < 0) return fail(INCIN_ROCM_EINVAL, "scaled_dot_product_attention: negative num_splits");
 
@@ -130,9 +129,9 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         else if (split_ok && R <= 8) impl = INCIN_ROCM_IMPL_SPLITKV;
         else impl = INCIN_ROCM_IMPL_GENERIC;
     }
-    if ((impl == INCIN_ROCM_IMPL_MFMA || impl == INCIN_ROCM_IMPL_MFMA_PIPE) && !mfma_ok)
+    if (impl == INCIN_ROCM_IMPL_MFMA && !mfma_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
-                    "scaled_dot_product_attention: the MFMA kernels need f16/bf16, D == Dv in {64,128}, scale > 0, no dense mask and 16-byte aligned rows");
+                    "scaled_dot_product_attention: the MFMA kernel needs f16/bf16, D == Dv in {64,128}, scale > 0, no dense mask and 16-byte aligned rows");
     if (impl == INCIN_ROCM_IMPL_SPLITKV && !split_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
                     "scaled_dot_product_attention: the split-KV kernel needs D == Dv in {64,128}, Sq <= 64, no dense mask and 16-byte aligned rows");
@@ -405,7 +404,6 @@ int incin_rocm_sdpa_fwd(const incin_rocm_sdpa_desc_t* desc, void* stream)
     hipError_t e;
     switch (plan.impl) {
         case INCIN_ROCM_IMPL_MFMA: e = incin_rocm::launch_sdpa_prefill_mfma(p, desc->dtype, s); break;
-        case INCIN_ROCM_IMPL_MFMA_PIPE: e = incin_rocm::launch_sdpa_prefill_pipe(p, desc->dtype, s); break;
         case INCIN_ROCM_IMPL_SPLITKV: e = incin_rocm::launch_sdpa_decode(p, desc->dtype, s); break;
         default: e = incin_rocm::launch_sdpa_generic(p, desc->dtype, s); break;
     }

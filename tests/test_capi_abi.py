@@ -56,7 +56,6 @@ def _plan(d):
 
 def test_dispatch_choices():
     assert _plan(_desc())[2] == capi.IMPL_MFMA
-    assert _plan(_desc(impl=capi.IMPL_MFMA_PIPE))[2] == capi.IMPL_MFMA_PIPE
     assert _plan(_desc(dtype=capi.F32))[2] == capi.IMPL_GENERIC
     assert _plan(_desc(D=80, Dv=80))[2] == capi.IMPL_GENERIC
     assert _plan(_desc(add_mask=0x20000))[2] == capi.IMPL_GENERIC

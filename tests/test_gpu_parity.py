@@ -172,7 +172,7 @@ def test_reference_golden_vectors_on_gpu(gpu):
 
 # ---- MFMA prefill kernel --------------------------------------------------------------------
 
-MFMA_IMPLS = [capi.IMPL_MFMA, capi.IMPL_MFMA_PIPE]
+MFMA_IMPLS = [capi.IMPL_MFMA]
 
 
 @pytest.mark.parametrize("impl", MFMA_IMPLS)
