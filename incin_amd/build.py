@@ -13,6 +13,10 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libincin_rocm.so")
 SOURCES = ["incin_rocm.hip", "sdpa_generic.hip", "sdpa_decode.hip", "sdpa_prefill_mfma.hip", "copy.hip"]
+HOST_DIR = os.path.join(HERE, "host")
+HOST_LIB = os.path.join(LIBDIR, "libincin_rocm_host.so")
+HOST_SOURCES = ["rocm_backend.cpp", "rocm_backend_c.cpp"]
+CXX = os.environ.get("CXX", "g++")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -packed-fp32-ops off: the compiler must not form packed-fp32 VALU instructions from float code.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
@@ -41,6 +45,21 @@ def build_library(verbose=False):
     return LIB
 
 
+def build_host_library(verbose=False):
+    """C++ host mirror of the backend interface; plain host code that links against the C ABI library."""
+    os.makedirs(LIBDIR, exist_ok=True)
+    cmd = [CXX, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra", "-o", HOST_LIB]
+    cmd += [os.path.join(HOST_DIR, f) for f in HOST_SOURCES]
+    cmd += ["-L" + LIBDIR, "-lincin_rocm", "-Wl,-rpath,$ORIGIN"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("host library build failed:\n%s\n%s" % (r.stdout, r.stderr))
+    if verbose:
+        print("built", HOST_LIB)
+    return HOST_LIB
+
+
 if __name__ == "__main__":
     build_library(verbose=True)
+    build_host_library(verbose=True)
     sys.exit(0)

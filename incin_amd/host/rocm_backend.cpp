@@ -1,0 +1,397 @@
+// See rocm_backend.hpp.  Everything that touches the device goes through the C ABI.
+#include "rocm_backend.hpp"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+
+#include "../../include/incin_rocm.h"
+
+namespace incin_rocm_host {
+
+namespace {
+
+thread_local int64_t g_launches = 0;
+
+Error ok() { return Error{}; }
+Error err(ErrorKind k, std::string m) { return Error{k, std::move(m)}; }
+
+std::string shape_str(const std::vector<int64_t>& s)
+{
+    std::string r = "[";
+    for (size_t i = 0; i < s.size(); ++i) r += (i ? ", " : "") + std::to_string(s[i]);
+    return r + "]";
+}
+
+// Status code of the C ABI -> the Error variant the Rust backend would return.
+Error from_status(int rc, int32_t device)
+{
+    if (rc == INCIN_ROCM_OK) return ok();
+    const std::string msg = incin_rocm_last_error();
+    switch (rc) {
+        case INCIN_ROCM_ESHAPE: return err(ErrorKind::ShapeMismatch, msg);
+        case INCIN_ROCM_EDTYPE: return err(ErrorKind::UnsupportedDType, msg);
+        case INCIN_ROCM_EDEVICE: return err(ErrorKind::InvalidDeviceOrdinal, "backend Rocm, ordinal " + std::to_string(device) + ": " + msg);
+        case INCIN_ROCM_ENOMEM: return err(ErrorKind::OutOfMemory, msg);
+        case INCIN_ROCM_EUNSUPPORTED: return err(ErrorKind::UnsupportedBackendOperation, msg);
+        default: return err(ErrorKind::Msg, msg);
+    }
+}
+
+std::vector<int64_t> contiguous_strides(const std::vector<int64_t>& shape)
+{
+    std::vector<int64_t> st(shape.size());
+    int64_t acc = 1;
+    for (int i = (int)shape.size() - 1; i >= 0; --i) {
+        st[i] = acc;
+        acc *= shape[i];
+    }
+    return st;
+}
+
+Error alloc_storage(const std::vector<int64_t>& dims, DType dtype, int32_t device, RocmStorage* out)
+{
+    int64_t n = 1;
+    for (int64_t d : dims) {
+        if (d < 0) return err(ErrorKind::ShapeMismatch, "negative extent in " + shape_str(dims));
+        n *= d;
+    }
+    void* p = nullptr;
+    const size_t bytes = (size_t)n * dtype_size(dtype);
+    if (Error e = from_status(incin_rocm_alloc(device, bytes, &p), device)) return e;
+    out->buffer = std::make_shared<RocmBuffer>(device, p, bytes);
+    out->shape = dims;
+    out->strides = contiguous_strides(dims);
+    out->offset_elements = 0;
+    out->dtype = dtype;
+    out->device = device;
+    out->mask_tag.reset();
+    return ok();
+}
+
+// strides of `s` seen through a right-aligned broadcast to `target` (rank >= s.rank); 0 where expanded
+bool broadcast_strides(const std::vector<int64_t>& shape, const std::vector<int64_t>& strides,
+                       const std::vector<int64_t>& target, std::vector<int64_t>* out)
+{
+    const size_t n = target.size(), r = shape.size();
+    if (r > n) return false;
+    out->assign(n, 0);
+    for (size_t i = 0; i < r; ++i) {
+        const size_t ti = n - r + i;
+        if (shape[i] == target[ti]) (*out)[ti] = shape[i] == 1 ? 0 : strides[i];
+        else if (shape[i] == 1) (*out)[ti] = 0;
+        else return false;
+    }
+    return true;
+}
+
+}  // namespace
+
+int64_t last_launch_count() { return g_launches; }
+
+RocmBuffer::~RocmBuffer()
+{
+    if (ptr_) incin_rocm_free(device_, ptr_);
+}
+
+int64_t RocmStorage::numel() const
+{
+    int64_t n = 1;
+    for (int64_t d : shape) n *= d;
+    return n;
+}
+
+bool RocmStorage::is_contiguous() const
+{
+    int64_t acc = 1;
+    for (int i = (int)shape.size() - 1; i >= 0; --i) {
+        if (shape[i] != 1 && strides[i] != acc) return false;
+        acc *= shape[i];
+    }
+    return true;
+}
+
+Error broadcast_shape(const std::vector<int64_t>& a, const std::vector<int64_t>& b, std::vector<int64_t>* out)
+{
+    const size_t n = std::max(a.size(), b.size());
+    out->assign(n, 1);
+    for (size_t i = 0; i < n; ++i) {
+        const int64_t da = i + a.size() >= n ? a[i + a.size() - n] : 1;
+        const int64_t db = i + b.size() >= n ? b[i + b.size() - n] : 1;
+        if (da != db && da != 1 && db != 1)
+            return err(ErrorKind::ShapeMismatch, "cannot broadcast shapes " + shape_str(a) + " and " + shape_str(b) +
+                                                     ": incompatible at right-aligned axis " + std::to_string(i));
+        (*out)[i] = std::max(da, db);
+    }
+    return ok();
+}
+
+Error RocmBackend::from_bytes(const void* bytes, size_t nbytes, const std::vector<int64_t>& dims, DType dtype, int32_t device,
+                              RocmStorage* out)
+{
+    if ((int)dtype < 0 || (int)dtype > 2) return err(ErrorKind::UnsupportedDType, "dtype tag " + std::to_string((int)dtype) + " on backend Rocm");
+    RocmStorage s;
+    if (Error e = alloc_storage(dims, dtype, device, &s)) return e;
+    if ((size_t)s.numel() * dtype_size(dtype) != nbytes)
+        return err(ErrorKind::Msg, "from_bytes: " + std::to_string(nbytes) + " bytes do not fill shape " + shape_str(dims));
+    if (nbytes && !bytes) return err(ErrorKind::Msg, "from_bytes: null source");
+    if (Error e = from_status(incin_rocm_memcpy_h2d(device, s.buffer->ptr(), bytes, nbytes), device)) return e;
+    *out = std::move(s);
+    return ok();
+}
+
+Error RocmBackend::to_bytes(const RocmStorage& s, std::vector<uint8_t>* out)
+{
+    const size_t isz = dtype_size(s.dtype);
+    const int64_t n = s.numel();
+    out->assign((size_t)n * isz, 0);
+    if (n == 0) return ok();
+    if (s.is_contiguous())
+        return from_status(incin_rocm_memcpy_d2h(s.device, out->data(), s.data(), (size_t)n * isz), s.device);
+    // strided or broadcast view: fetch the whole allocation once, gather on the host
+    std::vector<uint8_t> raw(s.buffer->bytes());
+    if (Error e = from_status(incin_rocm_memcpy_d2h(s.device, raw.data(), s.buffer->ptr(), raw.size()), s.device)) return e;
+    std::vector<int64_t> idx(s.shape.size(), 0);
+    for (int64_t flat = 0; flat < n; ++flat) {
+        int64_t off = s.offset_elements;
+        for (size_t a = 0; a < idx.size(); ++a) off += idx[a] * s.strides[a];
+        std::memcpy(out->data() + (size_t)flat * isz, raw.data() + (size_t)off * isz, isz);
+        for (int a = (int)idx.size() - 1; a >= 0; --a) {
+            if (++idx[a] < s.shape[a]) break;
+            idx[a] = 0;
+        }
+    }
+    return ok();
+}
+
+Error RocmBackend::transpose(const RocmStorage& s, int a, int b, RocmStorage* out)
+{
+    const int r = (int)s.shape.size();
+    if (a < 0 || b < 0 || a >= r || b >= r) return err(ErrorKind::ShapeMismatch, "transpose: axis out of range for rank " + std::to_string(r));
+    *out = s;
+    std::swap(out->shape[a], out->shape[b]);
+    std::swap(out->strides[a], out->strides[b]);
+    out->mask_tag.reset();
+    return ok();
+}
+
+Error RocmBackend::broadcast_as(const RocmStorage& s, const std::vector<int64_t>& dims, RocmStorage* out)
+{
+    std::vector<int64_t> st;
+    if (!broadcast_strides(s.shape, s.strides, dims, &st))
+        return err(ErrorKind::ShapeMismatch, "cannot broadcast " + shape_str(s.shape) + " to " + shape_str(dims));
+    *out = s;
+    out->shape = dims;
+    out->strides = st;
+    out->mask_tag.reset();
+    return ok();
+}
+
+Error RocmBackend::narrow(const RocmStorage& s, int dim, int64_t start, int64_t len, RocmStorage* out)
+{
+    const int r = (int)s.shape.size();
+    if (dim < 0 || dim >= r || start < 0 || len < 0 || start + len > s.shape[dim])
+        return err(ErrorKind::ShapeMismatch, "narrow: range out of bounds for " + shape_str(s.shape));
+    *out = s;
+    out->shape[dim] = len;
+    out->offset_elements += start * s.strides[dim];
+    out->mask_tag.reset();
+    return ok();
+}
+
+Error RocmBackend::tag_causal(const RocmStorage& mask, RocmStorage* out)
+{
+    if (mask.shape.size() < 2) return err(ErrorKind::ShapeMismatch, "a causal mask has at least two axes");
+    *out = mask;
+    out->mask_tag = MaskTag{MaskTag::Causal, nullptr, 0};
+    return ok();
+}
+
+Error RocmBackend::tag_key_padding(const RocmStorage& mask, const std::vector<int32_t>& lens, RocmStorage* out)
+{
+    void* p = nullptr;
+    if (Error e = from_status(incin_rocm_alloc(mask.device, lens.size() * sizeof(int32_t), &p), mask.device)) return e;
+    auto buf = std::make_shared<RocmBuffer>(mask.device, p, lens.size() * sizeof(int32_t));
+    if (Error e = from_status(incin_rocm_memcpy_h2d(mask.device, p, lens.data(), lens.size() * sizeof(int32_t)), mask.device)) return e;
+    *out = mask;
+    out->mask_tag = MaskTag{MaskTag::KeyPadding, buf, (int64_t)lens.size()};
+    return ok();
+}
+
+Error RocmBackend::scaled_dot_product_attention(const RocmStorage& q, const RocmStorage& k, const RocmStorage& v,
+                                                const RocmStorage* mask, std::optional<double> scale, RocmStorage* out)
+{
+    static const char* OP = "scaled_dot_product_attention";
+    // -- devices and dtypes, in the order the reference's checks fire ------------------------------------
+    if (q.device != k.device || q.device != v.device || (mask && mask->device != q.device))
+        return err(ErrorKind::DeviceMismatch, std::string(OP) + ": operands live on different devices");
+    if (k.dtype != q.dtype || v.dtype != q.dtype || (mask && mask->dtype != q.dtype))
+        return err(ErrorKind::DTypeStorageMismatch, std::string(OP) + ": operands have different dtypes");
+    // -- shapes (cpu/ops/matmul.rs:170-196) ------------------------------------------------------------
+    const int qr = (int)q.shape.size(), kr = (int)k.shape.size(), vr = (int)v.shape.size();
+    if (qr < 2 || kr < 2 || vr < 2)
+        return err(ErrorKind::ShapeMismatch, std::string(OP) + ": operands need rank >= 2; got q " + shape_str(q.shape) +
+                                                 ", k " + shape_str(k.shape) + ", v " + shape_str(v.shape));
+    const int64_t Sq = q.shape[qr - 2], D = q.shape[qr - 1], Skv = k.shape[kr - 2], Dv = v.shape[vr - 1];
+    if (k.shape[kr - 1] != D)
+        return err(ErrorKind::ShapeMismatch, std::string(OP) + ": q and k inner dims must match: q " + shape_str(q.shape) + ", k " + shape_str(k.shape));
+    if (v.shape[vr - 2] != Skv)
+        return err(ErrorKind::ShapeMismatch, std::string(OP) + ": k and v key counts must match: k " + shape_str(k.shape) + ", v " + shape_str(v.shape));
+    if (q.strides[qr - 1] != 1 && D > 1) return err(ErrorKind::UnsupportedBackendOperation, std::string(OP) + ": q needs a contiguous last axis on backend Rocm");
+    if (k.strides[kr - 1] != 1 && D > 1) return err(ErrorKind::UnsupportedBackendOperation, std::string(OP) + ": k needs a contiguous last axis on backend Rocm");
+    if (v.strides[vr - 1] != 1 && Dv > 1) return err(ErrorKind::UnsupportedBackendOperation, std::string(OP) + ": v needs a contiguous last axis on backend Rocm");
+
+    // -- batch axes: broadcast(broadcast(q, k), v), NumPy rule (cpu/ops/matmul.rs:198-221) ------------------
+    const std::vector<int64_t> qb(q.shape.begin(), q.shape.end() - 2), kb(k.shape.begin(), k.shape.end() - 2),
+        vb(v.shape.begin(), v.shape.end() - 2);
+    std::vector<int64_t> bshape, tmp;
+    if (Error e = broadcast_shape(qb, kb, &tmp)) return e;
+    if (Error e = broadcast_shape(tmp, vb, &bshape)) return e;
+    const int nb = (int)bshape.size();
+    std::vector<int64_t> qs, ks, vs, ms;
+    broadcast_strides(qb, std::vector<int64_t>(q.strides.begin(), q.strides.end() - 2), bshape, &qs);
+    broadcast_strides(kb, std::vector<int64_t>(k.strides.begin(), k.strides.end() - 2), bshape, &ks);
+    broadcast_strides(vb, std::vector<int64_t>(v.strides.begin(), v.strides.end() - 2), bshape, &vs);
+
+    // -- mask: None | tagged | dense additive, broadcast against [..b, Sq, Skv] without enlarging it ------------
+    int64_t m_si = 0, m_sj = 0;
+    bool dense_mask = false;
+    if (mask) {
+        std::vector<int64_t> mshape = mask->shape, mstr = mask->strides;
+        while ((int)mshape.size() < 2) {
+            mshape.insert(mshape.begin(), 1);
+            mstr.insert(mstr.begin(), 0);
+        }
+        std::vector<int64_t> full = bshape;
+        full.push_back(Sq);
+        full.push_back(Skv);
+        std::vector<int64_t> mfull;
+        if (!broadcast_strides(mshape, mstr, full, &mfull))
+            return err(ErrorKind::ShapeMismatch, std::string(OP) + ": mask " + shape_str(mask->shape) +
+                                                     " does not broadcast to the scores " + shape_str(full));
+        if (!mask->mask_tag) {
+            dense_mask = true;
+            ms.assign(mfull.begin(), mfull.end() - 2);
+            m_si = mfull[nb];
+            m_sj = mfull[nb + 1];
+        }
+    }
+
+    // -- output: fresh contiguous [..b, Sq, Dv] of the input dtype -----------------------------------------------
+    std::vector<int64_t> oshape = bshape;
+    oshape.push_back(Sq);
+    oshape.push_back(Dv);
+    RocmStorage o;
+    if (Error e = alloc_storage(oshape, q.dtype, q.device, &o)) return e;
+    const std::vector<int64_t> os(o.strides.begin(), o.strides.end() - 2);
+
+    // -- collapse the batch axes into (outer..., B, Hkv, G) ----------------------------------------------------
+    // G: the last batch axis when k and v are broadcast along it and q is not (the reference's way to write
+    // grouped-query attention: q [.., Hkv, G, S, D] against k, v [.., Hkv, 1, S, D]); Hkv: the axis before it;
+    // B: the one before that; anything further left is looped over here, one launch per index.
+    int g_ax = -1, h_ax = -1, b_ax = -1;
+    int next = nb - 1;
+    if (next >= 0 && bshape[next] > 1 && ks[next] == 0 && vs[next] == 0 && qs[next] != 0) g_ax = next--;
+    // rank-4 operands read [B, H, S, D] (k, v broadcast over H: one shared kv head); rank-5 and up read
+    // [.., B, Hkv, G, S, D]
+    if (next >= 0 && !(g_ax >= 0 && next == 0)) h_ax = next--;
+    if (next >= 0) b_ax = next--;
+    const int n_outer = next + 1;
+    int64_t G = g_ax >= 0 ? bshape[g_ax] : 1;
+    int64_t Hkv = h_ax >= 0 ? bshape[h_ax] : 1;
+    const int64_t B = b_ax >= 0 ? bshape[b_ax] : 1;
+    // query head hq = hkv * G + g must be one stride for q, o and the mask
+    bool fold_g = g_ax >= 0 && h_ax >= 0;
+    if (fold_g) {
+        const bool q_ok = qs[h_ax] == G * qs[g_ax] || Hkv == 1;
+        const bool o_ok = os[h_ax] == G * os[g_ax] || Hkv == 1;
+        const bool m_ok = !dense_mask || (ms[h_ax] == G * ms[g_ax]) || Hkv == 1;
+        if (!(q_ok && o_ok && m_ok)) fold_g = false;
+    }
+    // when the group axis cannot be folded into the head axis, the kv-head axis joins the outer loop
+    std::vector<int> outer_axes;
+    for (int a = 0; a < n_outer; ++a) outer_axes.push_back(a);
+    int head_ax = h_ax;       // axis whose stride is the head stride of q / o / mask
+    int64_t Hq = Hkv * G, Hkv_launch = Hkv;
+    if (g_ax >= 0 && !fold_g) {
+        if (h_ax >= 0) outer_axes.push_back(h_ax);
+        head_ax = g_ax;
+        Hq = G;
+        Hkv_launch = 1;
+    } else if (g_ax >= 0) {
+        head_ax = g_ax;       // stride of one query head is the stride of the group axis
+    }
+
+    const double s64 = scale ? *scale : 1.0 / std::sqrt((double)D);       // shape_ops.rs:1259-1260 (q's last dim)
+    incin_rocm_sdpa_desc_t d;
+    std::memset(&d, 0, sizeof(d));
+    d.dtype = (int32_t)q.dtype;
+    d.device = q.device;
+    d.B = B; d.Hq = Hq; d.Hkv = Hkv_launch; d.Sq = Sq; d.Skv = Skv; d.D = D; d.Dv = Dv;
+    auto st = [&](const std::vector<int64_t>& s, int ax) { return ax >= 0 ? s[ax] : 0; };
+    d.q_stride[0] = st(qs, b_ax); d.q_stride[1] = st(qs, head_ax); d.q_stride[2] = q.strides[qr - 2];
+    d.o_stride[0] = st(os, b_ax); d.o_stride[1] = st(os, head_ax); d.o_stride[2] = o.strides[nb];
+    // k, v: one stride per kv head (the axis before the group axis, or the head axis itself when there is no group)
+    const int kv_head_ax = (g_ax >= 0) ? (fold_g ? h_ax : -1) : h_ax;
+    d.k_stride[0] = st(ks, b_ax); d.k_stride[1] = st(ks, kv_head_ax); d.k_stride[2] = k.strides[kr - 2];
+    d.v_stride[0] = st(vs, b_ax); d.v_stride[1] = st(vs, kv_head_ax); d.v_stride[2] = v.strides[vr - 2];
+    d.scale = (float)s64;                                                   // elementwise_kernel.rs:87
+    if (mask && mask->mask_tag) {
+        if (mask->mask_tag->kind == MaskTag::Causal) d.causal = 1;
+        else {
+            if (mask->mask_tag->lens_count != B || n_outer != 0 || (g_ax >= 0 && !fold_g))
+                return err(ErrorKind::ShapeMismatch, std::string(OP) + ": key-padding lengths must have one entry per batch index");
+            d.kv_lens = static_cast<const int32_t*>(mask->mask_tag->lens->ptr());
+        }
+    } else if (dense_mask) {
+        d.mask_stride[0] = st(ms, b_ax); d.mask_stride[1] = st(ms, head_ax); d.mask_stride[2] = m_si; d.mask_stride[3] = m_sj;
+    }
+
+    const size_t isz = dtype_size(q.dtype);
+    // iterate the outer axes
+    std::vector<int64_t> oidx(outer_axes.size(), 0);
+    int64_t n_launch = 1;
+    for (int a : outer_axes) n_launch *= bshape[a];
+    std::shared_ptr<RocmBuffer> workspace;
+    g_launches = 0;
+    for (int64_t it = 0; it < n_launch; ++it) {
+        int64_t qo = q.offset_elements, ko = k.offset_elements, vo = v.offset_elements, oo = 0, mo = mask ? mask->offset_elements : 0;
+        for (size_t a = 0; a < outer_axes.size(); ++a) {
+            const int ax = outer_axes[a];
+            qo += oidx[a] * qs[ax]; ko += oidx[a] * ks[ax]; vo += oidx[a] * vs[ax]; oo += oidx[a] * os[ax];
+            if (dense_mask) mo += oidx[a] * ms[ax];
+        }
+        d.q = static_cast<const char*>(q.buffer->ptr()) + qo * (int64_t)isz;
+        d.k = static_cast<const char*>(k.buffer->ptr()) + ko * (int64_t)isz;
+        d.v = static_cast<const char*>(v.buffer->ptr()) + vo * (int64_t)isz;
+        d.o = static_cast<char*>(o.buffer->ptr()) + oo * (int64_t)isz;
+        d.add_mask = dense_mask ? static_cast<const char*>(mask->buffer->ptr()) + mo * (int64_t)isz : nullptr;
+        size_t ws_bytes = 0;
+        int32_t splits = 0;
+        d.workspace = nullptr;
+        d.workspace_bytes = 0;
+        if (Error e = from_status(incin_rocm_sdpa_workspace(&d, &ws_bytes, &splits, nullptr), q.device)) return e;
+        if (ws_bytes) {
+            if (!workspace || workspace->bytes() < ws_bytes) {
+                void* wp = nullptr;
+                if (Error e = from_status(incin_rocm_alloc(q.device, ws_bytes, &wp), q.device)) return e;
+                workspace = std::make_shared<RocmBuffer>(q.device, wp, ws_bytes);
+            }
+            d.workspace = workspace->ptr();
+            d.workspace_bytes = workspace->bytes();
+        }
+        if (Error e = from_status(incin_rocm_sdpa_fwd(&d, nullptr), q.device)) return e;
+        ++g_launches;
+        for (int a = (int)oidx.size() - 1; a >= 0; --a) {
+            if (++oidx[a] < bshape[outer_axes[a]]) break;
+            oidx[a] = 0;
+        }
+    }
+    // the workspace is used stream-ordered: finish before it is released
+    if (workspace)
+        if (Error e = from_status(incin_rocm_sync(q.device), q.device)) return e;
+    *out = std::move(o);
+    return ok();
+}
+
+}  // namespace incin_rocm_host

@@ -1,0 +1,110 @@
+// Host-side mirror of the part of incin's backend interface that the attention path uses, written
+// in C++ because no Rust toolchain exists in this build pipeline.  It stands where
+// crates/incin-backends/src/rocm/{storage,backend}.rs would stand: storage with shape / strides /
+// dtype / device (cf. cuda/storage.rs:24-59, cpu/storage.rs:199-204), byte round trips
+// (Backend::from_bytes / to_bytes, cuda/backend.rs:1905-1937), metadata-only views
+// (cpu/storage.rs:308-325) and TensorOps::scaled_dot_product_attention
+// (incin-core/src/tensor/backend.rs:485-492) with the reference's argument meaning and error kinds
+// (incin-core/src/err.rs:109-223).  All device work goes through the C ABI in include/incin_rocm.h.
+#pragma once
+#include <cstddef>
+#include <cstdint>
+#include <memory>
+#include <optional>
+#include <string>
+#include <vector>
+
+namespace incin_rocm_host {
+
+enum class DType : int32_t { F32 = 0, F16 = 1, BF16 = 2 };
+inline size_t dtype_size(DType d) { return d == DType::F32 ? 4 : 2; }
+
+// The variants of incin_core::Error this path can produce.
+enum class ErrorKind : int32_t {
+    None = 0,
+    Msg = 1,
+    ShapeMismatch = 2,
+    DTypeStorageMismatch = 3,
+    DeviceMismatch = 4,
+    UnsupportedDType = 5,
+    InvalidDeviceOrdinal = 6,
+    OutOfMemory = 7,
+    UnsupportedBackendOperation = 8,
+};
+
+struct Error {
+    ErrorKind kind = ErrorKind::None;
+    std::string message;
+    explicit operator bool() const { return kind != ErrorKind::None; }
+};
+
+// One device allocation, freed when the last storage that views it goes away.
+class RocmBuffer {
+  public:
+    RocmBuffer(int32_t device, void* ptr, size_t bytes) : device_(device), ptr_(ptr), bytes_(bytes) {}
+    ~RocmBuffer();
+    RocmBuffer(const RocmBuffer&) = delete;
+    RocmBuffer& operator=(const RocmBuffer&) = delete;
+    void* ptr() const { return ptr_; }
+    size_t bytes() const { return bytes_; }
+    int32_t device() const { return device_; }
+
+  private:
+    int32_t device_;
+    void* ptr_;
+    size_t bytes_;
+};
+
+// What a mask storage may declare about its contents so the backend need not read them.
+struct MaskTag {
+    enum Kind { Causal, KeyPadding } kind;
+    std::shared_ptr<RocmBuffer> lens;      // KeyPadding: int32 key counts, one per batch entry
+    int64_t lens_count = 0;
+};
+
+struct RocmStorage {
+    std::shared_ptr<RocmBuffer> buffer;
+    std::vector<int64_t> shape;
+    std::vector<int64_t> strides;          // elements; 0 on a broadcast axis
+    int64_t offset_elements = 0;
+    DType dtype = DType::F32;
+    int32_t device = 0;
+    std::optional<MaskTag> mask_tag;
+
+    int64_t numel() const;
+    bool is_contiguous() const;
+    const char* data() const { return static_cast<const char*>(buffer->ptr()) + offset_elements * (int64_t)dtype_size(dtype); }
+};
+
+struct RocmBackend {
+    // Backend::from_bytes: one allocation + one host-to-device copy; row-major contiguous.
+    static Error from_bytes(const void* bytes, size_t nbytes, const std::vector<int64_t>& dims, DType dtype, int32_t device,
+                            RocmStorage* out);
+    // Backend::to_bytes: logical (row-major) contents of the view.
+    static Error to_bytes(const RocmStorage& s, std::vector<uint8_t>* out);
+    static std::vector<int64_t> shape(const RocmStorage& s) { return s.shape; }
+
+    // Metadata-only views, as the reference's storages provide.
+    static Error transpose(const RocmStorage& s, int a, int b, RocmStorage* out);
+    static Error broadcast_as(const RocmStorage& s, const std::vector<int64_t>& dims, RocmStorage* out);
+    static Error narrow(const RocmStorage& s, int dim, int64_t start, int64_t len, RocmStorage* out);
+
+    // Declarations about a mask's contents (the caller vouches for them): `tag_causal` says the storage holds
+    // full(-inf).triu(1 + Skv - Sq) over its last two axes; `tag_key_padding` says it holds 0 for keys j < lens[b]
+    // and -inf for the rest, constant over query rows and heads.
+    static Error tag_causal(const RocmStorage& mask, RocmStorage* out);
+    static Error tag_key_padding(const RocmStorage& mask, const std::vector<int32_t>& lens, RocmStorage* out);
+
+    // TensorOps::scaled_dot_product_attention.
+    static Error scaled_dot_product_attention(const RocmStorage& q, const RocmStorage& k, const RocmStorage& v,
+                                              const RocmStorage* mask, std::optional<double> scale, RocmStorage* out);
+};
+
+// NumPy-style right-aligned broadcast of two shapes (cpu/stride.rs:86-106).
+Error broadcast_shape(const std::vector<int64_t>& a, const std::vector<int64_t>& b, std::vector<int64_t>* out);
+
+// Number of C-ABI attention calls the last scaled_dot_product_attention on this thread needed (1 unless batch
+// axes could not be collapsed into the descriptor's batch / head strides).
+int64_t last_launch_count();
+
+}  // namespace incin_rocm_host

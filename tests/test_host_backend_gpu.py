@@ -1,0 +1,197 @@
+"""The attention op through the C++ host mirror of the reference's backend interface, written the way
+the reference's own tests use the op (crates/incin/tests/medium_priority_ops_tests.rs:57-67:
+storages in, optional mask and scale, storage out) and checked against the CPU oracle."""
+import sys
+
+import numpy as np
+import pytest
+
+from incin_amd import dtypes
+from incin_amd import rocm_backend as RB
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+TOL = {RB.F32: 1e-5, RB.F16: 2e-2, RB.BF16: 2e-2}
+
+
+def say(msg):
+    print(msg, file=sys.stderr, flush=True)
+
+
+def rnd(seed, shape, dtype):
+    r = np.random.Generator(np.random.PCG64(seed))
+    return dtypes.round_to(r.standard_normal(shape, dtype=np.float32), dtype)
+
+
+def close(got, ref, tol, what):
+    assert got.shape == ref.shape, "%s: shape %s vs %s" % (what, got.shape, ref.shape)
+    nr = np.isnan(ref)
+    assert np.array_equal(np.isnan(got), nr), what + ": NaN pattern differs"
+    err = float(np.abs(np.where(nr, 0, got) - np.where(nr, 0, ref)).max()) if got.size else 0.0
+    say("%s: max-abs err %.3e" % (what, err))
+    assert err <= tol, "%s: %.3e > %.0e" % (what, err, tol)
+
+
+def test_ones_like_the_reference_test(gpu):
+    # medium_priority_ops_tests.rs:57-67: ones [1,2,4] everywhere, no mask, default scale -> dims [1,2,4]
+    say("host mirror: ones [1,2,4]")
+    one = np.ones((1, 2, 4), np.float32)
+    q, k, v = (RB.RocmStorage.from_numpy(one) for _ in range(3))
+    attn = RB.scaled_dot_product_attention(q, k, v, None, None)
+    assert attn.shape == (1, 2, 4)
+    # softmax of equal scores is uniform, so the output is the mean of v's rows: all ones
+    assert np.array_equal(attn.to_numpy(), one)
+
+
+def test_bytes_round_trip_and_views(gpu):
+    say("host mirror: from_bytes / to_bytes / views")
+    a = rnd(1, (3, 4, 5), RB.F32)
+    s = RB.RocmStorage.from_numpy(a)
+    assert s.shape == (3, 4, 5)
+    assert np.array_equal(s.to_numpy(), a)
+    assert np.array_equal(s.transpose(0, 2).to_numpy(), a.transpose(2, 1, 0))
+    assert np.array_equal(s.narrow(1, 1, 2).to_numpy(), a[:, 1:3])
+    b = RB.RocmStorage.from_numpy(a[:, :1])
+    assert np.array_equal(b.broadcast_as((2, 3, 4, 5)).to_numpy(), np.broadcast_to(a[:, :1], (2, 3, 4, 5)))
+    h = rnd(2, (7, 9), RB.BF16)
+    assert np.array_equal(RB.RocmStorage.from_numpy(h, RB.BF16).to_numpy(), h)
+    with pytest.raises(RB.BackendError) as e:
+        b.broadcast_as((3, 2, 4))
+    assert e.value.kind == "ShapeMismatch"
+
+
+@pytest.mark.parametrize("dtype", [RB.F32, RB.BF16, RB.F16])
+@pytest.mark.parametrize("shape", [
+    # (q shape, k shape, v shape)
+    ((5, 8), (7, 8), (7, 6)),                                      # rank 2: one head, no batch axes
+    ((3, 5, 16), (3, 9, 16), (3, 9, 16)),                          # rank 3
+    ((2, 3, 40, 64), (2, 3, 72, 64), (2, 3, 72, 64)),              # [B, H, S, D]
+    ((2, 6, 33, 64), (2, 1, 50, 64), (2, 1, 50, 64)),              # k, v broadcast over heads (one shared kv head)
+    ((2, 2, 4, 130, 128), (2, 2, 1, 200, 128), (2, 2, 1, 200, 128)),     # grouped-query: q [B,Hkv,G,S,D], kv [B,Hkv,1,S,D]
+    ((2, 1, 2, 3, 17, 32), (1, 2, 2, 1, 21, 32), (2, 2, 2, 1, 21, 32)),  # rank 6: leading axis looped on the host
+], ids=["rank2", "rank3", "bhsd", "mqa_broadcast", "gqa5d", "rank6"])
+def test_shapes_against_oracle(gpu, dtype, shape):
+    qs, ks, vs = shape
+    say("host mirror: q%s k%s v%s dtype %d" % (qs, ks, vs, dtype))
+    q, k, v = rnd(10, qs, dtype), rnd(11, ks, dtype), rnd(12, vs, dtype)
+    out = RB.scaled_dot_product_attention(RB.RocmStorage.from_numpy(q, dtype), RB.RocmStorage.from_numpy(k, dtype),
+                                          RB.RocmStorage.from_numpy(v, dtype))
+    ref = O.sdpa(q, k, v)
+    assert out.dtype == dtype
+    close(out.to_numpy(), ref, TOL[dtype], "shape %s" % (qs,))
+    if len(qs) <= 5:
+        assert RB.last_launch_count() == 1
+
+
+@pytest.mark.parametrize("dtype", [RB.F32, RB.BF16])
+def test_dense_masks_broadcast_like_the_reference(gpu, dtype):
+    B, Hkv, G, Sq, Skv, D = 2, 2, 3, 37, 53, 64
+    q, k, v = rnd(20, (B, Hkv, G, Sq, D), dtype), rnd(21, (B, Hkv, 1, Skv, D), dtype), rnd(22, (B, Hkv, 1, Skv, D), dtype)
+    Q, K, V = (RB.RocmStorage.from_numpy(x, dtype) for x in (q, k, v))
+    r = np.random.Generator(np.random.PCG64(23))
+    for mshape in [(Sq, Skv), (1, Skv), (B, 1, 1, Sq, Skv), (B, Hkv, G, Sq, Skv), (1, Hkv, 1, Sq, 1), (B, Hkv, 1, 1, Skv)]:
+        say("host mirror: dense mask %s dtype %d" % (mshape, dtype))
+        m = dtypes.round_to(r.standard_normal(mshape, dtype=np.float32), dtype)
+        m[r.random(mshape) < 0.2] = -np.inf
+        m[..., 0] = 0.0                            # keep every row alive
+        out = RB.scaled_dot_product_attention(Q, K, V, RB.RocmStorage.from_numpy(m, dtype), 0.3)
+        close(out.to_numpy(), O.sdpa(q, k, v, mask=m, scale=0.3), TOL[dtype], "mask %s" % (mshape,))
+    # a per-kv-head mask that is constant over the group cannot be folded into one head stride: the kv-head
+    # axis is then looped on the host
+    assert RB.last_launch_count() == Hkv
+    # fully masked row -> NaN, as exp(log_softmax) of an all -inf row gives on the reference
+    m = np.zeros((Sq, Skv), np.float32)
+    m[5, :] = -np.inf
+    out = RB.scaled_dot_product_attention(Q, K, V, RB.RocmStorage.from_numpy(m, dtype), None).to_numpy()
+    assert np.isnan(out[:, :, :, 5]).all() and not np.isnan(np.delete(out, 5, axis=3)).any()
+
+
+@pytest.mark.parametrize("dtype", [RB.F32, RB.BF16])
+def test_tagged_masks_equal_their_dense_form(gpu, dtype):
+    B, Hkv, G, Sq, Skv, D = 2, 2, 4, 96, 160, 128
+    q, k, v = rnd(30, (B, Hkv, G, Sq, D), dtype), rnd(31, (B, Hkv, 1, Skv, D), dtype), rnd(32, (B, Hkv, 1, Skv, D), dtype)
+    Q, K, V = (RB.RocmStorage.from_numpy(x, dtype) for x in (q, k, v))
+    say("host mirror: causal tag dtype %d" % dtype)
+    cm = O.causal_additive_mask(Sq, Skv)
+    M = RB.RocmStorage.from_numpy(cm, dtype)
+    dense = RB.scaled_dot_product_attention(Q, K, V, M).to_numpy()
+    tagged = RB.scaled_dot_product_attention(Q, K, V, M.tag_causal()).to_numpy()
+    ref = O.sdpa(q, k, v, mask=cm)
+    close(dense, ref, TOL[dtype], "dense causal")
+    close(tagged, ref, TOL[dtype], "tagged causal")
+    say("host mirror: key-padding tag dtype %d" % dtype)
+    lens = [160, 47]
+    pm = np.zeros((B, 1, 1, 1, Skv), np.float32)
+    for b, n in enumerate(lens):
+        pm[b, ..., n:] = -np.inf
+    P = RB.RocmStorage.from_numpy(pm, dtype)
+    ref = O.sdpa(q, k, v, mask=pm)
+    close(RB.scaled_dot_product_attention(Q, K, V, P).to_numpy(), ref, TOL[dtype], "dense padding")
+    close(RB.scaled_dot_product_attention(Q, K, V, P.tag_key_padding(lens)).to_numpy(), ref, TOL[dtype], "tagged padding")
+
+
+def test_views_as_operands(gpu):
+    # k handed over as a narrowed, transposed-back view of a larger cache; q as a slice of a [B,S,H,D] layout
+    say("host mirror: strided operands")
+    dtype = RB.BF16
+    B, H, S, D, CAP = 2, 4, 48, 64, 80
+    q_bshd = rnd(40, (B, S, H, D), dtype)
+    kc, vc = rnd(41, (B, H, CAP, D), dtype), rnd(42, (B, H, CAP, D), dtype)
+    Q = RB.RocmStorage.from_numpy(q_bshd, dtype).transpose(1, 2)
+    K = RB.RocmStorage.from_numpy(kc, dtype).narrow(2, 8, 60)
+    V = RB.RocmStorage.from_numpy(vc, dtype).narrow(2, 8, 60)
+    out = RB.scaled_dot_product_attention(Q, K, V)
+    ref = O.sdpa(q_bshd.transpose(0, 2, 1, 3), kc[:, :, 8:68], vc[:, :, 8:68])
+    close(out.to_numpy(), ref, TOL[dtype], "strided operands")
+
+
+def test_decode_step(gpu):
+    # one query token per head against a long cache: the split-KV path behind the same call
+    say("host mirror: decode step")
+    dtype = RB.BF16
+    B, Hkv, G, Skv, D = 3, 2, 4, 3000, 128
+    q, k, v = rnd(50, (B, Hkv, G, 1, D), dtype), rnd(51, (B, Hkv, 1, Skv, D), dtype), rnd(52, (B, Hkv, 1, Skv, D), dtype)
+    out = RB.scaled_dot_product_attention(*(RB.RocmStorage.from_numpy(x, dtype) for x in (q, k, v)))
+    close(out.to_numpy(), O.sdpa(q, k, v), TOL[dtype], "decode")
+
+
+def test_empty_extents(gpu):
+    say("host mirror: empty extents")
+    q, k, v = np.zeros((2, 3, 4), np.float32), np.zeros((2, 0, 4), np.float32), np.zeros((2, 0, 5), np.float32)
+    out = RB.scaled_dot_product_attention(*(RB.RocmStorage.from_numpy(x) for x in (q, k, v)))
+    assert out.shape == (2, 3, 5) and np.array_equal(out.to_numpy(), np.zeros((2, 3, 5), np.float32))
+    q0 = np.zeros((2, 0, 4), np.float32)
+    k1, v1 = np.ones((2, 6, 4), np.float32), np.ones((2, 6, 5), np.float32)
+    out = RB.scaled_dot_product_attention(*(RB.RocmStorage.from_numpy(x) for x in (q0, k1, v1)))
+    assert out.shape == (2, 0, 5)
+
+
+def test_error_behaviour(gpu):
+    say("host mirror: error kinds")
+    f = RB.RocmStorage.from_numpy
+    q, k, v = f(np.ones((2, 4, 8), np.float32)), f(np.ones((2, 6, 8), np.float32)), f(np.ones((2, 6, 8), np.float32))
+
+    def kind(*a, **kw):
+        with pytest.raises(RB.BackendError) as e:
+            RB.scaled_dot_product_attention(*a, **kw)
+        return e.value.kind
+
+    assert kind(q, f(np.ones((2, 6, 7), np.float32)), v) == "ShapeMismatch"          # q.D != k.D
+    assert kind(q, k, f(np.ones((2, 5, 8), np.float32))) == "ShapeMismatch"          # k and v key counts differ
+    assert kind(q, f(np.ones((3, 6, 8), np.float32)), f(np.ones((3, 6, 8), np.float32))) == "ShapeMismatch"   # batch 2 vs 3
+    assert kind(f(np.ones((8,), np.float32)), k, v) == "ShapeMismatch"               # rank 1
+    assert kind(q, k, v, f(np.ones((4, 5), np.float32))) == "ShapeMismatch"          # mask does not broadcast
+    assert kind(q, f(np.ones((2, 6, 8), np.float32), RB.BF16), v) == "DTypeStorageMismatch"
+    assert kind(q, k, v, f(np.zeros((4, 6), np.float32), RB.F16)) == "DTypeStorageMismatch"
+    with pytest.raises(RB.BackendError) as e:
+        RB.RocmStorage.from_numpy(np.ones(4, np.float32), device=99)
+    assert e.value.kind == "InvalidDeviceOrdinal"
+    with pytest.raises(RB.BackendError) as e:
+        RB.RocmStorage.from_bytes(b"\0" * 8, (4,), 7)
+    assert e.value.kind == "UnsupportedDType"
+    with pytest.raises(RB.BackendError) as e:
+        RB.RocmStorage.from_bytes(b"\0" * 8, (4,), RB.F32)
+    assert e.value.kind == "Msg"
+    # k with a strided last axis has no kernel on this backend
+    kt = f(np.ones((2, 8, 6), np.float32)).transpose(1, 2)
+    assert kind(q, kt, v) == "UnsupportedBackendOperation"
