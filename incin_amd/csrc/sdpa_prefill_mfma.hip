@@ -31,14 +31,19 @@
 // patterns (16 lanes x 16 bytes down a column of rows for K; 4 rows x 64 bytes
 // for the transposing V read) touch every bank once.
 //
-// Latency: with two wavefronts per SIMD the kernel is bound by LDS read latency
-// unless many operand reads are in flight, so matrix operands are fetched far
-// ahead of the MFMAs that use them: K operands four k-steps (8 MFMAs) ahead, V
-// operands 8 MFMAs ahead.  The one barrier per tile sits between the S^T product
-// and the softmax of the same tile; right after it the wavefront starts the
-// global loads of K(t+2) and V(t+1), the V(t) operand reads (their latency hides
-// under the softmax arithmetic) and, during O^T += V^T P^T, the first K(t+1)
-// operand reads for the next tile.
+// Overlap: the vector ALU work of the softmax and the matrix instructions of a wavefront only run
+// side by side when they are interleaved in that wavefront's own instruction stream (instructions of
+// the two wavefronts that share a SIMD take turns instead).  So the kernel is software-pipelined over
+// key tiles: while the matrix pipe computes S^T(t+1), the vector ALU turns S^T(t) into P^T(t) (two
+// exponentials, one pack per MFMA; the order is pinned with scheduling group barriers), and while the
+// matrix pipe computes O^T += V(t)^T P(t)^T the vector ALU takes the maxima of S^T(t+1).  Two score
+// tiles are alive at a time.  This loop runs over the tiles that need no mask; a wavefront's last
+// tiles (the diagonal ones of a causal mask, the ragged end of a key length) go through a plain
+// one-tile-at-a-time loop with masking.
+//
+// One barrier per tile, at the top of the iteration: it publishes K(t+1) and V(t), whose global loads
+// were started one iteration earlier, and frees the buffers of K(t) and V(t-1), into which the loads
+// of K(t+2) and V(t+1) start right away.  Matrix operands are read from LDS a few MFMAs ahead of use.
 //
 // The reference maximum is set from the first tile that holds a visible key and
 // afterwards only raised when a tile's maximum exceeds it by more than 2^8 (the
@@ -51,6 +56,12 @@
 
 namespace incin_rocm {
 
+#ifndef PF_KD
+#define PF_KD 2     // K operand reads run this many k-steps ahead of their MFMAs
+#endif
+#ifndef PF_VD
+#define PF_VD 4     // V operand reads run this many MFMAs ahead
+#endif
 
 template <typename T, int D>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
@@ -196,9 +207,9 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     float l_run = 0.0f;           // this lane's share of the running denominator
 
     // ---- matrix operands in flight ---------------------------------------------------------------
-    constexpr int KD = NSTEP < 4 ? NSTEP : 4;      // K operands are fetched KD k-steps ahead
+    constexpr int KD = PF_KD < NSTEP ? PF_KD : NSTEP;   // K operands are fetched KD k-steps (2*KD MFMAs) ahead
     constexpr int NPV = 4 * NDB;                   // MFMAs of one O^T update (4 k-steps of 16 keys x NDB blocks)
-    constexpr int VD = 8;                          // V operands are fetched VD MFMAs ahead
+    constexpr int VD = PF_VD;                      // V operands are fetched VD MFMAs ahead
     vec8 kbuf[KD][2];
     vec8 vbuf[VD];
     auto read_k = [&](const char* kb, int s) __attribute__((always_inline)) {
@@ -215,126 +226,186 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
         vbuf[i % VD] = __builtin_bit_cast(vec8, av);
     };
 
-    // One tile.  On entry kbuf holds the K(t) operands of k-steps 0..KD-1.  `par` = t % 2.
-    auto tile = [&](int t, auto PAR_) __attribute__((always_inline)) {
-        constexpr int par = decltype(PAR_)::value;
-        const char* k_cur = smem + par * L::TILE_BYTES;              // K(t)
-        const char* k_nxt = smem + (1 - par) * L::TILE_BYTES;        // K(t+1)
-        const char* v_cur = smem + (2 + par) * L::TILE_BYTES;        // V(t)
-        const int j0 = t * PF_BN;
-        const bool active = j0 < lim_wave_max;                       // some query of this wavefront sees this tile
-        floatx16 s_acc[2];
-        vec8 pb[4];
-        // ---- S^T = K Q'^T - m_ref ------------------------------------------------------------
-        if (active) {
-#pragma unroll
-            for (int s = 0; s < NSTEP; ++s) {
-#pragma unroll
-                for (int b2 = 0; b2 < 2; ++b2)
-                    s_acc[b2] = Mma<T>::run(kbuf[s % KD][b2], qreg[s], s == 0 ? neg_ref : s_acc[b2]);
-                if (s + KD < NSTEP) read_k(k_cur, s + KD);
-            }
-        }
-        // ---- the tile's barrier: K(t+1) and V(t) are in LDS for everyone, everyone is past
-        //      S^T(t) (K buffer `par` is free) and past O^T(t-1) (V buffer `1-par` is free) ----
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        if (t + 2 < n_tiles) issue_k(t + 2, par);
-        if (t + 1 < n_tiles) issue_v(t + 1, 1 - par);
-        if (active) {
-#pragma unroll
-            for (int i = 0; i < VD; ++i) read_v(v_cur, i);            // latency hides under the softmax arithmetic
-            __builtin_amdgcn_sched_barrier(0);
+    // Two score tiles are alive at a time: S(t) is turned into probabilities while the matrix pipe
+    // already computes S(t+1).  sacc[t % 2] holds S(t) - m_ref.
+    floatx16 sacc[2][2];
+    vec8 pb[4];
+    float tmax = -INFINITY;       // maximum of the current score tile relative to m_ref (both halves of the query's lanes)
+    float rsum = 0.0f;
 
-            // ---- masking (only tiles that cross a limit) --------------------------------
-            // register r of block kb is key j0 + 32*kb + 8*(r/4) + 4*g + (r%4)
-            if (j0 + PF_BN > lim_wave_min) {
-                const int rel = lim_lane - (j0 + 4 * g);
+    // register r of block kb of a score tile that starts at key j0 is key j0 + 32*kb + 8*(r/4) + 4*g + (r%4)
+    auto mask_tile = [&](floatx16 (&sx)[2], int j0) __attribute__((always_inline)) {
+        const int rel = lim_lane - (j0 + 4 * g);
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
+        for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int kofs = 32 * kb + 8 * (r / 4) + (r % 4);
-                        if (kofs >= rel) s_acc[kb][r] = -INFINITY;
-                    }
+            for (int r = 0; r < 16; ++r) {
+                const int kofs = 32 * kb + 8 * (r / 4) + (r % 4);
+                if (kofs >= rel) sx[kb][r] = -INFINITY;
             }
-
-            // ---- online softmax with lazy rescaling ------------------------------------------
-            float tmax = s_acc[0][0];
+    };
+    // Move the reference maximum when the pending tile maximum asks for it (first visible tile, or more
+    // than the threshold above the reference): rescales what has been accumulated and the pending tile.
+    auto adjust_reference = [&](floatx16 (&sx)[2]) __attribute__((always_inline)) {
+        const bool need = inited ? (tmax > PF_RESCALE_THRESHOLD) : (tmax > -INFINITY);
+        if (__builtin_amdgcn_ballot_w64(need) != 0) {
+            const float delta = need ? tmax : 0.0f;       // lanes that do not need it move by 0
+            const float alpha = inited ? __builtin_amdgcn_exp2f(-delta) : 1.0f;   // nothing accumulated yet: nothing to rescale
+            m_ref += delta;
+            inited = inited || need;
+            l_run *= alpha;
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) o_acc[db][r] *= alpha;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) neg_ref[r] = -m_ref;
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, s_acc[kb][r]);
-            tmax = xor32_max(tmax);                       // this tile's maximum relative to m_ref
-            const bool need = inited ? (tmax > PF_RESCALE_THRESHOLD) : (tmax > -INFINITY);
-            if (__builtin_amdgcn_ballot_w64(need) != 0) {
-                // move the reference to this tile's maximum (lanes that do not need it move by 0)
-                const float delta = need ? tmax : 0.0f;
-                const float alpha = inited ? __builtin_amdgcn_exp2f(-delta) : 1.0f;   // nothing accumulated yet: nothing to rescale
-                m_ref += delta;
-                inited = inited || need;
-                l_run *= alpha;
-#pragma unroll
-                for (int db = 0; db < NDB; ++db)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) o_acc[db][r] *= alpha;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) neg_ref[r] = -m_ref;
-#pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) s_acc[kb][r] -= delta;
-            }
-            // P^T in storage precision; element e of k-step ks is register 8*(ks%2)+e of key block ks/2,
-            // i.e. key 16*ks + 8*(e/4) + 4*g + (e%4)
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    pb[ks][e] = (T)__builtin_amdgcn_exp2f(s_acc[ks / 2][8 * (ks % 2) + e]);
-            // denominator from the rounded probabilities (the same values the numerator uses),
-            // two per instruction (v_dot2 with a vector of ones, f32 accumulate)
-            float rsum = 0.0f;
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-                for (int e = 0; e < 8; e += 2) {
-                    typename Mma<T>::vec2 pr = {pb[ks][e], pb[ks][e + 1]};
-                    rsum = Mma<T>::add2(pr, rsum);
-                }
-            l_run += rsum;
-            __builtin_amdgcn_sched_barrier(0);
-
-            // ---- O^T += V^T P^T; the next tile's first K operands are fetched underneath --------
-            const bool next_active = (t + 1 < n_tiles) && (j0 + PF_BN < lim_wave_max);
-#pragma unroll
-            for (int i = 0; i < NPV; ++i) {
-                o_acc[i % NDB] = Mma<T>::run(vbuf[i % VD], pb[i / NDB], o_acc[i % NDB]);
-                if (i + VD < NPV) read_v(v_cur, i + VD);
-                if (i == 1 && next_active) {
-#pragma unroll
-                    for (int s = 0; s < KD; ++s) read_k(k_nxt, s);
-                }
-            }
+                for (int r = 0; r < 16; ++r) sx[kb][r] -= delta;
         }
     };
+    // Probabilities of 4 score registers (slice sl = 0..7 of a tile): P^T in storage precision; element e of
+    // k-step ks is register 8*(ks%2)+e of key block ks/2, i.e. key 16*ks + 8*(e/4) + 4*g + (e%4).  The
+    // denominator is summed from the rounded values, two per instruction (dot2 with ones, f32 accumulate).
+    auto softmax_slice = [&](floatx16 (&sx)[2], int sl) __attribute__((always_inline)) {
+        const int ks = sl / 2, e0 = 4 * (sl % 2);
+#pragma unroll
+        for (int e = e0; e < e0 + 4; ++e) pb[ks][e] = (T)__builtin_amdgcn_exp2f(sx[ks / 2][8 * (ks % 2) + e]);
+#pragma unroll
+        for (int e = e0; e < e0 + 4; e += 2) {
+            typename Mma<T>::vec2 pr = {pb[ks][e], pb[ks][e + 1]};
+            rsum = Mma<T>::add2(pr, rsum);
+        }
+    };
+    auto max_of = [&](floatx16 (&sx)[2]) __attribute__((always_inline)) {
+        float m = sx[0][0];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) m = fmaxf(m, sx[kb][r]);
+        return xor32_max(m);
+    };
 
-    // prologue: K(0), K(1), V(0) in flight; first K operands of tile 0
-    if (n_tiles > 0) {
-        issue_k(0, 0);
-        if (n_tiles > 1) issue_k(1, 1);
-        issue_v(0, 0);
+#define SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
+    constexpr int SG_MFMA = 0x8, SG_VALU = 0x2, SG_TRANS = 0x400, SG_DSR = 0x100;
+
+    // start of every iteration t: K(t+1) and V(t) are in LDS for everyone, everyone is past S^T(t) (K buffer
+    // t%2 is free) and past O^T(t-1) (V buffer (t+1)%2 is free); start the next global loads into those.
+    auto turn = [&](int t) __attribute__((always_inline)) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if (lim_wave_max > 0) {
+        if (t + 2 < n_tiles) issue_k(t + 2, t & 1);
+        if (t + 1 < n_tiles) issue_v(t + 1, (t + 1) & 1);
+    };
+
+    // Hot iteration (tiles t and t+1 both computed by this wavefront, tile t+1 needs no mask):
+    // probabilities of tile t (scores in sacc[par], their maximum in tmax) on the vector ALU while the matrix
+    // pipe computes the scores of tile t+1; then O^T += V(t)^T P(t)^T with the maximum of S^T(t+1) underneath.
+    auto iter = [&](int t, auto PAR_) __attribute__((always_inline)) {
+        constexpr int par = decltype(PAR_)::value;
+        floatx16 (&sc)[2] = sacc[par];
+        floatx16 (&sn)[2] = sacc[1 - par];
+        const char* k_nxt = smem + (1 - par) * L::TILE_BYTES;        // K(t+1)
+        const char* v_cur = smem + (2 + par) * L::TILE_BYTES;        // V(t)
+        turn(t);
 #pragma unroll
-            for (int s = 0; s < KD; ++s) read_k(smem, s);
+        for (int s = 0; s < KD; ++s) read_k(k_nxt, s);
+        adjust_reference(sc);
+        rsum = 0.0f;
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < NSTEP; ++s) {
+#pragma unroll
+            for (int b2 = 0; b2 < 2; ++b2)
+                sn[b2] = Mma<T>::run(kbuf[s % KD][b2], qreg[s], s == 0 ? neg_ref : sn[b2]);
+            if (s + KD < NSTEP) read_k(k_nxt, s + KD);
+            if (NSTEP == 8) softmax_slice(sc, s);
+            else { softmax_slice(sc, 2 * s); softmax_slice(sc, 2 * s + 1); }
+            if (s >= NSTEP - VD / 2) { read_v(v_cur, 2 * (s - (NSTEP - VD / 2))); read_v(v_cur, 2 * (s - (NSTEP - VD / 2)) + 1); }
         }
-        for (int t = 0; t < n_tiles; t += 2) {
-            tile(t, std::integral_constant<int, 0>{});
-            if (t + 1 < n_tiles) tile(t + 1, std::integral_constant<int, 1>{});
+#pragma unroll
+        for (int s = 0; s < NSTEP; ++s) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                SGB(SG_MFMA, 1);
+                if (NSTEP == 8) { SGB(SG_TRANS, 2); SGB(SG_VALU, 2); } else { SGB(SG_TRANS, 4); SGB(SG_VALU, 4); }
+                if (s + KD < NSTEP) SGB(SG_DSR, 1);
+                if (s >= NSTEP - VD / 2) SGB(SG_DSR, 2);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        l_run += rsum;
+        float m0 = sn[0][0], m1 = sn[1][0];
+#pragma unroll
+        for (int i = 0; i < NPV; ++i) {
+            o_acc[i % NDB] = Mma<T>::run(vbuf[i % VD], pb[i / NDB], o_acc[i % NDB]);
+            if (i + VD < NPV) read_v(v_cur, i + VD);
+            if (NPV == 16) {
+                m0 = fmaxf(m0, sn[0][i]);
+                m1 = fmaxf(m1, sn[1][i]);
+            } else {
+                m0 = fmaxf(fmaxf(m0, sn[0][2 * i]), sn[0][2 * i + 1]);
+                m1 = fmaxf(fmaxf(m1, sn[1][2 * i]), sn[1][2 * i + 1]);
+            }
+        }
+        tmax = xor32_max(fmaxf(m0, m1));
+    };
+
+    // scores of one tile without overlap (prologue and the last tiles of a wavefront); kb = K tile in LDS
+    auto scores_plain = [&](const char* kb, floatx16 (&sx)[2], int j0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int s = 0; s < KD; ++s) read_k(kb, s);
+#pragma unroll
+        for (int s = 0; s < NSTEP; ++s) {
+#pragma unroll
+            for (int b2 = 0; b2 < 2; ++b2) sx[b2] = Mma<T>::run(kbuf[s % KD][b2], qreg[s], s == 0 ? neg_ref : sx[b2]);
+            if (s + KD < NSTEP) read_k(kb, s + KD);
+        }
+        if (j0 + PF_BN > lim_wave_min) mask_tile(sx, j0);
+        tmax = max_of(sx);
+    };
+
+    // tiles this wavefront computes, and how many of them the hot loop may produce scores for
+    const int n_act = lim_wave_max > 0 ? (lim_wave_max + PF_BN - 1) / PF_BN : 0;
+    const int n_hot = lim_wave_min > 0 ? min(lim_wave_min / PF_BN, n_act) : 0;      // tiles 0..n_hot-1 need no mask
+
+    if (n_tiles > 0) {
+        // prologue: K(0) first, then K(1), V(0) in flight; scores of tile 0
+        issue_k(0, 0);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (n_tiles > 1) issue_k(1, 1);
+        issue_v(0, 0);
+        if (n_act > 0) scores_plain(smem, sacc[0], 0);
+        int t = 0;
+        for (; t + 2 < n_hot; t += 2) {
+            iter(t, std::integral_constant<int, 0>{});
+            iter(t + 1, std::integral_constant<int, 1>{});
+        }
+        // the rest, one tile at a time without overlap; the pending scores are in sacc[0]
+        for (; t < n_tiles; ++t) {
+            turn(t);
+            if (t < n_act) {
+                const char* v_cur = smem + (2 + (t & 1)) * L::TILE_BYTES;
+#pragma unroll
+                for (int i = 0; i < VD; ++i) read_v(v_cur, i);
+                adjust_reference(sacc[0]);
+                rsum = 0.0f;
+#pragma unroll
+                for (int sl = 0; sl < 8; ++sl) softmax_slice(sacc[0], sl);
+                l_run += rsum;
+#pragma unroll
+                for (int i = 0; i < NPV; ++i) {
+                    o_acc[i % NDB] = Mma<T>::run(vbuf[i % VD], pb[i / NDB], o_acc[i % NDB]);
+                    if (i + VD < NPV) read_v(v_cur, i + VD);
+                }
+                if (t + 1 < n_act) scores_plain(smem + ((t + 1) & 1) * L::TILE_BYTES, sacc[0], (t + 1) * PF_BN);
+            }
         }
     }
+#undef SGB
 
     // ---- normalise and store ------------------------------------------------------------------
     const float l_tot = xor32_sum(l_run);
