@@ -31,7 +31,7 @@ PEAK_BF16_TFLOPS = 2516.6   # 256 CUs x 2.4 GHz x 4096 dense bf16 FLOP/clk/CU (v
 PEAK_HBM_GBS = 8000.0       # HBM3E, vendor figure
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same command (KiB per dispatch,
 # FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0 after calibration against the 1 GiB copy kernel): profiles/*.txt
-PREFILL_TRAFFIC_BYTES = (196696 * 2.0 + 131072) * 1024     # 5.37e8: |Q|+|K|+|V| read once, |O| written once
+PREFILL_TRAFFIC_BYTES = (196751 * 2.0 + 131073) * 1024     # 5.37e8: |Q|+|K|+|V| read once, |O| written once
 DECODE_TRAFFIC_BYTES = (2097470 * 2.0 + 1088 + 256) * 1024  # 4.297e9: K and V read once + split partials
 METRIC = "attn fwd TFLOP/s + % bf16 MFMA peak; decode KV GB/s + % HBM peak (1 GPU)"
 
