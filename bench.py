@@ -138,6 +138,20 @@ def cpu_baseline_prefill(D, S, slices, dtype):
     return causal_flops(1, slices, S, S, D) / dt / 1e12, dt
 
 
+def host_cpu():
+    """CPU model name and logical CPU count of the box the baseline runs on."""
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return "%s, %d logical CPUs" % (model, os.cpu_count() or 0)
+
+
 def cpu_baseline_decode(D, Skv, B, H, dtype):
     from oracle import oracle as O
     q, k, v = make_inputs(SEED0 + 3, B, H, H, 1, Skv, D, dtype)
@@ -214,8 +228,8 @@ def main():
                 "value": val, "unit": "TFLOP/s", "cores": threads, "kind": "port",
                 "sample": "%d of 128 (b,h) slices of config 3 (S=4096, D=128, explicit 0/-inf causal mask), oracle's "
                           "materialising restatement of the reference CPU op (not the Rust binary): matmuls and "
-                          "reductions on 1 thread, elementwise maps on %d OpenMP threads; %.1f s; same causal FLOP count"
-                          % (slices, threads, dt)}
+                          "reductions on 1 thread, elementwise maps on %d OpenMP threads; %.1f s; same causal FLOP count; host: %s"
+                          % (slices, threads, dt, host_cpu())}
 
     if args.only in (None, "decode"):
         B, H, Skv, D = 32, 32, 8192, 128
@@ -236,7 +250,7 @@ def main():
             val, dt = cpu_baseline_decode(D, Skv, 32, 32, capi.BF16)
             dec["cpu_baseline"] = {"value": val, "unit": "GB/s", "cores": threads, "kind": "port",
                                    "sample": "all of config 4 (B=32, H=32, KV=8192, D=128), oracle's materialising restatement of "
-                                             "the reference CPU op (serial matmuls and reductions); %.1f s" % dt}
+                                             "the reference CPU op (serial matmuls and reductions); %.1f s; host: %s" % (dt, host_cpu())}
         result["decode"] = dec
 
     print(json.dumps(result))
