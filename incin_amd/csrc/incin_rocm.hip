@@ -15,6 +15,7 @@
 namespace incin_rocm {
 hipError_t launch_sdpa_generic(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_sdpa_prefill_mfma(const SdpaParams& p, int dtype, hipStream_t stream);
+hipError_t launch_sdpa_prefill_mfma64(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_sdpa_decode(const SdpaParams& p, int dtype, hipStream_t stream);
 int decode_keys_per_tile(int dtype, int D, int R);
 hipError_t launch_copy16(void* dst, const void* src, size_t bytes, hipStream_t stream);
@@ -109,7 +110,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         return fail(INCIN_ROCM_ESHAPE, "scaled_dot_product_attention: batch and head counts are limited to 65535 per launch");
     if (!d->q || !d->o || (d->Skv > 0 && (!d->k || !d->v)))
         return fail(INCIN_ROCM_EINVAL, "scaled_dot_product_attention: null tensor pointer");
-    if (d->impl < INCIN_ROCM_IMPL_AUTO || d->impl > INCIN_ROCM_IMPL_SPLITKV)
+    if (d->impl < INCIN_ROCM_IMPL_AUTO || d->impl > INCIN_ROCM_IMPL_MFMA64)
         return fail(INCIN_ROCM_EINVAL, "scaled_dot_product_attention: unknown impl %d", d->impl);
     if (d->num_splits < 0) return fail(INCIN_ROCM_EINVAL, "scaled_dot_product_attention: negative num_splits");
 
@@ -120,6 +121,8 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     // the MFMA kernel addresses a K/V tile with 32-bit byte offsets from the tile's first row
     const bool tile_off_ok = d->k_stride[2] >= 0 && d->v_stride[2] >= 0 && d->k_stride[2] < (1 << 24) && d->v_stride[2] < (1 << 24);
     const bool mfma_ok = fast_ok && tile_off_ok && d->dtype != INCIN_ROCM_F32 && d->scale > 0.0f && std::isfinite(d->scale);
+    // the 64-row kernel keeps a tile's remaining byte count in 32 bits
+    const bool mfma64_ok = mfma_ok && d->D == 128 && d->Skv * d->k_stride[2] * 2 < (1LL << 31) && d->Skv * d->v_stride[2] * 2 < (1LL << 31);
     const bool split_ok = fast_ok && d->Sq <= 64;
 
     int impl = d->impl;
@@ -132,6 +135,9 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     if (impl == INCIN_ROCM_IMPL_MFMA && !mfma_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
                     "scaled_dot_product_attention: the MFMA kernel needs f16/bf16, D == Dv in {64,128}, scale > 0, no dense mask and 16-byte aligned rows");
+    if (impl == INCIN_ROCM_IMPL_MFMA64 && !mfma64_ok)
+        return fail(INCIN_ROCM_EUNSUPPORTED,
+                    "scaled_dot_product_attention: the 64-row MFMA kernel needs what the MFMA kernel needs, D == Dv == 128 and key/value slices below 2 GiB");
     if (impl == INCIN_ROCM_IMPL_SPLITKV && !split_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
                     "scaled_dot_product_attention: the split-KV kernel needs D == Dv in {64,128}, Sq <= 64, no dense mask and 16-byte aligned rows");
@@ -404,6 +410,7 @@ int incin_rocm_sdpa_fwd(const incin_rocm_sdpa_desc_t* desc, void* stream)
     hipError_t e;
     switch (plan.impl) {
         case INCIN_ROCM_IMPL_MFMA: e = incin_rocm::launch_sdpa_prefill_mfma(p, desc->dtype, s); break;
+        case INCIN_ROCM_IMPL_MFMA64: e = incin_rocm::launch_sdpa_prefill_mfma64(p, desc->dtype, s); break;
         case INCIN_ROCM_IMPL_SPLITKV: e = incin_rocm::launch_sdpa_decode(p, desc->dtype, s); break;
         default: e = incin_rocm::launch_sdpa_generic(p, desc->dtype, s); break;
     }

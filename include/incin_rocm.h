@@ -46,7 +46,8 @@ enum {
     INCIN_ROCM_IMPL_AUTO = 0,
     INCIN_ROCM_IMPL_GENERIC = 1,   /* fp32-FMA tiled kernel: any dtype, D and Dv <= 256, dense masks     */
     INCIN_ROCM_IMPL_MFMA = 2,      /* bf16/f16 MFMA prefill kernel: D == Dv in {64,128}                    */
-    INCIN_ROCM_IMPL_SPLITKV = 3    /* split-KV decode kernel + combine: D == Dv in {64,128}, few query rows */
+    INCIN_ROCM_IMPL_SPLITKV = 3,   /* split-KV decode kernel + combine: D == Dv in {64,128}, few query rows */
+    INCIN_ROCM_IMPL_MFMA64 = 4     /* bf16/f16 MFMA prefill kernel, 64 query rows per wavefront: D == Dv == 128 */
 };
 
 /* Thread-local message of the last failing call on this thread ("" if none).
