@@ -49,6 +49,9 @@ SC0, SC1 = 62, 64                # s[62:63], s[64:65]: lane masks in the rescali
 LDSW = 53                        # LDS byte address of this wavefront's first 1 KiB piece of K ring slot 0
 M0SAVE = 56
 KREM, VREM = 57, 58              # signed bytes from the next tile's first row to the end of the tensor slice
+DRAWADDR = 66                    # s[66:67] address of the work counter this workgroup draws its items from
+DRAWAT = 68                      # draw the next item when this many tiles are left (never reached: no draw from this wavefront)
+DRAWN, DRAWONE = 192, 193        # AGPRs: the counter's answer (lane 0) and the constant 1 it is advanced by
 # ---- AGPR map ---------------------------------------------------------------------------------------------
 def O(db, qb):                   # O^T accumulators
     return (db * QB + qb) * 16
@@ -225,6 +228,28 @@ def rescale(par):
     return L
 
 
+def prologue():
+    """State of a new work item: the K operands of tile 0 on their way from LDS, Q^T moved from the registers it
+    arrives in (the score registers, free until the first product) to its AGPRs, O^T, row sums, reference maxima
+    zero, no reference maximum set."""
+    L = []
+    for s_ in range(NSTEP):
+        L.append("ds_read_b128 %s, %s" % (v(KB + 4 * s_, 4), v(KADDR + s_)))
+    for i in range(QB * NSTEP * 4):
+        L.append("v_accvgpr_write_b32 a%d, v%d" % (Q(0, 0) + i, i))
+    for i in range(NDB * QB * 16):
+        L.append("v_accvgpr_write_b32 a%d, 0" % i)
+    for qb in range(QB):
+        for i in range(16):
+            L.append("v_mov_b32 %s, 0" % v(NR[qb] + i))
+    for qb in range(QB):
+        L.append("v_mov_b32 %s, %s" % (v(MX[qb]), v(NEGINF)))
+        L.append("v_mov_b32 %s, %s" % (v(THR[qb]), v(NEGINF)))
+        L.append("v_mov_b32 %s, 0" % v(MREF[qb]))
+        L.append("v_mov_b32 %s, 0" % v(LRUN[qb]))
+    return L
+
+
 def first_scores(ty):
     """Scores of tile 0 from the K operands in KB (nothing to overlap with yet); K operands of tile 1 behind them."""
     mfma = "v_mfma_f32_32x32x16_%s" % ty
@@ -245,11 +270,24 @@ def first_scores(ty):
     return L
 
 
+def draw(slot):
+    """Out of line, once per work item and workgroup: lane 0 advances the work counter.  The answer is not waited
+    for here; it is one more (older) entry in the queue the turns count, which only makes their wait safer."""
+    return [".Ldraw%d_%%=:" % slot,
+            "s_mov_b64 s[%d:%d], exec" % (SC0, SC0 + 1),
+            "s_mov_b64 exec, 1",
+            "v_mov_b32 %s, 0" % v(E),
+            "global_atomic_add a%d, %s, a%d, s[%d:%d] sc0" % (DRAWN, v(E), DRAWONE, DRAWADDR, DRAWADDR + 1),
+            "s_mov_b64 exec, s[%d:%d]" % (SC0, SC0 + 1),
+            "s_branch .Ldrawn%d_%%=" % slot]
+
+
 def loop(ty):
-    """The whole main path of a wavefront: tiles 0 .. LEFT-1.  Entry: T = 0, the K operands of tile 0 in KB, O^T and
-    the row sums zero, MREF 0, THR -inf, NR 0, REL for tile 0, the copies of K(0..7), V(0..5) started (K(0..3), V(0),
-    V(1) complete).  Exit: T = LEFT tiles done; if T is even its turn has NOT been taken."""
+    """The whole main path of a wavefront: tiles 0 .. LEFT-1.  Entry: T = 0, Q^T (scaled) in v0..v63, REL for tile 0,
+    the copies of K(0..7), V(0..5) started (K(0..3), V(0), V(1) complete and visible).  Exit: T = LEFT tiles done (if
+    T is even its turn has NOT been taken), O^T in its AGPRs, the row sums in LRUN."""
     L = ["s_mov_b32 s%d, m0" % M0SAVE]
+    L += prologue()
     L += first_scores(ty)
     L += ["s_branch .Lresc0_%="]                        # the first reference maximum
     for slot in range(RING):
@@ -259,12 +297,15 @@ def loop(ty):
             L += [".Lpre%d_%%=:" % slot]
         L += [".Lslot%d_%%=:" % slot]
         L += block(slot, ty) + ["s_add_i32 s%d, s%d, 1" % (T, T), "s_sub_i32 s%d, s%d, 1" % (LEFT, LEFT)]
+        L += ["s_cmp_eq_u32 s%d, s%d" % (LEFT, DRAWAT), "s_cbranch_scc1 .Ldraw%d_%%=" % slot, ".Ldrawn%d_%%=:" % slot]
         L += check(1 - slot % 2)
         L += ["s_cmp_eq_u32 s%d, 0" % LEFT, "s_cbranch_scc1 .Lexit_%="]
     L += [".Lpre0_%=:"] + turn(0)
     L += ["s_branch .Lslot0_%="]
     L += rescale(0)
     L += rescale(1)
+    for slot in range(RING):
+        L += draw(slot)
     L += [".Lexit_%=:", "s_mov_b32 m0, s%d" % M0SAVE, "s_nop 15"]
     return L
 
@@ -281,30 +322,25 @@ def main():
                       ("KB", KB), ("KADDR", KADDR), ("VADDR", VADDR), ("MX0", MX[0]), ("MX1", MX[1]),
                       ("LRUN0", LRUN[0]), ("LRUN1", LRUN[1])):
         out.append("#define PF_R_%s %d" % (name, val))
-    clob = list(range(P, P + 16)) + list(range(VB, VB + 32)) + list(range(E, E + 4)) + TT
+    clob = (list(range(NR[0], NR[0] + 16)) + list(range(NR[1], NR[1] + 16)) + list(range(P, P + 16)) + list(range(KB, KB + 32)) +
+            list(range(VB, VB + 32)) + list(range(E, E + 4)) + MX + THR + MREF + TT)
+    aclob = list(range(Q(0, 0), Q(0, 0) + QB * NSTEP * 4))
     # operand lists of the asm statement; the kernel source declares variables with these names
     outs = []
-    for par in range(2):
-        for qb in range(QB):
-            outs.append('"+{%s}"(sacc[%d][%d])' % (v(S[par][qb], 16), par, qb))
-    for s_ in range(NSTEP):
-        outs.append('"+{%s}"(kb[%d])' % (v(KB + 4 * s_, 4), s_))
     for qb in range(QB):
-        outs.append('"+{%s}"(mx[%d])' % (v(MX[qb]), qb))
+        for s_ in range(NSTEP):            # Q^T arrives in the score registers, which the loop then overwrites
+            outs.append('"+{%s}"(qreg[%d][%d])' % (v((qb * NSTEP + s_) * 4, 4), qb, s_))
     for qb in range(QB):
-        outs.append('"+{%s}"(l_run[%d])' % (v(LRUN[qb]), qb))
+        outs.append('"={%s}"(l_run[%d])' % (v(LRUN[qb]), qb))
     for db in range(NDB):
         for qb in range(QB):
-            outs.append('"+{%s}"(o_acc[%d][%d])' % (a_(O(db, qb), 16), db, qb))
+            outs.append('"={%s}"(o_acc[%d][%d])' % (a_(O(db, qb), 16), db, qb))
     ins = []
     for s_ in range(NSTEP):
         ins.append('"{%s}"(k_addr[%d])' % (v(KADDR + s_), s_))
     for db in range(NDB):
         for h in range(2):
             ins.append('"{%s}"(v_addr[%d][%d])' % (v(VADDR + 2 * db + h), db, h))
-    for qb in range(QB):
-        for s_ in range(NSTEP):
-            ins.append('"{%s}"(qreg[%d][%d])' % (a_(Q(qb, s_), 4), qb, s_))
     for c in range(2):
         ins.append('"{%s}"(k_voff[%d])' % (v(KVOFF[c]), c))
     for c in range(2):
@@ -312,12 +348,6 @@ def main():
     for qb in range(QB):
         outs.append('"+{%s}"(hot_rel[%d])' % (v(REL[qb]), qb))
     ins.append('"{%s}"(hot_neg_inf)' % v(NEGINF))
-    for qb in range(QB):
-        outs.append('"+{%s}"(hot_thr[%d])' % (v(THR[qb]), qb))
-    for qb in range(QB):
-        outs.append('"+{%s}"(hot_mref[%d])' % (v(MREF[qb]), qb))
-    for qb in range(QB):
-        outs.append('"+{%s}"(neg_ref[%d])' % (v(NR[qb], 16), qb))
     # scalar state of the loop
     outs.append('"+{s[%d:%d]}"(hot_kdesc)' % (KDESC, KDESC + 3))
     outs.append('"+{s[%d:%d]}"(hot_vdesc)' % (VDESC, VDESC + 3))
@@ -329,7 +359,11 @@ def main():
     ins.append('"{s%d}"(hot_vstep)' % VSTEP)
     ins.append('"{s%d}"(hot_ldsw)' % LDSW)
     ins.append('"{s%d}"(hot_nhot)' % NHOT)
-    clob_all = ['"v%d"' % r for r in clob] + ['"s%d"' % r for r in (M0SAVE, TMP, SC0, SC0 + 1, SC1, SC1 + 1)] + ['"vcc"', '"scc"', '"memory"']
+    ins.append('"{s[%d:%d]}"(hot_drawaddr)' % (DRAWADDR, DRAWADDR + 1))
+    ins.append('"{s%d}"(hot_drawat)' % DRAWAT)
+    ins.append('"{a%d}"(hot_one)' % DRAWONE)
+    outs.append('"+{a%d}"(drawn)' % DRAWN)
+    clob_all = ['"v%d"' % r for r in clob] + ['"a%d"' % r for r in aclob] + ['"s%d"' % r for r in (M0SAVE, TMP, SC0, SC0 + 1, SC1, SC1 + 1)] + ['"vcc"', '"scc"', '"memory"']
     out.append("#define PF_HOT_OPERANDS \\")
     out.append("    : %s \\" % ", ".join(outs))
     out.append("    : %s \\" % ", ".join(ins))

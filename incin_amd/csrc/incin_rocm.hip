@@ -121,13 +121,17 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     // the MFMA kernel addresses a K/V tile with 32-bit byte offsets from the tile's first row
     const bool tile_off_ok = d->k_stride[2] >= 0 && d->v_stride[2] >= 0 && d->k_stride[2] < (1 << 24) && d->v_stride[2] < (1 << 24);
     const bool mfma_ok = fast_ok && tile_off_ok && d->dtype != INCIN_ROCM_F32 && d->scale > 0.0f && std::isfinite(d->scale);
-    // the 64-row kernel keeps a tile's remaining byte count in 32 bits
-    const bool mfma64_ok = mfma_ok && d->D == 128 && d->Skv * d->k_stride[2] * 2 < (1LL << 31) && d->Skv * d->v_stride[2] * 2 < (1LL << 31);
+    // the 64-row kernel does its byte arithmetic on a head's K and V in 32 bits, up to 16 tiles of 32 rows past the end
+    const bool mfma64_ok = mfma_ok && d->D == 128 && (d->Skv + 512) * d->k_stride[2] * 2 < (1LL << 31) &&
+                           (d->Skv + 512) * d->v_stride[2] * 2 < (1LL << 31);
     const bool split_ok = fast_ok && d->Sq <= 64;
 
     int impl = d->impl;
     if (impl == INCIN_ROCM_IMPL_AUTO) {
         if (split_ok && R <= 8 && d->Skv >= 256) impl = INCIN_ROCM_IMPL_SPLITKV;
+        // long sequences with work for every compute unit twice over: the 64-row kernel's halved LDS traffic outweighs
+        // what it pays per 256-row work item (measured crossover: a few thousand keys)
+        else if (mfma64_ok && d->Skv >= 8192 && d->B * d->Hq * ((d->Sq + 255) / 256) >= 512) impl = INCIN_ROCM_IMPL_MFMA64;
         else if (mfma_ok) impl = INCIN_ROCM_IMPL_MFMA;
         else if (split_ok && R <= 8) impl = INCIN_ROCM_IMPL_SPLITKV;
         else impl = INCIN_ROCM_IMPL_GENERIC;

@@ -65,6 +65,18 @@ def test_dispatch_choices():
     nbytes, splits, impl = _plan(_desc(Sq=1, Skv=8192, B=1, Hq=8, Hkv=2, num_splits=4))
     assert impl == capi.IMPL_SPLITKV and splits == 4 and nbytes == 8 * 4 * 130 * 4
     assert _plan(_desc(Sq=1, Skv=64))[2] in (capi.IMPL_MFMA, capi.IMPL_SPLITKV)
+    # long sequences with at least 512 work items of 256 query rows: the 64-row kernel (head dimension 128 only)
+    def long(**kw):
+        S = kw.pop("S", 16384)
+        d = _desc(B=4, Hq=32, Hkv=8, Sq=S, Skv=S, **kw)
+        for name, heads in (("q_stride", 32), ("k_stride", 8), ("v_stride", 8), ("o_stride", 32)):
+            st = getattr(d, name)
+            st[0], st[1], st[2] = heads * S * d.D, S * d.D, d.D
+        return d
+    assert _plan(long())[2] == capi.IMPL_MFMA64
+    assert _plan(long(S=4096))[2] == capi.IMPL_MFMA
+    assert _plan(long(D=64, Dv=64))[2] == capi.IMPL_MFMA
+    assert _plan(_desc(Sq=8192, Skv=8192))[2] == capi.IMPL_MFMA          # 2 x 4 heads x 32 blocks: too few items
     # empty problems need nothing
     assert _plan(_desc(Sq=0))[0] == 0
 
