@@ -191,6 +191,7 @@ void fill_params(const incin_rocm_sdpa_desc_t* d, const Plan& plan, SdpaParams* 
     p->Sq = (int)d->Sq; p->Skv = (int)d->Skv; p->D = (int)d->D; p->Dv = (int)d->Dv;
     p->scale = d->scale;
     p->causal = d->causal ? 1 : 0;
+    p->interleave = 1;
     p->num_splits = plan.splits;
     p->split_len = plan.split_len;
     p->ws_acc = (float*)d->workspace;

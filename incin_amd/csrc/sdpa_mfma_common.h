@@ -2,6 +2,8 @@
 // instruction wrappers, the LDS tile layout (chunk-slot swizzle) and the
 // lane <-> lane^32 exchanges.
 #pragma once
+#include <atomic>
+
 #include "sdpa_params.h"
 
 namespace incin_rocm {
@@ -70,6 +72,53 @@ template <int D> struct PfLayout {
         return ((r >> 1) & 1) << 2;
     }
 };
+
+// CU count of the current device (256 if the query fails: only launch geometry depends on it).
+inline int device_cus()
+{
+    static std::atomic<int> cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
+
+// ---- order of the work list ------------------------------------------------------------------------------------
+// A work item is (batch, KV head, query head of its group, block of query rows).  The list runs over groups of F
+// (batch, KV head) pairs; inside a group the query blocks go longest-first (under a causal mask the last block sees
+// the most keys), and for each block all F * G heads of the group follow one another.  With F * G * (blocks per head)
+// a multiple of the workgroups an XCD runs at a time, every round of workgroups gets items of equal length, which
+// list scheduling in plain head order does not give (it ends each head on its shortest blocks while the next head's
+// longest start, and the last round is left ragged: about 9 % at 4096 x 4096 causal).  F is kept small: F KV heads
+// are in an XCD's L2 at a time.
+struct WorkItem { int bhkv, gq, qblk; };
+__device__ __forceinline__ WorkItem work_item(int vid, int F, int G, int nqb)
+{
+    const int per_group = F * G * nqb;
+    const int grp = vid / per_group, r = vid - grp * per_group;
+    const int rank = r / (F * G), m = r - rank * (F * G);
+    WorkItem w;
+    w.bhkv = grp * F + m / G;
+    w.gq = m % G;
+    w.qblk = nqb - 1 - rank;
+    return w;
+}
+// F for a launch: `slots` workgroups run on an XCD at a time, a range of the list (the whole list, or an eighth of it
+// when it divides by 8 and each XCD takes one) holds `range_items` items.
+inline int work_interleave(bool causal, int slots, int G, int nqb, long long range_items)
+{
+    if (!causal || slots <= 0) return 1;
+    int a = slots, b = (G * nqb) % slots;
+    while (b) { const int t = a % b; a = b; b = t; }          // a = gcd(slots, G * nqb)
+    int f = slots / a;
+    if (f > 8) f = 8;
+    while (f > 1 && range_items % ((long long)f * G * nqb)) --f;
+    return f;
+}
 
 __device__ __forceinline__ float xor32_max(float x)
 {

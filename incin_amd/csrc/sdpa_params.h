@@ -22,6 +22,7 @@ struct SdpaParams {
     int32_t Sq, Skv, D, Dv;
     float scale;
     int32_t causal;
+    int32_t interleave;        // MFMA prefill kernels: (batch, KV head) pairs per group of the work list, set by their launchers
     // split-KV only
     int32_t num_splits;
     int32_t split_len;         // keys per split (multiple of the kernel's key tile)

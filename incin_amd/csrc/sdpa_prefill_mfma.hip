@@ -83,15 +83,13 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
 
     // ---- which (batch, head, query block) -----------------------------------
     // Workgroups reach the 8 XCDs round-robin by id; hand each XCD a contiguous
-    // range of the work list so heads that share K/V stay in one L2, and order
-    // each head's query blocks longest-first.
+    // range of the work list so heads that share K/V stay in one L2.
     const int nqb = (Sq + PF_BM - 1) / PF_BM;
     const int total = gridDim.x;
     int vid = blockIdx.x;
     if ((total & 7) == 0) vid = (blockIdx.x & 7) * (total >> 3) + (blockIdx.x >> 3);
-    const int gq = vid % p.G;
-    const int qb = nqb - 1 - (vid / p.G) % nqb;
-    const int bhkv = vid / (p.G * nqb);
+    const WorkItem wi = work_item(vid, p.interleave, p.G, nqb);
+    const int gq = wi.gq, qb = wi.qblk, bhkv = wi.bhkv;
     const int hkv = bhkv % p.Hkv, b = bhkv / p.Hkv;
     const int hq = hkv * p.G + gq;
     const int q0 = qb * PF_BM;
@@ -427,10 +425,13 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
 }
 
 template <typename T, int D>
-static hipError_t launch_prefill_t(const SdpaParams& p, hipStream_t stream)
+static hipError_t launch_prefill_t(const SdpaParams& p0, hipStream_t stream)
 {
+    SdpaParams p = p0;
     const int nqb = (p.Sq + PF_BM - 1) / PF_BM;
     const int64_t total = (int64_t)nqb * p.Hq * p.B;
+    // two workgroups per CU (register budget), an eighth of the CUs per XCD
+    p.interleave = work_interleave(p.causal != 0, 2 * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
     hipLaunchKernelGGL((sdpa_prefill_mfma_kernel<T, D>), dim3((unsigned)total), dim3(256), 0, stream, p);
     return hipGetLastError();
 }
