@@ -13,7 +13,7 @@ ITEMSIZE = {F32: 4, F16: 2, BF16: 2}
 
 
 def f32_to_bf16_bits(x):
-    x = np.ascontiguousarray(x, dtype=np.float32)
+    x = np.asarray(x, dtype=np.float32, order="C")
     u = x.view(np.uint32).astype(np.uint64)
     rounded = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
     nan = np.isnan(x)
@@ -23,7 +23,7 @@ def f32_to_bf16_bits(x):
 
 
 def bf16_bits_to_f32(b):
-    b = np.ascontiguousarray(b, dtype=np.uint16)
+    b = np.asarray(b, dtype=np.uint16, order="C")
     return (b.astype(np.uint32) << 16).view(np.float32).reshape(b.shape)
 
 
@@ -31,10 +31,10 @@ def encode(x, dtype):
     """f32 array -> array holding the storage encoding (f32, f16, or bf16 bits as uint16)."""
     x = np.asarray(x, dtype=np.float32)
     if dtype == F32:
-        return np.ascontiguousarray(x)
+        return np.asarray(x, order="C")
     if dtype == F16:
         with np.errstate(over="ignore"):
-            return np.ascontiguousarray(x.astype(np.float16))
+            return np.asarray(x.astype(np.float16), order="C")
     return f32_to_bf16_bits(x)
 
 

@@ -4,6 +4,7 @@
 #include <string>
 
 #include "rocm_backend.hpp"
+#include "rocm_capability.hpp"
 
 using namespace incin_rocm_host;
 
@@ -104,5 +105,80 @@ int incin_host_scaled_dot_product_attention(const incin_host_storage* q, const i
 void incin_host_release(incin_host_storage* s) { delete s; }
 
 int64_t incin_host_last_launch_count(void) { return incin_rocm_host::last_launch_count(); }
+
+
+// ---- capability registry ------------------------------------------------------------------------------------
+namespace cap = incin_rocm_host::capability;
+
+const char* incin_host_capability_name(int32_t what, int32_t value)
+{
+    switch (what) {
+        case 0: return cap::name((cap::OperationKind)value);
+        case 1: return cap::name((cap::DTypeId)value);
+        case 2: return cap::as_str((cap::LayoutClass)value);
+        case 3: return cap::as_str((cap::MathMode)value);
+        case 4: return cap::name((cap::ImplementationKind)value);
+        case 5: return value >= 0 && value <= 4 ? cap::name((cap::DeviceKind)value) : "?";
+        default: return "?";
+    }
+}
+
+int32_t incin_host_capability_max_rank(void) { return cap::MAX_RANK; }
+
+int incin_host_capability_support(int32_t device_kind, int32_t operation, int32_t dtype, int32_t layout, int32_t rank,
+                                  int32_t training, int32_t math_mode, int32_t* reason_kind, char* reason, size_t capacity)
+{
+    cap::CapabilityQuery q{(cap::OperationKind)operation, (cap::DTypeId)dtype, (cap::LayoutClass)layout, rank, training != 0,
+                           (cap::MathMode)math_mode};
+    const cap::SupportLevel lv = cap::support((cap::DeviceKind)device_kind, q);
+    if (!lv.is_supported()) {
+        if (reason_kind) *reason_kind = (int32_t)lv.reason.kind;
+        if (reason && capacity) {
+            const std::string text = lv.reason.to_string();
+            const size_t n = text.size() < capacity - 1 ? text.size() : capacity - 1;
+            std::memcpy(reason, text.data(), n);
+            reason[n] = 0;
+        }
+    }
+    return (int)lv.kind;
+}
+
+int32_t incin_host_capability_rule_count(int32_t device_kind)
+{
+    return (int32_t)cap::registry((cap::DeviceKind)device_kind).registrations().size();
+}
+
+int incin_host_capability_rule(int32_t device_kind, int32_t index, int32_t* operation, uint32_t* dtypes, uint32_t* layouts,
+                               int32_t* min_rank, int32_t* max_rank, int32_t* training, uint32_t* math_modes,
+                               int32_t* implementation)
+{
+    const std::vector<cap::CapabilityRule>& rules = cap::registry((cap::DeviceKind)device_kind).registrations();
+    if (index < 0 || (size_t)index >= rules.size()) return finish(Error{ErrorKind::Msg, "capability rule index out of range"});
+    const cap::CapabilityRule& r = rules[index];
+    *operation = (int32_t)r.operation;
+    *dtypes = *layouts = *math_modes = 0;
+    for (cap::DTypeId d : r.dtypes) *dtypes |= 1u << (int)d;
+    for (cap::LayoutClass l : r.layouts) *layouts |= 1u << (int)l;
+    for (cap::MathMode m : r.math_modes) *math_modes |= 1u << (int)m;
+    *min_rank = r.min_rank;
+    *max_rank = r.max_rank;
+    *training = r.training ? 1 : 0;
+    *implementation = (int32_t)r.implementation;
+    return 0;
+}
+
+size_t incin_host_capability_docs(char* out, size_t capacity)
+{
+    const std::string text = cap::summary({{cap::DeviceKind::Cpu, &cap::cpu_attention_capabilities()},
+                                           {cap::DeviceKind::Rocm, &cap::rocm_capabilities()}}) +
+                             cap::device_section(cap::DeviceKind::Cpu, cap::cpu_attention_capabilities()) +
+                             cap::device_section(cap::DeviceKind::Rocm, cap::rocm_capabilities());
+    if (out && capacity) {
+        const size_t n = text.size() < capacity - 1 ? text.size() : capacity - 1;
+        std::memcpy(out, text.data(), n);
+        out[n] = 0;
+    }
+    return text.size();
+}
 
 }  // extern "C"

@@ -33,6 +33,25 @@ void incin_host_release(incin_host_storage* s);
 /* number of kernel launches (C-ABI sdpa calls) the last attention call on this thread made */
 int64_t incin_host_last_launch_count(void);
 
+
+/* ---- capability registry (rocm_capability.hpp).  Enumerations travel as their integer values, in the order the
+ * header declares them.  device_kind: 0 cpu, 1 cuda, 2 wgpu, 3 metal, 4 rocm. ---- */
+/* spelling of an enumeration value; what: 0 operation, 1 dtype, 2 layout, 3 math mode, 4 implementation, 5 device */
+const char* incin_host_capability_name(int32_t what, int32_t value);
+int32_t incin_host_capability_max_rank(void);
+/* support level of a query: 0 native, 1 composed, 2 fallback, 3 unsupported.  For 3, *reason_kind gets the
+ * UnsupportedReason variant (0 operation, 1 dtype, 2 layout, 3 rank, 4 training, 5 math mode) and `reason` its text. */
+int incin_host_capability_support(int32_t device_kind, int32_t operation, int32_t dtype, int32_t layout, int32_t rank,
+                                  int32_t training, int32_t math_mode, int32_t* reason_kind, char* reason, size_t capacity);
+int32_t incin_host_capability_rule_count(int32_t device_kind);
+/* one registration; dtypes / layouts / math_modes come back as bit masks over the enumeration values */
+int incin_host_capability_rule(int32_t device_kind, int32_t index, int32_t* operation, uint32_t* dtypes, uint32_t* layouts,
+                               int32_t* min_rank, int32_t* max_rank, int32_t* training, uint32_t* math_modes,
+                               int32_t* implementation);
+/* the generated tables for the rows this backend adds (summary over cpu and rocm, then both sections); returns the
+ * length of the text, of which at most capacity - 1 bytes are written */
+size_t incin_host_capability_docs(char* out, size_t capacity);
+
 #ifdef __cplusplus
 }
 #endif

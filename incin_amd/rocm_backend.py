@@ -25,6 +25,8 @@ EXPORTS = [
     "incin_host_dtype", "incin_host_to_bytes", "incin_host_transpose", "incin_host_broadcast_as",
     "incin_host_narrow", "incin_host_tag_causal", "incin_host_tag_key_padding",
     "incin_host_scaled_dot_product_attention", "incin_host_release", "incin_host_last_launch_count",
+    "incin_host_capability_name", "incin_host_capability_max_rank", "incin_host_capability_support",
+    "incin_host_capability_rule_count", "incin_host_capability_rule", "incin_host_capability_docs",
 ]
 
 
@@ -62,6 +64,17 @@ def lib():
         L.incin_host_tag_key_padding.argtypes = [C.c_void_p, C.POINTER(C.c_int32), C.c_int64, C.POINTER(C.c_void_p)]
         L.incin_host_scaled_dot_product_attention.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32,
                                                               C.c_double, C.POINTER(C.c_void_p)]
+        L.incin_host_capability_name.restype = C.c_char_p
+        L.incin_host_capability_name.argtypes = [C.c_int32, C.c_int32]
+        L.incin_host_capability_max_rank.restype = C.c_int32
+        L.incin_host_capability_support.argtypes = [C.c_int32] * 7 + [C.POINTER(C.c_int32), C.c_char_p, C.c_size_t]
+        L.incin_host_capability_rule_count.restype = C.c_int32
+        L.incin_host_capability_rule_count.argtypes = [C.c_int32]
+        L.incin_host_capability_rule.argtypes = [C.c_int32, C.c_int32, C.POINTER(C.c_int32), C.POINTER(C.c_uint32),
+                                                 C.POINTER(C.c_uint32), C.POINTER(C.c_int32), C.POINTER(C.c_int32),
+                                                 C.POINTER(C.c_int32), C.POINTER(C.c_uint32), C.POINTER(C.c_int32)]
+        L.incin_host_capability_docs.restype = C.c_size_t
+        L.incin_host_capability_docs.argtypes = [C.c_char_p, C.c_size_t]
         _lib = L
     return _lib
 
@@ -90,7 +103,7 @@ class RocmStorage:
     @classmethod
     def from_numpy(cls, a, dtype=F32, device=0):
         """`a` holds float values; they are stored on the device as `dtype` (round-to-nearest-even)."""
-        a = np.ascontiguousarray(a)
+        a = np.asarray(a, order="C")          # (ascontiguousarray would turn a rank-0 array into rank 1)
         if dtype == F32:
             raw = a.astype(np.float32).tobytes()
         elif dtype == F16:
@@ -99,7 +112,7 @@ class RocmStorage:
             raw = DT.f32_to_bf16_bits(a.astype(np.float32)).tobytes()
         else:
             raw = a.tobytes()
-        return cls.from_bytes(raw, a.shape, dtype, device)
+        return cls.from_bytes(raw, tuple(a.shape), dtype, device)
 
     @classmethod
     def from_bytes(cls, raw, dims, dtype, device=0):

@@ -1,0 +1,115 @@
+"""Executes what the rocm capability table advertises, the way the reference's capability_matrix suite executes the
+boundary cases of its CPU rules (crates/incin-backends/tests/capability_matrix.rs:222-330): every dtype x layout x
+{min rank, max rank} of every rule runs on the device and matches the CPU oracle / the host data, and cells the
+registry refuses are refused by the operator too, with the error kind the refusal names."""
+import sys
+
+import numpy as np
+import pytest
+
+from incin_amd import dtypes
+from incin_amd import rocm_backend as RB
+from incin_amd import rocm_capability as RC
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+CODE = {"f32": RB.F32, "f16": RB.F16, "bf16": RB.BF16}
+TOL = {"f32": 1e-5, "f16": 2e-2, "bf16": 2e-2}
+RULES = {r.operation: r for r in RC.registrations("rocm")}
+
+
+def say(msg):
+    print(msg, file=sys.stderr, flush=True)
+
+
+def rnd(seed, shape, dtype):
+    r = np.random.Generator(np.random.PCG64(seed))
+    return dtypes.round_to(r.standard_normal(shape, dtype=np.float32), CODE[dtype])
+
+
+def operand(a, dtype, layout):
+    """Storage holding `a` in the given layout class: dense, or a view with dense rows carved out of a larger
+    allocation (narrow along the row axis and, with batch axes, a transpose of two of them)."""
+    if layout == "contiguous":
+        return RB.RocmStorage.from_numpy(a, CODE[dtype])
+    assert layout == "row-wise"
+    if a.ndim >= 4:        # store with the first two batch axes swapped and 2 spare rows, view it back
+        big = np.zeros(a.shape[:-2] + (a.shape[-2] + 2, a.shape[-1]), np.float32)
+        big[..., 1:-1, :] = a
+        s = RB.RocmStorage.from_numpy(np.ascontiguousarray(np.swapaxes(big, 0, 1)), CODE[dtype])
+        s = s.transpose(0, 1)
+    else:
+        big = np.zeros(a.shape[:-2] + (a.shape[-2] + 2, a.shape[-1]), np.float32)
+        big[..., 1:-1, :] = a
+        s = RB.RocmStorage.from_numpy(big, CODE[dtype])
+    s = s.narrow(a.ndim - 2, 1, a.shape[-2])
+    assert s.shape == a.shape and np.array_equal(s.to_numpy(), a)
+    return s
+
+
+def shapes_of_rank(rank):
+    """q, k, v shapes of that rank: rank 2 is one head; rank 8 has four leading axes the host loops over or folds."""
+    if rank == 2:
+        return (9, 32), (13, 32), (13, 32)
+    lead = (1, 2, 1, 2)[: rank - 4] if rank > 4 else ()
+    core = {3: ((3,), (3,)), 4: ((2, 3), (2, 3))}.get(rank, ((2, 2), (2, 2)))
+    q = lead + core[0] + (17, 64)
+    k = lead + core[1] + (29, 64)
+    return q, k, k
+
+
+@pytest.mark.parametrize("dtype", RULES["attention"].dtypes)
+@pytest.mark.parametrize("layout", RULES["attention"].layouts)
+@pytest.mark.parametrize("rank", [RULES["attention"].min_rank, RULES["attention"].max_rank])
+def test_attention_rule_boundary_cases_execute(gpu, dtype, layout, rank):
+    case = RC.CapabilityQuery("attention", dtype, layout, rank)
+    assert RC.support("rocm", case).level == "native"
+    qs, ks, vs = shapes_of_rank(rank)
+    say("capability cell %s: q%s k%s" % (case, qs, ks))
+    q, k, v = rnd(1, qs, dtype), rnd(2, ks, dtype), rnd(3, vs, dtype)
+    out = RB.scaled_dot_product_attention(operand(q, dtype, layout), operand(k, dtype, layout), operand(v, dtype, layout))
+    ref = O.sdpa(q, k, v)
+    assert out.shape == ref.shape
+    err = float(np.abs(out.to_numpy() - ref).max())
+    say("   max-abs err %.3e" % err)
+    assert err <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", RULES["storage"].dtypes)
+@pytest.mark.parametrize("rank", [RULES["storage"].min_rank, RULES["storage"].max_rank])
+def test_storage_and_broadcast_rules_execute(gpu, dtype, rank):
+    say("capability cells storage / broadcast %s rank %d" % (dtype, rank))
+    shape = (2, 1, 2, 1, 3, 1, 2, 5)[8 - rank:] if rank else ()
+    a = rnd(4, shape, dtype)
+    s = RB.RocmStorage.from_numpy(a, CODE[dtype])
+    assert s.shape == shape and np.array_equal(s.to_numpy(), a)                  # storage, contiguous
+    if rank >= 2:
+        t = s.transpose(rank - 1, rank - 2)                                       # storage family, strided view
+        assert np.array_equal(t.to_numpy(), np.swapaxes(a, -1, -2))
+        wide = tuple(3 if d == 1 else d for d in shape)
+        assert np.array_equal(s.broadcast_as(wide).to_numpy(), np.broadcast_to(a, wide))     # broadcast
+    else:
+        assert np.array_equal(s.broadcast_as((2, 3)).to_numpy(), np.broadcast_to(a, (2, 3)))
+
+
+def test_refused_cells_are_refused_by_the_operator_too(gpu):
+    say("capability cells the registry refuses")
+    q = rnd(5, (2, 8, 16), "f32")
+    s = RB.RocmStorage.from_numpy(q)
+    # layout `strided` (last axis not dense): the registry says Layout, the operator UnsupportedBackendOperation
+    assert RC.support("rocm", RC.CapabilityQuery("attention", "f32", "strided", 3)).reason == "Layout"
+    with pytest.raises(RB.BackendError) as e:
+        t = RB.RocmStorage.from_numpy(np.ascontiguousarray(np.swapaxes(q, -1, -2))).transpose(1, 2)
+        RB.scaled_dot_product_attention(t, s, s)
+    assert e.value.kind == "UnsupportedBackendOperation"
+    # rank 1: registry says Rank, operator ShapeMismatch
+    assert RC.support("rocm", RC.CapabilityQuery("attention", "f32", "contiguous", 1)).reason == "Rank"
+    with pytest.raises(RB.BackendError) as e:
+        v1 = RB.RocmStorage.from_numpy(np.ones(16, np.float32))
+        RB.scaled_dot_product_attention(v1, v1, v1)
+    assert e.value.kind == "ShapeMismatch"
+    # a dtype the storage rule does not list cannot be created
+    assert RC.support("rocm", RC.CapabilityQuery("storage", "f64", "contiguous", 1)).reason == "DType"
+    with pytest.raises(RB.BackendError) as e:
+        RB.RocmStorage.from_bytes(b"\0" * 16, (2,), 3)
+    assert e.value.kind == "UnsupportedDType"
