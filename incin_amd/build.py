@@ -16,7 +16,7 @@ SOURCES = ["incin_rocm.hip", "sdpa_generic.hip", "sdpa_decode.hip", "sdpa_prefil
 EXTRA_FLAGS = {}    # per-file flags
 HOST_DIR = os.path.join(HERE, "host")
 HOST_LIB = os.path.join(LIBDIR, "libincin_rocm_host.so")
-HOST_SOURCES = ["rocm_backend.cpp", "rocm_capability.cpp", "rocm_backend_c.cpp"]
+HOST_SOURCES = ["rocm_backend.cpp", "rocm_capability.cpp", "rocm_exec.cpp", "rocm_conformance.cpp", "rocm_backend_c.cpp"]
 CXX = os.environ.get("CXX", "g++")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -packed-fp32-ops off: the compiler must not form packed-fp32 VALU instructions from float code.

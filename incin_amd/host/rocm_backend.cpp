@@ -199,6 +199,38 @@ Error RocmBackend::narrow(const RocmStorage& s, int dim, int64_t start, int64_t 
     return ok();
 }
 
+Error RocmBackend::reshape(const RocmStorage& s, const std::vector<int64_t>& dims, RocmStorage* out)
+{
+    int64_t n = 1;
+    for (int64_t d : dims) {
+        if (d < 0) return err(ErrorKind::ShapeMismatch, "reshape: negative extent in " + shape_str(dims));
+        n *= d;
+    }
+    if (n != s.numel())
+        return err(ErrorKind::ShapeMismatch, "reshape: " + shape_str(s.shape) + " has " + std::to_string(s.numel()) +
+                                                 " elements, " + shape_str(dims) + " has " + std::to_string(n));
+    if (!s.is_contiguous())
+        return err(ErrorKind::UnsupportedBackendOperation, "reshape: only contiguous storage can be re-addressed on backend Rocm");
+    *out = s;
+    out->shape = dims;
+    out->strides.assign(dims.size(), 1);
+    for (int i = (int)dims.size() - 2; i >= 0; --i) out->strides[i] = out->strides[i + 1] * dims[i + 1];
+    out->mask_tag.reset();
+    return ok();
+}
+
+Error RocmBackend::upload_i32(const std::vector<int32_t>& values, int32_t device, std::shared_ptr<RocmBuffer>* out)
+{
+    void* p = nullptr;
+    const size_t bytes = values.size() * sizeof(int32_t);
+    if (Error e = from_status(incin_rocm_alloc(device, bytes ? bytes : 4, &p), device)) return e;
+    auto buf = std::make_shared<RocmBuffer>(device, p, bytes);
+    if (bytes)
+        if (Error e = from_status(incin_rocm_memcpy_h2d(device, p, values.data(), bytes), device)) return e;
+    *out = std::move(buf);
+    return ok();
+}
+
 Error RocmBackend::tag_causal(const RocmStorage& mask, RocmStorage* out)
 {
     if (mask.shape.size() < 2) return err(ErrorKind::ShapeMismatch, "a causal mask has at least two axes");
@@ -220,6 +252,12 @@ Error RocmBackend::tag_key_padding(const RocmStorage& mask, const std::vector<in
 
 Error RocmBackend::scaled_dot_product_attention(const RocmStorage& q, const RocmStorage& k, const RocmStorage& v,
                                                 const RocmStorage* mask, std::optional<double> scale, RocmStorage* out)
+{
+    return attention(q, k, v, mask, scale, MaskFacts{}, out);
+}
+
+Error RocmBackend::attention(const RocmStorage& q, const RocmStorage& k, const RocmStorage& v, const RocmStorage* mask,
+                             std::optional<double> scale, const MaskFacts& facts, RocmStorage* out)
 {
     static const char* OP = "scaled_dot_product_attention";
     // -- devices and dtypes, in the order the reference's checks fire ------------------------------------
@@ -345,6 +383,15 @@ Error RocmBackend::scaled_dot_product_attention(const RocmStorage& q, const Rocm
         }
     } else if (dense_mask) {
         d.mask_stride[0] = st(ms, b_ax); d.mask_stride[1] = st(ms, head_ax); d.mask_stride[2] = m_si; d.mask_stride[3] = m_sj;
+    }
+
+    // facts stated by the caller's descriptor rather than by a mask storage; they combine with either kind of mask
+    if (facts.causal) d.causal = 1;
+    if (facts.kv_lens) {
+        if (d.kv_lens) return err(ErrorKind::ShapeMismatch, std::string(OP) + ": key lengths given twice (descriptor and mask tag)");
+        if (facts.kv_lens_count != B || n_outer != 0 || (g_ax >= 0 && !fold_g))
+            return err(ErrorKind::ShapeMismatch, std::string(OP) + ": key-padding lengths must have one entry per batch index");
+        d.kv_lens = static_cast<const int32_t*>(facts.kv_lens->ptr());
     }
 
     const size_t isz = dtype_size(q.dtype);

@@ -98,6 +98,21 @@ struct RocmBackend {
     // TensorOps::scaled_dot_product_attention.
     static Error scaled_dot_product_attention(const RocmStorage& q, const RocmStorage& k, const RocmStorage& v,
                                               const RocmStorage* mask, std::optional<double> scale, RocmStorage* out);
+
+    // The same operator with what a descriptor states about masking (rocm_exec.hpp) instead of, or on top of, a mask
+    // storage: causal alignment and per-batch key counts; both may hold at once.
+    struct MaskFacts {
+        bool causal = false;
+        std::shared_ptr<RocmBuffer> kv_lens;      // int32 key counts on the device, one per batch entry
+        int64_t kv_lens_count = 0;
+    };
+    static Error attention(const RocmStorage& q, const RocmStorage& k, const RocmStorage& v, const RocmStorage* mask,
+                           std::optional<double> scale, const MaskFacts& facts, RocmStorage* out);
+
+    // Reinterpret a contiguous storage under another shape of the same element count (metadata only).
+    static Error reshape(const RocmStorage& s, const std::vector<int64_t>& dims, RocmStorage* out);
+    // int32 values on the device (key counts of a descriptor).
+    static Error upload_i32(const std::vector<int32_t>& values, int32_t device, std::shared_ptr<RocmBuffer>* out);
 };
 
 // NumPy-style right-aligned broadcast of two shapes (cpu/stride.rs:86-106).

@@ -5,11 +5,16 @@
 
 #include "rocm_backend.hpp"
 #include "rocm_capability.hpp"
+#include "rocm_conformance.hpp"
+#include "rocm_exec.hpp"
 
 using namespace incin_rocm_host;
 
 struct incin_host_storage {
     RocmStorage s;
+};
+struct incin_host_attention_spec {
+    AttentionSpec spec;
 };
 
 namespace {
@@ -179,6 +184,80 @@ size_t incin_host_capability_docs(char* out, size_t capacity)
         out[n] = 0;
     }
     return text.size();
+}
+
+
+// ---- descriptors, conformance, detection ----------------------------------------------------------------------
+int incin_host_lower_attention(const int64_t* q_dims, int32_t q_rank, const int64_t* k_dims, int32_t k_rank, const int64_t* v_dims,
+                               int32_t v_rank, int32_t dtype, int32_t causal, const int32_t* kv_lens, int64_t kv_lens_count,
+                               int32_t has_scale, double scale, incin_host_attention_spec** out)
+{
+    std::optional<std::vector<int32_t>> lens;
+    if (kv_lens_count >= 0) lens = std::vector<int32_t>(kv_lens, kv_lens + kv_lens_count);
+    AttentionSpec spec;
+    Error e = lower_attention(std::vector<int64_t>(q_dims, q_dims + q_rank), std::vector<int64_t>(k_dims, k_dims + k_rank),
+                              std::vector<int64_t>(v_dims, v_dims + v_rank), (DType)dtype, causal != 0, lens,
+                              has_scale ? std::optional<double>(scale) : std::nullopt, &spec);
+    if (!e) *out = new incin_host_attention_spec{std::move(spec)};
+    return finish(e);
+}
+
+int incin_host_attention_spec_out_dims(const incin_host_attention_spec* spec, int64_t* dims_out, int32_t* rank_out, int64_t* group_out)
+{
+    for (size_t i = 0; i < spec->spec.out_dims.size(); ++i) dims_out[i] = spec->spec.out_dims[i];
+    *rank_out = (int32_t)spec->spec.out_dims.size();
+    if (group_out) *group_out = spec->spec.group;
+    return 0;
+}
+
+int incin_host_execute_attention(const incin_host_attention_spec* spec, const incin_host_storage* const* inputs, int32_t n_inputs,
+                                 incin_host_storage** out)
+{
+    std::vector<const RocmStorage*> in;
+    for (int32_t i = 0; i < n_inputs; ++i) in.push_back(&inputs[i]->s);
+    RocmStorage o;
+    Error e = execute(spec->spec, in, &o);
+    return give(e, std::move(o), out);
+}
+
+void incin_host_release_attention_spec(incin_host_attention_spec* spec) { delete spec; }
+
+int incin_host_reshape(const incin_host_storage* s, const int64_t* dims, int32_t rank, incin_host_storage** out)
+{
+    RocmStorage o;
+    Error e = RocmBackend::reshape(s->s, std::vector<int64_t>(dims, dims + rank), &o);
+    return give(e, std::move(o), out);
+}
+
+size_t incin_host_conformance_run(int32_t device, char* text, size_t capacity, int32_t* passed, int32_t* skipped, int32_t* failed)
+{
+    const conformance::Report r = conformance::run(device);
+    if (passed) *passed = r.count(conformance::Check::Outcome::Passed);
+    if (skipped) *skipped = r.count(conformance::Check::Outcome::Skipped);
+    if (failed) *failed = r.count(conformance::Check::Outcome::Failed);
+    const std::string t = r.to_text();
+    if (text && capacity) {
+        const size_t n = t.size() < capacity - 1 ? t.size() : capacity - 1;
+        std::memcpy(text, t.data(), n);
+        text[n] = 0;
+    }
+    return t.size();
+}
+
+int32_t incin_host_is_compiled_in(int32_t kind) { return is_compiled_in(kind) ? 1 : 0; }
+
+int32_t incin_host_probe(int32_t kind)
+{
+    const std::optional<DeviceId> d = probe(kind);
+    return d ? d->ordinal : -1;
+}
+
+int incin_host_detect_device(const int32_t* pref, int32_t n, int32_t* kind, int32_t* ordinal)
+{
+    const DeviceId d = detect_device_in(n < 0 ? preference() : std::vector<int32_t>(pref, pref + n));
+    *kind = d.kind;
+    *ordinal = d.ordinal;
+    return 0;
 }
 
 }  // extern "C"

@@ -52,6 +52,29 @@ int incin_host_capability_rule(int32_t device_kind, int32_t index, int32_t* oper
  * length of the text, of which at most capacity - 1 bytes are written */
 size_t incin_host_capability_docs(char* out, size_t capacity);
 
+
+/* ---- validated descriptors and their executor (rocm_exec.hpp) ---- */
+typedef struct incin_host_attention_spec incin_host_attention_spec;
+/* the shape rule; kv_lens_count < 0: no key counts; has_scale = 0: default 1/sqrt(D).  Needs no device. */
+int incin_host_lower_attention(const int64_t* q_dims, int32_t q_rank, const int64_t* k_dims, int32_t k_rank, const int64_t* v_dims,
+                               int32_t v_rank, int32_t dtype, int32_t causal, const int32_t* kv_lens, int64_t kv_lens_count,
+                               int32_t has_scale, double scale, incin_host_attention_spec** out);
+int incin_host_attention_spec_out_dims(const incin_host_attention_spec* spec, int64_t* dims_out, int32_t* rank_out, int64_t* group_out);
+int incin_host_execute_attention(const incin_host_attention_spec* spec, const incin_host_storage* const* inputs, int32_t n_inputs,
+                                 incin_host_storage** out);
+void incin_host_release_attention_spec(incin_host_attention_spec* spec);
+int incin_host_reshape(const incin_host_storage* s, const int64_t* dims, int32_t rank, incin_host_storage** out);
+
+/* ---- conformance suite (rocm_conformance.hpp): the report text (at most capacity - 1 bytes written, full length
+ * returned) and how many checks passed, were skipped, failed ---- */
+size_t incin_host_conformance_run(int32_t device, char* text, size_t capacity, int32_t* passed, int32_t* skipped, int32_t* failed);
+
+/* ---- device detection (rocm_exec.hpp); kinds as for the capability registry ---- */
+int32_t incin_host_is_compiled_in(int32_t kind);
+int32_t incin_host_probe(int32_t kind);                    /* device ordinal, or -1 */
+/* n < 0: the default preference order (cuda, rocm, metal, wgpu, cpu) */
+int incin_host_detect_device(const int32_t* preference, int32_t n, int32_t* kind, int32_t* ordinal);
+
 #ifdef __cplusplus
 }
 #endif

@@ -157,8 +157,11 @@ const std::vector<CapabilityRule>& rocm_capabilities()
     static const std::vector<CapabilityRule> rules = {
         // from_bytes / to_bytes: to_bytes gathers any view, from_bytes creates contiguous storage
         {OperationKind::Storage, ROCM_DTYPES, ANY_VIEW, 0, MAX_RANK, false, PRECISE, ImplementationKind::Native},
-        // metadata-only views: transpose / narrow answer through the `storage` family, broadcast_as here
+        // metadata-only views: transpose / narrow answer through the `storage` family, broadcast_as and reshape by rules of
+        // their own
         {OperationKind::Broadcast, ROCM_DTYPES, ANY_VIEW, 0, MAX_RANK, false, PRECISE, ImplementationKind::Native},
+        // reshape re-addresses contiguous storage; a view has to be materialised by the caller first
+        {OperationKind::Reshape, ROCM_DTYPES, {LayoutClass::Contiguous}, 0, MAX_RANK, false, PRECISE, ImplementationKind::Native},
         // scaled_dot_product_attention, forward only
         {OperationKind::Attention, ROCM_DTYPES, ROW_VIEWS, 2, MAX_RANK, false, PRECISE, ImplementationKind::Native},
     };

@@ -71,13 +71,17 @@ def test_unsupported_cells_return_the_documented_constraint():
 
 
 def test_operations_without_rules_of_their_own_resolve_through_their_family():
-    # transpose / narrow (slice) / reshape are metadata operations: family `storage`
+    # transpose / narrow (slice) and the like are metadata operations: family `storage`
     # (incin-core/src/shapes/error.rs:112-124), answered by the storage rule
-    for op in ("transpose", "slice", "reshape", "permute", "squeeze"):
+    for op in ("transpose", "slice", "permute", "squeeze"):
         assert RC.support("rocm", Q(op, "bf16", "strided", 5)).level == "native"
         assert RC.support("rocm", Q(op, "i64", "contiguous", 5)).reason == "DType"
-    # broadcast has a rule of its own, which then is the only one consulted
+    # broadcast and reshape have rules of their own, which then are the only ones consulted: reshape re-addresses
+    # contiguous storage only
     assert RC.support("rocm", Q("broadcast", "f16", "row-wise", 8)).level == "native"
+    assert RC.support("rocm", Q("reshape", "f16", "contiguous", 8)).level == "native"
+    s = RC.support("rocm", Q("reshape", "f16", "strided", 3))
+    assert (s.reason, s.message) == ("Layout", "layout strided is unsupported for reshape")
 
 
 @pytest.mark.parametrize("device", ["cuda", "wgpu", "metal"])
