@@ -56,14 +56,17 @@ def causal_flops(B, Hq, Sq, Skv, D):
 class Workload:
     """Device-resident operands + descriptor for one configuration."""
 
-    def __init__(self, name, seed, B, Hq, Hkv, Sq, Skv, D, dtype, causal):
+    def __init__(self, name, seed, B, Hq, Hkv, Sq, Skv, D, dtype, causal, kv_lens=None, pad_queries=False):
         self.name, self.shape = name, (B, Hq, Hkv, Sq, Skv, D)
-        self.dtype, self.causal = dtype, causal
+        self.dtype, self.causal, self.kv_lens = dtype, causal, kv_lens
         q, k, v = make_inputs(seed, B, Hq, Hkv, Sq, Skv, D, dtype)
         self.host = (q, k, v)
         self.tq, self.tk, self.tv = (host.DeviceTensor.from_f32(x, dtype) for x in (q, k, v))
         self.to = host.DeviceTensor((B, Hq, Sq, D), dtype)
-        self.desc = host.make_desc(self.tq, self.tk, self.tv, self.to, causal=causal)
+        self.tl = capi.DeviceBuffer.from_numpy(np.asarray(kv_lens, dtype=np.int32)) if kv_lens is not None else None
+        # a padded self-attention batch: the same lengths say which keys and which query rows are padding
+        self.desc = host.make_desc(self.tq, self.tk, self.tv, self.to, causal=causal, kv_lens=self.tl,
+                                   q_lens=self.tl if pad_queries else None)
         nbytes, self.splits, self.impl = capi.sdpa_workspace(self.desc)
         self.ws = capi.DeviceBuffer(nbytes) if nbytes else None
         if self.ws is not None:
@@ -115,12 +118,17 @@ class Workload:
         rows = np.stack([r.integers(0, B * Hq, n_rows), r.integers(0, Sq, n_rows)], axis=1)
         rows[0] = (0, 0)
         rows[1] = (B * Hq - 1, Sq - 1)
-        ref = O.sdpa_rows(q.reshape(B, Hkv, G, Sq, D), k[:, :, None], v[:, :, None], rows, causal=self.causal)
+        lens = None
+        if self.kv_lens is not None:       # sample inside each sequence's valid length (rows past it are padding queries)
+            lens = np.asarray(self.kv_lens, dtype=np.int32)
+            rows[:, 1] %= lens[rows[:, 0] // Hq]
+            lens = lens.reshape(B, 1, 1)
+        ref = O.sdpa_rows(q.reshape(B, Hkv, G, Sq, D), k[:, :, None], v[:, :, None], rows, causal=self.causal, kv_lens=lens)
         got = out.reshape(B * Hq, Sq, D)[rows[:, 0], rows[:, 1]]
         return float(np.abs(got - ref).max())
 
     def free(self):
-        for t in (self.tq.buf, self.tk.buf, self.tv.buf, self.to.buf, self.ws):
+        for t in (self.tq.buf, self.tk.buf, self.tv.buf, self.to.buf, self.ws, self.tl):
             if t is not None:
                 t.free()
 
@@ -168,7 +176,7 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["prefill", "decode", "copy"], default=None,
+    ap.add_argument("--only", choices=["prefill", "prefill_long", "decode", "copy"], default=None,
                     help="run a single workload (profiling). 'copy' runs --steps device-to-device copies of 1 GiB "
                          "through the library's plain copy kernel: the known-size dispatch that hardware byte "
                          "counters (FETCH_SIZE / WRITE_SIZE) are calibrated against")
@@ -230,6 +238,36 @@ def main():
                           "materialising restatement of the reference CPU op (not the Rust binary): matmuls and "
                           "reductions on 1 thread, elementwise maps on %d OpenMP threads; %.1f s; same causal FLOP count; host: %s"
                           % (slices, threads, dt, host_cpu())}
+
+    if args.only in (None, "prefill_long"):
+        # BASELINE config 5: grouped queries, 16384-token padded batch, causal + key padding; lengths U[2048, 16384]
+        # from the same seeded generator, one sequence at full length
+        B, Hq, Hkv, S, D = 4, 32, 8, 16384, 128
+        lens = rng(SEED0 + 4).integers(2048, S + 1, B).astype(np.int64)
+        lens[0] = S
+        w = Workload("prefill_c5", SEED0 + 4, B, Hq, Hkv, S, S, D, capi.BF16, True, kv_lens=lens, pad_queries=True)
+        steps = max(5, min(args.steps, 20))                 # ~5 ms per launch
+        wall, ev_mean, ev_med, ev_min = w.time(steps, min(args.warmup, 5))
+        # the same batch with the padding rows computed (what a caller gets who can only hand over a key mask)
+        w.desc.q_lens = None
+        wall_all_rows = w.time(steps, 2)[0]
+        w.desc.q_lens = w.tl.ptr
+        w.launch()
+        capi.sync()
+        flops = 4.0 * D * Hq * float(sum(int(n) * (int(n) + 1) // 2 for n in lens))      # rows i < lens[b] only
+        kernel = {capi.IMPL_MFMA64: "sdpa_prefill_mfma64_kernel<bf16>", capi.IMPL_MFMA: "sdpa_prefill_mfma_kernel<bf16,128>"}.get(w.impl, str(w.impl))
+        result["prefill_long"] = {
+            "workload": "BASELINE config 5: bf16 GQA causal prefill B=4 Hq=32 Hkv=8 S=16384 (padded) D=128, key padding with "
+                        "lengths %s given as kv_lens and q_lens (padding rows not computed); FLOPs count rows and keys inside "
+                        "each length only" % lens.tolist(),
+            "metric": "attn fwd TFLOP/s", "value": flops / (wall * 1e-3) / 1e12, "unit": "TFLOP/s", "ms_per_step": wall, "steps": steps,
+            "roofline": {"bound": "mfma", "achieved": flops / (ev_mean * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                         "frac": flops / (ev_mean * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": None, "kernel": kernel,
+                         "algorithmic_flops_per_launch": flops, "launch_ms_mean": ev_mean, "launch_ms_median": ev_med,
+                         "launch_ms_min": ev_min},
+            "ms_per_step_with_padding_rows_computed": wall_all_rows,
+            "parity_max_abs_err": w.parity(16)}
+        w.free()
 
     if args.only in (None, "decode"):
         B, H, Skv, D = 32, 32, 8192, 128

@@ -65,6 +65,7 @@ class SdpaDesc(C.Structure):
         ("workspace_bytes", C.c_size_t),
         ("num_splits", C.c_int32),
         ("impl", C.c_int32),
+        ("q_lens", C.c_void_p),
     ]
 
 

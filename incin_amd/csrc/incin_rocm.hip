@@ -182,6 +182,7 @@ void fill_params(const incin_rocm_sdpa_desc_t* d, const Plan& plan, SdpaParams* 
     p->q = d->q; p->k = d->k; p->v = d->v; p->o = d->o;
     p->mask = d->add_mask;
     p->kv_lens = d->kv_lens;
+    p->q_lens = d->q_lens;
     p->q_sb = d->q_stride[0]; p->q_sh = d->q_stride[1]; p->q_ss = d->q_stride[2];
     p->k_sb = d->k_stride[0]; p->k_sh = d->k_stride[1]; p->k_ss = d->k_stride[2];
     p->v_sb = d->v_stride[0]; p->v_sh = d->v_stride[1]; p->v_ss = d->v_stride[2];
@@ -192,6 +193,7 @@ void fill_params(const incin_rocm_sdpa_desc_t* d, const Plan& plan, SdpaParams* 
     p->scale = d->scale;
     p->causal = d->causal ? 1 : 0;
     p->interleave = 1;
+    p->deal_groups = 0;
     p->num_splits = plan.splits;
     p->split_len = plan.split_len;
     p->ws_acc = (float*)d->workspace;

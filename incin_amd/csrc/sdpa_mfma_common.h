@@ -107,6 +107,22 @@ __device__ __forceinline__ WorkItem work_item(int vid, int F, int G, int nqb)
     w.qblk = nqb - 1 - rank;
     return w;
 }
+// Which entry of the work list is item `item` of XCD `xcd`'s share (a share holds share_len items).  Shares are
+// dealt group by group (group g goes to XCD g % 8) when the groups divide evenly: batch entries of different
+// lengths then spread over all XCDs instead of one long sequence filling the shares of two of them.  Otherwise
+// a share is a contiguous eighth of the list.
+__device__ __forceinline__ int work_vid(int xcd, int item, int share_len, int F, int G, int nqb, int deal_groups)
+{
+    if (!deal_groups) return xcd * share_len + item;
+    const int per_group = F * G * nqb;
+    const int g_local = item / per_group;
+    return (g_local * 8 + xcd) * per_group + (item - g_local * per_group);
+}
+inline int work_deal_groups(int F, int G, int nqb, long long share_items)
+{
+    return share_items % ((long long)F * G * nqb) == 0 ? 1 : 0;
+}
+
 // F for a launch: `slots` workgroups run on an XCD at a time, a range of the list (the whole list, or an eighth of it
 // when it divides by 8 and each XCD takes one) holds `range_items` items.
 inline int work_interleave(bool causal, int slots, int G, int nqb, long long range_items)

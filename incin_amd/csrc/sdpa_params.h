@@ -13,6 +13,7 @@ struct SdpaParams {
     void* o;
     const void* mask;          // nullable dense additive mask (same dtype as q)
     const int32_t* kv_lens;    // nullable, B entries
+    const int32_t* q_lens;     // nullable, B entries: query rows at and beyond are padding (output unspecified)
     int64_t q_sb, q_sh, q_ss;
     int64_t k_sb, k_sh, k_ss;
     int64_t v_sb, v_sh, v_ss;
@@ -23,6 +24,7 @@ struct SdpaParams {
     float scale;
     int32_t causal;
     int32_t interleave;        // MFMA prefill kernels: (batch, KV head) pairs per group of the work list, set by their launchers
+    int32_t deal_groups;       // MFMA prefill kernels: groups of the work list are dealt to the 8 XCDs in turn (else: contiguous eighths)
     // split-KV only
     int32_t num_splits;
     int32_t split_len;         // keys per split (multiple of the kernel's key tile)

@@ -87,7 +87,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     const int nqb = (Sq + PF_BM - 1) / PF_BM;
     const int total = gridDim.x;
     int vid = blockIdx.x;
-    if ((total & 7) == 0) vid = (blockIdx.x & 7) * (total >> 3) + (blockIdx.x >> 3);
+    if ((total & 7) == 0) vid = work_vid(blockIdx.x & 7, blockIdx.x >> 3, total >> 3, p.interleave, p.G, nqb, p.deal_groups);
     const WorkItem wi = work_item(vid, p.interleave, p.G, nqb);
     const int gq = wi.gq, qb = wi.qblk, bhkv = wi.bhkv;
     const int hkv = bhkv % p.Hkv, b = bhkv / p.Hkv;
@@ -101,18 +101,22 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
 
     int kv_len = Skv;
     if (p.kv_lens) kv_len = clampi(p.kv_lens[b], 0, Skv);
+    // query rows at and beyond rows_b are padding: nothing is computed or stored for them
+    const int rows_b = p.q_lens ? clampi(p.q_lens[b], 0, Sq) : Sq;
+    if (q0 >= rows_b) return;                          // the whole block is padding (uniform: before any barrier)
     const int coff = Skv - Sq;
     // keys visible to this workgroup / this wavefront / this lane's query
     int j_end = kv_len;
     const int my_i = q0 + wave * 32 + ql;
     int lim_lane = kv_len, lim_wave_min = kv_len, lim_wave_max = kv_len;
     if (p.causal) {
-        const int last_row = min(q0 + PF_BM - 1, Sq - 1);
+        const int last_row = min(q0 + PF_BM - 1, rows_b - 1);
         j_end = clampi(last_row + coff + 1, 0, kv_len);
         lim_lane = clampi(my_i + coff + 1, 0, kv_len);
         lim_wave_min = clampi(q0 + wave * 32 + coff + 1, 0, kv_len);
-        lim_wave_max = clampi(min(q0 + wave * 32 + 31, Sq - 1) + coff + 1, 0, kv_len);
+        lim_wave_max = clampi(min(q0 + wave * 32 + 31, rows_b - 1) + coff + 1, 0, kv_len);
     }
+    if (q0 + wave * 32 >= rows_b) lim_wave_min = lim_wave_max = 0;      // a wavefront of padding rows only keeps the barriers company
     const int n_tiles = (j_end + PF_BN - 1) / PF_BN;
 
     // ---- global -> LDS copy plan ---------------------------------------------------
@@ -408,7 +412,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     // ---- normalise and store ------------------------------------------------------------------
     const float l_tot = xor32_sum(l_run);
     const float inv = (l_tot == 0.0f) ? __builtin_nanf("") : 1.0f / l_tot;   // no visible key: NaN, as the reference
-    if (my_i < Sq) {
+    if (my_i < rows_b) {
         T* orow = op + (int64_t)my_i * p.o_ss;
 #pragma unroll
         for (int db = 0; db < NDB; ++db)
@@ -432,6 +436,7 @@ static hipError_t launch_prefill_t(const SdpaParams& p0, hipStream_t stream)
     const int64_t total = (int64_t)nqb * p.Hq * p.B;
     // two workgroups per CU (register budget), an eighth of the CUs per XCD
     p.interleave = work_interleave(p.causal != 0, 2 * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
+    p.deal_groups = (total & 7) == 0 ? work_deal_groups(p.interleave, p.G, nqb, total >> 3) : 0;
     hipLaunchKernelGGL((sdpa_prefill_mfma_kernel<T, D>), dim3((unsigned)total), dim3(256), 0, stream, p);
     return hipGetLastError();
 }

@@ -48,7 +48,7 @@ def resolve_scale(scale, d):
 
 
 def make_desc(q, k, v, o, scale=None, causal=False, kv_lens=None, mask=None, mask_strides=None,
-              num_splits=0, impl=capi.IMPL_AUTO, workspace=None):
+              num_splits=0, impl=capi.IMPL_AUTO, workspace=None, q_lens=None):
     B, Hq, Sq, D = q.shape
     Bk, Hkv, Skv, Dk = k.shape
     Bv, Hv, Skv2, Dv = v.shape
@@ -63,6 +63,7 @@ def make_desc(q, k, v, o, scale=None, causal=False, kv_lens=None, mask=None, mas
     d.scale = resolve_scale(scale, D)
     d.causal = 1 if causal else 0
     d.kv_lens = kv_lens.ptr if kv_lens is not None else None
+    d.q_lens = q_lens.ptr if q_lens is not None else None
     if mask is not None:
         d.add_mask = mask.ptr
         for i in range(4):
@@ -88,7 +89,7 @@ def mask_strides_for(mask_shape, B, Hq, Sq, Skv):
 
 
 def sdpa(q, k, v, dtype=capi.F32, scale=None, causal=False, kv_lens=None, mask=None,
-         num_splits=0, impl=capi.IMPL_AUTO, dev=0, return_info=False):
+         num_splits=0, impl=capi.IMPL_AUTO, dev=0, return_info=False, q_lens=None):
     """Run attention on the GPU for f32 numpy operands [B,Hq,Sq,D], [B,Hkv,Skv,D], [B,Hkv,Skv,Dv].
 
     Operands are rounded to `dtype` on upload; the result is returned as f32
@@ -102,12 +103,13 @@ def sdpa(q, k, v, dtype=capi.F32, scale=None, causal=False, kv_lens=None, mask=N
     tq, tk, tv = (DeviceTensor.from_f32(x, dtype, dev) for x in (q, k, v))
     to = DeviceTensor((B, Hq, Sq, Dv), dtype, dev)
     tl = capi.DeviceBuffer.from_numpy(np.asarray(kv_lens, dtype=np.int32), dev) if kv_lens is not None else None
+    tql = capi.DeviceBuffer.from_numpy(np.asarray(q_lens, dtype=np.int32), dev) if q_lens is not None else None
     tm, ms = None, None
     if mask is not None:
         mask = np.asarray(mask, dtype=np.float32)
         ms = mask_strides_for(mask.shape, B, Hq, Sq, k.shape[2])
         tm = capi.DeviceBuffer.from_numpy(dtypes.encode(mask, dtype), dev)
-    d = make_desc(tq, tk, tv, to, scale, causal, tl, tm, ms, num_splits, impl)
+    d = make_desc(tq, tk, tv, to, scale, causal, tl, tm, ms, num_splits, impl, q_lens=tql)
     nbytes, splits, chosen = capi.sdpa_workspace(d)
     ws = capi.DeviceBuffer(nbytes, dev) if nbytes else None
     if ws is not None:
@@ -115,7 +117,7 @@ def sdpa(q, k, v, dtype=capi.F32, scale=None, causal=False, kv_lens=None, mask=N
     capi.sdpa_fwd(d)
     capi.sync(dev)
     out = to.to_f32()
-    for t in (tq.buf, tk.buf, tv.buf, to.buf, tl, tm, ws):
+    for t in (tq.buf, tk.buf, tv.buf, to.buf, tl, tm, ws, tql):
         if t is not None:
             t.free()
     if return_info:

@@ -393,6 +393,11 @@ Error RocmBackend::attention(const RocmStorage& q, const RocmStorage& k, const R
             return err(ErrorKind::ShapeMismatch, std::string(OP) + ": key-padding lengths must have one entry per batch index");
         d.kv_lens = static_cast<const int32_t*>(facts.kv_lens->ptr());
     }
+    if (facts.q_lens) {
+        if (facts.q_lens_count != B || n_outer != 0 || (g_ax >= 0 && !fold_g))
+            return err(ErrorKind::ShapeMismatch, std::string(OP) + ": query lengths must have one entry per batch index");
+        d.q_lens = static_cast<const int32_t*>(facts.q_lens->ptr());
+    }
 
     const size_t isz = dtype_size(q.dtype);
     // iterate the outer axes

@@ -105,6 +105,8 @@ struct RocmBackend {
         bool causal = false;
         std::shared_ptr<RocmBuffer> kv_lens;      // int32 key counts on the device, one per batch entry
         int64_t kv_lens_count = 0;
+        std::shared_ptr<RocmBuffer> q_lens;       // int32 query counts: rows at and beyond are padding, their output unspecified
+        int64_t q_lens_count = 0;
     };
     static Error attention(const RocmStorage& q, const RocmStorage& k, const RocmStorage& v, const RocmStorage* mask,
                            std::optional<double> scale, const MaskFacts& facts, RocmStorage* out);

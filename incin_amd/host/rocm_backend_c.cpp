@@ -190,14 +190,16 @@ size_t incin_host_capability_docs(char* out, size_t capacity)
 // ---- descriptors, conformance, detection ----------------------------------------------------------------------
 int incin_host_lower_attention(const int64_t* q_dims, int32_t q_rank, const int64_t* k_dims, int32_t k_rank, const int64_t* v_dims,
                                int32_t v_rank, int32_t dtype, int32_t causal, const int32_t* kv_lens, int64_t kv_lens_count,
-                               int32_t has_scale, double scale, incin_host_attention_spec** out)
+                               int32_t has_scale, double scale, const int32_t* q_lens, int64_t q_lens_count,
+                               incin_host_attention_spec** out)
 {
-    std::optional<std::vector<int32_t>> lens;
+    std::optional<std::vector<int32_t>> lens, qlens;
     if (kv_lens_count >= 0) lens = std::vector<int32_t>(kv_lens, kv_lens + kv_lens_count);
+    if (q_lens_count >= 0) qlens = std::vector<int32_t>(q_lens, q_lens + q_lens_count);
     AttentionSpec spec;
     Error e = lower_attention(std::vector<int64_t>(q_dims, q_dims + q_rank), std::vector<int64_t>(k_dims, k_dims + k_rank),
                               std::vector<int64_t>(v_dims, v_dims + v_rank), (DType)dtype, causal != 0, lens,
-                              has_scale ? std::optional<double>(scale) : std::nullopt, &spec);
+                              has_scale ? std::optional<double>(scale) : std::nullopt, &spec, qlens);
     if (!e) *out = new incin_host_attention_spec{std::move(spec)};
     return finish(e);
 }

@@ -55,10 +55,11 @@ size_t incin_host_capability_docs(char* out, size_t capacity);
 
 /* ---- validated descriptors and their executor (rocm_exec.hpp) ---- */
 typedef struct incin_host_attention_spec incin_host_attention_spec;
-/* the shape rule; kv_lens_count < 0: no key counts; has_scale = 0: default 1/sqrt(D).  Needs no device. */
+/* the shape rule; kv_lens_count / q_lens_count < 0: no such counts; has_scale = 0: default 1/sqrt(D).  Needs no device. */
 int incin_host_lower_attention(const int64_t* q_dims, int32_t q_rank, const int64_t* k_dims, int32_t k_rank, const int64_t* v_dims,
                                int32_t v_rank, int32_t dtype, int32_t causal, const int32_t* kv_lens, int64_t kv_lens_count,
-                               int32_t has_scale, double scale, incin_host_attention_spec** out);
+                               int32_t has_scale, double scale, const int32_t* q_lens, int64_t q_lens_count,
+                               incin_host_attention_spec** out);
 int incin_host_attention_spec_out_dims(const incin_host_attention_spec* spec, int64_t* dims_out, int32_t* rank_out, int64_t* group_out);
 int incin_host_execute_attention(const incin_host_attention_spec* spec, const incin_host_storage* const* inputs, int32_t n_inputs,
                                  incin_host_storage** out);

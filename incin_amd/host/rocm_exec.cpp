@@ -19,7 +19,7 @@ const char* OP = "scaled_dot_product_attention";
 
 Error lower_attention(const std::vector<int64_t>& q, const std::vector<int64_t>& k, const std::vector<int64_t>& v, DType dtype,
                       bool causal, const std::optional<std::vector<int32_t>>& kv_lens, std::optional<double> scale,
-                      AttentionSpec* out)
+                      AttentionSpec* out, const std::optional<std::vector<int32_t>>& q_lens)
 {
     if (q.size() < 2 || k.size() < 2 || v.size() < 2)
         return bad(std::string(OP) + ": operands need rank >= 2; got q " + dims_str(q) + ", k " + dims_str(k) + ", v " + dims_str(v));
@@ -43,20 +43,25 @@ Error lower_attention(const std::vector<int64_t>& q, const std::vector<int64_t>&
     if (!b.empty() && qb.size() == b.size() && kb.size() == b.size() && vb.size() == b.size() && qb.back() > 1 && kb.back() == 1 &&
         vb.back() == 1 && b.size() >= 2)
         s.group = qb.back();
-    if (kv_lens) {
+    for (int which = 0; which < 2; ++which) {
+        const std::optional<std::vector<int32_t>>& lens = which ? q_lens : kv_lens;
+        const int64_t limit = which ? Sq : Skv;
+        const char* what = which ? "query" : "key";
+        if (!lens) continue;
         // one count per index of the batch axis: none below rank 4 (one set of sequences), the first axis at rank 4, the
         // axis before [kv heads] or [kv heads, group] above
         const int nb = (int)b.size();
         const int b_ax = nb <= 1 ? -1 : nb == 2 ? 0 : (s.group > 1 ? nb - 3 : nb - 2);      // a single batch axis counts heads
         const int64_t B = b_ax >= 0 ? b[b_ax] : 1;
-        if ((int64_t)kv_lens->size() != B)
-            return bad(std::string(OP) + ": " + std::to_string(kv_lens->size()) + " key counts for a batch axis of " + std::to_string(B));
-        for (int32_t n : *kv_lens)
-            if (n < 0 || n > Skv) return bad(std::string(OP) + ": key count " + std::to_string(n) + " outside 0..=" + std::to_string(Skv));
+        if ((int64_t)lens->size() != B)
+            return bad(std::string(OP) + ": " + std::to_string(lens->size()) + " " + what + " counts for a batch axis of " + std::to_string(B));
+        for (int32_t n : *lens)
+            if (n < 0 || n > limit) return bad(std::string(OP) + ": " + what + " count " + std::to_string(n) + " outside 0..=" + std::to_string(limit));
     }
     if (scale && !(*scale == *scale)) return Error{ErrorKind::Msg, std::string(OP) + ": scale is NaN"};
     s.causal = causal;
     s.kv_lens = kv_lens;
+    s.q_lens = q_lens;
     s.scale = scale;
     s.dtype = dtype;
     *out = std::move(s);
@@ -93,12 +98,16 @@ Error execute(const AttentionSpec& spec, const std::vector<const RocmStorage*>& 
         if (Error e = RocmBackend::upload_i32(*spec.kv_lens, q.device, &facts.kv_lens)) return e;
         facts.kv_lens_count = (int64_t)spec.kv_lens->size();
     }
+    if (spec.q_lens) {
+        if (Error e = RocmBackend::upload_i32(*spec.q_lens, q.device, &facts.q_lens)) return e;
+        facts.q_lens_count = (int64_t)spec.q_lens->size();
+    }
     RocmStorage o;
     if (Error e = RocmBackend::attention(q, k, v, nullptr, spec.scale, facts, &o)) return e;
     if (o.shape != spec.out_dims)
         return Error{ErrorKind::Msg, std::string(OP) + ": produced " + dims_str(o.shape) + ", the descriptor proves " + dims_str(spec.out_dims)};
     // the key counts are read by work that is only stream-ordered: finish before they are released
-    if (facts.kv_lens)
+    if (facts.kv_lens || facts.q_lens)
         if (incin_rocm_sync(q.device) != 0) return Error{ErrorKind::Msg, std::string("ROCm sync failed: ") + incin_rocm_last_error()};
     *out = std::move(o);
     return ok();

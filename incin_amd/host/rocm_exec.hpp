@@ -19,6 +19,7 @@ struct AttentionSpec {
     int64_t group = 1;                                // query heads per key/value head (last batch axis of q over 1 of k, v)
     bool causal = false;                              // query i sees keys j <= i + Skv - Sq
     std::optional<std::vector<int32_t>> kv_lens;      // keys j >= kv_lens[b] masked; one entry per index of the batch axis
+    std::optional<std::vector<int32_t>> q_lens;       // query rows i >= q_lens[b] are padding: output rows unspecified
     std::optional<double> scale;                      // None: 1/sqrt(D)
     DType dtype = DType::F32;
 };
@@ -30,7 +31,7 @@ struct ReshapeSpec {
 // Shape rules.  Errors are ShapeMismatch with the operation's name, as the reference's rules report them.
 Error lower_attention(const std::vector<int64_t>& q_dims, const std::vector<int64_t>& k_dims, const std::vector<int64_t>& v_dims,
                       DType dtype, bool causal, const std::optional<std::vector<int32_t>>& kv_lens, std::optional<double> scale,
-                      AttentionSpec* out);
+                      AttentionSpec* out, const std::optional<std::vector<int32_t>>& q_lens = std::nullopt);
 Error lower_reshape(const std::vector<int64_t>& in_dims, const std::vector<int64_t>& out_dims, ReshapeSpec* out);
 
 // Executors: inputs are borrowed storages, the output is a new storage (attention) or a view (reshape).

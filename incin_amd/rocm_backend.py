@@ -80,7 +80,7 @@ def lib():
         L.incin_host_capability_docs.argtypes = [C.c_char_p, C.c_size_t]
         I64P, I32P = C.POINTER(C.c_int64), C.POINTER(C.c_int32)
         L.incin_host_lower_attention.argtypes = [I64P, C.c_int32, I64P, C.c_int32, I64P, C.c_int32, C.c_int32, C.c_int32, I32P,
-                                                 C.c_int64, C.c_int32, C.c_double, C.POINTER(C.c_void_p)]
+                                                 C.c_int64, C.c_int32, C.c_double, I32P, C.c_int64, C.POINTER(C.c_void_p)]
         L.incin_host_attention_spec_out_dims.argtypes = [C.c_void_p, I64P, I32P, I64P]
         L.incin_host_execute_attention.argtypes = [C.c_void_p, C.POINTER(C.c_void_p), C.c_int32, C.POINTER(C.c_void_p)]
         L.incin_host_release_attention_spec.restype = None

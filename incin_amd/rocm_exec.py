@@ -19,13 +19,15 @@ class AttentionSpec:
             self._h = None
 
     @classmethod
-    def lower(cls, q_dims, k_dims, v_dims, dtype=RB.F32, causal=False, kv_lens=None, scale=None):
+    def lower(cls, q_dims, k_dims, v_dims, dtype=RB.F32, causal=False, kv_lens=None, scale=None, q_lens=None):
         out = C.c_void_p()
         lens = None if kv_lens is None else (C.c_int32 * max(len(kv_lens), 1))(*[int(x) for x in kv_lens])
+        qlens = None if q_lens is None else (C.c_int32 * max(len(q_lens), 1))(*[int(x) for x in q_lens])
         RB._check(RB.lib().incin_host_lower_attention(
             RB._dims(q_dims), len(q_dims), RB._dims(k_dims), len(k_dims), RB._dims(v_dims), len(v_dims), dtype,
             1 if causal else 0, lens, -1 if kv_lens is None else len(kv_lens),
-            0 if scale is None else 1, 0.0 if scale is None else float(scale), C.byref(out)))
+            0 if scale is None else 1, 0.0 if scale is None else float(scale), qlens,
+            -1 if q_lens is None else len(q_lens), C.byref(out)))
         return cls(out.value)
 
     def _out(self):

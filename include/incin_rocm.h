@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define INCIN_ROCM_ABI_VERSION 1
+#define INCIN_ROCM_ABI_VERSION 2
 
 /* ---- status codes (mapped to incin_core::Error variants by the Rust side;
  *      crates/incin-core/src/err.rs:109-223) --------------------------------- */
@@ -129,6 +129,11 @@ int incin_rocm_event_elapsed_ms(int32_t dev, void* start, void* stop, float* out
  * j >= kv_lens[b].  All three may be combined.  A query row with every key
  * masked yields NaN, as the reference's softmax does (-inf - -inf).
  *
+ * Padded batches.  `q_lens` has no counterpart in the reference's operator (a mask tensor can hide keys, not
+ * say that a query row is padding): when given, query rows i >= q_lens[b] are declared padding, their output
+ * rows are unspecified (a kernel may skip them or compute them), and a caller that pads both sides of a
+ * self-attention batch passes the same lengths here and in `kv_lens`.  Rows below the length are unaffected.
+ *
  * Output dtype equals the input dtype; accumulation is f32
  * (crates/incin-backends/src/dtype_policy.rs:64-104).
  */
@@ -154,6 +159,7 @@ typedef struct {
     size_t workspace_bytes;
     int32_t num_splits;            /* 0 = library chooses */
     int32_t impl;                  /* INCIN_ROCM_IMPL_*; AUTO unless a test pins a kernel */
+    const int32_t* q_lens;         /* nullable device pointer, B entries: rows at and beyond are padding */
 } incin_rocm_sdpa_desc_t;
 
 /* Validates the descriptor and reports the scratch bytes and the split count the

@@ -132,6 +132,12 @@ def test_config5_gqa_ragged_causal_full(gpu):
     ref = O.sdpa_rows(q.reshape(B, Hkv, G, S, D), k[:, :, None], v[:, :, None], rows, causal=True,
                       kv_lens=lens.reshape(B, 1, 1))
     check_rows(got.reshape(B * Hq, S, D)[rows[:, 0], rows[:, 1]], ref, TOL[dt], "config 5")
+    # declaring the padding rows (q_lens) leaves every valid row bit-identical; what it saves is in the bench
+    say("config 5: padded-query property")
+    got_q = host.sdpa(q, k, v, dt, causal=True, kv_lens=lens, q_lens=lens)
+    for b in range(B):
+        n = int(lens[b])
+        assert np.array_equal(got[b, :, :n], got_q[b, :, :n])
     # padding keys carry weight exactly 0 in a valid row: other (finite) contents behind each length change
     # nothing there
     say("config 5: key-padding property")

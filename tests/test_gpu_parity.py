@@ -217,6 +217,28 @@ def test_mfma_prefill_ragged_lengths(gpu, impl):
     check(padded, trunc, 1e-6, "mfma padded == truncated")
 
 
+@pytest.mark.parametrize("impl", [capi.IMPL_AUTO, capi.IMPL_GENERIC] + MFMA_IMPLS)
+@pytest.mark.parametrize("causal", [True, False])
+def test_padded_queries(gpu, impl, causal):
+    """q_lens declares query rows padding: rows below the length are what they are without it (bit for bit);
+    rows at and beyond it are unspecified and not looked at."""
+    B, Hq, Hkv, S, D = 4, 4, 2, 600, 128
+    q, k, v = inputs(41, B, Hq, Hkv, S, S, D, D, capi.BF16)
+    lens = np.array([600, 257, 64, 0], np.int32)          # full, inside a block, a block boundary, nothing
+    say("padded queries: impl %d causal %s lens %s" % (impl, causal, lens.tolist()))
+    plain = host.sdpa(q, k, v, capi.BF16, causal=causal, kv_lens=lens, impl=impl)
+    got = host.sdpa(q, k, v, capi.BF16, causal=causal, kv_lens=lens, q_lens=lens, impl=impl)
+    ref = oracle_full(q, k, v, G=2, causal=causal, kv_lens=lens)
+    for b in range(B):
+        n = int(lens[b])
+        assert np.array_equal(got[b, :, :n], plain[b, :, :n]), "batch %d" % b
+        if n:
+            check(got[b:b + 1, :, :n], ref[b:b + 1, :, :n], 2e-2, "padded queries, batch %d" % b)
+    # lengths of Sq and beyond change nothing at all
+    same = host.sdpa(q, k, v, capi.BF16, causal=causal, kv_lens=lens, q_lens=np.full(B, S, np.int32), impl=impl)
+    assert np.array_equal(np.nan_to_num(same, nan=7.0), np.nan_to_num(plain, nan=7.0))
+
+
 # ---- split-KV decode -----------------------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", [capi.BF16, capi.F16, capi.F32])
