@@ -63,6 +63,25 @@ def test_descriptor_with_causal_and_key_counts_and_groups(gpu, dtype):
     assert err <= TOL[dtype]
 
 
+def test_descriptor_padded_queries(gpu):
+    # a padded self-attention batch: the same lengths for keys and queries; rows inside the lengths are what they
+    # are without q_lens, bit for bit
+    B, H, S, D = 3, 4, 300, 128
+    lens = [300, 129, 1]
+    q, k, v = rnd(8, (B, H, S, D), RB.BF16), rnd(9, (B, H, S, D), RB.BF16), rnd(10, (B, H, S, D), RB.BF16)
+    sq, sk, sv = (RB.RocmStorage.from_numpy(x, RB.BF16) for x in (q, k, v))
+    plain = RX.AttentionSpec.lower(q.shape, k.shape, v.shape, RB.BF16, causal=True, kv_lens=lens).execute(sq, sk, sv).to_numpy()
+    got = RX.AttentionSpec.lower(q.shape, k.shape, v.shape, RB.BF16, causal=True, kv_lens=lens, q_lens=lens).execute(sq, sk, sv).to_numpy()
+    ref = O.sdpa(q, k, v, causal=True, kv_lens=np.asarray(lens, np.int32).reshape(B, 1, 1))
+    for b in range(B):
+        n = lens[b]
+        assert np.array_equal(got[b, :, :n], plain[b, :, :n])
+        assert float(np.abs(got[b, :, :n] - ref[b, :, :n]).max()) <= TOL[RB.BF16]
+    with pytest.raises(RB.BackendError) as e:
+        RX.AttentionSpec.lower(q.shape, k.shape, v.shape, RB.BF16, q_lens=[300, 301, 0])
+    assert e.value.kind == "ShapeMismatch" and "query count 301 outside 0..=300" in e.value.message
+
+
 def test_descriptor_scale_and_views(gpu):
     q, k, v = rnd(4, (2, 3, 33, 64), RB.F32), rnd(5, (2, 3, 50, 64), RB.F32), rnd(6, (2, 3, 50, 64), RB.F32)
     spec = RX.AttentionSpec.lower(q.shape, k.shape, v.shape, RB.F32, scale=0.3)
