@@ -91,7 +91,8 @@ inline int device_cus()
 // A work item is (batch, KV head, query head of its group, block of query rows).  The list runs over groups of F
 // (batch, KV head) pairs; inside a group the query blocks go longest-first (under a causal mask the last block sees
 // the most keys), and for each block all F * G heads of the group follow one another.  With F * G * (blocks per head)
-// a multiple of the workgroups an XCD runs at a time, every round of workgroups gets items of equal length, which
+// a multiple (twice, measured best) of the workgroups an XCD runs at a time, every round of workgroups gets items of
+// nearly equal length, which
 // list scheduling in plain head order does not give (it ends each head on its shortest blocks while the next head's
 // longest start, and the last round is left ragged: about 9 % at 4096 x 4096 causal).  F is kept small: F KV heads
 // are in an XCD's L2 at a time.
@@ -107,18 +108,23 @@ __device__ __forceinline__ WorkItem work_item(int vid, int F, int G, int nqb)
     w.qblk = nqb - 1 - rank;
     return w;
 }
-// Which entry of the work list is item `item` of XCD `xcd`'s share (a share holds share_len items).  Shares are
-// dealt group by group (group g goes to XCD g % 8) when the groups divide evenly: batch entries of different
-// lengths then spread over all XCDs instead of one long sequence filling the shares of two of them.  Otherwise
-// a share is a contiguous eighth of the list.
-__device__ __forceinline__ int work_vid(int xcd, int item, int share_len, int F, int G, int nqb, int deal_groups)
+// Item `item` of XCD `xcd`'s share of the work list (a share holds share_len items).  When a share holds whole
+// groups, (batch, KV head) pairs are dealt to the XCDs in turn - pair h goes to XCD h % 8, and an XCD groups the
+// pairs it holds F at a time - so the sequences of a ragged batch spread over all XCDs instead of one long sequence
+// filling the shares of two of them.  Otherwise a share is a contiguous eighth of the list.
+__device__ __forceinline__ WorkItem work_item_of_share(int xcd, int item, int share_len, int F, int G, int nqb, int deal)
 {
-    if (!deal_groups) return xcd * share_len + item;
+    if (!deal) return work_item(xcd * share_len + item, F, G, nqb);
     const int per_group = F * G * nqb;
-    const int g_local = item / per_group;
-    return (g_local * 8 + xcd) * per_group + (item - g_local * per_group);
+    const int g_local = item / per_group, r = item - g_local * per_group;
+    const int rank = r / (F * G), m = r - rank * (F * G);
+    WorkItem w;
+    w.bhkv = (g_local * F + m / G) * 8 + xcd;
+    w.gq = m % G;
+    w.qblk = nqb - 1 - rank;
+    return w;
 }
-inline int work_deal_groups(int F, int G, int nqb, long long share_items)
+inline int work_deal(int F, int G, int nqb, long long share_items)
 {
     return share_items % ((long long)F * G * nqb) == 0 ? 1 : 0;
 }
@@ -130,7 +136,7 @@ inline int work_interleave(bool causal, int slots, int G, int nqb, long long ran
     if (!causal || slots <= 0) return 1;
     int a = slots, b = (G * nqb) % slots;
     while (b) { const int t = a % b; a = b; b = t; }          // a = gcd(slots, G * nqb)
-    int f = slots / a;
+    int f = 2 * (slots / a);          // two rounds per group: a slot that drew a long block first draws a short one next
     if (f > 8) f = 8;
     while (f > 1 && range_items % ((long long)f * G * nqb)) --f;
     return f;

@@ -24,7 +24,7 @@ struct SdpaParams {
     float scale;
     int32_t causal;
     int32_t interleave;        // MFMA prefill kernels: (batch, KV head) pairs per group of the work list, set by their launchers
-    int32_t deal_groups;       // MFMA prefill kernels: groups of the work list are dealt to the 8 XCDs in turn (else: contiguous eighths)
+    int32_t deal_groups;       // MFMA prefill kernels: (batch, KV head) pairs are dealt to the 8 XCDs in turn (else: contiguous eighths)
     // split-KV only
     int32_t num_splits;
     int32_t split_len;         // keys per split (multiple of the kernel's key tile)

@@ -86,9 +86,8 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     // range of the work list so heads that share K/V stay in one L2.
     const int nqb = (Sq + PF_BM - 1) / PF_BM;
     const int total = gridDim.x;
-    int vid = blockIdx.x;
-    if ((total & 7) == 0) vid = work_vid(blockIdx.x & 7, blockIdx.x >> 3, total >> 3, p.interleave, p.G, nqb, p.deal_groups);
-    const WorkItem wi = work_item(vid, p.interleave, p.G, nqb);
+    const WorkItem wi = (total & 7) == 0 ? work_item_of_share(blockIdx.x & 7, blockIdx.x >> 3, total >> 3, p.interleave, p.G, nqb, p.deal_groups)
+                                         : work_item(blockIdx.x, p.interleave, p.G, nqb);
     const int gq = wi.gq, qb = wi.qblk, bhkv = wi.bhkv;
     const int hkv = bhkv % p.Hkv, b = bhkv / p.Hkv;
     const int hq = hkv * p.G + gq;
@@ -436,7 +435,7 @@ static hipError_t launch_prefill_t(const SdpaParams& p0, hipStream_t stream)
     const int64_t total = (int64_t)nqb * p.Hq * p.B;
     // two workgroups per CU (register budget), an eighth of the CUs per XCD
     p.interleave = work_interleave(p.causal != 0, 2 * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
-    p.deal_groups = (total & 7) == 0 ? work_deal_groups(p.interleave, p.G, nqb, total >> 3) : 0;
+    p.deal_groups = (total & 7) == 0 ? work_deal(p.interleave, p.G, nqb, total >> 3) : 0;
     hipLaunchKernelGGL((sdpa_prefill_mfma_kernel<T, D>), dim3((unsigned)total), dim3(256), 0, stream, p);
     return hipGetLastError();
 }
