@@ -27,6 +27,7 @@ EXPORTS = [
     "incin_rocm_stream_create", "incin_rocm_stream_destroy", "incin_rocm_stream_sync",
     "incin_rocm_event_create", "incin_rocm_event_destroy", "incin_rocm_event_record",
     "incin_rocm_event_sync", "incin_rocm_event_elapsed_ms",
+    "incin_rocm_graph_begin", "incin_rocm_graph_end", "incin_rocm_graph_launch", "incin_rocm_graph_destroy",
     "incin_rocm_sdpa_workspace", "incin_rocm_sdpa_fwd",
 ]
 
@@ -112,6 +113,10 @@ def load():
     lib.incin_rocm_event_record.argtypes = [C.c_int32, C.c_void_p, C.c_void_p]
     lib.incin_rocm_event_sync.argtypes = [C.c_int32, C.c_void_p]
     lib.incin_rocm_event_elapsed_ms.argtypes = [C.c_int32, C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]
+    lib.incin_rocm_graph_begin.argtypes = [C.c_int32, C.c_void_p]
+    lib.incin_rocm_graph_end.argtypes = [C.c_int32, C.c_void_p, C.POINTER(C.c_void_p)]
+    lib.incin_rocm_graph_launch.argtypes = [C.c_int32, C.c_void_p, C.c_void_p]
+    lib.incin_rocm_graph_destroy.argtypes = [C.c_int32, C.c_void_p]
     lib.incin_rocm_sdpa_workspace.argtypes = [C.POINTER(SdpaDesc), C.POINTER(C.c_size_t), C.POINTER(C.c_int32),
                                               C.POINTER(C.c_int32)]
     lib.incin_rocm_sdpa_fwd.argtypes = [C.POINTER(SdpaDesc), C.c_void_p]
@@ -224,4 +229,35 @@ class Stream:
     def destroy(self):
         if self.ptr:
             check(load().incin_rocm_stream_destroy(self.dev, self.ptr))
+            self.ptr = None
+
+
+class Graph:
+    """Launches recorded on a stream (`with Graph.record(stream) as g: ...`), replayed with `launch`."""
+
+    def __init__(self, stream):
+        self.dev, self.stream, self.ptr = stream.dev, stream, None
+
+    @classmethod
+    def record(cls, stream):
+        return cls(stream)
+
+    def __enter__(self):
+        check(load().incin_rocm_graph_begin(self.dev, self.stream.ptr))
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        p = C.c_void_p()
+        rc = load().incin_rocm_graph_end(self.dev, self.stream.ptr, C.byref(p))
+        if exc_type is None:
+            check(rc)
+            self.ptr = p.value
+        return False
+
+    def launch(self, stream=None):
+        check(load().incin_rocm_graph_launch(self.dev, self.ptr, (stream or self.stream).ptr))
+
+    def destroy(self):
+        if self.ptr:
+            check(load().incin_rocm_graph_destroy(self.dev, self.ptr))
             self.ptr = None

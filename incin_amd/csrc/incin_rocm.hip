@@ -345,6 +345,46 @@ int incin_rocm_stream_sync(int32_t dev, void* stream)
     return 0;
 }
 
+int incin_rocm_graph_begin(int32_t dev, void* stream)
+{
+    if (!stream) return fail(INCIN_ROCM_EINVAL, "graph_begin: recording needs a stream of its own, not the default stream");
+    if (int rc = use_device(dev)) return rc;
+    // thread-local mode: other threads may go on allocating and launching while this one records
+    HIP_TRY(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
+    return 0;
+}
+
+int incin_rocm_graph_end(int32_t dev, void* stream, void** graph_out)
+{
+    if (!graph_out) return fail(INCIN_ROCM_EINVAL, "graph_end: null output");
+    *graph_out = nullptr;
+    if (int rc = use_device(dev)) return rc;
+    hipGraph_t g = nullptr;
+    HIP_TRY(hipStreamEndCapture((hipStream_t)stream, &g), "hipStreamEndCapture");
+    hipGraphExec_t exec = nullptr;
+    hipError_t e = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(g);
+    if (e != hipSuccess) return fail(INCIN_ROCM_ERUNTIME, "ROCm hipGraphInstantiate failed: %s", hipGetErrorString(e));
+    *graph_out = (void*)exec;
+    return 0;
+}
+
+int incin_rocm_graph_launch(int32_t dev, void* graph, void* stream)
+{
+    if (!graph) return fail(INCIN_ROCM_EINVAL, "graph_launch: null graph");
+    if (int rc = use_device(dev)) return rc;
+    HIP_TRY(hipGraphLaunch((hipGraphExec_t)graph, (hipStream_t)stream), "hipGraphLaunch");
+    return 0;
+}
+
+int incin_rocm_graph_destroy(int32_t dev, void* graph)
+{
+    if (!graph) return 0;
+    if (int rc = use_device(dev)) return rc;
+    HIP_TRY(hipGraphExecDestroy((hipGraphExec_t)graph), "hipGraphExecDestroy");
+    return 0;
+}
+
 int incin_rocm_event_create(int32_t dev, void** out)
 {
     if (!out) return fail(INCIN_ROCM_EINVAL, "event_create: null output");

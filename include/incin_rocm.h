@@ -108,6 +108,17 @@ int incin_rocm_event_record(int32_t dev, void* event, void* stream);
 int incin_rocm_event_sync(int32_t dev, void* event);
 int incin_rocm_event_elapsed_ms(int32_t dev, void* start, void* stop, float* out_ms);
 
+/* ---- launch graphs ------------------------------------------------------------
+ * No counterpart in the reference (its backends launch eagerly).  For callers that replay a fixed sequence of
+ * launches, a decode loop for one: everything enqueued on `stream` between begin and end is recorded instead of
+ * run, and the recording is replayed with incin_rocm_graph_launch.  incin_rocm_sdpa_fwd can be recorded: it
+ * neither allocates nor clears memory (the workspace is the caller's).  The allocating and copying entry points
+ * above must not be called on a stream that is recording. */
+int incin_rocm_graph_begin(int32_t dev, void* stream);
+int incin_rocm_graph_end(int32_t dev, void* stream, void** graph_out);
+int incin_rocm_graph_launch(int32_t dev, void* graph, void* stream);
+int incin_rocm_graph_destroy(int32_t dev, void* graph);
+
 /* ---- attention forward --------------------------------------------------------
  * Replaces CpuBackendImpl::scaled_dot_product_attention
  * (crates/incin-backends/src/cpu/ops/shape_ops.rs:1245-1269), the only

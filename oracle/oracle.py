@@ -113,6 +113,9 @@ def _prepare(q, k, v, mask, scale, causal, kv_lens, host_has_fma):
         raise ValueError("inner dims must match")
     b = broadcast_shape(q.shape[:-2], k.shape[:-2])
     b = broadcast_shape(b, v.shape[:-2])
+    if mask is not None and (causal or kv_lens is not None):
+        # the reference knows one mask tensor; the synthesised forms stand in for it, they do not add to it
+        raise ValueError("give either an explicit mask or causal / kv_lens; fold them into the mask to combine them")
     if mask is not None:
         mask = np.asarray(mask, dtype=np.float32)
         mshape = list(mask.shape)

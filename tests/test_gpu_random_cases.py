@@ -1,0 +1,105 @@
+"""Randomised differential test through the C ABI: seeded random shapes, dtypes, masks, lengths, scales and kernel
+choices, each compared with the CPU oracle.  The fixed sweeps of test_gpu_parity.py pick cases by hand; this one
+draws combinations nobody thought of (odd extents, broadcast mask axes, lengths of 0, Sq != Skv with causal
+alignment, every kernel the planner accepts for the case)."""
+import sys
+
+import numpy as np
+import pytest
+
+from incin_amd import capi, dtypes, host
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+TOL = {capi.F32: 1e-5, capi.F16: 2e-2, capi.BF16: 2e-2}
+N_CASES = 160
+
+
+def say(msg):
+    print(msg, file=sys.stderr, flush=True)
+
+
+def draw_case(r):
+    dtype = int(r.choice([capi.F32, capi.F16, capi.BF16]))
+    D = int(r.choice([16, 32, 64, 64, 80, 128, 128, 128, 256]))
+    Dv = D if r.random() < 0.8 else int(r.choice([16, 64, 128]))
+    Hkv = int(r.integers(1, 4))
+    G = int(r.choice([1, 1, 2, 4]))
+    B = int(r.integers(1, 4))
+    kind = r.choice(["prefill", "prefill", "decode", "rect"])
+    if kind == "decode":
+        Sq, Skv = int(r.integers(1, 5)), int(r.integers(1, 1500))
+    elif kind == "rect":
+        Sq, Skv = int(r.integers(1, 200)), int(r.integers(1, 400))
+    else:
+        Sq = Skv = int(r.integers(1, 420))
+    causal = bool(r.random() < 0.5)
+    lens = r.integers(0, Skv + 1, B).astype(np.int32) if r.random() < 0.4 else None
+    mask = None
+    if r.random() < 0.25:
+        shp = [B if r.random() < 0.5 else 1, Hkv * G if r.random() < 0.5 else 1, Sq if r.random() < 0.7 else 1, Skv]
+        mask = r.standard_normal(shp, dtype=np.float32)
+        mask[r.random(shp) < 0.2] = -np.inf
+    scale = None if r.random() < 0.6 else float(r.uniform(0.02, 0.6))
+    return dict(dtype=dtype, B=B, Hkv=Hkv, G=G, Sq=Sq, Skv=Skv, D=D, Dv=Dv, causal=causal, lens=lens, mask=mask, scale=scale)
+
+
+def run_case(i, c, r):
+    B, Hkv, G, Sq, Skv, D, Dv, dt = c["B"], c["Hkv"], c["G"], c["Sq"], c["Skv"], c["D"], c["Dv"], c["dtype"]
+    Hq = Hkv * G
+    q = dtypes.round_to(r.standard_normal((B, Hq, Sq, D), dtype=np.float32), dt)
+    k = dtypes.round_to(r.standard_normal((B, Hkv, Skv, D), dtype=np.float32), dt)
+    v = dtypes.round_to(r.standard_normal((B, Hkv, Skv, Dv), dtype=np.float32), dt)
+    mask = None if c["mask"] is None else dtypes.round_to(c["mask"], dt)
+    kw = dict(scale=c["scale"], causal=c["causal"], kv_lens=c["lens"], mask=mask)
+    if mask is None:
+        ref = O.sdpa(q.reshape(B, Hkv, G, Sq, D), k[:, :, None], v[:, :, None], scale=c["scale"], causal=c["causal"],
+                     kv_lens=None if c["lens"] is None else c["lens"].reshape(B, 1, 1))
+    else:
+        # the reference has one mask tensor: what the descriptor states beside it (causal, key counts) is folded into
+        # an explicit [B, Hkv, G, Sq, Skv] mask for the oracle
+        full = np.broadcast_to(mask, (B, Hq, Sq, Skv)).copy()
+        if c["causal"]:
+            full += np.triu(np.full((Sq, Skv), -np.inf, np.float32), 1 + Skv - Sq)
+        if c["lens"] is not None:
+            full += np.where(np.arange(Skv)[None, :] < c["lens"][:, None], 0.0, -np.inf).astype(np.float32)[:, None, None, :]
+        ref = O.sdpa(q.reshape(B, Hkv, G, Sq, D), k[:, :, None], v[:, :, None], mask=full.reshape(B, Hkv, G, Sq, Skv), scale=c["scale"])
+    ref = ref.reshape(B, Hq, Sq, Dv)
+    impls = [capi.IMPL_AUTO]
+    for impl in (capi.IMPL_GENERIC, capi.IMPL_MFMA, capi.IMPL_MFMA64, capi.IMPL_SPLITKV):
+        try:
+            got, info = host.sdpa(q, k, v, dt, impl=impl, return_info=True, **kw)
+        except capi.RocmError as e:
+            assert e.code == 7, "case %d impl %d: %s" % (i, impl, e)       # EUNSUPPORTED: outside that kernel's domain
+            continue
+        impls.append(impl)
+        check(i, c, impl, got, ref)
+    got = host.sdpa(q, k, v, dt, **kw)
+    check(i, c, capi.IMPL_AUTO, got, ref)
+    return impls
+
+
+def check(i, c, impl, got, ref):
+    what = "case %d impl %d %s" % (i, impl, {k: (v if not isinstance(v, np.ndarray) else v.shape) for k, v in c.items()})
+    nr = np.isnan(ref)
+    assert np.array_equal(np.isnan(got), nr), what + ": NaN pattern"
+    err = float(np.abs(np.where(nr, 0, got) - np.where(nr, 0, ref)).max()) if got.size else 0.0
+    # The stated bars (1e-5, 2e-2) are absolute and meant for outputs of order one, as the default scale gives; a drawn
+    # scale several times the default makes the softmax pick single values of v (|o| up to ~4), where one bf16 rounding
+    # of the output is already 8e-3: the bar scales with the largest output magnitude there.
+    big = float(np.abs(np.where(nr, 0, ref)).max()) if got.size else 0.0
+    assert err <= TOL[c["dtype"]] * max(1.0, big), "%s: %.3e (outputs up to %.2f)" % (what, err, big)
+
+
+def test_random_cases(gpu):
+    r = np.random.Generator(np.random.PCG64(20261125))
+    used = {}
+    for i in range(N_CASES):
+        c = draw_case(r)
+        if i % 20 == 0:
+            say("random case %d/%d" % (i, N_CASES))
+        for impl in run_case(i, c, r):
+            used[impl] = used.get(impl, 0) + 1
+    say("kernels exercised: %s" % used)
+    for impl in (capi.IMPL_GENERIC, capi.IMPL_MFMA, capi.IMPL_MFMA64, capi.IMPL_SPLITKV):
+        assert used.get(impl, 0) >= 5, "kernel %d was hardly reached: %s" % (impl, used)

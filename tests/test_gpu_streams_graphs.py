@@ -1,0 +1,95 @@
+"""The launch path under conditions a serving loop puts it in: several host threads launching on streams of their
+own at once (the C ABI promises this is safe), and launches captured into a HIP graph and replayed (the launch path
+neither allocates nor clears memory).  Results must equal the plain launch bit for bit."""
+import sys
+import threading
+
+import numpy as np
+import pytest
+
+from incin_amd import capi, dtypes, host
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print(msg, file=sys.stderr, flush=True)
+
+
+class Case:
+    def __init__(self, seed, B, Hq, Hkv, Sq, Skv, D, causal, impl):
+        r = np.random.Generator(np.random.PCG64(seed))
+        mk = lambda *s: dtypes.round_to(r.standard_normal(s, dtype=np.float32), capi.BF16)
+        self.tq, self.tk, self.tv = (host.DeviceTensor.from_f32(x, capi.BF16) for x in
+                                     (mk(B, Hq, Sq, D), mk(B, Hkv, Skv, D), mk(B, Hkv, Skv, D)))
+        self.to = host.DeviceTensor((B, Hq, Sq, D), capi.BF16)
+        self.desc = host.make_desc(self.tq, self.tk, self.tv, self.to, causal=causal, impl=impl)
+        nbytes, _, self.impl = capi.sdpa_workspace(self.desc)
+        self.ws = capi.DeviceBuffer(nbytes) if nbytes else None
+        if self.ws is not None:
+            self.desc.workspace, self.desc.workspace_bytes = self.ws.ptr, self.ws.nbytes
+
+    def plain(self):
+        capi.sdpa_fwd(self.desc)
+        capi.sync()
+        return self.to.to_f32()
+
+    def clear(self):
+        capi.check(capi.load().incin_rocm_memset(0, self.to.ptr, 0xFF, self.to.buf.nbytes))
+        capi.sync()
+
+
+CASES = [
+    ("prefill 32-row kernel", dict(B=2, Hq=8, Hkv=8, Sq=512, Skv=512, D=128, causal=True, impl=capi.IMPL_MFMA)),
+    ("prefill 64-row kernel", dict(B=2, Hq=8, Hkv=2, Sq=1024, Skv=1024, D=128, causal=True, impl=capi.IMPL_MFMA64)),
+    ("decode split-KV", dict(B=4, Hq=8, Hkv=8, Sq=1, Skv=4096, D=128, causal=False, impl=capi.IMPL_SPLITKV)),
+    ("generic", dict(B=1, Hq=2, Hkv=2, Sq=100, Skv=130, D=80, causal=True, impl=capi.IMPL_GENERIC)),
+]
+
+
+def test_threads_on_their_own_streams(gpu):
+    cases = [Case(100 + i, **kw) for i, (_, kw) in enumerate(CASES)]
+    expect = [c.plain() for c in cases]
+    for c in cases:
+        c.clear()
+    errors = []
+
+    def worker(c):
+        try:
+            s = capi.Stream()
+            for _ in range(25):
+                capi.sdpa_fwd(c.desc, s.ptr)
+            s.sync()
+        except Exception as e:      # noqa: BLE001 - reported below
+            errors.append(e)
+
+    say("4 threads x 25 launches, one stream and one kernel each")
+    threads = [threading.Thread(target=worker, args=(c,)) for c in cases]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for (name, _), c, e in zip(CASES, cases, expect):
+        got = c.to.to_f32()
+        assert np.array_equal(np.nan_to_num(got, nan=3.0), np.nan_to_num(e, nan=3.0)), name
+
+
+@pytest.mark.parametrize("name, kw", CASES, ids=[n for n, _ in CASES])
+def test_graph_capture_and_replay(gpu, name, kw):
+    c = Case(200, **kw)
+    expect = c.plain()
+    say("graph capture: %s" % name)
+    stream = capi.Stream()
+    with capi.Graph.record(stream) as graph:
+        capi.sdpa_fwd(c.desc, stream.ptr)
+        capi.sdpa_fwd(c.desc, stream.ptr)          # twice in one graph: the second must see what the first leaves behind
+    for replay in range(3):
+        c.clear()
+        graph.launch()
+        stream.sync()
+        got = c.to.to_f32()
+        assert np.array_equal(np.nan_to_num(got, nan=3.0), np.nan_to_num(expect, nan=3.0)), "%s, replay %d" % (name, replay)
+        # eager work of the program's own between replays
+        assert np.array_equal(np.nan_to_num(c.plain(), nan=3.0), np.nan_to_num(expect, nan=3.0))
+    graph.destroy()
