@@ -10,7 +10,7 @@
  * What each entry point stands in for in the reference (paths relative to the
  * reference checkout) is cited on its declaration.  The reference's GPU backends
  * reach their driver through the `cudarc` crate; the same call shapes are what a
- * Rust `incin-rocm-sys` crate binds here (bindings shown in INTEGRATION.md).
+ * Rust `incin-rocm-sys` crate binds here.
  */
 #ifndef INCIN_ROCM_H
 #define INCIN_ROCM_H
