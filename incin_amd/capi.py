@@ -29,6 +29,7 @@ EXPORTS = [
     "incin_rocm_event_sync", "incin_rocm_event_elapsed_ms",
     "incin_rocm_graph_begin", "incin_rocm_graph_end", "incin_rocm_graph_launch", "incin_rocm_graph_destroy",
     "incin_rocm_sdpa_workspace", "incin_rocm_sdpa_fwd",
+    "incin_rocm_sizeof_kv_append_desc", "incin_rocm_kv_append",
 ]
 
 
@@ -67,6 +68,19 @@ class SdpaDesc(C.Structure):
         ("num_splits", C.c_int32),
         ("impl", C.c_int32),
         ("q_lens", C.c_void_p),
+    ]
+
+
+class KvAppendDesc(C.Structure):
+    _fields_ = [
+        ("dtype", C.c_int32),
+        ("device", C.c_int32),
+        ("B", C.c_int64), ("Hkv", C.c_int64), ("S_new", C.c_int64), ("S_max", C.c_int64), ("D", C.c_int64), ("Dv", C.c_int64),
+        ("k_new", C.c_void_p), ("v_new", C.c_void_p),
+        ("k_new_stride", C.c_int64 * 3), ("v_new_stride", C.c_int64 * 3),
+        ("k_cache", C.c_void_p), ("v_cache", C.c_void_p),
+        ("k_cache_stride", C.c_int64 * 3), ("v_cache_stride", C.c_int64 * 3),
+        ("kv_lens", C.c_void_p),
     ]
 
 
@@ -120,6 +134,8 @@ def load():
     lib.incin_rocm_sdpa_workspace.argtypes = [C.POINTER(SdpaDesc), C.POINTER(C.c_size_t), C.POINTER(C.c_int32),
                                               C.POINTER(C.c_int32)]
     lib.incin_rocm_sdpa_fwd.argtypes = [C.POINTER(SdpaDesc), C.c_void_p]
+    lib.incin_rocm_sizeof_kv_append_desc.restype = C.c_size_t
+    lib.incin_rocm_kv_append.argtypes = [C.POINTER(KvAppendDesc), C.c_void_p]
     _lib = lib
     return lib
 
@@ -186,6 +202,10 @@ def sdpa_workspace(desc):
     nbytes, splits, impl = C.c_size_t(0), C.c_int32(0), C.c_int32(0)
     check(load().incin_rocm_sdpa_workspace(C.byref(desc), C.byref(nbytes), C.byref(splits), C.byref(impl)))
     return nbytes.value, splits.value, impl.value
+
+
+def kv_append(desc, stream=None):
+    check(load().incin_rocm_kv_append(C.byref(desc), stream))
 
 
 def sdpa_fwd(desc, stream=None):

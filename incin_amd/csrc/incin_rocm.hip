@@ -10,6 +10,7 @@
 #include <cstring>
 
 #include "../../include/incin_rocm.h"
+#include "kv_append.h"
 #include "sdpa_params.h"
 
 namespace incin_rocm {
@@ -462,6 +463,45 @@ int incin_rocm_sdpa_fwd(const incin_rocm_sdpa_desc_t* desc, void* stream)
         default: e = incin_rocm::launch_sdpa_generic(p, desc->dtype, s); break;
     }
     if (e != hipSuccess) return hip_fail(e, "attention kernel launch");
+    return 0;
+}
+
+
+size_t incin_rocm_sizeof_kv_append_desc(void) { return sizeof(incin_rocm_kv_append_desc_t); }
+
+int incin_rocm_kv_append(const incin_rocm_kv_append_desc_t* d, void* stream)
+{
+    if (!d) return fail(INCIN_ROCM_EINVAL, "kv_append: null descriptor");
+    if (d->dtype != INCIN_ROCM_F32 && d->dtype != INCIN_ROCM_F16 && d->dtype != INCIN_ROCM_BF16)
+        return fail(INCIN_ROCM_EDTYPE, "kv_append: dtype %d is not one of f32, f16, bf16", (int)d->dtype);
+    if (d->B < 0 || d->Hkv < 0 || d->S_new < 0 || d->S_max < 0 || d->D < 0 || d->Dv < 0)
+        return fail(INCIN_ROCM_ESHAPE, "kv_append: negative extent");
+    const int64_t lim = 0x7fffffffLL;
+    if (d->B > lim || d->Hkv > lim || d->S_new > lim || d->S_max > lim || d->D > (1 << 20) || d->Dv > (1 << 20) ||
+        d->B * d->Hkv * d->S_new > lim)
+        return fail(INCIN_ROCM_ESHAPE, "kv_append: extent exceeds 2^31-1");
+    if (d->B == 0 || d->Hkv == 0 || d->S_new == 0) return 0;
+    if (!d->k_new || !d->v_new || !d->k_cache || !d->v_cache || !d->kv_lens)
+        return fail(INCIN_ROCM_EINVAL, "kv_append: null operand");
+    if (int rc = use_device(d->device)) return rc;
+    const int elem = d->dtype == INCIN_ROCM_F32 ? 4 : 2;
+    incin_rocm::KvAppendParams p;
+    p.k_new = (const char*)d->k_new; p.v_new = (const char*)d->v_new;
+    p.k_cache = (char*)d->k_cache; p.v_cache = (char*)d->v_cache;
+    p.kv_lens = d->kv_lens;
+    p.kn_sb = d->k_new_stride[0]; p.kn_sh = d->k_new_stride[1]; p.kn_ss = d->k_new_stride[2];
+    p.vn_sb = d->v_new_stride[0]; p.vn_sh = d->v_new_stride[1]; p.vn_ss = d->v_new_stride[2];
+    p.kc_sb = d->k_cache_stride[0]; p.kc_sh = d->k_cache_stride[1]; p.kc_ss = d->k_cache_stride[2];
+    p.vc_sb = d->v_cache_stride[0]; p.vc_sh = d->v_cache_stride[1]; p.vc_ss = d->v_cache_stride[2];
+    p.B = (int32_t)d->B; p.Hkv = (int32_t)d->Hkv; p.S_new = (int32_t)d->S_new; p.S_max = (int32_t)d->S_max;
+    p.k_row_bytes = (int32_t)(d->D * elem); p.v_row_bytes = (int32_t)(d->Dv * elem); p.elem = elem;
+    // 16-byte copies need every row start and every row length to be a multiple of 16 bytes
+    auto mult16 = [&](int64_t stride_elems) { return (stride_elems * elem) % 16 == 0; };
+    bool vec16 = p.k_row_bytes % 16 == 0 && p.v_row_bytes % 16 == 0 && (uintptr_t)d->k_new % 16 == 0 && (uintptr_t)d->v_new % 16 == 0 &&
+                 (uintptr_t)d->k_cache % 16 == 0 && (uintptr_t)d->v_cache % 16 == 0;
+    for (int i = 0; i < 3; ++i)
+        vec16 = vec16 && mult16(d->k_new_stride[i]) && mult16(d->v_new_stride[i]) && mult16(d->k_cache_stride[i]) && mult16(d->v_cache_stride[i]);
+    HIP_TRY(incin_rocm::launch_kv_append(p, vec16, (hipStream_t)stream), "kv_append launch");
     return 0;
 }
 

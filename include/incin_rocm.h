@@ -184,6 +184,31 @@ int incin_rocm_sdpa_workspace(const incin_rocm_sdpa_desc_t* desc, size_t* bytes,
  * keeps alive until the stream has been synchronised. */
 int incin_rocm_sdpa_fwd(const incin_rocm_sdpa_desc_t* desc, void* stream);
 
+/* ---- key/value cache append ----------------------------------------------------
+ * No counterpart in the reference (it has no cache: a decode loop there concatenates tensors,
+ * TensorOps::cat, and re-runs the operator).  Copies S_new new key and value rows per (batch, kv head) into
+ * preallocated caches [B, Hkv, S_max, D] / [.., Dv] at row kv_lens[b], then advances kv_lens[b] by S_new - all
+ * on the device and stream-ordered, so that (append, incin_rocm_sdpa_fwd with the same kv_lens) is a decode step
+ * that needs nothing from the host and can be recorded into a launch graph once and replayed per token.
+ * Rows that would land at or beyond S_max are dropped and kv_lens saturates at S_max: the caller sizes the cache.
+ * Strides are in elements (batch, head, row), the last axis has stride 1. */
+typedef struct {
+    int32_t dtype;                 /* INCIN_ROCM_F32 / F16 / BF16 */
+    int32_t device;
+    int64_t B, Hkv, S_new, S_max, D, Dv;
+    const void* k_new;
+    const void* v_new;
+    int64_t k_new_stride[3];
+    int64_t v_new_stride[3];
+    void* k_cache;
+    void* v_cache;
+    int64_t k_cache_stride[3];
+    int64_t v_cache_stride[3];
+    int32_t* kv_lens;              /* device pointer, B entries, read and advanced */
+} incin_rocm_kv_append_desc_t;
+size_t incin_rocm_sizeof_kv_append_desc(void);
+int incin_rocm_kv_append(const incin_rocm_kv_append_desc_t* desc, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
