@@ -68,6 +68,7 @@ class SdpaDesc(C.Structure):
         ("num_splits", C.c_int32),
         ("impl", C.c_int32),
         ("q_lens", C.c_void_p),
+        ("lse", C.c_void_p),
     ]
 
 

@@ -285,7 +285,7 @@ def draw(slot):
 def loop(ty):
     """The whole main path of a wavefront: tiles 0 .. LEFT-1.  Entry: T = 0, Q^T (scaled) in v0..v63, REL for tile 0,
     the copies of K(0..7), V(0..5) started (K(0..3), V(0), V(1) complete and visible).  Exit: T = LEFT tiles done (if
-    T is even its turn has NOT been taken), O^T in its AGPRs, the row sums in LRUN."""
+    T is even its turn has NOT been taken), O^T in its AGPRs, the row sums in LRUN, the reference maxima in MREF."""
     L = ["s_mov_b32 s%d, m0" % M0SAVE]
     L += prologue()
     L += first_scores(ty)
@@ -323,7 +323,7 @@ def main():
                       ("LRUN0", LRUN[0]), ("LRUN1", LRUN[1])):
         out.append("#define PF_R_%s %d" % (name, val))
     clob = (list(range(NR[0], NR[0] + 16)) + list(range(NR[1], NR[1] + 16)) + list(range(P, P + 16)) + list(range(KB, KB + 32)) +
-            list(range(VB, VB + 32)) + list(range(E, E + 4)) + MX + THR + MREF + TT)
+            list(range(VB, VB + 32)) + list(range(E, E + 4)) + MX + THR + TT)
     aclob = list(range(Q(0, 0), Q(0, 0) + QB * NSTEP * 4))
     # operand lists of the asm statement; the kernel source declares variables with these names
     outs = []
@@ -332,6 +332,8 @@ def main():
             outs.append('"+{%s}"(qreg[%d][%d])' % (v((qb * NSTEP + s_) * 4, 4), qb, s_))
     for qb in range(QB):
         outs.append('"={%s}"(l_run[%d])' % (v(LRUN[qb]), qb))
+    for qb in range(QB):
+        outs.append('"={%s}"(m_ref[%d])' % (v(MREF[qb]), qb))
     for db in range(NDB):
         for qb in range(QB):
             outs.append('"={%s}"(o_acc[%d][%d])' % (a_(O(db, qb), 16), db, qb))

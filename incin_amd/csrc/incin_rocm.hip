@@ -129,12 +129,12 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
 
     int impl = d->impl;
     if (impl == INCIN_ROCM_IMPL_AUTO) {
-        if (split_ok && R <= 8 && d->Skv >= 256) impl = INCIN_ROCM_IMPL_SPLITKV;
+        if (split_ok && R <= 8 && d->Skv >= 256 && !d->lse) impl = INCIN_ROCM_IMPL_SPLITKV;
         // long sequences with work for every compute unit twice over: the 64-row kernel's halved LDS traffic outweighs
         // what it pays per 256-row work item (measured crossover: a few thousand keys)
         else if (mfma64_ok && d->Skv >= 8192 && d->B * d->Hq * ((d->Sq + 255) / 256) >= 512) impl = INCIN_ROCM_IMPL_MFMA64;
         else if (mfma_ok) impl = INCIN_ROCM_IMPL_MFMA;
-        else if (split_ok && R <= 8) impl = INCIN_ROCM_IMPL_SPLITKV;
+        else if (split_ok && R <= 8 && !d->lse) impl = INCIN_ROCM_IMPL_SPLITKV;
         else impl = INCIN_ROCM_IMPL_GENERIC;
     }
     if (impl == INCIN_ROCM_IMPL_MFMA && !mfma_ok)
@@ -143,6 +143,8 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     if (impl == INCIN_ROCM_IMPL_MFMA64 && !mfma64_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
                     "scaled_dot_product_attention: the 64-row MFMA kernel needs what the MFMA kernel needs, D == Dv == 128 and key/value slices below 2 GiB");
+    if (impl == INCIN_ROCM_IMPL_SPLITKV && d->lse)
+        return fail(INCIN_ROCM_EUNSUPPORTED, "scaled_dot_product_attention: the split-KV kernel does not write the row normalisers (lse)");
     if (impl == INCIN_ROCM_IMPL_SPLITKV && !split_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
                     "scaled_dot_product_attention: the split-KV kernel needs D == Dv in {64,128}, Sq <= 64, no dense mask and 16-byte aligned rows");
@@ -184,6 +186,7 @@ void fill_params(const incin_rocm_sdpa_desc_t* d, const Plan& plan, SdpaParams* 
     p->mask = d->add_mask;
     p->kv_lens = d->kv_lens;
     p->q_lens = d->q_lens;
+    p->lse = d->lse;
     p->q_sb = d->q_stride[0]; p->q_sh = d->q_stride[1]; p->q_ss = d->q_stride[2];
     p->k_sb = d->k_stride[0]; p->k_sh = d->k_stride[1]; p->k_ss = d->k_stride[2];
     p->v_sb = d->v_stride[0]; p->v_sh = d->v_stride[1]; p->v_ss = d->v_stride[2];

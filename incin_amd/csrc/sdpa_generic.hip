@@ -152,6 +152,8 @@ __global__ __launch_bounds__(256) void sdpa_generic_kernel(SdpaParams p)
         const int i = q0 + ty * 4 + r;
         if (i >= Sq) continue;
         const float inv = 1.0f / l_run[r];                  // l == 0 (no visible key): 0 * inf = NaN, as the reference
+        if (p.lse && tx == 0)
+            p.lse[((int64_t)b * p.Hq + hq) * Sq + i] = l_run[r] == 0.0f ? -INFINITY : m_run[r] + logf(l_run[r]);
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
             const int col = tx + 16 * c;

@@ -14,6 +14,7 @@ struct SdpaParams {
     const void* mask;          // nullable dense additive mask (same dtype as q)
     const int32_t* kv_lens;    // nullable, B entries
     const int32_t* q_lens;     // nullable, B entries: query rows at and beyond are padding (output unspecified)
+    float* lse;                // nullable, [B, Hq, Sq]: natural-log softmax normaliser of every row (generic and MFMA prefill kernels)
     int64_t q_sb, q_sh, q_ss;
     int64_t k_sb, k_sh, k_ss;
     int64_t v_sb, v_sh, v_ss;

@@ -411,6 +411,8 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     // ---- normalise and store ------------------------------------------------------------------
     const float l_tot = xor32_sum(l_run);
     const float inv = (l_tot == 0.0f) ? __builtin_nanf("") : 1.0f / l_tot;   // no visible key: NaN, as the reference
+    if (p.lse && g == 0 && my_i < rows_b)       // m_ref and the sum are in log2 units of the scaled scores
+        p.lse[((int64_t)b * p.Hq + hq) * Sq + my_i] = l_tot == 0.0f ? -INFINITY : (m_ref + __builtin_log2f(l_tot)) * 0.6931471805599453f;
     if (my_i < rows_b) {
         T* orow = op + (int64_t)my_i * p.o_ss;
 #pragma unroll

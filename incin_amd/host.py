@@ -48,7 +48,7 @@ def resolve_scale(scale, d):
 
 
 def make_desc(q, k, v, o, scale=None, causal=False, kv_lens=None, mask=None, mask_strides=None,
-              num_splits=0, impl=capi.IMPL_AUTO, workspace=None, q_lens=None):
+              num_splits=0, impl=capi.IMPL_AUTO, workspace=None, q_lens=None, lse=None):
     B, Hq, Sq, D = q.shape
     Bk, Hkv, Skv, Dk = k.shape
     Bv, Hv, Skv2, Dv = v.shape
@@ -64,6 +64,7 @@ def make_desc(q, k, v, o, scale=None, causal=False, kv_lens=None, mask=None, mas
     d.causal = 1 if causal else 0
     d.kv_lens = kv_lens.ptr if kv_lens is not None else None
     d.q_lens = q_lens.ptr if q_lens is not None else None
+    d.lse = lse.ptr if lse is not None else None
     if mask is not None:
         d.add_mask = mask.ptr
         for i in range(4):
@@ -89,7 +90,7 @@ def mask_strides_for(mask_shape, B, Hq, Sq, Skv):
 
 
 def sdpa(q, k, v, dtype=capi.F32, scale=None, causal=False, kv_lens=None, mask=None,
-         num_splits=0, impl=capi.IMPL_AUTO, dev=0, return_info=False, q_lens=None):
+         num_splits=0, impl=capi.IMPL_AUTO, dev=0, return_info=False, q_lens=None, return_lse=False):
     """Run attention on the GPU for f32 numpy operands [B,Hq,Sq,D], [B,Hkv,Skv,D], [B,Hkv,Skv,Dv].
 
     Operands are rounded to `dtype` on upload; the result is returned as f32
@@ -109,7 +110,8 @@ def sdpa(q, k, v, dtype=capi.F32, scale=None, causal=False, kv_lens=None, mask=N
         mask = np.asarray(mask, dtype=np.float32)
         ms = mask_strides_for(mask.shape, B, Hq, Sq, k.shape[2])
         tm = capi.DeviceBuffer.from_numpy(dtypes.encode(mask, dtype), dev)
-    d = make_desc(tq, tk, tv, to, scale, causal, tl, tm, ms, num_splits, impl, q_lens=tql)
+    tlse = capi.DeviceBuffer(B * Hq * Sq * 4, dev) if return_lse else None
+    d = make_desc(tq, tk, tv, to, scale, causal, tl, tm, ms, num_splits, impl, q_lens=tql, lse=tlse)
     nbytes, splits, chosen = capi.sdpa_workspace(d)
     ws = capi.DeviceBuffer(nbytes, dev) if nbytes else None
     if ws is not None:
@@ -117,9 +119,13 @@ def sdpa(q, k, v, dtype=capi.F32, scale=None, causal=False, kv_lens=None, mask=N
     capi.sdpa_fwd(d)
     capi.sync(dev)
     out = to.to_f32()
-    for t in (tq.buf, tk.buf, tv.buf, to.buf, tl, tm, ws, tql):
+    lse = tlse.to_numpy(np.float32, (B, Hq, Sq)) if return_lse else None
+    for t in (tq.buf, tk.buf, tv.buf, to.buf, tl, tm, ws, tql, tlse):
         if t is not None:
             t.free()
+    info = {"impl": chosen, "splits": splits, "workspace_bytes": nbytes}
+    if return_lse:
+        return (out, lse, info) if return_info else (out, lse)
     if return_info:
-        return out, {"impl": chosen, "splits": splits, "workspace_bytes": nbytes}
+        return out, info
     return out

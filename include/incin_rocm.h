@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define INCIN_ROCM_ABI_VERSION 2
+#define INCIN_ROCM_ABI_VERSION 3
 
 /* ---- status codes (mapped to incin_core::Error variants by the Rust side;
  *      crates/incin-core/src/err.rs:109-223) --------------------------------- */
@@ -171,6 +171,10 @@ typedef struct {
     int32_t num_splits;            /* 0 = library chooses */
     int32_t impl;                  /* INCIN_ROCM_IMPL_*; AUTO unless a test pins a kernel */
     const int32_t* q_lens;         /* nullable device pointer, B entries: rows at and beyond are padding */
+    float* lse;                    /* nullable device pointer, contiguous f32 [B, Hq, Sq]: receives log sum_j exp(x_ij) of
+                                      every row (natural log of the softmax normaliser; -inf for a row with no visible
+                                      key) - what incin_rocm_sdpa_bwd needs from the forward.  Written by the generic and
+                                      the MFMA prefill kernels; AUTO keeps to those when it is set */
 } incin_rocm_sdpa_desc_t;
 
 /* Validates the descriptor and reports the scratch bytes and the split count the

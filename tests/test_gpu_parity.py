@@ -239,6 +239,29 @@ def test_padded_queries(gpu, impl, causal):
     assert np.array_equal(np.nan_to_num(same, nan=7.0), np.nan_to_num(plain, nan=7.0))
 
 
+@pytest.mark.parametrize("impl", [capi.IMPL_AUTO, capi.IMPL_GENERIC] + MFMA_IMPLS)
+def test_row_normalisers(gpu, impl):
+    """lse = log sum_j exp(x_ij) of every row, the forward's by-product that the backward needs."""
+    from oracle import sdpa_backward as BW
+    B, Hq, Hkv, Sq, Skv, D = 2, 4, 2, 300, 420, 128
+    q, k, v = inputs(51, B, Hq, Hkv, Sq, Skv, D, D, capi.BF16)
+    lens = np.array([420, 77], np.int32)
+    for causal in (False, True):
+        got, lse, info = host.sdpa(q, k, v, capi.BF16, causal=causal, kv_lens=lens, impl=impl, return_lse=True, return_info=True)
+        assert info["impl"] != capi.IMPL_SPLITKV
+        want = BW.logsumexp(q.reshape(B, Hkv, 2, Sq, D), k[:, :, None], causal=causal, kv_lens=lens.reshape(B, 1, 1)).reshape(B, Hq, Sq)
+        fin = np.isfinite(want)
+        assert np.array_equal(np.isfinite(lse), fin) and np.all(lse[~fin] == -np.inf)
+        err = float(np.abs(lse[fin] - want[fin]).max())
+        say("row normalisers impl %d causal %s: max-abs err %.3e" % (impl, causal, err))
+        assert err <= 2e-2                # the scores come from bf16 products of a Q pre-multiplied by the scale in bf16
+        plain = host.sdpa(q, k, v, capi.BF16, causal=causal, kv_lens=lens, impl=info["impl"])
+        assert np.array_equal(np.nan_to_num(got, nan=7.0), np.nan_to_num(plain, nan=7.0))
+    # a decode-shaped request with lse keeps away from the split-KV kernel, which does not write it
+    _, _, info = host.sdpa(q[:, :, :1], k, v, capi.BF16, return_lse=True, return_info=True)
+    assert info["impl"] != capi.IMPL_SPLITKV
+
+
 # ---- split-KV decode -----------------------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", [capi.BF16, capi.F16, capi.F32])
