@@ -30,6 +30,7 @@ EXPORTS = [
     "incin_rocm_graph_begin", "incin_rocm_graph_end", "incin_rocm_graph_launch", "incin_rocm_graph_destroy",
     "incin_rocm_sdpa_workspace", "incin_rocm_sdpa_fwd",
     "incin_rocm_sizeof_kv_append_desc", "incin_rocm_kv_append",
+    "incin_rocm_sizeof_sdpa_bwd_desc", "incin_rocm_sdpa_bwd_workspace", "incin_rocm_sdpa_bwd",
 ]
 
 
@@ -69,6 +70,18 @@ class SdpaDesc(C.Structure):
         ("impl", C.c_int32),
         ("q_lens", C.c_void_p),
         ("lse", C.c_void_p),
+    ]
+
+
+class SdpaBwdDesc(C.Structure):
+    _fields_ = [
+        ("fwd", SdpaDesc),
+        ("d_o", C.c_void_p), ("d_o_stride", C.c_int64 * 3),
+        ("d_q", C.c_void_p), ("d_q_stride", C.c_int64 * 3),
+        ("d_k", C.c_void_p), ("d_k_stride", C.c_int64 * 3),
+        ("d_v", C.c_void_p), ("d_v_stride", C.c_int64 * 3),
+        ("workspace", C.c_void_p),
+        ("workspace_bytes", C.c_size_t),
     ]
 
 
@@ -136,6 +149,9 @@ def load():
                                               C.POINTER(C.c_int32)]
     lib.incin_rocm_sdpa_fwd.argtypes = [C.POINTER(SdpaDesc), C.c_void_p]
     lib.incin_rocm_sizeof_kv_append_desc.restype = C.c_size_t
+    lib.incin_rocm_sizeof_sdpa_bwd_desc.restype = C.c_size_t
+    lib.incin_rocm_sdpa_bwd_workspace.argtypes = [C.POINTER(SdpaBwdDesc), C.POINTER(C.c_size_t)]
+    lib.incin_rocm_sdpa_bwd.argtypes = [C.POINTER(SdpaBwdDesc), C.c_void_p]
     lib.incin_rocm_kv_append.argtypes = [C.POINTER(KvAppendDesc), C.c_void_p]
     _lib = lib
     return lib
@@ -203,6 +219,16 @@ def sdpa_workspace(desc):
     nbytes, splits, impl = C.c_size_t(0), C.c_int32(0), C.c_int32(0)
     check(load().incin_rocm_sdpa_workspace(C.byref(desc), C.byref(nbytes), C.byref(splits), C.byref(impl)))
     return nbytes.value, splits.value, impl.value
+
+
+def sdpa_bwd_workspace(desc):
+    n = C.c_size_t()
+    check(load().incin_rocm_sdpa_bwd_workspace(C.byref(desc), C.byref(n)))
+    return n.value
+
+
+def sdpa_bwd(desc, stream=None):
+    check(load().incin_rocm_sdpa_bwd(C.byref(desc), stream))
 
 
 def kv_append(desc, stream=None):

@@ -188,6 +188,35 @@ int incin_rocm_sdpa_workspace(const incin_rocm_sdpa_desc_t* desc, size_t* bytes,
  * keeps alive until the stream has been synchronised. */
 int incin_rocm_sdpa_fwd(const incin_rocm_sdpa_desc_t* desc, void* stream);
 
+/* ---- attention backward --------------------------------------------------------
+ * The reference has no backward kernel for attention: its gradient is what walking the tape of the composed ops
+ * gives (crates/incin-backends/src/cpu/ops/shape_ops.rs:1245-1269 records matmul, mul_scalar, add, log_softmax,
+ * exp, matmul; crates/incin-backends/src/cpu/tape.rs:149-176 walks it).  This computes the same dq, dk, dv in
+ * three launches from q, k, v, the forward's output o and row normalisers lse, and the upstream gradient d_o.
+ *
+ * `fwd` is the forward's descriptor as it was launched with `lse` set (o and lse are inputs here); causal,
+ * kv_lens and the grouped-query layout carry over; d_k and d_v are summed over the query heads of a group.
+ * Covered: f16 / bf16, D == Dv == 128, no dense additive mask, no q_lens; anything else is
+ * INCIN_ROCM_EUNSUPPORTED.  A query row with no visible key (NaN in the forward) gets a zero gradient and
+ * contributes nothing to d_k and d_v, where the reference's tape would spread NaN over the whole head.
+ * The workspace holds one float per query row ([B, Hq, Sq]); d_q, d_k, d_v are fully overwritten. */
+typedef struct {
+    incin_rocm_sdpa_desc_t fwd;
+    const void* d_o;               /* [B, Hq, Sq, D], dtype of the operands */
+    int64_t d_o_stride[3];
+    void* d_q;                     /* [B, Hq, Sq, D] */
+    int64_t d_q_stride[3];
+    void* d_k;                     /* [B, Hkv, Skv, D] */
+    int64_t d_k_stride[3];
+    void* d_v;                     /* [B, Hkv, Skv, D] */
+    int64_t d_v_stride[3];
+    void* workspace;
+    size_t workspace_bytes;
+} incin_rocm_sdpa_bwd_desc_t;
+size_t incin_rocm_sizeof_sdpa_bwd_desc(void);
+int incin_rocm_sdpa_bwd_workspace(const incin_rocm_sdpa_bwd_desc_t* desc, size_t* bytes);
+int incin_rocm_sdpa_bwd(const incin_rocm_sdpa_bwd_desc_t* desc, void* stream);
+
 /* ---- key/value cache append ----------------------------------------------------
  * No counterpart in the reference (it has no cache: a decode loop there concatenates tensors,
  * TensorOps::cat, and re-runs the operator).  Copies S_new new key and value rows per (batch, kv head) into

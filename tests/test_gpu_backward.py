@@ -1,0 +1,100 @@
+"""Attention backward through the C ABI against the backward oracle (the gradients the reference's tape walk
+gives, oracle/sdpa_backward.py): dq, dk, dv for f16 / bf16 operands, D = 128, grouped queries, causal masks with
+Sq != Skv, ragged key counts.  Tolerance: 2e-2 relative to the largest magnitude of the gradient tensor compared
+(bf16 / f16 inputs, bf16 / f16 probabilities and dS as matrix operands, f32 accumulation)."""
+import sys
+
+import numpy as np
+import pytest
+
+from incin_amd import capi, dtypes, host
+from oracle import sdpa_backward as BW
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print(msg, file=sys.stderr, flush=True)
+
+
+def make(seed, B, Hq, Hkv, Sq, Skv, D, dtype):
+    r = np.random.Generator(np.random.PCG64(seed))
+    mk = lambda *s: dtypes.round_to(r.standard_normal(s, dtype=np.float32), dtype)
+    return mk(B, Hq, Sq, D), mk(B, Hkv, Skv, D), mk(B, Hkv, Skv, D), mk(B, Hq, Sq, D)
+
+
+def compare(name, got, ref, tol=2e-2):
+    ref = np.asarray(ref, np.float64)
+    scale = float(np.abs(ref).max()) or 1.0
+    err = float(np.abs(got - ref).max()) / scale
+    say("   %s: max-abs err / max|ref| = %.3e (max|ref| %.3g)" % (name, err, scale))
+    assert not np.isnan(got).any(), name
+    assert err <= tol, "%s: %.3e" % (name, err)
+
+
+@pytest.mark.parametrize("dtype", [capi.BF16, capi.F16])
+@pytest.mark.parametrize("shape", [
+    # B, Hq, Hkv, Sq, Skv, causal, kv_lens
+    (1, 1, 1, 32, 32, False, None),
+    (1, 1, 1, 128, 128, True, None),
+    (2, 4, 4, 200, 333, False, None),
+    (2, 4, 2, 300, 300, True, None),
+    (1, 8, 2, 130, 450, True, None),                  # Sq < Skv: causal alignment, grouped queries
+    (3, 2, 2, 257, 257, True, [257, 100, 31]),
+    (2, 2, 1, 64, 700, False, [700, 1]),
+], ids=["tiny", "one_tile_causal", "rect", "gqa_causal", "gqa_rect_causal", "ragged_causal", "ragged"])
+def test_backward_against_the_oracle(gpu, dtype, shape):
+    B, Hq, Hkv, Sq, Skv, causal, lens = shape
+    D, G = 128, Hq // Hkv
+    say("backward: %s dtype %d" % (shape, dtype))
+    q, k, v, go = make(11, B, Hq, Hkv, Sq, Skv, D, dtype)
+    lens_a = None if lens is None else np.asarray(lens, np.int32)
+    out, dq, dk, dv = host.sdpa_backward(q, k, v, go, dtype, causal=causal, kv_lens=lens_a)
+    rq, rk, rv = BW.sdpa_backward(q.reshape(B, Hkv, G, Sq, D), k[:, :, None], v[:, :, None], go.reshape(B, Hkv, G, Sq, D),
+                                  causal=causal, kv_lens=None if lens is None else lens_a.reshape(B, 1, 1))
+    compare("dq", dq, rq.reshape(B, Hq, Sq, D))
+    compare("dk", dk, rk.reshape(B, Hkv, Skv, D))
+    compare("dv", dv, rv.reshape(B, Hkv, Skv, D))
+    if lens is not None:
+        for b in range(B):
+            assert not dk[b, :, lens[b]:].any() and not dv[b, :, lens[b]:].any()      # padded keys: exactly zero
+
+
+def test_rows_without_visible_keys_get_zero_gradients(gpu):
+    # Sq > Skv under causal alignment: the first Sq - Skv rows see nothing (NaN in the forward).  They get a zero dq
+    # and contribute nothing to dk, dv; the other rows are what the oracle gives for them alone.
+    B, H, Sq, Skv, D = 1, 2, 96, 40, 128
+    q, k, v, go = make(12, B, H, H, Sq, Skv, D, capi.BF16)
+    out, dq, dk, dv = host.sdpa_backward(q, k, v, go, capi.BF16, causal=True)
+    dead = Sq - Skv
+    assert np.isnan(out[:, :, :dead]).all() and not np.isnan(out[:, :, dead:]).any()
+    assert not dq[:, :, :dead].any()
+    rq, rk, rv = BW.sdpa_backward(q[:, :, dead:], k, v, go[:, :, dead:], causal=True)
+    compare("dq (live rows)", dq[:, :, dead:], rq)
+    compare("dk", dk, rk)
+    compare("dv", dv, rv)
+    # a sequence with no keys at all: zero gradients everywhere for it
+    lens = np.array([0], np.int32)
+    out, dq, dk, dv = host.sdpa_backward(q[:, :, :40], k, v, go[:, :, :40], capi.BF16, kv_lens=lens)
+    assert not dq.any() and not dk.any() and not dv.any()
+
+
+def test_backward_at_a_few_thousand_tokens(gpu):
+    B, Hq, Hkv, S, D = 1, 4, 2, 2048, 128
+    q, k, v, go = make(13, B, Hq, Hkv, S, S, D, capi.BF16)
+    out, dq, dk, dv = host.sdpa_backward(q, k, v, go, capi.BF16, causal=True)
+    rq, rk, rv = BW.sdpa_backward(q.reshape(B, Hkv, 2, S, D), k[:, :, None], v[:, :, None], go.reshape(B, Hkv, 2, S, D), causal=True)
+    compare("dq", dq, rq.reshape(B, Hq, S, D))
+    compare("dk", dk, rk.reshape(B, Hkv, S, D))
+    compare("dv", dv, rv.reshape(B, Hkv, S, D))
+
+
+def test_backward_refuses_what_it_does_not_cover(gpu):
+    q, k, v, go = make(14, 1, 1, 1, 32, 32, 64, capi.BF16)
+    with pytest.raises(capi.RocmError) as e:
+        host.sdpa_backward(q, k, v, go, capi.BF16)
+    assert e.value.code == capi.EUNSUPPORTED and "D == Dv == 128" in e.value.message
+    q, k, v, go = make(14, 1, 1, 1, 32, 32, 128, capi.F32)
+    with pytest.raises(capi.RocmError) as e:
+        host.sdpa_backward(q, k, v, go, capi.F32)
+    assert e.value.code == capi.EUNSUPPORTED
