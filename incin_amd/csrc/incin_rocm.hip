@@ -506,7 +506,7 @@ int incin_rocm_sdpa_bwd_workspace(const incin_rocm_sdpa_bwd_desc_t* bd, size_t* 
     *bytes = 0;
     bool empty = false;
     if (int rc = check_bwd(bd, &empty)) return rc;
-    if (!empty) *bytes = (size_t)(bd->fwd.B * bd->fwd.Hq * bd->fwd.Sq) * sizeof(float);
+    if (!empty) *bytes = 2 * (size_t)(bd->fwd.B * bd->fwd.Hq * bd->fwd.Sq) * sizeof(float);
     return 0;
 }
 
@@ -515,7 +515,7 @@ int incin_rocm_sdpa_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, void* stream)
     bool empty = false;
     if (int rc = check_bwd(bd, &empty)) return rc;
     if (empty) return 0;        // (gradients of an empty problem: nothing to write)
-    const size_t need = (size_t)(bd->fwd.B * bd->fwd.Hq * bd->fwd.Sq) * sizeof(float);
+    const size_t need = 2 * (size_t)(bd->fwd.B * bd->fwd.Hq * bd->fwd.Sq) * sizeof(float);      // two f32 per query row
     if (!bd->workspace || bd->workspace_bytes < need || !aligned16(bd->workspace))
         return fail(INCIN_ROCM_EWORKSPACE, "scaled_dot_product_attention backward: %zu workspace bytes needed (16-byte aligned), %zu given",
                     need, bd->workspace ? bd->workspace_bytes : (size_t)0);
@@ -527,7 +527,8 @@ int incin_rocm_sdpa_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, void* stream)
     memset(&bp, 0, sizeof(bp));
     fill_params(&bd->fwd, plan, &bp.f);
     bp.d_o = bd->d_o; bp.d_q = bd->d_q; bp.d_k = bd->d_k; bp.d_v = bd->d_v;
-    bp.delta = (float*)bd->workspace;
+    bp.neg_l2 = (float*)bd->workspace;
+    bp.neg_delta = bp.neg_l2 + bd->fwd.B * bd->fwd.Hq * bd->fwd.Sq;
     bp.do_sb = bd->d_o_stride[0]; bp.do_sh = bd->d_o_stride[1]; bp.do_ss = bd->d_o_stride[2];
     bp.dq_sb = bd->d_q_stride[0]; bp.dq_sh = bd->d_q_stride[1]; bp.dq_ss = bd->d_q_stride[2];
     bp.dk_sb = bd->d_k_stride[0]; bp.dk_sh = bd->d_k_stride[1]; bp.dk_ss = bd->d_k_stride[2];

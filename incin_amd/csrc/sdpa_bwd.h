@@ -12,7 +12,8 @@ struct SdpaBwdParams {
     void* d_q;
     void* d_k;
     void* d_v;
-    float* delta;                  // workspace, [B, Hq, Sq]
+    float* neg_l2;                 // workspace, [B, Hq, Sq]: -L_i log2(e) (the normalisers, negated, in log2 units)
+    float* neg_delta;              // workspace, [B, Hq, Sq]: -D_i = -(dO_i . O_i)
     int64_t do_sb, do_sh, do_ss;
     int64_t dq_sb, dq_sh, dq_ss;
     int64_t dk_sb, dk_sh, dk_ss;

@@ -41,7 +41,10 @@ __global__ __launch_bounds__(256) void sdpa_bwd_delta_kernel(SdpaBwdParams p)
     for (int d = lane; d < p.f.D; d += 64) acc = fmaf((float)o[d], (float)g[d], acc);
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 64);
-    if (lane == 0) p.delta[row] = acc;
+    if (lane == 0) {
+        p.neg_delta[row] = -acc;
+        p.neg_l2[row] = -p.f.lse[row] * 1.4426950408889634f;
+    }
 }
 
 // What both big kernels share: 64-row tiles of two tensors streamed through LDS in the forward's layout (rows of
@@ -85,16 +88,14 @@ struct BwdTiles {
     }
     // start the copy of rows [row0, row0 + 64) of tensor `which` (base pointer of the head, `rows` rows of `stride`
     // elements) into `dst`; rows at and beyond `rows` arrive as zeros
-    __device__ __forceinline__ void issue(int which, const T* base, int64_t stride, int rows, int row0, char* dst, int wave) const
+    __device__ __forceinline__ void issue(int which, const T* base, int64_t stride, int rows, int row0, unsigned dst, int wave) const
     {
         int64_t rem = (int64_t)(rows - row0 - 1) * stride * 2 + 256;
         if (rem > 0x7fffffffLL) rem = 0x7fffffffLL;
         if (rem < 0) rem = 0;
-        __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)base + (int64_t)row0 * stride * 2), 0, (int)rem, 0x00020000);
+        const uint4v r = dma_descriptor((const char*)base + (int64_t)row0 * stride * 2, (int)rem);
 #pragma unroll
-        for (int c = 0; c < LPW; ++c)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)(dst + (wave * LPW + c) * 1024), 16,
-                                                     voff[which][c], 0, 0, 0);
+        for (int c = 0; c < LPW; ++c) dma_copy16(r, dst + (wave * LPW + c) * 1024, voff[which][c]);
     }
     // A operand by rows: rows 32*blk + ql of the tile, k-step s
     __device__ __forceinline__ vec8 rows_op(int which, const char* tile, int blk, int s) const
@@ -177,8 +178,8 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
         }
     }
     const int64_t stat = ((int64_t)b * p.Hq + hq) * Sq + qi;
-    const float l2 = p.lse[stat] * 1.4426950408889634f;
-    const float dlt = bp.delta[stat];
+    const float l2 = -bp.neg_l2[stat];
+    const float dlt = -bp.neg_delta[stat];
 
     floatx16 dq_acc[NDB];
 #pragma unroll
@@ -189,17 +190,18 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
 #pragma unroll
     for (int r = 0; r < 16; ++r) zero16[r] = 0.0f;
 
+    const unsigned lds0 = lds_address(smem);
     if (n_tiles > 0) {
-        tl.issue(0, kp, p.k_ss, Skv, 0, smem, wave);
-        tl.issue(1, vp, p.v_ss, Skv, 0, smem + 2 * L::TILE_BYTES, wave);
+        tl.issue(0, kp, p.k_ss, Skv, 0, lds0, wave);
+        tl.issue(1, vp, p.v_ss, Skv, 0, lds0 + 2 * L::TILE_BYTES, wave);
     }
     for (int t = 0; t < n_tiles; ++t) {
         // K(t), V(t) have landed for everyone and everyone is done with tile t-1: the other pair of buffers is free
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         if (t + 1 < n_tiles) {
-            tl.issue(0, kp, p.k_ss, Skv, (t + 1) * PF_BN, smem + ((t + 1) & 1) * L::TILE_BYTES, wave);
-            tl.issue(1, vp, p.v_ss, Skv, (t + 1) * PF_BN, smem + (2 + ((t + 1) & 1)) * L::TILE_BYTES, wave);
+            tl.issue(0, kp, p.k_ss, Skv, (t + 1) * PF_BN, lds0 + ((t + 1) & 1) * L::TILE_BYTES, wave);
+            tl.issue(1, vp, p.v_ss, Skv, (t + 1) * PF_BN, lds0 + (2 + ((t + 1) & 1)) * L::TILE_BYTES, wave);
         }
         if (t >= n_act) continue;
         const char* kt = smem + (t & 1) * L::TILE_BYTES;
@@ -248,7 +250,15 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
 
 // ---- dK, dV ---------------------------------------------------------------------------------------------------------------
 constexpr int BWD_KEYS = 128;      // keys per workgroup of the dK/dV kernel (32 per wavefront)
+constexpr int BWD_RING = 8;        // matrix operands in flight from LDS (reads run this many matrix instructions ahead)
 
+// One wavefront per SIMD, so nothing hides a latency but the wavefront's own instruction order.  A 64-query tile is
+// 64 matrix instructions per wavefront in four runs of 16:
+//   A0  S, dP of query rows 0-31        A1  S, dP of rows 32-63, with P and dS of rows 0-31 on the vector ALU underneath
+//   B0  dV, dK from rows 0-31, with P and dS of rows 32-63 underneath                  B1  dV, dK from rows 32-63
+// and the LDS operand of instruction i + BWD_RING is requested right after instruction i is issued.  The S and dP
+// accumulators do not start from zero but from -L_i log2(e) and -D_i (staged per tile next to the Q and dO rows), so
+// P = exp2(S) and dS = P * dP need no subtraction.
 template <typename T>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
@@ -256,17 +266,32 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
 #if defined(__HIP_DEVICE_COMPILE__)
     typedef typename Mma<T>::vec8 vec8;
     typedef PfLayout<128> L;
-    constexpr int NSTEP = 8, NDB = 4;
+    typedef float float4v __attribute__((ext_vector_type(4)));
+    constexpr int NSTEP = 8, NDB = 4, R = BWD_RING;
+    constexpr int STAGE = 2 * L::TILE_BYTES + 1024;     // Q rows, dO rows, 64 x -L_i log2(e), 64 x -D_i (and padding)
     const SdpaParams& p = bp.f;
-    __shared__ __attribute__((aligned(1024))) char smem[4 * L::TILE_BYTES];      // Q buffers 0, 1, dO buffers 0, 1
+    __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int ql = lane & 31, g = lane >> 5;
     const int Sq = p.Sq, Skv = p.Skv;
     const int nkb = (Skv + BWD_KEYS - 1) / BWD_KEYS;
-    const int kblk = blockIdx.x % nkb;
-    const int bhkv = blockIdx.x / nkb;
+    // Workgroups reach the 8 XCDs round-robin by id.  All key blocks of a (batch, KV head) pair read the same Q and dO
+    // rows, so a pair is given to one XCD (pair h to XCD h % 8) and its key blocks run there side by side, the
+    // block with the most visible queries (the first, under a causal mask) first.
+    int kblk, bhkv;
+    {
+        const int pairs = p.B * p.Hkv;
+        if ((pairs & 7) == 0) {
+            const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+            kblk = slot % nkb;
+            bhkv = (slot / nkb) * 8 + xcd;
+        } else {
+            kblk = blockIdx.x % nkb;
+            bhkv = blockIdx.x / nkb;
+        }
+    }
     const int hkv = bhkv % p.Hkv, b = bhkv / p.Hkv;
     const int j0 = kblk * BWD_KEYS;
     const int my_j = j0 + wave * 32 + ql;              // this lane's key
@@ -283,6 +308,9 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
     const int i_begin_wg = p.causal ? clampi(j0 - coff, 0, Sq) : 0;
     const int i_begin_wave = p.causal ? clampi(j0 + wave * 32 - coff, 0, Sq) : 0;
     const bool wave_has_keys = j0 + wave * 32 < kv_len;
+    // first query row that sees every key of this wavefront (tiles from there on, wholly inside Sq, need no mask)
+    const bool wave_keys_whole = j0 + wave * 32 + 31 < kv_len;
+    const int i_all_wave = p.causal ? max(j0 + wave * 32 + 31 - coff, 0) : 0;
     const int t_begin = i_begin_wg / PF_BN;
     const int n_qt = (Sq + PF_BN - 1) / PF_BN;
     const int tiles_per_head = j0 < kv_len ? max(n_qt - t_begin, 0) : 0;
@@ -307,73 +335,155 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
             vreg[s] = *(const vec8*)(vrow + s * 16);
         }
     }
-    const bool key_ok = my_j < kv_len;
+    // rows i with lo_i <= i < Sq see this lane's key
+    const int lo_i = my_j < kv_len ? (p.causal ? my_j - coff : 0) : 0x7fffffff;
 
-    floatx16 dk_acc[NDB], dv_acc[NDB], zero16;
+    floatx16 dk_acc[NDB], dv_acc[NDB];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) zero16[r] = 0.0f;
+    for (int db = 0; db < NDB; ++db)
 #pragma unroll
-    for (int db = 0; db < NDB; ++db) { dk_acc[db] = zero16; dv_acc[db] = zero16; }
+        for (int r = 0; r < 16; ++r) { dk_acc[db][r] = 0.0f; dv_acc[db][r] = 0.0f; }
 
     auto head_of = [&](int t) { return hkv * p.G + t / tiles_per_head; };
     auto row0_of = [&](int t) { return (t_begin + t % tiles_per_head) * PF_BN; };
+    const unsigned lds0 = lds_address(smem);
     auto issue = [&](int t) __attribute__((always_inline)) {
-        const int hq = head_of(t);
+        const int hq = head_of(t), r0 = row0_of(t);
         const T* qp = (const T*)p.q + (int64_t)b * p.q_sb + (int64_t)hq * p.q_sh;
         const T* gp = (const T*)bp.d_o + (int64_t)b * bp.do_sb + (int64_t)hq * bp.do_sh;
-        tl.issue(0, qp, p.q_ss, Sq, row0_of(t), smem + (t & 1) * L::TILE_BYTES, wave);
-        tl.issue(1, gp, bp.do_ss, Sq, row0_of(t), smem + (2 + (t & 1)) * L::TILE_BYTES, wave);
+        const unsigned st = lds0 + (t & 1) * STAGE;
+        tl.issue(0, qp, p.q_ss, Sq, r0, st, wave);
+        tl.issue(1, gp, bp.do_ss, Sq, r0, st + L::TILE_BYTES, wave);
+        if (wave < 2) {         // 64 floats of one of the two per-row arrays; rows past Sq arrive as zeros
+            const float* src = (wave == 0 ? bp.neg_l2 : bp.neg_delta) + ((int64_t)b * p.Hq + hq) * Sq + r0;
+            dma_copy4(dma_descriptor(src, (Sq - r0) * 4), st + 2 * L::TILE_BYTES + wave * 256, lane * 4);
+        }
+    };
+
+    constexpr int SG_MFMA = 0x8, SG_VALU = 0x2, SG_TRANS = 0x400, SG_DSR = 0x100;
+#define SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
+
+    auto tile = [&](int t, auto MASKED_) __attribute__((always_inline)) {
+        constexpr bool MASKED = decltype(MASKED_)::value;
+        const char* qt = smem + (t & 1) * STAGE;
+        const char* gt = qt + L::TILE_BYTES;
+        const char* nl = gt + L::TILE_BYTES;
+        const int i0 = row0_of(t);
+        // matrix instruction i of the tile: its LDS operand ...
+        vec8 ring[R];
+        auto fetch = [&](int i) __attribute__((always_inline)) {
+            if (i < 32) {
+                const int qb = i / 16, s = (i % 16) / 2, which = i % 2;
+                ring[i % R] = tl.rows_op(which, which ? gt : qt, qb, s);
+            } else {
+                const int j = i - 32, qb = j / 16, h = (j % 16) / 8, db = (j % 8) / 2, which = 1 - j % 2;
+                ring[i % R] = tl.tr_op(which, which ? gt : qt, db, 2 * qb + h);
+            }
+        };
+        floatx16 sa[2], da[2];
+        vec8 pp[2][2], ds[2][2];
+        // ... and the instruction itself
+        auto mma = [&](int i) __attribute__((always_inline)) {
+            if (i < 32) {
+                const int qb = i / 16, s = (i % 16) / 2;
+                if (i % 2 == 0) sa[qb] = Mma<T>::run(ring[i % R], kreg[s], sa[qb]);
+                else da[qb] = Mma<T>::run(ring[i % R], vreg[s], da[qb]);
+            } else {
+                const int j = i - 32, qb = j / 16, h = (j % 16) / 8, db = (j % 8) / 2;
+                if (j % 2 == 0) dv_acc[db] = Mma<T>::run(ring[i % R], pp[qb][h], dv_acc[db]);
+                else dk_acc[db] = Mma<T>::run(ring[i % R], ds[qb][h], dk_acc[db]);
+            }
+        };
+        // P and dS of register r of query block qb: row i0 + 32*qb + 8*(r/4) + 4*g + (r%4)
+        const int rel_lo = lo_i - i0 - 4 * g, rel_hi = Sq - i0 - 4 * g;
+        auto soft = [&](int qb, int r) __attribute__((always_inline)) {
+            const float pr = __builtin_amdgcn_exp2f(sa[qb][r]);
+            const float dsv = pr * da[qb][r];
+            if (MASKED) {
+                // (selected, not multiplied by zero: a row without visible keys has NaN in D_i and P = +inf)
+                const int kofs = 32 * qb + 8 * (r / 4) + (r % 4);
+                const bool seen = kofs >= rel_lo && kofs < rel_hi;
+                pp[qb][r / 8][r % 8] = (T)(seen ? pr : 0.0f);
+                ds[qb][r / 8][r % 8] = (T)(seen ? dsv : 0.0f);
+            } else {
+                pp[qb][r / 8][r % 8] = (T)pr;
+                ds[qb][r / 8][r % 8] = (T)dsv;
+            }
+        };
+
+        // accumulators start from -L_i log2(e) and -D_i
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                const float4v a = *(const float4v*)(nl + (32 * qb + 8 * r4 + 4 * g) * 4);
+                const float4v d = *(const float4v*)(nl + 256 + (32 * qb + 8 * r4 + 4 * g) * 4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { sa[qb][4 * r4 + e] = a[e]; da[qb][4 * r4 + e] = d[e]; }
+            }
+#pragma unroll
+        for (int i = 0; i < R; ++i) fetch(i);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {          // A0
+            mma(i);
+            fetch(i + R);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 16; i < 32; ++i) {         // A1 over the vector work of rows 0-31
+            mma(i);
+            fetch(i + R);
+            soft(0, i - 16);
+        }
+        if (!MASKED) {
+#pragma unroll
+            for (int i = 16; i < 32; ++i) {
+                SGB(SG_MFMA, 1);
+                if (i + R < 32) SGB(SG_DSR, 1);
+                else SGB(SG_DSR, 2);         // (a transposed operand is two reads)
+                SGB(SG_TRANS, 1);
+                SGB(SG_VALU, 2);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 32; i < 48; ++i) {         // B0 over the vector work of rows 32-63
+            mma(i);
+            fetch(i + R);
+            soft(1, i - 32);
+        }
+        if (!MASKED) {
+#pragma unroll
+            for (int i = 32; i < 48; ++i) {
+                SGB(SG_MFMA, 1);
+                SGB(SG_DSR, 2);
+                SGB(SG_TRANS, 1);
+                SGB(SG_VALU, 2);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 48; i < 64; ++i) {         // B1
+            mma(i);
+            if (i + R < 64) fetch(i + R);
+        }
+        __builtin_amdgcn_sched_barrier(0);
     };
 
     if (n_tiles > 0) issue(0);
     for (int t = 0; t < n_tiles; ++t) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        // tile t has landed for everyone and everyone is done with tile t-1: the other stage is free
+        __builtin_amdgcn_s_waitcnt(0x0F70);             // vmcnt(0)
+        asm volatile("" ::: "memory");
         __syncthreads();
         if (t + 1 < n_tiles) issue(t + 1);
         const int i0 = row0_of(t);
-        if (!wave_has_keys || i0 + PF_BN <= i_begin_wave) continue;      // no row of this tile sees a key of this wavefront
-        const char* qt = smem + (t & 1) * L::TILE_BYTES;
-        const char* gt = smem + (2 + (t & 1)) * L::TILE_BYTES;
-        const int64_t stat0 = ((int64_t)b * p.Hq + head_of(t)) * Sq;
-#pragma unroll
-        for (int qb = 0; qb < 2; ++qb) {
-            floatx16 s_acc = zero16, dp_acc = zero16;
-#pragma unroll
-            for (int s = 0; s < NSTEP; ++s) {
-                s_acc = Mma<T>::run(tl.rows_op(0, qt, qb, s), kreg[s], s_acc);
-                dp_acc = Mma<T>::run(tl.rows_op(1, gt, qb, s), vreg[s], dp_acc);
-            }
-            // register r is query row i0 + 32*qb + 8*(r/4) + 4*g + (r%4); this lane's key is my_j
-            vec8 pp[2], ds[2];
-#pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-                const int i4 = i0 + 32 * qb + 8 * r4 + 4 * g;
-                float l2[4], dl[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int i = min(i4 + e, Sq - 1);
-                    l2[e] = p.lse[stat0 + i] * 1.4426950408889634f;
-                    dl[e] = bp.delta[stat0 + i];
-                }
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int r = 4 * r4 + e, i = i4 + e;
-                    const float pr = __builtin_amdgcn_exp2f(s_acc[r] - l2[e]);
-                    const bool seen = key_ok && i < Sq && (!p.causal || my_j <= i + coff);
-                    // (selected, not multiplied by zero: a row without visible keys has NaN in D_i and +inf here)
-                    pp[r / 8][r % 8] = (T)(seen ? pr : 0.0f);
-                    ds[r / 8][r % 8] = (T)(seen ? pr * (dp_acc[r] - dl[e]) : 0.0f);
-                }
-            }
-#pragma unroll
-            for (int h = 0; h < 2; ++h)
-#pragma unroll
-                for (int db = 0; db < NDB; ++db) {
-                    dv_acc[db] = Mma<T>::run(tl.tr_op(1, gt, db, 2 * qb + h), pp[h], dv_acc[db]);
-                    dk_acc[db] = Mma<T>::run(tl.tr_op(0, qt, db, 2 * qb + h), ds[h], dk_acc[db]);
-                }
-        }
+        if (!(wave_has_keys && i0 + PF_BN > i_begin_wave)) continue;      // no row of this tile sees a key of this wavefront
+        if (wave_keys_whole && i0 >= i_all_wave && i0 + PF_BN <= Sq) tile(t, std::false_type{});
+        else tile(t, std::true_type{});
     }
+#undef SGB
 
     if (my_j < Skv) {
         T* krow = dkp + (int64_t)my_j * bp.dk_ss;

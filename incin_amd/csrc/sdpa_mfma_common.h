@@ -73,6 +73,34 @@ template <int D> struct PfLayout {
     }
 };
 
+// One wavefront-wide global -> LDS copy (64 lanes x 16 bytes land at lds_addr .. lds_addr + 1023 in lane order; lanes
+// whose offset is outside the descriptor's range deliver zeros).  Issued through inline assembly on purpose: the
+// compiler makes every LDS access it cannot prove disjoint from a copy it knows of wait until that copy has landed -
+// for the transposing reads that is a full memory latency in the middle of every tile - whereas the kernels here
+// order copies and reads themselves (s_waitcnt vmcnt + barrier before a buffer is read, a barrier after its last read
+// before it is refilled).  Counting the copy in vmcnt stays correct for the compiler's own loads: memory operations
+// complete in order, so its waits only become stricter.
+__device__ __forceinline__ uint4v dma_descriptor(const void* base, int bytes)
+{
+    const unsigned long long a = (unsigned long long)base;
+    const uint4v d = {(unsigned)a, (unsigned)(a >> 32) & 0xffffu, (unsigned)bytes, 0x00020000u};
+    return d;
+}
+__device__ __forceinline__ unsigned lds_address(const void* p)
+{
+    return (unsigned)(unsigned long long)(const __attribute__((address_space(3))) char*)p;
+}
+__device__ __forceinline__ void dma_copy16(uint4v desc, unsigned lds_addr, int byte_offset)
+{
+    // (one wait state between the write of m0 and the copy that reads it)
+    asm volatile("s_nop 0\n\tbuffer_load_dwordx4 %0, %1, 0 offen lds" ::"v"(byte_offset), "s"(desc), "{m0}"(lds_addr) : "memory");
+}
+// The same for 64 lanes x 4 bytes (256 bytes of LDS).
+__device__ __forceinline__ void dma_copy4(uint4v desc, unsigned lds_addr, int byte_offset)
+{
+    asm volatile("s_nop 0\n\tbuffer_load_dword %0, %1, 0 offen lds" ::"v"(byte_offset), "s"(desc), "{m0}"(lds_addr) : "memory");
+}
+
 // CU count of the current device (256 if the query fails: only launch geometry depends on it).
 inline int device_cus()
 {

@@ -134,20 +134,18 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     auto issue_k = [&](int t, int buf) __attribute__((always_inline)) {
         int64_t rem = (int64_t)(Skv - t * PF_BN - 1) * p.k_ss * 2 + D * 2;   // bytes to the end of the last valid row: loads past that return 0
         if (rem > 0x7fffffffLL) rem = 0x7fffffffLL;
-        __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)kp + t * k_tile_bytes), 0, (int)rem, 0x00020000);
-        char* dst = smem + buf * L::TILE_BYTES + wave * LPW * 1024;
+        const uint4v r = dma_descriptor((const char*)kp + t * k_tile_bytes, (int)rem);
+        const unsigned dst = lds_address(smem) + buf * L::TILE_BYTES + wave * LPW * 1024;
 #pragma unroll
-        for (int c = 0; c < LPW; ++c)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)(dst + c * 1024), 16, k_voff[c], 0, 0, 0);
+        for (int c = 0; c < LPW; ++c) dma_copy16(r, dst + c * 1024, k_voff[c]);
     };
     auto issue_v = [&](int t, int buf) __attribute__((always_inline)) {
         int64_t rem = (int64_t)(Skv - t * PF_BN - 1) * p.v_ss * 2 + D * 2;
         if (rem > 0x7fffffffLL) rem = 0x7fffffffLL;
-        __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)((const char*)vp + t * v_tile_bytes), 0, (int)rem, 0x00020000);
-        char* dst = smem + (2 + buf) * L::TILE_BYTES + wave * LPW * 1024;
+        const uint4v r = dma_descriptor((const char*)vp + t * v_tile_bytes, (int)rem);
+        const unsigned dst = lds_address(smem) + (2 + buf) * L::TILE_BYTES + wave * LPW * 1024;
 #pragma unroll
-        for (int c = 0; c < LPW; ++c)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)(dst + c * 1024), 16, v_voff[c], 0, 0, 0);
+        for (int c = 0; c < LPW; ++c) dma_copy16(r, dst + c * 1024, v_voff[c]);
     };
 
     // ---- LDS read addresses (bytes inside a tile buffer) ------------------------------------
@@ -375,7 +373,8 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     if (n_tiles > 0) {
         // prologue: K(0) first, then K(1), V(0) in flight; scores of tile 0
         issue_k(0, 0);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0), told to the compiler too: it then knows the Q rows have arrived
+        asm volatile("" ::: "memory");
         __syncthreads();
         if (n_tiles > 1) issue_k(1, 1);
         issue_v(0, 0);
