@@ -25,40 +25,50 @@
 namespace incin_rocm {
 
 // ---- D_i = dO_i . O_i ---------------------------------------------------------------------------------------------
+// Sixteen lanes per row (16 bytes of O and of dO each), four rows per wavefront.
 template <typename T>
 __global__ __launch_bounds__(256) void sdpa_bwd_delta_kernel(SdpaBwdParams p)
 {
-    const int lane = threadIdx.x & 63;
-    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);     // (b * Hq + hq) * Sq + i
+    typedef typename Mma<T>::vec8 vec8;
+    const int lane = threadIdx.x & 63, sub = lane & 15;
+    const int64_t row = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 4 + (lane >> 4);     // (b * Hq + hq) * Sq + i
     const int64_t rows = (int64_t)p.f.B * p.f.Hq * p.f.Sq;
-    if (row >= rows) return;
-    const int i = (int)(row % p.f.Sq);
-    const int64_t bh = row / p.f.Sq;
-    const int hq = (int)(bh % p.f.Hq), b = (int)(bh / p.f.Hq);
-    const T* o = (const T*)p.f.o + b * p.f.o_sb + hq * p.f.o_sh + (int64_t)i * p.f.o_ss;
-    const T* g = (const T*)p.d_o + b * p.do_sb + hq * p.do_sh + (int64_t)i * p.do_ss;
     float acc = 0.0f;
-    for (int d = lane; d < p.f.D; d += 64) acc = fmaf((float)o[d], (float)g[d], acc);
+    if (row < rows) {
+        const int i = (int)(row % p.f.Sq);
+        const int64_t bh = row / p.f.Sq;
+        const int hq = (int)(bh % p.f.Hq), b = (int)(bh / p.f.Hq);
+        const T* o = (const T*)p.f.o + b * p.f.o_sb + hq * p.f.o_sh + (int64_t)i * p.f.o_ss;
+        const T* g = (const T*)p.d_o + b * p.do_sb + hq * p.do_sh + (int64_t)i * p.do_ss;
+        for (int d = sub * 8; d < p.f.D; d += 128) {
+            const vec8 x = *(const vec8*)(o + d), y = *(const vec8*)(g + d);
 #pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 64);
-    if (lane == 0) {
-        p.neg_delta[row] = -acc;
-        p.neg_l2[row] = -p.f.lse[row] * 1.4426950408889634f;
+            for (int e = 0; e < 8; ++e) acc = fmaf((float)x[e], (float)y[e], acc);
+        }
+    }
+#pragma unroll
+    for (int off = 8; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 64);
+    if (row < rows && sub == 0) {
+        // A row without a visible key (L_i = -inf, O and so D_i NaN) gets -inf and 0: its P is then 0 everywhere.
+        const float l = p.f.lse[row];
+        p.neg_delta[row] = l == -INFINITY ? 0.0f : -acc;
+        p.neg_l2[row] = l == -INFINITY ? -INFINITY : -l * 1.4426950408889634f;
     }
 }
 
-// What both big kernels share: 64-row tiles of two tensors streamed through LDS in the forward's layout (rows of
-// 256 bytes, 16-byte chunks XOR-swizzled by fk in the first tensor's buffers and by fv in the second's), read either
-// by rows (16 bytes of one row per lane: an A operand whose M index is the row) or transposed (the gfx950
-// transposing read: an A operand whose M index is the column block).
+// What both big kernels share: 64-row tiles of two tensors streamed through LDS in the layout of the forward's K tiles
+// (rows of 256 bytes, 16-byte chunks XOR-swizzled by fk), read either by rows (16 bytes of one row per lane: an A
+// operand whose M index is the row) or transposed (the gfx950 transposing read: an A operand whose M index is the
+// column block).  fk serves both reads without bank conflicts: 16 consecutive rows put one logical chunk into 16
+// different slots, and the 4 rows x 64 bytes a half-wavefront transposes land in 4 different 64-byte column groups.
 template <typename T>
 struct BwdTiles {
     typedef typename Mma<T>::vec8 vec8;
     typedef PfLayout<128> L;
     static constexpr int NSTEP = 8, NDB = 4, LPW = L::LOADS_PER_WAVE;
 
-    int row_addr[2][NSTEP];        // [tensor][k-step]: byte offset of this lane's 16 bytes of row ql, chunk 2*s + g
-    int tr_addr[2][NDB][2];        // [tensor][column block][half]: byte offset of the transposing read
+    int row_addr[NSTEP];           // [k-step]: byte offset of this lane's 16 bytes of row ql, chunk 2*s + g
+    int tr_addr[NDB][2];           // [column block][half]: byte offset of the transposing read
     int voff[2][LPW];              // [tensor][load]: global byte offset of this lane's 16 bytes of a tile
 
     __device__ __forceinline__ void init(int wave, int lane, int64_t stride0, int64_t stride1)
@@ -66,8 +76,7 @@ struct BwdTiles {
         const int ql = lane & 31, g = lane >> 5, n = lane & 15, dh = (lane >> 4) & 1;
 #pragma unroll
         for (int s = 0; s < NSTEP; ++s) {
-            row_addr[0][s] = ql * L::ROWB + (((2 * s + g) ^ L::fk(ql)) << 4);
-            row_addr[1][s] = ql * L::ROWB + (((2 * s + g) ^ L::fv(ql)) << 4);
+            row_addr[s] = ql * L::ROWB + (((2 * s + g) ^ L::fk(ql)) << 4);
         }
 #pragma unroll
         for (int db = 0; db < NDB; ++db)
@@ -75,15 +84,14 @@ struct BwdTiles {
             for (int h = 0; h < 2; ++h) {
                 const int r = 8 * h + 4 * g + (n >> 2);
                 const int chunk = 4 * db + 2 * dh + ((n & 3) >> 1);
-                tr_addr[0][db][h] = r * L::ROWB + ((chunk ^ L::fk(r)) << 4) + (n & 1) * 8;
-                tr_addr[1][db][h] = r * L::ROWB + ((chunk ^ L::fv(r)) << 4) + (n & 1) * 8;
+                tr_addr[db][h] = r * L::ROWB + ((chunk ^ L::fk(r)) << 4) + (n & 1) * 8;
             }
 #pragma unroll
         for (int c = 0; c < LPW; ++c) {
             const int pos = (wave * LPW + c) * 64 + lane;
             const int row = pos / L::CPR, slot = pos % L::CPR;
             voff[0][c] = row * (int)stride0 * 2 + (slot ^ L::fk(row)) * 16;
-            voff[1][c] = row * (int)stride1 * 2 + (slot ^ L::fv(row)) * 16;
+            voff[1][c] = row * (int)stride1 * 2 + (slot ^ L::fk(row)) * 16;
         }
     }
     // start the copy of rows [row0, row0 + 64) of tensor `which` (base pointer of the head, `rows` rows of `stride`
@@ -98,17 +106,17 @@ struct BwdTiles {
         for (int c = 0; c < LPW; ++c) dma_copy16(r, dst + (wave * LPW + c) * 1024, voff[which][c]);
     }
     // A operand by rows: rows 32*blk + ql of the tile, k-step s
-    __device__ __forceinline__ vec8 rows_op(int which, const char* tile, int blk, int s) const
+    __device__ __forceinline__ vec8 rows_op(const char* tile, int blk, int s) const
     {
-        return *(const vec8*)(tile + row_addr[which][s] + blk * 32 * L::ROWB);
+        return *(const vec8*)(tile + row_addr[s] + blk * 32 * L::ROWB);
     }
     // A operand transposed: column block db (32 columns), rows 16*ks .. 16*ks + 15 of the tile in the order the
     // accumulator registers of a 16-row half hold them
-    __device__ __forceinline__ vec8 tr_op(int which, const char* tile, int db, int ks) const
+    __device__ __forceinline__ vec8 tr_op(const char* tile, int db, int ks) const
     {
         short8v av;
-        av.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((short4v __attribute__((address_space(3)))*)(tile + tr_addr[which][db][0] + ks * 16 * L::ROWB));
-        av.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((short4v __attribute__((address_space(3)))*)(tile + tr_addr[which][db][1] + ks * 16 * L::ROWB));
+        av.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((short4v __attribute__((address_space(3)))*)(tile + tr_addr[db][0] + ks * 16 * L::ROWB));
+        av.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((short4v __attribute__((address_space(3)))*)(tile + tr_addr[db][1] + ks * 16 * L::ROWB));
         return __builtin_bit_cast(vec8, av);
     }
 };
@@ -130,10 +138,11 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
     const int ql = lane & 31, g = lane >> 5;
     const int Sq = p.Sq, Skv = p.Skv;
     const int nqb = (Sq + PF_BM - 1) / PF_BM;
-    const int vid = blockIdx.x;
-    const int gq = vid % p.G;
-    const int qb = nqb - 1 - (vid / p.G) % nqb;
-    const int bhkv = vid / (p.G * nqb);
+    // the forward's work order: an eighth of the list per XCD, query blocks longest-first, heads interleaved
+    const int total = gridDim.x;
+    const WorkItem wi = (total & 7) == 0 ? work_item_of_share(blockIdx.x & 7, blockIdx.x >> 3, total >> 3, p.interleave, p.G, nqb, p.deal_groups)
+                                         : work_item(blockIdx.x, p.interleave, p.G, nqb);
+    const int gq = wi.gq, qb = wi.qblk, bhkv = wi.bhkv;
     const int hkv = bhkv % p.Hkv, b = bhkv / p.Hkv;
     const int hq = hkv * p.G + gq;
     const int q0 = qb * PF_BM;
@@ -212,8 +221,8 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
             floatx16 s_acc = zero16, dp_acc = zero16;
 #pragma unroll
             for (int s = 0; s < NSTEP; ++s) {
-                s_acc = Mma<T>::run(tl.rows_op(0, kt, kb, s), qreg[s], s_acc);
-                dp_acc = Mma<T>::run(tl.rows_op(1, vt, kb, s), greg[s], dp_acc);
+                s_acc = Mma<T>::run(tl.rows_op(kt, kb, s), qreg[s], s_acc);
+                dp_acc = Mma<T>::run(tl.rows_op(vt, kb, s), greg[s], dp_acc);
             }
             // register r is key j0 + 32*kb + 8*(r/4) + 4*g + (r%4)
             vec8 ds[2];
@@ -228,7 +237,7 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
 #pragma unroll
             for (int h = 0; h < 2; ++h)
 #pragma unroll
-                for (int db = 0; db < NDB; ++db) dq_acc[db] = Mma<T>::run(tl.tr_op(0, kt, db, 2 * kb + h), ds[h], dq_acc[db]);
+                for (int db = 0; db < NDB; ++db) dq_acc[db] = Mma<T>::run(tl.tr_op(kt, db, 2 * kb + h), ds[h], dq_acc[db]);
         }
     }
 
@@ -250,7 +259,10 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
 
 // ---- dK, dV ---------------------------------------------------------------------------------------------------------------
 constexpr int BWD_KEYS = 128;      // keys per workgroup of the dK/dV kernel (32 per wavefront)
-constexpr int BWD_RING = 8;        // matrix operands in flight from LDS (reads run this many matrix instructions ahead)
+#ifndef BWD_RING_N
+#define BWD_RING_N 8
+#endif
+constexpr int BWD_RING = BWD_RING_N;        // matrix operands in flight from LDS (reads run this many matrix instructions ahead)
 
 // One wavefront per SIMD, so nothing hides a latency but the wavefront's own instruction order.  A 64-query tile is
 // 64 matrix instructions per wavefront in four runs of 16:
@@ -304,12 +316,9 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
     int kv_len = Skv;
     if (p.kv_lens) kv_len = clampi(p.kv_lens[b], 0, Skv);
     const int coff = Skv - Sq;
-    // query rows that see any key of this workgroup / of this wavefront: i >= j - coff for its first key (causal)
+    // query rows that see any key of this workgroup: i >= j - coff for its first key (causal)
     const int i_begin_wg = p.causal ? clampi(j0 - coff, 0, Sq) : 0;
-    const int i_begin_wave = p.causal ? clampi(j0 + wave * 32 - coff, 0, Sq) : 0;
-    const bool wave_has_keys = j0 + wave * 32 < kv_len;
-    // first query row that sees every key of this wavefront (tiles from there on, wholly inside Sq, need no mask)
-    const bool wave_keys_whole = j0 + wave * 32 + 31 < kv_len;
+    // first query row that sees every key of this wavefront: tiles from there on need no mask
     const int i_all_wave = p.causal ? max(j0 + wave * 32 + 31 - coff, 0) : 0;
     const int t_begin = i_begin_wg / PF_BN;
     const int n_qt = (Sq + PF_BN - 1) / PF_BN;
@@ -335,8 +344,8 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
             vreg[s] = *(const vec8*)(vrow + s * 16);
         }
     }
-    // rows i with lo_i <= i < Sq see this lane's key
-    const int lo_i = my_j < kv_len ? (p.causal ? my_j - coff : 0) : 0x7fffffff;
+    // rows i >= lo_i see this lane's key under the causal mask
+    const int lo_i = p.causal ? my_j - coff : -0x40000000;
 
     floatx16 dk_acc[NDB], dv_acc[NDB];
 #pragma unroll
@@ -363,8 +372,7 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
     constexpr int SG_MFMA = 0x8, SG_VALU = 0x2, SG_TRANS = 0x400, SG_DSR = 0x100;
 #define SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
 
-    auto tile = [&](int t, auto MASKED_) __attribute__((always_inline)) {
-        constexpr bool MASKED = decltype(MASKED_)::value;
+    auto tile = [&](int t) __attribute__((always_inline)) {
         const char* qt = smem + (t & 1) * STAGE;
         const char* gt = qt + L::TILE_BYTES;
         const char* nl = gt + L::TILE_BYTES;
@@ -374,10 +382,10 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
         auto fetch = [&](int i) __attribute__((always_inline)) {
             if (i < 32) {
                 const int qb = i / 16, s = (i % 16) / 2, which = i % 2;
-                ring[i % R] = tl.rows_op(which, which ? gt : qt, qb, s);
+                ring[i % R] = tl.rows_op(which ? gt : qt, qb, s);
             } else {
                 const int j = i - 32, qb = j / 16, h = (j % 16) / 8, db = (j % 8) / 2, which = 1 - j % 2;
-                ring[i % R] = tl.tr_op(which, which ? gt : qt, db, 2 * qb + h);
+                ring[i % R] = tl.tr_op(which ? gt : qt, db, 2 * qb + h);
             }
         };
         floatx16 sa[2], da[2];
@@ -394,24 +402,16 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
                 else dk_acc[db] = Mma<T>::run(ring[i % R], ds[qb][h], dk_acc[db]);
             }
         };
-        // P and dS of register r of query block qb: row i0 + 32*qb + 8*(r/4) + 4*g + (r%4)
-        const int rel_lo = lo_i - i0 - 4 * g, rel_hi = Sq - i0 - 4 * g;
+        // P and dS of register r of query block qb (row i0 + 32*qb + 8*(r/4) + 4*g + (r%4)), rounded for the next products
         auto soft = [&](int qb, int r) __attribute__((always_inline)) {
             const float pr = __builtin_amdgcn_exp2f(sa[qb][r]);
-            const float dsv = pr * da[qb][r];
-            if (MASKED) {
-                // (selected, not multiplied by zero: a row without visible keys has NaN in D_i and P = +inf)
-                const int kofs = 32 * qb + 8 * (r / 4) + (r % 4);
-                const bool seen = kofs >= rel_lo && kofs < rel_hi;
-                pp[qb][r / 8][r % 8] = (T)(seen ? pr : 0.0f);
-                ds[qb][r / 8][r % 8] = (T)(seen ? dsv : 0.0f);
-            } else {
-                pp[qb][r / 8][r % 8] = (T)pr;
-                ds[qb][r / 8][r % 8] = (T)dsv;
-            }
+            pp[qb][r / 8][r % 8] = (T)pr;
+            ds[qb][r / 8][r % 8] = (T)(pr * da[qb][r]);
         };
 
-        // accumulators start from -L_i log2(e) and -D_i
+        // The accumulators start from -L_i log2(e) and -D_i.  What the mask hides starts from -inf instead and ends as
+        // P = 0, dS = 0 * (finite): only the causal edge needs that here, rows past Sq arrive as zeros throughout (dO = 0,
+        // dP = 0), rows without any visible key carry -inf already, and keys past kv_len are zeroed at the end.
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb)
 #pragma unroll
@@ -423,6 +423,14 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
             }
 #pragma unroll
         for (int i = 0; i < R; ++i) fetch(i);
+        if (i0 < i_all_wave) {          // some row of the tile does not see every key of this wavefront
+            const int rel = lo_i - i0 - 4 * g;
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    if (32 * qb + 8 * (r / 4) + (r % 4) < rel) sa[qb][r] = -INFINITY;
+        }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < 16; ++i) {          // A0
@@ -436,15 +444,13 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
             fetch(i + R);
             soft(0, i - 16);
         }
-        if (!MASKED) {
 #pragma unroll
-            for (int i = 16; i < 32; ++i) {
-                SGB(SG_MFMA, 1);
-                if (i + R < 32) SGB(SG_DSR, 1);
-                else SGB(SG_DSR, 2);         // (a transposed operand is two reads)
-                SGB(SG_TRANS, 1);
-                SGB(SG_VALU, 2);
-            }
+        for (int i = 16; i < 32; ++i) {
+            SGB(SG_MFMA, 1);
+            if (i + R < 32) SGB(SG_DSR, 1);
+            else SGB(SG_DSR, 2);         // (a transposed operand is two reads)
+            SGB(SG_TRANS, 1);
+            SGB(SG_VALU, 2);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -453,14 +459,12 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
             fetch(i + R);
             soft(1, i - 32);
         }
-        if (!MASKED) {
 #pragma unroll
-            for (int i = 32; i < 48; ++i) {
-                SGB(SG_MFMA, 1);
-                SGB(SG_DSR, 2);
-                SGB(SG_TRANS, 1);
-                SGB(SG_VALU, 2);
-            }
+        for (int i = 32; i < 48; ++i) {
+            SGB(SG_MFMA, 1);
+            SGB(SG_DSR, 2);
+            SGB(SG_TRANS, 1);
+            SGB(SG_VALU, 2);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -478,10 +482,17 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
         asm volatile("" ::: "memory");
         __syncthreads();
         if (t + 1 < n_tiles) issue(t + 1);
-        const int i0 = row0_of(t);
-        if (!(wave_has_keys && i0 + PF_BN > i_begin_wave)) continue;      // no row of this tile sees a key of this wavefront
-        if (wave_keys_whole && i0 >= i_all_wave && i0 + PF_BN <= Sq) tile(t, std::false_type{});
-        else tile(t, std::true_type{});
+        // (The K and V rows are pinned to the architectural half of the register file: the accumulators - dK, dV and
+        // the tile's S and dP, 192 registers - then fit the accumulation half together, where dK and dV are pinned in
+        // turn.  Left alone, the register allocator parks dK and dV in the architectural half around every tile.)
+#pragma unroll
+        for (int s = 0; s < NSTEP; ++s) asm volatile("" : "+v"(kreg[s]), "+v"(vreg[s]));
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) asm volatile("" : "+a"(dk_acc[db]), "+a"(dv_acc[db]));
+        // Every wavefront computes every tile: one whose keys no row of the tile sees (the first tile or two under a
+        // causal mask) works on -inf, and would wait at the next barrier for the others anyway.  A tile skipped by
+        // some is also a second path the accumulators take around the loop, which costs register shuffling.
+        tile(t);
     }
 #undef SGB
 
@@ -495,9 +506,9 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
                 typedef T vec4 __attribute__((ext_vector_type(4)));
                 vec4 wk, wv;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    wk[e] = (T)(dk_acc[db][r4 * 4 + e] * p.scale);
-                    wv[e] = (T)dv_acc[db][r4 * 4 + e];
+                for (int e = 0; e < 4; ++e) {       // (a key past kv_len met no mask above: its sums are not gradients)
+                    wk[e] = (T)(my_j < kv_len ? dk_acc[db][r4 * 4 + e] * p.scale : 0.0f);
+                    wv[e] = (T)(my_j < kv_len ? dv_acc[db][r4 * 4 + e] : 0.0f);
                 }
                 *(vec4*)(krow + db * 32 + r4 * 8 + g * 4) = wk;
                 *(vec4*)(vrow + db * 32 + r4 * 8 + g * 4) = wv;
@@ -512,9 +523,13 @@ static hipError_t launch_bwd_t(const SdpaBwdParams& bp, hipStream_t stream)
     const SdpaParams& p = bp.f;
     const int64_t rows = (int64_t)p.B * p.Hq * p.Sq;
     if (rows > 0) {
-        hipLaunchKernelGGL((sdpa_bwd_delta_kernel<T>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, bp);
+        hipLaunchKernelGGL((sdpa_bwd_delta_kernel<T>), dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, stream, bp);
         const int nqb = (p.Sq + PF_BM - 1) / PF_BM;
-        hipLaunchKernelGGL((sdpa_bwd_dq_kernel<T>), dim3((unsigned)((int64_t)nqb * p.Hq * p.B)), dim3(256), 0, stream, bp);
+        const int64_t total = (int64_t)nqb * p.Hq * p.B;
+        SdpaBwdParams bq = bp;      // two workgroups per CU, an eighth of the CUs per XCD
+        bq.f.interleave = work_interleave(p.causal != 0, 2 * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
+        bq.f.deal_groups = (total & 7) == 0 ? work_deal(bq.f.interleave, p.G, nqb, total >> 3) : 0;
+        hipLaunchKernelGGL((sdpa_bwd_dq_kernel<T>), dim3((unsigned)total), dim3(256), 0, stream, bq);
     }
     const int nkb = (p.Skv + BWD_KEYS - 1) / BWD_KEYS;
     if ((int64_t)nkb * p.Hkv * p.B > 0)
