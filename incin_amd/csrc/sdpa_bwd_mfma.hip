@@ -259,10 +259,7 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
 
 // ---- dK, dV ---------------------------------------------------------------------------------------------------------------
 constexpr int BWD_KEYS = 128;      // keys per workgroup of the dK/dV kernel (32 per wavefront)
-#ifndef BWD_RING_N
-#define BWD_RING_N 8
-#endif
-constexpr int BWD_RING = BWD_RING_N;        // matrix operands in flight from LDS (reads run this many matrix instructions ahead)
+constexpr int BWD_RING = 8;        // matrix operands in flight from LDS (reads run this many matrix instructions ahead)
 
 // One wavefront per SIMD, so nothing hides a latency but the wavefront's own instruction order.  A 64-query tile is
 // 64 matrix instructions per wavefront in four runs of 16:
@@ -353,30 +350,46 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
 #pragma unroll
         for (int r = 0; r < 16; ++r) { dk_acc[db][r] = 0.0f; dv_acc[db][r] = 0.0f; }
 
-    auto head_of = [&](int t) { return hkv * p.G + t / tiles_per_head; };
-    auto row0_of = [&](int t) { return (t_begin + t % tiles_per_head) * PF_BN; };
+    // The copies walk the tiles with running addresses (the wavefront issues one instruction every four clocks and has
+    // the SIMD to itself: index arithmetic per tile would cost as much as the matrix instructions it feeds).
     const unsigned lds0 = lds_address(smem);
-    auto issue = [&](int t) __attribute__((always_inline)) {
-        const int hq = head_of(t), r0 = row0_of(t);
-        const T* qp = (const T*)p.q + (int64_t)b * p.q_sb + (int64_t)hq * p.q_sh;
-        const T* gp = (const T*)bp.d_o + (int64_t)b * bp.do_sb + (int64_t)hq * bp.do_sh;
-        const unsigned st = lds0 + (t & 1) * STAGE;
-        tl.issue(0, qp, p.q_ss, Sq, r0, st, wave);
-        tl.issue(1, gp, bp.do_ss, Sq, r0, st + L::TILE_BYTES, wave);
-        if (wave < 2) {         // 64 floats of one of the two per-row arrays; rows past Sq arrive as zeros
-            const float* src = (wave == 0 ? bp.neg_l2 : bp.neg_delta) + ((int64_t)b * p.Hq + hq) * Sq + r0;
-            dma_copy4(dma_descriptor(src, (Sq - r0) * 4), st + 2 * L::TILE_BYTES + wave * 256, lane * 4);
+    const int64_t q_step = (int64_t)PF_BN * p.q_ss * 2, g_step = (int64_t)PF_BN * bp.do_ss * 2;
+    const char *nx_q = nullptr, *nx_g = nullptr, *nx_s = nullptr;      // next tile to copy: Q rows, dO rows, per-row floats
+    int64_t nx_qrem = 0, nx_grem = 0;                                  // bytes from there to the end of the last row
+    int nx_rows = 0, nx_r = 0, nx_h = 0;                               // rows left, tile within the head, head within the group
+    auto to_head = [&](int h) __attribute__((always_inline)) {
+        const int hq = hkv * p.G + h, r0 = t_begin * PF_BN;
+        nx_q = (const char*)p.q + ((int64_t)b * p.q_sb + (int64_t)hq * p.q_sh + (int64_t)r0 * p.q_ss) * 2;
+        nx_g = (const char*)bp.d_o + ((int64_t)b * bp.do_sb + (int64_t)hq * bp.do_sh + (int64_t)r0 * bp.do_ss) * 2;
+        nx_s = (const char*)((wave == 0 ? bp.neg_l2 : bp.neg_delta) + ((int64_t)b * p.Hq + hq) * Sq + r0);
+        nx_rows = Sq - r0;
+        nx_qrem = (int64_t)(nx_rows - 1) * p.q_ss * 2 + 256;
+        nx_grem = (int64_t)(nx_rows - 1) * bp.do_ss * 2 + 256;
+        nx_r = 0;
+        nx_h = h;
+    };
+    auto clamp31 = [](int64_t x) { return (x >> 31) ? 0x7fffffff : (int)x; };       // (x is never negative here)
+    auto issue = [&](int stage) __attribute__((always_inline)) {
+        const unsigned st = lds0 + stage * STAGE;
+        const uint4v dq_ = dma_descriptor(nx_q, clamp31(nx_qrem)), dg_ = dma_descriptor(nx_g, clamp31(nx_grem));
+#pragma unroll
+        for (int c = 0; c < tl.LPW; ++c) dma_copy16(dq_, st + (wave * tl.LPW + c) * 1024, tl.voff[0][c]);
+#pragma unroll
+        for (int c = 0; c < tl.LPW; ++c) dma_copy16(dg_, st + L::TILE_BYTES + (wave * tl.LPW + c) * 1024, tl.voff[1][c]);
+        if (wave < 2)           // 64 floats of one of the two per-row arrays; rows past Sq arrive as zeros
+            dma_copy4(dma_descriptor(nx_s, nx_rows * 4), st + 2 * L::TILE_BYTES + wave * 256, lane * 4);
+        if (++nx_r == tiles_per_head) {
+            if (nx_h + 1 < p.G) to_head(nx_h + 1);
+        } else {
+            nx_q += q_step; nx_g += g_step; nx_s += PF_BN * 4;
+            nx_qrem -= q_step; nx_grem -= g_step; nx_rows -= PF_BN;
         }
     };
 
-    constexpr int SG_MFMA = 0x8, SG_VALU = 0x2, SG_TRANS = 0x400, SG_DSR = 0x100;
-#define SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
-
-    auto tile = [&](int t) __attribute__((always_inline)) {
-        const char* qt = smem + (t & 1) * STAGE;
+    auto tile = [&](int stage, int i0) __attribute__((always_inline)) {
+        const char* qt = smem + stage * STAGE;
         const char* gt = qt + L::TILE_BYTES;
         const char* nl = gt + L::TILE_BYTES;
-        const int i0 = row0_of(t);
         // matrix instruction i of the tile: its LDS operand ...
         vec8 ring[R];
         auto fetch = [&](int i) __attribute__((always_inline)) {
@@ -402,11 +415,23 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
                 else dk_acc[db] = Mma<T>::run(ring[i % R], ds[qb][h], dk_acc[db]);
             }
         };
+        // S and dP of a query block leave the accumulation registers in one go, at the seam between two runs, where the
+        // matrix pipe drains anyway: a read of an accumulation register waits until no matrix instruction is in
+        // flight (about one instruction's time each when the reads are spread among them).
+        float sv[16], dv[16];
+        auto take = [&](int qb) __attribute__((always_inline)) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                sv[r] = sa[qb][r];
+                dv[r] = da[qb][r];
+                asm volatile("" : "+v"(sv[r]), "+v"(dv[r]));
+            }
+        };
         // P and dS of register r of query block qb (row i0 + 32*qb + 8*(r/4) + 4*g + (r%4)), rounded for the next products
         auto soft = [&](int qb, int r) __attribute__((always_inline)) {
-            const float pr = __builtin_amdgcn_exp2f(sa[qb][r]);
+            const float pr = __builtin_amdgcn_exp2f(sv[r]);
             pp[qb][r / 8][r % 8] = (T)pr;
-            ds[qb][r / 8][r % 8] = (T)(pr * da[qb][r]);
+            ds[qb][r / 8][r % 8] = (T)(pr * dv[r]);
         };
 
         // The accumulators start from -L_i log2(e) and -D_i.  What the mask hides starts from -inf instead and ends as
@@ -432,56 +457,51 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
                     if (32 * qb + 8 * (r / 4) + (r % 4) < rel) sa[qb][r] = -INFINITY;
         }
         __builtin_amdgcn_sched_barrier(0);
+        // The order is pinned two matrix instructions at a time (the scheduler, left a whole run, strings the
+        // instructions of one accumulator together, each waiting for the one before).
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {          // A0
-            mma(i);
-            fetch(i + R);
+        for (int i = 0; i < 16; i += 2) {       // A0
+            mma(i); mma(i + 1);
+            fetch(i + R); fetch(i + R + 1);
+            __builtin_amdgcn_sched_barrier(0);
         }
+        take(0);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = 16; i < 32; ++i) {         // A1 over the vector work of rows 0-31
-            mma(i);
-            fetch(i + R);
-            soft(0, i - 16);
+        for (int i = 16; i < 32; i += 2) {      // A1 over the vector work of rows 0-31
+            mma(i); mma(i + 1);
+            fetch(i + R); fetch(i + R + 1);
+            soft(0, i - 16); soft(0, i - 15);
+            __builtin_amdgcn_sched_barrier(0);
         }
-#pragma unroll
-        for (int i = 16; i < 32; ++i) {
-            SGB(SG_MFMA, 1);
-            if (i + R < 32) SGB(SG_DSR, 1);
-            else SGB(SG_DSR, 2);         // (a transposed operand is two reads)
-            SGB(SG_TRANS, 1);
-            SGB(SG_VALU, 2);
-        }
+        take(1);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = 32; i < 48; ++i) {         // B0 over the vector work of rows 32-63
-            mma(i);
-            fetch(i + R);
-            soft(1, i - 32);
+        for (int i = 32; i < 48; i += 2) {      // B0 over the vector work of rows 32-63
+            mma(i); mma(i + 1);
+            fetch(i + R); fetch(i + R + 1);
+            soft(1, i - 32); soft(1, i - 31);
+            __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
-        for (int i = 32; i < 48; ++i) {
-            SGB(SG_MFMA, 1);
-            SGB(SG_DSR, 2);
-            SGB(SG_TRANS, 1);
-            SGB(SG_VALU, 2);
+        for (int i = 48; i < 64; i += 2) {      // B1
+            mma(i); mma(i + 1);
+            if (i + R < 64) { fetch(i + R); fetch(i + R + 1); }
+            __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int i = 48; i < 64; ++i) {         // B1
-            mma(i);
-            if (i + R < 64) fetch(i + R);
-        }
-        __builtin_amdgcn_sched_barrier(0);
     };
 
-    if (n_tiles > 0) issue(0);
+    if (n_tiles > 0) {
+        to_head(0);
+        issue(0);
+    }
+    int i0 = t_begin * PF_BN;
     for (int t = 0; t < n_tiles; ++t) {
         // tile t has landed for everyone and everyone is done with tile t-1: the other stage is free
         __builtin_amdgcn_s_waitcnt(0x0F70);             // vmcnt(0)
         asm volatile("" ::: "memory");
         __syncthreads();
-        if (t + 1 < n_tiles) issue(t + 1);
+        if (t + 1 < n_tiles) issue((t + 1) & 1);
         // (The K and V rows are pinned to the architectural half of the register file: the accumulators - dK, dV and
         // the tile's S and dP, 192 registers - then fit the accumulation half together, where dK and dV are pinned in
         // turn.  Left alone, the register allocator parks dK and dV in the architectural half around every tile.)
@@ -492,9 +512,10 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
         // Every wavefront computes every tile: one whose keys no row of the tile sees (the first tile or two under a
         // causal mask) works on -inf, and would wait at the next barrier for the others anyway.  A tile skipped by
         // some is also a second path the accumulators take around the loop, which costs register shuffling.
-        tile(t);
+        tile(t & 1, i0);
+        i0 += PF_BN;
+        if (i0 >= n_qt * PF_BN) i0 = t_begin * PF_BN;       // next head of the group
     }
-#undef SGB
 
     if (my_j < Skv) {
         T* krow = dkp + (int64_t)my_j * bp.dk_ss;
