@@ -61,17 +61,17 @@ __global__ __launch_bounds__(256) void sdpa_bwd_delta_kernel(SdpaBwdParams p)
 // operand whose M index is the row) or transposed (the gfx950 transposing read: an A operand whose M index is the
 // column block).  fk serves both reads without bank conflicts: 16 consecutive rows put one logical chunk into 16
 // different slots, and the 4 rows x 64 bytes a half-wavefront transposes land in 4 different 64-byte column groups.
-template <typename T>
+template <typename T, int NW, int NDBU>      // NW wavefronts share a tile copy; a wavefront transposes NDBU column blocks
 struct BwdTiles {
     typedef typename Mma<T>::vec8 vec8;
     typedef PfLayout<128> L;
-    static constexpr int NSTEP = 8, NDB = 4, LPW = L::LOADS_PER_WAVE;
+    static constexpr int NSTEP = 8, LPW = L::TILE_BYTES / 1024 / NW;
 
     int row_addr[NSTEP];           // [k-step]: byte offset of this lane's 16 bytes of row ql, chunk 2*s + g
-    int tr_addr[NDB][2];           // [column block][half]: byte offset of the transposing read
+    int tr_addr[NDBU][2];          // [column block - db0][half]: byte offset of the transposing read
     int voff[2][LPW];              // [tensor][load]: global byte offset of this lane's 16 bytes of a tile
 
-    __device__ __forceinline__ void init(int wave, int lane, int64_t stride0, int64_t stride1)
+    __device__ __forceinline__ void init(int wave, int lane, int64_t stride0, int64_t stride1, int db0)
     {
         const int ql = lane & 31, g = lane >> 5, n = lane & 15, dh = (lane >> 4) & 1;
 #pragma unroll
@@ -79,11 +79,11 @@ struct BwdTiles {
             row_addr[s] = ql * L::ROWB + (((2 * s + g) ^ L::fk(ql)) << 4);
         }
 #pragma unroll
-        for (int db = 0; db < NDB; ++db)
+        for (int db = 0; db < NDBU; ++db)
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 const int r = 8 * h + 4 * g + (n >> 2);
-                const int chunk = 4 * db + 2 * dh + ((n & 3) >> 1);
+                const int chunk = 4 * (db0 + db) + 2 * dh + ((n & 3) >> 1);
                 tr_addr[db][h] = r * L::ROWB + ((chunk ^ L::fk(r)) << 4) + (n & 1) * 8;
             }
 #pragma unroll
@@ -110,7 +110,7 @@ struct BwdTiles {
     {
         return *(const vec8*)(tile + row_addr[s] + blk * 32 * L::ROWB);
     }
-    // A operand transposed: column block db (32 columns), rows 16*ks .. 16*ks + 15 of the tile in the order the
+    // A operand transposed: column block db0 + db (32 columns), rows 16*ks .. 16*ks + 15 of the tile in the order the
     // accumulator registers of a 16-row half hold them
     __device__ __forceinline__ vec8 tr_op(const char* tile, int db, int ks) const
     {
@@ -167,8 +167,8 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
     const int n_tiles = (j_end + PF_BN - 1) / PF_BN;
     const int n_act = lim_wave_max > 0 ? (lim_wave_max + PF_BN - 1) / PF_BN : 0;
 
-    BwdTiles<T> tl;
-    tl.init(wave, lane, p.k_ss, p.v_ss);
+    BwdTiles<T, 4, 4> tl;
+    tl.init(wave, lane, p.k_ss, p.v_ss, 0);
 
     // this lane's query: Q row (scaled into log2 units, as the forward does) and dO row, the row's normaliser and D_i
     vec8 qreg[NSTEP], greg[NSTEP];
@@ -258,31 +258,38 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
 }
 
 // ---- dK, dV ---------------------------------------------------------------------------------------------------------------
-constexpr int BWD_KEYS = 128;      // keys per workgroup of the dK/dV kernel (32 per wavefront)
-constexpr int BWD_RING = 8;        // matrix operands in flight from LDS (reads run this many matrix instructions ahead)
+constexpr int BWD_KEYS = 128;      // keys per workgroup of the dK/dV kernel
+constexpr int BWD_RING = 4;        // matrix operands in flight from LDS (reads run this many matrix instructions ahead)
 
-// One wavefront per SIMD, so nothing hides a latency but the wavefront's own instruction order.  A 64-query tile is
-// 64 matrix instructions per wavefront in four runs of 16:
-//   A0  S, dP of query rows 0-31        A1  S, dP of rows 32-63, with P and dS of rows 0-31 on the vector ALU underneath
-//   B0  dV, dK from rows 0-31, with P and dS of rows 32-63 underneath                  B1  dV, dK from rows 32-63
-// and the LDS operand of instruction i + BWD_RING is requested right after instruction i is issued.  The S and dP
-// accumulators do not start from zero but from -L_i log2(e) and -D_i (staged per tile next to the Q and dO rows), so
-// P = exp2(S) and dS = P * dP need no subtraction.
+// A wavefront that has a SIMD to itself pays for every instruction it issues on top of its matrix instructions (nothing
+// of its own overlaps them), and 32 keys' dK and dV (128 accumulators) with the K and V rows (64 registers) and a tile's
+// S and dP leave no room for a second one.  So two wavefronts share each block of 32 keys, eight per workgroup, two
+// per SIMD, and split a 64-query tile both ways:
+//   first   S and dP of ONE 32-row query block (16 matrix instructions), P and dS from them, written to LDS;
+//   then    (after a barrier) dV and dK of the 32 keys for ONE half of the head dimension, over both query blocks
+//           (16 matrix instructions; the other block's P and dS come from the partner through LDS).
+// Each holds 64 accumulators, the matrix work is not duplicated, and what one wavefront issues runs under the matrix
+// instructions of the other.  The S and dP accumulators do not start from zero but from -L_i log2(e) and -D_i (staged
+// per tile next to the Q and dO rows), so P = exp2(S) and dS = P * dP need no subtraction.
 template <typename T>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
 {
 #if defined(__HIP_DEVICE_COMPILE__)
     typedef typename Mma<T>::vec8 vec8;
     typedef PfLayout<128> L;
     typedef float float4v __attribute__((ext_vector_type(4)));
-    constexpr int NSTEP = 8, NDB = 4, R = BWD_RING;
+    constexpr int NSTEP = 8, R = BWD_RING;
     constexpr int STAGE = 2 * L::TILE_BYTES + 1024;     // Q rows, dO rows, 64 x -L_i log2(e), 64 x -D_i (and padding)
+    constexpr int XCHG = 4 * 2 * 4 * 1024;              // [key block][query block][P lo, P hi, dS lo, dS hi]: 64 lanes x 16 bytes
     const SdpaParams& p = bp.f;
-    __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE];
+    constexpr int NS = 3;                               // stages: copies run two tiles ahead
+    __shared__ __attribute__((aligned(1024))) char smem[NS * STAGE + XCHG];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int kb = wave & 3;           // block of 32 keys
+    const int role = wave >> 2;        // query block of the first half, half of the head dimension of the second
     const int ql = lane & 31, g = lane >> 5;
     const int Sq = p.Sq, Skv = p.Skv;
     const int nkb = (Skv + BWD_KEYS - 1) / BWD_KEYS;
@@ -303,7 +310,7 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
     }
     const int hkv = bhkv % p.Hkv, b = bhkv / p.Hkv;
     const int j0 = kblk * BWD_KEYS;
-    const int my_j = j0 + wave * 32 + ql;              // this lane's key
+    const int my_j = j0 + kb * 32 + ql;                // this lane's key
 
     const T* kp = (const T*)p.k + (int64_t)b * p.k_sb + (int64_t)hkv * p.k_sh;
     const T* vp = (const T*)p.v + (int64_t)b * p.v_sb + (int64_t)hkv * p.v_sh;
@@ -316,14 +323,14 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
     // query rows that see any key of this workgroup: i >= j - coff for its first key (causal)
     const int i_begin_wg = p.causal ? clampi(j0 - coff, 0, Sq) : 0;
     // first query row that sees every key of this wavefront: tiles from there on need no mask
-    const int i_all_wave = p.causal ? max(j0 + wave * 32 + 31 - coff, 0) : 0;
+    const int i_all_wave = p.causal ? max(j0 + kb * 32 + 31 - coff, 0) : 0;
     const int t_begin = i_begin_wg / PF_BN;
     const int n_qt = (Sq + PF_BN - 1) / PF_BN;
     const int tiles_per_head = j0 < kv_len ? max(n_qt - t_begin, 0) : 0;
     const int n_tiles = tiles_per_head * p.G;           // the group's query heads one after another
 
-    BwdTiles<T> tl;
-    tl.init(wave, lane, p.q_ss, bp.do_ss);
+    BwdTiles<T, 8, 2> tl;
+    tl.init(wave, lane, p.q_ss, bp.do_ss, 2 * role);
 
     // this lane's key: K row (scaled into log2 units) and V row as B operands
     vec8 kreg[NSTEP], vreg[NSTEP];
@@ -344,14 +351,13 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
     // rows i >= lo_i see this lane's key under the causal mask
     const int lo_i = p.causal ? my_j - coff : -0x40000000;
 
-    floatx16 dk_acc[NDB], dv_acc[NDB];
+    floatx16 dk_acc[2], dv_acc[2];         // column blocks 2*role, 2*role + 1
 #pragma unroll
-    for (int db = 0; db < NDB; ++db)
+    for (int d = 0; d < 2; ++d)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) { dk_acc[db][r] = 0.0f; dv_acc[db][r] = 0.0f; }
+        for (int r = 0; r < 16; ++r) { dk_acc[d][r] = 0.0f; dv_acc[d][r] = 0.0f; }
 
-    // The copies walk the tiles with running addresses (the wavefront issues one instruction every four clocks and has
-    // the SIMD to itself: index arithmetic per tile would cost as much as the matrix instructions it feeds).
+    // The copies walk the tiles with running addresses instead of index arithmetic per tile.
     const unsigned lds0 = lds_address(smem);
     const int64_t q_step = (int64_t)PF_BN * p.q_ss * 2, g_step = (int64_t)PF_BN * bp.do_ss * 2;
     const char *nx_q = nullptr, *nx_g = nullptr, *nx_s = nullptr;      // next tile to copy: Q rows, dO rows, per-row floats
@@ -386,153 +392,125 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
         }
     };
 
+    char* const xmine = smem + NS * STAGE + ((kb * 2 + role) * 4) * 1024 + lane * 16;
+    const char* const xother = smem + NS * STAGE + ((kb * 2 + 1 - role) * 4) * 1024 + lane * 16;
+    const int own_rows = role * 32 * L::ROWB, other_rows = (1 - role) * 32 * L::ROWB;
+
     auto tile = [&](int stage, int i0) __attribute__((always_inline)) {
         const char* qt = smem + stage * STAGE;
         const char* gt = qt + L::TILE_BYTES;
-        const char* nl = gt + L::TILE_BYTES;
-        // matrix instruction i of the tile: its LDS operand ...
+        const char* nl = gt + L::TILE_BYTES + role * 128;
+        // Matrix instruction i of the tile and its LDS operand.  0..15: S (even i) and dP (odd i) of the own query block,
+        // k-step i / 2.  16..31: m = i - 16; the own block's rows first (m < 8), then the partner's; 16-row half (m / 4) % 2;
+        // column block (m / 2) % 2 of this wavefront's two; dV from dO^T and P (even m), dK from Q^T and dS (odd m).
         vec8 ring[R];
         auto fetch = [&](int i) __attribute__((always_inline)) {
-            if (i < 32) {
-                const int qb = i / 16, s = (i % 16) / 2, which = i % 2;
-                ring[i % R] = tl.rows_op(which ? gt : qt, qb, s);
+            if (i < 16) {
+                ring[i % R] = *(const vec8*)((i % 2 ? gt : qt) + own_rows + tl.row_addr[i / 2]);
             } else {
-                const int j = i - 32, qb = j / 16, h = (j % 16) / 8, db = (j % 8) / 2, which = 1 - j % 2;
-                ring[i % R] = tl.tr_op(which ? gt : qt, db, 2 * qb + h);
+                const int m = i - 16, h = (m / 4) % 2, d = (m / 2) % 2;
+                ring[i % R] = tl.tr_op((m % 2 ? qt : gt) + (m < 8 ? own_rows : other_rows), d, h);
             }
         };
-        floatx16 sa[2], da[2];
-        vec8 pp[2][2], ds[2][2];
-        // ... and the instruction itself
+        floatx16 sa, da;
+        vec8 pp[2], ds[2], opp[2], ods[2];
         auto mma = [&](int i) __attribute__((always_inline)) {
-            if (i < 32) {
-                const int qb = i / 16, s = (i % 16) / 2;
-                if (i % 2 == 0) sa[qb] = Mma<T>::run(ring[i % R], kreg[s], sa[qb]);
-                else da[qb] = Mma<T>::run(ring[i % R], vreg[s], da[qb]);
+            if (i < 16) {
+                if (i % 2 == 0) sa = Mma<T>::run(ring[i % R], kreg[i / 2], sa);
+                else da = Mma<T>::run(ring[i % R], vreg[i / 2], da);
             } else {
-                const int j = i - 32, qb = j / 16, h = (j % 16) / 8, db = (j % 8) / 2;
-                if (j % 2 == 0) dv_acc[db] = Mma<T>::run(ring[i % R], pp[qb][h], dv_acc[db]);
-                else dk_acc[db] = Mma<T>::run(ring[i % R], ds[qb][h], dk_acc[db]);
+                const int m = i - 16, h = (m / 4) % 2, d = (m / 2) % 2;
+                if (m % 2 == 0) dv_acc[d] = Mma<T>::run(ring[i % R], m < 8 ? pp[h] : opp[h], dv_acc[d]);
+                else dk_acc[d] = Mma<T>::run(ring[i % R], m < 8 ? ds[h] : ods[h], dk_acc[d]);
             }
-        };
-        // S and dP of a query block leave the accumulation registers in one go, at the seam between two runs, where the
-        // matrix pipe drains anyway: a read of an accumulation register waits until no matrix instruction is in
-        // flight (about one instruction's time each when the reads are spread among them).
-        float sv[16], dv[16];
-        auto take = [&](int qb) __attribute__((always_inline)) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                sv[r] = sa[qb][r];
-                dv[r] = da[qb][r];
-                asm volatile("" : "+v"(sv[r]), "+v"(dv[r]));
-            }
-        };
-        // P and dS of register r of query block qb (row i0 + 32*qb + 8*(r/4) + 4*g + (r%4)), rounded for the next products
-        auto soft = [&](int qb, int r) __attribute__((always_inline)) {
-            const float pr = __builtin_amdgcn_exp2f(sv[r]);
-            pp[qb][r / 8][r % 8] = (T)pr;
-            ds[qb][r / 8][r % 8] = (T)(pr * dv[r]);
         };
 
         // The accumulators start from -L_i log2(e) and -D_i.  What the mask hides starts from -inf instead and ends as
         // P = 0, dS = 0 * (finite): only the causal edge needs that here, rows past Sq arrive as zeros throughout (dO = 0,
         // dP = 0), rows without any visible key carry -inf already, and keys past kv_len are zeroed at the end.
 #pragma unroll
-        for (int qb = 0; qb < 2; ++qb)
+        for (int r4 = 0; r4 < 4; ++r4) {
+            const float4v a = *(const float4v*)(nl + (8 * r4 + 4 * g) * 4);
+            const float4v d = *(const float4v*)(nl + 256 + (8 * r4 + 4 * g) * 4);
 #pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-                const float4v a = *(const float4v*)(nl + (32 * qb + 8 * r4 + 4 * g) * 4);
-                const float4v d = *(const float4v*)(nl + 256 + (32 * qb + 8 * r4 + 4 * g) * 4);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) { sa[qb][4 * r4 + e] = a[e]; da[qb][4 * r4 + e] = d[e]; }
-            }
+            for (int e = 0; e < 4; ++e) { sa[4 * r4 + e] = a[e]; da[4 * r4 + e] = d[e]; }
+        }
 #pragma unroll
         for (int i = 0; i < R; ++i) fetch(i);
         if (i0 < i_all_wave) {          // some row of the tile does not see every key of this wavefront
-            const int rel = lo_i - i0 - 4 * g;
+            const int rel = lo_i - i0 - 4 * g - 32 * role;      // register r is row i0 + 32*role + 8*(r/4) + 4*g + (r%4)
 #pragma unroll
-            for (int qb = 0; qb < 2; ++qb)
-#pragma unroll
-                for (int r = 0; r < 16; ++r)
-                    if (32 * qb + 8 * (r / 4) + (r % 4) < rel) sa[qb][r] = -INFINITY;
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        // The order is pinned two matrix instructions at a time (the scheduler, left a whole run, strings the
-        // instructions of one accumulator together, each waiting for the one before).
-#pragma unroll
-        for (int i = 0; i < 16; i += 2) {       // A0
-            mma(i); mma(i + 1);
-            fetch(i + R); fetch(i + R + 1);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        take(0);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int i = 16; i < 32; i += 2) {      // A1 over the vector work of rows 0-31
-            mma(i); mma(i + 1);
-            fetch(i + R); fetch(i + R + 1);
-            soft(0, i - 16); soft(0, i - 15);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        take(1);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int i = 32; i < 48; i += 2) {      // B0 over the vector work of rows 32-63
-            mma(i); mma(i + 1);
-            fetch(i + R); fetch(i + R + 1);
-            soft(1, i - 32); soft(1, i - 31);
-            __builtin_amdgcn_sched_barrier(0);
+            for (int r = 0; r < 16; ++r)
+                if (8 * (r / 4) + (r % 4) < rel) sa[r] = -INFINITY;
         }
 #pragma unroll
-        for (int i = 48; i < 64; i += 2) {      // B1
-            mma(i); mma(i + 1);
-            if (i + R < 64) { fetch(i + R); fetch(i + R + 1); }
-            __builtin_amdgcn_sched_barrier(0);
+        for (int i = 0; i < 16; ++i) {
+            mma(i);
+            fetch(i + R);
+        }
+        // P and dS, rounded for the next products
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const float pr = __builtin_amdgcn_exp2f(sa[r]);
+            pp[r / 8][r % 8] = (T)pr;
+            ds[r / 8][r % 8] = (T)(pr * da[r]);
+        }
+        *(vec8*)(xmine) = pp[0];
+        *(vec8*)(xmine + 1024) = pp[1];
+        *(vec8*)(xmine + 2048) = ds[0];
+        *(vec8*)(xmine + 3072) = ds[1];
+        __syncthreads();
+        opp[0] = *(const vec8*)(xother);
+        opp[1] = *(const vec8*)(xother + 1024);
+        ods[0] = *(const vec8*)(xother + 2048);
+        ods[1] = *(const vec8*)(xother + 3072);
+#pragma unroll
+        for (int i = 16; i < 32; ++i) {
+            mma(i);
+            if (i + R < 32) fetch(i + R);
         }
     };
 
     if (n_tiles > 0) {
         to_head(0);
         issue(0);
+        if (n_tiles > 1) issue(1);
     }
-    int i0 = t_begin * PF_BN;
+    int i0 = t_begin * PF_BN, stage = 0;
     for (int t = 0; t < n_tiles; ++t) {
-        // tile t has landed for everyone and everyone is done with tile t-1: the other stage is free
-        __builtin_amdgcn_s_waitcnt(0x0F70);             // vmcnt(0)
+        // Tile t has landed for everyone (memory operations complete in order: all but the copies of tile t + 1, which
+        // are 4 per wavefront and one more in the two that fetch the per-row floats) and everyone is done with tile
+        // t - 1: its stage and the exchange buffer are free.
+        if (t + 1 >= n_tiles) __builtin_amdgcn_s_waitcnt(0x0F70);        // vmcnt(0)
+        else if (wave < 2) __builtin_amdgcn_s_waitcnt(0x0F75);           // vmcnt(5)
+        else __builtin_amdgcn_s_waitcnt(0x0F74);                         // vmcnt(4)
         asm volatile("" ::: "memory");
         __syncthreads();
-        if (t + 1 < n_tiles) issue((t + 1) & 1);
-        // (The K and V rows are pinned to the architectural half of the register file: the accumulators - dK, dV and
-        // the tile's S and dP, 192 registers - then fit the accumulation half together, where dK and dV are pinned in
-        // turn.  Left alone, the register allocator parks dK and dV in the architectural half around every tile.)
-#pragma unroll
-        for (int s = 0; s < NSTEP; ++s) asm volatile("" : "+v"(kreg[s]), "+v"(vreg[s]));
-#pragma unroll
-        for (int db = 0; db < NDB; ++db) asm volatile("" : "+a"(dk_acc[db]), "+a"(dv_acc[db]));
+        if (t + 2 < n_tiles) issue(stage == 0 ? 2 : stage - 1);          // stage of tile t + 2 = stage of tile t - 1
         // Every wavefront computes every tile: one whose keys no row of the tile sees (the first tile or two under a
-        // causal mask) works on -inf, and would wait at the next barrier for the others anyway.  A tile skipped by
-        // some is also a second path the accumulators take around the loop, which costs register shuffling.
-        tile(t & 1, i0);
+        // causal mask) works on -inf, and would wait at the barriers for the others anyway.
+        tile(stage, i0);
+        stage = stage == 2 ? 0 : stage + 1;
         i0 += PF_BN;
         if (i0 >= n_qt * PF_BN) i0 = t_begin * PF_BN;       // next head of the group
     }
 
     if (my_j < Skv) {
-        T* krow = dkp + (int64_t)my_j * bp.dk_ss;
-        T* vrow = dvp + (int64_t)my_j * bp.dv_ss;
+        T* krow = dkp + (int64_t)my_j * bp.dk_ss + role * 64;
+        T* vrow = dvp + (int64_t)my_j * bp.dv_ss + role * 64;
 #pragma unroll
-        for (int db = 0; db < NDB; ++db)
+        for (int d = 0; d < 2; ++d)
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4) {
                 typedef T vec4 __attribute__((ext_vector_type(4)));
                 vec4 wk, wv;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {       // (a key past kv_len met no mask above: its sums are not gradients)
-                    wk[e] = (T)(my_j < kv_len ? dk_acc[db][r4 * 4 + e] * p.scale : 0.0f);
-                    wv[e] = (T)(my_j < kv_len ? dv_acc[db][r4 * 4 + e] : 0.0f);
+                    wk[e] = (T)(my_j < kv_len ? dk_acc[d][r4 * 4 + e] * p.scale : 0.0f);
+                    wv[e] = (T)(my_j < kv_len ? dv_acc[d][r4 * 4 + e] : 0.0f);
                 }
-                *(vec4*)(krow + db * 32 + r4 * 8 + g * 4) = wk;
-                *(vec4*)(vrow + db * 32 + r4 * 8 + g * 4) = wv;
+                *(vec4*)(krow + d * 32 + r4 * 8 + g * 4) = wk;
+                *(vec4*)(vrow + d * 32 + r4 * 8 + g * 4) = wv;
             }
     }
 #endif
@@ -554,7 +532,7 @@ static hipError_t launch_bwd_t(const SdpaBwdParams& bp, hipStream_t stream)
     }
     const int nkb = (p.Skv + BWD_KEYS - 1) / BWD_KEYS;
     if ((int64_t)nkb * p.Hkv * p.B > 0)
-        hipLaunchKernelGGL((sdpa_bwd_dkv_kernel<T>), dim3((unsigned)((int64_t)nkb * p.Hkv * p.B)), dim3(256), 0, stream, bp);
+        hipLaunchKernelGGL((sdpa_bwd_dkv_kernel<T>), dim3((unsigned)((int64_t)nkb * p.Hkv * p.B)), dim3(512), 0, stream, bp);
     return hipGetLastError();
 }
 
