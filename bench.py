@@ -204,13 +204,62 @@ def decode_step_graph(w, B, H, Skv, D, steps):
             "ms_per_step": ms, "kv_GBps": 2.0 * B * H * Skv * D * 2 / (ms * 1e-3) / 1e9}
 
 
+def backward_config3(steps, warmup):
+    """Forward (keeping the row normalisers) and then the timed backward of BASELINE config 3's shape: dQ, dK, dV for a
+    synthetic upstream gradient.  The figure counts 2.5 x the forward's FLOPs (five matrix products against the
+    forward's two; the recomputation of S and dP in both big kernels is not counted)."""
+    B, H, S, D = 8, 16, 4096, 128
+    q, k, v = make_inputs(SEED0 + 5, B, H, H, S, S, D, capi.BF16)
+    g = rng(SEED0 + 6).standard_normal((B, H, S, D), dtype=np.float32)
+    tq, tk, tv, tg = (host.DeviceTensor.from_f32(x, capi.BF16) for x in (q, k, v, g))
+    to, tdq, tdk, tdv = (host.DeviceTensor((B, H, S, D), capi.BF16) for _ in range(4))
+    lse = capi.DeviceBuffer(B * H * S * 4)
+    bd = capi.SdpaBwdDesc()
+    bd.fwd = host.make_desc(tq, tk, tv, to, causal=True, lse=lse)
+    capi.sdpa_fwd(bd.fwd)
+    for name, t in (("d_o", tg), ("d_q", tdq), ("d_k", tdk), ("d_v", tdv)):
+        setattr(bd, name, t.ptr)
+        st = host._strides3(t.shape)
+        for i in range(3):
+            getattr(bd, name + "_stride")[i] = st[i]
+    ws = capi.DeviceBuffer(capi.sdpa_bwd_workspace(bd))
+    bd.workspace, bd.workspace_bytes = ws.ptr, ws.nbytes
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < 0.15:          # clocks settle (set-up, not measurement)
+        capi.sdpa_bwd(bd)
+        capi.sync()
+    for _ in range(warmup):
+        capi.sdpa_bwd(bd)
+    capi.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        capi.sdpa_bwd(bd)
+    capi.sync()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    # at-size check of one (batch, head) slice against the float64 backward oracle (checker only)
+    from oracle import sdpa_backward as OB
+    b, h = B - 1, H - 1
+    rq, rk, rv, rg = (dtypes.round_to(x[b, h], capi.BF16) for x in (q, k, v, g))
+    ref = OB.sdpa_backward(rq, rk, rv, rg, causal=True)
+    err = max(float(np.abs(t.to_f32()[b, h] - r).max() / np.abs(r).max()) for t, r in zip((tdq, tdk, tdv), ref))
+    flops = 2.5 * causal_flops(B, H, S, S, D)
+    for t in (tq.buf, tk.buf, tv.buf, tg.buf, to.buf, tdq.buf, tdk.buf, tdv.buf, lse, ws):
+        t.free()
+    return {"workload": "backward of BASELINE config 3's shape: bf16 causal B=8 H=16 S=4096 D=128, dQ dK dV from Q K V O dO and the "
+                        "forward's row normalisers", "step": "one incin_rocm_sdpa_bwd call (3 kernels: row dots, dQ, dK/dV)",
+            "metric": "attn bwd TFLOP/s (2.5 x forward FLOPs)", "value": flops / (wall * 1e-3) / 1e12, "unit": "TFLOP/s",
+            "ms_per_step": wall, "steps": steps, "frac_of_bf16_mfma_peak": flops / (wall * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+            "parity_max_err_rel_to_max_abs_ref": err,
+            "parity_sample": "dQ, dK, dV of slice (b=%d, h=%d) against the float64 oracle of the reference's tape gradients" % (b, h)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["prefill", "prefill_long", "decode", "copy"], default=None,
+    ap.add_argument("--only", choices=["prefill", "prefill_long", "decode", "backward", "copy"], default=None,
                     help="run a single workload (profiling). 'copy' runs --steps device-to-device copies of 1 GiB "
                          "through the library's plain copy kernel: the known-size dispatch that hardware byte "
                          "counters (FETCH_SIZE / WRITE_SIZE) are calibrated against")
@@ -323,6 +372,9 @@ def main():
                                    "sample": "all of config 4 (B=32, H=32, KV=8192, D=128), oracle's materialising restatement of "
                                              "the reference CPU op (serial matmuls and reductions); %.1f s; host: %s" % (dt, host_cpu())}
         result["decode"] = dec
+
+    if args.only in (None, "backward"):
+        result["backward"] = backward_config3(max(5, min(args.steps, 30)), min(args.warmup, 5))
 
     print(json.dumps(result))
     return 0

@@ -199,7 +199,8 @@ int incin_rocm_sdpa_fwd(const incin_rocm_sdpa_desc_t* desc, void* stream);
  * Covered: f16 / bf16, D == Dv == 128, no dense additive mask, no q_lens; anything else is
  * INCIN_ROCM_EUNSUPPORTED.  A query row with no visible key (NaN in the forward) gets a zero gradient and
  * contributes nothing to d_k and d_v, where the reference's tape would spread NaN over the whole head.
- * The workspace holds one float per query row ([B, Hq, Sq]); d_q, d_k, d_v are fully overwritten. */
+ * The workspace holds two floats per query row (2 x [B, Hq, Sq]; ask incin_rocm_sdpa_bwd_workspace for the size);
+ * d_q, d_k, d_v are fully overwritten. */
 typedef struct {
     incin_rocm_sdpa_desc_t fwd;
     const void* d_o;               /* [B, Hq, Sq, D], dtype of the operands */
