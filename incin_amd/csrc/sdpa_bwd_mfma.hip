@@ -7,16 +7,15 @@
 //   dV_j = sum_i P_ij dO_i      dK_j = s sum_i dS_ij Q_i      dQ_i = s sum_j dS_ij K_j
 //
 // Three kernels, no atomics, P and dP recomputed in both big ones:
-//   sdpa_bwd_delta_kernel   D_i (f32) into the workspace
+//   sdpa_bwd_delta_kernel   per query row, into the workspace: -L_i log2(e) and -D_i (f32), the values both big kernels
+//                           start their S and dP accumulators from
 //   sdpa_bwd_dq_kernel      the forward's shape of work: a wavefront owns 32 query rows (Q and dO rows resident in
 //                           registers), K / V tiles stream through LDS; S^T = K Q'^T and dP^T = V dO^T have the
 //                           lane-owns-a-query accumulator layout of the forward, which is again the B-operand layout
 //                           of the next product, dQ^T += K^T dS^T (K^T through the transposing LDS read)
-//   sdpa_bwd_dkv_kernel     the same with the roles swapped: a wavefront owns 32 keys (K and V rows resident), Q / dO
-//                           tiles of the group's query heads stream through LDS; S = Q K'^T and dP = dO V^T have a
+//   sdpa_bwd_dkv_kernel     the same with the roles swapped: a pair of wavefronts owns 32 keys (K and V rows resident),
+//                           Q / dO tiles of the group's query heads stream through LDS; S = Q K'^T and dP = dO V^T have a
 //                           lane-owns-a-key layout, the B-operand layout of dV^T += dO^T P and dK^T += Q^T dS
-// Both big kernels are plain loops (one tile at a time, operands read just ahead of use); they rely on two
-// wavefronts per SIMD (dQ) or none (dK/dV, 512 registers) for overlap and are not software-pipelined.
 #include <type_traits>
 
 #include "sdpa_bwd.h"

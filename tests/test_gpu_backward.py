@@ -60,6 +60,36 @@ def test_backward_against_the_oracle(gpu, dtype, shape):
             assert not dk[b, :, lens[b]:].any() and not dv[b, :, lens[b]:].any()      # padded keys: exactly zero
 
 
+def test_backward_random_cases(gpu):
+    """Seeded random shapes: batch, heads, group size, lengths on either side of the 64-row tiles and the 128-key
+    workgroups, causal alignment with Sq <= Skv, ragged key counts >= 1 (every query row keeps a visible key, so the
+    oracle has no NaN), scales.  Each case is printed before it runs."""
+    r = np.random.Generator(np.random.PCG64(2026))
+    D = 128
+    for case in range(28):
+        B, Hkv, G = int(r.integers(1, 4)), int(r.integers(1, 4)), int(r.choice([1, 2, 4]))
+        Skv = int(r.choice([r.integers(1, 70), r.integers(60, 140), r.integers(120, 420)]))
+        causal = bool(r.integers(0, 2))
+        Sq = int(r.integers(1, Skv + 1)) if causal else int(r.integers(1, 300))
+        lens = None
+        if r.integers(0, 2):
+            lens = r.integers(1, Skv + 1, B).astype(np.int32)      # (row 0 sees key 0 whenever Sq <= Skv and the count is >= 1)
+        dtype = capi.BF16 if case % 2 else capi.F16
+        scale = float(r.choice([0.0883883461356163, 0.05, 0.2]))
+        Hq = Hkv * G
+        say("backward random case %d: B=%d Hq=%d Hkv=%d Sq=%d Skv=%d causal=%s lens=%s dtype=%d scale=%g"
+            % (case, B, Hq, Hkv, Sq, Skv, causal, None if lens is None else lens.tolist(), dtype, scale))
+        q, k, v, go = make(100 + case, B, Hq, Hkv, Sq, Skv, D, dtype)
+        out, dq, dk, dv = host.sdpa_backward(q, k, v, go, dtype, scale=scale, causal=causal, kv_lens=lens)
+        rq, rk, rv = BW.sdpa_backward(q.reshape(B, Hkv, G, Sq, D), k[:, :, None], v[:, :, None], go.reshape(B, Hkv, G, Sq, D),
+                                      scale=scale, causal=causal, kv_lens=None if lens is None else lens.reshape(B, 1, 1))
+        rq, rk, rv = rq.reshape(B, Hq, Sq, D), rk.reshape(B, Hkv, Skv, D), rv.reshape(B, Hkv, Skv, D)
+        assert not np.isnan(rq).any(), "case construction: a row without keys"
+        compare("dq", dq, rq)
+        compare("dk", dk, rk)
+        compare("dv", dv, rv)
+
+
 def test_rows_without_visible_keys_get_zero_gradients(gpu):
     # Sq > Skv under causal alignment: the first Sq - Skv rows see nothing (NaN in the forward).  They get a zero dq
     # and contribute nothing to dk, dv; the other rows are what the oracle gives for them alone.
