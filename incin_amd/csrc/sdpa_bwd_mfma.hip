@@ -194,9 +194,14 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
     for (int db = 0; db < NDB; ++db)
 #pragma unroll
         for (int r = 0; r < 16; ++r) dq_acc[db][r] = 0.0f;
-    floatx16 zero16;
+    // The S and dP accumulators start from -L_i log2(e) and -D_i of the lane's query (what the mask hides: from -inf, which
+    // ends as P = 0 and dS = 0), so P = exp2(S) and dS = P * dP need neither a subtraction nor a select.
+    floatx16 seed_s, seed_d;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) zero16[r] = 0.0f;
+    for (int r = 0; r < 16; ++r) { seed_s[r] = -l2; seed_d[r] = -dlt; }
+    // first key some lane of this wavefront does not see: tiles that end at or before it need no mask
+    int lim_wave_min = kv_len;
+    if (p.causal) lim_wave_min = clampi(q0 + wave * 32 + coff + 1, 0, kv_len);
 
     const unsigned lds0 = lds_address(smem);
     if (n_tiles > 0) {
@@ -215,24 +220,25 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
         const char* kt = smem + (t & 1) * L::TILE_BYTES;
         const char* vt = smem + (2 + (t & 1)) * L::TILE_BYTES;
         const int j0 = t * PF_BN;
+        const bool edge = j0 + PF_BN > lim_wave_min;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
-            floatx16 s_acc = zero16, dp_acc = zero16;
+            floatx16 s_acc = seed_s, dp_acc = seed_d;
+            if (edge) {
+                // register r is key j0 + 32*kb + 8*(r/4) + 4*g + (r%4)
+                const int rel = lim_lane - (j0 + 32 * kb + 4 * g);
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    if (8 * (r / 4) + (r % 4) >= rel) s_acc[r] = -INFINITY;
+            }
 #pragma unroll
             for (int s = 0; s < NSTEP; ++s) {
                 s_acc = Mma<T>::run(tl.rows_op(kt, kb, s), qreg[s], s_acc);
                 dp_acc = Mma<T>::run(tl.rows_op(vt, kb, s), greg[s], dp_acc);
             }
-            // register r is key j0 + 32*kb + 8*(r/4) + 4*g + (r%4)
             vec8 ds[2];
-            const int rel = lim_lane - (j0 + 32 * kb + 4 * g);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int kofs = 8 * (r / 4) + (r % 4);
-                const float pr = __builtin_amdgcn_exp2f(s_acc[r] - l2);
-                // (selected, not multiplied by zero: a row without visible keys has NaN in D_i and +inf here)
-                ds[r / 8][r % 8] = (T)(kofs >= rel ? 0.0f : pr * (dp_acc[r] - dlt));
-            }
+            for (int r = 0; r < 16; ++r) ds[r / 8][r % 8] = (T)(__builtin_amdgcn_exp2f(s_acc[r]) * dp_acc[r]);
 #pragma unroll
             for (int h = 0; h < 2; ++h)
 #pragma unroll
