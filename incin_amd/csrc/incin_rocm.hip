@@ -473,30 +473,43 @@ int incin_rocm_sdpa_fwd(const incin_rocm_sdpa_desc_t* desc, void* stream)
 
 size_t incin_rocm_sizeof_sdpa_bwd_desc(void) { return sizeof(incin_rocm_sdpa_bwd_desc_t); }
 
-// Validates a backward request; *empty is set when there is nothing to compute.
-static int check_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, bool* empty)
+// Validates a backward request; *empty is set when there is nothing to compute, *mfma when the matrix-core kernels
+// take it (else the generic ones do).
+static int check_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, bool* empty, bool* mfma)
 {
     static const char* OP = "scaled_dot_product_attention backward";
     if (!bd) return fail(INCIN_ROCM_EINVAL, "%s: null descriptor", OP);
     const incin_rocm_sdpa_desc_t* d = &bd->fwd;
     Plan plan;
-    if (int rc = make_plan(d, &plan)) return rc;
+    {
+        incin_rocm_sdpa_desc_t any = *d;            // shapes, dtype, strides, mask: whatever some forward kernel accepts
+        any.impl = INCIN_ROCM_IMPL_AUTO;
+        if (int rc = make_plan(&any, &plan)) return rc;
+    }
     *empty = plan.empty || d->Skv == 0;
+    *mfma = false;
     if (*empty) return 0;
-    if (d->dtype == INCIN_ROCM_F32 || d->D != 128 || d->Dv != 128)
-        return fail(INCIN_ROCM_EUNSUPPORTED, "%s: f16 / bf16 with D == Dv == 128 only", OP);
-    if (d->add_mask) return fail(INCIN_ROCM_EUNSUPPORTED, "%s: no kernel takes a dense additive mask", OP);
     if (d->q_lens) return fail(INCIN_ROCM_EUNSUPPORTED, "%s: no kernel takes q_lens", OP);
-    if (!(d->scale > 0.0f) || !std::isfinite(d->scale)) return fail(INCIN_ROCM_EUNSUPPORTED, "%s: the scale must be positive and finite", OP);
     if (!d->lse) return fail(INCIN_ROCM_EINVAL, "%s: fwd.lse (the forward's row normalisers) is required", OP);
     if (!bd->d_o || !bd->d_q || !bd->d_k || !bd->d_v) return fail(INCIN_ROCM_EINVAL, "%s: null gradient pointer", OP);
-    bool ok = fast_layout_ok(d, 8) && aligned16(bd->d_o) && aligned16(bd->d_q) && aligned16(bd->d_k) && aligned16(bd->d_v);
+    if (d->D > 256 || d->Dv > 256) return fail(INCIN_ROCM_EUNSUPPORTED, "%s: D and Dv up to 256", OP);
+
+    bool ok = d->dtype != INCIN_ROCM_F32 && d->D == 128 && d->Dv == 128 && !d->add_mask && d->scale > 0.0f && std::isfinite(d->scale);
+    ok = ok && fast_layout_ok(d, 8) && aligned16(bd->d_o) && aligned16(bd->d_q) && aligned16(bd->d_k) && aligned16(bd->d_v);
     for (int a = 0; a < 3; ++a)
         ok = ok && bd->d_o_stride[a] % 8 == 0 && bd->d_q_stride[a] % 8 == 0 && bd->d_k_stride[a] % 8 == 0 && bd->d_v_stride[a] % 8 == 0;
     const int64_t big = 1 << 24;
     ok = ok && d->q_stride[2] >= 0 && d->q_stride[2] < big && d->k_stride[2] >= 0 && d->k_stride[2] < big && d->v_stride[2] >= 0 &&
          d->v_stride[2] < big && bd->d_o_stride[2] >= 0 && bd->d_o_stride[2] < big;
-    if (!ok) return fail(INCIN_ROCM_EUNSUPPORTED, "%s: rows must be 16-byte aligned with strides that are multiples of 8 elements below 2^24", OP);
+    if (d->impl == INCIN_ROCM_IMPL_AUTO) *mfma = ok;
+    else if (d->impl == INCIN_ROCM_IMPL_GENERIC) *mfma = false;
+    else if (d->impl == INCIN_ROCM_IMPL_MFMA) {
+        if (!ok)
+            return fail(INCIN_ROCM_EUNSUPPORTED, "%s: the MFMA kernels need f16 / bf16, D == Dv == 128, scale > 0, no dense mask, and rows "
+                        "16-byte aligned with strides that are multiples of 8 elements below 2^24", OP);
+        *mfma = true;
+    } else
+        return fail(INCIN_ROCM_EUNSUPPORTED, "%s: impl is one of AUTO, GENERIC, MFMA", OP);
     return 0;
 }
 
@@ -504,16 +517,16 @@ int incin_rocm_sdpa_bwd_workspace(const incin_rocm_sdpa_bwd_desc_t* bd, size_t* 
 {
     if (!bytes) return fail(INCIN_ROCM_EINVAL, "scaled_dot_product_attention backward: null output");
     *bytes = 0;
-    bool empty = false;
-    if (int rc = check_bwd(bd, &empty)) return rc;
+    bool empty = false, mfma = false;
+    if (int rc = check_bwd(bd, &empty, &mfma)) return rc;
     if (!empty) *bytes = 2 * (size_t)(bd->fwd.B * bd->fwd.Hq * bd->fwd.Sq) * sizeof(float);
     return 0;
 }
 
 int incin_rocm_sdpa_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, void* stream)
 {
-    bool empty = false;
-    if (int rc = check_bwd(bd, &empty)) return rc;
+    bool empty = false, mfma = false;
+    if (int rc = check_bwd(bd, &empty, &mfma)) return rc;
     if (empty) return 0;        // (gradients of an empty problem: nothing to write)
     const size_t need = 2 * (size_t)(bd->fwd.B * bd->fwd.Hq * bd->fwd.Sq) * sizeof(float);      // two f32 per query row
     if (!bd->workspace || bd->workspace_bytes < need || !aligned16(bd->workspace))
@@ -533,7 +546,8 @@ int incin_rocm_sdpa_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, void* stream)
     bp.dq_sb = bd->d_q_stride[0]; bp.dq_sh = bd->d_q_stride[1]; bp.dq_ss = bd->d_q_stride[2];
     bp.dk_sb = bd->d_k_stride[0]; bp.dk_sh = bd->d_k_stride[1]; bp.dk_ss = bd->d_k_stride[2];
     bp.dv_sb = bd->d_v_stride[0]; bp.dv_sh = bd->d_v_stride[1]; bp.dv_ss = bd->d_v_stride[2];
-    hipError_t e = incin_rocm::launch_sdpa_bwd_mfma(bp, bd->fwd.dtype, (hipStream_t)stream);
+    hipError_t e = mfma ? incin_rocm::launch_sdpa_bwd_mfma(bp, bd->fwd.dtype, (hipStream_t)stream)
+                        : incin_rocm::launch_sdpa_bwd_generic(bp, bd->fwd.dtype, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "attention backward launch");
     return 0;
 }

@@ -21,5 +21,6 @@ struct SdpaBwdParams {
 };
 
 hipError_t launch_sdpa_bwd_mfma(const SdpaBwdParams& bp, int dtype, hipStream_t stream);
+hipError_t launch_sdpa_bwd_generic(const SdpaBwdParams& bp, int dtype, hipStream_t stream);
 
 }  // namespace incin_rocm

@@ -131,21 +131,28 @@ def sdpa(q, k, v, dtype=capi.F32, scale=None, causal=False, kv_lens=None, mask=N
     return out
 
 
-def sdpa_backward(q, k, v, d_out, dtype=capi.BF16, scale=None, causal=False, kv_lens=None, impl=capi.IMPL_AUTO, dev=0):
+def sdpa_backward(q, k, v, d_out, dtype=capi.BF16, scale=None, causal=False, kv_lens=None, impl=capi.IMPL_AUTO, dev=0, mask=None):
     """Forward (with row normalisers) then backward on the GPU for f32 numpy operands [B,Hq,Sq,D], [B,Hkv,Skv,D],
-    d_out [B,Hq,Sq,D]; returns (out, dq, dk, dv) as f32 holding the `dtype`-rounded results."""
+    [B,Hkv,Skv,Dv], d_out [B,Hq,Sq,Dv] and an optional dense additive mask broadcastable to [B,Hq,Sq,Skv]; returns
+    (out, dq, dk, dv) as f32 holding the `dtype`-rounded results.  `impl` pins the kernels of both passes."""
     q, k, v, d_out = (np.asarray(x, dtype=np.float32) for x in (q, k, v, d_out))
     B, Hq, Sq, D = q.shape
+    Dv = v.shape[-1]
     tq, tk, tv, tg = (DeviceTensor.from_f32(x, dtype, dev) for x in (q, k, v, d_out))
-    to, tdq = DeviceTensor(q.shape, dtype, dev), DeviceTensor(q.shape, dtype, dev)
+    to, tdq = DeviceTensor((B, Hq, Sq, Dv), dtype, dev), DeviceTensor(q.shape, dtype, dev)
     tdk, tdv = DeviceTensor(k.shape, dtype, dev), DeviceTensor(v.shape, dtype, dev)
     tl = capi.DeviceBuffer.from_numpy(np.asarray(kv_lens, dtype=np.int32), dev) if kv_lens is not None else None
+    tm, ms = None, None
+    if mask is not None:
+        mask = np.asarray(mask, dtype=np.float32)
+        ms = mask_strides_for(mask.shape, B, Hq, Sq, k.shape[2])
+        tm = capi.DeviceBuffer.from_numpy(dtypes.encode(mask, dtype), dev)
     tlse = capi.DeviceBuffer(max(B * Hq * Sq, 1) * 4, dev)
     bd = capi.SdpaBwdDesc()
-    bd.fwd = make_desc(tq, tk, tv, to, scale, causal, tl, impl=impl, lse=tlse)
+    bd.fwd = make_desc(tq, tk, tv, to, scale, causal, tl, tm, ms, impl=impl, lse=tlse)
     capi.sdpa_fwd(bd.fwd)
-    for name, t, ptr in (("d_o", tg, "d_o"), ("d_q", tdq, "d_q"), ("d_k", tdk, "d_k"), ("d_v", tdv, "d_v")):
-        setattr(bd, ptr, t.ptr)
+    for name, t in (("d_o", tg), ("d_q", tdq), ("d_k", tdk), ("d_v", tdv)):
+        setattr(bd, name, t.ptr)
         st = _strides3(t.shape)
         for i in range(3):
             getattr(bd, name + "_stride")[i] = st[i]
@@ -156,7 +163,7 @@ def sdpa_backward(q, k, v, d_out, dtype=capi.BF16, scale=None, causal=False, kv_
     capi.sdpa_bwd(bd)
     capi.sync(dev)
     res = tuple(t.to_f32() for t in (to, tdq, tdk, tdv))
-    for t in (tq.buf, tk.buf, tv.buf, tg.buf, to.buf, tdq.buf, tdk.buf, tdv.buf, tl, tlse, ws):
+    for t in (tq.buf, tk.buf, tv.buf, tg.buf, to.buf, tdq.buf, tdk.buf, tdv.buf, tl, tm, tlse, ws):
         if t is not None:
             t.free()
     return res

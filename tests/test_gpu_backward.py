@@ -119,12 +119,69 @@ def test_backward_at_a_few_thousand_tokens(gpu):
     compare("dv", dv, rv.reshape(B, Hkv, S, D))
 
 
+def make_d(seed, B, Hq, Hkv, Sq, Skv, D, Dv, dtype):
+    r = np.random.Generator(np.random.PCG64(seed))
+    mk = lambda *s: dtypes.round_to(r.standard_normal(s, dtype=np.float32), dtype)
+    return mk(B, Hq, Sq, D), mk(B, Hkv, Skv, D), mk(B, Hkv, Skv, Dv), mk(B, Hq, Sq, Dv)
+
+
+@pytest.mark.parametrize("shape", [
+    # B, Hq, Hkv, Sq, Skv, D, Dv, causal, kv_lens, mask kind
+    (2, 2, 2, 4, 4, 8, 8, False, None, None),                    # the reference's smoke shape (shape_ops.rs:1575-1591)
+    (1, 3, 3, 33, 65, 16, 24, False, None, None),                # D != Dv, lengths off the 32-wide tiles
+    (2, 4, 2, 70, 70, 64, 64, True, None, None),
+    (2, 4, 1, 50, 90, 40, 40, True, [90, 37], None),             # grouped queries, causal alignment, ragged keys
+    (2, 2, 2, 45, 61, 32, 32, False, None, "full"),              # dense additive mask with -inf holes
+    (2, 3, 3, 40, 40, 128, 128, False, None, "row"),             # [1, 1, 1, Skv] mask: broadcast over batch, head, row
+    (1, 2, 2, 20, 30, 256, 200, True, None, "head"),             # the widest heads, [1, H, Sq, Skv] mask on top of causal
+], ids=["ref_smoke", "d_ne_dv", "causal", "gqa_ragged", "mask_full", "mask_row", "wide_mask_head"])
+def test_generic_backward_f32_against_the_oracle(gpu, shape):
+    """The reference's own dtype through the generic kernels: 1e-5 of the largest gradient magnitude against the f64 oracle
+    (f32 products and sums in a different order than the reference's tape; measured about 1e-6)."""
+    B, Hq, Hkv, Sq, Skv, D, Dv, causal, lens, mk = shape
+    G = Hq // Hkv
+    say("generic backward f32: %s" % (shape,))
+    q, k, v, go = make_d(21, B, Hq, Hkv, Sq, Skv, D, Dv, capi.F32)
+    r = np.random.Generator(np.random.PCG64(22))
+    mask = None
+    if mk is not None:
+        mshape = {"full": (B, Hq, Sq, Skv), "row": (1, 1, 1, Skv), "head": (1, Hq, Sq, Skv)}[mk]
+        mask = r.standard_normal(mshape, dtype=np.float32)
+        mask[r.random(mshape) < 0.25] = -np.inf
+        mask[..., 0] = 0.0                                       # every row keeps a visible key
+    lens_a = None if lens is None else np.asarray(lens, np.int32)
+    out, dq, dk, dv = host.sdpa_backward(q, k, v, go, capi.F32, causal=causal, kv_lens=lens_a, mask=mask)
+    m5 = None if mask is None else np.broadcast_to(mask, (B, Hq, Sq, Skv)).reshape(B, Hkv, G, Sq, Skv)
+    rq, rk, rv = BW.sdpa_backward(q.reshape(B, Hkv, G, Sq, D), k[:, :, None], v[:, :, None], go.reshape(B, Hkv, G, Sq, Dv),
+                                  mask=m5, causal=causal, kv_lens=None if lens is None else lens_a.reshape(B, 1, 1))
+    compare("dq", dq, rq.reshape(B, Hq, Sq, D), tol=1e-5)
+    compare("dk", dk, rk.reshape(B, Hkv, Skv, D), tol=1e-5)
+    compare("dv", dv, rv.reshape(B, Hkv, Skv, Dv), tol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [capi.BF16, capi.F16])
+def test_generic_and_matrix_core_backward_agree(gpu, dtype):
+    """The same 16-bit problem through both sets of kernels: each within tolerance of the oracle, and of each other."""
+    B, Hq, Hkv, S, D = 2, 4, 2, 200, 128
+    q, k, v, go = make(31, B, Hq, Hkv, S, S, D, dtype)
+    lens = np.array([200, 77], np.int32)
+    a = host.sdpa_backward(q, k, v, go, dtype, causal=True, kv_lens=lens, impl=capi.IMPL_GENERIC)
+    b = host.sdpa_backward(q, k, v, go, dtype, causal=True, kv_lens=lens, impl=capi.IMPL_MFMA)
+    ref = BW.sdpa_backward(q.reshape(B, Hkv, 2, S, D), k[:, :, None], v[:, :, None], go.reshape(B, Hkv, 2, S, D),
+                           causal=True, kv_lens=lens.reshape(B, 1, 1))
+    shapes = [(B, Hq, S, D), (B, Hkv, S, D), (B, Hkv, S, D)]
+    for name, x, y, r_, shp in zip(("dq", "dk", "dv"), a[1:], b[1:], ref, shapes):
+        compare(name + " generic", x, r_.reshape(shp))
+        compare(name + " mfma", y, r_.reshape(shp))
+        compare(name + " generic vs mfma", x, y)
+
+
 def test_backward_refuses_what_it_does_not_cover(gpu):
     q, k, v, go = make(14, 1, 1, 1, 32, 32, 64, capi.BF16)
-    with pytest.raises(capi.RocmError) as e:
-        host.sdpa_backward(q, k, v, go, capi.BF16)
-    assert e.value.code == capi.EUNSUPPORTED and "D == Dv == 128" in e.value.message
-    q, k, v, go = make(14, 1, 1, 1, 32, 32, 128, capi.F32)
+    with pytest.raises(capi.RocmError) as e:                     # the matrix-core kernels, pinned, outside their domain
+        host.sdpa_backward(q, k, v, go, capi.BF16, impl=capi.IMPL_MFMA)
+    assert e.value.code == capi.EUNSUPPORTED
+    q, k, v, go = make(14, 1, 1, 1, 8, 8, 320, capi.F32)         # wider than any kernel
     with pytest.raises(capi.RocmError) as e:
         host.sdpa_backward(q, k, v, go, capi.F32)
     assert e.value.code == capi.EUNSUPPORTED
