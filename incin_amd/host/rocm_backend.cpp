@@ -259,6 +259,22 @@ Error RocmBackend::scaled_dot_product_attention(const RocmStorage& q, const Rocm
 Error RocmBackend::attention(const RocmStorage& q, const RocmStorage& k, const RocmStorage& v, const RocmStorage* mask,
                              std::optional<double> scale, const MaskFacts& facts, RocmStorage* out)
 {
+    return attention_impl(q, k, v, mask, scale, facts, nullptr, out, nullptr);
+}
+
+Error RocmBackend::attention_backward(const RocmStorage& q, const RocmStorage& k, const RocmStorage& v, const RocmStorage* mask,
+                                      std::optional<double> scale, const MaskFacts& facts, const RocmStorage& grad_out,
+                                      RocmStorage* out, AttentionGrads* grads)
+{
+    return attention_impl(q, k, v, mask, scale, facts, &grad_out, out, grads);
+}
+
+// Forward, and with `grads` the backward after it: every launch of the forward keeps its row normalisers, and
+// incin_rocm_sdpa_bwd turns them, the output and the upstream gradient into dq, dk, dv of that launch's slice.
+Error RocmBackend::attention_impl(const RocmStorage& q, const RocmStorage& k, const RocmStorage& v, const RocmStorage* mask,
+                                  std::optional<double> scale, const MaskFacts& facts, const RocmStorage* grad_out,
+                                  RocmStorage* out, AttentionGrads* grads)
+{
     static const char* OP = "scaled_dot_product_attention";
     // -- devices and dtypes, in the order the reference's checks fire ------------------------------------
     if (q.device != k.device || q.device != v.device || (mask && mask->device != q.device))
@@ -323,6 +339,24 @@ Error RocmBackend::attention(const RocmStorage& q, const RocmStorage& k, const R
     if (Error e = alloc_storage(oshape, q.dtype, q.device, &o)) return e;
     const std::vector<int64_t> os(o.strides.begin(), o.strides.end() - 2);
 
+    // -- gradients: fresh contiguous storages of the operands' own shapes -------------------------------------------------
+    RocmStorage gq, gk, gv;
+    std::vector<int64_t> gqs, gks, gvs;
+    if (grads) {
+        if (!grad_out || grad_out->device != q.device) return err(ErrorKind::DeviceMismatch, std::string(OP) + " backward: the upstream gradient lives on another device");
+        if (grad_out->dtype != q.dtype) return err(ErrorKind::DTypeStorageMismatch, std::string(OP) + " backward: the upstream gradient has another dtype");
+        if (grad_out->shape != oshape)
+            return err(ErrorKind::ShapeMismatch, std::string(OP) + " backward: upstream gradient " + shape_str(grad_out->shape) + ", output " + shape_str(oshape));
+        if (!grad_out->is_contiguous())
+            return err(ErrorKind::UnsupportedBackendOperation, std::string(OP) + " backward: the upstream gradient must be contiguous on backend Rocm");
+        if (Error e = alloc_storage(q.shape, q.dtype, q.device, &gq)) return e;
+        if (Error e = alloc_storage(k.shape, k.dtype, k.device, &gk)) return e;
+        if (Error e = alloc_storage(v.shape, v.dtype, v.device, &gv)) return e;
+        broadcast_strides(qb, std::vector<int64_t>(gq.strides.begin(), gq.strides.end() - 2), bshape, &gqs);
+        broadcast_strides(kb, std::vector<int64_t>(gk.strides.begin(), gk.strides.end() - 2), bshape, &gks);
+        broadcast_strides(vb, std::vector<int64_t>(gv.strides.begin(), gv.strides.end() - 2), bshape, &gvs);
+    }
+
     // -- collapse the batch axes into (outer..., B, Hkv, G) ----------------------------------------------------
     // G: the last batch axis when k and v are broadcast along it and q is not (the reference's way to write
     // grouped-query attention: q [.., Hkv, G, S, D] against k, v [.., Hkv, 1, S, D]); Hkv: the axis before it;
@@ -335,6 +369,17 @@ Error RocmBackend::attention(const RocmStorage& q, const RocmStorage& k, const R
     if (next >= 0 && !(g_ax >= 0 && next == 0)) h_ax = next--;
     if (next >= 0) b_ax = next--;
     const int n_outer = next + 1;
+    if (grads) {
+        // A gradient of a broadcast operand is a sum over the broadcast axis (cpu/tape.rs:247-280).  The kernels sum over the
+        // group axis of grouped queries; any other broadcast would need sums across launches, which nothing here does.
+        for (int a = 0; a < nb; ++a) {
+            if (bshape[a] <= 1) continue;
+            if (qs[a] == 0 || ((ks[a] == 0 || vs[a] == 0) && a != g_ax))
+                return err(ErrorKind::UnsupportedBackendOperation,
+                           std::string(OP) + " backward: operands broadcast along batch axis " + std::to_string(a) +
+                               " (only keys and values shared by a group of query heads are summed) on backend Rocm");
+        }
+    }
     int64_t G = g_ax >= 0 ? bshape[g_ax] : 1;
     int64_t Hkv = h_ax >= 0 ? bshape[h_ax] : 1;
     const int64_t B = b_ax >= 0 ? bshape[b_ax] : 1;
@@ -404,7 +449,7 @@ Error RocmBackend::attention(const RocmStorage& q, const RocmStorage& k, const R
     std::vector<int64_t> oidx(outer_axes.size(), 0);
     int64_t n_launch = 1;
     for (int a : outer_axes) n_launch *= bshape[a];
-    std::shared_ptr<RocmBuffer> workspace;
+    std::shared_ptr<RocmBuffer> workspace, bwd_workspace, lse;
     g_launches = 0;
     for (int64_t it = 0; it < n_launch; ++it) {
         int64_t qo = q.offset_elements, ko = k.offset_elements, vo = v.offset_elements, oo = 0, mo = mask ? mask->offset_elements : 0;
@@ -418,6 +463,15 @@ Error RocmBackend::attention(const RocmStorage& q, const RocmStorage& k, const R
         d.v = static_cast<const char*>(v.buffer->ptr()) + vo * (int64_t)isz;
         d.o = static_cast<char*>(o.buffer->ptr()) + oo * (int64_t)isz;
         d.add_mask = dense_mask ? static_cast<const char*>(mask->buffer->ptr()) + mo * (int64_t)isz : nullptr;
+        if (grads) {
+            if (!lse) {
+                void* lp = nullptr;
+                const size_t lbytes = (size_t)std::max<int64_t>(B * Hq * Sq, 1) * sizeof(float);
+                if (Error e = from_status(incin_rocm_alloc(q.device, lbytes, &lp), q.device)) return e;
+                lse = std::make_shared<RocmBuffer>(q.device, lp, lbytes);
+            }
+            d.lse = static_cast<float*>(lse->ptr());
+        }
         size_t ws_bytes = 0;
         int32_t splits = 0;
         d.workspace = nullptr;
@@ -434,15 +488,52 @@ Error RocmBackend::attention(const RocmStorage& q, const RocmStorage& k, const R
         }
         if (Error e = from_status(incin_rocm_sdpa_fwd(&d, nullptr), q.device)) return e;
         ++g_launches;
+        if (grads) {
+            int64_t gqo = 0, gko = 0, gvo = 0;
+            for (size_t a = 0; a < outer_axes.size(); ++a) {
+                const int ax = outer_axes[a];
+                gqo += oidx[a] * gqs[ax]; gko += oidx[a] * gks[ax]; gvo += oidx[a] * gvs[ax];
+            }
+            incin_rocm_sdpa_bwd_desc_t bd;
+            std::memset(&bd, 0, sizeof(bd));
+            bd.fwd = d;
+            bd.fwd.workspace = nullptr;
+            bd.fwd.workspace_bytes = 0;
+            bd.d_o = static_cast<const char*>(grad_out->data()) + oo * (int64_t)isz;
+            bd.d_q = static_cast<char*>(gq.buffer->ptr()) + gqo * (int64_t)isz;
+            bd.d_k = static_cast<char*>(gk.buffer->ptr()) + gko * (int64_t)isz;
+            bd.d_v = static_cast<char*>(gv.buffer->ptr()) + gvo * (int64_t)isz;
+            for (int a = 0; a < 3; ++a) bd.d_o_stride[a] = d.o_stride[a];
+            bd.d_q_stride[0] = st(gqs, b_ax); bd.d_q_stride[1] = st(gqs, head_ax); bd.d_q_stride[2] = D;
+            bd.d_k_stride[0] = st(gks, b_ax); bd.d_k_stride[1] = st(gks, kv_head_ax); bd.d_k_stride[2] = D;
+            bd.d_v_stride[0] = st(gvs, b_ax); bd.d_v_stride[1] = st(gvs, kv_head_ax); bd.d_v_stride[2] = Dv;
+            size_t bws = 0;
+            if (Error e = from_status(incin_rocm_sdpa_bwd_workspace(&bd, &bws), q.device)) return e;
+            if (bws) {
+                if (!bwd_workspace || bwd_workspace->bytes() < bws) {
+                    void* wp = nullptr;
+                    if (Error e = from_status(incin_rocm_alloc(q.device, bws, &wp), q.device)) return e;
+                    bwd_workspace = std::make_shared<RocmBuffer>(q.device, wp, bws);
+                }
+                bd.workspace = bwd_workspace->ptr();
+                bd.workspace_bytes = bwd_workspace->bytes();
+            }
+            if (Error e = from_status(incin_rocm_sdpa_bwd(&bd, nullptr), q.device)) return e;
+        }
         for (int a = (int)oidx.size() - 1; a >= 0; --a) {
             if (++oidx[a] < bshape[outer_axes[a]]) break;
             oidx[a] = 0;
         }
     }
-    // the workspace is used stream-ordered: finish before it is released
-    if (workspace)
+    // the workspaces are used stream-ordered: finish before they are released
+    if (workspace || bwd_workspace || lse)
         if (Error e = from_status(incin_rocm_sync(q.device), q.device)) return e;
     *out = std::move(o);
+    if (grads) {
+        grads->dq = std::move(gq);
+        grads->dk = std::move(gk);
+        grads->dv = std::move(gv);
+    }
     return ok();
 }
 

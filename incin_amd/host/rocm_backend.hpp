@@ -111,10 +111,27 @@ struct RocmBackend {
     static Error attention(const RocmStorage& q, const RocmStorage& k, const RocmStorage& v, const RocmStorage* mask,
                            std::optional<double> scale, const MaskFacts& facts, RocmStorage* out);
 
+    // Gradients of the operator for an upstream gradient of the output's shape: the forward is run once more keeping its
+    // row normalisers, then one backward call per forward launch.  The reference gets these by walking its tape of the
+    // composed ops (cpu/tape.rs:149-176); like there, the mask is a constant.  dq, dk, dv are fresh contiguous storages of
+    // the operands' shapes.  Keys and values shared by a group of query heads get the sum over the group; operands
+    // broadcast along any other batch axis, a non-contiguous upstream gradient and q_lens are UnsupportedBackendOperation.
+    struct AttentionGrads {
+        RocmStorage dq, dk, dv;
+    };
+    static Error attention_backward(const RocmStorage& q, const RocmStorage& k, const RocmStorage& v, const RocmStorage* mask,
+                                    std::optional<double> scale, const MaskFacts& facts, const RocmStorage& grad_out,
+                                    RocmStorage* out, AttentionGrads* grads);
+
     // Reinterpret a contiguous storage under another shape of the same element count (metadata only).
     static Error reshape(const RocmStorage& s, const std::vector<int64_t>& dims, RocmStorage* out);
     // int32 values on the device (key counts of a descriptor).
     static Error upload_i32(const std::vector<int32_t>& values, int32_t device, std::shared_ptr<RocmBuffer>* out);
+
+private:
+    static Error attention_impl(const RocmStorage& q, const RocmStorage& k, const RocmStorage& v, const RocmStorage* mask,
+                                std::optional<double> scale, const MaskFacts& facts, const RocmStorage* grad_out, RocmStorage* out,
+                                AttentionGrads* grads);
 };
 
 // NumPy-style right-aligned broadcast of two shapes (cpu/stride.rs:86-106).

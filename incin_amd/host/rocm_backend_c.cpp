@@ -107,6 +107,22 @@ int incin_host_scaled_dot_product_attention(const incin_host_storage* q, const i
     return give(e, std::move(r), out);
 }
 
+int incin_host_attention_backward(const incin_host_storage* q, const incin_host_storage* k, const incin_host_storage* v,
+                                  const incin_host_storage* mask, int32_t has_scale, double scale, const incin_host_storage* grad_out,
+                                  incin_host_storage** out, incin_host_storage** dq, incin_host_storage** dk, incin_host_storage** dv)
+{
+    RocmStorage r;
+    RocmBackend::AttentionGrads g;
+    Error e = RocmBackend::attention_backward(q->s, k->s, v->s, mask ? &mask->s : nullptr,
+                                              has_scale ? std::optional<double>(scale) : std::nullopt, RocmBackend::MaskFacts{},
+                                              grad_out->s, &r, &g);
+    if (e) return give(e, std::move(r), out);
+    give(e, std::move(g.dq), dq);
+    give(e, std::move(g.dk), dk);
+    give(e, std::move(g.dv), dv);
+    return give(e, std::move(r), out);
+}
+
 void incin_host_release(incin_host_storage* s) { delete s; }
 
 int64_t incin_host_last_launch_count(void) { return incin_rocm_host::last_launch_count(); }

@@ -29,6 +29,10 @@ int incin_host_tag_key_padding(const incin_host_storage* mask, const int32_t* le
 int incin_host_scaled_dot_product_attention(const incin_host_storage* q, const incin_host_storage* k, const incin_host_storage* v,
                                             const incin_host_storage* mask, int32_t has_scale, double scale,
                                             incin_host_storage** out);
+/* the same forward and, for an upstream gradient of the output's shape, the gradients of q, k, v (fresh contiguous storages) */
+int incin_host_attention_backward(const incin_host_storage* q, const incin_host_storage* k, const incin_host_storage* v,
+                                  const incin_host_storage* mask, int32_t has_scale, double scale, const incin_host_storage* grad_out,
+                                  incin_host_storage** out, incin_host_storage** dq, incin_host_storage** dk, incin_host_storage** dv);
 void incin_host_release(incin_host_storage* s);
 /* number of kernel launches (C-ABI sdpa calls) the last attention call on this thread made */
 int64_t incin_host_last_launch_count(void);

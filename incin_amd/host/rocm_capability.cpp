@@ -162,8 +162,9 @@ const std::vector<CapabilityRule>& rocm_capabilities()
         {OperationKind::Broadcast, ROCM_DTYPES, ANY_VIEW, 0, MAX_RANK, false, PRECISE, ImplementationKind::Native},
         // reshape re-addresses contiguous storage; a view has to be materialised by the caller first
         {OperationKind::Reshape, ROCM_DTYPES, {LayoutClass::Contiguous}, 0, MAX_RANK, false, PRECISE, ImplementationKind::Native},
-        // scaled_dot_product_attention, forward only
-        {OperationKind::Attention, ROCM_DTYPES, ROW_VIEWS, 2, MAX_RANK, false, PRECISE, ImplementationKind::Native},
+        // scaled_dot_product_attention and its gradients (RocmBackend::attention_backward; broadcast batch axes other than
+        // the group axis of grouped queries are refused by the operator itself)
+        {OperationKind::Attention, ROCM_DTYPES, ROW_VIEWS, 2, MAX_RANK, true, PRECISE, ImplementationKind::Native},
     };
     return rules;
 }

@@ -265,6 +265,91 @@ std::vector<Check> attention_checks(const Subject& s)
     };
 }
 
+// Gradients of the same hand-composed heads for an upstream gradient g, evaluated in f64 from the definition (the chain
+// the reference's tape walks, cpu/tape.rs:149-176): P = softmax rows, dV_j = sum_i P_ij g_i, dP_ij = g_i v_j,
+// dS_ij = P_ij (dP_ij - sum_l P_il dP_il), dq_i = sum_j dS_ij k_j, dk_j = sum_i dS_ij q_i (scale 1, D = 1).
+void closed_form_gradients(const float q[2], const float k[2], const float v[2], const float g[2], double dq[2], double dk[2], double dv[2])
+{
+    double P[2][2], dS[2][2];
+    for (int i = 0; i < 2; ++i) {
+        const double s0 = (double)q[i] * k[0], s1 = (double)q[i] * k[1], m = std::fmax(s0, s1);
+        const double e0 = std::exp(s0 - m), e1 = std::exp(s1 - m);
+        P[i][0] = e0 / (e0 + e1);
+        P[i][1] = e1 / (e0 + e1);
+        const double dP0 = (double)g[i] * v[0], dP1 = (double)g[i] * v[1], D = P[i][0] * dP0 + P[i][1] * dP1;
+        dS[i][0] = P[i][0] * (dP0 - D);
+        dS[i][1] = P[i][1] * (dP1 - D);
+        dq[i] = dS[i][0] * k[0] + dS[i][1] * k[1];
+    }
+    for (int j = 0; j < 2; ++j) {
+        dv[j] = P[0][j] * g[0] + P[1][j] * g[1];
+        dk[j] = dS[0][j] * q[0] + dS[1][j] * q[1];
+    }
+}
+
+std::vector<Check> attention_training_checks(const Subject& s)
+{
+    cap::CapabilityQuery tq = query(cap::OperationKind::Attention, 3);
+    tq.training = true;
+    const cap::SupportLevel support = cap::support(cap::DeviceKind::Rocm, tq);
+    const std::vector<const char*> names = {"attention_gradients_are_within_tolerance", "attention_gradients_have_their_operands_shapes"};
+    if (!support.is_supported()) return skipped(names, support);
+    const std::vector<float> q = {1, 2, 0.5f, -0.5f}, k = {1, -1, 2, 1}, v = {3, 5, 7, 11}, g = {1, -2, 0.5f, 3};      // [2 heads, 2, 1]
+    return {
+        guarded(names[0], [&]() -> std::string {
+            RocmStorage sq, sk, sv, sg, o;
+            for (auto [st, vals] : {std::pair{&sq, &q}, std::pair{&sk, &k}, std::pair{&sv, &v}, std::pair{&sg, &g}})
+                if (std::string e = s.storage({2, 2, 1}, *vals, st); !e.empty()) return e;
+            RocmBackend::AttentionGrads grads;
+            if (Error e = RocmBackend::attention_backward(sq, sk, sv, nullptr, 1.0, RocmBackend::MaskFacts{}, sg, &o, &grads)) return e.message;
+            std::vector<float> gq, gk, gv;
+            if (std::string e = s.values(grads.dq, &gq); !e.empty()) return e;
+            if (std::string e = s.values(grads.dk, &gk); !e.empty()) return e;
+            if (std::string e = s.values(grads.dv, &gv); !e.empty()) return e;
+            if (gq.size() != 4 || gk.size() != 4 || gv.size() != 4) return "gradients of [2, 2, 1] operands do not hold 4 values each";
+            for (int h = 0; h < 2; ++h) {
+                double wq[2], wk[2], wv[2];
+                closed_form_gradients(&q[2 * h], &k[2 * h], &v[2 * h], &g[2 * h], wq, wk, wv);
+                for (int i = 0; i < 2; ++i) {
+                    const std::pair<const char*, std::pair<double, float>> rows[] = {
+                        {"dq", {wq[i], gq[2 * h + i]}}, {"dk", {wk[i], gk[2 * h + i]}}, {"dv", {wv[i], gv[2 * h + i]}}};
+                    for (const auto& [what, pr] : rows)
+                        if (!F32_ACCUMULATED.accepts(pr.first, pr.second))
+                            return std::string(what) + " of head " + std::to_string(h) + " row " + std::to_string(i) + " is " +
+                                   std::to_string(pr.second) + ", outside 1e-5 of " + std::to_string(pr.first);
+                }
+            }
+            return "";
+        }),
+        guarded(names[1], [&]() -> std::string {
+            // grouped queries: k and v shared by 3 query heads get gradients of their own shape, summed over the group; with
+            // all values equal the output does not depend on the weights, so dq = dk = 0 and every dv row adds up the upstream rows
+            RocmStorage sq, sk, sv, sg, o;
+            if (std::string e = s.storage({2, 1, 3, 5, 8}, std::vector<float>(240, 0.25f), &sq); !e.empty()) return e;
+            if (std::string e = s.storage({2, 1, 1, 7, 8}, std::vector<float>(112, 0.5f), &sk); !e.empty()) return e;
+            if (std::string e = s.storage({2, 1, 1, 7, 4}, std::vector<float>(56, 2.0f), &sv); !e.empty()) return e;
+            if (std::string e = s.storage({2, 1, 3, 5, 4}, std::vector<float>(120, 1.0f), &sg); !e.empty()) return e;
+            RocmBackend::AttentionGrads grads;
+            if (Error e = RocmBackend::attention_backward(sq, sk, sv, nullptr, std::nullopt, RocmBackend::MaskFacts{}, sg, &o, &grads)) return e.message;
+            if (grads.dq.shape != sq.shape || grads.dk.shape != sk.shape || grads.dv.shape != sv.shape)
+                return "gradients report " + dims_str(grads.dq.shape) + ", " + dims_str(grads.dk.shape) + ", " + dims_str(grads.dv.shape) +
+                       " for operands " + dims_str(sq.shape) + ", " + dims_str(sk.shape) + ", " + dims_str(sv.shape);
+            std::vector<float> gq, gk, gv;
+            if (std::string e = s.values(grads.dq, &gq); !e.empty()) return e;
+            if (std::string e = s.values(grads.dk, &gk); !e.empty()) return e;
+            if (std::string e = s.values(grads.dv, &gv); !e.empty()) return e;
+            for (float x : gq)
+                if (!F32_ACCUMULATED.accepts(0.0, x)) return "dq of an output that does not depend on q came out as " + std::to_string(x);
+            for (float x : gk)
+                if (!F32_ACCUMULATED.accepts(0.0, x)) return "dk of an output that does not depend on k came out as " + std::to_string(x);
+            // uniform weights 1/7 from 3 heads x 5 rows of ones: 15 / 7 per element
+            for (float x : gv)
+                if (!F32_ACCUMULATED.accepts(15.0 / 7.0, x)) return "dv under uniform weights came out as " + std::to_string(x) + ", not 15/7";
+            return "";
+        }),
+    };
+}
+
 std::string registry_agrees(const Subject& s)
 {
     auto word = [](bool b, const char* yes, const char* no) { return std::string(b ? yes : no); };
@@ -291,6 +376,14 @@ std::string registry_agrees(const Subject& s)
     if (attn_claimed != attn_ran)
         return "the registry says attention is " + word(attn_claimed, "supported", "unsupported") + " and executing it " +
                word(attn_ran, "succeeded", "failed");
+    cap::CapabilityQuery training = query(cap::OperationKind::Attention, 2);
+    training.training = true;
+    const bool train_claimed = cap::support(cap::DeviceKind::Rocm, training).is_supported();
+    RocmBackend::AttentionGrads grads;
+    const bool train_ran = !RocmBackend::attention_backward(in, in, in, nullptr, std::nullopt, RocmBackend::MaskFacts{}, in, &o, &grads);
+    if (train_claimed != train_ran)
+        return "the registry says training attention is " + word(train_claimed, "supported", "unsupported") + " and its backward " +
+               word(train_ran, "succeeded", "failed");
     // a dtype the storage cannot represent must be refused by the registry rather than discovered in a kernel
     bool refuses = false;
     for (cap::DTypeId d : {cap::DTypeId::Q8_0, cap::DTypeId::F64, cap::DTypeId::U8}) {
@@ -324,6 +417,7 @@ Report run(int device)
     for (Check& c : matmul_checks(s)) r.checks.push_back(std::move(c));
     for (Check& c : reshape_checks(s)) r.checks.push_back(std::move(c));
     for (Check& c : attention_checks(s)) r.checks.push_back(std::move(c));
+    for (Check& c : attention_training_checks(s)) r.checks.push_back(std::move(c));
     r.checks.push_back(guarded("the_registry_and_the_executor_agree", [&] { return registry_agrees(s); }));
     return r;
 }

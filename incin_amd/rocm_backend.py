@@ -24,7 +24,7 @@ EXPORTS = [
     "incin_host_last_error", "incin_host_from_bytes", "incin_host_numel", "incin_host_rank", "incin_host_shape",
     "incin_host_dtype", "incin_host_to_bytes", "incin_host_transpose", "incin_host_broadcast_as",
     "incin_host_narrow", "incin_host_tag_causal", "incin_host_tag_key_padding",
-    "incin_host_scaled_dot_product_attention", "incin_host_release", "incin_host_last_launch_count",
+    "incin_host_scaled_dot_product_attention", "incin_host_attention_backward", "incin_host_release", "incin_host_last_launch_count",
     "incin_host_capability_name", "incin_host_capability_max_rank", "incin_host_capability_support",
     "incin_host_capability_rule_count", "incin_host_capability_rule", "incin_host_capability_docs",
     "incin_host_lower_attention", "incin_host_attention_spec_out_dims", "incin_host_execute_attention",
@@ -67,6 +67,8 @@ def lib():
         L.incin_host_tag_key_padding.argtypes = [C.c_void_p, C.POINTER(C.c_int32), C.c_int64, C.POINTER(C.c_void_p)]
         L.incin_host_scaled_dot_product_attention.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32,
                                                               C.c_double, C.POINTER(C.c_void_p)]
+        L.incin_host_attention_backward.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_double, C.c_void_p] + \
+                                                   [C.POINTER(C.c_void_p)] * 4
         L.incin_host_capability_name.restype = C.c_char_p
         L.incin_host_capability_name.argtypes = [C.c_int32, C.c_int32]
         L.incin_host_capability_max_rank.restype = C.c_int32
@@ -201,6 +203,15 @@ def scaled_dot_product_attention(q, k, v, mask=None, scale=None):
         q._h, k._h, v._h, mask._h if mask is not None else None,
         0 if scale is None else 1, 0.0 if scale is None else float(scale), C.byref(out)))
     return RocmStorage(out.value)
+
+
+def attention_backward(q, k, v, grad_out, mask=None, scale=None):
+    """(out, dq, dk, dv): the operator and its gradients for an upstream gradient of the output's shape."""
+    hs = [C.c_void_p() for _ in range(4)]
+    _check(lib().incin_host_attention_backward(
+        q._h, k._h, v._h, mask._h if mask is not None else None,
+        0 if scale is None else 1, 0.0 if scale is None else float(scale), grad_out._h, *[C.byref(h) for h in hs]))
+    return tuple(RocmStorage(h.value) for h in hs)
 
 
 def last_launch_count():

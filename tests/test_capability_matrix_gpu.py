@@ -75,6 +75,29 @@ def test_attention_rule_boundary_cases_execute(gpu, dtype, layout, rank):
     assert err <= TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", RULES["attention"].dtypes)
+@pytest.mark.parametrize("layout", RULES["attention"].layouts)
+@pytest.mark.parametrize("rank", [RULES["attention"].min_rank, RULES["attention"].max_rank])
+def test_attention_rule_boundary_cases_train(gpu, dtype, layout, rank):
+    """The same cells with `training` set: the rule says yes, so the gradients come out and match the backward oracle
+    (1e-5 of the largest gradient magnitude for f32, 2e-2 for the 16-bit types)."""
+    from oracle import sdpa_backward as BW
+    assert RULES["attention"].training
+    case = RC.CapabilityQuery("attention", dtype, layout, rank, training=True)
+    assert RC.support("rocm", case).level == "native"
+    qs, ks, vs = shapes_of_rank(rank)
+    say("capability cell %s: q%s k%s" % (case, qs, ks))
+    q, k, v = rnd(1, qs, dtype), rnd(2, ks, dtype), rnd(3, vs, dtype)
+    go = rnd(6, qs[:-1] + (vs[-1],), dtype)
+    out, dq, dk, dv = RB.attention_backward(operand(q, dtype, layout), operand(k, dtype, layout), operand(v, dtype, layout),
+                                            RB.RocmStorage.from_numpy(go, CODE[dtype]))
+    tol = 1e-5 if dtype == "f32" else 2e-2
+    for name, got, ref in zip(("dq", "dk", "dv"), (dq, dk, dv), BW.sdpa_backward(q, k, v, go)):
+        err = float(np.abs(got.to_numpy() - ref).max() / np.abs(ref).max())
+        say("   %s: max-abs err / max|ref| %.3e" % (name, err))
+        assert got.shape == ref.shape and err <= tol
+
+
 @pytest.mark.parametrize("dtype", RULES["storage"].dtypes)
 @pytest.mark.parametrize("rank", [RULES["storage"].min_rank, RULES["storage"].max_rank])
 def test_storage_and_broadcast_rules_execute(gpu, dtype, rank):

@@ -56,8 +56,9 @@ def test_unsupported_cells_return_the_documented_constraint():
     assert (s.reason, s.message) == ("Layout", "layout strided is unsupported for attention")
     s = RC.support("rocm", Q("attention", "f32", "contiguous", 1))
     assert (s.reason, s.message) == ("Rank", "rank 1 is unsupported for attention; expected 2..=8")
-    s = RC.support("rocm", Q("attention", "bf16", "contiguous", 4, training=True))
-    assert (s.reason, s.message) == ("Training", "training is unsupported for attention")
+    assert RC.support("rocm", Q("attention", "bf16", "contiguous", 4, training=True)).level == "native"
+    s = RC.support("rocm", Q("reshape", "bf16", "contiguous", 4, training=True))
+    assert (s.reason, s.message) == ("Training", "training is unsupported for reshape")
     s = RC.support("rocm", Q("attention", "bf16", "contiguous", 4, math_mode="fast"))
     assert (s.reason, s.message) == ("MathMode", "math mode fast is unsupported for attention")
     # not registered at all: pointwise has no family rule either
@@ -97,5 +98,5 @@ def test_checked_in_table_is_what_the_renderer_produces():
             f.write(text)
     assert open(DOC).read() == text, "regenerate with INCIN_DOCS=overwrite python -m pytest tests/test_capability_registry.py"
     assert "| `attention` | `f32` | `bf16`, `f16`, `f32` |" in text
-    assert "| `attention` | `bf16`, `f16`, `f32` | `contiguous`, `row-wise` | 2+ | no | native |" in text
+    assert "| `attention` | `bf16`, `f16`, `f32` | `contiguous`, `row-wise` | 2+ | yes | native |" in text
     assert "| `broadcast` | — | `bf16`, `f16`, `f32` |" in text

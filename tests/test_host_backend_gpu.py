@@ -195,3 +195,60 @@ def test_error_behaviour(gpu):
     # k with a strided last axis has no kernel on this backend
     kt = f(np.ones((2, 8, 6), np.float32)).transpose(1, 2)
     assert kind(q, kt, v) == "UnsupportedBackendOperation"
+
+
+# ---- gradients through the host mirror ------------------------------------------------------------------------------
+def grad_close(name, got, ref, tol):
+    ref = np.asarray(ref, np.float64)
+    scale = float(np.abs(ref).max()) or 1.0
+    err = float(np.abs(got - ref).max()) / scale
+    say("   %s: max-abs err / max|ref| = %.3e" % (name, err))
+    assert got.shape == ref.shape and err <= tol, "%s: %.3e" % (name, err)
+
+
+@pytest.mark.parametrize("case", [
+    # q shape, k shape, v shape, dtype, mask kind
+    ((5, 8), (7, 8), (7, 6), RB.F32, None),                              # rank 2, the shape of the reference's matmul tests
+    ((2, 3, 9, 16), (2, 3, 11, 16), (2, 3, 11, 16), RB.F32, "dense"),    # [B, H, S, D] with a dense mask
+    ((2, 2, 4, 20, 128), (2, 2, 1, 20, 128), (2, 2, 1, 20, 128), RB.BF16, "causal"),    # grouped queries the reference's way
+    ((3, 2, 2, 10, 32), (3, 2, 2, 12, 32), (3, 2, 2, 12, 32), RB.F32, None),            # an outer axis: one launch per index
+    ((2, 6, 40, 128), (2, 1, 40, 128), (2, 1, 40, 128), RB.F16, "causal"),              # one shared kv head
+], ids=["rank2", "dense_mask", "gqa_causal", "outer_axis", "shared_kv_head"])
+def test_gradients_through_the_host_mirror(gpu, case):
+    from oracle import sdpa_backward as BW
+    qs, ks, vs, dtype, mk = case
+    say("host mirror backward: %s" % (case,))
+    q, k, v = rnd(41, qs, dtype), rnd(42, ks, dtype), rnd(43, vs, dtype)
+    go = rnd(44, np.broadcast_shapes(qs[:-2], ks[:-2]) + (qs[-2], vs[-1]), dtype)
+    Sq, Skv = qs[-2], ks[-2]
+    mask_np, mask = None, None
+    if mk == "dense":
+        mask_np = rnd(45, (1, qs[1], Sq, Skv), dtype)
+        mask_np[..., 3] = -np.inf
+        mask = RB.RocmStorage.from_numpy(mask_np, dtype)
+    elif mk == "causal":
+        mask_np = np.triu(np.full((Sq, Skv), -np.inf, np.float32), 1 + Skv - Sq)
+        mask = RB.RocmStorage.from_numpy(mask_np, dtype).tag_causal()
+    S = lambda a: RB.RocmStorage.from_numpy(a, dtype)
+    out, dq, dk, dv = RB.attention_backward(S(q), S(k), S(v), S(go), mask, None)
+    assert dq.shape == qs and dk.shape == ks and dv.shape == vs
+    rq, rk, rv = BW.sdpa_backward(q, k, v, go, mask=mask_np)
+    tol = 1e-5 if dtype == RB.F32 else 2e-2
+    grad_close("dq", dq.to_numpy(), rq, tol)
+    grad_close("dk", dk.to_numpy(), rk, tol)
+    grad_close("dv", dv.to_numpy(), rv, tol)
+    ref = O.sdpa(q, k, v, mask=mask_np) if hasattr(O, "sdpa") else None
+    if ref is not None:
+        close(out.to_numpy(), ref, TOL[dtype], "forward beside the gradients")
+
+
+def test_gradients_refused_for_broadcast_operands(gpu):
+    q, k, v = rnd(51, (2, 3, 4, 8), RB.F32), rnd(52, (1, 3, 5, 8), RB.F32), rnd(53, (1, 3, 5, 8), RB.F32)
+    go = rnd(54, (2, 3, 4, 8), RB.F32)
+    S = RB.RocmStorage.from_numpy
+    with pytest.raises(RB.BackendError) as e:       # k, v shared by the batch entries: their gradient is a sum over launches
+        RB.attention_backward(S(q), S(k), S(v), S(go))
+    assert e.value.kind == "UnsupportedBackendOperation" and "broadcast" in e.value.message
+    with pytest.raises(RB.BackendError) as e:
+        RB.attention_backward(S(q), S(rnd(55, (2, 3, 5, 8), RB.F32)), S(rnd(56, (2, 3, 5, 8), RB.F32)), S(go[:, :, :3]))
+    assert e.value.kind == "ShapeMismatch"
