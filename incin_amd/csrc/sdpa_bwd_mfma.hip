@@ -271,11 +271,15 @@ constexpr int BWD_RING = 4;        // matrix operands in flight from LDS (reads 
 // S and dP leave no room for a second one.  So two wavefronts share each block of 32 keys, eight per workgroup, two
 // per SIMD, and split a 64-query tile both ways:
 //   first   S and dP of ONE 32-row query block (16 matrix instructions), P and dS from them, written to LDS;
-//   then    (after a barrier) dV and dK of the 32 keys for ONE half of the head dimension, over both query blocks
-//           (16 matrix instructions; the other block's P and dS come from the partner through LDS).
-// Each holds 64 accumulators, the matrix work is not duplicated, and what one wavefront issues runs under the matrix
-// instructions of the other.  The S and dP accumulators do not start from zero but from -L_i log2(e) and -D_i (staged
-// per tile next to the Q and dO rows), so P = exp2(S) and dS = P * dP need no subtraction.
+//   then    dV and dK of the 32 keys for ONE half of the head dimension, over both query blocks (16 matrix
+//           instructions; P and dS of both blocks come back from LDS, the partner's and the wavefront's own).
+// Each holds 64 accumulators and the matrix work is not duplicated.  The two halves are pipelined over tiles: a step
+// computes S, dP of tile t, then dV, dK of tile t - 1 with the exponentials and products that make P, dS of tile t
+// issued between those matrix instructions (the workgroup's barriers keep the two wavefronts of a SIMD in the same
+// phase, so what overlaps a wavefront's matrix instructions has to come from its own stream), and writes P, dS of tile
+// t after a barrier.  Tiles t - 1 and t stay resident while tile t + 1 is copied: three stages.  The S and dP
+// accumulators do not start from zero but from -L_i log2(e) and -D_i (staged per tile next to the Q and dO rows), so
+// P = exp2(S) and dS = P * dP need no subtraction.
 template <typename T>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
@@ -288,7 +292,7 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
     constexpr int STAGE = 2 * L::TILE_BYTES + 1024;     // Q rows, dO rows, 64 x -L_i log2(e), 64 x -D_i (and padding)
     constexpr int XCHG = 4 * 2 * 4 * 1024;              // [key block][query block][P lo, P hi, dS lo, dS hi]: 64 lanes x 16 bytes
     const SdpaParams& p = bp.f;
-    constexpr int NS = 3;                               // stages: copies run two tiles ahead
+    constexpr int NS = 3;                               // stages: tiles t - 1 and t in use, tile t + 1 arriving
     __shared__ __attribute__((aligned(1024))) char smem[NS * STAGE + XCHG];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -401,103 +405,119 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
     const char* const xother = smem + NS * STAGE + ((kb * 2 + 1 - role) * 4) * 1024 + lane * 16;
     const int own_rows = role * 32 * L::ROWB, other_rows = (1 - role) * 32 * L::ROWB;
 
-    auto tile = [&](int stage, int i0) __attribute__((always_inline)) {
+    // One step of the pipeline: S, dP of tile t (16 matrix instructions), then dV, dK of tile t - 1 (16 more, operands from
+    // that tile's stage and from the exchange buffer) with P and dS of tile t computed on the vector ALU between them, then
+    // - after a barrier, when everyone has read tile t - 1's P and dS - this wavefront's P and dS of tile t into the buffer.
+    // WITH_A = false is the step after the last tile: only the second half.
+    auto step = [&](int stage, int pstage, int i0, bool has_prev, auto WITH_A_) __attribute__((always_inline)) {
+        constexpr bool WITH_A = decltype(WITH_A_)::value;
         const char* qt = smem + stage * STAGE;
         const char* gt = qt + L::TILE_BYTES;
         const char* nl = gt + L::TILE_BYTES + role * 128;
-        // Matrix instruction i of the tile and its LDS operand.  0..15: S (even i) and dP (odd i) of the own query block,
-        // k-step i / 2.  16..31: m = i - 16; the own block's rows first (m < 8), then the partner's; 16-row half (m / 4) % 2;
-        // column block (m / 2) % 2 of this wavefront's two; dV from dO^T and P (even m), dK from Q^T and dS (odd m).
+        const char* pq = smem + pstage * STAGE;
+        const char* pg = pq + L::TILE_BYTES;
         vec8 ring[R];
-        auto fetch = [&](int i) __attribute__((always_inline)) {
-            if (i < 16) {
-                ring[i % R] = *(const vec8*)((i % 2 ? gt : qt) + own_rows + tl.row_addr[i / 2]);
-            } else {
-                const int m = i - 16, h = (m / 4) % 2, d = (m / 2) % 2;
-                ring[i % R] = tl.tr_op((m % 2 ? qt : gt) + (m < 8 ? own_rows : other_rows), d, h);
-            }
-        };
         floatx16 sa, da;
-        vec8 pp[2], ds[2], opp[2], ods[2];
-        auto mma = [&](int i) __attribute__((always_inline)) {
-            if (i < 16) {
+        vec8 pp[2], ds[2];
+        if (WITH_A) {
+            // The accumulators start from -L_i log2(e) and -D_i.  What the mask hides starts from -inf instead and ends as
+            // P = 0, dS = 0 * (finite): only the causal edge needs that here, rows past Sq arrive as zeros throughout (dO = 0,
+            // dP = 0), rows without any visible key carry -inf already, and keys past kv_len are zeroed at the end.
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                const float4v a = *(const float4v*)(nl + (8 * r4 + 4 * g) * 4);
+                const float4v d = *(const float4v*)(nl + 256 + (8 * r4 + 4 * g) * 4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { sa[4 * r4 + e] = a[e]; da[4 * r4 + e] = d[e]; }
+            }
+            // S (even i) and dP (odd i) of the own query block, k-step i / 2
+            auto fetch_a = [&](int i) __attribute__((always_inline)) {
+                ring[i % R] = *(const vec8*)((i % 2 ? gt : qt) + own_rows + tl.row_addr[i / 2]);
+            };
+#pragma unroll
+            for (int i = 0; i < R; ++i) fetch_a(i);
+            if (i0 < i_all_wave) {          // some row of the tile does not see every key of this wavefront
+                const int rel = lo_i - i0 - 4 * g - 32 * role;      // register r is row i0 + 32*role + 8*(r/4) + 4*g + (r%4)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    if (8 * (r / 4) + (r % 4) < rel) sa[r] = -INFINITY;
+            }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
                 if (i % 2 == 0) sa = Mma<T>::run(ring[i % R], kreg[i / 2], sa);
                 else da = Mma<T>::run(ring[i % R], vreg[i / 2], da);
-            } else {
-                const int m = i - 16, h = (m / 4) % 2, d = (m / 2) % 2;
-                if (m % 2 == 0) dv_acc[d] = Mma<T>::run(ring[i % R], m < 8 ? pp[h] : opp[h], dv_acc[d]);
-                else dk_acc[d] = Mma<T>::run(ring[i % R], m < 8 ? ds[h] : ods[h], dk_acc[d]);
+                if (i + R < 16) fetch_a(i + R);
             }
-        };
-
-        // The accumulators start from -L_i log2(e) and -D_i.  What the mask hides starts from -inf instead and ends as
-        // P = 0, dS = 0 * (finite): only the causal edge needs that here, rows past Sq arrive as zeros throughout (dO = 0,
-        // dP = 0), rows without any visible key carry -inf already, and keys past kv_len are zeroed at the end.
-#pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) {
-            const float4v a = *(const float4v*)(nl + (8 * r4 + 4 * g) * 4);
-            const float4v d = *(const float4v*)(nl + 256 + (8 * r4 + 4 * g) * 4);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) { sa[4 * r4 + e] = a[e]; da[4 * r4 + e] = d[e]; }
         }
-#pragma unroll
-        for (int i = 0; i < R; ++i) fetch(i);
-        if (i0 < i_all_wave) {          // some row of the tile does not see every key of this wavefront
-            const int rel = lo_i - i0 - 4 * g - 32 * role;      // register r is row i0 + 32*role + 8*(r/4) + 4*g + (r%4)
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-                if (8 * (r / 4) + (r % 4) < rel) sa[r] = -INFINITY;
-        }
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            mma(i);
-            fetch(i + R);
-        }
-        // P and dS, rounded for the next products
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
+        // P and dS of register r of the own query block, rounded for the next products
+        auto soft = [&](int r) __attribute__((always_inline)) {
+            if (!WITH_A) return;
             const float pr = __builtin_amdgcn_exp2f(sa[r]);
             pp[r / 8][r % 8] = (T)pr;
             ds[r / 8][r % 8] = (T)(pr * da[r]);
-        }
-        *(vec8*)(xmine) = pp[0];
-        *(vec8*)(xmine + 1024) = pp[1];
-        *(vec8*)(xmine + 2048) = ds[0];
-        *(vec8*)(xmine + 3072) = ds[1];
-        __syncthreads();
-        opp[0] = *(const vec8*)(xother);
-        opp[1] = *(const vec8*)(xother + 1024);
-        ods[0] = *(const vec8*)(xother + 2048);
-        ods[1] = *(const vec8*)(xother + 3072);
+        };
+        if (has_prev) {
+            // Matrix instruction m of the second half: group m / 4 = (own query block, rows 0-15), (own, 16-31), (partner's, 0-15),
+            // (partner's, 16-31); column block (m / 2) % 2 of this wavefront's two; dV from dO^T and P (even m), dK from Q^T and dS (odd).
+            auto fetch_b = [&](int m) __attribute__((always_inline)) {
+                ring[m % R] = tl.tr_op((m % 2 ? pq : pg) + (m < 8 ? own_rows : other_rows), (m / 2) % 2, (m / 4) % 2);
+            };
+            vec8 bp_[2], bs_[2];        // P and dS of a group, two groups in flight
+            auto fetch_group = [&](int grp) __attribute__((always_inline)) {
+                const char* x = (grp < 2 ? (const char*)xmine : xother) + (grp % 2) * 1024;
+                bp_[grp % 2] = *(const vec8*)x;
+                bs_[grp % 2] = *(const vec8*)(x + 2048);
+            };
+            fetch_group(0);
+            fetch_group(1);
 #pragma unroll
-        for (int i = 16; i < 32; ++i) {
-            mma(i);
-            if (i + R < 32) fetch(i + R);
+            for (int m = 0; m < R; ++m) fetch_b(m);
+#pragma unroll
+            for (int m = 0; m < 16; ++m) {
+                const int d = (m / 2) % 2;
+                if (m % 2 == 0) dv_acc[d] = Mma<T>::run(ring[m % R], bp_[(m / 4) % 2], dv_acc[d]);
+                else dk_acc[d] = Mma<T>::run(ring[m % R], bs_[(m / 4) % 2], dk_acc[d]);
+                if (m + R < 16) fetch_b(m + R);
+                if (m % 4 == 3 && m / 4 + 2 < 4) fetch_group(m / 4 + 2);
+                soft(m);
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) soft(r);
+        }
+        if (WITH_A) {
+            __syncthreads();            // everyone has read the previous tile's P and dS
+            *(vec8*)(xmine) = pp[0];
+            *(vec8*)(xmine + 1024) = pp[1];
+            *(vec8*)(xmine + 2048) = ds[0];
+            *(vec8*)(xmine + 3072) = ds[1];
         }
     };
 
     if (n_tiles > 0) {
         to_head(0);
         issue(0);
-        if (n_tiles > 1) issue(1);
     }
-    int i0 = t_begin * PF_BN, stage = 0;
+    int i0 = t_begin * PF_BN, stage = 0, pstage = 0;
     for (int t = 0; t < n_tiles; ++t) {
-        // Tile t has landed for everyone (memory operations complete in order: all but the copies of tile t + 1, which
-        // are 4 per wavefront and one more in the two that fetch the per-row floats) and everyone is done with tile
-        // t - 1: its stage and the exchange buffer are free.
-        if (t + 1 >= n_tiles) __builtin_amdgcn_s_waitcnt(0x0F70);        // vmcnt(0)
-        else if (wave < 2) __builtin_amdgcn_s_waitcnt(0x0F75);           // vmcnt(5)
-        else __builtin_amdgcn_s_waitcnt(0x0F74);                         // vmcnt(4)
+        // Tile t has landed for everyone, tile t - 1's P and dS are in the exchange buffer, and everyone is done with tile
+        // t - 2: its stage is free for tile t + 1.
+        __builtin_amdgcn_s_waitcnt(0x0F70);             // vmcnt(0)
         asm volatile("" ::: "memory");
         __syncthreads();
-        if (t + 2 < n_tiles) issue(stage == 0 ? 2 : stage - 1);          // stage of tile t + 2 = stage of tile t - 1
+        const int nstage = stage == 2 ? 0 : stage + 1;
+        if (t + 1 < n_tiles) issue(nstage);
         // Every wavefront computes every tile: one whose keys no row of the tile sees (the first tile or two under a
         // causal mask) works on -inf, and would wait at the barriers for the others anyway.
-        tile(stage, i0);
-        stage = stage == 2 ? 0 : stage + 1;
+        step(stage, pstage, i0, t > 0, std::true_type{});
+        pstage = stage;
+        stage = nstage;
         i0 += PF_BN;
         if (i0 >= n_qt * PF_BN) i0 = t_begin * PF_BN;       // next head of the group
+    }
+    if (n_tiles > 0) {
+        __syncthreads();
+        step(stage, pstage, i0, true, std::false_type{});
     }
 
     if (my_j < Skv) {
