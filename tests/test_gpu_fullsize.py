@@ -150,3 +150,31 @@ def test_config5_gqa_ragged_causal_full(gpu):
         n = int(lens[b])
         assert np.array_equal(got[b, :, :n], got2[b, :, :n])
         assert not np.isnan(got2[b, :, :n]).any()
+
+
+def test_config3_backward_full(gpu):
+    """The backward at configuration 3's full size (bf16 causal, B=8 H=16 S=4096 D=128): two (batch, head) slices against
+    the float64 backward oracle, and properties that hold for every head and need no oracle - the weights of a row sum to
+    one, so sum_j dV_j = sum_i dO_i; the last key is seen by the last query only, so its dV is P_last,last * dO_last."""
+    from oracle import sdpa_backward as BW
+    B, H, S, D = 8, 16, 4096, 128
+    say("config 3 backward at full size")
+    q, k, v, go = (gen(70 + i, (B, H, S, D), capi.BF16) for i in range(4))
+    out, dq, dk, dv = host.sdpa_backward(q, k, v, go, capi.BF16, causal=True)
+    assert not np.isnan(dq).any() and not np.isnan(dk).any() and not np.isnan(dv).any()
+    # every head: total mass of dV (f32 sums of bf16-rounded rows; 4096 rows of magnitude ~1 summed: tolerance on the sum)
+    mass_got, mass_ref = dv.astype(np.float64).sum(2), go.astype(np.float64).sum(2)
+    err = float(np.abs(mass_got - mass_ref).max())
+    say("   sum_j dV_j = sum_i dO_i over all %d heads: max-abs err %.3e (sums of magnitude %.1f)" % (B * H, err, float(np.abs(mass_ref).max())))
+    assert err <= 2e-2 * float(np.abs(mass_ref).max())
+    # three slices against the oracle; in them also: the last key meets the last query only -> dV_last = P_last,last * dO_last
+    x_last = (q[:, :, -1].astype(np.float64) * k[:, :, -1]).sum(-1) / np.sqrt(D)
+    for (b, h) in [(0, 0), (B - 1, H - 1), (3, 7)]:
+        rq, rk, rv = BW.sdpa_backward(q[b, h], k[b, h], v[b, h], go[b, h], causal=True)
+        for name, got, ref in (("dq", dq[b, h], rq), ("dk", dk[b, h], rk), ("dv", dv[b, h], rv)):
+            e = float(np.abs(got - ref).max() / np.abs(ref).max())
+            say("   slice (%d, %d) %s: max-abs err / max|ref| %.3e" % (b, h, name, e))
+            assert e <= 2e-2
+        lse_row = BW.logsumexp(q[b, h], k[b, h], causal=True)[-1]
+        p_last = np.exp(x_last[b, h] - lse_row)
+        assert np.abs(dv[b, h, -1] - p_last * go[b, h, -1]).max() <= 2e-2 * max(1.0, float(np.abs(p_last * go[b, h, -1]).max()))
