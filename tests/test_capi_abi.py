@@ -110,3 +110,41 @@ def test_null_descriptor_and_missing_workspace():
         capi.sdpa_fwd(d)
     assert e.value.code == capi.EWORKSPACE
     assert lib.incin_rocm_device_count(None) == capi.EINVAL
+
+
+def _bwd(fwd_kw=None, **kw):
+    bd = capi.SdpaBwdDesc()
+    bd.fwd = _desc(**{**dict(lse=0x30000), **(fwd_kw or {})})
+    for name, heads in (("d_o", 4), ("d_q", 4), ("d_k", 4), ("d_v", 4)):
+        setattr(bd, name, 0x40000)
+        st = getattr(bd, name + "_stride")
+        st[0], st[1], st[2] = heads * 128 * 128, 128 * 128, 128
+    for k, v in kw.items():
+        setattr(bd, k, v)
+    return bd
+
+
+def test_backward_validation_and_workspace_size():
+    # two f32 per query row, whichever kernels take the request
+    assert capi.sdpa_bwd_workspace(_bwd()) == 2 * 2 * 4 * 128 * 4
+    assert capi.sdpa_bwd_workspace(_bwd(dict(dtype=capi.F32))) == 2 * 2 * 4 * 128 * 4
+    assert capi.sdpa_bwd_workspace(_bwd(dict(add_mask=0x20000))) == 2 * 2 * 4 * 128 * 4
+    assert capi.sdpa_bwd_workspace(_bwd(dict(Sq=0))) == 0            # nothing to compute
+    for bd, code in [
+        (_bwd(dict(lse=None)), capi.EINVAL),                          # the forward's normalisers are an input
+        (_bwd(d_k=None), capi.EINVAL),
+        (_bwd(dict(q_lens=0x50000)), capi.EUNSUPPORTED),
+        (_bwd(dict(impl=capi.IMPL_MFMA, dtype=capi.F32)), capi.EUNSUPPORTED),      # pinned to kernels that do not take it
+        (_bwd(dict(impl=capi.IMPL_MFMA, add_mask=0x20000)), capi.EUNSUPPORTED),
+        (_bwd(dict(impl=capi.IMPL_SPLITKV)), capi.EUNSUPPORTED),
+        (_bwd(dict(D=320, Dv=320)), capi.EUNSUPPORTED),
+        (_bwd(dict(Hq=6, Hkv=4)), capi.ESHAPE),
+    ]:
+        with pytest.raises(capi.RocmError) as e:
+            capi.sdpa_bwd_workspace(bd)
+        assert e.value.code == code, e.value.message
+    lib = capi.load()
+    assert lib.incin_rocm_sdpa_bwd(None, None) == capi.EINVAL
+    with pytest.raises(capi.RocmError) as e:          # no workspace: rejected before any device is touched
+        capi.sdpa_bwd(_bwd())
+    assert e.value.code == capi.EWORKSPACE
