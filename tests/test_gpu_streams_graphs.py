@@ -93,3 +93,55 @@ def test_graph_capture_and_replay(gpu, name, kw):
         # eager work of the program's own between replays
         assert np.array_equal(np.nan_to_num(c.plain(), nan=3.0), np.nan_to_num(expect, nan=3.0))
     graph.destroy()
+
+
+@pytest.mark.parametrize("dtype, impl", [(capi.BF16, capi.IMPL_AUTO), (capi.F32, capi.IMPL_AUTO)], ids=["bf16_matrix_core", "f32_generic"])
+def test_training_step_in_a_graph(gpu, dtype, impl):
+    """Forward (keeping the row normalisers) and backward recorded into one launch graph and replayed: every replay gives
+    the bytes the eager calls gave, with the program's own eager work between replays.  The backward launches three kernels
+    and neither allocates nor clears memory."""
+    B, Hq, Hkv, S, D = 2, 4, 2, 300, 128
+    r = np.random.Generator(np.random.PCG64(300))
+    mk = lambda *s: r.standard_normal(s, dtype=np.float32)
+    tq, tk, tv, tg = (host.DeviceTensor.from_f32(x, dtype) for x in (mk(B, Hq, S, D), mk(B, Hkv, S, D), mk(B, Hkv, S, D), mk(B, Hq, S, D)))
+    to, tdq = host.DeviceTensor((B, Hq, S, D), dtype), host.DeviceTensor((B, Hq, S, D), dtype)
+    tdk, tdv = host.DeviceTensor((B, Hkv, S, D), dtype), host.DeviceTensor((B, Hkv, S, D), dtype)
+    lse = capi.DeviceBuffer(B * Hq * S * 4)
+    bd = capi.SdpaBwdDesc()
+    bd.fwd = host.make_desc(tq, tk, tv, to, causal=True, impl=impl, lse=lse)
+    for name, t in (("d_o", tg), ("d_q", tdq), ("d_k", tdk), ("d_v", tdv)):
+        setattr(bd, name, t.ptr)
+        st = host._strides3(t.shape)
+        for i in range(3):
+            getattr(bd, name + "_stride")[i] = st[i]
+    ws = capi.DeviceBuffer(capi.sdpa_bwd_workspace(bd))
+    bd.workspace, bd.workspace_bytes = ws.ptr, ws.nbytes
+    outs = (to, tdq, tdk, tdv)
+
+    def eager():
+        capi.sdpa_fwd(bd.fwd)
+        capi.sdpa_bwd(bd)
+        capi.sync()
+        return [t.to_f32() for t in outs]
+
+    def clear():
+        for t in outs:
+            capi.check(capi.load().incin_rocm_memset(0, t.ptr, 0x7f, t.buf.nbytes))
+        capi.sync()
+
+    expect = eager()
+    say("graph capture: forward + backward, dtype %d" % dtype)
+    stream = capi.Stream()
+    with capi.Graph.record(stream) as graph:
+        capi.sdpa_fwd(bd.fwd, stream.ptr)
+        capi.sdpa_bwd(bd, stream.ptr)
+    for replay in range(3):
+        clear()
+        graph.launch()
+        stream.sync()
+        for name, t, e in zip(("out", "dq", "dk", "dv"), outs, expect):
+            assert np.array_equal(t.to_f32(), e), "%s, replay %d" % (name, replay)
+        for got, e in zip(eager(), expect):          # eager work of the program's own between replays
+            assert np.array_equal(got, e)
+    graph.destroy()
+    stream.destroy()
