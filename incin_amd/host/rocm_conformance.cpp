@@ -350,6 +350,33 @@ std::vector<Check> attention_training_checks(const Subject& s)
     };
 }
 
+// The runtime-dispatch arm (dispatch.rs:1196-1225): operands held by the rocm backend reach its operator and come back
+// wrapped; an operand or a mask held by no backend is an error with the reference's message, not a silent copy.
+std::string dispatch_routes(const Subject& s)
+{
+    const std::vector<float> q = {1, 2, 0.5f, -0.5f}, k = {1, -1, 2, 1}, v = {3, 5, 7, 11};
+    RocmStorage sq, sk, sv;
+    for (auto [st, vals] : {std::pair{&sq, &q}, std::pair{&sk, &k}, std::pair{&sv, &v}})
+        if (std::string e = s.storage({2, 2, 1}, *vals, st); !e.empty()) return e;
+    const DispatchStorage dq = DispatchStorage::on_rocm(sq), dk = DispatchStorage::on_rocm(sk), dv = DispatchStorage::on_rocm(sv), nowhere;
+    DispatchStorage out;
+    if (Error e = DispatchBackend::scaled_dot_product_attention(dq, dk, dv, nullptr, 1.0, &out)) return e.message;
+    if (out.holder != DispatchStorage::Holder::Rocm) return "the result of a rocm attention is not held by rocm";
+    std::vector<float> got;
+    if (std::string e = s.values(out.rocm, &got); !e.empty()) return e;
+    for (int h = 0; h < 2; ++h) {
+        double want[2];
+        closed_form(&q[2 * h], &k[2 * h], &v[2 * h], want);
+        for (int i = 0; i < 2; ++i)
+            if (!F32_ACCUMULATED.accepts(want[i], got[2 * h + i])) return "dispatched attention is outside 1e-5 of the closed form";
+    }
+    Error e = DispatchBackend::scaled_dot_product_attention(dq, nowhere, dv, nullptr, 1.0, &out);
+    if (!e || e.message != "mismatched backends in SDPA") return "an operand held by no backend gave: " + (e ? e.message : std::string("success"));
+    e = DispatchBackend::scaled_dot_product_attention(dq, dk, dv, &nowhere, 1.0, &out);
+    if (!e || e.message != "mismatched mask backend") return "a mask held by no backend gave: " + (e ? e.message : std::string("success"));
+    return "";
+}
+
 std::string registry_agrees(const Subject& s)
 {
     auto word = [](bool b, const char* yes, const char* no) { return std::string(b ? yes : no); };
@@ -418,6 +445,7 @@ Report run(int device)
     for (Check& c : reshape_checks(s)) r.checks.push_back(std::move(c));
     for (Check& c : attention_checks(s)) r.checks.push_back(std::move(c));
     for (Check& c : attention_training_checks(s)) r.checks.push_back(std::move(c));
+    r.checks.push_back(guarded("dispatch_routes_attention_to_the_holder_of_its_operands", [&] { return dispatch_routes(s); }));
     r.checks.push_back(guarded("the_registry_and_the_executor_agree", [&] { return registry_agrees(s); }));
     return r;
 }

@@ -149,4 +149,26 @@ DeviceId detect_device_in(const std::vector<int32_t>& pref)
     return DeviceId{0, 0};
 }
 
+DispatchStorage DispatchStorage::on_rocm(RocmStorage s)
+{
+    DispatchStorage d;
+    d.holder = Holder::Rocm;
+    d.rocm = std::move(s);
+    return d;
+}
+
+Error DispatchBackend::scaled_dot_product_attention(const DispatchStorage& q, const DispatchStorage& k, const DispatchStorage& v,
+                                                    const DispatchStorage* mask, std::optional<double> scale, DispatchStorage* out)
+{
+    using H = DispatchStorage::Holder;
+    if (q.holder == H::Rocm && k.holder == H::Rocm && v.holder == H::Rocm) {
+        if (mask && mask->holder != H::Rocm) return Error{ErrorKind::Msg, "mismatched mask backend"};
+        RocmStorage o;
+        if (Error e = RocmBackend::scaled_dot_product_attention(q.rocm, k.rocm, v.rocm, mask ? &mask->rocm : nullptr, scale, &o)) return e;
+        *out = DispatchStorage::on_rocm(std::move(o));
+        return Error{};
+    }
+    return Error{ErrorKind::Msg, "mismatched backends in SDPA"};
+}
+
 }  // namespace incin_rocm_host

@@ -49,4 +49,19 @@ std::optional<DeviceId> probe(int32_t kind);               // rocm: a device exi
 DeviceId detect_device_in(const std::vector<int32_t>& preference);     // first kind that probes; cpu ends the chain
 const std::vector<int32_t>& preference();                  // cuda, rocm, metal, wgpu, cpu
 
+// ---- runtime dispatch (crates/incin-backends/src/dispatch.rs:54-66, 1196-1225 with the rocm arm) ---------------
+// A storage that says which backend holds the data.  The reference's enum has one variant per compiled-in backend plus
+// `Unavailable`; this mirror compiles in the rocm arm only, so the others never occur here.
+struct DispatchStorage {
+    enum class Holder { Unavailable, Rocm } holder = Holder::Unavailable;
+    RocmStorage rocm;
+    static DispatchStorage on_rocm(RocmStorage s);
+};
+struct DispatchBackend {
+    // Routes to the backend that holds q, k and v; operands (or a mask) held elsewhere are an error, never a copy:
+    // "mismatched backends in SDPA" / "mismatched mask backend", the reference's messages.
+    static Error scaled_dot_product_attention(const DispatchStorage& q, const DispatchStorage& k, const DispatchStorage& v,
+                                              const DispatchStorage* mask, std::optional<double> scale, DispatchStorage* out);
+};
+
 }  // namespace incin_rocm_host

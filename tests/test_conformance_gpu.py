@@ -39,9 +39,9 @@ def test_conformance_report(gpu):
                  "attention_is_within_tolerance", "attention_output_matches_its_descriptor",
                  "attention_rejects_a_wrong_input_count", "attention_descriptor_facts_equal_an_explicit_mask",
                  "attention_gradients_are_within_tolerance", "attention_gradients_have_their_operands_shapes",
-                 "the_registry_and_the_executor_agree"):
+                 "dispatch_routes_attention_to_the_holder_of_its_operands", "the_registry_and_the_executor_agree"):
         assert "  pass  " + name in lines, name
-    assert rep.passed == 11
+    assert rep.passed == 12
 
 
 @pytest.mark.parametrize("dtype", [RB.F32, RB.BF16, RB.F16])
