@@ -132,8 +132,10 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     if (impl == INCIN_ROCM_IMPL_AUTO) {
         if (split_ok && R <= 8 && d->Skv >= 256 && !d->lse) impl = INCIN_ROCM_IMPL_SPLITKV;
         // long sequences with work for every compute unit twice over: the 64-row kernel's halved LDS traffic outweighs
-        // what it pays per 256-row work item (measured crossover: a few thousand keys)
-        else if (mfma64_ok && d->Skv >= 8192 && d->B * d->Hq * ((d->Sq + 255) / 256) >= 512) impl = INCIN_ROCM_IMPL_MFMA64;
+        // what it pays per 256-row work item (measured crossover: 4096 keys without a causal mask, where every item runs the
+        // full key range; 8192 with one)
+        else if (mfma64_ok && d->Skv >= (d->causal ? 8192 : 4096) && d->B * d->Hq * ((d->Sq + 255) / 256) >= 512)
+            impl = INCIN_ROCM_IMPL_MFMA64;
         else if (mfma_ok) impl = INCIN_ROCM_IMPL_MFMA;
         else if (split_ok && R <= 8 && !d->lse) impl = INCIN_ROCM_IMPL_SPLITKV;
         else impl = INCIN_ROCM_IMPL_GENERIC;

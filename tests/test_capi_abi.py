@@ -74,7 +74,10 @@ def test_dispatch_choices():
             st[0], st[1], st[2] = heads * S * d.D, S * d.D, d.D
         return d
     assert _plan(long())[2] == capi.IMPL_MFMA64
-    assert _plan(long(S=4096))[2] == capi.IMPL_MFMA
+    assert _plan(long(causal=1))[2] == capi.IMPL_MFMA64
+    assert _plan(long(S=4096))[2] == capi.IMPL_MFMA64          # without a causal mask the crossover is at 4096 keys
+    assert _plan(long(S=4096, causal=1))[2] == capi.IMPL_MFMA
+    assert _plan(long(S=2048))[2] == capi.IMPL_MFMA
     assert _plan(long(D=64, Dv=64))[2] == capi.IMPL_MFMA
     assert _plan(_desc(Sq=8192, Skv=8192))[2] == capi.IMPL_MFMA          # 2 x 4 heads x 32 blocks: too few items
     # empty problems need nothing
