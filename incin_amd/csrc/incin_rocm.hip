@@ -67,6 +67,8 @@ int use_device(int32_t dev)
 
 size_t dtype_size(int dtype) { return dtype == INCIN_ROCM_F32 ? 4 : 2; }
 
+constexpr size_t MFMA64_WS_BYTES = 256;     // work counters of one launch of the 64-row prefill kernel
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // What the dispatcher decided for one descriptor.
@@ -179,6 +181,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         plan->split_len = (int)split_len;
         plan->ws_bytes = splits > 1 ? (size_t)(d->B * d->Hq * d->Sq * splits) * (size_t)(d->Dv + 2) * sizeof(float) : 0;
     }
+    if (impl == INCIN_ROCM_IMPL_MFMA64) plan->ws_bytes = MFMA64_WS_BYTES;      // the launch's work counters
     return 0;
 }
 
@@ -203,7 +206,8 @@ void fill_params(const incin_rocm_sdpa_desc_t* d, const Plan& plan, SdpaParams* 
     p->deal_groups = 0;
     p->num_splits = plan.splits;
     p->split_len = plan.split_len;
-    p->ws_acc = (float*)d->workspace;
+    if (plan.impl == INCIN_ROCM_IMPL_MFMA64) p->sched = (int32_t*)d->workspace;
+    else p->ws_acc = (float*)d->workspace;
     if (plan.splits > 1) {
         const size_t rows = (size_t)(d->B * d->Hq * d->Sq * plan.splits);
         p->ws_ml = (float*)d->workspace + rows * (size_t)d->Dv;
@@ -445,16 +449,15 @@ int incin_rocm_sdpa_workspace(const incin_rocm_sdpa_desc_t* desc, size_t* bytes,
     return 0;
 }
 
-int incin_rocm_sdpa_fwd(const incin_rocm_sdpa_desc_t* desc, void* stream)
+// Launches a validated request; the scratch memory is what desc->workspace names.
+static int launch_fwd(const incin_rocm_sdpa_desc_t* desc, const Plan& plan, void* stream)
 {
-    Plan plan;
-    if (int rc = make_plan(desc, &plan)) return rc;
-    if (plan.empty) return 0;
     if (plan.ws_bytes > 0) {
         if (!desc->workspace || desc->workspace_bytes < plan.ws_bytes)
             return fail(INCIN_ROCM_EWORKSPACE,
-                        "scaled_dot_product_attention: split-KV needs %zu workspace bytes, %zu given",
-                        plan.ws_bytes, desc->workspace ? desc->workspace_bytes : (size_t)0);
+                        "scaled_dot_product_attention: %s needs %zu workspace bytes, %zu given",
+                        plan.impl == INCIN_ROCM_IMPL_MFMA64 ? "the 64-row MFMA kernel" : "split-KV", plan.ws_bytes,
+                        desc->workspace ? desc->workspace_bytes : (size_t)0);
         if (!aligned16(desc->workspace)) return fail(INCIN_ROCM_EWORKSPACE, "scaled_dot_product_attention: workspace must be 16-byte aligned");
     }
     if (int rc = use_device(desc->device)) return rc;
@@ -470,6 +473,14 @@ int incin_rocm_sdpa_fwd(const incin_rocm_sdpa_desc_t* desc, void* stream)
     }
     if (e != hipSuccess) return hip_fail(e, "attention kernel launch");
     return 0;
+}
+
+int incin_rocm_sdpa_fwd(const incin_rocm_sdpa_desc_t* desc, void* stream)
+{
+    Plan plan;
+    if (int rc = make_plan(desc, &plan)) return rc;
+    if (plan.empty) return 0;
+    return launch_fwd(desc, plan, stream);
 }
 
 
@@ -536,6 +547,7 @@ int incin_rocm_sdpa_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, void* stream)
                     need, bd->workspace ? bd->workspace_bytes : (size_t)0);
     if (int rc = use_device(bd->fwd.device)) return rc;
     Plan plan;
+    plan.impl = INCIN_ROCM_IMPL_GENERIC;
     plan.splits = 1;
     plan.split_len = (int)bd->fwd.Skv;
     incin_rocm::SdpaBwdParams bp;

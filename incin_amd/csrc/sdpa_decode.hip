@@ -15,6 +15,8 @@
 // ws_ml[b,hq,i,split] = (m, sum_j exp(s_j - m)); the combine kernel rescales
 // them to a common max.  With num_splits == 1 the first kernel writes the
 // final output itself.
+#include <atomic>
+
 #include "sdpa_params.h"
 
 namespace incin_rocm {
@@ -118,18 +120,22 @@ __global__ __launch_bounds__(256) void sdpa_decode_split_kernel(SdpaParams p)
     const T* kp = (const T*)p.k + (int64_t)b * p.k_sb + (int64_t)hkv * p.k_sh + dl;
     const T* vp = (const T*)p.v + (int64_t)b * p.v_sb + (int64_t)hkv * p.v_sh + dl;
 
+    // Rows at and beyond k_end (the end of the split, at most the batch entry's key count) are never read: a lane whose
+    // key lies there re-reads the split's last row, and its score is masked below.  What an unwritten cache tail holds
+    // (NaN bit patterns included) therefore cannot reach the result through 0 * v.
+    const int k_last = k_end - 1;
     for (int t0 = k_begin + wave * KT; t0 < k_end; t0 += 4 * KT) {
         vec_t kreg[U], vreg[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             int key = t0 + u * KPL + sub;
-            if (key > Skv - 1) key = Skv - 1;                 // stay inside the buffer; such keys are masked below
+            if (key > k_last) key = k_last;
             kreg[u] = __builtin_nontemporal_load((const vec_t*)(kp + (int64_t)key * p.k_ss));
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             int key = t0 + u * KPL + sub;
-            if (key > Skv - 1) key = Skv - 1;
+            if (key > k_last) key = k_last;
             vreg[u] = __builtin_nontemporal_load((const vec_t*)(vp + (int64_t)key * p.v_ss));
         }
 
@@ -253,8 +259,17 @@ static hipError_t launch_decode_t(const SdpaParams& p, hipStream_t stream)
     constexpr int NSTREAM = 4 * (64 / (D / VEC));
     size_t lds = (size_t)(NSTREAM * RMAX * D + NSTREAM * RMAX * 2) * sizeof(float);
     auto kern = sdpa_decode_split_kernel<T, D, RMAX, U>;
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
+    hipError_t e;
+    // the dynamic-LDS limit of this instance is raised once per device, not per launch
+    static std::atomic<uint64_t> prepared{0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+    const uint64_t bit = 1ull << (dev & 63);
+    if (!(prepared.load(std::memory_order_acquire) & bit)) {
+        e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        prepared.fetch_or(bit, std::memory_order_release);
+    }
     const int R = p.G * p.Sq;
     const int nchunks = (R + RMAX - 1) / RMAX;
     dim3 grid(p.num_splits, p.Hkv * nchunks, p.B);

@@ -13,6 +13,8 @@
 // output columns tx + 16*c of the accumulator.  Q, the current K (then V) tile
 // and the probability tile live in LDS as f32 with one float of row padding,
 // which makes every LDS access of the two inner loops conflict-free.
+#include <atomic>
+
 #include "sdpa_params.h"
 
 namespace incin_rocm {
@@ -71,7 +73,7 @@ __global__ __launch_bounds__(256) void sdpa_generic_kernel(SdpaParams p)
         for (int idx = tid; idx < GEN_BN * D; idx += 256) {
             int r = idx / D, d = idx - r * D;
             int j = j0 + r;
-            KVs[r * DP + d] = j < Skv ? to_f32(kp[(int64_t)j * p.k_ss + d]) : 0.0f;
+            KVs[r * DP + d] = j < kv_len ? to_f32(kp[(int64_t)j * p.k_ss + d]) : 0.0f;     // rows past the key count are never read
         }
         __syncthreads();
 
@@ -129,7 +131,7 @@ __global__ __launch_bounds__(256) void sdpa_generic_kernel(SdpaParams p)
         for (int idx = tid; idx < GEN_BN * Dv; idx += 256) {
             int r = idx / Dv, d = idx - r * Dv;
             int j = j0 + r;
-            KVs[r * DP + d] = j < Skv ? to_f32(vp[(int64_t)j * p.v_ss + d]) : 0.0f;
+            KVs[r * DP + d] = j < kv_len ? to_f32(vp[(int64_t)j * p.v_ss + d]) : 0.0f;
         }
         __syncthreads();
         for (int jj = 0; jj < GEN_BN; ++jj) {
@@ -171,8 +173,17 @@ static hipError_t launch_generic_t(const SdpaParams& p, hipStream_t stream)
 {
     size_t lds = (size_t)(GEN_BM * (DMAX + 1) + GEN_BN * (DMAX + 1) + GEN_BM * (GEN_BN + 1)) * sizeof(float);
     auto kern = sdpa_generic_kernel<T, DMAX>;
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
+    hipError_t e;
+    // the dynamic-LDS limit of this instance is raised once per device, not per launch
+    static std::atomic<uint64_t> prepared{0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+    const uint64_t bit = 1ull << (dev & 63);
+    if (!(prepared.load(std::memory_order_acquire) & bit)) {
+        e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        prepared.fetch_or(bit, std::memory_order_release);
+    }
     dim3 grid((p.Sq + GEN_BM - 1) / GEN_BM, p.Hq, p.B);
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, p);
     return hipGetLastError();

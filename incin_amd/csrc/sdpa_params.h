@@ -31,6 +31,9 @@ struct SdpaParams {
     int32_t split_len;         // keys per split (multiple of the kernel's key tile)
     float* ws_acc;             // [B, Hq, Sq, num_splits, Dv] f32 partial numerators
     float* ws_ml;              // [B, Hq, Sq, num_splits, 2]  running max (natural-log domain) and denominator
+    // 64-row MFMA prefill kernel only
+    int32_t* sched;            // 16 work counters of this launch's persistent workgroups (in the caller's workspace; the
+                               // launcher clears them with a one-workgroup kernel ahead of the attention kernel)
 };
 
 typedef __bf16 bf16_t;

@@ -132,7 +132,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     const int64_t k_tile_bytes = (int64_t)PF_BN * p.k_ss * 2, v_tile_bytes = (int64_t)PF_BN * p.v_ss * 2;
     // K buffer b at smem + b*TILE, V buffer b at smem + (2+b)*TILE
     auto issue_k = [&](int t, int buf) __attribute__((always_inline)) {
-        int64_t rem = (int64_t)(Skv - t * PF_BN - 1) * p.k_ss * 2 + D * 2;   // bytes to the end of the last valid row: loads past that return 0
+        int64_t rem = (int64_t)(j_end - t * PF_BN - 1) * p.k_ss * 2 + D * 2;   // bytes to the end of the last row this workgroup may see: loads past that return 0
         if (rem > 0x7fffffffLL) rem = 0x7fffffffLL;
         const uint4v r = dma_descriptor((const char*)kp + t * k_tile_bytes, (int)rem);
         const unsigned dst = lds_address(smem) + buf * L::TILE_BYTES + wave * LPW * 1024;
@@ -140,7 +140,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
         for (int c = 0; c < LPW; ++c) dma_copy16(r, dst + c * 1024, k_voff[c]);
     };
     auto issue_v = [&](int t, int buf) __attribute__((always_inline)) {
-        int64_t rem = (int64_t)(Skv - t * PF_BN - 1) * p.v_ss * 2 + D * 2;
+        int64_t rem = (int64_t)(j_end - t * PF_BN - 1) * p.v_ss * 2 + D * 2;     // (rows past a batch entry's key count are never read)
         if (rem > 0x7fffffffLL) rem = 0x7fffffffLL;
         const uint4v r = dma_descriptor((const char*)vp + t * v_tile_bytes, (int)rem);
         const unsigned dst = lds_address(smem) + (2 + buf) * L::TILE_BYTES + wave * LPW * 1024;

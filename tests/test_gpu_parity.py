@@ -300,3 +300,33 @@ def test_decode_lengths_and_prefill_consistency(gpu):
     full = host.sdpa(qf, kf, vf, capi.BF16, causal=True, impl=capi.IMPL_MFMA)
     last = host.sdpa(qf[:, :, -1:], kf, vf, capi.BF16, causal=True)
     check(last, full[:, :, -1:], 8e-3, "decode == last row of causal prefill")
+
+
+@pytest.mark.parametrize("impl, dtype, sq", [(capi.IMPL_GENERIC, capi.F32, 70), (capi.IMPL_GENERIC, capi.BF16, 70),
+                                             (capi.IMPL_MFMA, capi.BF16, 200), (capi.IMPL_MFMA64, capi.BF16, 200),
+                                             (capi.IMPL_MFMA, capi.F16, 200), (capi.IMPL_SPLITKV, capi.BF16, 1),
+                                             (capi.IMPL_SPLITKV, capi.F32, 2)],
+                         ids=["generic_f32", "generic_bf16", "mfma_bf16", "mfma64_bf16", "mfma_f16", "splitkv_bf16", "splitkv_f32"])
+def test_rows_beyond_the_key_count_are_never_read(gpu, impl, dtype, sq):
+    """A preallocated cache holds whatever the allocator left behind its valid rows.  With NaN and infinity bit patterns
+    in every key and value row at and beyond kv_lens[b], each kernel gives the bytes it gives over a zeroed tail, and
+    those agree with the oracle on the truncated operands."""
+    B, Hq, Hkv, Skv, D = 3, 4, 2, 333, 128
+    lens = np.array([333, 97, 1], np.int32)
+    q, k, v = inputs(SEED0 + 71, B, Hq, Hkv, sq, Skv, D, D, dtype)
+    k_bad, v_bad = k.copy(), v.copy()
+    junk = np.array([np.nan, np.inf, -np.inf, np.nan], np.float32)
+    for b in range(B):
+        n = Skv - lens[b]
+        if n:
+            k[b, :, lens[b]:], v[b, :, lens[b]:] = 0.0, 0.0
+            fill = np.resize(junk, n * D).reshape(n, D)
+            k_bad[b, :, lens[b]:], v_bad[b, :, lens[b]:] = fill, fill[::-1]
+    say("junk beyond kv_lens: impl %d dtype %d" % (impl, dtype))
+    kw = dict(causal=False, kv_lens=lens, impl=impl, num_splits=3 if impl == capi.IMPL_SPLITKV else 0)
+    clean, info = host.sdpa(q, k, v, dtype, return_info=True, **kw)
+    assert info["impl"] == impl
+    dirty = host.sdpa(q, k_bad, v_bad, dtype, **kw)
+    assert np.isfinite(dirty).all()
+    assert np.array_equal(dirty, clean)
+    check(dirty, oracle_full(q, k, v, G=Hq // Hkv, kv_lens=lens), TOL[dtype], "junk tail")

@@ -145,3 +145,52 @@ def test_training_step_in_a_graph(gpu, dtype, impl):
             assert np.array_equal(got, e)
     graph.destroy()
     stream.destroy()
+
+
+def test_overlapping_launches_of_the_64_row_kernel(gpu):
+    """Two host threads launch the same problem through the 64-row prefill kernel 50 times each on streams of their own
+    while a recorded graph of the same launch replays on a third stream.  The kernel's persistent workgroups draw their
+    work from counters in the launch's workspace; each party has a workspace and an output of its own, so whatever
+    overlaps, every output equals the plain launch bit for bit."""
+    kw = dict(B=2, Hq=8, Hkv=2, Sq=1024, Skv=1024, D=128, causal=True, impl=capi.IMPL_MFMA64)
+    parties = [Case(400, **kw) for _ in range(3)]          # same seed: same problem, separate buffers
+    assert all(c.impl == capi.IMPL_MFMA64 and c.ws is not None for c in parties)
+    expect = parties[0].plain()
+    for c in parties:
+        c.clear()
+    gstream = capi.Stream()
+    with capi.Graph.record(gstream) as graph:
+        capi.sdpa_fwd(parties[2].desc, gstream.ptr)
+    errors = []
+
+    def eager(c):
+        try:
+            s = capi.Stream()
+            for _ in range(50):
+                capi.sdpa_fwd(c.desc, s.ptr)
+            s.sync()
+            s.destroy()
+        except Exception as e:      # noqa: BLE001 - reported below
+            errors.append(e)
+
+    def replay():
+        try:
+            for _ in range(50):
+                graph.launch()
+            gstream.sync()
+        except Exception as e:      # noqa: BLE001
+            errors.append(e)
+
+    say("2 threads x 50 eager launches + 50 graph replays of the 64-row kernel, three streams")
+    threads = [threading.Thread(target=eager, args=(parties[0],)), threading.Thread(target=eager, args=(parties[1],)),
+               threading.Thread(target=replay)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    capi.sync()
+    for i, c in enumerate(parties):
+        assert np.array_equal(c.to.to_f32(), expect), "party %d" % i
+    graph.destroy()
+    gstream.destroy()
