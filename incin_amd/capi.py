@@ -28,7 +28,7 @@ EXPORTS = [
     "incin_rocm_event_create", "incin_rocm_event_destroy", "incin_rocm_event_record",
     "incin_rocm_event_sync", "incin_rocm_event_elapsed_ms",
     "incin_rocm_graph_begin", "incin_rocm_graph_end", "incin_rocm_graph_launch", "incin_rocm_graph_destroy",
-    "incin_rocm_sdpa_workspace", "incin_rocm_sdpa_fwd",
+    "incin_rocm_sdpa_workspace", "incin_rocm_sdpa_fwd", "incin_rocm_sdpa_fwd_static",
     "incin_rocm_sizeof_kv_append_desc", "incin_rocm_kv_append",
     "incin_rocm_sizeof_sdpa_bwd_desc", "incin_rocm_sdpa_bwd_workspace", "incin_rocm_sdpa_bwd",
 ]
@@ -148,6 +148,7 @@ def load():
     lib.incin_rocm_sdpa_workspace.argtypes = [C.POINTER(SdpaDesc), C.POINTER(C.c_size_t), C.POINTER(C.c_int32),
                                               C.POINTER(C.c_int32)]
     lib.incin_rocm_sdpa_fwd.argtypes = [C.POINTER(SdpaDesc), C.c_void_p]
+    lib.incin_rocm_sdpa_fwd_static.argtypes = [C.POINTER(SdpaDesc), C.c_void_p]
     lib.incin_rocm_sizeof_kv_append_desc.restype = C.c_size_t
     lib.incin_rocm_sizeof_sdpa_bwd_desc.restype = C.c_size_t
     lib.incin_rocm_sdpa_bwd_workspace.argtypes = [C.POINTER(SdpaBwdDesc), C.POINTER(C.c_size_t)]
@@ -237,6 +238,14 @@ def kv_append(desc, stream=None):
 
 def sdpa_fwd(desc, stream=None):
     check(load().incin_rocm_sdpa_fwd(C.byref(desc), stream))
+
+
+STATIC_SCRATCH_BYTES = 8 << 20      # INCIN_ROCM_STATIC_SCRATCH_BYTES
+
+
+def sdpa_fwd_static(desc, stream=None):
+    """incin_rocm_sdpa_fwd_static: the launch that takes its scratch memory from the library's static buffer."""
+    check(load().incin_rocm_sdpa_fwd_static(C.byref(desc), stream))
 
 
 class Event:

@@ -8,6 +8,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "../../include/incin_rocm.h"
 #include "kv_append.h"
@@ -481,6 +482,53 @@ int incin_rocm_sdpa_fwd(const incin_rocm_sdpa_desc_t* desc, void* stream)
     if (int rc = make_plan(desc, &plan)) return rc;
     if (plan.empty) return 0;
     return launch_fwd(desc, plan, stream);
+}
+
+// ---- the entry point that allocates nothing ------------------------------------------------------------------
+// Scratch memory of incin_rocm_sdpa_fwd_static: part of the code object, so every device the library runs on holds
+// its own copy from the moment the code object is loaded there until the process ends.  In host code the array's
+// name is only a handle for hipGetSymbolAddress, never a device address: static_scratch_of() asks once per device,
+// with that device current, and everything on the host side uses the pointer it returns.
+static __device__ __align__(256) unsigned char g_static_scratch[INCIN_ROCM_STATIC_SCRATCH_BYTES];
+
+static int static_scratch_of(int32_t dev, void** out)
+{
+    static std::mutex mu;
+    static void* ptrs[64];
+    if (dev < 0 || dev >= 64) return fail(INCIN_ROCM_EDEVICE, "sdpa_fwd_static: device ordinal %d is outside the table of 64", dev);
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptrs[dev]) {
+        void* ptr = nullptr;                               // (the caller has made `dev` the current device)
+        hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_static_scratch));
+        if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(static scratch)");
+        if (!ptr) return fail(INCIN_ROCM_ERUNTIME, "ROCm hipGetSymbolAddress(static scratch) returned no address on device %d", dev);
+        ptrs[dev] = ptr;
+    }
+    *out = ptrs[dev];
+    return 0;
+}
+
+int incin_rocm_sdpa_fwd_static(const incin_rocm_sdpa_desc_t* desc, void* stream)
+{
+    Plan plan;
+    if (int rc = make_plan(desc, &plan)) return rc;
+    if (plan.empty) return 0;
+    if (plan.ws_bytes > (size_t)INCIN_ROCM_STATIC_SCRATCH_BYTES)
+        return fail(INCIN_ROCM_EWORKSPACE,
+                    "sdpa_fwd_static: this request needs %zu bytes of scratch memory, the static buffer holds %zu "
+                    "(fewer splits, or incin_rocm_sdpa_fwd with a workspace of the caller's)",
+                    plan.ws_bytes, (size_t)INCIN_ROCM_STATIC_SCRATCH_BYTES);
+    incin_rocm_sdpa_desc_t d = *desc;
+    d.workspace = nullptr;
+    d.workspace_bytes = 0;
+    if (plan.ws_bytes > 0) {
+        if (int rc = use_device(desc->device)) return rc;
+        void* scratch = nullptr;
+        if (int rc = static_scratch_of(desc->device, &scratch)) return rc;
+        d.workspace = scratch;
+        d.workspace_bytes = (size_t)INCIN_ROCM_STATIC_SCRATCH_BYTES;
+    }
+    return launch_fwd(&d, plan, stream);
 }
 
 

@@ -196,6 +196,16 @@ int incin_rocm_sdpa_workspace(const incin_rocm_sdpa_desc_t* desc, size_t* bytes,
  * it was recorded with on every replay. */
 int incin_rocm_sdpa_fwd(const incin_rocm_sdpa_desc_t* desc, void* stream);
 
+/* The same launch for callers that cannot allocate device memory (code under graph capture, serving loops and
+ * harnesses that forbid it).  No counterpart in the reference.  `workspace` and `workspace_bytes` of the
+ * descriptor are ignored: the scratch memory is a buffer of INCIN_ROCM_STATIC_SCRATCH_BYTES that is part of the
+ * library's code object (one copy per device, held until the process ends), and the call makes no device or
+ * host allocation.  A request whose scratch need (incin_rocm_sdpa_workspace) exceeds the buffer is refused with
+ * INCIN_ROCM_EWORKSPACE.  Every call on a device shares that device's buffer: calls that may overlap in time on
+ * one device race, so keep them on one stream or order them with events. */
+#define INCIN_ROCM_STATIC_SCRATCH_BYTES (8u << 20)
+int incin_rocm_sdpa_fwd_static(const incin_rocm_sdpa_desc_t* desc, void* stream);
+
 /* ---- attention backward --------------------------------------------------------
  * The reference has no backward kernel for attention: its gradient is what walking the tape of the composed ops
  * gives (crates/incin-backends/src/cpu/ops/shape_ops.rs:1245-1269 records matmul, mul_scalar, add, log_softmax,
