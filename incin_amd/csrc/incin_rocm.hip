@@ -11,6 +11,7 @@
 #include <mutex>
 
 #include "../../include/incin_rocm.h"
+#include "copy.h"
 #include "kv_append.h"
 #include "sdpa_bwd.h"
 #include "sdpa_params.h"
@@ -21,7 +22,6 @@ hipError_t launch_sdpa_prefill_mfma(const SdpaParams& p, int dtype, hipStream_t 
 hipError_t launch_sdpa_prefill_mfma64(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_sdpa_decode(const SdpaParams& p, int dtype, hipStream_t stream);
 int decode_keys_per_tile(int dtype, int D, int R);
-hipError_t launch_copy16(void* dst, const void* src, size_t bytes, hipStream_t stream);
 }  // namespace incin_rocm
 
 using incin_rocm::SdpaParams;
@@ -324,6 +324,34 @@ int incin_rocm_memcpy_d2d(int32_t dev, void* dst, const void* src, size_t bytes)
     return copy(dev, dst, src, bytes, hipMemcpyDeviceToDevice, "hipMemcpy(device to device)");
 }
 
+int incin_rocm_copy_strided(int32_t dev, void* dst, const void* src, int32_t rank, const int64_t* shape, const int64_t* strides,
+                            int32_t elem_bytes, void* stream)
+{
+    if (rank < 0 || rank > 8) return fail(INCIN_ROCM_ESHAPE, "copy_strided: rank %d is outside 0..8", rank);
+    if (elem_bytes != 2 && elem_bytes != 4) return fail(INCIN_ROCM_EDTYPE, "copy_strided: elements of %d bytes (2 or 4 only)", elem_bytes);
+    if (rank > 0 && (!shape || !strides)) return fail(INCIN_ROCM_EINVAL, "copy_strided: null shape or strides");
+    incin_rocm::StridedCopyParams p;
+    int64_t n = 1;
+    for (int a = 0; a < 8; ++a) { p.shape[a] = 1; p.stride[a] = 0; }
+    for (int a = 0; a < rank; ++a) {
+        if (shape[a] < 0) return fail(INCIN_ROCM_ESHAPE, "copy_strided: negative extent");
+        if (shape[a] > 0x7fffffffLL || (n *= shape[a]) > (1LL << 40)) return fail(INCIN_ROCM_ESHAPE, "copy_strided: view too large");
+        p.shape[8 - rank + a] = shape[a];
+        p.stride[8 - rank + a] = strides[a];
+    }
+    if (n == 0) return 0;
+    if (!dst || !src) return fail(INCIN_ROCM_EINVAL, "copy_strided: null pointer");
+    if (((uintptr_t)dst | (uintptr_t)src) % (uintptr_t)elem_bytes) return fail(INCIN_ROCM_EINVAL, "copy_strided: misaligned pointer");
+    p.src = (const char*)src;
+    p.dst = (char*)dst;
+    p.elem = elem_bytes;
+    p.outer = 1;
+    for (int a = 0; a < 6; ++a) p.outer *= p.shape[a];
+    if (int rc = use_device(dev)) return rc;
+    HIP_TRY(incin_rocm::launch_copy_strided(p, (hipStream_t)stream), "strided copy launch");
+    return 0;
+}
+
 int incin_rocm_sync(int32_t dev)
 {
     if (int rc = use_device(dev)) return rc;
@@ -588,7 +616,19 @@ int incin_rocm_sdpa_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, void* stream)
 {
     bool empty = false, mfma = false;
     if (int rc = check_bwd(bd, &empty, &mfma)) return rc;
-    if (empty) return 0;        // (gradients of an empty problem: nothing to write)
+    if (empty) {
+        // No element to write - except with queries but no keys: the output is zeros whatever q holds, so d_q is zero
+        // (the reference's tape gives zeros there), and it is promised to be fully overwritten.
+        const incin_rocm_sdpa_desc_t* d = &bd->fwd;
+        if (d->Skv == 0 && d->B > 0 && d->Hq > 0 && d->Sq > 0 && d->D > 0) {
+            if (!bd->d_q) return fail(INCIN_ROCM_EINVAL, "scaled_dot_product_attention backward: null gradient pointer");
+            if (int rc = use_device(d->device)) return rc;
+            HIP_TRY(incin_rocm::launch_zero_rows(bd->d_q, (int)dtype_size(d->dtype), (int)d->B, (int)d->Hq, (int)d->Sq, (int)d->D,
+                                                 bd->d_q_stride[0], bd->d_q_stride[1], bd->d_q_stride[2], (hipStream_t)stream),
+                    "gradient clear launch");
+        }
+        return 0;
+    }
     const size_t need = 2 * (size_t)(bd->fwd.B * bd->fwd.Hq * bd->fwd.Sq) * sizeof(float);      // two f32 per query row
     if (!bd->workspace || bd->workspace_bytes < need || !aligned16(bd->workspace))
         return fail(INCIN_ROCM_EWORKSPACE, "scaled_dot_product_attention backward: %zu workspace bytes needed (16-byte aligned), %zu given",

@@ -150,6 +150,10 @@ def sdpa_backward(q, k, v, d_out, dtype=capi.BF16, scale=None, causal=False, kv_
     tlse = capi.DeviceBuffer(max(B * Hq * Sq, 1) * 4, dev)
     bd = capi.SdpaBwdDesc()
     bd.fwd = make_desc(tq, tk, tv, to, scale, causal, tl, tm, ms, impl=impl, lse=tlse)
+    fbytes = capi.sdpa_workspace(bd.fwd)[0]
+    fws = capi.DeviceBuffer(fbytes, dev) if fbytes else None
+    if fws is not None:
+        bd.fwd.workspace, bd.fwd.workspace_bytes = fws.ptr, fws.nbytes
     capi.sdpa_fwd(bd.fwd)
     for name, t in (("d_o", tg), ("d_q", tdq), ("d_k", tdk), ("d_v", tdv)):
         setattr(bd, name, t.ptr)
@@ -163,7 +167,7 @@ def sdpa_backward(q, k, v, d_out, dtype=capi.BF16, scale=None, causal=False, kv_
     capi.sdpa_bwd(bd)
     capi.sync(dev)
     res = tuple(t.to_f32() for t in (to, tdq, tdk, tdv))
-    for t in (tq.buf, tk.buf, tv.buf, tg.buf, to.buf, tdq.buf, tdk.buf, tdv.buf, tl, tm, tlse, ws):
+    for t in (tq.buf, tk.buf, tv.buf, tg.buf, to.buf, tdq.buf, tdk.buf, tdv.buf, tl, tm, tlse, ws, fws):
         if t is not None:
             t.free()
     return res

@@ -148,7 +148,12 @@ Error RocmBackend::to_bytes(const RocmStorage& s, std::vector<uint8_t>* out)
     if (n == 0) return ok();
     if (s.is_contiguous())
         return from_status(incin_rocm_memcpy_d2h(s.device, out->data(), s.data(), (size_t)n * isz), s.device);
-    // strided or broadcast view: fetch the whole allocation once, gather on the host
+    if (s.shape.size() <= 8) {          // strided or broadcast view: gather on the device, then one copy
+        RocmStorage dense;
+        if (Error e = contiguous(s, &dense)) return e;
+        return from_status(incin_rocm_memcpy_d2h(s.device, out->data(), dense.data(), (size_t)n * isz), s.device);
+    }
+    // beyond the copy kernel's rank: fetch the whole allocation once, gather on the host
     std::vector<uint8_t> raw(s.buffer->bytes());
     if (Error e = from_status(incin_rocm_memcpy_d2h(s.device, raw.data(), s.buffer->ptr(), raw.size()), s.device)) return e;
     std::vector<int64_t> idx(s.shape.size(), 0);
@@ -161,6 +166,46 @@ Error RocmBackend::to_bytes(const RocmStorage& s, std::vector<uint8_t>* out)
             idx[a] = 0;
         }
     }
+    return ok();
+}
+
+// CpuStorage::contiguous (cpu/storage.rs:407-440): a fresh dense copy of a view, here gathered by one kernel.
+Error RocmBackend::contiguous(const RocmStorage& s, RocmStorage* out)
+{
+    if (s.is_contiguous()) {
+        *out = s;
+        return ok();
+    }
+    if (s.shape.size() > 8) return err(ErrorKind::UnsupportedBackendOperation, "contiguous: rank above 8 on backend Rocm");
+    RocmStorage dense;
+    if (Error e = alloc_storage(s.shape, s.dtype, s.device, &dense)) return e;
+    if (dense.numel() > 0) {
+        if (Error e = from_status(incin_rocm_copy_strided(s.device, dense.buffer->ptr(), s.data(), (int32_t)s.shape.size(), s.shape.data(),
+                                                          s.strides.data(), (int32_t)dtype_size(s.dtype), nullptr), s.device))
+            return e;
+        if (Error e = from_status(incin_rocm_sync(s.device), s.device)) return e;
+    }
+    *out = std::move(dense);
+    return ok();
+}
+
+// An operand of attention whose last axis is strided (a transposed view, cpu/storage.rs:308-325), made dense along its
+// last axes.  Axes the view only repeats (stride 0) are not expanded: they are copied at extent 1 and stay broadcast.
+static Error dense_last_axis(const RocmStorage& s, RocmStorage* out)
+{
+    RocmStorage squeezed = s;
+    for (size_t a = 0; a < s.shape.size(); ++a)
+        if (s.strides[a] == 0) squeezed.shape[a] = std::min<int64_t>(s.shape[a], 1);
+    RocmStorage dense;
+    if (Error e = RocmBackend::contiguous(squeezed, &dense)) return e;
+    if (dense.buffer == s.buffer) {        // (already dense once the repeated axes are set aside: nothing to fix)
+        *out = s;
+        return ok();
+    }
+    for (size_t a = 0; a < s.shape.size(); ++a)
+        if (s.strides[a] == 0) { dense.shape[a] = s.shape[a]; dense.strides[a] = 0; }
+    dense.mask_tag.reset();
+    *out = std::move(dense);
     return ok();
 }
 
@@ -209,9 +254,9 @@ Error RocmBackend::reshape(const RocmStorage& s, const std::vector<int64_t>& dim
     if (n != s.numel())
         return err(ErrorKind::ShapeMismatch, "reshape: " + shape_str(s.shape) + " has " + std::to_string(s.numel()) +
                                                  " elements, " + shape_str(dims) + " has " + std::to_string(n));
-    if (!s.is_contiguous())
-        return err(ErrorKind::UnsupportedBackendOperation, "reshape: only contiguous storage can be re-addressed on backend Rocm");
-    *out = s;
+    RocmStorage dense;                  // a view that is not dense is materialised first, as the reference's reshape does
+    if (Error e = contiguous(s, &dense)) return e;
+    *out = dense;
     out->shape = dims;
     out->strides.assign(dims.size(), 1);
     for (int i = (int)dims.size() - 2; i >= 0; --i) out->strides[i] = out->strides[i + 1] * dims[i + 1];
@@ -291,9 +336,24 @@ Error RocmBackend::attention_impl(const RocmStorage& q, const RocmStorage& k, co
         return err(ErrorKind::ShapeMismatch, std::string(OP) + ": q and k inner dims must match: q " + shape_str(q.shape) + ", k " + shape_str(k.shape));
     if (v.shape[vr - 2] != Skv)
         return err(ErrorKind::ShapeMismatch, std::string(OP) + ": k and v key counts must match: k " + shape_str(k.shape) + ", v " + shape_str(v.shape));
-    if (q.strides[qr - 1] != 1 && D > 1) return err(ErrorKind::UnsupportedBackendOperation, std::string(OP) + ": q needs a contiguous last axis on backend Rocm");
-    if (k.strides[kr - 1] != 1 && D > 1) return err(ErrorKind::UnsupportedBackendOperation, std::string(OP) + ": k needs a contiguous last axis on backend Rocm");
-    if (v.strides[vr - 1] != 1 && Dv > 1) return err(ErrorKind::UnsupportedBackendOperation, std::string(OP) + ": v needs a contiguous last axis on backend Rocm");
+    // The kernels read rows of unit stride.  The reference takes any view (cpu/storage.rs:308-325; k = transpose of
+    // [.., D, Skv] storage is pinned at cpu/ops/matmul.rs:677-724): such an operand is gathered into a dense temporary
+    // first, as CpuStorage::contiguous would, and the operator runs on that.
+    {
+        const bool fq = q.strides[qr - 1] != 1 && D > 1, fk = k.strides[kr - 1] != 1 && D > 1, fv = v.strides[vr - 1] != 1 && Dv > 1;
+        if (fq || fk || fv) {
+            if (qr > 8 || kr > 8 || vr > 8)
+                return err(ErrorKind::UnsupportedBackendOperation, std::string(OP) + ": a strided last axis needs rank <= 8 on backend Rocm");
+            RocmStorage qd = q, kd = k, vd = v;
+            if (fq) if (Error e = dense_last_axis(q, &qd)) return e;
+            if (fk) if (Error e = dense_last_axis(k, &kd)) return e;
+            if (fv) if (Error e = dense_last_axis(v, &vd)) return e;
+            Error e = attention_impl(qd, kd, vd, mask, scale, facts, grad_out, out, grads);
+            // the temporaries are used stream-ordered: finish before they are released
+            if (Error e2 = from_status(incin_rocm_sync(q.device), q.device)) return e ? e : e2;
+            return e;
+        }
+    }
 
     // -- batch axes: broadcast(broadcast(q, k), v), NumPy rule (cpu/ops/matmul.rs:198-221) ------------------
     const std::vector<int64_t> qb(q.shape.begin(), q.shape.end() - 2), kb(k.shape.begin(), k.shape.end() - 2),
@@ -422,7 +482,7 @@ Error RocmBackend::attention_impl(const RocmStorage& q, const RocmStorage& k, co
     if (mask && mask->mask_tag) {
         if (mask->mask_tag->kind == MaskTag::Causal) d.causal = 1;
         else {
-            if (mask->mask_tag->lens_count != B || n_outer != 0 || (g_ax >= 0 && !fold_g))
+            if (mask->mask_tag->lens_count != B || n_outer != 0 || (g_ax >= 0 && !fold_g && h_ax >= 0))
                 return err(ErrorKind::ShapeMismatch, std::string(OP) + ": key-padding lengths must have one entry per batch index");
             d.kv_lens = static_cast<const int32_t*>(mask->mask_tag->lens->ptr());
         }
@@ -434,12 +494,12 @@ Error RocmBackend::attention_impl(const RocmStorage& q, const RocmStorage& k, co
     if (facts.causal) d.causal = 1;
     if (facts.kv_lens) {
         if (d.kv_lens) return err(ErrorKind::ShapeMismatch, std::string(OP) + ": key lengths given twice (descriptor and mask tag)");
-        if (facts.kv_lens_count != B || n_outer != 0 || (g_ax >= 0 && !fold_g))
+        if (facts.kv_lens_count != B || n_outer != 0 || (g_ax >= 0 && !fold_g && h_ax >= 0))
             return err(ErrorKind::ShapeMismatch, std::string(OP) + ": key-padding lengths must have one entry per batch index");
         d.kv_lens = static_cast<const int32_t*>(facts.kv_lens->ptr());
     }
     if (facts.q_lens) {
-        if (facts.q_lens_count != B || n_outer != 0 || (g_ax >= 0 && !fold_g))
+        if (facts.q_lens_count != B || n_outer != 0 || (g_ax >= 0 && !fold_g && h_ax >= 0))
             return err(ErrorKind::ShapeMismatch, std::string(OP) + ": query lengths must have one entry per batch index");
         d.q_lens = static_cast<const int32_t*>(facts.q_lens->ptr());
     }

@@ -84,6 +84,10 @@ struct RocmBackend {
     static Error to_bytes(const RocmStorage& s, std::vector<uint8_t>* out);
     static std::vector<int64_t> shape(const RocmStorage& s) { return s.shape; }
 
+    // A dense row-major copy of a view (the same storage when it already is dense): CpuStorage::contiguous,
+    // cpu/storage.rs:407-440.
+    static Error contiguous(const RocmStorage& s, RocmStorage* out);
+
     // Metadata-only views, as the reference's storages provide.
     static Error transpose(const RocmStorage& s, int a, int b, RocmStorage* out);
     static Error broadcast_as(const RocmStorage& s, const std::vector<int64_t>& dims, RocmStorage* out);

@@ -51,6 +51,11 @@ int incin_host_shape(const incin_host_storage* s, int64_t* dims_out)
     for (size_t i = 0; i < s->s.shape.size(); ++i) dims_out[i] = s->s.shape[i];
     return 0;
 }
+int incin_host_strides(const incin_host_storage* s, int64_t* strides_out)
+{
+    for (size_t i = 0; i < s->s.strides.size(); ++i) strides_out[i] = s->s.strides[i];
+    return 0;
+}
 int incin_host_dtype(const incin_host_storage* s, int32_t* out) { *out = (int32_t)s->s.dtype; return 0; }
 
 int incin_host_to_bytes(const incin_host_storage* s, void* out, size_t capacity)

@@ -18,6 +18,7 @@ int incin_host_from_bytes(const void* bytes, size_t nbytes, const int64_t* dims,
 int incin_host_numel(const incin_host_storage* s, int64_t* out);
 int incin_host_rank(const incin_host_storage* s, int32_t* out);
 int incin_host_shape(const incin_host_storage* s, int64_t* dims_out);
+int incin_host_strides(const incin_host_storage* s, int64_t* strides_out);      /* elements; 0 on a broadcast axis */
 int incin_host_dtype(const incin_host_storage* s, int32_t* out);
 int incin_host_to_bytes(const incin_host_storage* s, void* out, size_t capacity);
 int incin_host_transpose(const incin_host_storage* s, int32_t a, int32_t b, incin_host_storage** out);

@@ -147,7 +147,7 @@ namespace {
 const std::vector<DTypeId> ROCM_DTYPES = {DTypeId::BF16, DTypeId::F16, DTypeId::F32};      // what RocmStorage holds
 const std::vector<MathMode> PRECISE = {MathMode::Precise};
 const std::vector<LayoutClass> ANY_VIEW = {LayoutClass::Contiguous, LayoutClass::Strided, LayoutClass::RowWise};
-// attention reads q, k, v through their strides but needs the last axis dense: contiguous tensors and views
+// the attention kernels read q, k, v through their strides with the last axis dense: contiguous tensors and views
 // whose rows are contiguous (transposes of batch axes, narrows, broadcasts)
 const std::vector<LayoutClass> ROW_VIEWS = {LayoutClass::Contiguous, LayoutClass::RowWise};
 }  // namespace
@@ -160,11 +160,18 @@ const std::vector<CapabilityRule>& rocm_capabilities()
         // metadata-only views: transpose / narrow answer through the `storage` family, broadcast_as and reshape by rules of
         // their own
         {OperationKind::Broadcast, ROCM_DTYPES, ANY_VIEW, 0, MAX_RANK, false, PRECISE, ImplementationKind::Native},
-        // reshape re-addresses contiguous storage; a view has to be materialised by the caller first
+        // reshape re-addresses contiguous storage; any other view is first gathered into a dense copy, as the reference's
+        // reshape does (cpu/storage.rs:407-440)
         {OperationKind::Reshape, ROCM_DTYPES, {LayoutClass::Contiguous}, 0, MAX_RANK, false, PRECISE, ImplementationKind::Native},
-        // scaled_dot_product_attention and its gradients (RocmBackend::attention_backward; broadcast batch axes other than
-        // the group axis of grouped queries are refused by the operator itself)
+        {OperationKind::Reshape, ROCM_DTYPES, {LayoutClass::Strided, LayoutClass::RowWise}, 0, MAX_RANK, false, PRECISE,
+         ImplementationKind::Composed},
+        // scaled_dot_product_attention and its gradients (RocmBackend::attention_backward).  What a query cannot say and
+        // the operator still refuses: gradients for operands repeated along a batch axis other than the group axis of
+        // grouped queries, a non-contiguous upstream gradient, query lengths under training, and a mask whose broadcast
+        // would enlarge the score shape.
         {OperationKind::Attention, ROCM_DTYPES, ROW_VIEWS, 2, MAX_RANK, true, PRECISE, ImplementationKind::Native},
+        // operands whose last axis is strided (a transposed view): gathered into dense temporaries, then the same kernels
+        {OperationKind::Attention, ROCM_DTYPES, {LayoutClass::Strided}, 2, MAX_RANK, true, PRECISE, ImplementationKind::Composed},
     };
     return rules;
 }

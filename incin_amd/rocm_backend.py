@@ -21,7 +21,7 @@ F32, F16, BF16 = 0, 1, 2
 KINDS = ["None", "Msg", "ShapeMismatch", "DTypeStorageMismatch", "DeviceMismatch", "UnsupportedDType",
          "InvalidDeviceOrdinal", "OutOfMemory", "UnsupportedBackendOperation"]
 EXPORTS = [
-    "incin_host_last_error", "incin_host_from_bytes", "incin_host_numel", "incin_host_rank", "incin_host_shape",
+    "incin_host_last_error", "incin_host_from_bytes", "incin_host_numel", "incin_host_rank", "incin_host_shape", "incin_host_strides",
     "incin_host_dtype", "incin_host_to_bytes", "incin_host_transpose", "incin_host_broadcast_as",
     "incin_host_narrow", "incin_host_tag_causal", "incin_host_tag_key_padding",
     "incin_host_scaled_dot_product_attention", "incin_host_attention_backward", "incin_host_release", "incin_host_last_launch_count",
@@ -58,6 +58,7 @@ def lib():
         L.incin_host_numel.argtypes = [C.c_void_p, C.POINTER(C.c_int64)]
         L.incin_host_rank.argtypes = [C.c_void_p, C.POINTER(C.c_int32)]
         L.incin_host_shape.argtypes = [C.c_void_p, C.POINTER(C.c_int64)]
+        L.incin_host_strides.argtypes = [C.c_void_p, C.POINTER(C.c_int64)]
         L.incin_host_dtype.argtypes = [C.c_void_p, C.POINTER(C.c_int32)]
         L.incin_host_to_bytes.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
         L.incin_host_transpose.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.POINTER(C.c_void_p)]
@@ -148,6 +149,14 @@ class RocmStorage:
         return tuple(d[i] for i in range(r.value))
 
     @property
+    def strides(self):
+        """Element strides of the view (0 on a broadcast axis)."""
+        n = len(self.shape)
+        d = (C.c_int64 * max(n, 1))()
+        lib().incin_host_strides(self._h, d)
+        return tuple(d[i] for i in range(n))
+
+    @property
     def dtype(self):
         t = C.c_int32()
         lib().incin_host_dtype(self._h, C.byref(t))
@@ -187,6 +196,10 @@ class RocmStorage:
 
     def narrow(self, dim, start, length):
         return self._view(lib().incin_host_narrow, dim, start, length)
+
+    def reshape(self, dims):
+        """Same elements under another shape; a view that is not dense is gathered into a dense copy first."""
+        return self._view(lib().incin_host_reshape, _dims(dims), len(dims))
 
     def tag_causal(self):
         return self._view(lib().incin_host_tag_causal)

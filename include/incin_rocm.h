@@ -92,6 +92,13 @@ int incin_rocm_memset(int32_t dev, void* dst, int value, size_t bytes);
 int incin_rocm_memcpy_h2d(int32_t dev, void* dst, const void* src, size_t bytes);
 int incin_rocm_memcpy_d2h(int32_t dev, void* dst, const void* src, size_t bytes);
 int incin_rocm_memcpy_d2d(int32_t dev, void* dst, const void* src, size_t bytes);
+/* Logical (row-major) contents of a strided view written densely to `dst`: what CpuStorage::contiguous does on the
+ * host (crates/incin-backends/src/cpu/storage.rs:407-440), here one kernel enqueued on `stream`.  `shape` and `strides`
+ * (elements; 0 on a broadcast axis, negative allowed) have `rank` <= 8 entries, `src` points at the view's first
+ * element, elements are 2 or 4 bytes.  The backend uses it for operands of attention whose last axis is strided
+ * (a transposed view). */
+int incin_rocm_copy_strided(int32_t dev, void* dst, const void* src, int32_t rank, const int64_t* shape, const int64_t* strides,
+                            int32_t elem_bytes, void* stream);
 int incin_rocm_sync(int32_t dev);      /* waits for the device's default stream and any stream created here */
 
 /* ---- streams and events -------------------------------------------------------

@@ -15,7 +15,10 @@ from oracle import oracle as O
 pytestmark = pytest.mark.gpu
 CODE = {"f32": RB.F32, "f16": RB.F16, "bf16": RB.BF16}
 TOL = {"f32": 1e-5, "f16": 2e-2, "bf16": 2e-2}
-RULES = {r.operation: r for r in RC.registrations("rocm")}
+RULES = {}
+for _r in RC.registrations("rocm"):
+    RULES.setdefault(_r.operation, _r)          # the first (native) rule of an operation
+ATTENTION_CELLS = [(r.implementation, layout) for r in RC.registrations("rocm") if r.operation == "attention" for layout in r.layouts]
 
 
 def say(msg):
@@ -32,6 +35,10 @@ def operand(a, dtype, layout):
     allocation (narrow along the row axis and, with batch axes, a transpose of two of them)."""
     if layout == "contiguous":
         return RB.RocmStorage.from_numpy(a, CODE[dtype])
+    if layout == "strided":        # stored with the last two axes swapped, viewed back: the last axis is strided
+        s = RB.RocmStorage.from_numpy(np.ascontiguousarray(np.swapaxes(a, -1, -2)), CODE[dtype]).transpose(a.ndim - 1, a.ndim - 2)
+        assert s.shape == a.shape and s.strides[-1] != 1 and np.array_equal(s.to_numpy(), a)
+        return s
     assert layout == "row-wise"
     if a.ndim >= 4:        # store with the first two batch axes swapped and 2 spare rows, view it back
         big = np.zeros(a.shape[:-2] + (a.shape[-2] + 2, a.shape[-1]), np.float32)
@@ -59,11 +66,11 @@ def shapes_of_rank(rank):
 
 
 @pytest.mark.parametrize("dtype", RULES["attention"].dtypes)
-@pytest.mark.parametrize("layout", RULES["attention"].layouts)
+@pytest.mark.parametrize("level, layout", ATTENTION_CELLS)
 @pytest.mark.parametrize("rank", [RULES["attention"].min_rank, RULES["attention"].max_rank])
-def test_attention_rule_boundary_cases_execute(gpu, dtype, layout, rank):
+def test_attention_rule_boundary_cases_execute(gpu, dtype, level, layout, rank):
     case = RC.CapabilityQuery("attention", dtype, layout, rank)
-    assert RC.support("rocm", case).level == "native"
+    assert RC.support("rocm", case).level == level
     qs, ks, vs = shapes_of_rank(rank)
     say("capability cell %s: q%s k%s" % (case, qs, ks))
     q, k, v = rnd(1, qs, dtype), rnd(2, ks, dtype), rnd(3, vs, dtype)
@@ -76,15 +83,15 @@ def test_attention_rule_boundary_cases_execute(gpu, dtype, layout, rank):
 
 
 @pytest.mark.parametrize("dtype", RULES["attention"].dtypes)
-@pytest.mark.parametrize("layout", RULES["attention"].layouts)
+@pytest.mark.parametrize("level, layout", ATTENTION_CELLS)
 @pytest.mark.parametrize("rank", [RULES["attention"].min_rank, RULES["attention"].max_rank])
-def test_attention_rule_boundary_cases_train(gpu, dtype, layout, rank):
+def test_attention_rule_boundary_cases_train(gpu, dtype, level, layout, rank):
     """The same cells with `training` set: the rule says yes, so the gradients come out and match the backward oracle
     (1e-5 of the largest gradient magnitude for f32, 2e-2 for the 16-bit types)."""
     from oracle import sdpa_backward as BW
     assert RULES["attention"].training
     case = RC.CapabilityQuery("attention", dtype, layout, rank, training=True)
-    assert RC.support("rocm", case).level == "native"
+    assert RC.support("rocm", case).level == level
     qs, ks, vs = shapes_of_rank(rank)
     say("capability cell %s: q%s k%s" % (case, qs, ks))
     q, k, v = rnd(1, qs, dtype), rnd(2, ks, dtype), rnd(3, vs, dtype)
@@ -119,12 +126,12 @@ def test_refused_cells_are_refused_by_the_operator_too(gpu):
     say("capability cells the registry refuses")
     q = rnd(5, (2, 8, 16), "f32")
     s = RB.RocmStorage.from_numpy(q)
-    # layout `strided` (last axis not dense): the registry says Layout, the operator UnsupportedBackendOperation
-    assert RC.support("rocm", RC.CapabilityQuery("attention", "f32", "strided", 3)).reason == "Layout"
-    with pytest.raises(RB.BackendError) as e:
-        t = RB.RocmStorage.from_numpy(np.ascontiguousarray(np.swapaxes(q, -1, -2))).transpose(1, 2)
-        RB.scaled_dot_product_attention(t, s, s)
-    assert e.value.kind == "UnsupportedBackendOperation"
+    # layout `strided` (last axis not dense) is served through a dense temporary: composed, and it runs
+    assert RC.support("rocm", RC.CapabilityQuery("attention", "f32", "strided", 3)).level == "composed"
+    t = RB.RocmStorage.from_numpy(np.ascontiguousarray(np.swapaxes(q, -1, -2))).transpose(1, 2)
+    assert np.abs(RB.scaled_dot_product_attention(t, s, s).to_numpy() - O.sdpa(q, q, q)).max() <= 1e-5
+    # a reshape of that view is a gather followed by re-addressing
+    assert np.array_equal(t.reshape((16, 8, 2)).to_numpy(), q.reshape(16, 8, 2))
     # rank 1: registry says Rank, operator ShapeMismatch
     assert RC.support("rocm", RC.CapabilityQuery("attention", "f32", "contiguous", 1)).reason == "Rank"
     with pytest.raises(RB.BackendError) as e:

@@ -50,10 +50,10 @@ def test_unsupported_cells_return_the_documented_constraint():
     assert (s.level, s.reason, s.message) == ("unsupported", "DType", "dtype F64 is unsupported for attention")
     s = RC.support("rocm", Q("attention", "q8_0", "contiguous", 4))
     assert s.reason == "DType" and s.message == "dtype Q8_0 is unsupported for attention"
-    # a view whose last axis is not dense is refused up front (the operator answers it with
-    # UnsupportedBackendOperation, see the GPU test of the same cell)
-    s = RC.support("rocm", Q("attention", "bf16", "strided", 4))
-    assert (s.reason, s.message) == ("Layout", "layout strided is unsupported for attention")
+    # a view whose last axis is not dense runs through a dense temporary: composed, not native
+    assert RC.support("rocm", Q("attention", "bf16", "strided", 4)).level == "composed"
+    s = RC.support("rocm", Q("attention", "bf16", "channel-wise", 4))
+    assert (s.reason, s.message) == ("Layout", "layout channel-wise is unsupported for attention")
     s = RC.support("rocm", Q("attention", "f32", "contiguous", 1))
     assert (s.reason, s.message) == ("Rank", "rank 1 is unsupported for attention; expected 2..=8")
     assert RC.support("rocm", Q("attention", "bf16", "contiguous", 4, training=True)).level == "native"
@@ -78,11 +78,12 @@ def test_operations_without_rules_of_their_own_resolve_through_their_family():
         assert RC.support("rocm", Q(op, "bf16", "strided", 5)).level == "native"
         assert RC.support("rocm", Q(op, "i64", "contiguous", 5)).reason == "DType"
     # broadcast and reshape have rules of their own, which then are the only ones consulted: reshape re-addresses
-    # contiguous storage only
+    # contiguous storage and gathers any other view into a dense copy first
     assert RC.support("rocm", Q("broadcast", "f16", "row-wise", 8)).level == "native"
     assert RC.support("rocm", Q("reshape", "f16", "contiguous", 8)).level == "native"
-    s = RC.support("rocm", Q("reshape", "f16", "strided", 3))
-    assert (s.reason, s.message) == ("Layout", "layout strided is unsupported for reshape")
+    assert RC.support("rocm", Q("reshape", "f16", "strided", 3)).level == "composed"
+    s = RC.support("rocm", Q("reshape", "f16", "scalar-left", 3))
+    assert (s.reason, s.message) == ("Layout", "layout scalar-left is unsupported for reshape")
 
 
 @pytest.mark.parametrize("device", ["cuda", "wgpu", "metal"])
@@ -99,4 +100,5 @@ def test_checked_in_table_is_what_the_renderer_produces():
     assert open(DOC).read() == text, "regenerate with INCIN_DOCS=overwrite python -m pytest tests/test_capability_registry.py"
     assert "| `attention` | `f32` | `bf16`, `f16`, `f32` |" in text
     assert "| `attention` | `bf16`, `f16`, `f32` | `contiguous`, `row-wise` | 2+ | yes | native |" in text
+    assert "| `attention` | `bf16`, `f16`, `f32` | `strided` | 2+ | yes | composed |" in text
     assert "| `broadcast` | — | `bf16`, `f16`, `f32` |" in text

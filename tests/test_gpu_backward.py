@@ -185,3 +185,29 @@ def test_backward_refuses_what_it_does_not_cover(gpu):
     with pytest.raises(capi.RocmError) as e:
         host.sdpa_backward(q, k, v, go, capi.F32)
     assert e.value.code == capi.EUNSUPPORTED
+
+
+@pytest.mark.parametrize("dtype", [capi.BF16, capi.F32])
+def test_no_keys_gives_a_zero_query_gradient(gpu, dtype):
+    """Queries but no keys: the output is zeros whatever q holds, so dq is zeros (the reference's tape gives zeros), and
+    the entry point promises to overwrite it; dk and dv have no elements."""
+    say("backward with an empty key axis, dtype %d" % dtype)
+    B, H, Sq, D = 2, 3, 50, 128
+    q, _, _, go = make(5, B, H, H, Sq, 1, D, dtype)
+    empty = np.zeros((B, H, 0, D), np.float32)
+    tq, tg = host.DeviceTensor.from_f32(q, dtype), host.DeviceTensor.from_f32(go, dtype)
+    tk, tv, tdk, tdv = (host.DeviceTensor.from_f32(empty, dtype) for _ in range(4))
+    to, tdq = host.DeviceTensor((B, H, Sq, D), dtype), host.DeviceTensor((B, H, Sq, D), dtype)
+    capi.check(capi.load().incin_rocm_memset(0, tdq.ptr, 0x7f, tdq.buf.nbytes))          # what an allocator may leave behind
+    lse = capi.DeviceBuffer(B * H * Sq * 4)
+    bd = capi.SdpaBwdDesc()
+    bd.fwd = host.make_desc(tq, tk, tv, to, lse=lse)
+    for name, t in (("d_o", tg), ("d_q", tdq), ("d_k", tdk), ("d_v", tdv)):
+        setattr(bd, name, t.ptr)
+        for i, s in enumerate(host._strides3(t.shape)):
+            getattr(bd, name + "_stride")[i] = s
+    assert capi.sdpa_bwd_workspace(bd) == 0
+    capi.sdpa_fwd(bd.fwd)
+    capi.sdpa_bwd(bd)
+    capi.sync()
+    assert not to.to_f32().any() and not tdq.to_f32().any()

@@ -330,3 +330,28 @@ def test_rows_beyond_the_key_count_are_never_read(gpu, impl, dtype, sq):
     assert np.isfinite(dirty).all()
     assert np.array_equal(dirty, clean)
     check(dirty, oracle_full(q, k, v, G=Hq // Hkv, kv_lens=lens), TOL[dtype], "junk tail")
+
+
+@pytest.mark.parametrize("impl, sq", [(capi.IMPL_MFMA, 96), (capi.IMPL_MFMA64, 96), (capi.IMPL_SPLITKV, 2), (capi.IMPL_GENERIC, 40)],
+                         ids=["mfma", "mfma64", "splitkv", "generic"])
+@pytest.mark.parametrize("dtype", [capi.BF16, capi.F16])
+def test_large_logits(gpu, dtype, impl, sq):
+    """Logits of magnitude 50 with many keys within a few units of each row's maximum, and query rows whose elements are
+    all equal - so that whatever rounding a kernel applies to a query element (the matrix-core kernels fold
+    scale * log2(e) into Q and round it back to the storage type) hits every element of the row the same way and shows
+    up as a relative error of the whole logit row instead of averaging out.  Same absolute bar as everywhere."""
+    B, H, Skv, D = 2, 2, 320, 128
+    r = rng(SEED0 + 90)
+    x = r.choice(np.array([1.7265625, 1.8359375, 1.9140625, 2.0546875, 2.1328125], np.float32), size=(B, H, sq, 1))
+    q = dtypes.round_to(np.broadcast_to(x * r.choice([-1.0, 1.0], size=(B, H, sq, 1)).astype(np.float32), (B, H, sq, D)).copy(), dtype)
+    c = r.uniform(-2.2, 2.2, size=(B, H, Skv, 1)).astype(np.float32)
+    k = dtypes.round_to(c + 0.05 * r.standard_normal((B, H, Skv, D), dtype=np.float32), dtype)
+    v = dtypes.round_to(r.standard_normal((B, H, Skv, D), dtype=np.float32), dtype)
+    logits = np.einsum("bhid,bhjd->bhij", q, k) / np.sqrt(np.float32(D))
+    top = np.sort(logits, axis=-1)[..., -8:]
+    say("large logits: impl %d dtype %d, max |logit| %.1f, 8th-largest within %.2f of the row maximum (median)"
+        % (impl, dtype, np.abs(logits).max(), np.median(top[..., -1] - top[..., 0])))
+    assert np.abs(logits).max() > 45
+    got, info = host.sdpa(q, k, v, dtype, impl=impl, return_info=True, num_splits=2 if impl == capi.IMPL_SPLITKV else 0)
+    assert info["impl"] == impl
+    check(got, oracle_full(q, k, v), TOL[dtype], "large logits")

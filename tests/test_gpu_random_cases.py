@@ -79,16 +79,25 @@ def run_case(i, c, r):
     return impls
 
 
+WORST = {}       # dtype -> (absolute error, what): the largest error seen, for the log
+
+
 def check(i, c, impl, got, ref):
     what = "case %d impl %d %s" % (i, impl, {k: (v if not isinstance(v, np.ndarray) else v.shape) for k, v in c.items()})
     nr = np.isnan(ref)
     assert np.array_equal(np.isnan(got), nr), what + ": NaN pattern"
     err = float(np.abs(np.where(nr, 0, got) - np.where(nr, 0, ref)).max()) if got.size else 0.0
-    # The stated bars (1e-5, 2e-2) are absolute and meant for outputs of order one, as the default scale gives; a drawn
-    # scale several times the default makes the softmax pick single values of v (|o| up to ~4), where one bf16 rounding
-    # of the output is already 8e-3: the bar scales with the largest output magnitude there.
     big = float(np.abs(np.where(nr, 0, ref)).max()) if got.size else 0.0
-    assert err <= TOL[c["dtype"]] * max(1.0, big), "%s: %.3e (outputs up to %.2f)" % (what, err, big)
+    if err > WORST.get(c["dtype"], (-1.0, ""))[0]:
+        WORST[c["dtype"]] = (err, "%s (outputs up to %.2f)" % (what, big))
+    if c["dtype"] == capi.F32:
+        bar = TOL[capi.F32]                 # absolute, whatever the magnitudes
+    else:
+        # 16-bit outputs: the stated bar (2e-2) is absolute and meant for outputs of order one, as the default scale gives;
+        # a drawn scale several times the default makes the softmax pick single values of v (|o| up to ~4), where one
+        # bf16 rounding of the output is already 8e-3: there the bar scales with the largest output magnitude.
+        bar = TOL[c["dtype"]] * max(1.0, big)
+    assert err <= bar, "%s: %.3e (outputs up to %.2f)" % (what, err, big)
 
 
 def test_random_cases(gpu):
@@ -101,5 +110,7 @@ def test_random_cases(gpu):
         for impl in run_case(i, c, r):
             used[impl] = used.get(impl, 0) + 1
     say("kernels exercised: %s" % used)
+    for dt, (err, what) in sorted(WORST.items()):
+        say("worst absolute error, dtype %d: %.3e in %s" % (dt, err, what))
     for impl in (capi.IMPL_GENERIC, capi.IMPL_MFMA, capi.IMPL_MFMA64, capi.IMPL_SPLITKV):
         assert used.get(impl, 0) >= 5, "kernel %d was hardly reached: %s" % (impl, used)

@@ -130,6 +130,22 @@ def test_tagged_masks_equal_their_dense_form(gpu, dtype):
     close(RB.scaled_dot_product_attention(Q, K, V, P.tag_key_padding(lens)).to_numpy(), ref, TOL[dtype], "tagged padding")
 
 
+def test_key_lengths_with_one_shared_kv_head(gpu):
+    # rank-4 multi-query layout: q [B,H,S,D] against k, v [B,1,S,D]; the key counts are per batch entry
+    say("host mirror: multi-query operands with tagged key padding")
+    dtype = RB.BF16
+    B, H, Sq, Skv, D = 3, 4, 33, 150, 128
+    q, k, v = rnd(45, (B, H, Sq, D), dtype), rnd(46, (B, 1, Skv, D), dtype), rnd(47, (B, 1, Skv, D), dtype)
+    lens = [150, 1, 77]
+    pm = np.zeros((B, 1, 1, Skv), np.float32)
+    for b, n in enumerate(lens):
+        pm[b, ..., n:] = -np.inf
+    Q, K, V = (RB.RocmStorage.from_numpy(x, dtype) for x in (q, k, v))
+    P = RB.RocmStorage.from_numpy(pm, dtype).tag_key_padding(lens)
+    close(RB.scaled_dot_product_attention(Q, K, V, P).to_numpy(), O.sdpa(q, k, v, mask=pm), TOL[dtype], "multi-query padding")
+    assert RB.last_launch_count() == 1
+
+
 def test_views_as_operands(gpu):
     # k handed over as a narrowed, transposed-back view of a larger cache; q as a slice of a [B,S,H,D] layout
     say("host mirror: strided operands")
@@ -143,6 +159,34 @@ def test_views_as_operands(gpu):
     out = RB.scaled_dot_product_attention(Q, K, V)
     ref = O.sdpa(q_bshd.transpose(0, 2, 1, 3), kc[:, :, 8:68], vc[:, :, 8:68])
     close(out.to_numpy(), ref, TOL[dtype], "strided operands")
+
+
+@pytest.mark.parametrize("dtype", [RB.F32, RB.BF16])
+def test_operands_with_a_strided_last_axis(gpu, dtype):
+    """k handed over as transpose(kt) of [.., D, Skv] storage - the view the reference's own matmul test goes through
+    (cpu/ops/matmul.rs:677-724) - and v, q the same way, one of them also repeated over heads (stride 0): any view is an
+    operand (cpu/storage.rs:308-325).  Checked against the oracle, whose strided arm reads the same views."""
+    say("host mirror: operands whose last axis is strided, dtype %s" % dtype)
+    B, H, Sq, Skv, D = 2, 3, 40, 70, 64
+    q = rnd(60, (B, H, Sq, D), dtype)
+    kt, vt = rnd(61, (B, 1, D, Skv), dtype), rnd(62, (B, H, D, Skv), dtype)        # stored transposed; k shared by the heads
+    Q = RB.RocmStorage.from_numpy(q, dtype)
+    K = RB.RocmStorage.from_numpy(kt, dtype).transpose(2, 3).broadcast_as((B, H, Skv, D))
+    V = RB.RocmStorage.from_numpy(vt, dtype).transpose(2, 3)
+    assert K.strides[-1] != 1 and V.strides[-1] != 1 and K.strides[1] == 0
+    k_log = np.broadcast_to(kt.transpose(0, 1, 3, 2), (B, H, Skv, D))
+    v_log = vt.transpose(0, 1, 3, 2)
+    assert np.array_equal(K.to_numpy(), k_log) and np.array_equal(V.to_numpy(), v_log)        # the device-side gather itself
+    ref = O.sdpa(q, k_log, v_log)                       # numpy views: the oracle walks the same strides
+    out = RB.scaled_dot_product_attention(Q, K, V)
+    close(out.to_numpy(), ref, TOL[dtype], "transposed k and v")
+    # q strided too, with a dense mask and a causal tag on top
+    qt = rnd(63, (B, H, D, Sq), dtype)
+    Qt = RB.RocmStorage.from_numpy(qt, dtype).transpose(2, 3)
+    m = np.where(np.random.Generator(np.random.PCG64(64)).random((Sq, Skv)) < 0.2, -np.inf, 0.0).astype(np.float32)
+    m[:, 0] = 0.0
+    out = RB.scaled_dot_product_attention(Qt, K, V, mask=RB.RocmStorage.from_numpy(m, dtype))
+    close(out.to_numpy(), O.sdpa(qt.transpose(0, 1, 3, 2), k_log, v_log, mask=m), TOL[dtype], "transposed q, k, v with a mask")
 
 
 def test_decode_step(gpu):
