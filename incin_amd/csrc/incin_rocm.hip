@@ -20,6 +20,7 @@ namespace incin_rocm {
 hipError_t launch_sdpa_generic(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_sdpa_prefill_mfma(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_sdpa_prefill_mfma64(const SdpaParams& p, int dtype, hipStream_t stream);
+hipError_t launch_sdpa_prefill_f32(const SdpaParams& p, hipStream_t stream);
 hipError_t launch_sdpa_decode(const SdpaParams& p, int dtype, hipStream_t stream);
 int decode_keys_per_tile(int dtype, int D, int R);
 }  // namespace incin_rocm
@@ -122,12 +123,17 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     const int vec = d->dtype == INCIN_ROCM_F32 ? 4 : 8;
     const int64_t R = (d->Hq / d->Hkv) * d->Sq;
     const bool head_ok = d->D == d->Dv && (d->D == 64 || d->D == 128);
-    const bool fast_ok = head_ok && !d->add_mask && fast_layout_ok(d, vec) && d->Skv > 0;
-    // the MFMA kernel addresses a K/V tile with 32-bit byte offsets from the tile's first row
-    const bool tile_off_ok = d->k_stride[2] >= 0 && d->v_stride[2] >= 0 && d->k_stride[2] < (1 << 24) && d->v_stride[2] < (1 << 24);
-    const bool mfma_ok = fast_ok && tile_off_ok && d->dtype != INCIN_ROCM_F32 && d->scale > 0.0f && std::isfinite(d->scale);
+    const bool layout_ok = head_ok && fast_layout_ok(d, vec) && d->Skv > 0;
+    const bool fast_ok = layout_ok && !d->add_mask;
+    // the MFMA kernels address a K/V tile with 32-bit byte offsets from the tile's first row
+    const int64_t stride_lim = d->dtype == INCIN_ROCM_F32 ? (1 << 22) : (1 << 24);
+    const bool tile_off_ok = d->k_stride[2] >= 0 && d->v_stride[2] >= 0 && d->k_stride[2] < stride_lim && d->v_stride[2] < stride_lim;
+    // f32: the IEEE-f32 matrix-core kernel, which also takes a dense additive mask and any finite scale;
+    // f16 / bf16: the 16-bit kernels fold the scale into Q in a way that needs it positive, and take no dense mask
+    const bool mfma_ok = d->dtype == INCIN_ROCM_F32 ? (layout_ok && tile_off_ok && std::isfinite(d->scale))
+                                                    : (fast_ok && tile_off_ok && d->scale > 0.0f && std::isfinite(d->scale));
     // the 64-row kernel does its byte arithmetic on a head's K and V in 32 bits, up to 16 tiles of 32 rows past the end
-    const bool mfma64_ok = mfma_ok && d->D == 128 && (d->Skv + 512) * d->k_stride[2] * 2 < (1LL << 31) &&
+    const bool mfma64_ok = mfma_ok && d->dtype != INCIN_ROCM_F32 && d->D == 128 && (d->Skv + 512) * d->k_stride[2] * 2 < (1LL << 31) &&
                            (d->Skv + 512) * d->v_stride[2] * 2 < (1LL << 31);
     const bool split_ok = fast_ok && d->Sq <= 64;
 
@@ -145,7 +151,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     }
     if (impl == INCIN_ROCM_IMPL_MFMA && !mfma_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
-                    "scaled_dot_product_attention: the MFMA kernel needs f16/bf16, D == Dv in {64,128}, scale > 0, no dense mask and 16-byte aligned rows");
+                    "scaled_dot_product_attention: the MFMA kernels need D == Dv in {64,128} and 16-byte aligned rows; for f16/bf16 also scale > 0 and no dense mask");
     if (impl == INCIN_ROCM_IMPL_MFMA64 && !mfma64_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
                     "scaled_dot_product_attention: the 64-row MFMA kernel needs what the MFMA kernel needs, D == Dv == 128 and key/value slices below 2 GiB");
@@ -495,7 +501,9 @@ static int launch_fwd(const incin_rocm_sdpa_desc_t* desc, const Plan& plan, void
     hipStream_t s = (hipStream_t)stream;
     hipError_t e;
     switch (plan.impl) {
-        case INCIN_ROCM_IMPL_MFMA: e = incin_rocm::launch_sdpa_prefill_mfma(p, desc->dtype, s); break;
+        case INCIN_ROCM_IMPL_MFMA:
+            e = desc->dtype == INCIN_ROCM_F32 ? incin_rocm::launch_sdpa_prefill_f32(p, s) : incin_rocm::launch_sdpa_prefill_mfma(p, desc->dtype, s);
+            break;
         case INCIN_ROCM_IMPL_MFMA64: e = incin_rocm::launch_sdpa_prefill_mfma64(p, desc->dtype, s); break;
         case INCIN_ROCM_IMPL_SPLITKV: e = incin_rocm::launch_sdpa_decode(p, desc->dtype, s); break;
         default: e = incin_rocm::launch_sdpa_generic(p, desc->dtype, s); break;

@@ -45,7 +45,8 @@ enum { INCIN_ROCM_F32 = 0, INCIN_ROCM_F16 = 1, INCIN_ROCM_BF16 = 2 };
 enum {
     INCIN_ROCM_IMPL_AUTO = 0,
     INCIN_ROCM_IMPL_GENERIC = 1,   /* fp32-FMA tiled kernel: any dtype, D and Dv <= 256, dense masks     */
-    INCIN_ROCM_IMPL_MFMA = 2,      /* bf16/f16 MFMA prefill kernel: D == Dv in {64,128}                    */
+    INCIN_ROCM_IMPL_MFMA = 2,      /* MFMA prefill kernels, D == Dv in {64,128}: bf16/f16 (no dense mask, scale > 0), and
+                                      IEEE-f32 matrix instructions for f32 (dense mask allowed)                    */
     INCIN_ROCM_IMPL_SPLITKV = 3,   /* split-KV decode kernel + combine: D == Dv in {64,128}, few query rows */
     INCIN_ROCM_IMPL_MFMA64 = 4     /* bf16/f16 MFMA prefill kernel, 64 query rows per wavefront: D == Dv == 128 */
 };

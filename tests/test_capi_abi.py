@@ -56,7 +56,9 @@ def _plan(d):
 
 def test_dispatch_choices():
     assert _plan(_desc())[2] == capi.IMPL_MFMA
-    assert _plan(_desc(dtype=capi.F32))[2] == capi.IMPL_GENERIC
+    assert _plan(_desc(dtype=capi.F32))[2] == capi.IMPL_MFMA                  # the IEEE-f32 matrix-core kernel
+    assert _plan(_desc(dtype=capi.F32, add_mask=0x20000))[2] == capi.IMPL_MFMA  # which also takes a dense mask
+    assert _plan(_desc(dtype=capi.F32, D=80, Dv=80))[2] == capi.IMPL_GENERIC
     assert _plan(_desc(D=80, Dv=80))[2] == capi.IMPL_GENERIC
     assert _plan(_desc(add_mask=0x20000))[2] == capi.IMPL_GENERIC
     nbytes, splits, impl = _plan(_desc(Sq=1, Skv=8192, B=32, Hq=32, Hkv=32))
@@ -91,7 +93,8 @@ def test_dispatch_choices():
     (dict(q=None), capi.EINVAL),
     (dict(impl=9), capi.EINVAL),
     (dict(num_splits=-2), capi.EINVAL),
-    (dict(impl=capi.IMPL_MFMA, dtype=capi.F32), capi.EUNSUPPORTED),
+    (dict(impl=capi.IMPL_MFMA64, dtype=capi.F32), capi.EUNSUPPORTED),
+    (dict(impl=capi.IMPL_MFMA, add_mask=0x20000), capi.EUNSUPPORTED),
     (dict(impl=capi.IMPL_MFMA, D=80, Dv=80), capi.EUNSUPPORTED),
     (dict(impl=capi.IMPL_SPLITKV, Sq=4096), capi.EUNSUPPORTED),
     (dict(D=512, Dv=512), capi.EUNSUPPORTED),

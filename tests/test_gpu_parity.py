@@ -90,21 +90,28 @@ def test_buffer_round_trip(gpu):
 def test_config1_f32_single_head_noncausal(gpu):
     q, k, v = inputs(SEED0 + 0, 1, 1, 1, 128, 128, 64, 64, capi.F32)
     got, info = host.sdpa(q, k, v, capi.F32, scale=0.125, return_info=True)
-    assert info["impl"] == capi.IMPL_GENERIC
+    assert info["impl"] == capi.IMPL_MFMA               # the IEEE-f32 matrix-core kernel
     ref = O.sdpa(q, k, v, scale=0.125)
     check(got, ref, 1e-5, "C1 f32 B1 H1 S128 D64")
+    check(host.sdpa(q, k, v, capi.F32, scale=0.125, impl=capi.IMPL_GENERIC), ref, 1e-5, "C1, generic kernel")
     assert np.abs(ref - O.brute_f64(q, k, v, scale=0.125)).max() < 1e-6
 
 
 def test_config2_f32_multi_head_causal(gpu):
     q, k, v = inputs(SEED0 + 1, 4, 8, 8, 1024, 1024, 64, 64, capi.F32)
-    got = host.sdpa(q, k, v, capi.F32, causal=True)
+    got, info = host.sdpa(q, k, v, capi.F32, causal=True, return_info=True)
+    assert info["impl"] == capi.IMPL_MFMA
     mask = O.causal_additive_mask(1024, 1024)                       # the explicit 0/-inf tensor the CPU op is given
     ref = O.sdpa(q, k, v, mask=mask)
     check(got, ref, 1e-5, "C2 f32 B4 H8 S1024 D64 causal")
-    # the same mask handed over as a dense additive tensor goes through the mask path of the kernel
-    got2 = host.sdpa(q[:1, :2], k[:1, :2], v[:1, :2], capi.F32, mask=mask)
-    check(got2, ref[:1, :2], 1e-5, "C2 slice, dense additive mask")
+    check(host.sdpa(q, k, v, capi.F32, causal=True, impl=capi.IMPL_GENERIC), ref, 1e-5, "C2, generic kernel")
+    # the same mask handed over as a dense additive tensor, as a caller of the reference's operator passes it, goes
+    # through the mask path of either kernel
+    got2, info = host.sdpa(q, k, v, capi.F32, mask=mask, return_info=True)
+    assert info["impl"] == capi.IMPL_MFMA
+    check(got2, ref, 1e-5, "C2, dense additive mask")
+    got3 = host.sdpa(q[:1, :2], k[:1, :2], v[:1, :2], capi.F32, mask=mask, impl=capi.IMPL_GENERIC)
+    check(got3, ref[:1, :2], 1e-5, "C2 slice, dense additive mask, generic kernel")
 
 
 # ---- generic kernel: shapes, masks, dtypes ----------------------------------------------
@@ -201,6 +208,51 @@ def test_mfma_prefill(gpu, dtype, shape, impl):
         check(got, ref, TOL[dtype], "mfma %s %r causal=%d" % (dtypes.NAMES[dtype], shape, causal))
         gen = host.sdpa(q, k, v, dtype, causal=causal, impl=capi.IMPL_GENERIC)
         check(got, gen, TOL[dtype], "mfma vs generic kernel %r causal=%d" % (shape, causal))
+
+
+@pytest.mark.parametrize("shape", [
+    # B, Hq, Hkv, Sq, Skv, D
+    (1, 1, 1, 128, 128, 64),
+    (2, 4, 4, 512, 512, 128),
+    (1, 2, 2, 200, 333, 128),
+    (2, 8, 2, 256, 256, 64),
+    (1, 4, 1, 100, 1000, 64),
+    (1, 2, 2, 384, 129, 128),
+    (1, 1, 1, 17, 64, 128),
+    (1, 2, 1, 1000, 1000, 64),
+    (1, 1, 1, 300, 40, 64),
+    (2, 3, 3, 1, 70, 128),
+])
+def test_f32_matrix_core_prefill(gpu, shape):
+    """The IEEE-f32 matrix-core kernel on f32 operands - the reference's own dtype - against the oracle at 1e-5:
+    no mask, causal, ragged key counts with a causal mask, and dense additive masks of several broadcast shapes."""
+    B, Hq, Hkv, Sq, Skv, D = shape
+    G = Hq // Hkv
+    q, k, v = inputs(400 + sum(shape), B, Hq, Hkv, Sq, Skv, D, D, capi.F32)
+    for causal in (False, True):
+        got, info = host.sdpa(q, k, v, capi.F32, causal=causal, impl=capi.IMPL_MFMA, return_info=True)
+        assert info["impl"] == capi.IMPL_MFMA
+        check(got, oracle_full(q, k, v, G=G, causal=causal), 1e-5, "f32 mfma %r causal=%d" % (shape, causal))
+    r = rng(sum(shape))
+    lens = r.integers(0, Skv + 1, B).astype(np.int32)
+    got = host.sdpa(q, k, v, capi.F32, causal=True, kv_lens=lens, impl=capi.IMPL_MFMA)
+    check(got, oracle_full(q, k, v, G=G, causal=True, kv_lens=lens), 1e-5, "f32 mfma %r causal + kv_lens %s" % (shape, lens.tolist()))
+    for mshape in [(Sq, Skv), (1, Skv), (B, 1, Sq, Skv), (B, Hq, Sq, Skv), (1, Hq, 1, Skv)]:
+        m = r.standard_normal(mshape, dtype=np.float32)
+        m = np.where(r.random(mshape) < 0.25, -np.inf, m).astype(np.float32)
+        m[..., 0] = 0.0                                             # keep every row alive
+        got, info = host.sdpa(q, k, v, capi.F32, mask=m, scale=0.3 / np.sqrt(D / 32), return_info=True)
+        assert info["impl"] == capi.IMPL_MFMA
+        check(got, oracle_full(q, k, v, G=G, mask=m, scale=0.3 / np.sqrt(D / 32)), 1e-5, "f32 mfma %r mask %r" % (shape, mshape))
+    m = np.zeros((Sq, Skv), np.float32)
+    m[Sq // 2, :] = -np.inf                                         # one fully masked row: NaN, as the reference
+    got = host.sdpa(q, k, v, capi.F32, mask=m, impl=capi.IMPL_MFMA)
+    check(got, oracle_full(q, k, v, G=G, mask=m), 1e-5, "f32 mfma fully masked row")
+    got, lse = host.sdpa(q, k, v, capi.F32, causal=True, impl=capi.IMPL_MFMA, return_lse=True)
+    _, lse_g = host.sdpa(q, k, v, capi.F32, causal=True, impl=capi.IMPL_GENERIC, return_lse=True)
+    fin = np.isfinite(lse_g)                                        # rows without a visible key: -inf in both
+    assert np.array_equal(np.isfinite(lse), fin) and np.all(lse[~fin] == -np.inf)
+    assert not fin.any() or np.abs(lse[fin] - lse_g[fin]).max() <= 1e-5
 
 
 @pytest.mark.parametrize("impl", MFMA_IMPLS)

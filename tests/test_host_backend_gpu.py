@@ -236,9 +236,9 @@ def test_error_behaviour(gpu):
     with pytest.raises(RB.BackendError) as e:
         RB.RocmStorage.from_bytes(b"\0" * 8, (4,), RB.F32)
     assert e.value.kind == "Msg"
-    # k with a strided last axis has no kernel on this backend
-    kt = f(np.ones((2, 8, 6), np.float32)).transpose(1, 2)
-    assert kind(q, kt, v) == "UnsupportedBackendOperation"
+    # a head dimension beyond every kernel is a refusal, never a host fallback
+    big = f(np.ones((2, 4, 300), np.float32))
+    assert kind(big, big, big) == "UnsupportedBackendOperation"
 
 
 # ---- gradients through the host mirror ------------------------------------------------------------------------------
