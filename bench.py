@@ -28,11 +28,20 @@ from incin_amd import capi, dtypes, host  # noqa: E402
 
 SEED0 = 20261125
 PEAK_BF16_TFLOPS = 2516.6   # 256 CUs x 2.4 GHz x 4096 dense bf16 FLOP/clk/CU (vendor: 2.5 PFLOP/s)
+PEAK_F32_TFLOPS = 157.3      # dense fp32 matrix peak, vendor figure (256 CUs x 2.4 GHz x 256 FLOP/clk/CU)
 PEAK_HBM_GBS = 8000.0       # HBM3E, vendor figure
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same command (KiB per dispatch,
 # FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0 after calibration against the 1 GiB copy kernel): profiles/*.txt
 PREFILL_TRAFFIC_BYTES = (209881 * 2.0 + 131113) * 1024     # 5.64e8: |Q|+|K|+|V| read 1.07 times, |O| written once
 DECODE_TRAFFIC_BYTES = (2097470 * 2.0 + 1088 + 256) * 1024  # 4.297e9: K and V read once + split partials
+PREFILL_LONG_TRAFFIC_BYTES = None                           # filled from its counter run below when one exists
+# These three are constants taken from counter runs, not measured by this script: each roofline object says so and
+# names the summary the figures come from.
+TRAFFIC_SOURCE = {
+    "prefill": "constant from profiles/sdpa_prefill_mfma_bf16_d128_config3.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of `bench.py --only prefill`)",
+    "decode": "constant from profiles/sdpa_decode_splitkv_bf16_d128_config4.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of `bench.py --only decode`)",
+    "prefill_long": "profiles/sdpa_prefill_mfma64_bf16_d128_config5.txt",
+}
 METRIC = "attn fwd TFLOP/s + % bf16 MFMA peak; decode KV GB/s + % HBM peak (1 GPU)"
 
 
@@ -253,13 +262,72 @@ def backward_config3(steps, warmup):
             "parity_sample": "dQ, dK, dV of slice (b=%d, h=%d) against the float64 oracle of the reference's tape gradients" % (b, h)}
 
 
+def f32_configs(steps, warmup, with_cpu, threads):
+    """BASELINE configs 1 and 2 - f32, the one dtype the reference's operator runs end to end - on the IEEE-f32
+    matrix-core kernel: absolute TFLOP/s against the fp32 matrix peak, config 2 also with the causal mask handed over
+    as the explicit [S, S] tensor of 0 / -inf a caller of the reference's operator passes, and the oracle's
+    materialising restatement timed on all of config 2 beside it."""
+    from oracle import oracle as O
+    out = {}
+    for key, (B, H, S, D, causal, scale_note) in (("f32_c1", (1, 1, 128, 64, False, "scale=0.125")),
+                                                  ("f32_c2", (4, 8, 1024, 64, True, "scale=1/sqrt(64)"))):
+        w = Workload(key, SEED0 + (0 if key == "f32_c1" else 1), B, H, H, S, S, D, capi.F32, causal)
+        n = max(steps, 200)                                 # launches of tens of microseconds
+        wall, ev_mean, ev_med, ev_min = w.time(n, warmup)
+        flops = causal_flops(B, H, S, S, D) if causal else 4.0 * D * B * H * S * S
+        kernel = {capi.IMPL_MFMA: "sdpa_prefill_f32_kernel<%d>" % D, capi.IMPL_GENERIC: "sdpa_generic_kernel<float>"}.get(w.impl, str(w.impl))
+        rec = {"workload": "BASELINE config %s: f32 %s attention fwd B=%d H=%d S_q=S_kv=%d D=%d, %s" %
+                           (key[-1], "causal" if causal else "non-causal", B, H, S, D, scale_note),
+               "metric": "attn fwd TFLOP/s", "value": flops / (wall * 1e-3) / 1e12, "unit": "TFLOP/s", "dtype": "f32",
+               "ms_per_step": wall, "steps": n,
+               "roofline": {"bound": "mfma", "achieved": flops / (ev_mean * 1e-3) / 1e12, "peak": PEAK_F32_TFLOPS, "unit": "TFLOP/s",
+                            "frac": flops / (ev_mean * 1e-3) / 1e12 / PEAK_F32_TFLOPS, "traffic": None, "kernel": kernel,
+                            "algorithmic_flops_per_launch": flops, "launch_ms_mean": ev_mean, "launch_ms_median": ev_med,
+                            "launch_ms_min": ev_min},
+               "parity_max_abs_err": w.parity()}
+        if causal:
+            # the same problem with the mask as a tensor: the launch first classifies the tensor by blocks of 32 x 32 (hidden
+            # blocks are skipped, zero blocks run unmasked), FLOPs counted as above
+            mask = O.causal_additive_mask(S, S)
+            tm = capi.DeviceBuffer.from_numpy(mask)
+            w.desc.causal = 0
+            w.desc.add_mask = tm.ptr
+            for i, st in enumerate((0, 0, S, 1)):
+                w.desc.mask_stride[i] = st
+            mbytes = capi.sdpa_workspace(w.desc)[0]            # block flags of the mask
+            mws = capi.DeviceBuffer(mbytes) if mbytes else None
+            if mws is not None:
+                w.desc.workspace, w.desc.workspace_bytes = mws.ptr, mws.nbytes
+            wall_m = w.time(n, warmup)[0]
+            rec["with_dense_mask_tensor"] = {"what": "causal mask passed as an f32 [S, S] additive tensor (add_mask) instead of the causal flag",
+                                             "ms_per_step": wall_m, "value": flops / (wall_m * 1e-3) / 1e12, "unit": "TFLOP/s",
+                                             "parity_max_abs_err": w.parity()}
+            tm.free()
+            if mws is not None:
+                mws.free()
+            if with_cpu:
+                q, k, v = w.host
+                t0 = time.perf_counter()
+                O.sdpa_materialised(q, k, v, mask=mask)
+                dt = time.perf_counter() - t0
+                rec["cpu_baseline"] = {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                                       "sample": "all of config 2 (32 (b,h) slices, explicit 0/-inf causal mask), oracle's materialising "
+                                                 "restatement of the reference CPU op (not the Rust binary); %.1f s; host: %s" % (dt, host_cpu())}
+        w.free()
+        out[key] = rec
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["prefill", "prefill_long", "decode", "backward", "copy"], default=None,
+    ap.add_argument("--no-padding-compare", action="store_true",
+                    help="prefill_long: skip the extra timing of the batch with its padding rows computed (profiling: every "
+                         "launch of the run is then the same launch)")
+    ap.add_argument("--only", choices=["prefill", "prefill_long", "decode", "backward", "f32", "copy"], default=None,
                     help="run a single workload (profiling). 'copy' runs --steps device-to-device copies of 1 GiB "
                          "through the library's plain copy kernel: the known-size dispatch that hardware byte "
                          "counters (FETCH_SIZE / WRITE_SIZE) are calibrated against")
@@ -283,8 +351,8 @@ def main():
         "data": "synthetic: Q,K,V i.i.d. N(0,1) from numpy PCG64(seed 20261125+config), rounded to bf16",
         "config": {"workload": "BASELINE config 3: bf16 causal prefill B=8 H=16 S_q=S_kv=4096 D=128, scale=1/sqrt(128), "
                                "f32 accumulate, bf16 out", "step": "one incin_rocm_sdpa_fwd launch"},
-        "device": {"name": info.name.decode(), "arch": info.arch.decode(), "compute_units": info.compute_units,
-                   "clock_khz": info.clock_khz},
+        "device": {"name": info.name.decode() or info.arch.decode().split(":")[0], "arch": info.arch.decode(),
+                   "compute_units": info.compute_units, "clock_khz": info.clock_khz},
     }
 
     if args.only == "copy":
@@ -308,7 +376,7 @@ def main():
         result["ms_per_step"] = wall
         result["roofline"] = {"bound": "mfma", "achieved": flops / (ev_mean * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
                               "unit": "TFLOP/s", "frac": flops / (ev_mean * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": PREFILL_TRAFFIC_BYTES,
-                              "kernel": "sdpa_prefill_mfma_kernel<bf16,128>", "algorithmic_flops_per_launch": flops,
+                              "traffic_source": TRAFFIC_SOURCE["prefill"], "kernel": "sdpa_prefill_mfma_kernel<bf16,128>", "algorithmic_flops_per_launch": flops,
                               "launch_ms_mean": ev_mean, "launch_ms_median": ev_med, "launch_ms_min": ev_min}
         result["parity_max_abs_err"] = w.parity()
         w.free()
@@ -323,17 +391,18 @@ def main():
                           % (slices, threads, dt, host_cpu())}
 
     if args.only in (None, "prefill_long"):
-        # BASELINE config 5: grouped queries, 16384-token padded batch, causal + key padding; lengths U[2048, 16384]
-        # from the same seeded generator, one sequence at full length
+        # BASELINE config 5: grouped queries, batch padded to 16384 tokens, causal + key padding; lengths U[2048, 16384]
+        # from the same seeded generator
         B, Hq, Hkv, S, D = 4, 32, 8, 16384, 128
         lens = rng(SEED0 + 4).integers(2048, S + 1, B).astype(np.int64)
-        lens[0] = S
         w = Workload("prefill_c5", SEED0 + 4, B, Hq, Hkv, S, S, D, capi.BF16, True, kv_lens=lens, pad_queries=True)
         steps = max(5, min(args.steps, 20))                 # ~5 ms per launch
         # first the same batch with the padding rows computed (what a caller gets who can only hand over a key mask)
-        w.desc.q_lens = None
-        wall_all_rows = w.time(steps, 2)[0]
-        w.desc.q_lens = w.tl.ptr
+        wall_all_rows = None
+        if not args.no_padding_compare:
+            w.desc.q_lens = None
+            wall_all_rows = w.time(steps, 2)[0]
+            w.desc.q_lens = w.tl.ptr
         wall, ev_mean, ev_med, ev_min = w.time(steps, min(args.warmup, 5))
         flops = 4.0 * D * Hq * float(sum(int(n) * (int(n) + 1) // 2 for n in lens))      # rows i < lens[b] only
         kernel = {capi.IMPL_MFMA64: "sdpa_prefill_mfma64_kernel<bf16>", capi.IMPL_MFMA: "sdpa_prefill_mfma_kernel<bf16,128>"}.get(w.impl, str(w.impl))
@@ -343,7 +412,8 @@ def main():
                         "each length only" % lens.tolist(),
             "metric": "attn fwd TFLOP/s", "value": flops / (wall * 1e-3) / 1e12, "unit": "TFLOP/s", "ms_per_step": wall, "steps": steps,
             "roofline": {"bound": "mfma", "achieved": flops / (ev_mean * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                         "frac": flops / (ev_mean * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": None, "kernel": kernel,
+                         "frac": flops / (ev_mean * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": PREFILL_LONG_TRAFFIC_BYTES,
+                         "traffic_source": TRAFFIC_SOURCE["prefill_long"], "kernel": kernel,
                          "algorithmic_flops_per_launch": flops, "launch_ms_mean": ev_mean, "launch_ms_median": ev_med,
                          "launch_ms_min": ev_min},
             "ms_per_step_with_padding_rows_computed": wall_all_rows,
@@ -360,6 +430,7 @@ def main():
                "num_splits": w.splits,
                "roofline": {"bound": "hbm", "achieved": kv_bytes / (ev_mean * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                             "frac": kv_bytes / (ev_mean * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": DECODE_TRAFFIC_BYTES,
+                            "traffic_source": TRAFFIC_SOURCE["decode"],
                             "kernel": "sdpa_decode_split_kernel<bf16,128,1,8> + sdpa_combine_kernel",
                             "algorithmic_bytes_per_launch": kv_bytes,
                             "launch_ms_mean": ev_mean, "launch_ms_median": ev_med, "launch_ms_min": ev_min},
@@ -372,6 +443,9 @@ def main():
                                    "sample": "all of config 4 (B=32, H=32, KV=8192, D=128), oracle's materialising restatement of "
                                              "the reference CPU op (serial matmuls and reductions); %.1f s; host: %s" % (dt, host_cpu())}
         result["decode"] = dec
+
+    if args.only in (None, "f32"):
+        result.update(f32_configs(args.steps, args.warmup, not args.no_cpu_baseline, threads))
 
     if args.only in (None, "backward"):
         result["backward"] = backward_config3(max(5, min(args.steps, 30)), min(args.warmup, 5))

@@ -21,6 +21,7 @@ hipError_t launch_sdpa_generic(const SdpaParams& p, int dtype, hipStream_t strea
 hipError_t launch_sdpa_prefill_mfma(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_sdpa_prefill_mfma64(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_sdpa_prefill_f32(const SdpaParams& p, hipStream_t stream);
+hipError_t launch_mask_classify(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_sdpa_decode(const SdpaParams& p, int dtype, hipStream_t stream);
 int decode_keys_per_tile(int dtype, int D, int R);
 }  // namespace incin_rocm
@@ -189,6 +190,13 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         plan->ws_bytes = splits > 1 ? (size_t)(d->B * d->Hq * d->Sq * splits) * (size_t)(d->Dv + 2) * sizeof(float) : 0;
     }
     if (impl == INCIN_ROCM_IMPL_MFMA64) plan->ws_bytes = MFMA64_WS_BYTES;      // the launch's work counters
+    if (impl == INCIN_ROCM_IMPL_MFMA && d->add_mask) {
+        // one flag per block of 32 query rows x 32 keys of the mask, per mask batch entry and head
+        const int64_t nbh = (d->mask_stride[0] ? d->B : 1) * (d->mask_stride[1] ? d->Hq : 1);
+        if (nbh > 65535 || (d->Sq + 31) / 32 > 65535)
+            return fail(INCIN_ROCM_ESHAPE, "scaled_dot_product_attention: mask too large for one launch of the matrix-core kernels");
+        plan->ws_bytes = (size_t)(nbh * ((d->Sq + 31) / 32) * ((d->Skv + 31) / 32) + 255) / 256 * 256;
+    }
     return 0;
 }
 
@@ -214,6 +222,7 @@ void fill_params(const incin_rocm_sdpa_desc_t* d, const Plan& plan, SdpaParams* 
     p->num_splits = plan.splits;
     p->split_len = plan.split_len;
     if (plan.impl == INCIN_ROCM_IMPL_MFMA64) p->sched = (int32_t*)d->workspace;
+    else if (plan.impl == INCIN_ROCM_IMPL_MFMA) p->mask_flags = d->add_mask ? (const uint8_t*)d->workspace : nullptr;
     else p->ws_acc = (float*)d->workspace;
     if (plan.splits > 1) {
         const size_t rows = (size_t)(d->B * d->Hq * d->Sq * plan.splits);
@@ -491,7 +500,8 @@ static int launch_fwd(const incin_rocm_sdpa_desc_t* desc, const Plan& plan, void
         if (!desc->workspace || desc->workspace_bytes < plan.ws_bytes)
             return fail(INCIN_ROCM_EWORKSPACE,
                         "scaled_dot_product_attention: %s needs %zu workspace bytes, %zu given",
-                        plan.impl == INCIN_ROCM_IMPL_MFMA64 ? "the 64-row MFMA kernel" : "split-KV", plan.ws_bytes,
+                        plan.impl == INCIN_ROCM_IMPL_MFMA64 ? "the 64-row MFMA kernel" : plan.impl == INCIN_ROCM_IMPL_MFMA ? "a dense mask on the MFMA kernels" : "split-KV",
+                        plan.ws_bytes,
                         desc->workspace ? desc->workspace_bytes : (size_t)0);
         if (!aligned16(desc->workspace)) return fail(INCIN_ROCM_EWORKSPACE, "scaled_dot_product_attention: workspace must be 16-byte aligned");
     }
@@ -502,6 +512,10 @@ static int launch_fwd(const incin_rocm_sdpa_desc_t* desc, const Plan& plan, void
     hipError_t e;
     switch (plan.impl) {
         case INCIN_ROCM_IMPL_MFMA:
+            if (p.mask) {           // block flags of the mask first, on the same stream
+                e = incin_rocm::launch_mask_classify(p, desc->dtype, s);
+                if (e != hipSuccess) break;
+            }
             e = desc->dtype == INCIN_ROCM_F32 ? incin_rocm::launch_sdpa_prefill_f32(p, s) : incin_rocm::launch_sdpa_prefill_mfma(p, desc->dtype, s);
             break;
         case INCIN_ROCM_IMPL_MFMA64: e = incin_rocm::launch_sdpa_prefill_mfma64(p, desc->dtype, s); break;

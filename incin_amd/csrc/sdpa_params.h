@@ -31,6 +31,10 @@ struct SdpaParams {
     int32_t split_len;         // keys per split (multiple of the kernel's key tile)
     float* ws_acc;             // [B, Hq, Sq, num_splits, Dv] f32 partial numerators
     float* ws_ml;              // [B, Hq, Sq, num_splits, 2]  running max (natural-log domain) and denominator
+    // matrix-core prefill kernels with a dense mask: one byte per block of 32 query rows x 32 keys (0 mixed, 1 all zero,
+    // 2 all -inf), written by mask_classify_kernel ahead of the attention kernel, in the caller's workspace;
+    // [mask batch entries][mask heads][ceil(Sq / 32)][ceil(Skv / 32)], an extent of 1 where the mask is broadcast
+    const uint8_t* mask_flags;
     // 64-row MFMA prefill kernel only
     int32_t* sched;            // 16 work counters of this launch's persistent workgroups (in the caller's workspace; the
                                // launcher clears them with a one-workgroup kernel ahead of the attention kernel)
@@ -47,5 +51,14 @@ template <typename T> __device__ __forceinline__ T from_f32(float x) { return (T
 __device__ __forceinline__ int causal_limit(int i, int Sq, int Skv) { return i + (Skv - Sq) + 1; }
 
 __device__ __forceinline__ int clampi(int x, int lo, int hi) { return x < lo ? lo : (x > hi ? hi : x); }
+
+// Where the block flags of (batch b, query head hq) start, and the flags per row of blocks.
+__device__ __forceinline__ const uint8_t* mask_flags_of(const SdpaParams& p, int b, int hq)
+{
+    const int nkb = (p.Skv + 31) / 32, nrb = (p.Sq + 31) / 32;
+    const int Hm = p.m_sh ? p.Hq : 1;
+    const int64_t bh = (int64_t)(p.m_sb ? b : 0) * Hm + (p.m_sh ? hq : 0);
+    return p.mask_flags + bh * nrb * nkb;
+}
 
 }  // namespace incin_rocm

@@ -20,6 +20,9 @@
 //   O^T += V^T P^T     A = V^T: lane (d = lane % 32, g) supplies V[kappa(r, g)][32 db + d]: a 4-byte LDS read of
 //                      32 consecutive floats of one row per half-wavefront; no transposition anywhere.
 //
+// A dense additive mask comes with one flag per block of 32 rows x 32 keys (mask_blocks.hip): blocks the mask hides
+// completely are skipped, blocks where it is zero run without it, the rest add its values to the scores.
+//
 // The matrix pipe is the bound by a wide margin (an instruction occupies it for 64 cycles and needs one register of
 // each operand), so the loop is plain: per key tile one barrier, the global -> LDS copies of the next tile (K and V,
 // two buffers each, 16 KiB tiles: 64 keys at D = 64, 32 at D = 128), scores, exact online softmax, second product.
@@ -153,7 +156,11 @@ void sdpa_prefill_f32_kernel(SdpaParams p)
         }
     }
     const float* mrow = nullptr;          // this lane's row of the dense mask
-    if (DENSE) mrow = (const float*)p.mask + (int64_t)b * p.m_sb + (int64_t)hq * p.m_sh + (int64_t)min(my_i, Sq - 1) * p.m_si;
+    const uint8_t* mflags = nullptr;      // block flags of this wavefront's 32 rows: 0 mixed, 1 all zero, 2 all -inf
+    if (DENSE) {
+        mrow = (const float*)p.mask + (int64_t)b * p.m_sb + (int64_t)hq * p.m_sh + (int64_t)min(my_i, Sq - 1) * p.m_si;
+        mflags = mask_flags_of(p, b, hq) + (int64_t)((q0 >> 5) + wave) * ((Skv + 31) / 32);
+    }
 
     floatx16 o_acc[NDB];
 #pragma unroll
@@ -176,9 +183,14 @@ void sdpa_prefill_f32_kernel(SdpaParams p)
         for (int kb = 0; kb < NB; ++kb) {
             const int j0 = t * KT + kb * 32;
             if (j0 >= lim_wave_max) break;                    // (uniform) nothing of this block is visible to the wavefront
+            int flag = 1;
+            if (DENSE) {
+                flag = __builtin_amdgcn_readfirstlane((int)mflags[j0 >> 5]);
+                if (flag == 2) continue;                      // the mask hides the whole block from these rows
+            }
             // dense mask values of this lane's 16 keys, fetched ahead of the product that hides their latency
             float mv[16];
-            if (DENSE) {
+            if (DENSE && flag == 0) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int j = min(j0 + 8 * (r / 4) + 4 * g + (r % 4), Skv - 1);
@@ -202,7 +214,7 @@ void sdpa_prefill_f32_kernel(SdpaParams p)
             floatx16 s;
 #pragma unroll
             for (int r = 0; r < 16; ++r) s[r] = s0[r] + s1[r];
-            if (DENSE) {
+            if (DENSE && flag == 0) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) s[r] = __builtin_fmaf(mv[r], 1.4426950408889634f, s[r]);
             }

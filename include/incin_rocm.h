@@ -195,9 +195,11 @@ int incin_rocm_sdpa_workspace(const incin_rocm_sdpa_desc_t* desc, size_t* bytes,
  * stream-ordered use of the buffers named in the descriptor, which the caller
  * keeps alive until the stream has been synchronised.
  *
- * Workspace.  Two kernels need scratch memory, of the size incin_rocm_sdpa_workspace reports: the split-KV
- * kernel (partial results of the splits) and the 64-row MFMA prefill kernel (256 bytes: the work counters its
- * persistent workgroups draw from, cleared by the launch itself).  The contents need not survive the launch and
+ * Workspace.  Three launches need scratch memory, of the size incin_rocm_sdpa_workspace reports: the split-KV
+ * kernel (partial results of the splits), the 64-row MFMA prefill kernel (256 bytes: the work counters its
+ * persistent workgroups draw from, cleared by the launch itself) and the MFMA prefill kernels with a dense mask
+ * (one byte per block of 32 query rows x 32 keys of the mask: which blocks it hides, which it leaves alone;
+ * written by a small kernel of the same launch).  The contents need not survive the launch and
  * need no initialisation, but two launches that may run at the same time - other streams, other host threads, a
  * recorded graph replayed beside eager launches - must not be given the same workspace: they would draw from
  * each other's counters or overwrite each other's partial results.  A recorded launch keeps using the workspace
