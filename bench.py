@@ -32,15 +32,15 @@ PEAK_F32_TFLOPS = 157.3      # dense fp32 matrix peak, vendor figure (256 CUs x 
 PEAK_HBM_GBS = 8000.0       # HBM3E, vendor figure
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same command (KiB per dispatch,
 # FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0 after calibration against the 1 GiB copy kernel): profiles/*.txt
-PREFILL_TRAFFIC_BYTES = (209881 * 2.0 + 131113) * 1024     # 5.64e8: |Q|+|K|+|V| read 1.07 times, |O| written once
+PREFILL_TRAFFIC_BYTES = (287112 * 2.0 + 131169) * 1024     # 7.22e8: |Q|+|K|+|V| read 1.46 times (1.07 on another box), |O| written once
 DECODE_TRAFFIC_BYTES = (2097470 * 2.0 + 1088 + 256) * 1024  # 4.297e9: K and V read once + split partials
-PREFILL_LONG_TRAFFIC_BYTES = None                           # filled from its counter run below when one exists
+PREFILL_LONG_TRAFFIC_BYTES = (600683 * 2.0 + 319192) * 1024    # 1.56e9: valid |O| written once, inputs read 2.5 times
 # These three are constants taken from counter runs, not measured by this script: each roofline object says so and
 # names the summary the figures come from.
 TRAFFIC_SOURCE = {
     "prefill": "constant from profiles/sdpa_prefill_mfma_bf16_d128_config3.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of `bench.py --only prefill`)",
     "decode": "constant from profiles/sdpa_decode_splitkv_bf16_d128_config4.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of `bench.py --only decode`)",
-    "prefill_long": "profiles/sdpa_prefill_mfma64_bf16_d128_config5.txt",
+    "prefill_long": "constant from profiles/sdpa_prefill_mfma64_bf16_d128_config5.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of `bench.py --only prefill_long --no-padding-compare`)",
 }
 METRIC = "attn fwd TFLOP/s + % bf16 MFMA peak; decode KV GB/s + % HBM peak (1 GPU)"
 
@@ -379,6 +379,24 @@ def main():
                               "traffic_source": TRAFFIC_SOURCE["prefill"], "kernel": "sdpa_prefill_mfma_kernel<bf16,128>", "algorithmic_flops_per_launch": flops,
                               "launch_ms_mean": ev_mean, "launch_ms_median": ev_med, "launch_ms_min": ev_min}
         result["parity_max_abs_err"] = w.parity()
+        if args.only is None:
+            # the same batch with the causal mask handed over the way the reference's operator takes it: an explicit
+            # [S, S] tensor of 0 / -inf (bf16, broadcast over batch and heads) instead of the causal flag
+            from oracle import oracle as O
+            tm = capi.DeviceBuffer.from_numpy(dtypes.encode(O.causal_additive_mask(S, S), capi.BF16))
+            w.desc.causal = 0
+            w.desc.add_mask = tm.ptr
+            for i, st in enumerate((0, 0, S, 1)):
+                w.desc.mask_stride[i] = st
+            mws = capi.DeviceBuffer(capi.sdpa_workspace(w.desc)[0])
+            w.desc.workspace, w.desc.workspace_bytes = mws.ptr, mws.nbytes
+            wall_m = w.time(args.steps, args.warmup)[0]
+            result["prefill_with_dense_mask_tensor"] = {
+                "what": "config 3 with the causal mask passed as a bf16 [S, S] additive tensor (add_mask); the launch classifies it "
+                        "by 32 x 32 blocks first; same FLOP count", "ms_per_step": wall_m, "value": flops / (wall_m * 1e-3) / 1e12,
+                "unit": "TFLOP/s", "ratio_to_causal_flag": wall / wall_m, "parity_max_abs_err": w.parity()}
+            tm.free()
+            mws.free()
         w.free()
         if not args.no_cpu_baseline:
             slices = 12

@@ -129,12 +129,11 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     // the MFMA kernels address a K/V tile with 32-bit byte offsets from the tile's first row
     const int64_t stride_lim = d->dtype == INCIN_ROCM_F32 ? (1 << 22) : (1 << 24);
     const bool tile_off_ok = d->k_stride[2] >= 0 && d->v_stride[2] >= 0 && d->k_stride[2] < stride_lim && d->v_stride[2] < stride_lim;
-    // f32: the IEEE-f32 matrix-core kernel, which also takes a dense additive mask and any finite scale;
-    // f16 / bf16: the 16-bit kernels fold the scale into Q in a way that needs it positive, and take no dense mask
-    const bool mfma_ok = d->dtype == INCIN_ROCM_F32 ? (layout_ok && tile_off_ok && std::isfinite(d->scale))
-                                                    : (fast_ok && tile_off_ok && d->scale > 0.0f && std::isfinite(d->scale));
+    // f32: the IEEE-f32 matrix-core kernel, any finite scale; f16 / bf16: the 16-bit kernels fold the scale into Q in
+    // a way that needs it positive.  Both take a dense additive mask (any strides); the 64-row kernel does not.
+    const bool mfma_ok = layout_ok && tile_off_ok && std::isfinite(d->scale) && (d->dtype == INCIN_ROCM_F32 || d->scale > 0.0f);
     // the 64-row kernel does its byte arithmetic on a head's K and V in 32 bits, up to 16 tiles of 32 rows past the end
-    const bool mfma64_ok = mfma_ok && d->dtype != INCIN_ROCM_F32 && d->D == 128 && (d->Skv + 512) * d->k_stride[2] * 2 < (1LL << 31) &&
+    const bool mfma64_ok = mfma_ok && !d->add_mask && d->dtype != INCIN_ROCM_F32 && d->D == 128 && (d->Skv + 512) * d->k_stride[2] * 2 < (1LL << 31) &&
                            (d->Skv + 512) * d->v_stride[2] * 2 < (1LL << 31);
     const bool split_ok = fast_ok && d->Sq <= 64;
 
@@ -152,10 +151,10 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     }
     if (impl == INCIN_ROCM_IMPL_MFMA && !mfma_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
-                    "scaled_dot_product_attention: the MFMA kernels need D == Dv in {64,128} and 16-byte aligned rows; for f16/bf16 also scale > 0 and no dense mask");
+                    "scaled_dot_product_attention: the MFMA kernels need D == Dv in {64,128} and 16-byte aligned rows; for f16/bf16 also scale > 0");
     if (impl == INCIN_ROCM_IMPL_MFMA64 && !mfma64_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
-                    "scaled_dot_product_attention: the 64-row MFMA kernel needs what the MFMA kernel needs, D == Dv == 128 and key/value slices below 2 GiB");
+                    "scaled_dot_product_attention: the 64-row MFMA kernel needs f16/bf16, what the MFMA kernel needs, D == Dv == 128, no dense mask and key/value slices below 2 GiB");
     if (impl == INCIN_ROCM_IMPL_SPLITKV && d->lse)
         return fail(INCIN_ROCM_EUNSUPPORTED, "scaled_dot_product_attention: the split-KV kernel does not write the row normalisers (lse)");
     if (impl == INCIN_ROCM_IMPL_SPLITKV && !split_ok)
@@ -213,6 +212,8 @@ void fill_params(const incin_rocm_sdpa_desc_t* d, const Plan& plan, SdpaParams* 
     p->v_sb = d->v_stride[0]; p->v_sh = d->v_stride[1]; p->v_ss = d->v_stride[2];
     p->o_sb = d->o_stride[0]; p->o_sh = d->o_stride[1]; p->o_ss = d->o_stride[2];
     p->m_sb = d->mask_stride[0]; p->m_sh = d->mask_stride[1]; p->m_si = d->mask_stride[2]; p->m_sj = d->mask_stride[3];
+    p->mask_vec = d->add_mask && d->mask_stride[3] == 1 && (reinterpret_cast<uintptr_t>(d->add_mask) & 7u) == 0 &&
+                  d->mask_stride[0] % 4 == 0 && d->mask_stride[1] % 4 == 0 && d->mask_stride[2] % 4 == 0;
     p->B = (int)d->B; p->Hq = (int)d->Hq; p->Hkv = (int)d->Hkv; p->G = (int)(d->Hq / d->Hkv);
     p->Sq = (int)d->Sq; p->Skv = (int)d->Skv; p->D = (int)d->D; p->Dv = (int)d->Dv;
     p->scale = d->scale;

@@ -63,7 +63,7 @@ namespace incin_rocm {
 #define PF_VD 4     // V operand reads run this many MFMAs ahead
 #endif
 
-template <typename T, int D>
+template <typename T, int D, bool DENSE>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void sdpa_prefill_mfma_kernel(SdpaParams p)
 {
@@ -116,7 +116,40 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
         lim_wave_max = clampi(min(q0 + wave * 32 + 31, rows_b - 1) + coff + 1, 0, kv_len);
     }
     if (q0 + wave * 32 >= rows_b) lim_wave_min = lim_wave_max = 0;      // a wavefront of padding rows only keeps the barriers company
-    const int n_tiles = (j_end + PF_BN - 1) / PF_BN;
+    int n_tiles = (j_end + PF_BN - 1) / PF_BN;
+    // ---- dense additive mask: what its block flags say about this workgroup's rows ---------------------------------
+    // mflags: one byte per 32-key block for this wavefront's 32 rows (0 mixed, 1 all zero, 2 all -inf).  Tiles before
+    // the first and after the last one in which some wavefront has a visible block are never copied; in between, a
+    // wavefront skips the tiles hidden from its own rows.
+    const uint8_t* mflags = nullptr;
+    const T* mrow = nullptr;
+    const int nkb32 = (Skv + 31) >> 5;
+    int t_first = 0;
+    [[maybe_unused]] int w_first = 0, w_last = 0x7fffffff;      // this wavefront's first and last tile with a visible block
+    __shared__ int s_range[8];
+    if (DENSE) {
+        mflags = mask_flags_of(p, b, hq) + (int64_t)((q0 >> 5) + wave) * nkb32;
+        mrow = (const T*)p.mask + (int64_t)b * p.m_sb + (int64_t)hq * p.m_sh + (int64_t)min(my_i, Sq - 1) * p.m_si;
+        int lo = 0x7fffffff, hi = -1;
+        if (q0 + wave * 32 < rows_b)
+            for (int t = lane; t < n_tiles; t += 64) {
+                const int f0 = mflags[2 * t], f1 = 2 * t + 1 < nkb32 ? mflags[2 * t + 1] : 2;
+                if (f0 != 2 || f1 != 2) { lo = min(lo, t); hi = max(hi, t); }
+            }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            lo = min(lo, __shfl_xor(lo, off, 64));
+            hi = max(hi, __shfl_xor(hi, off, 64));
+        }
+        w_first = lo;
+        w_last = hi;
+        if (lane == 0) { s_range[wave] = lo; s_range[4 + wave] = hi; }
+        __syncthreads();
+        const int g_lo = min(min(s_range[0], s_range[1]), min(s_range[2], s_range[3]));
+        const int g_hi = max(max(s_range[4], s_range[5]), max(s_range[6], s_range[7]));
+        t_first = g_hi < 0 ? 0 : g_lo;
+        n_tiles = g_hi + 1;                           // (0 when the mask hides everything from these 128 rows)
+    }
 
     // ---- global -> LDS copy plan ---------------------------------------------------
     // wavefront-wide load number ii = wave*LPW + c fills LDS bytes [ii*1024, ii*1024 + 1024)
@@ -352,6 +385,35 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
         tmax = xor32_max(fmaxf(m0, m1));
     };
 
+    // Dense mask on the scores of the tile that starts at key j0 (scores are in log2 units): per 32-key half, nothing
+    // where the flag says zeros, -inf where it says hidden, else the values themselves - 4 consecutive keys per load
+    // where the mask's layout allows (unit key stride, 8-byte aligned rows), element by element otherwise.
+    auto add_dense_mask = [&](floatx16 (&sx)[2], int j0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            const int blk = (j0 >> 5) + kb;
+            const int flag = blk < nkb32 ? __builtin_amdgcn_readfirstlane((int)mflags[blk]) : 2;
+            if (flag == 1) continue;
+            if (flag == 2) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sx[kb][r] = -INFINITY;
+                continue;
+            }
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                const int j = j0 + 32 * kb + 8 * r4 + 4 * g;
+                typedef T vec4 __attribute__((ext_vector_type(4)));
+                vec4 mv;
+                if (p.mask_vec && j + 3 < Skv) mv = *(const vec4*)(mrow + j);
+                else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) mv[e] = mrow[(int64_t)min(j + e, Skv - 1) * p.m_sj];
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) sx[kb][4 * r4 + e] = __builtin_fmaf((float)mv[e], 1.4426950408889634f, sx[kb][4 * r4 + e]);
+            }
+        }
+    };
     // scores of one tile without overlap (prologue and the last tiles of a wavefront); kb = K tile in LDS
     auto scores_plain = [&](const char* kb, floatx16 (&sx)[2], int j0) __attribute__((always_inline)) {
 #pragma unroll
@@ -362,6 +424,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
             for (int b2 = 0; b2 < 2; ++b2) sx[b2] = Mma<T>::run(kbuf[s % KD][b2], qreg[s], s == 0 ? neg_ref : sx[b2]);
             if (s + KD < NSTEP) read_k(kb, s + KD);
         }
+        if (DENSE) add_dense_mask(sx, j0);
         if (j0 + PF_BN > lim_wave_min) mask_tile(sx, j0);
         tmax = max_of(sx);
     };
@@ -370,7 +433,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     const int n_act = lim_wave_max > 0 ? (lim_wave_max + PF_BN - 1) / PF_BN : 0;
     const int n_hot = lim_wave_min > 0 ? min(lim_wave_min / PF_BN, n_act) : 0;      // tiles 0..n_hot-1 need no mask
 
-    if (n_tiles > 0) {
+    if (!DENSE && n_tiles > 0) {
         // prologue: K(0) first, then K(1), V(0) in flight; scores of tile 0
         issue_k(0, 0);
         __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0), told to the compiler too: it then knows the Q rows have arrived
@@ -405,6 +468,44 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
             }
         }
     }
+    if (DENSE && n_tiles > t_first) {
+        // The same one-tile-at-a-time loop over the tiles t_first .. n_tiles - 1 the mask leaves to this workgroup; a
+        // wavefront computes tile t if its limits (causal, key count) and the mask's flags leave it a visible block.
+        auto mine = [&](int t) __attribute__((always_inline)) {
+            if (t >= n_act || t < w_first || t > w_last) return false;
+            const int f0 = __builtin_amdgcn_readfirstlane((int)mflags[2 * t]);
+            const int f1 = 2 * t + 1 < nkb32 ? __builtin_amdgcn_readfirstlane((int)mflags[2 * t + 1]) : 2;
+            return f0 != 2 || f1 != 2;
+        };
+        issue_k(t_first, t_first & 1);
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        asm volatile("" ::: "memory");
+        __syncthreads();
+        if (t_first + 1 < n_tiles) issue_k(t_first + 1, (t_first + 1) & 1);
+        issue_v(t_first, t_first & 1);
+        bool pending = mine(t_first);
+        if (pending) scores_plain(smem + (t_first & 1) * L::TILE_BYTES, sacc[0], t_first * PF_BN);
+        for (int t = t_first; t < n_tiles; ++t) {
+            turn(t);
+            if (pending) {
+                const char* v_cur = smem + (2 + (t & 1)) * L::TILE_BYTES;
+#pragma unroll
+                for (int i = 0; i < VD; ++i) read_v(v_cur, i);
+                adjust_reference(sacc[0]);
+                rsum = 0.0f;
+#pragma unroll
+                for (int sl = 0; sl < 8; ++sl) softmax_slice(sacc[0], sl);
+                l_run += rsum;
+#pragma unroll
+                for (int i = 0; i < NPV; ++i) {
+                    o_acc[i % NDB] = Mma<T>::run(vbuf[i % VD], pb[i / NDB], o_acc[i % NDB]);
+                    if (i + VD < NPV) read_v(v_cur, i + VD);
+                }
+            }
+            pending = t + 1 < n_tiles && mine(t + 1);
+            if (pending) scores_plain(smem + ((t + 1) & 1) * L::TILE_BYTES, sacc[0], (t + 1) * PF_BN);
+        }
+    }
 #undef SGB
 
     // ---- normalise and store ------------------------------------------------------------------
@@ -428,7 +529,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
 #endif
 }
 
-template <typename T, int D>
+template <typename T, int D, bool DENSE>
 static hipError_t launch_prefill_t(const SdpaParams& p0, hipStream_t stream)
 {
     SdpaParams p = p0;
@@ -437,17 +538,20 @@ static hipError_t launch_prefill_t(const SdpaParams& p0, hipStream_t stream)
     // two workgroups per CU (register budget), an eighth of the CUs per XCD
     p.interleave = work_interleave(p.causal != 0, 2 * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
     p.deal_groups = (total & 7) == 0 ? work_deal(p.interleave, p.G, nqb, total >> 3) : 0;
-    hipLaunchKernelGGL((sdpa_prefill_mfma_kernel<T, D>), dim3((unsigned)total), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((sdpa_prefill_mfma_kernel<T, D, DENSE>), dim3((unsigned)total), dim3(256), 0, stream, p);
     return hipGetLastError();
 }
 
-// Host has validated: dtype f16/bf16, D == Dv in {64,128}, scale > 0, no dense
-// mask, rows 16-byte aligned with unit last-dim stride, row strides below 2^24
+// Host has validated: dtype f16/bf16, D == Dv in {64,128}, scale > 0, rows 16-byte aligned with unit last-dim stride, row strides below 2^24
 // elements (tile offsets fit the 32-bit buffer offset).
 hipError_t launch_sdpa_prefill_mfma(const SdpaParams& p, int dtype, hipStream_t stream)
 {
-    if (dtype == 1) return p.D == 128 ? launch_prefill_t<f16_t, 128>(p, stream) : launch_prefill_t<f16_t, 64>(p, stream);
-    return p.D == 128 ? launch_prefill_t<bf16_t, 128>(p, stream) : launch_prefill_t<bf16_t, 64>(p, stream);
+    if (p.mask) {
+        if (dtype == 1) return p.D == 128 ? launch_prefill_t<f16_t, 128, true>(p, stream) : launch_prefill_t<f16_t, 64, true>(p, stream);
+        return p.D == 128 ? launch_prefill_t<bf16_t, 128, true>(p, stream) : launch_prefill_t<bf16_t, 64, true>(p, stream);
+    }
+    if (dtype == 1) return p.D == 128 ? launch_prefill_t<f16_t, 128, false>(p, stream) : launch_prefill_t<f16_t, 64, false>(p, stream);
+    return p.D == 128 ? launch_prefill_t<bf16_t, 128, false>(p, stream) : launch_prefill_t<bf16_t, 64, false>(p, stream);
 }
 
 }  // namespace incin_rocm

@@ -60,7 +60,9 @@ def test_dispatch_choices():
     assert _plan(_desc(dtype=capi.F32, add_mask=0x20000))[2] == capi.IMPL_MFMA  # which also takes a dense mask
     assert _plan(_desc(dtype=capi.F32, D=80, Dv=80))[2] == capi.IMPL_GENERIC
     assert _plan(_desc(D=80, Dv=80))[2] == capi.IMPL_GENERIC
-    assert _plan(_desc(add_mask=0x20000))[2] == capi.IMPL_GENERIC
+    nbytes, _, impl = _plan(_desc(add_mask=0x20000))                            # dense mask: still the matrix cores,
+    assert impl == capi.IMPL_MFMA and nbytes == 256                           # with 2 x 4 x 4 x 4 block flags (rounded up)
+    assert _plan(_desc(add_mask=0x20000, D=80, Dv=80))[2] == capi.IMPL_GENERIC
     nbytes, splits, impl = _plan(_desc(Sq=1, Skv=8192, B=32, Hq=32, Hkv=32))
     assert impl == capi.IMPL_SPLITKV and splits >= 1
     assert nbytes == (0 if splits == 1 else 32 * 32 * 1 * splits * (128 + 2) * 4)
@@ -94,7 +96,7 @@ def test_dispatch_choices():
     (dict(impl=9), capi.EINVAL),
     (dict(num_splits=-2), capi.EINVAL),
     (dict(impl=capi.IMPL_MFMA64, dtype=capi.F32), capi.EUNSUPPORTED),
-    (dict(impl=capi.IMPL_MFMA, add_mask=0x20000), capi.EUNSUPPORTED),
+    (dict(impl=capi.IMPL_MFMA64, add_mask=0x20000), capi.EUNSUPPORTED),
     (dict(impl=capi.IMPL_MFMA, D=80, Dv=80), capi.EUNSUPPORTED),
     (dict(impl=capi.IMPL_SPLITKV, Sq=4096), capi.EUNSUPPORTED),
     (dict(D=512, Dv=512), capi.EUNSUPPORTED),

@@ -255,6 +255,52 @@ def test_f32_matrix_core_prefill(gpu, shape):
     assert not fin.any() or np.abs(lse[fin] - lse_g[fin]).max() <= 1e-5
 
 
+@pytest.mark.parametrize("dtype", [capi.BF16, capi.F16])
+@pytest.mark.parametrize("shape", [
+    # B, Hq, Hkv, Sq, Skv, D
+    (2, 4, 2, 70, 90, 128),            # the shapes of the generic-kernel mask test, at the matrix-core head dimensions
+    (1, 2, 2, 300, 333, 128),          # key count not a multiple of 4: element-wise mask loads
+    (2, 4, 4, 512, 512, 64),
+    (1, 2, 1, 1000, 1000, 128),
+    (1, 1, 1, 17, 64, 64),
+])
+def test_mfma_prefill_dense_masks(gpu, dtype, shape):
+    """A dense additive mask keeps a 16-bit request on the matrix-core kernel: random masks of every broadcast shape
+    (values, -inf entries), the causal mask as the tensor full(-inf).triu(1) a caller of the reference builds (equal to
+    the causal flag bit for bit where whole blocks are hidden or zero), a banded mask (hidden blocks on both sides),
+    masks combined with the causal flag and key counts, and a fully masked row."""
+    B, Hq, Hkv, Sq, Skv, D = shape
+    G = Hq // Hkv
+    q, k, v = inputs(500 + sum(shape), B, Hq, Hkv, Sq, Skv, D, D, dtype)
+    r = rng(sum(shape))
+    for mshape in [(Sq, Skv), (1, Skv), (B, 1, Sq, Skv), (B, Hq, Sq, Skv), (1, Hq, 1, Skv)]:
+        m = dtypes.round_to(r.standard_normal(mshape, dtype=np.float32), dtype)
+        m = np.where(r.random(mshape) < 0.25, -np.inf, m).astype(np.float32)
+        m[..., 0] = 0.0                                             # keep every row alive
+        got, info = host.sdpa(q, k, v, dtype, mask=m, scale=0.3 / np.sqrt(D / 32), return_info=True)
+        assert info["impl"] == capi.IMPL_MFMA and info["workspace_bytes"] > 0
+        check(got, oracle_full(q, k, v, G=G, mask=m, scale=0.3 / np.sqrt(D / 32)), TOL[dtype], "mfma %s %r mask %r" % (dtypes.NAMES[dtype], shape, mshape))
+    cm = O.causal_additive_mask(Sq, Skv)
+    got, info = host.sdpa(q, k, v, dtype, mask=cm, return_info=True)
+    assert info["impl"] == capi.IMPL_MFMA
+    check(got, oracle_full(q, k, v, G=G, causal=True), TOL[dtype], "mfma causal mask as a tensor")
+    flagged = host.sdpa(q, k, v, dtype, causal=True, impl=capi.IMPL_MFMA)
+    check(got, flagged, 8e-3, "causal tensor vs causal flag")
+    band = np.where(np.abs(np.arange(Sq)[:, None] + (Skv - Sq) - np.arange(Skv)[None, :]) <= 100, 0.0, -np.inf).astype(np.float32)
+    got = host.sdpa(q, k, v, dtype, mask=band)
+    check(got, oracle_full(q, k, v, G=G, mask=band), TOL[dtype], "mfma banded mask")
+    lens = r.integers(1, Skv + 1, B).astype(np.int32)
+    m = dtypes.round_to(r.standard_normal((Sq, Skv), dtype=np.float32), dtype)
+    got = host.sdpa(q, k, v, dtype, mask=m, causal=True, kv_lens=lens)
+    full = np.broadcast_to(m, (B, Hq, Sq, Skv)) + cm + np.where(np.arange(Skv)[None, :] < lens[:, None], 0.0, -np.inf).astype(np.float32)[:, None, None, :]
+    check(got, oracle_full(q, k, v, G=G, mask=full), TOL[dtype], "mfma mask + causal flag + kv_lens")
+    m = np.zeros((Sq, Skv), np.float32)
+    m[Sq // 2, :] = -np.inf
+    check(host.sdpa(q, k, v, dtype, mask=m), oracle_full(q, k, v, G=G, mask=m), TOL[dtype], "mfma fully masked row")
+    hidden = np.full((Sq, Skv), -np.inf, np.float32)                # the mask hides everything: NaN everywhere, as the reference
+    assert np.isnan(host.sdpa(q, k, v, dtype, mask=hidden)).all()
+
+
 @pytest.mark.parametrize("impl", MFMA_IMPLS)
 def test_mfma_prefill_ragged_lengths(gpu, impl):
     B, Hq, Hkv, S, D = 3, 8, 2, 640, 128
