@@ -270,14 +270,16 @@ def f32_configs(steps, warmup, with_cpu, threads):
     from oracle import oracle as O
     out = {}
     for key, (B, H, S, D, causal, scale_note) in (("f32_c1", (1, 1, 128, 64, False, "scale=0.125")),
-                                                  ("f32_c2", (4, 8, 1024, 64, True, "scale=1/sqrt(64)"))):
-        w = Workload(key, SEED0 + (0 if key == "f32_c1" else 1), B, H, H, S, S, D, capi.F32, causal)
-        n = max(steps, 200)                                 # launches of tens of microseconds
+                                                  ("f32_c2", (4, 8, 1024, 64, True, "scale=1/sqrt(64)")),
+                                                  ("f32_large", (8, 16, 4096, 128, True, "scale=1/sqrt(128)"))):
+        w = Workload(key, SEED0 + {"f32_c1": 0, "f32_c2": 1, "f32_large": 7}[key], B, H, H, S, S, D, capi.F32, causal)
+        n = max(steps, 200) if key != "f32_large" else max(5, min(steps, 20))      # launches of tens of microseconds / of ~5 ms
         wall, ev_mean, ev_med, ev_min = w.time(n, warmup)
         flops = causal_flops(B, H, S, S, D) if causal else 4.0 * D * B * H * S * S
         kernel = {capi.IMPL_MFMA: "sdpa_prefill_f32_kernel<%d>" % D, capi.IMPL_GENERIC: "sdpa_generic_kernel<float>"}.get(w.impl, str(w.impl))
-        rec = {"workload": "BASELINE config %s: f32 %s attention fwd B=%d H=%d S_q=S_kv=%d D=%d, %s" %
-                           (key[-1], "causal" if causal else "non-causal", B, H, S, D, scale_note),
+        what = "BASELINE config %s" % key[-1] if key != "f32_large" else "not a BASELINE config (the shape of config 3 in f32: a launch that fills the machine)"
+        rec = {"workload": "%s: f32 %s attention fwd B=%d H=%d S_q=S_kv=%d D=%d, %s" %
+                           (what, "causal" if causal else "non-causal", B, H, S, D, scale_note),
                "metric": "attn fwd TFLOP/s", "value": flops / (wall * 1e-3) / 1e12, "unit": "TFLOP/s", "dtype": "f32",
                "ms_per_step": wall, "steps": n,
                "roofline": {"bound": "mfma", "achieved": flops / (ev_mean * 1e-3) / 1e12, "peak": PEAK_F32_TFLOPS, "unit": "TFLOP/s",
@@ -285,7 +287,7 @@ def f32_configs(steps, warmup, with_cpu, threads):
                             "algorithmic_flops_per_launch": flops, "launch_ms_mean": ev_mean, "launch_ms_median": ev_med,
                             "launch_ms_min": ev_min},
                "parity_max_abs_err": w.parity()}
-        if causal:
+        if key == "f32_c2":
             # the same problem with the mask as a tensor: the launch first classifies the tensor by blocks of 32 x 32 (hidden
             # blocks are skipped, zero blocks run unmasked), FLOPs counted as above
             mask = O.causal_additive_mask(S, S)

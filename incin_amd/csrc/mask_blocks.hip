@@ -5,36 +5,57 @@
 // The reference's operator knows one mask form, an additive tensor (crates/incin-backends/src/cpu/ops/shape_ops.rs:
 // 1262-1266), and its callers build the causal mask as full(-inf).triu(1): with the flags, such a tensor costs about
 // what the causal flag costs - blocks above the diagonal are skipped, blocks below it run the unmasked path.
-// One workgroup per block: 1024 elements, 4 per thread; rows beyond Sq and keys beyond Skv do not vote.
+// One workgroup per strip of 32 rows x 256 keys (8 blocks): a thread takes 8 consecutive keys of 4 rows - one 16-byte
+// load each for 16-bit masks with unit key stride and aligned rows, element-wise loads otherwise - and the votes of a
+// block meet in LDS; rows beyond Sq and keys beyond Skv do not vote.
 #include "sdpa_params.h"
 
 namespace incin_rocm {
 
-template <typename T>
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void mask_classify_kernel(const T* mask, int64_t m_sb, int64_t m_sh, int64_t m_si, int64_t m_sj,
-                                                           int Hm, int Sq, int Skv, uint8_t* flags)
+                                                           int Hm, int Sq, int Skv, int nkb, uint8_t* flags)
 {
-    const int kb = blockIdx.x, rb = blockIdx.y, bh = blockIdx.z;
+    __shared__ int votes[8][2];
+    const int strip = blockIdx.x, rb = blockIdx.y, bh = blockIdx.z;
     const int b = bh / Hm, h = bh % Hm;
     const T* base = mask + (int64_t)b * m_sb + (int64_t)h * m_sh;
-    const int c = threadIdx.x & 31, r0 = threadIdx.x >> 5;
-    const int j = kb * 32 + c;
+    const int c8 = threadIdx.x & 31, r0 = threadIdx.x >> 5;       // 8 keys starting at strip * 256 + c8 * 8; rows r0, r0 + 8, ..
+    if (threadIdx.x < 16) votes[threadIdx.x >> 1][threadIdx.x & 1] = 0;
+    __syncthreads();
+    const int j0 = strip * 256 + c8 * 8;
     int not_zero = 0, not_hidden = 0;
-    if (j < Skv) {
+    if (j0 < Skv) {
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int i = rb * 32 + r0 + 8 * u;
-            if (i < Sq) {
-                const float x = to_f32(base[(int64_t)i * m_si + (int64_t)j * m_sj]);
-                not_zero |= !(x == 0.0f);
-                not_hidden |= !(x == -INFINITY);
+            if (i >= Sq) continue;
+            const T* row = base + (int64_t)i * m_si;
+            if (VEC && j0 + 7 < Skv) {
+                typedef T vec8 __attribute__((ext_vector_type(8)));
+                const vec8 x = *(const vec8*)(row + j0);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float f = to_f32(x[e]);
+                    not_zero |= !(f == 0.0f);
+                    not_hidden |= !(f == -INFINITY);
+                }
+            } else {
+                for (int e = 0; e < 8 && j0 + e < Skv; ++e) {
+                    const float f = to_f32(row[(int64_t)(j0 + e) * m_sj]);
+                    not_zero |= !(f == 0.0f);
+                    not_hidden |= !(f == -INFINITY);
+                }
             }
         }
+        if (not_zero) atomicOr(&votes[c8 >> 2][0], 1);
+        if (not_hidden) atomicOr(&votes[c8 >> 2][1], 1);
     }
-    not_zero = __syncthreads_or(not_zero);
-    not_hidden = __syncthreads_or(not_hidden);
-    if (threadIdx.x == 0)
-        flags[((int64_t)bh * gridDim.y + rb) * gridDim.x + kb] = !not_zero ? 1 : (!not_hidden ? 2 : 0);
+    __syncthreads();
+    if (threadIdx.x < 8) {
+        const int kb = strip * 8 + threadIdx.x;
+        if (kb < nkb) flags[((int64_t)bh * gridDim.y + rb) * nkb + kb] = !votes[threadIdx.x][0] ? 1 : (!votes[threadIdx.x][1] ? 2 : 0);
+    }
 }
 
 // Host has validated the extents; nbh = mask batch entries x mask heads (1 where the mask is broadcast).
@@ -44,13 +65,18 @@ hipError_t launch_mask_classify(const SdpaParams& p, int dtype, hipStream_t stre
     const int Bm = p.m_sb ? p.B : 1, Hm = p.m_sh ? p.Hq : 1;
     if (nkb <= 0 || nrb <= 0) return hipSuccess;
     if (nrb > 65535 || (int64_t)Bm * Hm > 65535) return hipErrorInvalidValue;
-    const dim3 grid(nkb, nrb, Bm * Hm);
+    const dim3 grid((nkb + 7) / 8, nrb, Bm * Hm);
     uint8_t* flags = (uint8_t*)p.mask_flags;
+    const int esz = dtype == 0 ? 4 : 2;
+    // 8 consecutive elements in one vector load: unit key stride, every row start a multiple of the vector
+    const bool vec = p.m_sj == 1 && ((uintptr_t)p.mask % (8 * esz)) == 0 && p.m_sb % 8 == 0 && p.m_sh % 8 == 0 && p.m_si % 8 == 0;
+#define CLASSIFY(T, V) hipLaunchKernelGGL((mask_classify_kernel<T, V>), grid, dim3(256), 0, stream, (const T*)p.mask, p.m_sb, p.m_sh, p.m_si, p.m_sj, Hm, p.Sq, p.Skv, nkb, flags)
     switch (dtype) {
-        case 0: hipLaunchKernelGGL(mask_classify_kernel<float>, grid, dim3(256), 0, stream, (const float*)p.mask, p.m_sb, p.m_sh, p.m_si, p.m_sj, Hm, p.Sq, p.Skv, flags); break;
-        case 1: hipLaunchKernelGGL(mask_classify_kernel<f16_t>, grid, dim3(256), 0, stream, (const f16_t*)p.mask, p.m_sb, p.m_sh, p.m_si, p.m_sj, Hm, p.Sq, p.Skv, flags); break;
-        default: hipLaunchKernelGGL(mask_classify_kernel<bf16_t>, grid, dim3(256), 0, stream, (const bf16_t*)p.mask, p.m_sb, p.m_sh, p.m_si, p.m_sj, Hm, p.Sq, p.Skv, flags); break;
+        case 0: if (vec) CLASSIFY(float, true); else CLASSIFY(float, false); break;
+        case 1: if (vec) CLASSIFY(f16_t, true); else CLASSIFY(f16_t, false); break;
+        default: if (vec) CLASSIFY(bf16_t, true); else CLASSIFY(bf16_t, false); break;
     }
+#undef CLASSIFY
     return hipGetLastError();
 }
 

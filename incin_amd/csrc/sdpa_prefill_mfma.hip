@@ -126,7 +126,13 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     const int nkb32 = (Skv + 31) >> 5;
     int t_first = 0;
     [[maybe_unused]] int w_first = 0, w_last = 0x7fffffff;      // this wavefront's first and last tile with a visible block
+    [[maybe_unused]] int z_end = 0;
     __shared__ int s_range[8];
+    // the flags of this wavefront's tiles, two per tile, kept in LDS when they fit (up to 32768 keys): a flag is on
+    // the path of every tile, and a global load there costs a memory latency per tile
+    constexpr int FLAG_TILES = 512;
+    __shared__ uint8_t s_flags[DENSE ? 4 * 2 * FLAG_TILES : 4];
+    const bool flags_in_lds = DENSE && n_tiles <= FLAG_TILES;
     if (DENSE) {
         mflags = mask_flags_of(p, b, hq) + (int64_t)((q0 >> 5) + wave) * nkb32;
         mrow = (const T*)p.mask + (int64_t)b * p.m_sb + (int64_t)hq * p.m_sh + (int64_t)min(my_i, Sq - 1) * p.m_si;
@@ -135,20 +141,30 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
             for (int t = lane; t < n_tiles; t += 64) {
                 const int f0 = mflags[2 * t], f1 = 2 * t + 1 < nkb32 ? mflags[2 * t + 1] : 2;
                 if (f0 != 2 || f1 != 2) { lo = min(lo, t); hi = max(hi, t); }
+                if (flags_in_lds) { s_flags[(wave * FLAG_TILES + t) * 2] = (uint8_t)f0; s_flags[(wave * FLAG_TILES + t) * 2 + 1] = (uint8_t)f1; }
             }
 #pragma unroll
         for (int off = 32; off >= 1; off >>= 1) {
             lo = min(lo, __shfl_xor(lo, off, 64));
             hi = max(hi, __shfl_xor(hi, off, 64));
         }
-        w_first = lo;
-        w_last = hi;
+        w_first = __builtin_amdgcn_readfirstlane(lo);
+        w_last = __builtin_amdgcn_readfirstlane(hi);
         if (lane == 0) { s_range[wave] = lo; s_range[4 + wave] = hi; }
         __syncthreads();
         const int g_lo = min(min(s_range[0], s_range[1]), min(s_range[2], s_range[3]));
         const int g_hi = max(max(s_range[4], s_range[5]), max(s_range[6], s_range[7]));
-        t_first = g_hi < 0 ? 0 : g_lo;
-        n_tiles = g_hi + 1;                           // (0 when the mask hides everything from these 128 rows)
+        // (uniform by construction; said explicitly, because tile numbers end up in scalar DMA descriptors)
+        t_first = __builtin_amdgcn_readfirstlane(g_hi < 0 ? 0 : g_lo);
+        n_tiles = __builtin_amdgcn_readfirstlane(g_hi + 1);      // (0 when the mask hides everything from these 128 rows)
+        // z_end: the first tile after t_first in which the mask does something to this wavefront's rows; the tiles
+        // t_first + 1 .. z_end - 1 run through the pipelined loop like tiles of a launch without a mask
+        int z = n_tiles;
+        for (int t = t_first + 1 + lane; t < n_tiles; t += 64)
+            if (mflags[2 * t] != 1 || (2 * t + 1 < nkb32 ? mflags[2 * t + 1] : 2) != 1) { z = t; break; }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) z = min(z, __shfl_xor(z, off, 64));
+        z_end = __builtin_amdgcn_readfirstlane(z);
     }
 
     // ---- global -> LDS copy plan ---------------------------------------------------
@@ -388,11 +404,16 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     // Dense mask on the scores of the tile that starts at key j0 (scores are in log2 units): per 32-key half, nothing
     // where the flag says zeros, -inf where it says hidden, else the values themselves - 4 consecutive keys per load
     // where the mask's layout allows (unit key stride, 8-byte aligned rows), element by element otherwise.
+    // flag of 32-key block blk (= 2 * tile + half) for this wavefront's rows; past the last block: hidden
+    auto flag_of = [&](int blk) __attribute__((always_inline)) -> int {
+        if (blk >= nkb32) return 2;
+        const int f = flags_in_lds ? (int)s_flags[wave * FLAG_TILES * 2 + blk] : (int)mflags[blk];
+        return __builtin_amdgcn_readfirstlane(f);
+    };
     auto add_dense_mask = [&](floatx16 (&sx)[2], int j0) __attribute__((always_inline)) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
-            const int blk = (j0 >> 5) + kb;
-            const int flag = blk < nkb32 ? __builtin_amdgcn_readfirstlane((int)mflags[blk]) : 2;
+            const int flag = flag_of((j0 >> 5) + kb);
             if (flag == 1) continue;
             if (flag == 2) {
 #pragma unroll
@@ -473,9 +494,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
         // wavefront computes tile t if its limits (causal, key count) and the mask's flags leave it a visible block.
         auto mine = [&](int t) __attribute__((always_inline)) {
             if (t >= n_act || t < w_first || t > w_last) return false;
-            const int f0 = __builtin_amdgcn_readfirstlane((int)mflags[2 * t]);
-            const int f1 = 2 * t + 1 < nkb32 ? __builtin_amdgcn_readfirstlane((int)mflags[2 * t + 1]) : 2;
-            return f0 != 2 || f1 != 2;
+            return flag_of(2 * t) != 2 || flag_of(2 * t + 1) != 2;
         };
         issue_k(t_first, t_first & 1);
         __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -485,7 +504,8 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
         issue_v(t_first, t_first & 1);
         bool pending = mine(t_first);
         if (pending) scores_plain(smem + (t_first & 1) * L::TILE_BYTES, sacc[0], t_first * PF_BN);
-        for (int t = t_first; t < n_tiles; ++t) {
+        int t = t_first;
+        auto plain_step = [&]() __attribute__((always_inline)) {
             turn(t);
             if (pending) {
                 const char* v_cur = smem + (2 + (t & 1)) * L::TILE_BYTES;
@@ -504,7 +524,18 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
             }
             pending = t + 1 < n_tiles && mine(t + 1);
             if (pending) scores_plain(smem + ((t + 1) & 1) * L::TILE_BYTES, sacc[0], (t + 1) * PF_BN);
-        }
+            ++t;
+        };
+        // the run of tiles after the first one that neither the mask nor a limit touches: pipelined, two at a time
+        // from an even tile on
+        const int hot_end = min(min(z_end, n_hot), n_tiles);
+        if ((t & 1) && t < n_tiles) plain_step();
+        if (pending)
+            for (; t + 2 < hot_end; t += 2) {
+                iter(t, std::integral_constant<int, 0>{});
+                iter(t + 1, std::integral_constant<int, 1>{});
+            }
+        while (t < n_tiles) plain_step();
     }
 #undef SGB
 
