@@ -16,7 +16,10 @@ SOURCES = ["incin_rocm.hip", "sdpa_generic.hip", "sdpa_decode.hip", "sdpa_prefil
 EXTRA_FLAGS = {}    # per-file flags
 HOST_DIR = os.path.join(HERE, "host")
 HOST_LIB = os.path.join(LIBDIR, "libincin_rocm_host.so")
-HOST_SOURCES = ["rocm_backend.cpp", "rocm_capability.cpp", "rocm_exec.cpp", "rocm_conformance.cpp", "rocm_backend_c.cpp"]
+HOST_SOURCES = ["rocm_backend.cpp", "rocm_capability.cpp", "rocm_exec.cpp", "rocm_backend_c.cpp"]
+# test-side harness: the conformance suite, linked against the host library but not part of it
+TEST_DIR = os.path.join(os.path.dirname(HERE), "tests", "native")
+TEST_LIB = os.path.join(TEST_DIR, "libincin_rocm_conformance.so")
 CXX = os.environ.get("CXX", "g++")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -packed-fp32-ops off: the compiler must not form packed-fp32 VALU instructions from float code.
@@ -60,7 +63,20 @@ def build_host_library(verbose=False):
     return HOST_LIB
 
 
+def build_test_library(verbose=False):
+    """The conformance harness of the tests (tests/native/), a library of its own beside the product libraries."""
+    cmd = [CXX, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra", "-o", TEST_LIB, os.path.join(TEST_DIR, "rocm_conformance.cpp"),
+           "-L" + LIBDIR, "-lincin_rocm_host", "-lincin_rocm", "-Wl,-rpath," + LIBDIR]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("conformance harness build failed:\n%s\n%s" % (r.stdout, r.stderr))
+    if verbose:
+        print("built", TEST_LIB)
+    return TEST_LIB
+
+
 if __name__ == "__main__":
     build_library(verbose=True)
     build_host_library(verbose=True)
+    build_test_library(verbose=True)
     sys.exit(0)

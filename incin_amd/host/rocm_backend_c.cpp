@@ -5,7 +5,6 @@
 
 #include "rocm_backend.hpp"
 #include "rocm_capability.hpp"
-#include "rocm_conformance.hpp"
 #include "rocm_exec.hpp"
 
 using namespace incin_rocm_host;
@@ -208,7 +207,7 @@ size_t incin_host_capability_docs(char* out, size_t capacity)
 }
 
 
-// ---- descriptors, conformance, detection ----------------------------------------------------------------------
+// ---- descriptors, detection ----------------------------------------------------------------------
 int incin_host_lower_attention(const int64_t* q_dims, int32_t q_rank, const int64_t* k_dims, int32_t k_rank, const int64_t* v_dims,
                                int32_t v_rank, int32_t dtype, int32_t causal, const int32_t* kv_lens, int64_t kv_lens_count,
                                int32_t has_scale, double scale, const int32_t* q_lens, int64_t q_lens_count,
@@ -250,21 +249,6 @@ int incin_host_reshape(const incin_host_storage* s, const int64_t* dims, int32_t
     RocmStorage o;
     Error e = RocmBackend::reshape(s->s, std::vector<int64_t>(dims, dims + rank), &o);
     return give(e, std::move(o), out);
-}
-
-size_t incin_host_conformance_run(int32_t device, char* text, size_t capacity, int32_t* passed, int32_t* skipped, int32_t* failed)
-{
-    const conformance::Report r = conformance::run(device);
-    if (passed) *passed = r.count(conformance::Check::Outcome::Passed);
-    if (skipped) *skipped = r.count(conformance::Check::Outcome::Skipped);
-    if (failed) *failed = r.count(conformance::Check::Outcome::Failed);
-    const std::string t = r.to_text();
-    if (text && capacity) {
-        const size_t n = t.size() < capacity - 1 ? t.size() : capacity - 1;
-        std::memcpy(text, t.data(), n);
-        text[n] = 0;
-    }
-    return t.size();
 }
 
 int32_t incin_host_is_compiled_in(int32_t kind) { return is_compiled_in(kind) ? 1 : 0; }

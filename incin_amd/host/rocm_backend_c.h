@@ -71,10 +71,6 @@ int incin_host_execute_attention(const incin_host_attention_spec* spec, const in
 void incin_host_release_attention_spec(incin_host_attention_spec* spec);
 int incin_host_reshape(const incin_host_storage* s, const int64_t* dims, int32_t rank, incin_host_storage** out);
 
-/* ---- conformance suite (rocm_conformance.hpp): the report text (at most capacity - 1 bytes written, full length
- * returned) and how many checks passed, were skipped, failed ---- */
-size_t incin_host_conformance_run(int32_t device, char* text, size_t capacity, int32_t* passed, int32_t* skipped, int32_t* failed);
-
 /* ---- device detection (rocm_exec.hpp); kinds as for the capability registry ---- */
 int32_t incin_host_is_compiled_in(int32_t kind);
 int32_t incin_host_probe(int32_t kind);                    /* device ordinal, or -1 */

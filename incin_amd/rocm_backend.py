@@ -28,7 +28,7 @@ EXPORTS = [
     "incin_host_capability_name", "incin_host_capability_max_rank", "incin_host_capability_support",
     "incin_host_capability_rule_count", "incin_host_capability_rule", "incin_host_capability_docs",
     "incin_host_lower_attention", "incin_host_attention_spec_out_dims", "incin_host_execute_attention",
-    "incin_host_release_attention_spec", "incin_host_reshape", "incin_host_conformance_run",
+    "incin_host_release_attention_spec", "incin_host_reshape",
     "incin_host_is_compiled_in", "incin_host_probe", "incin_host_detect_device",
 ]
 
@@ -89,8 +89,6 @@ def lib():
         L.incin_host_release_attention_spec.restype = None
         L.incin_host_release_attention_spec.argtypes = [C.c_void_p]
         L.incin_host_reshape.argtypes = [C.c_void_p, I64P, C.c_int32, C.POINTER(C.c_void_p)]
-        L.incin_host_conformance_run.restype = C.c_size_t
-        L.incin_host_conformance_run.argtypes = [C.c_int32, C.c_char_p, C.c_size_t, I32P, I32P, I32P]
         L.incin_host_is_compiled_in.argtypes = [C.c_int32]
         L.incin_host_probe.argtypes = [C.c_int32]
         L.incin_host_detect_device.argtypes = [I32P, C.c_int32, I32P, I32P]

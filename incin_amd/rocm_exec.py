@@ -1,5 +1,5 @@
-"""ctypes view of the descriptor / executor layer, the conformance suite and device detection of the C++ host
-mirror (incin_amd/host/rocm_exec.hpp, rocm_conformance.hpp)."""
+"""ctypes view of the descriptor / executor layer and device detection of the C++ host mirror
+(incin_amd/host/rocm_exec.hpp)."""
 import ctypes as C
 from collections import namedtuple
 
@@ -55,18 +55,6 @@ def reshape(storage, dims):
     out = C.c_void_p()
     RB._check(RB.lib().incin_host_reshape(storage._h, RB._dims(dims), len(dims), C.byref(out)))
     return RB.RocmStorage(out.value)
-
-
-Report = namedtuple("Report", "text passed skipped failed")
-
-
-def conformance(device=0):
-    """Runs the conformance suite on a device; the report in the reference's text form plus the three counts."""
-    L = RB.lib()
-    p, s, f = C.c_int32(), C.c_int32(), C.c_int32()
-    buf = C.create_string_buffer(16384)
-    L.incin_host_conformance_run(device, buf, len(buf), C.byref(p), C.byref(s), C.byref(f))
-    return Report(buf.value.decode(), p.value, s.value, f.value)
 
 
 def is_compiled_in(kind):

@@ -5,9 +5,9 @@
 #include <exception>
 #include <functional>
 
-#include "rocm_backend.hpp"
-#include "rocm_capability.hpp"
-#include "rocm_exec.hpp"
+#include "../../incin_amd/host/rocm_backend.hpp"
+#include "../../incin_amd/host/rocm_capability.hpp"
+#include "../../incin_amd/host/rocm_exec.hpp"
 
 namespace incin_rocm_host {
 namespace conformance {
@@ -452,3 +452,21 @@ Report run(int device)
 
 }  // namespace conformance
 }  // namespace incin_rocm_host
+
+// Flat C entry for the Python test: the report text (at most capacity - 1 bytes written, full length returned) and how
+// many checks passed, were skipped, failed.
+extern "C" size_t incin_conformance_run(int32_t device, char* text, size_t capacity, int32_t* passed, int32_t* skipped, int32_t* failed)
+{
+    namespace conf = incin_rocm_host::conformance;
+    const conf::Report r = conf::run(device);
+    if (passed) *passed = r.count(conf::Check::Outcome::Passed);
+    if (skipped) *skipped = r.count(conf::Check::Outcome::Skipped);
+    if (failed) *failed = r.count(conf::Check::Outcome::Failed);
+    const std::string t = r.to_text();
+    if (text && capacity) {
+        const size_t n = t.size() < capacity - 1 ? t.size() : capacity - 1;
+        std::memcpy(text, t.data(), n);
+        text[n] = 0;
+    }
+    return t.size();
+}

@@ -1,4 +1,5 @@
-// The backend conformance suite for the rocm backend mirror: the checks of
+// Test-side harness (built into tests/native/libincin_rocm_conformance.so, not into the product libraries): the backend
+// conformance suite for the rocm backend mirror: the checks of
 // crates/incin-backends/src/external/conformance.rs:199-216 (storage round trip, metadata, matmul and reshape through
 // validated descriptors, registry and executor agreeing), reported the same way (pass / skip with the registry's
 // reason / FAIL with what went wrong, :93-160), plus the same three kinds of check for attention.  An operation the
