@@ -4,6 +4,7 @@
 // request no GPU kernel covers is an error, never a host fallback.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -57,14 +58,21 @@ int hip_fail(hipError_t e, const char* what)
 
 int use_device(int32_t dev)
 {
-    int n = 0;
-    hipError_t e = hipGetDeviceCount(&n);
-    if (e != hipSuccess) {
-        (void)hipGetLastError();
-        return fail(INCIN_ROCM_EDEVICE, "ROCm device query failed: %s", hipGetErrorString(e));
+    // the device count does not change while the process lives: asked once; the current device is only switched when
+    // it is another one (both calls are per-thread state lookups, no driver round trip on the launch path)
+    static std::atomic<int> count{-1};
+    int n = count.load(std::memory_order_relaxed);
+    if (n < 0) {
+        hipError_t e = hipGetDeviceCount(&n);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(INCIN_ROCM_EDEVICE, "ROCm device query failed: %s", hipGetErrorString(e));
+        }
+        count.store(n, std::memory_order_relaxed);
     }
     if (dev < 0 || dev >= n) return fail(INCIN_ROCM_EDEVICE, "invalid ROCm device ordinal %d (%d device(s) present)", dev, n);
-    HIP_TRY(hipSetDevice(dev), "hipSetDevice");
+    int cur = -1;
+    if (hipGetDevice(&cur) != hipSuccess || cur != dev) HIP_TRY(hipSetDevice(dev), "hipSetDevice");
     return 0;
 }
 
