@@ -17,13 +17,18 @@ def say(msg):
 
 
 class Case:
-    def __init__(self, seed, B, Hq, Hkv, Sq, Skv, D, causal, impl):
+    def __init__(self, seed, B, Hq, Hkv, Sq, Skv, D, causal, impl, dtype=capi.BF16, banded_mask=False):
         r = np.random.Generator(np.random.PCG64(seed))
-        mk = lambda *s: dtypes.round_to(r.standard_normal(s, dtype=np.float32), capi.BF16)
-        self.tq, self.tk, self.tv = (host.DeviceTensor.from_f32(x, capi.BF16) for x in
+        mk = lambda *s: dtypes.round_to(r.standard_normal(s, dtype=np.float32), dtype)
+        self.tq, self.tk, self.tv = (host.DeviceTensor.from_f32(x, dtype) for x in
                                      (mk(B, Hq, Sq, D), mk(B, Hkv, Skv, D), mk(B, Hkv, Skv, D)))
-        self.to = host.DeviceTensor((B, Hq, Sq, D), capi.BF16)
-        self.desc = host.make_desc(self.tq, self.tk, self.tv, self.to, causal=causal, impl=impl)
+        self.to = host.DeviceTensor((B, Hq, Sq, D), dtype)
+        self.tm, ms = None, None
+        if banded_mask:         # a [Sq, Skv] additive tensor: values near the diagonal, -inf away from it, zeros between
+            d = np.abs(np.arange(Sq)[:, None] - np.arange(Skv)[None, :])
+            m = np.where(d > 200, -np.inf, np.where(d < 40, r.standard_normal((Sq, Skv)), 0.0)).astype(np.float32)
+            self.tm, ms = capi.DeviceBuffer.from_numpy(dtypes.encode(dtypes.round_to(m, dtype), dtype)), (0, 0, Skv, 1)
+        self.desc = host.make_desc(self.tq, self.tk, self.tv, self.to, causal=causal, impl=impl, mask=self.tm, mask_strides=ms)
         nbytes, _, self.impl = capi.sdpa_workspace(self.desc)
         self.ws = capi.DeviceBuffer(nbytes) if nbytes else None
         if self.ws is not None:
@@ -44,6 +49,8 @@ CASES = [
     ("prefill 64-row kernel", dict(B=2, Hq=8, Hkv=2, Sq=1024, Skv=1024, D=128, causal=True, impl=capi.IMPL_MFMA64)),
     ("decode split-KV", dict(B=4, Hq=8, Hkv=8, Sq=1, Skv=4096, D=128, causal=False, impl=capi.IMPL_SPLITKV)),
     ("generic", dict(B=1, Hq=2, Hkv=2, Sq=100, Skv=130, D=80, causal=True, impl=capi.IMPL_GENERIC)),
+    ("f32 matrix-core prefill", dict(B=2, Hq=4, Hkv=2, Sq=300, Skv=300, D=64, causal=True, impl=capi.IMPL_MFMA, dtype=capi.F32)),
+    ("prefill with a dense mask", dict(B=1, Hq=4, Hkv=4, Sq=512, Skv=512, D=128, causal=False, impl=capi.IMPL_MFMA, banded_mask=True)),
 ]
 
 
@@ -63,7 +70,7 @@ def test_threads_on_their_own_streams(gpu):
         except Exception as e:      # noqa: BLE001 - reported below
             errors.append(e)
 
-    say("4 threads x 25 launches, one stream and one kernel each")
+    say("%d threads x 25 launches, one stream and one kernel each" % len(cases))
     threads = [threading.Thread(target=worker, args=(c,)) for c in cases]
     for t in threads:
         t.start()

@@ -1,7 +1,8 @@
 """incin_rocm_sdpa_fwd_static, the launch that takes its scratch memory from the library's static device buffer instead
 of a workspace of the caller's: its output must equal incin_rocm_sdpa_fwd's bit for bit, on two calls in a row of which
-the second is the smaller one (the buffer keeps the first call's contents), for both kernels that use scratch memory:
-split-KV decode (partial results) and the 64-row prefill kernel (work counters)."""
+the second is the smaller one (the buffer keeps the first call's contents), for the three launches that use scratch
+memory: split-KV decode (partial results), the 64-row prefill kernel (work counters) and a matrix-core prefill with a
+dense mask (block flags of the mask)."""
 import sys
 
 import numpy as np
@@ -17,15 +18,19 @@ def say(msg):
 
 
 class Problem:
-    def __init__(self, seed, B, Hq, Hkv, Sq, Skv, D, causal, impl, num_splits=0, kv_lens=None):
+    def __init__(self, seed, B, Hq, Hkv, Sq, Skv, D, causal, impl, num_splits=0, kv_lens=None, causal_mask_tensor=False):
         r = np.random.Generator(np.random.PCG64(seed))
         mk = lambda *s: dtypes.round_to(r.standard_normal(s, dtype=np.float32), capi.BF16)
         self.tq, self.tk, self.tv = (host.DeviceTensor.from_f32(x, capi.BF16) for x in
                                      (mk(B, Hq, Sq, D), mk(B, Hkv, Skv, D), mk(B, Hkv, Skv, D)))
         self.to = host.DeviceTensor((B, Hq, Sq, D), capi.BF16)
         self.lens = capi.DeviceBuffer.from_numpy(np.asarray(kv_lens, dtype=np.int32)) if kv_lens is not None else None
+        self.tm, ms = None, None
+        if causal_mask_tensor:
+            m = np.triu(np.full((Sq, Skv), -np.inf, np.float32), 1 + Skv - Sq)
+            self.tm, ms = capi.DeviceBuffer.from_numpy(dtypes.encode(m, capi.BF16)), (0, 0, Skv, 1)
         self.desc = host.make_desc(self.tq, self.tk, self.tv, self.to, causal=causal, impl=impl, num_splits=num_splits,
-                                   kv_lens=self.lens)
+                                   kv_lens=self.lens, mask=self.tm, mask_strides=ms)
         self.nbytes, self.splits, self.impl = capi.sdpa_workspace(self.desc)
         assert self.impl == impl and self.nbytes > 0
 
@@ -60,6 +65,9 @@ def test_static_scratch_matches_workspace_launch(gpu):
         ("64-row prefill",
          dict(B=2, Hq=8, Hkv=2, Sq=1024, Skv=1024, D=128, causal=True, impl=capi.IMPL_MFMA64),
          dict(B=1, Hq=3, Hkv=3, Sq=300, Skv=300, D=128, causal=True, impl=capi.IMPL_MFMA64)),
+        ("prefill with a dense mask (block flags)",
+         dict(B=2, Hq=4, Hkv=2, Sq=700, Skv=700, D=128, causal=False, impl=capi.IMPL_MFMA, causal_mask_tensor=True),
+         dict(B=1, Hq=2, Hkv=2, Sq=100, Skv=333, D=128, causal=False, impl=capi.IMPL_MFMA, causal_mask_tensor=True)),
     ]
     for name, big, small in big_small:
         pb, ps = Problem(7, **big), Problem(8, **small)
