@@ -105,8 +105,7 @@ def test_config5_gqa_ragged_causal_full(gpu):
     G = Hq // Hkv
     dt = capi.BF16
     r = np.random.Generator(np.random.PCG64(50))
-    lens = r.integers(2048, 16385, B).astype(np.int32)
-    lens[0] = 16384                                    # one full-length sequence
+    lens = r.integers(2048, 16385, B).astype(np.int32)           # drawn uniform in [2048, 16384], as the configuration says
     say("config 5: GQA bf16 causal prefill, ragged lengths %s padded to %d" % (lens.tolist(), S))
     q = gen(51, (B, Hq, S, D), dt)
     k, v = gen(52, (B, Hkv, S, D), dt), gen(53, (B, Hkv, S, D), dt)

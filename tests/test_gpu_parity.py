@@ -455,3 +455,42 @@ def test_large_logits(gpu, dtype, impl, sq):
     got, info = host.sdpa(q, k, v, dtype, impl=impl, return_info=True, num_splits=2 if impl == capi.IMPL_SPLITKV else 0)
     assert info["impl"] == impl
     check(got, oracle_full(q, k, v), TOL[dtype], "large logits")
+
+
+def test_copy_strided_gathers_any_view(gpu):
+    """incin_rocm_copy_strided against numpy's own view semantics: transposes of the last two axes and of outer axes,
+    broadcast (stride 0) and reversed (negative stride) axes, offsets into a larger buffer, ranks 0 to 8, 2- and 4-byte
+    elements, extents on either side of the 32 x 32 tiles."""
+    import ctypes as C
+    lib = capi.load()
+    r = rng(SEED0 + 200)
+
+    def gather(base, view):
+        """`view` is a numpy view of the contiguous array `base`; returns its logical contents gathered on the device."""
+        src = capi.DeviceBuffer.from_numpy(base)
+        dst = capi.DeviceBuffer(max(view.size * view.itemsize, 1))
+        off = view.__array_interface__["data"][0] - base.__array_interface__["data"][0]
+        shape = (C.c_int64 * max(view.ndim, 1))(*view.shape)
+        strides = (C.c_int64 * max(view.ndim, 1))(*[s // view.itemsize for s in view.strides])
+        capi.check(lib.incin_rocm_copy_strided(0, dst.ptr, src.ptr + off, view.ndim, shape, strides, view.itemsize, None))
+        capi.sync()
+        out = dst.to_numpy(view.dtype, view.shape) if view.size else np.empty(view.shape, view.dtype)
+        src.free()
+        dst.free()
+        return out
+
+    for dtype in (np.float32, np.uint16):
+        a = (r.standard_normal((3, 5, 70, 45)) * 100).astype(dtype)
+        views = [a.transpose(0, 1, 3, 2), a.transpose(1, 0, 2, 3), a[:, :, 5:60, 3:40], a[:, ::-1], a[..., ::-1],
+                 np.broadcast_to(a[:, :1], a.shape), a[1, 2], a[1, 2].T, a[0, 0, 0], a[0, 0, :, 0], a[2, 4, 33:34, 7:8],
+                 a.reshape(3, 5, 7, 10, 45).transpose(0, 2, 1, 4, 3), a[:, :, :0]]
+        for v in views:
+            say("copy_strided: %s shape %s strides %s" % (np.dtype(dtype).name, v.shape, v.strides))
+            assert np.array_equal(gather(a, v), v)
+        s = np.asarray(r.integers(0, 1000), dtype=dtype)               # rank 0
+        assert np.array_equal(gather(s.reshape(1), s.reshape(1)[0:1].reshape(())), s)
+    b = r.standard_normal((2, 1, 2, 1, 2, 3, 2, 5)).astype(np.float32)         # rank 8, last two axes swapped
+    assert np.array_equal(gather(b, b.swapaxes(-1, -2)), b.swapaxes(-1, -2))
+    bad = (C.c_int64 * 9)(*[1] * 9)
+    assert lib.incin_rocm_copy_strided(0, None, None, 9, bad, bad, 4, None) == capi.ESHAPE
+    assert lib.incin_rocm_copy_strided(0, None, None, 1, bad, bad, 3, None) == capi.EDTYPE
