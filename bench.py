@@ -213,24 +213,24 @@ def decode_step_graph(w, B, H, Skv, D, steps):
             "ms_per_step": ms, "kv_GBps": 2.0 * B * H * Skv * D * 2 / (ms * 1e-3) / 1e9}
 
 
-def backward_config3(steps, warmup):
-    """Forward (keeping the row normalisers) and then the timed backward of BASELINE config 3's shape: dQ, dK, dV for a
-    synthetic upstream gradient.  The figure counts 2.5 x the forward's FLOPs (five matrix products against the
-    forward's two; the recomputation of S and dP in both big kernels is not counted)."""
-    B, H, S, D = 8, 16, 4096, 128
-    q, k, v = make_inputs(SEED0 + 5, B, H, H, S, S, D, capi.BF16)
+def backward_leg(steps, warmup, dtype=capi.BF16, B=8, H=16, S=4096, D=128, what="BASELINE config 3's shape"):
+    """Forward (keeping the row normalisers) and then the timed backward: dQ, dK, dV for a synthetic upstream gradient.
+    The figure counts 2.5 x the forward's FLOPs (five matrix products against the forward's two; the recomputation of S
+    and dP in both big kernels is not counted)."""
+    name = {capi.BF16: "bf16", capi.F16: "f16", capi.F32: "f32"}[dtype]
+    q, k, v = make_inputs(SEED0 + 5, B, H, H, S, S, D, dtype)
     g = rng(SEED0 + 6).standard_normal((B, H, S, D), dtype=np.float32)
-    tq, tk, tv, tg = (host.DeviceTensor.from_f32(x, capi.BF16) for x in (q, k, v, g))
-    to, tdq, tdk, tdv = (host.DeviceTensor((B, H, S, D), capi.BF16) for _ in range(4))
+    tq, tk, tv, tg = (host.DeviceTensor.from_f32(x, dtype) for x in (q, k, v, g))
+    to, tdq, tdk, tdv = (host.DeviceTensor((B, H, S, D), dtype) for _ in range(4))
     lse = capi.DeviceBuffer(B * H * S * 4)
     bd = capi.SdpaBwdDesc()
     bd.fwd = host.make_desc(tq, tk, tv, to, causal=True, lse=lse)
     capi.sdpa_fwd(bd.fwd)
-    for name, t in (("d_o", tg), ("d_q", tdq), ("d_k", tdk), ("d_v", tdv)):
-        setattr(bd, name, t.ptr)
+    for field, t in (("d_o", tg), ("d_q", tdq), ("d_k", tdk), ("d_v", tdv)):
+        setattr(bd, field, t.ptr)
         st = host._strides3(t.shape)
         for i in range(3):
-            getattr(bd, name + "_stride")[i] = st[i]
+            getattr(bd, field + "_stride")[i] = st[i]
     ws = capi.DeviceBuffer(capi.sdpa_bwd_workspace(bd))
     bd.workspace, bd.workspace_bytes = ws.ptr, ws.nbytes
     t0 = time.perf_counter()
@@ -248,16 +248,18 @@ def backward_config3(steps, warmup):
     # at-size check of one (batch, head) slice against the float64 backward oracle (checker only)
     from oracle import sdpa_backward as OB
     b, h = B - 1, H - 1
-    rq, rk, rv, rg = (dtypes.round_to(x[b, h], capi.BF16) for x in (q, k, v, g))
+    rq, rk, rv, rg = (dtypes.round_to(x[b, h], dtype) for x in (q, k, v, g))
     ref = OB.sdpa_backward(rq, rk, rv, rg, causal=True)
     err = max(float(np.abs(t.to_f32()[b, h] - r).max() / np.abs(r).max()) for t, r in zip((tdq, tdk, tdv), ref))
     flops = 2.5 * causal_flops(B, H, S, S, D)
     for t in (tq.buf, tk.buf, tv.buf, tg.buf, to.buf, tdq.buf, tdk.buf, tdv.buf, lse, ws):
         t.free()
-    return {"workload": "backward of BASELINE config 3's shape: bf16 causal B=8 H=16 S=4096 D=128, dQ dK dV from Q K V O dO and the "
-                        "forward's row normalisers", "step": "one incin_rocm_sdpa_bwd call (3 kernels: row dots, dQ, dK/dV)",
+    peak = PEAK_F32_TFLOPS if dtype == capi.F32 else PEAK_BF16_TFLOPS
+    return {"workload": "backward of %s: %s causal B=%d H=%d S=%d D=%d, dQ dK dV from Q K V O dO and the "
+                        "forward's row normalisers" % (what, name, B, H, S, D),
+            "step": "one incin_rocm_sdpa_bwd call (3 kernels: row dots, dQ, dK/dV)", "dtype": name,
             "metric": "attn bwd TFLOP/s (2.5 x forward FLOPs)", "value": flops / (wall * 1e-3) / 1e12, "unit": "TFLOP/s",
-            "ms_per_step": wall, "steps": steps, "frac_of_bf16_mfma_peak": flops / (wall * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+            "ms_per_step": wall, "steps": steps, "frac_of_%s_mfma_peak" % ("fp32" if dtype == capi.F32 else "bf16"): flops / (wall * 1e-3) / 1e12 / peak,
             "parity_max_err_rel_to_max_abs_ref": err,
             "parity_sample": "dQ, dK, dV of slice (b=%d, h=%d) against the float64 oracle of the reference's tape gradients" % (b, h)}
 
@@ -468,7 +470,10 @@ def main():
         result.update(f32_configs(args.steps, args.warmup, not args.no_cpu_baseline, threads))
 
     if args.only in (None, "backward"):
-        result["backward"] = backward_config3(max(5, min(args.steps, 30)), min(args.warmup, 5))
+        result["backward"] = backward_leg(max(5, min(args.steps, 30)), min(args.warmup, 5))
+        # f32, the dtype the reference trains in: BASELINE config 2's shape (launches of ~100 us) and config 3's
+        result["backward_f32_c2"] = backward_leg(max(args.steps, 100), min(args.warmup, 5), capi.F32, 4, 8, 1024, 64, "BASELINE config 2's shape")
+        result["backward_f32_large"] = backward_leg(max(5, min(args.steps, 10)), min(args.warmup, 3), capi.F32, what="BASELINE config 3's shape in f32")
 
     print(json.dumps(result))
     return 0

@@ -593,9 +593,9 @@ int incin_rocm_sdpa_fwd_static(const incin_rocm_sdpa_desc_t* desc, void* stream)
 
 size_t incin_rocm_sizeof_sdpa_bwd_desc(void) { return sizeof(incin_rocm_sdpa_bwd_desc_t); }
 
-// Validates a backward request; *empty is set when there is nothing to compute, *mfma when the matrix-core kernels
-// take it (else the generic ones do).
-static int check_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, bool* empty, bool* mfma)
+// Validates a backward request; *empty is set when there is nothing to compute, *kind says which kernels take it:
+// 0 the generic ones, 1 the 16-bit matrix-core ones, 2 the IEEE-f32 matrix-core ones.
+static int check_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, bool* empty, int* kind)
 {
     static const char* OP = "scaled_dot_product_attention backward";
     if (!bd) return fail(INCIN_ROCM_EINVAL, "%s: null descriptor", OP);
@@ -607,27 +607,32 @@ static int check_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, bool* empty, bool* mf
         if (int rc = make_plan(&any, &plan)) return rc;
     }
     *empty = plan.empty || d->Skv == 0;
-    *mfma = false;
+    *kind = 0;
     if (*empty) return 0;
     if (d->q_lens) return fail(INCIN_ROCM_EUNSUPPORTED, "%s: no kernel takes q_lens", OP);
     if (!d->lse) return fail(INCIN_ROCM_EINVAL, "%s: fwd.lse (the forward's row normalisers) is required", OP);
     if (!bd->d_o || !bd->d_q || !bd->d_k || !bd->d_v) return fail(INCIN_ROCM_EINVAL, "%s: null gradient pointer", OP);
     if (d->D > 256 || d->Dv > 256) return fail(INCIN_ROCM_EUNSUPPORTED, "%s: D and Dv up to 256", OP);
 
-    bool ok = d->dtype != INCIN_ROCM_F32 && d->D == 128 && d->Dv == 128 && !d->add_mask && d->scale > 0.0f && std::isfinite(d->scale);
-    ok = ok && fast_layout_ok(d, 8) && aligned16(bd->d_o) && aligned16(bd->d_q) && aligned16(bd->d_k) && aligned16(bd->d_v);
+    // both matrix-core families: whole rows move as 16-byte vectors, tiles are addressed with 32-bit byte offsets
+    const bool f32 = d->dtype == INCIN_ROCM_F32;
+    const int vec = f32 ? 4 : 8;
+    bool ok = d->D == d->Dv && (d->D == 128 || (f32 && d->D == 64)) && !d->add_mask && std::isfinite(d->scale) && (f32 || d->scale > 0.0f);
+    ok = ok && fast_layout_ok(d, vec) && aligned16(bd->d_o) && aligned16(bd->d_q) && aligned16(bd->d_k) && aligned16(bd->d_v);
     for (int a = 0; a < 3; ++a)
-        ok = ok && bd->d_o_stride[a] % 8 == 0 && bd->d_q_stride[a] % 8 == 0 && bd->d_k_stride[a] % 8 == 0 && bd->d_v_stride[a] % 8 == 0;
-    const int64_t big = 1 << 24;
+        ok = ok && bd->d_o_stride[a] % vec == 0 && bd->d_q_stride[a] % vec == 0 && bd->d_k_stride[a] % vec == 0 && bd->d_v_stride[a] % vec == 0;
+    const int64_t big = f32 ? (1 << 22) : (1 << 24);
     ok = ok && d->q_stride[2] >= 0 && d->q_stride[2] < big && d->k_stride[2] >= 0 && d->k_stride[2] < big && d->v_stride[2] >= 0 &&
          d->v_stride[2] < big && bd->d_o_stride[2] >= 0 && bd->d_o_stride[2] < big;
-    if (d->impl == INCIN_ROCM_IMPL_AUTO) *mfma = ok;
-    else if (d->impl == INCIN_ROCM_IMPL_GENERIC) *mfma = false;
+    const int fast = f32 ? 2 : 1;
+    if (d->impl == INCIN_ROCM_IMPL_AUTO) *kind = ok ? fast : 0;
+    else if (d->impl == INCIN_ROCM_IMPL_GENERIC) *kind = 0;
     else if (d->impl == INCIN_ROCM_IMPL_MFMA) {
         if (!ok)
-            return fail(INCIN_ROCM_EUNSUPPORTED, "%s: the MFMA kernels need f16 / bf16, D == Dv == 128, scale > 0, no dense mask, and rows "
-                        "16-byte aligned with strides that are multiples of 8 elements below 2^24", OP);
-        *mfma = true;
+            return fail(INCIN_ROCM_EUNSUPPORTED, "%s: the MFMA kernels need D == Dv == 128 (f32: 64 as well), a finite scale (f16 / bf16: "
+                        "positive), no dense mask, and rows 16-byte aligned with strides that are multiples of 16 bytes below 2^%d elements",
+                        OP, f32 ? 22 : 24);
+        *kind = fast;
     } else
         return fail(INCIN_ROCM_EUNSUPPORTED, "%s: impl is one of AUTO, GENERIC, MFMA", OP);
     return 0;
@@ -637,16 +642,18 @@ int incin_rocm_sdpa_bwd_workspace(const incin_rocm_sdpa_bwd_desc_t* bd, size_t* 
 {
     if (!bytes) return fail(INCIN_ROCM_EINVAL, "scaled_dot_product_attention backward: null output");
     *bytes = 0;
-    bool empty = false, mfma = false;
-    if (int rc = check_bwd(bd, &empty, &mfma)) return rc;
+    bool empty = false;
+    int kind = 0;
+    if (int rc = check_bwd(bd, &empty, &kind)) return rc;
     if (!empty) *bytes = 2 * (size_t)(bd->fwd.B * bd->fwd.Hq * bd->fwd.Sq) * sizeof(float);
     return 0;
 }
 
 int incin_rocm_sdpa_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, void* stream)
 {
-    bool empty = false, mfma = false;
-    if (int rc = check_bwd(bd, &empty, &mfma)) return rc;
+    bool empty = false;
+    int kind = 0;
+    if (int rc = check_bwd(bd, &empty, &kind)) return rc;
     if (empty) {
         // No element to write - except with queries but no keys: the output is zeros whatever q holds, so d_q is zero
         // (the reference's tape gives zeros there), and it is promised to be fully overwritten.
@@ -679,8 +686,9 @@ int incin_rocm_sdpa_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, void* stream)
     bp.dq_sb = bd->d_q_stride[0]; bp.dq_sh = bd->d_q_stride[1]; bp.dq_ss = bd->d_q_stride[2];
     bp.dk_sb = bd->d_k_stride[0]; bp.dk_sh = bd->d_k_stride[1]; bp.dk_ss = bd->d_k_stride[2];
     bp.dv_sb = bd->d_v_stride[0]; bp.dv_sh = bd->d_v_stride[1]; bp.dv_ss = bd->d_v_stride[2];
-    hipError_t e = mfma ? incin_rocm::launch_sdpa_bwd_mfma(bp, bd->fwd.dtype, (hipStream_t)stream)
-                        : incin_rocm::launch_sdpa_bwd_generic(bp, bd->fwd.dtype, (hipStream_t)stream);
+    hipError_t e = kind == 2   ? incin_rocm::launch_sdpa_bwd_f32(bp, (hipStream_t)stream)
+                   : kind == 1 ? incin_rocm::launch_sdpa_bwd_mfma(bp, bd->fwd.dtype, (hipStream_t)stream)
+                               : incin_rocm::launch_sdpa_bwd_generic(bp, bd->fwd.dtype, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "attention backward launch");
     return 0;
 }

@@ -1,4 +1,4 @@
-// Launch parameters of the attention backward kernels (sdpa_bwd_mfma.hip), shared with the C ABI layer.
+// Launch parameters of the attention backward kernels (sdpa_bwd_mfma.hip, sdpa_bwd_f32.hip, sdpa_bwd_generic.hip), shared with the C ABI layer.
 #pragma once
 #include <hip/hip_runtime.h>
 
@@ -21,6 +21,7 @@ struct SdpaBwdParams {
 };
 
 hipError_t launch_sdpa_bwd_mfma(const SdpaBwdParams& bp, int dtype, hipStream_t stream);
+hipError_t launch_sdpa_bwd_f32(const SdpaBwdParams& bp, hipStream_t stream);
 hipError_t launch_sdpa_bwd_generic(const SdpaBwdParams& bp, int dtype, hipStream_t stream);
 
 }  // namespace incin_rocm

@@ -150,13 +150,97 @@ def test_generic_backward_f32_against_the_oracle(gpu, shape):
         mask[r.random(mshape) < 0.25] = -np.inf
         mask[..., 0] = 0.0                                       # every row keeps a visible key
     lens_a = None if lens is None else np.asarray(lens, np.int32)
-    out, dq, dk, dv = host.sdpa_backward(q, k, v, go, capi.F32, causal=causal, kv_lens=lens_a, mask=mask)
+    out, dq, dk, dv = host.sdpa_backward(q, k, v, go, capi.F32, causal=causal, kv_lens=lens_a, mask=mask, impl=capi.IMPL_GENERIC)
     m5 = None if mask is None else np.broadcast_to(mask, (B, Hq, Sq, Skv)).reshape(B, Hkv, G, Sq, Skv)
     rq, rk, rv = BW.sdpa_backward(q.reshape(B, Hkv, G, Sq, D), k[:, :, None], v[:, :, None], go.reshape(B, Hkv, G, Sq, Dv),
                                   mask=m5, causal=causal, kv_lens=None if lens is None else lens_a.reshape(B, 1, 1))
     compare("dq", dq, rq.reshape(B, Hq, Sq, D), tol=1e-5)
     compare("dk", dk, rk.reshape(B, Hkv, Skv, D), tol=1e-5)
     compare("dv", dv, rv.reshape(B, Hkv, Skv, Dv), tol=1e-5)
+
+
+@pytest.mark.parametrize("shape", [
+    # B, Hq, Hkv, Sq, Skv, D, causal, kv_lens, scale
+    (1, 1, 1, 32, 32, 64, False, None, None),
+    (1, 1, 1, 32, 32, 128, True, None, None),
+    (2, 3, 3, 128, 128, 64, True, None, None),                   # the reference's bench head shape, causal
+    (2, 4, 4, 200, 333, 64, False, None, 0.3),
+    (2, 4, 2, 300, 300, 128, True, None, None),
+    (1, 8, 2, 130, 450, 64, True, None, None),                   # Sq < Skv: causal alignment, grouped queries
+    (3, 2, 2, 257, 257, 64, True, [257, 100, 31], None),
+    (2, 2, 1, 64, 700, 128, False, [700, 2], None),
+    (1, 2, 2, 513, 129, 64, False, None, -0.125),                # a negative scale is a scale like any other in f32
+    (8, 2, 1, 77, 140, 128, True, [140, 70, 64, 65, 128, 129, 100, 96], None),      # (batch, KV head) pairs dealt over the XCDs
+], ids=["tiny64", "tiny128_causal", "bench_head", "rect", "gqa_causal128", "gqa_rect_causal", "ragged_causal", "ragged128",
+        "negative_scale", "dealt_pairs"])
+def test_matrix_core_backward_f32_against_the_oracle(gpu, shape):
+    """f32 through the IEEE-f32 matrix-core kernels (D = 64 and 128), picked by AUTO and pinned: 1e-5 of the largest
+    gradient magnitude against the f64 oracle, and the generic f32 kernels within the same distance."""
+    B, Hq, Hkv, Sq, Skv, D, causal, lens, scale = shape
+    G = Hq // Hkv
+    say("matrix-core backward f32: %s" % (shape,))
+    q, k, v, go = make(41, B, Hq, Hkv, Sq, Skv, D, capi.F32)
+    lens_a = None if lens is None else np.asarray(lens, np.int32)
+    kw = dict(causal=causal, kv_lens=lens_a, scale=scale)
+    out, dq, dk, dv = host.sdpa_backward(q, k, v, go, capi.F32, impl=capi.IMPL_MFMA, **kw)
+    auto = host.sdpa_backward(q, k, v, go, capi.F32, **kw)
+    gen = host.sdpa_backward(q, k, v, go, capi.F32, impl=capi.IMPL_GENERIC, **kw)
+    rq, rk, rv = BW.sdpa_backward(q.reshape(B, Hkv, G, Sq, D), k[:, :, None], v[:, :, None], go.reshape(B, Hkv, G, Sq, D),
+                                  scale=scale, causal=causal, kv_lens=None if lens is None else lens_a.reshape(B, 1, 1))
+    refs = (rq.reshape(B, Hq, Sq, D), rk.reshape(B, Hkv, Skv, D), rv.reshape(B, Hkv, Skv, D))
+    for name, x, a, g_, r_ in zip(("dq", "dk", "dv"), (dq, dk, dv), auto[1:], gen[1:], refs):
+        compare(name, x, r_, tol=1e-5)
+        assert np.array_equal(x, a), name + ": AUTO takes the same kernels, which have no run-to-run variation"
+        compare(name + " generic vs matrix-core", g_, x, tol=2e-5)
+    if lens is not None:
+        for b in range(B):
+            assert not dk[b, :, lens[b]:].any() and not dv[b, :, lens[b]:].any()      # padded keys: exactly zero
+
+
+def test_matrix_core_backward_f32_rows_without_keys(gpu):
+    # Sq > Skv under causal alignment: the first Sq - Skv rows see nothing; they get a zero dq and add nothing to dk, dv
+    B, H, Sq, Skv, D = 1, 2, 96, 40, 64
+    q, k, v, go = make(42, B, H, H, Sq, Skv, D, capi.F32)
+    out, dq, dk, dv = host.sdpa_backward(q, k, v, go, capi.F32, causal=True, impl=capi.IMPL_MFMA)
+    dead = Sq - Skv
+    assert np.isnan(out[:, :, :dead]).all() and not dq[:, :, :dead].any()
+    rq, rk, rv = BW.sdpa_backward(q[:, :, dead:], k, v, go[:, :, dead:], causal=True)
+    compare("dq (live rows)", dq[:, :, dead:], rq, tol=1e-5)
+    compare("dk", dk, rk, tol=1e-5)
+    compare("dv", dv, rv, tol=1e-5)
+    lens = np.array([0], np.int32)
+    out, dq, dk, dv = host.sdpa_backward(q[:, :, :40], k, v, go[:, :, :40], capi.F32, kv_lens=lens, impl=capi.IMPL_MFMA)
+    assert not dq.any() and not dk.any() and not dv.any()
+
+
+def test_matrix_core_backward_f32_single_key(gpu):
+    """One visible key: P = 1, dS = dP - D = 0 and dq = dk = 0 in real arithmetic.  The reference's tape subtracts dP from
+    itself there (cpu/ops/elementwise.rs:1062-1077: the sum over one element) and gets an exact zero; the kernels subtract
+    D_i = dO_i . O_i from dP_i0 = dO_i . V_0, two f32 evaluations of one sum of D products, each off by the rounding of its
+    partial sums (of the order of sqrt(D) half units in the last place).  What reaches the gradients is bounded by that:
+    2 sqrt(D) 2^-24 max|dP| per dS, times |scale| sum_i |Q_id| for dk and |scale| |K_0d| for dq; dv is the plain column sum
+    of dO."""
+    B, Hq, Hkv, Sq, Skv, D = 1, 2, 1, 64, 70, 128
+    q, k, v, go = make(44, B, Hq, Hkv, Sq, Skv, D, capi.F32)
+    lens = np.array([1], np.int32)
+    out, dq, dk, dv = host.sdpa_backward(q, k, v, go, capi.F32, kv_lens=lens, impl=capi.IMPL_MFMA)
+    s = 1.0 / np.sqrt(D)
+    eps_ds = 2.0 * np.sqrt(D) * 2.0 ** -24 * float(np.abs(go.astype(np.float64) @ v[0, 0, 0].astype(np.float64)).max())
+    say("   single key: max|dq| %.3e max|dk| %.3e, dS rounding level %.3e" % (np.abs(dq).max(), np.abs(dk).max(), eps_ds))
+    assert np.abs(dq).max() <= eps_ds * s * np.abs(k[0, 0, 0]).max()
+    assert np.abs(dk[0, 0, 0]).max() <= eps_ds * s * np.abs(q).sum(axis=(1, 2)).max()
+    assert not dk[0, 0, 1:].any() and not dv[0, 0, 1:].any()
+    compare("dv", dv[0, 0, 0], go.astype(np.float64).sum(axis=(0, 1, 2)), tol=1e-5)
+
+
+def test_matrix_core_backward_f32_at_a_few_thousand_tokens(gpu):
+    B, Hq, Hkv, S, D = 1, 4, 2, 2048, 128
+    q, k, v, go = make(43, B, Hq, Hkv, S, S, D, capi.F32)
+    out, dq, dk, dv = host.sdpa_backward(q, k, v, go, capi.F32, causal=True, impl=capi.IMPL_MFMA)
+    rq, rk, rv = BW.sdpa_backward(q.reshape(B, Hkv, 2, S, D), k[:, :, None], v[:, :, None], go.reshape(B, Hkv, 2, S, D), causal=True)
+    compare("dq", dq, rq.reshape(B, Hq, S, D), tol=1e-5)
+    compare("dk", dk, rk.reshape(B, Hkv, S, D), tol=1e-5)
+    compare("dv", dv, rv.reshape(B, Hkv, S, D), tol=1e-5)
 
 
 @pytest.mark.parametrize("dtype", [capi.BF16, capi.F16])
