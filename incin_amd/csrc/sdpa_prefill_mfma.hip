@@ -50,6 +50,18 @@
 // accumulator and the running sum are rescaled then); otherwise probabilities
 // are taken against the stale maximum, which is exact in exact arithmetic and
 // keeps every intermediate within f32 / storage range.
+//
+// bf16 without a dense mask goes one step further in the pipelined loop and takes no maxima there at
+// all.  bf16 has the exponent range of f32, so the probabilities are carried 2^-64 times smaller
+// (the reference is kept 64 above the maximum it was taken from) and the only thing to know about a
+// tile is whether some probability reached 2.0 - bit 14 of a bf16 - i.e. whether a score passed the
+// stale maximum by more than 2^64: the packed probabilities are OR-ed together as they are made
+// (8 instructions per tile instead of 21 for the maxima) and one test of the result decides.  If the
+// bit is set, the exact path runs before anything of that tile is accumulated: maximum of the tile,
+// reference raised, O^T and the row sum rescaled, the probabilities taken again.  Scores more than
+// 2^62 below the reference flush to zero, which is far below what bf16 resolves.  The vector ALU
+// instructions saved are the point: on N(0,1) inputs this kernel is limited by power (the same
+// launch on zero inputs runs 1.4 times faster), and every instruction not issued is clock gained.
 #include <type_traits>
 
 #include "sdpa_mfma_common.h"
@@ -73,6 +85,10 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     constexpr int NSTEP = D / 16;          // k-steps of the S^T product
     constexpr int NDB = D / 32;            // 32-wide blocks of the head dimension
     constexpr int LPW = L::LOADS_PER_WAVE;
+    // bf16 without a dense mask: probabilities are taken 2^-SHIFT times smaller, so that "some probability reached 2"
+    // - one bit of the packed values - says that a score passed the reference by more than 2^SHIFT
+    constexpr bool ORCHK = std::is_same<T, bf16_t>::value && !DENSE;
+    constexpr float SHIFT = ORCHK ? 64.0f : 0.0f;
 
     __shared__ __attribute__((aligned(1024))) char smem[4 * L::TILE_BYTES];   // K buffers 0, 1, V buffers 0, 1
 
@@ -179,23 +195,41 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
         v_voff[c] = row * (int)p.v_ss * 2 + (slot ^ L::fv(row)) * 16;
     }
     const int64_t k_tile_bytes = (int64_t)PF_BN * p.k_ss * 2, v_tile_bytes = (int64_t)PF_BN * p.v_ss * 2;
-    // K buffer b at smem + b*TILE, V buffer b at smem + (2+b)*TILE
-    auto issue_k = [&](int t, int buf) __attribute__((always_inline)) {
-        int64_t rem = (int64_t)(j_end - t * PF_BN - 1) * p.k_ss * 2 + D * 2;   // bytes to the end of the last row this workgroup may see: loads past that return 0
-        if (rem > 0x7fffffffLL) rem = 0x7fffffffLL;
-        const uint4v r = dma_descriptor((const char*)kp + t * k_tile_bytes, (int)rem);
+    // K buffer b at smem + b*TILE, V buffer b at smem + (2+b)*TILE.  Tiles are copied in order from tile t_first on, so
+    // the copy state runs along: address of the next tile and the bytes from there to the end of the last row this
+    // workgroup may see (loads past that return 0; rows past a batch entry's key count are never read).
+    const char* k_next = (const char*)kp + t_first * k_tile_bytes;
+    const char* v_next = (const char*)vp + t_first * v_tile_bytes;
+    int64_t k_rem = (int64_t)(j_end - t_first * PF_BN - 1) * p.k_ss * 2 + D * 2;
+    int64_t v_rem = (int64_t)(j_end - t_first * PF_BN - 1) * p.v_ss * 2 + D * 2;
+    auto clamp31 = [](int64_t x) __attribute__((always_inline)) {
+        const unsigned hi = (unsigned)((unsigned long long)x >> 32), lo = (unsigned)x;
+        return (hi | (lo >> 31)) != 0 ? 0x7fffffff : (int)lo;
+    };
+    auto issue_k = [&](int /*t: the next tile in order*/, int buf) __attribute__((always_inline)) {
+        const uint4v r = dma_descriptor(k_next, clamp31(k_rem));
         const unsigned dst = lds_address(smem) + buf * L::TILE_BYTES + wave * LPW * 1024;
 #pragma unroll
         for (int c = 0; c < LPW; ++c) dma_copy16(r, dst + c * 1024, k_voff[c]);
+        k_next += k_tile_bytes;
+        k_rem -= k_tile_bytes;
     };
-    auto issue_v = [&](int t, int buf) __attribute__((always_inline)) {
-        int64_t rem = (int64_t)(j_end - t * PF_BN - 1) * p.v_ss * 2 + D * 2;     // (rows past a batch entry's key count are never read)
-        if (rem > 0x7fffffffLL) rem = 0x7fffffffLL;
-        const uint4v r = dma_descriptor((const char*)vp + t * v_tile_bytes, (int)rem);
+    auto issue_v = [&](int, int buf) __attribute__((always_inline)) {
+        const uint4v r = dma_descriptor(v_next, clamp31(v_rem));
         const unsigned dst = lds_address(smem) + (2 + buf) * L::TILE_BYTES + wave * LPW * 1024;
 #pragma unroll
         for (int c = 0; c < LPW; ++c) dma_copy16(r, dst + c * 1024, v_voff[c]);
+        v_next += v_tile_bytes;
+        v_rem -= v_tile_bytes;
     };
+
+    // The first copies start before anything else waits on memory (the Q rows, a dense mask's flags): K of the first
+    // two tiles and V of the first; nothing in this workgroup's LDS is in use yet.
+    if (n_tiles > t_first) {
+        issue_k(t_first, t_first & 1);
+        if (t_first + 1 < n_tiles) issue_k(t_first + 1, (t_first + 1) & 1);
+        issue_v(t_first, t_first & 1);
+    }
 
     // ---- LDS read addresses (bytes inside a tile buffer) ------------------------------------
     // K operand: lane (ql, g) reads row 32*kb + ql, logical chunk 2*s + g
@@ -295,9 +329,10 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     // Move the reference maximum when the pending tile maximum asks for it (first visible tile, or more
     // than the threshold above the reference): rescales what has been accumulated and the pending tile.
     auto adjust_reference = [&](floatx16 (&sx)[2]) __attribute__((always_inline)) {
-        const bool need = inited ? (tmax > PF_RESCALE_THRESHOLD) : (tmax > -INFINITY);
+        const bool need = inited ? (tmax > PF_RESCALE_THRESHOLD - SHIFT) : (tmax > -INFINITY);
         if (__builtin_amdgcn_ballot_w64(need) != 0) {
-            const float delta = need ? tmax : 0.0f;       // lanes that do not need it move by 0
+            const float delta = need ? tmax + SHIFT : 0.0f;       // lanes that do not need it move by 0
+            tmax -= delta;
             const float alpha = inited ? __builtin_amdgcn_exp2f(-delta) : 1.0f;   // nothing accumulated yet: nothing to rescale
             m_ref += delta;
             inited = inited || need;
@@ -341,11 +376,17 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
 
     // start of every iteration t: K(t+1) and V(t) are in LDS for everyone, everyone is past S^T(t) (K buffer
     // t%2 is free) and past O^T(t-1) (V buffer (t+1)%2 is free); start the next global loads into those.
-    auto turn = [&](int t) __attribute__((always_inline)) {
+    auto turn_sync = [&]() __attribute__((always_inline)) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
+    };
+    auto turn_issue = [&](int t) __attribute__((always_inline)) {
         if (t + 2 < n_tiles) issue_k(t + 2, t & 1);
         if (t + 1 < n_tiles) issue_v(t + 1, (t + 1) & 1);
+    };
+    auto turn = [&](int t) __attribute__((always_inline)) {
+        turn_sync();
+        turn_issue(t);
     };
 
     // Hot iteration (tiles t and t+1 both computed by this wavefront, tile t+1 needs no mask):
@@ -357,9 +398,10 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
         floatx16 (&sn)[2] = sacc[1 - par];
         const char* k_nxt = smem + (1 - par) * L::TILE_BYTES;        // K(t+1)
         const char* v_cur = smem + (2 + par) * L::TILE_BYTES;        // V(t)
-        turn(t);
+        turn_sync();
 #pragma unroll
         for (int s = 0; s < KD; ++s) read_k(k_nxt, s);
+        turn_issue(t);
         adjust_reference(sc);
         rsum = 0.0f;
         __builtin_amdgcn_sched_barrier(0);
@@ -399,6 +441,128 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
             }
         }
         tmax = xor32_max(fmaxf(m0, m1));
+    };
+
+    // The same iteration with the cheap overflow check (ORCHK): no maxima.  The probabilities of tile t are OR-ed
+    // together as they are packed; a set bit 14 in either half of the result says that one of them reached 2, i.e. that
+    // a score of tile t passed the reference by more than 2^SHIFT.  Only then (rare: the reference is the maximum of
+    // an earlier tile) the exact path runs: maximum of tile t, reference moved, O^T and the row sum rescaled, both score
+    // tiles shifted and the probabilities of tile t taken again - before anything of tile t has been accumulated.
+    auto iter_or = [&](int t, auto PAR_) __attribute__((always_inline)) {
+        constexpr int par = decltype(PAR_)::value;
+        floatx16 (&sc)[2] = sacc[par];
+        floatx16 (&sn)[2] = sacc[1 - par];
+        const char* k_nxt = smem + (1 - par) * L::TILE_BYTES;        // K(t+1)
+        const char* v_cur = smem + (2 + par) * L::TILE_BYTES;        // V(t)
+        turn_sync();
+#pragma unroll
+        for (int s = 0; s < KD; ++s) read_k(k_nxt, s);
+        turn_issue(t);
+        unsigned orv = 0;
+        // exponentials of slice sl (4 scores) now, their packing one slice later: a pack never waits for its operands
+        float ex[2][4];
+        typedef unsigned uint4w __attribute__((ext_vector_type(4)));
+        auto exps_of = [&](int sl) __attribute__((always_inline)) {
+            const int ks = sl / 2, e0 = 4 * (sl % 2);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) ex[sl % 2][e] = __builtin_amdgcn_exp2f(sc[ks / 2][8 * (ks % 2) + e0 + e]);
+        };
+        auto pack_of = [&](int sl) __attribute__((always_inline)) {
+            const int ks = sl / 2, e0 = 4 * (sl % 2);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) pb[ks][e0 + e] = (T)ex[sl % 2][e];
+            const uint4w w = __builtin_bit_cast(uint4w, pb[ks]);
+            orv = orv | w[e0 / 2] | w[e0 / 2 + 1];
+        };
+        constexpr int NSL = 8;
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < NSTEP; ++s) {
+#pragma unroll
+            for (int b2 = 0; b2 < 2; ++b2)
+                sn[b2] = Mma<T>::run(kbuf[s % KD][b2], qreg[s], s == 0 ? neg_ref : sn[b2]);
+            if (s + KD < NSTEP) read_k(k_nxt, s + KD);
+            if (NSTEP == 8) {
+                exps_of(s);
+                if (s > 0) pack_of(s - 1);
+            } else {
+                exps_of(2 * s);
+                if (s > 0) pack_of(2 * s - 1);
+                exps_of(2 * s + 1);
+                pack_of(2 * s);
+            }
+            if (s >= NSTEP - VD / 2) { read_v(v_cur, 2 * (s - (NSTEP - VD / 2))); read_v(v_cur, 2 * (s - (NSTEP - VD / 2)) + 1); }
+        }
+        pack_of(NSL - 1);
+#pragma unroll
+        for (int s = 0; s < NSTEP; ++s) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                SGB(SG_MFMA, 1);
+                if (NSTEP == 8) {
+                    SGB(SG_TRANS, 1);
+                    if (s > 0) SGB(SG_VALU, 1);
+                    SGB(SG_TRANS, 1);
+                    if (s > 0 && h == 1) SGB(SG_VALU, 1);
+                } else {
+                    SGB(SG_TRANS, 2); SGB(SG_VALU, 2); SGB(SG_TRANS, 2); SGB(SG_VALU, 1);
+                }
+                if (s + KD < NSTEP) SGB(SG_DSR, 1);
+                if (s >= NSTEP - VD / 2) SGB(SG_DSR, 2);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (__builtin_amdgcn_ballot_w64((orv & 0x40004000u) != 0) != 0) {
+            tmax = max_of(sc);
+            const bool need = tmax > PF_RESCALE_THRESHOLD - SHIFT;
+            const float delta = need ? tmax + SHIFT : 0.0f;
+            const float alpha = __builtin_amdgcn_exp2f(-delta);
+            m_ref += delta;
+            l_run *= alpha;
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) o_acc[db][r] *= alpha;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) neg_ref[r] = -m_ref;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) { sc[kb][r] -= delta; sn[kb][r] -= delta; }
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) pb[ks][e] = (T)__builtin_amdgcn_exp2f(sc[ks / 2][8 * (ks % 2) + e]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        float rs[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int i = 0; i < NPV; ++i) {
+            o_acc[i % NDB] = Mma<T>::run(vbuf[i % VD], pb[i / NDB], o_acc[i % NDB]);
+            if (i + VD < NPV) read_v(v_cur, i + VD);
+            // row sum of the rounded probabilities, two per instruction, four chains
+            if (NPV == 16) {
+                typename Mma<T>::vec2 pr = {pb[i / 4][2 * (i % 4)], pb[i / 4][2 * (i % 4) + 1]};
+                rs[i % 4] = Mma<T>::add2(pr, rs[i % 4]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int ii = 2 * i + j;
+                    typename Mma<T>::vec2 pr = {pb[ii / 4][2 * (ii % 4)], pb[ii / 4][2 * (ii % 4) + 1]};
+                    rs[ii % 4] = Mma<T>::add2(pr, rs[ii % 4]);
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NPV; ++i) {
+            SGB(SG_MFMA, 1);
+            SGB(SG_VALU, NPV == 16 ? 1 : 2);
+            if (i + VD < NPV) SGB(SG_DSR, 2);
+        }
+        asm volatile("" : "+v"(rs[0]), "+v"(rs[1]), "+v"(rs[2]), "+v"(rs[3]));      // (keeps the sums from being sunk below the next barrier)
+        __builtin_amdgcn_sched_barrier(0);
+        rsum = (rs[0] + rs[1]) + (rs[2] + rs[3]);
+        l_run += rsum;
     };
 
     // Dense mask on the scores of the tile that starts at key j0 (scores are in log2 units): per 32-key half, nothing
@@ -455,18 +619,26 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     const int n_hot = lim_wave_min > 0 ? min(lim_wave_min / PF_BN, n_act) : 0;      // tiles 0..n_hot-1 need no mask
 
     if (!DENSE && n_tiles > 0) {
-        // prologue: K(0) first, then K(1), V(0) in flight; scores of tile 0
-        issue_k(0, 0);
+        // prologue: K(0), K(1), V(0) are in flight since the start; scores of tile 0
         __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0), told to the compiler too: it then knows the Q rows have arrived
         asm volatile("" ::: "memory");
         __syncthreads();
-        if (n_tiles > 1) issue_k(1, 1);
-        issue_v(0, 0);
         if (n_act > 0) scores_plain(smem, sacc[0], 0);
         int t = 0;
-        for (; t + 2 < n_hot; t += 2) {
-            iter(t, std::integral_constant<int, 0>{});
-            iter(t + 1, std::integral_constant<int, 1>{});
+        if constexpr (ORCHK) {
+            if (2 < n_hot) {
+                adjust_reference(sacc[0]);        // the reference of every row of this wavefront: the maximum of tile 0
+                for (; t + 2 < n_hot; t += 2) {
+                    iter_or(t, std::integral_constant<int, 0>{});
+                    iter_or(t + 1, std::integral_constant<int, 1>{});
+                }
+                tmax = max_of(sacc[0]);           // the masked loop below decides by maxima
+            }
+        } else {
+            for (; t + 2 < n_hot; t += 2) {
+                iter(t, std::integral_constant<int, 0>{});
+                iter(t + 1, std::integral_constant<int, 1>{});
+            }
         }
         // the rest, one tile at a time without overlap; the pending scores are in sacc[0]
         for (; t < n_tiles; ++t) {
@@ -496,12 +668,9 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
             if (t >= n_act || t < w_first || t > w_last) return false;
             return flag_of(2 * t) != 2 || flag_of(2 * t + 1) != 2;
         };
-        issue_k(t_first, t_first & 1);
         __builtin_amdgcn_s_waitcnt(0x0F70);
         asm volatile("" ::: "memory");
         __syncthreads();
-        if (t_first + 1 < n_tiles) issue_k(t_first + 1, (t_first + 1) & 1);
-        issue_v(t_first, t_first & 1);
         bool pending = mine(t_first);
         if (pending) scores_plain(smem + (t_first & 1) * L::TILE_BYTES, sacc[0], t_first * PF_BN);
         int t = t_first;

@@ -457,6 +457,40 @@ def test_large_logits(gpu, dtype, impl, sq):
     check(got, oracle_full(q, k, v), TOL[dtype], "large logits")
 
 
+@pytest.mark.parametrize("causal", [False, True], ids=["full", "causal"])
+@pytest.mark.parametrize("impl", [capi.IMPL_MFMA, capi.IMPL_MFMA64], ids=["mfma", "mfma64"])
+@pytest.mark.parametrize("dtype", [capi.BF16, capi.F16])
+def test_scores_far_above_the_first_tiles(gpu, dtype, impl, causal):
+    """Keys whose logits lie 60 to 130 units above everything a row has seen before, in the second, the fourth and the
+    seventh key tile: the reference maximum a kernel carries from earlier tiles is useless there.  The 16-bit prefill
+    kernel takes no maxima in its pipelined loop for bf16 (it watches one bit of the probabilities instead) and has to
+    notice, rescale and take the probabilities of that tile again; rows of the opposite sign see the same keys fall
+    130 units below their maximum and must not notice at all, and rows of half the magnitude stay under the trigger
+    while sharing a wavefront with rows that pull it.  Keys of one class are identical, so every row's answer is a
+    plain mean of V rows and the rounding of the pre-scaled queries cannot matter."""
+    B, H, S, D = 1, 2, 640, 128
+    r = rng(SEED0 + 93)
+    a = r.choice(np.array([1.0, -1.0, 0.5], np.float32), size=(B, H, S, 1))
+    q = np.broadcast_to(a, (B, H, S, D)).copy()
+    b = np.full((B, H, S, 1), -4.0, np.float32)
+    b[:, :, [70, 200, 201, 207, 231, 250]] = 2.0
+    b[:, :, [400, 401, 437]] = 8.0
+    b[:, 1, 100] = 8.0                                       # head 1: the largest class already in the second tile
+    k = np.broadcast_to(b, (B, H, S, D)).copy()
+    v = dtypes.round_to(r.standard_normal((B, H, S, D), dtype=np.float32), dtype)
+    got, info = host.sdpa(q, k, v, dtype, causal=causal, impl=impl, return_info=True)
+    assert info["impl"] == impl
+    ref = oracle_full(q, k, v, causal=causal)
+    check(got, ref, TOL[dtype], "scores far above the first tiles")
+    # the closed form: mean of the V rows of the visible keys with the row's largest logit
+    logit = a * np.swapaxes(b, 2, 3)                                  # [B, H, S, S] up to a positive factor
+    if causal:
+        logit = np.where(np.tril(np.ones((S, S), bool)), logit, -np.inf)
+    top = logit == logit.max(axis=-1, keepdims=True)
+    mean = np.einsum("bhij,bhjd->bhid", top.astype(np.float64), v.astype(np.float64)) / top.sum(axis=-1, keepdims=True)
+    check(got, mean.astype(np.float32), TOL[dtype], "scores far above the first tiles, closed form")
+
+
 def test_copy_strided_gathers_any_view(gpu):
     """incin_rocm_copy_strided against numpy's own view semantics: transposes of the last two axes and of outer axes,
     broadcast (stride 0) and reversed (negative stride) axes, offsets into a larger buffer, ranks 0 to 8, 2- and 4-byte
