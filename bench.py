@@ -264,6 +264,41 @@ def backward_leg(steps, warmup, dtype=capi.BF16, B=8, H=16, S=4096, D=128, what=
             "parity_sample": "dQ, dK, dV of slice (b=%d, h=%d) against the float64 oracle of the reference's tape gradients" % (b, h)}
 
 
+def matrix_rate():
+    """What rate of bf16 matrix instructions the device sustains, by the data they work on: a loop of
+    v_mfma_f32_32x32x16_bf16 on every compute unit (incin_rocm_matrix_rate), about 20 ms per launch, on zeros, on N(0,1)
+    values rounded to bf16 (what the attention inputs are) and with the vector / LDS instructions the prefill kernel issues
+    per matrix instruction.  The device lowers its clock under the switching activity of real data; these figures are the
+    ceilings the 16-bit attention kernels live under, reported beside the nominal peak the roofline is priced against."""
+    out = {"what": "sustained rate of a loop of v_mfma_f32_32x32x16_bf16, 2 wavefronts per SIMD on every CU, ~20 ms launches; "
+                   "operands: 256 KiB of zeros or of N(0,1) rounded to bf16; mix 1 adds, per matrix instruction, 2 v_exp_f32, "
+                   "3 v_fma_f32 and one ds_read_b128", "unit": "TFLOP/s", "nominal_peak": PEAK_BF16_TFLOPS}
+    sink = capi.DeviceBuffer(2048 * 1024)
+    data = {"zeros": np.zeros(65536, np.uint32),
+            "normal": dtypes.f32_to_bf16_bits(rng(SEED0 + 9).standard_normal(131072, dtype=np.float32)).view(np.uint32)}
+    for name, arr in data.items():
+        src = capi.DeviceBuffer.from_numpy(arr)
+        for mix in (0, 1):
+            iters = 150000 if mix == 0 else 100000
+            capi.matrix_rate(src, sink, mix, 2000)
+            capi.sync()
+            best = None
+            for _ in range(3):
+                e0, e1 = capi.Event(), capi.Event()
+                e0.record()
+                fl = capi.matrix_rate(src, sink, mix, iters)
+                e1.record()
+                capi.sync()
+                ms = e0.elapsed_ms(e1)
+                best = ms if best is None else min(best, ms)
+                e0.destroy(); e1.destroy()
+            out["%s_operands_mix%d" % (name, mix)] = {"value": fl / (best * 1e-3) / 1e12, "ms": best,
+                                                       "frac_of_nominal": fl / (best * 1e-3) / 1e12 / PEAK_BF16_TFLOPS}
+        src.free()
+    sink.free()
+    return out
+
+
 def f32_configs(steps, warmup, with_cpu, threads):
     """BASELINE configs 1 and 2 - f32, the one dtype the reference's operator runs end to end - on the IEEE-f32
     matrix-core kernel: absolute TFLOP/s against the fp32 matrix peak, config 2 also with the causal mask handed over
@@ -331,7 +366,7 @@ def main():
     ap.add_argument("--no-padding-compare", action="store_true",
                     help="prefill_long: skip the extra timing of the batch with its padding rows computed (profiling: every "
                          "launch of the run is then the same launch)")
-    ap.add_argument("--only", choices=["prefill", "prefill_long", "decode", "backward", "f32", "copy"], default=None,
+    ap.add_argument("--only", choices=["prefill", "prefill_long", "decode", "backward", "f32", "copy", "matrix_rate"], default=None,
                     help="run a single workload (profiling). 'copy' runs --steps device-to-device copies of 1 GiB "
                          "through the library's plain copy kernel: the known-size dispatch that hardware byte "
                          "counters (FETCH_SIZE / WRITE_SIZE) are calibrated against")
@@ -468,6 +503,9 @@ def main():
 
     if args.only in (None, "f32"):
         result.update(f32_configs(args.steps, args.warmup, not args.no_cpu_baseline, threads))
+
+    if args.only in (None, "matrix_rate"):
+        result["matrix_rate"] = matrix_rate()
 
     if args.only in (None, "backward"):
         result["backward"] = backward_leg(max(5, min(args.steps, 30)), min(args.warmup, 5))

@@ -31,6 +31,7 @@ EXPORTS = [
     "incin_rocm_sdpa_workspace", "incin_rocm_sdpa_fwd", "incin_rocm_sdpa_fwd_static",
     "incin_rocm_sizeof_kv_append_desc", "incin_rocm_kv_append",
     "incin_rocm_sizeof_sdpa_bwd_desc", "incin_rocm_sdpa_bwd_workspace", "incin_rocm_sdpa_bwd",
+    "incin_rocm_matrix_rate",
 ]
 
 
@@ -156,6 +157,7 @@ def load():
     lib.incin_rocm_sdpa_bwd_workspace.argtypes = [C.POINTER(SdpaBwdDesc), C.POINTER(C.c_size_t)]
     lib.incin_rocm_sdpa_bwd.argtypes = [C.POINTER(SdpaBwdDesc), C.c_void_p]
     lib.incin_rocm_kv_append.argtypes = [C.POINTER(KvAppendDesc), C.c_void_p]
+    lib.incin_rocm_matrix_rate.argtypes = [C.c_int32, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.POINTER(C.c_double), C.c_void_p]
     _lib = lib
     return lib
 
@@ -232,6 +234,13 @@ def sdpa_bwd_workspace(desc):
 
 def sdpa_bwd(desc, stream=None):
     check(load().incin_rocm_sdpa_bwd(C.byref(desc), stream))
+
+
+def matrix_rate(operands, sink, mix, iterations, stream=None, dev=0):
+    """One launch of the matrix-instruction loop on the 256 KiB at `operands`; returns the FLOPs of the launch."""
+    fl = C.c_double(0.0)
+    check(load().incin_rocm_matrix_rate(dev, operands.ptr, sink.ptr, mix, iterations, C.byref(fl), stream))
+    return fl.value
 
 
 def kv_append(desc, stream=None):

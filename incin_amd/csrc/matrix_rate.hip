@@ -1,0 +1,82 @@
+// Diagnostic kernel behind incin_rocm_matrix_rate: what rate of bf16 matrix instructions this device sustains, as a function of
+// the DATA the instructions work on.  No counterpart in the reference; it exists because the bound of the 16-bit attention
+// kernels on this hardware is not a pipe but the power the chip may draw: a loop of nothing but v_mfma_f32_32x32x16_bf16 runs
+// near the nominal peak on zeros and about a third slower on random values, and the attention kernels sit under the second
+// figure.  bench.py reports both beside the roofline of the prefill kernel.
+#include <hip/hip_runtime.h>
+
+#include "sdpa_mfma_common.h"
+
+namespace incin_rocm {
+
+// MIX 0: matrix instructions only.  MIX 1: per matrix instruction two v_exp_f32, three other vector instructions and one
+// 16-byte LDS read - the instruction mix of the prefill kernel's pipelined loop - all independent of the products.
+// 512 threads: two wavefronts per SIMD.  Operands: 16 bytes per lane and operand from `src` (64 Ki dwords, whatever they hold).
+template <int MIX>
+__global__ __launch_bounds__(512) void matrix_rate_kernel(const unsigned* __restrict__ src, float* __restrict__ sink, int iterations)
+{
+    __shared__ unsigned lds[16 * 1024];
+    union { bf16x8 v; unsigned u[4]; } a[4], b[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            a[j].u[e] = src[(threadIdx.x * 16 + j * 4 + e) & 65535];
+            b[j].u[e] = src[(threadIdx.x * 16 + 7 + j * 4 + e + 32768) & 65535];
+        }
+    for (int i = threadIdx.x; i < 16 * 1024; i += blockDim.x) lds[i] = src[i];
+    __syncthreads();
+    floatx16 c[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) c[j][r] = 0.0f;
+    float v[12], t[8];
+#pragma unroll
+    for (int i = 0; i < 12; ++i) v[i] = threadIdx.x * 0.001f + i;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) t[i] = -(threadIdx.x * 0.01f) - i;
+    const unsigned laddr = lds_address(lds) + (threadIdx.x & 63) * 16;
+    float4 ld[4] = {};
+    for (int it = 0; it < iterations; ++it) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            c[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[j].v, b[j].v, c[j], 0, 0, 0);
+            if (MIX == 1) {
+                t[2 * j] = __builtin_amdgcn_exp2f(t[2 * j]);
+                v[3 * j] = __builtin_fmaf(v[3 * j], 1.0001f, 0.5f);
+                t[2 * j + 1] = __builtin_amdgcn_exp2f(t[2 * j + 1]);
+                v[3 * j + 1] = __builtin_fmaf(v[3 * j + 1], 1.0001f, 0.5f);
+                v[3 * j + 2] = __builtin_fmaf(v[3 * j + 2], 1.0001f, 0.5f);
+                asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(ld[j]) : "v"(laddr), "n"(j * 1024));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (MIX == 1) asm volatile("s_waitcnt lgkmcnt(0)");
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 12; ++i) s += v[i];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s += t[i];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        s += ld[j].x + ld[j].w;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s += c[j][r];
+    }
+    sink[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
+// One workgroup per compute unit; `src` holds 256 KiB, `sink` takes 4 bytes per thread (compute units x 2 KiB).
+// *flops = the FLOPs of the matrix instructions of one launch.
+hipError_t launch_matrix_rate(const void* src, void* sink, int mix, int iterations, double* flops, hipStream_t stream)
+{
+    const int cus = device_cus();
+    if (mix == 1) hipLaunchKernelGGL(matrix_rate_kernel<1>, dim3(cus), dim3(512), 0, stream, (const unsigned*)src, (float*)sink, iterations);
+    else hipLaunchKernelGGL(matrix_rate_kernel<0>, dim3(cus), dim3(512), 0, stream, (const unsigned*)src, (float*)sink, iterations);
+    *flops = (double)cus * 8.0 * (double)iterations * 4.0 * 32768.0;
+    return hipGetLastError();
+}
+
+}  // namespace incin_rocm

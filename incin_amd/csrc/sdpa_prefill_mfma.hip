@@ -627,7 +627,21 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
         int t = 0;
         if constexpr (ORCHK) {
             if (2 < n_hot) {
-                adjust_reference(sacc[0]);        // the reference of every row of this wavefront: the maximum of tile 0
+                // the reference of every row of this wavefront: the maximum of tile 0 (nothing accumulated yet, so
+                // nothing to rescale)
+                {
+                    const bool need = tmax > -INFINITY;
+                    const float delta = need ? tmax + SHIFT : 0.0f;
+                    m_ref += delta;
+                    tmax -= delta;
+                    inited = inited || need;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) neg_ref[r] = -m_ref;
+#pragma unroll
+                    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) sacc[0][kb][r] -= delta;
+                }
                 for (; t + 2 < n_hot; t += 2) {
                     iter_or(t, std::integral_constant<int, 0>{});
                     iter_or(t + 1, std::integral_constant<int, 1>{});

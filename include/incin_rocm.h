@@ -249,6 +249,16 @@ size_t incin_rocm_sizeof_sdpa_bwd_desc(void);
 int incin_rocm_sdpa_bwd_workspace(const incin_rocm_sdpa_bwd_desc_t* desc, size_t* bytes);
 int incin_rocm_sdpa_bwd(const incin_rocm_sdpa_bwd_desc_t* desc, void* stream);
 
+/* ---- diagnostics ------------------------------------------------------------------
+ * No counterpart in the reference.  One launch of a loop of bf16 matrix instructions (v_mfma_f32_32x32x16_bf16, one
+ * workgroup of two wavefronts per SIMD on every compute unit, `iterations` x 4 instructions per wavefront) whose operands
+ * are whatever the 256 KiB at `operands` hold - zeros, random values, a slice of real inputs.  mix 0: matrix instructions
+ * only; mix 1: with the vector and LDS instructions the prefill kernel issues per matrix instruction.  The rate a device
+ * sustains depends on that data (its power management lowers the clock under the switching activity of random values),
+ * and it is the ceiling the 16-bit attention kernels live under; bench.py reports it beside their roofline.
+ * `sink` takes 2 KiB per compute unit.  *flops = FLOPs of the launch; time it with events on `stream`. */
+int incin_rocm_matrix_rate(int32_t dev, const void* operands, void* sink, int32_t mix, int32_t iterations, double* flops, void* stream);
+
 /* ---- key/value cache append ----------------------------------------------------
  * No counterpart in the reference (it has no cache: a decode loop there concatenates tensors,
  * TensorOps::cat, and re-runs the operator).  Copies S_new new key and value rows per (batch, kv head) into

@@ -69,7 +69,7 @@ def test_dispatch_choices():
     nbytes, splits, impl = _plan(_desc(Sq=1, Skv=8192, B=1, Hq=8, Hkv=2, num_splits=4))
     assert impl == capi.IMPL_SPLITKV and splits == 4 and nbytes == 8 * 4 * 130 * 4
     assert _plan(_desc(Sq=1, Skv=64))[2] in (capi.IMPL_MFMA, capi.IMPL_SPLITKV)
-    # long sequences with at least 512 work items of 256 query rows: the 64-row kernel (head dimension 128 only)
+    # long sequences: the 32-row kernel as well (the 64-row kernel is level with it or behind at every length; by name only)
     def long(**kw):
         S = kw.pop("S", 16384)
         d = _desc(B=4, Hq=32, Hkv=8, Sq=S, Skv=S, **kw)
@@ -77,9 +77,11 @@ def test_dispatch_choices():
             st = getattr(d, name)
             st[0], st[1], st[2] = heads * S * d.D, S * d.D, d.D
         return d
-    assert _plan(long())[2] == capi.IMPL_MFMA64
-    assert _plan(long(causal=1))[2] == capi.IMPL_MFMA64
-    assert _plan(long(S=4096))[2] == capi.IMPL_MFMA64          # without a causal mask the crossover is at 4096 keys
+    assert _plan(long())[2] == capi.IMPL_MFMA
+    assert _plan(long(causal=1))[2] == capi.IMPL_MFMA
+    assert _plan(long(S=4096))[2] == capi.IMPL_MFMA
+    nbytes, _, impl = _plan(long(impl=capi.IMPL_MFMA64))
+    assert impl == capi.IMPL_MFMA64 and nbytes == 256           # pinned: its work counters come from the workspace
     assert _plan(long(S=4096, causal=1))[2] == capi.IMPL_MFMA
     assert _plan(long(S=2048))[2] == capi.IMPL_MFMA
     assert _plan(long(D=64, Dv=64))[2] == capi.IMPL_MFMA
