@@ -437,6 +437,7 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
 #pragma unroll
             for (int i = 0; i < R; ++i) fetch_a(i);
             if (i0 < i_all_wave) {          // some row of the tile does not see every key of this wavefront
+                asm volatile("" ::: "memory");      // (a real branch: as selects this would cost every tile 32 vector instructions)
                 const int rel = lo_i - i0 - 4 * g - 32 * role;      // register r is row i0 + 32*role + 8*(r/4) + 4*g + (r%4)
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
