@@ -87,8 +87,9 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     constexpr int LPW = L::LOADS_PER_WAVE;
     // bf16 without a dense mask: probabilities are taken 2^-SHIFT times smaller, so that "some probability reached 2"
     // - one bit of the packed values - says that a score passed the reference by more than 2^SHIFT
-    constexpr bool ORCHK = std::is_same<T, bf16_t>::value && !DENSE;
-    constexpr float SHIFT = ORCHK ? 64.0f : 0.0f;
+    constexpr bool BF16 = std::is_same<T, bf16_t>::value;
+    constexpr bool ORCHK = BF16 && !DENSE;
+    constexpr float SHIFT = BF16 ? 64.0f : 0.0f;
 
     __shared__ __attribute__((aligned(1024))) char smem[4 * L::TILE_BYTES];   // K buffers 0, 1, V buffers 0, 1
 
@@ -712,13 +713,29 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
         // the run of tiles after the first one that neither the mask nor a limit touches: pipelined, two at a time
         // from an even tile on
         const int hot_end = min(min(z_end, n_hot), n_tiles);
-        if ((t & 1) && t < n_tiles) plain_step();
-        if (pending)
-            for (; t + 2 < hot_end; t += 2) {
-                iter(t, std::integral_constant<int, 0>{});
-                iter(t + 1, std::integral_constant<int, 1>{});
+        if constexpr (BF16) {
+            // bf16: without maxima, as in a launch without a mask - once every row of the wavefront has a reference.  A
+            // row the mask has hidden entirely so far has none; the plain iteration knows how to give it one.
+            while (t < n_tiles) {
+                if (pending && !(t & 1) && t + 2 < hot_end && __builtin_amdgcn_ballot_w64(!inited) == 0) {
+                    adjust_reference(sacc[0]);
+                    for (; t + 2 < hot_end; t += 2) {
+                        iter_or(t, std::integral_constant<int, 0>{});
+                        iter_or(t + 1, std::integral_constant<int, 1>{});
+                    }
+                    tmax = max_of(sacc[0]);
+                }
+                plain_step();
             }
-        while (t < n_tiles) plain_step();
+        } else {
+            if ((t & 1) && t < n_tiles) plain_step();
+            if (pending)
+                for (; t + 2 < hot_end; t += 2) {
+                    iter(t, std::integral_constant<int, 0>{});
+                    iter(t + 1, std::integral_constant<int, 1>{});
+                }
+            while (t < n_tiles) plain_step();
+        }
     }
 #undef SGB
 
