@@ -34,13 +34,13 @@ PEAK_HBM_GBS = 8000.0       # HBM3E, vendor figure
 # FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0 after calibration against the 1 GiB copy kernel): profiles/*.txt
 PREFILL_TRAFFIC_BYTES = (290791 * 2.0 + 131236) * 1024     # 7.30e8: |Q|+|K|+|V| read 1.48 times (1.07 on another box), |O| written once
 DECODE_TRAFFIC_BYTES = (2097470 * 2.0 + 1088 + 256) * 1024  # 4.297e9: K and V read once + split partials
-PREFILL_LONG_TRAFFIC_BYTES = (600683 * 2.0 + 319192) * 1024    # 1.56e9: valid |O| written once, inputs read 2.5 times
+PREFILL_LONG_TRAFFIC_BYTES = (493652 * 2.0 + 318987) * 1024    # 1.34e9: valid |O| written once, inputs read 2.1 times
 # These three are constants taken from counter runs, not measured by this script: each roofline object says so and
 # names the summary the figures come from.
 TRAFFIC_SOURCE = {
     "prefill": "constant from profiles/sdpa_prefill_mfma_bf16_d128_config3.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of `bench.py --only prefill`)",
     "decode": "constant from profiles/sdpa_decode_splitkv_bf16_d128_config4.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of `bench.py --only decode`)",
-    "prefill_long": "constant from profiles/sdpa_prefill_mfma64_bf16_d128_config5.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of `bench.py --only prefill_long --no-padding-compare`)",
+    "prefill_long": "constant from profiles/sdpa_prefill_mfma_bf16_d128_config5.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of `bench.py --only prefill_long --no-padding-compare`)",
 }
 METRIC = "attn fwd TFLOP/s + % bf16 MFMA peak; decode KV GB/s + % HBM peak (1 GPU)"
 
