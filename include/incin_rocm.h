@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define INCIN_ROCM_ABI_VERSION 4
+#define INCIN_ROCM_ABI_VERSION 5
 
 /* ---- status codes (mapped to incin_core::Error variants by the Rust side;
  *      crates/incin-core/src/err.rs:109-223) --------------------------------- */
