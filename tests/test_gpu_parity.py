@@ -457,7 +457,7 @@ def test_large_logits(gpu, dtype, impl, sq):
     check(got, oracle_full(q, k, v), TOL[dtype], "large logits")
 
 
-@pytest.mark.parametrize("causal", [False, True], ids=["full", "causal"])
+@pytest.mark.parametrize("causal", [False, True, "tensor"], ids=["full", "causal", "causal_as_tensor"])
 @pytest.mark.parametrize("impl", [capi.IMPL_MFMA, capi.IMPL_MFMA64], ids=["mfma", "mfma64"])
 @pytest.mark.parametrize("dtype", [capi.BF16, capi.F16])
 def test_scores_far_above_the_first_tiles(gpu, dtype, impl, causal):
@@ -478,7 +478,16 @@ def test_scores_far_above_the_first_tiles(gpu, dtype, impl, causal):
     b[:, 1, 100] = 8.0                                       # head 1: the largest class already in the second tile
     k = np.broadcast_to(b, (B, H, S, D)).copy()
     v = dtypes.round_to(r.standard_normal((B, H, S, D), dtype=np.float32), dtype)
-    got, info = host.sdpa(q, k, v, dtype, causal=causal, impl=impl, return_info=True)
+    if causal == "tensor":
+        # the causal mask the way the reference's operator takes it: the dense-mask instance of the kernel, whose
+        # mask-free stretch of tiles runs the same bit check
+        if impl == capi.IMPL_MFMA64:
+            pytest.skip("the 64-row kernel takes no dense mask")
+        mask = O.causal_additive_mask(S, S).reshape(1, 1, S, S)
+        got, info = host.sdpa(q, k, v, dtype, mask=mask, impl=impl, return_info=True)
+        causal = True
+    else:
+        got, info = host.sdpa(q, k, v, dtype, causal=causal, impl=impl, return_info=True)
     assert info["impl"] == impl
     ref = oracle_full(q, k, v, causal=causal)
     check(got, ref, TOL[dtype], "scores far above the first tiles")
