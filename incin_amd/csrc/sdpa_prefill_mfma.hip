@@ -62,6 +62,7 @@
 // 2^62 below the reference flush to zero, which is far below what bf16 resolves.  The vector ALU
 // instructions saved are the point: on N(0,1) inputs this kernel is limited by power (the same
 // launch on zero inputs runs 1.4 times faster), and every instruction not issued is clock gained.
+#include <cstdlib>
 #include <type_traits>
 
 #include "sdpa_mfma_common.h"
@@ -75,8 +76,10 @@ namespace incin_rocm {
 #define PF_VD 4     // V operand reads run this many MFMAs ahead
 #endif
 
-template <typename T, int D, bool DENSE>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+// NW wavefronts = 32 * NW query rows per workgroup: 4 (two workgroups per compute unit) or 8 (one, whose K / V tiles then
+// serve 256 rows: half the global -> LDS copies per matrix instruction).
+template <typename T, int D, bool DENSE, int NW>
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void sdpa_prefill_mfma_kernel(SdpaParams p)
 {
 #if defined(__HIP_DEVICE_COMPILE__)   // the body uses device-only types (buffer descriptors); the host pass needs only the stub
@@ -84,7 +87,8 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     typedef PfLayout<D> L;
     constexpr int NSTEP = D / 16;          // k-steps of the S^T product
     constexpr int NDB = D / 32;            // 32-wide blocks of the head dimension
-    constexpr int LPW = L::LOADS_PER_WAVE;
+    constexpr int LPW = L::TILE_BYTES / 1024 / NW;     // wavefront-wide 1 KiB copies per tensor per tile
+    constexpr int BM = 32 * NW;                        // query rows per workgroup
     // bf16 without a dense mask: probabilities are taken 2^-SHIFT times smaller, so that "some probability reached 2"
     // - one bit of the packed values - says that a score passed the reference by more than 2^SHIFT
     constexpr bool BF16 = std::is_same<T, bf16_t>::value;
@@ -101,14 +105,14 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     // ---- which (batch, head, query block) -----------------------------------
     // Workgroups reach the 8 XCDs round-robin by id; hand each XCD a contiguous
     // range of the work list so heads that share K/V stay in one L2.
-    const int nqb = (Sq + PF_BM - 1) / PF_BM;
+    const int nqb = (Sq + BM - 1) / BM;
     const int total = gridDim.x;
     const WorkItem wi = (total & 7) == 0 ? work_item_of_share(blockIdx.x & 7, blockIdx.x >> 3, total >> 3, p.interleave, p.G, nqb, p.deal_groups)
                                          : work_item(blockIdx.x, p.interleave, p.G, nqb);
     const int gq = wi.gq, qb = wi.qblk, bhkv = wi.bhkv;
     const int hkv = bhkv % p.Hkv, b = bhkv / p.Hkv;
     const int hq = hkv * p.G + gq;
-    const int q0 = qb * PF_BM;
+    const int q0 = qb * BM;
 
     const T* qp = (const T*)p.q + (int64_t)b * p.q_sb + (int64_t)hq * p.q_sh;
     const T* kp = (const T*)p.k + (int64_t)b * p.k_sb + (int64_t)hkv * p.k_sh;
@@ -126,7 +130,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     const int my_i = q0 + wave * 32 + ql;
     int lim_lane = kv_len, lim_wave_min = kv_len, lim_wave_max = kv_len;
     if (p.causal) {
-        const int last_row = min(q0 + PF_BM - 1, rows_b - 1);
+        const int last_row = min(q0 + BM - 1, rows_b - 1);
         j_end = clampi(last_row + coff + 1, 0, kv_len);
         lim_lane = clampi(my_i + coff + 1, 0, kv_len);
         lim_wave_min = clampi(q0 + wave * 32 + coff + 1, 0, kv_len);
@@ -144,11 +148,11 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     int t_first = 0;
     [[maybe_unused]] int w_first = 0, w_last = 0x7fffffff;      // this wavefront's first and last tile with a visible block
     [[maybe_unused]] int z_end = 0;
-    __shared__ int s_range[8];
+    __shared__ int s_range[2 * NW];
     // the flags of this wavefront's tiles, two per tile, kept in LDS when they fit (up to 32768 keys): a flag is on
     // the path of every tile, and a global load there costs a memory latency per tile
     constexpr int FLAG_TILES = 512;
-    __shared__ uint8_t s_flags[DENSE ? 4 * 2 * FLAG_TILES : 4];
+    __shared__ uint8_t s_flags[DENSE ? NW * 2 * FLAG_TILES : 4];
     const bool flags_in_lds = DENSE && n_tiles <= FLAG_TILES;
     if (DENSE) {
         mflags = mask_flags_of(p, b, hq) + (int64_t)((q0 >> 5) + wave) * nkb32;
@@ -167,10 +171,11 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
         }
         w_first = __builtin_amdgcn_readfirstlane(lo);
         w_last = __builtin_amdgcn_readfirstlane(hi);
-        if (lane == 0) { s_range[wave] = lo; s_range[4 + wave] = hi; }
+        if (lane == 0) { s_range[wave] = lo; s_range[NW + wave] = hi; }
         __syncthreads();
-        const int g_lo = min(min(s_range[0], s_range[1]), min(s_range[2], s_range[3]));
-        const int g_hi = max(max(s_range[4], s_range[5]), max(s_range[6], s_range[7]));
+        int g_lo = s_range[0], g_hi = s_range[NW];
+#pragma unroll
+        for (int w2 = 1; w2 < NW; ++w2) { g_lo = min(g_lo, s_range[w2]); g_hi = max(g_hi, s_range[NW + w2]); }
         // (uniform by construction; said explicitly, because tile numbers end up in scalar DMA descriptors)
         t_first = __builtin_amdgcn_readfirstlane(g_hi < 0 ? 0 : g_lo);
         n_tiles = __builtin_amdgcn_readfirstlane(g_hi + 1);      // (0 when the mask hides everything from these 128 rows)
@@ -760,17 +765,35 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
 #endif
 }
 
-template <typename T, int D, bool DENSE>
-static hipError_t launch_prefill_t(const SdpaParams& p0, hipStream_t stream)
+template <typename T, int D, bool DENSE, int NW>
+static hipError_t launch_prefill_nw(const SdpaParams& p0, hipStream_t stream)
 {
     SdpaParams p = p0;
-    const int nqb = (p.Sq + PF_BM - 1) / PF_BM;
+    const int nqb = (p.Sq + 32 * NW - 1) / (32 * NW);
     const int64_t total = (int64_t)nqb * p.Hq * p.B;
-    // two workgroups per CU (register budget), an eighth of the CUs per XCD
-    p.interleave = work_interleave(p.causal != 0, 2 * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
+    // 256 registers per lane: eight wavefronts per compute unit, i.e. two workgroups of four or one of eight; an eighth
+    // of the compute units per XCD
+    p.interleave = work_interleave(p.causal != 0, (8 / NW) * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
     p.deal_groups = (total & 7) == 0 ? work_deal(p.interleave, p.G, nqb, total >> 3) : 0;
-    hipLaunchKernelGGL((sdpa_prefill_mfma_kernel<T, D, DENSE>), dim3((unsigned)total), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((sdpa_prefill_mfma_kernel<T, D, DENSE, NW>), dim3((unsigned)total), dim3(64 * NW), 0, stream, p);
     return hipGetLastError();
+}
+
+// 256-row workgroups where there is work enough for them (measured: level with 128-row workgroups at six 256-row blocks per
+// compute unit and 2048 keys, 2 - 3.5 % ahead from 4096 keys on, far behind when the launch does not fill the device) -
+// head dimension 128 without a dense mask; 128-row workgroups otherwise.
+template <typename T, int D, bool DENSE>
+static hipError_t launch_prefill_t(const SdpaParams& p, hipStream_t stream)
+{
+    if constexpr (D == 128 && !DENSE) {
+        // INCIN_ROCM_PREFILL_BLOCK_ROWS = 128 or 256 overrides the rule (for tests: small shapes through the 256-row form)
+        const char* forced = getenv("INCIN_ROCM_PREFILL_BLOCK_ROWS");
+        const int rows = forced ? atoi(forced) : 0;
+        const int64_t blocks256 = (int64_t)((p.Sq + 255) / 256) * p.Hq * p.B;
+        if (rows == 256 || (rows != 128 && p.Skv >= 4096 && blocks256 >= 6 * (int64_t)device_cus()))
+            return launch_prefill_nw<T, D, DENSE, 8>(p, stream);
+    }
+    return launch_prefill_nw<T, D, DENSE, 4>(p, stream);
 }
 
 // Host has validated: dtype f16/bf16, D == Dv in {64,128}, scale > 0, rows 16-byte aligned with unit last-dim stride, row strides below 2^24

@@ -457,10 +457,45 @@ def test_large_logits(gpu, dtype, impl, sq):
     check(got, oracle_full(q, k, v), TOL[dtype], "large logits")
 
 
+@pytest.mark.parametrize("dtype", [capi.BF16, capi.F16])
+@pytest.mark.parametrize("shape", [
+    # B, Hq, Hkv, Sq, Skv, causal, kv_lens, q_lens
+    (1, 2, 2, 640, 640, True, None, None),
+    (1, 2, 1, 700, 700, False, None, None),                       # rows and keys not multiples of the blocks
+    (2, 4, 2, 513, 900, True, [900, 311], None),                  # Sq < Skv: causal alignment; ragged keys
+    (2, 2, 2, 900, 300, True, None, None),                        # Sq > Skv: rows without keys
+    (3, 2, 2, 768, 768, True, [768, 200, 0], [768, 200, 0]),      # a padded batch: padding rows, an empty sequence
+    (1, 1, 1, 255, 257, False, [129], None),
+], ids=["square", "ragged_edges", "gqa_lens", "rows_without_keys", "padded_batch", "short"])
+def test_256_row_workgroups(gpu, dtype, shape, monkeypatch):
+    """The 16-bit prefill kernel runs with 128 or 256 query rows per workgroup (the launcher picks by the size of the
+    problem; INCIN_ROCM_PREFILL_BLOCK_ROWS forces one).  A row's arithmetic does not depend on which: both forms must agree
+    bit for bit on every valid row, normalisers included, and with the oracle."""
+    B, Hq, Hkv, Sq, Skv, causal, kv_lens, q_lens = shape
+    q, k, v = inputs(700 + Sq + Skv, B, Hq, Hkv, Sq, Skv, 128, 128, dtype)
+    kl = None if kv_lens is None else np.asarray(kv_lens, np.int32)
+    qlens = None if q_lens is None else np.asarray(q_lens, np.int32)
+    outs = {}
+    for rows in ("128", "256"):
+        monkeypatch.setenv("INCIN_ROCM_PREFILL_BLOCK_ROWS", rows)
+        outs[rows] = host.sdpa(q, k, v, dtype, causal=causal, kv_lens=kl, q_lens=qlens, impl=capi.IMPL_MFMA, return_lse=True)
+    monkeypatch.delenv("INCIN_ROCM_PREFILL_BLOCK_ROWS")
+    (o128, l128), (o256, l256) = outs["128"], outs["256"]
+    valid = np.ones((B, Hq, Sq), bool)
+    if qlens is not None:
+        valid &= np.arange(Sq)[None, None, :] < qlens[:, None, None]
+    assert np.array_equal(o128[valid], o256[valid], equal_nan=True)
+    assert np.array_equal(l128[valid], l256[valid], equal_nan=True)
+    ref = oracle_full(q, k, v, G=Hq // Hkv, causal=causal, kv_lens=kl)
+    got = np.where(valid[..., None], o256, ref)
+    check(got, ref, TOL[dtype], "256-row workgroups %r" % (shape,))
+
+
 @pytest.mark.parametrize("causal", [False, True, "tensor"], ids=["full", "causal", "causal_as_tensor"])
 @pytest.mark.parametrize("impl", [capi.IMPL_MFMA, capi.IMPL_MFMA64], ids=["mfma", "mfma64"])
 @pytest.mark.parametrize("dtype", [capi.BF16, capi.F16])
-def test_scores_far_above_the_first_tiles(gpu, dtype, impl, causal):
+@pytest.mark.parametrize("rows", ["128", "256"])
+def test_scores_far_above_the_first_tiles(gpu, dtype, impl, causal, rows, monkeypatch):
     """Keys whose logits lie 60 to 130 units above everything a row has seen before, in the second, the fourth and the
     seventh key tile: the reference maximum a kernel carries from earlier tiles is useless there.  The 16-bit prefill
     kernel takes no maxima in its pipelined loop for bf16 (it watches one bit of the probabilities instead) and has to
@@ -468,6 +503,9 @@ def test_scores_far_above_the_first_tiles(gpu, dtype, impl, causal):
     130 units below their maximum and must not notice at all, and rows of half the magnitude stay under the trigger
     while sharing a wavefront with rows that pull it.  Keys of one class are identical, so every row's answer is a
     plain mean of V rows and the rounding of the pre-scaled queries cannot matter."""
+    if rows == "256" and (impl != capi.IMPL_MFMA or causal == "tensor"):
+        pytest.skip("256-row workgroups: the 32-row kernel without a dense mask")
+    monkeypatch.setenv("INCIN_ROCM_PREFILL_BLOCK_ROWS", rows)
     B, H, S, D = 1, 2, 640, 128
     r = rng(SEED0 + 93)
     a = r.choice(np.array([1.0, -1.0, 0.5], np.float32), size=(B, H, S, 1))
