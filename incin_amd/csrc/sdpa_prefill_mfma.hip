@@ -781,7 +781,8 @@ static hipError_t launch_prefill_nw(const SdpaParams& p0, hipStream_t stream)
 
 // 256-row workgroups where there is work enough for them (measured: level with 128-row workgroups at six 256-row blocks per
 // compute unit and 2048 keys, 2 - 3.5 % ahead from 4096 keys on, far behind when the launch does not fill the device) -
-// head dimension 128 without a dense mask; 128-row workgroups otherwise.
+// head dimension 128 without a dense mask (with one the 256-row form is 6 % behind: the wavefronts of a workgroup see
+// different stretches of the mask and wait for each other at every tile); 128-row workgroups otherwise.
 template <typename T, int D, bool DENSE>
 static hipError_t launch_prefill_t(const SdpaParams& p, hipStream_t stream)
 {
