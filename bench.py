@@ -34,7 +34,7 @@ PEAK_HBM_GBS = 8000.0       # HBM3E, vendor figure
 # FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0 after calibration against the 1 GiB copy kernel): profiles/*.txt
 PREFILL_TRAFFIC_BYTES = (273324 * 2.0 + 131085) * 1024     # 6.94e8: |Q|+|K|+|V| read 1.39 times, |O| written once
 DECODE_TRAFFIC_BYTES = (2097470 * 2.0 + 1088 + 256) * 1024  # 4.297e9: K and V read once + split partials
-PREFILL_LONG_TRAFFIC_BYTES = (493652 * 2.0 + 318987) * 1024    # 1.34e9: valid |O| written once, inputs read 2.1 times
+PREFILL_LONG_TRAFFIC_BYTES = (537192 * 2.0 + 318930) * 1024    # 1.43e9: valid |O| written once, inputs read 2.2 times
 # These three are constants taken from counter runs, not measured by this script: each roofline object says so and
 # names the summary the figures come from.
 TRAFFIC_SOURCE = {
