@@ -296,6 +296,32 @@ def matrix_rate():
                                                        "frac_of_nominal": fl / (best * 1e-3) / 1e12 / PEAK_BF16_TFLOPS}
         src.free()
     sink.free()
+    # the attention kernel itself, same launch (configuration 3), by what its inputs hold: N(0,1) (the headline figure),
+    # the same values scaled by 0.01 (near-uniform probabilities) and zeros - identical instruction stream and traffic
+    B, H, S, D = 8, 16, 4096, 128
+    flops = causal_flops(B, H, S, S, D)
+    r = rng(SEED0 + 10)
+    x = r.standard_normal((B, H, S, D), dtype=np.float32)
+    by_data = {}
+    for name, scale in (("normal", 1.0), ("normal_times_0.01", 0.01), ("zeros", 0.0)):
+        tq, tk, tv = (host.DeviceTensor.from_f32(np.roll(x, sh, axis=2) * np.float32(scale), capi.BF16) for sh in (0, 1, 2))
+        to = host.DeviceTensor((B, H, S, D), capi.BF16)
+        d = host.make_desc(tq, tk, tv, to, causal=True)
+        for _ in range(120):
+            capi.sdpa_fwd(d)
+        capi.sync()
+        e0, e1 = capi.Event(), capi.Event()
+        e0.record()
+        for _ in range(60):
+            capi.sdpa_fwd(d)
+        e1.record()
+        capi.sync()
+        ms = e0.elapsed_ms(e1) / 60
+        e0.destroy(); e1.destroy()
+        by_data[name] = {"ms_per_launch": ms, "value": flops / (ms * 1e-3) / 1e12}
+        for t in (tq, tk, tv, to):
+            t.buf.free()
+    out["prefill_config3_by_input_data"] = by_data
     return out
 
 
