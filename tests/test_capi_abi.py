@@ -122,6 +122,18 @@ def test_null_descriptor_and_missing_workspace():
     assert lib.incin_rocm_device_count(None) == capi.EINVAL
 
 
+def test_matrix_rate_validation():
+    # the diagnostic refuses malformed requests before any device is touched
+    import ctypes as C
+    lib = capi.load()
+    fl = C.c_double(0.0)
+    assert lib.incin_rocm_matrix_rate(0, None, 0x1000, 0, 10, C.byref(fl), None) == capi.EINVAL
+    assert lib.incin_rocm_matrix_rate(0, 0x1000, 0x1000, 0, 10, None, None) == capi.EINVAL
+    assert lib.incin_rocm_matrix_rate(0, 0x1000, 0x1000, 2, 10, C.byref(fl), None) == capi.EINVAL
+    assert lib.incin_rocm_matrix_rate(0, 0x1000, 0x1000, 0, 0, C.byref(fl), None) == capi.EINVAL
+    assert b"matrix_rate" in lib.incin_rocm_last_error()
+
+
 def _bwd(fwd_kw=None, **kw):
     bd = capi.SdpaBwdDesc()
     bd.fwd = _desc(**{**dict(lse=0x30000), **(fwd_kw or {})})
