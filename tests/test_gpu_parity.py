@@ -538,6 +538,19 @@ def test_scores_far_above_the_first_tiles(gpu, dtype, impl, causal, rows, monkey
     check(got, mean.astype(np.float32), TOL[dtype], "scores far above the first tiles, closed form")
 
 
+def test_matrix_rate_diagnostic(gpu):
+    """The matrix-instruction loop behind bench.py's matrix_rate figures: it runs, and counts its own work."""
+    info = capi.device_info(0)
+    sink = capi.DeviceBuffer(2048 * info.compute_units)
+    src = capi.DeviceBuffer.from_numpy(np.zeros(65536, np.uint32))
+    for mix in (0, 1):
+        fl = capi.matrix_rate(src, sink, mix, 100)
+        capi.sync()
+        assert fl == info.compute_units * 8 * 100 * 4 * 32768.0
+    src.free()
+    sink.free()
+
+
 def test_copy_strided_gathers_any_view(gpu):
     """incin_rocm_copy_strided against numpy's own view semantics: transposes of the last two axes and of outer axes,
     broadcast (stride 0) and reversed (negative stride) axes, offsets into a larger buffer, ranks 0 to 8, 2- and 4-byte
