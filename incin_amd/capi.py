@@ -15,7 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("INCIN_ROCM_LIBRARY") or os.path.join(_HERE, "lib", "libincin_rocm.so")
 
 F32, F16, BF16 = 0, 1, 2
-IMPL_AUTO, IMPL_GENERIC, IMPL_MFMA, IMPL_SPLITKV, IMPL_MFMA64 = 0, 1, 2, 3, 4
+IMPL_AUTO, IMPL_GENERIC, IMPL_MFMA, IMPL_SPLITKV, IMPL_MFMA64, IMPL_SPLITKV_MFMA = 0, 1, 2, 3, 4, 5
 OK, EINVAL, ESHAPE, EDTYPE, EDEVICE, ENOMEM, EWORKSPACE, EUNSUPPORTED, ERUNTIME = range(9)
 
 EXPORTS = [

@@ -4,6 +4,7 @@
 // request no GPU kernel covers is an error, never a host fallback.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <atomic>
 #include <cmath>
 #include <cstdarg>
@@ -25,6 +26,8 @@ hipError_t launch_matrix_rate(const void* src, void* sink, int mix, int iteratio
 hipError_t launch_sdpa_prefill_f32(const SdpaParams& p, hipStream_t stream);
 hipError_t launch_mask_classify(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_sdpa_decode(const SdpaParams& p, int dtype, hipStream_t stream);
+hipError_t launch_sdpa_decode_mfma(const SdpaParams& p, int dtype, hipStream_t stream);
+int decode_mfma_chunk_rows(int R);
 int decode_keys_per_tile(int dtype, int D, int R);
 }  // namespace incin_rocm
 
@@ -81,6 +84,23 @@ size_t dtype_size(int dtype) { return dtype == INCIN_ROCM_F32 ? 4 : 2; }
 
 constexpr size_t MFMA64_WS_BYTES = 256;     // work counters of one launch of the 64-row prefill kernel
 
+// Compute units of device `dev` (256 when it cannot be asked, e.g. a workspace query on a machine without a device:
+// only launch geometry depends on it).
+int compute_units_of(int dev)
+{
+    static std::atomic<int> cached[64];
+    if (dev < 0 || dev >= 64) return 256;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+            (void)hipGetLastError();
+            n = 256;
+        }
+        cached[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // What the dispatcher decided for one descriptor.
@@ -126,7 +146,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         return fail(INCIN_ROCM_ESHAPE, "scaled_dot_product_attention: batch and head counts are limited to 65535 per launch");
     if (!d->q || !d->o || (d->Skv > 0 && (!d->k || !d->v)))
         return fail(INCIN_ROCM_EINVAL, "scaled_dot_product_attention: null tensor pointer");
-    if (d->impl < INCIN_ROCM_IMPL_AUTO || d->impl > INCIN_ROCM_IMPL_MFMA64)
+    if (d->impl < INCIN_ROCM_IMPL_AUTO || d->impl > INCIN_ROCM_IMPL_SPLITKV_MFMA)
         return fail(INCIN_ROCM_EINVAL, "scaled_dot_product_attention: unknown impl %d", d->impl);
     if (d->num_splits < 0) return fail(INCIN_ROCM_EINVAL, "scaled_dot_product_attention: negative num_splits");
 
@@ -145,10 +165,24 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     const bool mfma64_ok = mfma_ok && !d->add_mask && d->dtype != INCIN_ROCM_F32 && d->D == 128 && (d->Skv + 512) * d->k_stride[2] * 2 < (1LL << 31) &&
                            (d->Skv + 512) * d->v_stride[2] * 2 < (1LL << 31);
     const bool split_ok = fast_ok && d->Sq <= 64;
+    // the matrix-core split-KV kernel: 16-bit storage, head dimension 128, tiles addressed like the prefill kernels'
+    const bool split_mfma_ok = split_ok && tile_off_ok && d->dtype != INCIN_ROCM_F32 && d->D == 128 && std::isfinite(d->scale);
 
     int impl = d->impl;
     if (impl == INCIN_ROCM_IMPL_AUTO) {
-        if (split_ok && R <= 8 && d->Skv >= 256 && !d->lse) impl = INCIN_ROCM_IMPL_SPLITKV;
+        // Few rows per KV head (query heads of the group x query positions) over a long cache: split-KV.  One row stays
+        // on the vector-ALU kernel; with more it runs out of arithmetic before it runs out of bandwidth (measured on
+        // 32 x 8 KV heads x 8192 keys: 83 / 82 / 77 / 76 / 54 % of the memory bandwidth at 1 / 2 / 3 / 4 / 5 rows, the
+        // matrix-core kernel 85 % at each), except over short caches, where the matrix-core kernel's one workgroup per
+        // compute unit has too little to stream.  Up to 64 rows the matrix-core kernel reads the cache once; beyond, once
+        // per 64 rows, which still beats the prefill kernel when that one would leave most of the device idle (it does
+        // not split the keys).
+        const int64_t prefill_wgs = d->B * d->Hq * ((d->Sq + 127) / 128);
+        if (split_mfma_ok && !d->lse && d->Skv >= 256 &&
+            ((R >= 2 && R <= 4 && d->Skv >= 1024) || (R >= 5 && R <= 64) ||
+             (R > 64 && d->Skv >= 2048 && prefill_wgs * 4 <= compute_units_of(d->device))))
+            impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
+        else if (split_ok && R <= 8 && d->Skv >= 256 && !d->lse) impl = INCIN_ROCM_IMPL_SPLITKV;
         // (the 64-row kernel is never picked: since the 32-row kernel stopped taking maxima in its pipelined loop it is
         // level with or ahead of it at every length measured, 4096 to 16384 keys, with and without a causal mask and
         // on ragged batches; INCIN_ROCM_IMPL_MFMA64 stays available by name)
@@ -162,8 +196,11 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     if (impl == INCIN_ROCM_IMPL_MFMA64 && !mfma64_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
                     "scaled_dot_product_attention: the 64-row MFMA kernel needs f16/bf16, what the MFMA kernel needs, D == Dv == 128, no dense mask and key/value slices below 2 GiB");
-    if (impl == INCIN_ROCM_IMPL_SPLITKV && d->lse)
-        return fail(INCIN_ROCM_EUNSUPPORTED, "scaled_dot_product_attention: the split-KV kernel does not write the row normalisers (lse)");
+    if ((impl == INCIN_ROCM_IMPL_SPLITKV || impl == INCIN_ROCM_IMPL_SPLITKV_MFMA) && d->lse)
+        return fail(INCIN_ROCM_EUNSUPPORTED, "scaled_dot_product_attention: the split-KV kernels do not write the row normalisers (lse)");
+    if (impl == INCIN_ROCM_IMPL_SPLITKV_MFMA && !split_mfma_ok)
+        return fail(INCIN_ROCM_EUNSUPPORTED,
+                    "scaled_dot_product_attention: the matrix-core split-KV kernel needs f16/bf16, D == Dv == 128, Sq <= 64, no dense mask, a finite scale and 16-byte aligned rows");
     if (impl == INCIN_ROCM_IMPL_SPLITKV && !split_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
                     "scaled_dot_product_attention: the split-KV kernel needs D == Dv in {64,128}, Sq <= 64, no dense mask and 16-byte aligned rows");
@@ -188,6 +225,37 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         }
         int64_t split_len = (d->Skv + splits - 1) / splits;
         split_len = (split_len + tile - 1) / tile * tile;
+        splits = (d->Skv + split_len - 1) / split_len;
+        if (splits > 65535) return fail(INCIN_ROCM_ESHAPE, "scaled_dot_product_attention: too many splits");
+        if (d->Hkv * nchunks > 65535) return fail(INCIN_ROCM_ESHAPE, "scaled_dot_product_attention: too many head groups for one launch");
+        plan->splits = (int)splits;
+        plan->split_len = (int)split_len;
+        plan->ws_bytes = splits > 1 ? (size_t)(d->B * d->Hq * d->Sq * splits) * (size_t)(d->Dv + 2) * sizeof(float) : 0;
+    }
+    if (impl == INCIN_ROCM_IMPL_SPLITKV_MFMA) {
+        // One workgroup per (batch, KV head, chunk of 32 or 64 rows, split), and a compute unit holds one at a time (its LDS is
+        // the ring of tiles in flight): the workgroups of a launch run in rounds of one per compute unit, all of equal
+        // length.  Take the number of splits that leaves the last round fullest, among those that keep at least 256
+        // keys per split, preferring fewer splits at equal filling (fewer partial results to combine).
+        const int64_t chunk = incin_rocm::decode_mfma_chunk_rows((int)std::min<int64_t>(R, 1 << 20));
+        const int64_t nchunks = (R + chunk - 1) / chunk;
+        const int64_t groups = d->B * d->Hkv * nchunks;
+        int64_t splits = d->num_splits;
+        if (splits == 0) {
+            const int64_t cus = compute_units_of(d->device);
+            const int64_t max_by_len = d->Skv / 256 > 0 ? d->Skv / 256 : 1;
+            const int64_t max_splits = std::min<int64_t>(max_by_len, std::max<int64_t>(1, 2 * cus / groups));
+            auto fill = [&](int64_t s) {
+                const int64_t wgs = groups * s, rounds = (wgs + cus - 1) / cus;
+                return (double)wgs / (double)(rounds * cus);
+            };
+            double best = 0.0;
+            for (int64_t s = 1; s <= max_splits; ++s) best = std::max(best, fill(s));
+            splits = 1;
+            while (splits < max_splits && fill(splits) < 0.98 * best) ++splits;
+        }
+        int64_t split_len = (d->Skv + splits - 1) / splits;
+        split_len = (split_len + 127) / 128 * 128;      // whole rounds of the four wavefronts' 32-key blocks
         splits = (d->Skv + split_len - 1) / split_len;
         if (splits > 65535) return fail(INCIN_ROCM_ESHAPE, "scaled_dot_product_attention: too many splits");
         if (d->Hkv * nchunks > 65535) return fail(INCIN_ROCM_ESHAPE, "scaled_dot_product_attention: too many head groups for one launch");
@@ -528,6 +596,7 @@ static int launch_fwd(const incin_rocm_sdpa_desc_t* desc, const Plan& plan, void
             break;
         case INCIN_ROCM_IMPL_MFMA64: e = incin_rocm::launch_sdpa_prefill_mfma64(p, desc->dtype, s); break;
         case INCIN_ROCM_IMPL_SPLITKV: e = incin_rocm::launch_sdpa_decode(p, desc->dtype, s); break;
+        case INCIN_ROCM_IMPL_SPLITKV_MFMA: e = incin_rocm::launch_sdpa_decode_mfma(p, desc->dtype, s); break;
         default: e = incin_rocm::launch_sdpa_generic(p, desc->dtype, s); break;
     }
     if (e != hipSuccess) return hip_fail(e, "attention kernel launch");

@@ -227,29 +227,90 @@ __global__ __launch_bounds__(256) void sdpa_decode_split_kernel(SdpaParams p)
     }
 }
 
-// One workgroup of D threads per (b, hq, i) row: rescale the partials of all
-// splits to their common max and normalise.
+// One workgroup per (b, hq, i) row: rescale the partials of all splits to their common maximum and normalise.  A
+// thread holds 4 consecutive output elements; the D / 4 threads of a group walk the splits group, group + NG, ..., so
+// that NG splits are read side by side (a launch with hundreds of splits and few rows would otherwise walk them one
+// after the other), and the groups' sums meet in LDS.  blockDim.x = NG * D / 4, a multiple of 64.
 template <typename T, int D>
-__global__ __launch_bounds__(D) void sdpa_combine_kernel(SdpaParams p)
+__global__ __launch_bounds__(256) void sdpa_combine_kernel(SdpaParams p)
 {
+    constexpr int TPR = D / 4;
+    constexpr int NG_MAX = 256 / TPR;
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    __shared__ float s_max[4];
+    __shared__ f4 s_acc[NG_MAX][TPR];
+    __shared__ float s_l[NG_MAX];
     const int64_t row = blockIdx.x;                    // (b * Hq + hq) * Sq + i
-    const int d = threadIdx.x;
+    const int tid = threadIdx.x;
+    const int ng = blockDim.x / TPR;
     const int i = (int)(row % p.Sq);
     const int64_t bh = row / p.Sq;
     const int hq = (int)(bh % p.Hq), b = (int)(bh / p.Hq);
     const float* ml = p.ws_ml + row * p.num_splits * 2;
     const float* ac = p.ws_acc + row * p.num_splits * D;
-    float M = -INFINITY;
-    for (int s = 0; s < p.num_splits; ++s) M = fmaxf(M, ml[s * 2]);
+    float m = -INFINITY;
+    for (int s = tid; s < p.num_splits; s += blockDim.x) m = fmaxf(m, ml[s * 2]);
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+    if ((tid & 63) == 0) s_max[tid >> 6] = m;
+    __syncthreads();
+    float M = s_max[0];
+    for (int w = 1; w < (int)(blockDim.x >> 6); ++w) M = fmaxf(M, s_max[w]);
     const float M_use = (M == -INFINITY) ? 0.0f : M;
-    float L = 0.0f, A = 0.0f;
-    for (int s = 0; s < p.num_splits; ++s) {
+    const int grp = tid / TPR, c = tid % TPR;
+    f4 A = {0.0f, 0.0f, 0.0f, 0.0f};
+    float L = 0.0f;
+    for (int s = grp; s < p.num_splits; s += ng) {
         const float w = Softexp<T>::ex(ml[s * 2] - M_use);
         L = fmaf(w, ml[s * 2 + 1], L);
-        A = fmaf(w, ac[s * D + d], A);
+        const f4 a = *(const f4*)(ac + (int64_t)s * D + 4 * c);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) A[e] = fmaf(w, a[e], A[e]);
     }
-    T* op = (T*)p.o + (int64_t)b * p.o_sb + (int64_t)hq * p.o_sh + (int64_t)i * p.o_ss;
-    op[d] = from_f32<T>(L == 0.0f ? __builtin_nanf("") : A / L);
+    s_acc[grp][c] = A;
+    if (c == 0) s_l[grp] = L;
+    __syncthreads();
+    if (tid < TPR) {
+        for (int g2 = 1; g2 < ng; ++g2) {
+            const f4 a = s_acc[g2][tid];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) A[e] += a[e];
+            L += s_l[g2];
+        }
+        typedef T vec4 __attribute__((ext_vector_type(4)));
+        vec4 w;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w[e] = from_f32<T>(L == 0.0f ? __builtin_nanf("") : A[e] / L);
+        T* op = (T*)p.o + (int64_t)b * p.o_sb + (int64_t)hq * p.o_sh + (int64_t)i * p.o_ss;
+        *(vec4*)(op + 4 * tid) = w;
+    }
+}
+
+template <typename T, int D>
+static hipError_t launch_combine_t(const SdpaParams& p, hipStream_t stream)
+{
+    constexpr int TPR = D / 4;
+    int ng = 64 / TPR;                                  // at least one wavefront
+    while (ng < 256 / TPR && ng < p.num_splits) ng *= 2;
+    hipLaunchKernelGGL((sdpa_combine_kernel<T, D>), dim3((unsigned)((int64_t)p.B * p.Hq * p.Sq)), dim3(ng * TPR), 0, stream, p);
+    return hipGetLastError();
+}
+
+// The partial results of a split-KV launch (D == Dv in {64, 128}) into the output.
+hipError_t launch_sdpa_combine(const SdpaParams& p, int dtype, hipStream_t stream)
+{
+    if (p.D == 128) {
+        switch (dtype) {
+            case 0: return launch_combine_t<float, 128>(p, stream);
+            case 1: return launch_combine_t<f16_t, 128>(p, stream);
+            default: return launch_combine_t<bf16_t, 128>(p, stream);
+        }
+    }
+    switch (dtype) {
+        case 0: return launch_combine_t<float, 64>(p, stream);
+        case 1: return launch_combine_t<f16_t, 64>(p, stream);
+        default: return launch_combine_t<bf16_t, 64>(p, stream);
+    }
 }
 
 template <typename T, int D, int RMAX, int U>
@@ -276,10 +337,7 @@ static hipError_t launch_decode_t(const SdpaParams& p, hipStream_t stream)
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, p);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
-    if (p.num_splits > 1) {
-        hipLaunchKernelGGL((sdpa_combine_kernel<T, D>), dim3((unsigned)((int64_t)p.B * p.Hq * p.Sq)), dim3(D), 0, stream, p);
-        e = hipGetLastError();
-    }
+    if (p.num_splits > 1) e = launch_combine_t<T, D>(p, stream);
     return e;
 }
 

@@ -1,0 +1,400 @@
+// Split-KV attention for the query rows that share one key/value head, on the gfx950 matrix cores (f16 / bf16,
+// D == Dv == 128): grouped-query decode, where the vector-ALU split-KV kernel runs out of arithmetic (it spends
+// ~24 vector instructions per query row on every 2 KiB of cache it reads), and short runs of query rows over a long
+// cache.  Same function as the other attention kernels (crates/incin-backends/src/cpu/ops/shape_ops.rs:1245-1269),
+// same partial-result format as the vector-ALU split-KV kernel, same combine kernel.
+//
+// The work is bound by the bandwidth of the cache reads, so the design serves the memory system first:
+//
+//   * one workgroup (4 wavefronts) per (batch, KV head, chunk of 32 or 64 query rows, split), one workgroup per compute
+//     unit.  The split's keys are dealt to the wavefronts in blocks of 32 (wavefront w takes blocks w, w + 4, ...), and
+//     a wavefront works through its blocks on its own: no barrier in the loop, nothing shared.  Each wavefront owns a
+//     ring of NSLOT 8 KiB slots in LDS that the K and V blocks pass through in the order they are needed
+//     (K0 V0 K1 V1 ...), filled straight from global memory (buffer_load ... lds, whole rows, 1 KiB per instruction);
+//     a slot is refilled the moment its block has been used, so NSLOT - 1 blocks per wavefront - 128 KiB per compute
+//     unit with five slots - are in flight at any time;
+//   * 32 rows are the 32 columns of S^T = K Q^T (v_mfma_f32_32x32x16, a lane owns one row's scores of the block; rows
+//     that do not exist are zero columns - matrix throughput is not what is scarce here), the softmax is the usual
+//     online one per wavefront, and O^T += V^T P^T takes V through transposing LDS reads; with 64 rows every K and V
+//     operand read from LDS serves two such products;
+//   * at the end the four wavefronts' (maximum, sum, O^T) meet once in LDS (the rings are done with by then) and
+//     wavefront w writes columns 32 w .. 32 w + 31 of every row.
+//
+// Rows: row r of a chunk is (query head hkv * G + r / Sq, position r % Sq) - the G heads of the group times the Sq
+// positions.  The scale is applied to the f32 scores (any sign), masks as -inf before the maximum.
+#include "sdpa_mfma_common.h"
+
+namespace incin_rocm {
+
+constexpr int DM_BLOCK = 32;            // keys per block
+constexpr int DM_SLOT_BYTES = DM_BLOCK * 256;
+#ifndef DM_NSLOT
+#define DM_NSLOT 5       // slots per wavefront: 4 wavefronts x 5 x 8 KiB = the 160 KiB of a compute unit
+#endif
+
+// One wavefront-wide global -> LDS copy of 64 x 16 bytes, as dma_copy16, marked non-temporal: every byte of the cache
+// is read once per launch, and leaving it out of the caches' replacement order is worth 12 - 13 points of the memory
+// bandwidth (measured on 32 x 32 heads x 8192 keys: 6.05 TB/s without the mark, 7.04 with it).
+#ifndef DM_CACHE
+#define DM_CACHE " nt"
+#endif
+__device__ __forceinline__ void dm_copy16(uint4v desc, unsigned lds_addr, int byte_offset)
+{
+    asm volatile("s_nop 0\n\tbuffer_load_dwordx4 %0, %1, 0 offen" DM_CACHE " lds" ::"v"(byte_offset), "s"(desc), "{m0}"(lds_addr) : "memory");
+}
+
+// All but the newest NSLOT - 1 copies of this wavefront (8 instructions each) have landed.
+template <int NSLOT> __device__ __forceinline__ void wait_oldest_copy()
+{
+    static_assert(NSLOT >= 3 && NSLOT <= 5, "s_waitcnt takes an immediate");
+    if (NSLOT == 5) asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
+    else if (NSLOT == 4) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+}
+
+template <typename T, int NSLOT, int NRB>
+__global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    constexpr int D = 128;
+    typedef typename Mma<T>::vec8 vec8;
+    typedef PfLayout<D> L;
+    constexpr int NSTEP = D / 16, NDB = D / 32;
+    constexpr int CPB = DM_SLOT_BYTES / 1024;          // wavefront-wide 1 KiB copies per block
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ql = lane & 31, g = lane >> 5;
+    const int Sq = p.Sq, Skv = p.Skv;
+    const int R = p.G * Sq;
+    constexpr int CHUNK = 32 * NRB;                    // rows per workgroup
+    const int nchunks = (R + CHUNK - 1) / CHUNK;
+    const int split = blockIdx.x;
+    const int hkv = blockIdx.y / nchunks, r0 = (blockIdx.y % nchunks) * CHUNK;
+    const int b = blockIdx.z;
+
+    int kv_len = Skv;
+    if (p.kv_lens) kv_len = clampi(p.kv_lens[b], 0, Skv);
+    const int k_begin = split * p.split_len;
+
+    // this lane's rows, one per block of 32 (lanes l and l + 32 share them), and the keys each may see inside this split
+    bool valid[NRB];
+    int hq[NRB], qi[NRB], lim[NRB];
+    int lim_hi = 0, lim_lo = 0x7fffffff;
+#pragma unroll
+    for (int rb = 0; rb < NRB; ++rb) {
+        const int row = r0 + 32 * rb + ql;
+        valid[rb] = row < R;
+        const int gq = valid[rb] ? row / Sq : 0;
+        qi[rb] = valid[rb] ? row % Sq : 0;
+        hq[rb] = hkv * p.G + gq;
+        int l = min(k_begin + p.split_len, kv_len);
+        if (p.causal) l = min(l, causal_limit(qi[rb], Sq, Skv));
+        lim[rb] = valid[rb] ? l : 0;
+        lim_hi = max(lim_hi, lim[rb]);
+        if (valid[rb]) lim_lo = min(lim_lo, l);
+    }
+#pragma unroll
+    for (int off = 16; off >= 1; off >>= 1) {
+        lim_hi = max(lim_hi, __shfl_xor(lim_hi, off, 64));
+        lim_lo = min(lim_lo, __shfl_xor(lim_lo, off, 64));
+    }
+    const int k_end = __builtin_amdgcn_readfirstlane(lim_hi);          // rows at and beyond are never read
+    const int mask_from = __builtin_amdgcn_readfirstlane(lim_lo);      // blocks that end at or before need no mask
+    const int n_blocks = k_end > k_begin ? (k_end - k_begin + DM_BLOCK - 1) / DM_BLOCK : 0;
+    const int my_blocks = n_blocks > wave ? (n_blocks - wave + 3) >> 2 : 0;      // blocks wave, wave + 4, ...
+
+    // ---- global -> LDS copy plan (rows of 256 bytes, chunk slot c ^ f(row) as in the prefill kernels' tiles) ---------
+    int k_voff[CPB], v_voff[CPB];
+#pragma unroll
+    for (int c = 0; c < CPB; ++c) {
+        const int pos = c * 64 + lane;
+        const int r = pos / L::CPR, slot = pos % L::CPR;
+        k_voff[c] = r * (int)p.k_ss * 2 + (slot ^ L::fk(r)) * 16;
+        v_voff[c] = r * (int)p.v_ss * 2 + (slot ^ L::fv(r)) * 16;
+    }
+    const T* kp = (const T*)p.k + (int64_t)b * p.k_sb + (int64_t)hkv * p.k_sh;
+    const T* vp = (const T*)p.v + (int64_t)b * p.v_sb + (int64_t)hkv * p.v_sh;
+    // The copies of this wavefront go K(block 0) V(0) K(1) V(1) ...; copy number n lands in slot n % NSLOT.  Address of
+    // the next block of each tensor and the bytes from there to the end of row k_end - 1 (loads past that deliver
+    // zeros: what an unwritten cache tail holds never enters LDS).
+    const int64_t k_step = (int64_t)4 * DM_BLOCK * p.k_ss * 2, v_step = (int64_t)4 * DM_BLOCK * p.v_ss * 2;
+    const int first_key = k_begin + wave * DM_BLOCK;
+    const char* k_next = (const char*)kp + (int64_t)first_key * p.k_ss * 2;
+    const char* v_next = (const char*)vp + (int64_t)first_key * p.v_ss * 2;
+    int64_t k_rem = (int64_t)(k_end - first_key - 1) * p.k_ss * 2 + D * 2;
+    int64_t v_rem = (int64_t)(k_end - first_key - 1) * p.v_ss * 2 + D * 2;
+    // bytes a descriptor may cover: none once the tensor's blocks are used up, 2^31 - 1 at most
+    auto clamp31 = [](int64_t x) __attribute__((always_inline)) {
+        const unsigned hi = (unsigned)((unsigned long long)x >> 32), lo = (unsigned)x;
+        return x <= 0 ? 0 : (hi | (lo >> 31)) != 0 ? 0x7fffffff : (int)lo;
+    };
+    const unsigned ring = lds_address(smem) + wave * NSLOT * DM_SLOT_BYTES;
+    // Copies are started unconditionally, NSLOT ahead of their use: past the wavefront's last block the descriptor
+    // covers nothing, such a copy fetches nothing and delivers zeros into a slot nobody reads any more - which keeps the
+    // count of copies in flight, and with it the wait for the oldest, the same from the first block to the last.
+    int issued = 0, slot_in = 0;
+    auto issue_next = [&]() __attribute__((always_inline)) {
+        const unsigned dst = ring + slot_in * DM_SLOT_BYTES;
+        if ((issued & 1) == 0) {
+            const uint4v rk = dma_descriptor(k_next, clamp31(k_rem));
+#pragma unroll
+            for (int c = 0; c < CPB; ++c) dm_copy16(rk, dst + c * 1024, k_voff[c]);
+            k_next += k_step;
+            k_rem -= k_step;
+        } else {
+            const uint4v rv = dma_descriptor(v_next, clamp31(v_rem));
+#pragma unroll
+            for (int c = 0; c < CPB; ++c) dm_copy16(rv, dst + c * 1024, v_voff[c]);
+            v_next += v_step;
+            v_rem -= v_step;
+        }
+        ++issued;
+        slot_in = slot_in + 1 == NSLOT ? 0 : slot_in + 1;
+    };
+    for (int u = 0; u < NSLOT; ++u) issue_next();
+
+    // ---- operands ----------------------------------------------------------------------------------------------
+    // Q^T (B operand, resident): this lane's row, elements 16 s + 8 g .. + 7 of it per k-step s
+    vec8 qreg[NRB][NSTEP];
+#pragma unroll
+    for (int rb = 0; rb < NRB; ++rb) {
+        const T* qrow = (const T*)p.q + (int64_t)b * p.q_sb + (int64_t)hq[rb] * p.q_sh + (int64_t)qi[rb] * p.q_ss + g * 8;
+#pragma unroll
+        for (int s = 0; s < NSTEP; ++s) {
+            qreg[rb][s] = *(const vec8*)(qrow + s * 16);
+            if (!valid[rb])
+#pragma unroll
+                for (int e = 0; e < 8; ++e) qreg[rb][s][e] = (T)0.0f;
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0), told to the compiler too: the Q rows (and the first copies) have arrived
+    asm volatile("" ::: "memory");
+    // K operand: lane (ql, g) reads row ql, logical chunk 2 s + g
+    int k_addr[NSTEP];
+    {
+        const int F = L::fk(ql);
+#pragma unroll
+        for (int s = 0; s < NSTEP; ++s) k_addr[s] = ql * L::ROWB + (((2 * s + g) ^ F) << 4);
+    }
+    // V operand (transposing read): the 16 lanes of a group fetch a 4-key x 16-d patch (lane n: key n / 4,
+    // d 4 (n % 4) .. + 3) and receive (d = n, keys 0 .. 3).  Row within a 16-row block: 8 h + 4 g + n / 4; logical chunk
+    // 4 db + 2 dh + (n % 4) / 2.
+    int v_addr[NDB][2];
+    {
+        const int n = lane & 15, dh = (lane >> 4) & 1;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int r = 8 * h + 4 * g + (n >> 2);
+                const int chunk = 4 * db + 2 * dh + ((n & 3) >> 1);
+                v_addr[db][h] = r * L::ROWB + ((chunk ^ L::fv(r)) << 4) + (n & 1) * 8;
+            }
+    }
+
+    const float sc2 = p.scale * 1.4426950408889634f;      // scores in log2 units
+    float m_run[NRB], l_run[NRB];
+    floatx16 o_acc[NRB][NDB];
+#pragma unroll
+    for (int rb = 0; rb < NRB; ++rb) {
+        m_run[rb] = -INFINITY;
+        l_run[rb] = 0.0f;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o_acc[rb][db][r] = 0.0f;
+    }
+
+    int slot_out = 0;              // slot of the copy consumed next
+    for (int j = 0; j < my_blocks; ++j) {
+        const int j0 = first_key + j * 4 * DM_BLOCK;
+        // ---- S^T = K Q^T ----
+        wait_oldest_copy<NSLOT>();
+        const char* kb = smem + (wave * NSLOT + slot_out) * DM_SLOT_BYTES;
+        slot_out = slot_out + 1 == NSLOT ? 0 : slot_out + 1;
+        floatx16 sacc[NRB];
+#pragma unroll
+        for (int rb = 0; rb < NRB; ++rb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sacc[rb][r] = 0.0f;
+#pragma unroll
+        for (int s = 0; s < NSTEP; ++s) {
+            const vec8 a = *(const vec8*)(kb + k_addr[s]);
+#pragma unroll
+            for (int rb = 0; rb < NRB; ++rb) sacc[rb] = Mma<T>::run(a, qreg[rb][s], sacc[rb]);
+        }
+        // (the matrix instructions above hold the block's values: its slot can take the next copy)
+#pragma unroll
+        for (int rb = 0; rb < NRB; ++rb) asm volatile("" : "+v"(sacc[rb]));
+        issue_next();
+        // register r is key j0 + 8 (r / 4) + 4 g + (r % 4)
+        const bool masked = j0 + DM_BLOCK > mask_from;
+        vec8 pb[NRB][2];
+#pragma unroll
+        for (int rb = 0; rb < NRB; ++rb) {
+            const int rel = lim[rb] - (j0 + 4 * g);
+            float tmax = -INFINITY;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float x = sacc[rb][r] * sc2;
+                if (masked && 8 * (r / 4) + (r % 4) >= rel) x = -INFINITY;
+                sacc[rb][r] = x;
+                tmax = fmaxf(tmax, x);
+            }
+            tmax = xor32_max(tmax);
+            const float m_new = fmaxf(m_run[rb], tmax);
+            const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f(m_run[rb] - m_use);
+            m_run[rb] = m_new;
+            // P^T in storage precision: element e of k-step ks is register 8 ks + e; the denominator is summed from
+            // the rounded values
+            float rsum = 0.0f;
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) pb[rb][ks][e] = (T)__builtin_amdgcn_exp2f(sacc[rb][8 * ks + e] - m_use);
+#pragma unroll
+                for (int e = 0; e < 8; e += 2) {
+                    typename Mma<T>::vec2 pr = {pb[rb][ks][e], pb[rb][ks][e + 1]};
+                    rsum = Mma<T>::add2(pr, rsum);
+                }
+            }
+            l_run[rb] = l_run[rb] * alpha + rsum;
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) o_acc[rb][db][r] *= alpha;
+        }
+        // ---- O^T += V^T P^T ----
+        wait_oldest_copy<NSLOT>();
+        const char* vb = smem + (wave * NSLOT + slot_out) * DM_SLOT_BYTES;
+        slot_out = slot_out + 1 == NSLOT ? 0 : slot_out + 1;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int db = 0; db < NDB; ++db) {
+                short8v av;
+                av.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((short4v __attribute__((address_space(3)))*)(vb + v_addr[db][0] + ks * 16 * L::ROWB));
+                av.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((short4v __attribute__((address_space(3)))*)(vb + v_addr[db][1] + ks * 16 * L::ROWB));
+#pragma unroll
+                for (int rb = 0; rb < NRB; ++rb) o_acc[rb][db] = Mma<T>::run(__builtin_bit_cast(vec8, av), pb[rb][ks], o_acc[rb][db]);
+            }
+#pragma unroll
+        for (int rb = 0; rb < NRB; ++rb) asm volatile("" : "+v"(o_acc[rb][0]), "+v"(o_acc[rb][1]), "+v"(o_acc[rb][2]), "+v"(o_acc[rb][3]));
+        issue_next();
+    }
+
+    // ---- the four wavefronts' results meet (the rings are done with) --------------------------------------------------
+    float* s_m = (float*)smem;                               // [4][CHUNK] maxima
+    float* s_l = s_m + 4 * CHUNK;                            // [4][CHUNK] sums, rescaled
+    float* s_o = s_l + 4 * CHUNK;                            // [4 wavefronts][NRB][NDB][16][64] O^T registers, rescaled
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // (the empty copies started past the last block too)
+    __syncthreads();
+#pragma unroll
+    for (int rb = 0; rb < NRB; ++rb)
+        if (g == 0) s_m[wave * CHUNK + 32 * rb + ql] = m_run[rb];
+    __syncthreads();
+    float M[NRB];
+#pragma unroll
+    for (int rb = 0; rb < NRB; ++rb) {
+        M[rb] = s_m[32 * rb + ql];
+#pragma unroll
+        for (int w = 1; w < 4; ++w) M[rb] = fmaxf(M[rb], s_m[w * CHUNK + 32 * rb + ql]);
+        const float M_use = (M[rb] == -INFINITY) ? 0.0f : M[rb];
+        const float f = __builtin_amdgcn_exp2f(m_run[rb] - M_use);
+        const float l_w = xor32_sum(l_run[rb]) * f;
+        if (g == 0) s_l[wave * CHUNK + 32 * rb + ql] = l_w;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s_o[(((wave * NRB + rb) * NDB + db) * 16 + r) * 64 + lane] = o_acc[rb][db][r] * f;
+    }
+    __syncthreads();
+    // ---- this wavefront's 32 columns of every row ----------------------------------------------------------------
+#pragma unroll
+    for (int rb = 0; rb < NRB; ++rb) {
+        if (!valid[rb]) continue;
+        float l_tot = 0.0f;
+        floatx16 o;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[r] = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            l_tot += s_l[w * CHUNK + 32 * rb + ql];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[r] += s_o[(((w * NRB + rb) * NDB + wave) * 16 + r) * 64 + lane];
+        }
+        if (p.num_splits == 1) {
+            const float inv = (l_tot == 0.0f) ? __builtin_nanf("") : 1.0f / l_tot;      // no visible key: NaN, as the reference
+            T* orow = (T*)p.o + (int64_t)b * p.o_sb + (int64_t)hq[rb] * p.o_sh + (int64_t)qi[rb] * p.o_ss + 32 * wave + 4 * g;
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                typedef T vec4 __attribute__((ext_vector_type(4)));
+                vec4 w;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) w[e] = (T)(o[r4 * 4 + e] * inv);
+                *(vec4*)(orow + r4 * 8) = w;
+            }
+        } else {
+            const int64_t slot = (((int64_t)b * p.Hq + hq[rb]) * Sq + qi[rb]) * p.num_splits + split;
+            float* arow = p.ws_acc + slot * D + 32 * wave + 4 * g;
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                typedef float f4 __attribute__((ext_vector_type(4)));
+                f4 w = {o[r4 * 4], o[r4 * 4 + 1], o[r4 * 4 + 2], o[r4 * 4 + 3]};
+                *(f4*)(arow + r4 * 8) = w;
+            }
+            if (wave == 0 && g == 0) {
+                p.ws_ml[slot * 2 + 0] = M[rb];      // log2 units, as the combine kernel takes them for 16-bit storage
+                p.ws_ml[slot * 2 + 1] = l_tot;
+            }
+        }
+    }
+#endif
+}
+
+hipError_t launch_sdpa_combine(const SdpaParams& p, int dtype, hipStream_t stream);
+
+template <typename T, int NSLOT, int NRB>
+static hipError_t launch_decode_mfma_t(const SdpaParams& p, hipStream_t stream)
+{
+    constexpr size_t lds = (size_t)4 * NSLOT * DM_SLOT_BYTES;
+    auto kern = sdpa_decode_mfma_kernel<T, NSLOT, NRB>;
+    // the dynamic-LDS limit of this instance is raised once per device, not per launch
+    static std::atomic<uint64_t> prepared{0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+    const uint64_t bit = 1ull << (dev & 63);
+    if (!(prepared.load(std::memory_order_acquire) & bit)) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        prepared.fetch_or(bit, std::memory_order_release);
+    }
+    const int R = p.G * p.Sq;
+    const int nchunks = (R + 32 * NRB - 1) / (32 * NRB);
+    dim3 grid(p.num_splits, p.Hkv * nchunks, p.B);
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, p);
+    return hipGetLastError();
+}
+
+// Rows a workgroup takes: 32, or 64 (two blocks of 32 against the same K and V operands) when more than 32 rows share a KV
+// head - the cache is then read once for 64 rows instead of once per 32.
+int decode_mfma_chunk_rows(int R) { return R > 32 ? 64 : 32; }
+
+// Host has validated: dtype f16 / bf16, D == Dv == 128, rows 16-byte aligned with unit last-dim stride, row strides
+// below 2^24 elements, split_len a multiple of 128 (every wavefront's blocks then start where its
+// neighbour's end in every split).
+hipError_t launch_sdpa_decode_mfma(const SdpaParams& p, int dtype, hipStream_t stream)
+{
+    hipError_t e;
+    if (decode_mfma_chunk_rows(p.G * p.Sq) == 64)
+        e = dtype == 1 ? launch_decode_mfma_t<f16_t, DM_NSLOT, 2>(p, stream) : launch_decode_mfma_t<bf16_t, DM_NSLOT, 2>(p, stream);
+    else
+        e = dtype == 1 ? launch_decode_mfma_t<f16_t, DM_NSLOT, 1>(p, stream) : launch_decode_mfma_t<bf16_t, DM_NSLOT, 1>(p, stream);
+    if (e != hipSuccess || p.num_splits == 1) return e;
+    return launch_sdpa_combine(p, dtype, stream);
+}
+
+}  // namespace incin_rocm

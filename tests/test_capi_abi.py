@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), "missing export %s" % n
     assert set(names) == set(capi.EXPORTS)
-    assert lib.incin_rocm_abi_version() == 5
+    assert lib.incin_rocm_abi_version() == 6
 
 
 def test_descriptor_layout_matches():
@@ -66,8 +66,25 @@ def test_dispatch_choices():
     nbytes, splits, impl = _plan(_desc(Sq=1, Skv=8192, B=32, Hq=32, Hkv=32))
     assert impl == capi.IMPL_SPLITKV and splits >= 1
     assert nbytes == (0 if splits == 1 else 32 * 32 * 1 * splits * (128 + 2) * 4)
+    # grouped-query decode, 4 rows per KV head: the matrix-core split-KV kernel (the vector-ALU one by name)
     nbytes, splits, impl = _plan(_desc(Sq=1, Skv=8192, B=1, Hq=8, Hkv=2, num_splits=4))
+    assert impl == capi.IMPL_SPLITKV_MFMA and splits == 4 and nbytes == 8 * 4 * 130 * 4
+    nbytes, splits, impl = _plan(_desc(Sq=1, Skv=8192, B=1, Hq=8, Hkv=2, num_splits=4, impl=capi.IMPL_SPLITKV))
     assert impl == capi.IMPL_SPLITKV and splits == 4 and nbytes == 8 * 4 * 130 * 4
+    # its split count fills the device's compute units once (256 here: no device to ask): 2 groups x 128 splits of 64 keys
+    # would, but a split keeps at least 256 keys
+    _, splits, impl = _plan(_desc(Sq=1, Skv=8192, B=1, Hq=8, Hkv=2))
+    assert impl == capi.IMPL_SPLITKV_MFMA and splits == 32
+    _, splits, impl = _plan(_desc(Sq=1, Skv=8192, B=32, Hq=32, Hkv=8))
+    assert impl == capi.IMPL_SPLITKV_MFMA and splits == 1                     # 256 groups: one round, nothing to combine
+    assert _plan(_desc(Sq=1, Skv=8192, B=2, Hq=8, Hkv=2, dtype=capi.F32))[2] == capi.IMPL_SPLITKV   # f32, D = 64: vector ALU
+    assert _plan(_desc(Sq=1, Skv=8192, B=2, Hq=8, Hkv=2, D=64, Dv=64))[2] == capi.IMPL_SPLITKV
+    assert _plan(_desc(Sq=4, Skv=8192, B=2, Hq=32, Hkv=2))[2] == capi.IMPL_SPLITKV_MFMA             # 64 rows per KV head: one workgroup's worth
+    assert _plan(_desc(Sq=8, Skv=8192, B=2, Hq=32, Hkv=2))[2] == capi.IMPL_SPLITKV_MFMA             # 128, but the prefill kernel would run 64 workgroups
+    assert _plan(_desc(Sq=8, Skv=8192, B=8, Hq=32, Hkv=2))[2] == capi.IMPL_MFMA                     # 256 of them: a prefill shape
+    assert _plan(_desc(Sq=1, Skv=512, B=2, Hq=8, Hkv=2))[2] == capi.IMPL_SPLITKV                    # 4 rows, short cache: vector ALU
+    assert _plan(_desc(Sq=1, Skv=512, B=2, Hq=16, Hkv=2))[2] == capi.IMPL_SPLITKV_MFMA              # 8 rows
+    assert _plan(_desc(Sq=1, Skv=8192, B=2, Hq=4, Hkv=2))[2] == capi.IMPL_SPLITKV_MFMA              # 2 rows, long cache
     assert _plan(_desc(Sq=1, Skv=64))[2] in (capi.IMPL_MFMA, capi.IMPL_SPLITKV)
     # long sequences: the 32-row kernel as well (the 64-row kernel is level with it or behind at every length; by name only)
     def long(**kw):
@@ -101,6 +118,10 @@ def test_dispatch_choices():
     (dict(impl=capi.IMPL_MFMA64, add_mask=0x20000), capi.EUNSUPPORTED),
     (dict(impl=capi.IMPL_MFMA, D=80, Dv=80), capi.EUNSUPPORTED),
     (dict(impl=capi.IMPL_SPLITKV, Sq=4096), capi.EUNSUPPORTED),
+    (dict(impl=capi.IMPL_SPLITKV_MFMA, Sq=4096), capi.EUNSUPPORTED),
+    (dict(impl=capi.IMPL_SPLITKV_MFMA, Sq=1, dtype=capi.F32), capi.EUNSUPPORTED),
+    (dict(impl=capi.IMPL_SPLITKV_MFMA, Sq=1, D=64, Dv=64), capi.EUNSUPPORTED),
+    (dict(impl=capi.IMPL_SPLITKV_MFMA, Sq=1, add_mask=0x20000), capi.EUNSUPPORTED),
     (dict(D=512, Dv=512), capi.EUNSUPPORTED),
     (dict(B=70000), capi.ESHAPE),
 ])

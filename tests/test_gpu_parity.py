@@ -385,6 +385,63 @@ def test_decode_splitkv(gpu, dtype, shape):
         check(o, outs[1], 1e-5 if dtype == capi.F32 else 8e-3, "decode split-count invariance")
 
 
+@pytest.mark.parametrize("dtype", [capi.BF16, capi.F16])
+@pytest.mark.parametrize("shape", [
+    # B, Hq, Hkv, Sq, Skv, causal
+    (2, 8, 2, 1, 4096, False),        # grouped-query decode, 4 rows per KV head
+    (1, 32, 4, 1, 3000, False),       # 8 rows, ragged last tile
+    (3, 16, 1, 1, 700, True),         # multi-query, 16 rows
+    (1, 8, 2, 5, 1500, True),         # 20 rows per KV head with a causal edge among the 5 positions
+    (1, 40, 1, 1, 333, False),        # 40 rows: two chunks of 32, the second mostly empty
+    (2, 12, 4, 9, 1000, True),        # 27 rows
+    (1, 4, 4, 40, 2500, True),        # one head per KV head, 40 positions: two chunks, causal
+    (1, 8, 8, 1, 200, False),         # a single row per KV head, fewer keys than a split asks for
+    (2, 64, 1, 1, 900, False),        # 64 rows: one workgroup of two 32-row blocks
+    (1, 16, 2, 9, 1200, True),        # 72 rows per KV head: two chunks of 64, the second with 8 rows
+    (1, 6, 2, 64, 1500, True),        # 192 rows per KV head: three chunks, causal over 64 positions
+])
+def test_decode_splitkv_matrix_cores(gpu, dtype, shape):
+    """The matrix-core split-KV kernel against the oracle, with the split count left to the library, forced to one
+    (the kernel writes the output itself) and forced to counts that leave ragged and empty last splits; and against
+    the vector-ALU split-KV kernel where that one takes the shape."""
+    B, Hq, Hkv, Sq, Skv, causal = shape
+    D = 128
+    q, k, v = inputs(700 + sum(shape[:5]), B, Hq, Hkv, Sq, Skv, D, D, dtype)
+    ref = oracle_full(q, k, v, G=Hq // Hkv, causal=causal)
+    outs = []
+    for splits in (0, 1, 3, 7, 40):
+        say("matrix-core split-KV: %s %r splits=%d" % (dtypes.NAMES[dtype], shape, splits))
+        got, info = host.sdpa(q, k, v, dtype, causal=causal, num_splits=splits, impl=capi.IMPL_SPLITKV_MFMA, return_info=True)
+        assert info["impl"] == capi.IMPL_SPLITKV_MFMA
+        check(got, ref, TOL[dtype], "matrix-core split-KV %s %r splits=%d->%d" % (dtypes.NAMES[dtype], shape, splits, info["splits"]))
+        outs.append(got)
+    for o in outs:
+        check(o, outs[1], 8e-3, "matrix-core split-KV: split-count invariance")
+    if (Hq // Hkv) * Sq <= 8:
+        valu = host.sdpa(q, k, v, dtype, causal=causal, impl=capi.IMPL_SPLITKV)
+        check(outs[0], valu, 8e-3, "matrix-core vs vector-ALU split-KV")
+
+
+def test_decode_splitkv_matrix_cores_lengths_strides_scale(gpu):
+    """Key counts per batch entry (one of them 0: NaN rows, as the reference), a negative scale (the scale is applied to
+    the f32 scores, so its sign does not matter to this kernel), and AUTO's choice for grouped-query decode."""
+    B, Hq, Hkv, Skv, D = 4, 16, 4, 1100, 128
+    q, k, v = inputs(733, B, Hq, Hkv, 1, Skv, D, D, capi.BF16)
+    lens = np.array([1100, 64, 0, 257], np.int32)
+    for splits in (0, 1, 5):
+        got, info = host.sdpa(q, k, v, capi.BF16, kv_lens=lens, num_splits=splits, impl=capi.IMPL_SPLITKV_MFMA, return_info=True)
+        ref = oracle_full(q, k, v, G=4, kv_lens=lens)
+        assert np.isnan(ref[2]).all()
+        check(got, ref, 2e-2, "matrix-core split-KV kv_lens incl. empty, splits=%d" % splits)
+    got = host.sdpa(q, k, v, capi.BF16, scale=-0.07, impl=capi.IMPL_SPLITKV_MFMA)
+    check(got, oracle_full(q, k, v, G=4, scale=-0.07), 2e-2, "matrix-core split-KV negative scale")
+    got, info = host.sdpa(q, k, v, capi.BF16, return_info=True)
+    assert info["impl"] == capi.IMPL_SPLITKV_MFMA           # 4 rows per KV head, 16-bit, D = 128: AUTO's choice
+    check(got, oracle_full(q, k, v, G=4), 2e-2, "AUTO grouped-query decode")
+    _, info = host.sdpa(q[:, :4], k, v, capi.BF16, return_info=True)
+    assert info["impl"] == capi.IMPL_SPLITKV                # one row per KV head stays on the vector-ALU kernel
+
+
 def test_decode_lengths_and_prefill_consistency(gpu):
     B, H, Skv, D = 3, 4, 2048, 128
     q, k, v = inputs(41, B, H, H, 1, Skv, D, D, capi.BF16)
@@ -405,8 +462,9 @@ def test_decode_lengths_and_prefill_consistency(gpu):
     pytest.param(capi.IMPL_MFMA64, capi.BF16, 200, marks=pytest.mark.skip(
         reason="this case did not finish on the device once in three runs (the launch of the 64-row kernel never completed; "
                "cause not found by reading the kernel): kept off the device until a cause can be shown")),
-    (capi.IMPL_MFMA, capi.F16, 200), (capi.IMPL_SPLITKV, capi.BF16, 1), (capi.IMPL_SPLITKV, capi.F32, 2)],
-    ids=["generic_f32", "generic_bf16", "mfma_bf16", "mfma64_bf16", "mfma_f16", "splitkv_bf16", "splitkv_f32"])
+    (capi.IMPL_MFMA, capi.F16, 200), (capi.IMPL_SPLITKV, capi.BF16, 1), (capi.IMPL_SPLITKV, capi.F32, 2),
+    (capi.IMPL_SPLITKV_MFMA, capi.BF16, 3), (capi.IMPL_SPLITKV_MFMA, capi.F16, 1)],
+    ids=["generic_f32", "generic_bf16", "mfma_bf16", "mfma64_bf16", "mfma_f16", "splitkv_bf16", "splitkv_f32", "splitkv_mfma_bf16", "splitkv_mfma_f16"])
 def test_rows_beyond_the_key_count_are_never_read(gpu, impl, dtype, sq):
     """A preallocated cache holds whatever the allocator left behind its valid rows.  With NaN and infinity bit patterns
     in every key and value row at and beyond kv_lens[b], each kernel gives the bytes it gives over a zeroed tail, and
@@ -423,7 +481,7 @@ def test_rows_beyond_the_key_count_are_never_read(gpu, impl, dtype, sq):
             fill = np.resize(junk, n * D).reshape(n, D)
             k_bad[b, :, lens[b]:], v_bad[b, :, lens[b]:] = fill, fill[::-1]
     say("junk beyond kv_lens: impl %d dtype %d" % (impl, dtype))
-    kw = dict(causal=False, kv_lens=lens, impl=impl, num_splits=3 if impl == capi.IMPL_SPLITKV else 0)
+    kw = dict(causal=False, kv_lens=lens, impl=impl, num_splits=3 if impl in (capi.IMPL_SPLITKV, capi.IMPL_SPLITKV_MFMA) else 0)
     clean, info = host.sdpa(q, k, v, dtype, return_info=True, **kw)
     assert info["impl"] == impl
     dirty = host.sdpa(q, k_bad, v_bad, dtype, **kw)
@@ -432,8 +490,9 @@ def test_rows_beyond_the_key_count_are_never_read(gpu, impl, dtype, sq):
     check(dirty, oracle_full(q, k, v, G=Hq // Hkv, kv_lens=lens), TOL[dtype], "junk tail")
 
 
-@pytest.mark.parametrize("impl, sq", [(capi.IMPL_MFMA, 96), (capi.IMPL_MFMA64, 96), (capi.IMPL_SPLITKV, 2), (capi.IMPL_GENERIC, 40)],
-                         ids=["mfma", "mfma64", "splitkv", "generic"])
+@pytest.mark.parametrize("impl, sq", [(capi.IMPL_MFMA, 96), (capi.IMPL_MFMA64, 96), (capi.IMPL_SPLITKV, 2), (capi.IMPL_GENERIC, 40),
+                                      (capi.IMPL_SPLITKV_MFMA, 6)],
+                         ids=["mfma", "mfma64", "splitkv", "generic", "splitkv_mfma"])
 @pytest.mark.parametrize("dtype", [capi.BF16, capi.F16])
 def test_large_logits(gpu, dtype, impl, sq):
     """Logits of magnitude 50 with many keys within a few units of each row's maximum, and query rows whose elements are
@@ -452,7 +511,7 @@ def test_large_logits(gpu, dtype, impl, sq):
     say("large logits: impl %d dtype %d, max |logit| %.1f, 8th-largest within %.2f of the row maximum (median)"
         % (impl, dtype, np.abs(logits).max(), np.median(top[..., -1] - top[..., 0])))
     assert np.abs(logits).max() > 45
-    got, info = host.sdpa(q, k, v, dtype, impl=impl, return_info=True, num_splits=2 if impl == capi.IMPL_SPLITKV else 0)
+    got, info = host.sdpa(q, k, v, dtype, impl=impl, return_info=True, num_splits=2 if impl in (capi.IMPL_SPLITKV, capi.IMPL_SPLITKV_MFMA) else 0)
     assert info["impl"] == impl
     check(got, oracle_full(q, k, v), TOL[dtype], "large logits")
 
