@@ -65,7 +65,7 @@ def causal_flops(B, Hq, Sq, Skv, D):
 class Workload:
     """Device-resident operands + descriptor for one configuration."""
 
-    def __init__(self, name, seed, B, Hq, Hkv, Sq, Skv, D, dtype, causal, kv_lens=None, pad_queries=False):
+    def __init__(self, name, seed, B, Hq, Hkv, Sq, Skv, D, dtype, causal, kv_lens=None, pad_queries=False, impl=capi.IMPL_AUTO):
         self.name, self.shape = name, (B, Hq, Hkv, Sq, Skv, D)
         self.dtype, self.causal, self.kv_lens = dtype, causal, kv_lens
         q, k, v = make_inputs(seed, B, Hq, Hkv, Sq, Skv, D, dtype)
@@ -75,7 +75,7 @@ class Workload:
         self.tl = capi.DeviceBuffer.from_numpy(np.asarray(kv_lens, dtype=np.int32)) if kv_lens is not None else None
         # a padded self-attention batch: the same lengths say which keys and which query rows are padding
         self.desc = host.make_desc(self.tq, self.tk, self.tv, self.to, causal=causal, kv_lens=self.tl,
-                                   q_lens=self.tl if pad_queries else None)
+                                   q_lens=self.tl if pad_queries else None, impl=impl)
         nbytes, self.splits, self.impl = capi.sdpa_workspace(self.desc)
         self.ws = capi.DeviceBuffer(nbytes) if nbytes else None
         if self.ws is not None:
@@ -177,6 +177,39 @@ def cpu_baseline_decode(D, Skv, B, H, dtype):
     O.sdpa_materialised(q, k, v)
     dt = time.perf_counter() - t0
     return 2.0 * B * H * Skv * D * 2 / dt / 1e9, dt
+
+
+def decode_gqa_leg(steps, warmup, only_shape=None):
+    """Decode shapes beyond BASELINE config 4, where several query rows share a KV head: grouped-query decode at config
+    4's batch and cache length, one long sequence, and a short run of query positions (causal among themselves).  Each
+    through the kernel AUTO picks (the matrix-core split-KV kernel) and, where it takes the shape, through the
+    vector-ALU split-KV kernel; KV bytes read once / launch time against the HBM peak."""
+    out = {}
+    shapes = [("gqa4_b32_kv8192", 32, 32, 8, 1, 8192, False), ("gqa4_b1_kv131072", 1, 32, 8, 1, 131072, False),
+              ("gqa8_b32_kv8192", 32, 64, 8, 1, 8192, False), ("gqa4_sq4_b8_kv8192", 8, 32, 8, 4, 8192, True)]
+    names = {capi.IMPL_SPLITKV: "sdpa_decode_split_kernel (vector ALU)", capi.IMPL_SPLITKV_MFMA: "sdpa_decode_mfma_kernel (matrix cores)",
+             capi.IMPL_MFMA: "sdpa_prefill_mfma_kernel"}
+    for i, (name, B, Hq, Hkv, Sq, Skv, causal) in enumerate(shapes):
+        if only_shape is not None and name != only_shape:
+            continue
+        kv_bytes = 2.0 * B * Hkv * Skv * 128 * 2
+        n = max(steps, min(200, int(0.02 / (kv_bytes / 6e12))))
+        entry = {"workload": "bf16 decode B=%d Hq=%d Hkv=%d S_q=%d KV=%d D=128%s" % (B, Hq, Hkv, Sq, Skv, " causal" if causal else "")}
+        for impl in (capi.IMPL_AUTO, capi.IMPL_SPLITKV):
+            if impl == capi.IMPL_SPLITKV and (Hq // Hkv) * Sq > 8:
+                continue
+            w = Workload("decode_" + name, SEED0 + 40 + i, B, Hq, Hkv, Sq, Skv, 128, capi.BF16, causal, impl=impl)
+            wall, ev_mean, ev_med, ev_min = w.time(n, warmup)
+            entry["auto" if impl == capi.IMPL_AUTO else "vector_alu_kernel"] = {
+                "kernel": names.get(w.impl, str(w.impl)), "num_splits": w.splits, "ms_per_step": wall,
+                "kv_gb_per_s": kv_bytes / (wall * 1e-3) / 1e9,
+                "roofline": {"bound": "hbm", "achieved": kv_bytes / (ev_mean * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                             "frac": kv_bytes / (ev_mean * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None,
+                             "algorithmic_bytes_per_launch": kv_bytes, "launch_ms_mean": ev_mean, "launch_ms_min": ev_min},
+                "parity_max_abs_err": w.parity(16)}
+            w.free()
+        out[name] = entry
+    return out
 
 
 def decode_step_graph(w, B, H, Skv, D, steps):
@@ -392,7 +425,8 @@ def main():
     ap.add_argument("--no-padding-compare", action="store_true",
                     help="prefill_long: skip the extra timing of the batch with its padding rows computed (profiling: every "
                          "launch of the run is then the same launch)")
-    ap.add_argument("--only", choices=["prefill", "prefill_long", "decode", "backward", "f32", "copy", "matrix_rate"], default=None,
+    ap.add_argument("--decode-gqa-shape", default=None, help="with --only decode_gqa: one of its shapes by name (for profiles)")
+    ap.add_argument("--only", choices=["prefill", "prefill_long", "decode", "decode_gqa", "backward", "f32", "copy", "matrix_rate"], default=None,
                     help="run a single workload (profiling). 'copy' runs --steps device-to-device copies of 1 GiB "
                          "through the library's plain copy kernel: the known-size dispatch that hardware byte "
                          "counters (FETCH_SIZE / WRITE_SIZE) are calibrated against")
@@ -508,17 +542,25 @@ def main():
         w = Workload("decode_c4", SEED0 + 3, B, H, H, 1, Skv, D, capi.BF16, False)
         wall, ev_mean, ev_med, ev_min = w.time(args.steps, args.warmup)
         kv_bytes = 2.0 * B * H * Skv * D * 2
-        dec = {"workload": "BASELINE config 4: bf16 decode MHA B=32 H=32 S_q=1 KV=8192 D=128, split-KV partials + combine",
+        dec = {"workload": "BASELINE config 4: bf16 decode MHA B=32 H=32 S_q=1 KV=8192 D=128",
                "metric": "decode KV GB/s", "value": kv_bytes / (wall * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": wall,
                "num_splits": w.splits,
                "roofline": {"bound": "hbm", "achieved": kv_bytes / (ev_mean * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                             "frac": kv_bytes / (ev_mean * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": DECODE_TRAFFIC_BYTES,
                             "traffic_source": TRAFFIC_SOURCE["decode"],
-                            "kernel": "sdpa_decode_split_kernel<bf16,128,1,8> + sdpa_combine_kernel",
+                            "kernel": {capi.IMPL_SPLITKV: "sdpa_decode_split_kernel<bf16,128,1,8> + sdpa_combine_kernel",
+                                       capi.IMPL_SPLITKV_MFMA: "sdpa_decode_mfma_kernel<bf16,5,1>"}.get(w.impl, str(w.impl)),
                             "algorithmic_bytes_per_launch": kv_bytes,
                             "launch_ms_mean": ev_mean, "launch_ms_median": ev_med, "launch_ms_min": ev_min},
                "parity_max_abs_err": w.parity()}
         dec["decode_step_graph"] = decode_step_graph(w, B, H, Skv, D, args.steps)
+        w.free()
+        # the same through the vector-ALU split-KV kernel (what f32 caches and short caches run on)
+        w = Workload("decode_c4", SEED0 + 3, B, H, H, 1, Skv, D, capi.BF16, False, impl=capi.IMPL_SPLITKV)
+        wall_v, ev_v, _, _ = w.time(args.steps, args.warmup)
+        dec["vector_alu_kernel"] = {"kernel": "sdpa_decode_split_kernel<bf16,128,1,8> + sdpa_combine_kernel", "num_splits": w.splits,
+                                    "ms_per_step": wall_v, "launch_ms_mean": ev_v, "frac": kv_bytes / (ev_v * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                                    "parity_max_abs_err": w.parity()}
         w.free()
         if not args.no_cpu_baseline:
             val, dt = cpu_baseline_decode(D, Skv, 32, 32, capi.BF16)
@@ -526,6 +568,9 @@ def main():
                                    "sample": "all of config 4 (B=32, H=32, KV=8192, D=128), oracle's materialising restatement of "
                                              "the reference CPU op (serial matmuls and reductions); %.1f s; host: %s" % (dt, host_cpu())}
         result["decode"] = dec
+
+    if args.only in (None, "decode_gqa"):
+        result["decode_gqa"] = decode_gqa_leg(args.steps, args.warmup, args.decode_gqa_shape)
 
     if args.only in (None, "f32"):
         result.update(f32_configs(args.steps, args.warmup, not args.no_cpu_baseline, threads))

@@ -170,16 +170,16 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
 
     int impl = d->impl;
     if (impl == INCIN_ROCM_IMPL_AUTO) {
-        // Few rows per KV head (query heads of the group x query positions) over a long cache: split-KV.  One row stays
-        // on the vector-ALU kernel; with more it runs out of arithmetic before it runs out of bandwidth (measured on
+        // Few rows per KV head (query heads of the group x query positions) over a long cache: split-KV.  With more
+        // than a row or two the vector-ALU kernel runs out of arithmetic before it runs out of bandwidth (measured on
         // 32 x 8 KV heads x 8192 keys: 83 / 82 / 77 / 76 / 54 % of the memory bandwidth at 1 / 2 / 3 / 4 / 5 rows, the
-        // matrix-core kernel 85 % at each), except over short caches, where the matrix-core kernel's one workgroup per
-        // compute unit has too little to stream.  Up to 64 rows the matrix-core kernel reads the cache once; beyond, once
-        // per 64 rows, which still beats the prefill kernel when that one would leave most of the device idle (it does
-        // not split the keys).
+        // matrix-core kernel 86 - 87 % at each); over short caches the matrix-core kernel's one workgroup per compute
+        // unit has too little to stream, and the vector-ALU kernel keeps those (the thresholds are where the two cross).
+        // Up to 64 rows the matrix-core kernel reads the cache once; beyond, once per 64 rows, which still beats the
+        // prefill kernel when that one would leave most of the device idle (it does not split the keys).
         const int64_t prefill_wgs = d->B * d->Hq * ((d->Sq + 127) / 128);
         if (split_mfma_ok && !d->lse && d->Skv >= 256 &&
-            ((R >= 2 && R <= 4 && d->Skv >= 1024) || (R >= 5 && R <= 64) ||
+            ((R == 1 && d->Skv >= 4096) || (R >= 2 && R <= 4 && d->Skv >= 1024) || (R >= 5 && R <= 64) ||
              (R > 64 && d->Skv >= 2048 && prefill_wgs * 4 <= compute_units_of(d->device))))
             impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
         else if (split_ok && R <= 8 && d->Skv >= 256 && !d->lse) impl = INCIN_ROCM_IMPL_SPLITKV;

@@ -136,6 +136,9 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
     // count of copies in flight, and with it the wait for the oldest, the same from the first block to the last.
     int issued = 0, slot_in = 0;
     auto issue_next = [&]() __attribute__((always_inline)) {
+        // The slot about to be refilled was read by this wavefront's LDS loads just before: those loads have delivered
+        // once lgkmcnt is 0 (the "memory" clobber keeps them above this point in program order).
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         const unsigned dst = ring + slot_in * DM_SLOT_BYTES;
         if ((issued & 1) == 0) {
             const uint4v rk = dma_descriptor(k_next, clamp31(k_rem));
@@ -225,29 +228,38 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
 #pragma unroll
             for (int rb = 0; rb < NRB; ++rb) sacc[rb] = Mma<T>::run(a, qreg[rb][s], sacc[rb]);
         }
-        // (the matrix instructions above hold the block's values: its slot can take the next copy)
-#pragma unroll
-        for (int rb = 0; rb < NRB; ++rb) asm volatile("" : "+v"(sacc[rb]));
-        issue_next();
+        issue_next();              // (the block's values are in registers: its slot takes the next copy)
         // register r is key j0 + 8 (r / 4) + 4 g + (r % 4)
         const bool masked = j0 + DM_BLOCK > mask_from;
         vec8 pb[NRB][2];
 #pragma unroll
         for (int rb = 0; rb < NRB; ++rb) {
-            const int rel = lim[rb] - (j0 + 4 * g);
-            float tmax = -INFINITY;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                float x = sacc[rb][r] * sc2;
-                if (masked && 8 * (r / 4) + (r % 4) >= rel) x = -INFINITY;
-                sacc[rb][r] = x;
-                tmax = fmaxf(tmax, x);
+            for (int r = 0; r < 16; ++r) sacc[rb][r] *= sc2;
+            if (masked) {
+                const int rel = lim[rb] - (j0 + 4 * g);
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    if (8 * (r / 4) + (r % 4) >= rel) sacc[rb][r] = -INFINITY;
             }
-            tmax = xor32_max(tmax);
-            const float m_new = fmaxf(m_run[rb], tmax);
-            const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
-            const float alpha = __builtin_amdgcn_exp2f(m_run[rb] - m_use);
-            m_run[rb] = m_new;
+            float tmax = sacc[rb][0];
+#pragma unroll
+            for (int r = 1; r < 16; ++r) tmax = fmaxf(tmax, sacc[rb][r]);
+            tmax = xor32_max(tmax);              // largest score of the row in this block (log2 units)
+            // The reference the probabilities are taken against moves only when a block's maximum passes it by more
+            // than 2^8 (or the row sees its first key): exact in exact arithmetic, probabilities stay <= 2^8, and O^T -
+            // 64 accumulator registers - is rescaled on the first block and then hardly ever.
+            const bool need = tmax > m_run[rb] + PF_RESCALE_THRESHOLD;      // (-inf + 8 = -inf: any finite maximum passes it)
+            if (__builtin_amdgcn_ballot_w64(need) != 0) {
+                const float alpha = need ? __builtin_amdgcn_exp2f(m_run[rb] - tmax) : 1.0f;   // (first key: exp2(-inf) = 0 times 0)
+                if (need) m_run[rb] = tmax;
+                l_run[rb] *= alpha;
+#pragma unroll
+                for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) o_acc[rb][db][r] *= alpha;
+            }
+            const float m_use = (m_run[rb] == -INFINITY) ? 0.0f : m_run[rb];
             // P^T in storage precision: element e of k-step ks is register 8 ks + e; the denominator is summed from
             // the rounded values
             float rsum = 0.0f;
@@ -261,11 +273,7 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
                     rsum = Mma<T>::add2(pr, rsum);
                 }
             }
-            l_run[rb] = l_run[rb] * alpha + rsum;
-#pragma unroll
-            for (int db = 0; db < NDB; ++db)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) o_acc[rb][db][r] *= alpha;
+            l_run[rb] += rsum;
         }
         // ---- O^T += V^T P^T ----
         wait_oldest_copy<NSLOT>();
@@ -281,8 +289,6 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
 #pragma unroll
                 for (int rb = 0; rb < NRB; ++rb) o_acc[rb][db] = Mma<T>::run(__builtin_bit_cast(vec8, av), pb[rb][ks], o_acc[rb][db]);
             }
-#pragma unroll
-        for (int rb = 0; rb < NRB; ++rb) asm volatile("" : "+v"(o_acc[rb][0]), "+v"(o_acc[rb][1]), "+v"(o_acc[rb][2]), "+v"(o_acc[rb][3]));
         issue_next();
     }
 

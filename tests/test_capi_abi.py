@@ -64,7 +64,9 @@ def test_dispatch_choices():
     assert impl == capi.IMPL_MFMA and nbytes == 256                           # with 2 x 4 x 4 x 4 block flags (rounded up)
     assert _plan(_desc(add_mask=0x20000, D=80, Dv=80))[2] == capi.IMPL_GENERIC
     nbytes, splits, impl = _plan(_desc(Sq=1, Skv=8192, B=32, Hq=32, Hkv=32))
-    assert impl == capi.IMPL_SPLITKV and splits >= 1
+    assert impl == capi.IMPL_SPLITKV_MFMA and splits == 1 and nbytes == 0      # 1024 workgroups, four rounds of 256
+    nbytes, splits, impl = _plan(_desc(Sq=1, Skv=2048, B=32, Hq=32, Hkv=32))
+    assert impl == capi.IMPL_SPLITKV and splits >= 1                             # one row per KV head, short cache: vector ALU
     assert nbytes == (0 if splits == 1 else 32 * 32 * 1 * splits * (128 + 2) * 4)
     # grouped-query decode, 4 rows per KV head: the matrix-core split-KV kernel (the vector-ALU one by name)
     nbytes, splits, impl = _plan(_desc(Sq=1, Skv=8192, B=1, Hq=8, Hkv=2, num_splits=4))

@@ -87,17 +87,22 @@ def test_config4_bf16_decode_full(gpu):
     q = gen(40, (B, H, 1, D), dt)
     k, v = gen(41, (B, H, KV, D), dt), gen(42, (B, H, KV, D), dt)
     got, info = host.sdpa(q, k, v, dt, return_info=True)
-    assert info["impl"] == capi.IMPL_SPLITKV and info["splits"] >= 1
+    assert info["impl"] == capi.IMPL_SPLITKV_MFMA and info["splits"] >= 1      # a long cache: the matrix-core split-KV kernel
     ref = O.sdpa(q, k, v)
     err = float(np.abs(got - ref).max())
     say("config 4: splits %d, max-abs err %.3e" % (info["splits"], err))
     assert err <= TOL[dt]
     # split invariance: other split counts agree with the chosen one to rounding of the bf16 output
-    for ns in (1, 4, 16):
-        other = host.sdpa(q, k, v, dt, num_splits=ns, impl=capi.IMPL_SPLITKV)
-        d = float(np.abs(other - got).max())
-        say("config 4: %d splits vs %d: max-abs diff %.3e" % (ns, info["splits"], d))
-        assert d <= 2.0 ** -8
+    # and so does the vector-ALU split-KV kernel, which also stands against the oracle on its own
+    for impl in (capi.IMPL_SPLITKV_MFMA, capi.IMPL_SPLITKV):
+        for ns in (0, 1, 4, 16):
+            other, oi = host.sdpa(q, k, v, dt, num_splits=ns, impl=impl, return_info=True)
+            assert oi["impl"] == impl
+            d = float(np.abs(other - got).max())
+            say("config 4: kernel %d, %d splits vs %d: max-abs diff %.3e" % (impl, oi["splits"], info["splits"], d))
+            assert d <= 2.0 ** -8
+            if impl == capi.IMPL_SPLITKV and ns == 0:
+                assert float(np.abs(other - ref).max()) <= TOL[dt]
 
 
 def test_config5_gqa_ragged_causal_full(gpu):

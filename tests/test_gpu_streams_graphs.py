@@ -48,6 +48,7 @@ CASES = [
     ("prefill 32-row kernel", dict(B=2, Hq=8, Hkv=8, Sq=512, Skv=512, D=128, causal=True, impl=capi.IMPL_MFMA)),
     ("prefill 64-row kernel", dict(B=2, Hq=8, Hkv=2, Sq=1024, Skv=1024, D=128, causal=True, impl=capi.IMPL_MFMA64)),
     ("decode split-KV", dict(B=4, Hq=8, Hkv=8, Sq=1, Skv=4096, D=128, causal=False, impl=capi.IMPL_SPLITKV)),
+    ("grouped-query decode, matrix-core split-KV", dict(B=2, Hq=16, Hkv=2, Sq=1, Skv=4096, D=128, causal=False, impl=capi.IMPL_SPLITKV_MFMA)),
     ("generic", dict(B=1, Hq=2, Hkv=2, Sq=100, Skv=130, D=80, causal=True, impl=capi.IMPL_GENERIC)),
     ("f32 matrix-core prefill", dict(B=2, Hq=4, Hkv=2, Sq=300, Skv=300, D=64, causal=True, impl=capi.IMPL_MFMA, dtype=capi.F32)),
     ("prefill with a dense mask", dict(B=1, Hq=4, Hkv=4, Sq=512, Skv=512, D=128, causal=False, impl=capi.IMPL_MFMA, banded_mask=True)),

@@ -62,6 +62,9 @@ def test_static_scratch_matches_workspace_launch(gpu):
         ("split-KV decode",
          dict(B=4, Hq=8, Hkv=8, Sq=1, Skv=4096, D=128, causal=False, impl=capi.IMPL_SPLITKV, num_splits=8),
          dict(B=2, Hq=4, Hkv=2, Sq=1, Skv=1500, D=128, causal=False, impl=capi.IMPL_SPLITKV, num_splits=3, kv_lens=[1500, 700])),
+        ("matrix-core split-KV decode",
+         dict(B=2, Hq=16, Hkv=2, Sq=1, Skv=4096, D=128, causal=False, impl=capi.IMPL_SPLITKV_MFMA, num_splits=8),
+         dict(B=2, Hq=12, Hkv=2, Sq=3, Skv=1500, D=128, causal=True, impl=capi.IMPL_SPLITKV_MFMA, num_splits=3, kv_lens=[1500, 700])),
         ("64-row prefill",
          dict(B=2, Hq=8, Hkv=2, Sq=1024, Skv=1024, D=128, causal=True, impl=capi.IMPL_MFMA64),
          dict(B=1, Hq=3, Hkv=3, Sq=300, Skv=300, D=128, causal=True, impl=capi.IMPL_MFMA64)),
