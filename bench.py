@@ -33,13 +33,13 @@ PEAK_HBM_GBS = 8000.0       # HBM3E, vendor figure
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same command (KiB per dispatch,
 # FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0 after calibration against the 1 GiB copy kernel): profiles/*.txt
 PREFILL_TRAFFIC_BYTES = (273324 * 2.0 + 131085) * 1024     # 6.94e8: |Q|+|K|+|V| read 1.39 times, |O| written once
-DECODE_TRAFFIC_BYTES = (2097470 * 2.0 + 1088 + 256) * 1024  # 4.297e9: K and V read once + split partials
+DECODE_TRAFFIC_BYTES = (2097360 * 2.0 + 256) * 1024        # 4.2957e9: K and V read once, O written once
 PREFILL_LONG_TRAFFIC_BYTES = (537192 * 2.0 + 318930) * 1024    # 1.43e9: valid |O| written once, inputs read 2.2 times
 # These three are constants taken from counter runs, not measured by this script: each roofline object says so and
 # names the summary the figures come from.
 TRAFFIC_SOURCE = {
     "prefill": "constant from profiles/sdpa_prefill_mfma_bf16_d128_config3.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of `bench.py --only prefill`)",
-    "decode": "constant from profiles/sdpa_decode_splitkv_bf16_d128_config4.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of `bench.py --only decode`)",
+    "decode": "constant from profiles/sdpa_decode_mfma_bf16_d128_config4.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of `bench.py --only decode`)",
     "prefill_long": "constant from profiles/sdpa_prefill_mfma_bf16_d128_config5.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of `bench.py --only prefill_long --no-padding-compare`)",
 }
 METRIC = "attn fwd TFLOP/s + % bf16 MFMA peak; decode KV GB/s + % HBM peak (1 GPU)"

@@ -198,7 +198,7 @@ int incin_rocm_sdpa_workspace(const incin_rocm_sdpa_desc_t* desc, size_t* bytes,
  * keeps alive until the stream has been synchronised.
  *
  * Workspace.  Three launches need scratch memory, of the size incin_rocm_sdpa_workspace reports: the split-KV
- * kernel (partial results of the splits), the 64-row MFMA prefill kernel (256 bytes: the work counters its
+ * kernels when they split (partial results of the splits), the 64-row MFMA prefill kernel (256 bytes: the work counters its
  * persistent workgroups draw from, cleared by the launch itself) and the MFMA prefill kernels with a dense mask
  * (one byte per block of 32 query rows x 32 keys of the mask: which blocks it hides, which it leaves alone;
  * written by a small kernel of the same launch).  The contents need not survive the launch and
