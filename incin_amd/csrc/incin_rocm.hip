@@ -28,6 +28,7 @@ hipError_t launch_mask_classify(const SdpaParams& p, int dtype, hipStream_t stre
 hipError_t launch_sdpa_decode(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_sdpa_decode_mfma(const SdpaParams& p, int dtype, hipStream_t stream);
 int decode_mfma_chunk_rows(int R);
+int decode_mfma_workgroups_per_cu(int chunk_rows, int64_t split_len);
 int decode_keys_per_tile(int dtype, int D, int R);
 }  // namespace incin_rocm
 
@@ -173,13 +174,17 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         // Few rows per KV head (query heads of the group x query positions) over a long cache: split-KV.  With more
         // than a row or two the vector-ALU kernel runs out of arithmetic before it runs out of bandwidth (measured on
         // 32 x 8 KV heads x 8192 keys: 83 / 82 / 77 / 76 / 54 % of the memory bandwidth at 1 / 2 / 3 / 4 / 5 rows, the
-        // matrix-core kernel 86 - 87 % at each); over short caches the matrix-core kernel's one workgroup per compute
-        // unit has too little to stream, and the vector-ALU kernel keeps those (the thresholds are where the two cross).
+        // matrix-core kernel 86 - 87 % at each); over the shortest caches the matrix-core kernel's one or two workgroups
+        // per compute unit have too little to stream, and the vector-ALU kernel keeps those (the thresholds are where
+        // the two cross on launches of 268 MB of cache).  With one row per KV head the two kernels are within a few per
+        // cent of each other everywhere; the matrix-core one is ahead on launches that run long enough for its longer
+        // start-up not to show (3 - 4 % from 1 GB of cache on, behind by 4 - 9 % at 64 - 268 MB).
         // Up to 64 rows the matrix-core kernel reads the cache once; beyond, once per 64 rows, which still beats the
         // prefill kernel when that one would leave most of the device idle (it does not split the keys).
         const int64_t prefill_wgs = d->B * d->Hq * ((d->Sq + 127) / 128);
+        const int64_t kv_bytes = 2 * d->B * d->Hkv * d->Skv * d->D * 2;       // (16-bit storage where it matters)
         if (split_mfma_ok && !d->lse && d->Skv >= 256 &&
-            ((R == 1 && d->Skv >= 4096) || (R >= 2 && R <= 4 && d->Skv >= 1024) || (R >= 5 && R <= 64) ||
+            ((R == 1 && d->Skv >= 1024 && kv_bytes >= (512LL << 20)) || (R >= 2 && R <= 3 && d->Skv >= 512) || (R >= 4 && R <= 64) ||
              (R > 64 && d->Skv >= 2048 && prefill_wgs * 4 <= compute_units_of(d->device))))
             impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
         else if (split_ok && R <= 8 && d->Skv >= 256 && !d->lse) impl = INCIN_ROCM_IMPL_SPLITKV;
@@ -233,10 +238,11 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         plan->ws_bytes = splits > 1 ? (size_t)(d->B * d->Hq * d->Sq * splits) * (size_t)(d->Dv + 2) * sizeof(float) : 0;
     }
     if (impl == INCIN_ROCM_IMPL_SPLITKV_MFMA) {
-        // One workgroup per (batch, KV head, chunk of 32 or 64 rows, split), and a compute unit holds one at a time (its LDS is
-        // the ring of tiles in flight): the workgroups of a launch run in rounds of one per compute unit, all of equal
-        // length.  Take the number of splits that leaves the last round fullest, among those that keep at least 256
-        // keys per split, preferring fewer splits at equal filling (fewer partial results to combine).
+        // One workgroup per (batch, KV head, chunk of 32 or 64 rows, split).  A compute unit holds one at a time (its LDS
+        // is the ring of blocks in flight) - two when the splits are short enough for the two-slot rings - so the
+        // workgroups of a launch, all of equal length, run in rounds.  Take the number of splits that leaves the last
+        // round fullest, among those that keep at least 256 keys per split, preferring fewer splits at (nearly) equal
+        // filling: fewer partial results to combine.
         const int64_t chunk = incin_rocm::decode_mfma_chunk_rows((int)std::min<int64_t>(R, 1 << 20));
         const int64_t nchunks = (R + chunk - 1) / chunk;
         const int64_t groups = d->B * d->Hkv * nchunks;
@@ -244,10 +250,12 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         if (splits == 0) {
             const int64_t cus = compute_units_of(d->device);
             const int64_t max_by_len = d->Skv / 256 > 0 ? d->Skv / 256 : 1;
-            const int64_t max_splits = std::min<int64_t>(max_by_len, std::max<int64_t>(1, 2 * cus / groups));
-            auto fill = [&](int64_t s) {
-                const int64_t wgs = groups * s, rounds = (wgs + cus - 1) / cus;
-                return (double)wgs / (double)(rounds * cus);
+            const int64_t max_splits = std::min<int64_t>(max_by_len, std::max<int64_t>(1, 4 * cus / groups));
+            auto fill = [&](int64_t s) {           // (with the split length, and so the count, s really leads to)
+                const int64_t len = ((d->Skv + s - 1) / s + 127) / 128 * 128;
+                const int64_t at_a_time = cus * incin_rocm::decode_mfma_workgroups_per_cu((int)chunk, len);
+                const int64_t wgs = groups * ((d->Skv + len - 1) / len), rounds = (wgs + at_a_time - 1) / at_a_time;
+                return (double)wgs / (double)(rounds * at_a_time);
             };
             double best = 0.0;
             for (int64_t s = 1; s <= max_splits; ++s) best = std::max(best, fill(s));

@@ -22,12 +22,17 @@
 //
 // Rows: row r of a chunk is (query head hkv * G + r / Sq, position r % Sq) - the G heads of the group times the Sq
 // positions.  The scale is applied to the f32 scores (any sign), masks as -inf before the maximum.
+#include <cstdlib>
+
 #include "sdpa_mfma_common.h"
 
 namespace incin_rocm {
 
 constexpr int DM_BLOCK = 32;            // keys per block
 constexpr int DM_SLOT_BYTES = DM_BLOCK * 256;
+#ifndef DM_SHORT_KEYS
+#define DM_SHORT_KEYS 2048
+#endif
 #ifndef DM_NSLOT
 #define DM_NSLOT 5       // slots per wavefront: 4 wavefronts x 5 x 8 KiB = the 160 KiB of a compute unit
 #endif
@@ -46,10 +51,11 @@ __device__ __forceinline__ void dm_copy16(uint4v desc, unsigned lds_addr, int by
 // All but the newest NSLOT - 1 copies of this wavefront (8 instructions each) have landed.
 template <int NSLOT> __device__ __forceinline__ void wait_oldest_copy()
 {
-    static_assert(NSLOT >= 3 && NSLOT <= 5, "s_waitcnt takes an immediate");
+    static_assert(NSLOT >= 2 && NSLOT <= 5, "s_waitcnt takes an immediate");
     if (NSLOT == 5) asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
     else if (NSLOT == 4) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else if (NSLOT == 3) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
 }
 
 template <typename T, int NSLOT, int NRB>
@@ -366,7 +372,9 @@ hipError_t launch_sdpa_combine(const SdpaParams& p, int dtype, hipStream_t strea
 template <typename T, int NSLOT, int NRB>
 static hipError_t launch_decode_mfma_t(const SdpaParams& p, hipStream_t stream)
 {
-    constexpr size_t lds = (size_t)4 * NSLOT * DM_SLOT_BYTES;
+    // the rings, or what the wavefronts' results need when they meet at the end, whichever is more
+    constexpr size_t ring_bytes = (size_t)4 * NSLOT * DM_SLOT_BYTES, merge_bytes = (size_t)NRB * (4 * 32 * 2 + 4 * 4 * 16 * 64) * sizeof(float);
+    constexpr size_t lds = ring_bytes > merge_bytes ? ring_bytes : merge_bytes;
     auto kern = sdpa_decode_mfma_kernel<T, NSLOT, NRB>;
     // the dynamic-LDS limit of this instance is raised once per device, not per launch
     static std::atomic<uint64_t> prepared{0};
@@ -389,16 +397,32 @@ static hipError_t launch_decode_mfma_t(const SdpaParams& p, hipStream_t stream)
 // head - the cache is then read once for 64 rows instead of once per 32.
 int decode_mfma_chunk_rows(int R) { return R > 32 ? 64 : 32; }
 
+// Workgroups a compute unit holds at a time: two of the two-slot form (32 rows, splits of up to DM_SHORT_KEYS keys), one
+// otherwise.  The planner fills rounds of this many.
+int decode_mfma_workgroups_per_cu(int chunk_rows, int64_t split_len) { return chunk_rows == 32 && split_len <= DM_SHORT_KEYS ? 2 : 1; }
+
 // Host has validated: dtype f16 / bf16, D == Dv == 128, rows 16-byte aligned with unit last-dim stride, row strides
 // below 2^24 elements, split_len a multiple of 128 (every wavefront's blocks then start where its
 // neighbour's end in every split).
 hipError_t launch_sdpa_decode_mfma(const SdpaParams& p, int dtype, hipStream_t stream)
 {
     hipError_t e;
-    if (decode_mfma_chunk_rows(p.G * p.Sq) == 64)
+    if (decode_mfma_chunk_rows(p.G * p.Sq) == 64) {
         e = dtype == 1 ? launch_decode_mfma_t<f16_t, DM_NSLOT, 2>(p, stream) : launch_decode_mfma_t<bf16_t, DM_NSLOT, 2>(p, stream);
-    else
-        e = dtype == 1 ? launch_decode_mfma_t<f16_t, DM_NSLOT, 1>(p, stream) : launch_decode_mfma_t<bf16_t, DM_NSLOT, 1>(p, stream);
+    } else {
+        // Short splits (up to DM_SHORT_KEYS keys: 16 blocks per wavefront) take rings of two slots, which lets a compute
+        // unit hold two workgroups: with so little to stream, what counts is that one workgroup's start-up (its first
+        // copies' latency) and end (the wavefronts' results meeting, the stores) overlap another's arithmetic.  Measured
+        // on launches of 268 MB of cache, two slots against five: 256-key splits 73 against 46 % of the memory bandwidth,
+        // 512: 81 / 63, 1024: 80 / 73, 2048: 87.5 / 86.3; 4096: 78.5 / 80 (one sequence of 131072 keys); 8192: 84 / 86.7.
+        // INCIN_ROCM_DECODE_SLOTS = 2 or 5 overrides the rule (for tests: both forms on any shape).
+        const char* forced = getenv("INCIN_ROCM_DECODE_SLOTS");
+        const int slots = forced ? atoi(forced) : 0;
+        if (slots == 2 || (slots != DM_NSLOT && decode_mfma_workgroups_per_cu(32, p.split_len) == 2))
+            e = dtype == 1 ? launch_decode_mfma_t<f16_t, 2, 1>(p, stream) : launch_decode_mfma_t<bf16_t, 2, 1>(p, stream);
+        else
+            e = dtype == 1 ? launch_decode_mfma_t<f16_t, DM_NSLOT, 1>(p, stream) : launch_decode_mfma_t<bf16_t, DM_NSLOT, 1>(p, stream);
+    }
     if (e != hipSuccess || p.num_splits == 1) return e;
     return launch_sdpa_combine(p, dtype, stream);
 }

@@ -65,9 +65,9 @@ def test_dispatch_choices():
     assert _plan(_desc(add_mask=0x20000, D=80, Dv=80))[2] == capi.IMPL_GENERIC
     nbytes, splits, impl = _plan(_desc(Sq=1, Skv=8192, B=32, Hq=32, Hkv=32))
     assert impl == capi.IMPL_SPLITKV_MFMA and splits == 1 and nbytes == 0      # 1024 workgroups, four rounds of 256
-    nbytes, splits, impl = _plan(_desc(Sq=1, Skv=2048, B=32, Hq=32, Hkv=32))
-    assert impl == capi.IMPL_SPLITKV and splits >= 1                             # one row per KV head, short cache: vector ALU
-    assert nbytes == (0 if splits == 1 else 32 * 32 * 1 * splits * (128 + 2) * 4)
+    nbytes, splits, impl = _plan(_desc(Sq=1, Skv=2048, B=8, Hq=32, Hkv=32))
+    assert impl == capi.IMPL_SPLITKV and splits >= 1                             # one row per KV head, 268 MB of cache: vector ALU
+    assert nbytes == (0 if splits == 1 else 8 * 32 * 1 * splits * (128 + 2) * 4)
     # grouped-query decode, 4 rows per KV head: the matrix-core split-KV kernel (the vector-ALU one by name)
     nbytes, splits, impl = _plan(_desc(Sq=1, Skv=8192, B=1, Hq=8, Hkv=2, num_splits=4))
     assert impl == capi.IMPL_SPLITKV_MFMA and splits == 4 and nbytes == 8 * 4 * 130 * 4
@@ -84,7 +84,7 @@ def test_dispatch_choices():
     assert _plan(_desc(Sq=4, Skv=8192, B=2, Hq=32, Hkv=2))[2] == capi.IMPL_SPLITKV_MFMA             # 64 rows per KV head: one workgroup's worth
     assert _plan(_desc(Sq=8, Skv=8192, B=2, Hq=32, Hkv=2))[2] == capi.IMPL_SPLITKV_MFMA             # 128, but the prefill kernel would run 64 workgroups
     assert _plan(_desc(Sq=8, Skv=8192, B=8, Hq=32, Hkv=2))[2] == capi.IMPL_MFMA                     # 256 of them: a prefill shape
-    assert _plan(_desc(Sq=1, Skv=512, B=2, Hq=8, Hkv=2))[2] == capi.IMPL_SPLITKV                    # 4 rows, short cache: vector ALU
+    assert _plan(_desc(Sq=1, Skv=400, B=2, Hq=4, Hkv=2))[2] == capi.IMPL_SPLITKV                    # 2 rows, short cache: vector ALU
     assert _plan(_desc(Sq=1, Skv=512, B=2, Hq=16, Hkv=2))[2] == capi.IMPL_SPLITKV_MFMA              # 8 rows
     assert _plan(_desc(Sq=1, Skv=8192, B=2, Hq=4, Hkv=2))[2] == capi.IMPL_SPLITKV_MFMA              # 2 rows, long cache
     assert _plan(_desc(Sq=1, Skv=64))[2] in (capi.IMPL_MFMA, capi.IMPL_SPLITKV)

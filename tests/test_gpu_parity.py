@@ -400,10 +400,13 @@ def test_decode_splitkv(gpu, dtype, shape):
     (1, 16, 2, 9, 1200, True),        # 72 rows per KV head: two chunks of 64, the second with 8 rows
     (1, 6, 2, 64, 1500, True),        # 192 rows per KV head: three chunks, causal over 64 positions
 ])
-def test_decode_splitkv_matrix_cores(gpu, dtype, shape):
+@pytest.mark.parametrize("slots", ["2", "5"], ids=["two_slot_rings", "five_slot_rings"])
+def test_decode_splitkv_matrix_cores(gpu, dtype, shape, slots, monkeypatch):
     """The matrix-core split-KV kernel against the oracle, with the split count left to the library, forced to one
     (the kernel writes the output itself) and forced to counts that leave ragged and empty last splits; and against
-    the vector-ALU split-KV kernel where that one takes the shape."""
+    the vector-ALU split-KV kernel where that one takes the shape.  Both forms of the 32-row instance on every shape:
+    rings of two slots (two workgroups per compute unit; the library's choice for short splits) and of five."""
+    monkeypatch.setenv("INCIN_ROCM_DECODE_SLOTS", slots)
     B, Hq, Hkv, Sq, Skv, causal = shape
     D = 128
     q, k, v = inputs(700 + sum(shape[:5]), B, Hq, Hkv, Sq, Skv, D, D, dtype)
