@@ -399,6 +399,7 @@ def test_decode_splitkv(gpu, dtype, shape):
     (2, 64, 1, 1, 900, False),        # 64 rows: one workgroup of two 32-row blocks
     (1, 16, 2, 9, 1200, True),        # 72 rows per KV head: two chunks of 64, the second with 8 rows
     (1, 6, 2, 64, 1500, True),        # 192 rows per KV head: three chunks, causal over 64 positions
+    (1, 4, 2, 8, 5, True),            # more positions than keys: the first three see none (NaN rows, as the reference)
 ])
 @pytest.mark.parametrize("slots", ["2", "5"], ids=["two_slot_rings", "five_slot_rings"])
 def test_decode_splitkv_matrix_cores(gpu, dtype, shape, slots, monkeypatch):
@@ -443,6 +444,37 @@ def test_decode_splitkv_matrix_cores_lengths_strides_scale(gpu):
     check(got, oracle_full(q, k, v, G=4), 2e-2, "AUTO grouped-query decode")
     _, info = host.sdpa(q[:, :4], k, v, capi.BF16, return_info=True)
     assert info["impl"] == capi.IMPL_SPLITKV                # one row per KV head stays on the vector-ALU kernel
+
+
+@pytest.mark.parametrize("impl", [capi.IMPL_SPLITKV_MFMA, capi.IMPL_SPLITKV], ids=["matrix_cores", "vector_alu"])
+def test_decode_over_a_token_major_cache(gpu, impl):
+    """Cache, queries and output stored [B, S, H, D] (token-major, as serving stacks keep them) and handed over as
+    [B, H, S, D] views by strides alone: both split-KV kernels read rows 'Hkv * D' elements apart in place."""
+    B, Hq, Hkv, Sq, Skv, D = 2, 8, 2, 2, 1111, 128
+    dt = capi.BF16
+    q, k, v = inputs(811, B, Hq, Hkv, Sq, Skv, D, D, dt)
+    ref = oracle_full(q, k, v, G=Hq // Hkv, causal=True)
+    tq, tk, tv = (host.DeviceTensor.from_f32(np.ascontiguousarray(x.transpose(0, 2, 1, 3)), dt) for x in (q, k, v))
+    to = host.DeviceTensor((B, Sq, Hq, D), dt)
+
+    class View:                                   # logical [B, H, S, D] over the stored [B, S, H, D]
+        def __init__(self, t, H, S):
+            self.shape, self.dtype, self.dev, self.ptr = (B, H, S, D), t.dtype, t.dev, t.ptr
+    d = host.make_desc(View(tq, Hq, Sq), View(tk, Hkv, Skv), View(tv, Hkv, Skv), View(to, Hq, Sq), causal=True, impl=impl, num_splits=3)
+    for name, H, S in (("q_stride", Hq, Sq), ("k_stride", Hkv, Skv), ("v_stride", Hkv, Skv), ("o_stride", Hq, Sq)):
+        st = getattr(d, name)
+        st[0], st[1], st[2] = S * H * D, D, H * D
+    nbytes, splits, chosen = capi.sdpa_workspace(d)
+    assert chosen == impl and splits == 3
+    ws = capi.DeviceBuffer(nbytes)
+    d.workspace, d.workspace_bytes = ws.ptr, ws.nbytes
+    capi.sdpa_fwd(d)
+    capi.sync()
+    got = to.to_f32().transpose(0, 2, 1, 3)
+    check(got, ref, TOL[dt], "token-major cache, impl %d" % impl)
+    for t in (tq, tk, tv, to):
+        t.buf.free()
+    ws.free()
 
 
 def test_decode_lengths_and_prefill_consistency(gpu):
