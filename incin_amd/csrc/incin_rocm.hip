@@ -166,8 +166,8 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     const bool mfma64_ok = mfma_ok && !d->add_mask && d->dtype != INCIN_ROCM_F32 && d->D == 128 && (d->Skv + 512) * d->k_stride[2] * 2 < (1LL << 31) &&
                            (d->Skv + 512) * d->v_stride[2] * 2 < (1LL << 31);
     const bool split_ok = fast_ok && d->Sq <= 64;
-    // the matrix-core split-KV kernel: 16-bit storage, head dimension 128, tiles addressed like the prefill kernels'
-    const bool split_mfma_ok = split_ok && tile_off_ok && d->dtype != INCIN_ROCM_F32 && d->D == 128 && std::isfinite(d->scale);
+    // the matrix-core split-KV kernel: 16-bit storage, blocks addressed like the prefill kernels' tiles
+    const bool split_mfma_ok = split_ok && tile_off_ok && d->dtype != INCIN_ROCM_F32 && std::isfinite(d->scale);
 
     int impl = d->impl;
     if (impl == INCIN_ROCM_IMPL_AUTO) {
@@ -183,9 +183,10 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         // prefill kernel when that one would leave most of the device idle (it does not split the keys).
         const int64_t prefill_wgs = d->B * d->Hq * ((d->Sq + 127) / 128);
         const int64_t kv_bytes = 2 * d->B * d->Hkv * d->Skv * d->D * 2;       // (16-bit storage where it matters)
-        if (split_mfma_ok && !d->lse && d->Skv >= 256 &&
-            ((R == 1 && d->Skv >= 1024 && kv_bytes >= (512LL << 20)) || (R >= 2 && R <= 3 && d->Skv >= 512) || (R >= 4 && R <= 64) ||
-             (R > 64 && d->Skv >= 2048 && prefill_wgs * 4 <= compute_units_of(d->device))))
+        const int64_t len128 = d->Skv * d->D / 128;      // cache length in keys of 128 elements (what the thresholds were measured in)
+        if (split_mfma_ok && !d->lse && len128 >= 256 &&
+            ((R == 1 && len128 >= 1024 && kv_bytes >= (512LL << 20)) || (R >= 2 && R <= 3 && len128 >= 512) || (R >= 4 && R <= 64) ||
+             (R > 64 && len128 >= 2048 && prefill_wgs * 4 <= compute_units_of(d->device))))
             impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
         else if (split_ok && R <= 8 && d->Skv >= 256 && !d->lse) impl = INCIN_ROCM_IMPL_SPLITKV;
         // (the 64-row kernel is never picked: since the 32-row kernel stopped taking maxima in its pipelined loop it is
@@ -205,7 +206,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         return fail(INCIN_ROCM_EUNSUPPORTED, "scaled_dot_product_attention: the split-KV kernels do not write the row normalisers (lse)");
     if (impl == INCIN_ROCM_IMPL_SPLITKV_MFMA && !split_mfma_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
-                    "scaled_dot_product_attention: the matrix-core split-KV kernel needs f16/bf16, D == Dv == 128, Sq <= 64, no dense mask, a finite scale and 16-byte aligned rows");
+                    "scaled_dot_product_attention: the matrix-core split-KV kernel needs f16/bf16, D == Dv in {64,128}, Sq <= 64, no dense mask, a finite scale and 16-byte aligned rows");
     if (impl == INCIN_ROCM_IMPL_SPLITKV && !split_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
                     "scaled_dot_product_attention: the split-KV kernel needs D == Dv in {64,128}, Sq <= 64, no dense mask and 16-byte aligned rows");
@@ -252,7 +253,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
             const int64_t max_by_len = d->Skv / 256 > 0 ? d->Skv / 256 : 1;
             const int64_t max_splits = std::min<int64_t>(max_by_len, std::max<int64_t>(1, 4 * cus / groups));
             auto fill = [&](int64_t s) {           // (with the split length, and so the count, s really leads to)
-                const int64_t len = ((d->Skv + s - 1) / s + 127) / 128 * 128;
+                const int64_t len = ((d->Skv + s - 1) / s + 255) / 256 * 256;
                 const int64_t at_a_time = cus * incin_rocm::decode_mfma_workgroups_per_cu((int)chunk, len);
                 const int64_t wgs = groups * ((d->Skv + len - 1) / len), rounds = (wgs + at_a_time - 1) / at_a_time;
                 return (double)wgs / (double)(rounds * at_a_time);
@@ -263,7 +264,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
             while (splits < max_splits && fill(splits) < 0.98 * best) ++splits;
         }
         int64_t split_len = (d->Skv + splits - 1) / splits;
-        split_len = (split_len + 127) / 128 * 128;      // whole rounds of the four wavefronts' 32-key blocks
+        split_len = (split_len + 255) / 256 * 256;      // whole rounds of the four wavefronts' blocks of 32 (D = 128) or 64 keys
         splits = (d->Skv + split_len - 1) / split_len;
         if (splits > 65535) return fail(INCIN_ROCM_ESHAPE, "scaled_dot_product_attention: too many splits");
         if (d->Hkv * nchunks > 65535) return fail(INCIN_ROCM_ESHAPE, "scaled_dot_product_attention: too many head groups for one launch");

@@ -1,5 +1,5 @@
 // Split-KV attention for the query rows that share one key/value head, on the gfx950 matrix cores (f16 / bf16,
-// D == Dv == 128): grouped-query decode, where the vector-ALU split-KV kernel runs out of arithmetic (it spends
+// D == Dv in {64, 128}): grouped-query decode, where the vector-ALU split-KV kernel runs out of arithmetic (it spends
 // ~24 vector instructions per query row on every 2 KiB of cache it reads), and short runs of query rows over a long
 // cache.  Same function as the other attention kernels (crates/incin-backends/src/cpu/ops/shape_ops.rs:1245-1269),
 // same partial-result format as the vector-ALU split-KV kernel, same combine kernel.
@@ -7,7 +7,7 @@
 // The work is bound by the bandwidth of the cache reads, so the design serves the memory system first:
 //
 //   * one workgroup (4 wavefronts) per (batch, KV head, chunk of 32 or 64 query rows, split), one workgroup per compute
-//     unit.  The split's keys are dealt to the wavefronts in blocks of 32 (wavefront w takes blocks w, w + 4, ...), and
+//     unit.  The split's keys are dealt to the wavefronts in blocks of 32 (D = 64: 64; wavefront w takes blocks w, w + 4, ...), and
 //     a wavefront works through its blocks on its own: no barrier in the loop, nothing shared.  Each wavefront owns a
 //     ring of NSLOT 8 KiB slots in LDS that the K and V blocks pass through in the order they are needed
 //     (K0 V0 K1 V1 ...), filled straight from global memory (buffer_load ... lds, whole rows, 1 KiB per instruction);
@@ -28,8 +28,7 @@
 
 namespace incin_rocm {
 
-constexpr int DM_BLOCK = 32;            // keys per block
-constexpr int DM_SLOT_BYTES = DM_BLOCK * 256;
+constexpr int DM_SLOT_BYTES = 8192;      // a block of K or of V: 32 keys at D = 128, 64 keys at D = 64
 #ifndef DM_SHORT_KEYS
 #define DM_SHORT_KEYS 2048
 #endif
@@ -58,14 +57,15 @@ template <int NSLOT> __device__ __forceinline__ void wait_oldest_copy()
     else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
 }
 
-template <typename T, int NSLOT, int NRB>
+template <typename T, int D, int NSLOT, int NRB>
 __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
 {
 #if defined(__HIP_DEVICE_COMPILE__)
-    constexpr int D = 128;
     typedef typename Mma<T>::vec8 vec8;
     typedef PfLayout<D> L;
     constexpr int NSTEP = D / 16, NDB = D / 32;
+    constexpr int KB = 128 / D;                        // 32-key sub-blocks of a block: a slot holds 8 KiB either way
+    constexpr int BLOCK = 32 * KB;                     // keys per block
     constexpr int CPB = DM_SLOT_BYTES / 1024;          // wavefront-wide 1 KiB copies per block
     extern __shared__ __attribute__((aligned(1024))) char smem[];
 
@@ -108,7 +108,7 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
     }
     const int k_end = __builtin_amdgcn_readfirstlane(lim_hi);          // rows at and beyond are never read
     const int mask_from = __builtin_amdgcn_readfirstlane(lim_lo);      // blocks that end at or before need no mask
-    const int n_blocks = k_end > k_begin ? (k_end - k_begin + DM_BLOCK - 1) / DM_BLOCK : 0;
+    const int n_blocks = k_end > k_begin ? (k_end - k_begin + BLOCK - 1) / BLOCK : 0;
     const int my_blocks = n_blocks > wave ? (n_blocks - wave + 3) >> 2 : 0;      // blocks wave, wave + 4, ...
 
     // ---- global -> LDS copy plan (rows of 256 bytes, chunk slot c ^ f(row) as in the prefill kernels' tiles) ---------
@@ -125,8 +125,8 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
     // The copies of this wavefront go K(block 0) V(0) K(1) V(1) ...; copy number n lands in slot n % NSLOT.  Address of
     // the next block of each tensor and the bytes from there to the end of row k_end - 1 (loads past that deliver
     // zeros: what an unwritten cache tail holds never enters LDS).
-    const int64_t k_step = (int64_t)4 * DM_BLOCK * p.k_ss * 2, v_step = (int64_t)4 * DM_BLOCK * p.v_ss * 2;
-    const int first_key = k_begin + wave * DM_BLOCK;
+    const int64_t k_step = (int64_t)4 * BLOCK * p.k_ss * 2, v_step = (int64_t)4 * BLOCK * p.v_ss * 2;
+    const int first_key = k_begin + wave * BLOCK;
     const char* k_next = (const char*)kp + (int64_t)first_key * p.k_ss * 2;
     const char* v_next = (const char*)vp + (int64_t)first_key * p.v_ss * 2;
     int64_t k_rem = (int64_t)(k_end - first_key - 1) * p.k_ss * 2 + D * 2;
@@ -218,39 +218,49 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
 
     int slot_out = 0;              // slot of the copy consumed next
     for (int j = 0; j < my_blocks; ++j) {
-        const int j0 = first_key + j * 4 * DM_BLOCK;
+        const int j0 = first_key + j * 4 * BLOCK;
         // ---- S^T = K Q^T ----
         wait_oldest_copy<NSLOT>();
         const char* kb = smem + (wave * NSLOT + slot_out) * DM_SLOT_BYTES;
         slot_out = slot_out + 1 == NSLOT ? 0 : slot_out + 1;
-        floatx16 sacc[NRB];
+        floatx16 sacc[NRB][KB];
 #pragma unroll
         for (int rb = 0; rb < NRB; ++rb)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) sacc[rb][r] = 0.0f;
+            for (int kb2 = 0; kb2 < KB; ++kb2)
 #pragma unroll
-        for (int s = 0; s < NSTEP; ++s) {
-            const vec8 a = *(const vec8*)(kb + k_addr[s]);
+                for (int r = 0; r < 16; ++r) sacc[rb][kb2][r] = 0.0f;
 #pragma unroll
-            for (int rb = 0; rb < NRB; ++rb) sacc[rb] = Mma<T>::run(a, qreg[rb][s], sacc[rb]);
-        }
+        for (int s = 0; s < NSTEP; ++s)
+#pragma unroll
+            for (int kb2 = 0; kb2 < KB; ++kb2) {
+                const vec8 a = *(const vec8*)(kb + k_addr[s] + kb2 * 32 * L::ROWB);
+#pragma unroll
+                for (int rb = 0; rb < NRB; ++rb) sacc[rb][kb2] = Mma<T>::run(a, qreg[rb][s], sacc[rb][kb2]);
+            }
         issue_next();              // (the block's values are in registers: its slot takes the next copy)
-        // register r is key j0 + 8 (r / 4) + 4 g + (r % 4)
-        const bool masked = j0 + DM_BLOCK > mask_from;
-        vec8 pb[NRB][2];
+        // register r of sub-block kb2 is key j0 + 32 kb2 + 8 (r / 4) + 4 g + (r % 4)
+        const bool masked = j0 + BLOCK > mask_from;
+        vec8 pb[NRB][2 * KB];
 #pragma unroll
         for (int rb = 0; rb < NRB; ++rb) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) sacc[rb][r] *= sc2;
+            for (int kb2 = 0; kb2 < KB; ++kb2)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sacc[rb][kb2][r] *= sc2;
             if (masked) {
                 const int rel = lim[rb] - (j0 + 4 * g);
 #pragma unroll
-                for (int r = 0; r < 16; ++r)
-                    if (8 * (r / 4) + (r % 4) >= rel) sacc[rb][r] = -INFINITY;
-            }
-            float tmax = sacc[rb][0];
+                for (int kb2 = 0; kb2 < KB; ++kb2)
 #pragma unroll
-            for (int r = 1; r < 16; ++r) tmax = fmaxf(tmax, sacc[rb][r]);
+                    for (int r = 0; r < 16; ++r)
+                        if (32 * kb2 + 8 * (r / 4) + (r % 4) >= rel) sacc[rb][kb2][r] = -INFINITY;
+            }
+            float tmax = sacc[rb][0][0];
+#pragma unroll
+            for (int kb2 = 0; kb2 < KB; ++kb2)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, sacc[rb][kb2][r]);
             tmax = xor32_max(tmax);              // largest score of the row in this block (log2 units)
             // The reference the probabilities are taken against moves only when a block's maximum passes it by more
             // than 2^8 (or the row sees its first key): exact in exact arithmetic, probabilities stay <= 2^8, and O^T -
@@ -266,13 +276,13 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
                     for (int r = 0; r < 16; ++r) o_acc[rb][db][r] *= alpha;
             }
             const float m_use = (m_run[rb] == -INFINITY) ? 0.0f : m_run[rb];
-            // P^T in storage precision: element e of k-step ks is register 8 ks + e; the denominator is summed from
-            // the rounded values
+            // P^T in storage precision: element e of k-step ks is register 8 (ks % 2) + e of sub-block ks / 2; the
+            // denominator is summed from the rounded values
             float rsum = 0.0f;
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
+            for (int ks = 0; ks < 2 * KB; ++ks) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) pb[rb][ks][e] = (T)__builtin_amdgcn_exp2f(sacc[rb][8 * ks + e] - m_use);
+                for (int e = 0; e < 8; ++e) pb[rb][ks][e] = (T)__builtin_amdgcn_exp2f(sacc[rb][ks / 2][8 * (ks % 2) + e] - m_use);
 #pragma unroll
                 for (int e = 0; e < 8; e += 2) {
                     typename Mma<T>::vec2 pr = {pb[rb][ks][e], pb[rb][ks][e + 1]};
@@ -286,7 +296,7 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
         const char* vb = smem + (wave * NSLOT + slot_out) * DM_SLOT_BYTES;
         slot_out = slot_out + 1 == NSLOT ? 0 : slot_out + 1;
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks)
+        for (int ks = 0; ks < 2 * KB; ++ks)
 #pragma unroll
             for (int db = 0; db < NDB; ++db) {
                 short8v av;
@@ -324,7 +334,8 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
             for (int r = 0; r < 16; ++r) s_o[(((wave * NRB + rb) * NDB + db) * 16 + r) * 64 + lane] = o_acc[rb][db][r] * f;
     }
     __syncthreads();
-    // ---- this wavefront's 32 columns of every row ----------------------------------------------------------------
+    // ---- this wavefront's 32 columns of every row (D = 64: the first two wavefronts') -------------------------------
+    if (wave >= NDB) return;
 #pragma unroll
     for (int rb = 0; rb < NRB; ++rb) {
         if (!valid[rb]) continue;
@@ -369,13 +380,13 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
 
 hipError_t launch_sdpa_combine(const SdpaParams& p, int dtype, hipStream_t stream);
 
-template <typename T, int NSLOT, int NRB>
+template <typename T, int D, int NSLOT, int NRB>
 static hipError_t launch_decode_mfma_t(const SdpaParams& p, hipStream_t stream)
 {
     // the rings, or what the wavefronts' results need when they meet at the end, whichever is more
-    constexpr size_t ring_bytes = (size_t)4 * NSLOT * DM_SLOT_BYTES, merge_bytes = (size_t)NRB * (4 * 32 * 2 + 4 * 4 * 16 * 64) * sizeof(float);
+    constexpr size_t ring_bytes = (size_t)4 * NSLOT * DM_SLOT_BYTES, merge_bytes = (size_t)NRB * (4 * 32 * 2 + 4 * (D / 32) * 16 * 64) * sizeof(float);
     constexpr size_t lds = ring_bytes > merge_bytes ? ring_bytes : merge_bytes;
-    auto kern = sdpa_decode_mfma_kernel<T, NSLOT, NRB>;
+    auto kern = sdpa_decode_mfma_kernel<T, D, NSLOT, NRB>;
     // the dynamic-LDS limit of this instance is raised once per device, not per launch
     static std::atomic<uint64_t> prepared{0};
     int dev = 0;
@@ -401,28 +412,29 @@ int decode_mfma_chunk_rows(int R) { return R > 32 ? 64 : 32; }
 // otherwise.  The planner fills rounds of this many.
 int decode_mfma_workgroups_per_cu(int chunk_rows, int64_t split_len) { return chunk_rows == 32 && split_len <= DM_SHORT_KEYS ? 2 : 1; }
 
-// Host has validated: dtype f16 / bf16, D == Dv == 128, rows 16-byte aligned with unit last-dim stride, row strides
-// below 2^24 elements, split_len a multiple of 128 (every wavefront's blocks then start where its
-// neighbour's end in every split).
+// Host has validated: dtype f16 / bf16, D == Dv in {64, 128}, rows 16-byte aligned with unit last-dim stride, row strides
+// below 2^24 elements, split_len a multiple of 256 (whole rounds of the four wavefronts' blocks of 32 or 64 keys).
+template <typename T, int D>
+static hipError_t launch_decode_mfma_d(const SdpaParams& p, hipStream_t stream)
+{
+    if (decode_mfma_chunk_rows(p.G * p.Sq) == 64) return launch_decode_mfma_t<T, D, DM_NSLOT, 2>(p, stream);
+    // Short splits (up to DM_SHORT_KEYS keys: 16 blocks per wavefront) take rings of two slots, which lets a compute
+    // unit hold two workgroups: with so little to stream, what counts is that one workgroup's start-up (its first
+    // copies' latency) and end (the wavefronts' results meeting, the stores) overlap another's arithmetic.  Measured
+    // on launches of 268 MB of cache, two slots against five: 256-key splits 73 against 46 % of the memory bandwidth,
+    // 512: 81 / 63, 1024: 80 / 73, 2048: 87.5 / 86.3; 4096: 78.5 / 80 (one sequence of 131072 keys); 8192: 84 / 86.7.
+    // INCIN_ROCM_DECODE_SLOTS = 2 or 5 overrides the rule (for tests: both forms on any shape).
+    const char* forced = getenv("INCIN_ROCM_DECODE_SLOTS");
+    const int slots = forced ? atoi(forced) : 0;
+    if (slots == 2 || (slots != DM_NSLOT && decode_mfma_workgroups_per_cu(32, p.split_len) == 2)) return launch_decode_mfma_t<T, D, 2, 1>(p, stream);
+    return launch_decode_mfma_t<T, D, DM_NSLOT, 1>(p, stream);
+}
+
 hipError_t launch_sdpa_decode_mfma(const SdpaParams& p, int dtype, hipStream_t stream)
 {
     hipError_t e;
-    if (decode_mfma_chunk_rows(p.G * p.Sq) == 64) {
-        e = dtype == 1 ? launch_decode_mfma_t<f16_t, DM_NSLOT, 2>(p, stream) : launch_decode_mfma_t<bf16_t, DM_NSLOT, 2>(p, stream);
-    } else {
-        // Short splits (up to DM_SHORT_KEYS keys: 16 blocks per wavefront) take rings of two slots, which lets a compute
-        // unit hold two workgroups: with so little to stream, what counts is that one workgroup's start-up (its first
-        // copies' latency) and end (the wavefronts' results meeting, the stores) overlap another's arithmetic.  Measured
-        // on launches of 268 MB of cache, two slots against five: 256-key splits 73 against 46 % of the memory bandwidth,
-        // 512: 81 / 63, 1024: 80 / 73, 2048: 87.5 / 86.3; 4096: 78.5 / 80 (one sequence of 131072 keys); 8192: 84 / 86.7.
-        // INCIN_ROCM_DECODE_SLOTS = 2 or 5 overrides the rule (for tests: both forms on any shape).
-        const char* forced = getenv("INCIN_ROCM_DECODE_SLOTS");
-        const int slots = forced ? atoi(forced) : 0;
-        if (slots == 2 || (slots != DM_NSLOT && decode_mfma_workgroups_per_cu(32, p.split_len) == 2))
-            e = dtype == 1 ? launch_decode_mfma_t<f16_t, 2, 1>(p, stream) : launch_decode_mfma_t<bf16_t, 2, 1>(p, stream);
-        else
-            e = dtype == 1 ? launch_decode_mfma_t<f16_t, DM_NSLOT, 1>(p, stream) : launch_decode_mfma_t<bf16_t, DM_NSLOT, 1>(p, stream);
-    }
+    if (p.D == 128) e = dtype == 1 ? launch_decode_mfma_d<f16_t, 128>(p, stream) : launch_decode_mfma_d<bf16_t, 128>(p, stream);
+    else e = dtype == 1 ? launch_decode_mfma_d<f16_t, 64>(p, stream) : launch_decode_mfma_d<bf16_t, 64>(p, stream);
     if (e != hipSuccess || p.num_splits == 1) return e;
     return launch_sdpa_combine(p, dtype, stream);
 }

@@ -49,7 +49,7 @@ enum {
                                       IEEE-f32 matrix instructions for f32 (dense mask allowed)                    */
     INCIN_ROCM_IMPL_SPLITKV = 3,   /* split-KV decode kernel + combine: D == Dv in {64,128}, few query rows */
     INCIN_ROCM_IMPL_MFMA64 = 4,    /* bf16/f16 MFMA prefill kernel, 64 query rows per wavefront: D == Dv == 128 */
-    INCIN_ROCM_IMPL_SPLITKV_MFMA = 5 /* bf16/f16 split-KV kernel on the matrix cores + combine: D == Dv == 128, Sq <= 64; the rows that
+    INCIN_ROCM_IMPL_SPLITKV_MFMA = 5 /* bf16/f16 split-KV kernel on the matrix cores + combine: D == Dv in {64,128}, Sq <= 64; the rows that
                                       share a KV head (query heads of the group x query positions) go through it 32 at a time */
 };
 

@@ -79,8 +79,8 @@ def test_dispatch_choices():
     assert impl == capi.IMPL_SPLITKV_MFMA and splits == 32
     _, splits, impl = _plan(_desc(Sq=1, Skv=8192, B=32, Hq=32, Hkv=8))
     assert impl == capi.IMPL_SPLITKV_MFMA and splits == 1                     # 256 groups: one round, nothing to combine
-    assert _plan(_desc(Sq=1, Skv=8192, B=2, Hq=8, Hkv=2, dtype=capi.F32))[2] == capi.IMPL_SPLITKV   # f32, D = 64: vector ALU
-    assert _plan(_desc(Sq=1, Skv=8192, B=2, Hq=8, Hkv=2, D=64, Dv=64))[2] == capi.IMPL_SPLITKV
+    assert _plan(_desc(Sq=1, Skv=8192, B=2, Hq=8, Hkv=2, dtype=capi.F32))[2] == capi.IMPL_SPLITKV   # f32: vector ALU
+    assert _plan(_desc(Sq=1, Skv=8192, B=2, Hq=8, Hkv=2, D=64, Dv=64))[2] == capi.IMPL_SPLITKV_MFMA            # D = 64 too
     assert _plan(_desc(Sq=4, Skv=8192, B=2, Hq=32, Hkv=2))[2] == capi.IMPL_SPLITKV_MFMA             # 64 rows per KV head: one workgroup's worth
     assert _plan(_desc(Sq=8, Skv=8192, B=2, Hq=32, Hkv=2))[2] == capi.IMPL_SPLITKV_MFMA             # 128, but the prefill kernel would run 64 workgroups
     assert _plan(_desc(Sq=8, Skv=8192, B=8, Hq=32, Hkv=2))[2] == capi.IMPL_MFMA                     # 256 of them: a prefill shape
@@ -122,7 +122,7 @@ def test_dispatch_choices():
     (dict(impl=capi.IMPL_SPLITKV, Sq=4096), capi.EUNSUPPORTED),
     (dict(impl=capi.IMPL_SPLITKV_MFMA, Sq=4096), capi.EUNSUPPORTED),
     (dict(impl=capi.IMPL_SPLITKV_MFMA, Sq=1, dtype=capi.F32), capi.EUNSUPPORTED),
-    (dict(impl=capi.IMPL_SPLITKV_MFMA, Sq=1, D=64, Dv=64), capi.EUNSUPPORTED),
+    (dict(impl=capi.IMPL_SPLITKV_MFMA, Sq=1, D=32, Dv=32), capi.EUNSUPPORTED),
     (dict(impl=capi.IMPL_SPLITKV_MFMA, Sq=1, add_mask=0x20000), capi.EUNSUPPORTED),
     (dict(D=512, Dv=512), capi.EUNSUPPORTED),
     (dict(B=70000), capi.ESHAPE),

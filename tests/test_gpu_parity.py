@@ -426,6 +426,36 @@ def test_decode_splitkv_matrix_cores(gpu, dtype, shape, slots, monkeypatch):
         check(outs[0], valu, 8e-3, "matrix-core vs vector-ALU split-KV")
 
 
+@pytest.mark.parametrize("dtype", [capi.BF16, capi.F16])
+@pytest.mark.parametrize("slots", ["2", "5"], ids=["two_slot_rings", "five_slot_rings"])
+@pytest.mark.parametrize("shape", [
+    # B, Hq, Hkv, Sq, Skv, causal      (head dimension 64: blocks of 64 keys)
+    (2, 8, 2, 1, 4096, False),
+    (1, 14, 2, 1, 3001, False),       # 7 query heads per KV head, ragged last block
+    (2, 16, 1, 3, 777, True),         # 48 rows: the 64-row instance, causal among the positions
+    (1, 4, 4, 1, 130, False),         # two blocks and a bit
+    (1, 2, 1, 40, 2000, True),        # 80 rows: two chunks of 64
+])
+def test_decode_splitkv_matrix_cores_d64(gpu, dtype, shape, slots, monkeypatch):
+    """The same kernel at head dimension 64 (a slot holds 64 keys there) against the oracle and the vector-ALU kernel."""
+    monkeypatch.setenv("INCIN_ROCM_DECODE_SLOTS", slots)
+    B, Hq, Hkv, Sq, Skv, causal = shape
+    D = 64
+    q, k, v = inputs(900 + sum(shape[:5]), B, Hq, Hkv, Sq, Skv, D, D, dtype)
+    ref = oracle_full(q, k, v, G=Hq // Hkv, causal=causal)
+    lens = np.asarray([Skv - 1 - 37 * b for b in range(B)], np.int32)
+    ref_l = oracle_full(q, k, v, G=Hq // Hkv, causal=causal, kv_lens=lens)
+    for splits in (0, 1, 3, 9):
+        say("matrix-core split-KV, D = 64: %s %r splits=%d" % (dtypes.NAMES[dtype], shape, splits))
+        got, info = host.sdpa(q, k, v, dtype, causal=causal, num_splits=splits, impl=capi.IMPL_SPLITKV_MFMA, return_info=True)
+        assert info["impl"] == capi.IMPL_SPLITKV_MFMA
+        check(got, ref, TOL[dtype], "matrix-core split-KV D=64 %s %r splits=%d->%d" % (dtypes.NAMES[dtype], shape, splits, info["splits"]))
+        got = host.sdpa(q, k, v, dtype, causal=causal, kv_lens=lens, num_splits=splits, impl=capi.IMPL_SPLITKV_MFMA)
+        check(got, ref_l, TOL[dtype], "matrix-core split-KV D=64 with key counts")
+    if (Hq // Hkv) * Sq <= 8:
+        check(got, host.sdpa(q, k, v, dtype, causal=causal, kv_lens=lens, impl=capi.IMPL_SPLITKV), 8e-3, "matrix-core vs vector-ALU split-KV, D = 64")
+
+
 def test_decode_splitkv_matrix_cores_lengths_strides_scale(gpu):
     """Key counts per batch entry (one of them 0: NaN rows, as the reference), a negative scale (the scale is applied to
     the f32 scores, so its sign does not matter to this kernel), and AUTO's choice for grouped-query decode."""
