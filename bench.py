@@ -65,7 +65,7 @@ def causal_flops(B, Hq, Sq, Skv, D):
 class Workload:
     """Device-resident operands + descriptor for one configuration."""
 
-    def __init__(self, name, seed, B, Hq, Hkv, Sq, Skv, D, dtype, causal, kv_lens=None, pad_queries=False, impl=capi.IMPL_AUTO):
+    def __init__(self, name, seed, B, Hq, Hkv, Sq, Skv, D, dtype, causal, kv_lens=None, pad_queries=False, impl=capi.IMPL_AUTO, num_splits=0):
         self.name, self.shape = name, (B, Hq, Hkv, Sq, Skv, D)
         self.dtype, self.causal, self.kv_lens = dtype, causal, kv_lens
         q, k, v = make_inputs(seed, B, Hq, Hkv, Sq, Skv, D, dtype)
@@ -75,7 +75,7 @@ class Workload:
         self.tl = capi.DeviceBuffer.from_numpy(np.asarray(kv_lens, dtype=np.int32)) if kv_lens is not None else None
         # a padded self-attention batch: the same lengths say which keys and which query rows are padding
         self.desc = host.make_desc(self.tq, self.tk, self.tv, self.to, causal=causal, kv_lens=self.tl,
-                                   q_lens=self.tl if pad_queries else None, impl=impl)
+                                   q_lens=self.tl if pad_queries else None, impl=impl, num_splits=num_splits)
         nbytes, self.splits, self.impl = capi.sdpa_workspace(self.desc)
         self.ws = capi.DeviceBuffer(nbytes) if nbytes else None
         if self.ws is not None:
@@ -177,6 +177,29 @@ def cpu_baseline_decode(D, Skv, B, H, dtype):
     O.sdpa_materialised(q, k, v)
     dt = time.perf_counter() - t0
     return 2.0 * B * H * Skv * D * 2 / dt / 1e9, dt
+
+
+def prefill_chunk_leg(steps, warmup):
+    """A chunk of a long prompt: few query rows (one sequence, 128 or 512 new positions) over a long cache, causal.  The
+    launch has 32 or 128 (head, row block) items for 256 compute units, so the library splits the key axis and combines
+    the partial results; beside it the same launch unsplit (num_splits = 1)."""
+    out = {}
+    for i, (Sq, Skv) in enumerate(((128, 32768), (512, 32768))):
+        B, Hq, Hkv, D = 1, 32, 8, 128
+        flops = 4.0 * D * Hq * B * (Sq * Skv - Sq * (Sq - 1) / 2.0)
+        entry = {"workload": "bf16 causal prefill chunk B=%d Hq=%d Hkv=%d S_q=%d over KV=%d D=128" % (B, Hq, Hkv, Sq, Skv)}
+        for name, ns in (("auto", 0), ("unsplit", 1)):
+            w = Workload("chunk", SEED0 + 60 + i, B, Hq, Hkv, Sq, Skv, D, capi.BF16, True, num_splits=ns)
+            wall, ev_mean, ev_med, ev_min = w.time(max(steps, 100), warmup)
+            entry[name] = {"num_splits": w.splits, "ms_per_step": wall, "tflops": flops / (wall * 1e-3) / 1e12,
+                           "roofline": {"bound": "mfma", "achieved": flops / (ev_mean * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                                        "frac": flops / (ev_mean * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": None,
+                                        "kernel": "sdpa_prefill_mfma_kernel<bf16,128>" + (" over splits of the keys + sdpa_combine_kernel" if w.splits > 1 else ""),
+                                        "algorithmic_flops_per_launch": flops, "launch_ms_mean": ev_mean, "launch_ms_min": ev_min},
+                           "parity_max_abs_err": w.parity(16)}
+            w.free()
+        out["sq%d_kv%d" % (Sq, Skv)] = entry
+    return out
 
 
 def decode_gqa_leg(steps, warmup, only_shape=None):
@@ -426,7 +449,7 @@ def main():
                     help="prefill_long: skip the extra timing of the batch with its padding rows computed (profiling: every "
                          "launch of the run is then the same launch)")
     ap.add_argument("--decode-gqa-shape", default=None, help="with --only decode_gqa: one of its shapes by name (for profiles)")
-    ap.add_argument("--only", choices=["prefill", "prefill_long", "decode", "decode_gqa", "backward", "f32", "copy", "matrix_rate"], default=None,
+    ap.add_argument("--only", choices=["prefill", "prefill_long", "prefill_chunk", "decode", "decode_gqa", "backward", "f32", "copy", "matrix_rate"], default=None,
                     help="run a single workload (profiling). 'copy' runs --steps device-to-device copies of 1 GiB "
                          "through the library's plain copy kernel: the known-size dispatch that hardware byte "
                          "counters (FETCH_SIZE / WRITE_SIZE) are calibrated against")
@@ -568,6 +591,9 @@ def main():
                                    "sample": "all of config 4 (B=32, H=32, KV=8192, D=128), oracle's materialising restatement of "
                                              "the reference CPU op (serial matmuls and reductions); %.1f s; host: %s" % (dt, host_cpu())}
         result["decode"] = dec
+
+    if args.only in (None, "prefill_chunk"):
+        result["prefill_chunk"] = prefill_chunk_leg(args.steps, args.warmup)
 
     if args.only in (None, "decode_gqa"):
         result["decode_gqa"] = decode_gqa_leg(args.steps, args.warmup, args.decode_gqa_shape)

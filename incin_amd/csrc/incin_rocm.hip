@@ -273,6 +273,32 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         plan->ws_bytes = splits > 1 ? (size_t)(d->B * d->Hq * d->Sq * splits) * (size_t)(d->Dv + 2) * sizeof(float) : 0;
     }
     if (impl == INCIN_ROCM_IMPL_MFMA64) plan->ws_bytes = MFMA64_WS_BYTES;      // the launch's work counters
+    if (impl == INCIN_ROCM_IMPL_MFMA && d->dtype != INCIN_ROCM_F32 && !d->add_mask && !d->lse && !d->q_lens) {
+        // The 16-bit prefill kernel runs one workgroup per (batch, query head, 128 rows) and a compute unit holds two:
+        // when a launch has at most one per compute unit and a long key axis - a chunk of a long prompt, a single
+        // sequence - the keys are split as for decode, as many ways as fill the device (1024 keys per split at least:
+        // measured best on 32 heads x 128 rows x 8192 keys, 8 splits 32 us against 40 with 4 and 35 with 16), and the
+        // splits' partial results go through the split-KV kernels' combine pass.  num_splits > 0 in the descriptor forces
+        // a count.
+        const int64_t cus = compute_units_of(d->device);
+        const int64_t wgs = d->B * d->Hq * ((d->Sq + 127) / 128);
+        int64_t splits = d->num_splits;
+        if (splits == 0) {
+            splits = 1;
+            if (wgs <= cus && d->Skv >= 4096) splits = std::min<int64_t>(2 * cus / wgs, d->Skv / 1024);
+        }
+        if (splits > 1) {
+            int64_t split_len = (d->Skv + splits - 1) / splits;
+            split_len = (split_len + 127) / 128 * 128;       // whole pairs of 64-key tiles: every split starts on an even tile
+            splits = (d->Skv + split_len - 1) / split_len;
+            if (splits > 65535) return fail(INCIN_ROCM_ESHAPE, "scaled_dot_product_attention: too many splits");
+            if (splits > 1) {
+                plan->splits = (int)splits;
+                plan->split_len = (int)split_len;
+                plan->ws_bytes = (size_t)(d->B * d->Hq * d->Sq * splits) * (size_t)(d->Dv + 2) * sizeof(float);
+            }
+        }
+    }
     if (impl == INCIN_ROCM_IMPL_MFMA && d->add_mask) {
         // one flag per block of 32 query rows x 32 keys of the mask, per mask batch entry and head
         const int64_t nbh = (d->mask_stride[0] ? d->B : 1) * (d->mask_stride[1] ? d->Hq : 1);
@@ -308,7 +334,7 @@ void fill_params(const incin_rocm_sdpa_desc_t* d, const Plan& plan, SdpaParams* 
     p->split_len = plan.split_len;
     if (plan.impl == INCIN_ROCM_IMPL_MFMA64) p->sched = (int32_t*)d->workspace;
     else if (plan.impl == INCIN_ROCM_IMPL_MFMA) p->mask_flags = d->add_mask ? (const uint8_t*)d->workspace : nullptr;
-    else p->ws_acc = (float*)d->workspace;
+    if (plan.impl != INCIN_ROCM_IMPL_MFMA64 && !(plan.impl == INCIN_ROCM_IMPL_MFMA && d->add_mask)) p->ws_acc = (float*)d->workspace;
     if (plan.splits > 1) {
         const size_t rows = (size_t)(d->B * d->Hq * d->Sq * plan.splits);
         p->ws_ml = (float*)d->workspace + rows * (size_t)d->Dv;
@@ -585,7 +611,7 @@ static int launch_fwd(const incin_rocm_sdpa_desc_t* desc, const Plan& plan, void
         if (!desc->workspace || desc->workspace_bytes < plan.ws_bytes)
             return fail(INCIN_ROCM_EWORKSPACE,
                         "scaled_dot_product_attention: %s needs %zu workspace bytes, %zu given",
-                        plan.impl == INCIN_ROCM_IMPL_MFMA64 ? "the 64-row MFMA kernel" : plan.impl == INCIN_ROCM_IMPL_MFMA ? "a dense mask on the MFMA kernels" : "split-KV",
+                        plan.impl == INCIN_ROCM_IMPL_MFMA64 ? "the 64-row MFMA kernel" : plan.impl != INCIN_ROCM_IMPL_MFMA ? "split-KV" : desc->add_mask ? "a dense mask on the MFMA kernels" : "the MFMA prefill kernel with the keys split",
                         plan.ws_bytes,
                         desc->workspace ? desc->workspace_bytes : (size_t)0);
         if (!aligned16(desc->workspace)) return fail(INCIN_ROCM_EWORKSPACE, "scaled_dot_product_attention: workspace must be 16-byte aligned");
@@ -649,6 +675,14 @@ int incin_rocm_sdpa_fwd_static(const incin_rocm_sdpa_desc_t* desc, void* stream)
     Plan plan;
     if (int rc = make_plan(desc, &plan)) return rc;
     if (plan.empty) return 0;
+    if (plan.ws_bytes > (size_t)INCIN_ROCM_STATIC_SCRATCH_BYTES && plan.impl == INCIN_ROCM_IMPL_MFMA && !desc->add_mask &&
+        desc->num_splits == 0) {
+        // a prefill launch whose keys the library chose to split, with more partial results than the buffer holds: the
+        // same launch without splits needs no scratch memory at all
+        incin_rocm_sdpa_desc_t whole = *desc;
+        whole.num_splits = 1;
+        if (int rc = make_plan(&whole, &plan)) return rc;
+    }
     if (plan.ws_bytes > (size_t)INCIN_ROCM_STATIC_SCRATCH_BYTES)
         return fail(INCIN_ROCM_EWORKSPACE,
                     "sdpa_fwd_static: this request needs %zu bytes of scratch memory, the static buffer holds %zu "

@@ -78,7 +78,12 @@ namespace incin_rocm {
 
 // NW wavefronts = 32 * NW query rows per workgroup: 4 (two workgroups per compute unit) or 8 (one, whose K / V tiles then
 // serve 256 rows: half the global -> LDS copies per matrix instruction).
-template <typename T, int D, bool DENSE, int NW>
+//
+// SPLIT: the launch is a grid of (work items) x (splits of the key axis); a workgroup handles the keys of its split only and
+// writes, per row, the unnormalised O, the reference and the sum - the partial-result format of the split-KV kernels, whose
+// combine kernel finishes the job.  For launches with too few (batch, head, row block) items to fill the device over a long
+// key axis (a chunk of a long prompt, a single sequence): the key axis supplies the parallelism the rows lack.
+template <typename T, int D, bool DENSE, int NW, bool SPLIT = false>
 __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void sdpa_prefill_mfma_kernel(SdpaParams p)
 {
@@ -121,6 +126,9 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
 
     int kv_len = Skv;
     if (p.kv_lens) kv_len = clampi(p.kv_lens[b], 0, Skv);
+    // a split ends where the next begins: to this workgroup the keys beyond do not exist (split_len is a multiple of two tiles)
+    const int split = SPLIT ? (int)blockIdx.y : 0;
+    if (SPLIT) kv_len = min(kv_len, (split + 1) * p.split_len);
     // query rows at and beyond rows_b are padding: nothing is computed or stored for them
     const int rows_b = p.q_lens ? clampi(p.q_lens[b], 0, Sq) : Sq;
     if (q0 >= rows_b) return;                          // the whole block is padding (uniform: before any barrier)
@@ -145,7 +153,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     const uint8_t* mflags = nullptr;
     const T* mrow = nullptr;
     const int nkb32 = (Skv + 31) >> 5;
-    int t_first = 0;
+    int t_first = SPLIT ? min(split * (p.split_len / PF_BN), n_tiles) : 0;
     [[maybe_unused]] int w_first = 0, w_last = 0x7fffffff;      // this wavefront's first and last tile with a visible block
     [[maybe_unused]] int z_end = 0;
     __shared__ int s_range[2 * NW];
@@ -624,17 +632,18 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     const int n_act = lim_wave_max > 0 ? (lim_wave_max + PF_BN - 1) / PF_BN : 0;
     const int n_hot = lim_wave_min > 0 ? min(lim_wave_min / PF_BN, n_act) : 0;      // tiles 0..n_hot-1 need no mask
 
-    if (!DENSE && n_tiles > 0) {
-        // prologue: K(0), K(1), V(0) are in flight since the start; scores of tile 0
+    if (!DENSE && n_tiles > t_first) {
+        // prologue: K and V of the first tile (tile 0, or a split's first: an even one) and K of the next are in flight since
+        // the start; scores of the first tile
         __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0), told to the compiler too: it then knows the Q rows have arrived
         asm volatile("" ::: "memory");
         __syncthreads();
-        if (n_act > 0) scores_plain(smem, sacc[0], 0);
-        int t = 0;
+        if (n_act > t_first) scores_plain(smem, sacc[0], t_first * PF_BN);
+        int t = t_first;
         if constexpr (ORCHK) {
-            if (2 < n_hot) {
-                // the reference of every row of this wavefront: the maximum of tile 0 (nothing accumulated yet, so
-                // nothing to rescale)
+            if (t_first + 2 < n_hot) {
+                // the reference of every row of this wavefront: the maximum of the first tile (nothing accumulated yet,
+                // so nothing to rescale)
                 {
                     const bool need = tmax > -INFINITY;
                     const float delta = need ? tmax + SHIFT : 0.0f;
@@ -746,6 +755,27 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
 
     // ---- normalise and store ------------------------------------------------------------------
     const float l_tot = xor32_sum(l_run);
+    if constexpr (SPLIT) {
+        // partial result of this split: unnormalised O, and (reference, sum) in the log2 units the combine kernel takes for
+        // 16-bit storage; a row that saw no key in this split says so with a reference of -inf
+        if (my_i < rows_b) {
+            const int64_t slot = (((int64_t)b * p.Hq + hq) * Sq + my_i) * p.num_splits + split;
+            float* arow = p.ws_acc + slot * D + g * 4;
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    typedef float f4 __attribute__((ext_vector_type(4)));
+                    f4 w = {o_acc[db][r4 * 4], o_acc[db][r4 * 4 + 1], o_acc[db][r4 * 4 + 2], o_acc[db][r4 * 4 + 3]};
+                    *(f4*)(arow + db * 32 + r4 * 8) = w;
+                }
+            if (g == 0) {
+                p.ws_ml[slot * 2 + 0] = l_tot == 0.0f ? -INFINITY : m_ref;
+                p.ws_ml[slot * 2 + 1] = l_tot;
+            }
+        }
+        return;
+    }
     const float inv = (l_tot == 0.0f) ? __builtin_nanf("") : 1.0f / l_tot;   // no visible key: NaN, as the reference
     if (p.lse && g == 0 && my_i < rows_b)       // m_ref and the sum are in log2 units of the scaled scores
         p.lse[((int64_t)b * p.Hq + hq) * Sq + my_i] = l_tot == 0.0f ? -INFINITY : (m_ref + __builtin_log2f(l_tot)) * 0.6931471805599453f;
@@ -765,6 +795,8 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
 #endif
 }
 
+hipError_t launch_sdpa_combine(const SdpaParams& p, int dtype, hipStream_t stream);
+
 template <typename T, int D, bool DENSE, int NW>
 static hipError_t launch_prefill_nw(const SdpaParams& p0, hipStream_t stream)
 {
@@ -775,6 +807,13 @@ static hipError_t launch_prefill_nw(const SdpaParams& p0, hipStream_t stream)
     // of the compute units per XCD
     p.interleave = work_interleave(p.causal != 0, (8 / NW) * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
     p.deal_groups = (total & 7) == 0 ? work_deal(p.interleave, p.G, nqb, total >> 3) : 0;
+    if constexpr (!DENSE && NW == 4) {
+        if (p.num_splits > 1) {          // split launch: partial results, then the split-KV kernels' combine pass
+            hipLaunchKernelGGL((sdpa_prefill_mfma_kernel<T, D, false, 4, true>), dim3((unsigned)total, (unsigned)p.num_splits), dim3(256), 0, stream, p);
+            hipError_t e = hipGetLastError();
+            return e != hipSuccess ? e : launch_sdpa_combine(p, std::is_same<T, f16_t>::value ? 1 : 2, stream);
+        }
+    }
     hipLaunchKernelGGL((sdpa_prefill_mfma_kernel<T, D, DENSE, NW>), dim3((unsigned)total), dim3(64 * NW), 0, stream, p);
     return hipGetLastError();
 }
@@ -791,7 +830,7 @@ static hipError_t launch_prefill_t(const SdpaParams& p, hipStream_t stream)
         const char* forced = getenv("INCIN_ROCM_PREFILL_BLOCK_ROWS");
         const int rows = forced ? atoi(forced) : 0;
         const int64_t blocks256 = (int64_t)((p.Sq + 255) / 256) * p.Hq * p.B;
-        if (rows == 256 || (rows != 128 && p.Skv >= 4096 && blocks256 >= 6 * (int64_t)device_cus()))
+        if (p.num_splits <= 1 && (rows == 256 || (rows != 128 && p.Skv >= 4096 && blocks256 >= 6 * (int64_t)device_cus())))
             return launch_prefill_nw<T, D, DENSE, 8>(p, stream);
     }
     return launch_prefill_nw<T, D, DENSE, 4>(p, stream);

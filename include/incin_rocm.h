@@ -178,7 +178,7 @@ typedef struct {
     int64_t mask_stride[4];        /* elements: batch, query head, query row, key; 0 = broadcast */
     void* workspace;               /* device scratch for split-KV partials; see incin_rocm_sdpa_workspace */
     size_t workspace_bytes;
-    int32_t num_splits;            /* 0 = library chooses */
+    int32_t num_splits;            /* splits of the key axis (split-KV kernels; 16-bit MFMA prefill kernel): 0 = library chooses, 1 = none */
     int32_t impl;                  /* INCIN_ROCM_IMPL_*; AUTO unless a test pins a kernel */
     const int32_t* q_lens;         /* nullable device pointer, B entries: rows at and beyond are padding */
     float* lse;                    /* nullable device pointer, contiguous f32 [B, Hq, Sq]: receives log sum_j exp(x_ij) of
@@ -197,8 +197,9 @@ int incin_rocm_sdpa_workspace(const incin_rocm_sdpa_desc_t* desc, size_t* bytes,
  * stream-ordered use of the buffers named in the descriptor, which the caller
  * keeps alive until the stream has been synchronised.
  *
- * Workspace.  Three launches need scratch memory, of the size incin_rocm_sdpa_workspace reports: the split-KV
- * kernels when they split (partial results of the splits), the 64-row MFMA prefill kernel (256 bytes: the work counters its
+ * Workspace.  Three launches need scratch memory, of the size incin_rocm_sdpa_workspace reports: launches that split
+ * the key axis - the split-KV kernels, and the 16-bit MFMA prefill kernel when few row blocks meet many keys - (partial
+ * results of the splits), the 64-row MFMA prefill kernel (256 bytes: the work counters its
  * persistent workgroups draw from, cleared by the launch itself) and the MFMA prefill kernels with a dense mask
  * (one byte per block of 32 query rows x 32 keys of the mask: which blocks it hides, which it leaves alone;
  * written by a small kernel of the same launch).  The contents need not survive the launch and

@@ -105,6 +105,22 @@ def test_dispatch_choices():
     assert _plan(long(S=2048))[2] == capi.IMPL_MFMA
     assert _plan(long(D=64, Dv=64))[2] == capi.IMPL_MFMA
     assert _plan(_desc(Sq=8192, Skv=8192))[2] == capi.IMPL_MFMA          # 2 x 4 heads x 32 blocks: too few items
+    # few row blocks over many keys: the prefill launch splits the keys (and then needs a workspace for the partial results)
+    def chunk(B, Hq, Hkv, Sq, Skv, **kw):
+        d = _desc(B=B, Hq=Hq, Hkv=Hkv, Sq=Sq, Skv=Skv, **kw)
+        for name, heads, rows in (("q_stride", Hq, Sq), ("k_stride", Hkv, Skv), ("v_stride", Hkv, Skv), ("o_stride", Hq, Sq)):
+            st = getattr(d, name)
+            st[0], st[1], st[2] = heads * rows * d.D, rows * d.D, d.D
+        return d
+    nbytes, splits, impl = _plan(chunk(1, 8, 8, 128, 4096, causal=1))
+    assert impl == capi.IMPL_MFMA and splits == 4 and nbytes == 1 * 8 * 128 * 4 * 130 * 4       # 8 workgroups, 1024 keys per split at least
+    nbytes, splits, impl = _plan(chunk(1, 32, 8, 512, 32768))
+    assert impl == capi.IMPL_MFMA and splits == 4                                               # 128 workgroups: 4 x fills both slots of every compute unit
+    assert _plan(chunk(1, 32, 8, 512, 32768, num_splits=1))[1] == 1
+    assert _plan(chunk(4, 32, 8, 512, 32768))[1] == 1                                           # 512 workgroups: the rows fill the device
+    assert _plan(chunk(1, 8, 8, 128, 2048))[1] == 1                                             # too few keys to split
+    assert _plan(chunk(1, 32, 8, 512, 32768, lse=0x30000))[1] == 1                              # the row normalisers come from the unsplit kernel
+    assert _plan(chunk(1, 32, 8, 512, 32768, dtype=capi.F32))[1] == 1                           # (the f32 kernel does not split)
     # empty problems need nothing
     assert _plan(_desc(Sq=0))[0] == 0
 

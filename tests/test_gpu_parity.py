@@ -360,6 +360,34 @@ def test_row_normalisers(gpu, impl):
     assert info["impl"] != capi.IMPL_SPLITKV
 
 
+@pytest.mark.parametrize("dtype", [capi.BF16, capi.F16])
+@pytest.mark.parametrize("shape", [
+    # B, Hq, Hkv, Sq, Skv, D, causal, key counts
+    (1, 8, 2, 300, 5000, 128, True, None),          # a chunk of a long prompt: 24 workgroups, the keys supply the rest
+    (1, 4, 4, 128, 4608, 128, False, None),
+    (2, 2, 1, 77, 9000, 128, True, [9000, 4100]),   # the second sequence ends inside a split
+    (1, 6, 3, 200, 4500, 64, True, None),           # head dimension 64
+    (1, 2, 2, 130, 4096, 128, True, [300]),         # most splits see no key at all
+])
+def test_prefill_with_the_keys_split(gpu, dtype, shape):
+    """The 16-bit prefill kernel over splits of the key axis + combine (what AUTO does for launches with few row blocks
+    over many keys): against the oracle with the library's split count and forced ones, and against the unsplit launch."""
+    B, Hq, Hkv, Sq, Skv, D, causal, lens = shape
+    q, k, v = inputs(1200 + Sq + Skv, B, Hq, Hkv, Sq, Skv, D, D, dtype)
+    lens = None if lens is None else np.asarray(lens, np.int32)
+    ref = oracle_full(q, k, v, G=Hq // Hkv, causal=causal, kv_lens=lens)
+    whole, info = host.sdpa(q, k, v, dtype, causal=causal, kv_lens=lens, impl=capi.IMPL_MFMA, num_splits=1, return_info=True)
+    assert info["splits"] == 1
+    for splits in (0, 2, 5, 13):
+        say("prefill with the keys split: %s %r splits=%d" % (dtypes.NAMES[dtype], shape, splits))
+        got, info = host.sdpa(q, k, v, dtype, causal=causal, kv_lens=lens, impl=capi.IMPL_MFMA, num_splits=splits, return_info=True)
+        assert info["impl"] == capi.IMPL_MFMA and info["splits"] > 1 and info["workspace_bytes"] > 0
+        check(got, ref, TOL[dtype], "prefill, keys split %d ways" % info["splits"])
+        check(got, whole, 8e-3, "split vs whole")
+    got, info = host.sdpa(q, k, v, dtype, causal=causal, kv_lens=lens, return_info=True)      # AUTO comes to the same launch
+    assert info["impl"] == capi.IMPL_MFMA and info["splits"] > 1
+
+
 # ---- split-KV decode -----------------------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", [capi.BF16, capi.F16, capi.F32])

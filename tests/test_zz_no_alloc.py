@@ -65,6 +65,9 @@ def test_static_scratch_matches_workspace_launch(gpu):
         ("matrix-core split-KV decode",
          dict(B=2, Hq=16, Hkv=2, Sq=1, Skv=4096, D=128, causal=False, impl=capi.IMPL_SPLITKV_MFMA, num_splits=8),
          dict(B=2, Hq=12, Hkv=2, Sq=3, Skv=1500, D=128, causal=True, impl=capi.IMPL_SPLITKV_MFMA, num_splits=3, kv_lens=[1500, 700])),
+        ("prefill with the keys split",
+         dict(B=1, Hq=4, Hkv=2, Sq=100, Skv=4500, D=128, causal=True, impl=capi.IMPL_MFMA),
+         dict(B=1, Hq=2, Hkv=2, Sq=40, Skv=4100, D=128, causal=False, impl=capi.IMPL_MFMA, num_splits=3)),
         ("64-row prefill",
          dict(B=2, Hq=8, Hkv=2, Sq=1024, Skv=1024, D=128, causal=True, impl=capi.IMPL_MFMA64),
          dict(B=1, Hq=3, Hkv=3, Sq=300, Skv=300, D=128, causal=True, impl=capi.IMPL_MFMA64)),
@@ -103,3 +106,27 @@ def test_static_scratch_limit_and_no_workspace_needed(gpu):
     capi.sdpa_fwd_static(d)
     capi.sync()
     assert np.array_equal(to.to_f32(), want)
+
+
+def test_static_scratch_takes_a_prefill_launch_whole_when_its_partials_do_not_fit(gpu):
+    """The library would split the keys of this launch (few row blocks, many keys) and the splits' partial results
+    exceed the static buffer: the entry point runs the launch unsplit - no scratch memory needed - instead of refusing."""
+    B, Hq, Hkv, Sq, Skv, D = 1, 32, 8, 256, 16384, 128
+    r = np.random.Generator(np.random.PCG64(5))
+    mk = lambda *s: dtypes.round_to(r.standard_normal(s, dtype=np.float32), capi.BF16)
+    q, k, v = mk(B, Hq, Sq, D), mk(B, Hkv, Skv, D), mk(B, Hkv, Skv, D)
+    tq, tk, tv = (host.DeviceTensor.from_f32(x, capi.BF16) for x in (q, k, v))
+    to = host.DeviceTensor((B, Hq, Sq, D), capi.BF16)
+    d = host.make_desc(tq, tk, tv, to, causal=True)
+    nbytes, splits, impl = capi.sdpa_workspace(d)
+    assert impl == capi.IMPL_MFMA and splits > 1 and nbytes > capi.STATIC_SCRATCH_BYTES
+    capi.sdpa_fwd_static(d)
+    capi.sync()
+    got = to.to_f32()
+    whole = host.sdpa(q, k, v, capi.BF16, causal=True, impl=capi.IMPL_MFMA, num_splits=1)
+    assert np.array_equal(got, whole)
+    # a forced split count beyond the buffer is refused as before
+    d.num_splits = splits
+    with pytest.raises(capi.RocmError) as e:
+        capi.sdpa_fwd_static(d)
+    assert e.value.code == capi.EWORKSPACE
