@@ -184,21 +184,23 @@ def prefill_chunk_leg(steps, warmup):
     launch has 32 or 128 (head, row block) items for 256 compute units, so the library splits the key axis and combines
     the partial results; beside it the same launch unsplit (num_splits = 1)."""
     out = {}
-    for i, (Sq, Skv) in enumerate(((128, 32768), (512, 32768))):
+    for i, (dt, Sq, Skv) in enumerate(((capi.BF16, 128, 32768), (capi.BF16, 512, 32768), (capi.F32, 128, 32768))):
         B, Hq, Hkv, D = 1, 32, 8, 128
         flops = 4.0 * D * Hq * B * (Sq * Skv - Sq * (Sq - 1) / 2.0)
-        entry = {"workload": "bf16 causal prefill chunk B=%d Hq=%d Hkv=%d S_q=%d over KV=%d D=128" % (B, Hq, Hkv, Sq, Skv)}
+        peak = PEAK_F32_TFLOPS if dt == capi.F32 else PEAK_BF16_TFLOPS
+        kernel = "sdpa_prefill_f32_kernel<128>" if dt == capi.F32 else "sdpa_prefill_mfma_kernel<bf16,128>"
+        entry = {"workload": "%s causal prefill chunk B=%d Hq=%d Hkv=%d S_q=%d over KV=%d D=128" % (dtypes.NAMES[dt], B, Hq, Hkv, Sq, Skv)}
         for name, ns in (("auto", 0), ("unsplit", 1)):
-            w = Workload("chunk", SEED0 + 60 + i, B, Hq, Hkv, Sq, Skv, D, capi.BF16, True, num_splits=ns)
-            wall, ev_mean, ev_med, ev_min = w.time(max(steps, 100), warmup)
+            w = Workload("chunk", SEED0 + 60 + i, B, Hq, Hkv, Sq, Skv, D, dt, True, num_splits=ns)
+            wall, ev_mean, ev_med, ev_min = w.time(max(steps, 100) if dt != capi.F32 else 20, warmup if dt != capi.F32 else 3)
             entry[name] = {"num_splits": w.splits, "ms_per_step": wall, "tflops": flops / (wall * 1e-3) / 1e12,
-                           "roofline": {"bound": "mfma", "achieved": flops / (ev_mean * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                                        "frac": flops / (ev_mean * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": None,
-                                        "kernel": "sdpa_prefill_mfma_kernel<bf16,128>" + (" over splits of the keys + sdpa_combine_kernel" if w.splits > 1 else ""),
+                           "roofline": {"bound": "mfma", "achieved": flops / (ev_mean * 1e-3) / 1e12, "peak": peak, "unit": "TFLOP/s",
+                                        "frac": flops / (ev_mean * 1e-3) / 1e12 / peak, "traffic": None,
+                                        "kernel": kernel + (" over splits of the keys + sdpa_combine_kernel" if w.splits > 1 else ""),
                                         "algorithmic_flops_per_launch": flops, "launch_ms_mean": ev_mean, "launch_ms_min": ev_min},
                            "parity_max_abs_err": w.parity(16)}
             w.free()
-        out["sq%d_kv%d" % (Sq, Skv)] = entry
+        out["%s_sq%d_kv%d" % (dtypes.NAMES[dt], Sq, Skv)] = entry
     return out
 
 

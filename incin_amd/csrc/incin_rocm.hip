@@ -273,8 +273,8 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         plan->ws_bytes = splits > 1 ? (size_t)(d->B * d->Hq * d->Sq * splits) * (size_t)(d->Dv + 2) * sizeof(float) : 0;
     }
     if (impl == INCIN_ROCM_IMPL_MFMA64) plan->ws_bytes = MFMA64_WS_BYTES;      // the launch's work counters
-    if (impl == INCIN_ROCM_IMPL_MFMA && d->dtype != INCIN_ROCM_F32 && !d->add_mask && !d->lse && !d->q_lens) {
-        // The 16-bit prefill kernel runs one workgroup per (batch, query head, 128 rows) and a compute unit holds two:
+    if (impl == INCIN_ROCM_IMPL_MFMA && !d->add_mask && !d->lse && !d->q_lens) {
+        // The prefill kernels (16-bit and f32) run one workgroup per (batch, query head, 128 rows) and a compute unit holds two:
         // when a launch has at most one per compute unit and a long key axis - a chunk of a long prompt, a single
         // sequence - the keys are split as for decode, as many ways as fill the device (1024 keys per split at least:
         // measured best on 32 heads x 128 rows x 8192 keys, 8 splits 32 us against 40 with 4 and 35 with 16), and the

@@ -47,7 +47,10 @@ template <int D> struct F32Layout {
     static __device__ __forceinline__ int f(int r) { return (r & 3) | ((r & 4) << 1) | ((r & 8) >> 1); }
 };
 
-template <int D, bool DENSE>
+// SPLIT: the launch is a grid of (work items) x (splits of the key axis); a workgroup handles the keys of its split only and
+// writes, per row, the unnormalised O, the maximum and the sum in the partial-result format of the split-KV kernels, whose
+// combine kernel finishes - for launches with too few (batch, head, row block) items to fill the device over a long key axis.
+template <int D, bool DENSE, bool SPLIT = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void sdpa_prefill_f32_kernel(SdpaParams p)
 {
@@ -84,6 +87,9 @@ void sdpa_prefill_f32_kernel(SdpaParams p)
 
     int kv_len = Skv;
     if (p.kv_lens) kv_len = clampi(p.kv_lens[b], 0, Skv);
+    // a split ends where the next begins: to this workgroup the keys beyond do not exist (split_len is a multiple of the tile)
+    const int split = SPLIT ? (int)blockIdx.y : 0;
+    if (SPLIT) kv_len = min(kv_len, (split + 1) * p.split_len);
     const int rows_b = p.q_lens ? clampi(p.q_lens[b], 0, Sq) : Sq;      // query rows at and beyond are padding
     if (q0 >= rows_b) return;                                           // (uniform: before any barrier)
     const int coff = Skv - Sq;
@@ -99,6 +105,7 @@ void sdpa_prefill_f32_kernel(SdpaParams p)
     }
     if (q0 + wave * 32 >= rows_b) lim_wave_min = lim_wave_max = 0;      // a wavefront of padding rows only keeps the barriers company
     const int n_tiles = (j_end + KT - 1) / KT;
+    const int t_first = SPLIT ? min(split * (p.split_len / KT), n_tiles) : 0;
     const int n_act = lim_wave_max > 0 ? (lim_wave_max + KT - 1) / KT : 0;      // tiles this wavefront computes
 
     // ---- global -> LDS copy plan: wavefront-wide load ii = wave * LPW + c fills LDS bytes [ii * 1024, +1024) of a tile
@@ -170,8 +177,8 @@ void sdpa_prefill_f32_kernel(SdpaParams p)
     float m_run = -INFINITY;      // running maximum (log2 units) of this lane's query, the same in lanes l and l ^ 32
     float l_run = 0.0f;           // this lane's share of the running denominator
 
-    if (n_tiles > 0) issue_kv(0);
-    for (int t = 0; t < n_tiles; ++t) {
+    if (n_tiles > t_first) issue_kv(t_first);
+    for (int t = t_first; t < n_tiles; ++t) {
         // K(t), V(t) have arrived for everyone, everyone is done with tile t - 1: its buffers take tile t + 1
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
@@ -262,6 +269,26 @@ void sdpa_prefill_f32_kernel(SdpaParams p)
 
     // ---- normalise and store --------------------------------------------------------------------------------------
     const float l_tot = xor32_sum(l_run);
+    if constexpr (SPLIT) {
+        // partial result of this split: unnormalised O, and (maximum, sum) in the natural-log units the combine kernel takes
+        // for f32 storage; a row that saw no key in this split has the maximum -inf
+        if (my_i < rows_b) {
+            const int64_t slot = (((int64_t)b * p.Hq + hq) * Sq + my_i) * p.num_splits + split;
+            float* arow = p.ws_acc + slot * D + g * 4;
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    float4v w = {o_acc[db][r4 * 4], o_acc[db][r4 * 4 + 1], o_acc[db][r4 * 4 + 2], o_acc[db][r4 * 4 + 3]};
+                    *(float4v*)(arow + db * 32 + r4 * 8) = w;
+                }
+            if (g == 0) {
+                p.ws_ml[slot * 2 + 0] = l_tot == 0.0f ? -INFINITY : m_run * 0.6931471805599453f;
+                p.ws_ml[slot * 2 + 1] = l_tot;
+            }
+        }
+        return;
+    }
     const float inv = (l_tot == 0.0f) ? __builtin_nanf("") : 1.0f / l_tot;   // no visible key: NaN, as the reference
     if (p.lse && g == 0 && my_i < rows_b)
         p.lse[((int64_t)b * p.Hq + hq) * Sq + my_i] = l_tot == 0.0f ? -INFINITY : (m_run + __builtin_log2f(l_tot)) * 0.6931471805599453f;
@@ -280,6 +307,8 @@ void sdpa_prefill_f32_kernel(SdpaParams p)
 #endif
 }
 
+hipError_t launch_sdpa_combine(const SdpaParams& p, int dtype, hipStream_t stream);
+
 template <int D, bool DENSE>
 static hipError_t launch_prefill_f32_t(const SdpaParams& p0, hipStream_t stream)
 {
@@ -290,6 +319,13 @@ static hipError_t launch_prefill_f32_t(const SdpaParams& p0, hipStream_t stream)
     if (total > 0x7fffffffLL) return hipErrorInvalidValue;
     p.interleave = work_interleave(p.causal != 0, 2 * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
     p.deal_groups = (total & 7) == 0 ? work_deal(p.interleave, p.G, nqb, total >> 3) : 0;
+    if constexpr (!DENSE) {
+        if (p.num_splits > 1) {          // split launch: partial results, then the split-KV kernels' combine pass
+            hipLaunchKernelGGL((sdpa_prefill_f32_kernel<D, false, true>), dim3((unsigned)total, (unsigned)p.num_splits), dim3(256), 0, stream, p);
+            hipError_t e = hipGetLastError();
+            return e != hipSuccess ? e : launch_sdpa_combine(p, 0, stream);
+        }
+    }
     hipLaunchKernelGGL((sdpa_prefill_f32_kernel<D, DENSE>), dim3((unsigned)total), dim3(256), 0, stream, p);
     return hipGetLastError();
 }

@@ -120,7 +120,8 @@ def test_dispatch_choices():
     assert _plan(chunk(4, 32, 8, 512, 32768))[1] == 1                                           # 512 workgroups: the rows fill the device
     assert _plan(chunk(1, 8, 8, 128, 2048))[1] == 1                                             # too few keys to split
     assert _plan(chunk(1, 32, 8, 512, 32768, lse=0x30000))[1] == 1                              # the row normalisers come from the unsplit kernel
-    assert _plan(chunk(1, 32, 8, 512, 32768, dtype=capi.F32))[1] == 1                           # (the f32 kernel does not split)
+    assert _plan(chunk(1, 32, 8, 512, 32768, dtype=capi.F32))[1] == 4                           # the f32 matrix-core kernel splits the same way
+    assert _plan(chunk(1, 32, 8, 512, 32768, add_mask=0x20000))[1] == 1                          # not with a dense mask
     # empty problems need nothing
     assert _plan(_desc(Sq=0))[0] == 0
 
