@@ -179,14 +179,13 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         // the two cross on launches of 268 MB of cache).  With one row per KV head the two kernels are within a few per
         // cent of each other everywhere; the matrix-core one is ahead on launches that run long enough for its longer
         // start-up not to show (3 - 4 % from 1 GB of cache on, behind by 4 - 9 % at 64 - 268 MB).
-        // Up to 64 rows the matrix-core kernel reads the cache once; beyond, once per 64 rows, which still beats the
-        // prefill kernel when that one would leave most of the device idle (it does not split the keys).
-        const int64_t prefill_wgs = d->B * d->Hq * ((d->Sq + 127) / 128);
+        // Up to 64 rows the matrix-core kernel reads the cache once; beyond (it would read it once per 64 rows) the
+        // prefill kernel takes over, which splits the keys itself when its launch is small (measured level or ahead from
+        // 128 rows per KV head on).
         const int64_t kv_bytes = 2 * d->B * d->Hkv * d->Skv * d->D * 2;       // (16-bit storage where it matters)
         const int64_t len128 = d->Skv * d->D / 128;      // cache length in keys of 128 elements (what the thresholds were measured in)
         if (split_mfma_ok && !d->lse && len128 >= 256 &&
-            ((R == 1 && len128 >= 1024 && kv_bytes >= (512LL << 20)) || (R >= 2 && R <= 3 && len128 >= 512) || (R >= 4 && R <= 64) ||
-             (R > 64 && len128 >= 2048 && prefill_wgs * 4 <= compute_units_of(d->device))))
+            ((R == 1 && len128 >= 1024 && kv_bytes >= (512LL << 20)) || (R >= 2 && R <= 3 && len128 >= 512) || (R >= 4 && R <= 64)))
             impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
         else if (split_ok && R <= 8 && d->Skv >= 256 && !d->lse) impl = INCIN_ROCM_IMPL_SPLITKV;
         // (the 64-row kernel is never picked: since the 32-row kernel stopped taking maxima in its pipelined loop it is

@@ -82,8 +82,8 @@ def test_dispatch_choices():
     assert _plan(_desc(Sq=1, Skv=8192, B=2, Hq=8, Hkv=2, dtype=capi.F32))[2] == capi.IMPL_SPLITKV   # f32: vector ALU
     assert _plan(_desc(Sq=1, Skv=8192, B=2, Hq=8, Hkv=2, D=64, Dv=64))[2] == capi.IMPL_SPLITKV_MFMA            # D = 64 too
     assert _plan(_desc(Sq=4, Skv=8192, B=2, Hq=32, Hkv=2))[2] == capi.IMPL_SPLITKV_MFMA             # 64 rows per KV head: one workgroup's worth
-    assert _plan(_desc(Sq=8, Skv=8192, B=2, Hq=32, Hkv=2))[2] == capi.IMPL_SPLITKV_MFMA             # 128, but the prefill kernel would run 64 workgroups
-    assert _plan(_desc(Sq=8, Skv=8192, B=8, Hq=32, Hkv=2))[2] == capi.IMPL_MFMA                     # 256 of them: a prefill shape
+    _, splits, impl = _plan(_desc(Sq=8, Skv=8192, B=2, Hq=32, Hkv=2))
+    assert impl == capi.IMPL_MFMA and splits == 8                                                   # 128 rows per KV head: the prefill kernel, keys split
     assert _plan(_desc(Sq=1, Skv=400, B=2, Hq=4, Hkv=2))[2] == capi.IMPL_SPLITKV                    # 2 rows, short cache: vector ALU
     assert _plan(_desc(Sq=1, Skv=512, B=2, Hq=16, Hkv=2))[2] == capi.IMPL_SPLITKV_MFMA              # 8 rows
     assert _plan(_desc(Sq=1, Skv=8192, B=2, Hq=4, Hkv=2))[2] == capi.IMPL_SPLITKV_MFMA              # 2 rows, long cache
