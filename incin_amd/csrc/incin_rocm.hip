@@ -277,14 +277,16 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         // when a launch has at most one per compute unit and a long key axis - a chunk of a long prompt, a single
         // sequence - the keys are split as for decode, as many ways as fill the device (1024 keys per split at least:
         // measured best on 32 heads x 128 rows x 8192 keys, 8 splits 32 us against 40 with 4 and 35 with 16), and the
-        // splits' partial results go through the split-KV kernels' combine pass.  num_splits > 0 in the descriptor forces
-        // a count.
+        // splits' partial results go through the split-KV kernels' combine pass.  Only where the key axis is the long one
+        // (four times the rows or more): the partial results are rows x splits x D floats, and on a square causal launch
+        // writing and combining them costs what the splits gain (one sequence, 8 heads, 4096 x 4096: 61 us whole, 64 in
+        // two splits, 74 in four).  num_splits > 0 in the descriptor forces a count.
         const int64_t cus = compute_units_of(d->device);
         const int64_t wgs = d->B * d->Hq * ((d->Sq + 127) / 128);
         int64_t splits = d->num_splits;
         if (splits == 0) {
             splits = 1;
-            if (wgs <= cus && d->Skv >= 4096) splits = std::min<int64_t>(2 * cus / wgs, d->Skv / 1024);
+            if (wgs <= cus && d->Skv >= 4096 && d->Skv >= 4 * d->Sq) splits = std::min<int64_t>(2 * cus / wgs, d->Skv / 1024);
         }
         if (splits > 1) {
             int64_t split_len = (d->Skv + splits - 1) / splits;
