@@ -34,7 +34,7 @@ PEAK_HBM_GBS = 8000.0       # HBM3E, vendor figure
 # FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0 after calibration against the 1 GiB copy kernel): profiles/*.txt
 PREFILL_TRAFFIC_BYTES = (273141 * 2.0 + 131084) * 1024     # 6.94e8: |Q|+|K|+|V| read 1.39 times, |O| written once
 DECODE_TRAFFIC_BYTES = (2097360 * 2.0 + 256) * 1024        # 4.2957e9: K and V read once, O written once
-PREFILL_LONG_TRAFFIC_BYTES = (537192 * 2.0 + 318930) * 1024    # 1.43e9: valid |O| written once, inputs read 2.2 times
+PREFILL_LONG_TRAFFIC_BYTES = (534477 * 2.0 + 318950) * 1024    # 1.43e9: valid |O| written once, inputs read 2.2 times
 # These three are constants taken from counter runs, not measured by this script: each roofline object says so and
 # names the summary the figures come from.
 TRAFFIC_SOURCE = {
