@@ -184,15 +184,15 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         // 128 rows per KV head on).
         const int64_t kv_bytes = 2 * d->B * d->Hkv * d->Skv * d->D * 2;       // (16-bit storage where it matters)
         const int64_t len128 = d->Skv * d->D / 128;      // cache length in keys of 128 elements (what the thresholds were measured in)
-        if (split_mfma_ok && !d->lse && len128 >= 256 &&
+        if (split_mfma_ok && len128 >= 256 &&
             ((R == 1 && len128 >= 1024 && kv_bytes >= (512LL << 20)) || (R >= 2 && R <= 3 && len128 >= 512) || (R >= 4 && R <= 64)))
             impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
-        else if (split_ok && R <= 8 && d->Skv >= 256 && !d->lse) impl = INCIN_ROCM_IMPL_SPLITKV;
+        else if (split_ok && R <= 8 && d->Skv >= 256) impl = INCIN_ROCM_IMPL_SPLITKV;
         // (the 64-row kernel is never picked: since the 32-row kernel stopped taking maxima in its pipelined loop it is
         // level with or ahead of it at every length measured, 4096 to 16384 keys, with and without a causal mask and
         // on ragged batches; INCIN_ROCM_IMPL_MFMA64 stays available by name)
         else if (mfma_ok) impl = INCIN_ROCM_IMPL_MFMA;
-        else if (split_ok && R <= 8 && !d->lse) impl = INCIN_ROCM_IMPL_SPLITKV;
+        else if (split_ok && R <= 8) impl = INCIN_ROCM_IMPL_SPLITKV;
         else impl = INCIN_ROCM_IMPL_GENERIC;
     }
     if (impl == INCIN_ROCM_IMPL_MFMA && !mfma_ok)
@@ -201,8 +201,6 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     if (impl == INCIN_ROCM_IMPL_MFMA64 && !mfma64_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
                     "scaled_dot_product_attention: the 64-row MFMA kernel needs f16/bf16, what the MFMA kernel needs, D == Dv == 128, no dense mask and key/value slices below 2 GiB");
-    if ((impl == INCIN_ROCM_IMPL_SPLITKV || impl == INCIN_ROCM_IMPL_SPLITKV_MFMA) && d->lse)
-        return fail(INCIN_ROCM_EUNSUPPORTED, "scaled_dot_product_attention: the split-KV kernels do not write the row normalisers (lse)");
     if (impl == INCIN_ROCM_IMPL_SPLITKV_MFMA && !split_mfma_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
                     "scaled_dot_product_attention: the matrix-core split-KV kernel needs f16/bf16, D == Dv in {64,128}, Sq <= 64, no dense mask, a finite scale and 16-byte aligned rows");
@@ -272,7 +270,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         plan->ws_bytes = splits > 1 ? (size_t)(d->B * d->Hq * d->Sq * splits) * (size_t)(d->Dv + 2) * sizeof(float) : 0;
     }
     if (impl == INCIN_ROCM_IMPL_MFMA64) plan->ws_bytes = MFMA64_WS_BYTES;      // the launch's work counters
-    if (impl == INCIN_ROCM_IMPL_MFMA && !d->add_mask && !d->lse && !d->q_lens) {
+    if (impl == INCIN_ROCM_IMPL_MFMA && !d->add_mask && !d->q_lens) {
         // The prefill kernels (16-bit and f32) run one workgroup per (batch, query head, 128 rows) and a compute unit holds two:
         // when a launch has at most one per compute unit and a long key axis - a chunk of a long prompt, a single
         // sequence - the keys are split as for decode, as many ways as fill the device (1024 keys per split at least:

@@ -216,6 +216,7 @@ __global__ __launch_bounds__(256) void sdpa_decode_split_kernel(SdpaParams p)
         if (p.num_splits == 1) {
             T* op = (T*)p.o + (int64_t)b * p.o_sb + (int64_t)hq * p.o_sh + (int64_t)i * p.o_ss;
             op[d] = from_f32<T>(L == 0.0f ? __builtin_nanf("") : A / L);
+            if (p.lse && d == 0) p.lse[((int64_t)b * p.Hq + hq) * Sq + i] = L == 0.0f ? -INFINITY : M / Softexp<T>::kPre + logf(L);
         } else {
             const int64_t slot = (((int64_t)b * p.Hq + hq) * Sq + i) * p.num_splits + split;
             p.ws_acc[slot * D + d] = A;
@@ -283,6 +284,8 @@ __global__ __launch_bounds__(256) void sdpa_combine_kernel(SdpaParams p)
         for (int e = 0; e < 4; ++e) w[e] = from_f32<T>(L == 0.0f ? __builtin_nanf("") : A[e] / L);
         T* op = (T*)p.o + (int64_t)b * p.o_sb + (int64_t)hq * p.o_sh + (int64_t)i * p.o_ss;
         *(vec4*)(op + 4 * tid) = w;
+        // the row's softmax normaliser, natural log (the maxima are in log2 units for 16-bit storage)
+        if (p.lse && tid == 0) p.lse[row] = L == 0.0f ? -INFINITY : M / Softexp<T>::kPre + logf(L);
     }
 }
 

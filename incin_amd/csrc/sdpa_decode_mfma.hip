@@ -360,6 +360,8 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
                 for (int e = 0; e < 4; ++e) w[e] = (T)(o[r4 * 4 + e] * inv);
                 *(vec4*)(orow + r4 * 8) = w;
             }
+            if (p.lse && wave == 0 && g == 0)       // the row's softmax normaliser, natural log (M and the sum are in log2 units)
+                p.lse[((int64_t)b * p.Hq + hq[rb]) * Sq + qi[rb]] = l_tot == 0.0f ? -INFINITY : (M[rb] + __builtin_log2f(l_tot)) * 0.6931471805599453f;
         } else {
             const int64_t slot = (((int64_t)b * p.Hq + hq[rb]) * Sq + qi[rb]) * p.num_splits + split;
             float* arow = p.ws_acc + slot * D + 32 * wave + 4 * g;

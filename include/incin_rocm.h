@@ -183,8 +183,8 @@ typedef struct {
     const int32_t* q_lens;         /* nullable device pointer, B entries: rows at and beyond are padding */
     float* lse;                    /* nullable device pointer, contiguous f32 [B, Hq, Sq]: receives log sum_j exp(x_ij) of
                                       every row (natural log of the softmax normaliser; -inf for a row with no visible
-                                      key) - what incin_rocm_sdpa_bwd needs from the forward.  Written by the generic and
-                                      the MFMA prefill kernels; AUTO keeps to those when it is set */
+                                      key) - what incin_rocm_sdpa_bwd needs from the forward.  Every kernel writes it
+                                      (launches that split the key axis: their combine pass) */
 } incin_rocm_sdpa_desc_t;
 
 /* Validates the descriptor and reports the scratch bytes and the split count the

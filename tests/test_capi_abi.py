@@ -120,7 +120,7 @@ def test_dispatch_choices():
     assert _plan(chunk(4, 32, 8, 512, 32768))[1] == 1                                           # 512 workgroups: the rows fill the device
     assert _plan(chunk(1, 8, 8, 128, 2048))[1] == 1                                             # too few keys to split
     assert _plan(chunk(1, 8, 8, 4096, 4096, causal=1))[1] == 1                                  # square: the partial results would cost what the splits gain
-    assert _plan(chunk(1, 32, 8, 512, 32768, lse=0x30000))[1] == 1                              # the row normalisers come from the unsplit kernel
+    assert _plan(chunk(1, 32, 8, 512, 32768, lse=0x30000))[1] == 4                              # (the combine pass writes the row normalisers)
     assert _plan(chunk(1, 32, 8, 512, 32768, dtype=capi.F32))[1] == 4                           # the f32 matrix-core kernel splits the same way
     assert _plan(chunk(1, 32, 8, 512, 32768, add_mask=0x20000))[1] == 1                          # not with a dense mask
     # empty problems need nothing

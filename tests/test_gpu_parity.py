@@ -346,7 +346,6 @@ def test_row_normalisers(gpu, impl):
     lens = np.array([420, 77], np.int32)
     for causal in (False, True):
         got, lse, info = host.sdpa(q, k, v, capi.BF16, causal=causal, kv_lens=lens, impl=impl, return_lse=True, return_info=True)
-        assert info["impl"] != capi.IMPL_SPLITKV
         want = BW.logsumexp(q.reshape(B, Hkv, 2, Sq, D), k[:, :, None], causal=causal, kv_lens=lens.reshape(B, 1, 1)).reshape(B, Hq, Sq)
         fin = np.isfinite(want)
         assert np.array_equal(np.isfinite(lse), fin) and np.all(lse[~fin] == -np.inf)
@@ -355,9 +354,37 @@ def test_row_normalisers(gpu, impl):
         assert err <= 2e-2                # the scores come from bf16 products of a Q pre-multiplied by the scale in bf16
         plain = host.sdpa(q, k, v, capi.BF16, causal=causal, kv_lens=lens, impl=info["impl"])
         assert np.array_equal(np.nan_to_num(got, nan=7.0), np.nan_to_num(plain, nan=7.0))
-    # a decode-shaped request with lse keeps away from the split-KV kernel, which does not write it
-    _, _, info = host.sdpa(q[:, :, :1], k, v, capi.BF16, return_lse=True, return_info=True)
-    assert info["impl"] != capi.IMPL_SPLITKV
+
+
+@pytest.mark.parametrize("case", [
+    # impl, dtype, B, Hq, Hkv, Sq, Skv, D, splits
+    (capi.IMPL_SPLITKV, capi.BF16, 2, 4, 2, 1, 1500, 128, 0), (capi.IMPL_SPLITKV, capi.BF16, 2, 4, 2, 2, 1500, 128, 1),
+    (capi.IMPL_SPLITKV, capi.F32, 1, 4, 4, 1, 900, 64, 3),
+    (capi.IMPL_SPLITKV_MFMA, capi.BF16, 2, 16, 2, 1, 1500, 128, 0), (capi.IMPL_SPLITKV_MFMA, capi.F16, 2, 16, 2, 3, 1500, 128, 1),
+    (capi.IMPL_SPLITKV_MFMA, capi.BF16, 1, 8, 1, 9, 700, 64, 4),
+    (capi.IMPL_MFMA, capi.BF16, 1, 4, 2, 100, 4500, 128, 0), (capi.IMPL_MFMA, capi.F32, 1, 2, 2, 70, 4200, 64, 3),
+])
+def test_row_normalisers_from_split_launches(gpu, case):
+    """The same by-product from the launches that split the key axis - the split-KV kernels (their combine pass, or the
+    kernel itself with one split) and the prefill kernels over key splits - with a sequence that ends inside a split and
+    one without keys."""
+    from oracle import sdpa_backward as BW
+    impl, dtype, B, Hq, Hkv, Sq, Skv, D, splits = case
+    G = Hq // Hkv
+    q, k, v = inputs(61 + Skv, B, Hq, Hkv, Sq, Skv, D, D, dtype)
+    lens = np.array([Skv - 13, 0][:B], np.int32)
+    got, lse, info = host.sdpa(q, k, v, dtype, causal=True, kv_lens=lens, impl=impl, num_splits=splits, return_lse=True, return_info=True)
+    assert info["impl"] == impl
+    say("row normalisers: impl %d dtype %d, %d splits" % (impl, dtype, info["splits"]))
+    want = BW.logsumexp(q.reshape(B, Hkv, G, Sq, D), k[:, :, None], causal=True, kv_lens=lens.reshape(B, 1, 1)).reshape(B, Hq, Sq)
+    fin = np.isfinite(want)
+    assert np.array_equal(np.isfinite(lse), fin) and np.all(lse[~fin] == -np.inf)
+    err = float(np.abs(lse[fin] - want[fin]).max())
+    say("row normalisers from split launches: max-abs err %.3e" % err)
+    assert err <= (2e-5 if dtype == capi.F32 else 2e-2)
+    plain = host.sdpa(q, k, v, dtype, causal=True, kv_lens=lens, impl=impl, num_splits=splits)
+    assert np.array_equal(np.nan_to_num(got, nan=7.0), np.nan_to_num(plain, nan=7.0))
+    check(got, oracle_full(q, k, v, G=G, causal=True, kv_lens=lens), TOL[dtype], "output beside the row normalisers")
 
 
 @pytest.mark.parametrize("dtype", [capi.BF16, capi.F16, capi.F32])
