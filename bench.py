@@ -547,7 +547,7 @@ def main():
             w.desc.q_lens = w.tl.ptr
         wall, ev_mean, ev_med, ev_min = w.time(steps, min(args.warmup, 5))
         flops = 4.0 * D * Hq * float(sum(int(n) * (int(n) + 1) // 2 for n in lens))      # rows i < lens[b] only
-        kernel = {capi.IMPL_MFMA64: "sdpa_prefill_mfma64_kernel<bf16>", capi.IMPL_MFMA: "sdpa_prefill_mfma_kernel<bf16,128>"}.get(w.impl, str(w.impl))
+        kernel = {capi.IMPL_MFMA: "sdpa_prefill_mfma_kernel<bf16,128>"}.get(w.impl, str(w.impl))
         result["prefill_long"] = {
             "workload": "BASELINE config 5: bf16 GQA causal prefill B=4 Hq=32 Hkv=8 S=16384 (padded) D=128, key padding with "
                         "lengths %s given as kv_lens and q_lens (padding rows not computed); FLOPs count rows and keys inside "

@@ -21,7 +21,6 @@
 namespace incin_rocm {
 hipError_t launch_sdpa_generic(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_sdpa_prefill_mfma(const SdpaParams& p, int dtype, hipStream_t stream);
-hipError_t launch_sdpa_prefill_mfma64(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_matrix_rate(const void* src, void* sink, int mix, int iterations, double* flops, hipStream_t stream);
 hipError_t launch_sdpa_prefill_f32(const SdpaParams& p, hipStream_t stream);
 hipError_t launch_mask_classify(const SdpaParams& p, int dtype, hipStream_t stream);
@@ -83,7 +82,6 @@ int use_device(int32_t dev)
 
 size_t dtype_size(int dtype) { return dtype == INCIN_ROCM_F32 ? 4 : 2; }
 
-constexpr size_t MFMA64_WS_BYTES = 256;     // work counters of one launch of the 64-row prefill kernel
 
 // Compute units of device `dev` (256 when it cannot be asked, e.g. a workspace query on a machine without a device:
 // only launch geometry depends on it).
@@ -162,9 +160,6 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     // f32: the IEEE-f32 matrix-core kernel, any finite scale; f16 / bf16: the 16-bit kernels fold the scale into Q in
     // a way that needs it positive.  Both take a dense additive mask (any strides); the 64-row kernel does not.
     const bool mfma_ok = layout_ok && tile_off_ok && std::isfinite(d->scale) && (d->dtype == INCIN_ROCM_F32 || d->scale > 0.0f);
-    // the 64-row kernel does its byte arithmetic on a head's K and V in 32 bits, up to 16 tiles of 32 rows past the end
-    const bool mfma64_ok = mfma_ok && !d->add_mask && d->dtype != INCIN_ROCM_F32 && d->D == 128 && (d->Skv + 512) * d->k_stride[2] * 2 < (1LL << 31) &&
-                           (d->Skv + 512) * d->v_stride[2] * 2 < (1LL << 31);
     const bool split_ok = fast_ok && d->Sq <= 64;
     // the matrix-core split-KV kernel: 16-bit storage, blocks addressed like the prefill kernels' tiles
     const bool split_mfma_ok = split_ok && tile_off_ok && d->dtype != INCIN_ROCM_F32 && std::isfinite(d->scale);
@@ -188,9 +183,6 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
             ((R == 1 && len128 >= 1024 && kv_bytes >= (512LL << 20)) || (R >= 2 && R <= 3 && len128 >= 512) || (R >= 4 && R <= 64)))
             impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
         else if (split_ok && R <= 8 && d->Skv >= 256) impl = INCIN_ROCM_IMPL_SPLITKV;
-        // (the 64-row kernel is never picked: since the 32-row kernel stopped taking maxima in its pipelined loop it is
-        // level with or ahead of it at every length measured, 4096 to 16384 keys, with and without a causal mask and
-        // on ragged batches; INCIN_ROCM_IMPL_MFMA64 stays available by name)
         else if (mfma_ok) impl = INCIN_ROCM_IMPL_MFMA;
         else if (split_ok && R <= 8) impl = INCIN_ROCM_IMPL_SPLITKV;
         else impl = INCIN_ROCM_IMPL_GENERIC;
@@ -198,9 +190,9 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     if (impl == INCIN_ROCM_IMPL_MFMA && !mfma_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
                     "scaled_dot_product_attention: the MFMA kernels need D == Dv in {64,128} and 16-byte aligned rows; for f16/bf16 also scale > 0");
-    if (impl == INCIN_ROCM_IMPL_MFMA64 && !mfma64_ok)
+    if (impl == INCIN_ROCM_IMPL_MFMA64)
         return fail(INCIN_ROCM_EUNSUPPORTED,
-                    "scaled_dot_product_attention: the 64-row MFMA kernel needs f16/bf16, what the MFMA kernel needs, D == Dv == 128, no dense mask and key/value slices below 2 GiB");
+                    "scaled_dot_product_attention: the 64-row MFMA prefill kernel has been retired (INCIN_ROCM_IMPL_MFMA covers its shapes)");
     if (impl == INCIN_ROCM_IMPL_SPLITKV_MFMA && !split_mfma_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
                     "scaled_dot_product_attention: the matrix-core split-KV kernel needs f16/bf16, D == Dv in {64,128}, Sq <= 64, no dense mask, a finite scale and 16-byte aligned rows");
@@ -269,7 +261,6 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         plan->split_len = (int)split_len;
         plan->ws_bytes = splits > 1 ? (size_t)(d->B * d->Hq * d->Sq * splits) * (size_t)(d->Dv + 2) * sizeof(float) : 0;
     }
-    if (impl == INCIN_ROCM_IMPL_MFMA64) plan->ws_bytes = MFMA64_WS_BYTES;      // the launch's work counters
     if (impl == INCIN_ROCM_IMPL_MFMA && !d->add_mask && !d->q_lens) {
         // The prefill kernels (16-bit and f32) run one workgroup per (batch, query head, 128 rows) and a compute unit holds two:
         // when a launch has at most one per compute unit and a long key axis - a chunk of a long prompt, a single
@@ -331,9 +322,8 @@ void fill_params(const incin_rocm_sdpa_desc_t* d, const Plan& plan, SdpaParams* 
     p->deal_groups = 0;
     p->num_splits = plan.splits;
     p->split_len = plan.split_len;
-    if (plan.impl == INCIN_ROCM_IMPL_MFMA64) p->sched = (int32_t*)d->workspace;
-    else if (plan.impl == INCIN_ROCM_IMPL_MFMA) p->mask_flags = d->add_mask ? (const uint8_t*)d->workspace : nullptr;
-    if (plan.impl != INCIN_ROCM_IMPL_MFMA64 && !(plan.impl == INCIN_ROCM_IMPL_MFMA && d->add_mask)) p->ws_acc = (float*)d->workspace;
+    if (plan.impl == INCIN_ROCM_IMPL_MFMA) p->mask_flags = d->add_mask ? (const uint8_t*)d->workspace : nullptr;
+    if (!(plan.impl == INCIN_ROCM_IMPL_MFMA && d->add_mask)) p->ws_acc = (float*)d->workspace;
     if (plan.splits > 1) {
         const size_t rows = (size_t)(d->B * d->Hq * d->Sq * plan.splits);
         p->ws_ml = (float*)d->workspace + rows * (size_t)d->Dv;
@@ -610,7 +600,7 @@ static int launch_fwd(const incin_rocm_sdpa_desc_t* desc, const Plan& plan, void
         if (!desc->workspace || desc->workspace_bytes < plan.ws_bytes)
             return fail(INCIN_ROCM_EWORKSPACE,
                         "scaled_dot_product_attention: %s needs %zu workspace bytes, %zu given",
-                        plan.impl == INCIN_ROCM_IMPL_MFMA64 ? "the 64-row MFMA kernel" : plan.impl != INCIN_ROCM_IMPL_MFMA ? "split-KV" : desc->add_mask ? "a dense mask on the MFMA kernels" : "the MFMA prefill kernel with the keys split",
+                        plan.impl != INCIN_ROCM_IMPL_MFMA ? "split-KV" : desc->add_mask ? "a dense mask on the MFMA kernels" : "the MFMA prefill kernel with the keys split",
                         plan.ws_bytes,
                         desc->workspace ? desc->workspace_bytes : (size_t)0);
         if (!aligned16(desc->workspace)) return fail(INCIN_ROCM_EWORKSPACE, "scaled_dot_product_attention: workspace must be 16-byte aligned");
@@ -628,7 +618,6 @@ static int launch_fwd(const incin_rocm_sdpa_desc_t* desc, const Plan& plan, void
             }
             e = desc->dtype == INCIN_ROCM_F32 ? incin_rocm::launch_sdpa_prefill_f32(p, s) : incin_rocm::launch_sdpa_prefill_mfma(p, desc->dtype, s);
             break;
-        case INCIN_ROCM_IMPL_MFMA64: e = incin_rocm::launch_sdpa_prefill_mfma64(p, desc->dtype, s); break;
         case INCIN_ROCM_IMPL_SPLITKV: e = incin_rocm::launch_sdpa_decode(p, desc->dtype, s); break;
         case INCIN_ROCM_IMPL_SPLITKV_MFMA: e = incin_rocm::launch_sdpa_decode_mfma(p, desc->dtype, s); break;
         default: e = incin_rocm::launch_sdpa_generic(p, desc->dtype, s); break;

@@ -1,4 +1,4 @@
-// Shared pieces of the two MFMA attention kernels: operand types, the matrix
+// Shared pieces of the MFMA attention kernels: operand types, the matrix
 // instruction wrappers, the LDS tile layout (chunk-slot swizzle) and the
 // lane <-> lane^32 exchanges.
 #pragma once

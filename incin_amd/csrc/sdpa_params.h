@@ -36,9 +36,6 @@ struct SdpaParams {
     // [mask batch entries][mask heads][ceil(Sq / 32)][ceil(Skv / 32)], an extent of 1 where the mask is broadcast
     const uint8_t* mask_flags;
     int32_t mask_vec;          // 16-bit MFMA kernel: the mask's rows allow 8-byte loads of 4 consecutive keys
-    // 64-row MFMA prefill kernel only
-    int32_t* sched;            // 16 work counters of this launch's persistent workgroups (in the caller's workspace; the
-                               // launcher clears them with a one-workgroup kernel ahead of the attention kernel)
 };
 
 typedef __bf16 bf16_t;

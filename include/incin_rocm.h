@@ -48,7 +48,7 @@ enum {
     INCIN_ROCM_IMPL_MFMA = 2,      /* MFMA prefill kernels, D == Dv in {64,128}: bf16/f16 (no dense mask, scale > 0), and
                                       IEEE-f32 matrix instructions for f32 (dense mask allowed)                    */
     INCIN_ROCM_IMPL_SPLITKV = 3,   /* split-KV decode kernel + combine: D == Dv in {64,128}, few query rows */
-    INCIN_ROCM_IMPL_MFMA64 = 4,    /* bf16/f16 MFMA prefill kernel, 64 query rows per wavefront: D == Dv == 128 */
+    INCIN_ROCM_IMPL_MFMA64 = 4,    /* retired (a prefill kernel with 64 query rows per wavefront): refused with INCIN_ROCM_EUNSUPPORTED */
     INCIN_ROCM_IMPL_SPLITKV_MFMA = 5 /* bf16/f16 split-KV kernel on the matrix cores + combine: D == Dv in {64,128}, Sq <= 64; the rows that
                                       share a KV head (query heads of the group x query positions) go through it 32 at a time */
 };
@@ -197,15 +197,14 @@ int incin_rocm_sdpa_workspace(const incin_rocm_sdpa_desc_t* desc, size_t* bytes,
  * stream-ordered use of the buffers named in the descriptor, which the caller
  * keeps alive until the stream has been synchronised.
  *
- * Workspace.  Three launches need scratch memory, of the size incin_rocm_sdpa_workspace reports: launches that split
- * the key axis - the split-KV kernels, and the 16-bit MFMA prefill kernel when few row blocks meet many keys - (partial
- * results of the splits), the 64-row MFMA prefill kernel (256 bytes: the work counters its
- * persistent workgroups draw from, cleared by the launch itself) and the MFMA prefill kernels with a dense mask
+ * Workspace.  Two kinds of launch need scratch memory, of the size incin_rocm_sdpa_workspace reports: launches that split
+ * the key axis - the split-KV kernels, and the MFMA prefill kernels when few row blocks meet many keys - (partial
+ * results of the splits) and the MFMA prefill kernels with a dense mask
  * (one byte per block of 32 query rows x 32 keys of the mask: which blocks it hides, which it leaves alone;
  * written by a small kernel of the same launch).  The contents need not survive the launch and
  * need no initialisation, but two launches that may run at the same time - other streams, other host threads, a
- * recorded graph replayed beside eager launches - must not be given the same workspace: they would draw from
- * each other's counters or overwrite each other's partial results.  A recorded launch keeps using the workspace
+ * recorded graph replayed beside eager launches - must not be given the same workspace: they would overwrite
+ * each other's partial results or block flags.  A recorded launch keeps using the workspace
  * it was recorded with on every replay. */
 int incin_rocm_sdpa_fwd(const incin_rocm_sdpa_desc_t* desc, void* stream);
 

@@ -88,7 +88,7 @@ def test_dispatch_choices():
     assert _plan(_desc(Sq=1, Skv=512, B=2, Hq=16, Hkv=2))[2] == capi.IMPL_SPLITKV_MFMA              # 8 rows
     assert _plan(_desc(Sq=1, Skv=8192, B=2, Hq=4, Hkv=2))[2] == capi.IMPL_SPLITKV_MFMA              # 2 rows, long cache
     assert _plan(_desc(Sq=1, Skv=64))[2] in (capi.IMPL_MFMA, capi.IMPL_SPLITKV)
-    # long sequences: the 32-row kernel as well (the 64-row kernel is level with it or behind at every length; by name only)
+    # long sequences: the same kernel
     def long(**kw):
         S = kw.pop("S", 16384)
         d = _desc(B=4, Hq=32, Hkv=8, Sq=S, Skv=S, **kw)
@@ -99,8 +99,6 @@ def test_dispatch_choices():
     assert _plan(long())[2] == capi.IMPL_MFMA
     assert _plan(long(causal=1))[2] == capi.IMPL_MFMA
     assert _plan(long(S=4096))[2] == capi.IMPL_MFMA
-    nbytes, _, impl = _plan(long(impl=capi.IMPL_MFMA64))
-    assert impl == capi.IMPL_MFMA64 and nbytes == 256           # pinned: its work counters come from the workspace
     assert _plan(long(S=4096, causal=1))[2] == capi.IMPL_MFMA
     assert _plan(long(S=2048))[2] == capi.IMPL_MFMA
     assert _plan(long(D=64, Dv=64))[2] == capi.IMPL_MFMA
@@ -134,8 +132,7 @@ def test_dispatch_choices():
     (dict(q=None), capi.EINVAL),
     (dict(impl=9), capi.EINVAL),
     (dict(num_splits=-2), capi.EINVAL),
-    (dict(impl=capi.IMPL_MFMA64, dtype=capi.F32), capi.EUNSUPPORTED),
-    (dict(impl=capi.IMPL_MFMA64, add_mask=0x20000), capi.EUNSUPPORTED),
+    (dict(impl=capi.IMPL_MFMA64), capi.EUNSUPPORTED),                 # retired: the value is refused
     (dict(impl=capi.IMPL_MFMA, D=80, Dv=80), capi.EUNSUPPORTED),
     (dict(impl=capi.IMPL_SPLITKV, Sq=4096), capi.EUNSUPPORTED),
     (dict(impl=capi.IMPL_SPLITKV_MFMA, Sq=4096), capi.EUNSUPPORTED),

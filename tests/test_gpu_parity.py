@@ -179,7 +179,7 @@ def test_reference_golden_vectors_on_gpu(gpu):
 
 # ---- MFMA prefill kernel --------------------------------------------------------------------
 
-MFMA_IMPLS = [capi.IMPL_MFMA, capi.IMPL_MFMA64]
+MFMA_IMPLS = [capi.IMPL_MFMA]
 
 
 @pytest.mark.parametrize("impl", MFMA_IMPLS)
@@ -198,8 +198,6 @@ MFMA_IMPLS = [capi.IMPL_MFMA, capi.IMPL_MFMA64]
 ])
 def test_mfma_prefill(gpu, dtype, shape, impl):
     B, Hq, Hkv, Sq, Skv, D = shape
-    if impl == capi.IMPL_MFMA64 and D != 128:
-        pytest.skip("the 64-row kernel covers head dimension 128 only")
     q, k, v = inputs(200 + sum(shape), B, Hq, Hkv, Sq, Skv, D, D, dtype)
     for causal in (False, True):
         got, info = host.sdpa(q, k, v, dtype, causal=causal, impl=impl, return_info=True)
@@ -579,12 +577,9 @@ def test_decode_lengths_and_prefill_consistency(gpu):
 
 @pytest.mark.parametrize("impl, dtype, sq", [
     (capi.IMPL_GENERIC, capi.F32, 70), (capi.IMPL_GENERIC, capi.BF16, 70), (capi.IMPL_MFMA, capi.BF16, 200),
-    pytest.param(capi.IMPL_MFMA64, capi.BF16, 200, marks=pytest.mark.skip(
-        reason="this case did not finish on the device once in three runs (the launch of the 64-row kernel never completed; "
-               "cause not found by reading the kernel): kept off the device until a cause can be shown")),
     (capi.IMPL_MFMA, capi.F16, 200), (capi.IMPL_SPLITKV, capi.BF16, 1), (capi.IMPL_SPLITKV, capi.F32, 2),
     (capi.IMPL_SPLITKV_MFMA, capi.BF16, 3), (capi.IMPL_SPLITKV_MFMA, capi.F16, 1)],
-    ids=["generic_f32", "generic_bf16", "mfma_bf16", "mfma64_bf16", "mfma_f16", "splitkv_bf16", "splitkv_f32", "splitkv_mfma_bf16", "splitkv_mfma_f16"])
+    ids=["generic_f32", "generic_bf16", "mfma_bf16", "mfma_f16", "splitkv_bf16", "splitkv_f32", "splitkv_mfma_bf16", "splitkv_mfma_f16"])
 def test_rows_beyond_the_key_count_are_never_read(gpu, impl, dtype, sq):
     """A preallocated cache holds whatever the allocator left behind its valid rows.  With NaN and infinity bit patterns
     in every key and value row at and beyond kv_lens[b], each kernel gives the bytes it gives over a zeroed tail, and
@@ -610,9 +605,9 @@ def test_rows_beyond_the_key_count_are_never_read(gpu, impl, dtype, sq):
     check(dirty, oracle_full(q, k, v, G=Hq // Hkv, kv_lens=lens), TOL[dtype], "junk tail")
 
 
-@pytest.mark.parametrize("impl, sq", [(capi.IMPL_MFMA, 96), (capi.IMPL_MFMA64, 96), (capi.IMPL_SPLITKV, 2), (capi.IMPL_GENERIC, 40),
+@pytest.mark.parametrize("impl, sq", [(capi.IMPL_MFMA, 96), (capi.IMPL_SPLITKV, 2), (capi.IMPL_GENERIC, 40),
                                       (capi.IMPL_SPLITKV_MFMA, 6)],
-                         ids=["mfma", "mfma64", "splitkv", "generic", "splitkv_mfma"])
+                         ids=["mfma", "splitkv", "generic", "splitkv_mfma"])
 @pytest.mark.parametrize("dtype", [capi.BF16, capi.F16])
 def test_large_logits(gpu, dtype, impl, sq):
     """Logits of magnitude 50 with many keys within a few units of each row's maximum, and query rows whose elements are
@@ -671,7 +666,7 @@ def test_256_row_workgroups(gpu, dtype, shape, monkeypatch):
 
 
 @pytest.mark.parametrize("causal", [False, True, "tensor"], ids=["full", "causal", "causal_as_tensor"])
-@pytest.mark.parametrize("impl", [capi.IMPL_MFMA, capi.IMPL_MFMA64], ids=["mfma", "mfma64"])
+@pytest.mark.parametrize("impl", [capi.IMPL_MFMA], ids=["mfma"])
 @pytest.mark.parametrize("dtype", [capi.BF16, capi.F16])
 @pytest.mark.parametrize("rows", ["128", "256"])
 def test_scores_far_above_the_first_tiles(gpu, dtype, impl, causal, rows, monkeypatch):
@@ -698,8 +693,6 @@ def test_scores_far_above_the_first_tiles(gpu, dtype, impl, causal, rows, monkey
     if causal == "tensor":
         # the causal mask the way the reference's operator takes it: the dense-mask instance of the kernel, whose
         # mask-free stretch of tiles runs the same bit check
-        if impl == capi.IMPL_MFMA64:
-            pytest.skip("the 64-row kernel takes no dense mask")
         mask = O.causal_additive_mask(S, S).reshape(1, 1, S, S)
         got, info = host.sdpa(q, k, v, dtype, mask=mask, impl=impl, return_info=True)
         causal = True

@@ -68,7 +68,7 @@ def run_case(i, c, r):
     sc = c["scale"] if c["scale"] is not None else 1.0 / np.sqrt(D)
     c["max_logit"] = float(np.abs(np.einsum("bhgid,bhjd->bhgij", q.reshape(B, Hkv, G, Sq, D).astype(np.float64), k.astype(np.float64))).max() * sc) if q.size and k.size else 0.0
     impls = [capi.IMPL_AUTO]
-    for impl in (capi.IMPL_GENERIC, capi.IMPL_MFMA, capi.IMPL_MFMA64, capi.IMPL_SPLITKV, capi.IMPL_SPLITKV_MFMA):
+    for impl in (capi.IMPL_GENERIC, capi.IMPL_MFMA, capi.IMPL_SPLITKV, capi.IMPL_SPLITKV_MFMA):
         try:
             got, info = host.sdpa(q, k, v, dt, impl=impl, return_info=True, **kw)
         except capi.RocmError as e:
@@ -119,5 +119,5 @@ def test_random_cases(gpu):
     say("kernels exercised: %s" % used)
     for dt, (err, what) in sorted(WORST.items()):
         say("worst absolute error, dtype %d: %.3e in %s" % (dt, err, what))
-    for impl in (capi.IMPL_GENERIC, capi.IMPL_MFMA, capi.IMPL_MFMA64, capi.IMPL_SPLITKV, capi.IMPL_SPLITKV_MFMA):
+    for impl in (capi.IMPL_GENERIC, capi.IMPL_MFMA, capi.IMPL_SPLITKV, capi.IMPL_SPLITKV_MFMA):
         assert used.get(impl, 0) >= 5, "kernel %d was hardly reached: %s" % (impl, used)

@@ -46,7 +46,7 @@ class Case:
 
 CASES = [
     ("prefill 32-row kernel", dict(B=2, Hq=8, Hkv=8, Sq=512, Skv=512, D=128, causal=True, impl=capi.IMPL_MFMA)),
-    ("prefill 64-row kernel", dict(B=2, Hq=8, Hkv=2, Sq=1024, Skv=1024, D=128, causal=True, impl=capi.IMPL_MFMA64)),
+    ("prefill over key splits", dict(B=1, Hq=4, Hkv=2, Sq=128, Skv=4200, D=128, causal=True, impl=capi.IMPL_MFMA)),
     ("decode split-KV", dict(B=4, Hq=8, Hkv=8, Sq=1, Skv=4096, D=128, causal=False, impl=capi.IMPL_SPLITKV)),
     ("grouped-query decode, matrix-core split-KV", dict(B=2, Hq=16, Hkv=2, Sq=1, Skv=4096, D=128, causal=False, impl=capi.IMPL_SPLITKV_MFMA)),
     ("generic", dict(B=1, Hq=2, Hkv=2, Sq=100, Skv=130, D=80, causal=True, impl=capi.IMPL_GENERIC)),
@@ -155,14 +155,14 @@ def test_training_step_in_a_graph(gpu, dtype, impl):
     stream.destroy()
 
 
-def test_overlapping_launches_of_the_64_row_kernel(gpu):
-    """Two host threads launch the same problem through the 64-row prefill kernel 50 times each on streams of their own
-    while a recorded graph of the same launch replays on a third stream.  The kernel's persistent workgroups draw their
-    work from counters in the launch's workspace; each party has a workspace and an output of its own, so whatever
-    overlaps, every output equals the plain launch bit for bit."""
-    kw = dict(B=2, Hq=8, Hkv=2, Sq=1024, Skv=1024, D=128, causal=True, impl=capi.IMPL_MFMA64)
+def test_overlapping_launches_with_workspaces_of_their_own(gpu):
+    """Two host threads launch the same problem - grouped-query decode through the matrix-core split-KV kernel, whose
+    splits leave their partial results in the launch's workspace for the combine pass - 50 times each on streams of their
+    own while a recorded graph of the same launch replays on a third stream.  Each party has a workspace and an output
+    of its own, so whatever overlaps, every output equals the plain launch bit for bit."""
+    kw = dict(B=2, Hq=16, Hkv=2, Sq=1, Skv=6000, D=128, causal=False, impl=capi.IMPL_SPLITKV_MFMA)
     parties = [Case(400, **kw) for _ in range(3)]          # same seed: same problem, separate buffers
-    assert all(c.impl == capi.IMPL_MFMA64 and c.ws is not None for c in parties)
+    assert all(c.impl == capi.IMPL_SPLITKV_MFMA and c.ws is not None for c in parties)
     expect = parties[0].plain()
     for c in parties:
         c.clear()
@@ -189,7 +189,7 @@ def test_overlapping_launches_of_the_64_row_kernel(gpu):
         except Exception as e:      # noqa: BLE001
             errors.append(e)
 
-    say("2 threads x 50 eager launches + 50 graph replays of the 64-row kernel, three streams")
+    say("2 threads x 50 eager launches + 50 graph replays of a split-KV launch, three streams")
     threads = [threading.Thread(target=eager, args=(parties[0],)), threading.Thread(target=eager, args=(parties[1],)),
                threading.Thread(target=replay)]
     for t in threads:

@@ -1,7 +1,7 @@
 """incin_rocm_sdpa_fwd_static, the launch that takes its scratch memory from the library's static device buffer instead
 of a workspace of the caller's: its output must equal incin_rocm_sdpa_fwd's bit for bit, on two calls in a row of which
 the second is the smaller one (the buffer keeps the first call's contents), for the three launches that use scratch
-memory: split-KV decode (partial results), the 64-row prefill kernel (work counters) and a matrix-core prefill with a
+memory: split-KV decode (partial results), a prefill launch over key splits (the same) and a matrix-core prefill with a
 dense mask (block flags of the mask)."""
 import sys
 
@@ -68,9 +68,6 @@ def test_static_scratch_matches_workspace_launch(gpu):
         ("prefill with the keys split",
          dict(B=1, Hq=4, Hkv=2, Sq=100, Skv=4500, D=128, causal=True, impl=capi.IMPL_MFMA),
          dict(B=1, Hq=2, Hkv=2, Sq=40, Skv=4100, D=128, causal=False, impl=capi.IMPL_MFMA, num_splits=3)),
-        ("64-row prefill",
-         dict(B=2, Hq=8, Hkv=2, Sq=1024, Skv=1024, D=128, causal=True, impl=capi.IMPL_MFMA64),
-         dict(B=1, Hq=3, Hkv=3, Sq=300, Skv=300, D=128, causal=True, impl=capi.IMPL_MFMA64)),
         ("prefill with a dense mask (block flags)",
          dict(B=2, Hq=4, Hkv=2, Sq=700, Skv=700, D=128, causal=False, impl=capi.IMPL_MFMA, causal_mask_tensor=True),
          dict(B=1, Hq=2, Hkv=2, Sq=100, Skv=333, D=128, causal=False, impl=capi.IMPL_MFMA, causal_mask_tensor=True)),
