@@ -609,6 +609,7 @@ def main():
     if args.only in (None, "backward"):
         result["backward"] = backward_leg(max(5, min(args.steps, 30)), min(args.warmup, 5))
         # f32, the dtype the reference trains in: BASELINE config 2's shape (launches of ~100 us) and config 3's
+        result["backward_d64"] = backward_leg(max(5, min(args.steps, 30)), min(args.warmup, 5), capi.BF16, 8, 32, 4096, 64, "config 3 with 32 heads of 64 (the same FLOPs)")
         result["backward_f32_c2"] = backward_leg(max(args.steps, 100), min(args.warmup, 5), capi.F32, 4, 8, 1024, 64, "BASELINE config 2's shape")
         result["backward_f32_large"] = backward_leg(max(5, min(args.steps, 10)), min(args.warmup, 3), capi.F32, what="BASELINE config 3's shape in f32")
 

@@ -1,4 +1,4 @@
-// bf16 / f16 attention backward on the gfx950 matrix cores, head dimension 128: dQ, dK, dV of
+// bf16 / f16 attention backward on the gfx950 matrix cores, head dimension 64 or 128 (described for 128): dQ, dK, dV of
 // O = softmax(Q K^T s + mask) V for an upstream gradient dO, from Q, K, V, O, dO and the forward's row
 // normalisers L_i = log sum_j exp(x_ij) (the reference reaches the same gradients by walking its tape of
 // composed ops: crates/incin-backends/src/cpu/ops/matmul.rs:264-281, cpu/ops/elementwise.rs:1062-1077).
@@ -60,11 +60,11 @@ __global__ __launch_bounds__(256) void sdpa_bwd_delta_kernel(SdpaBwdParams p)
 // operand whose M index is the row) or transposed (the gfx950 transposing read: an A operand whose M index is the
 // column block).  fk serves both reads without bank conflicts: 16 consecutive rows put one logical chunk into 16
 // different slots, and the 4 rows x 64 bytes a half-wavefront transposes land in 4 different 64-byte column groups.
-template <typename T, int NW, int NDBU>      // NW wavefronts share a tile copy; a wavefront transposes NDBU column blocks
+template <typename T, int D, int NW, int NDBU>      // NW wavefronts share a tile copy; a wavefront transposes NDBU column blocks
 struct BwdTiles {
     typedef typename Mma<T>::vec8 vec8;
-    typedef PfLayout<128> L;
-    static constexpr int NSTEP = 8, LPW = L::TILE_BYTES / 1024 / NW;
+    typedef PfLayout<D> L;
+    static constexpr int NSTEP = D / 16, LPW = L::TILE_BYTES / 1024 / NW;
 
     int row_addr[NSTEP];           // [k-step]: byte offset of this lane's 16 bytes of row ql, chunk 2*s + g
     int tr_addr[NDBU][2];          // [column block - db0][half]: byte offset of the transposing read
@@ -97,7 +97,7 @@ struct BwdTiles {
     // elements) into `dst`; rows at and beyond `rows` arrive as zeros
     __device__ __forceinline__ void issue(int which, const T* base, int64_t stride, int rows, int row0, unsigned dst, int wave) const
     {
-        int64_t rem = (int64_t)(rows - row0 - 1) * stride * 2 + 256;
+        int64_t rem = (int64_t)(rows - row0 - 1) * stride * 2 + D * 2;
         if (rem > 0x7fffffffLL) rem = 0x7fffffffLL;
         if (rem < 0) rem = 0;
         const uint4v r = dma_descriptor((const char*)base + (int64_t)row0 * stride * 2, (int)rem);
@@ -121,14 +121,14 @@ struct BwdTiles {
 };
 
 // ---- dQ ----------------------------------------------------------------------------------------------------------------
-template <typename T>
+template <typename T, int D>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
 {
 #if defined(__HIP_DEVICE_COMPILE__)
     typedef typename Mma<T>::vec8 vec8;
-    typedef PfLayout<128> L;
-    constexpr int NSTEP = 8, NDB = 4, D = 128;
+    typedef PfLayout<D> L;
+    constexpr int NSTEP = D / 16, NDB = D / 32;
     const SdpaParams& p = bp.f;
     __shared__ __attribute__((aligned(1024))) char smem[4 * L::TILE_BYTES];      // K buffers 0, 1, V buffers 0, 1
 
@@ -166,7 +166,7 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
     const int n_tiles = (j_end + PF_BN - 1) / PF_BN;
     const int n_act = lim_wave_max > 0 ? (lim_wave_max + PF_BN - 1) / PF_BN : 0;
 
-    BwdTiles<T, 4, 4> tl;
+    BwdTiles<T, D, 4, NDB> tl;
     tl.init(wave, lane, p.k_ss, p.v_ss, 0);
 
     // this lane's query: Q row (scaled into log2 units, as the forward does) and dO row, the row's normaliser and D_i
@@ -280,15 +280,18 @@ constexpr int BWD_RING = 4;        // matrix operands in flight from LDS (reads 
 // t after a barrier.  Tiles t - 1 and t stay resident while tile t + 1 is copied: three stages.  The S and dP
 // accumulators do not start from zero but from -L_i log2(e) and -D_i (staged per tile next to the Q and dO rows), so
 // P = exp2(S) and dS = P * dP need no subtraction.
-template <typename T>
+template <typename T, int D>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
 {
 #if defined(__HIP_DEVICE_COMPILE__)
     typedef typename Mma<T>::vec8 vec8;
-    typedef PfLayout<128> L;
+    typedef PfLayout<D> L;
     typedef float float4v __attribute__((ext_vector_type(4)));
-    constexpr int NSTEP = 8, R = BWD_RING;
+    constexpr int NSTEP = D / 16, R = BWD_RING;
+    constexpr int NCB = D / 64;                         // 32-wide column blocks of dK / dV per wavefront (its half of the head dimension)
+    constexpr int NA = 2 * NSTEP;                       // matrix instructions of the first half of a step (S and dP)
+    constexpr int NB2 = 8 * NCB;                        // of the second half: 4 groups of 16 query rows x NCB blocks x (dV, dK)
     constexpr int STAGE = 2 * L::TILE_BYTES + 1024;     // Q rows, dO rows, 64 x -L_i log2(e), 64 x -D_i (and padding)
     constexpr int XCHG = 4 * 2 * 4 * 1024;              // [key block][query block][P lo, P hi, dS lo, dS hi]: 64 lanes x 16 bytes
     const SdpaParams& p = bp.f;
@@ -338,8 +341,8 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
     const int tiles_per_head = j0 < kv_len ? max(n_qt - t_begin, 0) : 0;
     const int n_tiles = tiles_per_head * p.G;           // the group's query heads one after another
 
-    BwdTiles<T, 8, 2> tl;
-    tl.init(wave, lane, p.q_ss, bp.do_ss, 2 * role);
+    BwdTiles<T, D, 8, NCB> tl;
+    tl.init(wave, lane, p.q_ss, bp.do_ss, NCB * role);
 
     // this lane's key: K row (scaled into log2 units) and V row as B operands
     vec8 kreg[NSTEP], vreg[NSTEP];
@@ -360,9 +363,9 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
     // rows i >= lo_i see this lane's key under the causal mask
     const int lo_i = p.causal ? my_j - coff : -0x40000000;
 
-    floatx16 dk_acc[2], dv_acc[2];         // column blocks 2*role, 2*role + 1
+    floatx16 dk_acc[NCB], dv_acc[NCB];     // column blocks NCB * role .. NCB * role + NCB - 1
 #pragma unroll
-    for (int d = 0; d < 2; ++d)
+    for (int d = 0; d < NCB; ++d)
 #pragma unroll
         for (int r = 0; r < 16; ++r) { dk_acc[d][r] = 0.0f; dv_acc[d][r] = 0.0f; }
 
@@ -378,8 +381,8 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
         nx_g = (const char*)bp.d_o + ((int64_t)b * bp.do_sb + (int64_t)hq * bp.do_sh + (int64_t)r0 * bp.do_ss) * 2;
         nx_s = (const char*)((wave == 0 ? bp.neg_l2 : bp.neg_delta) + ((int64_t)b * p.Hq + hq) * Sq + r0);
         nx_rows = Sq - r0;
-        nx_qrem = (int64_t)(nx_rows - 1) * p.q_ss * 2 + 256;
-        nx_grem = (int64_t)(nx_rows - 1) * bp.do_ss * 2 + 256;
+        nx_qrem = (int64_t)(nx_rows - 1) * p.q_ss * 2 + D * 2;
+        nx_grem = (int64_t)(nx_rows - 1) * bp.do_ss * 2 + D * 2;
         nx_r = 0;
         nx_h = h;
     };
@@ -444,10 +447,10 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
                     if (8 * (r / 4) + (r % 4) < rel) sa[r] = -INFINITY;
             }
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
+            for (int i = 0; i < NA; ++i) {
                 if (i % 2 == 0) sa = Mma<T>::run(ring[i % R], kreg[i / 2], sa);
                 else da = Mma<T>::run(ring[i % R], vreg[i / 2], da);
-                if (i + R < 16) fetch_a(i + R);
+                if (i + R < NA) fetch_a(i + R);
             }
         }
         // P and dS of register r of the own query block, rounded for the next products
@@ -458,10 +461,12 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
             ds[r / 8][r % 8] = (T)(pr * da[r]);
         };
         if (has_prev) {
-            // Matrix instruction m of the second half: group m / 4 = (own query block, rows 0-15), (own, 16-31), (partner's, 0-15),
-            // (partner's, 16-31); column block (m / 2) % 2 of this wavefront's two; dV from dO^T and P (even m), dK from Q^T and dS (odd).
+            // Matrix instruction m of the second half: group m / (2 NCB) = (own query block, rows 0-15), (own, 16-31),
+            // (partner's, 0-15), (partner's, 16-31); column block (m / 2) % NCB of this wavefront's; dV from dO^T and P (even m),
+            // dK from Q^T and dS (odd).
             auto fetch_b = [&](int m) __attribute__((always_inline)) {
-                ring[m % R] = tl.tr_op((m % 2 ? pq : pg) + (m < 8 ? own_rows : other_rows), (m / 2) % 2, (m / 4) % 2);
+                const int grp = m / (2 * NCB);
+                ring[m % R] = tl.tr_op((m % 2 ? pq : pg) + (grp < 2 ? own_rows : other_rows), (m / 2) % NCB, grp % 2);
             };
             vec8 bp_[2], bs_[2];        // P and dS of a group, two groups in flight
             auto fetch_group = [&](int grp) __attribute__((always_inline)) {
@@ -474,13 +479,14 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
 #pragma unroll
             for (int m = 0; m < R; ++m) fetch_b(m);
 #pragma unroll
-            for (int m = 0; m < 16; ++m) {
-                const int d = (m / 2) % 2;
-                if (m % 2 == 0) dv_acc[d] = Mma<T>::run(ring[m % R], bp_[(m / 4) % 2], dv_acc[d]);
-                else dk_acc[d] = Mma<T>::run(ring[m % R], bs_[(m / 4) % 2], dk_acc[d]);
-                if (m + R < 16) fetch_b(m + R);
-                if (m % 4 == 3 && m / 4 + 2 < 4) fetch_group(m / 4 + 2);
-                soft(m);
+            for (int m = 0; m < NB2; ++m) {
+                const int d = (m / 2) % NCB, grp = m / (2 * NCB);
+                if (m % 2 == 0) dv_acc[d] = Mma<T>::run(ring[m % R], bp_[grp % 2], dv_acc[d]);
+                else dk_acc[d] = Mma<T>::run(ring[m % R], bs_[grp % 2], dk_acc[d]);
+                if (m + R < NB2) fetch_b(m + R);
+                if (m % (2 * NCB) == 2 * NCB - 1 && grp + 2 < 4) fetch_group(grp + 2);
+#pragma unroll
+                for (int r = m * (16 / NB2); r < (m + 1) * (16 / NB2); ++r) soft(r);
             }
         } else {
 #pragma unroll
@@ -522,10 +528,10 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
     }
 
     if (my_j < Skv) {
-        T* krow = dkp + (int64_t)my_j * bp.dk_ss + role * 64;
-        T* vrow = dvp + (int64_t)my_j * bp.dv_ss + role * 64;
+        T* krow = dkp + (int64_t)my_j * bp.dk_ss + role * (D / 2);
+        T* vrow = dvp + (int64_t)my_j * bp.dv_ss + role * (D / 2);
 #pragma unroll
-        for (int d = 0; d < 2; ++d)
+        for (int d = 0; d < NCB; ++d)
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4) {
                 typedef T vec4 __attribute__((ext_vector_type(4)));
@@ -542,7 +548,7 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
 #endif
 }
 
-template <typename T>
+template <typename T, int D>
 static hipError_t launch_bwd_t(const SdpaBwdParams& bp, hipStream_t stream)
 {
     const SdpaParams& p = bp.f;
@@ -554,20 +560,20 @@ static hipError_t launch_bwd_t(const SdpaBwdParams& bp, hipStream_t stream)
         SdpaBwdParams bq = bp;      // two workgroups per CU, an eighth of the CUs per XCD
         bq.f.interleave = work_interleave(p.causal != 0, 2 * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
         bq.f.deal_groups = (total & 7) == 0 ? work_deal(bq.f.interleave, p.G, nqb, total >> 3) : 0;
-        hipLaunchKernelGGL((sdpa_bwd_dq_kernel<T>), dim3((unsigned)total), dim3(256), 0, stream, bq);
+        hipLaunchKernelGGL((sdpa_bwd_dq_kernel<T, D>), dim3((unsigned)total), dim3(256), 0, stream, bq);
     }
     const int nkb = (p.Skv + BWD_KEYS - 1) / BWD_KEYS;
     if ((int64_t)nkb * p.Hkv * p.B > 0)
-        hipLaunchKernelGGL((sdpa_bwd_dkv_kernel<T>), dim3((unsigned)((int64_t)nkb * p.Hkv * p.B)), dim3(512), 0, stream, bp);
+        hipLaunchKernelGGL((sdpa_bwd_dkv_kernel<T, D>), dim3((unsigned)((int64_t)nkb * p.Hkv * p.B)), dim3(512), 0, stream, bp);
     return hipGetLastError();
 }
 
-// Host has validated: dtype f16/bf16, D == Dv == 128, no dense mask, unit last-axis strides, 16-byte aligned rows,
+// Host has validated: dtype f16/bf16, D == Dv in {64, 128}, no dense mask, unit last-axis strides, 16-byte aligned rows,
 // row strides below 2^24 elements, lse and the delta workspace present.
 hipError_t launch_sdpa_bwd_mfma(const SdpaBwdParams& bp, int dtype, hipStream_t stream)
 {
-    if (dtype == 1) return launch_bwd_t<f16_t>(bp, stream);
-    return launch_bwd_t<bf16_t>(bp, stream);
+    if (bp.f.D == 128) return dtype == 1 ? launch_bwd_t<f16_t, 128>(bp, stream) : launch_bwd_t<bf16_t, 128>(bp, stream);
+    return dtype == 1 ? launch_bwd_t<f16_t, 64>(bp, stream) : launch_bwd_t<bf16_t, 64>(bp, stream);
 }
 
 }  // namespace incin_rocm

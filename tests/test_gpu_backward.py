@@ -43,10 +43,11 @@ def compare(name, got, ref, tol=2e-2):
     (3, 2, 2, 257, 257, True, [257, 100, 31]),
     (2, 2, 1, 64, 700, False, [700, 1]),
 ], ids=["tiny", "one_tile_causal", "rect", "gqa_causal", "gqa_rect_causal", "ragged_causal", "ragged"])
-def test_backward_against_the_oracle(gpu, dtype, shape):
+@pytest.mark.parametrize("D", [128, 64])
+def test_backward_against_the_oracle(gpu, dtype, shape, D):
     B, Hq, Hkv, Sq, Skv, causal, lens = shape
-    D, G = 128, Hq // Hkv
-    say("backward: %s dtype %d" % (shape, dtype))
+    G = Hq // Hkv
+    say("backward: %s D=%d dtype %d" % (shape, D, dtype))
     q, k, v, go = make(11, B, Hq, Hkv, Sq, Skv, D, dtype)
     lens_a = None if lens is None else np.asarray(lens, np.int32)
     out, dq, dk, dv = host.sdpa_backward(q, k, v, go, dtype, causal=causal, kv_lens=lens_a)
@@ -65,8 +66,8 @@ def test_backward_random_cases(gpu):
     workgroups, causal alignment with Sq <= Skv, ragged key counts >= 1 (every query row keeps a visible key, so the
     oracle has no NaN), scales.  Each case is printed before it runs."""
     r = np.random.Generator(np.random.PCG64(2026))
-    D = 128
     for case in range(28):
+        D = 128 if case % 3 else 64
         B, Hkv, G = int(r.integers(1, 4)), int(r.integers(1, 4)), int(r.choice([1, 2, 4]))
         Skv = int(r.choice([r.integers(1, 70), r.integers(60, 140), r.integers(120, 420)]))
         causal = bool(r.integers(0, 2))
@@ -109,8 +110,9 @@ def test_rows_without_visible_keys_get_zero_gradients(gpu):
     assert not dq.any() and not dk.any() and not dv.any()
 
 
-def test_backward_at_a_few_thousand_tokens(gpu):
-    B, Hq, Hkv, S, D = 1, 4, 2, 2048, 128
+@pytest.mark.parametrize("D", [128, 64])
+def test_backward_at_a_few_thousand_tokens(gpu, D):
+    B, Hq, Hkv, S = 1, 4, 2, 2048
     q, k, v, go = make(13, B, Hq, Hkv, S, S, D, capi.BF16)
     out, dq, dk, dv = host.sdpa_backward(q, k, v, go, capi.BF16, causal=True)
     rq, rk, rv = BW.sdpa_backward(q.reshape(B, Hkv, 2, S, D), k[:, :, None], v[:, :, None], go.reshape(B, Hkv, 2, S, D), causal=True)
@@ -244,9 +246,10 @@ def test_matrix_core_backward_f32_at_a_few_thousand_tokens(gpu):
 
 
 @pytest.mark.parametrize("dtype", [capi.BF16, capi.F16])
-def test_generic_and_matrix_core_backward_agree(gpu, dtype):
+@pytest.mark.parametrize("D", [128, 64])
+def test_generic_and_matrix_core_backward_agree(gpu, dtype, D):
     """The same 16-bit problem through both sets of kernels: each within tolerance of the oracle, and of each other."""
-    B, Hq, Hkv, S, D = 2, 4, 2, 200, 128
+    B, Hq, Hkv, S = 2, 4, 2, 200
     q, k, v, go = make(31, B, Hq, Hkv, S, S, D, dtype)
     lens = np.array([200, 77], np.int32)
     a = host.sdpa_backward(q, k, v, go, dtype, causal=True, kv_lens=lens, impl=capi.IMPL_GENERIC)
@@ -261,7 +264,7 @@ def test_generic_and_matrix_core_backward_agree(gpu, dtype):
 
 
 def test_backward_refuses_what_it_does_not_cover(gpu):
-    q, k, v, go = make(14, 1, 1, 1, 32, 32, 64, capi.BF16)
+    q, k, v, go = make(14, 1, 1, 1, 32, 32, 32, capi.BF16)
     with pytest.raises(capi.RocmError) as e:                     # the matrix-core kernels, pinned, outside their domain
         host.sdpa_backward(q, k, v, go, capi.BF16, impl=capi.IMPL_MFMA)
     assert e.value.code == capi.EUNSUPPORTED
