@@ -322,6 +322,37 @@ def backward_leg(steps, warmup, dtype=capi.BF16, B=8, H=16, S=4096, D=128, what=
             "parity_sample": "dQ, dK, dV of slice (b=%d, h=%d) against the float64 oracle of the reference's tape gradients" % (b, h)}
 
 
+def read_rate():
+    """What the memory system delivers to a kernel that only reads (incin_rocm_read_rate: 16-byte loads of 4 GiB, 8 in
+    flight per lane, summed and thrown away), with non-temporal loads and with plain ones - the measured ceiling the
+    split-KV kernels live under, reported beside the nominal HBM figure their roofline is priced against."""
+    nbytes = 4 << 30
+    src = capi.DeviceBuffer(nbytes)
+    capi.check(capi.load().incin_rocm_memset(0, src.ptr, 0x11, nbytes))
+    sink = capi.DeviceBuffer(16384)
+    out = {"what": "rate of a read-only kernel over 4 GiB (16-byte loads, 4096 workgroups of 256 threads, 8 loads in flight per lane)",
+           "unit": "GB/s", "nominal_peak": PEAK_HBM_GBS}
+    for name, nt in (("non_temporal_loads", True), ("plain_loads", False)):
+        for _ in range(5):
+            capi.read_rate(src, nbytes, nt, sink)
+        capi.sync()
+        best = None
+        for _ in range(3):
+            e0, e1 = capi.Event(), capi.Event()
+            e0.record()
+            for _ in range(10):
+                capi.read_rate(src, nbytes, nt, sink)
+            e1.record()
+            capi.sync()
+            ms = e0.elapsed_ms(e1) / 10
+            best = ms if best is None else min(best, ms)
+            e0.destroy(); e1.destroy()
+        out[name] = {"value": nbytes / (best * 1e-3) / 1e9, "ms": best, "frac_of_nominal": nbytes / (best * 1e-3) / 1e9 / PEAK_HBM_GBS}
+    src.free()
+    sink.free()
+    return out
+
+
 def matrix_rate():
     """What rate of bf16 matrix instructions the device sustains, by the data they work on: a loop of
     v_mfma_f32_32x32x16_bf16 on every compute unit (incin_rocm_matrix_rate), about 20 ms per launch, on zeros, on N(0,1)
@@ -451,7 +482,7 @@ def main():
                     help="prefill_long: skip the extra timing of the batch with its padding rows computed (profiling: every "
                          "launch of the run is then the same launch)")
     ap.add_argument("--decode-gqa-shape", default=None, help="with --only decode_gqa: one of its shapes by name (for profiles)")
-    ap.add_argument("--only", choices=["prefill", "prefill_long", "prefill_chunk", "decode", "decode_gqa", "backward", "f32", "copy", "matrix_rate"], default=None,
+    ap.add_argument("--only", choices=["prefill", "prefill_long", "prefill_chunk", "decode", "decode_gqa", "backward", "f32", "copy", "matrix_rate", "read_rate"], default=None,
                     help="run a single workload (profiling). 'copy' runs --steps device-to-device copies of 1 GiB "
                          "through the library's plain copy kernel: the known-size dispatch that hardware byte "
                          "counters (FETCH_SIZE / WRITE_SIZE) are calibrated against")
@@ -605,6 +636,9 @@ def main():
 
     if args.only in (None, "matrix_rate"):
         result["matrix_rate"] = matrix_rate()
+
+    if args.only in (None, "read_rate"):
+        result["read_rate"] = read_rate()
 
     if args.only in (None, "backward"):
         result["backward"] = backward_leg(max(5, min(args.steps, 30)), min(args.warmup, 5))

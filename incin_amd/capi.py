@@ -31,7 +31,7 @@ EXPORTS = [
     "incin_rocm_sdpa_workspace", "incin_rocm_sdpa_fwd", "incin_rocm_sdpa_fwd_static",
     "incin_rocm_sizeof_kv_append_desc", "incin_rocm_kv_append",
     "incin_rocm_sizeof_sdpa_bwd_desc", "incin_rocm_sdpa_bwd_workspace", "incin_rocm_sdpa_bwd",
-    "incin_rocm_matrix_rate",
+    "incin_rocm_matrix_rate", "incin_rocm_read_rate",
 ]
 
 
@@ -158,6 +158,7 @@ def load():
     lib.incin_rocm_sdpa_bwd.argtypes = [C.POINTER(SdpaBwdDesc), C.c_void_p]
     lib.incin_rocm_kv_append.argtypes = [C.POINTER(KvAppendDesc), C.c_void_p]
     lib.incin_rocm_matrix_rate.argtypes = [C.c_int32, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.POINTER(C.c_double), C.c_void_p]
+    lib.incin_rocm_read_rate.argtypes = [C.c_int32, C.c_void_p, C.c_size_t, C.c_int32, C.c_void_p, C.c_void_p]
     _lib = lib
     return lib
 
@@ -234,6 +235,11 @@ def sdpa_bwd_workspace(desc):
 
 def sdpa_bwd(desc, stream=None):
     check(load().incin_rocm_sdpa_bwd(C.byref(desc), stream))
+
+
+def read_rate(src, nbytes, nontemporal, sink, stream=None, dev=0):
+    """One launch of the read-only kernel over nbytes of src (DeviceBuffer); time it with events."""
+    check(load().incin_rocm_read_rate(dev, src.ptr, nbytes, 1 if nontemporal else 0, sink.ptr, stream))
 
 
 def matrix_rate(operands, sink, mix, iterations, stream=None, dev=0):

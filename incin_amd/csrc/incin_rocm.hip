@@ -26,6 +26,7 @@ hipError_t launch_sdpa_prefill_f32(const SdpaParams& p, hipStream_t stream);
 hipError_t launch_mask_classify(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_sdpa_decode(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_sdpa_decode_mfma(const SdpaParams& p, int dtype, hipStream_t stream);
+hipError_t launch_read_rate(const void* src, void* sink, size_t bytes, int nontemporal, hipStream_t stream);
 int decode_mfma_chunk_rows(int R);
 int decode_mfma_workgroups_per_cu(int chunk_rows, int64_t split_len);
 int decode_keys_per_tile(int dtype, int D, int R);
@@ -697,6 +698,17 @@ int incin_rocm_matrix_rate(int32_t dev, const void* operands, void* sink, int32_
     if (int rc = use_device(dev)) return rc;
     const hipError_t e = incin_rocm::launch_matrix_rate(operands, sink, mix, iterations, flops, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "matrix rate launch");
+    return 0;
+}
+
+int incin_rocm_read_rate(int32_t dev, const void* src, size_t bytes, int32_t nontemporal, void* sink, void* stream)
+{
+    if (!src || !sink) return fail(INCIN_ROCM_EINVAL, "read_rate: null pointer");
+    if (bytes == 0 || bytes % ((size_t)4096 * 32768) != 0) return fail(INCIN_ROCM_EINVAL, "read_rate: bytes is a positive multiple of 128 MiB");
+    if (!aligned16(src)) return fail(INCIN_ROCM_EINVAL, "read_rate: src must be 16-byte aligned");
+    if (int rc = use_device(dev)) return rc;
+    const hipError_t e = incin_rocm::launch_read_rate(src, sink, bytes, nontemporal != 0, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "read rate launch");
     return 0;
 }
 

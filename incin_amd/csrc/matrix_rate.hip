@@ -79,4 +79,33 @@ hipError_t launch_matrix_rate(const void* src, void* sink, int mix, int iteratio
     return hipGetLastError();
 }
 
+// ---- read rate -----------------------------------------------------------------------------------------------------
+// Nothing but 16-byte loads of `bytes` bytes, 8 in flight per lane, summed and thrown away: what the memory system
+// delivers to a kernel that only reads - the ceiling the split-KV kernels live under, below the nominal HBM figure.
+typedef float float4r __attribute__((ext_vector_type(4)));
+template <bool NT>
+__global__ __launch_bounds__(256) void read_rate_kernel(const float4r* __restrict__ src, float* sink, size_t vecs_per_wg)
+{
+    const float4r* p = src + (size_t)blockIdx.x * vecs_per_wg + threadIdx.x;
+    float4r acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (size_t i = 0; i < vecs_per_wg; i += 256 * 8) {
+        float4r v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = NT ? __builtin_nontemporal_load(p + i + u * 256) : p[i + u * 256];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc += v[u];
+    }
+    if (acc[0] + acc[1] + acc[2] + acc[3] == 12345.678f) sink[blockIdx.x] = acc[0];      // (never: keeps the loads alive)
+}
+
+// bytes: a multiple of 4096 workgroups x 32 KiB; sink: 16 KiB.
+hipError_t launch_read_rate(const void* src, void* sink, size_t bytes, int nontemporal, hipStream_t stream)
+{
+    const int wgs = 4096;
+    const size_t vecs_per_wg = bytes / 16 / wgs;
+    if (nontemporal) hipLaunchKernelGGL((read_rate_kernel<true>), dim3(wgs), dim3(256), 0, stream, (const float4r*)src, (float*)sink, vecs_per_wg);
+    else hipLaunchKernelGGL((read_rate_kernel<false>), dim3(wgs), dim3(256), 0, stream, (const float4r*)src, (float*)sink, vecs_per_wg);
+    return hipGetLastError();
+}
+
 }  // namespace incin_rocm

@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define INCIN_ROCM_ABI_VERSION 6
+#define INCIN_ROCM_ABI_VERSION 7
 
 /* ---- status codes (mapped to incin_core::Error variants by the Rust side;
  *      crates/incin-core/src/err.rs:109-223) --------------------------------- */
@@ -260,6 +260,12 @@ int incin_rocm_sdpa_bwd(const incin_rocm_sdpa_bwd_desc_t* desc, void* stream);
  * and it is the ceiling the 16-bit attention kernels live under; bench.py reports it beside their roofline.
  * `sink` takes 2 KiB per compute unit.  *flops = FLOPs of the launch; time it with events on `stream`. */
 int incin_rocm_matrix_rate(int32_t dev, const void* operands, void* sink, int32_t mix, int32_t iterations, double* flops, void* stream);
+
+/* No counterpart in the reference.  One launch of a kernel that does nothing but read `bytes` bytes at `src` (a positive
+ * multiple of 128 MiB) with 16-byte loads, marked non-temporal or not, and throw them away: the rate the memory system
+ * delivers to a kernel that only reads, the ceiling the split-KV kernels live under; bench.py reports it beside their
+ * roofline.  `sink` takes 16 KiB.  Time it with events on `stream`. */
+int incin_rocm_read_rate(int32_t dev, const void* src, size_t bytes, int32_t nontemporal, void* sink, void* stream);
 
 /* ---- key/value cache append ----------------------------------------------------
  * No counterpart in the reference (it has no cache: a decode loop there concatenates tensors,

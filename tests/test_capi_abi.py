@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), "missing export %s" % n
     assert set(names) == set(capi.EXPORTS)
-    assert lib.incin_rocm_abi_version() == 6
+    assert lib.incin_rocm_abi_version() == 7
 
 
 def test_descriptor_layout_matches():
@@ -170,6 +170,13 @@ def test_matrix_rate_validation():
     assert lib.incin_rocm_matrix_rate(0, 0x1000, 0x1000, 2, 10, C.byref(fl), None) == capi.EINVAL
     assert lib.incin_rocm_matrix_rate(0, 0x1000, 0x1000, 0, 0, C.byref(fl), None) == capi.EINVAL
     assert b"matrix_rate" in lib.incin_rocm_last_error()
+    # and so does the read-rate one
+    assert lib.incin_rocm_read_rate(0, None, 1 << 27, 1, 0x1000, None) == capi.EINVAL
+    assert lib.incin_rocm_read_rate(0, 0x1000, 1 << 27, 1, None, None) == capi.EINVAL
+    assert lib.incin_rocm_read_rate(0, 0x1000, 0, 1, 0x1000, None) == capi.EINVAL
+    assert lib.incin_rocm_read_rate(0, 0x1000, (1 << 27) + 4096, 1, 0x1000, None) == capi.EINVAL      # not a multiple of 128 MiB
+    assert lib.incin_rocm_read_rate(0, 0x1008, 1 << 27, 1, 0x1000, None) == capi.EINVAL               # misaligned
+    assert b"read_rate" in lib.incin_rocm_last_error()
 
 
 def _bwd(fwd_kw=None, **kw):

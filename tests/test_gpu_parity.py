@@ -723,6 +723,30 @@ def test_matrix_rate_diagnostic(gpu):
     sink.free()
 
 
+def test_read_rate_diagnostic(gpu):
+    """The read-only kernel runs, writes nothing (its sink keeps what it held) and takes about the time the memory system
+    needs for the bytes (between 2 and 8 TB/s: a sanity range, the figure itself is bench.py's business)."""
+    nbytes = 1 << 30
+    src = capi.DeviceBuffer(nbytes)
+    capi.check(capi.load().incin_rocm_memset(0, src.ptr, 0x11, nbytes))
+    sink = capi.DeviceBuffer.from_numpy(np.full(4096, 7.0, np.float32))
+    for nt in (True, False):
+        capi.read_rate(src, nbytes, nt, sink)
+        capi.sync()
+        e0, e1 = capi.Event(), capi.Event()
+        e0.record()
+        for _ in range(5):
+            capi.read_rate(src, nbytes, nt, sink)
+        e1.record()
+        capi.sync()
+        rate = 5 * nbytes / (e0.elapsed_ms(e1) * 1e-3) / 1e12
+        say("read rate, %s loads: %.2f TB/s" % ("non-temporal" if nt else "plain", rate))
+        assert 2.0 < rate < 8.0
+    assert np.array_equal(sink.to_numpy(np.float32, (4096,)), np.full(4096, 7.0, np.float32))
+    src.free()
+    sink.free()
+
+
 def test_copy_strided_gathers_any_view(gpu):
     """incin_rocm_copy_strided against numpy's own view semantics: transposes of the last two axes and of outer axes,
     broadcast (stride 0) and reversed (negative stride) axes, offsets into a larger buffer, ranks 0 to 8, 2- and 4-byte
