@@ -7,12 +7,13 @@
 // The work is bound by the bandwidth of the cache reads, so the design serves the memory system first:
 //
 //   * one workgroup (4 wavefronts) per (batch, KV head, chunk of 32 or 64 query rows, split), one workgroup per compute
-//     unit.  The split's keys are dealt to the wavefronts in blocks of 32 (D = 64: 64; wavefront w takes blocks w, w + 4, ...), and
+//     unit (two of the two-slot form that short splits take: see the launcher).  The split's keys are dealt to the wavefronts in blocks of 32 (D = 64: 64; wavefront w takes blocks w, w + 4, ...), and
 //     a wavefront works through its blocks on its own: no barrier in the loop, nothing shared.  Each wavefront owns a
 //     ring of NSLOT 8 KiB slots in LDS that the K and V blocks pass through in the order they are needed
 //     (K0 V0 K1 V1 ...), filled straight from global memory (buffer_load ... lds, whole rows, 1 KiB per instruction);
 //     a slot is refilled the moment its block has been used, so NSLOT - 1 blocks per wavefront - 128 KiB per compute
-//     unit with five slots - are in flight at any time;
+//     unit with five slots - are in flight at any time, and the wait for the oldest copy is a constant s_waitcnt: copies
+//     past a wavefront's last block are started all the same, with a descriptor that covers nothing;
 //   * 32 rows are the 32 columns of S^T = K Q^T (v_mfma_f32_32x32x16, a lane owns one row's scores of the block; rows
 //     that do not exist are zero columns - matrix throughput is not what is scarce here), the softmax is the usual
 //     online one per wavefront, and O^T += V^T P^T takes V through transposing LDS reads; with 64 rows every K and V
