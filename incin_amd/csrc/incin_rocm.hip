@@ -730,7 +730,6 @@ static int check_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, bool* empty, int* kin
     *empty = plan.empty || d->Skv == 0;
     *kind = 0;
     if (*empty) return 0;
-    if (d->q_lens) return fail(INCIN_ROCM_EUNSUPPORTED, "%s: no kernel takes q_lens", OP);
     if (!d->lse) return fail(INCIN_ROCM_EINVAL, "%s: fwd.lse (the forward's row normalisers) is required", OP);
     if (!bd->d_o || !bd->d_q || !bd->d_k || !bd->d_v) return fail(INCIN_ROCM_EINVAL, "%s: null gradient pointer", OP);
     if (d->D > 256 || d->Dv > 256) return fail(INCIN_ROCM_EUNSUPPORTED, "%s: D and Dv up to 256", OP);

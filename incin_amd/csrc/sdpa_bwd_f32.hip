@@ -137,18 +137,22 @@ void bwd_f32_dq_kernel(SdpaBwdParams bp)
 
     int kv_len = Skv;
     if (p.kv_lens) kv_len = clampi(p.kv_lens[b], 0, Skv);
+    // query rows at and beyond rows_b are padding (q_lens): their dQ is written as zero; a lane's row stays in its own
+    // column of every product here, so a padding row next to real ones computes in isolation
+    const int rows_b = p.q_lens ? clampi(p.q_lens[b], 0, Sq) : Sq;
     const int coff = Skv - Sq;
     int j_end = kv_len;
     const int my_i = q0 + wave * 32 + ql;
     int lim_lane = kv_len, lim_wave_min = kv_len, lim_wave_max = kv_len;
     if (p.causal) {
-        const int last_row = min(q0 + PF_BM - 1, Sq - 1);
+        const int last_row = min(q0 + PF_BM - 1, rows_b - 1);
         j_end = clampi(last_row + coff + 1, 0, kv_len);
         lim_lane = clampi(my_i + coff + 1, 0, kv_len);
         lim_wave_min = clampi(q0 + wave * 32 + coff + 1, 0, kv_len);
-        lim_wave_max = clampi(min(q0 + wave * 32 + 31, Sq - 1) + coff + 1, 0, kv_len);
+        lim_wave_max = clampi(min(q0 + wave * 32 + 31, rows_b - 1) + coff + 1, 0, kv_len);
     }
-    if (q0 + wave * 32 >= Sq) lim_wave_min = lim_wave_max = 0;
+    if (q0 >= rows_b) j_end = 0;
+    if (q0 + wave * 32 >= rows_b) lim_wave_min = lim_wave_max = 0;
     const int n_tiles = (j_end + KT - 1) / KT;
     const int n_act = lim_wave_max > 0 ? (lim_wave_max + KT - 1) / KT : 0;
 
@@ -264,7 +268,7 @@ void bwd_f32_dq_kernel(SdpaBwdParams bp)
             for (int r4 = 0; r4 < 4; ++r4) {
                 float4v w;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) w[e] = dq_acc[db][r4 * 4 + e] * p.scale;
+                for (int e = 0; e < 4; ++e) w[e] = my_i < rows_b ? dq_acc[db][r4 * 4 + e] * p.scale : 0.0f;
                 *(float4v*)(row + db * 32 + r4 * 8 + g * 4) = w;
             }
     }
@@ -320,7 +324,10 @@ void bwd_f32_dkv_kernel(SdpaBwdParams bp)
     // first query row that sees every key of this wavefront: tiles from there on need no mask
     const int i_all_wave = p.causal ? max(j0 + wave * 32 + 31 - coff, 0) : 0;
     const int t_begin = i_begin_wg / QT;
-    const int n_qt = (Sq + QT - 1) / QT;
+    // query rows at and beyond rows_b are padding (q_lens): the tiles end there, and the rows between there and the end of
+    // the last tile arrive as zeros like rows past Sq
+    const int rows_b = p.q_lens ? clampi(p.q_lens[b], 0, Sq) : Sq;
+    const int n_qt = (rows_b + QT - 1) / QT;
     const int tiles_per_head = j0 < kv_len ? max(n_qt - t_begin, 0) : 0;
     const int n_tiles = tiles_per_head * p.G;           // the group's query heads one after another
 
@@ -360,11 +367,11 @@ void bwd_f32_dkv_kernel(SdpaBwdParams bp)
         const int h = n / tiles_per_head, r0 = (t_begin + n % tiles_per_head) * QT;
         const int hq = hkv * p.G + h;
         const unsigned st = lds0 + stage * STAGE;
-        ad.issue(0, (const float*)p.q + (int64_t)b * p.q_sb + (int64_t)hq * p.q_sh, p.q_ss, Sq, r0, st, wave);
-        ad.issue(1, (const float*)bp.d_o + (int64_t)b * bp.do_sb + (int64_t)hq * bp.do_sh, bp.do_ss, Sq, r0, st + L::TILE_BYTES, wave);
+        ad.issue(0, (const float*)p.q + (int64_t)b * p.q_sb + (int64_t)hq * p.q_sh, p.q_ss, rows_b, r0, st, wave);
+        ad.issue(1, (const float*)bp.d_o + (int64_t)b * bp.do_sb + (int64_t)hq * bp.do_sh, bp.do_ss, rows_b, r0, st + L::TILE_BYTES, wave);
         if (wave < 2) {          // 64 floats (a tile has at most that many rows) of one of the two per-row arrays; rows past Sq arrive as zeros
             const float* src = (wave == 0 ? bp.neg_l2 : bp.neg_delta) + ((int64_t)b * p.Hq + hq) * Sq + r0;
-            dma_copy4(dma_descriptor(src, (Sq - r0) * 4), st + 2 * L::TILE_BYTES + wave * 256, lane * 4);
+            dma_copy4(dma_descriptor(src, (rows_b - r0) * 4), st + 2 * L::TILE_BYTES + wave * 256, lane * 4);
         }
     };
 
@@ -380,7 +387,7 @@ void bwd_f32_dkv_kernel(SdpaBwdParams bp)
 #pragma unroll
         for (int qb = 0; qb < NB; ++qb) {
             const int ib = i0 + qb * 32;               // first query row of the block
-            if (ib >= Sq) break;
+            if (ib >= rows_b) break;
             // S - L and dP - D in the lane-owns-a-key layout: register r is query row ib + 8 (r / 4) + 4 g + r % 4.
             // Operands of a step are read from LDS one step ahead, as in the dQ kernel.
             floatx16 s, dp;

@@ -54,10 +54,10 @@ __device__ __forceinline__ void load_tile(float* dst, int pitch, const T* base, 
 // P and dS of one (query i, key j) pair from the raw products s = q_i.k_j and dp = dO_i.v_j
 struct Pair { float p, ds; };
 template <typename T>
-__device__ __forceinline__ Pair pair_of(const SdpaParams& f, const T* mp, int i, int j, int kv_len, int coff, float s, float dp, float L, float negD)
+__device__ __forceinline__ Pair pair_of(const SdpaParams& f, int rows_b, const T* mp, int i, int j, int kv_len, int coff, float s, float dp, float L, float negD)
 {
     Pair r = {0.0f, 0.0f};
-    if (i >= f.Sq || j >= kv_len || (f.causal && j > i + coff) || L == -INFINITY) return r;
+    if (i >= rows_b || j >= kv_len || (f.causal && j > i + coff) || L == -INFINITY) return r;
     float x = s * f.scale;
     if (mp) x += to_f32(mp[(int64_t)i * f.m_si + (int64_t)j * f.m_sj]);
     if (x == -INFINITY) return r;         // hidden by the dense mask
@@ -89,14 +89,17 @@ __global__ __launch_bounds__(256) void bwd_generic_dq_kernel(SdpaBwdParams bp)
     T* dqp = (T*)bp.d_q + (int64_t)b * bp.dq_sb + (int64_t)hq * bp.dq_sh;
     const T* mp = p.mask ? (const T*)p.mask + (int64_t)b * p.m_sb + (int64_t)hq * p.m_sh : nullptr;
 
-    load_tile(Qs, DP, qp, p.q_ss, q0, Sq, D, tid);
-    load_tile(Gs, DP, gp, bp.do_ss, q0, Sq, Dv, tid);
+    // query rows at and beyond rows_b are padding (q_lens): they arrive as zeros, weigh nothing and get a zero dQ
+    const int rows_b = p.q_lens ? clampi(p.q_lens[b], 0, Sq) : Sq;
+    load_tile(Qs, DP, qp, p.q_ss, q0, rows_b, D, tid);
+    load_tile(Gs, DP, gp, bp.do_ss, q0, rows_b, Dv, tid);
 
     int kv_len = Skv;
     if (p.kv_lens) kv_len = clampi(p.kv_lens[b], 0, Skv);
     const int coff = Skv - Sq;
     int j_end = kv_len;
     if (p.causal) j_end = clampi(min(q0 + GB - 1, Sq - 1) + coff + 1, 0, kv_len);
+    if (q0 >= rows_b) j_end = 0;
 
     float L[2], negD[2];
 #pragma unroll
@@ -135,7 +138,7 @@ __global__ __launch_bounds__(256) void bwd_generic_dq_kernel(SdpaBwdParams bp)
 #pragma unroll
             for (int c = 0; c < 2; ++c)
                 Ss[(2 * ty + r) * (GB + 1) + tx + 16 * c] =
-                    pair_of(p, mp, q0 + 2 * ty + r, j0 + tx + 16 * c, kv_len, coff, s[r][c], dp[r][c], L[r], negD[r]).ds;
+                    pair_of(p, rows_b, mp, q0 + 2 * ty + r, j0 + tx + 16 * c, kv_len, coff, s[r][c], dp[r][c], L[r], negD[r]).ds;
         __syncthreads();
         for (int jj = 0; jj < GB; ++jj) {
             const float d0 = Ss[(2 * ty) * (GB + 1) + jj], d1 = Ss[(2 * ty + 1) * (GB + 1) + jj];
@@ -153,7 +156,7 @@ __global__ __launch_bounds__(256) void bwd_generic_dq_kernel(SdpaBwdParams bp)
         if (i >= Sq) continue;
 #pragma unroll
         for (int c = 0; c < NC; ++c)
-            if (tx + 16 * c < D) dqp[(int64_t)i * bp.dq_ss + tx + 16 * c] = from_f32<T>(acc[r][c] * p.scale);
+            if (tx + 16 * c < D) dqp[(int64_t)i * bp.dq_ss + tx + 16 * c] = from_f32<T>(i < rows_b ? acc[r][c] * p.scale : 0.0f);
     }
 }
 
@@ -188,7 +191,8 @@ __global__ __launch_bounds__(256) void bwd_generic_dkv_kernel(SdpaBwdParams bp)
     const int coff = Skv - Sq;
     // first query row that sees a key of this block (causal: i >= j - coff)
     const int i_begin = p.causal ? clampi(j0 - coff, 0, Sq) / GB * GB : 0;
-    const int i_end = j0 < kv_len ? Sq : 0;
+    const int rows_b = p.q_lens ? clampi(p.q_lens[b], 0, Sq) : Sq;      // query rows at and beyond are padding (q_lens)
+    const int i_end = j0 < kv_len ? rows_b : 0;
 
     float dk[2][NC], dv[2][NC];
 #pragma unroll
@@ -204,8 +208,8 @@ __global__ __launch_bounds__(256) void bwd_generic_dkv_kernel(SdpaBwdParams bp)
         const int64_t stat0 = ((int64_t)b * p.Hq + hq) * Sq;
         for (int i0 = i_begin; i0 < i_end; i0 += GB) {
             __syncthreads();                     // the previous tile is consumed (and K, V are stored)
-            load_tile(Qs, DP, qp, p.q_ss, i0, Sq, D, tid);
-            load_tile(Gs, DP, gp, bp.do_ss, i0, Sq, Dv, tid);
+            load_tile(Qs, DP, qp, p.q_ss, i0, rows_b, D, tid);
+            load_tile(Gs, DP, gp, bp.do_ss, i0, rows_b, Dv, tid);
             if (tid < GB) {
                 const int i = min(i0 + tid, Sq - 1);
                 Ls[tid] = p.lse[stat0 + i];
@@ -231,7 +235,7 @@ __global__ __launch_bounds__(256) void bwd_generic_dkv_kernel(SdpaBwdParams bp)
 #pragma unroll
                 for (int c = 0; c < 2; ++c) {
                     const int ii = tx + 16 * c;
-                    const Pair pr = pair_of(p, mp, i0 + ii, j0 + 2 * ty + r, kv_len, coff, s[r][c], dp[r][c], Ls[ii], Ds[ii]);
+                    const Pair pr = pair_of(p, rows_b, mp, i0 + ii, j0 + 2 * ty + r, kv_len, coff, s[r][c], dp[r][c], Ls[ii], Ds[ii]);
                     Ps[(2 * ty + r) * (GB + 1) + ii] = pr.p;
                     Ss[(2 * ty + r) * (GB + 1) + ii] = pr.ds;
                 }

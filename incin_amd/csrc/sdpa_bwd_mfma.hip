@@ -154,15 +154,20 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
 
     int kv_len = Skv;
     if (p.kv_lens) kv_len = clampi(p.kv_lens[b], 0, Skv);
+    // query rows at and beyond rows_b are padding (q_lens): what the forward left in their O and lse, and what their dO
+    // holds, is never used - their dQ is written as zero and they add nothing to dK and dV.  A lane's row stays in its
+    // own column of every product here, so a padding row inside a wavefront that has real ones computes in isolation.
+    const int rows_b = p.q_lens ? clampi(p.q_lens[b], 0, Sq) : Sq;
     const int coff = Skv - Sq;
     const int my_i = q0 + wave * 32 + ql;
     int j_end = kv_len, lim_lane = kv_len, lim_wave_max = kv_len;
     if (p.causal) {
-        j_end = clampi(min(q0 + PF_BM - 1, Sq - 1) + coff + 1, 0, kv_len);
+        j_end = clampi(min(q0 + PF_BM - 1, rows_b - 1) + coff + 1, 0, kv_len);
         lim_lane = clampi(my_i + coff + 1, 0, kv_len);
-        lim_wave_max = clampi(min(q0 + wave * 32 + 31, Sq - 1) + coff + 1, 0, kv_len);
+        lim_wave_max = clampi(min(q0 + wave * 32 + 31, rows_b - 1) + coff + 1, 0, kv_len);
     }
-    if (q0 + wave * 32 >= Sq) lim_wave_max = 0;
+    if (q0 >= rows_b) j_end = 0;
+    if (q0 + wave * 32 >= rows_b) lim_wave_max = 0;
     const int n_tiles = (j_end + PF_BN - 1) / PF_BN;
     const int n_act = lim_wave_max > 0 ? (lim_wave_max + PF_BN - 1) / PF_BN : 0;
 
@@ -255,7 +260,7 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
                 typedef T vec4 __attribute__((ext_vector_type(4)));
                 vec4 w;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) w[e] = (T)(dq_acc[db][r4 * 4 + e] * p.scale);
+                for (int e = 0; e < 4; ++e) w[e] = (T)(my_i < rows_b ? dq_acc[db][r4 * 4 + e] * p.scale : 0.0f);
                 *(vec4*)(row + db * 32 + r4 * 8 + g * 4) = w;
             }
     }
@@ -337,7 +342,10 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
     // first query row that sees every key of this wavefront: tiles from there on need no mask
     const int i_all_wave = p.causal ? max(j0 + kb * 32 + 31 - coff, 0) : 0;
     const int t_begin = i_begin_wg / PF_BN;
-    const int n_qt = (Sq + PF_BN - 1) / PF_BN;
+    // query rows at and beyond rows_b are padding (q_lens): the tiles end there, and the rows between there and the end of
+    // the last tile arrive as zeros like rows past Sq (Q, dO and the per-row values), which leaves dS and P^T dO at zero
+    const int rows_b = p.q_lens ? clampi(p.q_lens[b], 0, Sq) : Sq;
+    const int n_qt = (rows_b + PF_BN - 1) / PF_BN;
     const int tiles_per_head = j0 < kv_len ? max(n_qt - t_begin, 0) : 0;
     const int n_tiles = tiles_per_head * p.G;           // the group's query heads one after another
 
@@ -380,7 +388,7 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
         nx_q = (const char*)p.q + ((int64_t)b * p.q_sb + (int64_t)hq * p.q_sh + (int64_t)r0 * p.q_ss) * 2;
         nx_g = (const char*)bp.d_o + ((int64_t)b * bp.do_sb + (int64_t)hq * bp.do_sh + (int64_t)r0 * bp.do_ss) * 2;
         nx_s = (const char*)((wave == 0 ? bp.neg_l2 : bp.neg_delta) + ((int64_t)b * p.Hq + hq) * Sq + r0);
-        nx_rows = Sq - r0;
+        nx_rows = rows_b - r0;
         nx_qrem = (int64_t)(nx_rows - 1) * p.q_ss * 2 + D * 2;
         nx_grem = (int64_t)(nx_rows - 1) * bp.do_ss * 2 + D * 2;
         nx_r = 0;

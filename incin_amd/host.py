@@ -131,10 +131,13 @@ def sdpa(q, k, v, dtype=capi.F32, scale=None, causal=False, kv_lens=None, mask=N
     return out
 
 
-def sdpa_backward(q, k, v, d_out, dtype=capi.BF16, scale=None, causal=False, kv_lens=None, impl=capi.IMPL_AUTO, dev=0, mask=None):
+def sdpa_backward(q, k, v, d_out, dtype=capi.BF16, scale=None, causal=False, kv_lens=None, impl=capi.IMPL_AUTO, dev=0, mask=None,
+                  q_lens=None, poison_padding=False):
     """Forward (with row normalisers) then backward on the GPU for f32 numpy operands [B,Hq,Sq,D], [B,Hkv,Skv,D],
     [B,Hkv,Skv,Dv], d_out [B,Hq,Sq,Dv] and an optional dense additive mask broadcastable to [B,Hq,Sq,Skv]; returns
-    (out, dq, dk, dv) as f32 holding the `dtype`-rounded results.  `impl` pins the kernels of both passes."""
+    (out, dq, dk, dv) as f32 holding the `dtype`-rounded results.  `impl` pins the kernels of both passes.  q_lens: query
+    rows at and beyond are padding; poison_padding overwrites what the forward left in their O and lse rows with NaN
+    bit patterns before the backward runs (it must not read them)."""
     q, k, v, d_out = (np.asarray(x, dtype=np.float32) for x in (q, k, v, d_out))
     B, Hq, Sq, D = q.shape
     Dv = v.shape[-1]
@@ -147,14 +150,24 @@ def sdpa_backward(q, k, v, d_out, dtype=capi.BF16, scale=None, causal=False, kv_
         mask = np.asarray(mask, dtype=np.float32)
         ms = mask_strides_for(mask.shape, B, Hq, Sq, k.shape[2])
         tm = capi.DeviceBuffer.from_numpy(dtypes.encode(mask, dtype), dev)
+    tql = capi.DeviceBuffer.from_numpy(np.asarray(q_lens, dtype=np.int32), dev) if q_lens is not None else None
     tlse = capi.DeviceBuffer(max(B * Hq * Sq, 1) * 4, dev)
     bd = capi.SdpaBwdDesc()
-    bd.fwd = make_desc(tq, tk, tv, to, scale, causal, tl, tm, ms, impl=impl, lse=tlse)
+    bd.fwd = make_desc(tq, tk, tv, to, scale, causal, tl, tm, ms, impl=impl, lse=tlse, q_lens=tql)
     fbytes = capi.sdpa_workspace(bd.fwd)[0]
     fws = capi.DeviceBuffer(fbytes, dev) if fbytes else None
     if fws is not None:
         bd.fwd.workspace, bd.fwd.workspace_bytes = fws.ptr, fws.nbytes
     capi.sdpa_fwd(bd.fwd)
+    if poison_padding and q_lens is not None:
+        capi.sync(dev)
+        o_host, l_host = to.to_f32(), tlse.to_numpy(np.float32, (B, Hq, Sq))
+        for b in range(B):
+            o_host[b, :, int(q_lens[b]):] = np.nan
+            l_host[b, :, int(q_lens[b]):] = np.nan
+        raw = dtypes.encode(o_host, dtype)
+        capi.check(capi.load().incin_rocm_memcpy_h2d(dev, to.ptr, raw.ctypes.data, raw.nbytes))
+        capi.check(capi.load().incin_rocm_memcpy_h2d(dev, tlse.ptr, l_host.ctypes.data, l_host.nbytes))
     for name, t in (("d_o", tg), ("d_q", tdq), ("d_k", tdk), ("d_v", tdv)):
         setattr(bd, name, t.ptr)
         st = _strides3(t.shape)
@@ -167,7 +180,7 @@ def sdpa_backward(q, k, v, d_out, dtype=capi.BF16, scale=None, causal=False, kv_
     capi.sdpa_bwd(bd)
     capi.sync(dev)
     res = tuple(t.to_f32() for t in (to, tdq, tdk, tdv))
-    for t in (tq.buf, tk.buf, tv.buf, tg.buf, to.buf, tdq.buf, tdk.buf, tdv.buf, tl, tm, tlse, ws, fws):
+    for t in (tq.buf, tk.buf, tv.buf, tg.buf, to.buf, tdq.buf, tdk.buf, tdv.buf, tl, tm, tlse, ws, fws, tql):
         if t is not None:
             t.free()
     return res

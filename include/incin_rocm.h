@@ -226,7 +226,8 @@ int incin_rocm_sdpa_fwd_static(const incin_rocm_sdpa_desc_t* desc, void* stream)
  *
  * `fwd` is the forward's descriptor as it was launched with `lse` set (o and lse are inputs here); causal,
  * kv_lens and the grouped-query layout carry over; d_k and d_v are summed over the query heads of a group.
- * Covered: f32 / f16 / bf16, D and Dv up to 256, dense additive mask, causal, kv_lens (no q_lens: INCIN_ROCM_EUNSUPPORTED).
+ * Covered: f32 / f16 / bf16, D and Dv up to 256, dense additive mask, causal, kv_lens, q_lens (padding query rows: their
+ * O, lse and d_o rows are never read, their d_q rows are written as zero and they add nothing to d_k and d_v).
  * fwd.impl picks the kernels: AUTO = matrix-core kernels where they apply - f16 / bf16 with D == Dv in {64, 128} and a positive
  * scale, f32 (IEEE single-precision matrix instructions) with D == Dv in {64, 128} and any finite scale; both without a
  * dense mask and with 16-byte aligned rows - and generic f32-arithmetic kernels otherwise; GENERIC and MFMA pin one or

@@ -298,3 +298,32 @@ def test_no_keys_gives_a_zero_query_gradient(gpu, dtype):
     capi.sdpa_bwd(bd)
     capi.sync()
     assert not to.to_f32().any() and not tdq.to_f32().any()
+
+
+@pytest.mark.parametrize("case", [
+    # dtype, impl, D
+    (capi.BF16, capi.IMPL_AUTO, 128), (capi.F16, capi.IMPL_MFMA, 64), (capi.F32, capi.IMPL_AUTO, 64), (capi.F32, capi.IMPL_MFMA, 128),
+    (capi.F32, capi.IMPL_GENERIC, 80), (capi.BF16, capi.IMPL_GENERIC, 128),
+], ids=["bf16_auto", "f16_mfma_d64", "f32_auto_d64", "f32_mfma", "f32_generic_d80", "bf16_generic"])
+def test_backward_of_a_padded_batch(gpu, case):
+    """A padded self-attention batch: sequence b has lens[b] real positions, the rest of its rows and keys are padding
+    (q_lens = kv_lens = lens).  The forward leaves the padding rows of O and lse unspecified - here they are overwritten
+    with NaN, and the padding rows of dO hold NaN too - and the backward must give, per sequence, the gradients of that
+    sequence alone: dQ, dK, dV of the truncated problem inside the lengths, exact zeros outside."""
+    dtype, impl, D = case
+    B, Hq, Hkv, S = 3, 4, 2, 300
+    G = Hq // Hkv
+    lens = np.array([300, 131, 64], np.int32)
+    q, k, v, go = make(71, B, Hq, Hkv, S, S, D, dtype)
+    for b in range(B):
+        go[b, :, lens[b]:] = np.nan
+    out, dq, dk, dv = host.sdpa_backward(q, k, v, go, dtype, causal=True, kv_lens=lens, q_lens=lens, impl=impl, poison_padding=True)
+    tol = 1e-5 if dtype == capi.F32 else 2e-2
+    for b in range(B):
+        n = int(lens[b])
+        rq, rk, rv = BW.sdpa_backward(q[b:b + 1, :, :n].reshape(1, Hkv, G, n, D), k[b:b + 1, :, None, :n], v[b:b + 1, :, None, :n],
+                                      go[b:b + 1, :, :n].reshape(1, Hkv, G, n, D), causal=True)
+        compare("dq[%d]" % b, dq[b:b + 1, :, :n], rq.reshape(1, Hq, n, D), tol)
+        compare("dk[%d]" % b, dk[b:b + 1, :, :n], rk.reshape(1, Hkv, n, D), tol)
+        compare("dv[%d]" % b, dv[b:b + 1, :, :n], rv.reshape(1, Hkv, n, D), tol)
+        assert not dq[b, :, n:].any() and not dk[b, :, n:].any() and not dv[b, :, n:].any()
