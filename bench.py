@@ -210,23 +210,29 @@ def decode_gqa_leg(steps, warmup, only_shape=None):
     through the kernel AUTO picks (the matrix-core split-KV kernel) and, where it takes the shape, through the
     vector-ALU split-KV kernel; KV bytes read once / launch time against the HBM peak."""
     out = {}
-    shapes = [("gqa4_b32_kv8192", 32, 32, 8, 1, 8192, False), ("gqa4_b1_kv131072", 1, 32, 8, 1, 131072, False),
-              ("gqa8_b32_kv8192", 32, 64, 8, 1, 8192, False), ("gqa4_sq4_b8_kv8192", 8, 32, 8, 4, 8192, True)]
+    BF, F = capi.BF16, capi.F32
+    shapes = [("gqa4_b32_kv8192", 32, 32, 8, 1, 8192, False, BF), ("gqa4_b1_kv131072", 1, 32, 8, 1, 131072, False, BF),
+              ("gqa8_b32_kv8192", 32, 64, 8, 1, 8192, False, BF), ("gqa4_sq4_b8_kv8192", 8, 32, 8, 4, 8192, True, BF),
+              # f32 caches (the reference's own dtype): 4 rows per KV head, and 32 (8 heads x 4 positions), where the IEEE-f32
+              # matrix instructions - half a PFLOP/s short of the 16-bit ones - come close to being the bound
+              ("f32_gqa4_b32_kv8192", 32, 32, 8, 1, 8192, False, F), ("f32_gqa8_sq4_b8_kv8192", 8, 64, 8, 4, 8192, True, F)]
     names = {capi.IMPL_SPLITKV: "sdpa_decode_split_kernel (vector ALU)", capi.IMPL_SPLITKV_MFMA: "sdpa_decode_mfma_kernel (matrix cores)",
              capi.IMPL_MFMA: "sdpa_prefill_mfma_kernel"}
-    for i, (name, B, Hq, Hkv, Sq, Skv, causal) in enumerate(shapes):
+    names_f32 = {capi.IMPL_SPLITKV: "sdpa_decode_split_kernel (vector ALU)", capi.IMPL_SPLITKV_MFMA: "sdpa_decode_f32_kernel (matrix cores, IEEE f32)",
+                 capi.IMPL_MFMA: "sdpa_prefill_f32_kernel"}
+    for i, (name, B, Hq, Hkv, Sq, Skv, causal, dt) in enumerate(shapes):
         if only_shape is not None and name != only_shape:
             continue
-        kv_bytes = 2.0 * B * Hkv * Skv * 128 * 2
+        kv_bytes = 2.0 * B * Hkv * Skv * 128 * (4 if dt == F else 2)
         n = max(steps, min(200, int(0.02 / (kv_bytes / 6e12))))
-        entry = {"workload": "bf16 decode B=%d Hq=%d Hkv=%d S_q=%d KV=%d D=128%s" % (B, Hq, Hkv, Sq, Skv, " causal" if causal else "")}
+        entry = {"workload": "%s decode B=%d Hq=%d Hkv=%d S_q=%d KV=%d D=128%s" % (dtypes.NAMES[dt], B, Hq, Hkv, Sq, Skv, " causal" if causal else "")}
         for impl in (capi.IMPL_AUTO, capi.IMPL_SPLITKV):
             if impl == capi.IMPL_SPLITKV and (Hq // Hkv) * Sq > 8:
                 continue
-            w = Workload("decode_" + name, SEED0 + 40 + i, B, Hq, Hkv, Sq, Skv, 128, capi.BF16, causal, impl=impl)
+            w = Workload("decode_" + name, SEED0 + 40 + i, B, Hq, Hkv, Sq, Skv, 128, dt, causal, impl=impl)
             wall, ev_mean, ev_med, ev_min = w.time(n, warmup)
             entry["auto" if impl == capi.IMPL_AUTO else "vector_alu_kernel"] = {
-                "kernel": names.get(w.impl, str(w.impl)), "num_splits": w.splits, "ms_per_step": wall,
+                "kernel": (names_f32 if dt == F else names).get(w.impl, str(w.impl)), "num_splits": w.splits, "ms_per_step": wall,
                 "kv_gb_per_s": kv_bytes / (wall * 1e-3) / 1e9,
                 "roofline": {"bound": "hbm", "achieved": kv_bytes / (ev_mean * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                              "frac": kv_bytes / (ev_mean * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None,

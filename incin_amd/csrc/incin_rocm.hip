@@ -27,8 +27,8 @@ hipError_t launch_mask_classify(const SdpaParams& p, int dtype, hipStream_t stre
 hipError_t launch_sdpa_decode(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_sdpa_decode_mfma(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_read_rate(const void* src, void* sink, size_t bytes, int nontemporal, hipStream_t stream);
-int decode_mfma_chunk_rows(int R);
-int decode_mfma_workgroups_per_cu(int chunk_rows, int64_t split_len);
+int decode_mfma_chunk_rows(int R, int dtype);
+int decode_mfma_workgroups_per_cu(int chunk_rows, int64_t split_len, int dtype);
 int decode_keys_per_tile(int dtype, int D, int R);
 }  // namespace incin_rocm
 
@@ -162,8 +162,8 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     // a way that needs it positive.  Both take a dense additive mask (any strides); the 64-row kernel does not.
     const bool mfma_ok = layout_ok && tile_off_ok && std::isfinite(d->scale) && (d->dtype == INCIN_ROCM_F32 || d->scale > 0.0f);
     const bool split_ok = fast_ok && d->Sq <= 64;
-    // the matrix-core split-KV kernel: 16-bit storage, blocks addressed like the prefill kernels' tiles
-    const bool split_mfma_ok = split_ok && tile_off_ok && d->dtype != INCIN_ROCM_F32 && std::isfinite(d->scale);
+    // the matrix-core split-KV kernels (16-bit and f32): blocks addressed like the prefill kernels' tiles
+    const bool split_mfma_ok = split_ok && tile_off_ok && std::isfinite(d->scale);
 
     int impl = d->impl;
     if (impl == INCIN_ROCM_IMPL_AUTO) {
@@ -178,9 +178,18 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         // Up to 64 rows the matrix-core kernel reads the cache once; beyond (it would read it once per 64 rows) the
         // prefill kernel takes over, which splits the keys itself when its launch is small (measured level or ahead from
         // 128 rows per KV head on).
-        const int64_t kv_bytes = 2 * d->B * d->Hkv * d->Skv * d->D * 2;       // (16-bit storage where it matters)
-        const int64_t len128 = d->Skv * d->D / 128;      // cache length in keys of 128 elements (what the thresholds were measured in)
-        if (split_mfma_ok && len128 >= 256 &&
+        const int64_t esize = (int64_t)dtype_size(d->dtype);
+        const int64_t kv_bytes = 2 * d->B * d->Hkv * d->Skv * d->D * esize;
+        const int64_t len128 = d->Skv * d->D * esize / 256;      // cache length in keys of 256 bytes (what the thresholds were measured in)
+        // f32 (sdpa_decode_f32.hip): from two rows per KV head on, whatever the count - the f32 prefill kernel would spend a
+        // 32-row matrix instruction on every query head's few rows (32 heads of a group at one position each: 8.4 ms
+        // against 0.23), and where it packs as well (64 positions of one head) the split-KV form is still ahead (0.22
+        // against 0.28 ms on 8 x 8 heads x 8192 keys); the vector-ALU kernel is level at 2 rows and behind from 4 on
+        // (4 rows, 268 MB of cache: 5.6 against 4.8 TB/s; 8 rows: 6.6 against 3.4).  More than 32 rows over fewer than 512
+        // keys stay with the prefill kernel (64 positions x 16 heads x 64 sequences of 256 keys: 0.14 against 0.17 ms).
+        if (d->dtype == INCIN_ROCM_F32 && split_mfma_ok && len128 >= 256 && R >= 2 && (R <= 32 || d->Skv >= 512))
+            impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
+        else if (d->dtype != INCIN_ROCM_F32 && split_mfma_ok && len128 >= 256 &&
             ((R == 1 && len128 >= 1024 && kv_bytes >= (512LL << 20)) || (R >= 2 && R <= 3 && len128 >= 512) || (R >= 4 && R <= 64)))
             impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
         else if (split_ok && R <= 8 && d->Skv >= 256) impl = INCIN_ROCM_IMPL_SPLITKV;
@@ -196,7 +205,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
                     "scaled_dot_product_attention: the 64-row MFMA prefill kernel has been retired (INCIN_ROCM_IMPL_MFMA covers its shapes)");
     if (impl == INCIN_ROCM_IMPL_SPLITKV_MFMA && !split_mfma_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
-                    "scaled_dot_product_attention: the matrix-core split-KV kernel needs f16/bf16, D == Dv in {64,128}, Sq <= 64, no dense mask, a finite scale and 16-byte aligned rows");
+                    "scaled_dot_product_attention: the matrix-core split-KV kernels need D == Dv in {64,128}, Sq <= 64, no dense mask, a finite scale and 16-byte aligned rows");
     if (impl == INCIN_ROCM_IMPL_SPLITKV && !split_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
                     "scaled_dot_product_attention: the split-KV kernel needs D == Dv in {64,128}, Sq <= 64, no dense mask and 16-byte aligned rows");
@@ -234,7 +243,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         // workgroups of a launch, all of equal length, run in rounds.  Take the number of splits that leaves the last
         // round fullest, among those that keep at least 256 keys per split, preferring fewer splits at (nearly) equal
         // filling: fewer partial results to combine.
-        const int64_t chunk = incin_rocm::decode_mfma_chunk_rows((int)std::min<int64_t>(R, 1 << 20));
+        const int64_t chunk = incin_rocm::decode_mfma_chunk_rows((int)std::min<int64_t>(R, 1 << 20), d->dtype);
         const int64_t nchunks = (R + chunk - 1) / chunk;
         const int64_t groups = d->B * d->Hkv * nchunks;
         int64_t splits = d->num_splits;
@@ -244,7 +253,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
             const int64_t max_splits = std::min<int64_t>(max_by_len, std::max<int64_t>(1, 4 * cus / groups));
             auto fill = [&](int64_t s) {           // (with the split length, and so the count, s really leads to)
                 const int64_t len = ((d->Skv + s - 1) / s + 255) / 256 * 256;
-                const int64_t at_a_time = cus * incin_rocm::decode_mfma_workgroups_per_cu((int)chunk, len);
+                const int64_t at_a_time = cus * incin_rocm::decode_mfma_workgroups_per_cu((int)chunk, len, d->dtype);
                 const int64_t wgs = groups * ((d->Skv + len - 1) / len), rounds = (wgs + at_a_time - 1) / at_a_time;
                 return (double)wgs / (double)(rounds * at_a_time);
             };

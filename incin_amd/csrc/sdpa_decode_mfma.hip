@@ -25,38 +25,9 @@
 // positions.  The scale is applied to the f32 scores (any sign), masks as -inf before the maximum.
 #include <cstdlib>
 
-#include "sdpa_mfma_common.h"
+#include "sdpa_decode_ring.h"
 
 namespace incin_rocm {
-
-constexpr int DM_SLOT_BYTES = 8192;      // a block of K or of V: 32 keys at D = 128, 64 keys at D = 64
-#ifndef DM_SHORT_KEYS
-#define DM_SHORT_KEYS 2048
-#endif
-#ifndef DM_NSLOT
-#define DM_NSLOT 5       // slots per wavefront: 4 wavefronts x 5 x 8 KiB = the 160 KiB of a compute unit
-#endif
-
-// One wavefront-wide global -> LDS copy of 64 x 16 bytes, as dma_copy16, marked non-temporal: every byte of the cache
-// is read once per launch, and leaving it out of the caches' replacement order is worth 12 - 13 points of the memory
-// bandwidth (measured on 32 x 32 heads x 8192 keys: 6.05 TB/s without the mark, 7.04 with it).
-#ifndef DM_CACHE
-#define DM_CACHE " nt"
-#endif
-__device__ __forceinline__ void dm_copy16(uint4v desc, unsigned lds_addr, int byte_offset)
-{
-    asm volatile("s_nop 0\n\tbuffer_load_dwordx4 %0, %1, 0 offen" DM_CACHE " lds" ::"v"(byte_offset), "s"(desc), "{m0}"(lds_addr) : "memory");
-}
-
-// All but the newest NSLOT - 1 copies of this wavefront (8 instructions each) have landed.
-template <int NSLOT> __device__ __forceinline__ void wait_oldest_copy()
-{
-    static_assert(NSLOT >= 2 && NSLOT <= 5, "s_waitcnt takes an immediate");
-    if (NSLOT == 5) asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
-    else if (NSLOT == 4) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
-    else if (NSLOT == 3) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-}
 
 template <typename T, int D, int NSLOT, int NRB>
 __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
@@ -407,34 +378,49 @@ static hipError_t launch_decode_mfma_t(const SdpaParams& p, hipStream_t stream)
     return hipGetLastError();
 }
 
-// Rows a workgroup takes: 32, or 64 (two blocks of 32 against the same K and V operands) when more than 32 rows share a KV
-// head - the cache is then read once for 64 rows instead of once per 32.
-int decode_mfma_chunk_rows(int R) { return R > 32 ? 64 : 32; }
+int decode_f32_chunk_rows(int R);
+hipError_t launch_sdpa_decode_f32(const SdpaParams& p, bool two_slots, hipStream_t stream);
 
-// Workgroups a compute unit holds at a time: two of the two-slot form (32 rows, splits of up to DM_SHORT_KEYS keys), one
-// otherwise.  The planner fills rounds of this many.
-int decode_mfma_workgroups_per_cu(int chunk_rows, int64_t split_len) { return chunk_rows == 32 && split_len <= DM_SHORT_KEYS ? 2 : 1; }
+// Rows a workgroup takes: 32, or 64 (two blocks of 32 against the same K and V operands) when more than 32 rows share a KV
+// head - the cache is then read once for 64 rows instead of once per 32.  (f32, dtype 0: 16 or 32, sdpa_decode_f32.hip.)
+int decode_mfma_chunk_rows(int R, int dtype) { return dtype == 0 ? decode_f32_chunk_rows(R) : R > 32 ? 64 : 32; }
+
+// Workgroups a compute unit holds at a time: two of the two-slot form (one block of rows, splits of up to DM_SHORT_KEYS
+// keys of 16-bit storage or half as many of f32), one otherwise.  The planner fills rounds of this many.
+int decode_mfma_workgroups_per_cu(int chunk_rows, int64_t split_len, int dtype)
+{
+    if (dtype == 0) return chunk_rows == 16 && 2 * split_len <= DM_SHORT_KEYS ? 2 : 1;
+    return chunk_rows == 32 && split_len <= DM_SHORT_KEYS ? 2 : 1;
+}
+
+// INCIN_ROCM_DECODE_SLOTS = 2 or 5 overrides the choice between the two forms of the one-block kernels (for tests: both
+// forms on any shape).
+static bool decode_two_slots(const SdpaParams& p, int dtype)
+{
+    const char* forced = getenv("INCIN_ROCM_DECODE_SLOTS");
+    const int slots = forced ? atoi(forced) : 0;
+    const int one_block = dtype == 0 ? 16 : 32;
+    return slots == 2 || (slots != DM_NSLOT && decode_mfma_workgroups_per_cu(one_block, p.split_len, dtype) == 2);
+}
 
 // Host has validated: dtype f16 / bf16, D == Dv in {64, 128}, rows 16-byte aligned with unit last-dim stride, row strides
 // below 2^24 elements, split_len a multiple of 256 (whole rounds of the four wavefronts' blocks of 32 or 64 keys).
 template <typename T, int D>
 static hipError_t launch_decode_mfma_d(const SdpaParams& p, hipStream_t stream)
 {
-    if (decode_mfma_chunk_rows(p.G * p.Sq) == 64) return launch_decode_mfma_t<T, D, DM_NSLOT, 2>(p, stream);
+    if (decode_mfma_chunk_rows(p.G * p.Sq, 2) == 64) return launch_decode_mfma_t<T, D, DM_NSLOT, 2>(p, stream);
     // Short splits (up to DM_SHORT_KEYS keys: 16 blocks per wavefront) take rings of two slots, which lets a compute
     // unit hold two workgroups: with so little to stream, what counts is that one workgroup's start-up (its first
     // copies' latency) and end (the wavefronts' results meeting, the stores) overlap another's arithmetic.  Measured
     // on launches of 268 MB of cache, two slots against five: 256-key splits 73 against 46 % of the memory bandwidth,
     // 512: 81 / 63, 1024: 80 / 73, 2048: 87.5 / 86.3; 4096: 78.5 / 80 (one sequence of 131072 keys); 8192: 84 / 86.7.
-    // INCIN_ROCM_DECODE_SLOTS = 2 or 5 overrides the rule (for tests: both forms on any shape).
-    const char* forced = getenv("INCIN_ROCM_DECODE_SLOTS");
-    const int slots = forced ? atoi(forced) : 0;
-    if (slots == 2 || (slots != DM_NSLOT && decode_mfma_workgroups_per_cu(32, p.split_len) == 2)) return launch_decode_mfma_t<T, D, 2, 1>(p, stream);
+    if (decode_two_slots(p, 2)) return launch_decode_mfma_t<T, D, 2, 1>(p, stream);
     return launch_decode_mfma_t<T, D, DM_NSLOT, 1>(p, stream);
 }
 
 hipError_t launch_sdpa_decode_mfma(const SdpaParams& p, int dtype, hipStream_t stream)
 {
+    if (dtype == 0) return launch_sdpa_decode_f32(p, decode_two_slots(p, 0), stream);
     hipError_t e;
     if (p.D == 128) e = dtype == 1 ? launch_decode_mfma_d<f16_t, 128>(p, stream) : launch_decode_mfma_d<bf16_t, 128>(p, stream);
     else e = dtype == 1 ? launch_decode_mfma_d<f16_t, 64>(p, stream) : launch_decode_mfma_d<bf16_t, 64>(p, stream);

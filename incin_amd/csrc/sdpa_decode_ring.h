@@ -1,0 +1,38 @@
+// The per-wavefront ring of LDS slots that the matrix-core split-KV kernels (sdpa_decode_mfma.hip: f16 / bf16,
+// sdpa_decode_f32.hip: f32) stream the key/value cache through: slot size, the non-temporal global -> LDS copy and
+// the constant wait for the oldest copy in flight.
+#pragma once
+#include "sdpa_mfma_common.h"
+
+namespace incin_rocm {
+
+constexpr int DM_SLOT_BYTES = 8192;      // a block of K or of V: 16-bit storage 32 keys at D = 128, 64 at D = 64; f32 half as many
+#ifndef DM_SHORT_KEYS
+#define DM_SHORT_KEYS 2048      // (keys of 256 bytes: 16-bit storage at D = 128)
+#endif
+#ifndef DM_NSLOT
+#define DM_NSLOT 5       // slots per wavefront: 4 wavefronts x 5 x 8 KiB = the 160 KiB of a compute unit
+#endif
+
+// One wavefront-wide global -> LDS copy of 64 x 16 bytes, as dma_copy16, marked non-temporal: every byte of the cache
+// is read once per launch, and leaving it out of the caches' replacement order is worth 12 - 13 points of the memory
+// bandwidth (measured on 32 x 32 heads x 8192 keys: 6.05 TB/s without the mark, 7.04 with it).
+#ifndef DM_CACHE
+#define DM_CACHE " nt"
+#endif
+__device__ __forceinline__ void dm_copy16(uint4v desc, unsigned lds_addr, int byte_offset)
+{
+    asm volatile("s_nop 0\n\tbuffer_load_dwordx4 %0, %1, 0 offen" DM_CACHE " lds" ::"v"(byte_offset), "s"(desc), "{m0}"(lds_addr) : "memory");
+}
+
+// All but the newest NSLOT - 1 copies of this wavefront (8 instructions each) have landed.
+template <int NSLOT> __device__ __forceinline__ void wait_oldest_copy()
+{
+    static_assert(NSLOT >= 2 && NSLOT <= 5, "s_waitcnt takes an immediate");
+    if (NSLOT == 5) asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
+    else if (NSLOT == 4) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+    else if (NSLOT == 3) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+}
+
+}  // namespace incin_rocm

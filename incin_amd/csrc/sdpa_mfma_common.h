@@ -73,6 +73,20 @@ template <int D> struct PfLayout {
     }
 };
 
+// The same for rows of f32 (the IEEE-f32 kernels: sdpa_prefill_f32.hip, sdpa_decode_f32.hip).
+template <int D> struct F32Layout {
+    static constexpr int ROWB = D * 4;                       // bytes per K/V row in LDS (unpadded)
+    static constexpr int CPR = D / 4;                        // 16-byte chunks per row
+    static constexpr int TILE_BYTES = 16384;
+    static constexpr int KT = TILE_BYTES / ROWB;             // keys per tile: 64 (D = 64), 32 (D = 128)
+    static constexpr int NB = KT / 32;                       // 32-key blocks per tile
+    static constexpr int LOADS_PER_WAVE = TILE_BYTES / 1024 / 4;
+    // Chunk c of row r sits at chunk c ^ f(r).  K reads go down 16 consecutive rows at one logical chunk: f takes 16
+    // values there.  V reads take rows r and r + 4 (r % 8 < 4) in the two halves of a wavefront, eight consecutive
+    // chunks each: f(r) and f(r + 4) differ in bit 3, which sends the halves to different halves of the banks.
+    static __device__ __forceinline__ int f(int r) { return (r & 3) | ((r & 4) << 1) | ((r & 8) >> 1); }
+};
+
 // One wavefront-wide global -> LDS copy (64 lanes x 16 bytes land at lds_addr .. lds_addr + 1023 in lane order; lanes
 // whose offset is outside the descriptor's range deliver zeros).  Issued through inline assembly on purpose: the
 // compiler makes every LDS access it cannot prove disjoint from a copy it knows of wait until that copy has landed -

@@ -34,19 +34,6 @@
 
 namespace incin_rocm {
 
-template <int D> struct F32Layout {
-    static constexpr int ROWB = D * 4;                       // bytes per K/V row in LDS (unpadded)
-    static constexpr int CPR = D / 4;                        // 16-byte chunks per row
-    static constexpr int TILE_BYTES = 16384;
-    static constexpr int KT = TILE_BYTES / ROWB;             // keys per tile: 64 (D = 64), 32 (D = 128)
-    static constexpr int NB = KT / 32;                       // 32-key blocks per tile
-    static constexpr int LOADS_PER_WAVE = TILE_BYTES / 1024 / 4;
-    // Chunk c of row r sits at chunk c ^ f(r).  K reads go down 16 consecutive rows at one logical chunk: f takes 16
-    // values there.  V reads take rows r and r + 4 (r % 8 < 4) in the two halves of a wavefront, eight consecutive
-    // chunks each: f(r) and f(r + 4) differ in bit 3, which sends the halves to different halves of the banks.
-    static __device__ __forceinline__ int f(int r) { return (r & 3) | ((r & 4) << 1) | ((r & 8) >> 1); }
-};
-
 // SPLIT: the launch is a grid of (work items) x (splits of the key axis); a workgroup handles the keys of its split only and
 // writes, per row, the unnormalised O, the maximum and the sum in the partial-result format of the split-KV kernels, whose
 // combine kernel finishes - for launches with too few (batch, head, row block) items to fill the device over a long key axis.

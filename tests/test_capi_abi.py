@@ -79,7 +79,14 @@ def test_dispatch_choices():
     assert impl == capi.IMPL_SPLITKV_MFMA and splits == 32
     _, splits, impl = _plan(_desc(Sq=1, Skv=8192, B=32, Hq=32, Hkv=8))
     assert impl == capi.IMPL_SPLITKV_MFMA and splits == 1                     # 256 groups: one round, nothing to combine
-    assert _plan(_desc(Sq=1, Skv=8192, B=2, Hq=8, Hkv=2, dtype=capi.F32))[2] == capi.IMPL_SPLITKV   # f32: vector ALU
+    # f32: its own matrix-core split-KV kernel (chunks of 16 or 32 rows) from two rows per KV head on, any number of rows
+    assert _plan(_desc(Sq=1, Skv=8192, B=2, Hq=8, Hkv=2, dtype=capi.F32))[2] == capi.IMPL_SPLITKV_MFMA
+    assert _plan(_desc(Sq=1, Skv=8192, B=2, Hq=8, Hkv=8, dtype=capi.F32))[2] == capi.IMPL_SPLITKV             # one row: vector ALU
+    assert _plan(_desc(Sq=64, Skv=8192, B=2, Hq=32, Hkv=2, dtype=capi.F32))[2] == capi.IMPL_SPLITKV_MFMA      # 1024 rows per KV head
+    assert _plan(_desc(Sq=65, Skv=8192, B=2, Hq=32, Hkv=2, dtype=capi.F32))[2] == capi.IMPL_MFMA              # more positions: prefill
+    assert _plan(_desc(Sq=1, Skv=100, B=2, Hq=8, Hkv=2, dtype=capi.F32))[2] == capi.IMPL_MFMA                 # shortest caches: one workgroup per head
+    _, splits, impl = _plan(_desc(Sq=1, Skv=8192, B=32, Hq=32, Hkv=8, dtype=capi.F32))
+    assert impl == capi.IMPL_SPLITKV_MFMA and splits == 1
     assert _plan(_desc(Sq=1, Skv=8192, B=2, Hq=8, Hkv=2, D=64, Dv=64))[2] == capi.IMPL_SPLITKV_MFMA            # D = 64 too
     assert _plan(_desc(Sq=4, Skv=8192, B=2, Hq=32, Hkv=2))[2] == capi.IMPL_SPLITKV_MFMA             # 64 rows per KV head: one workgroup's worth
     _, splits, impl = _plan(_desc(Sq=8, Skv=8192, B=2, Hq=32, Hkv=2))
@@ -136,7 +143,6 @@ def test_dispatch_choices():
     (dict(impl=capi.IMPL_MFMA, D=80, Dv=80), capi.EUNSUPPORTED),
     (dict(impl=capi.IMPL_SPLITKV, Sq=4096), capi.EUNSUPPORTED),
     (dict(impl=capi.IMPL_SPLITKV_MFMA, Sq=4096), capi.EUNSUPPORTED),
-    (dict(impl=capi.IMPL_SPLITKV_MFMA, Sq=1, dtype=capi.F32), capi.EUNSUPPORTED),
     (dict(impl=capi.IMPL_SPLITKV_MFMA, Sq=1, D=32, Dv=32), capi.EUNSUPPORTED),
     (dict(impl=capi.IMPL_SPLITKV_MFMA, Sq=1, add_mask=0x20000), capi.EUNSUPPORTED),
     (dict(D=512, Dv=512), capi.EUNSUPPORTED),

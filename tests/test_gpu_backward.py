@@ -192,7 +192,10 @@ def test_matrix_core_backward_f32_against_the_oracle(gpu, shape):
     refs = (rq.reshape(B, Hq, Sq, D), rk.reshape(B, Hkv, Skv, D), rv.reshape(B, Hkv, Skv, D))
     for name, x, a, g_, r_ in zip(("dq", "dk", "dv"), (dq, dk, dv), auto[1:], gen[1:], refs):
         compare(name, x, r_, tol=1e-5)
-        assert np.array_equal(x, a), name + ": AUTO takes the same kernels, which have no run-to-run variation"
+        if Sq > 64:
+            assert np.array_equal(x, a), name + ": AUTO takes the same kernels, which have no run-to-run variation"
+        else:       # up to 64 positions AUTO's forward is the split-KV kernel: O and the row normalisers differ in the last bits
+            compare(name + " AUTO vs pinned", a, x, tol=2e-6)
         compare(name + " generic vs matrix-core", g_, x, tol=2e-5)
     if lens is not None:
         for b in range(B):

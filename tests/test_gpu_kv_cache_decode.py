@@ -57,8 +57,8 @@ def test_decode_loop_over_a_device_side_cache(gpu, dtype, replay):
     ws = capi.DeviceBuffer(nbytes) if nbytes else None
     if ws is not None:
         sd.workspace, sd.workspace_bytes = ws.ptr, ws.nbytes
-    # 4 query heads per KV head: the matrix-core split-KV kernel for 16-bit caches, the vector-ALU one for f32
-    assert impl == (capi.IMPL_SPLITKV if dtype == capi.F32 else capi.IMPL_SPLITKV_MFMA)
+    # 4 query heads per KV head: the matrix-core split-KV kernels (16-bit and f32)
+    assert impl == capi.IMPL_SPLITKV_MFMA
 
     stream = capi.Stream()
     graph = None

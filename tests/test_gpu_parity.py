@@ -509,6 +509,69 @@ def test_decode_splitkv_matrix_cores_d64(gpu, dtype, shape, slots, monkeypatch):
         check(got, host.sdpa(q, k, v, dtype, causal=causal, kv_lens=lens, impl=capi.IMPL_SPLITKV), 8e-3, "matrix-core vs vector-ALU split-KV, D = 64")
 
 
+@pytest.mark.parametrize("D", [128, 64])
+@pytest.mark.parametrize("slots", ["2", "5"], ids=["two_slot_rings", "five_slot_rings"])
+@pytest.mark.parametrize("shape", [
+    # B, Hq, Hkv, Sq, Skv, causal      (f32: chunks of 16 or 32 rows, blocks of 16 keys at D = 128 and 32 at D = 64)
+    (2, 8, 2, 1, 4096, False),        # grouped-query decode, 4 rows per KV head
+    (1, 32, 4, 1, 3000, False),       # 8 rows, ragged last block
+    (3, 16, 1, 1, 700, True),         # multi-query, 16 rows: a full block of rows
+    (1, 8, 2, 5, 1500, True),         # 20 rows: the 32-row instance, a causal edge among the 5 positions
+    (1, 40, 1, 1, 333, False),        # 40 rows: two chunks of 32, the second with 8 rows
+    (2, 12, 4, 9, 1000, True),        # 27 rows
+    (1, 8, 8, 1, 200, False),         # a single row per KV head, fewer keys than a split asks for
+    (1, 6, 2, 22, 1500, True),        # 66 rows per KV head: three chunks, causal over 22 positions
+    (1, 4, 2, 8, 5, True),            # more positions than keys: the first three see none (NaN rows, as the reference)
+])
+def test_decode_splitkv_matrix_cores_f32(gpu, D, shape, slots, monkeypatch):
+    """The f32 matrix-core split-KV kernel (IEEE-f32 matrix instructions) against the oracle at the f32 bar, with the
+    split count left to the library, forced to one and forced to counts that leave ragged and empty last splits, with key
+    counts per batch entry, and against the vector-ALU split-KV kernel where that one takes the shape; row normalisers
+    from the one-split and the combined launches."""
+    monkeypatch.setenv("INCIN_ROCM_DECODE_SLOTS", slots)
+    B, Hq, Hkv, Sq, Skv, causal = shape
+    dt = capi.F32
+    q, k, v = inputs(1300 + D + sum(shape[:5]), B, Hq, Hkv, Sq, Skv, D, D, dt)
+    ref = oracle_full(q, k, v, G=Hq // Hkv, causal=causal)
+    lens = np.asarray([max(Skv - 1 - 37 * b, 0) for b in range(B)], np.int32)
+    ref_l = oracle_full(q, k, v, G=Hq // Hkv, causal=causal, kv_lens=lens)
+    outs = []
+    for splits in (0, 1, 3, 7, 40):
+        say("f32 matrix-core split-KV: D=%d %r splits=%d" % (D, shape, splits))
+        got, info = host.sdpa(q, k, v, dt, causal=causal, num_splits=splits, impl=capi.IMPL_SPLITKV_MFMA, return_info=True)
+        assert info["impl"] == capi.IMPL_SPLITKV_MFMA
+        check(got, ref, TOL[dt], "f32 matrix-core split-KV D=%d %r splits=%d->%d" % (D, shape, splits, info["splits"]))
+        outs.append(got)
+        got = host.sdpa(q, k, v, dt, causal=causal, kv_lens=lens, num_splits=splits, impl=capi.IMPL_SPLITKV_MFMA)
+        check(got, ref_l, TOL[dt], "f32 matrix-core split-KV with key counts, splits=%d" % splits)
+    for o in outs:
+        check(o, outs[1], 2e-6, "f32 matrix-core split-KV: split-count invariance")
+    if (Hq // Hkv) * Sq <= 8:
+        check(outs[0], host.sdpa(q, k, v, dt, causal=causal, impl=capi.IMPL_SPLITKV), 2e-6, "f32 matrix-core vs vector-ALU split-KV")
+
+
+def test_decode_splitkv_matrix_cores_f32_scale_lse_auto(gpu):
+    """A negative scale, the row normalisers (one split and combined) against the generic kernel's, and AUTO's choice for
+    f32 grouped-query decode."""
+    B, Hq, Hkv, Skv, D = 2, 16, 4, 1100, 128
+    dt = capi.F32
+    q, k, v = inputs(1733, B, Hq, Hkv, 1, Skv, D, D, dt)
+    got = host.sdpa(q, k, v, dt, scale=-0.07, impl=capi.IMPL_SPLITKV_MFMA)
+    check(got, oracle_full(q, k, v, G=4, scale=-0.07), TOL[dt], "f32 matrix-core split-KV negative scale")
+    lens = np.array([1100, 0], np.int32)
+    _, lse_ref = host.sdpa(q, k, v, dt, kv_lens=lens, impl=capi.IMPL_GENERIC, return_lse=True)
+    for splits in (1, 4):
+        got, lse = host.sdpa(q, k, v, dt, kv_lens=lens, impl=capi.IMPL_SPLITKV_MFMA, num_splits=splits, return_lse=True)
+        check(got, oracle_full(q, k, v, G=4, kv_lens=lens), TOL[dt], "f32 matrix-core split-KV, an empty batch entry")
+        assert np.all(np.isneginf(lse[1])) and np.all(np.isneginf(lse_ref[1]))
+        assert np.max(np.abs(lse[0] - lse_ref[0])) < 2e-6
+    got, info = host.sdpa(q, k, v, dt, return_info=True)
+    assert info["impl"] == capi.IMPL_SPLITKV_MFMA           # 4 rows per KV head over 1100 keys, f32: AUTO's choice
+    check(got, oracle_full(q, k, v, G=4), TOL[dt], "AUTO f32 grouped-query decode")
+    _, info = host.sdpa(q[:, :4], k, v, dt, return_info=True)
+    assert info["impl"] == capi.IMPL_SPLITKV                # one row per KV head stays on the vector-ALU kernel
+
+
 def test_decode_splitkv_matrix_cores_lengths_strides_scale(gpu):
     """Key counts per batch entry (one of them 0: NaN rows, as the reference), a negative scale (the scale is applied to
     the f32 scores, so its sign does not matter to this kernel), and AUTO's choice for grouped-query decode."""
