@@ -49,8 +49,9 @@ enum {
                                       IEEE-f32 matrix instructions for f32 (dense mask allowed)                    */
     INCIN_ROCM_IMPL_SPLITKV = 3,   /* split-KV decode kernel + combine: D == Dv in {64,128}, few query rows */
     INCIN_ROCM_IMPL_MFMA64 = 4,    /* retired (a prefill kernel with 64 query rows per wavefront): refused with INCIN_ROCM_EUNSUPPORTED */
-    INCIN_ROCM_IMPL_SPLITKV_MFMA = 5 /* bf16/f16 split-KV kernel on the matrix cores + combine: D == Dv in {64,128}, Sq <= 64; the rows that
-                                      share a KV head (query heads of the group x query positions) go through it 32 at a time */
+    INCIN_ROCM_IMPL_SPLITKV_MFMA = 5 /* split-KV kernels on the matrix cores + combine: D == Dv in {64,128}, Sq <= 64; the rows that share a
+                                      KV head (query heads of the group x query positions) go through them 32 or 64 at a time (bf16/f16),
+                                      16 or 32 at a time on IEEE-f32 matrix instructions (f32) */
 };
 
 /* Thread-local message of the last failing call on this thread ("" if none).
