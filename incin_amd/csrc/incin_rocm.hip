@@ -152,8 +152,13 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
 
     const int vec = d->dtype == INCIN_ROCM_F32 ? 4 : 8;
     const int64_t R = (d->Hq / d->Hkv) * d->Sq;
-    const bool head_ok = d->D == d->Dv && (d->D == 64 || d->D == 128);
-    const bool layout_ok = head_ok && fast_layout_ok(d, vec) && d->Skv > 0;
+    // The matrix-core kernels are built for head dimensions 64 and 128; smaller ones (D and Dv need not be equal) run in
+    // the instance that holds them, padded with zeros on the way into LDS, as long as rows stay whole 16-byte vectors.
+    // The vector-ALU split-KV kernel takes the two dimensions as they are.
+    const bool head_pad_ok = d->D > 0 && d->D <= 128 && d->Dv <= 128 && d->D % vec == 0 && d->Dv % vec == 0;
+    const int64_t d_pad = std::max(d->D, d->Dv) <= 64 ? 64 : 128;
+    const bool head_exact = d->D == d->Dv && d->D == d_pad;
+    const bool layout_ok = head_pad_ok && fast_layout_ok(d, vec) && d->Skv > 0;
     const bool fast_ok = layout_ok && !d->add_mask;
     // the MFMA kernels address a K/V tile with 32-bit byte offsets from the tile's first row
     const int64_t stride_lim = d->dtype == INCIN_ROCM_F32 ? (1 << 22) : (1 << 24);
@@ -161,9 +166,9 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     // f32: the IEEE-f32 matrix-core kernel, any finite scale; f16 / bf16: the 16-bit kernels fold the scale into Q in
     // a way that needs it positive.  Both take a dense additive mask (any strides); the 64-row kernel does not.
     const bool mfma_ok = layout_ok && tile_off_ok && std::isfinite(d->scale) && (d->dtype == INCIN_ROCM_F32 || d->scale > 0.0f);
-    const bool split_ok = fast_ok && d->Sq <= 64;
+    const bool split_ok = fast_ok && head_exact && d->Sq <= 64;
     // the matrix-core split-KV kernels (16-bit and f32): blocks addressed like the prefill kernels' tiles
-    const bool split_mfma_ok = split_ok && tile_off_ok && std::isfinite(d->scale);
+    const bool split_mfma_ok = fast_ok && d->Sq <= 64 && tile_off_ok && std::isfinite(d->scale);
 
     int impl = d->impl;
     if (impl == INCIN_ROCM_IMPL_AUTO) {
@@ -180,7 +185,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         // 128 rows per KV head on).
         const int64_t esize = (int64_t)dtype_size(d->dtype);
         const int64_t kv_bytes = 2 * d->B * d->Hkv * d->Skv * d->D * esize;
-        const int64_t len128 = d->Skv * d->D * esize / 256;      // cache length in keys of 256 bytes (what the thresholds were measured in)
+        const int64_t len128 = d->Skv * d_pad * esize / 256;     // cache length in keys of 256 bytes (what the thresholds were measured in)
         // f32 (sdpa_decode_f32.hip): from two rows per KV head on, whatever the count - the f32 prefill kernel would spend a
         // 32-row matrix instruction on every query head's few rows (32 heads of a group at one position each: 8.4 ms
         // against 0.23), and where it packs as well (64 positions of one head) the split-KV form is still ahead (0.22
@@ -193,19 +198,22 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
             ((R == 1 && len128 >= 1024 && kv_bytes >= (512LL << 20)) || (R >= 2 && R <= 3 && len128 >= 512) || (R >= 4 && R <= 64)))
             impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
         else if (split_ok && R <= 8 && d->Skv >= 256) impl = INCIN_ROCM_IMPL_SPLITKV;
+        // a head dimension that is padded into its instance has no vector-ALU kernel: one row per KV head, too, goes through
+        // the matrix-core split-KV kernels
+        else if (!head_exact && split_mfma_ok && len128 >= 256 && (d->dtype == INCIN_ROCM_F32 || R <= 64)) impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
         else if (mfma_ok) impl = INCIN_ROCM_IMPL_MFMA;
         else if (split_ok && R <= 8) impl = INCIN_ROCM_IMPL_SPLITKV;
         else impl = INCIN_ROCM_IMPL_GENERIC;
     }
     if (impl == INCIN_ROCM_IMPL_MFMA && !mfma_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
-                    "scaled_dot_product_attention: the MFMA kernels need D == Dv in {64,128} and 16-byte aligned rows; for f16/bf16 also scale > 0");
+                    "scaled_dot_product_attention: the MFMA kernels need D and Dv <= 128 in whole 16-byte vectors and 16-byte aligned rows; for f16/bf16 also scale > 0");
     if (impl == INCIN_ROCM_IMPL_MFMA64)
         return fail(INCIN_ROCM_EUNSUPPORTED,
                     "scaled_dot_product_attention: the 64-row MFMA prefill kernel has been retired (INCIN_ROCM_IMPL_MFMA covers its shapes)");
     if (impl == INCIN_ROCM_IMPL_SPLITKV_MFMA && !split_mfma_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
-                    "scaled_dot_product_attention: the matrix-core split-KV kernels need D == Dv in {64,128}, Sq <= 64, no dense mask, a finite scale and 16-byte aligned rows");
+                    "scaled_dot_product_attention: the matrix-core split-KV kernels need D and Dv <= 128 in whole 16-byte vectors, Sq <= 64, no dense mask, a finite scale and 16-byte aligned rows");
     if (impl == INCIN_ROCM_IMPL_SPLITKV && !split_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
                     "scaled_dot_product_attention: the split-KV kernel needs D == Dv in {64,128}, Sq <= 64, no dense mask and 16-byte aligned rows");
@@ -235,7 +243,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         if (d->Hkv * nchunks > 65535) return fail(INCIN_ROCM_ESHAPE, "scaled_dot_product_attention: too many head groups for one launch");
         plan->splits = (int)splits;
         plan->split_len = (int)split_len;
-        plan->ws_bytes = splits > 1 ? (size_t)(d->B * d->Hq * d->Sq * splits) * (size_t)(d->Dv + 2) * sizeof(float) : 0;
+        plan->ws_bytes = splits > 1 ? (size_t)(d->B * d->Hq * d->Sq * splits) * (size_t)(d_pad + 2) * sizeof(float) : 0;
     }
     if (impl == INCIN_ROCM_IMPL_SPLITKV_MFMA) {
         // One workgroup per (batch, KV head, chunk of 32 or 64 rows, split).  A compute unit holds one at a time (its LDS
@@ -269,7 +277,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         if (d->Hkv * nchunks > 65535) return fail(INCIN_ROCM_ESHAPE, "scaled_dot_product_attention: too many head groups for one launch");
         plan->splits = (int)splits;
         plan->split_len = (int)split_len;
-        plan->ws_bytes = splits > 1 ? (size_t)(d->B * d->Hq * d->Sq * splits) * (size_t)(d->Dv + 2) * sizeof(float) : 0;
+        plan->ws_bytes = splits > 1 ? (size_t)(d->B * d->Hq * d->Sq * splits) * (size_t)(d_pad + 2) * sizeof(float) : 0;
     }
     if (impl == INCIN_ROCM_IMPL_MFMA && !d->add_mask && !d->q_lens) {
         // The prefill kernels (16-bit and f32) run one workgroup per (batch, query head, 128 rows) and a compute unit holds two:
@@ -295,7 +303,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
             if (splits > 1) {
                 plan->splits = (int)splits;
                 plan->split_len = (int)split_len;
-                plan->ws_bytes = (size_t)(d->B * d->Hq * d->Sq * splits) * (size_t)(d->Dv + 2) * sizeof(float);
+                plan->ws_bytes = (size_t)(d->B * d->Hq * d->Sq * splits) * (size_t)(d_pad + 2) * sizeof(float);
             }
         }
     }
@@ -326,6 +334,7 @@ void fill_params(const incin_rocm_sdpa_desc_t* d, const Plan& plan, SdpaParams* 
                   d->mask_stride[0] % 4 == 0 && d->mask_stride[1] % 4 == 0 && d->mask_stride[2] % 4 == 0;
     p->B = (int)d->B; p->Hq = (int)d->Hq; p->Hkv = (int)d->Hkv; p->G = (int)(d->Hq / d->Hkv);
     p->Sq = (int)d->Sq; p->Skv = (int)d->Skv; p->D = (int)d->D; p->Dv = (int)d->Dv;
+    p->Dp = std::max(d->D, d->Dv) <= 64 ? 64 : 128;      // (means something to the matrix-core and split-KV kernels only)
     p->scale = d->scale;
     p->causal = d->causal ? 1 : 0;
     p->interleave = 1;
@@ -336,7 +345,7 @@ void fill_params(const incin_rocm_sdpa_desc_t* d, const Plan& plan, SdpaParams* 
     if (!(plan.impl == INCIN_ROCM_IMPL_MFMA && d->add_mask)) p->ws_acc = (float*)d->workspace;
     if (plan.splits > 1) {
         const size_t rows = (size_t)(d->B * d->Hq * d->Sq * plan.splits);
-        p->ws_ml = (float*)d->workspace + rows * (size_t)d->Dv;
+        p->ws_ml = (float*)d->workspace + rows * (size_t)p->Dp;      // partial rows are as wide as the kernel instance
     }
 }
 

@@ -283,7 +283,7 @@ __global__ __launch_bounds__(256) void sdpa_combine_kernel(SdpaParams p)
 #pragma unroll
         for (int e = 0; e < 4; ++e) w[e] = from_f32<T>(L == 0.0f ? __builtin_nanf("") : A[e] / L);
         T* op = (T*)p.o + (int64_t)b * p.o_sb + (int64_t)hq * p.o_sh + (int64_t)i * p.o_ss;
-        *(vec4*)(op + 4 * tid) = w;
+        if (4 * tid < p.Dv) *(vec4*)(op + 4 * tid) = w;      // (the partial rows are as wide as the kernel instance, the output as V's rows)
         // the row's softmax normaliser, natural log (the maxima are in log2 units for 16-bit storage)
         if (p.lse && tid == 0) p.lse[row] = L == 0.0f ? -INFINITY : M / Softexp<T>::kPre + logf(L);
     }
@@ -299,10 +299,10 @@ static hipError_t launch_combine_t(const SdpaParams& p, hipStream_t stream)
     return hipGetLastError();
 }
 
-// The partial results of a split-KV launch (D == Dv in {64, 128}) into the output.
+// The partial results of a split-KV launch (rows of p.Dp floats, 64 or 128) into the output.
 hipError_t launch_sdpa_combine(const SdpaParams& p, int dtype, hipStream_t stream)
 {
-    if (p.D == 128) {
+    if (p.Dp == 128) {
         switch (dtype) {
             case 0: return launch_combine_t<float, 128>(p, stream);
             case 1: return launch_combine_t<f16_t, 128>(p, stream);

@@ -107,8 +107,8 @@ __global__ __launch_bounds__(256) void sdpa_decode_f32_kernel(SdpaParams p)
     for (int c = 0; c < CPB; ++c) {
         const int pos = c * 64 + lane;
         const int r = pos / L::CPR, slot = pos % L::CPR;
-        k_voff[c] = r * (int)p.k_ss * 4 + (slot ^ L::f(r)) * 16;
-        v_voff[c] = r * (int)p.v_ss * 4 + (slot ^ L::f(r)) * 16;
+        k_voff[c] = dma_chunk_offset(r, (int)p.k_ss * 4, slot ^ L::f(r), p.D * 4);
+        v_voff[c] = dma_chunk_offset(r, (int)p.v_ss * 4, slot ^ L::f(r), p.Dv * 4);
     }
     const float* kp = (const float*)p.k + (int64_t)b * p.k_sb + (int64_t)hkv * p.k_sh;
     const float* vp = (const float*)p.v + (int64_t)b * p.v_sb + (int64_t)hkv * p.v_sh;
@@ -119,8 +119,8 @@ __global__ __launch_bounds__(256) void sdpa_decode_f32_kernel(SdpaParams p)
     const int first_key = k_begin + wave * BLOCK;
     const char* k_next = (const char*)kp + (int64_t)first_key * p.k_ss * 4;
     const char* v_next = (const char*)vp + (int64_t)first_key * p.v_ss * 4;
-    int64_t k_rem = (int64_t)(k_end - first_key - 1) * p.k_ss * 4 + D * 4;
-    int64_t v_rem = (int64_t)(k_end - first_key - 1) * p.v_ss * 4 + D * 4;
+    int64_t k_rem = (int64_t)(k_end - first_key - 1) * p.k_ss * 4 + p.D * 4;
+    int64_t v_rem = (int64_t)(k_end - first_key - 1) * p.v_ss * 4 + p.Dv * 4;
     // bytes a descriptor may cover: none once the tensor's blocks are used up, 2^31 - 1 at most
     auto clamp31 = [](int64_t x) __attribute__((always_inline)) {
         const unsigned hi = (unsigned)((unsigned long long)x >> 32), lo = (unsigned)x;
@@ -164,9 +164,10 @@ __global__ __launch_bounds__(256) void sdpa_decode_f32_kernel(SdpaParams p)
             const float* qrow = (const float*)p.q + (int64_t)b * p.q_sb + (int64_t)hq[rb] * p.q_sh + (int64_t)qi[rb] * p.q_ss + g * 4;
 #pragma unroll
             for (int j = 0; j < NJ; ++j) {
-                qreg[rb][j] = *(const floatx4*)(qrow + j * 16);
+                const bool in = valid[rb] && j * 16 + g * 4 < p.D;      // (rows that do not exist, and beyond the head dimension: zeros, like K's)
+                if (j * 16 + g * 4 < p.D) qreg[rb][j] = *(const floatx4*)(qrow + j * 16);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) qreg[rb][j][e] = valid[rb] ? qreg[rb][j][e] * c2 : 0.0f;
+                for (int e = 0; e < 4; ++e) qreg[rb][j][e] = in ? qreg[rb][j][e] * c2 : 0.0f;
             }
         }
     }
@@ -363,7 +364,7 @@ __global__ __launch_bounds__(256) void sdpa_decode_f32_kernel(SdpaParams p)
                 float* orow = (float*)p.o + (int64_t)b * p.o_sb + (int64_t)hq[rb] * p.o_sh + (int64_t)qi[rb] * p.o_ss;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) o[r] *= inv;
-                *(floatx4*)(orow + 16 * db + 4 * g) = o;
+                if (16 * db + 4 * g < p.Dv) *(floatx4*)(orow + 16 * db + 4 * g) = o;
             } else {
                 *(floatx4*)(p.ws_acc + slot * D + 16 * db + 4 * g) = o;
             }
@@ -424,7 +425,7 @@ static hipError_t launch_decode_f32_d(const SdpaParams& p, bool two_slots, hipSt
 // chooses them for short splits.
 hipError_t launch_sdpa_decode_f32(const SdpaParams& p, bool two_slots, hipStream_t stream)
 {
-    hipError_t e = p.D == 128 ? launch_decode_f32_d<128>(p, two_slots, stream) : launch_decode_f32_d<64>(p, two_slots, stream);
+    hipError_t e = p.Dp == 128 ? launch_decode_f32_d<128>(p, two_slots, stream) : launch_decode_f32_d<64>(p, two_slots, stream);
     if (e != hipSuccess || p.num_splits == 1) return e;
     return launch_sdpa_combine(p, 0, stream);
 }

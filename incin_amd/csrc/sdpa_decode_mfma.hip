@@ -89,8 +89,8 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
     for (int c = 0; c < CPB; ++c) {
         const int pos = c * 64 + lane;
         const int r = pos / L::CPR, slot = pos % L::CPR;
-        k_voff[c] = r * (int)p.k_ss * 2 + (slot ^ L::fk(r)) * 16;
-        v_voff[c] = r * (int)p.v_ss * 2 + (slot ^ L::fv(r)) * 16;
+        k_voff[c] = dma_chunk_offset(r, (int)p.k_ss * 2, slot ^ L::fk(r), p.D * 2);
+        v_voff[c] = dma_chunk_offset(r, (int)p.v_ss * 2, slot ^ L::fv(r), p.Dv * 2);
     }
     const T* kp = (const T*)p.k + (int64_t)b * p.k_sb + (int64_t)hkv * p.k_sh;
     const T* vp = (const T*)p.v + (int64_t)b * p.v_sb + (int64_t)hkv * p.v_sh;
@@ -101,8 +101,8 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
     const int first_key = k_begin + wave * BLOCK;
     const char* k_next = (const char*)kp + (int64_t)first_key * p.k_ss * 2;
     const char* v_next = (const char*)vp + (int64_t)first_key * p.v_ss * 2;
-    int64_t k_rem = (int64_t)(k_end - first_key - 1) * p.k_ss * 2 + D * 2;
-    int64_t v_rem = (int64_t)(k_end - first_key - 1) * p.v_ss * 2 + D * 2;
+    int64_t k_rem = (int64_t)(k_end - first_key - 1) * p.k_ss * 2 + p.D * 2;
+    int64_t v_rem = (int64_t)(k_end - first_key - 1) * p.v_ss * 2 + p.Dv * 2;
     // bytes a descriptor may cover: none once the tensor's blocks are used up, 2^31 - 1 at most
     auto clamp31 = [](int64_t x) __attribute__((always_inline)) {
         const unsigned hi = (unsigned)((unsigned long long)x >> 32), lo = (unsigned)x;
@@ -144,8 +144,8 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
         const T* qrow = (const T*)p.q + (int64_t)b * p.q_sb + (int64_t)hq[rb] * p.q_sh + (int64_t)qi[rb] * p.q_ss + g * 8;
 #pragma unroll
         for (int s = 0; s < NSTEP; ++s) {
-            qreg[rb][s] = *(const vec8*)(qrow + s * 16);
-            if (!valid[rb])
+            if (s * 16 + g * 8 < p.D) qreg[rb][s] = *(const vec8*)(qrow + s * 16);
+            if (!valid[rb] || s * 16 + g * 8 >= p.D)      // (rows that do not exist, and beyond the head dimension: zeros, like K's)
 #pragma unroll
                 for (int e = 0; e < 8; ++e) qreg[rb][s][e] = (T)0.0f;
         }
@@ -330,7 +330,7 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
                 vec4 w;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) w[e] = (T)(o[r4 * 4 + e] * inv);
-                *(vec4*)(orow + r4 * 8) = w;
+                if (32 * wave + 4 * g + r4 * 8 < p.Dv) *(vec4*)(orow + r4 * 8) = w;
             }
             if (p.lse && wave == 0 && g == 0)       // the row's softmax normaliser, natural log (M and the sum are in log2 units)
                 p.lse[((int64_t)b * p.Hq + hq[rb]) * Sq + qi[rb]] = l_tot == 0.0f ? -INFINITY : (M[rb] + __builtin_log2f(l_tot)) * 0.6931471805599453f;
@@ -422,7 +422,7 @@ hipError_t launch_sdpa_decode_mfma(const SdpaParams& p, int dtype, hipStream_t s
 {
     if (dtype == 0) return launch_sdpa_decode_f32(p, decode_two_slots(p, 0), stream);
     hipError_t e;
-    if (p.D == 128) e = dtype == 1 ? launch_decode_mfma_d<f16_t, 128>(p, stream) : launch_decode_mfma_d<bf16_t, 128>(p, stream);
+    if (p.Dp == 128) e = dtype == 1 ? launch_decode_mfma_d<f16_t, 128>(p, stream) : launch_decode_mfma_d<bf16_t, 128>(p, stream);
     else e = dtype == 1 ? launch_decode_mfma_d<f16_t, 64>(p, stream) : launch_decode_mfma_d<bf16_t, 64>(p, stream);
     if (e != hipSuccess || p.num_splits == 1) return e;
     return launch_sdpa_combine(p, dtype, stream);

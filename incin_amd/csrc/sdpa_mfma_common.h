@@ -109,6 +109,14 @@ __device__ __forceinline__ void dma_copy16(uint4v desc, unsigned lds_addr, int b
     // (one wait state between the write of m0 and the copy that reads it)
     asm volatile("s_nop 0\n\tbuffer_load_dwordx4 %0, %1, 0 offen lds" ::"v"(byte_offset), "s"(desc), "{m0}"(lds_addr) : "memory");
 }
+// Offset for the lane of such a copy that fetches 16-byte chunk `chunk` of row `row` (rows `row_bytes` apart in memory,
+// `data_bytes` of data each): a chunk at or beyond the row's data gets an offset that no descriptor covers, so that lane
+// delivers zeros.  This is how a head dimension below the one a kernel instance is built for is padded: with zeros, on
+// the way into LDS, without touching the operands in memory.
+__device__ __forceinline__ int dma_chunk_offset(int row, int row_bytes, int chunk, int data_bytes)
+{
+    return chunk * 16 < data_bytes ? row * row_bytes + chunk * 16 : 0x7fffffff;
+}
 // The same for 64 lanes x 4 bytes (256 bytes of LDS).
 __device__ __forceinline__ void dma_copy4(uint4v desc, unsigned lds_addr, int byte_offset)
 {

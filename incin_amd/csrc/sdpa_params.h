@@ -22,6 +22,7 @@ struct SdpaParams {
     int64_t m_sb, m_sh, m_si, m_sj;
     int32_t B, Hq, Hkv, G;     // G = Hq / Hkv
     int32_t Sq, Skv, D, Dv;
+    int32_t Dp;                // matrix-core kernels: the head dimension their instance is built for (64 or 128); D and Dv fit in it, zero-padded
     float scale;
     int32_t causal;
     int32_t interleave;        // MFMA prefill kernels: (batch, KV head) pairs per group of the work list, set by their launchers

@@ -101,14 +101,14 @@ void sdpa_prefill_f32_kernel(SdpaParams p)
     for (int c = 0; c < LPW; ++c) {
         const int pos = (wave * LPW + c) * 64 + lane;
         const int row = pos / L::CPR, slot = pos % L::CPR;
-        k_voff[c] = row * (int)p.k_ss * 4 + (slot ^ L::f(row)) * 16;
-        v_voff[c] = row * (int)p.v_ss * 4 + (slot ^ L::f(row)) * 16;
+        k_voff[c] = dma_chunk_offset(row, (int)p.k_ss * 4, slot ^ L::f(row), p.D * 4);
+        v_voff[c] = dma_chunk_offset(row, (int)p.v_ss * 4, slot ^ L::f(row), p.Dv * 4);
     }
     const int64_t k_tile_bytes = (int64_t)KT * p.k_ss * 4, v_tile_bytes = (int64_t)KT * p.v_ss * 4;
-    auto issue = [&](const float* base, int64_t tile_bytes, int64_t row_stride, int t, int buf, const int (&voff)[LPW]) __attribute__((always_inline)) {
+    auto issue = [&](const float* base, int64_t tile_bytes, int64_t row_stride, int row_floats, int t, int buf, const int (&voff)[LPW]) __attribute__((always_inline)) {
         // bytes to the end of the last row this workgroup may see: loads past that return 0 (rows past a batch
         // entry's key count are never read)
-        int64_t rem = (int64_t)(j_end - t * KT - 1) * row_stride * 4 + D * 4;
+        int64_t rem = (int64_t)(j_end - t * KT - 1) * row_stride * 4 + row_floats * 4;
         if (rem > 0x7fffffffLL) rem = 0x7fffffffLL;
         const uint4v r = dma_descriptor((const char*)base + t * tile_bytes, (int)rem);
         const unsigned dst = lds_address(smem) + buf * L::TILE_BYTES + wave * LPW * 1024;
@@ -116,8 +116,8 @@ void sdpa_prefill_f32_kernel(SdpaParams p)
         for (int c = 0; c < LPW; ++c) dma_copy16(r, dst + c * 1024, voff[c]);
     };
     auto issue_kv = [&](int t) __attribute__((always_inline)) {
-        issue(kp, k_tile_bytes, p.k_ss, t, t & 1, k_voff);
-        issue(vp, v_tile_bytes, p.v_ss, t, 2 + (t & 1), v_voff);
+        issue(kp, k_tile_bytes, p.k_ss, p.D, t, t & 1, k_voff);
+        issue(vp, v_tile_bytes, p.v_ss, p.Dv, t, 2 + (t & 1), v_voff);
     };
 
     // ---- LDS read addresses (bytes inside a tile buffer), kept to a few registers: the rest is one vector
@@ -144,9 +144,10 @@ void sdpa_prefill_f32_kernel(SdpaParams p)
         const float c2 = p.scale * 1.4426950408889634f;      // scores in log2 units
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
-            qreg[j] = *(const float4v*)(qrow + j * 8);
+            const bool in = j * 8 + g * 4 < p.D;      // (beyond the head dimension: zeros, like K's)
+            if (in) qreg[j] = *(const float4v*)(qrow + j * 8);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) qreg[j][e] *= c2;
+            for (int e = 0; e < 4; ++e) qreg[j][e] = in ? qreg[j][e] * c2 : 0.0f;
         }
     }
     const float* mrow = nullptr;          // this lane's row of the dense mask
@@ -288,7 +289,7 @@ void sdpa_prefill_f32_kernel(SdpaParams p)
                 float4v w;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) w[e] = o_acc[db][r4 * 4 + e] * inv;
-                *(float4v*)(orow + db * 32 + r4 * 8 + g * 4) = w;
+                if (db * 32 + r4 * 8 + g * 4 < p.Dv) *(float4v*)(orow + db * 32 + r4 * 8 + g * 4) = w;
             }
     }
 #endif
@@ -321,8 +322,8 @@ static hipError_t launch_prefill_f32_t(const SdpaParams& p0, hipStream_t stream)
 // strides below 2^24 elements (tile offsets fit the 32-bit buffer offset); the dense mask, if any, has any strides.
 hipError_t launch_sdpa_prefill_f32(const SdpaParams& p, hipStream_t stream)
 {
-    if (p.mask) return p.D == 128 ? launch_prefill_f32_t<128, true>(p, stream) : launch_prefill_f32_t<64, true>(p, stream);
-    return p.D == 128 ? launch_prefill_f32_t<128, false>(p, stream) : launch_prefill_f32_t<64, false>(p, stream);
+    if (p.mask) return p.Dp == 128 ? launch_prefill_f32_t<128, true>(p, stream) : launch_prefill_f32_t<64, true>(p, stream);
+    return p.Dp == 128 ? launch_prefill_f32_t<128, false>(p, stream) : launch_prefill_f32_t<64, false>(p, stream);
 }
 
 }  // namespace incin_rocm

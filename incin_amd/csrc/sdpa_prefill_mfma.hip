@@ -205,8 +205,8 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     for (int c = 0; c < LPW; ++c) {
         const int pos = (wave * LPW + c) * 64 + lane;
         const int row = pos / L::CPR, slot = pos % L::CPR;
-        k_voff[c] = row * (int)p.k_ss * 2 + (slot ^ L::fk(row)) * 16;
-        v_voff[c] = row * (int)p.v_ss * 2 + (slot ^ L::fv(row)) * 16;
+        k_voff[c] = dma_chunk_offset(row, (int)p.k_ss * 2, slot ^ L::fk(row), p.D * 2);
+        v_voff[c] = dma_chunk_offset(row, (int)p.v_ss * 2, slot ^ L::fv(row), p.Dv * 2);
     }
     const int64_t k_tile_bytes = (int64_t)PF_BN * p.k_ss * 2, v_tile_bytes = (int64_t)PF_BN * p.v_ss * 2;
     // K buffer b at smem + b*TILE, V buffer b at smem + (2+b)*TILE.  Tiles are copied in order from tile t_first on, so
@@ -214,8 +214,8 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     // workgroup may see (loads past that return 0; rows past a batch entry's key count are never read).
     const char* k_next = (const char*)kp + t_first * k_tile_bytes;
     const char* v_next = (const char*)vp + t_first * v_tile_bytes;
-    int64_t k_rem = (int64_t)(j_end - t_first * PF_BN - 1) * p.k_ss * 2 + D * 2;
-    int64_t v_rem = (int64_t)(j_end - t_first * PF_BN - 1) * p.v_ss * 2 + D * 2;
+    int64_t k_rem = (int64_t)(j_end - t_first * PF_BN - 1) * p.k_ss * 2 + p.D * 2;
+    int64_t v_rem = (int64_t)(j_end - t_first * PF_BN - 1) * p.v_ss * 2 + p.Dv * 2;
     auto clamp31 = [](int64_t x) __attribute__((always_inline)) {
         const unsigned hi = (unsigned)((unsigned long long)x >> 32), lo = (unsigned)x;
         return (hi | (lo >> 31)) != 0 ? 0x7fffffff : (int)lo;
@@ -275,7 +275,12 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
         const int qi = min(my_i, Sq - 1);
         const T* qrow = qp + (int64_t)qi * p.q_ss + g * 8;
 #pragma unroll
-        for (int s = 0; s < NSTEP; ++s) qreg[s] = *(const vec8*)(qrow + s * 16);
+        for (int s = 0; s < NSTEP; ++s) {
+            if (s * 16 + g * 8 < p.D) qreg[s] = *(const vec8*)(qrow + s * 16);      // (beyond the head dimension: zeros, like K's)
+            else
+#pragma unroll
+                for (int e = 0; e < 8; ++e) qreg[s][e] = (T)0.0f;
+        }
     }
     // Fold scale * log2(e) into Q once (rounded back to the storage type): the matrix product then
     // yields the scores directly in the log2 units the softmax works in.
@@ -789,7 +794,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
                 vec4 w;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) w[e] = (T)(o_acc[db][r4 * 4 + e] * inv);
-                *(vec4*)(orow + db * 32 + r4 * 8 + g * 4) = w;
+                if (db * 32 + r4 * 8 + g * 4 < p.Dv) *(vec4*)(orow + db * 32 + r4 * 8 + g * 4) = w;
             }
     }
 #endif
@@ -841,11 +846,11 @@ static hipError_t launch_prefill_t(const SdpaParams& p, hipStream_t stream)
 hipError_t launch_sdpa_prefill_mfma(const SdpaParams& p, int dtype, hipStream_t stream)
 {
     if (p.mask) {
-        if (dtype == 1) return p.D == 128 ? launch_prefill_t<f16_t, 128, true>(p, stream) : launch_prefill_t<f16_t, 64, true>(p, stream);
-        return p.D == 128 ? launch_prefill_t<bf16_t, 128, true>(p, stream) : launch_prefill_t<bf16_t, 64, true>(p, stream);
+        if (dtype == 1) return p.Dp == 128 ? launch_prefill_t<f16_t, 128, true>(p, stream) : launch_prefill_t<f16_t, 64, true>(p, stream);
+        return p.Dp == 128 ? launch_prefill_t<bf16_t, 128, true>(p, stream) : launch_prefill_t<bf16_t, 64, true>(p, stream);
     }
-    if (dtype == 1) return p.D == 128 ? launch_prefill_t<f16_t, 128, false>(p, stream) : launch_prefill_t<f16_t, 64, false>(p, stream);
-    return p.D == 128 ? launch_prefill_t<bf16_t, 128, false>(p, stream) : launch_prefill_t<bf16_t, 64, false>(p, stream);
+    if (dtype == 1) return p.Dp == 128 ? launch_prefill_t<f16_t, 128, false>(p, stream) : launch_prefill_t<f16_t, 64, false>(p, stream);
+    return p.Dp == 128 ? launch_prefill_t<bf16_t, 128, false>(p, stream) : launch_prefill_t<bf16_t, 64, false>(p, stream);
 }
 
 }  // namespace incin_rocm

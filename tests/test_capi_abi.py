@@ -58,11 +58,25 @@ def test_dispatch_choices():
     assert _plan(_desc())[2] == capi.IMPL_MFMA
     assert _plan(_desc(dtype=capi.F32))[2] == capi.IMPL_MFMA                  # the IEEE-f32 matrix-core kernel
     assert _plan(_desc(dtype=capi.F32, add_mask=0x20000))[2] == capi.IMPL_MFMA  # which also takes a dense mask
-    assert _plan(_desc(dtype=capi.F32, D=80, Dv=80))[2] == capi.IMPL_GENERIC
-    assert _plan(_desc(D=80, Dv=80))[2] == capi.IMPL_GENERIC
+    # head dimensions up to 128 in whole 16-byte vectors (D and Dv need not be equal) run padded in the matrix-core kernels
+    assert _plan(_desc(dtype=capi.F32, D=80, Dv=80))[2] == capi.IMPL_MFMA
+    assert _plan(_desc(D=80, Dv=80))[2] == capi.IMPL_MFMA
+    assert _plan(_desc(D=128, Dv=64))[2] == capi.IMPL_MFMA
+    assert _plan(_desc(D=8, Dv=40))[2] == capi.IMPL_MFMA
+    assert _plan(_desc(D=84, Dv=84))[2] == capi.IMPL_GENERIC                    # 168-byte rows: not whole vectors
+    assert _plan(_desc(dtype=capi.F32, D=84, Dv=84))[2] == capi.IMPL_MFMA       # in f32 they are
+    assert _plan(_desc(D=160, Dv=160))[2] == capi.IMPL_GENERIC
+    assert _plan(_desc(D=128, Dv=136))[2] == capi.IMPL_GENERIC
+    # decode over such a cache: the matrix-core split-KV kernels, also at one row per KV head (no vector-ALU kernel there);
+    # partial rows are as wide as the kernel instance
+    nbytes, splits, impl = _plan(_desc(Sq=1, Skv=8192, B=2, Hq=8, Hkv=8, D=96, Dv=96, num_splits=4))
+    assert impl == capi.IMPL_SPLITKV_MFMA and splits == 4 and nbytes == 2 * 8 * 4 * 130 * 4
+    nbytes, splits, impl = _plan(_desc(Sq=1, Skv=8192, B=2, Hq=8, Hkv=2, D=48, Dv=32, num_splits=4, dtype=capi.F32))
+    assert impl == capi.IMPL_SPLITKV_MFMA and splits == 4 and nbytes == 2 * 8 * 4 * 66 * 4
     nbytes, _, impl = _plan(_desc(add_mask=0x20000))                            # dense mask: still the matrix cores,
     assert impl == capi.IMPL_MFMA and nbytes == 256                           # with 2 x 4 x 4 x 4 block flags (rounded up)
-    assert _plan(_desc(add_mask=0x20000, D=80, Dv=80))[2] == capi.IMPL_GENERIC
+    assert _plan(_desc(add_mask=0x20000, D=80, Dv=80))[2] == capi.IMPL_MFMA
+    assert _plan(_desc(add_mask=0x20000, D=160, Dv=160))[2] == capi.IMPL_GENERIC
     nbytes, splits, impl = _plan(_desc(Sq=1, Skv=8192, B=32, Hq=32, Hkv=32))
     assert impl == capi.IMPL_SPLITKV_MFMA and splits == 1 and nbytes == 0      # 1024 workgroups, four rounds of 256
     nbytes, splits, impl = _plan(_desc(Sq=1, Skv=2048, B=8, Hq=32, Hkv=32))
@@ -140,10 +154,12 @@ def test_dispatch_choices():
     (dict(impl=9), capi.EINVAL),
     (dict(num_splits=-2), capi.EINVAL),
     (dict(impl=capi.IMPL_MFMA64), capi.EUNSUPPORTED),                 # retired: the value is refused
-    (dict(impl=capi.IMPL_MFMA, D=80, Dv=80), capi.EUNSUPPORTED),
+    (dict(impl=capi.IMPL_MFMA, D=160, Dv=160), capi.EUNSUPPORTED),
+    (dict(impl=capi.IMPL_MFMA, D=84, Dv=84), capi.EUNSUPPORTED),
+    (dict(impl=capi.IMPL_SPLITKV, Sq=1, D=96, Dv=96), capi.EUNSUPPORTED),             # the vector-ALU kernel takes 64 and 128 only
     (dict(impl=capi.IMPL_SPLITKV, Sq=4096), capi.EUNSUPPORTED),
     (dict(impl=capi.IMPL_SPLITKV_MFMA, Sq=4096), capi.EUNSUPPORTED),
-    (dict(impl=capi.IMPL_SPLITKV_MFMA, Sq=1, D=32, Dv=32), capi.EUNSUPPORTED),
+    (dict(impl=capi.IMPL_SPLITKV_MFMA, Sq=1, D=36, Dv=36), capi.EUNSUPPORTED),
     (dict(impl=capi.IMPL_SPLITKV_MFMA, Sq=1, add_mask=0x20000), capi.EUNSUPPORTED),
     (dict(D=512, Dv=512), capi.EUNSUPPORTED),
     (dict(B=70000), capi.ESHAPE),

@@ -572,6 +572,65 @@ def test_decode_splitkv_matrix_cores_f32_scale_lse_auto(gpu):
     assert info["impl"] == capi.IMPL_SPLITKV                # one row per KV head stays on the vector-ALU kernel
 
 
+HEAD_DIMS_16 = [(96, 96), (80, 80), (40, 40), (8, 8), (112, 72), (128, 64), (64, 128), (32, 16), (120, 128)]
+HEAD_DIMS_F32 = [(96, 96), (20, 20), (4, 4), (100, 36), (128, 64), (60, 128)]
+
+
+@pytest.mark.parametrize("dtype,dims", [(dt, dd) for dt in (capi.BF16, capi.F16) for dd in HEAD_DIMS_16] +
+                         [(capi.F32, dd) for dd in HEAD_DIMS_F32],
+                         ids=lambda x: dtypes.NAMES[x] if isinstance(x, int) else "D%d_Dv%d" % x)
+def test_head_dimensions_padded_into_the_matrix_core_kernels(gpu, dtype, dims):
+    """Head dimensions up to 128 in whole 16-byte vectors, D and Dv not necessarily equal, run in the matrix-core kernels'
+    64 or 128 instance (zeros on the way into LDS, stores cut at Dv): prefill with a causal mask, with key counts and with
+    a dense mask, a chunk with the keys split, decode (one and several rows per KV head) through the split-KV kernels,
+    row normalisers - each against the oracle, and AUTO must pick those kernels."""
+    D, Dv = dims
+    tol = TOL[dtype]
+    # prefill, grouped queries, causal with S_q < S_kv, key counts
+    B, Hq, Hkv, Sq, Skv = 2, 4, 2, 200, 333
+    q, k, v = inputs(2100 + D + 3 * Dv, B, Hq, Hkv, Sq, Skv, D, Dv, dtype)
+    lens = np.array([333, 97], np.int32)
+    say("padded head dimensions: %s D=%d Dv=%d prefill" % (dtypes.NAMES[dtype], D, Dv))
+    got, lse, info = host.sdpa(q, k, v, dtype, causal=True, kv_lens=lens, return_info=True, return_lse=True)
+    assert info["impl"] == capi.IMPL_MFMA
+    check(got, oracle_full(q, k, v, G=2, causal=True, kv_lens=lens), tol, "prefill D=%d Dv=%d" % (D, Dv))
+    _, lse_g = host.sdpa(q, k, v, dtype, causal=True, kv_lens=lens, impl=capi.IMPL_GENERIC, return_lse=True)
+    assert np.max(np.abs(lse - lse_g)) < (2e-5 if dtype == capi.F32 else 2e-2)
+    # a dense additive mask (values and hidden blocks)
+    r = rng(5)
+    m = (r.standard_normal((1, 1, Sq, Skv)) * 0.5).astype(np.float32)
+    m[..., 64:160, 32:128] = -np.inf
+    m = dtypes.round_to(m, dtype)
+    got, info = host.sdpa(q, k, v, dtype, mask=m, return_info=True)
+    assert info["impl"] == capi.IMPL_MFMA
+    check(got, oracle_full(q, k, v, G=2, mask=m), tol, "dense mask D=%d Dv=%d" % (D, Dv))
+    # a chunk of a long prompt: the library splits the keys, the combine pass cuts the partial rows at Dv
+    q2, k2, v2 = inputs(2200 + D, 1, 4, 4, 128, 8192, D, Dv, dtype)
+    got, info = host.sdpa(q2, k2, v2, dtype, causal=True, return_info=True)
+    assert info["impl"] == capi.IMPL_MFMA and info["splits"] > 1
+    check(got, oracle_full(q2, k2, v2, causal=True), tol, "prefill with the keys split, D=%d Dv=%d" % (D, Dv))
+    # decode: one row per KV head and a short causal run of a group's heads, split counts chosen and forced
+    for Hq3, Sq3 in ((2, 1), (8, 3)):
+        q3, k3, v3 = inputs(2300 + D + Hq3, 2, Hq3, 2, Sq3, 1500, D, Dv, dtype)
+        ref = oracle_full(q3, k3, v3, G=Hq3 // 2, causal=True)
+        for splits in (0, 1, 5):
+            say("padded head dimensions: decode Hq=%d Sq=%d splits=%d" % (Hq3, Sq3, splits))
+            got, lse, info = host.sdpa(q3, k3, v3, dtype, causal=True, num_splits=splits, return_info=True, return_lse=True)
+            assert info["impl"] == capi.IMPL_SPLITKV_MFMA
+            check(got, ref, tol, "decode D=%d Dv=%d rows=%d splits=%d" % (D, Dv, Hq3 // 2 * Sq3, splits))
+        _, lse_g = host.sdpa(q3, k3, v3, dtype, causal=True, impl=capi.IMPL_GENERIC, return_lse=True)
+        assert np.max(np.abs(lse - lse_g)) < (2e-5 if dtype == capi.F32 else 2e-2)
+
+
+def test_head_dimensions_outside_the_matrix_core_kernels(gpu):
+    """Rows that are not whole 16-byte vectors, and head dimensions above 128, stay on the generic kernel."""
+    for dtype, D in ((capi.BF16, 20), (capi.F32, 6), (capi.BF16, 160), (capi.F32, 136)):
+        q, k, v = inputs(2400 + D, 1, 2, 2, 40, 70, D, D, dtype)
+        got, info = host.sdpa(q, k, v, dtype, causal=True, return_info=True)
+        assert info["impl"] == capi.IMPL_GENERIC
+        check(got, oracle_full(q, k, v, causal=True), TOL[dtype], "generic D=%d" % D)
+
+
 def test_decode_splitkv_matrix_cores_lengths_strides_scale(gpu):
     """Key counts per batch entry (one of them 0: NaN rows, as the reference), a negative scale (the scale is applied to
     the f32 scores, so its sign does not matter to this kernel), and AUTO's choice for grouped-query decode."""
