@@ -27,8 +27,8 @@ hipError_t launch_mask_classify(const SdpaParams& p, int dtype, hipStream_t stre
 hipError_t launch_sdpa_decode(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_sdpa_decode_mfma(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_read_rate(const void* src, void* sink, size_t bytes, int nontemporal, hipStream_t stream);
-int decode_mfma_chunk_rows(int R, int dtype);
-int decode_mfma_workgroups_per_cu(int chunk_rows, int64_t split_len, int dtype);
+int decode_mfma_chunk_rows(int R, int dtype, int d_pad);
+int decode_mfma_workgroups_per_cu(int chunk_rows, int64_t split_len, int dtype, int d_pad);
 int decode_keys_per_tile(int dtype, int D, int R);
 }  // namespace incin_rocm
 
@@ -154,10 +154,13 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     const int64_t R = (d->Hq / d->Hkv) * d->Sq;
     // The matrix-core kernels are built for head dimensions 64 and 128; smaller ones (D and Dv need not be equal) run in
     // the instance that holds them, padded with zeros on the way into LDS, as long as rows stay whole 16-byte vectors.
-    // The vector-ALU split-KV kernel takes the two dimensions as they are.
-    const bool head_pad_ok = d->D > 0 && d->D <= 128 && d->Dv <= 128 && d->D % vec == 0 && d->Dv % vec == 0;
-    const int64_t d_pad = std::max(d->D, d->Dv) <= 64 ? 64 : 128;
-    const bool head_exact = d->D == d->Dv && d->D == d_pad;
+    // The 16-bit split-KV kernel has an instance for 256 as well, which takes every launch with a head dimension above
+    // 128 - prefill shapes too, 32 rows per workgroup.  The vector-ALU split-KV kernel takes the two dimensions as they are.
+    const int64_t d_max = std::max(d->D, d->Dv);
+    const int64_t d_pad = d_max <= 64 ? 64 : d_max <= 128 ? 128 : 256;
+    const bool wide = d_pad == 256;
+    const bool head_pad_ok = d->D > 0 && d_max <= (d->dtype == INCIN_ROCM_F32 ? 128 : 256) && d->D % vec == 0 && d->Dv % vec == 0;
+    const bool head_exact = d->D == d->Dv && d->D == d_pad && !wide;
     const bool layout_ok = head_pad_ok && fast_layout_ok(d, vec) && d->Skv > 0;
     const bool fast_ok = layout_ok && !d->add_mask;
     // the MFMA kernels address a K/V tile with 32-bit byte offsets from the tile's first row
@@ -165,10 +168,10 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     const bool tile_off_ok = d->k_stride[2] >= 0 && d->v_stride[2] >= 0 && d->k_stride[2] < stride_lim && d->v_stride[2] < stride_lim;
     // f32: the IEEE-f32 matrix-core kernel, any finite scale; f16 / bf16: the 16-bit kernels fold the scale into Q in
     // a way that needs it positive.  Both take a dense additive mask (any strides); the 64-row kernel does not.
-    const bool mfma_ok = layout_ok && tile_off_ok && std::isfinite(d->scale) && (d->dtype == INCIN_ROCM_F32 || d->scale > 0.0f);
+    const bool mfma_ok = layout_ok && !wide && tile_off_ok && std::isfinite(d->scale) && (d->dtype == INCIN_ROCM_F32 || d->scale > 0.0f);
     const bool split_ok = fast_ok && head_exact && d->Sq <= 64;
     // the matrix-core split-KV kernels (16-bit and f32): blocks addressed like the prefill kernels' tiles
-    const bool split_mfma_ok = fast_ok && d->Sq <= 64 && tile_off_ok && std::isfinite(d->scale);
+    const bool split_mfma_ok = fast_ok && (d->Sq <= 64 || wide) && tile_off_ok && std::isfinite(d->scale);
 
     int impl = d->impl;
     if (impl == INCIN_ROCM_IMPL_AUTO) {
@@ -192,7 +195,8 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         // against 0.28 ms on 8 x 8 heads x 8192 keys); the vector-ALU kernel is level at 2 rows and behind from 4 on
         // (4 rows, 268 MB of cache: 5.6 against 4.8 TB/s; 8 rows: 6.6 against 3.4).  More than 32 rows over fewer than 512
         // keys stay with the prefill kernel (64 positions x 16 heads x 64 sequences of 256 keys: 0.14 against 0.17 ms).
-        if (d->dtype == INCIN_ROCM_F32 && split_mfma_ok && len128 >= 256 && R >= 2 && (R <= 32 || d->Skv >= 512))
+        if (wide && split_mfma_ok) impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
+        else if (d->dtype == INCIN_ROCM_F32 && split_mfma_ok && len128 >= 256 && R >= 2 && (R <= 32 || d->Skv >= 512))
             impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
         else if (d->dtype != INCIN_ROCM_F32 && split_mfma_ok && len128 >= 256 &&
             ((R == 1 && len128 >= 1024 && kv_bytes >= (512LL << 20)) || (R >= 2 && R <= 3 && len128 >= 512) || (R >= 4 && R <= 64)))
@@ -207,13 +211,13 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     }
     if (impl == INCIN_ROCM_IMPL_MFMA && !mfma_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
-                    "scaled_dot_product_attention: the MFMA kernels need D and Dv <= 128 in whole 16-byte vectors and 16-byte aligned rows; for f16/bf16 also scale > 0");
+                    "scaled_dot_product_attention: the MFMA prefill kernels need D and Dv <= 128 in whole 16-byte vectors and 16-byte aligned rows; for f16/bf16 also scale > 0");
     if (impl == INCIN_ROCM_IMPL_MFMA64)
         return fail(INCIN_ROCM_EUNSUPPORTED,
                     "scaled_dot_product_attention: the 64-row MFMA prefill kernel has been retired (INCIN_ROCM_IMPL_MFMA covers its shapes)");
     if (impl == INCIN_ROCM_IMPL_SPLITKV_MFMA && !split_mfma_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
-                    "scaled_dot_product_attention: the matrix-core split-KV kernels need D and Dv <= 128 in whole 16-byte vectors, Sq <= 64, no dense mask, a finite scale and 16-byte aligned rows");
+                    "scaled_dot_product_attention: the matrix-core split-KV kernels need D and Dv <= 128 (f16/bf16: 256) in whole 16-byte vectors, Sq <= 64 (any Sq above 128), no dense mask, a finite scale and 16-byte aligned rows");
     if (impl == INCIN_ROCM_IMPL_SPLITKV && !split_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
                     "scaled_dot_product_attention: the split-KV kernel needs D == Dv in {64,128}, Sq <= 64, no dense mask and 16-byte aligned rows");
@@ -251,7 +255,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         // workgroups of a launch, all of equal length, run in rounds.  Take the number of splits that leaves the last
         // round fullest, among those that keep at least 256 keys per split, preferring fewer splits at (nearly) equal
         // filling: fewer partial results to combine.
-        const int64_t chunk = incin_rocm::decode_mfma_chunk_rows((int)std::min<int64_t>(R, 1 << 20), d->dtype);
+        const int64_t chunk = incin_rocm::decode_mfma_chunk_rows((int)std::min<int64_t>(R, 1 << 20), d->dtype, (int)d_pad);
         const int64_t nchunks = (R + chunk - 1) / chunk;
         const int64_t groups = d->B * d->Hkv * nchunks;
         int64_t splits = d->num_splits;
@@ -261,7 +265,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
             const int64_t max_splits = std::min<int64_t>(max_by_len, std::max<int64_t>(1, 4 * cus / groups));
             auto fill = [&](int64_t s) {           // (with the split length, and so the count, s really leads to)
                 const int64_t len = ((d->Skv + s - 1) / s + 255) / 256 * 256;
-                const int64_t at_a_time = cus * incin_rocm::decode_mfma_workgroups_per_cu((int)chunk, len, d->dtype);
+                const int64_t at_a_time = cus * incin_rocm::decode_mfma_workgroups_per_cu((int)chunk, len, d->dtype, (int)d_pad);
                 const int64_t wgs = groups * ((d->Skv + len - 1) / len), rounds = (wgs + at_a_time - 1) / at_a_time;
                 return (double)wgs / (double)(rounds * at_a_time);
             };
@@ -334,7 +338,7 @@ void fill_params(const incin_rocm_sdpa_desc_t* d, const Plan& plan, SdpaParams* 
                   d->mask_stride[0] % 4 == 0 && d->mask_stride[1] % 4 == 0 && d->mask_stride[2] % 4 == 0;
     p->B = (int)d->B; p->Hq = (int)d->Hq; p->Hkv = (int)d->Hkv; p->G = (int)(d->Hq / d->Hkv);
     p->Sq = (int)d->Sq; p->Skv = (int)d->Skv; p->D = (int)d->D; p->Dv = (int)d->Dv;
-    p->Dp = std::max(d->D, d->Dv) <= 64 ? 64 : 128;      // (means something to the matrix-core and split-KV kernels only)
+    p->Dp = std::max(d->D, d->Dv) <= 64 ? 64 : std::max(d->D, d->Dv) <= 128 ? 128 : 256;      // (means something to the matrix-core and split-KV kernels only)
     p->scale = d->scale;
     p->causal = d->causal ? 1 : 0;
     p->interleave = 1;

@@ -36,9 +36,11 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
     typedef typename Mma<T>::vec8 vec8;
     typedef PfLayout<D> L;
     constexpr int NSTEP = D / 16, NDB = D / 32;
-    constexpr int KB = 128 / D;                        // 32-key sub-blocks of a block: a slot holds 8 KiB either way
+    constexpr int SLOT = D > 128 ? 2 * DM_SLOT_BYTES : DM_SLOT_BYTES;      // a slot holds 8 KiB, at D = 256 the 16 KiB of 32 keys
+    constexpr int KB = SLOT / (32 * L::ROWB);          // 32-key sub-blocks of a block: 2 at D = 64, else 1
     constexpr int BLOCK = 32 * KB;                     // keys per block
-    constexpr int CPB = DM_SLOT_BYTES / 1024;          // wavefront-wide 1 KiB copies per block
+    constexpr int CPB = SLOT / 1024;                   // wavefront-wide 1 KiB copies per block
+    constexpr int NDBW = NDB >= 4 ? NDB / 4 : 1;       // 32-wide blocks of the head dimension a wavefront stores at the end
     extern __shared__ __attribute__((aligned(1024))) char smem[];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -108,7 +110,7 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
         const unsigned hi = (unsigned)((unsigned long long)x >> 32), lo = (unsigned)x;
         return x <= 0 ? 0 : (hi | (lo >> 31)) != 0 ? 0x7fffffff : (int)lo;
     };
-    const unsigned ring = lds_address(smem) + wave * NSLOT * DM_SLOT_BYTES;
+    const unsigned ring = lds_address(smem) + wave * NSLOT * SLOT;
     // Copies are started unconditionally, NSLOT ahead of their use: past the wavefront's last block the descriptor
     // covers nothing, such a copy fetches nothing and delivers zeros into a slot nobody reads any more - which keeps the
     // count of copies in flight, and with it the wait for the oldest, the same from the first block to the last.
@@ -117,7 +119,7 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
         // The slot about to be refilled was read by this wavefront's LDS loads just before: those loads have delivered
         // once lgkmcnt is 0 (the "memory" clobber keeps them above this point in program order).
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        const unsigned dst = ring + slot_in * DM_SLOT_BYTES;
+        const unsigned dst = ring + slot_in * SLOT;
         if ((issued & 1) == 0) {
             const uint4v rk = dma_descriptor(k_next, clamp31(k_rem));
 #pragma unroll
@@ -192,8 +194,8 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
     for (int j = 0; j < my_blocks; ++j) {
         const int j0 = first_key + j * 4 * BLOCK;
         // ---- S^T = K Q^T ----
-        wait_oldest_copy<NSLOT>();
-        const char* kb = smem + (wave * NSLOT + slot_out) * DM_SLOT_BYTES;
+        wait_oldest_copy<NSLOT, CPB>();
+        const char* kb = smem + (wave * NSLOT + slot_out) * SLOT;
         slot_out = slot_out + 1 == NSLOT ? 0 : slot_out + 1;
         floatx16 sacc[NRB][KB];
 #pragma unroll
@@ -264,8 +266,8 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
             l_run[rb] += rsum;
         }
         // ---- O^T += V^T P^T ----
-        wait_oldest_copy<NSLOT>();
-        const char* vb = smem + (wave * NSLOT + slot_out) * DM_SLOT_BYTES;
+        wait_oldest_copy<NSLOT, CPB>();
+        const char* vb = smem + (wave * NSLOT + slot_out) * SLOT;
         slot_out = slot_out + 1 == NSLOT ? 0 : slot_out + 1;
 #pragma unroll
         for (int ks = 0; ks < 2 * KB; ++ks)
@@ -306,44 +308,51 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
             for (int r = 0; r < 16; ++r) s_o[(((wave * NRB + rb) * NDB + db) * 16 + r) * 64 + lane] = o_acc[rb][db][r] * f;
     }
     __syncthreads();
-    // ---- this wavefront's 32 columns of every row (D = 64: the first two wavefronts') -------------------------------
-    if (wave >= NDB) return;
+    // ---- this wavefront's NDBW blocks of 32 columns of every row (D = 64: the first two wavefronts' one) --------------
+    if (wave * NDBW >= NDB) return;
 #pragma unroll
     for (int rb = 0; rb < NRB; ++rb) {
         if (!valid[rb]) continue;
         float l_tot = 0.0f;
-        floatx16 o;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) o[r] = 0.0f;
+        for (int w = 0; w < 4; ++w) l_tot += s_l[w * CHUNK + 32 * rb + ql];
+        const float inv = (l_tot == 0.0f) ? __builtin_nanf("") : 1.0f / l_tot;      // no visible key: NaN, as the reference
+        const int64_t slot = (((int64_t)b * p.Hq + hq[rb]) * Sq + qi[rb]) * p.num_splits + split;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            l_tot += s_l[w * CHUNK + 32 * rb + ql];
+        for (int d2 = 0; d2 < NDBW; ++d2) {
+            const int db = wave * NDBW + d2;
+            floatx16 o;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) o[r] += s_o[(((w * NRB + rb) * NDB + wave) * 16 + r) * 64 + lane];
+            for (int r = 0; r < 16; ++r) o[r] = 0.0f;
+#pragma unroll
+            for (int w = 0; w < 4; ++w)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) o[r] += s_o[(((w * NRB + rb) * NDB + db) * 16 + r) * 64 + lane];
+            if (p.num_splits == 1) {
+                T* orow = (T*)p.o + (int64_t)b * p.o_sb + (int64_t)hq[rb] * p.o_sh + (int64_t)qi[rb] * p.o_ss + 32 * db + 4 * g;
+#pragma unroll
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    typedef T vec4 __attribute__((ext_vector_type(4)));
+                    vec4 w;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) w[e] = (T)(o[r4 * 4 + e] * inv);
+                    if (32 * db + 4 * g + r4 * 8 < p.Dv) *(vec4*)(orow + r4 * 8) = w;
+                }
+            } else {
+                float* arow = p.ws_acc + slot * D + 32 * db + 4 * g;
+#pragma unroll
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    typedef float f4 __attribute__((ext_vector_type(4)));
+                    f4 w = {o[r4 * 4], o[r4 * 4 + 1], o[r4 * 4 + 2], o[r4 * 4 + 3]};
+                    *(f4*)(arow + r4 * 8) = w;
+                }
+            }
         }
-        if (p.num_splits == 1) {
-            const float inv = (l_tot == 0.0f) ? __builtin_nanf("") : 1.0f / l_tot;      // no visible key: NaN, as the reference
-            T* orow = (T*)p.o + (int64_t)b * p.o_sb + (int64_t)hq[rb] * p.o_sh + (int64_t)qi[rb] * p.o_ss + 32 * wave + 4 * g;
-#pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-                typedef T vec4 __attribute__((ext_vector_type(4)));
-                vec4 w;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) w[e] = (T)(o[r4 * 4 + e] * inv);
-                if (32 * wave + 4 * g + r4 * 8 < p.Dv) *(vec4*)(orow + r4 * 8) = w;
-            }
-            if (p.lse && wave == 0 && g == 0)       // the row's softmax normaliser, natural log (M and the sum are in log2 units)
-                p.lse[((int64_t)b * p.Hq + hq[rb]) * Sq + qi[rb]] = l_tot == 0.0f ? -INFINITY : (M[rb] + __builtin_log2f(l_tot)) * 0.6931471805599453f;
-        } else {
-            const int64_t slot = (((int64_t)b * p.Hq + hq[rb]) * Sq + qi[rb]) * p.num_splits + split;
-            float* arow = p.ws_acc + slot * D + 32 * wave + 4 * g;
-#pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-                typedef float f4 __attribute__((ext_vector_type(4)));
-                f4 w = {o[r4 * 4], o[r4 * 4 + 1], o[r4 * 4 + 2], o[r4 * 4 + 3]};
-                *(f4*)(arow + r4 * 8) = w;
-            }
-            if (wave == 0 && g == 0) {
+        if (wave == 0 && g == 0) {
+            if (p.num_splits == 1) {
+                if (p.lse)      // the row's softmax normaliser, natural log (M and the sum are in log2 units)
+                    p.lse[((int64_t)b * p.Hq + hq[rb]) * Sq + qi[rb]] = l_tot == 0.0f ? -INFINITY : (M[rb] + __builtin_log2f(l_tot)) * 0.6931471805599453f;
+            } else {
                 p.ws_ml[slot * 2 + 0] = M[rb];      // log2 units, as the combine kernel takes them for 16-bit storage
                 p.ws_ml[slot * 2 + 1] = l_tot;
             }
@@ -358,7 +367,8 @@ template <typename T, int D, int NSLOT, int NRB>
 static hipError_t launch_decode_mfma_t(const SdpaParams& p, hipStream_t stream)
 {
     // the rings, or what the wavefronts' results need when they meet at the end, whichever is more
-    constexpr size_t ring_bytes = (size_t)4 * NSLOT * DM_SLOT_BYTES, merge_bytes = (size_t)NRB * (4 * 32 * 2 + 4 * (D / 32) * 16 * 64) * sizeof(float);
+    constexpr size_t slot_bytes = D > 128 ? 2 * DM_SLOT_BYTES : DM_SLOT_BYTES;
+    constexpr size_t ring_bytes = (size_t)4 * NSLOT * slot_bytes, merge_bytes = (size_t)NRB * (4 * 32 * 2 + 4 * (D / 32) * 16 * 64) * sizeof(float);
     constexpr size_t lds = ring_bytes > merge_bytes ? ring_bytes : merge_bytes;
     auto kern = sdpa_decode_mfma_kernel<T, D, NSLOT, NRB>;
     // the dynamic-LDS limit of this instance is raised once per device, not per launch
@@ -383,12 +393,13 @@ hipError_t launch_sdpa_decode_f32(const SdpaParams& p, bool two_slots, hipStream
 
 // Rows a workgroup takes: 32, or 64 (two blocks of 32 against the same K and V operands) when more than 32 rows share a KV
 // head - the cache is then read once for 64 rows instead of once per 32.  (f32, dtype 0: 16 or 32, sdpa_decode_f32.hip.)
-int decode_mfma_chunk_rows(int R, int dtype) { return dtype == 0 ? decode_f32_chunk_rows(R) : R > 32 ? 64 : 32; }
+int decode_mfma_chunk_rows(int R, int dtype, int d_pad) { return dtype == 0 ? decode_f32_chunk_rows(R) : R > 32 && d_pad <= 128 ? 64 : 32; }
 
 // Workgroups a compute unit holds at a time: two of the two-slot form (one block of rows, splits of up to DM_SHORT_KEYS
 // keys of 16-bit storage or half as many of f32), one otherwise.  The planner fills rounds of this many.
-int decode_mfma_workgroups_per_cu(int chunk_rows, int64_t split_len, int dtype)
+int decode_mfma_workgroups_per_cu(int chunk_rows, int64_t split_len, int dtype, int d_pad)
 {
+    if (d_pad > 128) return 1;
     if (dtype == 0) return chunk_rows == 16 && 2 * split_len <= DM_SHORT_KEYS ? 2 : 1;
     return chunk_rows == 32 && split_len <= DM_SHORT_KEYS ? 2 : 1;
 }
@@ -400,7 +411,7 @@ static bool decode_two_slots(const SdpaParams& p, int dtype)
     const char* forced = getenv("INCIN_ROCM_DECODE_SLOTS");
     const int slots = forced ? atoi(forced) : 0;
     const int one_block = dtype == 0 ? 16 : 32;
-    return slots == 2 || (slots != DM_NSLOT && decode_mfma_workgroups_per_cu(one_block, p.split_len, dtype) == 2);
+    return slots == 2 || (slots != DM_NSLOT && decode_mfma_workgroups_per_cu(one_block, p.split_len, dtype, p.Dp) == 2);
 }
 
 // Host has validated: dtype f16 / bf16, D == Dv in {64, 128}, rows 16-byte aligned with unit last-dim stride, row strides
@@ -408,7 +419,7 @@ static bool decode_two_slots(const SdpaParams& p, int dtype)
 template <typename T, int D>
 static hipError_t launch_decode_mfma_d(const SdpaParams& p, hipStream_t stream)
 {
-    if (decode_mfma_chunk_rows(p.G * p.Sq, 2) == 64) return launch_decode_mfma_t<T, D, DM_NSLOT, 2>(p, stream);
+    if (decode_mfma_chunk_rows(p.G * p.Sq, 2, D) == 64) return launch_decode_mfma_t<T, D, DM_NSLOT, 2>(p, stream);
     // Short splits (up to DM_SHORT_KEYS keys: 16 blocks per wavefront) take rings of two slots, which lets a compute
     // unit hold two workgroups: with so little to stream, what counts is that one workgroup's start-up (its first
     // copies' latency) and end (the wavefronts' results meeting, the stores) overlap another's arithmetic.  Measured
@@ -422,7 +433,9 @@ hipError_t launch_sdpa_decode_mfma(const SdpaParams& p, int dtype, hipStream_t s
 {
     if (dtype == 0) return launch_sdpa_decode_f32(p, decode_two_slots(p, 0), stream);
     hipError_t e;
-    if (p.Dp == 128) e = dtype == 1 ? launch_decode_mfma_d<f16_t, 128>(p, stream) : launch_decode_mfma_d<bf16_t, 128>(p, stream);
+    // head dimensions above 128: one form - 32 rows, two slots of 16 KiB (a block of 32 keys) per wavefront
+    if (p.Dp == 256) e = dtype == 1 ? launch_decode_mfma_t<f16_t, 256, 2, 1>(p, stream) : launch_decode_mfma_t<bf16_t, 256, 2, 1>(p, stream);
+    else if (p.Dp == 128) e = dtype == 1 ? launch_decode_mfma_d<f16_t, 128>(p, stream) : launch_decode_mfma_d<bf16_t, 128>(p, stream);
     else e = dtype == 1 ? launch_decode_mfma_d<f16_t, 64>(p, stream) : launch_decode_mfma_d<bf16_t, 64>(p, stream);
     if (e != hipSuccess || p.num_splits == 1) return e;
     return launch_sdpa_combine(p, dtype, stream);

@@ -25,13 +25,14 @@ __device__ __forceinline__ void dm_copy16(uint4v desc, unsigned lds_addr, int by
     asm volatile("s_nop 0\n\tbuffer_load_dwordx4 %0, %1, 0 offen" DM_CACHE " lds" ::"v"(byte_offset), "s"(desc), "{m0}"(lds_addr) : "memory");
 }
 
-// All but the newest NSLOT - 1 copies of this wavefront (8 instructions each) have landed.
-template <int NSLOT> __device__ __forceinline__ void wait_oldest_copy()
+// All but the newest NSLOT - 1 copies of this wavefront (CPB instructions each: 8 for an 8 KiB slot) have landed.
+template <int NSLOT, int CPB = 8> __device__ __forceinline__ void wait_oldest_copy()
 {
-    static_assert(NSLOT >= 2 && NSLOT <= 5, "s_waitcnt takes an immediate");
-    if (NSLOT == 5) asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
-    else if (NSLOT == 4) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
-    else if (NSLOT == 3) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    constexpr int N = (NSLOT - 1) * CPB;
+    static_assert(N == 8 || N == 16 || N == 24 || N == 32, "s_waitcnt takes an immediate");
+    if (N == 32) asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
+    else if (N == 24) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+    else if (N == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
 }
 

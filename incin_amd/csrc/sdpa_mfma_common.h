@@ -60,7 +60,7 @@ template <int D> struct PfLayout {
     // because two 128-byte rows already split the banks).
     static __device__ __forceinline__ int fk(int r)
     {
-        if (D == 128) return ((r & 3) << 2) | ((r >> 2) & 3);
+        if (D >= 128) return ((r & 3) << 2) | ((r >> 2) & 3);
         return (((r >> 1) & 1) << 2) | ((r >> 2) & 3);
     }
     // V tile: the transposing read takes 4 consecutive rows x 64 bytes per half-wavefront, so fv only
@@ -68,7 +68,7 @@ template <int D> struct PfLayout {
     // bits 0-1 (D = 64: bit 1) makes the read address base ^ (d_block << 6) + immediate.
     static __device__ __forceinline__ int fv(int r)
     {
-        if (D == 128) return (r & 3) << 2;
+        if (D >= 128) return (r & 3) << 2;
         return ((r >> 1) & 1) << 2;
     }
 };

@@ -622,9 +622,32 @@ def test_head_dimensions_padded_into_the_matrix_core_kernels(gpu, dtype, dims):
         assert np.max(np.abs(lse - lse_g)) < (2e-5 if dtype == capi.F32 else 2e-2)
 
 
+@pytest.mark.parametrize("dtype", [capi.BF16, capi.F16])
+@pytest.mark.parametrize("dims", [(256, 256), (192, 128), (160, 160), (136, 256), (64, 200)], ids=lambda x: "D%d_Dv%d" % x)
+def test_head_dimensions_above_128(gpu, dtype, dims):
+    """Head dimensions above 128 (16-bit storage) go through the 256 instance of the matrix-core split-KV kernel whatever
+    the shape: decode with one and with several rows per KV head, and prefill shapes 32 rows per workgroup - causal,
+    grouped queries, key counts, split counts chosen and forced, row normalisers - against the oracle."""
+    D, Dv = dims
+    tol = TOL[dtype]
+    for (B, Hq, Hkv, Sq, Skv), split_list in (((2, 2, 2, 1, 1500), (0, 1, 5)), ((2, 8, 2, 3, 1500), (0, 3)), ((2, 4, 2, 200, 333), (0, 1, 2)),
+                                              ((1, 2, 1, 70, 70), (0,)), ((1, 40, 1, 1, 40), (0,))):
+        q, k, v = inputs(2500 + D + Dv + Sq, B, Hq, Hkv, Sq, Skv, D, Dv, dtype)
+        lens = np.array([Skv, max(Skv // 3, 1)][:B], np.int32)
+        ref = oracle_full(q, k, v, G=Hq // Hkv, causal=True, kv_lens=lens)
+        for splits in split_list:
+            say("head dimension above 128: %s D=%d Dv=%d %r splits=%d" % (dtypes.NAMES[dtype], D, Dv, (B, Hq, Hkv, Sq, Skv), splits))
+            got, lse, info = host.sdpa(q, k, v, dtype, causal=True, kv_lens=lens, num_splits=splits, return_info=True, return_lse=True)
+            assert info["impl"] == capi.IMPL_SPLITKV_MFMA
+            check(got, ref, tol, "D=%d Dv=%d Sq=%d splits=%d->%d" % (D, Dv, Sq, splits, info["splits"]))
+        _, lse_g = host.sdpa(q, k, v, dtype, causal=True, kv_lens=lens, impl=capi.IMPL_GENERIC, return_lse=True)
+        fin = np.isfinite(lse_g)
+        assert np.array_equal(fin, np.isfinite(lse)) and np.max(np.abs(lse[fin] - lse_g[fin])) < 2e-2
+
+
 def test_head_dimensions_outside_the_matrix_core_kernels(gpu):
-    """Rows that are not whole 16-byte vectors, and head dimensions above 128, stay on the generic kernel."""
-    for dtype, D in ((capi.BF16, 20), (capi.F32, 6), (capi.BF16, 160), (capi.F32, 136)):
+    """Rows that are not whole 16-byte vectors, and f32 head dimensions above 128, stay on the generic kernel."""
+    for dtype, D in ((capi.BF16, 20), (capi.F32, 6), (capi.BF16, 132), (capi.F32, 136)):
         q, k, v = inputs(2400 + D, 1, 2, 2, 40, 70, D, D, dtype)
         got, info = host.sdpa(q, k, v, dtype, causal=True, return_info=True)
         assert info["impl"] == capi.IMPL_GENERIC
