@@ -154,12 +154,12 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     const int64_t R = (d->Hq / d->Hkv) * d->Sq;
     // The matrix-core kernels are built for head dimensions 64 and 128; smaller ones (D and Dv need not be equal) run in
     // the instance that holds them, padded with zeros on the way into LDS, as long as rows stay whole 16-byte vectors.
-    // The 16-bit split-KV kernel has an instance for 256 as well, which takes every launch with a head dimension above
+    // The split-KV kernels have an instance for 256 as well, which takes every launch with a head dimension above
     // 128 - prefill shapes too, 32 rows per workgroup.  The vector-ALU split-KV kernel takes the two dimensions as they are.
     const int64_t d_max = std::max(d->D, d->Dv);
     const int64_t d_pad = d_max <= 64 ? 64 : d_max <= 128 ? 128 : 256;
     const bool wide = d_pad == 256;
-    const bool head_pad_ok = d->D > 0 && d_max <= (d->dtype == INCIN_ROCM_F32 ? 128 : 256) && d->D % vec == 0 && d->Dv % vec == 0;
+    const bool head_pad_ok = d->D > 0 && d_max <= 256 && d->D % vec == 0 && d->Dv % vec == 0;
     const bool head_exact = d->D == d->Dv && d->D == d_pad && !wide;
     const bool layout_ok = head_pad_ok && fast_layout_ok(d, vec) && d->Skv > 0;
     const bool fast_ok = layout_ok && !d->add_mask;
@@ -217,7 +217,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
                     "scaled_dot_product_attention: the 64-row MFMA prefill kernel has been retired (INCIN_ROCM_IMPL_MFMA covers its shapes)");
     if (impl == INCIN_ROCM_IMPL_SPLITKV_MFMA && !split_mfma_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
-                    "scaled_dot_product_attention: the matrix-core split-KV kernels need D and Dv <= 128 (f16/bf16: 256) in whole 16-byte vectors, Sq <= 64 (any Sq above 128), no dense mask, a finite scale and 16-byte aligned rows");
+                    "scaled_dot_product_attention: the matrix-core split-KV kernels need D and Dv <= 256 in whole 16-byte vectors, Sq <= 64 (any Sq above 128), no dense mask, a finite scale and 16-byte aligned rows");
     if (impl == INCIN_ROCM_IMPL_SPLITKV && !split_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
                     "scaled_dot_product_attention: the split-KV kernel needs D == Dv in {64,128}, Sq <= 64, no dense mask and 16-byte aligned rows");

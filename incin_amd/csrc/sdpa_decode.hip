@@ -299,10 +299,10 @@ static hipError_t launch_combine_t(const SdpaParams& p, hipStream_t stream)
     return hipGetLastError();
 }
 
-// The partial results of a split-KV launch (rows of p.Dp floats: 64, 128 or - 16-bit storage - 256) into the output.
+// The partial results of a split-KV launch (rows of p.Dp floats: 64, 128 or 256) into the output.
 hipError_t launch_sdpa_combine(const SdpaParams& p, int dtype, hipStream_t stream)
 {
-    if (p.Dp == 256) return dtype == 1 ? launch_combine_t<f16_t, 256>(p, stream) : launch_combine_t<bf16_t, 256>(p, stream);
+    if (p.Dp == 256) return dtype == 0 ? launch_combine_t<float, 256>(p, stream) : dtype == 1 ? launch_combine_t<f16_t, 256>(p, stream) : launch_combine_t<bf16_t, 256>(p, stream);
     if (p.Dp == 128) {
         switch (dtype) {
             case 0: return launch_combine_t<float, 128>(p, stream);

@@ -53,9 +53,10 @@ __global__ __launch_bounds__(256) void sdpa_decode_f32_kernel(SdpaParams p)
     constexpr int NJ = D / 16;                         // groups of four k-steps of the S^T product
     constexpr int NDB = D / 16;                        // 16-wide blocks of the head dimension
     constexpr int NDBW = NDB / 4;                      // of which a wavefront stores this many at the end
-    constexpr int BLOCK = DM_SLOT_BYTES / L::ROWB;     // keys per block: 16 (D = 128), 32 (D = 64)
+    constexpr int SLOT = D > 128 ? 2 * DM_SLOT_BYTES : DM_SLOT_BYTES;      // a slot holds 8 KiB, at D = 256 the 16 KiB of 16 keys
+    constexpr int BLOCK = SLOT / L::ROWB;              // keys per block: 16 (D = 128, 256), 32 (D = 64)
     constexpr int KB = BLOCK / 16;                     // 16-key sub-blocks of a block
-    constexpr int CPB = DM_SLOT_BYTES / 1024;          // wavefront-wide 1 KiB copies per block
+    constexpr int CPB = SLOT / 1024;                   // wavefront-wide 1 KiB copies per block
     constexpr int CHUNK = 16 * NRB;                    // rows per workgroup
     constexpr float LN2 = 0.6931471805599453f;
     extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -126,7 +127,7 @@ __global__ __launch_bounds__(256) void sdpa_decode_f32_kernel(SdpaParams p)
         const unsigned hi = (unsigned)((unsigned long long)x >> 32), lo = (unsigned)x;
         return x <= 0 ? 0 : (hi | (lo >> 31)) != 0 ? 0x7fffffff : (int)lo;
     };
-    const unsigned ring = lds_address(smem) + wave * NSLOT * DM_SLOT_BYTES;
+    const unsigned ring = lds_address(smem) + wave * NSLOT * SLOT;
     // Copies are started unconditionally, NSLOT ahead of their use: past the wavefront's last block the descriptor
     // covers nothing, such a copy fetches nothing and delivers zeros into a slot nobody reads any more - which keeps the
     // count of copies in flight, and with it the wait for the oldest, the same from the first block to the last.
@@ -135,7 +136,7 @@ __global__ __launch_bounds__(256) void sdpa_decode_f32_kernel(SdpaParams p)
         // The slot about to be refilled was read by this wavefront's LDS loads just before: those loads have delivered
         // once lgkmcnt is 0 (the "memory" clobber keeps them above this point in program order).
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        const unsigned dst = ring + slot_in * DM_SLOT_BYTES;
+        const unsigned dst = ring + slot_in * SLOT;
         if ((issued & 1) == 0) {
             const uint4v rk = dma_descriptor(k_next, clamp31(k_rem));
 #pragma unroll
@@ -198,8 +199,8 @@ __global__ __launch_bounds__(256) void sdpa_decode_f32_kernel(SdpaParams p)
     for (int jb = 0; jb < my_blocks; ++jb) {
         const int j0 = first_key + jb * 4 * BLOCK;
         // ---- S^T = K Q'^T: two chains over the halves of the head dimension ----
-        wait_oldest_copy<NSLOT>();
-        const char* kb = smem + (wave * NSLOT + slot_out) * DM_SLOT_BYTES;
+        wait_oldest_copy<NSLOT, CPB>();
+        const char* kb = smem + (wave * NSLOT + slot_out) * SLOT;
         slot_out = slot_out + 1 == NSLOT ? 0 : slot_out + 1;
         floatx4 s0[NRB][KB], s1[NRB][KB];
 #pragma unroll
@@ -291,8 +292,8 @@ __global__ __launch_bounds__(256) void sdpa_decode_f32_kernel(SdpaParams p)
             l_run[rb] += rsum;
         }
         // ---- O^T += V^T P^T ----
-        wait_oldest_copy<NSLOT>();
-        const char* vb = smem + (wave * NSLOT + slot_out) * DM_SLOT_BYTES;
+        wait_oldest_copy<NSLOT, CPB>();
+        const char* vb = smem + (wave * NSLOT + slot_out) * SLOT;
         slot_out = slot_out + 1 == NSLOT ? 0 : slot_out + 1;
 #pragma unroll
         for (int kb2 = 0; kb2 < KB; ++kb2)
@@ -388,7 +389,8 @@ template <int D, int NSLOT, int NRB>
 static hipError_t launch_decode_f32_t(const SdpaParams& p, hipStream_t stream)
 {
     // the rings, or what the wavefronts' results need when they meet at the end, whichever is more
-    constexpr size_t ring_bytes = (size_t)4 * NSLOT * DM_SLOT_BYTES, merge_bytes = (size_t)NRB * (4 * 16 * 2 + 4 * (D / 16) * 4 * 64) * sizeof(float);
+    constexpr size_t slot_bytes = D > 128 ? 2 * DM_SLOT_BYTES : DM_SLOT_BYTES;
+    constexpr size_t ring_bytes = (size_t)4 * NSLOT * slot_bytes, merge_bytes = (size_t)NRB * (4 * 16 * 2 + 4 * (D / 16) * 4 * 64) * sizeof(float);
     constexpr size_t lds = ring_bytes > merge_bytes ? ring_bytes : merge_bytes;
     auto kern = sdpa_decode_f32_kernel<D, NSLOT, NRB>;
     // the dynamic-LDS limit of this instance is raised once per device, not per launch
@@ -425,7 +427,10 @@ static hipError_t launch_decode_f32_d(const SdpaParams& p, bool two_slots, hipSt
 // chooses them for short splits.
 hipError_t launch_sdpa_decode_f32(const SdpaParams& p, bool two_slots, hipStream_t stream)
 {
-    hipError_t e = p.Dp == 128 ? launch_decode_f32_d<128>(p, two_slots, stream) : launch_decode_f32_d<64>(p, two_slots, stream);
+    hipError_t e;
+    // head dimensions above 128: two slots of 16 KiB (a block of 16 keys) per wavefront, 16 or 32 rows
+    if (p.Dp == 256) e = decode_f32_chunk_rows(p.G * p.Sq) == 32 ? launch_decode_f32_t<256, 2, 2>(p, stream) : launch_decode_f32_t<256, 2, 1>(p, stream);
+    else e = p.Dp == 128 ? launch_decode_f32_d<128>(p, two_slots, stream) : launch_decode_f32_d<64>(p, two_slots, stream);
     if (e != hipSuccess || p.num_splits == 1) return e;
     return launch_sdpa_combine(p, 0, stream);
 }

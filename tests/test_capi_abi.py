@@ -65,11 +65,11 @@ def test_dispatch_choices():
     assert _plan(_desc(D=8, Dv=40))[2] == capi.IMPL_MFMA
     assert _plan(_desc(D=84, Dv=84))[2] == capi.IMPL_GENERIC                    # 168-byte rows: not whole vectors
     assert _plan(_desc(dtype=capi.F32, D=84, Dv=84))[2] == capi.IMPL_MFMA       # in f32 they are
-    # above 128, 16-bit storage: the 256 instance of the matrix-core split-KV kernel, prefill shapes too; f32 stays generic
+    # above 128: the 256 instance of the matrix-core split-KV kernels (16-bit and f32), prefill shapes too
     assert _plan(_desc(D=160, Dv=160))[2] == capi.IMPL_SPLITKV_MFMA
     assert _plan(_desc(D=128, Dv=136))[2] == capi.IMPL_SPLITKV_MFMA
     assert _plan(_desc(D=256, Dv=256, Sq=4096, Skv=4096, causal=1))[2] == capi.IMPL_SPLITKV_MFMA
-    assert _plan(_desc(dtype=capi.F32, D=160, Dv=160))[2] == capi.IMPL_GENERIC
+    assert _plan(_desc(dtype=capi.F32, D=160, Dv=160))[2] == capi.IMPL_SPLITKV_MFMA
     # decode over such a cache: the matrix-core split-KV kernels, also at one row per KV head (no vector-ALU kernel there);
     # partial rows are as wide as the kernel instance
     nbytes, splits, impl = _plan(_desc(Sq=1, Skv=8192, B=2, Hq=8, Hkv=8, D=96, Dv=96, num_splits=4))
