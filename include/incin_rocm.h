@@ -45,13 +45,15 @@ enum { INCIN_ROCM_F32 = 0, INCIN_ROCM_F16 = 1, INCIN_ROCM_BF16 = 2 };
 enum {
     INCIN_ROCM_IMPL_AUTO = 0,
     INCIN_ROCM_IMPL_GENERIC = 1,   /* fp32-FMA tiled kernel: any dtype, D and Dv <= 256, dense masks     */
-    INCIN_ROCM_IMPL_MFMA = 2,      /* MFMA prefill kernels, D == Dv in {64,128}: bf16/f16 (no dense mask, scale > 0), and
-                                      IEEE-f32 matrix instructions for f32 (dense mask allowed)                    */
-    INCIN_ROCM_IMPL_SPLITKV = 3,   /* split-KV decode kernel + combine: D == Dv in {64,128}, few query rows */
+    INCIN_ROCM_IMPL_MFMA = 2,      /* MFMA prefill kernels: D and Dv <= 128 in whole 16-byte vectors (instances for 64 and 128; smaller
+                                      and unequal head dimensions are zero-padded into LDS); bf16/f16 (scale > 0) and IEEE-f32
+                                      matrix instructions for f32; dense mask allowed                              */
+    INCIN_ROCM_IMPL_SPLITKV = 3,   /* vector-ALU split-KV decode kernel + combine: D == Dv in {64,128}, few query rows */
     INCIN_ROCM_IMPL_MFMA64 = 4,    /* retired (a prefill kernel with 64 query rows per wavefront): refused with INCIN_ROCM_EUNSUPPORTED */
-    INCIN_ROCM_IMPL_SPLITKV_MFMA = 5 /* split-KV kernels on the matrix cores + combine: D == Dv in {64,128}, Sq <= 64; the rows that share a
-                                      KV head (query heads of the group x query positions) go through them 32 or 64 at a time (bf16/f16),
-                                      16 or 32 at a time on IEEE-f32 matrix instructions (f32) */
+    INCIN_ROCM_IMPL_SPLITKV_MFMA = 5 /* split-KV kernels on the matrix cores + combine: D and Dv <= 256 in whole 16-byte vectors (instances for
+                                      64, 128 and 256), Sq <= 64 - any Sq when a head dimension is above 128, which only these kernels
+                                      cover; the rows that share a KV head (query heads of the group x query positions) go through
+                                      them 32 or 64 at a time (bf16/f16), 16 or 32 at a time on IEEE-f32 matrix instructions (f32) */
 };
 
 /* Thread-local message of the last failing call on this thread ("" if none).
