@@ -1,5 +1,6 @@
 // Split-KV attention for the query rows that share one key/value head, in IEEE single precision on the gfx950 matrix
-// cores (v_mfma_f32_16x16x4_f32: f32 operands, products and sums), D == Dv in {64, 128}: grouped-query decode and short
+// cores (v_mfma_f32_16x16x4_f32: f32 operands, products and sums), head dimensions up to 256 (instances for 64, 128 and
+// 256; a smaller D or Dv is zero-padded on the way into LDS): grouped-query decode and short
 // runs of query rows over a long f32 cache - f32 being the one dtype the reference's own operator runs end to end
 // (crates/incin-backends/src/cpu/ops/shape_ops.rs:1245-1269), with a 1e-5 bar.  The vector-ALU split-KV kernel
 // handles one to a few rows per KV head at the memory system's rate and then runs out of arithmetic; the prefill kernel
@@ -414,7 +415,7 @@ static hipError_t launch_decode_f32_t(const SdpaParams& p, hipStream_t stream)
 // 16 rows share a KV head.
 int decode_f32_chunk_rows(int R) { return R > 16 ? 32 : 16; }
 
-// Host has validated: f32, D == Dv in {64, 128}, rows 16-byte aligned with unit last-dim stride, row strides below 2^22
+// Host has validated: f32, D and Dv <= 128 in whole 16-byte vectors (p.Dp = the instance), rows 16-byte aligned with unit last-dim stride, row strides below 2^22
 // elements, split_len a multiple of 256 (whole rounds of the four wavefronts' blocks of 16 or 32 keys).
 template <int D>
 static hipError_t launch_decode_f32_d(const SdpaParams& p, bool two_slots, hipStream_t stream)

@@ -1,5 +1,5 @@
 // Split-KV attention for the query rows that share one key/value head, on the gfx950 matrix cores (f16 / bf16,
-// D == Dv in {64, 128}): grouped-query decode, where the vector-ALU split-KV kernel runs out of arithmetic (it spends
+// head dimensions up to 256: instances for 64, 128 and 256, a smaller D or Dv zero-padded on the way into LDS): grouped-query decode, where the vector-ALU split-KV kernel runs out of arithmetic (it spends
 // ~24 vector instructions per query row on every 2 KiB of cache it reads), and short runs of query rows over a long
 // cache.  Same function as the other attention kernels (crates/incin-backends/src/cpu/ops/shape_ops.rs:1245-1269),
 // same partial-result format as the vector-ALU split-KV kernel, same combine kernel.
@@ -414,7 +414,7 @@ static bool decode_two_slots(const SdpaParams& p, int dtype)
     return slots == 2 || (slots != DM_NSLOT && decode_mfma_workgroups_per_cu(one_block, p.split_len, dtype, p.Dp) == 2);
 }
 
-// Host has validated: dtype f16 / bf16, D == Dv in {64, 128}, rows 16-byte aligned with unit last-dim stride, row strides
+// Host has validated: dtype f16 / bf16, D and Dv <= 128 in whole 16-byte vectors (p.Dp = the instance), rows 16-byte aligned with unit last-dim stride, row strides
 // below 2^24 elements, split_len a multiple of 256 (whole rounds of the four wavefronts' blocks of 32 or 64 keys).
 template <typename T, int D>
 static hipError_t launch_decode_mfma_d(const SdpaParams& p, hipStream_t stream)

@@ -1,6 +1,6 @@
 // f32 attention forward on the gfx950 matrix cores with IEEE single-precision arithmetic
-// (v_mfma_f32_32x32x2_f32: f32 operands, f32 products and sums - no reduced-precision path), for D == Dv in
-// {64, 128}, optional causal mask, per-batch key lengths, a dense additive mask with arbitrary broadcast strides,
+// (v_mfma_f32_32x32x2_f32: f32 operands, f32 products and sums - no reduced-precision path), for head dimensions up to
+// 128 (instances for 64 and 128; a smaller D or Dv, in whole 16-byte vectors, is zero-padded on the way into LDS), optional causal mask, per-batch key lengths, a dense additive mask with arbitrary broadcast strides,
 // MHA and GQA.  f32 is the one dtype the reference's own operator runs end to end
 // (crates/incin-backends/src/cpu/ops/shape_ops.rs:1245-1269 over cpu/ops/matmul.rs:234,254), with a 1e-5 bar.
 //
@@ -318,7 +318,7 @@ static hipError_t launch_prefill_f32_t(const SdpaParams& p0, hipStream_t stream)
     return hipGetLastError();
 }
 
-// Host has validated: f32, D == Dv in {64, 128}, finite scale, rows 16-byte aligned with unit last-dim stride, row
+// Host has validated: f32, D and Dv <= 128 in whole 16-byte vectors (p.Dp = the instance: 64 or 128), finite scale, rows 16-byte aligned with unit last-dim stride, row
 // strides below 2^24 elements (tile offsets fit the 32-bit buffer offset); the dense mask, if any, has any strides.
 hipError_t launch_sdpa_prefill_f32(const SdpaParams& p, hipStream_t stream)
 {

@@ -1,8 +1,9 @@
 // bf16 / f16 attention forward on the gfx950 matrix cores (prefill shapes).
 //
 // Computes the function of the reference CPU composition
-// (crates/incin-backends/src/cpu/ops/shape_ops.rs:1245-1269) for D == Dv in
-// {64, 128}, optional causal mask and per-batch key lengths, MHA and GQA, with
+// (crates/incin-backends/src/cpu/ops/shape_ops.rs:1245-1269) for head dimensions up to 128 (instances for 64 and
+// 128; a smaller D or Dv, in whole 16-byte vectors, is zero-padded on the way into LDS and the stores are cut at Dv),
+// optional causal mask and per-batch key lengths, MHA and GQA, with
 // f32 accumulation and an online softmax: no score tensor is ever materialised.
 //
 // Shape of the computation (one workgroup = 4 wavefronts = 128 query rows, one
@@ -841,7 +842,7 @@ static hipError_t launch_prefill_t(const SdpaParams& p, hipStream_t stream)
     return launch_prefill_nw<T, D, DENSE, 4>(p, stream);
 }
 
-// Host has validated: dtype f16/bf16, D == Dv in {64,128}, scale > 0, rows 16-byte aligned with unit last-dim stride, row strides below 2^24
+// Host has validated: dtype f16/bf16, D and Dv <= 128 in whole 16-byte vectors (p.Dp = the instance: 64 or 128), scale > 0, rows 16-byte aligned with unit last-dim stride, row strides below 2^24
 // elements (tile offsets fit the 32-bit buffer offset).
 hipError_t launch_sdpa_prefill_mfma(const SdpaParams& p, int dtype, hipStream_t stream)
 {
