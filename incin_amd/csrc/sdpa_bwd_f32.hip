@@ -45,9 +45,12 @@ template <int D> struct F32Addr {
     int row_base;                  // by rows: address = row_base ^ (j << 5)
     int col_low[8], col_high[D / 32];
     int voff[2][L::LPW];
+    int width[2];                  // [tensor]: floats of data per row (a row's chunks beyond arrive as zeros: dma_chunk_offset)
 
-    __device__ __forceinline__ void init(int wave, int lane, int64_t stride0, int64_t stride1)
+    __device__ __forceinline__ void init(int wave, int lane, int64_t stride0, int64_t stride1, int width0, int width1)
     {
+        width[0] = width0;
+        width[1] = width1;
         const int ql = lane & 31, g = lane >> 5;
         row_base = ql * L::ROWB + (((g ^ L::f(ql)) & 1) << 4) + ((L::f(ql) & 0xe) << 4);
 #pragma unroll
@@ -58,8 +61,8 @@ template <int D> struct F32Addr {
         for (int c = 0; c < L::LPW; ++c) {
             const int pos = (wave * L::LPW + c) * 64 + lane;
             const int row = pos / L::CPR, slot = pos % L::CPR;
-            voff[0][c] = row * (int)stride0 * 4 + (slot ^ L::f(row)) * 16;
-            voff[1][c] = row * (int)stride1 * 4 + (slot ^ L::f(row)) * 16;
+            voff[0][c] = dma_chunk_offset(row, (int)stride0 * 4, slot ^ L::f(row), width0 * 4);
+            voff[1][c] = dma_chunk_offset(row, (int)stride1 * 4, slot ^ L::f(row), width1 * 4);
         }
     }
     __device__ __forceinline__ float4v by_rows(const char* tile, int blk, int j) const
@@ -73,7 +76,7 @@ template <int D> struct F32Addr {
     // rows [row0, row0 + ROWS) of tensor `which` (rows of `stride` floats, `rows` of them) into the tile at LDS address dst
     __device__ __forceinline__ void issue(int which, const float* base, int64_t stride, int rows, int row0, unsigned dst, int wave) const
     {
-        int64_t rem = (int64_t)(rows - row0 - 1) * stride * 4 + D * 4;
+        int64_t rem = (int64_t)(rows - row0 - 1) * stride * 4 + width[which] * 4;
         if (rem > 0x7fffffffLL) rem = 0x7fffffffLL;
         if (rem < 0) rem = 0;
         const uint4v r = dma_descriptor((const char*)base + (int64_t)row0 * stride * 4, (int)rem);
@@ -157,7 +160,7 @@ void bwd_f32_dq_kernel(SdpaBwdParams bp)
     const int n_act = lim_wave_max > 0 ? (lim_wave_max + KT - 1) / KT : 0;
 
     F32Addr<D> ad;
-    ad.init(wave, lane, p.k_ss, p.v_ss);
+    ad.init(wave, lane, p.k_ss, p.v_ss, p.D, p.Dv);
     const unsigned lds0 = lds_address(smem);
     auto issue_kv = [&](int t) __attribute__((always_inline)) {
         ad.issue(0, kp, p.k_ss, j_end, t * KT, lds0 + (t & 1) * L::TILE_BYTES, wave);
@@ -174,10 +177,15 @@ void bwd_f32_dq_kernel(SdpaBwdParams bp)
         const float c2 = p.scale * 1.4426950408889634f;
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
-            qreg[j] = *(const float4v*)(qrow + j * 8);
-            greg[j] = *(const float4v*)(grow + j * 8);
+            // (beyond the head dimensions: zeros, like the tiles' rows)
+            const bool in_q = j * 8 + g * 4 < p.D, in_g = j * 8 + g * 4 < p.Dv;
+            if (in_q) qreg[j] = *(const float4v*)(qrow + j * 8);
+            if (in_g) greg[j] = *(const float4v*)(grow + j * 8);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) qreg[j][e] *= c2;
+            for (int e = 0; e < 4; ++e) {
+                qreg[j][e] = in_q ? qreg[j][e] * c2 : 0.0f;
+                greg[j][e] = in_g ? greg[j][e] : 0.0f;
+            }
         }
         const int64_t stat = ((int64_t)b * p.Hq + hq) * Sq + qi;
         seed_s = bp.neg_l2[stat];
@@ -269,7 +277,7 @@ void bwd_f32_dq_kernel(SdpaBwdParams bp)
                 float4v w;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) w[e] = my_i < rows_b ? dq_acc[db][r4 * 4 + e] * p.scale : 0.0f;
-                *(float4v*)(row + db * 32 + r4 * 8 + g * 4) = w;
+                if (db * 32 + r4 * 8 + g * 4 < p.D) *(float4v*)(row + db * 32 + r4 * 8 + g * 4) = w;
             }
     }
 #endif
@@ -332,7 +340,7 @@ void bwd_f32_dkv_kernel(SdpaBwdParams bp)
     const int n_tiles = tiles_per_head * p.G;           // the group's query heads one after another
 
     F32Addr<D> ad;
-    ad.init(wave, lane, p.q_ss, bp.do_ss);
+    ad.init(wave, lane, p.q_ss, bp.do_ss, p.D, p.Dv);
 
     // this lane's key: K' = K * scale * log2(e) and V rows as B operands
     float4v kreg[NJ], vreg[NJ];
@@ -343,10 +351,14 @@ void bwd_f32_dkv_kernel(SdpaBwdParams bp)
         const float c2 = p.scale * 1.4426950408889634f;
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
-            kreg[j] = *(const float4v*)(krow + j * 8);
-            vreg[j] = *(const float4v*)(vrow + j * 8);
+            const bool in_k = j * 8 + g * 4 < p.D, in_v = j * 8 + g * 4 < p.Dv;
+            if (in_k) kreg[j] = *(const float4v*)(krow + j * 8);
+            if (in_v) vreg[j] = *(const float4v*)(vrow + j * 8);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) kreg[j][e] *= c2;
+            for (int e = 0; e < 4; ++e) {
+                kreg[j][e] = in_k ? kreg[j][e] * c2 : 0.0f;
+                vreg[j][e] = in_v ? vreg[j][e] : 0.0f;
+            }
         }
         // (arrived before the loop, as in the dQ kernel)
 #pragma unroll
@@ -470,8 +482,8 @@ void bwd_f32_dkv_kernel(SdpaBwdParams bp)
                     wk[e] = live ? dk_acc[db][r4 * 4 + e] * p.scale : 0.0f;
                     wv[e] = live ? dv_acc[db][r4 * 4 + e] : 0.0f;
                 }
-                *(float4v*)(krow + db * 32 + r4 * 8 + g * 4) = wk;
-                *(float4v*)(vrow + db * 32 + r4 * 8 + g * 4) = wv;
+                if (db * 32 + r4 * 8 + g * 4 < p.D) *(float4v*)(krow + db * 32 + r4 * 8 + g * 4) = wk;
+                if (db * 32 + r4 * 8 + g * 4 < p.Dv) *(float4v*)(vrow + db * 32 + r4 * 8 + g * 4) = wv;
             }
     }
 #endif
@@ -498,11 +510,11 @@ static hipError_t launch_bwd_f32_t(const SdpaBwdParams& bp, hipStream_t stream)
     return hipGetLastError();
 }
 
-// Host has validated: f32, D == Dv in {64, 128}, no dense mask, finite scale, unit last-axis strides, 16-byte aligned rows,
+// Host has validated: f32, D and Dv <= 128 in whole 16-byte vectors (bp.f.Dp = the instance: 64 or 128), no dense mask, finite scale, unit last-axis strides, 16-byte aligned rows,
 // row strides below 2^22 elements, lse and the workspace present.
 hipError_t launch_sdpa_bwd_f32(const SdpaBwdParams& bp, hipStream_t stream)
 {
-    return bp.f.D == 128 ? launch_bwd_f32_t<128>(bp, stream) : launch_bwd_f32_t<64>(bp, stream);
+    return bp.f.Dp == 128 ? launch_bwd_f32_t<128>(bp, stream) : launch_bwd_f32_t<64>(bp, stream);
 }
 
 }  // namespace incin_rocm

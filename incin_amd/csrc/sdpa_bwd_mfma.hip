@@ -39,7 +39,7 @@ __global__ __launch_bounds__(256) void sdpa_bwd_delta_kernel(SdpaBwdParams p)
         const int hq = (int)(bh % p.f.Hq), b = (int)(bh / p.f.Hq);
         const T* o = (const T*)p.f.o + b * p.f.o_sb + hq * p.f.o_sh + (int64_t)i * p.f.o_ss;
         const T* g = (const T*)p.d_o + b * p.do_sb + hq * p.do_sh + (int64_t)i * p.do_ss;
-        for (int d = sub * 8; d < p.f.D; d += 128) {
+        for (int d = sub * 8; d < p.f.Dv; d += 128) {
             const vec8 x = *(const vec8*)(o + d), y = *(const vec8*)(g + d);
 #pragma unroll
             for (int e = 0; e < 8; ++e) acc = fmaf((float)x[e], (float)y[e], acc);
@@ -70,8 +70,12 @@ struct BwdTiles {
     int tr_addr[NDBU][2];          // [column block - db0][half]: byte offset of the transposing read
     int voff[2][LPW];              // [tensor][load]: global byte offset of this lane's 16 bytes of a tile
 
-    __device__ __forceinline__ void init(int wave, int lane, int64_t stride0, int64_t stride1, int db0)
+    int width[2];                  // [tensor]: elements of data per row (a row's chunks beyond arrive as zeros: dma_chunk_offset)
+
+    __device__ __forceinline__ void init(int wave, int lane, int64_t stride0, int64_t stride1, int width0, int width1, int db0)
     {
+        width[0] = width0;
+        width[1] = width1;
         const int ql = lane & 31, g = lane >> 5, n = lane & 15, dh = (lane >> 4) & 1;
 #pragma unroll
         for (int s = 0; s < NSTEP; ++s) {
@@ -89,15 +93,15 @@ struct BwdTiles {
         for (int c = 0; c < LPW; ++c) {
             const int pos = (wave * LPW + c) * 64 + lane;
             const int row = pos / L::CPR, slot = pos % L::CPR;
-            voff[0][c] = row * (int)stride0 * 2 + (slot ^ L::fk(row)) * 16;
-            voff[1][c] = row * (int)stride1 * 2 + (slot ^ L::fk(row)) * 16;
+            voff[0][c] = dma_chunk_offset(row, (int)stride0 * 2, slot ^ L::fk(row), width0 * 2);
+            voff[1][c] = dma_chunk_offset(row, (int)stride1 * 2, slot ^ L::fk(row), width1 * 2);
         }
     }
     // start the copy of rows [row0, row0 + 64) of tensor `which` (base pointer of the head, `rows` rows of `stride`
     // elements) into `dst`; rows at and beyond `rows` arrive as zeros
     __device__ __forceinline__ void issue(int which, const T* base, int64_t stride, int rows, int row0, unsigned dst, int wave) const
     {
-        int64_t rem = (int64_t)(rows - row0 - 1) * stride * 2 + D * 2;
+        int64_t rem = (int64_t)(rows - row0 - 1) * stride * 2 + width[which] * 2;
         if (rem > 0x7fffffffLL) rem = 0x7fffffffLL;
         if (rem < 0) rem = 0;
         const uint4v r = dma_descriptor((const char*)base + (int64_t)row0 * stride * 2, (int)rem);
@@ -172,7 +176,7 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
     const int n_act = lim_wave_max > 0 ? (lim_wave_max + PF_BN - 1) / PF_BN : 0;
 
     BwdTiles<T, D, 4, NDB> tl;
-    tl.init(wave, lane, p.k_ss, p.v_ss, 0);
+    tl.init(wave, lane, p.k_ss, p.v_ss, p.D, p.Dv, 0);
 
     // this lane's query: Q row (scaled into log2 units, as the forward does) and dO row, the row's normaliser and D_i
     vec8 qreg[NSTEP], greg[NSTEP];
@@ -183,11 +187,16 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
         const float c2 = p.scale * 1.4426950408889634f;
 #pragma unroll
         for (int s = 0; s < NSTEP; ++s) {
-            vec8 x = *(const vec8*)(qrow + s * 16);
+            // (beyond the head dimensions: zeros, like the tiles' rows)
+            vec8 x, y;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) { x[e] = (T)0.0f; y[e] = (T)0.0f; }
+            if (s * 16 + g * 8 < p.D) x = *(const vec8*)(qrow + s * 16);
+            if (s * 16 + g * 8 < p.Dv) y = *(const vec8*)(grow + s * 16);
 #pragma unroll
             for (int e = 0; e < 8; ++e) x[e] = (T)((float)x[e] * c2);
             qreg[s] = x;
-            greg[s] = *(const vec8*)(grow + s * 16);
+            greg[s] = y;
         }
     }
     const int64_t stat = ((int64_t)b * p.Hq + hq) * Sq + qi;
@@ -261,7 +270,7 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
                 vec4 w;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) w[e] = (T)(my_i < rows_b ? dq_acc[db][r4 * 4 + e] * p.scale : 0.0f);
-                *(vec4*)(row + db * 32 + r4 * 8 + g * 4) = w;
+                if (db * 32 + r4 * 8 + g * 4 < p.D) *(vec4*)(row + db * 32 + r4 * 8 + g * 4) = w;
             }
     }
 #endif
@@ -350,7 +359,7 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
     const int n_tiles = tiles_per_head * p.G;           // the group's query heads one after another
 
     BwdTiles<T, D, 8, NCB> tl;
-    tl.init(wave, lane, p.q_ss, bp.do_ss, NCB * role);
+    tl.init(wave, lane, p.q_ss, bp.do_ss, p.D, p.Dv, NCB * role);
 
     // this lane's key: K row (scaled into log2 units) and V row as B operands
     vec8 kreg[NSTEP], vreg[NSTEP];
@@ -361,11 +370,15 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
         const float c2 = p.scale * 1.4426950408889634f;
 #pragma unroll
         for (int s = 0; s < NSTEP; ++s) {
-            vec8 x = *(const vec8*)(krow + s * 16);
+            vec8 x, y;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) { x[e] = (T)0.0f; y[e] = (T)0.0f; }
+            if (s * 16 + g * 8 < p.D) x = *(const vec8*)(krow + s * 16);
+            if (s * 16 + g * 8 < p.Dv) y = *(const vec8*)(vrow + s * 16);
 #pragma unroll
             for (int e = 0; e < 8; ++e) x[e] = (T)((float)x[e] * c2);
             kreg[s] = x;
-            vreg[s] = *(const vec8*)(vrow + s * 16);
+            vreg[s] = y;
         }
     }
     // rows i >= lo_i see this lane's key under the causal mask
@@ -389,8 +402,8 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
         nx_g = (const char*)bp.d_o + ((int64_t)b * bp.do_sb + (int64_t)hq * bp.do_sh + (int64_t)r0 * bp.do_ss) * 2;
         nx_s = (const char*)((wave == 0 ? bp.neg_l2 : bp.neg_delta) + ((int64_t)b * p.Hq + hq) * Sq + r0);
         nx_rows = rows_b - r0;
-        nx_qrem = (int64_t)(nx_rows - 1) * p.q_ss * 2 + D * 2;
-        nx_grem = (int64_t)(nx_rows - 1) * bp.do_ss * 2 + D * 2;
+        nx_qrem = (int64_t)(nx_rows - 1) * p.q_ss * 2 + p.D * 2;
+        nx_grem = (int64_t)(nx_rows - 1) * bp.do_ss * 2 + p.Dv * 2;
         nx_r = 0;
         nx_h = h;
     };
@@ -549,8 +562,9 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
                     wk[e] = (T)(my_j < kv_len ? dk_acc[d][r4 * 4 + e] * p.scale : 0.0f);
                     wv[e] = (T)(my_j < kv_len ? dv_acc[d][r4 * 4 + e] : 0.0f);
                 }
-                *(vec4*)(krow + d * 32 + r4 * 8 + g * 4) = wk;
-                *(vec4*)(vrow + d * 32 + r4 * 8 + g * 4) = wv;
+                const int col = role * (D / 2) + d * 32 + r4 * 8 + g * 4;
+                if (col < p.D) *(vec4*)(krow + d * 32 + r4 * 8 + g * 4) = wk;
+                if (col < p.Dv) *(vec4*)(vrow + d * 32 + r4 * 8 + g * 4) = wv;
             }
     }
 #endif
@@ -576,11 +590,12 @@ static hipError_t launch_bwd_t(const SdpaBwdParams& bp, hipStream_t stream)
     return hipGetLastError();
 }
 
-// Host has validated: dtype f16/bf16, D == Dv in {64, 128}, no dense mask, unit last-axis strides, 16-byte aligned rows,
+// Host has validated: dtype f16/bf16, D and Dv <= 128 in whole 16-byte vectors (bp.f.Dp = the instance: 64 or 128; smaller
+// or unequal head dimensions are zero-padded on the way into LDS and registers, stores are cut), no dense mask, unit last-axis strides, 16-byte aligned rows,
 // row strides below 2^24 elements, lse and the delta workspace present.
 hipError_t launch_sdpa_bwd_mfma(const SdpaBwdParams& bp, int dtype, hipStream_t stream)
 {
-    if (bp.f.D == 128) return dtype == 1 ? launch_bwd_t<f16_t, 128>(bp, stream) : launch_bwd_t<bf16_t, 128>(bp, stream);
+    if (bp.f.Dp == 128) return dtype == 1 ? launch_bwd_t<f16_t, 128>(bp, stream) : launch_bwd_t<bf16_t, 128>(bp, stream);
     return dtype == 1 ? launch_bwd_t<f16_t, 64>(bp, stream) : launch_bwd_t<bf16_t, 64>(bp, stream);
 }
 

@@ -231,9 +231,9 @@ int incin_rocm_sdpa_fwd_static(const incin_rocm_sdpa_desc_t* desc, void* stream)
  * kv_lens and the grouped-query layout carry over; d_k and d_v are summed over the query heads of a group.
  * Covered: f32 / f16 / bf16, D and Dv up to 256, dense additive mask, causal, kv_lens, q_lens (padding query rows: their
  * O, lse and d_o rows are never read, their d_q rows are written as zero and they add nothing to d_k and d_v).
- * fwd.impl picks the kernels: AUTO = matrix-core kernels where they apply - f16 / bf16 with D == Dv in {64, 128} and a positive
- * scale, f32 (IEEE single-precision matrix instructions) with D == Dv in {64, 128} and any finite scale; both without a
- * dense mask and with 16-byte aligned rows - and generic f32-arithmetic kernels otherwise; GENERIC and MFMA pin one or
+ * fwd.impl picks the kernels: AUTO = matrix-core kernels where they apply - D and Dv up to 128 in whole 16-byte vectors (zero-padded
+ * into instances for 64 and 128); f16 / bf16 with a positive scale, f32 (IEEE single-precision matrix instructions) with any finite
+ * scale; both without a dense mask and with 16-byte aligned rows - and generic f32-arithmetic kernels otherwise; GENERIC and MFMA pin one or
  * the other.  A query row with no visible key (NaN in the forward) gets a zero gradient and
  * contributes nothing to d_k and d_v, where the reference's tape would spread NaN over the whole head.
  * The workspace holds two floats per query row (2 x [B, Hq, Sq]; ask incin_rocm_sdpa_bwd_workspace for the size);

@@ -225,8 +225,9 @@ def test_backward_validation_and_workspace_size():
     for bd, code in [
         (_bwd(dict(lse=None)), capi.EINVAL),                          # the forward's normalisers are an input
         (_bwd(d_k=None), capi.EINVAL),
-        (_bwd(dict(impl=capi.IMPL_MFMA, D=32, Dv=32)), capi.EUNSUPPORTED),           # pinned to kernels that do not take it
-        (_bwd(dict(impl=capi.IMPL_MFMA, dtype=capi.F32, D=32, Dv=32)), capi.EUNSUPPORTED),
+        (_bwd(dict(impl=capi.IMPL_MFMA, D=160, Dv=160)), capi.EUNSUPPORTED),         # pinned to kernels that do not take it
+        (_bwd(dict(impl=capi.IMPL_MFMA, D=36, Dv=36)), capi.EUNSUPPORTED),           # (72-byte rows are not whole vectors)
+        (_bwd(dict(impl=capi.IMPL_MFMA, dtype=capi.F32, D=160, Dv=160)), capi.EUNSUPPORTED),
         (_bwd(dict(impl=capi.IMPL_MFMA, add_mask=0x20000)), capi.EUNSUPPORTED),
         (_bwd(dict(impl=capi.IMPL_SPLITKV)), capi.EUNSUPPORTED),
         (_bwd(dict(D=320, Dv=320)), capi.EUNSUPPORTED),

@@ -161,6 +161,28 @@ def test_generic_backward_f32_against_the_oracle(gpu, shape):
     compare("dv", dv, rv.reshape(B, Hkv, Skv, Dv), tol=1e-5)
 
 
+@pytest.mark.parametrize("dtype,dims", [(capi.BF16, (96, 96)), (capi.BF16, (40, 72)), (capi.F16, (128, 64)), (capi.BF16, (8, 8)), (capi.F16, (80, 80)),
+                                        (capi.F32, (96, 96)), (capi.F32, (20, 36)), (capi.F32, (128, 64)), (capi.F32, (4, 4))],
+                         ids=lambda x: dtypes.NAMES[x] if isinstance(x, int) else "D%d_Dv%d" % x)
+def test_matrix_core_backward_with_padded_head_dimensions(gpu, dtype, dims):
+    """Head dimensions up to 128 in whole 16-byte vectors, D and Dv not necessarily equal, through the matrix-core backward
+    kernels (pinned, and AUTO must pick them): zero-padded into the 64 / 128 instances, gradient stores cut at D and Dv."""
+    D, Dv = dims
+    tol = 1e-5 if dtype == capi.F32 else 2e-2
+    for B, Hq, Hkv, Sq, Skv, causal, lens in ((2, 4, 2, 150, 200, True, [200, 77]), (1, 2, 2, 70, 70, False, None)):
+        G = Hq // Hkv
+        say("padded backward: %s D=%d Dv=%d %r" % (dtypes.NAMES[dtype], D, Dv, (B, Hq, Hkv, Sq, Skv)))
+        q, k, v, go = make_d(61 + D, B, Hq, Hkv, Sq, Skv, D, Dv, dtype)
+        lens_a = None if lens is None else np.asarray(lens, np.int32)
+        out, dq, dk, dv = host.sdpa_backward(q, k, v, go, dtype, causal=causal, kv_lens=lens_a, impl=capi.IMPL_MFMA)
+        auto = host.sdpa_backward(q, k, v, go, dtype, causal=causal, kv_lens=lens_a)
+        rq, rk, rv = BW.sdpa_backward(q.reshape(B, Hkv, G, Sq, D), k[:, :, None], v[:, :, None], go.reshape(B, Hkv, G, Sq, Dv),
+                                      causal=causal, kv_lens=None if lens is None else lens_a.reshape(B, 1, 1))
+        for name, x, a, r_ in zip(("dq", "dk", "dv"), (dq, dk, dv), auto[1:], (rq.reshape(B, Hq, Sq, D), rk.reshape(B, Hkv, Skv, D), rv.reshape(B, Hkv, Skv, Dv))):
+            compare(name, x, r_, tol=tol)
+            assert np.array_equal(x, a), name + ": AUTO takes the same kernels"
+
+
 @pytest.mark.parametrize("shape", [
     # B, Hq, Hkv, Sq, Skv, D, causal, kv_lens, scale
     (1, 1, 1, 32, 32, 64, False, None, None),
@@ -267,8 +289,8 @@ def test_generic_and_matrix_core_backward_agree(gpu, dtype, D):
 
 
 def test_backward_refuses_what_it_does_not_cover(gpu):
-    q, k, v, go = make(14, 1, 1, 1, 32, 32, 32, capi.BF16)
-    with pytest.raises(capi.RocmError) as e:                     # the matrix-core kernels, pinned, outside their domain
+    q, k, v, go = make(14, 1, 1, 1, 32, 32, 36, capi.BF16)
+    with pytest.raises(capi.RocmError) as e:                     # the matrix-core kernels, pinned, outside their domain (72-byte rows)
         host.sdpa_backward(q, k, v, go, capi.BF16, impl=capi.IMPL_MFMA)
     assert e.value.code == capi.EUNSUPPORTED
     q, k, v, go = make(14, 1, 1, 1, 8, 8, 320, capi.F32)         # wider than any kernel
