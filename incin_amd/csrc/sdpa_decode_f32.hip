@@ -69,7 +69,9 @@ __global__ __launch_bounds__(256) void sdpa_decode_f32_kernel(SdpaParams p)
     const int R = p.G * Sq;
     const int nchunks = (R + CHUNK - 1) / CHUNK;
     const int split = blockIdx.x;
-    const int hkv = blockIdx.y / nchunks, r0 = (blockIdx.y % nchunks) * CHUNK;
+    int hkv, chunk_id;
+    decode_work_item(nchunks, &hkv, &chunk_id);
+    const int r0 = chunk_id * CHUNK;
     const int b = blockIdx.z;
 
     int kv_len = Skv;

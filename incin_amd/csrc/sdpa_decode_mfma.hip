@@ -51,7 +51,9 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
     constexpr int CHUNK = 32 * NRB;                    // rows per workgroup
     const int nchunks = (R + CHUNK - 1) / CHUNK;
     const int split = blockIdx.x;
-    const int hkv = blockIdx.y / nchunks, r0 = (blockIdx.y % nchunks) * CHUNK;
+    int hkv, chunk_id;
+    decode_work_item(nchunks, &hkv, &chunk_id);
+    const int r0 = chunk_id * CHUNK;
     const int b = blockIdx.z;
 
     int kv_len = Skv;

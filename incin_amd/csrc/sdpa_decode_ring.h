@@ -36,4 +36,22 @@ template <int NSLOT, int CPB = 8> __device__ __forceinline__ void wait_oldest_co
     else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
 }
 
+// Which (KV head, chunk of rows) a workgroup of the split-KV matrix-core kernels takes, from blockIdx.y.  With several
+// chunks per KV head (prefill shapes through these kernels) the chunks of a head read the same keys and values: workgroups
+// reach the 8 XCDs round-robin in dispatch order, so an unsplit launch hands each XCD a contiguous eighth of the list
+// (a head's chunks then meet in one L2 instead of all eight), and the chunks of a head go last-first (under a causal
+// mask the last rows see the most keys: longest first).
+__device__ __forceinline__ void decode_work_item(int nchunks, int* hkv, int* chunk)
+{
+    int y = blockIdx.y;
+    if (nchunks > 1) {
+        if (gridDim.x == 1 && (gridDim.y & 7) == 0) y = (y & 7) * (int)(gridDim.y >> 3) + (y >> 3);
+        *hkv = y / nchunks;
+        *chunk = nchunks - 1 - y % nchunks;
+    } else {
+        *hkv = y;
+        *chunk = 0;
+    }
+}
+
 }  // namespace incin_rocm
