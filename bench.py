@@ -243,6 +243,35 @@ def decode_gqa_leg(steps, warmup, only_shape=None):
     return out
 
 
+def head_dims_leg(steps, warmup):
+    """Head dimensions other than 64 and 128 (bf16): D = 96 runs zero-padded in the 128 instances of the prefill and split-KV
+    kernels, D = 256 in the 256 instance of the split-KV kernel (prefill shapes too).  Prefill: useful FLOPs (4 D per visible
+    pair) against the bf16 matrix peak; decode: KV bytes read once against the HBM peak."""
+    out = {}
+    names = {capi.IMPL_SPLITKV_MFMA: "sdpa_decode_mfma_kernel", capi.IMPL_MFMA: "sdpa_prefill_mfma_kernel", capi.IMPL_GENERIC: "sdpa_generic_kernel"}
+    for i, (name, B, Hq, Hkv, Sq, Skv, D, causal) in enumerate((("prefill_d96", 8, 16, 16, 2048, 2048, 96, True), ("prefill_d256", 4, 16, 16, 4096, 4096, 256, True),
+                                                                 ("decode_d96", 32, 32, 8, 1, 8192, 96, False), ("decode_d256", 32, 32, 8, 1, 8192, 256, False))):
+        w = Workload("head_dims_" + name, SEED0 + 80 + i, B, Hq, Hkv, Sq, Skv, D, capi.BF16, causal)
+        wall, ev_mean, ev_med, ev_min = w.time(max(steps, 50), warmup)
+        entry = {"workload": "bf16 %s B=%d Hq=%d Hkv=%d S_q=%d KV=%d D=%d" % ("causal prefill" if Sq > 1 else "decode", B, Hq, Hkv, Sq, Skv, D),
+                 "kernel": names.get(w.impl, str(w.impl)), "num_splits": w.splits, "ms_per_step": wall, "parity_max_abs_err": w.parity(16)}
+        if Sq > 1:
+            flops = causal_flops(B, Hq, Sq, Skv, D)
+            entry["tflops"] = flops / (wall * 1e-3) / 1e12
+            entry["roofline"] = {"bound": "mfma", "achieved": flops / (ev_mean * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                                 "frac": flops / (ev_mean * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": None,
+                                 "algorithmic_flops_per_launch": flops, "launch_ms_mean": ev_mean, "launch_ms_min": ev_min}
+        else:
+            kv_bytes = 2.0 * B * Hkv * Skv * D * 2
+            entry["kv_gb_per_s"] = kv_bytes / (wall * 1e-3) / 1e9
+            entry["roofline"] = {"bound": "hbm", "achieved": kv_bytes / (ev_mean * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                 "frac": kv_bytes / (ev_mean * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None,
+                                 "algorithmic_bytes_per_launch": kv_bytes, "launch_ms_mean": ev_mean, "launch_ms_min": ev_min}
+        w.free()
+        out[name] = entry
+    return out
+
+
 def decode_step_graph(w, B, H, Skv, D, steps):
     """One decode step as a serving loop runs it: append the token's K and V rows to the cache at kv_lens (device side),
     attend over the cache with kv_lens; both recorded into a launch graph once and replayed per token."""
@@ -488,7 +517,7 @@ def main():
                     help="prefill_long: skip the extra timing of the batch with its padding rows computed (profiling: every "
                          "launch of the run is then the same launch)")
     ap.add_argument("--decode-gqa-shape", default=None, help="with --only decode_gqa: one of its shapes by name (for profiles)")
-    ap.add_argument("--only", choices=["prefill", "prefill_long", "prefill_chunk", "decode", "decode_gqa", "backward", "f32", "copy", "matrix_rate", "read_rate"], default=None,
+    ap.add_argument("--only", choices=["prefill", "prefill_long", "prefill_chunk", "decode", "decode_gqa", "head_dims", "backward", "f32", "copy", "matrix_rate", "read_rate"], default=None,
                     help="run a single workload (profiling). 'copy' runs --steps device-to-device copies of 1 GiB "
                          "through the library's plain copy kernel: the known-size dispatch that hardware byte "
                          "counters (FETCH_SIZE / WRITE_SIZE) are calibrated against")
@@ -636,6 +665,9 @@ def main():
 
     if args.only in (None, "decode_gqa"):
         result["decode_gqa"] = decode_gqa_leg(args.steps, args.warmup, args.decode_gqa_shape)
+
+    if args.only in (None, "head_dims"):
+        result["head_dims"] = head_dims_leg(args.steps, args.warmup)
 
     if args.only in (None, "f32"):
         result.update(f32_configs(args.steps, args.warmup, not args.no_cpu_baseline, threads))
