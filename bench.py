@@ -81,6 +81,18 @@ class Workload:
         if self.ws is not None:
             self.desc.workspace, self.desc.workspace_bytes = self.ws.ptr, self.ws.nbytes
 
+    def replan(self, impl=capi.IMPL_AUTO, num_splits=0):
+        """The same operands through another kernel or split count (generating and uploading gigabytes of cache again
+        would cost more than the measurement)."""
+        if self.ws is not None:
+            self.ws.free()
+        self.desc.impl, self.desc.num_splits = impl, num_splits
+        self.desc.workspace, self.desc.workspace_bytes = None, 0
+        nbytes, self.splits, self.impl = capi.sdpa_workspace(self.desc)
+        self.ws = capi.DeviceBuffer(nbytes) if nbytes else None
+        if self.ws is not None:
+            self.desc.workspace, self.desc.workspace_bytes = self.ws.ptr, self.ws.nbytes
+
     def launch(self):
         capi.sdpa_fwd(self.desc)
 
@@ -226,10 +238,12 @@ def decode_gqa_leg(steps, warmup, only_shape=None):
         kv_bytes = 2.0 * B * Hkv * Skv * 128 * (4 if dt == F else 2)
         n = max(steps, min(200, int(0.02 / (kv_bytes / 6e12))))
         entry = {"workload": "%s decode B=%d Hq=%d Hkv=%d S_q=%d KV=%d D=128%s" % (dtypes.NAMES[dt], B, Hq, Hkv, Sq, Skv, " causal" if causal else "")}
+        w = Workload("decode_" + name, SEED0 + 40 + i, B, Hq, Hkv, Sq, Skv, 128, dt, causal)
         for impl in (capi.IMPL_AUTO, capi.IMPL_SPLITKV):
             if impl == capi.IMPL_SPLITKV and (Hq // Hkv) * Sq > 8:
                 continue
-            w = Workload("decode_" + name, SEED0 + 40 + i, B, Hq, Hkv, Sq, Skv, 128, dt, causal, impl=impl)
+            if impl != capi.IMPL_AUTO:
+                w.replan(impl=impl)
             wall, ev_mean, ev_med, ev_min = w.time(n, warmup)
             entry["auto" if impl == capi.IMPL_AUTO else "vector_alu_kernel"] = {
                 "kernel": (names_f32 if dt == F else names).get(w.impl, str(w.impl)), "num_splits": w.splits, "ms_per_step": wall,
@@ -238,7 +252,7 @@ def decode_gqa_leg(steps, warmup, only_shape=None):
                              "frac": kv_bytes / (ev_mean * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None,
                              "algorithmic_bytes_per_launch": kv_bytes, "launch_ms_mean": ev_mean, "launch_ms_min": ev_min},
                 "parity_max_abs_err": w.parity(16)}
-            w.free()
+        w.free()
         out[name] = entry
     return out
 
@@ -507,6 +521,14 @@ def f32_configs(steps, warmup, with_cpu, threads):
     return out
 
 
+_T0 = time.perf_counter()
+
+
+def note(leg):
+    """Progress on stderr (stdout carries the one JSON line): a run that prints nothing for minutes looks hung to a harness."""
+    print("[bench %6.1f s] %s" % (time.perf_counter() - _T0, leg), file=sys.stderr, flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -558,6 +580,7 @@ def main():
         return 0
 
     if args.only in (None, "prefill"):
+        note("prefill")
         B, H, S, D = 8, 16, 4096, 128
         w = Workload("prefill_c3", SEED0 + 2, B, H, H, S, S, D, capi.BF16, True)
         wall, ev_mean, ev_med, ev_min = w.time(args.steps, args.warmup)
@@ -599,6 +622,7 @@ def main():
                           % (slices, threads, dt, host_cpu())}
 
     if args.only in (None, "prefill_long"):
+        note("prefill_long")
         # BASELINE config 5: grouped queries, batch padded to 16384 tokens, causal + key padding; lengths U[2048, 16384]
         # from the same seeded generator
         B, Hq, Hkv, S, D = 4, 32, 8, 16384, 128
@@ -629,6 +653,7 @@ def main():
         w.free()
 
     if args.only in (None, "decode"):
+        note("decode")
         B, H, Skv, D = 32, 32, 8192, 128
         w = Workload("decode_c4", SEED0 + 3, B, H, H, 1, Skv, D, capi.BF16, False)
         wall, ev_mean, ev_med, ev_min = w.time(args.steps, args.warmup)
@@ -644,14 +669,15 @@ def main():
                             "algorithmic_bytes_per_launch": kv_bytes,
                             "launch_ms_mean": ev_mean, "launch_ms_median": ev_med, "launch_ms_min": ev_min},
                "parity_max_abs_err": w.parity()}
-        dec["decode_step_graph"] = decode_step_graph(w, B, H, Skv, D, args.steps)
-        w.free()
-        # the same through the vector-ALU split-KV kernel (what f32 caches and short caches run on)
-        w = Workload("decode_c4", SEED0 + 3, B, H, H, 1, Skv, D, capi.BF16, False, impl=capi.IMPL_SPLITKV)
+        # the same through the vector-ALU split-KV kernel (what one row per KV head over short caches runs on)
+        w.replan(impl=capi.IMPL_SPLITKV)
         wall_v, ev_v, _, _ = w.time(args.steps, args.warmup)
         dec["vector_alu_kernel"] = {"kernel": "sdpa_decode_split_kernel<bf16,128,1,8> + sdpa_combine_kernel", "num_splits": w.splits,
                                     "ms_per_step": wall_v, "launch_ms_mean": ev_v, "frac": kv_bytes / (ev_v * 1e-3) / 1e9 / PEAK_HBM_GBS,
                                     "parity_max_abs_err": w.parity()}
+        # (last: the appended rows overwrite the end of the cache)
+        w.replan()
+        dec["decode_step_graph"] = decode_step_graph(w, B, H, Skv, D, args.steps)
         w.free()
         if not args.no_cpu_baseline:
             val, dt = cpu_baseline_decode(D, Skv, 32, 32, capi.BF16)
@@ -661,24 +687,31 @@ def main():
         result["decode"] = dec
 
     if args.only in (None, "prefill_chunk"):
+        note("prefill_chunk")
         result["prefill_chunk"] = prefill_chunk_leg(args.steps, args.warmup)
 
     if args.only in (None, "decode_gqa"):
+        note("decode_gqa")
         result["decode_gqa"] = decode_gqa_leg(args.steps, args.warmup, args.decode_gqa_shape)
 
     if args.only in (None, "head_dims"):
+        note("head_dims")
         result["head_dims"] = head_dims_leg(args.steps, args.warmup)
 
     if args.only in (None, "f32"):
+        note("f32")
         result.update(f32_configs(args.steps, args.warmup, not args.no_cpu_baseline, threads))
 
     if args.only in (None, "matrix_rate"):
+        note("matrix_rate")
         result["matrix_rate"] = matrix_rate()
 
     if args.only in (None, "read_rate"):
+        note("read_rate")
         result["read_rate"] = read_rate()
 
     if args.only in (None, "backward"):
+        note("backward")
         result["backward"] = backward_leg(max(5, min(args.steps, 30)), min(args.warmup, 5))
         # f32, the dtype the reference trains in: BASELINE config 2's shape (launches of ~100 us) and config 3's
         result["backward_d64"] = backward_leg(max(5, min(args.steps, 30)), min(args.warmup, 5), capi.BF16, 8, 32, 4096, 64, "config 3 with 32 heads of 64 (the same FLOPs)")
