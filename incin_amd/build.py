@@ -12,7 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libincin_rocm.so")
-SOURCES = ["incin_rocm.hip", "sdpa_generic.hip", "sdpa_decode.hip", "sdpa_decode_mfma.hip", "sdpa_decode_f32.hip", "sdpa_prefill_mfma.hip", "sdpa_prefill_f32.hip", "sdpa_bwd_f32.hip", "mask_blocks.hip", "matrix_rate.hip", "copy.hip", "kv_append.hip", "sdpa_bwd_mfma.hip", "sdpa_bwd_generic.hip"]
+SOURCES = ["incin_rocm.hip", "sdpa_generic.hip", "sdpa_decode.hip", "sdpa_decode_mfma.hip", "sdpa_decode_f32.hip", "sdpa_prefill_mfma.hip", "sdpa_prefill_wide.hip", "sdpa_prefill_f32.hip", "sdpa_bwd_f32.hip", "mask_blocks.hip", "matrix_rate.hip", "copy.hip", "kv_append.hip", "sdpa_bwd_mfma.hip", "sdpa_bwd_generic.hip"]
 # per-file flags.  The split-KV matrix-core kernel keeps its accumulators in ordinary vector registers: it rescales them
 # only when a reference maximum moves, and with accumulation registers the compiler copies all of them out and back
 # around that rare branch on every key block.

@@ -23,6 +23,7 @@ hipError_t launch_sdpa_generic(const SdpaParams& p, int dtype, hipStream_t strea
 hipError_t launch_sdpa_prefill_mfma(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_matrix_rate(const void* src, void* sink, int mix, int iterations, double* flops, hipStream_t stream);
 hipError_t launch_sdpa_prefill_f32(const SdpaParams& p, hipStream_t stream);
+hipError_t launch_sdpa_prefill_wide(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_mask_classify(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_sdpa_decode(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_sdpa_decode_mfma(const SdpaParams& p, int dtype, hipStream_t stream);
@@ -168,7 +169,9 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     const bool tile_off_ok = d->k_stride[2] >= 0 && d->v_stride[2] >= 0 && d->k_stride[2] < stride_lim && d->v_stride[2] < stride_lim;
     // f32: the IEEE-f32 matrix-core kernel, any finite scale; f16 / bf16: the 16-bit kernels fold the scale into Q in
     // a way that needs it positive.  Both take a dense additive mask (any strides); the 64-row kernel does not.
-    const bool mfma_ok = layout_ok && !wide && tile_off_ok && std::isfinite(d->scale) && (d->dtype == INCIN_ROCM_F32 || d->scale > 0.0f);
+    // (above 128: sdpa_prefill_wide.hip - 16-bit storage, no dense mask, any finite scale)
+    const bool mfma_ok = wide ? fast_ok && d->dtype != INCIN_ROCM_F32 && tile_off_ok && std::isfinite(d->scale)
+                              : layout_ok && tile_off_ok && std::isfinite(d->scale) && (d->dtype == INCIN_ROCM_F32 || d->scale > 0.0f);
     const bool split_ok = fast_ok && head_exact && d->Sq <= 64;
     // the matrix-core split-KV kernels (16-bit and f32): blocks addressed like the prefill kernels' tiles
     const bool split_mfma_ok = fast_ok && (d->Sq <= 64 || wide) && tile_off_ok && std::isfinite(d->scale);
@@ -195,7 +198,10 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         // against 0.28 ms on 8 x 8 heads x 8192 keys); the vector-ALU kernel is level at 2 rows and behind from 4 on
         // (4 rows, 268 MB of cache: 5.6 against 4.8 TB/s; 8 rows: 6.6 against 3.4).  More than 32 rows over fewer than 512
         // keys stay with the prefill kernel (64 positions x 16 heads x 64 sequences of 256 keys: 0.14 against 0.17 ms).
-        if (wide && split_mfma_ok) impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
+        // above 128: the split-KV kernels' 256 instance for decode shapes (and for f32 whatever the shape), the 16-bit
+        // prefill kernel for 256 where there are more than 64 positions (128 rows share a K / V tile there instead of 32)
+        if (wide && mfma_ok && d->Sq > 64) impl = INCIN_ROCM_IMPL_MFMA;
+        else if (wide && split_mfma_ok) impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
         else if (d->dtype == INCIN_ROCM_F32 && split_mfma_ok && len128 >= 256 && R >= 2 && (R <= 32 || d->Skv >= 512))
             impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
         else if (d->dtype != INCIN_ROCM_F32 && split_mfma_ok && len128 >= 256 &&
@@ -211,7 +217,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     }
     if (impl == INCIN_ROCM_IMPL_MFMA && !mfma_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
-                    "scaled_dot_product_attention: the MFMA prefill kernels need D and Dv <= 128 in whole 16-byte vectors and 16-byte aligned rows; for f16/bf16 also scale > 0");
+                    "scaled_dot_product_attention: the MFMA prefill kernels need D and Dv <= 128 (f16/bf16 without a dense mask: 256) in whole 16-byte vectors and 16-byte aligned rows; for f16/bf16 up to 128 also scale > 0");
     if (impl == INCIN_ROCM_IMPL_MFMA64)
         return fail(INCIN_ROCM_EUNSUPPORTED,
                     "scaled_dot_product_attention: the 64-row MFMA prefill kernel has been retired (INCIN_ROCM_IMPL_MFMA covers its shapes)");
@@ -283,7 +289,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         plan->split_len = (int)split_len;
         plan->ws_bytes = splits > 1 ? (size_t)(d->B * d->Hq * d->Sq * splits) * (size_t)(d_pad + 2) * sizeof(float) : 0;
     }
-    if (impl == INCIN_ROCM_IMPL_MFMA && !d->add_mask && !d->q_lens) {
+    if (impl == INCIN_ROCM_IMPL_MFMA && !d->add_mask && !d->q_lens && !wide) {
         // The prefill kernels (16-bit and f32) run one workgroup per (batch, query head, 128 rows) and a compute unit holds two:
         // when a launch has at most one per compute unit and a long key axis - a chunk of a long prompt, a single
         // sequence - the keys are split as for decode, as many ways as fill the device (1024 keys per split at least:
@@ -639,7 +645,9 @@ static int launch_fwd(const incin_rocm_sdpa_desc_t* desc, const Plan& plan, void
                 e = incin_rocm::launch_mask_classify(p, desc->dtype, s);
                 if (e != hipSuccess) break;
             }
-            e = desc->dtype == INCIN_ROCM_F32 ? incin_rocm::launch_sdpa_prefill_f32(p, s) : incin_rocm::launch_sdpa_prefill_mfma(p, desc->dtype, s);
+            e = p.Dp == 256                    ? incin_rocm::launch_sdpa_prefill_wide(p, desc->dtype, s)
+                : desc->dtype == INCIN_ROCM_F32 ? incin_rocm::launch_sdpa_prefill_f32(p, s)
+                                                : incin_rocm::launch_sdpa_prefill_mfma(p, desc->dtype, s);
             break;
         case INCIN_ROCM_IMPL_SPLITKV: e = incin_rocm::launch_sdpa_decode(p, desc->dtype, s); break;
         case INCIN_ROCM_IMPL_SPLITKV_MFMA: e = incin_rocm::launch_sdpa_decode_mfma(p, desc->dtype, s); break;

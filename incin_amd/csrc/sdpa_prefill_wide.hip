@@ -1,0 +1,249 @@
+// bf16 / f16 attention forward on the gfx950 matrix cores for head dimensions above 128 (up to 256, D and Dv in whole
+// 16-byte vectors, zero-padded into the 256 instance on the way into LDS) on prefill shapes: the function of the
+// reference CPU composition (crates/incin-backends/src/cpu/ops/shape_ops.rs:1245-1269), optional causal mask, per-batch
+// key and query lengths, MHA and GQA.
+//
+// Decode shapes at these head dimensions run on the split-KV kernel's 256 instance (sdpa_decode_mfma.hip), and so did
+// prefill shapes before this kernel: 32 rows per workgroup there, each workgroup streaming K and V for itself, which
+// makes the traffic between L2 and LDS the bound (340 - 460 TFLOP/s).  Here a workgroup is 4 wavefronts = 128 query
+// rows sharing every K / V tile, the shape of sdpa_prefill_mfma.hip with the operand layouts of sdpa_decode_mfma.hip:
+//
+//   S^T = K_tile Q^T     v_mfma_f32_32x32x16 over the 16 k-steps of 256 elements: A = K rows from LDS (16-byte reads),
+//                        B = Q^T resident in registers (64 of them); a lane owns one query and 16 keys of the tile.
+//   softmax              scale applied to the f32 scores (any finite scale), masks as -inf before the maximum, the
+//                        reference maximum moved lazily (threshold 2^8), P rounded to the storage type in registers.
+//   O^T += V^T P^T       A = V^T through the transposing LDS read, 8 blocks of 32 columns: 128 accumulator registers.
+//
+// A tile is 32 keys (16 KiB of K, 16 KiB of V), two buffers each: 64 KiB of LDS and 256 registers per lane, so two
+// workgroups share a compute unit and one's softmax runs beside the other's matrix instructions.  One barrier per tile:
+// it publishes tile t, whose copies (global -> LDS, no register staging) were started an iteration earlier, and frees
+// the buffers of tile t - 1 for the copies of tile t + 1.  The loop is the plain one - with two matrix instructions per
+// key and row where head dimension 128 has one, the vector work between them weighs half as much.
+#include "sdpa_mfma_common.h"
+
+namespace incin_rocm {
+
+constexpr int PW_KT = 32;      // keys per tile
+
+template <typename T>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void sdpa_prefill_wide_kernel(SdpaParams p)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef typename Mma<T>::vec8 vec8;
+    constexpr int D = 256;
+    typedef PfLayout<D> L;
+    constexpr int NSTEP = D / 16, NDB = D / 32;
+    constexpr int TILE = PW_KT * L::ROWB;              // 16 KiB
+    constexpr int LPW = TILE / 1024 / 4;               // wavefront-wide 1 KiB copies per tensor per tile: 4
+    __shared__ __attribute__((aligned(1024))) char smem[4 * TILE];      // K buffers 0, 1, V buffers 0, 1
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ql = lane & 31, g = lane >> 5;
+    const int Sq = p.Sq, Skv = p.Skv;
+
+    // ---- which (batch, head, query block): the work order of the other prefill kernels ---------------------------------
+    const int nqb = (Sq + PF_BM - 1) / PF_BM;
+    const int total = gridDim.x;
+    const WorkItem wi = (total & 7) == 0 ? work_item_of_share(blockIdx.x & 7, blockIdx.x >> 3, total >> 3, p.interleave, p.G, nqb, p.deal_groups)
+                                         : work_item(blockIdx.x, p.interleave, p.G, nqb);
+    const int hkv = wi.bhkv % p.Hkv, b = wi.bhkv / p.Hkv;
+    const int hq = hkv * p.G + wi.gq;
+    const int q0 = wi.qblk * PF_BM;
+
+    const T* qp = (const T*)p.q + (int64_t)b * p.q_sb + (int64_t)hq * p.q_sh;
+    const T* kp = (const T*)p.k + (int64_t)b * p.k_sb + (int64_t)hkv * p.k_sh;
+    const T* vp = (const T*)p.v + (int64_t)b * p.v_sb + (int64_t)hkv * p.v_sh;
+    T* op = (T*)p.o + (int64_t)b * p.o_sb + (int64_t)hq * p.o_sh;
+
+    int kv_len = Skv;
+    if (p.kv_lens) kv_len = clampi(p.kv_lens[b], 0, Skv);
+    const int rows_b = p.q_lens ? clampi(p.q_lens[b], 0, Sq) : Sq;      // query rows at and beyond are padding
+    if (q0 >= rows_b) return;                                           // (uniform: before any barrier)
+    const int coff = Skv - Sq;
+    int j_end = kv_len;
+    const int my_i = q0 + wave * 32 + ql;
+    int lim_lane = kv_len, lim_wave_min = kv_len, lim_wave_max = kv_len;
+    if (p.causal) {
+        const int last_row = min(q0 + PF_BM - 1, rows_b - 1);
+        j_end = clampi(last_row + coff + 1, 0, kv_len);
+        lim_lane = clampi(my_i + coff + 1, 0, kv_len);
+        lim_wave_min = clampi(q0 + wave * 32 + coff + 1, 0, kv_len);
+        lim_wave_max = clampi(min(q0 + wave * 32 + 31, rows_b - 1) + coff + 1, 0, kv_len);
+    }
+    if (q0 + wave * 32 >= rows_b) lim_wave_min = lim_wave_max = 0;      // a wavefront of padding rows only keeps the barriers company
+    const int n_tiles = (j_end + PW_KT - 1) / PW_KT;
+    const int n_act = lim_wave_max > 0 ? (lim_wave_max + PW_KT - 1) / PW_KT : 0;      // tiles this wavefront computes
+
+    // ---- global -> LDS copy plan: wavefront-wide load ii = wave * LPW + c fills LDS bytes [ii * 1024, +1024) of a tile ----
+    int k_voff[LPW], v_voff[LPW];
+#pragma unroll
+    for (int c = 0; c < LPW; ++c) {
+        const int pos = (wave * LPW + c) * 64 + lane;
+        const int row = pos / L::CPR, slot = pos % L::CPR;
+        k_voff[c] = dma_chunk_offset(row, (int)p.k_ss * 2, slot ^ L::fk(row), p.D * 2);
+        v_voff[c] = dma_chunk_offset(row, (int)p.v_ss * 2, slot ^ L::fv(row), p.Dv * 2);
+    }
+    const int64_t k_tile_bytes = (int64_t)PW_KT * p.k_ss * 2, v_tile_bytes = (int64_t)PW_KT * p.v_ss * 2;
+    auto issue = [&](const T* base, int64_t tile_bytes, int64_t row_stride, int row_elems, int t, int buf, const int (&voff)[LPW]) __attribute__((always_inline)) {
+        // bytes to the end of the last row this workgroup may see: loads past that return 0 (rows past a batch entry's
+        // key count are never read)
+        int64_t rem = (int64_t)(j_end - t * PW_KT - 1) * row_stride * 2 + row_elems * 2;
+        if (rem > 0x7fffffffLL) rem = 0x7fffffffLL;
+        const uint4v r = dma_descriptor((const char*)base + t * tile_bytes, (int)rem);
+        const unsigned dst = lds_address(smem) + buf * TILE + wave * LPW * 1024;
+#pragma unroll
+        for (int c = 0; c < LPW; ++c) dma_copy16(r, dst + c * 1024, voff[c]);
+    };
+    auto issue_kv = [&](int t) __attribute__((always_inline)) {
+        issue(kp, k_tile_bytes, p.k_ss, p.D, t, t & 1, k_voff);
+        issue(vp, v_tile_bytes, p.v_ss, p.Dv, t, 2 + (t & 1), v_voff);
+    };
+    if (n_tiles > 0) issue_kv(0);
+
+    // ---- operands ----------------------------------------------------------------------------------------------
+    // Q^T (B operand, resident): this lane's row, elements 16 s + 8 g .. + 7 of it per k-step s (beyond D: zeros, like K's)
+    vec8 qreg[NSTEP];
+    {
+        const T* qrow = qp + (int64_t)min(my_i, Sq - 1) * p.q_ss + g * 8;
+#pragma unroll
+        for (int s = 0; s < NSTEP; ++s) {
+            if (s * 16 + g * 8 < p.D) qreg[s] = *(const vec8*)(qrow + s * 16);
+            else
+#pragma unroll
+                for (int e = 0; e < 8; ++e) qreg[s][e] = (T)0.0f;
+        }
+    }
+    // K operand of k-step s: row ql, logical chunk 2 s + g, stored at chunk (2 s + g) ^ fk(ql) = (g ^ fk(ql)) ^ 2 s; the
+    // row's offset and the chunk bits share none, so the address is k_base ^ (s << 5).
+    const int k_base = ql * L::ROWB + ((g ^ L::fk(ql)) << 4);
+    // V operand (transposing read) of column block db, half h: the 16 lanes of a group fetch a 4-key x 16-d patch (lane n:
+    // key n / 4, d 4 (n % 4) .. + 3).  Row 8 h + 4 g + n / 4, logical chunk 4 db + 2 dh + (n % 4) / 2 at chunk
+    // ^ fv(row) = ^ 4 (n / 4): v_base[h] ^ (db << 6).
+    int v_base[2];
+    {
+        const int n = lane & 15, dh = (lane >> 4) & 1;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int r = 8 * h + 4 * g + (n >> 2);
+            const int chunk = 2 * dh + ((n & 3) >> 1);
+            v_base[h] = r * L::ROWB + ((chunk ^ L::fv(r)) << 4) + (n & 1) * 8;
+        }
+    }
+
+    const float sc2 = p.scale * 1.4426950408889634f;      // scores in log2 units
+    float m_run = -INFINITY, l_run = 0.0f;
+    floatx16 o_acc[NDB];
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o_acc[db][r] = 0.0f;
+
+    for (int t = 0; t < n_tiles; ++t) {
+        // K(t), V(t) have arrived for everyone, everyone is done with tile t - 1: its buffers take tile t + 1
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (t + 1 < n_tiles) issue_kv(t + 1);
+        if (t >= n_act) continue;
+        const char* kb = smem + (t & 1) * TILE;
+        const char* vb = smem + (2 + (t & 1)) * TILE;
+        const int j0 = t * PW_KT;
+        // ---- S^T = K Q^T ----
+        floatx16 sacc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sacc[r] = 0.0f;
+#pragma unroll
+        for (int s = 0; s < NSTEP; ++s) {
+            const vec8 a = *(const vec8*)(kb + (k_base ^ (s << 5)));
+            sacc = Mma<T>::run(a, qreg[s], sacc);
+        }
+        // register r is key j0 + 8 (r / 4) + 4 g + (r % 4)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sacc[r] *= sc2;
+        if (j0 + PW_KT > lim_wave_min) {                  // (uniform) the tile crosses a limit of this wavefront
+            const int rel = lim_lane - (j0 + 4 * g);
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                if (8 * (r / 4) + (r % 4) >= rel) sacc[r] = -INFINITY;
+        }
+        float tmax = sacc[0];
+#pragma unroll
+        for (int r = 1; r < 16; ++r) tmax = fmaxf(tmax, sacc[r]);
+        tmax = xor32_max(tmax);
+        // the reference moves only when a tile's maximum passes it by more than 2^8 (or the row sees its first key)
+        const bool need = tmax > m_run + PF_RESCALE_THRESHOLD;
+        if (__builtin_amdgcn_ballot_w64(need) != 0) {
+            const float alpha = need ? __builtin_amdgcn_exp2f(m_run - tmax) : 1.0f;      // (first key: exp2(-inf) = 0 times 0)
+            if (need) m_run = tmax;
+            l_run *= alpha;
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) o_acc[db][r] *= alpha;
+        }
+        const float m_use = (m_run == -INFINITY) ? 0.0f : m_run;
+        // P^T in storage precision: element e of k-step ks is register 8 ks + e; the denominator is summed from the rounded values
+        vec8 pb[2];
+        float rsum = 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pb[ks][e] = (T)__builtin_amdgcn_exp2f(sacc[8 * ks + e] - m_use);
+#pragma unroll
+            for (int e = 0; e < 8; e += 2) {
+                typename Mma<T>::vec2 pr = {pb[ks][e], pb[ks][e + 1]};
+                rsum = Mma<T>::add2(pr, rsum);
+            }
+        }
+        l_run += rsum;
+        // ---- O^T += V^T P^T ----
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int db = 0; db < NDB; ++db) {
+                short8v av;
+                av.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((short4v __attribute__((address_space(3)))*)(vb + ks * 16 * L::ROWB + (v_base[0] ^ (db << 6))));
+                av.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((short4v __attribute__((address_space(3)))*)(vb + ks * 16 * L::ROWB + (v_base[1] ^ (db << 6))));
+                o_acc[db] = Mma<T>::run(__builtin_bit_cast(vec8, av), pb[ks], o_acc[db]);
+            }
+    }
+
+    // ---- normalise and store --------------------------------------------------------------------------------------
+    const float l_tot = xor32_sum(l_run);
+    const float inv = (l_tot == 0.0f) ? __builtin_nanf("") : 1.0f / l_tot;      // no visible key: NaN, as the reference
+    if (my_i < rows_b) {
+        if (p.lse && g == 0)       // m_run and the sum are in log2 units of the scaled scores
+            p.lse[((int64_t)b * p.Hq + hq) * Sq + my_i] = l_tot == 0.0f ? -INFINITY : (m_run + __builtin_log2f(l_tot)) * 0.6931471805599453f;
+        T* orow = op + (int64_t)my_i * p.o_ss;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                typedef T vec4 __attribute__((ext_vector_type(4)));
+                vec4 w;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) w[e] = (T)(o_acc[db][r4 * 4 + e] * inv);
+                if (db * 32 + r4 * 8 + g * 4 < p.Dv) *(vec4*)(orow + db * 32 + r4 * 8 + g * 4) = w;
+            }
+    }
+#endif
+}
+
+// Host has validated: dtype f16 / bf16, 128 < max(D, Dv) <= 256 in whole 16-byte vectors, finite scale, no dense mask,
+// rows 16-byte aligned with unit last-dim stride, row strides below 2^24 elements.
+hipError_t launch_sdpa_prefill_wide(const SdpaParams& p0, int dtype, hipStream_t stream)
+{
+    SdpaParams p = p0;
+    const int nqb = (p.Sq + PF_BM - 1) / PF_BM;
+    const int64_t total = (int64_t)nqb * p.Hq * p.B;
+    if (total <= 0) return hipSuccess;
+    if (total > 0x7fffffffLL) return hipErrorInvalidValue;
+    // two workgroups per compute unit, an eighth of the compute units per XCD
+    p.interleave = work_interleave(p.causal != 0, 2 * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
+    p.deal_groups = (total & 7) == 0 ? work_deal(p.interleave, p.G, nqb, total >> 3) : 0;
+    if (dtype == 1) hipLaunchKernelGGL(sdpa_prefill_wide_kernel<f16_t>, dim3((unsigned)total), dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL(sdpa_prefill_wide_kernel<bf16_t>, dim3((unsigned)total), dim3(256), 0, stream, p);
+    return hipGetLastError();
+}
+
+}  // namespace incin_rocm

@@ -65,10 +65,14 @@ def test_dispatch_choices():
     assert _plan(_desc(D=8, Dv=40))[2] == capi.IMPL_MFMA
     assert _plan(_desc(D=84, Dv=84))[2] == capi.IMPL_GENERIC                    # 168-byte rows: not whole vectors
     assert _plan(_desc(dtype=capi.F32, D=84, Dv=84))[2] == capi.IMPL_MFMA       # in f32 they are
-    # above 128: the 256 instance of the matrix-core split-KV kernels (16-bit and f32), prefill shapes too
-    assert _plan(_desc(D=160, Dv=160))[2] == capi.IMPL_SPLITKV_MFMA
-    assert _plan(_desc(D=128, Dv=136))[2] == capi.IMPL_SPLITKV_MFMA
-    assert _plan(_desc(D=256, Dv=256, Sq=4096, Skv=4096, causal=1))[2] == capi.IMPL_SPLITKV_MFMA
+    # above 128: 16-bit prefill shapes on the prefill kernel for 256, decode shapes (up to 64 positions) and f32 on the 256
+    # instance of the matrix-core split-KV kernels
+    assert _plan(_desc(D=160, Dv=160))[2] == capi.IMPL_MFMA
+    assert _plan(_desc(D=128, Dv=136))[2] == capi.IMPL_MFMA
+    assert _plan(_desc(D=256, Dv=256, Sq=4096, Skv=4096, causal=1))[2] == capi.IMPL_MFMA
+    assert _plan(_desc(D=256, Dv=256, Sq=4096, Skv=4096, causal=1, impl=capi.IMPL_SPLITKV_MFMA))[2] == capi.IMPL_SPLITKV_MFMA
+    assert _plan(_desc(D=256, Dv=256, Sq=64, Skv=4096, causal=1))[2] == capi.IMPL_SPLITKV_MFMA
+    assert _plan(_desc(D=256, Dv=256, Sq=1, Skv=4096, Hkv=1))[2] == capi.IMPL_SPLITKV_MFMA
     assert _plan(_desc(dtype=capi.F32, D=160, Dv=160))[2] == capi.IMPL_SPLITKV_MFMA
     # decode over such a cache: the matrix-core split-KV kernels, also at one row per KV head (no vector-ALU kernel there);
     # partial rows are as wide as the kernel instance
@@ -157,7 +161,8 @@ def test_dispatch_choices():
     (dict(impl=9), capi.EINVAL),
     (dict(num_splits=-2), capi.EINVAL),
     (dict(impl=capi.IMPL_MFMA64), capi.EUNSUPPORTED),                 # retired: the value is refused
-    (dict(impl=capi.IMPL_MFMA, D=160, Dv=160), capi.EUNSUPPORTED),
+    (dict(impl=capi.IMPL_MFMA, D=264, Dv=264), capi.EUNSUPPORTED),
+    (dict(impl=capi.IMPL_MFMA, D=160, Dv=160, dtype=capi.F32), capi.EUNSUPPORTED),          # above 128 the prefill kernel is 16-bit only
     (dict(impl=capi.IMPL_MFMA, D=84, Dv=84), capi.EUNSUPPORTED),
     (dict(impl=capi.IMPL_SPLITKV, Sq=1, D=96, Dv=96), capi.EUNSUPPORTED),             # the vector-ALU kernel takes 64 and 128 only
     (dict(impl=capi.IMPL_SPLITKV, Sq=4096), capi.EUNSUPPORTED),

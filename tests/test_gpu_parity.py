@@ -625,9 +625,10 @@ def test_head_dimensions_padded_into_the_matrix_core_kernels(gpu, dtype, dims):
 @pytest.mark.parametrize("dtype", [capi.BF16, capi.F16, capi.F32], ids=lambda x: dtypes.NAMES[x])
 @pytest.mark.parametrize("dims", [(256, 256), (192, 128), (160, 160), (136, 256), (64, 200)], ids=lambda x: "D%d_Dv%d" % x)
 def test_head_dimensions_above_128(gpu, dtype, dims):
-    """Head dimensions above 128 go through the 256 instance of the matrix-core split-KV kernels (16-bit and f32) whatever
-    the shape: decode with one and with several rows per KV head, and prefill shapes 32 rows per workgroup - causal,
-    grouped queries, key counts, split counts chosen and forced, row normalisers - against the oracle."""
+    """Head dimensions above 128: decode shapes (one and several rows per KV head) and every f32 shape go through the 256
+    instance of the matrix-core split-KV kernels, 16-bit prefill shapes through the prefill kernel for 256 (and through the
+    split-KV kernel when it is pinned) - causal, grouped queries, key counts, split counts chosen and forced, row
+    normalisers - against the oracle."""
     D, Dv = dims
     tol = TOL[dtype]
     for (B, Hq, Hkv, Sq, Skv), split_list in (((2, 2, 2, 1, 1500), (0, 1, 5)), ((2, 8, 2, 3, 1500), (0, 3)), ((2, 4, 2, 200, 333), (0, 1, 2)),
@@ -637,9 +638,12 @@ def test_head_dimensions_above_128(gpu, dtype, dims):
         ref = oracle_full(q, k, v, G=Hq // Hkv, causal=True, kv_lens=lens)
         for splits in split_list:
             say("head dimension above 128: %s D=%d Dv=%d %r splits=%d" % (dtypes.NAMES[dtype], D, Dv, (B, Hq, Hkv, Sq, Skv), splits))
-            got, lse, info = host.sdpa(q, k, v, dtype, causal=True, kv_lens=lens, num_splits=splits, return_info=True, return_lse=True)
-            assert info["impl"] == capi.IMPL_SPLITKV_MFMA
+            got, lse, info = host.sdpa(q, k, v, dtype, causal=True, kv_lens=lens, num_splits=splits, impl=capi.IMPL_SPLITKV_MFMA,
+                                       return_info=True, return_lse=True)
             check(got, ref, tol, "D=%d Dv=%d Sq=%d splits=%d->%d" % (D, Dv, Sq, splits, info["splits"]))
+        got, lse, info = host.sdpa(q, k, v, dtype, causal=True, kv_lens=lens, return_info=True, return_lse=True)
+        assert info["impl"] == (capi.IMPL_MFMA if Sq > 64 and dtype != capi.F32 else capi.IMPL_SPLITKV_MFMA)
+        check(got, ref, tol, "AUTO, D=%d Dv=%d Sq=%d" % (D, Dv, Sq))
         _, lse_g = host.sdpa(q, k, v, dtype, causal=True, kv_lens=lens, impl=capi.IMPL_GENERIC, return_lse=True)
         fin = np.isfinite(lse_g)
         assert np.array_equal(fin, np.isfinite(lse)) and np.max(np.abs(lse[fin] - lse_g[fin])) < (2e-5 if dtype == capi.F32 else 2e-2)
