@@ -157,6 +157,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             const vec8 a = *(const vec8*)(kb + (k_base ^ (s << 5)));
             sacc = Mma<T>::run(a, qreg[s], sacc);
         }
+        // (the order asked of the scheduler: K reads four matrix instructions ahead of their use: + 4 - 8 %)
+        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+        for (int i = 0; i < NSTEP - 4; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
         // register r is key j0 + 8 (r / 4) + 4 g + (r % 4)
 #pragma unroll
         for (int r = 0; r < 16; ++r) sacc[r] *= sc2;
@@ -206,6 +214,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 av.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((short4v __attribute__((address_space(3)))*)(vb + ks * 16 * L::ROWB + (v_base[1] ^ (db << 6))));
                 o_acc[db] = Mma<T>::run(__builtin_bit_cast(vec8, av), pb[ks], o_acc[db]);
             }
+        // (V reads - two per matrix instruction - four matrix instructions ahead)
+        __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+        for (int i = 0; i < 2 * NDB - 4; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
     }
 
     // ---- normalise and store --------------------------------------------------------------------------------------
