@@ -259,7 +259,7 @@ def decode_gqa_leg(steps, warmup, only_shape=None):
 
 def head_dims_leg(steps, warmup):
     """Head dimensions other than 64 and 128 (bf16): D = 96 runs zero-padded in the 128 instances of the prefill and split-KV
-    kernels, D = 256 in the 256 instance of the split-KV kernel (prefill shapes too).  Prefill: useful FLOPs (4 D per visible
+    kernels, D = 256 in the prefill kernel for 256 and in the 256 instance of the split-KV kernel.  Prefill: useful FLOPs (4 D per visible
     pair) against the bf16 matrix peak; decode: KV bytes read once against the HBM peak."""
     out = {}
     names = {capi.IMPL_SPLITKV_MFMA: "sdpa_decode_mfma_kernel", capi.IMPL_MFMA: "sdpa_prefill_mfma_kernel", capi.IMPL_GENERIC: "sdpa_generic_kernel"}
@@ -268,7 +268,8 @@ def head_dims_leg(steps, warmup):
         w = Workload("head_dims_" + name, SEED0 + 80 + i, B, Hq, Hkv, Sq, Skv, D, capi.BF16, causal)
         wall, ev_mean, ev_med, ev_min = w.time(max(steps, 50), warmup)
         entry = {"workload": "bf16 %s B=%d Hq=%d Hkv=%d S_q=%d KV=%d D=%d" % ("causal prefill" if Sq > 1 else "decode", B, Hq, Hkv, Sq, Skv, D),
-                 "kernel": names.get(w.impl, str(w.impl)), "num_splits": w.splits, "ms_per_step": wall, "parity_max_abs_err": w.parity(16)}
+                 "kernel": "sdpa_prefill_wide_kernel" if D > 128 and w.impl == capi.IMPL_MFMA else names.get(w.impl, str(w.impl)),
+                 "num_splits": w.splits, "ms_per_step": wall, "parity_max_abs_err": w.parity(16)}
         if Sq > 1:
             flops = causal_flops(B, Hq, Sq, Skv, D)
             entry["tflops"] = flops / (wall * 1e-3) / 1e12
