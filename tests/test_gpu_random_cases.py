@@ -19,10 +19,10 @@ def say(msg):
     print(msg, file=sys.stderr, flush=True)
 
 
-def draw_case(r):
+def draw_case(r, head_dims=(16, 32, 64, 64, 80, 128, 128, 128, 256), other_dv=(16, 64, 128)):
     dtype = int(r.choice([capi.F32, capi.F16, capi.BF16]))
-    D = int(r.choice([16, 32, 64, 64, 80, 128, 128, 128, 256]))
-    Dv = D if r.random() < 0.8 else int(r.choice([16, 64, 128]))
+    D = int(r.choice(head_dims))
+    Dv = D if r.random() < 0.8 else int(r.choice(other_dv))
     Hkv = int(r.integers(1, 4))
     G = int(r.choice([1, 1, 2, 4]))
     B = int(r.integers(1, 4))
@@ -120,4 +120,21 @@ def test_random_cases(gpu):
     for dt, (err, what) in sorted(WORST.items()):
         say("worst absolute error, dtype %d: %.3e in %s" % (dt, err, what))
     for impl in (capi.IMPL_GENERIC, capi.IMPL_MFMA, capi.IMPL_SPLITKV, capi.IMPL_SPLITKV_MFMA):
+        assert used.get(impl, 0) >= 5, "kernel %d was hardly reached: %s" % (impl, used)
+
+
+def test_random_cases_over_head_dimensions(gpu):
+    """The same draw over the head dimensions the matrix-core kernels take padded (whole 16-byte vectors up to 128, above
+    128 up to 256, D != Dv) and some they do not (rows of 4 or 12 bytes more than a vector), every kernel the planner
+    accepts for each case."""
+    r = np.random.Generator(np.random.PCG64(20261126))
+    used = {}
+    for i in range(80):
+        c = draw_case(r, head_dims=(8, 24, 40, 72, 96, 104, 120, 136, 160, 192, 200, 248, 20, 132), other_dv=(8, 48, 96, 144, 256))
+        if i % 20 == 0:
+            say("random case (head dimensions) %d/80" % i)
+        for impl in run_case(1000 + i, c, r):
+            used[impl] = used.get(impl, 0) + 1
+    say("kernels exercised: %s" % used)
+    for impl in (capi.IMPL_GENERIC, capi.IMPL_MFMA, capi.IMPL_SPLITKV_MFMA):
         assert used.get(impl, 0) >= 5, "kernel %d was hardly reached: %s" % (impl, used)
