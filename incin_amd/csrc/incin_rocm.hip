@@ -155,8 +155,9 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     const int64_t R = (d->Hq / d->Hkv) * d->Sq;
     // The matrix-core kernels are built for head dimensions 64 and 128; smaller ones (D and Dv need not be equal) run in
     // the instance that holds them, padded with zeros on the way into LDS, as long as rows stay whole 16-byte vectors.
-    // The split-KV kernels have an instance for 256 as well, which takes every launch with a head dimension above
-    // 128 - prefill shapes too, 32 rows per workgroup.  The vector-ALU split-KV kernel takes the two dimensions as they are.
+    // Above 128 (up to 256): an instance for 256 of the split-KV kernels (16-bit and f32, any number of query positions) and of
+    // the 16-bit prefill kernel (sdpa_prefill_wide.hip, no dense mask).  The vector-ALU split-KV kernel takes D == Dv in
+    // {64, 128} as they are.
     const int64_t d_max = std::max(d->D, d->Dv);
     const int64_t d_pad = d_max <= 64 ? 64 : d_max <= 128 ? 128 : 256;
     const bool wide = d_pad == 256;
@@ -192,18 +193,20 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         const int64_t esize = (int64_t)dtype_size(d->dtype);
         const int64_t kv_bytes = 2 * d->B * d->Hkv * d->Skv * d->D * esize;
         const int64_t len128 = d->Skv * d_pad * esize / 256;     // cache length in keys of 256 bytes (what the thresholds were measured in)
+        // Head dimensions above 128: the 16-bit prefill kernel for 256 where there are more than 64 query positions (128 rows
+        // share a K / V tile there, 32 in the split-KV kernel: D = 256 causal prefill 775 - 890 against 340 - 460 TFLOP/s), the
+        // split-KV kernels' 256 instance for decode shapes and - f32 has no such prefill kernel - for every f32 shape.
+        if (wide && mfma_ok && d->Sq > 64) impl = INCIN_ROCM_IMPL_MFMA;
+        else if (wide && split_mfma_ok) impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
         // f32 (sdpa_decode_f32.hip): from two rows per KV head on, whatever the count - the f32 prefill kernel would spend a
         // 32-row matrix instruction on every query head's few rows (32 heads of a group at one position each: 8.4 ms
         // against 0.23), and where it packs as well (64 positions of one head) the split-KV form is still ahead (0.22
         // against 0.28 ms on 8 x 8 heads x 8192 keys); the vector-ALU kernel is level at 2 rows and behind from 4 on
         // (4 rows, 268 MB of cache: 5.6 against 4.8 TB/s; 8 rows: 6.6 against 3.4).  More than 32 rows over fewer than 512
         // keys stay with the prefill kernel (64 positions x 16 heads x 64 sequences of 256 keys: 0.14 against 0.17 ms).
-        // above 128: the split-KV kernels' 256 instance for decode shapes (and for f32 whatever the shape), the 16-bit
-        // prefill kernel for 256 where there are more than 64 positions (128 rows share a K / V tile there instead of 32)
-        if (wide && mfma_ok && d->Sq > 64) impl = INCIN_ROCM_IMPL_MFMA;
-        else if (wide && split_mfma_ok) impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
         else if (d->dtype == INCIN_ROCM_F32 && split_mfma_ok && len128 >= 256 && R >= 2 && (R <= 32 || d->Skv >= 512))
             impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
+        // f16 / bf16 (sdpa_decode_mfma.hip): the thresholds described above
         else if (d->dtype != INCIN_ROCM_F32 && split_mfma_ok && len128 >= 256 &&
             ((R == 1 && len128 >= 1024 && kv_bytes >= (512LL << 20)) || (R >= 2 && R <= 3 && len128 >= 512) || (R >= 4 && R <= 64)))
             impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
