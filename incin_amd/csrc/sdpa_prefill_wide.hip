@@ -10,7 +10,7 @@
 //
 //   S^T = K_tile Q^T     v_mfma_f32_32x32x16 over the 16 k-steps of 256 elements: A = K rows from LDS (16-byte reads),
 //                        B = Q^T resident in registers (64 of them); a lane owns one query and 16 keys of the tile.
-//   softmax              scale applied to the f32 scores (any finite scale), masks as -inf before the maximum, the
+//   softmax              scale * log2(e) folded into Q (any finite scale), masks as -inf before the maximum, the
 //                        reference maximum moved lazily (threshold 2^8), P rounded to the storage type in registers.
 //   O^T += V^T P^T       A = V^T through the transposing LDS read, 8 blocks of 32 columns: 128 accumulator registers.
 //
@@ -113,6 +113,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
                 for (int e = 0; e < 8; ++e) qreg[s][e] = (T)0.0f;
         }
+        // scale * log2(e) folded into Q once (rounded back to the storage type, as sdpa_prefill_mfma.hip does): the product
+        // then yields the scores in the log2 units the softmax works in, whatever the sign of the scale
+        const float c2 = p.scale * 1.4426950408889634f;
+#pragma unroll
+        for (int s = 0; s < NSTEP; ++s)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) qreg[s][e] = (T)((float)qreg[s][e] * c2);
     }
     // K operand of k-step s: row ql, logical chunk 2 s + g, stored at chunk (2 s + g) ^ fk(ql) = (g ^ fk(ql)) ^ 2 s; the
     // row's offset and the chunk bits share none, so the address is k_base ^ (s << 5).
@@ -131,7 +138,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
     }
 
-    const float sc2 = p.scale * 1.4426950408889634f;      // scores in log2 units
     float m_run = -INFINITY, l_run = 0.0f;
     floatx16 o_acc[NDB];
 #pragma unroll
@@ -166,8 +172,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
         __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
         // register r is key j0 + 8 (r / 4) + 4 g + (r % 4)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) sacc[r] *= sc2;
         if (j0 + PW_KT > lim_wave_min) {                  // (uniform) the tile crosses a limit of this wavefront
             const int rel = lim_lane - (j0 + 4 * g);
 #pragma unroll
