@@ -123,6 +123,13 @@ bool fast_layout_ok(const incin_rocm_sdpa_desc_t* d, int vec)
     return true;
 }
 
+// The rows of a 16-bit dense mask can be read four keys (8 bytes) at a time: unit stride along the keys, every row 8-byte aligned.
+bool mask_rows_vector_loadable(const incin_rocm_sdpa_desc_t* d)
+{
+    return d->add_mask && d->mask_stride[3] == 1 && (reinterpret_cast<uintptr_t>(d->add_mask) & 7u) == 0 &&
+           d->mask_stride[0] % 4 == 0 && d->mask_stride[1] % 4 == 0 && d->mask_stride[2] % 4 == 0;
+}
+
 int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
 {
     if (!d) return fail(INCIN_ROCM_EINVAL, "scaled_dot_product_attention: null descriptor");
@@ -170,8 +177,8 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     const bool tile_off_ok = d->k_stride[2] >= 0 && d->v_stride[2] >= 0 && d->k_stride[2] < stride_lim && d->v_stride[2] < stride_lim;
     // f32: the IEEE-f32 matrix-core kernel, any finite scale; f16 / bf16: the 16-bit kernels fold the scale into Q in
     // a way that needs it positive.  Both take a dense additive mask (any strides); the 64-row kernel does not.
-    // (above 128: sdpa_prefill_wide.hip - 16-bit storage, no dense mask, any finite scale)
-    const bool mfma_ok = wide ? fast_ok && d->dtype != INCIN_ROCM_F32 && tile_off_ok && std::isfinite(d->scale)
+    // (above 128: sdpa_prefill_wide.hip - 16-bit storage, any finite scale, a dense mask whose rows it can read 8 bytes at a time)
+    const bool mfma_ok = wide ? layout_ok && d->dtype != INCIN_ROCM_F32 && tile_off_ok && std::isfinite(d->scale) && (!d->add_mask || mask_rows_vector_loadable(d))
                               : layout_ok && tile_off_ok && std::isfinite(d->scale) && (d->dtype == INCIN_ROCM_F32 || d->scale > 0.0f);
     const bool split_ok = fast_ok && head_exact && d->Sq <= 64;
     // the matrix-core split-KV kernels (16-bit and f32): blocks addressed like the prefill kernels' tiles
@@ -220,7 +227,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     }
     if (impl == INCIN_ROCM_IMPL_MFMA && !mfma_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
-                    "scaled_dot_product_attention: the MFMA prefill kernels need D and Dv <= 128 (f16/bf16 without a dense mask: 256) in whole 16-byte vectors and 16-byte aligned rows; for f16/bf16 up to 128 also scale > 0");
+                    "scaled_dot_product_attention: the MFMA prefill kernels need D and Dv <= 128 (f16/bf16: 256) in whole 16-byte vectors and 16-byte aligned rows; for f16/bf16 up to 128 also scale > 0");
     if (impl == INCIN_ROCM_IMPL_MFMA64)
         return fail(INCIN_ROCM_EUNSUPPORTED,
                     "scaled_dot_product_attention: the 64-row MFMA prefill kernel has been retired (INCIN_ROCM_IMPL_MFMA covers its shapes)");
@@ -343,8 +350,7 @@ void fill_params(const incin_rocm_sdpa_desc_t* d, const Plan& plan, SdpaParams* 
     p->v_sb = d->v_stride[0]; p->v_sh = d->v_stride[1]; p->v_ss = d->v_stride[2];
     p->o_sb = d->o_stride[0]; p->o_sh = d->o_stride[1]; p->o_ss = d->o_stride[2];
     p->m_sb = d->mask_stride[0]; p->m_sh = d->mask_stride[1]; p->m_si = d->mask_stride[2]; p->m_sj = d->mask_stride[3];
-    p->mask_vec = d->add_mask && d->mask_stride[3] == 1 && (reinterpret_cast<uintptr_t>(d->add_mask) & 7u) == 0 &&
-                  d->mask_stride[0] % 4 == 0 && d->mask_stride[1] % 4 == 0 && d->mask_stride[2] % 4 == 0;
+    p->mask_vec = mask_rows_vector_loadable(d);
     p->B = (int)d->B; p->Hq = (int)d->Hq; p->Hkv = (int)d->Hkv; p->G = (int)(d->Hq / d->Hkv);
     p->Sq = (int)d->Sq; p->Skv = (int)d->Skv; p->D = (int)d->D; p->Dv = (int)d->Dv;
     p->Dp = std::max(d->D, d->Dv) <= 64 ? 64 : std::max(d->D, d->Dv) <= 128 ? 128 : 256;      // (means something to the matrix-core and split-KV kernels only)

@@ -25,7 +25,10 @@ namespace incin_rocm {
 
 constexpr int PW_KT = 32;      // keys per tile
 
-template <typename T>
+// DENSE: a dense additive mask (any broadcast strides) comes with one flag per block of 32 rows x 32 keys (mask_blocks.hip) -
+// a tile of this kernel is one such block per wavefront: tiles where the mask is zero run without it, the others add its
+// values to the scores, and the tiles before the first and after the last one it shows to a wavefront are skipped.
+template <typename T, bool DENSE>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void sdpa_prefill_wide_kernel(SdpaParams p)
 {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -72,8 +75,38 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         lim_wave_max = clampi(min(q0 + wave * 32 + 31, rows_b - 1) + coff + 1, 0, kv_len);
     }
     if (q0 + wave * 32 >= rows_b) lim_wave_min = lim_wave_max = 0;      // a wavefront of padding rows only keeps the barriers company
-    const int n_tiles = (j_end + PW_KT - 1) / PW_KT;
-    const int n_act = lim_wave_max > 0 ? (lim_wave_max + PW_KT - 1) / PW_KT : 0;      // tiles this wavefront computes
+    int n_tiles = (j_end + PW_KT - 1) / PW_KT;
+    int n_act = lim_wave_max > 0 ? (lim_wave_max + PW_KT - 1) / PW_KT : 0;      // tiles this wavefront computes: [w_first, n_act)
+    int w_first = 0, t_first = 0;
+    // dense mask: this lane's row of it and the flags of this wavefront's 32 rows, one per tile.  The tiles before the first
+    // and after the last one the mask shows to a wavefront are not computed (a sliding window's past), and the workgroup's
+    // copies run from the first to the last tile any of its wavefronts computes; a hidden tile in between goes through the
+    // mask's values like a mixed one (-inf everywhere).
+    const T* mrow = nullptr;
+    const uint8_t* mflags = nullptr;
+    __shared__ int s_range[8];
+    if (DENSE) {
+        mrow = (const T*)p.mask + (int64_t)b * p.m_sb + (int64_t)hq * p.m_sh + (int64_t)min(my_i, Sq - 1) * p.m_si;
+        mflags = mask_flags_of(p, b, hq) + (int64_t)((q0 >> 5) + wave) * ((Skv + 31) >> 5);
+        int lo = 0x7fffffff, hi = -1;
+        for (int t = lane; t < n_act; t += 64)
+            if (mflags[t] != 2) { lo = min(lo, t); hi = max(hi, t); }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            lo = min(lo, __shfl_xor(lo, off, 64));
+            hi = max(hi, __shfl_xor(hi, off, 64));
+        }
+        w_first = __builtin_amdgcn_readfirstlane(hi < 0 ? 0 : lo);
+        n_act = __builtin_amdgcn_readfirstlane(hi + 1);
+        if (lane == 0) { s_range[wave] = hi < 0 ? 0x7fffffff : lo; s_range[4 + wave] = hi; }
+        __syncthreads();
+        int g_lo = s_range[0], g_hi = s_range[4];
+#pragma unroll
+        for (int w2 = 1; w2 < 4; ++w2) { g_lo = min(g_lo, s_range[w2]); g_hi = max(g_hi, s_range[4 + w2]); }
+        // (uniform by construction; said explicitly, because tile numbers end up in scalar copy descriptors)
+        t_first = __builtin_amdgcn_readfirstlane(g_hi < 0 ? 0 : g_lo);
+        n_tiles = __builtin_amdgcn_readfirstlane(g_hi + 1);      // (0 when the mask hides everything from these 128 rows)
+    }
 
     // ---- global -> LDS copy plan: wavefront-wide load ii = wave * LPW + c fills LDS bytes [ii * 1024, +1024) of a tile ----
     int k_voff[LPW], v_voff[LPW];
@@ -99,7 +132,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         issue(kp, k_tile_bytes, p.k_ss, p.D, t, t & 1, k_voff);
         issue(vp, v_tile_bytes, p.v_ss, p.Dv, t, 2 + (t & 1), v_voff);
     };
-    if (n_tiles > 0) issue_kv(0);
+    if (n_tiles > t_first) issue_kv(t_first);
+    int flag_next = 1;      // the flag of the next tile, read one tile ahead
+    if (DENSE && n_tiles > t_first) flag_next = mflags[t_first];
 
     // ---- operands ----------------------------------------------------------------------------------------------
     // Q^T (B operand, resident): this lane's row, elements 16 s + 8 g .. + 7 of it per k-step s (beyond D: zeros, like K's)
@@ -145,12 +180,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
         for (int r = 0; r < 16; ++r) o_acc[db][r] = 0.0f;
 
-    for (int t = 0; t < n_tiles; ++t) {
+    for (int t = t_first; t < n_tiles; ++t) {
         // K(t), V(t) have arrived for everyone, everyone is done with tile t - 1: its buffers take tile t + 1
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         if (t + 1 < n_tiles) issue_kv(t + 1);
-        if (t >= n_act) continue;
+        int flag = 1;
+        if (DENSE) {      // (arrived with the tile: the wait above covers it)
+            flag = __builtin_amdgcn_readfirstlane(flag_next);
+            if (t + 1 < n_tiles) flag_next = mflags[t + 1];
+        }
+        if (t >= n_act || t < w_first) continue;      // nothing of this tile is visible to the wavefront's rows
         const char* kb = smem + (t & 1) * TILE;
         const char* vb = smem + (2 + (t & 1)) * TILE;
         const int j0 = t * PW_KT;
@@ -172,6 +212,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
         __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
         // register r is key j0 + 8 (r / 4) + 4 g + (r % 4)
+        if (DENSE && flag != 1) {      // the mask's values of this lane's 16 keys (no registers to spare for asking earlier)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                const int j = j0 + 8 * r4 + 4 * g;
+                typedef T vec4 __attribute__((ext_vector_type(4)));
+                // (rows of the mask are contiguous and 8-byte aligned here - the host sends other masks elsewhere; keys at and
+                // beyond Skv are hidden by the limits below whatever is added to them)
+                vec4 m4 = {(T)0.0f, (T)0.0f, (T)0.0f, (T)0.0f};
+                if (j + 3 < Skv) m4 = *(const vec4*)(mrow + j);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) sacc[4 * r4 + e] = __builtin_fmaf((float)m4[e], 1.4426950408889634f, sacc[4 * r4 + e]);
+            }
+        }
         if (j0 + PW_KT > lim_wave_min) {                  // (uniform) the tile crosses a limit of this wavefront
             const int rel = lim_lane - (j0 + 4 * g);
 #pragma unroll
@@ -249,7 +302,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #endif
 }
 
-// Host has validated: dtype f16 / bf16, 128 < max(D, Dv) <= 256 in whole 16-byte vectors, finite scale, no dense mask,
+// Host has validated: dtype f16 / bf16, 128 < max(D, Dv) <= 256 in whole 16-byte vectors, finite scale; with a dense mask its
+// block flags have been written (launch_mask_classify);
 // rows 16-byte aligned with unit last-dim stride, row strides below 2^24 elements.
 hipError_t launch_sdpa_prefill_wide(const SdpaParams& p0, int dtype, hipStream_t stream)
 {
@@ -261,8 +315,11 @@ hipError_t launch_sdpa_prefill_wide(const SdpaParams& p0, int dtype, hipStream_t
     // two workgroups per compute unit, an eighth of the compute units per XCD
     p.interleave = work_interleave(p.causal != 0, 2 * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
     p.deal_groups = (total & 7) == 0 ? work_deal(p.interleave, p.G, nqb, total >> 3) : 0;
-    if (dtype == 1) hipLaunchKernelGGL(sdpa_prefill_wide_kernel<f16_t>, dim3((unsigned)total), dim3(256), 0, stream, p);
-    else hipLaunchKernelGGL(sdpa_prefill_wide_kernel<bf16_t>, dim3((unsigned)total), dim3(256), 0, stream, p);
+    if (p.mask) {
+        if (dtype == 1) hipLaunchKernelGGL((sdpa_prefill_wide_kernel<f16_t, true>), dim3((unsigned)total), dim3(256), 0, stream, p);
+        else hipLaunchKernelGGL((sdpa_prefill_wide_kernel<bf16_t, true>), dim3((unsigned)total), dim3(256), 0, stream, p);
+    } else if (dtype == 1) hipLaunchKernelGGL((sdpa_prefill_wide_kernel<f16_t, false>), dim3((unsigned)total), dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL((sdpa_prefill_wide_kernel<bf16_t, false>), dim3((unsigned)total), dim3(256), 0, stream, p);
     return hipGetLastError();
 }
 

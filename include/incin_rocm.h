@@ -47,8 +47,8 @@ enum {
     INCIN_ROCM_IMPL_GENERIC = 1,   /* fp32-FMA tiled kernel: any dtype, D and Dv <= 256, dense masks     */
     INCIN_ROCM_IMPL_MFMA = 2,      /* MFMA prefill kernels: D and Dv <= 128 in whole 16-byte vectors (instances for 64 and 128; smaller
                                       and unequal head dimensions are zero-padded into LDS); bf16/f16 (scale > 0) and IEEE-f32
-                                      matrix instructions for f32; dense mask allowed.  bf16/f16 without a dense mask also
-                                      above 128, up to 256 (an instance for 256, any finite scale)                 */
+                                      matrix instructions for f32; dense mask allowed.  bf16/f16 also above 128, up to 256
+                                      (an instance for 256, any finite scale; a dense mask with 8-byte aligned rows)  */
     INCIN_ROCM_IMPL_SPLITKV = 3,   /* vector-ALU split-KV decode kernel + combine: D == Dv in {64,128}, few query rows */
     INCIN_ROCM_IMPL_MFMA64 = 4,    /* retired (a prefill kernel with 64 query rows per wavefront): refused with INCIN_ROCM_EUNSUPPORTED */
     INCIN_ROCM_IMPL_SPLITKV_MFMA = 5 /* split-KV kernels on the matrix cores + combine: D and Dv <= 256 in whole 16-byte vectors (instances for

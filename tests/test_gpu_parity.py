@@ -649,6 +649,43 @@ def test_head_dimensions_above_128(gpu, dtype, dims):
         assert np.array_equal(fin, np.isfinite(lse)) and np.max(np.abs(lse[fin] - lse_g[fin])) < (2e-5 if dtype == capi.F32 else 2e-2)
 
 
+@pytest.mark.parametrize("dtype", [capi.BF16, capi.F16], ids=lambda x: dtypes.NAMES[x])
+@pytest.mark.parametrize("dims", [(256, 256), (192, 128)], ids=lambda x: "D%d_Dv%d" % x)
+def test_head_dimensions_above_128_with_a_dense_mask(gpu, dtype, dims):
+    """The prefill kernel for 256 with a dense additive mask: a sliding window given as a [1, 1, Sq, Skv] tensor (tiles before
+    the window are skipped by the mask's block flags), random values with hidden blocks per batch entry on top of the causal
+    flag, a decode-like launch with a mask; a mask whose rows are not 8-byte aligned falls to the generic kernel."""
+    D, Dv = dims
+    tol = TOL[dtype]
+    B, Hq, Hkv, Sq, Skv = 2, 4, 2, 300, 420
+    q, k, v = inputs(2600 + D, B, Hq, Hkv, Sq, Skv, D, Dv, dtype)
+    i, j = np.arange(Sq)[:, None], np.arange(Skv)[None, :]
+    window = np.where((j <= i + Skv - Sq) & (j > i + Skv - Sq - 100), 0.0, -np.inf).astype(np.float32)[None, None]
+    got, info = host.sdpa(q, k, v, dtype, mask=window, return_info=True)
+    assert info["impl"] == capi.IMPL_MFMA
+    check(got, oracle_full(q, k, v, G=2, mask=window), tol, "sliding window as a tensor, D=%d" % D)
+    r = rng(7)
+    m = (r.standard_normal((B, 1, Sq, Skv)) * 0.5).astype(np.float32)
+    m[0, :, 64:200, 32:160] = -np.inf
+    m[1, :, :, 300:] = -np.inf
+    m = dtypes.round_to(m, dtype)
+    got, lse, info = host.sdpa(q, k, v, dtype, mask=m, causal=True, return_info=True, return_lse=True)
+    assert info["impl"] == capi.IMPL_MFMA
+    full = np.broadcast_to(m, (B, Hq, Sq, Skv)) + np.triu(np.full((Sq, Skv), -np.inf, np.float32), 1 + Skv - Sq)
+    check(got, oracle_full(q, k, v, G=2, mask=full), tol, "random mask with hidden blocks + causal, D=%d" % D)
+    _, lse_g = host.sdpa(q, k, v, dtype, mask=m, causal=True, impl=capi.IMPL_GENERIC, return_lse=True)
+    assert np.max(np.abs(lse - lse_g)) < 2e-2
+    # decode-like: 3 positions over the cache with a mask
+    q3 = q[:, :, :3]
+    got, info = host.sdpa(q3, k, v, dtype, mask=m[:, :, :3], return_info=True)
+    assert info["impl"] == capi.IMPL_MFMA
+    check(got, oracle_full(q3, k, v, G=2, mask=m[:, :, :3]), tol, "decode-like with a mask, D=%d" % D)
+    # 418 keys: rows of the mask 836 bytes apart
+    got, info = host.sdpa(q, k[:, :, :418], v[:, :, :418], dtype, mask=m[..., :418], return_info=True)
+    assert info["impl"] == capi.IMPL_GENERIC
+    check(got, oracle_full(q, k[:, :, :418], v[:, :, :418], G=2, mask=m[..., :418]), tol, "mask rows not 8-byte aligned: generic")
+
+
 def test_head_dimensions_outside_the_matrix_core_kernels(gpu):
     """Rows that are not whole 16-byte vectors stay on the generic kernel."""
     for dtype, D in ((capi.BF16, 20), (capi.F32, 6), (capi.BF16, 132), (capi.F32, 134)):
