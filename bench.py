@@ -478,7 +478,9 @@ def f32_configs(steps, warmup, with_cpu, threads):
         n = max(steps, 200) if key != "f32_large" else max(5, min(steps, 20))      # launches of tens of microseconds / of ~5 ms
         wall, ev_mean, ev_med, ev_min = w.time(n, warmup)
         flops = causal_flops(B, H, S, S, D) if causal else 4.0 * D * B * H * S * S
-        kernel = {capi.IMPL_MFMA: "sdpa_prefill_f32_kernel<%d>" % D, capi.IMPL_GENERIC: "sdpa_generic_kernel<float>"}.get(w.impl, str(w.impl))
+        kernel = {capi.IMPL_MFMA: "sdpa_prefill_f32_kernel<%d>" % D, capi.IMPL_GENERIC: "sdpa_generic_kernel<float>",
+                  capi.IMPL_SPLITKV_MFMA: "sdpa_decode_f32_kernel<%d> (the f32 split-KV kernel, 32 rows per workgroup: AUTO's choice for launches "
+                                          "of at most one 128-row block per compute unit)" % D}.get(w.impl, str(w.impl))
         what = "BASELINE config %s" % key[-1] if key != "f32_large" else "not a BASELINE config (the shape of config 3 in f32: a launch that fills the machine)"
         rec = {"workload": "%s: f32 %s attention fwd B=%d H=%d S_q=S_kv=%d D=%d, %s" %
                            (what, "causal" if causal else "non-causal", B, H, S, D, scale_note),
@@ -489,6 +491,12 @@ def f32_configs(steps, warmup, with_cpu, threads):
                             "algorithmic_flops_per_launch": flops, "launch_ms_mean": ev_mean, "launch_ms_median": ev_med,
                             "launch_ms_min": ev_min},
                "parity_max_abs_err": w.parity()}
+        if w.impl != capi.IMPL_MFMA:        # the f32 prefill kernel on the same launch, pinned
+            w.replan(impl=capi.IMPL_MFMA)
+            wall_p = w.time(n, warmup)[0]
+            rec["prefill_kernel_pinned"] = {"kernel": "sdpa_prefill_f32_kernel<%d>" % D, "ms_per_step": wall_p,
+                                            "value": flops / (wall_p * 1e-3) / 1e12, "unit": "TFLOP/s", "parity_max_abs_err": w.parity()}
+            w.replan()
         if key == "f32_c2":
             # the same problem with the mask as a tensor: the launch first classifies the tensor by blocks of 32 x 32 (hidden
             # blocks are skipped, zero blocks run unmasked), FLOPs counted as above

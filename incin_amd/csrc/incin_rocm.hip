@@ -181,8 +181,9 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     const bool mfma_ok = wide ? layout_ok && d->dtype != INCIN_ROCM_F32 && tile_off_ok && std::isfinite(d->scale) && (!d->add_mask || mask_rows_vector_loadable(d))
                               : layout_ok && tile_off_ok && std::isfinite(d->scale) && (d->dtype == INCIN_ROCM_F32 || d->scale > 0.0f);
     const bool split_ok = fast_ok && head_exact && d->Sq <= 64;
-    // the matrix-core split-KV kernels (16-bit and f32): blocks addressed like the prefill kernels' tiles
-    const bool split_mfma_ok = fast_ok && (d->Sq <= 64 || wide) && tile_off_ok && std::isfinite(d->scale);
+    // the matrix-core split-KV kernels (16-bit and f32): blocks addressed like the prefill kernels' tiles; the f32 kernel and
+    // the 256 instances take any number of query positions
+    const bool split_mfma_ok = fast_ok && (d->Sq <= 64 || wide || d->dtype == INCIN_ROCM_F32) && tile_off_ok && std::isfinite(d->scale);
 
     int impl = d->impl;
     if (impl == INCIN_ROCM_IMPL_AUTO) {
@@ -211,7 +212,16 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         // against 0.28 ms on 8 x 8 heads x 8192 keys); the vector-ALU kernel is level at 2 rows and behind from 4 on
         // (4 rows, 268 MB of cache: 5.6 against 4.8 TB/s; 8 rows: 6.6 against 3.4).  More than 32 rows over fewer than 512
         // keys stay with the prefill kernel (64 positions x 16 heads x 64 sequences of 256 keys: 0.14 against 0.17 ms).
-        else if (d->dtype == INCIN_ROCM_F32 && split_mfma_ok && len128 >= 256 && R >= 2 && (R <= 32 || d->Skv >= 512))
+        else if (d->dtype == INCIN_ROCM_F32 && split_mfma_ok && d->Sq <= 64 && len128 >= 256 && R >= 2 && (R <= 32 || d->Skv >= 512))
+            impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
+        // f32 prefill launches that give the prefill kernel at most one 128-row workgroup per compute unit: the split-KV kernel
+        // takes them 32 rows per workgroup with the keys dealt to its four wavefronts - four times the workgroups, a quarter
+        // of the keys per wavefront - where the prefill kernel's wavefronts each walk all keys for their 32 rows behind
+        // 64-cycle matrix instructions (measured, causal: one head of 128 x 128 13.3 -> 8.6 us; 2 x 8 heads x 512 x 512 at
+        // D = 128 73 -> 28; 128 workgroups' worth of 1024 x 1024 80 -> 33; 256 - BASELINE config 2 - 80 -> 65; level at 512).
+        // Not the chunks of a long prompt, where the prefill kernel splits the keys itself (below) and runs at 80 % of the peak.
+        else if (d->dtype == INCIN_ROCM_F32 && split_mfma_ok && d->Sq > 64 && !(d->Skv >= 4096 && d->Skv >= 4 * d->Sq) &&
+                 d->B * d->Hq * ((d->Sq + 127) / 128) <= compute_units_of(d->device))
             impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
         // f16 / bf16 (sdpa_decode_mfma.hip): the thresholds described above
         else if (d->dtype != INCIN_ROCM_F32 && split_mfma_ok && len128 >= 256 &&
@@ -220,7 +230,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         else if (split_ok && R <= 8 && d->Skv >= 256) impl = INCIN_ROCM_IMPL_SPLITKV;
         // a head dimension that is padded into its instance has no vector-ALU kernel: one row per KV head, too, goes through
         // the matrix-core split-KV kernels
-        else if (!head_exact && split_mfma_ok && len128 >= 256 && (d->dtype == INCIN_ROCM_F32 || R <= 64)) impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
+        else if (!head_exact && split_mfma_ok && d->Sq <= 64 && len128 >= 256 && (d->dtype == INCIN_ROCM_F32 || R <= 64)) impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
         else if (mfma_ok) impl = INCIN_ROCM_IMPL_MFMA;
         else if (split_ok && R <= 8) impl = INCIN_ROCM_IMPL_SPLITKV;
         else impl = INCIN_ROCM_IMPL_GENERIC;
@@ -233,7 +243,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
                     "scaled_dot_product_attention: the 64-row MFMA prefill kernel has been retired (INCIN_ROCM_IMPL_MFMA covers its shapes)");
     if (impl == INCIN_ROCM_IMPL_SPLITKV_MFMA && !split_mfma_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
-                    "scaled_dot_product_attention: the matrix-core split-KV kernels need D and Dv <= 256 in whole 16-byte vectors, Sq <= 64 (any Sq above 128), no dense mask, a finite scale and 16-byte aligned rows");
+                    "scaled_dot_product_attention: the matrix-core split-KV kernels need D and Dv <= 256 in whole 16-byte vectors, Sq <= 64 (any Sq in f32 and above 128), no dense mask, a finite scale and 16-byte aligned rows");
     if (impl == INCIN_ROCM_IMPL_SPLITKV && !split_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
                     "scaled_dot_product_attention: the split-KV kernel needs D == Dv in {64,128}, Sq <= 64, no dense mask and 16-byte aligned rows");

@@ -56,15 +56,21 @@ def _plan(d):
 
 def test_dispatch_choices():
     assert _plan(_desc())[2] == capi.IMPL_MFMA
-    assert _plan(_desc(dtype=capi.F32))[2] == capi.IMPL_MFMA                  # the IEEE-f32 matrix-core kernel
+    # f32: the IEEE-f32 matrix-core prefill kernel where the launch gives it more than one 128-row workgroup per compute unit
+    # (256 here: no device to ask), the f32 split-KV kernel - 32 rows per workgroup, keys dealt to its wavefronts - below that
+    assert _plan(_desc(dtype=capi.F32, B=8, Hq=16, Sq=4096, Skv=4096))[2] == capi.IMPL_MFMA
+    assert _plan(_desc(dtype=capi.F32, B=4, Hq=8, Sq=1024, Skv=1024))[2] == capi.IMPL_SPLITKV_MFMA      # BASELINE config 2: 256 workgroups
+    assert _plan(_desc(dtype=capi.F32, B=4, Hq=8, Sq=1025, Skv=1025))[2] == capi.IMPL_MFMA              # 288
+    assert _plan(_desc(dtype=capi.F32))[2] == capi.IMPL_SPLITKV_MFMA
+    assert _plan(_desc(dtype=capi.F32, impl=capi.IMPL_MFMA))[2] == capi.IMPL_MFMA
     assert _plan(_desc(dtype=capi.F32, add_mask=0x20000))[2] == capi.IMPL_MFMA  # which also takes a dense mask
     # head dimensions up to 128 in whole 16-byte vectors (D and Dv need not be equal) run padded in the matrix-core kernels
-    assert _plan(_desc(dtype=capi.F32, D=80, Dv=80))[2] == capi.IMPL_MFMA
+    assert _plan(_desc(dtype=capi.F32, D=80, Dv=80, B=8, Hq=16, Sq=4096, Skv=4096))[2] == capi.IMPL_MFMA
     assert _plan(_desc(D=80, Dv=80))[2] == capi.IMPL_MFMA
     assert _plan(_desc(D=128, Dv=64))[2] == capi.IMPL_MFMA
     assert _plan(_desc(D=8, Dv=40))[2] == capi.IMPL_MFMA
     assert _plan(_desc(D=84, Dv=84))[2] == capi.IMPL_GENERIC                    # 168-byte rows: not whole vectors
-    assert _plan(_desc(dtype=capi.F32, D=84, Dv=84))[2] == capi.IMPL_MFMA       # in f32 they are
+    assert _plan(_desc(dtype=capi.F32, D=84, Dv=84, B=8, Hq=16, Sq=4096, Skv=4096))[2] == capi.IMPL_MFMA       # in f32 they are
     # above 128: 16-bit prefill shapes on the prefill kernel for 256, decode shapes (up to 64 positions) and f32 on the 256
     # instance of the matrix-core split-KV kernels
     assert _plan(_desc(D=160, Dv=160))[2] == capi.IMPL_MFMA
@@ -108,7 +114,7 @@ def test_dispatch_choices():
     assert _plan(_desc(Sq=1, Skv=8192, B=2, Hq=8, Hkv=2, dtype=capi.F32))[2] == capi.IMPL_SPLITKV_MFMA
     assert _plan(_desc(Sq=1, Skv=8192, B=2, Hq=8, Hkv=8, dtype=capi.F32))[2] == capi.IMPL_SPLITKV             # one row: vector ALU
     assert _plan(_desc(Sq=64, Skv=8192, B=2, Hq=32, Hkv=2, dtype=capi.F32))[2] == capi.IMPL_SPLITKV_MFMA      # 1024 rows per KV head
-    assert _plan(_desc(Sq=65, Skv=8192, B=2, Hq=32, Hkv=2, dtype=capi.F32))[2] == capi.IMPL_MFMA              # more positions: prefill
+    assert _plan(_desc(Sq=65, Skv=8192, B=8, Hq=64, Hkv=2, dtype=capi.F32))[2] == capi.IMPL_MFMA              # more positions, 512 row blocks: prefill
     assert _plan(_desc(Sq=1, Skv=100, B=2, Hq=8, Hkv=2, dtype=capi.F32))[2] == capi.IMPL_MFMA                 # shortest caches: one workgroup per head
     _, splits, impl = _plan(_desc(Sq=1, Skv=8192, B=32, Hq=32, Hkv=8, dtype=capi.F32))
     assert impl == capi.IMPL_SPLITKV_MFMA and splits == 1

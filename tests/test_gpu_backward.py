@@ -180,7 +180,10 @@ def test_matrix_core_backward_with_padded_head_dimensions(gpu, dtype, dims):
                                       causal=causal, kv_lens=None if lens is None else lens_a.reshape(B, 1, 1))
         for name, x, a, r_ in zip(("dq", "dk", "dv"), (dq, dk, dv), auto[1:], (rq.reshape(B, Hq, Sq, D), rk.reshape(B, Hkv, Skv, D), rv.reshape(B, Hkv, Skv, Dv))):
             compare(name, x, r_, tol=tol)
-            assert np.array_equal(x, a), name + ": AUTO takes the same kernels"
+            if dtype == capi.F32:       # (AUTO's forward of an f32 launch this small is the split-KV kernel: last-bit differences in O and lse)
+                compare(name + " AUTO vs pinned", a, x, tol=2e-6)
+            else:
+                assert np.array_equal(x, a), name + ": AUTO takes the same kernels"
 
 
 @pytest.mark.parametrize("shape", [
@@ -214,10 +217,8 @@ def test_matrix_core_backward_f32_against_the_oracle(gpu, shape):
     refs = (rq.reshape(B, Hq, Sq, D), rk.reshape(B, Hkv, Skv, D), rv.reshape(B, Hkv, Skv, D))
     for name, x, a, g_, r_ in zip(("dq", "dk", "dv"), (dq, dk, dv), auto[1:], gen[1:], refs):
         compare(name, x, r_, tol=1e-5)
-        if Sq > 64:
-            assert np.array_equal(x, a), name + ": AUTO takes the same kernels, which have no run-to-run variation"
-        else:       # up to 64 positions AUTO's forward is the split-KV kernel: O and the row normalisers differ in the last bits
-            compare(name + " AUTO vs pinned", a, x, tol=2e-6)
+        # (AUTO's forward of launches this small is the f32 split-KV kernel: O and the row normalisers differ in the last bits)
+        compare(name + " AUTO vs pinned", a, x, tol=2e-6)
         compare(name + " generic vs matrix-core", g_, x, tol=2e-5)
     if lens is not None:
         for b in range(B):

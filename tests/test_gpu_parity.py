@@ -90,9 +90,10 @@ def test_buffer_round_trip(gpu):
 def test_config1_f32_single_head_noncausal(gpu):
     q, k, v = inputs(SEED0 + 0, 1, 1, 1, 128, 128, 64, 64, capi.F32)
     got, info = host.sdpa(q, k, v, capi.F32, scale=0.125, return_info=True)
-    assert info["impl"] == capi.IMPL_MFMA               # the IEEE-f32 matrix-core kernel
+    assert info["impl"] == capi.IMPL_SPLITKV_MFMA       # one 128-row block: the f32 split-KV kernel, 32 rows per workgroup
     ref = O.sdpa(q, k, v, scale=0.125)
     check(got, ref, 1e-5, "C1 f32 B1 H1 S128 D64")
+    check(host.sdpa(q, k, v, capi.F32, scale=0.125, impl=capi.IMPL_MFMA), ref, 1e-5, "C1, the IEEE-f32 matrix-core prefill kernel")
     check(host.sdpa(q, k, v, capi.F32, scale=0.125, impl=capi.IMPL_GENERIC), ref, 1e-5, "C1, generic kernel")
     assert np.abs(ref - O.brute_f64(q, k, v, scale=0.125)).max() < 1e-6
 
@@ -100,10 +101,11 @@ def test_config1_f32_single_head_noncausal(gpu):
 def test_config2_f32_multi_head_causal(gpu):
     q, k, v = inputs(SEED0 + 1, 4, 8, 8, 1024, 1024, 64, 64, capi.F32)
     got, info = host.sdpa(q, k, v, capi.F32, causal=True, return_info=True)
-    assert info["impl"] == capi.IMPL_MFMA
+    assert info["impl"] == capi.IMPL_SPLITKV_MFMA       # 256 row blocks of 128 on 256 compute units: the f32 split-KV kernel
     mask = O.causal_additive_mask(1024, 1024)                       # the explicit 0/-inf tensor the CPU op is given
     ref = O.sdpa(q, k, v, mask=mask)
     check(got, ref, 1e-5, "C2 f32 B4 H8 S1024 D64 causal")
+    check(host.sdpa(q, k, v, capi.F32, causal=True, impl=capi.IMPL_MFMA), ref, 1e-5, "C2, the IEEE-f32 matrix-core prefill kernel")
     check(host.sdpa(q, k, v, capi.F32, causal=True, impl=capi.IMPL_GENERIC), ref, 1e-5, "C2, generic kernel")
     # the same mask handed over as a dense additive tensor, as a caller of the reference's operator passes it, goes
     # through the mask path of either kernel
@@ -591,9 +593,12 @@ def test_head_dimensions_padded_into_the_matrix_core_kernels(gpu, dtype, dims):
     q, k, v = inputs(2100 + D + 3 * Dv, B, Hq, Hkv, Sq, Skv, D, Dv, dtype)
     lens = np.array([333, 97], np.int32)
     say("padded head dimensions: %s D=%d Dv=%d prefill" % (dtypes.NAMES[dtype], D, Dv))
-    got, lse, info = host.sdpa(q, k, v, dtype, causal=True, kv_lens=lens, return_info=True, return_lse=True)
-    assert info["impl"] == capi.IMPL_MFMA
+    got, lse, info = host.sdpa(q, k, v, dtype, causal=True, kv_lens=lens, impl=capi.IMPL_MFMA, return_info=True, return_lse=True)
     check(got, oracle_full(q, k, v, G=2, causal=True, kv_lens=lens), tol, "prefill D=%d Dv=%d" % (D, Dv))
+    got_a, info = host.sdpa(q, k, v, dtype, causal=True, kv_lens=lens, return_info=True)
+    # (f32 launches this small go 32 rows per workgroup through the split-KV kernel)
+    assert info["impl"] == (capi.IMPL_SPLITKV_MFMA if dtype == capi.F32 else capi.IMPL_MFMA)
+    check(got_a, oracle_full(q, k, v, G=2, causal=True, kv_lens=lens), tol, "AUTO, prefill D=%d Dv=%d" % (D, Dv))
     _, lse_g = host.sdpa(q, k, v, dtype, causal=True, kv_lens=lens, impl=capi.IMPL_GENERIC, return_lse=True)
     assert np.max(np.abs(lse - lse_g)) < (2e-5 if dtype == capi.F32 else 2e-2)
     # a dense additive mask (values and hidden blocks)
