@@ -30,7 +30,7 @@ struct SdpaParams {
     // split-KV only
     int32_t num_splits;
     int32_t split_len;         // keys per split (multiple of the kernel's key tile)
-    float* ws_acc;             // [B, Hq, Sq, num_splits, Dv] f32 partial numerators
+    float* ws_acc;             // [B, Hq, Sq, num_splits, Dp] f32 partial numerators (Dp == Dv for the vector-ALU kernel)
     float* ws_ml;              // [B, Hq, Sq, num_splits, 2]  running max (natural-log domain) and denominator
     // matrix-core prefill kernels with a dense mask: one byte per block of 32 query rows x 32 keys (0 mixed, 1 all zero,
     // 2 all -inf), written by mask_classify_kernel ahead of the attention kernel, in the caller's workspace;
