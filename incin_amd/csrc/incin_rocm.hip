@@ -180,7 +180,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     // (above 128: sdpa_prefill_wide.hip - 16-bit storage, any finite scale, a dense mask whose rows it can read 8 bytes at a time)
     const bool mfma_ok = wide ? layout_ok && d->dtype != INCIN_ROCM_F32 && tile_off_ok && std::isfinite(d->scale) && (!d->add_mask || mask_rows_vector_loadable(d))
                               : layout_ok && tile_off_ok && std::isfinite(d->scale) && (d->dtype == INCIN_ROCM_F32 || d->scale > 0.0f);
-    const bool split_ok = fast_ok && head_exact && d->Sq <= 64;
+    const bool split_ok = layout_ok && head_exact && d->Sq <= 64;      // (the vector-ALU kernel takes a dense mask)
     // the matrix-core split-KV kernels (16-bit and f32): blocks addressed like the prefill kernels' tiles; the f32 kernel and
     // the 256 instances take any number of query positions
     const bool split_mfma_ok = fast_ok && (d->Sq <= 64 || wide || d->dtype == INCIN_ROCM_F32) && tile_off_ok && std::isfinite(d->scale);
@@ -246,7 +246,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
                     "scaled_dot_product_attention: the matrix-core split-KV kernels need D and Dv <= 256 in whole 16-byte vectors, Sq <= 64 (any Sq in f32 and above 128), no dense mask, a finite scale and 16-byte aligned rows");
     if (impl == INCIN_ROCM_IMPL_SPLITKV && !split_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
-                    "scaled_dot_product_attention: the split-KV kernel needs D == Dv in {64,128}, Sq <= 64, no dense mask and 16-byte aligned rows");
+                    "scaled_dot_product_attention: the split-KV kernel needs D == Dv in {64,128}, Sq <= 64 and 16-byte aligned rows");
     if (impl == INCIN_ROCM_IMPL_GENERIC && (d->D > 256 || d->Dv > 256))
         return fail(INCIN_ROCM_EUNSUPPORTED,
                     "scaled_dot_product_attention: head dimension %lld/%lld exceeds 256, no Rocm kernel covers it",

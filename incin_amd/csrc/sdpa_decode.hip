@@ -57,7 +57,9 @@ __device__ __forceinline__ float group_sum(float x)
     return x;
 }
 
-template <typename T, int D, int RMAX, int U>
+// DENSE: a dense additive mask (any broadcast strides): its value for (row, key) is added to the scaled score - what an
+// additive position bias or a mask tensor with holes needs at decode time.
+template <typename T, int D, int RMAX, int U, bool DENSE = false>
 __global__ __launch_bounds__(256) void sdpa_decode_split_kernel(SdpaParams p)
 {
     typedef typename Vec16<T>::type vec_t;
@@ -91,6 +93,7 @@ __global__ __launch_bounds__(256) void sdpa_decode_split_kernel(SdpaParams p)
     const float sc = p.scale * Softexp<T>::kPre;
     float qf[RMAX][VEC];
     int lim[RMAX];
+    [[maybe_unused]] const T* mrow[RMAX];      // this row of the dense mask
 #pragma unroll
     for (int r = 0; r < RMAX; ++r) {
         const int row = r0 + r;
@@ -106,6 +109,7 @@ __global__ __launch_bounds__(256) void sdpa_decode_split_kernel(SdpaParams p)
             if (cl < l) l = cl;
         }
         lim[r] = valid ? l : 0;
+        if (DENSE) mrow[r] = (const T*)p.mask + (int64_t)b * p.m_sb + (int64_t)(hkv * p.G + g) * p.m_sh + (int64_t)i * p.m_si;
     }
 
     float m_run[RMAX], l_run[RMAX], acc[RMAX][VEC];
@@ -151,8 +155,9 @@ __global__ __launch_bounds__(256) void sdpa_decode_split_kernel(SdpaParams p)
                 float part = 0.0f;
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) part = fmaf(qf[r][e], kf[e], part);
-                part = group_sum<LPR>(part);
-                s[r][u] = (key < lim[r]) ? part * sc : -INFINITY;
+                part = group_sum<LPR>(part) * sc;
+                if (DENSE) part = fmaf(to_f32(mrow[r][(int64_t)min(key, k_last) * p.m_sj]), Softexp<T>::kPre, part);
+                s[r][u] = (key < lim[r]) ? part : -INFINITY;
             }
         }
 #pragma unroll
@@ -317,13 +322,13 @@ hipError_t launch_sdpa_combine(const SdpaParams& p, int dtype, hipStream_t strea
     }
 }
 
-template <typename T, int D, int RMAX, int U>
+template <typename T, int D, int RMAX, int U, bool DENSE>
 static hipError_t launch_decode_t(const SdpaParams& p, hipStream_t stream)
 {
     constexpr int VEC = Vec16<T>::N;
     constexpr int NSTREAM = 4 * (64 / (D / VEC));
     size_t lds = (size_t)(NSTREAM * RMAX * D + NSTREAM * RMAX * 2) * sizeof(float);
-    auto kern = sdpa_decode_split_kernel<T, D, RMAX, U>;
+    auto kern = sdpa_decode_split_kernel<T, D, RMAX, U, DENSE>;
     hipError_t e;
     // the dynamic-LDS limit of this instance is raised once per device, not per launch
     static std::atomic<uint64_t> prepared{0};
@@ -345,14 +350,20 @@ static hipError_t launch_decode_t(const SdpaParams& p, hipStream_t stream)
     return e;
 }
 
+template <typename T, int D, bool DENSE>
+static hipError_t launch_decode_rd(const SdpaParams& p, hipStream_t stream)
+{
+    const int R = p.G * p.Sq;
+    if (R <= 1) return launch_decode_t<T, D, 1, 8, DENSE>(p, stream);
+    if (R <= 2) return launch_decode_t<T, D, 2, 8, DENSE>(p, stream);
+    if (R <= 4) return launch_decode_t<T, D, 4, 4, DENSE>(p, stream);
+    return launch_decode_t<T, D, 8, 4, DENSE>(p, stream);
+}
+
 template <typename T, int D>
 static hipError_t launch_decode_r(const SdpaParams& p, hipStream_t stream)
 {
-    const int R = p.G * p.Sq;
-    if (R <= 1) return launch_decode_t<T, D, 1, 8>(p, stream);
-    if (R <= 2) return launch_decode_t<T, D, 2, 8>(p, stream);
-    if (R <= 4) return launch_decode_t<T, D, 4, 4>(p, stream);
-    return launch_decode_t<T, D, 8, 4>(p, stream);
+    return p.mask ? launch_decode_rd<T, D, true>(p, stream) : launch_decode_rd<T, D, false>(p, stream);
 }
 
 // Keys per wavefront tile for the instance launch_sdpa_decode would pick; the

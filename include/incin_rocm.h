@@ -49,7 +49,7 @@ enum {
                                       and unequal head dimensions are zero-padded into LDS); bf16/f16 (scale > 0) and IEEE-f32
                                       matrix instructions for f32; dense mask allowed.  bf16/f16 also above 128, up to 256
                                       (an instance for 256, any finite scale; a dense mask with 8-byte aligned rows)  */
-    INCIN_ROCM_IMPL_SPLITKV = 3,   /* vector-ALU split-KV decode kernel + combine: D == Dv in {64,128}, few query rows */
+    INCIN_ROCM_IMPL_SPLITKV = 3,   /* vector-ALU split-KV decode kernel + combine: D == Dv in {64,128}, few query rows; dense mask allowed */
     INCIN_ROCM_IMPL_MFMA64 = 4,    /* retired (a prefill kernel with 64 query rows per wavefront): refused with INCIN_ROCM_EUNSUPPORTED */
     INCIN_ROCM_IMPL_SPLITKV_MFMA = 5 /* split-KV kernels on the matrix cores + combine: D and Dv <= 256 in whole 16-byte vectors (instances for
                                       64, 128 and 256), Sq <= 64 - any Sq when a head dimension is above 128, which only these kernels

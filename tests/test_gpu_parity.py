@@ -700,6 +700,38 @@ def test_head_dimensions_outside_the_matrix_core_kernels(gpu):
         check(got, oracle_full(q, k, v, causal=True), TOL[dtype], "generic D=%d" % D)
 
 
+@pytest.mark.parametrize("dtype", [capi.BF16, capi.F16, capi.F32], ids=lambda x: dtypes.NAMES[x])
+@pytest.mark.parametrize("shape", [
+    # B, Hq, Hkv, Sq, Skv, D
+    (2, 8, 2, 1, 1500, 128),          # grouped-query decode, 4 rows per KV head
+    (3, 4, 4, 1, 700, 64),            # one row per KV head
+    (1, 16, 2, 1, 2049, 128),         # 8 rows, a ragged last tile
+    (2, 4, 2, 3, 900, 64),            # 6 rows: a short causal run
+])
+def test_decode_with_a_dense_additive_mask(gpu, dtype, shape):
+    """Decode shapes with a mask tensor - an additive position bias per head ([1, Hq, 1, Skv]) and a [B, 1, Sq, Skv] mask with
+    hidden stretches, on top of key counts - go through the vector-ALU split-KV kernel (up to 8 rows per KV head), which
+    adds the mask's values to the scaled scores: against the oracle, split counts chosen and forced."""
+    B, Hq, Hkv, Sq, Skv, D = shape
+    q, k, v = inputs(2700 + sum(shape), B, Hq, Hkv, Sq, Skv, D, D, dtype)
+    bias = (-0.02 * np.arange(Skv)[::-1].astype(np.float32))[None, None, None, :] * (1.0 + np.arange(Hq, dtype=np.float32))[None, :, None, None]
+    bias = dtypes.round_to(np.broadcast_to(bias, (1, Hq, Sq, Skv)).copy(), dtype)
+    r = rng(17)
+    holes = (r.standard_normal((B, 1, Sq, Skv)) * 0.3).astype(np.float32)
+    holes[:, :, :, 100:400] = -np.inf
+    holes[0, :, :, Skv - 50:] = -np.inf
+    holes = dtypes.round_to(holes, dtype)
+    lens = np.array([Skv - 7 * b for b in range(B)], np.int32)
+    for name, m in (("bias per head", bias), ("holes per batch entry", holes)):
+        full = np.broadcast_to(m, (B, Hq, Sq, Skv)) + np.where(np.arange(Skv)[None, :] < lens[:, None], 0.0, -np.inf).astype(np.float32)[:, None, None, :]
+        ref = oracle_full(q, k, v, G=Hq // Hkv, mask=full)
+        for splits in (0, 1, 5):
+            say("decode with a mask: %s %r %s splits=%d" % (dtypes.NAMES[dtype], shape, name, splits))
+            got, info = host.sdpa(q, k, v, dtype, mask=m, kv_lens=lens, num_splits=splits, return_info=True)
+            assert info["impl"] == capi.IMPL_SPLITKV
+            check(got, ref, TOL[dtype], "decode with a mask (%s), splits=%d->%d" % (name, splits, info["splits"]))
+
+
 def test_decode_splitkv_matrix_cores_lengths_strides_scale(gpu):
     """Key counts per batch entry (one of them 0: NaN rows, as the reference), a negative scale (the scale is applied to
     the f32 scores, so its sign does not matter to this kernel), and AUTO's choice for grouped-query decode."""
