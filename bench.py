@@ -252,6 +252,26 @@ def decode_gqa_leg(steps, warmup, only_shape=None):
                              "frac": kv_bytes / (ev_mean * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None,
                              "algorithmic_bytes_per_launch": kv_bytes, "launch_ms_mean": ev_mean, "launch_ms_min": ev_min},
                 "parity_max_abs_err": w.parity(16)}
+        if name == "gqa4_b32_kv8192" and only_shape is None:
+            # the same launch with an additive position bias per query head, handed over as the reference's operator takes it: a
+            # [1, Hq, 1, KV] mask tensor.  AUTO sends it to the vector-ALU split-KV kernel, which adds the mask's values.
+            bias = (-0.02 * np.arange(Skv)[::-1].astype(np.float32))[None, None, None, :] * (1.0 + np.arange(Hq, dtype=np.float32))[None, :, None, None]
+            tm = capi.DeviceBuffer.from_numpy(dtypes.encode(np.ascontiguousarray(bias), dt))
+            w.desc.add_mask = tm.ptr
+            for a, st in enumerate((0, Skv, 0, 1)):
+                w.desc.mask_stride[a] = st
+            w.replan()
+            wall_b, ev_b, _, _ = w.time(n, warmup)
+            from oracle import oracle as O
+            q, k, v = (dtypes.round_to(x, dt) for x in w.host)
+            rows = np.array([[0, 0], [B * Hq - 1, 0], [5, 0], [B * Hq // 2, 0]])
+            ref = O.sdpa_rows(q.reshape(B, Hkv, Hq // Hkv, Sq, 128), k[:, :, None], v[:, :, None], rows,
+                              mask=dtypes.round_to(bias, dt).reshape(1, Hkv, Hq // Hkv, 1, Skv))
+            err = float(np.abs(w.to.to_f32().reshape(B * Hq, Sq, 128)[rows[:, 0], rows[:, 1]] - ref).max())
+            entry["with_bias_mask_tensor"] = {"kernel": names.get(w.impl, str(w.impl)), "num_splits": w.splits, "ms_per_step": wall_b,
+                                              "kv_gb_per_s": kv_bytes / (wall_b * 1e-3) / 1e9, "frac": kv_bytes / (ev_b * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                                              "parity_max_abs_err": err}
+            tm.free()
         w.free()
         out[name] = entry
     return out
