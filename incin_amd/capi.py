@@ -31,7 +31,7 @@ EXPORTS = [
     "incin_rocm_sdpa_workspace", "incin_rocm_sdpa_fwd", "incin_rocm_sdpa_fwd_static",
     "incin_rocm_sizeof_kv_append_desc", "incin_rocm_kv_append",
     "incin_rocm_sizeof_sdpa_bwd_desc", "incin_rocm_sdpa_bwd_workspace", "incin_rocm_sdpa_bwd",
-    "incin_rocm_matrix_rate", "incin_rocm_read_rate",
+    "incin_rocm_matrix_rate", "incin_rocm_read_rate", "incin_rocm_lds_fill",
 ]
 
 
@@ -159,6 +159,7 @@ def load():
     lib.incin_rocm_kv_append.argtypes = [C.POINTER(KvAppendDesc), C.c_void_p]
     lib.incin_rocm_matrix_rate.argtypes = [C.c_int32, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.POINTER(C.c_double), C.c_void_p]
     lib.incin_rocm_read_rate.argtypes = [C.c_int32, C.c_void_p, C.c_size_t, C.c_int32, C.c_void_p, C.c_void_p]
+    lib.incin_rocm_lds_fill.argtypes = [C.c_int32, C.c_uint32, C.c_void_p, C.c_void_p]
     _lib = lib
     return lib
 
@@ -240,6 +241,11 @@ def sdpa_bwd(desc, stream=None):
 def read_rate(src, nbytes, nontemporal, sink, stream=None, dev=0):
     """One launch of the read-only kernel over nbytes of src (DeviceBuffer); time it with events."""
     check(load().incin_rocm_read_rate(dev, src.ptr, nbytes, 1 if nontemporal else 0, sink.ptr, stream))
+
+
+def lds_fill(pattern, sink, stream=None, dev=0):
+    """Writes the 32-bit pattern into the whole LDS of every compute unit (sink: a DeviceBuffer of 4 bytes or more)."""
+    check(load().incin_rocm_lds_fill(dev, pattern, sink.ptr, stream))
 
 
 def matrix_rate(operands, sink, mix, iterations, stream=None, dev=0):

@@ -28,6 +28,7 @@ hipError_t launch_mask_classify(const SdpaParams& p, int dtype, hipStream_t stre
 hipError_t launch_sdpa_decode(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_sdpa_decode_mfma(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_read_rate(const void* src, void* sink, size_t bytes, int nontemporal, hipStream_t stream);
+hipError_t launch_lds_fill(void* sink, uint32_t pattern, hipStream_t stream);
 int decode_mfma_chunk_rows(int R, int dtype, int d_pad);
 int decode_mfma_workgroups_per_cu(int chunk_rows, int64_t split_len, int dtype, int d_pad);
 int decode_keys_per_tile(int dtype, int D, int R);
@@ -758,6 +759,15 @@ int incin_rocm_read_rate(int32_t dev, const void* src, size_t bytes, int32_t non
     if (int rc = use_device(dev)) return rc;
     const hipError_t e = incin_rocm::launch_read_rate(src, sink, bytes, nontemporal != 0, (hipStream_t)stream);
     if (e != hipSuccess) return hip_fail(e, "read rate launch");
+    return 0;
+}
+
+int incin_rocm_lds_fill(int32_t dev, uint32_t pattern, void* sink, void* stream)
+{
+    if (!sink) return fail(INCIN_ROCM_EINVAL, "lds_fill: null pointer");
+    if (int rc = use_device(dev)) return rc;
+    const hipError_t e = incin_rocm::launch_lds_fill(sink, pattern, (hipStream_t)stream);
+    if (e != hipSuccess) return hip_fail(e, "lds fill launch");
     return 0;
 }
 

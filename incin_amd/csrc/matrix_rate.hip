@@ -108,4 +108,35 @@ hipError_t launch_read_rate(const void* src, void* sink, size_t bytes, int nonte
     return hipGetLastError();
 }
 
+// Writes `pattern` into every 32-bit word of a 160 KiB LDS allocation, one workgroup per LDS in flight: what the next
+// kernels on those compute units find in LDS they have not written themselves.
+__global__ __launch_bounds__(256) void lds_fill_kernel(uint32_t* sink, uint32_t pattern)
+{
+    extern __shared__ uint32_t lds_words[];
+    constexpr int kWords = 160 * 1024 / 4;
+    for (int i = threadIdx.x; i < kWords; i += 256) lds_words[i] = pattern;
+    __syncthreads();
+    uint32_t acc = 0;
+    for (int i = threadIdx.x; i < kWords; i += 256 * 64) acc ^= lds_words[(i + 4099) % kWords];
+    if (acc == 0x9e3779b9u && pattern != 0x9e3779b9u) sink[0] = acc;                      // (never: keeps the stores alive)
+}
+
+// sink: 4 bytes.  1024 workgroups: four passes over 256 compute units, so each one's LDS is written whichever way the
+// dispatcher spreads them.
+hipError_t launch_lds_fill(void* sink, uint32_t pattern, hipStream_t stream)
+{
+    constexpr int kBytes = 160 * 1024;
+    static thread_local int configured_dev = -1;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (configured_dev != dev) {
+        e = hipFuncSetAttribute((const void*)lds_fill_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kBytes);
+        if (e != hipSuccess) return e;
+        configured_dev = dev;
+    }
+    hipLaunchKernelGGL(lds_fill_kernel, dim3(1024), dim3(256), kBytes, stream, (uint32_t*)sink, pattern);
+    return hipGetLastError();
+}
+
 }  // namespace incin_rocm

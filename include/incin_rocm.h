@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define INCIN_ROCM_ABI_VERSION 7
+#define INCIN_ROCM_ABI_VERSION 8
 
 /* ---- status codes (mapped to incin_core::Error variants by the Rust side;
  *      crates/incin-core/src/err.rs:109-223) --------------------------------- */
@@ -271,6 +271,12 @@ int incin_rocm_matrix_rate(int32_t dev, const void* operands, void* sink, int32_
  * delivers to a kernel that only reads, the ceiling the split-KV kernels live under; bench.py reports it beside their
  * roofline.  `sink` takes 16 KiB.  Time it with events on `stream`. */
 int incin_rocm_read_rate(int32_t dev, const void* src, size_t bytes, int32_t nontemporal, void* sink, void* stream);
+
+/* No counterpart in the reference.  One launch that writes `pattern` into every 32-bit word of the LDS of every compute
+ * unit (1024 workgroups of 160 KiB).  The matrix-core kernels pad a head dimension below their instance's with zeros
+ * that the copy engine writes into LDS, and read nothing else they have not written; a test fills LDS with the bit
+ * pattern of a NaN first and shows that no result depends on what LDS held.  `sink` takes 4 bytes and is never written. */
+int incin_rocm_lds_fill(int32_t dev, uint32_t pattern, void* sink, void* stream);
 
 /* ---- key/value cache append ----------------------------------------------------
  * No counterpart in the reference (it has no cache: a decode loop there concatenates tensors,

@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), "missing export %s" % n
     assert set(names) == set(capi.EXPORTS)
-    assert lib.incin_rocm_abi_version() == 7
+    assert lib.incin_rocm_abi_version() == 8
 
 
 def test_descriptor_layout_matches():
@@ -217,6 +217,8 @@ def test_matrix_rate_validation():
     assert lib.incin_rocm_read_rate(0, 0x1000, (1 << 27) + 4096, 1, 0x1000, None) == capi.EINVAL      # not a multiple of 128 MiB
     assert lib.incin_rocm_read_rate(0, 0x1008, 1 << 27, 1, 0x1000, None) == capi.EINVAL               # misaligned
     assert b"read_rate" in lib.incin_rocm_last_error()
+    assert lib.incin_rocm_lds_fill(0, 0x7fc00000, None, None) == capi.EINVAL
+    assert b"lds_fill" in lib.incin_rocm_last_error()
 
 
 def _bwd(fwd_kw=None, **kw):

@@ -946,6 +946,42 @@ def test_matrix_rate_diagnostic(gpu):
     sink.free()
 
 
+def test_padded_head_dimensions_do_not_depend_on_what_lds_held(gpu):
+    """The matrix-core kernels pad a head dimension below their instance's with zeros the copy engine writes into LDS
+    (lanes whose 16 bytes lie beyond a row's data address memory no descriptor covers and deliver zeros).  Were those
+    lanes to write nothing, the padding would be whatever the last kernel left in LDS - usually small numbers, so an
+    ordinary parity test could pass by luck.  Fill every compute unit's LDS with NaN bit patterns (as bf16/f16 pairs,
+    as f32, all ones) before each launch: results carry no NaN, match the oracle and are bit-identical to the launch
+    before the fill."""
+    BF, F = capi.BF16, capi.F32
+    cases = [  # dtype, D, Dv, Hq, Sq, Skv, causal, impl asked, impl run
+        (BF, 96, 96, 4, 200, 333, True, capi.IMPL_AUTO, capi.IMPL_MFMA),                 # prefill, 128 instance
+        (capi.F16, 40, 72, 4, 200, 333, True, capi.IMPL_AUTO, capi.IMPL_MFMA),           # prefill, D and Dv in different instances' reach
+        (BF, 40, 72, 4, 1, 1500, False, capi.IMPL_AUTO, capi.IMPL_SPLITKV_MFMA),         # decode
+        (BF, 192, 128, 4, 200, 333, True, capi.IMPL_AUTO, capi.IMPL_MFMA),               # prefill, 256 instance
+        (BF, 160, 160, 8, 1, 1500, False, capi.IMPL_AUTO, capi.IMPL_SPLITKV_MFMA),       # decode, 256 instance
+        (F, 20, 36, 4, 200, 333, True, capi.IMPL_AUTO, capi.IMPL_SPLITKV_MFMA),          # f32: a small prefill launch
+        (F, 20, 36, 4, 200, 333, True, capi.IMPL_MFMA, capi.IMPL_MFMA),                  # f32 prefill kernel
+        (F, 100, 100, 8, 1, 1500, False, capi.IMPL_AUTO, capi.IMPL_SPLITKV_MFMA),        # f32 decode
+    ]
+    sink = capi.DeviceBuffer.from_numpy(np.full(4, 7, np.uint32))
+    for dtype, D, Dv, Hq, Sq, Skv, causal, impl, impl_run in cases:
+        q, k, v = inputs(2700 + D + Dv, 2, Hq, 2, Sq, Skv, D, Dv, dtype)
+        ref = oracle_full(q, k, v, G=Hq // 2, causal=causal)
+        first, info = host.sdpa(q, k, v, dtype, causal=causal, impl=impl, return_info=True)
+        assert info["impl"] == impl_run
+        for pattern in (0x7fc07fc0, 0x7e007e00, 0x7fc00000, 0xffffffff):
+            say("LDS filled with %08x: %s D=%d Dv=%d Sq=%d impl %d" % (pattern, dtypes.NAMES[dtype], D, Dv, Sq, impl_run))
+            capi.lds_fill(pattern, sink)
+            got = host.sdpa(q, k, v, dtype, causal=causal, impl=impl)
+            assert not np.isnan(got).any(), "NaN after filling LDS with %08x, D=%d Dv=%d" % (pattern, D, Dv)
+            check(got, ref, TOL[dtype], "after filling LDS with %08x, D=%d Dv=%d" % (pattern, D, Dv))
+            assert np.array_equal(got, first)
+    capi.sync()
+    assert np.array_equal(sink.to_numpy(np.uint32, (4,)), np.full(4, 7, np.uint32))
+    sink.free()
+
+
 def test_read_rate_diagnostic(gpu):
     """The read-only kernel runs, writes nothing (its sink keeps what it held) and takes about the time the memory system
     needs for the bytes (between 2 and 8 TB/s: a sanity range, the figure itself is bench.py's business)."""
