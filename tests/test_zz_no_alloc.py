@@ -71,6 +71,12 @@ def test_static_scratch_matches_workspace_launch(gpu):
         ("prefill with a dense mask (block flags)",
          dict(B=2, Hq=4, Hkv=2, Sq=700, Skv=700, D=128, causal=False, impl=capi.IMPL_MFMA, causal_mask_tensor=True),
          dict(B=1, Hq=2, Hkv=2, Sq=100, Skv=333, D=128, causal=False, impl=capi.IMPL_MFMA, causal_mask_tensor=True)),
+        ("matrix-core split-KV decode, head dimensions padded to the 256 and the 128 instance (partial rows that wide)",
+         dict(B=2, Hq=16, Hkv=2, Sq=1, Skv=4096, D=192, causal=False, impl=capi.IMPL_SPLITKV_MFMA, num_splits=8),
+         dict(B=2, Hq=12, Hkv=2, Sq=3, Skv=1500, D=96, causal=True, impl=capi.IMPL_SPLITKV_MFMA, num_splits=3, kv_lens=[1500, 700])),
+        ("prefill with the keys split, head dimension 112 (128 instance) then 40 (64 instance)",
+         dict(B=1, Hq=4, Hkv=2, Sq=100, Skv=4500, D=112, causal=True, impl=capi.IMPL_MFMA),
+         dict(B=1, Hq=2, Hkv=2, Sq=40, Skv=4100, D=40, causal=False, impl=capi.IMPL_MFMA, num_splits=3)),
     ]
     for name, big, small in big_small:
         pb, ps = Problem(7, **big), Problem(8, **small)
