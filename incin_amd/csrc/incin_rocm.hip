@@ -205,7 +205,13 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         // Head dimensions above 128: the 16-bit prefill kernel for 256 where there are more than 64 query positions (128 rows
         // share a K / V tile there, 32 in the split-KV kernel: D = 256 causal prefill 775 - 890 against 340 - 460 TFLOP/s), the
         // split-KV kernels' 256 instance for decode shapes and - f32 has no such prefill kernel - for every f32 shape.
-        if (wide && mfma_ok && d->Sq > 64) impl = INCIN_ROCM_IMPL_MFMA;
+        // That prefill kernel does not split the keys: a launch that gives it workgroups for at most half the compute units
+        // (the chunks of a long prompt, few heads) goes 32 rows per workgroup, keys split as needed, through the split-KV
+        // kernel (measured, bf16 causal, D = 256: 8 heads x 128 x 8192 0.305 -> 0.039 ms; 32 x 256 x 16384 0.60 -> 0.26;
+        // 8 x 1024 x 32768 1.18 -> 0.56; 16 x 1024 x 4096 - 128 workgroups - 0.158 -> 0.121; at 256 workgroups
+        // (2 x 32 x 512 x 512) the prefill kernel is ahead, 0.031 against 0.057).
+        const bool wide_underfilled = d->B * d->Hq * ((d->Sq + 127) / 128) * 2 <= compute_units_of(d->device);
+        if (wide && mfma_ok && d->Sq > 64 && !(split_mfma_ok && wide_underfilled)) impl = INCIN_ROCM_IMPL_MFMA;
         else if (wide && split_mfma_ok) impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
         // f32 (sdpa_decode_f32.hip): from two rows per KV head on, whatever the count - the f32 prefill kernel would spend a
         // 32-row matrix instruction on every query head's few rows (32 heads of a group at one position each: 8.4 ms

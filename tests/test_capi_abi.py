@@ -73,8 +73,13 @@ def test_dispatch_choices():
     assert _plan(_desc(dtype=capi.F32, D=84, Dv=84, B=8, Hq=16, Sq=4096, Skv=4096))[2] == capi.IMPL_MFMA       # in f32 they are
     # above 128: 16-bit prefill shapes on the prefill kernel for 256, decode shapes (up to 64 positions) and f32 on the 256
     # instance of the matrix-core split-KV kernels
-    assert _plan(_desc(D=160, Dv=160))[2] == capi.IMPL_MFMA
-    assert _plan(_desc(D=128, Dv=136))[2] == capi.IMPL_MFMA
+    assert _plan(_desc(D=160, Dv=160, B=64))[2] == capi.IMPL_MFMA
+    assert _plan(_desc(D=128, Dv=136, B=64))[2] == capi.IMPL_MFMA
+    # (that prefill kernel does not split the keys: launches that give it workgroups for at most half the compute units go
+    # 32 rows per workgroup through the split-KV kernel - 8 and 128 workgroups here, then 136)
+    assert _plan(_desc(D=160, Dv=160))[2] == capi.IMPL_SPLITKV_MFMA
+    assert _plan(_desc(D=256, Dv=256, B=1, Hq=16, Hkv=16, Sq=1024, Skv=4096, causal=1))[2] == capi.IMPL_SPLITKV_MFMA
+    assert _plan(_desc(D=256, Dv=256, B=1, Hq=17, Hkv=17, Sq=1024, Skv=4096, causal=1))[2] == capi.IMPL_MFMA
     assert _plan(_desc(D=256, Dv=256, Sq=4096, Skv=4096, causal=1))[2] == capi.IMPL_MFMA
     assert _plan(_desc(D=256, Dv=256, Sq=4096, Skv=4096, causal=1, impl=capi.IMPL_SPLITKV_MFMA))[2] == capi.IMPL_SPLITKV_MFMA
     assert _plan(_desc(D=256, Dv=256, Sq=64, Skv=4096, causal=1))[2] == capi.IMPL_SPLITKV_MFMA

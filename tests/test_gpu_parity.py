@@ -637,7 +637,7 @@ def test_head_dimensions_above_128(gpu, dtype, dims):
     D, Dv = dims
     tol = TOL[dtype]
     for (B, Hq, Hkv, Sq, Skv), split_list in (((2, 2, 2, 1, 1500), (0, 1, 5)), ((2, 8, 2, 3, 1500), (0, 3)), ((2, 4, 2, 200, 333), (0, 1, 2)),
-                                              ((1, 2, 1, 70, 70), (0,)), ((1, 40, 1, 1, 40), (0,))):
+                                              ((1, 2, 1, 70, 70), (0,)), ((1, 40, 1, 1, 40), (0,)), ((1, 136, 8, 129, 140), (0,))):
         q, k, v = inputs(2500 + D + Dv + Sq, B, Hq, Hkv, Sq, Skv, D, Dv, dtype)
         lens = np.array([Skv, max(Skv // 3, 1)][:B], np.int32)
         ref = oracle_full(q, k, v, G=Hq // Hkv, causal=True, kv_lens=lens)
@@ -647,8 +647,16 @@ def test_head_dimensions_above_128(gpu, dtype, dims):
                                        return_info=True, return_lse=True)
             check(got, ref, tol, "D=%d Dv=%d Sq=%d splits=%d->%d" % (D, Dv, Sq, splits, info["splits"]))
         got, lse, info = host.sdpa(q, k, v, dtype, causal=True, kv_lens=lens, return_info=True, return_lse=True)
-        assert info["impl"] == (capi.IMPL_MFMA if Sq > 64 and dtype != capi.F32 else capi.IMPL_SPLITKV_MFMA)
+        # (16-bit: the prefill kernel for 256 once its 128-row workgroups cover more than half the compute units)
+        prefill_256 = Sq > 64 and dtype != capi.F32 and B * Hq * ((Sq + 127) // 128) * 2 > capi.device_info(0).compute_units
+        assert info["impl"] == (capi.IMPL_MFMA if prefill_256 else capi.IMPL_SPLITKV_MFMA)
         check(got, ref, tol, "AUTO, D=%d Dv=%d Sq=%d" % (D, Dv, Sq))
+        if Sq > 64 and dtype != capi.F32:
+            got, lse_p, info = host.sdpa(q, k, v, dtype, causal=True, kv_lens=lens, impl=capi.IMPL_MFMA, return_info=True, return_lse=True)
+            assert info["impl"] == capi.IMPL_MFMA
+            check(got, ref, tol, "prefill kernel for 256, D=%d Dv=%d Sq=%d" % (D, Dv, Sq))
+            fin = np.isfinite(lse)
+            assert np.array_equal(fin, np.isfinite(lse_p)) and np.max(np.abs(lse[fin] - lse_p[fin])) < 2e-2
         _, lse_g = host.sdpa(q, k, v, dtype, causal=True, kv_lens=lens, impl=capi.IMPL_GENERIC, return_lse=True)
         fin = np.isfinite(lse_g)
         assert np.array_equal(fin, np.isfinite(lse)) and np.max(np.abs(lse[fin] - lse_g[fin])) < (2e-5 if dtype == capi.F32 else 2e-2)
@@ -958,7 +966,8 @@ def test_padded_head_dimensions_do_not_depend_on_what_lds_held(gpu):
         (BF, 96, 96, 4, 200, 333, True, capi.IMPL_AUTO, capi.IMPL_MFMA),                 # prefill, 128 instance
         (capi.F16, 40, 72, 4, 200, 333, True, capi.IMPL_AUTO, capi.IMPL_MFMA),           # prefill, D and Dv in different instances' reach
         (BF, 40, 72, 4, 1, 1500, False, capi.IMPL_AUTO, capi.IMPL_SPLITKV_MFMA),         # decode
-        (BF, 192, 128, 4, 200, 333, True, capi.IMPL_AUTO, capi.IMPL_MFMA),               # prefill, 256 instance
+        (BF, 192, 128, 4, 200, 333, True, capi.IMPL_MFMA, capi.IMPL_MFMA),               # prefill kernel for 256
+        (BF, 192, 128, 4, 200, 333, True, capi.IMPL_AUTO, capi.IMPL_SPLITKV_MFMA),       # a launch this small: split-KV, 256 instance
         (BF, 160, 160, 8, 1, 1500, False, capi.IMPL_AUTO, capi.IMPL_SPLITKV_MFMA),       # decode, 256 instance
         (F, 20, 36, 4, 200, 333, True, capi.IMPL_AUTO, capi.IMPL_SPLITKV_MFMA),          # f32: a small prefill launch
         (F, 20, 36, 4, 200, 333, True, capi.IMPL_MFMA, capi.IMPL_MFMA),                  # f32 prefill kernel
