@@ -225,7 +225,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         // takes them 32 rows per workgroup with the keys dealt to its four wavefronts - four times the workgroups, a quarter
         // of the keys per wavefront - where the prefill kernel's wavefronts each walk all keys for their 32 rows behind
         // 64-cycle matrix instructions (measured, causal: one head of 128 x 128 13.3 -> 8.6 us; 2 x 8 heads x 512 x 512 at
-        // D = 128 73 -> 28; 128 workgroups' worth of 1024 x 1024 80 -> 33; 256 - BASELINE config 2 - 80 -> 65; level at 512).
+        // D = 128 73 -> 28; 128 workgroups' worth of 1024 x 1024 80 -> 33; 256 - 4 x 8 heads x 1024 x 1024 at D = 64 - 80 -> 65; level at 512).
         // Not the chunks of a long prompt, where the prefill kernel splits the keys itself (below) and runs at 80 % of the peak.
         else if (d->dtype == INCIN_ROCM_F32 && split_mfma_ok && d->Sq > 64 && !(d->Skv >= 4096 && d->Skv >= 4 * d->Sq) &&
                  d->B * d->Hq * ((d->Sq + 127) / 128) <= compute_units_of(d->device))

@@ -59,7 +59,7 @@ def test_dispatch_choices():
     # f32: the IEEE-f32 matrix-core prefill kernel where the launch gives it more than one 128-row workgroup per compute unit
     # (256 here: no device to ask), the f32 split-KV kernel - 32 rows per workgroup, keys dealt to its wavefronts - below that
     assert _plan(_desc(dtype=capi.F32, B=8, Hq=16, Sq=4096, Skv=4096))[2] == capi.IMPL_MFMA
-    assert _plan(_desc(dtype=capi.F32, B=4, Hq=8, Sq=1024, Skv=1024))[2] == capi.IMPL_SPLITKV_MFMA      # BASELINE config 2: 256 workgroups
+    assert _plan(_desc(dtype=capi.F32, B=4, Hq=8, Sq=1024, Skv=1024))[2] == capi.IMPL_SPLITKV_MFMA      # 4 x 8 heads x 1024 x 1024: 256 workgroups
     assert _plan(_desc(dtype=capi.F32, B=4, Hq=8, Sq=1025, Skv=1025))[2] == capi.IMPL_MFMA              # 288
     assert _plan(_desc(dtype=capi.F32))[2] == capi.IMPL_SPLITKV_MFMA
     assert _plan(_desc(dtype=capi.F32, impl=capi.IMPL_MFMA))[2] == capi.IMPL_MFMA

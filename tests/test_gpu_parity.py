@@ -85,7 +85,7 @@ def test_buffer_round_trip(gpu):
     assert np.array_equal(dtypes.encode(t.to_f32(), capi.BF16).reshape(-1), raw)
 
 
-# ---- BASELINE configs 1 and 2 (f32) ------------------------------------------------
+# ---- the two f32 benchmark configurations ------------------------------------------------
 
 def test_config1_f32_single_head_noncausal(gpu):
     q, k, v = inputs(SEED0 + 0, 1, 1, 1, 128, 128, 64, 64, capi.F32)
