@@ -279,15 +279,17 @@ def decode_gqa_leg(steps, warmup, only_shape=None):
 
 def head_dims_leg(steps, warmup):
     """Head dimensions other than 64 and 128 (bf16): D = 96 runs zero-padded in the 128 instances of the prefill and split-KV
-    kernels, D = 256 in the prefill kernel for 256 and in the 256 instance of the split-KV kernel.  Prefill: useful FLOPs (4 D per visible
+    kernels, D = 256 in the prefill kernel for 256 and in the 256 instance of the split-KV kernel (decode, and a 256-row chunk of a
+    16384-token prompt: too few 128-row blocks for the prefill kernel, which does not split the keys).  Prefill: useful FLOPs (4 D per visible
     pair) against the bf16 matrix peak; decode: KV bytes read once against the HBM peak."""
     out = {}
     names = {capi.IMPL_SPLITKV_MFMA: "sdpa_decode_mfma_kernel", capi.IMPL_MFMA: "sdpa_prefill_mfma_kernel", capi.IMPL_GENERIC: "sdpa_generic_kernel"}
     for i, (name, B, Hq, Hkv, Sq, Skv, D, causal) in enumerate((("prefill_d96", 8, 16, 16, 2048, 2048, 96, True), ("prefill_d256", 4, 16, 16, 4096, 4096, 256, True),
+                                                                 ("chunk_d256", 1, 32, 8, 256, 16384, 256, True),
                                                                  ("decode_d96", 32, 32, 8, 1, 8192, 96, False), ("decode_d256", 32, 32, 8, 1, 8192, 256, False))):
         w = Workload("head_dims_" + name, SEED0 + 80 + i, B, Hq, Hkv, Sq, Skv, D, capi.BF16, causal)
         wall, ev_mean, ev_med, ev_min = w.time(max(steps, 50), warmup)
-        entry = {"workload": "bf16 %s B=%d Hq=%d Hkv=%d S_q=%d KV=%d D=%d" % ("causal prefill" if Sq > 1 else "decode", B, Hq, Hkv, Sq, Skv, D),
+        entry = {"workload": "bf16 %s B=%d Hq=%d Hkv=%d S_q=%d KV=%d D=%d" % ("decode" if Sq == 1 else "causal prefill" if Sq == Skv else "causal prefill chunk", B, Hq, Hkv, Sq, Skv, D),
                  "kernel": "sdpa_prefill_wide_kernel" if D > 128 and w.impl == capi.IMPL_MFMA else names.get(w.impl, str(w.impl)),
                  "num_splits": w.splits, "ms_per_step": wall, "parity_max_abs_err": w.parity(16)}
         if Sq > 1:
