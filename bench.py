@@ -5,7 +5,9 @@ One "step" is one launch of `incin_rocm_sdpa_fwd` over one batch of synthetic
 input already resident in HBM.  The headline workload is BASELINE config 3
 (bf16 causal prefill, B=8 H=16 S=4096 D=128); BASELINE config 4 (bf16 decode,
 B=32 H=32 KV=8192 D=128, split-KV + combine) is measured in the same run and
-reported under "decode".  Prints ONE JSON line.
+reported under "decode".  The last line of stdout is ONE compact JSON line (the headline, its roofline and CPU
+baseline, and the decode and ragged-prefill figures); every other leg is written in full to `bench_detail.json`
+beside this file and echoed to stderr.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
 
@@ -552,6 +554,63 @@ def f32_configs(steps, warmup, with_cpu, threads):
     return out
 
 
+def _round(x, sig=6):
+    """Floats to `sig` significant digits, recursively: the compact line carries figures, not 17-digit reprs."""
+    if isinstance(x, float):
+        return float("%.*g" % (sig, x))
+    if isinstance(x, dict):
+        return {k: _round(v, sig) for k, v in x.items()}
+    if isinstance(x, (list, tuple)):
+        return [_round(v, sig) for v in x]
+    return x
+
+
+def _pick(d, keys):
+    return {k: d[k] for k in keys if d is not None and k in d}
+
+
+_ROOFLINE_KEYS = ("bound", "achieved", "peak", "unit", "frac", "traffic", "kernel", "algorithmic_flops_per_launch",
+                  "algorithmic_bytes_per_launch", "launch_ms_mean", "launch_ms_median", "launch_ms_min")
+COMPACT_LIMIT = 4096
+
+
+def compact_line(result, detail_file="bench_detail.json"):
+    """The one line a harness parses: the headline (config 3) with its roofline and CPU baseline, config 4's decode and
+    config 5's ragged prefill in short form.  Everything else the run measured stays in `detail_file`."""
+    out = _pick(result, ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                         "vs_baseline", "dtype", "data", "config"))
+    if "roofline" in result:
+        out["roofline"] = _pick(result["roofline"], _ROOFLINE_KEYS)
+    if "cpu_baseline" in result:
+        out["cpu_baseline"] = _pick(result["cpu_baseline"], ("value", "unit", "cores", "kind", "sample"))
+    if "parity_max_abs_err" in result:
+        out["parity_max_abs_err"] = result["parity_max_abs_err"]
+    dec = result.get("decode")
+    if dec:
+        d = _pick(dec, ("workload", "value", "unit", "ms_per_step", "parity_max_abs_err"))
+        d["roofline"] = _pick(dec.get("roofline"), _ROOFLINE_KEYS)
+        if "cpu_baseline" in dec:
+            d["cpu_baseline"] = _pick(dec["cpu_baseline"], ("value", "unit", "cores", "kind", "sample"))
+        out["decode"] = d
+    pl = result.get("prefill_long")
+    if pl:
+        d = _pick(pl, ("value", "unit", "ms_per_step", "parity_max_abs_err"))
+        d["roofline"] = _pick(pl.get("roofline"), ("frac", "launch_ms_mean"))
+        out["prefill_long"] = d
+    bw = result.get("backward")
+    if bw:
+        out["backward"] = _pick(bw, ("value", "unit", "ms_per_step", "frac_of_bf16_mfma_peak"))
+    out["detail"] = detail_file
+    line = json.dumps(_round(out), separators=(",", ":"))
+    if len(line) >= COMPACT_LIMIT:      # never let free text push the line past what a tail-reading harness keeps
+        for obj in (out.get("cpu_baseline"), out.get("decode", {}).get("cpu_baseline")):
+            if obj and "sample" in obj:
+                obj["sample"] = obj["sample"][:160]
+        line = json.dumps(_round(out), separators=(",", ":"))
+    assert len(line) < COMPACT_LIMIT, "compact bench line is %d bytes" % len(line)
+    return line
+
+
 _T0 = time.perf_counter()
 
 
@@ -749,7 +808,16 @@ def main():
         result["backward_f32_c2"] = backward_leg(max(args.steps, 100), min(args.warmup, 5), capi.F32, 4, 8, 1024, 64, "BASELINE config 2's shape")
         result["backward_f32_large"] = backward_leg(max(5, min(args.steps, 10)), min(args.warmup, 3), capi.F32, what="BASELINE config 3's shape in f32")
 
-    print(json.dumps(result))
+    for detail in (os.path.join(ROOT, "bench_detail.json"), os.path.join(ROOT, "gpurun_out", "bench_detail.json")):
+        if not os.path.isdir(os.path.dirname(detail)):
+            continue
+        try:
+            with open(detail, "w") as f:
+                json.dump(result, f, indent=1)
+        except OSError as e:                 # a read-only tree must not cost the run its headline
+            print("bench.py: could not write %s: %s" % (detail, e), file=sys.stderr)
+    print(json.dumps(result), file=sys.stderr, flush=True)
+    print(compact_line(result), flush=True)
     return 0
 
 

@@ -87,7 +87,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     __shared__ int s_range[8];
     if (DENSE) {
         mrow = (const T*)p.mask + (int64_t)b * p.m_sb + (int64_t)hq * p.m_sh + (int64_t)min(my_i, Sq - 1) * p.m_si;
-        mflags = mask_flags_of(p, b, hq) + (int64_t)((q0 >> 5) + wave) * ((Skv + 31) >> 5);
+        // (a wavefront whose 32 rows lie past Sq computes nothing; its flag reads stay inside the array on the last row block)
+        mflags = mask_flags_of(p, b, hq) + (int64_t)min((q0 >> 5) + wave, ((Sq + 31) >> 5) - 1) * ((Skv + 31) >> 5);
         int lo = 0x7fffffff, hi = -1;
         for (int t = lane; t < n_act; t += 64)
             if (mflags[t] != 2) { lo = min(lo, t); hi = max(hi, t); }
@@ -221,6 +222,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 // beyond Skv are hidden by the limits below whatever is added to them)
                 vec4 m4 = {(T)0.0f, (T)0.0f, (T)0.0f, (T)0.0f};
                 if (j + 3 < Skv) m4 = *(const vec4*)(mrow + j);
+                else if (j < Skv) {      // the group that straddles the last key: its keys below Skv one by one
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) m4[e] = mrow[min(j + e, Skv - 1)];
+                }
 #pragma unroll
                 for (int e = 0; e < 4; ++e) sacc[4 * r4 + e] = __builtin_fmaf((float)m4[e], 1.4426950408889634f, sacc[4 * r4 + e]);
             }

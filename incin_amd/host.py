@@ -90,11 +90,12 @@ def mask_strides_for(mask_shape, B, Hq, Sq, Skv):
 
 
 def sdpa(q, k, v, dtype=capi.F32, scale=None, causal=False, kv_lens=None, mask=None,
-         num_splits=0, impl=capi.IMPL_AUTO, dev=0, return_info=False, q_lens=None, return_lse=False):
+         num_splits=0, impl=capi.IMPL_AUTO, dev=0, return_info=False, q_lens=None, return_lse=False, mask_row_pitch=None):
     """Run attention on the GPU for f32 numpy operands [B,Hq,Sq,D], [B,Hkv,Skv,D], [B,Hkv,Skv,Dv].
 
     Operands are rounded to `dtype` on upload; the result is returned as f32
-    holding the `dtype`-rounded output.
+    holding the `dtype`-rounded output.  `mask_row_pitch`: the mask's rows are stored that many elements apart
+    (a view of a wider buffer whose padding holds a large value no kernel may read as a key's).
     """
     q = np.asarray(q, dtype=np.float32)
     k = np.asarray(k, dtype=np.float32)
@@ -108,7 +109,14 @@ def sdpa(q, k, v, dtype=capi.F32, scale=None, causal=False, kv_lens=None, mask=N
     tm, ms = None, None
     if mask is not None:
         mask = np.asarray(mask, dtype=np.float32)
-        ms = mask_strides_for(mask.shape, B, Hq, Sq, k.shape[2])
+        if mask_row_pitch is not None:
+            padded = np.full(mask.shape[:-1] + (mask_row_pitch,), 1e4, np.float32)
+            padded[..., :mask.shape[-1]] = mask
+            ms = mask_strides_for(mask.shape[:-1] + (k.shape[2],), B, Hq, Sq, k.shape[2])
+            ms = [st // k.shape[2] * mask_row_pitch for st in ms[:3]] + [ms[3]]
+            mask = padded
+        else:
+            ms = mask_strides_for(mask.shape, B, Hq, Sq, k.shape[2])
         tm = capi.DeviceBuffer.from_numpy(dtypes.encode(mask, dtype), dev)
     tlse = capi.DeviceBuffer(B * Hq * Sq * 4, dev) if return_lse else None
     d = make_desc(tq, tk, tv, to, scale, causal, tl, tm, ms, num_splits, impl, q_lens=tql, lse=tlse)

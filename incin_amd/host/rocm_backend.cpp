@@ -193,17 +193,19 @@ Error RocmBackend::contiguous(const RocmStorage& s, RocmStorage* out)
 // last axes.  Axes the view only repeats (stride 0) are not expanded: they are copied at extent 1 and stay broadcast.
 static Error dense_last_axis(const RocmStorage& s, RocmStorage* out)
 {
+    // (the last axis is the one the copy is for: a view that repeats one element along it - broadcast_as of [.., S, 1] -
+    // is written out at its full extent)
+    const size_t last = s.shape.size() - 1;
     RocmStorage squeezed = s;
-    for (size_t a = 0; a < s.shape.size(); ++a)
+    for (size_t a = 0; a < last; ++a)
         if (s.strides[a] == 0) squeezed.shape[a] = std::min<int64_t>(s.shape[a], 1);
     RocmStorage dense;
     if (Error e = RocmBackend::contiguous(squeezed, &dense)) return e;
-    if (dense.buffer == s.buffer) {        // (already dense once the repeated axes are set aside: nothing to fix)
-        *out = s;
-        return ok();
-    }
-    for (size_t a = 0; a < s.shape.size(); ++a)
+    for (size_t a = 0; a < last; ++a)
         if (s.strides[a] == 0) { dense.shape[a] = s.shape[a]; dense.strides[a] = 0; }
+    if (dense.strides[last] != 1 && dense.shape[last] > 1)
+        return err(ErrorKind::UnsupportedBackendOperation, "scaled_dot_product_attention: could not make the last axis of " +
+                                                               shape_str(s.shape) + " dense on backend Rocm");
     dense.mask_tag.reset();
     *out = std::move(dense);
     return ok();

@@ -699,6 +699,37 @@ def test_head_dimensions_above_128_with_a_dense_mask(gpu, dtype, dims):
     check(got, oracle_full(q, k[:, :, :418], v[:, :, :418], G=2, mask=m[..., :418]), tol, "mask rows not 8-byte aligned: generic")
 
 
+@pytest.mark.parametrize("dtype", [capi.BF16, capi.F16], ids=lambda x: dtypes.NAMES[x])
+@pytest.mark.parametrize("skv", [417, 418, 419, 33], ids=lambda x: "skv%d" % x)
+def test_head_dimensions_above_128_key_bias_on_the_last_keys(gpu, dtype, skv):
+    """A key bias [1, 1, 1, Skv] (every stride but the key's is 0, so the prefill kernel for 256 takes it) with Skv not a
+    multiple of 4: the last Skv % 4 keys carry -inf and a large bias, which the kernel must add like any other key's."""
+    D = Dv = 256
+    B, Hq, Hkv, Sq = 2, 4, 2, 200
+    q, k, v = inputs(2700 + skv, B, Hq, Hkv, Sq, skv, D, Dv, dtype)
+    bias = (rng(8).standard_normal((1, 1, 1, skv)) * 0.5).astype(np.float32)
+    bias[..., skv - 1] = -np.inf
+    if skv % 4 >= 2:
+        bias[..., skv - 2] = 6.0
+    if skv % 4 == 3:
+        bias[..., skv - 3] = -np.inf
+    bias = dtypes.round_to(bias, dtype)
+    say("key bias on the last keys: %s Skv=%d" % (dtypes.NAMES[dtype], skv))
+    got, info = host.sdpa(q, k, v, dtype, mask=bias, return_info=True)
+    assert info["impl"] == capi.IMPL_MFMA
+    ref = oracle_full(q, k, v, G=2, mask=np.broadcast_to(bias, (1, 1, Sq, skv)))
+    check(got, ref, TOL[dtype], "key bias with values on the last %d keys, D=256" % (skv % 4))
+    # the same with the rows of a [B, 1, Sq, Skv] mask padded to a pitch of whole 8-byte groups
+    pitch = (skv + 3) // 4 * 4 + 4
+    mp = (rng(9).standard_normal((B, 1, Sq, skv)) * 0.5).astype(np.float32)
+    mp[..., skv - 1] = -np.inf
+    mp[0, 0, 5, skv - 1] = 3.0
+    mp = dtypes.round_to(mp, dtype)
+    got, info = host.sdpa(q, k, v, dtype, mask=mp, mask_row_pitch=pitch, return_info=True)
+    assert info["impl"] == capi.IMPL_MFMA
+    check(got, oracle_full(q, k, v, G=2, mask=mp), TOL[dtype], "mask rows at a padded pitch, D=256")
+
+
 def test_head_dimensions_outside_the_matrix_core_kernels(gpu):
     """Rows that are not whole 16-byte vectors stay on the generic kernel."""
     for dtype, D in ((capi.BF16, 20), (capi.F32, 6), (capi.BF16, 132), (capi.F32, 134)):

@@ -189,6 +189,29 @@ def test_operands_with_a_strided_last_axis(gpu, dtype):
     close(out.to_numpy(), O.sdpa(qt.transpose(0, 1, 3, 2), k_log, v_log, mask=m), TOL[dtype], "transposed q, k, v with a mask")
 
 
+@pytest.mark.parametrize("dtype", [RB.F32, RB.BF16])
+def test_operands_repeated_along_the_last_axis(gpu, dtype):
+    """q and v as broadcast_as([.., S, 1] -> [.., S, D]) views: the last axis has stride 0.  The reference takes any view
+    (cpu/storage.rs:308-325); here the view is written out at its full extent before the launch."""
+    say("host mirror: operands with a stride-0 last axis, dtype %s" % dtype)
+    B, H, Sq, Skv, D = 2, 3, 33, 50, 64
+    q1, v1 = rnd(70, (B, H, Sq, 1), dtype), rnd(71, (B, H, Skv, 1), dtype)
+    k = rnd(72, (B, H, Skv, D), dtype)
+    Q = RB.RocmStorage.from_numpy(q1, dtype).broadcast_as((B, H, Sq, D))
+    V = RB.RocmStorage.from_numpy(v1, dtype).broadcast_as((B, H, Skv, D))
+    K = RB.RocmStorage.from_numpy(k, dtype)
+    assert Q.strides[-1] == 0 and V.strides[-1] == 0
+    ref = O.sdpa(np.broadcast_to(q1, (B, H, Sq, D)), k, np.broadcast_to(v1, (B, H, Skv, D)))
+    out = RB.scaled_dot_product_attention(Q, K, V)
+    close(out.to_numpy(), ref, TOL[dtype], "q and v repeated along the last axis")
+    # also repeated over the heads (two stride-0 axes, one of them the last)
+    q2 = rnd(73, (B, 1, Sq, 1), dtype)
+    Q2 = RB.RocmStorage.from_numpy(q2, dtype).broadcast_as((B, H, Sq, D))
+    out = RB.scaled_dot_product_attention(Q2, K, V)
+    close(out.to_numpy(), O.sdpa(np.broadcast_to(q2, (B, H, Sq, D)), k, np.broadcast_to(v1, (B, H, Skv, D))), TOL[dtype],
+          "q repeated along heads and the last axis")
+
+
 def test_decode_step(gpu):
     # one query token per head against a long cache: the split-KV path behind the same call
     say("host mirror: decode step")
