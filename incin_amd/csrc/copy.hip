@@ -106,3 +106,80 @@ hipError_t launch_zero_rows(void* base, int elem, int B, int H, int S, int row_e
 }
 
 }  // namespace incin_rocm
+
+// ---- gradient of a broadcast: sums over the axes an operand was repeated along -------------------------------------
+// What the reference's tape does with the gradient of a broadcast operand (crates/incin-backends/src/cpu/tape.rs:
+// 243-265, `unbroadcast`, through `sum_dim_keepdim`, :283-317): the axes along which the operand had extent 1 are summed
+// away, one axis after the other from the left, each sum running over the axis in ascending order from 0.  One thread
+// per destination element keeps that order (a partial sum per reduced axis, folded into the next axis's when the axis
+// wraps), so the f32 result has the reference's rounding sequence; 16-bit storage is summed in f32 and rounded once
+// (the reference rounds after every addition).
+namespace incin_rocm {
+
+template <int DT> struct SumElem;
+template <> struct SumElem<0> { typedef float T; static __device__ float load(const T* p) { return *p; } static __device__ void store(T* p, float v) { *p = v; } };
+template <> struct SumElem<1> { typedef _Float16 T; static __device__ float load(const T* p) { return (float)*p; } static __device__ void store(T* p, float v) { *p = (T)v; } };
+template <> struct SumElem<2> { typedef __bf16 T; static __device__ float load(const T* p) { return (float)*p; } static __device__ void store(T* p, float v) { *p = (T)v; } };
+
+template <int DT>
+__global__ __launch_bounds__(256) void sum_to_shape_kernel(SumToShapeParams p, int64_t n_dst)
+{
+    typedef typename SumElem<DT>::T T;
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_dst) return;
+    // destination index -> source offset of its first term; the reduced axes, leftmost first
+    int64_t sstride[8], acc_s = 1;
+#pragma unroll
+    for (int a = 7; a >= 0; --a) { sstride[a] = acc_s; acc_s *= p.src_shape[a]; }
+    int64_t off = 0, rem = i;
+#pragma unroll
+    for (int a = 7; a >= 0; --a) {
+        const int64_t n = p.dst_shape[a];
+        off += (rem % n) * sstride[a];
+        rem /= n;
+    }
+    int64_t rext[8], rstr[8];
+    int nred = 0;
+#pragma unroll
+    for (int a = 0; a < 8; ++a)
+        if (p.dst_shape[a] != p.src_shape[a]) { rext[nred] = p.src_shape[a]; rstr[nred] = sstride[a]; ++nred; }
+    const T* src = (const T*)p.src;
+    if (nred == 0) { SumElem<DT>::store((T*)p.dst + i, SumElem<DT>::load(src + off)); return; }
+    float acc[8];
+    int64_t idx[8];
+    for (int l = 0; l < 8; ++l) { acc[l] = 0.0f; idx[l] = 0; }
+    for (;;) {
+        acc[0] += SumElem<DT>::load(src + off);
+        int l = 0;
+        bool done = false;
+        for (;;) {
+            off += rstr[l];
+            if (++idx[l] < rext[l]) break;
+            off -= rstr[l] * rext[l];
+            idx[l] = 0;
+            if (l + 1 == nred) { done = true; break; }
+            acc[l + 1] += acc[l];
+            acc[l] = 0.0f;
+            ++l;
+        }
+        if (done) break;
+    }
+    SumElem<DT>::store((T*)p.dst + i, acc[nred - 1]);
+}
+
+hipError_t launch_sum_to_shape(const SumToShapeParams& p, hipStream_t stream)
+{
+    int64_t n_dst = 1;
+    for (int a = 0; a < 8; ++a) n_dst *= p.dst_shape[a];
+    if (n_dst <= 0) return hipSuccess;
+    const int64_t blocks = (n_dst + 255) / 256;
+    if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+    switch (p.dtype) {
+        case 0: hipLaunchKernelGGL(sum_to_shape_kernel<0>, dim3((unsigned)blocks), dim3(256), 0, stream, p, n_dst); break;
+        case 1: hipLaunchKernelGGL(sum_to_shape_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, stream, p, n_dst); break;
+        default: hipLaunchKernelGGL(sum_to_shape_kernel<2>, dim3((unsigned)blocks), dim3(256), 0, stream, p, n_dst); break;
+    }
+    return hipGetLastError();
+}
+
+}  // namespace incin_rocm

@@ -522,6 +522,42 @@ int incin_rocm_copy_strided(int32_t dev, void* dst, const void* src, int32_t ran
     return 0;
 }
 
+int incin_rocm_sum_to_shape(int32_t dev, int32_t dtype, void* dst, const void* src, int32_t rank, const int64_t* src_shape,
+                            const int64_t* dst_shape, void* stream)
+{
+    if (rank < 0 || rank > 8) return fail(INCIN_ROCM_ESHAPE, "sum_to_shape: rank %d is outside 0..8", rank);
+    if (dtype != INCIN_ROCM_F32 && dtype != INCIN_ROCM_F16 && dtype != INCIN_ROCM_BF16)
+        return fail(INCIN_ROCM_EDTYPE, "sum_to_shape: unsupported dtype tag %d on backend Rocm (f32, f16, bf16 only)", dtype);
+    if (rank > 0 && (!src_shape || !dst_shape)) return fail(INCIN_ROCM_EINVAL, "sum_to_shape: null shape");
+    incin_rocm::SumToShapeParams p;
+    int64_t n_src = 1, n_dst = 1;
+    for (int a = 0; a < 8; ++a) { p.src_shape[a] = 1; p.dst_shape[a] = 1; }
+    for (int a = 0; a < rank; ++a) {
+        if (src_shape[a] < 0 || dst_shape[a] < 0) return fail(INCIN_ROCM_ESHAPE, "sum_to_shape: negative extent");
+        if (dst_shape[a] != src_shape[a] && dst_shape[a] != 1)
+            return fail(INCIN_ROCM_ESHAPE, "sum_to_shape: axis %d has extent %lld in the source and %lld in the target (the same, or 1)", a,
+                        (long long)src_shape[a], (long long)dst_shape[a]);
+        if (src_shape[a] > 0x7fffffffLL || (n_src *= src_shape[a]) > (1LL << 40)) return fail(INCIN_ROCM_ESHAPE, "sum_to_shape: source too large");
+        n_dst *= dst_shape[a];
+        p.src_shape[8 - rank + a] = src_shape[a];
+        p.dst_shape[8 - rank + a] = dst_shape[a];
+    }
+    if (n_dst == 0) return 0;
+    if (!dst) return fail(INCIN_ROCM_EINVAL, "sum_to_shape: null pointer");
+    if (int rc = use_device(dev)) return rc;
+    if (n_dst > 0x7fffffffLL) return fail(INCIN_ROCM_ESHAPE, "sum_to_shape: target too large");
+    if (n_src == 0) {       // an empty sum is 0 (the reference starts every sum from the default value)
+        HIP_TRY(incin_rocm::launch_zero_rows(dst, dtype == INCIN_ROCM_F32 ? 4 : 2, 1, 1, 1, (int)n_dst, 0, 0, 0, (hipStream_t)stream), "zero fill launch");
+        return 0;
+    }
+    if (!src) return fail(INCIN_ROCM_EINVAL, "sum_to_shape: null pointer");
+    p.src = (const char*)src;
+    p.dst = (char*)dst;
+    p.dtype = dtype;
+    HIP_TRY(incin_rocm::launch_sum_to_shape(p, (hipStream_t)stream), "sum_to_shape launch");
+    return 0;
+}
+
 int incin_rocm_sync(int32_t dev)
 {
     if (int rc = use_device(dev)) return rc;

@@ -211,6 +211,27 @@ static Error dense_last_axis(const RocmStorage& s, RocmStorage* out)
     return ok();
 }
 
+// The gradient of an operand that was broadcast to `g`'s shape, summed back to the operand's shape `target`
+// (right-aligned; cpu/tape.rs:243-265): leading axes the operand does not have and axes where it has extent 1 are summed
+// away.  `g` is dense.
+static Error sum_to_shape(const RocmStorage& g, const std::vector<int64_t>& target, RocmStorage* out)
+{
+    const int r = (int)g.shape.size(), pad = r - (int)target.size();
+    if (pad < 0 || r > 8) return err(ErrorKind::UnsupportedBackendOperation, "unbroadcast: rank above 8 on backend Rocm");
+    std::vector<int64_t> kept(r, 1);
+    for (int a = pad; a < r; ++a) {
+        if (target[a - pad] != g.shape[a] && target[a - pad] != 1)
+            return err(ErrorKind::ShapeMismatch, "unbroadcast: " + shape_str(g.shape) + " does not reduce to " + shape_str(target));
+        kept[a] = target[a - pad];
+    }
+    RocmStorage dst;
+    if (Error e = alloc_storage(target, g.dtype, g.device, &dst)) return e;
+    if (Error e = from_status(incin_rocm_sum_to_shape(g.device, (int32_t)g.dtype, dst.buffer->ptr(), g.data(), r, g.shape.data(), kept.data(), nullptr), g.device))
+        return e;
+    *out = std::move(dst);
+    return ok();
+}
+
 Error RocmBackend::transpose(const RocmStorage& s, int a, int b, RocmStorage* out)
 {
     const int r = (int)s.shape.size();
@@ -357,11 +378,73 @@ Error RocmBackend::attention_impl(const RocmStorage& q, const RocmStorage& k, co
         }
     }
 
-    // -- batch axes: broadcast(broadcast(q, k), v), NumPy rule (cpu/ops/matmul.rs:198-221) ------------------
+    // -- gradients of a view that repeats its storage along a batch axis (stride 0 at an extent above 1): to the reference
+    // such an operand has the view's shape and every repeated slice gets a gradient of its own (cpu/tape.rs:243-246: no
+    // sum where the shapes agree), so the view is written out and treated like any dense operand.
+    if (grads) {
+        auto repeats = [](const RocmStorage& x) {
+            for (size_t a = 0; a + 2 < x.shape.size(); ++a)
+                if (x.shape[a] > 1 && x.strides[a] == 0) return true;
+            return false;
+        };
+        if (repeats(q) || repeats(k) || repeats(v)) {
+            RocmStorage qd = q, kd = k, vd = v;
+            if (repeats(q)) if (Error e = contiguous(q, &qd)) return e;
+            if (repeats(k)) if (Error e = contiguous(k, &kd)) return e;
+            if (repeats(v)) if (Error e = contiguous(v, &vd)) return e;
+            return attention_impl(qd, kd, vd, mask, scale, facts, grad_out, out, grads);
+        }
+    }
+
+    // -- a mask that adds query rows: scores [.., 1, Skv] + mask [.., R, Skv] is [.., R, Skv] in the reference (its add
+    // broadcasts both ways, cpu/ops/shape_ops.rs:1262-1266 with cpu/stride.rs:86-106): q's one row is repeated R times
+    // (a stride-0 view, written out so that every kernel sees rows of its own), and a gradient sums the rows back.
+    if (mask && mask->shape.size() >= 2 && Sq == 1) {
+        const int64_t mrows = mask->shape[mask->shape.size() - 2];
+        if (mrows > 1) {
+            std::vector<int64_t> dims = q.shape;
+            dims[qr - 2] = mrows;
+            RocmStorage qv, qd;
+            if (Error e = broadcast_as(q, dims, &qv)) return e;
+            if (Error e = contiguous(qv, &qd)) return e;
+            if (!grads) return attention_impl(qd, k, v, mask, scale, facts, grad_out, out, grads);
+            AttentionGrads g2;
+            if (Error e = attention_impl(qd, k, v, mask, scale, facts, grad_out, out, &g2)) return e;
+            if (Error e = sum_to_shape(g2.dq, q.shape, &grads->dq)) return e;
+            grads->dk = std::move(g2.dk);
+            grads->dv = std::move(g2.dv);
+            return ok();
+        }
+    }
+
+    // -- batch axes: broadcast(broadcast(broadcast(q, k), mask), v), NumPy rule (cpu/ops/matmul.rs:198-221 for the two
+    // products, cpu/stride.rs:86-106 for the mask's add, which may add leading axes or widen axes of extent 1) ------------
     const std::vector<int64_t> qb(q.shape.begin(), q.shape.end() - 2), kb(k.shape.begin(), k.shape.end() - 2),
         vb(v.shape.begin(), v.shape.end() - 2);
     std::vector<int64_t> bshape, tmp;
     if (Error e = broadcast_shape(qb, kb, &tmp)) return e;
+    std::vector<int64_t> mshape, mstr;
+    if (mask) {
+        mshape = mask->shape;
+        mstr = mask->strides;
+        while ((int)mshape.size() < 2) {
+            mshape.insert(mshape.begin(), 1);
+            mstr.insert(mstr.begin(), 0);
+        }
+        const int64_t mr = mshape[mshape.size() - 2], mc = mshape[mshape.size() - 1];
+        std::vector<int64_t> full = tmp;
+        full.push_back(Sq);
+        full.push_back(Skv);
+        // (a mask with more keys than k has would widen the scores past v's rows: the second product refuses that)
+        if ((mr != 1 && mr != Sq) || (mc != 1 && mc != Skv))
+            return err(ErrorKind::ShapeMismatch, std::string(OP) + ": mask " + shape_str(mask->shape) +
+                                                     " does not broadcast to the scores " + shape_str(full));
+        std::vector<int64_t> tmp2;
+        if (broadcast_shape(tmp, std::vector<int64_t>(mshape.begin(), mshape.end() - 2), &tmp2))
+            return err(ErrorKind::ShapeMismatch, std::string(OP) + ": mask " + shape_str(mask->shape) +
+                                                     " does not broadcast to the scores " + shape_str(full));
+        tmp = tmp2;
+    }
     if (Error e = broadcast_shape(tmp, vb, &bshape)) return e;
     const int nb = (int)bshape.size();
     std::vector<int64_t> qs, ks, vs, ms;
@@ -369,15 +452,10 @@ Error RocmBackend::attention_impl(const RocmStorage& q, const RocmStorage& k, co
     broadcast_strides(kb, std::vector<int64_t>(k.strides.begin(), k.strides.end() - 2), bshape, &ks);
     broadcast_strides(vb, std::vector<int64_t>(v.strides.begin(), v.strides.end() - 2), bshape, &vs);
 
-    // -- mask: None | tagged | dense additive, broadcast against [..b, Sq, Skv] without enlarging it ------------
+    // -- mask: None | tagged | dense additive, seen through the broadcast to [..b, Sq, Skv] ---------------------------
     int64_t m_si = 0, m_sj = 0;
     bool dense_mask = false;
     if (mask) {
-        std::vector<int64_t> mshape = mask->shape, mstr = mask->strides;
-        while ((int)mshape.size() < 2) {
-            mshape.insert(mshape.begin(), 1);
-            mstr.insert(mstr.begin(), 0);
-        }
         std::vector<int64_t> full = bshape;
         full.push_back(Sq);
         full.push_back(Skv);
@@ -401,22 +479,19 @@ Error RocmBackend::attention_impl(const RocmStorage& q, const RocmStorage& k, co
     if (Error e = alloc_storage(oshape, q.dtype, q.device, &o)) return e;
     const std::vector<int64_t> os(o.strides.begin(), o.strides.end() - 2);
 
-    // -- gradients: fresh contiguous storages of the operands' own shapes -------------------------------------------------
-    RocmStorage gq, gk, gv;
+    // -- gradients: dense storages over the batch axes the launches run over; an operand repeated along a batch axis gets its
+    // gradient summed over that axis afterwards (cpu/tape.rs:243-265) - except keys and values shared by a group of query
+    // heads, which the kernels sum themselves (the group axis is found below: the storages are laid out after it) -----------
+    RocmStorage gq, gk, gv, grad_dense;
     std::vector<int64_t> gqs, gks, gvs;
     if (grads) {
         if (!grad_out || grad_out->device != q.device) return err(ErrorKind::DeviceMismatch, std::string(OP) + " backward: the upstream gradient lives on another device");
         if (grad_out->dtype != q.dtype) return err(ErrorKind::DTypeStorageMismatch, std::string(OP) + " backward: the upstream gradient has another dtype");
         if (grad_out->shape != oshape)
             return err(ErrorKind::ShapeMismatch, std::string(OP) + " backward: upstream gradient " + shape_str(grad_out->shape) + ", output " + shape_str(oshape));
-        if (!grad_out->is_contiguous())
-            return err(ErrorKind::UnsupportedBackendOperation, std::string(OP) + " backward: the upstream gradient must be contiguous on backend Rocm");
-        if (Error e = alloc_storage(q.shape, q.dtype, q.device, &gq)) return e;
-        if (Error e = alloc_storage(k.shape, k.dtype, k.device, &gk)) return e;
-        if (Error e = alloc_storage(v.shape, v.dtype, v.device, &gv)) return e;
-        broadcast_strides(qb, std::vector<int64_t>(gq.strides.begin(), gq.strides.end() - 2), bshape, &gqs);
-        broadcast_strides(kb, std::vector<int64_t>(gk.strides.begin(), gk.strides.end() - 2), bshape, &gks);
-        broadcast_strides(vb, std::vector<int64_t>(gv.strides.begin(), gv.strides.end() - 2), bshape, &gvs);
+        // the kernels read the upstream gradient with the output's strides: any other view is gathered first
+        if (Error e = contiguous(*grad_out, &grad_dense)) return e;
+        grad_out = &grad_dense;
     }
 
     // -- collapse the batch axes into (outer..., B, Hkv, G) ----------------------------------------------------
@@ -431,16 +506,32 @@ Error RocmBackend::attention_impl(const RocmStorage& q, const RocmStorage& k, co
     if (next >= 0 && !(g_ax >= 0 && next == 0)) h_ax = next--;
     if (next >= 0) b_ax = next--;
     const int n_outer = next + 1;
+    bool sum_q = false, sum_k = false, sum_v = false;      // a gradient storage is wider than its operand
     if (grads) {
-        // A gradient of a broadcast operand is a sum over the broadcast axis (cpu/tape.rs:247-280).  The kernels sum over the
-        // group axis of grouped queries; any other broadcast would need sums across launches, which nothing here does.
-        for (int a = 0; a < nb; ++a) {
-            if (bshape[a] <= 1) continue;
-            if (qs[a] == 0 || ((ks[a] == 0 || vs[a] == 0) && a != g_ax))
-                return err(ErrorKind::UnsupportedBackendOperation,
-                           std::string(OP) + " backward: operands broadcast along batch axis " + std::to_string(a) +
-                               " (only keys and values shared by a group of query heads are summed) on backend Rocm");
-        }
+        // shape of an operand's gradient as the launches write it: the batch shape, with extent 1 kept only on the group axis
+        // of k and v
+        auto launch_shape = [&](const RocmStorage& x, bool kv, bool* wider) {
+            std::vector<int64_t> dims(bshape);
+            const int pad = nb - ((int)x.shape.size() - 2);
+            for (int a = 0; a < nb; ++a) {
+                const int64_t own = a >= pad ? x.shape[a - pad] : 1;
+                if (kv && a == g_ax) dims[a] = 1;
+                else if (own != bshape[a]) *wider = true;
+            }
+            dims.push_back(x.shape[x.shape.size() - 2]);
+            dims.push_back(x.shape[x.shape.size() - 1]);
+            return dims;
+        };
+        const std::vector<int64_t> gq_dims = launch_shape(q, false, &sum_q), gk_dims = launch_shape(k, true, &sum_k),
+                                   gv_dims = launch_shape(v, true, &sum_v);
+        if (nb + 2 > 8 && (sum_q || sum_k || sum_v))
+            return err(ErrorKind::UnsupportedBackendOperation, std::string(OP) + " backward: summing the gradient of a broadcast operand needs rank <= 8 on backend Rocm");
+        if (Error e = alloc_storage(gq_dims, q.dtype, q.device, &gq)) return e;
+        if (Error e = alloc_storage(gk_dims, k.dtype, k.device, &gk)) return e;
+        if (Error e = alloc_storage(gv_dims, v.dtype, v.device, &gv)) return e;
+        broadcast_strides(std::vector<int64_t>(gq_dims.begin(), gq_dims.end() - 2), std::vector<int64_t>(gq.strides.begin(), gq.strides.end() - 2), bshape, &gqs);
+        broadcast_strides(std::vector<int64_t>(gk_dims.begin(), gk_dims.end() - 2), std::vector<int64_t>(gk.strides.begin(), gk.strides.end() - 2), bshape, &gks);
+        broadcast_strides(std::vector<int64_t>(gv_dims.begin(), gv_dims.end() - 2), std::vector<int64_t>(gv.strides.begin(), gv.strides.end() - 2), bshape, &gvs);
     }
     int64_t G = g_ax >= 0 ? bshape[g_ax] : 1;
     int64_t Hkv = h_ax >= 0 ? bshape[h_ax] : 1;
@@ -592,9 +683,17 @@ Error RocmBackend::attention_impl(const RocmStorage& q, const RocmStorage& k, co
         if (Error e = from_status(incin_rocm_sync(q.device), q.device)) return e;
     *out = std::move(o);
     if (grads) {
-        grads->dq = std::move(gq);
-        grads->dk = std::move(gk);
-        grads->dv = std::move(gv);
+        // (a gradient storage of the operand's own extents only needs the operand's rank back)
+        auto finish = [&](RocmStorage& g, const RocmStorage& x, bool wider, RocmStorage* dst) -> Error {
+            if (wider) return sum_to_shape(g, x.shape, dst);
+            g.shape = x.shape;
+            g.strides = contiguous_strides(x.shape);
+            *dst = std::move(g);
+            return ok();
+        };
+        if (Error e = finish(gq, q, sum_q, &grads->dq)) return e;
+        if (Error e = finish(gk, k, sum_k, &grads->dk)) return e;
+        if (Error e = finish(gv, v, sum_v, &grads->dv)) return e;
     }
     return ok();
 }

@@ -118,8 +118,10 @@ struct RocmBackend {
     // Gradients of the operator for an upstream gradient of the output's shape: the forward is run once more keeping its
     // row normalisers, then one backward call per forward launch.  The reference gets these by walking its tape of the
     // composed ops (cpu/tape.rs:149-176); like there, the mask is a constant.  dq, dk, dv are fresh contiguous storages of
-    // the operands' shapes.  Keys and values shared by a group of query heads get the sum over the group; operands
-    // broadcast along any other batch axis, a non-contiguous upstream gradient and q_lens are UnsupportedBackendOperation.
+    // the operands' shapes.  Keys and values shared by a group of query heads get the sum over the group from the kernels;
+    // an operand broadcast along any other batch axis (or a query row repeated under a mask of several rows) gets its
+    // gradient at the launches' shape first and the sum over the repetitions after (cpu/tape.rs:243-265); the upstream
+    // gradient may be any view.  q_lens together with gradients is UnsupportedBackendOperation.
     struct AttentionGrads {
         RocmStorage dq, dk, dv;
     };

@@ -165,10 +165,10 @@ const std::vector<CapabilityRule>& rocm_capabilities()
         {OperationKind::Reshape, ROCM_DTYPES, {LayoutClass::Contiguous}, 0, MAX_RANK, false, PRECISE, ImplementationKind::Native},
         {OperationKind::Reshape, ROCM_DTYPES, {LayoutClass::Strided, LayoutClass::RowWise}, 0, MAX_RANK, false, PRECISE,
          ImplementationKind::Composed},
-        // scaled_dot_product_attention and its gradients (RocmBackend::attention_backward).  What a query cannot say and
-        // the operator still refuses: gradients for operands repeated along a batch axis other than the group axis of
-        // grouped queries, a non-contiguous upstream gradient, query lengths under training, and a mask whose broadcast
-        // would enlarge the score shape.
+        // scaled_dot_product_attention and its gradients (RocmBackend::attention_backward): operands repeated along batch
+        // axes get the sum of their repetitions' gradients, a mask may widen the scores, the upstream gradient may be any
+        // view.  Outside what a query can say, the operator refuses head dimensions above 256 and gradients together with
+        // query lengths (a descriptor field the reference's operator does not have).
         {OperationKind::Attention, ROCM_DTYPES, ROW_VIEWS, 2, MAX_RANK, true, PRECISE, ImplementationKind::Native},
         // operands whose last axis is strided (a transposed view): gathered into dense temporaries, then the same kernels
         {OperationKind::Attention, ROCM_DTYPES, {LayoutClass::Strided}, 2, MAX_RANK, true, PRECISE, ImplementationKind::Composed},

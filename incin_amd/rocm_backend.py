@@ -154,6 +154,14 @@ class RocmStorage:
         lib().incin_host_strides(self._h, d)
         return tuple(d[i] for i in range(n))
 
+    def is_contiguous(self):
+        acc = 1
+        for n, st in zip(reversed(self.shape), reversed(self.strides)):
+            if n != 1 and st != acc:
+                return False
+            acc *= n
+        return True
+
     @property
     def dtype(self):
         t = C.c_int32()

@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define INCIN_ROCM_ABI_VERSION 8
+#define INCIN_ROCM_ABI_VERSION 9
 
 /* ---- status codes (mapped to incin_core::Error variants by the Rust side;
  *      crates/incin-core/src/err.rs:109-223) --------------------------------- */
@@ -106,6 +106,13 @@ int incin_rocm_memcpy_d2d(int32_t dev, void* dst, const void* src, size_t bytes)
  * (a transposed view). */
 int incin_rocm_copy_strided(int32_t dev, void* dst, const void* src, int32_t rank, const int64_t* shape, const int64_t* strides,
                             int32_t elem_bytes, void* stream);
+/* Gradient of a broadcast operand: `src` (dense, `src_shape`) summed down to `dst` (dense, `dst_shape`), where
+ * dst_shape[a] is src_shape[a] or 1 - the axes with 1 are summed away.  Replaces `unbroadcast`
+ * (crates/incin-backends/src/cpu/tape.rs:243-265; `sum_dim_keepdim` :283-317): axis after axis from the left, each in
+ * ascending order, f32 partial sums (16-bit storage is rounded once at the end).  rank <= 8; a caller with fewer leading
+ * axes in the target pads its shape with 1s.  dtype: INCIN_ROCM_F32 / F16 / BF16.  Enqueued on `stream`. */
+int incin_rocm_sum_to_shape(int32_t dev, int32_t dtype, void* dst, const void* src, int32_t rank, const int64_t* src_shape,
+                            const int64_t* dst_shape, void* stream);
 int incin_rocm_sync(int32_t dev);      /* waits for the device's default stream and any stream created here */
 
 /* ---- streams and events -------------------------------------------------------

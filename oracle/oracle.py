@@ -122,6 +122,11 @@ def _prepare(q, k, v, mask, scale, causal, kv_lens, host_has_fma):
         while len(mshape) < 2:
             mshape.insert(0, 1)
         mask = mask.reshape(mshape)
+        if Sq == 1 and mshape[-2] > 1:
+            # the reference's add broadcasts both ways (shape_ops.rs:1262-1266, cpu/stride.rs:86-106): scores [.., 1, Skv]
+            # plus a mask of R rows are R rows of scores, each from q's one row - a stride-0 view of q says the same
+            Sq = mshape[-2]
+            q = np.broadcast_to(q, q.shape[:-2] + (Sq, D))
         if broadcast_shape(mshape[-2:], [Sq, Skv]) != [Sq, Skv]:
             raise ValueError("mask must broadcast to [..., Sq, Skv]")
         b = broadcast_shape(b, mshape[:-2])

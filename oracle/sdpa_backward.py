@@ -74,10 +74,13 @@ def sdpa_backward(q, k, v, grad_out, mask=None, scale=None, causal=False, kv_len
         mask = extra if mask is None else np.asarray(mask, np.float64) + extra
     out, p, s = sdpa_forward_f64(q, k, v, mask, scale)
     dv = np.matmul(np.swapaxes(p, -1, -2), go)                     # attn^T @ grad_out
-    dp = np.matmul(go, np.swapaxes(v, -1, -2))                     # grad_out @ v^T
+    dp = _unbroadcast(np.matmul(go, np.swapaxes(v, -1, -2)), p.shape)      # grad_out @ v^T, back to attn's shape
     dls = dp * p
     dx = dls - p * dls.sum(-1, keepdims=True)
-    dscores = dx * s
+    # the mask's add may have widened the scores (more batch axes, or rows where q has one): its gradient rule sums
+    # those back to the shape of q k^T before the scale and the first product's rules apply (cpu/tape.rs:243-265)
+    scores_shape = tuple(np.broadcast_shapes(q.shape[:-2], k.shape[:-2])) + (Sq, Skv)
+    dscores = _unbroadcast(dx, scores_shape) * s
     dq = np.matmul(dscores, k)
     dk = np.matmul(np.swapaxes(dscores, -1, -2), q)
     return _unbroadcast(dq, q.shape), _unbroadcast(dk, k.shape), _unbroadcast(dv, v.shape)

@@ -84,18 +84,28 @@ def test_attention_rule_boundary_cases_execute(gpu, dtype, level, layout, rank):
 
 @pytest.mark.parametrize("dtype", RULES["attention"].dtypes)
 @pytest.mark.parametrize("level, layout", ATTENTION_CELLS)
-@pytest.mark.parametrize("rank", [RULES["attention"].min_rank, RULES["attention"].max_rank])
-def test_attention_rule_boundary_cases_train(gpu, dtype, level, layout, rank):
+@pytest.mark.parametrize("rank", [RULES["attention"].min_rank, 3, RULES["attention"].max_rank])
+@pytest.mark.parametrize("shared", [False, True], ids=["own_batch", "broadcast_batch"])
+def test_attention_rule_boundary_cases_train(gpu, dtype, level, layout, rank, shared):
     """The same cells with `training` set: the rule says yes, so the gradients come out and match the backward oracle
-    (1e-5 of the largest gradient magnitude for f32, 2e-2 for the 16-bit types)."""
+    (1e-5 of the largest gradient magnitude for f32, 2e-2 for the 16-bit types).  `broadcast_batch`: k and v have extent 1
+    on a batch axis where q has more, and (from rank 5 on) q has extent 1 on another - operands the reference's matmul
+    broadcasts, whose gradients are sums over the repetitions (cpu/tape.rs:243-265)."""
     from oracle import sdpa_backward as BW
     assert RULES["attention"].training
     case = RC.CapabilityQuery("attention", dtype, layout, rank, training=True)
     assert RC.support("rocm", case).level == level
     qs, ks, vs = shapes_of_rank(rank)
+    if shared:
+        if rank == 2:
+            pytest.skip("rank 2 has no batch axis to share")
+        wide = [a for a in range(rank - 2) if qs[a] > 1]
+        ks = vs = tuple(1 if a == wide[0] else n for a, n in enumerate(ks))
+        if len(wide) > 1:
+            qs = tuple(1 if a == wide[-1] else n for a, n in enumerate(qs))
     say("capability cell %s: q%s k%s" % (case, qs, ks))
     q, k, v = rnd(1, qs, dtype), rnd(2, ks, dtype), rnd(3, vs, dtype)
-    go = rnd(6, qs[:-1] + (vs[-1],), dtype)
+    go = rnd(6, np.broadcast_shapes(qs[:-2], ks[:-2]) + (qs[-2], vs[-1]), dtype)
     out, dq, dk, dv = RB.attention_backward(operand(q, dtype, layout), operand(k, dtype, layout), operand(v, dtype, layout),
                                             RB.RocmStorage.from_numpy(go, CODE[dtype]))
     tol = 1e-5 if dtype == "f32" else 2e-2

@@ -309,13 +309,105 @@ def test_gradients_through_the_host_mirror(gpu, case):
         close(out.to_numpy(), ref, TOL[dtype], "forward beside the gradients")
 
 
-def test_gradients_refused_for_broadcast_operands(gpu):
-    q, k, v = rnd(51, (2, 3, 4, 8), RB.F32), rnd(52, (1, 3, 5, 8), RB.F32), rnd(53, (1, 3, 5, 8), RB.F32)
-    go = rnd(54, (2, 3, 4, 8), RB.F32)
+@pytest.mark.parametrize("dtype", [RB.F32, RB.BF16])
+@pytest.mark.parametrize("case", [
+    ((3, 5, 16), (3, 7, 16), (3, 7, 8), (2, 1, 5, 7)),              # the mask adds a leading axis
+    ((2, 3, 1, 16), (2, 3, 7, 16), (2, 3, 7, 16), (4, 7)),          # one query row, four mask rows
+    ((1, 3, 5, 16), (1, 3, 7, 16), (1, 3, 7, 16), (4, 1, 1, 7)),    # an axis of extent 1 widened by the mask
+    ((1, 16), (7, 16), (7, 8), (3, 2, 5, 7)),                       # rank-2 operands under a rank-4 mask
+    ((2, 2, 4, 9, 64), (2, 2, 1, 11, 64), (2, 2, 1, 11, 64), (3, 1, 1, 1, 9, 11)),      # grouped queries under a mask with one more axis
+], ids=["leading_axis", "rows", "widened_axis", "rank2", "gqa_leading_axis"])
+def test_masks_that_widen_the_scores(gpu, dtype, case):
+    """The reference adds the mask with a two-way broadcast (cpu/ops/shape_ops.rs:1262-1266, cpu/stride.rs:86-106): a mask
+    with more leading axes, or more rows than q has, widens the scores and the output with them."""
+    qs, ks, vs, msh = case
+    say("host mirror: mask %s widens the scores of q %s, dtype %s" % (msh, qs, dtype))
+    q, k, v = rnd(80, qs, dtype), rnd(81, ks, dtype), rnd(82, vs, dtype)
+    mask = rnd(83, msh, dtype)
+    mask[..., 2] = -np.inf
+    S = lambda a: RB.RocmStorage.from_numpy(a, dtype)
+    out = RB.scaled_dot_product_attention(S(q), S(k), S(v), mask=S(mask))
+    ref = O.sdpa(q, k, v, mask=mask)
+    assert out.shape == ref.shape
+    close(out.to_numpy(), ref, TOL[dtype], "widening mask")
+    # and its gradients: the widened axes are summed back (cpu/tape.rs:243-265)
+    from oracle import sdpa_backward as BW
+    go = rnd(84, ref.shape, dtype)
+    out2, dq, dk, dv = RB.attention_backward(S(q), S(k), S(v), S(go), S(mask))
+    assert dq.shape == qs and dk.shape == ks and dv.shape == vs
+    rq, rk, rv = BW.sdpa_backward(q, k, v, go, mask=mask)
+    tol = 1e-5 if dtype == RB.F32 else 2e-2
+    grad_close("dq", dq.to_numpy(), rq, tol)
+    grad_close("dk", dk.to_numpy(), rk, tol)
+    grad_close("dv", dv.to_numpy(), rv, tol)
+    close(out2.to_numpy(), ref, TOL[dtype], "forward beside the gradients")
+    # a mask with more keys than k has would widen the scores past v's rows
+    with pytest.raises(RB.BackendError) as e:
+        RB.scaled_dot_product_attention(S(q), S(k[..., :1, :]), S(v[..., :1, :]), mask=S(mask))
+    assert e.value.kind == "ShapeMismatch"
+
+
+@pytest.mark.parametrize("case", [
+    # q shape, k shape, v shape, dtype, causal tag
+    ((2, 3, 4, 8), (1, 3, 5, 8), (1, 3, 5, 8), RB.F32, False),          # k, v shared by the batch entries
+    ((2, 1, 6, 16), (2, 3, 5, 16), (2, 3, 5, 16), RB.F32, False),       # q shared by the heads
+    ((2, 3, 4, 8), (5, 8), (5, 8), RB.F32, False),                      # k, v of lower rank
+    ((2, 3, 4, 8), (2, 1, 5, 8), (2, 3, 5, 8), RB.F32, False),          # k shared by the heads, v not: no group axis
+    ((3, 1, 2, 4, 20, 64), (1, 2, 2, 1, 20, 64), (1, 2, 2, 1, 20, 64), RB.BF16, True),      # grouped queries + two more broadcast axes
+    ((2, 4, 40, 128), (1, 1, 40, 128), (1, 1, 40, 128), RB.BF16, True),  # one kv head for all batch entries (matrix-core kernels)
+    ((4, 2, 33, 64), (1, 2, 47, 64), (4, 1, 47, 64), RB.F16, False),
+], ids=["kv_shared_by_batch", "q_shared_by_heads", "kv_lower_rank", "k_only", "gqa_plus_outer", "one_kv_head_bf16", "mixed_f16"])
+def test_gradients_of_broadcast_operands(gpu, case):
+    """An operand repeated along a batch axis gets the sum of the gradients of its repetitions (cpu/tape.rs:243-265)."""
+    from oracle import sdpa_backward as BW
+    qs, ks, vs, dtype, causal = case
+    say("host mirror backward with broadcast operands: %s" % (case,))
+    q, k, v = rnd(51, qs, dtype), rnd(52, ks, dtype), rnd(53, vs, dtype)
+    oshape = np.broadcast_shapes(qs[:-2], ks[:-2], vs[:-2]) + (qs[-2], vs[-1])
+    go = rnd(54, oshape, dtype)
+    Sq, Skv = qs[-2], ks[-2]
+    S = lambda a: RB.RocmStorage.from_numpy(a, dtype)
+    mask_np, mask = None, None
+    if causal:
+        mask_np = np.triu(np.full((Sq, Skv), -np.inf, np.float32), 1 + Skv - Sq)
+        mask = S(mask_np).tag_causal()
+    out, dq, dk, dv = RB.attention_backward(S(q), S(k), S(v), S(go), mask)
+    assert out.shape == oshape and dq.shape == qs and dk.shape == ks and dv.shape == vs
+    rq, rk, rv = BW.sdpa_backward(q, k, v, go, mask=mask_np)
+    tol = 1e-5 if dtype == RB.F32 else 2e-2
+    grad_close("dq", dq.to_numpy(), rq, tol)
+    grad_close("dk", dk.to_numpy(), rk, tol)
+    grad_close("dv", dv.to_numpy(), rv, tol)
+    close(out.to_numpy(), O.sdpa(q, k, v, mask=mask_np), TOL[dtype], "forward beside the gradients")
+
+
+@pytest.mark.parametrize("dtype", [RB.F32, RB.BF16])
+def test_gradients_of_views(gpu, dtype):
+    """Operands that are views: k repeated over the heads by broadcast_as (to the reference an operand of the view's
+    shape: every repetition gets a gradient of its own), q transposed, and an upstream gradient that is a transposed view."""
+    from oracle import sdpa_backward as BW
+    B, H, Sq, Skv, D = 2, 3, 12, 17, 64
+    q_t = rnd(90, (B, H, D, Sq), dtype)                   # q stored transposed
+    k1, v = rnd(91, (B, 1, Skv, D), dtype), rnd(92, (B, H, Skv, D), dtype)
+    go_t = rnd(93, (B, H, D, Sq), dtype)                  # the upstream gradient too
+    S = lambda a: RB.RocmStorage.from_numpy(a, dtype)
+    Q = S(q_t).transpose(2, 3)
+    K = S(k1).broadcast_as((B, H, Skv, D))
+    GO = S(go_t).transpose(2, 3)
+    assert K.strides[1] == 0 and not GO.is_contiguous()
+    out, dq, dk, dv = RB.attention_backward(Q, K, S(v), GO)
+    q_log, k_log, go_log = q_t.transpose(0, 1, 3, 2), np.broadcast_to(k1, (B, H, Skv, D)), go_t.transpose(0, 1, 3, 2)
+    rq, rk, rv = BW.sdpa_backward(q_log, np.ascontiguousarray(k_log), v, go_log)
+    assert dq.shape == q_log.shape and dk.shape == (B, H, Skv, D) and dv.shape == v.shape
+    tol = 1e-5 if dtype == RB.F32 else 2e-2
+    grad_close("dq", dq.to_numpy(), rq, tol)
+    grad_close("dk (one per repetition)", dk.to_numpy(), rk, tol)
+    grad_close("dv", dv.to_numpy(), rv, tol)
+
+
+def test_gradient_shape_errors(gpu):
+    q, go = rnd(51, (2, 3, 4, 8), RB.F32), rnd(54, (2, 3, 4, 8), RB.F32)
     S = RB.RocmStorage.from_numpy
-    with pytest.raises(RB.BackendError) as e:       # k, v shared by the batch entries: their gradient is a sum over launches
-        RB.attention_backward(S(q), S(k), S(v), S(go))
-    assert e.value.kind == "UnsupportedBackendOperation" and "broadcast" in e.value.message
     with pytest.raises(RB.BackendError) as e:
         RB.attention_backward(S(q), S(rnd(55, (2, 3, 5, 8), RB.F32)), S(rnd(56, (2, 3, 5, 8), RB.F32)), S(go[:, :, :3]))
     assert e.value.kind == "ShapeMismatch"

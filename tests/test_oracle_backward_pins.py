@@ -110,3 +110,31 @@ def test_forward_of_the_backward_oracle_is_the_forward_oracle():
     x = np.einsum("bhid,bhjd->bhij", q.astype(np.float64), k.astype(np.float64)) * float(np.float32(0.25))
     x = x + BW.additive_mask(17, 23, (2, 3), True)
     assert np.allclose(lse, np.log(np.exp(x).sum(-1)), atol=1e-12)
+
+
+def test_gradients_under_a_mask_that_widens_the_scores_match_central_differences():
+    """q with one row under a mask of four rows and an extra leading axis: the gradient of the scores is summed back to the
+    shape of q k^T before the first product's rules apply (cpu/tape.rs:243-265).  Checked by central differences."""
+    r = np.random.Generator(np.random.PCG64(77))
+    q, k, v = r.standard_normal((2, 3, 1, 8)), r.standard_normal((2, 1, 7, 8)), r.standard_normal((3, 7, 5))
+    mask = r.standard_normal((5, 1, 1, 4, 7))
+    g = r.standard_normal((5, 2, 3, 4, 5))
+    dq, dk, dv = BW.sdpa_backward(q, k, v, g, mask=mask)
+    assert dq.shape == q.shape and dk.shape == k.shape and dv.shape == v.shape
+
+    def f(q_, k_, v_):
+        return float((BW.sdpa_forward_f64(q_, k_, v_, mask)[0] * g).sum())
+
+    eps = 1e-6
+    for which, x, d in ((0, q, dq), (1, k, dk), (2, v, dv)):
+        for _ in range(6):
+            idx = tuple(int(r.integers(0, n)) for n in x.shape)
+            xp, xm = x.copy(), x.copy()
+            xp[idx] += eps
+            xm[idx] -= eps
+            args_p = [q, k, v]
+            args_m = [q, k, v]
+            args_p[which], args_m[which] = xp, xm
+            num = (f(*args_p) - f(*args_m)) / (2 * eps)
+            assert abs(num - d[idx]) < 1e-6 * max(1.0, abs(num)), (which, idx, num, d[idx])
+

@@ -102,6 +102,34 @@ def test_reference_batch_broadcast_shapes():
         O.broadcast_shape([2, 3], [4, 3])
 
 
+# ---- a mask whose broadcast widens the scores (cpu/ops/shape_ops.rs:1262-1266, cpu/stride.rs:86-106) ----------------
+
+@pytest.mark.parametrize("case", [
+    ((3, 5, 8), (3, 7, 8), (3, 7, 6), (2, 1, 5, 7)),          # leading mask axis: the output gains it
+    ((2, 3, 1, 8), (2, 3, 7, 8), (2, 3, 7, 8), (4, 7)),      # one query row, four mask rows: four output rows
+    ((1, 3, 5, 8), (1, 3, 7, 8), (1, 3, 7, 8), (4, 1, 1, 7)),  # an axis of extent 1 widened by the mask
+    ((1, 8), (7, 8), (7, 4), (3, 2, 5, 7)),                  # rank-2 operands under a rank-4 mask
+], ids=["leading_axis", "rows", "widened_axis", "rank2"])
+def test_mask_that_widens_the_scores(case):
+    """The oracle against an independent float64 numpy evaluation, where numpy's own broadcasting does the widening, and
+    against the same call with the operands widened by hand (which takes the ordinary path)."""
+    from oracle import sdpa_backward as BW
+    qs, ks, vs, msh = case
+    r = rng(sum(qs) + sum(msh))
+    q, k, v = (r.standard_normal(sh, dtype=np.float32) for sh in (qs, ks, vs))
+    mask = r.standard_normal(msh, dtype=np.float32)
+    mask[..., 2] = -np.inf
+    got = O.sdpa(q, k, v, mask=mask)
+    ref = BW.sdpa_forward_f64(q, k, v, mask)[0]
+    assert got.shape == ref.shape
+    assert np.abs(got - ref).max() < 1e-6
+    rows = max(qs[-2], msh[-2] if len(msh) >= 2 else 1)
+    bshape = np.broadcast_shapes(qs[:-2], ks[:-2], vs[:-2], msh[:-2])
+    wide = O.sdpa(np.ascontiguousarray(np.broadcast_to(q, bshape + (rows, qs[-1]))), k, v, mask=mask)
+    assert np.array_equal(got, wide)
+    assert np.array_equal(got, O.sdpa_materialised(q, k, v, mask=mask))
+
+
 # ---- independent float64 evaluation ---------------------------------------------------
 
 @pytest.mark.parametrize("shape", [(1, 1, 8, 4), (2, 4, 64, 32), (1, 3, 17, 5), (2, 2, 33, 16)])
