@@ -210,7 +210,15 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         // kernel (measured, bf16 causal, D = 256: 8 heads x 128 x 8192 0.305 -> 0.039 ms; 32 x 256 x 16384 0.60 -> 0.26;
         // 8 x 1024 x 32768 1.18 -> 0.56; 16 x 1024 x 4096 - 128 workgroups - 0.158 -> 0.121; at 256 workgroups
         // (2 x 32 x 512 x 512) the prefill kernel is ahead, 0.031 against 0.057).
-        const bool wide_underfilled = d->B * d->Hq * ((d->Sq + 127) / 128) * 2 <= compute_units_of(d->device);
+        // Swept over 4 - 32 heads x 128 - 2048 rows x 1024 - 16384 keys (causal, one sequence): the split-KV kernel is ahead
+        // (to 0.06 of the prefill kernel's time) up to a quarter of the compute units' worth of 128-row workgroups, and up to
+        // half where its 32-row chunks come in whole rounds of the compute units (its workgroups then finish together);
+        // with a ragged last round (192, 288, 384 chunks) it is 1.1 - 1.5 times behind from 48 - 72 workgroups on, and over
+        // fewer than 2048 keys a ragged round is all there is.
+        const int64_t cus_w = compute_units_of(d->device);
+        const int64_t wgs_w = d->B * d->Hq * ((d->Sq + 127) / 128), chunks_w = d->B * d->Hkv * ((R + 31) / 32);
+        const bool wide_underfilled = (wgs_w * 4 <= cus_w && (d->Skv >= 2048 || chunks_w * 2 <= cus_w || chunks_w % cus_w == 0)) ||
+                                      (wgs_w * 2 <= cus_w && chunks_w % cus_w == 0);
         if (wide && mfma_ok && d->Sq > 64 && !(split_mfma_ok && wide_underfilled)) impl = INCIN_ROCM_IMPL_MFMA;
         else if (wide && split_mfma_ok) impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
         // f32 (sdpa_decode_f32.hip): from two rows per KV head on, whatever the count - the f32 prefill kernel would spend a
@@ -219,7 +227,11 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         // against 0.28 ms on 8 x 8 heads x 8192 keys); the vector-ALU kernel is level at 2 rows and behind from 4 on
         // (4 rows, 268 MB of cache: 5.6 against 4.8 TB/s; 8 rows: 6.6 against 3.4).  More than 32 rows over fewer than 512
         // keys stay with the prefill kernel (64 positions x 16 heads x 64 sequences of 256 keys: 0.14 against 0.17 ms).
-        else if (d->dtype == INCIN_ROCM_F32 && split_mfma_ok && d->Sq <= 64 && len128 >= 256 && R >= 2 && (R <= 32 || d->Skv >= 512))
+        // One row per KV head (swept over 1 - 32 sequences x 8 - 32 heads x 512 - 16384 keys): the matrix-core kernel is level
+        // from 500 MB of cache on and up to 2.8 times ahead below (its splits fill the device where the vector-ALU kernel's
+        // do not), except over the shortest caches at D = 64 (512 keys: 1.1 - 1.4 times behind).
+        else if (d->dtype == INCIN_ROCM_F32 && split_mfma_ok && d->Sq <= 64 && len128 >= 256 &&
+                 (R >= 2 ? (R <= 32 || d->Skv >= 512) : d->Skv >= (d_pad == 64 ? 1024 : 512)))
             impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
         // f32 prefill launches that give the prefill kernel at most one 128-row workgroup per compute unit: the split-KV kernel
         // takes them 32 rows per workgroup with the keys dealt to its four wavefronts - four times the workgroups, a quarter

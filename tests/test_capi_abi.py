@@ -80,6 +80,10 @@ def test_dispatch_choices():
     assert _plan(_desc(D=160, Dv=160))[2] == capi.IMPL_SPLITKV_MFMA
     assert _plan(_desc(D=256, Dv=256, B=1, Hq=16, Hkv=16, Sq=1024, Skv=4096, causal=1))[2] == capi.IMPL_SPLITKV_MFMA
     assert _plan(_desc(D=256, Dv=256, B=1, Hq=17, Hkv=17, Sq=1024, Skv=4096, causal=1))[2] == capi.IMPL_MFMA
+    # (72 workgroups, 288 chunks of 32 rows: a ragged second round for the split-KV kernel, measured 1.25 times behind)
+    assert _plan(_desc(D=256, Dv=256, B=1, Hq=12, Hkv=12, Sq=768, Skv=3000, causal=1))[2] == capi.IMPL_MFMA
+    assert _plan(_desc(D=256, Dv=256, B=1, Hq=8, Hkv=8, Sq=768, Skv=3000, causal=1))[2] == capi.IMPL_SPLITKV_MFMA      # 48 workgroups
+    assert _plan(_desc(D=256, Dv=256, B=1, Hq=8, Hkv=8, Sq=768, Skv=1024, causal=1))[2] == capi.IMPL_MFMA              # over 1024 keys: 192 chunks, one ragged round
     assert _plan(_desc(D=256, Dv=256, Sq=4096, Skv=4096, causal=1))[2] == capi.IMPL_MFMA
     assert _plan(_desc(D=256, Dv=256, Sq=4096, Skv=4096, causal=1, impl=capi.IMPL_SPLITKV_MFMA))[2] == capi.IMPL_SPLITKV_MFMA
     assert _plan(_desc(D=256, Dv=256, Sq=64, Skv=4096, causal=1))[2] == capi.IMPL_SPLITKV_MFMA
@@ -117,7 +121,9 @@ def test_dispatch_choices():
     assert impl == capi.IMPL_SPLITKV_MFMA and splits == 1                     # 256 groups: one round, nothing to combine
     # f32: its own matrix-core split-KV kernel (chunks of 16 or 32 rows) from two rows per KV head on, any number of rows
     assert _plan(_desc(Sq=1, Skv=8192, B=2, Hq=8, Hkv=2, dtype=capi.F32))[2] == capi.IMPL_SPLITKV_MFMA
-    assert _plan(_desc(Sq=1, Skv=8192, B=2, Hq=8, Hkv=8, dtype=capi.F32))[2] == capi.IMPL_SPLITKV             # one row: vector ALU
+    assert _plan(_desc(Sq=1, Skv=8192, B=2, Hq=8, Hkv=8, dtype=capi.F32))[2] == capi.IMPL_SPLITKV_MFMA        # one row too, from 512 keys on
+    assert _plan(_desc(Sq=1, Skv=400, B=2, Hq=8, Hkv=8, dtype=capi.F32))[2] == capi.IMPL_SPLITKV              # shortest caches: vector ALU
+    assert _plan(_desc(Sq=1, Skv=600, B=2, Hq=8, Hkv=8, D=64, Dv=64, dtype=capi.F32))[2] == capi.IMPL_SPLITKV  # (at D = 64 up to 1024 keys)
     assert _plan(_desc(Sq=64, Skv=8192, B=2, Hq=32, Hkv=2, dtype=capi.F32))[2] == capi.IMPL_SPLITKV_MFMA      # 1024 rows per KV head
     assert _plan(_desc(Sq=65, Skv=8192, B=8, Hq=64, Hkv=2, dtype=capi.F32))[2] == capi.IMPL_MFMA              # more positions, 512 row blocks: prefill
     assert _plan(_desc(Sq=1, Skv=100, B=2, Hq=8, Hkv=2, dtype=capi.F32))[2] == capi.IMPL_MFMA                 # shortest caches: one workgroup per head

@@ -570,8 +570,12 @@ def test_decode_splitkv_matrix_cores_f32_scale_lse_auto(gpu):
     got, info = host.sdpa(q, k, v, dt, return_info=True)
     assert info["impl"] == capi.IMPL_SPLITKV_MFMA           # 4 rows per KV head over 1100 keys, f32: AUTO's choice
     check(got, oracle_full(q, k, v, G=4), TOL[dt], "AUTO f32 grouped-query decode")
-    _, info = host.sdpa(q[:, :4], k, v, dt, return_info=True)
-    assert info["impl"] == capi.IMPL_SPLITKV                # one row per KV head stays on the vector-ALU kernel
+    got, info = host.sdpa(q[:, :4], k, v, dt, return_info=True)
+    assert info["impl"] == capi.IMPL_SPLITKV_MFMA           # one row per KV head too (from 512 keys on)
+    check(got, oracle_full(q[:, :4], k, v, G=1), TOL[dt], "AUTO f32 decode, one row per KV head")
+    got, info = host.sdpa(q[:, :4], k[:, :, :300], v[:, :, :300], dt, return_info=True)
+    assert info["impl"] == capi.IMPL_SPLITKV                # the shortest caches stay on the vector-ALU kernel
+    check(got, oracle_full(q[:, :4], k[:, :, :300], v[:, :, :300], G=1), TOL[dt], "AUTO f32 decode over a short cache")
 
 
 HEAD_DIMS_16 = [(96, 96), (80, 80), (40, 40), (8, 8), (112, 72), (128, 64), (64, 128), (32, 16), (120, 128)]
@@ -648,7 +652,9 @@ def test_head_dimensions_above_128(gpu, dtype, dims):
             check(got, ref, tol, "D=%d Dv=%d Sq=%d splits=%d->%d" % (D, Dv, Sq, splits, info["splits"]))
         got, lse, info = host.sdpa(q, k, v, dtype, causal=True, kv_lens=lens, return_info=True, return_lse=True)
         # (16-bit: the prefill kernel for 256 once its 128-row workgroups cover more than half the compute units)
-        prefill_256 = Sq > 64 and dtype != capi.F32 and B * Hq * ((Sq + 127) // 128) * 2 > capi.device_info(0).compute_units
+        cus, wgs, chunks = capi.device_info(0).compute_units, B * Hq * ((Sq + 127) // 128), B * Hkv * ((Hq // Hkv * Sq + 31) // 32)
+        split_ahead = (wgs * 4 <= cus and (Skv >= 2048 or chunks * 2 <= cus or chunks % cus == 0)) or (wgs * 2 <= cus and chunks % cus == 0)
+        prefill_256 = Sq > 64 and dtype != capi.F32 and not split_ahead
         assert info["impl"] == (capi.IMPL_MFMA if prefill_256 else capi.IMPL_SPLITKV_MFMA)
         check(got, ref, tol, "AUTO, D=%d Dv=%d Sq=%d" % (D, Dv, Sq))
         if Sq > 64 and dtype != capi.F32:

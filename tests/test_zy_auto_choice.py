@@ -1,0 +1,105 @@
+"""AUTO's choice of kernel against every kernel that accepts the same launch, timed on the device.
+
+The planner's thresholds were measured on a handful of shapes; this holds them to account on shapes between and beside
+those: for each, the launch is timed through AUTO and through every pinned kernel that takes it (HIP events around a run
+of launches, best of three runs), and AUTO may be at most 10 % slower than the fastest of them (15 % on launches under
+20 microseconds, where one launch's jitter is that large).  Collected late on purpose: a timing assertion should not
+hide the parity tests behind it in a run that stops at the first failure."""
+import sys
+
+import numpy as np
+import pytest
+
+from incin_amd import capi, dtypes, host
+
+pytestmark = pytest.mark.gpu
+BF, F32 = capi.BF16, capi.F32
+NAMES = {capi.IMPL_AUTO: "auto", capi.IMPL_GENERIC: "generic", capi.IMPL_MFMA: "prefill", capi.IMPL_SPLITKV: "split-kv (vector ALU)",
+         capi.IMPL_SPLITKV_MFMA: "split-kv (matrix cores)"}
+
+# (name, dtype, B, Hq, Hkv, Sq, Skv, D, causal)
+SHAPES = [
+    ("decode_mha_short", BF, 8, 32, 32, 1, 1536, 128, False),            # one row per KV head, 100 MB of cache
+    ("decode_mha_mid", BF, 16, 32, 32, 1, 3072, 128, False),             # 800 MB
+    ("decode_gqa2", BF, 8, 16, 8, 1, 3000, 128, False),                  # two rows per KV head
+    ("decode_gqa4_short", BF, 4, 32, 8, 1, 700, 128, False),
+    ("decode_gqa8_long", BF, 2, 64, 8, 1, 20000, 128, False),
+    ("decode_sq3", BF, 4, 8, 8, 3, 5000, 128, True),                     # three positions, causal among themselves
+    ("decode_gqa4_d64", BF, 8, 32, 8, 1, 6000, 64, False),
+    ("decode_sq16_gqa4", BF, 2, 32, 8, 16, 6000, 128, True),             # 64 rows per KV head
+    ("chunk_sq96", BF, 1, 16, 4, 96, 12000, 128, True),                  # more than 64 positions: prefill, keys split
+    ("prefill_small", BF, 2, 8, 8, 640, 640, 128, True),
+    ("prefill_mid", BF, 4, 16, 16, 1536, 1536, 128, True),
+    ("prefill_d64", BF, 4, 16, 16, 1024, 1024, 64, True),
+    ("prefill_d256_few_heads", BF, 1, 12, 12, 768, 3000, 256, True),
+    ("prefill_d256", BF, 2, 24, 24, 1024, 1024, 256, True),
+    ("decode_d256", BF, 8, 16, 4, 1, 5000, 256, False),
+    ("f32_decode_gqa2", F32, 4, 16, 8, 1, 5000, 128, False),
+    ("f32_decode_mha", F32, 8, 16, 16, 1, 3000, 128, False),
+    ("f32_decode_sq8", F32, 2, 32, 8, 8, 3000, 64, True),
+    ("f32_prefill_small", F32, 2, 8, 8, 768, 768, 64, True),
+    ("f32_prefill_mid", F32, 4, 16, 16, 1280, 1280, 64, True),
+    ("f32_prefill_d128", F32, 2, 16, 16, 2048, 2048, 128, True),
+    ("f32_short_cache", F32, 16, 16, 16, 48, 300, 64, True),
+]
+
+
+def say(msg):
+    print(msg, file=sys.stderr, flush=True)
+
+
+def time_launches(desc, n):
+    for _ in range(3):
+        capi.sdpa_fwd(desc)
+    capi.sync()
+    best = None
+    for _ in range(3):
+        e0, e1 = capi.Event(), capi.Event()
+        e0.record()
+        for _ in range(n):
+            capi.sdpa_fwd(desc)
+        e1.record()
+        capi.sync()
+        ms = e0.elapsed_ms(e1) / n
+        best = ms if best is None else min(best, ms)
+        e0.destroy()
+        e1.destroy()
+    return best
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=[s[0] for s in SHAPES])
+def test_auto_is_not_slower_than_a_pinned_kernel(gpu, shape):
+    name, dt, B, Hq, Hkv, Sq, Skv, D, causal = shape
+    r = np.random.Generator(np.random.PCG64(4242))
+    tq = host.DeviceTensor.from_f32(r.standard_normal((B, Hq, Sq, D), dtype=np.float32), dt)
+    tk = host.DeviceTensor.from_f32(r.standard_normal((B, Hkv, Skv, D), dtype=np.float32), dt)
+    tv = host.DeviceTensor.from_f32(r.standard_normal((B, Hkv, Skv, D), dtype=np.float32), dt)
+    to = host.DeviceTensor((B, Hq, Sq, D), dt)
+    times, chosen = {}, None
+    for impl in (capi.IMPL_AUTO, capi.IMPL_MFMA, capi.IMPL_SPLITKV, capi.IMPL_SPLITKV_MFMA):
+        d = host.make_desc(tq, tk, tv, to, causal=causal, impl=impl)
+        try:
+            nbytes, splits, got = capi.sdpa_workspace(d)
+        except capi.RocmError as e:
+            assert e.code == capi.EUNSUPPORTED, e
+            continue
+        if impl == capi.IMPL_AUTO:
+            chosen = got
+        ws = capi.DeviceBuffer(nbytes) if nbytes else None
+        if ws is not None:
+            d.workspace, d.workspace_bytes = ws.ptr, ws.nbytes
+        capi.sdpa_fwd(d)
+        capi.sync()
+        once = time_launches(d, 3)
+        times[impl] = time_launches(d, max(5, min(200, int(3.0 / max(once, 1e-3)))))
+        if ws is not None:
+            ws.free()
+    for t in (tq, tk, tv, to):
+        t.buf.free()
+    say("%s: AUTO -> %s; " % (name, NAMES[chosen]) + ", ".join("%s %.4f ms" % (NAMES[i], t) for i, t in times.items()))
+    pinned = {i: t for i, t in times.items() if i != capi.IMPL_AUTO}
+    assert chosen in pinned, "AUTO chose a kernel that refuses the launch when pinned"
+    best_impl = min(pinned, key=pinned.get)
+    slack = 1.15 if pinned[best_impl] < 0.02 else 1.10
+    assert times[capi.IMPL_AUTO] <= slack * pinned[best_impl], \
+        "%s: AUTO (%s) %.4f ms, %s %.4f ms" % (name, NAMES[chosen], times[capi.IMPL_AUTO], NAMES[best_impl], pinned[best_impl])
