@@ -256,7 +256,9 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
 #elif defined(PF_ABL_Q0)
                 qraw[h][ps] = *(const uint4v*)((const T*)p.q + (int64_t)(wave * 32 + rr) * p.q_ss + col);
 #else
-                qraw[h][ps] = col < p.D ? *(const uint4v*)(qp + (int64_t)min(row0 + rr, Sq - 1) * p.q_ss + col) : zero;      // (beyond the head dimension: zeros, like K's)
+                // (non-temporal, like the stores of O below: rows that are read or written once must not push the K / V tiles, which
+                // every workgroup of a head reads, out of the XCD's L2 - 3.7 % on 8 x 16 heads x 4096 x 4096 causal)
+                qraw[h][ps] = col < p.D ? __builtin_nontemporal_load((const uint4v*)(qp + (int64_t)min(row0 + rr, Sq - 1) * p.q_ss + col)) : zero;      // (beyond the head dimension: zeros, like K's)
 #endif
             }
     }
@@ -845,7 +847,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
                 const int rr = ps * 8 + (lane >> 3), c = lane & 7;
                 const uint4v val = *(const uint4v*)(stage + rr * 128 + ((c ^ (rr & 7)) << 4));
                 const int col = h * 64 + c * 8;
-                if (row0 + rr < rows_b && col < p.Dv) *(uint4v*)(op + (int64_t)(row0 + rr) * p.o_ss + col) = val;
+                if (row0 + rr < rows_b && col < p.Dv) __builtin_nontemporal_store(val, (uint4v*)(op + (int64_t)(row0 + rr) * p.o_ss + col));
             }
         }
     }
@@ -863,6 +865,9 @@ static hipError_t launch_prefill_nw(const SdpaParams& p0, hipStream_t stream)
     // 256 registers per lane: eight wavefronts per compute unit, i.e. two workgroups of four or one of eight; an eighth
     // of the compute units per XCD
     p.interleave = work_interleave(p.causal != 0, (8 / NW) * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
+#ifdef PF_FORCE_F
+    p.interleave = PF_FORCE_F;
+#endif
     p.deal_groups = (total & 7) == 0 ? work_deal(p.interleave, p.G, nqb, total >> 3) : 0;
     if constexpr (!DENSE && NW == 4) {
         if (p.num_splits > 1) {          // split launch: partial results, then the split-KV kernels' combine pass
