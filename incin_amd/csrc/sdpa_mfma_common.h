@@ -192,6 +192,94 @@ inline int work_interleave(bool causal, int slots, int G, int nqb, long long ran
     return f;
 }
 
+// ---- Q rows in, O rows out: 16 bytes per lane, eight lanes to a 128-byte run of a row -------------------------------
+// The prefill kernels keep a query per lane: lane (ql, g) of a wavefront holds, of row ql, the 16-byte chunks
+// 2 s + g of Q (one per k-step s; f32: per group of four k-steps) and of O the four columns db * 32 + r4 * 8 + g * 4 ..
+// per (db, r4).  Read and written
+// that way, every memory instruction touches 32 rows with 16 or 32 bytes each, and the compute unit's path to memory takes
+// such partial cache lines one at a time (512 of them per wavefront for 64 lines of data).  So both go through a
+// wavefront-private 4 KiB of LDS, 128 bytes per row (64 columns, 32 in f32) per pass: chunk c of row r at chunk c ^ (r % 8).  Both are
+// non-temporal: rows that are used once must not push the K / V tiles, which every workgroup of a head reads, out of L2.
+// No barrier is involved: the area belongs to one wavefront; the caller says which LDS nobody else touches meanwhile.
+template <typename T, int NQH>
+__device__ __forceinline__ void fetch_q_rows(uint4v (&qraw)[NQH][4], const T* qhead, int row0, int Sq, int64_t q_ss, int Dq, int lane)
+{
+#pragma unroll
+    for (int h = 0; h < NQH; ++h)
+#pragma unroll
+        for (int ps = 0; ps < 4; ++ps) {
+            const int rr = ps * 8 + (lane >> 3), col = h * (int)(128 / sizeof(T)) + (lane & 7) * (int)(16 / sizeof(T));
+            const uint4v zero = {0u, 0u, 0u, 0u};
+            // (rows past the last one repeat it: their results are never stored; beyond the head dimension: zeros, like K's)
+            qraw[h][ps] = col < Dq ? __builtin_nontemporal_load((const uint4v*)(qhead + (int64_t)min(row0 + rr, Sq - 1) * q_ss + col)) : zero;
+        }
+}
+template <typename V8, int NQH>
+__device__ __forceinline__ void stage_q_rows(V8 (&qreg)[4 * NQH], const uint4v (&qraw)[NQH][4], char* stage, int lane)
+{
+    const int ql = lane & 31, g = lane >> 5;
+#pragma unroll
+    for (int h = 0; h < NQH; ++h) {
+#pragma unroll
+        for (int ps = 0; ps < 4; ++ps) {
+            const int rr = ps * 8 + (lane >> 3), c = lane & 7;
+            *(uint4v*)(stage + rr * 128 + ((c ^ (rr & 7)) << 4)) = qraw[h][ps];
+        }
+#pragma unroll
+        for (int sl = 0; sl < 4; ++sl) qreg[h * 4 + sl] = *(const V8*)(stage + ql * 128 + (((2 * sl + g) ^ (ql & 7)) << 4));
+    }
+}
+template <typename T, int NDB>
+__device__ __forceinline__ void store_o_rows(const floatx16 (&o_acc)[NDB], float inv, char* stage, T* ohead, int row0, int rows_b, int64_t o_ss, int Dv, int lane)
+{
+    typedef T vec4 __attribute__((ext_vector_type(4)));
+    const int ql = lane & 31, g = lane >> 5;
+#pragma unroll
+    for (int h = 0; h < NDB / 2; ++h) {
+#pragma unroll
+        for (int dbl = 0; dbl < 2; ++dbl)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                vec4 w;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) w[e] = (T)(o_acc[2 * h + dbl][r4 * 4 + e] * inv);
+                *(vec4*)(stage + ql * 128 + (((dbl * 4 + r4) ^ (ql & 7)) << 4) + g * 8) = w;
+            }
+#pragma unroll
+        for (int ps = 0; ps < 4; ++ps) {
+            const int rr = ps * 8 + (lane >> 3), c = lane & 7;
+            const uint4v val = *(const uint4v*)(stage + rr * 128 + ((c ^ (rr & 7)) << 4));
+            const int col = h * 64 + c * 8;
+            if (row0 + rr < rows_b && col < Dv) __builtin_nontemporal_store(val, (uint4v*)(ohead + (int64_t)(row0 + rr) * o_ss + col));
+        }
+    }
+}
+
+// (f32: a pass is one 32-column block; the lane's four floats of (db, r4) are chunk 2 r4 + g of it)
+template <int NDB>
+__device__ __forceinline__ void store_o_rows_f32(const floatx16 (&o_acc)[NDB], float inv, char* stage, float* ohead, int row0, int rows_b, int64_t o_ss, int Dv, int lane)
+{
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    const int ql = lane & 31, g = lane >> 5;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) {
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+            f4 w;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[e] = o_acc[db][r4 * 4 + e] * inv;
+            *(f4*)(stage + ql * 128 + (((2 * r4 + g) ^ (ql & 7)) << 4)) = w;
+        }
+#pragma unroll
+        for (int ps = 0; ps < 4; ++ps) {
+            const int rr = ps * 8 + (lane >> 3), c = lane & 7;
+            const uint4v val = *(const uint4v*)(stage + rr * 128 + ((c ^ (rr & 7)) << 4));
+            const int col = db * 32 + c * 4;
+            if (row0 + rr < rows_b && col < Dv) __builtin_nontemporal_store(val, (uint4v*)(ohead + (int64_t)(row0 + rr) * o_ss + col));
+        }
+    }
+}
+
 __device__ __forceinline__ float xor32_max(float x)
 {
     // lanes l and l^32 exchange; both end with the maximum

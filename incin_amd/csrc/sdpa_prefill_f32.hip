@@ -137,18 +137,18 @@ void sdpa_prefill_f32_kernel(SdpaParams p)
     for (int db = 0; db < NDB; ++db) v_high[db] = (db ^ g) << 7;
 
     // ---- Q'^T operand, resident in registers ----------------------------------------------------------------------
+    // (fetched 16 bytes per lane, eight lanes to a 128-byte run of a row, and brought into the operand layout through this
+    // wavefront's 4 KiB of the K buffer the first copies do not fill: nothing is copied there before the loop's first barrier)
     float4v qreg[NJ];
     {
-        const int qi = min(my_i, Sq - 1);
-        const float* qrow = qp + (int64_t)qi * p.q_ss + g * 4;
+        uint4v qraw[NJ / 4][4];
+        fetch_q_rows(qraw, qp, q0 + wave * 32, Sq, p.q_ss, p.D, lane);
+        stage_q_rows(qreg, qraw, smem + ((t_first + 1) & 1) * L::TILE_BYTES + wave * 4096, lane);
         const float c2 = p.scale * 1.4426950408889634f;      // scores in log2 units
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-            const bool in = j * 8 + g * 4 < p.D;      // (beyond the head dimension: zeros, like K's)
-            if (in) qreg[j] = *(const float4v*)(qrow + j * 8);
+        for (int j = 0; j < NJ; ++j)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) qreg[j][e] = in ? qreg[j][e] * c2 : 0.0f;
-        }
+            for (int e = 0; e < 4; ++e) qreg[j][e] *= c2;
     }
     const float* mrow = nullptr;          // this lane's row of the dense mask
     const uint8_t* mflags = nullptr;      // block flags of this wavefront's 32 rows: 0 mixed, 1 all zero, 2 all -inf
@@ -280,18 +280,9 @@ void sdpa_prefill_f32_kernel(SdpaParams p)
     const float inv = (l_tot == 0.0f) ? __builtin_nanf("") : 1.0f / l_tot;   // no visible key: NaN, as the reference
     if (p.lse && g == 0 && my_i < rows_b)
         p.lse[((int64_t)b * p.Hq + hq) * Sq + my_i] = l_tot == 0.0f ? -INFINITY : (m_run + __builtin_log2f(l_tot)) * 0.6931471805599453f;
-    if (my_i < rows_b) {
-        float* orow = op + (int64_t)my_i * p.o_ss;
-#pragma unroll
-        for (int db = 0; db < NDB; ++db)
-#pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-                float4v w;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) w[e] = o_acc[db][r4 * 4 + e] * inv;
-                if (db * 32 + r4 * 8 + g * 4 < p.Dv) *(float4v*)(orow + db * 32 + r4 * 8 + g * 4) = w;
-            }
-    }
+    // through this wavefront's 4 KiB of the K buffer the last tile did not use (every wavefront is past the barrier of that
+    // tile, i.e. done with the tile before it, and nothing has been copied since)
+    store_o_rows_f32(o_acc, inv, smem + (n_tiles & 1) * L::TILE_BYTES + wave * 4096, op, q0 + wave * 32, rows_b, p.o_ss, p.Dv, lane);
 #endif
 }
 

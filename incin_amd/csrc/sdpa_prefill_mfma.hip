@@ -238,30 +238,11 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
         v_rem -= v_tile_bytes;
     };
 
-    // The Q rows are asked for first, 16 bytes per lane and eight lanes to a 128-byte run of a row (in the operand layout a
-    // lane would fetch 16 bytes of each of 32 different rows per instruction, and the compute unit's path to memory takes
-    // partial cache lines one at a time); they reach the operand layout through LDS below.
+    // The Q rows are asked for first (fetch_q_rows: 16 bytes per lane, eight lanes to a run of a row); they reach the operand
+    // layout through LDS below.
     constexpr int NQH = D / 64;      // passes of 64 columns
     uint4v qraw[NQH][4];
-    {
-        const int row0 = q0 + wave * 32;
-#pragma unroll
-        for (int h = 0; h < NQH; ++h)
-#pragma unroll
-            for (int ps = 0; ps < 4; ++ps) {
-                const int rr = ps * 8 + (lane >> 3), col = h * 64 + (lane & 7) * 8;
-                const uint4v zero = {0u, 0u, 0u, 0u};
-#ifdef PF_ABL_NOQ
-                qraw[h][ps] = zero;
-#elif defined(PF_ABL_Q0)
-                qraw[h][ps] = *(const uint4v*)((const T*)p.q + (int64_t)(wave * 32 + rr) * p.q_ss + col);
-#else
-                // (non-temporal, like the stores of O below: rows that are read or written once must not push the K / V tiles, which
-                // every workgroup of a head reads, out of the XCD's L2 - 3.7 % on 8 x 16 heads x 4096 x 4096 causal)
-                qraw[h][ps] = col < p.D ? __builtin_nontemporal_load((const uint4v*)(qp + (int64_t)min(row0 + rr, Sq - 1) * p.q_ss + col)) : zero;      // (beyond the head dimension: zeros, like K's)
-#endif
-            }
-    }
+    fetch_q_rows(qraw, qp, q0 + wave * 32, Sq, p.q_ss, p.D, lane);
     // The first copies start before anything waits on memory: K of the first two tiles.  V of the first tile follows after
     // the barrier below: until then the V buffers are the staging area of the Q rows.
     if (n_tiles > t_first) {
@@ -294,24 +275,10 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     }
 
     // ---- Q^T operand, resident in registers ---------------------------------------
-    // through this wavefront's 4 KiB of the V buffers, 64 columns per pass: chunk c of row r at chunk c ^ (r % 8); the lane
-    // of query ql takes chunk 2 s + g of its row for k-step s
+    // through this wavefront's 4 KiB of the V buffers, which nothing is copied into before the barrier below
     vec8 qreg[NSTEP];
-    {
-        char* stage = smem + 2 * L::TILE_BYTES + wave * 4096;
-        static_assert(2 * L::TILE_BYTES >= NW * 4096, "the V buffers hold a staging area per wavefront");
-#pragma unroll
-        for (int h = 0; h < NQH; ++h) {
-#pragma unroll
-            for (int ps = 0; ps < 4; ++ps) {
-                const int rr = ps * 8 + (lane >> 3), c = lane & 7;
-                *(uint4v*)(stage + rr * 128 + ((c ^ (rr & 7)) << 4)) = qraw[h][ps];
-            }
-#pragma unroll
-            for (int sl = 0; sl < 4; ++sl)
-                qreg[h * 4 + sl] = *(const vec8*)(stage + ql * 128 + (((2 * sl + g) ^ (ql & 7)) << 4));
-        }
-    }
+    static_assert(2 * L::TILE_BYTES >= NW * 4096, "the K buffers, and the V buffers, hold a 4 KiB staging area per wavefront");
+    stage_q_rows(qreg, qraw, smem + 2 * L::TILE_BYTES + wave * 4096, lane);
     // Fold scale * log2(e) into Q once (rounded back to the storage type): the matrix product then
     // yields the scores directly in the log2 units the softmax works in.
     const float c2 = p.scale * 1.4426950408889634f;
@@ -816,41 +783,9 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     const float inv = (l_tot == 0.0f) ? __builtin_nanf("") : 1.0f / l_tot;   // no visible key: NaN, as the reference
     if (p.lse && g == 0 && my_i < rows_b)       // m_ref and the sum are in log2 units of the scaled scores
         p.lse[((int64_t)b * p.Hq + hq) * Sq + my_i] = l_tot == 0.0f ? -INFINITY : (m_ref + __builtin_log2f(l_tot)) * 0.6931471805599453f;
-    // The lane-owns-a-row layout would store 8 bytes per lane into 32 different rows per instruction (512 partial cache
-    // lines per wavefront for 64 lines of data, and the compute unit's one path to memory takes them one at a time); so the
-    // normalised rows go through LDS once and leave 16 bytes per lane, eight lanes to a 128-byte run of a row.  The staging
-    // area is this wavefront's 4 KiB of the K buffers: nobody reads K after the barrier of the workgroup's last tile (a
-    // slower wavefront may still be reading V, which lies behind them), and the area is touched by no other wavefront, so
-    // no barrier is needed - 64 columns (32 rows x 128 bytes) per pass; chunk c of row r sits at chunk c ^ (r % 8).
-    {
-        char* stage = smem + wave * 4096;
-        static_assert(2 * L::TILE_BYTES >= NW * 4096, "the K buffers hold a staging area per wavefront");
-        const int row0 = q0 + wave * 32;
-        typedef T vec4 __attribute__((ext_vector_type(4)));
-#ifdef PF_ABL_NOEPI
-        if (l_tot == 12345.678f)
-#endif
-#pragma unroll
-        for (int h = 0; h < D / 64; ++h) {
-#pragma unroll
-            for (int dbl = 0; dbl < 2; ++dbl)
-#pragma unroll
-                for (int r4 = 0; r4 < 4; ++r4) {
-                    vec4 w;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) w[e] = (T)(o_acc[2 * h + dbl][r4 * 4 + e] * inv);
-                    const int c = dbl * 4 + r4;
-                    *(vec4*)(stage + ql * 128 + ((c ^ (ql & 7)) << 4) + g * 8) = w;
-                }
-#pragma unroll
-            for (int ps = 0; ps < 4; ++ps) {
-                const int rr = ps * 8 + (lane >> 3), c = lane & 7;
-                const uint4v val = *(const uint4v*)(stage + rr * 128 + ((c ^ (rr & 7)) << 4));
-                const int col = h * 64 + c * 8;
-                if (row0 + rr < rows_b && col < p.Dv) __builtin_nontemporal_store(val, (uint4v*)(op + (int64_t)(row0 + rr) * p.o_ss + col));
-            }
-        }
-    }
+    // store_o_rows through this wavefront's 4 KiB of the K buffers: nobody reads K after the barrier of the workgroup's last
+    // tile (a slower wavefront may still be reading V, which lies behind them).
+    store_o_rows(o_acc, inv, smem + wave * 4096, op, q0 + wave * 32, rows_b, p.o_ss, p.Dv, lane);
 #endif
 }
 
@@ -865,9 +800,6 @@ static hipError_t launch_prefill_nw(const SdpaParams& p0, hipStream_t stream)
     // 256 registers per lane: eight wavefronts per compute unit, i.e. two workgroups of four or one of eight; an eighth
     // of the compute units per XCD
     p.interleave = work_interleave(p.causal != 0, (8 / NW) * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
-#ifdef PF_FORCE_F
-    p.interleave = PF_FORCE_F;
-#endif
     p.deal_groups = (total & 7) == 0 ? work_deal(p.interleave, p.G, nqb, total >> 3) : 0;
     if constexpr (!DENSE && NW == 4) {
         if (p.num_splits > 1) {          // split launch: partial results, then the split-KV kernels' combine pass

@@ -138,17 +138,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     if (DENSE && n_tiles > t_first) flag_next = mflags[t_first];
 
     // ---- operands ----------------------------------------------------------------------------------------------
-    // Q^T (B operand, resident): this lane's row, elements 16 s + 8 g .. + 7 of it per k-step s (beyond D: zeros, like K's)
+    // Q^T (B operand, resident): this lane's row, elements 16 s + 8 g .. + 7 of it per k-step s (beyond D: zeros, like K's).
+    // Fetched 16 bytes per lane, eight lanes to a run of a row, and brought into that layout through this wavefront's 4 KiB
+    // of the K buffer the first copies do not fill (nothing is copied there before the loop's first barrier).
     vec8 qreg[NSTEP];
     {
-        const T* qrow = qp + (int64_t)min(my_i, Sq - 1) * p.q_ss + g * 8;
-#pragma unroll
-        for (int s = 0; s < NSTEP; ++s) {
-            if (s * 16 + g * 8 < p.D) qreg[s] = *(const vec8*)(qrow + s * 16);
-            else
-#pragma unroll
-                for (int e = 0; e < 8; ++e) qreg[s][e] = (T)0.0f;
-        }
+        uint4v qraw[NSTEP / 4][4];
+        fetch_q_rows(qraw, qp, q0 + wave * 32, Sq, p.q_ss, p.D, lane);
+        stage_q_rows(qreg, qraw, smem + ((t_first + 1) & 1) * TILE + wave * 4096, lane);
         // scale * log2(e) folded into Q once (rounded back to the storage type, as sdpa_prefill_mfma.hip does): the product
         // then yields the scores in the log2 units the softmax works in, whatever the sign of the scale
         const float c2 = p.scale * 1.4426950408889634f;
@@ -289,21 +286,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // ---- normalise and store --------------------------------------------------------------------------------------
     const float l_tot = xor32_sum(l_run);
     const float inv = (l_tot == 0.0f) ? __builtin_nanf("") : 1.0f / l_tot;      // no visible key: NaN, as the reference
-    if (my_i < rows_b) {
-        if (p.lse && g == 0)       // m_run and the sum are in log2 units of the scaled scores
-            p.lse[((int64_t)b * p.Hq + hq) * Sq + my_i] = l_tot == 0.0f ? -INFINITY : (m_run + __builtin_log2f(l_tot)) * 0.6931471805599453f;
-        T* orow = op + (int64_t)my_i * p.o_ss;
-#pragma unroll
-        for (int db = 0; db < NDB; ++db)
-#pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-                typedef T vec4 __attribute__((ext_vector_type(4)));
-                vec4 w;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) w[e] = (T)(o_acc[db][r4 * 4 + e] * inv);
-                if (db * 32 + r4 * 8 + g * 4 < p.Dv) *(vec4*)(orow + db * 32 + r4 * 8 + g * 4) = w;
-            }
-    }
+    if (my_i < rows_b && p.lse && g == 0)       // m_run and the sum are in log2 units of the scaled scores
+        p.lse[((int64_t)b * p.Hq + hq) * Sq + my_i] = l_tot == 0.0f ? -INFINITY : (m_run + __builtin_log2f(l_tot)) * 0.6931471805599453f;
+    // through this wavefront's 4 KiB of the K buffer the last tile did not use: every wavefront is past the barrier of that
+    // tile, i.e. done with the tile before it, and nothing has been copied since
+    store_o_rows(o_acc, inv, smem + (n_tiles & 1) * TILE + wave * 4096, op, q0 + wave * 32, rows_b, p.o_ss, p.Dv, lane);
 #endif
 }
 
