@@ -178,27 +178,29 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
     BwdTiles<T, D, 4, NDB> tl;
     tl.init(wave, lane, p.k_ss, p.v_ss, p.D, p.Dv, 0);
 
-    // this lane's query: Q row (scaled into log2 units, as the forward does) and dO row, the row's normaliser and D_i
+    // this lane's query: Q row (scaled into log2 units, as the forward does) and dO row, the row's normaliser and D_i.  The
+    // rows are fetched 16 bytes per lane, eight lanes to a 128-byte run of a row, and reach the operand layout through this
+    // wavefront's 4 KiB of the V buffers (fetch_q_rows / stage_q_rows), which nothing is copied into before the barrier below.
     vec8 qreg[NSTEP], greg[NSTEP];
     const int qi = min(my_i, Sq - 1);
+    const unsigned lds0 = lds_address(smem);
+    if (n_tiles > 0) tl.issue(0, kp, p.k_ss, Skv, 0, lds0, wave);
     {
-        const T* qrow = qp + (int64_t)qi * p.q_ss + g * 8;
-        const T* grow = gp + (int64_t)qi * bp.do_ss + g * 8;
+        static_assert(2 * L::TILE_BYTES >= 4 * 4096, "the V buffers hold a 4 KiB staging area per wavefront");
+        char* stage = smem + 2 * L::TILE_BYTES + wave * 4096;
+        uint4v qraw[NSTEP / 4][4], graw[NSTEP / 4][4];
+        fetch_q_rows(qraw, qp, q0 + wave * 32, Sq, p.q_ss, p.D, lane);
+        fetch_q_rows(graw, gp, q0 + wave * 32, Sq, bp.do_ss, p.Dv, lane);
+        stage_q_rows(qreg, qraw, stage, lane);
+        stage_q_rows(greg, graw, stage, lane);
         const float c2 = p.scale * 1.4426950408889634f;
 #pragma unroll
-        for (int s = 0; s < NSTEP; ++s) {
-            // (beyond the head dimensions: zeros, like the tiles' rows)
-            vec8 x, y;
+        for (int s = 0; s < NSTEP; ++s)
 #pragma unroll
-            for (int e = 0; e < 8; ++e) { x[e] = (T)0.0f; y[e] = (T)0.0f; }
-            if (s * 16 + g * 8 < p.D) x = *(const vec8*)(qrow + s * 16);
-            if (s * 16 + g * 8 < p.Dv) y = *(const vec8*)(grow + s * 16);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) x[e] = (T)((float)x[e] * c2);
-            qreg[s] = x;
-            greg[s] = y;
-        }
+            for (int e = 0; e < 8; ++e) qreg[s][e] = (T)((float)qreg[s][e] * c2);
     }
+    __syncthreads();      // every wavefront has its rows out of the V buffers
+    if (n_tiles > 0) tl.issue(1, vp, p.v_ss, Skv, 0, lds0 + 2 * L::TILE_BYTES, wave);
     const int64_t stat = ((int64_t)b * p.Hq + hq) * Sq + qi;
     const float l2 = -bp.neg_l2[stat];
     const float dlt = -bp.neg_delta[stat];
@@ -217,11 +219,6 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
     int lim_wave_min = kv_len;
     if (p.causal) lim_wave_min = clampi(q0 + wave * 32 + coff + 1, 0, kv_len);
 
-    const unsigned lds0 = lds_address(smem);
-    if (n_tiles > 0) {
-        tl.issue(0, kp, p.k_ss, Skv, 0, lds0, wave);
-        tl.issue(1, vp, p.v_ss, Skv, 0, lds0 + 2 * L::TILE_BYTES, wave);
-    }
     for (int t = 0; t < n_tiles; ++t) {
         // K(t), V(t) have landed for everyone and everyone is done with tile t-1: the other pair of buffers is free
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -260,18 +257,19 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
         }
     }
 
-    if (my_i < Sq) {
-        T* row = dqp + (int64_t)my_i * bp.dq_ss;
+    // dQ rows out (store_o_rows): padding rows inside Sq as zeros; staged through 4 KiB of the buffers the last tile did not
+    // use (every wavefront is past that tile's barrier, i.e. done with the tile before it) - at D = 64 a buffer holds two
+    // wavefronts' areas, so two wavefronts take the K buffer and two the V buffer
+    if (my_i >= rows_b) {
 #pragma unroll
         for (int db = 0; db < NDB; ++db)
 #pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-                typedef T vec4 __attribute__((ext_vector_type(4)));
-                vec4 w;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) w[e] = (T)(my_i < rows_b ? dq_acc[db][r4 * 4 + e] * p.scale : 0.0f);
-                if (db * 32 + r4 * 8 + g * 4 < p.D) *(vec4*)(row + db * 32 + r4 * 8 + g * 4) = w;
-            }
+            for (int r = 0; r < 16; ++r) dq_acc[db][r] = 0.0f;
+    }
+    {
+        constexpr int PER_BUF = L::TILE_BYTES / 4096;      // staging areas per buffer: 4 (D = 128) or 2
+        char* stage = smem + ((wave / PER_BUF) * 2 + (n_tiles & 1)) * L::TILE_BYTES + (wave % PER_BUF) * 4096;
+        store_o_rows(dq_acc, p.scale, stage, dqp, q0 + wave * 32, Sq, bp.dq_ss, p.D, lane);
     }
 #endif
 }
