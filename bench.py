@@ -256,7 +256,7 @@ def decode_gqa_leg(steps, warmup, only_shape=None):
                 "parity_max_abs_err": w.parity(16)}
         if name == "gqa4_b32_kv8192" and only_shape is None:
             # the same launch with an additive position bias per query head, handed over as the reference's operator takes it: a
-            # [1, Hq, 1, KV] mask tensor.  AUTO sends it to the vector-ALU split-KV kernel, which adds the mask's values.
+            # [1, Hq, 1, KV] mask tensor.  The matrix-core split-KV kernel copies the mask's values into LDS a block ahead.
             bias = (-0.02 * np.arange(Skv)[::-1].astype(np.float32))[None, None, None, :] * (1.0 + np.arange(Hq, dtype=np.float32))[None, :, None, None]
             tm = capi.DeviceBuffer.from_numpy(dtypes.encode(np.ascontiguousarray(bias), dt))
             w.desc.add_mask = tm.ptr

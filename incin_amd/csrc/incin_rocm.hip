@@ -131,6 +131,18 @@ bool mask_rows_vector_loadable(const incin_rocm_sdpa_desc_t* d)
            d->mask_stride[0] % 4 == 0 && d->mask_stride[1] % 4 == 0 && d->mask_stride[2] % 4 == 0;
 }
 
+// A 16-bit dense mask the matrix-core split-KV kernel can copy into LDS 16 bytes (8 keys) at a time: unit key stride, a key
+// count that is a multiple of 8, every row 16-byte aligned, non-negative strides, and offsets inside a batch entry that fit
+// the 32-bit offsets of its copies.
+bool mask_rows_chunk_copyable(const incin_rocm_sdpa_desc_t* d)
+{
+    if (!d->add_mask || d->mask_stride[3] != 1 || d->Skv % 8 != 0 || (reinterpret_cast<uintptr_t>(d->add_mask) & 15u) != 0) return false;
+    for (int a = 0; a < 3; ++a)
+        if (d->mask_stride[a] < 0 || d->mask_stride[a] % 8 != 0) return false;
+    const int64_t extent = (d->Hq - 1) * d->mask_stride[1] + (d->Sq - 1) * d->mask_stride[2] + d->Skv;
+    return extent < (1LL << 29);
+}
+
 int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
 {
     if (!d) return fail(INCIN_ROCM_EINVAL, "scaled_dot_product_attention: null descriptor");
@@ -184,7 +196,10 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     const bool split_ok = layout_ok && head_exact && d->Sq <= 64;      // (the vector-ALU kernel takes a dense mask)
     // the matrix-core split-KV kernels (16-bit and f32): blocks addressed like the prefill kernels' tiles; the f32 kernel and
     // the 256 instances take any number of query positions
-    const bool split_mfma_ok = fast_ok && (d->Sq <= 64 || wide || d->dtype == INCIN_ROCM_F32) && tile_off_ok && std::isfinite(d->scale);
+    // (the 16-bit kernel also takes a dense mask it can copy into LDS eight keys at a time - not in the form of 64 rows per
+    // workgroup at D = 64, where the mask's buffers do not fit beside the rings)
+    const bool split_mask_ok = !d->add_mask || (d->dtype != INCIN_ROCM_F32 && mask_rows_chunk_copyable(d) && !(d_pad == 64 && R > 32));
+    const bool split_mfma_ok = layout_ok && split_mask_ok && (d->Sq <= 64 || wide || d->dtype == INCIN_ROCM_F32) && tile_off_ok && std::isfinite(d->scale);
 
     int impl = d->impl;
     if (impl == INCIN_ROCM_IMPL_AUTO) {
@@ -219,7 +234,8 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         const int64_t wgs_w = d->B * d->Hq * ((d->Sq + 127) / 128), chunks_w = d->B * d->Hkv * ((R + 31) / 32);
         const bool wide_underfilled = (wgs_w * 4 <= cus_w && (d->Skv >= 2048 || chunks_w * 2 <= cus_w || chunks_w % cus_w == 0)) ||
                                       (wgs_w * 2 <= cus_w && chunks_w % cus_w == 0);
-        if (wide && mfma_ok && d->Sq > 64 && !(split_mfma_ok && wide_underfilled)) impl = INCIN_ROCM_IMPL_MFMA;
+        // (with a dense mask the prefill kernel keeps launches of more than 64 positions: its block flags skip what the mask hides)
+        if (wide && mfma_ok && d->Sq > 64 && !(split_mfma_ok && wide_underfilled && !d->add_mask)) impl = INCIN_ROCM_IMPL_MFMA;
         else if (wide && split_mfma_ok) impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
         // f32 (sdpa_decode_f32.hip): from two rows per KV head on, whatever the count - the f32 prefill kernel would spend a
         // 32-row matrix instruction on every query head's few rows (32 heads of a group at one position each: 8.4 ms
@@ -262,7 +278,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
                     "scaled_dot_product_attention: the 64-row MFMA prefill kernel has been retired (INCIN_ROCM_IMPL_MFMA covers its shapes)");
     if (impl == INCIN_ROCM_IMPL_SPLITKV_MFMA && !split_mfma_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
-                    "scaled_dot_product_attention: the matrix-core split-KV kernels need D and Dv <= 256 in whole 16-byte vectors, Sq <= 64 (any Sq in f32 and above 128), no dense mask, a finite scale and 16-byte aligned rows");
+                    "scaled_dot_product_attention: the matrix-core split-KV kernels need D and Dv <= 256 in whole 16-byte vectors, Sq <= 64 (any Sq in f32 and above 128), no dense mask in f32 (16-bit: one with unit key stride, 16-byte aligned rows and a key count that is a multiple of 8; at D = 64 up to 32 rows per KV head), a finite scale and 16-byte aligned rows");
     if (impl == INCIN_ROCM_IMPL_SPLITKV && !split_ok)
         return fail(INCIN_ROCM_EUNSUPPORTED,
                     "scaled_dot_product_attention: the split-KV kernel needs D == Dv in {64,128}, Sq <= 64 and 16-byte aligned rows");

@@ -23,13 +23,22 @@
 //
 // Rows: row r of a chunk is (query head hkv * G + r / Sq, position r % Sq) - the G heads of the group times the Sq
 // positions.  The scale is applied to the f32 scores (any sign), masks as -inf before the maximum.
+//
+// A dense additive mask (MASK instances; the reference's mask tensor: crates/incin-backends/src/cpu/ops/shape_ops.rs:
+// 1262-1266; unit key stride, 16-byte aligned rows, Skv a multiple of 8) is added to the scaled scores.  Its values take
+// the road the keys take: copied global -> LDS a block ahead (two copies of 64 x 16 bytes per 32 rows x 32 keys, into one
+// of two small buffers per wavefront behind the rings), read from there when the block's scores are ready.  The copies
+// share the counter of memory operations in flight with the ring's, so the wait for them is a count as well: three ring
+// copies and the next block's mask copies have been issued since - which asks of the ring only that the copy it needs
+// next anyway has landed.  (Loading the values into registers would leave the waiting to the compiler, which knows
+// nothing of the ring's copies and would drain it at every block.)
 #include <cstdlib>
 
 #include "sdpa_decode_ring.h"
 
 namespace incin_rocm {
 
-template <typename T, int D, int NSLOT, int NRB>
+template <typename T, int D, int NSLOT, int NRB, bool MASK = false>
 __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
 {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -179,6 +188,43 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
             }
     }
 
+    // dense mask: two buffers per wavefront behind the rings, each NRB x KB tiles of 32 rows x 32 keys (64 bytes per row; the
+    // 16-byte chunk c of row r at chunk c ^ (r / 4 % 4), which spreads the reads of a chunk down 32 rows over the banks).
+    // Copy c (of two per tile) brings rows 16 c + lane / 4, chunk lane % 4: the lane's offsets into the mask are those rows'.
+    constexpr int MTILE = 2048, MBUF = NRB * KB * MTILE, NMC = NRB * KB * 2;      // bytes per tile / buffer, copies per block
+    [[maybe_unused]] const unsigned mzone = lds_address(smem) + 4 * NSLOT * SLOT + wave * 2 * MBUF;
+    [[maybe_unused]] int m_voff[NRB][2];
+    [[maybe_unused]] uint4v m_desc = {0u, 0u, 0u, 0u};
+    if constexpr (MASK) {
+#pragma unroll
+        for (int rb = 0; rb < NRB; ++rb)
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                const int rr = 16 * c + (lane >> 2), row = r0 + 32 * rb + rr;
+                const int hq_r = hkv * p.G + (row < R ? row / Sq : 0), qi_r = row < R ? row % Sq : 0;
+                m_voff[rb][c] = (int)(((int64_t)hq_r * p.m_sh + (int64_t)qi_r * p.m_si) * 2) + ((((lane & 3) ^ ((rr >> 2) & 3))) << 4);
+            }
+        // everything from this batch entry's first mask byte to the last one any row reaches; chunks beyond arrive as zeros
+        // (they belong to keys past Skv in the last row, which the limits hide)
+        const int64_t extent = ((p.m_sh ? (int64_t)(p.Hq - 1) * p.m_sh : 0) + (p.m_si ? (int64_t)(Sq - 1) * p.m_si : 0) + Skv) * 2;
+        m_desc = dma_descriptor((const T*)p.mask + (int64_t)b * p.m_sb, (int)(extent > 0x7fffffffLL ? 0x7fffffffLL : extent));
+    }
+    // the mask's values for the block of this wavefront that starts at key jb, into buffer `buf`
+    [[maybe_unused]] auto issue_mask = [&](int jb, int buf) __attribute__((always_inline)) {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");      // (the buffer's last readers have their values)
+#pragma unroll
+        for (int rb = 0; rb < NRB; ++rb)
+#pragma unroll
+            for (int kb2 = 0; kb2 < KB; ++kb2)
+#pragma unroll
+                for (int c = 0; c < 2; ++c)
+                    dma_copy16_at(m_desc, mzone + buf * MBUF + (rb * KB + kb2) * MTILE + c * 1024, m_voff[rb][c], (jb + 32 * kb2) * 2);
+    };
+    if constexpr (MASK) {
+        issue_mask(first_key, 0);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // (start-up: the first block's values, with the first copies)
+    }
+
     const float sc2 = p.scale * 1.4426950408889634f;      // scores in log2 units
     float m_run[NRB], l_run[NRB];
     floatx16 o_acc[NRB][NDB];
@@ -195,6 +241,8 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
     int slot_out = 0;              // slot of the copy consumed next
     for (int j = 0; j < my_blocks; ++j) {
         const int j0 = first_key + j * 4 * BLOCK;
+        // the mask's values of this wavefront's next block start towards the buffer the block before this one used
+        if constexpr (MASK) issue_mask(j0 + 4 * BLOCK, (j + 1) & 1);
         // ---- S^T = K Q^T ----
         wait_oldest_copy<NSLOT, CPB>();
         const char* kb = smem + (wave * NSLOT + slot_out) * SLOT;
@@ -218,12 +266,31 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
         // register r of sub-block kb2 is key j0 + 32 kb2 + 8 (r / 4) + 4 g + (r % 4)
         const bool masked = j0 + BLOCK > mask_from;
         vec8 pb[NRB][2 * KB];
+        if constexpr (MASK) {
+            // issued since this block's mask copies: two ring copies in the last iteration, the next block's mask copies and
+            // one ring copy in this one - everything older has landed once no more than that is in flight
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * CPB + NMC) : "memory");
+        }
 #pragma unroll
         for (int rb = 0; rb < NRB; ++rb) {
 #pragma unroll
             for (int kb2 = 0; kb2 < KB; ++kb2)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) sacc[rb][kb2][r] *= sc2;
+            if constexpr (MASK) {
+                // registers 4 r4 .. 4 r4 + 3 of sub-block kb2 are keys 8 r4 + 4 g .. + 3 of it: half g of chunk r4 of row ql
+                const char* mt = smem + 4 * NSLOT * SLOT + wave * 2 * MBUF + (j & 1) * MBUF + rb * KB * MTILE;
+#pragma unroll
+                for (int kb2 = 0; kb2 < KB; ++kb2)
+#pragma unroll
+                    for (int r4 = 0; r4 < 4; ++r4) {
+                        typedef T vec4 __attribute__((ext_vector_type(4)));
+                        const vec4 mv = *(const vec4*)(mt + kb2 * MTILE + ql * 64 + ((r4 ^ ((ql >> 2) & 3)) << 4) + g * 8);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            sacc[rb][kb2][4 * r4 + e] = __builtin_fmaf((float)mv[e], 1.4426950408889634f, sacc[rb][kb2][4 * r4 + e]);
+                    }
+            }
             if (masked) {
                 const int rel = lim[rb] - (j0 + 4 * g);
 #pragma unroll
@@ -365,14 +432,17 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
 
 hipError_t launch_sdpa_combine(const SdpaParams& p, int dtype, hipStream_t stream);
 
-template <typename T, int D, int NSLOT, int NRB>
+template <typename T, int D, int NSLOT, int NRB, bool MASK = false>
 static hipError_t launch_decode_mfma_t(const SdpaParams& p, hipStream_t stream)
 {
-    // the rings, or what the wavefronts' results need when they meet at the end, whichever is more
+    // the rings (and behind them, with a dense mask, two buffers of its values per wavefront), or what the wavefronts'
+    // results need when they meet at the end, whichever is more
     constexpr size_t slot_bytes = D > 128 ? 2 * DM_SLOT_BYTES : DM_SLOT_BYTES;
-    constexpr size_t ring_bytes = (size_t)4 * NSLOT * slot_bytes, merge_bytes = (size_t)NRB * (4 * 32 * 2 + 4 * (D / 32) * 16 * 64) * sizeof(float);
+    constexpr size_t mask_bytes = MASK ? (size_t)4 * 2 * NRB * (slot_bytes / (32 * D * 2)) * 2048 : 0;
+    constexpr size_t ring_bytes = (size_t)4 * NSLOT * slot_bytes + mask_bytes, merge_bytes = (size_t)NRB * (4 * 32 * 2 + 4 * (D / 32) * 16 * 64) * sizeof(float);
     constexpr size_t lds = ring_bytes > merge_bytes ? ring_bytes : merge_bytes;
-    auto kern = sdpa_decode_mfma_kernel<T, D, NSLOT, NRB>;
+    static_assert(lds <= 160 * 1024, "a compute unit's LDS");
+    auto kern = sdpa_decode_mfma_kernel<T, D, NSLOT, NRB, MASK>;
     // the dynamic-LDS limit of this instance is raised once per device, not per launch
     static std::atomic<uint64_t> prepared{0};
     int dev = 0;
@@ -416,11 +486,29 @@ static bool decode_two_slots(const SdpaParams& p, int dtype)
     return slots == 2 || (slots != DM_NSLOT && decode_mfma_workgroups_per_cu(one_block, p.split_len, dtype, p.Dp) == 2);
 }
 
+// With a dense mask: the same forms with four slots per wavefront instead of five (the mask's buffers take the room); 64 rows
+// per workgroup at D = 64 do not fit and are not offered (the planner sends such launches elsewhere).
+template <typename T, int D>
+static hipError_t launch_decode_mfma_masked(const SdpaParams& p, hipStream_t stream)
+{
+    if constexpr (D <= 128) {
+        if (decode_mfma_chunk_rows(p.G * p.Sq, 2, D) == 64) {
+            if constexpr (D == 128) return launch_decode_mfma_t<T, D, 4, 2, true>(p, stream);
+            else return hipErrorInvalidValue;
+        }
+        if (decode_two_slots(p, 2)) return launch_decode_mfma_t<T, D, 2, 1, true>(p, stream);
+        return launch_decode_mfma_t<T, D, 4, 1, true>(p, stream);
+    } else {
+        return launch_decode_mfma_t<T, D, 2, 1, true>(p, stream);
+    }
+}
+
 // Host has validated: dtype f16 / bf16, D and Dv <= 128 in whole 16-byte vectors (p.Dp = the instance), rows 16-byte aligned with unit last-dim stride, row strides
 // below 2^24 elements, split_len a multiple of 256 (whole rounds of the four wavefronts' blocks of 32 or 64 keys).
 template <typename T, int D>
 static hipError_t launch_decode_mfma_d(const SdpaParams& p, hipStream_t stream)
 {
+    if (p.mask) return launch_decode_mfma_masked<T, D>(p, stream);
     if (decode_mfma_chunk_rows(p.G * p.Sq, 2, D) == 64) return launch_decode_mfma_t<T, D, DM_NSLOT, 2>(p, stream);
     // Short splits (up to DM_SHORT_KEYS keys: 16 blocks per wavefront) take rings of two slots, which lets a compute
     // unit hold two workgroups: with so little to stream, what counts is that one workgroup's start-up (its first
@@ -436,7 +524,8 @@ hipError_t launch_sdpa_decode_mfma(const SdpaParams& p, int dtype, hipStream_t s
     if (dtype == 0) return launch_sdpa_decode_f32(p, decode_two_slots(p, 0), stream);
     hipError_t e;
     // head dimensions above 128: one form - 32 rows, two slots of 16 KiB (a block of 32 keys) per wavefront
-    if (p.Dp == 256) e = dtype == 1 ? launch_decode_mfma_t<f16_t, 256, 2, 1>(p, stream) : launch_decode_mfma_t<bf16_t, 256, 2, 1>(p, stream);
+    if (p.Dp == 256 && p.mask) e = dtype == 1 ? launch_decode_mfma_masked<f16_t, 256>(p, stream) : launch_decode_mfma_masked<bf16_t, 256>(p, stream);
+    else if (p.Dp == 256) e = dtype == 1 ? launch_decode_mfma_t<f16_t, 256, 2, 1>(p, stream) : launch_decode_mfma_t<bf16_t, 256, 2, 1>(p, stream);
     else if (p.Dp == 128) e = dtype == 1 ? launch_decode_mfma_d<f16_t, 128>(p, stream) : launch_decode_mfma_d<bf16_t, 128>(p, stream);
     else e = dtype == 1 ? launch_decode_mfma_d<f16_t, 64>(p, stream) : launch_decode_mfma_d<bf16_t, 64>(p, stream);
     if (e != hipSuccess || p.num_splits == 1) return e;

@@ -109,6 +109,12 @@ __device__ __forceinline__ void dma_copy16(uint4v desc, unsigned lds_addr, int b
     // (one wait state between the write of m0 and the copy that reads it)
     asm volatile("s_nop 0\n\tbuffer_load_dwordx4 %0, %1, 0 offen lds" ::"v"(byte_offset), "s"(desc), "{m0}"(lds_addr) : "memory");
 }
+// The same with a wavefront-uniform byte offset added to every lane's (the instruction's scalar offset operand): copies that
+// differ only by such an offset share one register of lane offsets.
+__device__ __forceinline__ void dma_copy16_at(uint4v desc, unsigned lds_addr, int byte_offset, int uniform_offset)
+{
+    asm volatile("s_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds" ::"v"(byte_offset), "s"(desc), "s"(uniform_offset), "{m0}"(lds_addr) : "memory");
+}
 // Offset for the lane of such a copy that fetches 16-byte chunk `chunk` of row `row` (rows `row_bytes` apart in memory,
 // `data_bytes` of data each): a chunk at or beyond the row's data gets an offset that no descriptor covers, so that lane
 // delivers zeros.  This is how a head dimension below the one a kernel instance is built for is padded: with zeros, on

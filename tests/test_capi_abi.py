@@ -189,7 +189,8 @@ def test_dispatch_choices():
     (dict(impl=capi.IMPL_SPLITKV, Sq=4096), capi.EUNSUPPORTED),
     (dict(impl=capi.IMPL_SPLITKV_MFMA, Sq=4096), capi.EUNSUPPORTED),
     (dict(impl=capi.IMPL_SPLITKV_MFMA, Sq=1, D=36, Dv=36), capi.EUNSUPPORTED),
-    (dict(impl=capi.IMPL_SPLITKV_MFMA, Sq=1, add_mask=0x20000), capi.EUNSUPPORTED),
+    (dict(impl=capi.IMPL_SPLITKV_MFMA, Sq=1, add_mask=0x20000), capi.EUNSUPPORTED),          # (a mask without a unit key stride)
+    (dict(impl=capi.IMPL_SPLITKV_MFMA, Sq=1, add_mask=0x20000, dtype=capi.F32), capi.EUNSUPPORTED),
     (dict(D=512, Dv=512), capi.EUNSUPPORTED),
     (dict(B=70000), capi.ESHAPE),
 ])

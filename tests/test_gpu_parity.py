@@ -697,8 +697,11 @@ def test_head_dimensions_above_128_with_a_dense_mask(gpu, dtype, dims):
     # decode-like: 3 positions over the cache with a mask
     q3 = q[:, :, :3]
     got, info = host.sdpa(q3, k, v, dtype, mask=m[:, :, :3], return_info=True)
-    assert info["impl"] == capi.IMPL_MFMA
+    assert info["impl"] == capi.IMPL_MFMA          # (420 keys: not a multiple of 8, so not for the split-KV kernel's mask copies)
     check(got, oracle_full(q3, k, v, G=2, mask=m[:, :, :3]), tol, "decode-like with a mask, D=%d" % D)
+    got, info = host.sdpa(q3, k[:, :, :416], v[:, :, :416], dtype, mask=m[:, :, :3, :416], return_info=True)
+    assert info["impl"] == capi.IMPL_SPLITKV_MFMA          # (416 keys: up to 64 positions go to the split-KV kernel with their mask)
+    check(got, oracle_full(q3, k[:, :, :416], v[:, :, :416], G=2, mask=m[:, :, :3, :416]), tol, "decode-like with a mask on the split-KV kernel, D=%d" % D)
     # 418 keys: rows of the mask 836 bytes apart
     got, info = host.sdpa(q, k[:, :, :418], v[:, :, :418], dtype, mask=m[..., :418], return_info=True)
     assert info["impl"] == capi.IMPL_GENERIC
@@ -772,9 +775,62 @@ def test_decode_with_a_dense_additive_mask(gpu, dtype, shape):
         ref = oracle_full(q, k, v, G=Hq // Hkv, mask=full)
         for splits in (0, 1, 5):
             say("decode with a mask: %s %r %s splits=%d" % (dtypes.NAMES[dtype], shape, name, splits))
-            got, info = host.sdpa(q, k, v, dtype, mask=m, kv_lens=lens, num_splits=splits, return_info=True)
+            got, info = host.sdpa(q, k, v, dtype, mask=m, kv_lens=lens, num_splits=splits, impl=capi.IMPL_SPLITKV, return_info=True)
             assert info["impl"] == capi.IMPL_SPLITKV
             check(got, ref, TOL[dtype], "decode with a mask (%s), splits=%d->%d" % (name, splits, info["splits"]))
+            got, info = host.sdpa(q, k, v, dtype, mask=m, kv_lens=lens, num_splits=splits, return_info=True)
+            # (AUTO: f32 and key counts that are not multiples of 4 stay on the vector-ALU kernel, 16-bit launches follow the
+            # thresholds of launches without a mask)
+            assert info["impl"] in (capi.IMPL_SPLITKV, capi.IMPL_SPLITKV_MFMA)
+            if dtype == capi.F32 or Skv % 8:
+                assert info["impl"] == capi.IMPL_SPLITKV
+            check(got, ref, TOL[dtype], "decode with a mask (%s), AUTO, splits=%d->%d" % (name, splits, info["splits"]))
+
+
+@pytest.mark.parametrize("dtype", [capi.BF16, capi.F16], ids=lambda x: dtypes.NAMES[x])
+@pytest.mark.parametrize("shape", [
+    # B, Hq, Hkv, Sq, Skv, D
+    (2, 8, 2, 1, 1496, 128),          # grouped-query decode, 4 rows per KV head
+    (1, 16, 2, 1, 2056, 128),         # 8 rows, a ragged last block
+    (2, 4, 2, 3, 904, 64),            # 6 rows: a short causal run; blocks of 64 keys
+    (1, 48, 1, 1, 1000, 128),         # 48 rows: two blocks of rows per workgroup
+    (2, 8, 2, 5, 640, 64),            # 20 rows, causal among themselves
+    (1, 8, 2, 1, 1200, 256),          # the 256 instance
+    (3, 4, 4, 1, 4104, 128),          # one row per KV head
+    (2, 8, 2, 1, 40, 128),            # a cache shorter than one round of blocks
+], ids=lambda x: "x".join(map(str, x)))
+def test_decode_with_a_dense_additive_mask_on_the_matrix_cores(gpu, dtype, shape):
+    """The matrix-core split-KV kernel with a mask tensor: a position bias per head ([1, Hq, 1, Skv]), a [B, 1, Sq, Skv] mask
+    with hidden stretches and a full [B, Hq, Sq, Skv] one, with key counts and (where there are several positions) the causal
+    flag on top - against the oracle, for the split counts the planner chooses and forced ones (a split that ends inside a
+    block, splits whose keys the mask hides entirely), and against the vector-ALU kernel where that takes the launch."""
+    B, Hq, Hkv, Sq, Skv, D = shape
+    q, k, v = inputs(2900 + sum(shape), B, Hq, Hkv, Sq, Skv, D, D, dtype)
+    bias = (-0.02 * np.arange(Skv)[::-1].astype(np.float32))[None, None, None, :] * (1.0 + np.arange(Hq, dtype=np.float32))[None, :, None, None]
+    bias = dtypes.round_to(np.ascontiguousarray(np.broadcast_to(bias, (1, Hq, 1, Skv))), dtype)
+    r = rng(18)
+    holes = (r.standard_normal((B, 1, Sq, Skv)) * 0.3).astype(np.float32)
+    holes[:, :, :, 100:400] = -np.inf
+    holes[0, :, :, Skv - 50:] = -np.inf
+    holes = dtypes.round_to(holes, dtype)
+    full_m = dtypes.round_to((r.standard_normal((B, Hq, Sq, Skv)) * 0.5).astype(np.float32), dtype)
+    full_m[:, 0, :, :] = -np.inf                       # one head sees nothing: NaN rows, as the reference gives
+    lens = np.array([Skv - 7 * b for b in range(B)], np.int32)
+    causal = Sq > 1
+    tri = np.triu(np.full((Sq, Skv), -np.inf, np.float32), 1 + Skv - Sq) if causal else np.zeros((Sq, Skv), np.float32)
+    for name, m in (("bias per head", bias), ("holes per batch entry", holes), ("full mask", full_m)):
+        full = np.broadcast_to(m, (B, Hq, Sq, Skv)) + tri + np.where(np.arange(Skv)[None, :] < lens[:, None], 0.0, -np.inf).astype(np.float32)[:, None, None, :]
+        ref = oracle_full(q, k, v, G=Hq // Hkv, mask=full)
+        for splits in (0, 1, 3, 7):
+            say("matrix-core decode with a mask: %s %r %s splits=%d" % (dtypes.NAMES[dtype], shape, name, splits))
+            got, info = host.sdpa(q, k, v, dtype, mask=m, kv_lens=lens, causal=causal, num_splits=splits, impl=capi.IMPL_SPLITKV_MFMA, return_info=True)
+            assert info["impl"] == capi.IMPL_SPLITKV_MFMA
+            check(got, ref, TOL[dtype], "matrix-core decode with a mask (%s), splits=%d->%d" % (name, splits, info["splits"]))
+    # a mask it cannot copy eight keys at a time is refused by name and goes elsewhere under AUTO
+    with pytest.raises(capi.RocmError):
+        host.sdpa(q, k[:, :, :Skv - 4], v[:, :, :Skv - 4], dtype, mask=bias[..., :Skv - 4], impl=capi.IMPL_SPLITKV_MFMA)
+    got, info = host.sdpa(q, k[:, :, :Skv - 4], v[:, :, :Skv - 4], dtype, mask=bias[..., :Skv - 4], return_info=True)
+    assert info["impl"] != capi.IMPL_SPLITKV_MFMA
 
 
 def test_decode_splitkv_matrix_cores_lengths_strides_scale(gpu):
