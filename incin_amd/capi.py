@@ -26,7 +26,7 @@ EXPORTS = [
     "incin_rocm_memcpy_h2d", "incin_rocm_memcpy_d2h", "incin_rocm_memcpy_d2d", "incin_rocm_copy_strided", "incin_rocm_sum_to_shape", "incin_rocm_sync",
     "incin_rocm_stream_create", "incin_rocm_stream_destroy", "incin_rocm_stream_sync",
     "incin_rocm_event_create", "incin_rocm_event_destroy", "incin_rocm_event_record",
-    "incin_rocm_event_sync", "incin_rocm_event_elapsed_ms",
+    "incin_rocm_event_sync", "incin_rocm_event_query", "incin_rocm_event_elapsed_ms",
     "incin_rocm_graph_begin", "incin_rocm_graph_end", "incin_rocm_graph_launch", "incin_rocm_graph_destroy",
     "incin_rocm_sdpa_workspace", "incin_rocm_sdpa_fwd", "incin_rocm_sdpa_fwd_static",
     "incin_rocm_sizeof_kv_append_desc", "incin_rocm_kv_append",
@@ -145,6 +145,7 @@ def load():
     lib.incin_rocm_event_destroy.argtypes = [C.c_int32, C.c_void_p]
     lib.incin_rocm_event_record.argtypes = [C.c_int32, C.c_void_p, C.c_void_p]
     lib.incin_rocm_event_sync.argtypes = [C.c_int32, C.c_void_p]
+    lib.incin_rocm_event_query.argtypes = [C.c_int32, C.c_void_p, C.POINTER(C.c_int32)]
     lib.incin_rocm_event_elapsed_ms.argtypes = [C.c_int32, C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]
     lib.incin_rocm_graph_begin.argtypes = [C.c_int32, C.c_void_p]
     lib.incin_rocm_graph_end.argtypes = [C.c_int32, C.c_void_p, C.POINTER(C.c_void_p)]

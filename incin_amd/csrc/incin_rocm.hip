@@ -619,6 +619,16 @@ int incin_rocm_stream_sync(int32_t dev, void* stream)
     return 0;
 }
 
+int incin_rocm_event_query(int32_t dev, void* event, int32_t* done)
+{
+    if (!event || !done) return fail(INCIN_ROCM_EINVAL, "event_query: null argument");
+    if (int rc = use_device(dev)) return rc;
+    const hipError_t e = hipEventQuery((hipEvent_t)event);
+    if (e != hipSuccess && e != hipErrorNotReady) return fail(INCIN_ROCM_ERUNTIME, "ROCm hipEventQuery failed: %s", hipGetErrorString(e));
+    *done = e == hipSuccess ? 1 : 0;
+    return 0;
+}
+
 int incin_rocm_graph_begin(int32_t dev, void* stream)
 {
     if (!stream) return fail(INCIN_ROCM_EINVAL, "graph_begin: recording needs a stream of its own, not the default stream");

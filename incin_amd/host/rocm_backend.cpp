@@ -4,6 +4,8 @@
 #include <algorithm>
 #include <cmath>
 #include <cstring>
+#include <map>
+#include <mutex>
 
 #include "../../include/incin_rocm.h"
 
@@ -38,6 +40,99 @@ Error from_status(int rc, int32_t device)
     }
 }
 
+// ---- the calling thread's stream, its recording, and the buffer pools ---------------------------------------------------
+thread_local void* t_stream = nullptr;
+thread_local RecordedGraph* t_recording = nullptr;
+
+struct IdleBlock {
+    void* ptr;
+    size_t bytes;
+    void* stream;      // the stream whose work may still be using the block
+    void* event;       // recorded on that stream at release; nullptr: nothing can be using it
+};
+struct DevicePool {
+    std::mutex mu;
+    std::multimap<size_t, IdleBlock> idle;
+    int64_t device_allocs = 0, reused = 0, idle_bytes = 0;
+};
+DevicePool& pool_of(int32_t device)
+{
+    // never evicted, like the reference's device cache (cuda/gpu.rs:99-152), and never destroyed: buffers released while the
+    // process winds down still find their pool
+    static std::mutex* mu = new std::mutex();
+    static std::map<int32_t, DevicePool*>* pools = new std::map<int32_t, DevicePool*>();
+    std::lock_guard<std::mutex> lock(*mu);
+    DevicePool*& p = (*pools)[device];
+    if (!p) p = new DevicePool();
+    return *p;
+}
+size_t pool_size_class(size_t bytes)
+{
+    if (bytes == 0) bytes = 1;
+    const size_t unit = bytes <= (1u << 20) ? 512 : (64u << 10);      // little is wasted, and equal requests meet equal blocks
+    return (bytes + unit - 1) / unit * unit;
+}
+// A block of at least `bytes`: from the pool when one is there that this thread's stream may touch, else from the device.
+// *settled says whether nothing on the device can still be using the block (a host-side copy into it needs that).
+int pool_alloc(int32_t device, size_t bytes, void** out, size_t* granted, bool* settled)
+{
+    const size_t want = pool_size_class(bytes);
+    DevicePool& pool = pool_of(device);
+    {
+        std::lock_guard<std::mutex> lock(pool.mu);
+        for (auto it = pool.idle.lower_bound(want); it != pool.idle.end() && it->first <= want + want / 4 + 4096; ++it) {
+            IdleBlock& b = it->second;
+            bool done = b.event == nullptr;
+            if (!done && !t_recording) {      // (an event recorded into a graph cannot be asked; such blocks carry none)
+                int32_t d = 0;
+                if (incin_rocm_event_query(device, b.event, &d) == 0 && d) done = true;
+            }
+            if (!done && b.stream != t_stream) continue;
+            if (b.event) incin_rocm_event_destroy(device, b.event);
+            *out = b.ptr;
+            *granted = b.bytes;
+            *settled = done;
+            pool.idle_bytes -= (int64_t)b.bytes;
+            ++pool.reused;
+            pool.idle.erase(it);
+            return 0;
+        }
+    }
+    if (t_recording) {
+        // (no message from the C ABI for this one: the refusal is the pool's)
+        return -1;
+    }
+    int rc = incin_rocm_alloc(device, want, out);
+    if (rc == INCIN_ROCM_ENOMEM) {      // give back what is idle and try once more
+        RocmBackend::trim_pool(device);
+        rc = incin_rocm_alloc(device, want, out);
+    }
+    if (rc != 0) return rc;
+    *granted = want;
+    *settled = true;
+    std::lock_guard<std::mutex> lock(pool.mu);
+    ++pool.device_allocs;
+    return 0;
+}
+void pool_release(int32_t device, void* ptr, size_t bytes)
+{
+    if (t_recording && t_recording->device == device) {      // the recorded kernels use it at every replay
+        t_recording->retained.emplace_back(ptr, bytes);
+        return;
+    }
+    IdleBlock b{ptr, bytes, t_stream, nullptr};
+    if (incin_rocm_event_create(device, &b.event) != 0 || incin_rocm_event_record(device, b.event, t_stream) != 0) {
+        // no event to be had: make sure nothing uses the block, then it needs none
+        if (b.event) incin_rocm_event_destroy(device, b.event);
+        b.event = nullptr;
+        incin_rocm_sync(device);
+    }
+    DevicePool& pool = pool_of(device);
+    std::lock_guard<std::mutex> lock(pool.mu);
+    pool.idle_bytes += (int64_t)bytes;
+    pool.idle.emplace(bytes, b);
+}
+
 std::vector<int64_t> contiguous_strides(const std::vector<int64_t>& shape)
 {
     std::vector<int64_t> st(shape.size());
@@ -49,7 +144,23 @@ std::vector<int64_t> contiguous_strides(const std::vector<int64_t>& shape)
     return st;
 }
 
-Error alloc_storage(const std::vector<int64_t>& dims, DType dtype, int32_t device, RocmStorage* out)
+// A buffer of `bytes` (the pool may grant more).  *settled (may be null): nothing on the device can still be using it.
+Error alloc_buffer(int32_t device, size_t bytes, std::shared_ptr<RocmBuffer>* out, bool* settled = nullptr)
+{
+    void* p = nullptr;
+    size_t granted = 0;
+    bool s = true;
+    const int rc = pool_alloc(device, bytes, &p, &granted, &s);
+    if (rc == -1)
+        return err(ErrorKind::Msg, "ROCm allocation of " + std::to_string(bytes) + " bytes while a launch graph is being recorded: the pool holds no "
+                                   "buffer of that size for this stream (run the recorded operators once before recording)");
+    if (Error e = from_status(rc, device)) return e;
+    if (settled) *settled = s;
+    *out = std::make_shared<RocmBuffer>(device, p, granted);
+    return ok();
+}
+
+Error alloc_storage(const std::vector<int64_t>& dims, DType dtype, int32_t device, RocmStorage* out, bool* settled = nullptr)
 {
     int64_t n = 1;
     for (int64_t d : dims) {
@@ -58,8 +169,10 @@ Error alloc_storage(const std::vector<int64_t>& dims, DType dtype, int32_t devic
     }
     void* p = nullptr;
     const size_t bytes = (size_t)n * dtype_size(dtype);
-    if (Error e = from_status(incin_rocm_alloc(device, bytes, &p), device)) return e;
-    out->buffer = std::make_shared<RocmBuffer>(device, p, bytes);
+    std::shared_ptr<RocmBuffer> buf;
+    if (Error e = alloc_buffer(device, bytes, &buf, settled)) return e;
+    p = buf->ptr();
+    out->buffer = std::move(buf);
     out->shape = dims;
     out->strides = contiguous_strides(dims);
     out->offset_elements = 0;
@@ -91,7 +204,65 @@ int64_t last_launch_count() { return g_launches; }
 
 RocmBuffer::~RocmBuffer()
 {
-    if (ptr_) incin_rocm_free(device_, ptr_);
+    if (ptr_) pool_release(device_, ptr_, bytes_);
+}
+
+RecordedGraph::~RecordedGraph()
+{
+    if (graph) incin_rocm_graph_destroy(device, graph);
+    // (what the recording kept may be in use by a replay that is still running: release it like any other buffer, ordered
+    // behind the calling thread's stream - the caller replays and destroys on one stream)
+    for (auto& b : retained) pool_release(device, b.first, b.second);
+}
+
+void RocmBackend::set_stream(void* stream) { t_stream = stream; }
+void* RocmBackend::stream() { return t_stream; }
+
+Error RocmBackend::begin_recording(int32_t device)
+{
+    if (t_recording) return err(ErrorKind::Msg, "a launch graph is already being recorded on this thread");
+    if (!t_stream) return err(ErrorKind::Msg, "recording needs a stream of its own (set_stream), not the default stream");
+    if (Error e = from_status(incin_rocm_graph_begin(device, t_stream), device)) return e;
+    t_recording = new RecordedGraph();
+    t_recording->device = device;
+    return ok();
+}
+
+Error RocmBackend::end_recording(std::unique_ptr<RecordedGraph>* out)
+{
+    if (!t_recording) return err(ErrorKind::Msg, "no launch graph is being recorded on this thread");
+    std::unique_ptr<RecordedGraph> g(t_recording);
+    t_recording = nullptr;
+    if (Error e = from_status(incin_rocm_graph_end(g->device, t_stream, &g->graph), g->device)) return e;
+    *out = std::move(g);
+    return ok();
+}
+
+Error RocmBackend::replay(const RecordedGraph& g) { return from_status(incin_rocm_graph_launch(g.device, g.graph, t_stream), g.device); }
+
+RocmBackend::PoolStats RocmBackend::pool_stats(int32_t device)
+{
+    DevicePool& pool = pool_of(device);
+    std::lock_guard<std::mutex> lock(pool.mu);
+    PoolStats s;
+    s.device_allocs = pool.device_allocs;
+    s.reused = pool.reused;
+    s.idle_bytes = pool.idle_bytes;
+    return s;
+}
+
+Error RocmBackend::trim_pool(int32_t device)
+{
+    if (Error e = from_status(incin_rocm_sync(device), device)) return e;
+    DevicePool& pool = pool_of(device);
+    std::lock_guard<std::mutex> lock(pool.mu);
+    for (auto& kv : pool.idle) {
+        if (kv.second.event) incin_rocm_event_destroy(device, kv.second.event);
+        incin_rocm_free(device, kv.second.ptr);
+    }
+    pool.idle.clear();
+    pool.idle_bytes = 0;
+    return ok();
 }
 
 int64_t RocmStorage::numel() const
@@ -131,10 +302,15 @@ Error RocmBackend::from_bytes(const void* bytes, size_t nbytes, const std::vecto
 {
     if ((int)dtype < 0 || (int)dtype > 2) return err(ErrorKind::UnsupportedDType, "dtype tag " + std::to_string((int)dtype) + " on backend Rocm");
     RocmStorage s;
-    if (Error e = alloc_storage(dims, dtype, device, &s)) return e;
+    bool settled = true;
+    if (Error e = alloc_storage(dims, dtype, device, &s, &settled)) return e;
     if ((size_t)s.numel() * dtype_size(dtype) != nbytes)
         return err(ErrorKind::Msg, "from_bytes: " + std::to_string(nbytes) + " bytes do not fill shape " + shape_str(dims));
     if (nbytes && !bytes) return err(ErrorKind::Msg, "from_bytes: null source");
+    // (the copy does not go through the thread's stream: a block the pool handed over in stream order may still be read by
+    // that stream's earlier work)
+    if (!settled)
+        if (Error e = from_status(t_stream ? incin_rocm_stream_sync(device, t_stream) : incin_rocm_sync(device), device)) return e;
     if (Error e = from_status(incin_rocm_memcpy_h2d(device, s.buffer->ptr(), bytes, nbytes), device)) return e;
     *out = std::move(s);
     return ok();
@@ -146,6 +322,10 @@ Error RocmBackend::to_bytes(const RocmStorage& s, std::vector<uint8_t>* out)
     const int64_t n = s.numel();
     out->assign((size_t)n * isz, 0);
     if (n == 0) return ok();
+    // (the synchronous point of the contract, cuda/backend.rs:2007-2045: the copies below go through the default stream,
+    // which does not wait for a stream created here)
+    if (t_stream)
+        if (Error e = from_status(incin_rocm_stream_sync(s.device, t_stream), s.device)) return e;
     if (s.is_contiguous())
         return from_status(incin_rocm_memcpy_d2h(s.device, out->data(), s.data(), (size_t)n * isz), s.device);
     if (s.shape.size() <= 8) {          // strided or broadcast view: gather on the device, then one copy
@@ -181,9 +361,8 @@ Error RocmBackend::contiguous(const RocmStorage& s, RocmStorage* out)
     if (Error e = alloc_storage(s.shape, s.dtype, s.device, &dense)) return e;
     if (dense.numel() > 0) {
         if (Error e = from_status(incin_rocm_copy_strided(s.device, dense.buffer->ptr(), s.data(), (int32_t)s.shape.size(), s.shape.data(),
-                                                          s.strides.data(), (int32_t)dtype_size(s.dtype), nullptr), s.device))
+                                                          s.strides.data(), (int32_t)dtype_size(s.dtype), t_stream), s.device))
             return e;
-        if (Error e = from_status(incin_rocm_sync(s.device), s.device)) return e;
     }
     *out = std::move(dense);
     return ok();
@@ -226,7 +405,7 @@ static Error sum_to_shape(const RocmStorage& g, const std::vector<int64_t>& targ
     }
     RocmStorage dst;
     if (Error e = alloc_storage(target, g.dtype, g.device, &dst)) return e;
-    if (Error e = from_status(incin_rocm_sum_to_shape(g.device, (int32_t)g.dtype, dst.buffer->ptr(), g.data(), r, g.shape.data(), kept.data(), nullptr), g.device))
+    if (Error e = from_status(incin_rocm_sum_to_shape(g.device, (int32_t)g.dtype, dst.buffer->ptr(), g.data(), r, g.shape.data(), kept.data(), t_stream), g.device))
         return e;
     *out = std::move(dst);
     return ok();
@@ -289,12 +468,15 @@ Error RocmBackend::reshape(const RocmStorage& s, const std::vector<int64_t>& dim
 
 Error RocmBackend::upload_i32(const std::vector<int32_t>& values, int32_t device, std::shared_ptr<RocmBuffer>* out)
 {
-    void* p = nullptr;
     const size_t bytes = values.size() * sizeof(int32_t);
-    if (Error e = from_status(incin_rocm_alloc(device, bytes ? bytes : 4, &p), device)) return e;
-    auto buf = std::make_shared<RocmBuffer>(device, p, bytes);
-    if (bytes)
-        if (Error e = from_status(incin_rocm_memcpy_h2d(device, p, values.data(), bytes), device)) return e;
+    std::shared_ptr<RocmBuffer> buf;
+    bool settled = true;
+    if (Error e = alloc_buffer(device, bytes ? bytes : 4, &buf, &settled)) return e;
+    if (bytes) {
+        if (!settled)      // (a host-side copy into a block that earlier work of the stream may still read)
+            if (Error e = from_status(t_stream ? incin_rocm_stream_sync(device, t_stream) : incin_rocm_sync(device), device)) return e;
+        if (Error e = from_status(incin_rocm_memcpy_h2d(device, buf->ptr(), values.data(), bytes), device)) return e;
+    }
     *out = std::move(buf);
     return ok();
 }
@@ -309,10 +491,8 @@ Error RocmBackend::tag_causal(const RocmStorage& mask, RocmStorage* out)
 
 Error RocmBackend::tag_key_padding(const RocmStorage& mask, const std::vector<int32_t>& lens, RocmStorage* out)
 {
-    void* p = nullptr;
-    if (Error e = from_status(incin_rocm_alloc(mask.device, lens.size() * sizeof(int32_t), &p), mask.device)) return e;
-    auto buf = std::make_shared<RocmBuffer>(mask.device, p, lens.size() * sizeof(int32_t));
-    if (Error e = from_status(incin_rocm_memcpy_h2d(mask.device, p, lens.data(), lens.size() * sizeof(int32_t)), mask.device)) return e;
+    std::shared_ptr<RocmBuffer> buf;
+    if (Error e = upload_i32(lens, mask.device, &buf)) return e;
     *out = mask;
     out->mask_tag = MaskTag{MaskTag::KeyPadding, buf, (int64_t)lens.size()};
     return ok();
@@ -371,10 +551,8 @@ Error RocmBackend::attention_impl(const RocmStorage& q, const RocmStorage& k, co
             if (fq) if (Error e = dense_last_axis(q, &qd)) return e;
             if (fk) if (Error e = dense_last_axis(k, &kd)) return e;
             if (fv) if (Error e = dense_last_axis(v, &vd)) return e;
-            Error e = attention_impl(qd, kd, vd, mask, scale, facts, grad_out, out, grads);
-            // the temporaries are used stream-ordered: finish before they are released
-            if (Error e2 = from_status(incin_rocm_sync(q.device), q.device)) return e ? e : e2;
-            return e;
+            // (the temporaries are released in stream order when this returns: nothing to wait for)
+            return attention_impl(qd, kd, vd, mask, scale, facts, grad_out, out, grads);
         }
     }
 
@@ -618,10 +796,8 @@ Error RocmBackend::attention_impl(const RocmStorage& q, const RocmStorage& k, co
         d.add_mask = dense_mask ? static_cast<const char*>(mask->buffer->ptr()) + mo * (int64_t)isz : nullptr;
         if (grads) {
             if (!lse) {
-                void* lp = nullptr;
                 const size_t lbytes = (size_t)std::max<int64_t>(B * Hq * Sq, 1) * sizeof(float);
-                if (Error e = from_status(incin_rocm_alloc(q.device, lbytes, &lp), q.device)) return e;
-                lse = std::make_shared<RocmBuffer>(q.device, lp, lbytes);
+                if (Error e = alloc_buffer(q.device, lbytes, &lse)) return e;
             }
             d.lse = static_cast<float*>(lse->ptr());
         }
@@ -631,15 +807,12 @@ Error RocmBackend::attention_impl(const RocmStorage& q, const RocmStorage& k, co
         d.workspace_bytes = 0;
         if (Error e = from_status(incin_rocm_sdpa_workspace(&d, &ws_bytes, &splits, nullptr), q.device)) return e;
         if (ws_bytes) {
-            if (!workspace || workspace->bytes() < ws_bytes) {
-                void* wp = nullptr;
-                if (Error e = from_status(incin_rocm_alloc(q.device, ws_bytes, &wp), q.device)) return e;
-                workspace = std::make_shared<RocmBuffer>(q.device, wp, ws_bytes);
-            }
+            if (!workspace || workspace->bytes() < ws_bytes)
+                if (Error e = alloc_buffer(q.device, ws_bytes, &workspace)) return e;
             d.workspace = workspace->ptr();
             d.workspace_bytes = workspace->bytes();
         }
-        if (Error e = from_status(incin_rocm_sdpa_fwd(&d, nullptr), q.device)) return e;
+        if (Error e = from_status(incin_rocm_sdpa_fwd(&d, t_stream), q.device)) return e;
         ++g_launches;
         if (grads) {
             int64_t gqo = 0, gko = 0, gvo = 0;
@@ -663,24 +836,19 @@ Error RocmBackend::attention_impl(const RocmStorage& q, const RocmStorage& k, co
             size_t bws = 0;
             if (Error e = from_status(incin_rocm_sdpa_bwd_workspace(&bd, &bws), q.device)) return e;
             if (bws) {
-                if (!bwd_workspace || bwd_workspace->bytes() < bws) {
-                    void* wp = nullptr;
-                    if (Error e = from_status(incin_rocm_alloc(q.device, bws, &wp), q.device)) return e;
-                    bwd_workspace = std::make_shared<RocmBuffer>(q.device, wp, bws);
-                }
+                if (!bwd_workspace || bwd_workspace->bytes() < bws)
+                    if (Error e = alloc_buffer(q.device, bws, &bwd_workspace)) return e;
                 bd.workspace = bwd_workspace->ptr();
                 bd.workspace_bytes = bwd_workspace->bytes();
             }
-            if (Error e = from_status(incin_rocm_sdpa_bwd(&bd, nullptr), q.device)) return e;
+            if (Error e = from_status(incin_rocm_sdpa_bwd(&bd, t_stream), q.device)) return e;
         }
         for (int a = (int)oidx.size() - 1; a >= 0; --a) {
             if (++oidx[a] < bshape[outer_axes[a]]) break;
             oidx[a] = 0;
         }
     }
-    // the workspaces are used stream-ordered: finish before they are released
-    if (workspace || bwd_workspace || lse)
-        if (Error e = from_status(incin_rocm_sync(q.device), q.device)) return e;
+    // (the workspaces and the row normalisers are still in use by the launches above: they are released in stream order)
     *out = std::move(o);
     if (grads) {
         // (a gradient storage of the operand's own extents only needs the operand's rank back)

@@ -38,7 +38,11 @@ struct Error {
     explicit operator bool() const { return kind != ErrorKind::None; }
 };
 
-// One device allocation, freed when the last storage that views it goes away.
+// One device allocation, released when the last storage that views it goes away.  Released, not freed: the buffer goes back
+// to a pool per device, stamped with an event on the stream the releasing thread works on, and is handed out again to
+// that same stream at once (its work is ordered behind what still uses the buffer) or to another stream once the event
+// has passed - the stream-ordered lifetime the reference's CUDA buffers have (cuda/storage.rs:171-177, 225-233).  So an
+// operator can drop temporaries and workspaces that its kernels are still using without waiting for the device.
 class RocmBuffer {
   public:
     RocmBuffer(int32_t device, void* ptr, size_t bytes) : device_(device), ptr_(ptr), bytes_(bytes) {}
@@ -76,7 +80,35 @@ struct RocmStorage {
     const char* data() const { return static_cast<const char*>(buffer->ptr()) + offset_elements * (int64_t)dtype_size(dtype); }
 };
 
+// What a recording (launch graph) keeps alive: buffers released while it was being recorded - the recorded kernels use
+// them at every replay.  They return to the pool when the recording is destroyed.
+struct RecordedGraph {
+    void* graph = nullptr;        // incin_rocm_graph_* handle
+    int32_t device = 0;
+    std::vector<std::pair<void*, size_t>> retained;
+    ~RecordedGraph();
+    RecordedGraph() = default;
+    RecordedGraph(const RecordedGraph&) = delete;
+    RecordedGraph& operator=(const RecordedGraph&) = delete;
+};
+
 struct RocmBackend {
+    // The stream the calling thread's operators launch on and its buffers are ordered by (nullptr: the device's default
+    // stream, as the reference's backends use: cuda/ops/matmul.rs:57-90).  to_bytes waits for it.
+    static void set_stream(void* stream);
+    static void* stream();
+    // Recording of the calling thread's work on its stream (not the default stream) into a launch graph.  While recording,
+    // nothing may be allocated from or returned to the device: buffers come from the pool (run the same operators once
+    // beforehand: what they released is what the recording finds there) and released ones are kept with the recording.
+    static Error begin_recording(int32_t device);
+    static Error end_recording(std::unique_ptr<RecordedGraph>* out);
+    static Error replay(const RecordedGraph& g);
+    // Pool counters of a device (for tests): device allocations made so far, buffers handed out from the pool, bytes idle
+    // in the pool.  trim_pool waits for the device and frees what is idle.
+    struct PoolStats { int64_t device_allocs = 0, reused = 0, idle_bytes = 0; };
+    static PoolStats pool_stats(int32_t device);
+    static Error trim_pool(int32_t device);
+
     // Backend::from_bytes: one allocation + one host-to-device copy; row-major contiguous.
     static Error from_bytes(const void* bytes, size_t nbytes, const std::vector<int64_t>& dims, DType dtype, int32_t device,
                             RocmStorage* out);

@@ -1,6 +1,7 @@
 #include "rocm_backend_c.h"
 
 #include <cstring>
+#include <memory>
 #include <string>
 
 #include "rocm_backend.hpp"
@@ -11,6 +12,9 @@ using namespace incin_rocm_host;
 
 struct incin_host_storage {
     RocmStorage s;
+};
+struct incin_host_graph {
+    std::unique_ptr<RecordedGraph> g;
 };
 struct incin_host_attention_spec {
     AttentionSpec spec;
@@ -128,6 +132,28 @@ int incin_host_attention_backward(const incin_host_storage* q, const incin_host_
 }
 
 void incin_host_release(incin_host_storage* s) { delete s; }
+
+int incin_host_data_ptr(const incin_host_storage* s, void** out) { *out = const_cast<char*>(s->s.data()); return 0; }
+void incin_host_set_stream(void* stream) { RocmBackend::set_stream(stream); }
+int incin_host_begin_recording(int32_t device) { return finish(RocmBackend::begin_recording(device)); }
+int incin_host_end_recording(incin_host_graph** out)
+{
+    std::unique_ptr<RecordedGraph> g;
+    Error e = RocmBackend::end_recording(&g);
+    if (!e) *out = new incin_host_graph{std::move(g)};
+    return finish(e);
+}
+int incin_host_replay(const incin_host_graph* g) { return finish(RocmBackend::replay(*g->g)); }
+void incin_host_release_graph(incin_host_graph* g) { delete g; }
+int incin_host_pool_stats(int32_t device, int64_t* device_allocs, int64_t* reused, int64_t* idle_bytes)
+{
+    const RocmBackend::PoolStats s = RocmBackend::pool_stats(device);
+    *device_allocs = s.device_allocs;
+    *reused = s.reused;
+    *idle_bytes = s.idle_bytes;
+    return 0;
+}
+int incin_host_trim_pool(int32_t device) { return finish(RocmBackend::trim_pool(device)); }
 
 int64_t incin_host_last_launch_count(void) { return incin_rocm_host::last_launch_count(); }
 

@@ -35,6 +35,19 @@ int incin_host_attention_backward(const incin_host_storage* q, const incin_host_
                                   const incin_host_storage* mask, int32_t has_scale, double scale, const incin_host_storage* grad_out,
                                   incin_host_storage** out, incin_host_storage** dq, incin_host_storage** dk, incin_host_storage** dv);
 void incin_host_release(incin_host_storage* s);
+/* device address of the view's first element (for tests that rewrite an operand in place between replays of a recording) */
+int incin_host_data_ptr(const incin_host_storage* s, void** out);
+/* the stream the calling thread's operators launch on (NULL: the default stream) */
+void incin_host_set_stream(void* stream);
+/* recording of the calling thread's work on its stream into a launch graph; replays go to the calling thread's stream */
+typedef struct incin_host_graph incin_host_graph;
+int incin_host_begin_recording(int32_t device);
+int incin_host_end_recording(incin_host_graph** out);
+int incin_host_replay(const incin_host_graph* g);
+void incin_host_release_graph(incin_host_graph* g);
+/* pool counters of a device: allocations made on the device so far, buffers handed out from the pool, bytes idle in it */
+int incin_host_pool_stats(int32_t device, int64_t* device_allocs, int64_t* reused, int64_t* idle_bytes);
+int incin_host_trim_pool(int32_t device);
 /* number of kernel launches (C-ABI sdpa calls) the last attention call on this thread made */
 int64_t incin_host_last_launch_count(void);
 

@@ -30,6 +30,8 @@ EXPORTS = [
     "incin_host_lower_attention", "incin_host_attention_spec_out_dims", "incin_host_execute_attention",
     "incin_host_release_attention_spec", "incin_host_reshape",
     "incin_host_is_compiled_in", "incin_host_probe", "incin_host_detect_device",
+    "incin_host_data_ptr", "incin_host_set_stream", "incin_host_begin_recording", "incin_host_end_recording", "incin_host_replay",
+    "incin_host_release_graph", "incin_host_pool_stats", "incin_host_trim_pool",
 ]
 
 
@@ -92,6 +94,16 @@ def lib():
         L.incin_host_is_compiled_in.argtypes = [C.c_int32]
         L.incin_host_probe.argtypes = [C.c_int32]
         L.incin_host_detect_device.argtypes = [I32P, C.c_int32, I32P, I32P]
+        L.incin_host_data_ptr.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+        L.incin_host_set_stream.restype = None
+        L.incin_host_set_stream.argtypes = [C.c_void_p]
+        L.incin_host_begin_recording.argtypes = [C.c_int32]
+        L.incin_host_end_recording.argtypes = [C.POINTER(C.c_void_p)]
+        L.incin_host_replay.argtypes = [C.c_void_p]
+        L.incin_host_release_graph.restype = None
+        L.incin_host_release_graph.argtypes = [C.c_void_p]
+        L.incin_host_pool_stats.argtypes = [C.c_int32, I64P, I64P, I64P]
+        L.incin_host_trim_pool.argtypes = [C.c_int32]
         _lib = L
     return _lib
 
@@ -153,6 +165,12 @@ class RocmStorage:
         d = (C.c_int64 * max(n, 1))()
         lib().incin_host_strides(self._h, d)
         return tuple(d[i] for i in range(n))
+
+    @property
+    def data_ptr(self):
+        p = C.c_void_p()
+        lib().incin_host_data_ptr(self._h, C.byref(p))
+        return p.value
 
     def is_contiguous(self):
         acc = 1
@@ -231,6 +249,50 @@ def attention_backward(q, k, v, grad_out, mask=None, scale=None):
         q._h, k._h, v._h, mask._h if mask is not None else None,
         0 if scale is None else 1, 0.0 if scale is None else float(scale), grad_out._h, *[C.byref(h) for h in hs]))
     return tuple(RocmStorage(h.value) for h in hs)
+
+
+def set_stream(stream_ptr):
+    """The stream the calling thread's operators launch on from now on (None: the device's default stream)."""
+    lib().incin_host_set_stream(stream_ptr)
+
+
+class Recording:
+    """`with Recording(device) as rec:` records the calling thread's operators on its stream (set_stream) into a launch
+    graph; afterwards `rec.replay()` runs them again.  The recording keeps the buffers its kernels use."""
+
+    def __init__(self, device=0):
+        self.device, self._g = device, None
+
+    def __enter__(self):
+        _check(lib().incin_host_begin_recording(self.device))
+        return self
+
+    def __exit__(self, et, ev, tb):
+        g = C.c_void_p()
+        code = lib().incin_host_end_recording(C.byref(g))
+        if et is None:
+            _check(code)
+        self._g = g
+        return False
+
+    def replay(self):
+        _check(lib().incin_host_replay(self._g))
+
+    def release(self):
+        if self._g:
+            lib().incin_host_release_graph(self._g)
+            self._g = None
+
+
+def pool_stats(device=0):
+    """(device allocations so far, buffers handed out from the pool, bytes idle in the pool)"""
+    a, r, i = C.c_int64(), C.c_int64(), C.c_int64()
+    lib().incin_host_pool_stats(device, C.byref(a), C.byref(r), C.byref(i))
+    return a.value, r.value, i.value
+
+
+def trim_pool(device=0):
+    _check(lib().incin_host_trim_pool(device))
 
 
 def last_launch_count():

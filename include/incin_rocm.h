@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define INCIN_ROCM_ABI_VERSION 9
+#define INCIN_ROCM_ABI_VERSION 10
 
 /* ---- status codes (mapped to incin_core::Error variants by the Rust side;
  *      crates/incin-core/src/err.rs:109-223) --------------------------------- */
@@ -127,6 +127,10 @@ int incin_rocm_event_create(int32_t dev, void** out);
 int incin_rocm_event_destroy(int32_t dev, void* event);
 int incin_rocm_event_record(int32_t dev, void* event, void* stream);
 int incin_rocm_event_sync(int32_t dev, void* event);
+/* *done = 1 once everything recorded before the event has finished, else 0 (never blocks).  What a stream-ordered
+ * allocator needs to hand a released buffer to another stream: the reference's CUDA buffers are allocated and freed
+ * in stream order by its driver crate (crates/incin-backends/src/cuda/storage.rs:171-177, 225-233). */
+int incin_rocm_event_query(int32_t dev, void* event, int32_t* done);
 int incin_rocm_event_elapsed_ms(int32_t dev, void* start, void* stop, float* out_ms);
 
 /* ---- launch graphs ------------------------------------------------------------

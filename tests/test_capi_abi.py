@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), "missing export %s" % n
     assert set(names) == set(capi.EXPORTS)
-    assert lib.incin_rocm_abi_version() == 9
+    assert lib.incin_rocm_abi_version() == 10
 
 
 def test_descriptor_layout_matches():

@@ -411,3 +411,75 @@ def test_gradient_shape_errors(gpu):
     with pytest.raises(RB.BackendError) as e:
         RB.attention_backward(S(q), S(rnd(55, (2, 3, 5, 8), RB.F32)), S(rnd(56, (2, 3, 5, 8), RB.F32)), S(go[:, :, :3]))
     assert e.value.kind == "ShapeMismatch"
+
+
+# ---- buffers released in stream order; operators recorded into launch graphs ---------------------------------------------
+def test_operators_do_not_allocate_once_the_pool_is_warm(gpu):
+    """The operator drops its temporaries (gathered operands, workspaces, row normalisers) while its kernels still use them:
+    they go back to the pool in stream order (cuda/storage.rs:171-177 is the reference's counterpart) and the same call,
+    made again, is served from the pool without a single device allocation - with the same results."""
+    B, H, Sq, Skv, D = 2, 3, 40, 4160, 64
+    q, kt, v = rnd(60, (B, H, Sq, D), RB.BF16), rnd(61, (B, 1, D, Skv), RB.BF16), rnd(62, (B, H, Skv, D), RB.BF16)
+    go = rnd(63, (B, H, Sq, D), RB.BF16)
+    S = lambda a: RB.RocmStorage.from_numpy(a, RB.BF16)
+    Q, V, GO = S(q), S(v), S(go)
+    K = S(kt).transpose(2, 3).broadcast_as((B, H, Skv, D))              # gathered into a temporary by the operator
+    outs = []
+    for rep in range(3):
+        before = RB.pool_stats()
+        out = RB.scaled_dot_product_attention(Q, K, V)                   # (split launch: a workspace too)
+        o2, dq, dk, dv = RB.attention_backward(Q, K, V, GO)
+        after = RB.pool_stats()
+        outs.append((out.to_numpy(), dq.to_numpy(), dk.to_numpy(), dv.to_numpy()))
+        del out, o2, dq, dk, dv
+        if rep == 2:
+            assert after[0] == before[0], "device allocations on a warm pool: %r -> %r" % (before, after)
+            assert after[1] > before[1]
+    for a, b in zip(outs[0], outs[-1]):
+        assert np.array_equal(a, b)
+    k_log = np.broadcast_to(kt.transpose(0, 1, 3, 2), (B, H, Skv, D))
+    close(outs[0][0], O.sdpa(q, k_log, v), TOL[RB.BF16], "forward on a warm pool")
+    RB.trim_pool()
+    assert RB.pool_stats()[2] == 0
+
+
+def test_recorded_operator_with_a_transposed_k(gpu):
+    """The operator with k handed over as a transposed view (gathered into a temporary first), recorded into a launch graph on
+    a stream of the caller's and replayed: no step of it waits for the device or allocates while recording; every replay -
+    with eager work on the same operands and synchronisations in between - gives what an eager call gives on the operands'
+    current contents."""
+    from incin_amd import capi
+    B, H, Sq, Skv, D = 2, 4, 48, 300, 64
+    dtype = RB.BF16
+    q, kt, v = rnd(70, (B, H, Sq, D), dtype), rnd(71, (B, H, D, Skv), dtype), rnd(72, (B, H, Skv, D), dtype)
+    S = lambda a: RB.RocmStorage.from_numpy(a, dtype)
+    Q, Kt, V = S(q), S(kt), S(v)
+    K = Kt.transpose(2, 3)
+    stream = capi.Stream()
+    RB.set_stream(stream.ptr)
+    try:
+        warm = RB.scaled_dot_product_attention(Q, K, V)                  # fills the pool with what the recording will ask for
+        ref0 = warm.to_numpy()
+        del warm
+        with RB.Recording() as rec:
+            out = RB.scaled_dot_product_attention(Q, K, V)
+        stream.sync()
+        k_log = kt.transpose(0, 1, 3, 2)
+        close(ref0, O.sdpa(q, k_log, v), TOL[dtype], "eager call on the stream")
+        for rep in range(4):
+            # new contents for q, written in place; an eager call on the same operands between the replays
+            q_new = rnd(80 + rep, (B, H, Sq, D), dtype)
+            stream.sync()
+            raw = dtypes.encode(q_new, dtype)
+            capi.check(capi.load().incin_rocm_memcpy_h2d(0, Q.data_ptr, raw.ctypes.data, raw.nbytes))
+            rec.replay()
+            eager = RB.scaled_dot_product_attention(Q, K, V)
+            got, want = out.to_numpy(), eager.to_numpy()                 # (to_bytes waits for the stream)
+            assert np.array_equal(got, want), "replay %d differs from the eager call" % rep
+            close(got, O.sdpa(q_new, k_log, v), TOL[dtype], "replay %d" % rep)
+        rec.release()
+    finally:
+        RB.set_stream(None)
+        stream.sync()
+        stream.destroy()
+
