@@ -220,8 +220,9 @@ __device__ __forceinline__ void fetch_q_rows(uint4v (&qraw)[NQH][4], const T* qh
             qraw[h][ps] = col < Dq ? __builtin_nontemporal_load((const uint4v*)(qhead + (int64_t)min(row0 + rr, Sq - 1) * q_ss + col)) : zero;
         }
 }
-template <typename V8, int NQH>
-__device__ __forceinline__ void stage_q_rows(V8 (&qreg)[4 * NQH], const uint4v (&qraw)[NQH][4], char* stage, int lane)
+// (NS k-steps' worth of operands are taken out: 4 * NQH, or fewer when the last columns of the last pass are padding)
+template <typename V8, int NS, int NQH>
+__device__ __forceinline__ void stage_q_rows(V8 (&qreg)[NS], const uint4v (&qraw)[NQH][4], char* stage, int lane)
 {
     const int ql = lane & 31, g = lane >> 5;
 #pragma unroll
@@ -232,7 +233,8 @@ __device__ __forceinline__ void stage_q_rows(V8 (&qreg)[4 * NQH], const uint4v (
             *(uint4v*)(stage + rr * 128 + ((c ^ (rr & 7)) << 4)) = qraw[h][ps];
         }
 #pragma unroll
-        for (int sl = 0; sl < 4; ++sl) qreg[h * 4 + sl] = *(const V8*)(stage + ql * 128 + (((2 * sl + g) ^ (ql & 7)) << 4));
+        for (int sl = 0; sl < 4; ++sl)
+            if (h * 4 + sl < NS) qreg[h * 4 + sl] = *(const V8*)(stage + ql * 128 + (((2 * sl + g) ^ (ql & 7)) << 4));
     }
 }
 template <typename T, int NDB>
@@ -241,9 +243,9 @@ __device__ __forceinline__ void store_o_rows(const floatx16 (&o_acc)[NDB], float
     typedef T vec4 __attribute__((ext_vector_type(4)));
     const int ql = lane & 31, g = lane >> 5;
 #pragma unroll
-    for (int h = 0; h < NDB / 2; ++h) {
+    for (int h = 0; h < (NDB + 1) / 2; ++h) {      // (an odd NDB: the last pass is half full, and Dv cuts its stores)
 #pragma unroll
-        for (int dbl = 0; dbl < 2; ++dbl)
+        for (int dbl = 0; dbl < 2 && 2 * h + dbl < NDB; ++dbl)
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4) {
                 vec4 w;

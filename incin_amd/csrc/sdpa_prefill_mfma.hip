@@ -84,15 +84,25 @@ namespace incin_rocm {
 // writes, per row, the unnormalised O, the reference and the sum - the partial-result format of the split-KV kernels, whose
 // combine kernel finishes the job.  For launches with too few (batch, head, row block) items to fill the device over a long
 // key axis (a chunk of a long prompt, a single sequence): the key axis supplies the parallelism the rows lack.
-template <typename T, int D, bool DENSE, int NW, bool SPLIT = false>
+//
+// KS, NB: the k-steps of 16 head-dimension columns the score product runs over, and the 32-column blocks of the output it
+// keeps.  D fixes the layout of a tile in LDS (rows of D columns, zero beyond the tensors' own); head dimensions that fill only
+// part of it leave the rest out of the arithmetic as well: 6 k-steps and 3 blocks for head dimensions up to 96 in the 128 layout.
+template <typename T, int D, bool DENSE, int NW, bool SPLIT = false, int KS = D / 16, int NB = D / 32>
 __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void sdpa_prefill_mfma_kernel(SdpaParams p)
 {
 #if defined(__HIP_DEVICE_COMPILE__)   // the body uses device-only types (buffer descriptors); the host pass needs only the stub
     typedef typename Mma<T>::vec8 vec8;
     typedef PfLayout<D> L;
-    constexpr int NSTEP = D / 16;          // k-steps of the S^T product
-    constexpr int NDB = D / 32;            // 32-wide blocks of the head dimension
+    constexpr int NSTEP = KS;              // k-steps of the S^T product
+    constexpr int NDB = NB;                // 32-wide blocks of the head dimension
+    static_assert(KS <= D / 16 && NB <= D / 32 && KS >= 4 && NB >= 1, "");
+    // the 8 slices of 4 scores a tile's probabilities are taken in, dealt over the k-steps of the next tile's score product
+    // (slices slice_lo(s) .. slice_lo(s + 1) - 1 under k-step s), and the 16 pairs of the row sum (or the 16 registers of
+    // the maximum) over the MFMAs of the O^T update
+    auto slice_lo = [](int s) constexpr { return s * 8 / KS; };
+    auto pair_lo = [](int i) constexpr { return i * 16 / (4 * NB); };
     constexpr int LPW = L::TILE_BYTES / 1024 / NW;     // wavefront-wide 1 KiB copies per tensor per tile
     constexpr int BM = 32 * NW;                        // query rows per workgroup
     // bf16 without a dense mask: probabilities are taken 2^-SHIFT times smaller, so that "some probability reached 2"
@@ -427,8 +437,8 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
             for (int b2 = 0; b2 < 2; ++b2)
                 sn[b2] = Mma<T>::run(kbuf[s % KD][b2], qreg[s], s == 0 ? neg_ref : sn[b2]);
             if (s + KD < NSTEP) read_k(k_nxt, s + KD);
-            if (NSTEP == 8) softmax_slice(sc, s);
-            else { softmax_slice(sc, 2 * s); softmax_slice(sc, 2 * s + 1); }
+#pragma unroll
+            for (int sl = slice_lo(s); sl < slice_lo(s + 1); ++sl) softmax_slice(sc, sl);
             if (s >= NSTEP - VD / 2) { read_v(v_cur, 2 * (s - (NSTEP - VD / 2))); read_v(v_cur, 2 * (s - (NSTEP - VD / 2)) + 1); }
         }
 #pragma unroll
@@ -436,7 +446,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 SGB(SG_MFMA, 1);
-                if (NSTEP == 8) { SGB(SG_TRANS, 2); SGB(SG_VALU, 2); } else { SGB(SG_TRANS, 4); SGB(SG_VALU, 4); }
+                if (slice_lo(s + 1) - slice_lo(s) == 1) { SGB(SG_TRANS, 2); SGB(SG_VALU, 2); } else { SGB(SG_TRANS, 4); SGB(SG_VALU, 4); }
                 if (s + KD < NSTEP) SGB(SG_DSR, 1);
                 if (s >= NSTEP - VD / 2) SGB(SG_DSR, 2);
             }
@@ -448,12 +458,10 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
         for (int i = 0; i < NPV; ++i) {
             o_acc[i % NDB] = Mma<T>::run(vbuf[i % VD], pb[i / NDB], o_acc[i % NDB]);
             if (i + VD < NPV) read_v(v_cur, i + VD);
-            if (NPV == 16) {
-                m0 = fmaxf(m0, sn[0][i]);
-                m1 = fmaxf(m1, sn[1][i]);
-            } else {
-                m0 = fmaxf(fmaxf(m0, sn[0][2 * i]), sn[0][2 * i + 1]);
-                m1 = fmaxf(fmaxf(m1, sn[1][2 * i]), sn[1][2 * i + 1]);
+#pragma unroll
+            for (int r = pair_lo(i); r < pair_lo(i + 1); ++r) {
+                m0 = fmaxf(m0, sn[0][r]);
+                m1 = fmaxf(m1, sn[1][r]);
             }
         }
         tmax = xor32_max(fmaxf(m0, m1));
@@ -498,14 +506,10 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
             for (int b2 = 0; b2 < 2; ++b2)
                 sn[b2] = Mma<T>::run(kbuf[s % KD][b2], qreg[s], s == 0 ? neg_ref : sn[b2]);
             if (s + KD < NSTEP) read_k(k_nxt, s + KD);
-            if (NSTEP == 8) {
-                exps_of(s);
-                if (s > 0) pack_of(s - 1);
-            } else {
-                exps_of(2 * s);
-                if (s > 0) pack_of(2 * s - 1);
-                exps_of(2 * s + 1);
-                pack_of(2 * s);
+#pragma unroll
+            for (int sl = slice_lo(s); sl < slice_lo(s + 1); ++sl) {
+                exps_of(sl);
+                if (sl > 0) pack_of(sl - 1);
             }
             if (s >= NSTEP - VD / 2) { read_v(v_cur, 2 * (s - (NSTEP - VD / 2))); read_v(v_cur, 2 * (s - (NSTEP - VD / 2)) + 1); }
         }
@@ -515,7 +519,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 SGB(SG_MFMA, 1);
-                if (NSTEP == 8) {
+                if (slice_lo(s + 1) - slice_lo(s) == 1) {
                     SGB(SG_TRANS, 1);
                     if (s > 0) SGB(SG_VALU, 1);
                     SGB(SG_TRANS, 1);
@@ -557,22 +561,16 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
             o_acc[i % NDB] = Mma<T>::run(vbuf[i % VD], pb[i / NDB], o_acc[i % NDB]);
             if (i + VD < NPV) read_v(v_cur, i + VD);
             // row sum of the rounded probabilities, two per instruction, four chains
-            if (NPV == 16) {
-                typename Mma<T>::vec2 pr = {pb[i / 4][2 * (i % 4)], pb[i / 4][2 * (i % 4) + 1]};
-                rs[i % 4] = Mma<T>::add2(pr, rs[i % 4]);
-            } else {
 #pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const int ii = 2 * i + j;
-                    typename Mma<T>::vec2 pr = {pb[ii / 4][2 * (ii % 4)], pb[ii / 4][2 * (ii % 4) + 1]};
-                    rs[ii % 4] = Mma<T>::add2(pr, rs[ii % 4]);
-                }
+            for (int ii = pair_lo(i); ii < pair_lo(i + 1); ++ii) {
+                typename Mma<T>::vec2 pr = {pb[ii / 4][2 * (ii % 4)], pb[ii / 4][2 * (ii % 4) + 1]};
+                rs[ii % 4] = Mma<T>::add2(pr, rs[ii % 4]);
             }
         }
 #pragma unroll
         for (int i = 0; i < NPV; ++i) {
             SGB(SG_MFMA, 1);
-            SGB(SG_VALU, NPV == 16 ? 1 : 2);
+            if (pair_lo(i + 1) - pair_lo(i) == 1) SGB(SG_VALU, 1); else SGB(SG_VALU, 2);
             if (i + VD < NPV) SGB(SG_DSR, 2);
         }
         asm volatile("" : "+v"(rs[0]), "+v"(rs[1]), "+v"(rs[2]), "+v"(rs[3]));      // (keeps the sums from being sunk below the next barrier)
@@ -806,6 +804,12 @@ static hipError_t launch_prefill_nw(const SdpaParams& p0, hipStream_t stream)
             hipLaunchKernelGGL((sdpa_prefill_mfma_kernel<T, D, false, 4, true>), dim3((unsigned)total, (unsigned)p.num_splits), dim3(256), 0, stream, p);
             hipError_t e = hipGetLastError();
             return e != hipSuccess ? e : launch_sdpa_combine(p, std::is_same<T, f16_t>::value ? 1 : 2, stream);
+        }
+    }
+    if constexpr (!DENSE && D == 128) {
+        if (p.D <= 96 && p.Dv <= 96) {   // the last quarter of the layout is padding: the instance that leaves it out of the products
+            hipLaunchKernelGGL((sdpa_prefill_mfma_kernel<T, D, false, NW, false, 6, 3>), dim3((unsigned)total), dim3(64 * NW), 0, stream, p);
+            return hipGetLastError();
         }
     }
     hipLaunchKernelGGL((sdpa_prefill_mfma_kernel<T, D, DENSE, NW>), dim3((unsigned)total), dim3(64 * NW), 0, stream, p);

@@ -989,6 +989,48 @@ def test_256_row_workgroups(gpu, dtype, shape, monkeypatch):
     check(got, ref, TOL[dtype], "256-row workgroups %r" % (shape,))
 
 
+@pytest.mark.parametrize("dtype", [capi.BF16, capi.F16], ids=lambda x: dtypes.NAMES[x])
+@pytest.mark.parametrize("dims", [(96, 96), (80, 96), (96, 72), (72, 40)], ids=lambda x: "D%d_Dv%d" % x)
+@pytest.mark.parametrize("rows", ["128", "256"])
+def test_head_dimensions_up_to_96_in_the_128_layout(gpu, dtype, dims, rows, monkeypatch):
+    """Head dimensions between 65 and 96 (D and Dv both) run an instance of the 16-bit prefill kernel that keeps the 128-column
+    layout of a tile in LDS but leaves the last quarter out of both matrix products: 6 of 8 k-steps, 3 of 4 output blocks.
+    Its pipelined loop deals the softmax over the k-steps differently, so it gets what the full instance gets: enough
+    tiles for the loop to run in both workgroup forms, ragged edges, key counts, grouped queries, and the keys far above
+    the reference that make the loop back out of a tile."""
+    D, Dv = dims
+    monkeypatch.setenv("INCIN_ROCM_PREFILL_BLOCK_ROWS", rows)
+    for B, Hq, Hkv, Sq, Skv, causal, kv_lens in ((1, 2, 2, 640, 640, True, None), (1, 2, 1, 700, 900, False, None),
+                                                  (2, 4, 2, 513, 1100, True, [1100, 311])):
+        say("head dimension %d/%d, %s rows: %s" % (D, Dv, rows, (B, Hq, Hkv, Sq, Skv, causal, kv_lens)))
+        q, k, v = inputs(2900 + D + Dv + Sq, B, Hq, Hkv, Sq, Skv, D, Dv, dtype)
+        kl = None if kv_lens is None else np.asarray(kv_lens, np.int32)
+        got, lse, info = host.sdpa(q, k, v, dtype, causal=causal, kv_lens=kl, impl=capi.IMPL_MFMA, return_info=True, return_lse=True)
+        assert info["impl"] == capi.IMPL_MFMA and got.shape[-1] == Dv
+        check(got, oracle_full(q, k, v, G=Hq // Hkv, causal=causal, kv_lens=kl), TOL[dtype], "D=%d Dv=%d %s rows" % (D, Dv, rows))
+        _, lse_g = host.sdpa(q, k, v, dtype, causal=causal, kv_lens=kl, impl=capi.IMPL_GENERIC, return_lse=True)
+        assert np.max(np.abs(lse - lse_g)) < 2e-2
+    # keys 60 to 130 logit units above what a row saw before (as in the test below), identical within a class
+    B, H, S = 1, 2, 640
+    r = rng(SEED0 + 94)
+    a = r.choice(np.array([1.0, -1.0, 0.5], np.float32), size=(B, H, S, 1))
+    q = np.broadcast_to(a, (B, H, S, D)).copy()
+    b = np.full((B, H, S, 1), -4.0, np.float32)
+    b[:, :, [70, 200, 201, 207, 231, 250]] = 2.0
+    b[:, :, [400, 401, 437]] = 8.0
+    b[:, 1, 100] = 8.0
+    k = np.broadcast_to(b, (B, H, S, D)).copy()
+    v = dtypes.round_to(r.standard_normal((B, H, S, Dv), dtype=np.float32), dtype)
+    for causal in (False, True):
+        got = host.sdpa(q, k, v, dtype, causal=causal, impl=capi.IMPL_MFMA, scale=1.0 / np.sqrt(128.0))
+        logit = a * np.swapaxes(b, 2, 3)
+        if causal:
+            logit = np.where(np.tril(np.ones((S, S), bool)), logit, -np.inf)
+        top = logit == logit.max(axis=-1, keepdims=True)
+        mean = np.einsum("bhij,bhjd->bhid", top.astype(np.float64), v.astype(np.float64)) / top.sum(axis=-1, keepdims=True)
+        check(got, mean.astype(np.float32), TOL[dtype], "scores far above the first tiles, D=%d Dv=%d" % (D, Dv))
+
+
 @pytest.mark.parametrize("causal", [False, True, "tensor"], ids=["full", "causal", "causal_as_tensor"])
 @pytest.mark.parametrize("impl", [capi.IMPL_MFMA], ids=["mfma"])
 @pytest.mark.parametrize("dtype", [capi.BF16, capi.F16])
