@@ -78,25 +78,42 @@ class Workload:
         # a padded self-attention batch: the same lengths say which keys and which query rows are padding
         self.desc = host.make_desc(self.tq, self.tk, self.tv, self.to, causal=causal, kv_lens=self.tl,
                                    q_lens=self.tl if pad_queries else None, impl=impl, num_splits=num_splits)
-        nbytes, self.splits, self.impl = capi.sdpa_workspace(self.desc)
-        self.ws = capi.DeviceBuffer(nbytes) if nbytes else None
-        if self.ws is not None:
-            self.desc.workspace, self.desc.workspace_bytes = self.ws.ptr, self.ws.nbytes
+        self.descs, self.more_kv, self.turn = [self.desc], [], 0
+        self._make_kw = dict(causal=causal, kv_lens=self.tl, q_lens=self.tl if pad_queries else None)
+        self.ws = None
+        self.replan(impl, num_splits)
+
+    def rotate_kv(self, min_bytes=512 << 20):
+        """Launches that read less than `min_bytes` of K and V take turns over as many copies of the cache as add up to
+        that much: back-to-back launches over one small cache would be served by the 256 MB last-level cache, not by
+        HBM, and a fraction of the HBM peak taken from them would mean nothing.  Returns the number of copies."""
+        B, Hq, Hkv, Sq, Skv, D = self.shape
+        kv_bytes = 2 * B * Hkv * Skv * D * (4 if self.dtype == capi.F32 else 2)
+        n = min(8, -(-min_bytes // kv_bytes))
+        for _ in range(n - len(self.descs)):
+            tk, tv = (host.DeviceTensor.from_f32(x, self.dtype) for x in self.host[1:])
+            self.more_kv += [tk, tv]
+            self.descs.append(host.make_desc(self.tq, tk, tv, self.to, impl=self.desc.impl, num_splits=self.desc.num_splits, **self._make_kw))
+        self.replan(self.desc.impl, self.desc.num_splits)
+        return len(self.descs)
 
     def replan(self, impl=capi.IMPL_AUTO, num_splits=0):
         """The same operands through another kernel or split count (generating and uploading gigabytes of cache again
         would cost more than the measurement)."""
         if self.ws is not None:
             self.ws.free()
-        self.desc.impl, self.desc.num_splits = impl, num_splits
-        self.desc.workspace, self.desc.workspace_bytes = None, 0
+        for d in self.descs:
+            d.impl, d.num_splits = impl, num_splits
+            d.workspace, d.workspace_bytes = None, 0
         nbytes, self.splits, self.impl = capi.sdpa_workspace(self.desc)
         self.ws = capi.DeviceBuffer(nbytes) if nbytes else None
         if self.ws is not None:
-            self.desc.workspace, self.desc.workspace_bytes = self.ws.ptr, self.ws.nbytes
+            for d in self.descs:                 # (launches follow each other on one stream: one workspace serves every copy)
+                d.workspace, d.workspace_bytes = self.ws.ptr, self.ws.nbytes
 
     def launch(self):
-        capi.sdpa_fwd(self.desc)
+        capi.sdpa_fwd(self.descs[self.turn])
+        self.turn = self.turn + 1 if self.turn + 1 < len(self.descs) else 0
 
     def ramp(self, seconds=0.15):
         """Setup, not measurement: keep the GPU busy until its clocks have settled (the first ~30 launches
@@ -151,7 +168,7 @@ class Workload:
         return float(np.abs(got - ref).max())
 
     def free(self):
-        for t in (self.tq.buf, self.tk.buf, self.tv.buf, self.to.buf, self.ws, self.tl):
+        for t in [self.tq.buf, self.tk.buf, self.tv.buf, self.to.buf, self.ws, self.tl] + [x.buf for x in self.more_kv]:
             if t is not None:
                 t.free()
 
@@ -241,6 +258,7 @@ def decode_gqa_leg(steps, warmup, only_shape=None):
         n = max(steps, min(200, int(0.02 / (kv_bytes / 6e12))))
         entry = {"workload": "%s decode B=%d Hq=%d Hkv=%d S_q=%d KV=%d D=128%s" % (dtypes.NAMES[dt], B, Hq, Hkv, Sq, Skv, " causal" if causal else "")}
         w = Workload("decode_" + name, SEED0 + 40 + i, B, Hq, Hkv, Sq, Skv, 128, dt, causal)
+        entry["kv_copies_in_rotation"] = w.rotate_kv()
         for impl in (capi.IMPL_AUTO, capi.IMPL_SPLITKV):
             if impl == capi.IMPL_SPLITKV and (Hq // Hkv) * Sq > 8:
                 continue
@@ -290,10 +308,13 @@ def head_dims_leg(steps, warmup):
                                                                  ("chunk_d256", 1, 32, 8, 256, 16384, 256, True),
                                                                  ("decode_d96", 32, 32, 8, 1, 8192, 96, False), ("decode_d256", 32, 32, 8, 1, 8192, 256, False))):
         w = Workload("head_dims_" + name, SEED0 + 80 + i, B, Hq, Hkv, Sq, Skv, D, capi.BF16, causal)
+        copies = w.rotate_kv() if Sq == 1 else 1
         wall, ev_mean, ev_med, ev_min = w.time(max(steps, 50), warmup)
         entry = {"workload": "bf16 %s B=%d Hq=%d Hkv=%d S_q=%d KV=%d D=%d" % ("decode" if Sq == 1 else "causal prefill" if Sq == Skv else "causal prefill chunk", B, Hq, Hkv, Sq, Skv, D),
                  "kernel": "sdpa_prefill_wide_kernel" if D > 128 and w.impl == capi.IMPL_MFMA else names.get(w.impl, str(w.impl)),
                  "num_splits": w.splits, "ms_per_step": wall, "parity_max_abs_err": w.parity(16)}
+        if Sq == 1:
+            entry["kv_copies_in_rotation"] = copies
         if Sq > 1:
             flops = causal_flops(B, Hq, Sq, Skv, D)
             entry["tflops"] = flops / (wall * 1e-3) / 1e12

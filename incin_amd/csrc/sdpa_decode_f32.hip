@@ -70,9 +70,9 @@ __global__ __launch_bounds__(256) void sdpa_decode_f32_kernel(SdpaParams p)
     const int nchunks = (R + CHUNK - 1) / CHUNK;
     const int split = blockIdx.x;
     int hkv, chunk_id;
-    decode_work_item(nchunks, &hkv, &chunk_id);
+    int b;
+    decode_work_item(nchunks, p.causal && p.G == 1, NSLOT == 2, &b, &hkv, &chunk_id);
     const int r0 = chunk_id * CHUNK;
-    const int b = blockIdx.z;
 
     int kv_len = Skv;
     if (p.kv_lens) kv_len = clampi(p.kv_lens[b], 0, Skv);
@@ -422,7 +422,10 @@ int decode_f32_chunk_rows(int R) { return R > 16 ? 32 : 16; }
 template <int D>
 static hipError_t launch_decode_f32_d(const SdpaParams& p, bool two_slots, hipStream_t stream)
 {
-    if (decode_f32_chunk_rows(p.G * p.Sq) == 32) return launch_decode_f32_t<D, DM_NSLOT, 2>(p, stream);
+    // 32 rows: always the two-slot rings, two workgroups per compute unit - one wavefront per SIMD leaves nothing to cover a
+    // wavefront's start-up, softmax and waits (measured against five slots on prefill and decode shapes alike: level to 1.3
+    // times ahead, config 2 of the benchmark 65 -> 51 us)
+    if (decode_f32_chunk_rows(p.G * p.Sq) == 32) return launch_decode_f32_t<D, 2, 2>(p, stream);
     return two_slots ? launch_decode_f32_t<D, 2, 1>(p, stream) : launch_decode_f32_t<D, DM_NSLOT, 1>(p, stream);
 }
 

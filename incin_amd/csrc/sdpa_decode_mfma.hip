@@ -61,9 +61,9 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
     const int nchunks = (R + CHUNK - 1) / CHUNK;
     const int split = blockIdx.x;
     int hkv, chunk_id;
-    decode_work_item(nchunks, &hkv, &chunk_id);
+    int b;
+    decode_work_item(nchunks, p.causal && p.G == 1, NSLOT == 2, &b, &hkv, &chunk_id);
     const int r0 = chunk_id * CHUNK;
-    const int b = blockIdx.z;
 
     int kv_len = Skv;
     if (p.kv_lens) kv_len = clampi(p.kv_lens[b], 0, Skv);
@@ -472,7 +472,7 @@ int decode_mfma_chunk_rows(int R, int dtype, int d_pad) { return dtype == 0 ? de
 int decode_mfma_workgroups_per_cu(int chunk_rows, int64_t split_len, int dtype, int d_pad)
 {
     if (d_pad > 128) return 1;
-    if (dtype == 0) return chunk_rows == 16 && 2 * split_len <= DM_SHORT_KEYS ? 2 : 1;
+    if (dtype == 0) return chunk_rows == 32 || 2 * split_len <= DM_SHORT_KEYS ? 2 : 1;      // (f32, 32 rows: always two-slot rings)
     return chunk_rows == 32 && split_len <= DM_SHORT_KEYS ? 2 : 1;
 }
 

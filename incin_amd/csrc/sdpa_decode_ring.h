@@ -29,22 +29,47 @@ __device__ __forceinline__ void dm_copy16(uint4v desc, unsigned lds_addr, int by
 template <int NSLOT, int CPB = 8> __device__ __forceinline__ void wait_oldest_copy()
 {
     constexpr int N = (NSLOT - 1) * CPB;
-    static_assert(N == 8 || N == 16 || N == 24 || N == 32, "s_waitcnt takes an immediate");
-    if (N == 32) asm volatile("s_waitcnt vmcnt(32)" ::: "memory");
-    else if (N == 24) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
-    else if (N == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    static_assert(N >= 1 && N <= 63, "s_waitcnt takes an immediate of 6 bits");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-// Which (KV head, chunk of rows) a workgroup of the split-KV matrix-core kernels takes, from blockIdx.y.  With several
-// chunks per KV head (prefill shapes through these kernels) the chunks of a head read the same keys and values: workgroups
-// reach the 8 XCDs round-robin in dispatch order, so an unsplit launch hands each XCD a contiguous eighth of the list
-// (a head's chunks then meet in one L2 instead of all eight), and the chunks of a head go last-first (under a causal
-// mask the last rows see the most keys: longest first).
-__device__ __forceinline__ void decode_work_item(int nchunks, int* hkv, int* chunk)
+// Which (batch entry, KV head, chunk of rows) a workgroup of the split-KV matrix-core kernels takes, from blockIdx.y and .z.
+// With several chunks per KV head (prefill shapes through these kernels) the chunks of a head read the same keys and
+// values: workgroups reach the 8 XCDs round-robin in dispatch order, so an unsplit launch hands each XCD a contiguous eighth
+// of the list (a head's chunks then meet in one L2 instead of all eight), and the chunks of a head go last-first (under a
+// causal mask the last rows see the most keys: longest first).
+// longest_first (a causal launch of one query head per KV head, keys not split): the order is by length over the whole
+// launch, not head by head - every (batch, head)'s last chunk, then every second-to-last, ... - because the workgroups that
+// start last decide when the launch ends, and they should be the short ones; an XCD still keeps an eighth of the heads to itself.
+// pairs: a compute unit holds two workgroups at a time, and the first two rounds of 32 per XCD all start at once - odd rounds
+// go in reverse, so that a compute unit's pair is a long one and a short one.
+__device__ __forceinline__ void decode_work_item(int nchunks, bool longest_first, bool pairs, int* b, int* hkv, int* chunk)
 {
     int y = blockIdx.y;
+    *b = blockIdx.z;
     if (nchunks > 1) {
+        if (longest_first && gridDim.x == 1) {
+            const int heads = (int)gridDim.y / nchunks, BH = (int)gridDim.z * heads;
+            const int id = (int)blockIdx.z * (int)gridDim.y + y;      // dispatch order
+            int bh, c;
+            if ((BH & 7) == 0) {
+                const int per = BH >> 3;
+                int i = id >> 3;
+                if (pairs && ((i >> 5) & 1)) {       // (the last round may be a partial one: reversed within what it has)
+                    const int first = i & ~31, len = min(32, (BH * nchunks >> 3) - first);
+                    i = first + (len - 1 - (i - first));
+                }
+                c = i / per;
+                bh = (id & 7) * per + i % per;
+            } else {
+                c = id / BH;
+                bh = id % BH;
+            }
+            *chunk = nchunks - 1 - c;
+            *b = bh / heads;
+            *hkv = bh % heads;
+            return;
+        }
         if (gridDim.x == 1 && (gridDim.y & 7) == 0) y = (y & 7) * (int)(gridDim.y >> 3) + (y >> 3);
         *hkv = y / nchunks;
         *chunk = nchunks - 1 - y % nchunks;
