@@ -32,18 +32,46 @@ SEED0 = 20261125
 PEAK_BF16_TFLOPS = 2516.6   # 256 CUs x 2.4 GHz x 4096 dense bf16 FLOP/clk/CU (vendor: 2.5 PFLOP/s)
 PEAK_F32_TFLOPS = 157.3      # dense fp32 matrix peak, vendor figure (256 CUs x 2.4 GHz x 256 FLOP/clk/CU)
 PEAK_HBM_GBS = 8000.0       # HBM3E, vendor figure
-# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this same command (KiB per dispatch,
-# FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0 after calibration against the 1 GiB copy kernel): profiles/*.txt
-PREFILL_TRAFFIC_BYTES = (273141 * 2.0 + 131084) * 1024     # 6.94e8: |Q|+|K|+|V| read 1.39 times, |O| written once
-DECODE_TRAFFIC_BYTES = (2097360 * 2.0 + 256) * 1024        # 4.2957e9: K and V read once, O written once
-PREFILL_LONG_TRAFFIC_BYTES = (534477 * 2.0 + 318950) * 1024    # 1.43e9: valid |O| written once, inputs read 2.2 times
-# These three are constants taken from counter runs, not measured by this script: each roofline object says so and
-# names the summary the figures come from.
-TRAFFIC_SOURCE = {
-    "prefill": "constant from profiles/sdpa_prefill_mfma_bf16_d128_config3.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of `bench.py --only prefill`)",
-    "decode": "constant from profiles/sdpa_decode_mfma_bf16_d128_config4.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of `bench.py --only decode`)",
-    "prefill_long": "constant from profiles/sdpa_prefill_mfma_bf16_d128_config5.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of `bench.py --only prefill_long --no-padding-compare`)",
+# HBM bytes per launch, from rocprofv3 --pmc runs of this same script, one leg (and where a leg has several shapes on one
+# kernel, one shape) at a time: `rocprofv3 --pmc FETCH_SIZE -- python3 bench.py --only LEG [--shape NAME] --steps 10
+# --warmup 2 --no-cpu-baseline`, then the same with WRITE_SIZE; KiB per dispatch, mean of the leg's last 20 dispatches of each
+# kernel, the kernels of one launch (main + combine, the backward's three) added up.  The counters are calibrated against
+# the 1 GiB copy kernel (`--only copy`: FETCH_SIZE 524294, WRITE_SIZE 1048580 KiB), hence FETCH_SIZE x 2.0, WRITE_SIZE x 1.0.
+# These are constants taken from counter runs, not measured by this script: each roofline object says so and names the
+# summary under profiles/ that records the run.
+TRAFFIC_KIB = {   # leg/shape/variant: (FETCH_SIZE, WRITE_SIZE)
+    "prefill": (263343, 131074),                           # 5.39e8 + 1.34e8: |O| written once, |Q|+|K|+|V| read 1.34 times
+    "decode": (2097380, 256.0),                            # 4.295e9: K and V read once
+    "decode/vector_alu": (2097460 + 616.5, 1088.2 + 256),
+    "prefill_long": (453220, 318928),                      # valid |O| written once, the inputs read 1.9 times
+    "decode_gqa/gqa4_b32_kv8192/auto": (524504, 256), "decode_gqa/gqa4_b32_kv8192/vector_alu": (525386 + 2152.5, 4352 + 256),
+    "decode_gqa/gqa4_b32_kv8192/bias": (524760, 256),
+    "decode_gqa/gqa4_b1_kv131072/auto": (262264 + 2120.5, 544 + 8), "decode_gqa/gqa4_b1_kv131072/vector_alu": (262250 + 2120.5, 4352.2 + 8),
+    "decode_gqa/gqa8_b32_kv8192/auto": (524632, 512), "decode_gqa/gqa8_b32_kv8192/vector_alu": (526452 + 4264.5, 8704 + 512),
+    "decode_gqa/gqa4_sq4_b8_kv8192/auto": (132176 + 2152.5, 4352.1 + 256),
+    "decode_gqa/f32_gqa4_b32_kv8192/auto": (1048910, 512), "decode_gqa/f32_gqa4_b32_kv8192/vector_alu": (1050700 + 2152, 4352 + 512),
+    "decode_gqa/f32_gqa8_sq4_b8_kv8192/auto": (266342 + 4264, 8704.3 + 1024),
+    "head_dims/prefill_d96": (109157, 62546.7), "head_dims/prefill_d256": (556912, 131083), "head_dims/chunk_d256": (119352, 4096),
+    "head_dims/decode_d96": (393400, 192), "head_dims/decode_d256": (1048960, 512),
+    "prefill_chunk/bf16_sq128_kv32768/auto": (66326.4 + 16680.5, 33392.9 + 1024), "prefill_chunk/bf16_sq128_kv32768/unsplit": (66199.5, 1024),
+    "prefill_chunk/bf16_sq512_kv32768/auto": (67708 + 17448.5, 33677.2 + 4096), "prefill_chunk/bf16_sq512_kv32768/unsplit": (67735.5, 4096),
+    "prefill_chunk/f32_sq128_kv32768/auto": (132204 + 16680, 33316.9 + 2048), "prefill_chunk/f32_sq128_kv32768/unsplit": (132192, 2048),
+    "f32/f32_c1": (187.2, 32), "f32/f32_c2": (12378.4, 8192), "f32/f32_large": (1523050, 262144),
+    "backward/bf16_d128": (133146 + 368971 + 264723, 4096 + 131072 + 262358),          # (row dots + dQ + dK/dV kernels)
+    "backward/bf16_d64": (135194 + 302550 + 266323, 8192 + 131072 + 262144),
+    "backward/f32_d64": (8735 + 16600 + 16607.5, 512 + 8192 + 16423.3), "backward/f32_d128": (270367 + 885089 + 932720, 8192 + 262144 + 524288),
 }
+TRAFFIC_PROFILE = "profiles/fetch_write_size_bench_legs.txt"
+
+
+def traffic_of(key):
+    """(HBM bytes per launch, where the figure comes from) for one leg / shape / variant of the table above."""
+    if key not in TRAFFIC_KIB:
+        return None, None
+    fetch, write = TRAFFIC_KIB[key]
+    return (fetch * 2.0 + write) * 1024.0, "constant from %s (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of `bench.py --only %s`)" % (TRAFFIC_PROFILE, key.split("/")[0])
+
+
 METRIC = "attn fwd TFLOP/s + % bf16 MFMA peak; decode KV GB/s + % HBM peak (1 GPU)"
 
 
@@ -210,13 +238,15 @@ def cpu_baseline_decode(D, Skv, B, H, dtype):
     return 2.0 * B * H * Skv * D * 2 / dt / 1e9, dt
 
 
-def prefill_chunk_leg(steps, warmup):
+def prefill_chunk_leg(steps, warmup, only_shape=None):
     """A chunk of a long prompt: few query rows (one sequence, 128 or 512 new positions) over a long cache, causal.  The
     launch has 32 or 128 (head, row block) items for 256 compute units, so the library splits the key axis and combines
     the partial results; beside it the same launch unsplit (num_splits = 1)."""
     out = {}
     for i, (dt, Sq, Skv) in enumerate(((capi.BF16, 128, 32768), (capi.BF16, 512, 32768), (capi.F32, 128, 32768))):
         B, Hq, Hkv, D = 1, 32, 8, 128
+        if only_shape is not None and only_shape != "%s_sq%d_kv%d" % (dtypes.NAMES[dt], Sq, Skv):
+            continue
         flops = 4.0 * D * Hq * B * (Sq * Skv - Sq * (Sq - 1) / 2.0)
         peak = PEAK_F32_TFLOPS if dt == capi.F32 else PEAK_BF16_TFLOPS
         kernel = "sdpa_prefill_f32_kernel<128>" if dt == capi.F32 else "sdpa_prefill_mfma_kernel<bf16,128>"
@@ -226,7 +256,8 @@ def prefill_chunk_leg(steps, warmup):
             wall, ev_mean, ev_med, ev_min = w.time(max(steps, 100) if dt != capi.F32 else 20, warmup if dt != capi.F32 else 3)
             entry[name] = {"num_splits": w.splits, "ms_per_step": wall, "tflops": flops / (wall * 1e-3) / 1e12,
                            "roofline": {"bound": "mfma", "achieved": flops / (ev_mean * 1e-3) / 1e12, "peak": peak, "unit": "TFLOP/s",
-                                        "frac": flops / (ev_mean * 1e-3) / 1e12 / peak, "traffic": None,
+                                        "frac": flops / (ev_mean * 1e-3) / 1e12 / peak,
+                                        "traffic": traffic_of("prefill_chunk/%s_sq%d_kv%d/%s" % (dtypes.NAMES[dt], Sq, Skv, name))[0], "traffic_source": TRAFFIC_PROFILE,
                                         "kernel": kernel + (" over splits of the keys + sdpa_combine_kernel" if w.splits > 1 else ""),
                                         "algorithmic_flops_per_launch": flops, "launch_ms_mean": ev_mean, "launch_ms_min": ev_min},
                            "parity_max_abs_err": w.parity(16)}
@@ -269,7 +300,8 @@ def decode_gqa_leg(steps, warmup, only_shape=None):
                 "kernel": (names_f32 if dt == F else names).get(w.impl, str(w.impl)), "num_splits": w.splits, "ms_per_step": wall,
                 "kv_gb_per_s": kv_bytes / (wall * 1e-3) / 1e9,
                 "roofline": {"bound": "hbm", "achieved": kv_bytes / (ev_mean * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                             "frac": kv_bytes / (ev_mean * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None,
+                             "frac": kv_bytes / (ev_mean * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                             "traffic": traffic_of("decode_gqa/%s/%s" % (name, "auto" if impl == capi.IMPL_AUTO else "vector_alu"))[0], "traffic_source": TRAFFIC_PROFILE,
                              "algorithmic_bytes_per_launch": kv_bytes, "launch_ms_mean": ev_mean, "launch_ms_min": ev_min},
                 "parity_max_abs_err": w.parity(16)}
         if name == "gqa4_b32_kv8192" and only_shape is None:
@@ -290,6 +322,7 @@ def decode_gqa_leg(steps, warmup, only_shape=None):
             err = float(np.abs(w.to.to_f32().reshape(B * Hq, Sq, 128)[rows[:, 0], rows[:, 1]] - ref).max())
             entry["with_bias_mask_tensor"] = {"kernel": names.get(w.impl, str(w.impl)), "num_splits": w.splits, "ms_per_step": wall_b,
                                               "kv_gb_per_s": kv_bytes / (wall_b * 1e-3) / 1e9, "frac": kv_bytes / (ev_b * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                                              "traffic": traffic_of("decode_gqa/%s/bias" % name)[0], "traffic_source": TRAFFIC_PROFILE,
                                               "parity_max_abs_err": err}
             tm.free()
         w.free()
@@ -297,7 +330,7 @@ def decode_gqa_leg(steps, warmup, only_shape=None):
     return out
 
 
-def head_dims_leg(steps, warmup):
+def head_dims_leg(steps, warmup, only_shape=None):
     """Head dimensions other than 64 and 128 (bf16): D = 96 runs zero-padded in the 128 instances of the prefill and split-KV
     kernels, D = 256 in the prefill kernel for 256 and in the 256 instance of the split-KV kernel (decode, and a 256-row chunk of a
     16384-token prompt: too few 128-row blocks for the prefill kernel, which does not split the keys).  Prefill: useful FLOPs (4 D per visible
@@ -307,6 +340,8 @@ def head_dims_leg(steps, warmup):
     for i, (name, B, Hq, Hkv, Sq, Skv, D, causal) in enumerate((("prefill_d96", 8, 16, 16, 2048, 2048, 96, True), ("prefill_d256", 4, 16, 16, 4096, 4096, 256, True),
                                                                  ("chunk_d256", 1, 32, 8, 256, 16384, 256, True),
                                                                  ("decode_d96", 32, 32, 8, 1, 8192, 96, False), ("decode_d256", 32, 32, 8, 1, 8192, 256, False))):
+        if only_shape is not None and name != only_shape:
+            continue
         w = Workload("head_dims_" + name, SEED0 + 80 + i, B, Hq, Hkv, Sq, Skv, D, capi.BF16, causal)
         copies = w.rotate_kv() if Sq == 1 else 1
         wall, ev_mean, ev_med, ev_min = w.time(max(steps, 50), warmup)
@@ -319,13 +354,15 @@ def head_dims_leg(steps, warmup):
             flops = causal_flops(B, Hq, Sq, Skv, D)
             entry["tflops"] = flops / (wall * 1e-3) / 1e12
             entry["roofline"] = {"bound": "mfma", "achieved": flops / (ev_mean * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                                 "frac": flops / (ev_mean * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": None,
+                                 "frac": flops / (ev_mean * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+                                 "traffic": traffic_of("head_dims/" + name)[0], "traffic_source": TRAFFIC_PROFILE,
                                  "algorithmic_flops_per_launch": flops, "launch_ms_mean": ev_mean, "launch_ms_min": ev_min}
         else:
             kv_bytes = 2.0 * B * Hkv * Skv * D * 2
             entry["kv_gb_per_s"] = kv_bytes / (wall * 1e-3) / 1e9
             entry["roofline"] = {"bound": "hbm", "achieved": kv_bytes / (ev_mean * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                 "frac": kv_bytes / (ev_mean * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None,
+                                 "frac": kv_bytes / (ev_mean * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                                 "traffic": traffic_of("head_dims/" + name)[0], "traffic_source": TRAFFIC_PROFILE,
                                  "algorithmic_bytes_per_launch": kv_bytes, "launch_ms_mean": ev_mean, "launch_ms_min": ev_min}
         w.free()
         out[name] = entry
@@ -413,6 +450,7 @@ def backward_leg(steps, warmup, dtype=capi.BF16, B=8, H=16, S=4096, D=128, what=
             "step": "one incin_rocm_sdpa_bwd call (3 kernels: row dots, dQ, dK/dV)", "dtype": name,
             "metric": "attn bwd TFLOP/s (2.5 x forward FLOPs)", "value": flops / (wall * 1e-3) / 1e12, "unit": "TFLOP/s",
             "ms_per_step": wall, "steps": steps, "frac_of_%s_mfma_peak" % ("fp32" if dtype == capi.F32 else "bf16"): flops / (wall * 1e-3) / 1e12 / peak,
+            "traffic": traffic_of("backward/%s_d%d" % (name, D))[0], "traffic_source": TRAFFIC_PROFILE,
             "parity_max_err_rel_to_max_abs_ref": err,
             "parity_sample": "dQ, dK, dV of slice (b=%d, h=%d) against the float64 oracle of the reference's tape gradients" % (b, h)}
 
@@ -532,7 +570,8 @@ def f32_configs(steps, warmup, with_cpu, threads):
                "metric": "attn fwd TFLOP/s", "value": flops / (wall * 1e-3) / 1e12, "unit": "TFLOP/s", "dtype": "f32",
                "ms_per_step": wall, "steps": n,
                "roofline": {"bound": "mfma", "achieved": flops / (ev_mean * 1e-3) / 1e12, "peak": PEAK_F32_TFLOPS, "unit": "TFLOP/s",
-                            "frac": flops / (ev_mean * 1e-3) / 1e12 / PEAK_F32_TFLOPS, "traffic": None, "kernel": kernel,
+                            "frac": flops / (ev_mean * 1e-3) / 1e12 / PEAK_F32_TFLOPS,
+                            "traffic": traffic_of("f32/" + key)[0], "traffic_source": TRAFFIC_PROFILE, "kernel": kernel,
                             "algorithmic_flops_per_launch": flops, "launch_ms_mean": ev_mean, "launch_ms_median": ev_med,
                             "launch_ms_min": ev_min},
                "parity_max_abs_err": w.parity()}
@@ -649,7 +688,8 @@ def main():
     ap.add_argument("--no-padding-compare", action="store_true",
                     help="prefill_long: skip the extra timing of the batch with its padding rows computed (profiling: every "
                          "launch of the run is then the same launch)")
-    ap.add_argument("--decode-gqa-shape", default=None, help="with --only decode_gqa: one of its shapes by name (for profiles)")
+    ap.add_argument("--shape", "--decode-gqa-shape", dest="shape", default=None,
+                    help="with --only decode_gqa, head_dims or prefill_chunk: one of the leg's shapes by name (for profiles)")
     ap.add_argument("--only", choices=["prefill", "prefill_long", "prefill_chunk", "decode", "decode_gqa", "head_dims", "backward", "f32", "copy", "matrix_rate", "read_rate"], default=None,
                     help="run a single workload (profiling). 'copy' runs --steps device-to-device copies of 1 GiB "
                          "through the library's plain copy kernel: the known-size dispatch that hardware byte "
@@ -699,8 +739,8 @@ def main():
         result["value"] = flops / (wall * 1e-3) / 1e12
         result["ms_per_step"] = wall
         result["roofline"] = {"bound": "mfma", "achieved": flops / (ev_mean * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS,
-                              "unit": "TFLOP/s", "frac": flops / (ev_mean * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": PREFILL_TRAFFIC_BYTES,
-                              "traffic_source": TRAFFIC_SOURCE["prefill"], "kernel": "sdpa_prefill_mfma_kernel<bf16,128>", "algorithmic_flops_per_launch": flops,
+                              "unit": "TFLOP/s", "frac": flops / (ev_mean * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": traffic_of("prefill")[0],
+                              "traffic_source": traffic_of("prefill")[1], "kernel": "sdpa_prefill_mfma_kernel<bf16,128>", "algorithmic_flops_per_launch": flops,
                               "launch_ms_mean": ev_mean, "launch_ms_median": ev_med, "launch_ms_min": ev_min}
         result["parity_max_abs_err"] = w.parity()
         if args.only is None:
@@ -755,8 +795,8 @@ def main():
                         "each length only" % lens.tolist(),
             "metric": "attn fwd TFLOP/s", "value": flops / (wall * 1e-3) / 1e12, "unit": "TFLOP/s", "ms_per_step": wall, "steps": steps,
             "roofline": {"bound": "mfma", "achieved": flops / (ev_mean * 1e-3) / 1e12, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                         "frac": flops / (ev_mean * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": PREFILL_LONG_TRAFFIC_BYTES,
-                         "traffic_source": TRAFFIC_SOURCE["prefill_long"], "kernel": kernel,
+                         "frac": flops / (ev_mean * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, "traffic": traffic_of("prefill_long")[0],
+                         "traffic_source": traffic_of("prefill_long")[1], "kernel": kernel,
                          "algorithmic_flops_per_launch": flops, "launch_ms_mean": ev_mean, "launch_ms_median": ev_med,
                          "launch_ms_min": ev_min},
             "ms_per_step_with_padding_rows_computed": wall_all_rows,
@@ -773,8 +813,8 @@ def main():
                "metric": "decode KV GB/s", "value": kv_bytes / (wall * 1e-3) / 1e9, "unit": "GB/s", "ms_per_step": wall,
                "num_splits": w.splits,
                "roofline": {"bound": "hbm", "achieved": kv_bytes / (ev_mean * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                            "frac": kv_bytes / (ev_mean * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": DECODE_TRAFFIC_BYTES,
-                            "traffic_source": TRAFFIC_SOURCE["decode"],
+                            "frac": kv_bytes / (ev_mean * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": traffic_of("decode")[0],
+                            "traffic_source": traffic_of("decode")[1],
                             "kernel": {capi.IMPL_SPLITKV: "sdpa_decode_split_kernel<bf16,128,1,8> + sdpa_combine_kernel",
                                        capi.IMPL_SPLITKV_MFMA: "sdpa_decode_mfma_kernel<bf16,5,1>"}.get(w.impl, str(w.impl)),
                             "algorithmic_bytes_per_launch": kv_bytes,
@@ -785,6 +825,7 @@ def main():
         wall_v, ev_v, _, _ = w.time(args.steps, args.warmup)
         dec["vector_alu_kernel"] = {"kernel": "sdpa_decode_split_kernel<bf16,128,1,8> + sdpa_combine_kernel", "num_splits": w.splits,
                                     "ms_per_step": wall_v, "launch_ms_mean": ev_v, "frac": kv_bytes / (ev_v * 1e-3) / 1e9 / PEAK_HBM_GBS,
+                                    "traffic": traffic_of("decode/vector_alu")[0], "traffic_source": TRAFFIC_PROFILE,
                                     "parity_max_abs_err": w.parity()}
         # (last: the appended rows overwrite the end of the cache)
         w.replan()
@@ -799,15 +840,15 @@ def main():
 
     if args.only in (None, "prefill_chunk"):
         note("prefill_chunk")
-        result["prefill_chunk"] = prefill_chunk_leg(args.steps, args.warmup)
+        result["prefill_chunk"] = prefill_chunk_leg(args.steps, args.warmup, args.shape)
 
     if args.only in (None, "decode_gqa"):
         note("decode_gqa")
-        result["decode_gqa"] = decode_gqa_leg(args.steps, args.warmup, args.decode_gqa_shape)
+        result["decode_gqa"] = decode_gqa_leg(args.steps, args.warmup, args.shape)
 
     if args.only in (None, "head_dims"):
         note("head_dims")
-        result["head_dims"] = head_dims_leg(args.steps, args.warmup)
+        result["head_dims"] = head_dims_leg(args.steps, args.warmup, args.shape)
 
     if args.only in (None, "f32"):
         note("f32")
