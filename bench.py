@@ -51,7 +51,7 @@ TRAFFIC_KIB = {   # leg/shape/variant: (FETCH_SIZE, WRITE_SIZE)
     "decode_gqa/gqa4_sq4_b8_kv8192/auto": (132176 + 2152.5, 4352.1 + 256),
     "decode_gqa/f32_gqa4_b32_kv8192/auto": (1048910, 512), "decode_gqa/f32_gqa4_b32_kv8192/vector_alu": (1050700 + 2152, 4352 + 512),
     "decode_gqa/f32_gqa8_sq4_b8_kv8192/auto": (266342 + 4264, 8704.3 + 1024),
-    "head_dims/prefill_d96": (109157, 62546.7), "head_dims/prefill_d256": (556912, 131083), "head_dims/chunk_d256": (119352, 4096),
+    "head_dims/prefill_d96": (109157, 62546.7), "head_dims/prefill_d256": (556912, 131083), "head_dims/chunk_d256": (68960.5 + 33320.5, 67438.4 + 4096),
     "head_dims/decode_d96": (393400, 192), "head_dims/decode_d256": (1048960, 512),
     "prefill_chunk/bf16_sq128_kv32768/auto": (66326.4 + 16680.5, 33392.9 + 1024), "prefill_chunk/bf16_sq128_kv32768/unsplit": (66199.5, 1024),
     "prefill_chunk/bf16_sq512_kv32768/auto": (67708 + 17448.5, 33677.2 + 4096), "prefill_chunk/bf16_sq512_kv32768/unsplit": (67735.5, 4096),
@@ -66,7 +66,7 @@ TRAFFIC_PROFILE = "profiles/fetch_write_size_bench_legs.txt"
 
 def traffic_of(key):
     """(HBM bytes per launch, where the figure comes from) for one leg / shape / variant of the table above."""
-    if key not in TRAFFIC_KIB:
+    if TRAFFIC_KIB.get(key) is None:
         return None, None
     fetch, write = TRAFFIC_KIB[key]
     return (fetch * 2.0 + write) * 1024.0, "constant from %s (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of `bench.py --only %s`)" % (TRAFFIC_PROFILE, key.split("/")[0])

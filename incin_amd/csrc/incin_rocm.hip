@@ -234,29 +234,41 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         const int64_t wgs_w = d->B * d->Hq * ((d->Sq + 127) / 128), chunks_w = d->B * d->Hkv * ((R + 31) / 32);
         const bool wide_underfilled = (wgs_w * 4 <= cus_w && (d->Skv >= 2048 || chunks_w * 2 <= cus_w || chunks_w % cus_w == 0)) ||
                                       (wgs_w * 2 <= cus_w && chunks_w % cus_w == 0);
+        // The prefill kernel for 256 splits the keys like the one for 128 (a launch of at most one workgroup per compute unit over
+        // 4096 keys or more, four times the rows: see below); where those splits give every compute unit a workgroup it is well
+        // ahead of the split-KV kernel's 32 rows per pass over K and V (32 / 8 heads x 256 x 16384 0.257 -> 0.153 ms; 8 / 2 heads x
+        // 1024 x 32768 0.57 -> 0.27; 64 / 8 heads x 128 x 32768 0.59 -> 0.29; 16 heads x 1024 x 4096 0.138 -> 0.096), and behind
+        // where they do not (8 heads x 128 x 8192: 64 workgroups, 0.053 against 0.036).
+        const int64_t wide_splits = (wgs_w <= cus_w && d->Skv >= 4096 && d->Skv >= 4 * d->Sq && !d->q_lens && d->num_splits == 0)
+                                        ? std::min<int64_t>(2 * cus_w / wgs_w, d->Skv / 1024) : (d->num_splits > 1 ? d->num_splits : 1);
+        const bool wide_split_fills = wide_splits > 1 && wgs_w * wide_splits >= cus_w && !d->add_mask && d->dtype != INCIN_ROCM_F32;
         // (with a dense mask the prefill kernel keeps launches of more than 64 positions: its block flags skip what the mask hides)
-        if (wide && mfma_ok && d->Sq > 64 && !(split_mfma_ok && wide_underfilled && !d->add_mask)) impl = INCIN_ROCM_IMPL_MFMA;
+        if (wide && mfma_ok && d->Sq > 64 && (wide_split_fills || !(split_mfma_ok && wide_underfilled && !d->add_mask))) impl = INCIN_ROCM_IMPL_MFMA;
         else if (wide && split_mfma_ok) impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
         // f32 (sdpa_decode_f32.hip): from two rows per KV head on, whatever the count - the f32 prefill kernel would spend a
         // 32-row matrix instruction on every query head's few rows (32 heads of a group at one position each: 8.4 ms
         // against 0.23), and where it packs as well (64 positions of one head) the split-KV form is still ahead (0.22
         // against 0.28 ms on 8 x 8 heads x 8192 keys); the vector-ALU kernel is level at 2 rows and behind from 4 on
-        // (4 rows, 268 MB of cache: 5.6 against 4.8 TB/s; 8 rows: 6.6 against 3.4).  More than 32 rows over fewer than 512
-        // keys stay with the prefill kernel (64 positions x 16 heads x 64 sequences of 256 keys: 0.14 against 0.17 ms).
+        // (4 rows, 268 MB of cache: 5.6 against 4.8 TB/s; 8 rows: 6.6 against 3.4).  That holds over short caches too since the
+        // 32-row form runs two workgroups per compute unit (48 positions x 16 heads x 16 sequences of 300 keys: 0.020 against
+        // the prefill kernel's 0.030 ms).
         // One row per KV head (swept over 1 - 32 sequences x 8 - 32 heads x 512 - 16384 keys): the matrix-core kernel is level
         // from 500 MB of cache on and up to 2.8 times ahead below (its splits fill the device where the vector-ALU kernel's
         // do not), except over the shortest caches at D = 64 (512 keys: 1.1 - 1.4 times behind).
         else if (d->dtype == INCIN_ROCM_F32 && split_mfma_ok && d->Sq <= 64 && len128 >= 256 &&
-                 (R >= 2 ? (R <= 32 || d->Skv >= 512) : d->Skv >= (d_pad == 64 ? 1024 : 512)))
+                 (R >= 2 || d->Skv >= (d_pad == 64 ? 1024 : 512)))
             impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
-        // f32 prefill launches that give the prefill kernel at most one 128-row workgroup per compute unit: the split-KV kernel
+        // f32 prefill launches that give the prefill kernel at most two 128-row workgroups per compute unit (one round of what a
+        // compute unit holds; since the 32-row form runs two workgroups per compute unit, longest chunks first: 2 x 16 heads x
+        // 2048 x 2048 at D = 128, 512 workgroups' worth, 0.384 -> 0.316 ms; 4 x 16 x 1024 x 1024 0.197 -> 0.180; level at 640
+        // workgroups' worth at D = 64; the prefill kernel 1.1 - 1.3 times ahead from 1024 on): the split-KV kernel
         // takes them 32 rows per workgroup with the keys dealt to its four wavefronts - four times the workgroups, a quarter
         // of the keys per wavefront - where the prefill kernel's wavefronts each walk all keys for their 32 rows behind
         // 64-cycle matrix instructions (measured, causal: one head of 128 x 128 13.3 -> 8.6 us; 2 x 8 heads x 512 x 512 at
         // D = 128 73 -> 28; 128 workgroups' worth of 1024 x 1024 80 -> 33; 256 - 4 x 8 heads x 1024 x 1024 at D = 64 - 80 -> 65; level at 512).
         // Not the chunks of a long prompt, where the prefill kernel splits the keys itself (below) and runs at 80 % of the peak.
         else if (d->dtype == INCIN_ROCM_F32 && split_mfma_ok && d->Sq > 64 && !(d->Skv >= 4096 && d->Skv >= 4 * d->Sq) &&
-                 d->B * d->Hq * ((d->Sq + 127) / 128) <= compute_units_of(d->device))
+                 d->B * d->Hq * ((d->Sq + 127) / 128) <= 2 * compute_units_of(d->device))
             impl = INCIN_ROCM_IMPL_SPLITKV_MFMA;
         // f16 / bf16 (sdpa_decode_mfma.hip): the thresholds described above
         else if (d->dtype != INCIN_ROCM_F32 && split_mfma_ok && len128 >= 256 &&
@@ -344,7 +356,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         plan->split_len = (int)split_len;
         plan->ws_bytes = splits > 1 ? (size_t)(d->B * d->Hq * d->Sq * splits) * (size_t)(d_pad + 2) * sizeof(float) : 0;
     }
-    if (impl == INCIN_ROCM_IMPL_MFMA && !d->add_mask && !d->q_lens && !wide) {
+    if (impl == INCIN_ROCM_IMPL_MFMA && !d->add_mask && !d->q_lens && !(wide && d->dtype == INCIN_ROCM_F32)) {
         // The prefill kernels (16-bit and f32) run one workgroup per (batch, query head, 128 rows) and a compute unit holds two:
         // when a launch has at most one per compute unit and a long key axis - a chunk of a long prompt, a single
         // sequence - the keys are split as for decode, as many ways as fill the device (1024 keys per split at least:

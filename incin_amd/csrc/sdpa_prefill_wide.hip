@@ -28,7 +28,11 @@ constexpr int PW_KT = 32;      // keys per tile
 // DENSE: a dense additive mask (any broadcast strides) comes with one flag per block of 32 rows x 32 keys (mask_blocks.hip) -
 // a tile of this kernel is one such block per wavefront: tiles where the mask is zero run without it, the others add its
 // values to the scores, and the tiles before the first and after the last one it shows to a wavefront are skipped.
-template <typename T, bool DENSE>
+//
+// SPLIT: a grid of (work items) x (splits of the key axis), as in sdpa_prefill_mfma.hip - a workgroup handles the keys of its
+// split and writes, per row, the unnormalised O, the reference and the sum in the split-KV kernels' partial-result format; their
+// combine kernel finishes.  For launches with few 128-row blocks over a long key axis (a chunk of a long prompt).
+template <typename T, bool DENSE, bool SPLIT = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void sdpa_prefill_wide_kernel(SdpaParams p)
 {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -61,6 +65,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
     int kv_len = Skv;
     if (p.kv_lens) kv_len = clampi(p.kv_lens[b], 0, Skv);
+    // a split ends where the next begins: to this workgroup the keys beyond do not exist (split_len is a multiple of the tile)
+    const int split = SPLIT ? (int)blockIdx.y : 0;
+    if (SPLIT) kv_len = min(kv_len, (split + 1) * p.split_len);
     const int rows_b = p.q_lens ? clampi(p.q_lens[b], 0, Sq) : Sq;      // query rows at and beyond are padding
     if (q0 >= rows_b) return;                                           // (uniform: before any barrier)
     const int coff = Skv - Sq;
@@ -77,7 +84,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     if (q0 + wave * 32 >= rows_b) lim_wave_min = lim_wave_max = 0;      // a wavefront of padding rows only keeps the barriers company
     int n_tiles = (j_end + PW_KT - 1) / PW_KT;
     int n_act = lim_wave_max > 0 ? (lim_wave_max + PW_KT - 1) / PW_KT : 0;      // tiles this wavefront computes: [w_first, n_act)
-    int w_first = 0, t_first = 0;
+    int w_first = 0, t_first = SPLIT ? min(split * (p.split_len / PW_KT), n_tiles) : 0;
     // dense mask: this lane's row of it and the flags of this wavefront's 32 rows, one per tile.  The tiles before the first
     // and after the last one the mask shows to a wavefront are not computed (a sliding window's past), and the workgroup's
     // copies run from the first to the last tile any of its wavefronts computes; a hidden tile in between goes through the
@@ -285,6 +292,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
     // ---- normalise and store --------------------------------------------------------------------------------------
     const float l_tot = xor32_sum(l_run);
+    if constexpr (SPLIT) {
+        // partial result of this split: unnormalised O, and (reference, sum) in the log2 units the combine kernel takes for 16-bit
+        // storage; a row that saw no key in this split says so with a reference of -inf
+        if (my_i < rows_b) {
+            const int64_t slot = (((int64_t)b * p.Hq + hq) * Sq + my_i) * p.num_splits + split;
+            float* arow = p.ws_acc + slot * D + g * 4;
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    typedef float f4 __attribute__((ext_vector_type(4)));
+                    f4 w = {o_acc[db][r4 * 4], o_acc[db][r4 * 4 + 1], o_acc[db][r4 * 4 + 2], o_acc[db][r4 * 4 + 3]};
+                    *(f4*)(arow + db * 32 + r4 * 8) = w;
+                }
+            if (g == 0) {
+                p.ws_ml[slot * 2 + 0] = l_tot == 0.0f ? -INFINITY : m_run;
+                p.ws_ml[slot * 2 + 1] = l_tot;
+            }
+        }
+        return;
+    }
     const float inv = (l_tot == 0.0f) ? __builtin_nanf("") : 1.0f / l_tot;      // no visible key: NaN, as the reference
     if (my_i < rows_b && p.lse && g == 0)       // m_run and the sum are in log2 units of the scaled scores
         p.lse[((int64_t)b * p.Hq + hq) * Sq + my_i] = l_tot == 0.0f ? -INFINITY : (m_run + __builtin_log2f(l_tot)) * 0.6931471805599453f;
@@ -297,6 +325,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // Host has validated: dtype f16 / bf16, 128 < max(D, Dv) <= 256 in whole 16-byte vectors, finite scale; with a dense mask its
 // block flags have been written (launch_mask_classify);
 // rows 16-byte aligned with unit last-dim stride, row strides below 2^24 elements.
+hipError_t launch_sdpa_combine(const SdpaParams& p, int dtype, hipStream_t stream);
+
 hipError_t launch_sdpa_prefill_wide(const SdpaParams& p0, int dtype, hipStream_t stream)
 {
     SdpaParams p = p0;
@@ -307,6 +337,13 @@ hipError_t launch_sdpa_prefill_wide(const SdpaParams& p0, int dtype, hipStream_t
     // two workgroups per compute unit, an eighth of the compute units per XCD
     p.interleave = work_interleave(p.causal != 0, 2 * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
     p.deal_groups = (total & 7) == 0 ? work_deal(p.interleave, p.G, nqb, total >> 3) : 0;
+    if (!p.mask && p.num_splits > 1) {       // split launch: partial results, then the split-KV kernels' combine pass
+        const dim3 grid((unsigned)total, (unsigned)p.num_splits);
+        if (dtype == 1) hipLaunchKernelGGL((sdpa_prefill_wide_kernel<f16_t, false, true>), grid, dim3(256), 0, stream, p);
+        else hipLaunchKernelGGL((sdpa_prefill_wide_kernel<bf16_t, false, true>), grid, dim3(256), 0, stream, p);
+        hipError_t e = hipGetLastError();
+        return e != hipSuccess ? e : launch_sdpa_combine(p, dtype, stream);
+    }
     if (p.mask) {
         if (dtype == 1) hipLaunchKernelGGL((sdpa_prefill_wide_kernel<f16_t, true>), dim3((unsigned)total), dim3(256), 0, stream, p);
         else hipLaunchKernelGGL((sdpa_prefill_wide_kernel<bf16_t, true>), dim3((unsigned)total), dim3(256), 0, stream, p);

@@ -395,11 +395,15 @@ def test_row_normalisers_from_split_launches(gpu, case):
     (2, 2, 1, 77, 9000, 128, True, [9000, 4100]),   # the second sequence ends inside a split
     (1, 6, 3, 200, 4500, 64, True, None),           # head dimension 64
     (1, 2, 2, 130, 4096, 128, True, [300]),         # most splits see no key at all
+    (1, 4, 2, 200, 4500, 256, True, None),          # the prefill kernel for head dimensions above 128 (16-bit)
+    (2, 2, 2, 130, 4200, 160, True, [4200, 1000]),
 ])
 def test_prefill_with_the_keys_split(gpu, dtype, shape):
     """The matrix-core prefill kernels (16-bit and f32) over splits of the key axis + combine (what AUTO does for launches with few row blocks
     over many keys): against the oracle with the library's split count and forced ones, and against the unsplit launch."""
     B, Hq, Hkv, Sq, Skv, D, causal, lens = shape
+    if D > 128 and dtype == capi.F32:
+        pytest.skip("f32 has no prefill kernel above 128 (the split-KV kernel's 256 instance takes those launches)")
     q, k, v = inputs(1200 + Sq + Skv, B, Hq, Hkv, Sq, Skv, D, D, dtype)
     lens = None if lens is None else np.asarray(lens, np.int32)
     ref = oracle_full(q, k, v, G=Hq // Hkv, causal=causal, kv_lens=lens)
@@ -411,8 +415,27 @@ def test_prefill_with_the_keys_split(gpu, dtype, shape):
         assert info["impl"] == capi.IMPL_MFMA and info["splits"] > 1 and info["workspace_bytes"] > 0
         check(got, ref, TOL[dtype], "prefill, keys split %d ways" % info["splits"])
         check(got, whole, 8e-3 if dtype != capi.F32 else 2e-6, "split vs whole")
+    if D > 128:        # (AUTO keeps launches this small on the split-KV kernel: the test below)
+        return
     got, info = host.sdpa(q, k, v, dtype, causal=causal, kv_lens=lens, return_info=True)      # AUTO comes to the same launch
     assert info["impl"] == capi.IMPL_MFMA and info["splits"] > 1
+
+
+def test_auto_splits_the_keys_of_a_wide_prefill_launch_that_fills_the_device(gpu):
+    """Head dimensions above 128: a chunk of a long prompt goes to the prefill kernel with its keys split when the splits
+    give every compute unit a workgroup (64 row blocks x 8 splits here), and stays on the split-KV kernel when they do not
+    (8 row blocks).  Both against the split-KV kernel pinned (itself against the oracle in test_head_dimensions_above_128)."""
+    for Hq, Hkv, Sq, Skv, want in ((32, 8, 256, 16384, capi.IMPL_MFMA), (8, 8, 128, 8192, capi.IMPL_SPLITKV_MFMA)):
+        q, k, v = inputs(1300 + Hq, 1, Hq, Hkv, Sq, Skv, 256, 256, capi.BF16)
+        got, info = host.sdpa(q, k, v, capi.BF16, causal=True, return_info=True)
+        assert info["impl"] == want, info
+        if want == capi.IMPL_MFMA:
+            assert info["splits"] > 1 and info["workspace_bytes"] > 0
+        other = host.sdpa(q, k, v, capi.BF16, causal=True, impl=capi.IMPL_SPLITKV_MFMA)
+        check(got, other, 8e-3, "prefill kernel for 256 with split keys against the split-KV kernel")
+        rows = np.array([[0, 0], [Hq - 1, Sq - 1], [Hq // 2, Sq // 2], [1, 31]])
+        ref = O.sdpa_rows(q.reshape(1, Hkv, Hq // Hkv, Sq, 256), k[:, :, None], v[:, :, None], rows, causal=True)
+        assert np.abs(got.reshape(Hq, Sq, 256)[rows[:, 0], rows[:, 1]] - ref).max() <= TOL[capi.BF16]
 
 
 # ---- split-KV decode -----------------------------------------------------------------------------

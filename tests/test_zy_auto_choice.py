@@ -41,6 +41,9 @@ SHAPES = [
     ("f32_prefill_mid", F32, 4, 16, 16, 1280, 1280, 64, True),
     ("f32_prefill_d128", F32, 2, 16, 16, 2048, 2048, 128, True),
     ("f32_short_cache", F32, 16, 16, 16, 48, 300, 64, True),
+    ("f32_short_cache_64", F32, 64, 16, 16, 64, 256, 64, True),
+    ("f32_prefill_512_blocks", F32, 4, 16, 16, 1024, 1024, 128, True),
+    ("d256_chunk", BF, 1, 32, 8, 256, 16384, 256, True),
 ]
 
 
