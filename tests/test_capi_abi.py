@@ -56,11 +56,13 @@ def _plan(d):
 
 def test_dispatch_choices():
     assert _plan(_desc())[2] == capi.IMPL_MFMA
-    # f32: the IEEE-f32 matrix-core prefill kernel where the launch gives it more than one 128-row workgroup per compute unit
-    # (256 here: no device to ask), the f32 split-KV kernel - 32 rows per workgroup, keys dealt to its wavefronts - below that
+    # f32: the IEEE-f32 matrix-core prefill kernel where the launch gives it more than two 128-row workgroups per compute unit
+    # (256 compute units here: no device to ask), the f32 split-KV kernel - 32 rows per workgroup, keys dealt to its wavefronts,
+    # two workgroups per compute unit - up to that
     assert _plan(_desc(dtype=capi.F32, B=8, Hq=16, Sq=4096, Skv=4096))[2] == capi.IMPL_MFMA
     assert _plan(_desc(dtype=capi.F32, B=4, Hq=8, Sq=1024, Skv=1024))[2] == capi.IMPL_SPLITKV_MFMA      # 4 x 8 heads x 1024 x 1024: 256 workgroups
-    assert _plan(_desc(dtype=capi.F32, B=4, Hq=8, Sq=1025, Skv=1025))[2] == capi.IMPL_MFMA              # 288
+    assert _plan(_desc(dtype=capi.F32, B=4, Hq=8, Sq=2048, Skv=2048))[2] == capi.IMPL_SPLITKV_MFMA      # 512
+    assert _plan(_desc(dtype=capi.F32, B=4, Hq=8, Sq=2049, Skv=2049))[2] == capi.IMPL_MFMA              # 544
     assert _plan(_desc(dtype=capi.F32))[2] == capi.IMPL_SPLITKV_MFMA
     assert _plan(_desc(dtype=capi.F32, impl=capi.IMPL_MFMA))[2] == capi.IMPL_MFMA
     assert _plan(_desc(dtype=capi.F32, add_mask=0x20000))[2] == capi.IMPL_MFMA  # which also takes a dense mask
@@ -75,10 +77,16 @@ def test_dispatch_choices():
     # instance of the matrix-core split-KV kernels
     assert _plan(_desc(D=160, Dv=160, B=64))[2] == capi.IMPL_MFMA
     assert _plan(_desc(D=128, Dv=136, B=64))[2] == capi.IMPL_MFMA
-    # (that prefill kernel does not split the keys: launches that give it workgroups for at most half the compute units go
-    # 32 rows per workgroup through the split-KV kernel - 8 and 128 workgroups here, then 136)
+    # (launches that give that prefill kernel workgroups for at most half the compute units go 32 rows per workgroup through
+    # the split-KV kernel - 8 workgroups here, then 128 over 3000 keys - unless the keys are long enough to be split so that
+    # every compute unit gets a workgroup: 128 workgroups x 4 splits of 4096 keys, and a 256-row chunk of a 16384-token prompt)
     assert _plan(_desc(D=160, Dv=160))[2] == capi.IMPL_SPLITKV_MFMA
-    assert _plan(_desc(D=256, Dv=256, B=1, Hq=16, Hkv=16, Sq=1024, Skv=4096, causal=1))[2] == capi.IMPL_SPLITKV_MFMA
+    assert _plan(_desc(D=256, Dv=256, B=1, Hq=16, Hkv=16, Sq=1024, Skv=3000, causal=1))[2] == capi.IMPL_SPLITKV_MFMA
+    nbytes, splits, impl = _plan(_desc(D=256, Dv=256, B=1, Hq=16, Hkv=16, Sq=1024, Skv=4096, causal=1))
+    assert impl == capi.IMPL_MFMA and splits == 4 and nbytes == 16 * 1024 * 4 * 258 * 4
+    nbytes, splits, impl = _plan(_desc(D=256, Dv=256, B=1, Hq=32, Hkv=8, Sq=256, Skv=16384, causal=1))
+    assert impl == capi.IMPL_MFMA and splits == 8
+    assert _plan(_desc(D=256, Dv=256, B=1, Hq=8, Hkv=8, Sq=128, Skv=8192, causal=1))[2] == capi.IMPL_SPLITKV_MFMA      # 8 workgroups x 8 splits: not enough
     assert _plan(_desc(D=256, Dv=256, B=1, Hq=17, Hkv=17, Sq=1024, Skv=4096, causal=1))[2] == capi.IMPL_MFMA
     # (72 workgroups, 288 chunks of 32 rows: a ragged second round for the split-KV kernel, measured 1.25 times behind)
     assert _plan(_desc(D=256, Dv=256, B=1, Hq=12, Hkv=12, Sq=768, Skv=3000, causal=1))[2] == capi.IMPL_MFMA
