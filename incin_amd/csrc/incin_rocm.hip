@@ -111,6 +111,7 @@ struct Plan {
     int splits;
     int split_len;
     size_t ws_bytes;
+    size_t lims_offset;      // dense mask on the 16-bit prefill kernel for up to 128: where the mask's row limits start in the workspace (0: none)
     bool empty;      // nothing to compute
 };
 
@@ -157,6 +158,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     plan->splits = 1;
     plan->split_len = (int)d->Skv;
     plan->ws_bytes = 0;
+    plan->lims_offset = 0;
     plan->empty = (d->B == 0 || d->Hq == 0 || d->Sq == 0 || d->Dv == 0);
     if (plan->empty) return 0;
     if (d->Hkv <= 0 || d->Hq % d->Hkv != 0)
@@ -390,6 +392,10 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         if (nbh > 65535 || (d->Sq + 31) / 32 > 65535)
             return fail(INCIN_ROCM_ESHAPE, "scaled_dot_product_attention: mask too large for one launch of the matrix-core kernels");
         plan->ws_bytes = (size_t)(nbh * ((d->Sq + 31) / 32) * ((d->Skv + 31) / 32) + 255) / 256 * 256;
+        if (d->dtype != INCIN_ROCM_F32 && !wide) {      // and one int per mask row: its limit, if it is zeros up to one and -inf beyond
+            plan->lims_offset = plan->ws_bytes;
+            plan->ws_bytes += (size_t)(nbh * (d->mask_stride[2] ? d->Sq : 1) * 4 + 255) / 256 * 256;
+        }
     }
     return 0;
 }
@@ -418,6 +424,7 @@ void fill_params(const incin_rocm_sdpa_desc_t* d, const Plan& plan, SdpaParams* 
     p->num_splits = plan.splits;
     p->split_len = plan.split_len;
     if (plan.impl == INCIN_ROCM_IMPL_MFMA) p->mask_flags = d->add_mask ? (const uint8_t*)d->workspace : nullptr;
+    if (plan.impl == INCIN_ROCM_IMPL_MFMA && d->add_mask && plan.lims_offset) p->mask_lims = (const int32_t*)((const char*)d->workspace + plan.lims_offset);
     if (!(plan.impl == INCIN_ROCM_IMPL_MFMA && d->add_mask)) p->ws_acc = (float*)d->workspace;
     if (plan.splits > 1) {
         const size_t rows = (size_t)(d->B * d->Hq * d->Sq * plan.splits);

@@ -58,6 +58,55 @@ __global__ __launch_bounds__(256) void mask_classify_kernel(const T* mask, int64
     }
 }
 
+// Row limits: for every row of the mask, n if the row reads n zeros and then -inf to its end (n = Skv: all zeros, n = 0:
+// all -inf), else -1.  What a causal mask, a key-padding mask and their sum look like; a kernel that knows the limit of
+// every row it handles compares key numbers with it instead of reading the mask.  One wavefront per row: the first
+// position that is not zero and the number of -inf values decide.
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void mask_row_limits_kernel(const T* mask, int64_t m_sb, int64_t m_sh, int64_t m_si, int64_t m_sj,
+                                                             int Hm, int rows_m, int Skv, int64_t n_rows, int32_t* lims)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);       // (mask batch entry, mask head, row)
+    if (r >= n_rows) return;
+    const int i = (int)(r % rows_m);
+    const int64_t bh = r / rows_m;
+    const T* row = mask + (bh / Hm) * m_sb + (bh % Hm) * m_sh + (int64_t)i * m_si;
+    int first = Skv, ninf = 0;
+    if (VEC) {
+        typedef T vec8 __attribute__((ext_vector_type(8)));
+        for (int j0 = lane * 8; j0 < Skv; j0 += 512) {
+            if (j0 + 7 < Skv) {
+                const vec8 x = *(const vec8*)(row + j0);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float f = to_f32(x[e]);
+                    if (!(f == 0.0f)) first = min(first, j0 + e);
+                    ninf += f == -INFINITY;
+                }
+            } else {
+                for (int e = 0; j0 + e < Skv; ++e) {
+                    const float f = to_f32(row[j0 + e]);
+                    if (!(f == 0.0f)) first = min(first, j0 + e);
+                    ninf += f == -INFINITY;
+                }
+            }
+        }
+    } else {
+        for (int j = lane; j < Skv; j += 64) {
+            const float f = to_f32(row[(int64_t)j * m_sj]);
+            if (!(f == 0.0f)) first = min(first, j);
+            ninf += f == -INFINITY;
+        }
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        first = min(first, __shfl_xor(first, off, 64));
+        ninf += __shfl_xor(ninf, off, 64);
+    }
+    if (lane == 0) lims[r] = ninf == Skv - first ? first : -1;
+}
+
 // Host has validated the extents; nbh = mask batch entries x mask heads (1 where the mask is broadcast).
 hipError_t launch_mask_classify(const SdpaParams& p, int dtype, hipStream_t stream)
 {
@@ -77,6 +126,18 @@ hipError_t launch_mask_classify(const SdpaParams& p, int dtype, hipStream_t stre
         default: if (vec) CLASSIFY(bf16_t, true); else CLASSIFY(bf16_t, false); break;
     }
 #undef CLASSIFY
+    if (p.mask_lims) {
+        const int rows_m = p.m_si ? p.Sq : 1;
+        const int64_t n_rows = (int64_t)Bm * Hm * rows_m;
+        const dim3 lgrid((unsigned)((n_rows + 3) / 4));
+#define LIMITS(T, V) hipLaunchKernelGGL((mask_row_limits_kernel<T, V>), lgrid, dim3(256), 0, stream, (const T*)p.mask, p.m_sb, p.m_sh, p.m_si, p.m_sj, Hm, rows_m, p.Skv, n_rows, (int32_t*)p.mask_lims)
+        switch (dtype) {
+            case 0: if (vec) LIMITS(float, true); else LIMITS(float, false); break;
+            case 1: if (vec) LIMITS(f16_t, true); else LIMITS(f16_t, false); break;
+            default: if (vec) LIMITS(bf16_t, true); else LIMITS(bf16_t, false); break;
+        }
+#undef LIMITS
+    }
     return hipGetLastError();
 }
 

@@ -187,6 +187,8 @@ inline int work_deal(int F, int G, int nqb, long long share_items)
 
 // F for a launch: `slots` workgroups run on an XCD at a time, a range of the list (the whole list, or an eighth of it
 // when it divides by 8 and each XCD takes one) holds `range_items` items.
+// (`causal`: the blocks of a head differ in length - a causal flag, or a mask tensor, which more often than not is a causal
+// mask; with blocks of equal length the interleaved order costs nothing)
 inline int work_interleave(bool causal, int slots, int G, int nqb, long long range_items)
 {
     if (!causal || slots <= 0) return 1;

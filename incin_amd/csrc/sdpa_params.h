@@ -36,6 +36,11 @@ struct SdpaParams {
     // 2 all -inf), written by mask_classify_kernel ahead of the attention kernel, in the caller's workspace;
     // [mask batch entries][mask heads][ceil(Sq / 32)][ceil(Skv / 32)], an extent of 1 where the mask is broadcast
     const uint8_t* mask_flags;
+    // and, for the 16-bit prefill kernel, one int per mask row ([mask batch entries][mask heads][Sq, or 1 where the rows are
+    // broadcast]): n if the row is n zeros followed by -inf to its end - a causal mask, key padding, both - else -1, written by
+    // mask_row_limits_kernel.  A workgroup whose rows all have one needs no mask values, only the limits.  Null: not provided.
+    const int32_t* mask_lims;
+    int32_t lims_rows;         // rows per block of the launch that takes the blocks whose rows all have a limit (128 or 256; set by the launcher)
     int32_t mask_vec;          // 16-bit MFMA kernel: the mask's rows allow 8-byte loads of 4 consecutive keys
 };
 
@@ -58,6 +63,14 @@ __device__ __forceinline__ const uint8_t* mask_flags_of(const SdpaParams& p, int
     const int Hm = p.m_sh ? p.Hq : 1;
     const int64_t bh = (int64_t)(p.m_sb ? b : 0) * Hm + (p.m_sh ? hq : 0);
     return p.mask_flags + bh * nrb * nkb;
+}
+
+// Where the row limits of (batch b, query head hq) start.
+__device__ __forceinline__ const int32_t* mask_lims_of(const SdpaParams& p, int b, int hq)
+{
+    const int Hm = p.m_sh ? p.Hq : 1;
+    const int64_t bh = (int64_t)(p.m_sb ? b : 0) * Hm + (p.m_sh ? hq : 0);
+    return p.mask_lims + bh * (p.m_si ? p.Sq : 1);
 }
 
 }  // namespace incin_rocm

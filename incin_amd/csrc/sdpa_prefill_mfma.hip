@@ -88,10 +88,17 @@ namespace incin_rocm {
 // KS, NB: the k-steps of 16 head-dimension columns the score product runs over, and the 32-column blocks of the output it
 // keeps.  D fixes the layout of a tile in LDS (rows of D columns, zero beyond the tensors' own); head dimensions that fill only
 // part of it leave the rest out of the arithmetic as well: 6 k-steps and 3 blocks for head dimensions up to 96 in the 128 layout.
-template <typename T, int D, bool DENSE, int NW, bool SPLIT = false, int KS = D / 16, int NB = D / 32>
+//
+// MASK: 0 no mask tensor; 1 (DENSE) a dense additive mask, by block flags and values; 2 (LIMS) a launch with a dense mask for
+// the workgroups all of whose rows the mask gives n zeros and then -inf (mask_row_limits_kernel wrote n per row: a causal mask,
+// key padding, both): to them the tensor says nothing their limits do not, and they run exactly as without one.  A masked
+// request is two launches, LIMS then DENSE, and every block of p.lims_rows rows is computed by one of them: by LIMS if all
+// its rows have a limit, else by DENSE (whose 128-row workgroups look at the limits of the LIMS block that holds them).
+template <typename T, int D, int MASK, int NW, bool SPLIT = false, int KS = D / 16, int NB = D / 32>
 __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void sdpa_prefill_mfma_kernel(SdpaParams p)
 {
+    constexpr bool DENSE = MASK == 1, LIMS = MASK == 2;
 #if defined(__HIP_DEVICE_COMPILE__)   // the body uses device-only types (buffer descriptors); the host pass needs only the stub
     typedef typename Mma<T>::vec8 vec8;
     typedef PfLayout<D> L;
@@ -172,6 +179,42 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     // the path of every tile, and a global load there costs a memory latency per tile
     constexpr int FLAG_TILES = 512;
     __shared__ uint8_t s_flags[DENSE ? NW * 2 * FLAG_TILES : 4];
+    if ((DENSE || LIMS) && p.mask_lims != nullptr) {
+        // does every row of the block of lims_rows rows around this workgroup's have a limit?  (uniform over the workgroup)
+        const int32_t* lims = mask_lims_of(p, b, hq);
+        const int blk0 = (q0 / p.lims_rows) * p.lims_rows, blk1 = min(blk0 + p.lims_rows, rows_b);
+        bool ok = true;
+        for (int i = blk0 + tid; i < blk1; i += 64 * NW) ok = ok && lims[p.m_si ? i : 0] >= 0;
+        const bool wave_ok = __builtin_amdgcn_ballot_w64(!ok) == 0;
+        if (lane == 0) s_range[wave] = wave_ok ? 1 : 0;
+        __syncthreads();
+        bool all = true;
+#pragma unroll
+        for (int w2 = 0; w2 < NW; ++w2) all = all && s_range[w2] != 0;
+        all = __builtin_amdgcn_readfirstlane(all ? 1 : 0) != 0;
+        if (all != LIMS) return;                           // the other launch computes this block
+        __syncthreads();                                   // (s_range is used again below)
+        if (LIMS) {
+            // this lane's limit, the smallest and largest of the wavefront, the largest of the workgroup
+            const bool row_here = my_i < rows_b;
+            lim_lane = row_here ? min(lim_lane, lims[p.m_si ? my_i : 0]) : 0;
+            int lo = row_here ? lim_lane : 0x7fffffff, hi = lim_lane;
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) {
+                lo = min(lo, __shfl_xor(lo, off, 64));
+                hi = max(hi, __shfl_xor(hi, off, 64));
+            }
+            lim_wave_min = __builtin_amdgcn_readfirstlane(lo == 0x7fffffff ? 0 : lo);
+            lim_wave_max = __builtin_amdgcn_readfirstlane(hi);
+            if (lane == 0) s_range[wave] = lim_wave_max;
+            __syncthreads();
+            int je = 0;
+#pragma unroll
+            for (int w2 = 0; w2 < NW; ++w2) je = max(je, s_range[w2]);
+            j_end = __builtin_amdgcn_readfirstlane(je);
+            n_tiles = (j_end + PF_BN - 1) / PF_BN;
+        }
+    }
     const bool flags_in_lds = DENSE && n_tiles <= FLAG_TILES;
     if (DENSE) {
         mflags = mask_flags_of(p, b, hq) + (int64_t)((q0 >> 5) + wave) * nkb32;
@@ -789,7 +832,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
 
 hipError_t launch_sdpa_combine(const SdpaParams& p, int dtype, hipStream_t stream);
 
-template <typename T, int D, bool DENSE, int NW>
+template <typename T, int D, int MASK, int NW>
 static hipError_t launch_prefill_nw(const SdpaParams& p0, hipStream_t stream)
 {
     SdpaParams p = p0;
@@ -797,22 +840,24 @@ static hipError_t launch_prefill_nw(const SdpaParams& p0, hipStream_t stream)
     const int64_t total = (int64_t)nqb * p.Hq * p.B;
     // 256 registers per lane: eight wavefronts per compute unit, i.e. two workgroups of four or one of eight; an eighth
     // of the compute units per XCD
-    p.interleave = work_interleave(p.causal != 0, (8 / NW) * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
+    p.interleave = work_interleave(p.causal != 0 || p.mask != nullptr, (8 / NW) * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
     p.deal_groups = (total & 7) == 0 ? work_deal(p.interleave, p.G, nqb, total >> 3) : 0;
-    if constexpr (!DENSE && NW == 4) {
+    constexpr bool DENSE = MASK == 1;
+    if constexpr (MASK == 0 && NW == 4) {
         if (p.num_splits > 1) {          // split launch: partial results, then the split-KV kernels' combine pass
-            hipLaunchKernelGGL((sdpa_prefill_mfma_kernel<T, D, false, 4, true>), dim3((unsigned)total, (unsigned)p.num_splits), dim3(256), 0, stream, p);
+            hipLaunchKernelGGL((sdpa_prefill_mfma_kernel<T, D, 0, 4, true>), dim3((unsigned)total, (unsigned)p.num_splits), dim3(256), 0, stream, p);
             hipError_t e = hipGetLastError();
             return e != hipSuccess ? e : launch_sdpa_combine(p, std::is_same<T, f16_t>::value ? 1 : 2, stream);
         }
     }
-    if constexpr (!DENSE && D == 128) {
+    if constexpr (MASK == 0 && D == 128) {
         if (p.D <= 96 && p.Dv <= 96) {   // the last quarter of the layout is padding: the instance that leaves it out of the products
-            hipLaunchKernelGGL((sdpa_prefill_mfma_kernel<T, D, false, NW, false, 6, 3>), dim3((unsigned)total), dim3(64 * NW), 0, stream, p);
+            hipLaunchKernelGGL((sdpa_prefill_mfma_kernel<T, D, 0, NW, false, 6, 3>), dim3((unsigned)total), dim3(64 * NW), 0, stream, p);
             return hipGetLastError();
         }
     }
-    hipLaunchKernelGGL((sdpa_prefill_mfma_kernel<T, D, DENSE, NW>), dim3((unsigned)total), dim3(64 * NW), 0, stream, p);
+    (void)DENSE;
+    hipLaunchKernelGGL((sdpa_prefill_mfma_kernel<T, D, MASK, NW>), dim3((unsigned)total), dim3(64 * NW), 0, stream, p);
     return hipGetLastError();
 }
 
@@ -820,18 +865,34 @@ static hipError_t launch_prefill_nw(const SdpaParams& p0, hipStream_t stream)
 // compute unit and 2048 keys, 2 - 3.5 % ahead from 4096 keys on, far behind when the launch does not fill the device) -
 // head dimension 128 without a dense mask (with one the 256-row form is 6 % behind: the wavefronts of a workgroup see
 // different stretches of the mask and wait for each other at every tile); 128-row workgroups otherwise.
-template <typename T, int D, bool DENSE>
-static hipError_t launch_prefill_t(const SdpaParams& p, hipStream_t stream)
+// With a dense mask (MASK = 1): first the launch for the blocks whose rows all have a limit (MASK = 2, in the form the rule
+// picks), then the 128-row launch that reads the mask, for the others.
+template <typename T, int D, int MASK>
+static hipError_t launch_prefill_t(const SdpaParams& p0, hipStream_t stream)
 {
-    if constexpr (D == 128 && !DENSE) {
+    SdpaParams p = p0;
+    if constexpr (MASK == 1) {
+        if (p.mask_lims != nullptr) {
+            hipError_t e = launch_prefill_t<T, D, 2>(p, stream);
+            if (e != hipSuccess) return e;
+            const char* forced = getenv("INCIN_ROCM_PREFILL_BLOCK_ROWS");      // (the same rule as below: the block the first launch took)
+            const int rows = forced ? atoi(forced) : 0;
+            const int64_t blocks256 = (int64_t)((p.Sq + 255) / 256) * p.Hq * p.B;
+            p.lims_rows = D == 128 && (rows == 256 || (rows != 128 && p.Skv >= 4096 && blocks256 >= 6 * (int64_t)device_cus())) ? 256 : 128;
+        }
+    }
+    if constexpr (D == 128 && MASK != 1) {
         // INCIN_ROCM_PREFILL_BLOCK_ROWS = 128 or 256 overrides the rule (for tests: small shapes through the 256-row form)
         const char* forced = getenv("INCIN_ROCM_PREFILL_BLOCK_ROWS");
         const int rows = forced ? atoi(forced) : 0;
         const int64_t blocks256 = (int64_t)((p.Sq + 255) / 256) * p.Hq * p.B;
-        if (p.num_splits <= 1 && (rows == 256 || (rows != 128 && p.Skv >= 4096 && blocks256 >= 6 * (int64_t)device_cus())))
-            return launch_prefill_nw<T, D, DENSE, 8>(p, stream);
+        if (p.num_splits <= 1 && (rows == 256 || (rows != 128 && p.Skv >= 4096 && blocks256 >= 6 * (int64_t)device_cus()))) {
+            p.lims_rows = 256;
+            return launch_prefill_nw<T, D, MASK, 8>(p, stream);
+        }
     }
-    return launch_prefill_nw<T, D, DENSE, 4>(p, stream);
+    if constexpr (MASK == 2) p.lims_rows = 128;
+    return launch_prefill_nw<T, D, MASK, 4>(p, stream);
 }
 
 // Host has validated: dtype f16/bf16, D and Dv <= 128 in whole 16-byte vectors (p.Dp = the instance: 64 or 128), scale > 0, rows 16-byte aligned with unit last-dim stride, row strides below 2^24
@@ -839,11 +900,11 @@ static hipError_t launch_prefill_t(const SdpaParams& p, hipStream_t stream)
 hipError_t launch_sdpa_prefill_mfma(const SdpaParams& p, int dtype, hipStream_t stream)
 {
     if (p.mask) {
-        if (dtype == 1) return p.Dp == 128 ? launch_prefill_t<f16_t, 128, true>(p, stream) : launch_prefill_t<f16_t, 64, true>(p, stream);
-        return p.Dp == 128 ? launch_prefill_t<bf16_t, 128, true>(p, stream) : launch_prefill_t<bf16_t, 64, true>(p, stream);
+        if (dtype == 1) return p.Dp == 128 ? launch_prefill_t<f16_t, 128, 1>(p, stream) : launch_prefill_t<f16_t, 64, 1>(p, stream);
+        return p.Dp == 128 ? launch_prefill_t<bf16_t, 128, 1>(p, stream) : launch_prefill_t<bf16_t, 64, 1>(p, stream);
     }
-    if (dtype == 1) return p.Dp == 128 ? launch_prefill_t<f16_t, 128, false>(p, stream) : launch_prefill_t<f16_t, 64, false>(p, stream);
-    return p.Dp == 128 ? launch_prefill_t<bf16_t, 128, false>(p, stream) : launch_prefill_t<bf16_t, 64, false>(p, stream);
+    if (dtype == 1) return p.Dp == 128 ? launch_prefill_t<f16_t, 128, 0>(p, stream) : launch_prefill_t<f16_t, 64, 0>(p, stream);
+    return p.Dp == 128 ? launch_prefill_t<bf16_t, 128, 0>(p, stream) : launch_prefill_t<bf16_t, 64, 0>(p, stream);
 }
 
 }  // namespace incin_rocm

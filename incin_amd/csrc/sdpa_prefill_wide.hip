@@ -335,7 +335,7 @@ hipError_t launch_sdpa_prefill_wide(const SdpaParams& p0, int dtype, hipStream_t
     if (total <= 0) return hipSuccess;
     if (total > 0x7fffffffLL) return hipErrorInvalidValue;
     // two workgroups per compute unit, an eighth of the compute units per XCD
-    p.interleave = work_interleave(p.causal != 0, 2 * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
+    p.interleave = work_interleave(p.causal != 0 || p.mask != nullptr, 2 * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
     p.deal_groups = (total & 7) == 0 ? work_deal(p.interleave, p.G, nqb, total >> 3) : 0;
     if (!p.mask && p.num_splits > 1) {       // split launch: partial results, then the split-KV kernels' combine pass
         const dim3 grid((unsigned)total, (unsigned)p.num_splits);

@@ -103,8 +103,8 @@ def test_dispatch_choices():
     assert impl == capi.IMPL_SPLITKV_MFMA and splits == 4 and nbytes == 2 * 8 * 4 * 130 * 4
     nbytes, splits, impl = _plan(_desc(Sq=1, Skv=8192, B=2, Hq=8, Hkv=2, D=48, Dv=32, num_splits=4, dtype=capi.F32))
     assert impl == capi.IMPL_SPLITKV_MFMA and splits == 4 and nbytes == 2 * 8 * 4 * 66 * 4
-    nbytes, _, impl = _plan(_desc(add_mask=0x20000))                            # dense mask: still the matrix cores,
-    assert impl == capi.IMPL_MFMA and nbytes == 256                           # with 2 x 4 x 4 x 4 block flags (rounded up)
+    nbytes, _, impl = _plan(_desc(add_mask=0x20000))                            # dense mask: still the matrix cores, with
+    assert impl == capi.IMPL_MFMA and nbytes == 256 + 256                     # 2 x 4 x 4 x 4 block flags and a limit per mask row (each rounded up)
     assert _plan(_desc(add_mask=0x20000, D=80, Dv=80))[2] == capi.IMPL_MFMA
     assert _plan(_desc(add_mask=0x20000, D=160, Dv=160))[2] == capi.IMPL_GENERIC      # (a mask without strides: not readable 8 bytes at a time)
     wide_masked = _desc(add_mask=0x20000, D=160, Dv=160)

@@ -438,6 +438,62 @@ def test_auto_splits_the_keys_of_a_wide_prefill_launch_that_fills_the_device(gpu
         assert np.abs(got.reshape(Hq, Sq, 256)[rows[:, 0], rows[:, 1]] - ref).max() <= TOL[capi.BF16]
 
 
+@pytest.mark.parametrize("dtype", [capi.BF16, capi.F16], ids=lambda x: dtypes.NAMES[x])
+@pytest.mark.parametrize("rows", ["128", "256"])
+@pytest.mark.parametrize("D", [128, 64])
+def test_mask_tensors_whose_rows_are_zeros_then_minus_infinity(gpu, dtype, rows, D, monkeypatch):
+    """A mask tensor whose every row is n zeros followed by -inf - the causal mask as the reference's callers build it, a
+    key-padding mask, their sum - says nothing its row limits do not.  The 16-bit prefill launch writes a limit per mask row
+    and runs the blocks of rows that all have one as a launch without a mask tensor does, the others from the mask's flags
+    and values; every block is computed by exactly one of the two.  Against the oracle given the tensor: masks that are all
+    limits, masks where some blocks are and some are not (a bias in a few rows), limits of 0 (rows that see nothing: NaN)
+    and of Skv, rows broadcast over queries / heads / batch, on top of a causal flag and key counts, S_q not a multiple of
+    the blocks, both workgroup forms."""
+    monkeypatch.setenv("INCIN_ROCM_PREFILL_BLOCK_ROWS", rows)
+    tol = TOL[dtype]
+    r = rng(SEED0 + 120 + D)
+    B, Hq, Hkv, Sq, Skv = 2, 4, 2, 600, 700
+    q, k, v = inputs(3100 + D, B, Hq, Hkv, Sq, Skv, D, D, dtype)
+    NEG = -np.inf
+    causal = O.causal_additive_mask(Sq, Skv).reshape(1, 1, Sq, Skv)                       # aligned to the last key
+    cases = []
+    cases.append(("the causal tensor", causal, {}))
+    pad = np.zeros((B, 1, 1, Skv), np.float32)
+    pad[0, ..., 650:] = NEG
+    pad[1, ..., 90:] = NEG
+    cases.append(("key padding [B,1,1,Skv]", pad, {}))
+    cases.append(("causal + key padding [B,1,Sq,Skv]", causal + pad, {}))
+    lims = r.integers(0, Skv + 1, size=(B, Hq, Sq))                                        # any limit per row, 0 and Skv among them
+    lims[0, 0, :5] = 0
+    lims[1, 3, 300:310] = Skv
+    anyl = np.where(np.arange(Skv)[None, None, None, :] < lims[..., None], 0.0, NEG).astype(np.float32)
+    cases.append(("a limit of its own per row [B,Hq,Sq,Skv]", anyl, {}))
+    mixed = np.broadcast_to(causal, (1, Hq, Sq, Skv)).copy()
+    mixed[0, 1, 130:140, :20] = -1.5                                                       # head 1: rows 130..139 carry a bias: their block reads the mask
+    mixed[0, 2, 599, 100] = NEG                                                            # head 2: a hole in the last row
+    mixed[0, 3, 300, 400:] = 0.0                                                           # head 3: one row sees everything (a limit, too)
+    cases.append(("causal with a few rows that are not limits [1,Hq,Sq,Skv]", mixed, {}))
+    cases.append(("key padding under a causal flag and key counts", pad, dict(causal=True, kv_lens=np.array([700, 60], np.int32))))
+    for what, m, kw in cases:
+        say("limit masks: %s, %s rows, D=%d, %s" % (dtypes.NAMES[dtype], rows, D, what))
+        m = dtypes.round_to(np.ascontiguousarray(m), dtype)
+        got, lse, info = host.sdpa(q, k, v, dtype, mask=m, impl=capi.IMPL_MFMA, return_info=True, return_lse=True, **kw)
+        assert info["impl"] == capi.IMPL_MFMA
+        full = np.broadcast_to(m, (B, Hq, Sq, Skv)).copy()             # (the oracle takes one mask: the flag and the counts folded in)
+        if kw.get("causal"):
+            full += causal
+        if kw.get("kv_lens") is not None:
+            full += np.where(np.arange(Skv)[None, :] < kw["kv_lens"][:, None], 0.0, NEG).astype(np.float32)[:, None, None, :]
+        check(got, oracle_full(q, k, v, G=Hq // Hkv, mask=full), tol, what)
+        _, lse_g = host.sdpa(q, k, v, dtype, mask=m, impl=capi.IMPL_GENERIC, return_lse=True, **kw)
+        fin = np.isfinite(lse_g)
+        assert np.array_equal(np.isfinite(lse), fin) and np.max(np.abs(lse[fin] - lse_g[fin])) < 2e-2, what
+    # the causal tensor and the causal flag are the same computation row for row
+    flag = host.sdpa(q, k, v, dtype, causal=True, impl=capi.IMPL_MFMA)
+    tens = host.sdpa(q, k, v, dtype, mask=dtypes.round_to(causal, dtype), impl=capi.IMPL_MFMA)
+    assert np.array_equal(flag, tens, equal_nan=True)
+
+
 # ---- split-KV decode -----------------------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", [capi.BF16, capi.F16, capi.F32])
