@@ -111,7 +111,7 @@ struct Plan {
     int splits;
     int split_len;
     size_t ws_bytes;
-    size_t lims_offset;      // dense mask on the 16-bit prefill kernel for up to 128: where the mask's row limits start in the workspace (0: none)
+    size_t lims_offset;      // dense mask on the 16-bit prefill kernels: where the mask's row limits start in the workspace (0: none)
     bool empty;      // nothing to compute
 };
 
@@ -392,7 +392,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         if (nbh > 65535 || (d->Sq + 31) / 32 > 65535)
             return fail(INCIN_ROCM_ESHAPE, "scaled_dot_product_attention: mask too large for one launch of the matrix-core kernels");
         plan->ws_bytes = (size_t)(nbh * ((d->Sq + 31) / 32) * ((d->Skv + 31) / 32) + 255) / 256 * 256;
-        if (d->dtype != INCIN_ROCM_F32 && !wide) {      // and one int per mask row: its limit, if it is zeros up to one and -inf beyond
+        if (d->dtype != INCIN_ROCM_F32) {               // and (16-bit kernels) one int per mask row: its limit, if it is zeros up to one and -inf beyond
             plan->lims_offset = plan->ws_bytes;
             plan->ws_bytes += (size_t)(nbh * (d->mask_stride[2] ? d->Sq : 1) * 4 + 255) / 256 * 256;
         }

@@ -32,9 +32,14 @@ constexpr int PW_KT = 32;      // keys per tile
 // SPLIT: a grid of (work items) x (splits of the key axis), as in sdpa_prefill_mfma.hip - a workgroup handles the keys of its
 // split and writes, per row, the unnormalised O, the reference and the sum in the split-KV kernels' partial-result format; their
 // combine kernel finishes.  For launches with few 128-row blocks over a long key axis (a chunk of a long prompt).
-template <typename T, bool DENSE, bool SPLIT = false>
+//
+// MASK: 0 no mask tensor; 1 (DENSE) a dense additive mask by flags and values; 2 (LIMS) the launch for the 128-row blocks all
+// of whose rows the mask gives n zeros and then -inf (sdpa_prefill_mfma.hip has the scheme: a masked request is the LIMS
+// launch, whose other workgroups leave at once, and then the DENSE launch, whose workgroups leave if LIMS took their block).
+template <typename T, int MASK, bool SPLIT = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void sdpa_prefill_wide_kernel(SdpaParams p)
 {
+    constexpr bool DENSE = MASK == 1, LIMS = MASK == 2;
 #if defined(__HIP_DEVICE_COMPILE__)
     typedef typename Mma<T>::vec8 vec8;
     constexpr int D = 256;
@@ -92,6 +97,35 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const T* mrow = nullptr;
     const uint8_t* mflags = nullptr;
     __shared__ int s_range[8];
+    if ((DENSE || LIMS) && p.mask_lims != nullptr) {
+        // does every row of this workgroup have a limit?  (uniform over the workgroup)
+        const int32_t* lims = mask_lims_of(p, b, hq);
+        const bool row_here = my_i < rows_b;
+        const int lm = lims[p.m_si ? min(my_i, Sq - 1) : 0];
+        const bool wave_ok = __builtin_amdgcn_ballot_w64(row_here && lm < 0) == 0;
+        if (lane == 0) s_range[wave] = wave_ok ? 1 : 0;
+        __syncthreads();
+        const bool all = __builtin_amdgcn_readfirstlane((s_range[0] & s_range[1] & s_range[2] & s_range[3]) != 0 ? 1 : 0) != 0;
+        if (all != LIMS) return;                           // the other launch computes this block
+        __syncthreads();                                   // (s_range is used again below)
+        if (LIMS) {
+            // this lane's limit, the smallest and largest of the wavefront, the largest of the workgroup
+            lim_lane = row_here ? min(lim_lane, lm) : 0;
+            int lo = row_here ? lim_lane : 0x7fffffff, hi = lim_lane;
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) {
+                lo = min(lo, __shfl_xor(lo, off, 64));
+                hi = max(hi, __shfl_xor(hi, off, 64));
+            }
+            lim_wave_min = __builtin_amdgcn_readfirstlane(lo == 0x7fffffff ? 0 : lo);
+            lim_wave_max = __builtin_amdgcn_readfirstlane(hi);
+            if (lane == 0) s_range[wave] = lim_wave_max;
+            __syncthreads();
+            j_end = __builtin_amdgcn_readfirstlane(max(max(s_range[0], s_range[1]), max(s_range[2], s_range[3])));
+            n_tiles = (j_end + PW_KT - 1) / PW_KT;
+            n_act = lim_wave_max > 0 ? (lim_wave_max + PW_KT - 1) / PW_KT : 0;
+        }
+    }
     if (DENSE) {
         mrow = (const T*)p.mask + (int64_t)b * p.m_sb + (int64_t)hq * p.m_sh + (int64_t)min(my_i, Sq - 1) * p.m_si;
         // (a wavefront whose 32 rows lie past Sq computes nothing; its flag reads stay inside the array on the last row block)
@@ -337,18 +371,24 @@ hipError_t launch_sdpa_prefill_wide(const SdpaParams& p0, int dtype, hipStream_t
     // two workgroups per compute unit, an eighth of the compute units per XCD
     p.interleave = work_interleave(p.causal != 0 || p.mask != nullptr, 2 * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
     p.deal_groups = (total & 7) == 0 ? work_deal(p.interleave, p.G, nqb, total >> 3) : 0;
+    if (p.mask && p.mask_lims) {       // the blocks whose rows all have a limit; then, below, the others
+        if (dtype == 1) hipLaunchKernelGGL((sdpa_prefill_wide_kernel<f16_t, 2>), dim3((unsigned)total), dim3(256), 0, stream, p);
+        else hipLaunchKernelGGL((sdpa_prefill_wide_kernel<bf16_t, 2>), dim3((unsigned)total), dim3(256), 0, stream, p);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
     if (!p.mask && p.num_splits > 1) {       // split launch: partial results, then the split-KV kernels' combine pass
         const dim3 grid((unsigned)total, (unsigned)p.num_splits);
-        if (dtype == 1) hipLaunchKernelGGL((sdpa_prefill_wide_kernel<f16_t, false, true>), grid, dim3(256), 0, stream, p);
-        else hipLaunchKernelGGL((sdpa_prefill_wide_kernel<bf16_t, false, true>), grid, dim3(256), 0, stream, p);
+        if (dtype == 1) hipLaunchKernelGGL((sdpa_prefill_wide_kernel<f16_t, 0, true>), grid, dim3(256), 0, stream, p);
+        else hipLaunchKernelGGL((sdpa_prefill_wide_kernel<bf16_t, 0, true>), grid, dim3(256), 0, stream, p);
         hipError_t e = hipGetLastError();
         return e != hipSuccess ? e : launch_sdpa_combine(p, dtype, stream);
     }
     if (p.mask) {
-        if (dtype == 1) hipLaunchKernelGGL((sdpa_prefill_wide_kernel<f16_t, true>), dim3((unsigned)total), dim3(256), 0, stream, p);
-        else hipLaunchKernelGGL((sdpa_prefill_wide_kernel<bf16_t, true>), dim3((unsigned)total), dim3(256), 0, stream, p);
-    } else if (dtype == 1) hipLaunchKernelGGL((sdpa_prefill_wide_kernel<f16_t, false>), dim3((unsigned)total), dim3(256), 0, stream, p);
-    else hipLaunchKernelGGL((sdpa_prefill_wide_kernel<bf16_t, false>), dim3((unsigned)total), dim3(256), 0, stream, p);
+        if (dtype == 1) hipLaunchKernelGGL((sdpa_prefill_wide_kernel<f16_t, 1>), dim3((unsigned)total), dim3(256), 0, stream, p);
+        else hipLaunchKernelGGL((sdpa_prefill_wide_kernel<bf16_t, 1>), dim3((unsigned)total), dim3(256), 0, stream, p);
+    } else if (dtype == 1) hipLaunchKernelGGL((sdpa_prefill_wide_kernel<f16_t, 0>), dim3((unsigned)total), dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL((sdpa_prefill_wide_kernel<bf16_t, 0>), dim3((unsigned)total), dim3(256), 0, stream, p);
     return hipGetLastError();
 }
 

@@ -110,7 +110,7 @@ def test_dispatch_choices():
     wide_masked = _desc(add_mask=0x20000, D=160, Dv=160)
     wide_masked.mask_stride[2], wide_masked.mask_stride[3] = 128, 1                    # a [1, 1, Sq, Skv] mask
     nbytes, _, impl = _plan(wide_masked)
-    assert impl == capi.IMPL_MFMA and nbytes == 256                                    # block flags, as at 128
+    assert impl == capi.IMPL_MFMA and nbytes == 256 + 512                              # block flags and a limit per mask row (128 of them), as at 128
     nbytes, splits, impl = _plan(_desc(Sq=1, Skv=8192, B=32, Hq=32, Hkv=32))
     assert impl == capi.IMPL_SPLITKV_MFMA and splits == 1 and nbytes == 0      # 1024 workgroups, four rounds of 256
     nbytes, splits, impl = _plan(_desc(Sq=1, Skv=2048, B=8, Hq=32, Hkv=32))

@@ -440,7 +440,7 @@ def test_auto_splits_the_keys_of_a_wide_prefill_launch_that_fills_the_device(gpu
 
 @pytest.mark.parametrize("dtype", [capi.BF16, capi.F16], ids=lambda x: dtypes.NAMES[x])
 @pytest.mark.parametrize("rows", ["128", "256"])
-@pytest.mark.parametrize("D", [128, 64])
+@pytest.mark.parametrize("D", [128, 64, 256])
 def test_mask_tensors_whose_rows_are_zeros_then_minus_infinity(gpu, dtype, rows, D, monkeypatch):
     """A mask tensor whose every row is n zeros followed by -inf - the causal mask as the reference's callers build it, a
     key-padding mask, their sum - says nothing its row limits do not.  The 16-bit prefill launch writes a limit per mask row
