@@ -25,6 +25,7 @@ hipError_t launch_matrix_rate(const void* src, void* sink, int mix, int iteratio
 hipError_t launch_sdpa_prefill_f32(const SdpaParams& p, hipStream_t stream);
 hipError_t launch_sdpa_prefill_wide(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_mask_classify(const SdpaParams& p, int dtype, hipStream_t stream);
+hipError_t launch_sdpa_decode_f32_limits(const SdpaParams& p, hipStream_t stream);
 hipError_t launch_sdpa_decode(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_sdpa_decode_mfma(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_read_rate(const void* src, void* sink, size_t bytes, int nontemporal, hipStream_t stream);
@@ -111,7 +112,8 @@ struct Plan {
     int splits;
     int split_len;
     size_t ws_bytes;
-    size_t lims_offset;      // dense mask on the 16-bit prefill kernels: where the mask's row limits start in the workspace (0: none)
+    size_t lims_offset;      // dense mask on the prefill kernels: where the mask's row limits start in the workspace (0: none)
+    bool lims_splitkv;       // f32 with a dense mask: the blocks whose rows all have a limit go through the f32 split-KV kernel first
     bool empty;      // nothing to compute
 };
 
@@ -159,6 +161,7 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
     plan->split_len = (int)d->Skv;
     plan->ws_bytes = 0;
     plan->lims_offset = 0;
+    plan->lims_splitkv = false;
     plan->empty = (d->B == 0 || d->Hq == 0 || d->Sq == 0 || d->Dv == 0);
     if (plan->empty) return 0;
     if (d->Hkv <= 0 || d->Hq % d->Hkv != 0)
@@ -392,7 +395,13 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         if (nbh > 65535 || (d->Sq + 31) / 32 > 65535)
             return fail(INCIN_ROCM_ESHAPE, "scaled_dot_product_attention: mask too large for one launch of the matrix-core kernels");
         plan->ws_bytes = (size_t)(nbh * ((d->Sq + 31) / 32) * ((d->Skv + 31) / 32) + 255) / 256 * 256;
-        if (d->dtype != INCIN_ROCM_F32) {               // and (16-bit kernels) one int per mask row: its limit, if it is zeros up to one and -inf beyond
+        // f32: a small launch (what AUTO would hand the f32 split-KV kernel if there were no mask tensor: at most two 128-row
+        // blocks per compute unit) whose chunks of 32 rows do not straddle query heads gets the blocks whose mask rows all have
+        // a limit computed by that kernel, from the limits, ahead of the prefill kernel's dense-mask launch for the rest
+        // (benchmark config 2 with the causal mask as a tensor: 90 -> 66 us)
+        plan->lims_splitkv = d->dtype == INCIN_ROCM_F32 && !wide && d->impl == INCIN_ROCM_IMPL_AUTO && !d->q_lens && d->Sq > 64 &&
+                             (d->Hq == d->Hkv || d->Sq % 128 == 0) && d->B * d->Hq * ((d->Sq + 127) / 128) <= 2 * compute_units_of(d->device);
+        if (d->dtype != INCIN_ROCM_F32 || plan->lims_splitkv) {      // one int per mask row: its limit, if it is zeros up to one and -inf beyond
             plan->lims_offset = plan->ws_bytes;
             plan->ws_bytes += (size_t)(nbh * (d->mask_stride[2] ? d->Sq : 1) * 4 + 255) / 256 * 256;
         }
@@ -760,9 +769,16 @@ static int launch_fwd(const incin_rocm_sdpa_desc_t* desc, const Plan& plan, void
     hipError_t e;
     switch (plan.impl) {
         case INCIN_ROCM_IMPL_MFMA:
-            if (p.mask) {           // block flags of the mask first, on the same stream
+            if (p.mask) {           // block flags of the mask first (and its row limits), on the same stream
                 e = incin_rocm::launch_mask_classify(p, desc->dtype, s);
                 if (e != hipSuccess) break;
+                if (plan.lims_splitkv) {
+                    SdpaParams pl = p;
+                    pl.num_splits = 1;
+                    pl.split_len = (int)((desc->Skv + 255) / 256 * 256);
+                    e = incin_rocm::launch_sdpa_decode_f32_limits(pl, s);
+                    if (e != hipSuccess) break;
+                }
             }
             e = p.Dp == 256                    ? incin_rocm::launch_sdpa_prefill_wide(p, desc->dtype, s)
                 : desc->dtype == INCIN_ROCM_F32 ? incin_rocm::launch_sdpa_prefill_f32(p, s)

@@ -46,7 +46,12 @@ __device__ __forceinline__ float quad_sum(float x)
     return xor32_sum(x);
 }
 
-template <int D, int NSLOT, int NRB>
+//
+// LIMS: the launch is one half of a request with a mask tensor (one query head per KV head, or whole 128-row blocks per head):
+// mask_row_limits_kernel wrote, per mask row, n if the row is n zeros and then -inf, else -1.  A workgroup whose 128-row
+// block of rows all have a limit takes the limits - the tensor says nothing more - and the others leave at once: the f32
+// prefill kernel's dense-mask launch that follows computes those, and leaves the blocks computed here alone.
+template <int D, int NSLOT, int NRB, bool LIMS = false>
 __global__ __launch_bounds__(256) void sdpa_decode_f32_kernel(SdpaParams p)
 {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -71,7 +76,7 @@ __global__ __launch_bounds__(256) void sdpa_decode_f32_kernel(SdpaParams p)
     const int split = blockIdx.x;
     int hkv, chunk_id;
     int b;
-    decode_work_item(nchunks, p.causal && p.G == 1, NSLOT == 2, &b, &hkv, &chunk_id);
+    decode_work_item(nchunks, (p.causal || LIMS) && p.G == 1, NSLOT == 2, &b, &hkv, &chunk_id);
     const int r0 = chunk_id * CHUNK;
 
     int kv_len = Skv;
@@ -92,8 +97,27 @@ __global__ __launch_bounds__(256) void sdpa_decode_f32_kernel(SdpaParams p)
         int l = min(k_begin + p.split_len, kv_len);
         if (p.causal) l = min(l, causal_limit(qi[rb], Sq, Skv));
         lim[rb] = valid[rb] ? l : 0;
+    }
+    if (LIMS) {
+        // the 128-row block of this chunk's query head (rows of a chunk share a head: the host sends no other launches here)
+        __shared__ int s_ok[4];
+        const int head_row0 = (r0 / Sq) * Sq, i0 = r0 - head_row0;
+        const int blk0 = (i0 / 128) * 128, blk1 = min(blk0 + 128, Sq);
+        const int32_t* lims = mask_lims_of(p, b, hkv * p.G + r0 / Sq);
+        bool ok = true;
+        for (int i = blk0 + tid; i < blk1; i += 256) ok = ok && lims[p.m_si ? i : 0] >= 0;
+        const bool wave_ok = __builtin_amdgcn_ballot_w64(!ok) == 0;
+        if (lane == 0) s_ok[wave] = wave_ok ? 1 : 0;
+        __syncthreads();
+        if ((s_ok[0] & s_ok[1] & s_ok[2] & s_ok[3]) == 0) return;      // (uniform) the dense-mask launch computes this block
+#pragma unroll
+        for (int rb = 0; rb < NRB; ++rb)
+            if (valid[rb]) lim[rb] = min(lim[rb], lims[p.m_si ? qi[rb] : 0]);
+    }
+#pragma unroll
+    for (int rb = 0; rb < NRB; ++rb) {
         lim_hi = max(lim_hi, lim[rb]);
-        if (valid[rb]) lim_lo = min(lim_lo, l);
+        if (valid[rb]) lim_lo = min(lim_lo, lim[rb]);
     }
 #pragma unroll
     for (int off = 8; off >= 1; off >>= 1) {
@@ -388,14 +412,14 @@ __global__ __launch_bounds__(256) void sdpa_decode_f32_kernel(SdpaParams p)
 
 hipError_t launch_sdpa_combine(const SdpaParams& p, int dtype, hipStream_t stream);
 
-template <int D, int NSLOT, int NRB>
+template <int D, int NSLOT, int NRB, bool LIMS = false>
 static hipError_t launch_decode_f32_t(const SdpaParams& p, hipStream_t stream)
 {
     // the rings, or what the wavefronts' results need when they meet at the end, whichever is more
     constexpr size_t slot_bytes = D > 128 ? 2 * DM_SLOT_BYTES : DM_SLOT_BYTES;
     constexpr size_t ring_bytes = (size_t)4 * NSLOT * slot_bytes, merge_bytes = (size_t)NRB * (4 * 16 * 2 + 4 * (D / 16) * 4 * 64) * sizeof(float);
     constexpr size_t lds = ring_bytes > merge_bytes ? ring_bytes : merge_bytes;
-    auto kern = sdpa_decode_f32_kernel<D, NSLOT, NRB>;
+    auto kern = sdpa_decode_f32_kernel<D, NSLOT, NRB, LIMS>;
     // the dynamic-LDS limit of this instance is raised once per device, not per launch
     static std::atomic<uint64_t> prepared{0};
     int dev = 0;
@@ -439,6 +463,14 @@ hipError_t launch_sdpa_decode_f32(const SdpaParams& p, bool two_slots, hipStream
     else e = p.Dp == 128 ? launch_decode_f32_d<128>(p, two_slots, stream) : launch_decode_f32_d<64>(p, two_slots, stream);
     if (e != hipSuccess || p.num_splits == 1) return e;
     return launch_sdpa_combine(p, 0, stream);
+}
+
+// The row-limit half of an f32 request with a mask tensor (see the kernel): 32 rows per workgroup, one split, no combine
+// pass.  Host has validated what launch_sdpa_decode_f32 asks for, one query head per KV head or S_q a multiple of 128, D and
+// Dv <= 128, and p.mask_lims written.
+hipError_t launch_sdpa_decode_f32_limits(const SdpaParams& p, hipStream_t stream)
+{
+    return p.Dp == 128 ? launch_decode_f32_t<128, 2, 2, true>(p, stream) : launch_decode_f32_t<64, 2, 2, true>(p, stream);
 }
 
 }  // namespace incin_rocm

@@ -91,6 +91,16 @@ void sdpa_prefill_f32_kernel(SdpaParams p)
         lim_wave_max = clampi(min(q0 + wave * 32 + 31, rows_b - 1) + coff + 1, 0, kv_len);
     }
     if (q0 + wave * 32 >= rows_b) lim_wave_min = lim_wave_max = 0;      // a wavefront of padding rows only keeps the barriers company
+    if (DENSE && p.mask_lims != nullptr) {
+        // a launch of the f32 split-KV kernel went before this one and computed the 128-row blocks whose mask rows are all n
+        // zeros and then -inf from their limits (sdpa_decode_f32.hip, LIMS): such a block is done
+        __shared__ int s_ok[4];
+        const bool no_limit = my_i < rows_b && mask_lims_of(p, b, hq)[p.m_si ? my_i : 0] < 0;
+        const bool wave_ok = __builtin_amdgcn_ballot_w64(no_limit) == 0;
+        if (lane == 0) s_ok[wave] = wave_ok ? 1 : 0;
+        __syncthreads();
+        if ((s_ok[0] & s_ok[1] & s_ok[2] & s_ok[3]) != 0) return;      // (uniform)
+    }
     const int n_tiles = (j_end + KT - 1) / KT;
     const int t_first = SPLIT ? min(split * (p.split_len / KT), n_tiles) : 0;
     const int n_act = lim_wave_max > 0 ? (lim_wave_max + KT - 1) / KT : 0;      // tiles this wavefront computes

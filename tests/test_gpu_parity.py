@@ -494,6 +494,42 @@ def test_mask_tensors_whose_rows_are_zeros_then_minus_infinity(gpu, dtype, rows,
     assert np.array_equal(flag, tens, equal_nan=True)
 
 
+@pytest.mark.parametrize("shape", [(2, 3, 3, 300, 400, 64), (1, 4, 2, 256, 256, 128), (2, 2, 2, 130, 500, 128)],
+                         ids=["one_head_per_kv_head", "groups_of_whole_blocks", "a_ragged_last_block"])
+def test_f32_mask_tensors_whose_rows_are_zeros_then_minus_infinity(gpu, shape):
+    """f32, small launches: the 128-row blocks whose mask rows all have a limit are computed by the f32 split-KV kernel from
+    the limits (the kernel AUTO gives such launches when there is no mask tensor), the others by the prefill kernel's
+    dense-mask launch that follows.  Against the oracle at 1e-5; the causal tensor must reproduce the causal flag through
+    the split-KV kernel bit for bit - which also says the limit launch is the one that ran."""
+    B, Hq, Hkv, Sq, Skv, D = shape
+    dt = capi.F32
+    q, k, v = inputs(3200 + Sq + D, B, Hq, Hkv, Sq, Skv, D, D, dt)
+    NEG = -np.inf
+    causal = O.causal_additive_mask(Sq, Skv).reshape(1, 1, Sq, Skv)
+    pad = np.zeros((B, 1, 1, Skv), np.float32)
+    pad[0, ..., Skv - 30:] = NEG
+    pad[-1, ..., 90:] = NEG
+    mixed = np.broadcast_to(causal, (1, Hq, Sq, Skv)).copy()
+    mixed[0, 0, 5:9, :3] = 0.75                                    # head 0, first block: rows with values - that block reads the mask
+    mixed[0, Hq - 1, Sq - 1, 0] = NEG                              # last head, last block: a hole
+    hidden = causal + pad
+    hidden = np.broadcast_to(hidden, (B, 1, Sq, Skv)).copy()
+    hidden[0, 0, 17] = NEG                                         # a row that sees nothing: limit 0, NaN
+    for what, m in (("the causal tensor", causal), ("key padding", pad), ("causal with rows that are not limits", mixed),
+                    ("causal + key padding, one row hidden entirely", hidden)):
+        say("f32 limit masks %r: %s" % (shape, what))
+        m = np.ascontiguousarray(m)
+        got, lse, info = host.sdpa(q, k, v, dt, mask=m, return_info=True, return_lse=True)
+        assert info["impl"] == capi.IMPL_MFMA
+        check(got, oracle_full(q, k, v, G=Hq // Hkv, mask=m), TOL[dt], what)
+        _, lse_g = host.sdpa(q, k, v, dt, mask=m, impl=capi.IMPL_GENERIC, return_lse=True)
+        fin = np.isfinite(lse_g)
+        assert np.array_equal(np.isfinite(lse), fin) and np.max(np.abs(lse[fin] - lse_g[fin])) < 2e-5, what
+    flag = host.sdpa(q, k, v, dt, causal=True, impl=capi.IMPL_SPLITKV_MFMA, num_splits=1)
+    tens = host.sdpa(q, k, v, dt, mask=causal)
+    assert np.array_equal(flag, tens, equal_nan=True)
+
+
 # ---- split-KV decode -----------------------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", [capi.BF16, capi.F16, capi.F32])
