@@ -23,7 +23,7 @@ EXPORTS = [
     "incin_rocm_sizeof_sdpa_desc", "incin_rocm_sizeof_device_info",
     "incin_rocm_device_count", "incin_rocm_device_info",
     "incin_rocm_alloc", "incin_rocm_free", "incin_rocm_memset",
-    "incin_rocm_memcpy_h2d", "incin_rocm_memcpy_d2h", "incin_rocm_memcpy_d2d", "incin_rocm_copy_strided", "incin_rocm_sum_to_shape", "incin_rocm_sync",
+    "incin_rocm_memcpy_h2d", "incin_rocm_memcpy_d2h", "incin_rocm_memcpy_d2d", "incin_rocm_copy_strided", "incin_rocm_sum_to_shape", "incin_rocm_mask_row_limits", "incin_rocm_sync",
     "incin_rocm_stream_create", "incin_rocm_stream_destroy", "incin_rocm_stream_sync",
     "incin_rocm_event_create", "incin_rocm_event_destroy", "incin_rocm_event_record",
     "incin_rocm_event_sync", "incin_rocm_event_query", "incin_rocm_event_elapsed_ms",
@@ -134,6 +134,7 @@ def load():
     lib.incin_rocm_sync.argtypes = [C.c_int32]
     lib.incin_rocm_copy_strided.argtypes = [C.c_int32, C.c_void_p, C.c_void_p, C.c_int32, C.POINTER(C.c_int64), C.POINTER(C.c_int64),
                                             C.c_int32, C.c_void_p]
+    lib.incin_rocm_mask_row_limits.argtypes = [C.c_int32, C.c_int32, C.c_void_p, C.POINTER(C.c_int64), C.POINTER(C.c_int64), C.c_void_p, C.c_void_p]
     lib.incin_rocm_sum_to_shape.argtypes = [C.c_int32, C.c_int32, C.c_void_p, C.c_void_p, C.c_int32, C.POINTER(C.c_int64), C.POINTER(C.c_int64),
                                             C.c_void_p]
     lib.incin_rocm_device_count.argtypes = [C.POINTER(C.c_int32)]

@@ -25,6 +25,7 @@ hipError_t launch_matrix_rate(const void* src, void* sink, int mix, int iteratio
 hipError_t launch_sdpa_prefill_f32(const SdpaParams& p, hipStream_t stream);
 hipError_t launch_sdpa_prefill_wide(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_mask_classify(const SdpaParams& p, int dtype, hipStream_t stream);
+hipError_t launch_mask_row_limits(const void* mask, int dtype, const int64_t shape[4], const int64_t strides[4], int32_t* lims, hipStream_t stream);
 hipError_t launch_sdpa_decode_f32_limits(const SdpaParams& p, hipStream_t stream);
 hipError_t launch_sdpa_decode(const SdpaParams& p, int dtype, hipStream_t stream);
 hipError_t launch_sdpa_decode_mfma(const SdpaParams& p, int dtype, hipStream_t stream);
@@ -611,6 +612,24 @@ int incin_rocm_sum_to_shape(int32_t dev, int32_t dtype, void* dst, const void* s
     p.dst = (char*)dst;
     p.dtype = dtype;
     HIP_TRY(incin_rocm::launch_sum_to_shape(p, (hipStream_t)stream), "sum_to_shape launch");
+    return 0;
+}
+
+int incin_rocm_mask_row_limits(int32_t dev, int32_t dtype, const void* mask, const int64_t* shape, const int64_t* strides, int32_t* lims, void* stream)
+{
+    if (dtype != INCIN_ROCM_F32 && dtype != INCIN_ROCM_F16 && dtype != INCIN_ROCM_BF16)
+        return fail(INCIN_ROCM_EDTYPE, "mask_row_limits: unsupported dtype tag %d on backend Rocm (f32, f16, bf16 only)", dtype);
+    if (!shape || !strides) return fail(INCIN_ROCM_EINVAL, "mask_row_limits: null shape");
+    int64_t rows = 1;
+    for (int a = 0; a < 4; ++a) {
+        if (shape[a] < 0 || shape[a] > 0x7fffffffLL) return fail(INCIN_ROCM_ESHAPE, "mask_row_limits: extent %lld of axis %d", (long long)shape[a], a);
+        if (a < 3) rows *= shape[a];
+        if (rows > (1LL << 40)) return fail(INCIN_ROCM_ESHAPE, "mask_row_limits: mask too large");
+    }
+    if (rows == 0) return 0;
+    if (!lims || (!mask && shape[3] > 0)) return fail(INCIN_ROCM_EINVAL, "mask_row_limits: null pointer");
+    if (int rc = use_device(dev)) return rc;
+    HIP_TRY(incin_rocm::launch_mask_row_limits(mask, dtype, shape, strides, lims, (hipStream_t)stream), "mask_row_limits launch");
     return 0;
 }
 

@@ -141,4 +141,24 @@ hipError_t launch_mask_classify(const SdpaParams& p, int dtype, hipStream_t stre
     return hipGetLastError();
 }
 
+// The row limits of a mask given by itself: shape [A0, A1, rows, Skv] with element strides (0 where an axis is repeated),
+// one int per (a0, a1, row) in that order.  Behind incin_rocm_mask_row_limits.
+hipError_t launch_mask_row_limits(const void* mask, int dtype, const int64_t shape[4], const int64_t strides[4], int32_t* lims, hipStream_t stream)
+{
+    const int64_t n_rows = shape[0] * shape[1] * shape[2];
+    if (n_rows <= 0) return hipSuccess;
+    if ((n_rows + 3) / 4 > 0x7fffffffLL) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)((n_rows + 3) / 4));
+    const int esz = dtype == 0 ? 4 : 2;
+    const bool vec = strides[3] == 1 && ((uintptr_t)mask % (8 * esz)) == 0 && strides[0] % 8 == 0 && strides[1] % 8 == 0 && strides[2] % 8 == 0;
+#define LIMITS(T, V) hipLaunchKernelGGL((mask_row_limits_kernel<T, V>), grid, dim3(256), 0, stream, (const T*)mask, strides[0], strides[1], strides[2], strides[3], (int)shape[1], (int)shape[2], (int)shape[3], n_rows, lims)
+    switch (dtype) {
+        case 0: if (vec) LIMITS(float, true); else LIMITS(float, false); break;
+        case 1: if (vec) LIMITS(f16_t, true); else LIMITS(f16_t, false); break;
+        default: if (vec) LIMITS(bf16_t, true); else LIMITS(bf16_t, false); break;
+    }
+#undef LIMITS
+    return hipGetLastError();
+}
+
 }  // namespace incin_rocm

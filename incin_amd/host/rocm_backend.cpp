@@ -498,6 +498,65 @@ Error RocmBackend::tag_key_padding(const RocmStorage& mask, const std::vector<in
     return ok();
 }
 
+Error RocmBackend::infer_mask_tag(const RocmStorage& mask, RocmStorage* out, int* kind)
+{
+    *out = mask;
+    if (kind) *kind = 0;
+    const size_t r = mask.shape.size();
+    if (r < 2 || r > 4 || mask.mask_tag) return ok();
+    // [A0, A1, rows, Skv]: missing leading axes are 1
+    int64_t shape[4] = {1, 1, 1, 1}, strides[4] = {0, 0, 0, 0};
+    for (size_t a = 0; a < r; ++a) {
+        shape[4 - r + a] = mask.shape[a];
+        strides[4 - r + a] = mask.shape[a] == 1 ? 0 : mask.strides[a];
+    }
+    const int64_t A0 = shape[0], A1 = shape[1], R = shape[2], Skv = shape[3];
+    const int64_t n = A0 * A1 * R;
+    if (n <= 0 || Skv <= 0 || n > (1 << 26)) return ok();
+    std::shared_ptr<RocmBuffer> lims_dev;
+    if (Error e = alloc_buffer(mask.device, (size_t)n * sizeof(int32_t), &lims_dev)) return e;
+    if (Error e = from_status(incin_rocm_mask_row_limits(mask.device, (int32_t)mask.dtype, mask.data(), shape, strides,
+                                                         static_cast<int32_t*>(lims_dev->ptr()), t_stream), mask.device))
+        return e;
+    if (Error e = from_status(t_stream ? incin_rocm_stream_sync(mask.device, t_stream) : incin_rocm_sync(mask.device), mask.device)) return e;
+    std::vector<int32_t> lims((size_t)n);
+    if (Error e = from_status(incin_rocm_memcpy_d2h(mask.device, lims.data(), lims_dev->ptr(), (size_t)n * sizeof(int32_t)), mask.device)) return e;
+    // per index of the first axis: the count the last row states; then: are all rows that count (key padding), or the smaller
+    // of it and the causal limit of the row (both; without a count below Skv: causal)?
+    std::vector<int32_t> counts((size_t)A0);
+    bool plain = true, causal = R > 1;
+    for (int64_t a0 = 0; a0 < A0; ++a0) {
+        const int32_t L = lims[(size_t)((a0 * A1) * R + (R - 1))];
+        counts[(size_t)a0] = L;
+        for (int64_t a1 = 0; a1 < A1; ++a1)
+            for (int64_t i = 0; i < R; ++i) {
+                const int32_t lm = lims[(size_t)((a0 * A1 + a1) * R + i)];
+                if (lm < 0) return ok();
+                const int64_t c = std::min<int64_t>(std::max<int64_t>(i + 1 + Skv - R, 0), Skv);
+                plain = plain && lm == L;
+                causal = causal && lm == std::min<int64_t>(c, L);
+            }
+    }
+    if (!plain && !causal) return ok();
+    bool padded = false;
+    for (int32_t c : counts) padded = padded || c < Skv;
+    if (!padded) {
+        if (!causal) return ok();               // all zeros: the mask says nothing, and costs nothing that matters as it is
+        out->mask_tag = MaskTag{MaskTag::Causal, nullptr, 0};
+        if (kind) *kind = 1;
+        return ok();
+    }
+    // key counts go by batch entry: only a rank-4 mask with more than one entry on its first axis says which rows of the
+    // scores belong to which (under the operator's right-aligned broadcast a shorter mask's first axis is the head axis,
+    // and a single entry may be repeated over a batch whose size the mask does not know)
+    if (r != 4 || A0 == 1) return ok();
+    std::shared_ptr<RocmBuffer> buf;
+    if (Error e = upload_i32(counts, mask.device, &buf)) return e;
+    out->mask_tag = MaskTag{plain ? MaskTag::KeyPadding : MaskTag::CausalKeyPadding, buf, (int64_t)counts.size()};
+    if (kind) *kind = plain ? 2 : 3;
+    return ok();
+}
+
 Error RocmBackend::scaled_dot_product_attention(const RocmStorage& q, const RocmStorage& k, const RocmStorage& v,
                                                 const RocmStorage* mask, std::optional<double> scale, RocmStorage* out)
 {
@@ -751,8 +810,8 @@ Error RocmBackend::attention_impl(const RocmStorage& q, const RocmStorage& k, co
     d.v_stride[0] = st(vs, b_ax); d.v_stride[1] = st(vs, kv_head_ax); d.v_stride[2] = v.strides[vr - 2];
     d.scale = (float)s64;                                                   // elementwise_kernel.rs:87
     if (mask && mask->mask_tag) {
-        if (mask->mask_tag->kind == MaskTag::Causal) d.causal = 1;
-        else {
+        if (mask->mask_tag->kind != MaskTag::KeyPadding) d.causal = 1;
+        if (mask->mask_tag->kind != MaskTag::Causal) {
             if (mask->mask_tag->lens_count != B || n_outer != 0 || (g_ax >= 0 && !fold_g && h_ax >= 0))
                 return err(ErrorKind::ShapeMismatch, std::string(OP) + ": key-padding lengths must have one entry per batch index");
             d.kv_lens = static_cast<const int32_t*>(mask->mask_tag->lens->ptr());

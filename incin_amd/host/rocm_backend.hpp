@@ -61,8 +61,8 @@ class RocmBuffer {
 
 // What a mask storage may declare about its contents so the backend need not read them.
 struct MaskTag {
-    enum Kind { Causal, KeyPadding } kind;
-    std::shared_ptr<RocmBuffer> lens;      // KeyPadding: int32 key counts, one per batch entry
+    enum Kind { Causal, KeyPadding, CausalKeyPadding } kind;      // (the last: the sum of the two masks)
+    std::shared_ptr<RocmBuffer> lens;      // KeyPadding, CausalKeyPadding: int32 key counts, one per batch entry
     int64_t lens_count = 0;
 };
 
@@ -130,6 +130,16 @@ struct RocmBackend {
     // and -inf for the rest, constant over query rows and heads.
     static Error tag_causal(const RocmStorage& mask, RocmStorage* out);
     static Error tag_key_padding(const RocmStorage& mask, const std::vector<int32_t>& lens, RocmStorage* out);
+    // The same declarations read off the mask's contents.  The reference's operator knows a mask only as a tensor
+    // (cpu/ops/shape_ops.rs:1262-1266), and its callers build the causal mask as full(-inf).triu(1), key padding as 0 / -inf
+    // per key and add the two: every row of such a mask is n zeros followed by -inf.  This reads the mask once on the
+    // device (incin_rocm_mask_row_limits), waits for the result - the one synchronisation, which is why it is a call of its
+    // own and not part of the operator: a backend makes it where the mask is made, once per mask - and tags `out` as
+    // Causal, KeyPadding (one count per index of the first axis) or both, if that is what the rows say: *kind 0 none (out is
+    // the mask untouched: values, holes, a window, counts the tag could not hold), 1 causal, 2 key padding, 3 both.  A tagged
+    // mask runs on the facts in the forward and - where a mask tensor would send the gradients to the generic kernels -
+    // in the backward.  Masks of rank 2 to 4.
+    static Error infer_mask_tag(const RocmStorage& mask, RocmStorage* out, int* kind);
 
     // TensorOps::scaled_dot_product_attention.
     static Error scaled_dot_product_attention(const RocmStorage& q, const RocmStorage& k, const RocmStorage& v,

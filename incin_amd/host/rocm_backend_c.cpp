@@ -105,6 +105,15 @@ int incin_host_tag_key_padding(const incin_host_storage* mask, const int32_t* le
     return give(e, std::move(r), out);
 }
 
+int incin_host_infer_mask_tag(const incin_host_storage* mask, int32_t* kind, incin_host_storage** out)
+{
+    RocmStorage r;
+    int k = 0;
+    Error e = RocmBackend::infer_mask_tag(mask->s, &r, &k);
+    if (kind) *kind = k;
+    return give(e, std::move(r), out);
+}
+
 int incin_host_scaled_dot_product_attention(const incin_host_storage* q, const incin_host_storage* k, const incin_host_storage* v,
                                             const incin_host_storage* mask, int32_t has_scale, double scale,
                                             incin_host_storage** out)

@@ -26,6 +26,8 @@ int incin_host_broadcast_as(const incin_host_storage* s, const int64_t* dims, in
 int incin_host_narrow(const incin_host_storage* s, int32_t dim, int64_t start, int64_t len, incin_host_storage** out);
 int incin_host_tag_causal(const incin_host_storage* mask, incin_host_storage** out);
 int incin_host_tag_key_padding(const incin_host_storage* mask, const int32_t* lens, int64_t count, incin_host_storage** out);
+/* *kind: 0 untagged (out is the mask as it was), 1 causal, 2 key padding, 3 both; reads the mask on the device and waits */
+int incin_host_infer_mask_tag(const incin_host_storage* mask, int32_t* kind, incin_host_storage** out);
 /* mask may be null; has_scale = 0 means Option::None (default 1/sqrt(D)) */
 int incin_host_scaled_dot_product_attention(const incin_host_storage* q, const incin_host_storage* k, const incin_host_storage* v,
                                             const incin_host_storage* mask, int32_t has_scale, double scale,

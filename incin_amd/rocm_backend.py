@@ -23,7 +23,7 @@ KINDS = ["None", "Msg", "ShapeMismatch", "DTypeStorageMismatch", "DeviceMismatch
 EXPORTS = [
     "incin_host_last_error", "incin_host_from_bytes", "incin_host_numel", "incin_host_rank", "incin_host_shape", "incin_host_strides",
     "incin_host_dtype", "incin_host_to_bytes", "incin_host_transpose", "incin_host_broadcast_as",
-    "incin_host_narrow", "incin_host_tag_causal", "incin_host_tag_key_padding",
+    "incin_host_narrow", "incin_host_tag_causal", "incin_host_tag_key_padding", "incin_host_infer_mask_tag",
     "incin_host_scaled_dot_product_attention", "incin_host_attention_backward", "incin_host_release", "incin_host_last_launch_count",
     "incin_host_capability_name", "incin_host_capability_max_rank", "incin_host_capability_support",
     "incin_host_capability_rule_count", "incin_host_capability_rule", "incin_host_capability_docs",
@@ -68,6 +68,7 @@ def lib():
         L.incin_host_narrow.argtypes = [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.POINTER(C.c_void_p)]
         L.incin_host_tag_causal.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
         L.incin_host_tag_key_padding.argtypes = [C.c_void_p, C.POINTER(C.c_int32), C.c_int64, C.POINTER(C.c_void_p)]
+        L.incin_host_infer_mask_tag.argtypes = [C.c_void_p, C.POINTER(C.c_int32), C.POINTER(C.c_void_p)]
         L.incin_host_scaled_dot_product_attention.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32,
                                                               C.c_double, C.POINTER(C.c_void_p)]
         L.incin_host_attention_backward.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_double, C.c_void_p] + \
@@ -227,6 +228,14 @@ class RocmStorage:
 
     def tag_causal(self):
         return self._view(lib().incin_host_tag_causal)
+
+    def infer_mask_tag(self):
+        """(storage, kind): the mask tagged with what its rows state - kind 1 causal, 2 key padding, 3 both - or, kind 0,
+        the mask as it was.  Reads the mask on the device and waits for the answer: once per mask, where it is made."""
+        kind = C.c_int32(0)
+        out = C.c_void_p()
+        _check(lib().incin_host_infer_mask_tag(self._h, C.byref(kind), C.byref(out)))
+        return RocmStorage(out.value), int(kind.value)
 
     def tag_key_padding(self, lens):
         arr = (C.c_int32 * max(len(lens), 1))(*[int(x) for x in lens])

@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define INCIN_ROCM_ABI_VERSION 10
+#define INCIN_ROCM_ABI_VERSION 11
 
 /* ---- status codes (mapped to incin_core::Error variants by the Rust side;
  *      crates/incin-core/src/err.rs:109-223) --------------------------------- */
@@ -113,6 +113,15 @@ int incin_rocm_copy_strided(int32_t dev, void* dst, const void* src, int32_t ran
  * axes in the target pads its shape with 1s.  dtype: INCIN_ROCM_F32 / F16 / BF16.  Enqueued on `stream`. */
 int incin_rocm_sum_to_shape(int32_t dev, int32_t dtype, void* dst, const void* src, int32_t rank, const int64_t* src_shape,
                             const int64_t* dst_shape, void* stream);
+/* What a mask tensor of zeros and -inf states, row by row.  The reference's operator takes its mask as a tensor only
+ * (crates/incin-backends/src/cpu/ops/shape_ops.rs:1262-1266) and its callers build the causal mask as
+ * full(-inf).triu(1) and key padding as 0 / -inf per key: every row of such a mask is n zeros followed by -inf.  For a mask
+ * of shape [A0, A1, rows, Skv] (`shape`, `strides` in elements, 0 on a repeated axis) this writes one int per
+ * (a0, a1, row), in that order, to `lims`: n if the row has that form (n = Skv: all zeros, n = 0: all -inf), else -1.
+ * A backend that reads the result back can state the mask as `causal` / `kv_lens` in the descriptors (forward and backward)
+ * instead of passing the tensor.  Enqueued on `stream`; a row with Skv = 0 gets 0. */
+int incin_rocm_mask_row_limits(int32_t dev, int32_t dtype, const void* mask, const int64_t* shape, const int64_t* strides, int32_t* lims,
+                               void* stream);
 int incin_rocm_sync(int32_t dev);      /* waits for the device's default stream and any stream created here */
 
 /* ---- streams and events -------------------------------------------------------

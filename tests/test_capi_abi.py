@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), "missing export %s" % n
     assert set(names) == set(capi.EXPORTS)
-    assert lib.incin_rocm_abi_version() == 10
+    assert lib.incin_rocm_abi_version() == 11
 
 
 def test_descriptor_layout_matches():
@@ -218,6 +218,18 @@ def test_null_descriptor_and_missing_workspace():
         capi.sdpa_fwd(d)
     assert e.value.code == capi.EWORKSPACE
     assert lib.incin_rocm_device_count(None) == capi.EINVAL
+
+
+def test_mask_row_limits_validation():
+    """incin_rocm_mask_row_limits refuses what it cannot read before it touches a device."""
+    lib = capi.load()
+    shape = (C.c_int64 * 4)(1, 1, 8, 16)
+    strides = (C.c_int64 * 4)(0, 0, 16, 1)
+    assert lib.incin_rocm_mask_row_limits(0, 7, 0x1000, shape, strides, 0x2000, None) == capi.EDTYPE
+    assert lib.incin_rocm_mask_row_limits(0, capi.F32, 0x1000, None, strides, 0x2000, None) == capi.EINVAL
+    assert lib.incin_rocm_mask_row_limits(0, capi.F32, 0x1000, (C.c_int64 * 4)(1, -1, 8, 16), strides, 0x2000, None) == capi.ESHAPE
+    assert lib.incin_rocm_mask_row_limits(0, capi.F32, 0x1000, shape, strides, None, None) == capi.EINVAL
+    assert lib.incin_rocm_mask_row_limits(0, capi.F32, None, (C.c_int64 * 4)(1, 1, 0, 16), strides, None, None) == 0      # no rows: nothing to do
 
 
 def test_matrix_rate_validation():

@@ -130,6 +130,62 @@ def test_tagged_masks_equal_their_dense_form(gpu, dtype):
     close(RB.scaled_dot_product_attention(Q, K, V, P.tag_key_padding(lens)).to_numpy(), ref, TOL[dtype], "tagged padding")
 
 
+@pytest.mark.parametrize("dtype", [RB.F32, RB.BF16])
+def test_mask_tags_read_off_the_mask(gpu, dtype):
+    """infer_mask_tag: the causal mask as its callers build it, a key-padding mask and their sum are recognised from their
+    rows (n zeros, then -inf) and tagged; anything else - values, a hole, a window, counts the tag cannot hold - comes back
+    as it was.  A tagged mask gives what the tensor gives, forward and backward (where a mask tensor sends the gradients to
+    the generic kernels and the tag does not)."""
+    from oracle import sdpa_backward as BW
+    B, H, Sq, Skv, D = 3, 2, 70, 100, 64
+    q, k, v, go = rnd(60, (B, H, Sq, D), dtype), rnd(61, (B, H, Skv, D), dtype), rnd(62, (B, H, Skv, D), dtype), rnd(63, (B, H, Sq, D), dtype)
+    S = lambda a: RB.RocmStorage.from_numpy(a, dtype)
+    Q, K, V, GO = S(q), S(k), S(v), S(go)
+    NEG = -np.inf
+    causal = O.causal_additive_mask(Sq, Skv)                                   # [Sq, Skv], aligned to the last key
+    pad = np.zeros((B, 1, 1, Skv), np.float32)
+    for b, n in enumerate((100, 33, 71)):
+        pad[b, ..., n:] = NEG
+    both = causal[None, None] + pad
+    cases = [("causal [Sq,Skv]", causal, 1), ("causal [1,1,Sq,Skv]", causal[None, None], 1), ("causal [H,Sq,Skv]", np.broadcast_to(causal, (H, Sq, Skv)).copy(), 1),
+             ("key padding [B,1,1,Skv]", pad, 2), ("key padding [B,H,Sq,Skv]", np.broadcast_to(pad, (B, H, Sq, Skv)).copy(), 2),
+             ("causal + key padding [B,1,Sq,Skv]", both, 3)]
+    window = causal.copy()
+    window[np.tril(np.ones((Sq, Skv), bool), Skv - Sq - 20)] = NEG             # a sliding window: rows start with -inf
+    hole = causal.copy()
+    hole[40, 3] = NEG
+    values = causal.copy()
+    values[10, 2] = -0.5
+    one_padded = np.zeros((1, 1, 1, Skv), np.float32)
+    one_padded[..., 50:] = NEG                                                 # one entry for a batch of unknown size: not tagged
+    cases += [("window", window, 0), ("hole", hole, 0), ("values", values, 0), ("all zeros", np.zeros((Sq, Skv), np.float32), 0),
+              ("one padded entry [1,1,1,Skv]", one_padded, 0), ("padding per head [H,1,Skv]", pad[:H, 0], 0)]
+    tol = TOL[dtype]
+    for what, m, kind in cases:
+        say("host mirror: inferred mask tag, dtype %d: %s" % (dtype, what))
+        M = S(np.ascontiguousarray(m))
+        T, got_kind = M.infer_mask_tag()
+        assert got_kind == kind, what
+        assert T.shape == M.shape
+        ref = O.sdpa(q, k, v, mask=m)
+        close(RB.scaled_dot_product_attention(Q, K, V, T).to_numpy(), ref, tol, what)
+        if kind == 0 and what not in ("window", "hole"):
+            continue
+        out, dq, dk, dv = RB.attention_backward(Q, K, V, GO, T)
+        rq, rk, rv = BW.sdpa_backward(q, k, v, go, mask=m)
+        gtol = 1e-5 if dtype == RB.F32 else 2e-2
+        grad_close("dq " + what, dq.to_numpy(), rq, gtol)
+        grad_close("dk " + what, dk.to_numpy(), rk, gtol)
+        grad_close("dv " + what, dv.to_numpy(), rv, gtol)
+    # a tag is kept, not inferred again; a view of a mask is read through its strides
+    T, kind = S(causal).tag_causal().infer_mask_tag()
+    assert kind == 0
+    wide = np.full((Sq, Skv + 12), 7.0, np.float32)                            # a mask inside a wider buffer whose padding is not a mask
+    wide[:, :Skv] = causal
+    T, kind = S(wide).narrow(1, 0, Skv).infer_mask_tag()
+    assert kind == 1
+
+
 def test_key_lengths_with_one_shared_kv_head(gpu):
     # rank-4 multi-query layout: q [B,H,S,D] against k, v [B,1,S,D]; the key counts are per batch entry
     say("host mirror: multi-query operands with tagged key padding")
