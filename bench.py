@@ -706,6 +706,7 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--with-mask-tensor", action="store_true", help="with --only prefill: also the launch with the causal mask as a tensor (for profiles)")
     ap.add_argument("--no-padding-compare", action="store_true",
                     help="prefill_long: skip the extra timing of the batch with its padding rows computed (profiling: every "
                          "launch of the run is then the same launch)")
@@ -764,7 +765,7 @@ def main():
                               "traffic_source": traffic_of("prefill")[1], "kernel": "sdpa_prefill_mfma_kernel<bf16,128>", "algorithmic_flops_per_launch": flops,
                               "launch_ms_mean": ev_mean, "launch_ms_median": ev_med, "launch_ms_min": ev_min}
         result["parity_max_abs_err"] = w.parity()
-        if args.only is None:
+        if args.only is None or args.with_mask_tensor:
             # the same batch with the causal mask handed over the way the reference's operator takes it: an explicit
             # [S, S] tensor of 0 / -inf (bf16, broadcast over batch and heads) instead of the causal flag
             from oracle import oracle as O
@@ -778,7 +779,8 @@ def main():
             wall_m = w.time(args.steps, args.warmup)[0]
             result["prefill_with_dense_mask_tensor"] = {
                 "what": "config 3 with the causal mask passed as a bf16 [S, S] additive tensor (add_mask); the launch classifies it "
-                        "by 32 x 32 blocks first; same FLOP count", "ms_per_step": wall_m, "value": flops / (wall_m * 1e-3) / 1e12,
+                        "by 32 x 32 blocks and takes a limit per mask row first, then runs the blocks whose rows all have a limit "
+                        "from the limits; same FLOP count", "ms_per_step": wall_m, "value": flops / (wall_m * 1e-3) / 1e12,
                 "unit": "TFLOP/s", "ratio_to_causal_flag": wall / wall_m, "parity_max_abs_err": w.parity()}
             tm.free()
             mws.free()

@@ -182,22 +182,13 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     if ((DENSE || LIMS) && p.mask_lims != nullptr) {
         // does every row of the block of lims_rows rows around this workgroup's have a limit?  (uniform over the workgroup)
         const int32_t* lims = mask_lims_of(p, b, hq);
-        const int blk0 = (q0 / p.lims_rows) * p.lims_rows, blk1 = min(blk0 + p.lims_rows, rows_b);
-        bool ok = true;
-        for (int i = blk0 + tid; i < blk1; i += 64 * NW) ok = ok && lims[p.m_si ? i : 0] >= 0;
-        const bool wave_ok = __builtin_amdgcn_ballot_w64(!ok) == 0;
-        if (lane == 0) s_range[wave] = wave_ok ? 1 : 0;
-        __syncthreads();
-        bool all = true;
-#pragma unroll
-        for (int w2 = 0; w2 < NW; ++w2) all = all && s_range[w2] != 0;
-        all = __builtin_amdgcn_readfirstlane(all ? 1 : 0) != 0;
-        if (all != LIMS) return;                           // the other launch computes this block
-        __syncthreads();                                   // (s_range is used again below)
         if (LIMS) {
-            // this lane's limit, the smallest and largest of the wavefront, the largest of the workgroup
+            // (the block is this workgroup's: one row per lane, and one exchange through LDS says both whether every row has a
+            // limit and what the largest is) this lane's limit, the smallest and largest of the wavefront, the largest of the workgroup
             const bool row_here = my_i < rows_b;
-            lim_lane = row_here ? min(lim_lane, lims[p.m_si ? my_i : 0]) : 0;
+            const int lm = lims[p.m_si ? min(my_i, Sq - 1) : 0];
+            const bool wave_ok = __builtin_amdgcn_ballot_w64(row_here && lm < 0) == 0;
+            lim_lane = row_here ? min(lim_lane, lm) : 0;
             int lo = row_here ? lim_lane : 0x7fffffff, hi = lim_lane;
 #pragma unroll
             for (int off = 32; off >= 1; off >>= 1) {
@@ -206,13 +197,27 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
             }
             lim_wave_min = __builtin_amdgcn_readfirstlane(lo == 0x7fffffff ? 0 : lo);
             lim_wave_max = __builtin_amdgcn_readfirstlane(hi);
-            if (lane == 0) s_range[wave] = lim_wave_max;
+            if (lane == 0) { s_range[wave] = wave_ok ? 1 : 0; s_range[NW + wave] = lim_wave_max; }
             __syncthreads();
+            bool all = true;
             int je = 0;
 #pragma unroll
-            for (int w2 = 0; w2 < NW; ++w2) je = max(je, s_range[w2]);
+            for (int w2 = 0; w2 < NW; ++w2) { all = all && s_range[w2] != 0; je = max(je, s_range[NW + w2]); }
+            if (__builtin_amdgcn_readfirstlane(all ? 1 : 0) == 0) return;      // the dense-mask launch computes this block
             j_end = __builtin_amdgcn_readfirstlane(je);
             n_tiles = (j_end + PF_BN - 1) / PF_BN;
+        } else {
+            const int blk0 = (q0 / p.lims_rows) * p.lims_rows, blk1 = min(blk0 + p.lims_rows, rows_b);
+            bool ok = true;
+            for (int i = blk0 + tid; i < blk1; i += 64 * NW) ok = ok && lims[p.m_si ? i : 0] >= 0;
+            const bool wave_ok = __builtin_amdgcn_ballot_w64(!ok) == 0;
+            if (lane == 0) s_range[wave] = wave_ok ? 1 : 0;
+            __syncthreads();
+            bool all = true;
+#pragma unroll
+            for (int w2 = 0; w2 < NW; ++w2) all = all && s_range[w2] != 0;
+            if (__builtin_amdgcn_readfirstlane(all ? 1 : 0) != 0) return;      // the launch before this one computed the block from its limits
+            __syncthreads();                                                   // (s_range is used again below)
         }
     }
     const bool flags_in_lds = DENSE && n_tiles <= FLAG_TILES;

@@ -98,18 +98,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const uint8_t* mflags = nullptr;
     __shared__ int s_range[8];
     if ((DENSE || LIMS) && p.mask_lims != nullptr) {
-        // does every row of this workgroup have a limit?  (uniform over the workgroup)
+        // does every row of this workgroup have a limit?  One exchange through LDS says that and, for LIMS, the largest limit.
         const int32_t* lims = mask_lims_of(p, b, hq);
         const bool row_here = my_i < rows_b;
         const int lm = lims[p.m_si ? min(my_i, Sq - 1) : 0];
         const bool wave_ok = __builtin_amdgcn_ballot_w64(row_here && lm < 0) == 0;
-        if (lane == 0) s_range[wave] = wave_ok ? 1 : 0;
-        __syncthreads();
-        const bool all = __builtin_amdgcn_readfirstlane((s_range[0] & s_range[1] & s_range[2] & s_range[3]) != 0 ? 1 : 0) != 0;
-        if (all != LIMS) return;                           // the other launch computes this block
-        __syncthreads();                                   // (s_range is used again below)
         if (LIMS) {
-            // this lane's limit, the smallest and largest of the wavefront, the largest of the workgroup
+            // this lane's limit, the smallest and largest of the wavefront
             lim_lane = row_here ? min(lim_lane, lm) : 0;
             int lo = row_here ? lim_lane : 0x7fffffff, hi = lim_lane;
 #pragma unroll
@@ -119,12 +114,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             }
             lim_wave_min = __builtin_amdgcn_readfirstlane(lo == 0x7fffffff ? 0 : lo);
             lim_wave_max = __builtin_amdgcn_readfirstlane(hi);
-            if (lane == 0) s_range[wave] = lim_wave_max;
-            __syncthreads();
-            j_end = __builtin_amdgcn_readfirstlane(max(max(s_range[0], s_range[1]), max(s_range[2], s_range[3])));
+        }
+        if (lane == 0) { s_range[wave] = wave_ok ? 1 : 0; s_range[4 + wave] = lim_wave_max; }
+        __syncthreads();
+        const bool all = __builtin_amdgcn_readfirstlane((s_range[0] & s_range[1] & s_range[2] & s_range[3]) != 0 ? 1 : 0) != 0;
+        if (all != LIMS) return;                           // the other launch computes this block
+        if (LIMS) {
+            j_end = __builtin_amdgcn_readfirstlane(max(max(s_range[4], s_range[5]), max(s_range[6], s_range[7])));
             n_tiles = (j_end + PW_KT - 1) / PW_KT;
             n_act = lim_wave_max > 0 ? (lim_wave_max + PW_KT - 1) / PW_KT : 0;
         }
+        __syncthreads();                                   // (s_range is used again below)
     }
     if (DENSE) {
         mrow = (const T*)p.mask + (int64_t)b * p.m_sb + (int64_t)hq * p.m_sh + (int64_t)min(my_i, Sq - 1) * p.m_si;
