@@ -14,10 +14,19 @@ namespace incin_rocm {
 
 template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void mask_classify_kernel(const T* mask, int64_t m_sb, int64_t m_sh, int64_t m_si, int64_t m_sj,
-                                                           int Hm, int Sq, int Skv, int nkb, uint8_t* flags)
+                                                           int Hm, int Sq, int Skv, int nkb, uint8_t* flags, const int32_t* lims, int rows_m)
 {
     __shared__ int votes[8][2];
     const int strip = blockIdx.x, rb = blockIdx.y, bh = blockIdx.z;
+    if (lims != nullptr) {
+        // Row limits are known (mask_row_limits_kernel ran before): the attention launches read the flags only of blocks of 128
+        // or 256 rows in which some row has no limit.  If every row of the 256 around these 32 has one, nobody will ask.
+        const int blk0 = (rb * 32 / 256) * 256, blk1 = min(blk0 + 256, Sq);
+        const int32_t* l = lims + (int64_t)bh * rows_m;
+        bool ok = true;
+        for (int i = blk0 + (int)threadIdx.x; i < blk1; i += 256) ok = ok && l[rows_m > 1 ? i : 0] >= 0;
+        if (__syncthreads_and(ok)) return;
+    }
     const int b = bh / Hm, h = bh % Hm;
     const T* base = mask + (int64_t)b * m_sb + (int64_t)h * m_sh;
     const int c8 = threadIdx.x & 31, r0 = threadIdx.x >> 5;       // 8 keys starting at strip * 256 + c8 * 8; rows r0, r0 + 8, ..
@@ -119,15 +128,8 @@ hipError_t launch_mask_classify(const SdpaParams& p, int dtype, hipStream_t stre
     const int esz = dtype == 0 ? 4 : 2;
     // 8 consecutive elements in one vector load: unit key stride, every row start a multiple of the vector
     const bool vec = p.m_sj == 1 && ((uintptr_t)p.mask % (8 * esz)) == 0 && p.m_sb % 8 == 0 && p.m_sh % 8 == 0 && p.m_si % 8 == 0;
-#define CLASSIFY(T, V) hipLaunchKernelGGL((mask_classify_kernel<T, V>), grid, dim3(256), 0, stream, (const T*)p.mask, p.m_sb, p.m_sh, p.m_si, p.m_sj, Hm, p.Sq, p.Skv, nkb, flags)
-    switch (dtype) {
-        case 0: if (vec) CLASSIFY(float, true); else CLASSIFY(float, false); break;
-        case 1: if (vec) CLASSIFY(f16_t, true); else CLASSIFY(f16_t, false); break;
-        default: if (vec) CLASSIFY(bf16_t, true); else CLASSIFY(bf16_t, false); break;
-    }
-#undef CLASSIFY
-    if (p.mask_lims) {
-        const int rows_m = p.m_si ? p.Sq : 1;
+    const int rows_m = p.m_si ? p.Sq : 1;
+    if (p.mask_lims) {       // the limits first: the flags of blocks whose rows all have one are not needed
         const int64_t n_rows = (int64_t)Bm * Hm * rows_m;
         const dim3 lgrid((unsigned)((n_rows + 3) / 4));
 #define LIMITS(T, V) hipLaunchKernelGGL((mask_row_limits_kernel<T, V>), lgrid, dim3(256), 0, stream, (const T*)p.mask, p.m_sb, p.m_sh, p.m_si, p.m_sj, Hm, rows_m, p.Skv, n_rows, (int32_t*)p.mask_lims)
@@ -138,6 +140,13 @@ hipError_t launch_mask_classify(const SdpaParams& p, int dtype, hipStream_t stre
         }
 #undef LIMITS
     }
+#define CLASSIFY(T, V) hipLaunchKernelGGL((mask_classify_kernel<T, V>), grid, dim3(256), 0, stream, (const T*)p.mask, p.m_sb, p.m_sh, p.m_si, p.m_sj, Hm, p.Sq, p.Skv, nkb, flags, p.mask_lims, rows_m)
+    switch (dtype) {
+        case 0: if (vec) CLASSIFY(float, true); else CLASSIFY(float, false); break;
+        case 1: if (vec) CLASSIFY(f16_t, true); else CLASSIFY(f16_t, false); break;
+        default: if (vec) CLASSIFY(bf16_t, true); else CLASSIFY(bf16_t, false); break;
+    }
+#undef CLASSIFY
     return hipGetLastError();
 }
 
