@@ -931,7 +931,7 @@ static int check_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, bool* empty, int* kin
     const bool f32 = d->dtype == INCIN_ROCM_F32;
     const int vec = f32 ? 4 : 8;
     // (head dimensions up to 128 in whole 16-byte vectors, D and Dv not necessarily equal: zero-padded into the 64 / 128 instances)
-    bool ok = d->D > 0 && d->D <= 128 && d->Dv <= 128 && d->D % vec == 0 && d->Dv % vec == 0 && !d->add_mask && std::isfinite(d->scale) && (f32 || d->scale > 0.0f);
+    bool ok = d->D > 0 && d->D <= 128 && d->Dv <= 128 && d->D % vec == 0 && d->Dv % vec == 0 && (!d->add_mask || !f32) && std::isfinite(d->scale) && (f32 || d->scale > 0.0f);
     ok = ok && fast_layout_ok(d, vec) && aligned16(bd->d_o) && aligned16(bd->d_q) && aligned16(bd->d_k) && aligned16(bd->d_v);
     for (int a = 0; a < 3; ++a)
         ok = ok && bd->d_o_stride[a] % vec == 0 && bd->d_q_stride[a] % vec == 0 && bd->d_k_stride[a] % vec == 0 && bd->d_v_stride[a] % vec == 0;
@@ -944,7 +944,7 @@ static int check_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, bool* empty, int* kin
     else if (d->impl == INCIN_ROCM_IMPL_MFMA) {
         if (!ok)
             return fail(INCIN_ROCM_EUNSUPPORTED, "%s: the MFMA kernels need D and Dv <= 128 in whole 16-byte vectors, a finite scale (f16 / bf16: "
-                        "positive), no dense mask, and rows 16-byte aligned with strides that are multiples of 16 bytes below 2^%d elements",
+                        "positive), no dense mask in f32, and rows 16-byte aligned with strides that are multiples of 16 bytes below 2^%d elements",
                         OP, f32 ? 22 : 24);
         *kind = fast;
     } else

@@ -125,7 +125,9 @@ struct BwdTiles {
 };
 
 // ---- dQ ----------------------------------------------------------------------------------------------------------------
-template <typename T, int D>
+// DENSE: a dense additive mask - its values (times log2 e) are added to the scores before the exponential, fetched while
+// the matrix instructions of the scores run; what the mask hides (-inf) ends as P = 0 like the causal edge.
+template <typename T, int D, bool DENSE = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
 {
@@ -202,6 +204,8 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
     __syncthreads();      // every wavefront has its rows out of the V buffers
     if (n_tiles > 0) tl.issue(1, vp, p.v_ss, Skv, 0, lds0 + 2 * L::TILE_BYTES, wave);
     const int64_t stat = ((int64_t)b * p.Hq + hq) * Sq + qi;
+    [[maybe_unused]] const T* mrow = nullptr;      // DENSE: this lane's row of the mask
+    if (DENSE) mrow = (const T*)p.mask + (int64_t)b * p.m_sb + (int64_t)hq * p.m_sh + (int64_t)qi * p.m_si;
     const float l2 = -bp.neg_l2[stat];
     const float dlt = -bp.neg_delta[stat];
 
@@ -242,10 +246,27 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
                 for (int r = 0; r < 16; ++r)
                     if (8 * (r / 4) + (r % 4) >= rel) s_acc[r] = -INFINITY;
             }
+            typedef T vec4 __attribute__((ext_vector_type(4)));
+            [[maybe_unused]] vec4 mv[4];
+            if (DENSE) {      // the mask's values of this lane's 16 keys, asked for ahead of the products
+#pragma unroll
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    const int j = j0 + 32 * kb + 8 * r4 + 4 * g;
+                    if (p.mask_vec && j + 3 < Skv) mv[r4] = *(const vec4*)(mrow + j);
+                    else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) mv[r4][e] = mrow[(int64_t)min(j + e, Skv - 1) * p.m_sj];
+                    }
+                }
+            }
 #pragma unroll
             for (int s = 0; s < NSTEP; ++s) {
                 s_acc = Mma<T>::run(tl.rows_op(kt, kb, s), qreg[s], s_acc);
                 dp_acc = Mma<T>::run(tl.rows_op(vt, kb, s), greg[s], dp_acc);
+            }
+            if (DENSE) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) s_acc[r] = __builtin_fmaf((float)mv[r / 4][r % 4], 1.4426950408889634f, s_acc[r]);
             }
             vec8 ds[2];
 #pragma unroll
@@ -292,7 +313,9 @@ constexpr int BWD_RING = 4;        // matrix operands in flight from LDS (reads 
 // t after a barrier.  Tiles t - 1 and t stay resident while tile t + 1 is copied: three stages.  The S and dP
 // accumulators do not start from zero but from -L_i log2(e) and -D_i (staged per tile next to the Q and dO rows), so
 // P = exp2(S) and dS = P * dP need no subtraction.
-template <typename T, int D>
+// DENSE: a dense additive mask - a lane holds one key and 16 query rows of a block, so its mask values are 16 loads down a
+// column of the mask, asked for at the start of a step and added (times log2 e) to the scores where P is taken.
+template <typename T, int D, bool DENSE = false>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
 {
@@ -431,7 +454,9 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
     // that tile's stage and from the exchange buffer) with P and dS of tile t computed on the vector ALU between them, then
     // - after a barrier, when everyone has read tile t - 1's P and dS - this wavefront's P and dS of tile t into the buffer.
     // WITH_A = false is the step after the last tile: only the second half.
-    auto step = [&](int stage, int pstage, int i0, bool has_prev, auto WITH_A_) __attribute__((always_inline)) {
+    // DENSE: the mask's column of this lane's key, for the query head in hand
+    [[maybe_unused]] const int64_t m_col = (int64_t)min(my_j, Skv - 1) * p.m_sj;
+    auto step = [&](int stage, int pstage, int i0, bool has_prev, [[maybe_unused]] int head, auto WITH_A_) __attribute__((always_inline)) {
         constexpr bool WITH_A = decltype(WITH_A_)::value;
         const char* qt = smem + stage * STAGE;
         const char* gt = qt + L::TILE_BYTES;
@@ -441,6 +466,13 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
         vec8 ring[R];
         floatx16 sa, da;
         vec8 pp[2], ds[2];
+        [[maybe_unused]] T mval[16];
+        if (WITH_A && DENSE) {      // register r is row i0 + 32 * role + 8 * (r / 4) + 4 * g + (r % 4); rows past the last repeat it
+            const T* mc = (const T*)p.mask + (int64_t)b * p.m_sb + (int64_t)(hkv * p.G + head) * p.m_sh + m_col;
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                mval[r] = mc[(int64_t)min(i0 + 32 * role + 8 * (r / 4) + 4 * g + (r % 4), Sq - 1) * p.m_si];
+        }
         if (WITH_A) {
             // The accumulators start from -L_i log2(e) and -D_i.  What the mask hides starts from -inf instead and ends as
             // P = 0, dS = 0 * (finite): only the causal edge needs that here, rows past Sq arrive as zeros throughout (dO = 0,
@@ -475,7 +507,7 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
         // P and dS of register r of the own query block, rounded for the next products
         auto soft = [&](int r) __attribute__((always_inline)) {
             if (!WITH_A) return;
-            const float pr = __builtin_amdgcn_exp2f(sa[r]);
+            const float pr = __builtin_amdgcn_exp2f(DENSE ? __builtin_fmaf((float)mval[r], 1.4426950408889634f, sa[r]) : sa[r]);
             pp[r / 8][r % 8] = (T)pr;
             ds[r / 8][r % 8] = (T)(pr * da[r]);
         };
@@ -524,7 +556,7 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
         to_head(0);
         issue(0);
     }
-    int i0 = t_begin * PF_BN, stage = 0, pstage = 0;
+    int i0 = t_begin * PF_BN, stage = 0, pstage = 0, head = 0;
     for (int t = 0; t < n_tiles; ++t) {
         // Tile t has landed for everyone, tile t - 1's P and dS are in the exchange buffer, and everyone is done with tile
         // t - 2: its stage is free for tile t + 1.
@@ -535,15 +567,15 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
         if (t + 1 < n_tiles) issue(nstage);
         // Every wavefront computes every tile: one whose keys no row of the tile sees (the first tile or two under a
         // causal mask) works on -inf, and would wait at the barriers for the others anyway.
-        step(stage, pstage, i0, t > 0, std::true_type{});
+        step(stage, pstage, i0, t > 0, head, std::true_type{});
         pstage = stage;
         stage = nstage;
         i0 += PF_BN;
-        if (i0 >= n_qt * PF_BN) i0 = t_begin * PF_BN;       // next head of the group
+        if (i0 >= n_qt * PF_BN) { i0 = t_begin * PF_BN; ++head; }      // next head of the group
     }
     if (n_tiles > 0) {
         __syncthreads();
-        step(stage, pstage, i0, true, std::false_type{});
+        step(stage, pstage, i0, true, head, std::false_type{});
     }
 
     if (my_j < Skv) {
@@ -568,7 +600,7 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
 #endif
 }
 
-template <typename T, int D>
+template <typename T, int D, bool DENSE = false>
 static hipError_t launch_bwd_t(const SdpaBwdParams& bp, hipStream_t stream)
 {
     const SdpaParams& p = bp.f;
@@ -580,19 +612,23 @@ static hipError_t launch_bwd_t(const SdpaBwdParams& bp, hipStream_t stream)
         SdpaBwdParams bq = bp;      // two workgroups per CU, an eighth of the CUs per XCD
         bq.f.interleave = work_interleave(p.causal != 0, 2 * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
         bq.f.deal_groups = (total & 7) == 0 ? work_deal(bq.f.interleave, p.G, nqb, total >> 3) : 0;
-        hipLaunchKernelGGL((sdpa_bwd_dq_kernel<T, D>), dim3((unsigned)total), dim3(256), 0, stream, bq);
+        hipLaunchKernelGGL((sdpa_bwd_dq_kernel<T, D, DENSE>), dim3((unsigned)total), dim3(256), 0, stream, bq);
     }
     const int nkb = (p.Skv + BWD_KEYS - 1) / BWD_KEYS;
     if ((int64_t)nkb * p.Hkv * p.B > 0)
-        hipLaunchKernelGGL((sdpa_bwd_dkv_kernel<T, D>), dim3((unsigned)((int64_t)nkb * p.Hkv * p.B)), dim3(512), 0, stream, bp);
+        hipLaunchKernelGGL((sdpa_bwd_dkv_kernel<T, D, DENSE>), dim3((unsigned)((int64_t)nkb * p.Hkv * p.B)), dim3(512), 0, stream, bp);
     return hipGetLastError();
 }
 
 // Host has validated: dtype f16/bf16, D and Dv <= 128 in whole 16-byte vectors (bp.f.Dp = the instance: 64 or 128; smaller
-// or unequal head dimensions are zero-padded on the way into LDS and registers, stores are cut), no dense mask, unit last-axis strides, 16-byte aligned rows,
+// or unequal head dimensions are zero-padded on the way into LDS and registers, stores are cut), a dense mask of any strides (the DENSE instances), unit last-axis strides, 16-byte aligned rows,
 // row strides below 2^24 elements, lse and the delta workspace present.
 hipError_t launch_sdpa_bwd_mfma(const SdpaBwdParams& bp, int dtype, hipStream_t stream)
 {
+    if (bp.f.mask) {
+        if (bp.f.Dp == 128) return dtype == 1 ? launch_bwd_t<f16_t, 128, true>(bp, stream) : launch_bwd_t<bf16_t, 128, true>(bp, stream);
+        return dtype == 1 ? launch_bwd_t<f16_t, 64, true>(bp, stream) : launch_bwd_t<bf16_t, 64, true>(bp, stream);
+    }
     if (bp.f.Dp == 128) return dtype == 1 ? launch_bwd_t<f16_t, 128>(bp, stream) : launch_bwd_t<bf16_t, 128>(bp, stream);
     return dtype == 1 ? launch_bwd_t<f16_t, 64>(bp, stream) : launch_bwd_t<bf16_t, 64>(bp, stream);
 }

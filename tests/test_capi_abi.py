@@ -277,7 +277,7 @@ def test_backward_validation_and_workspace_size():
         (_bwd(dict(impl=capi.IMPL_MFMA, D=160, Dv=160)), capi.EUNSUPPORTED),         # pinned to kernels that do not take it
         (_bwd(dict(impl=capi.IMPL_MFMA, D=36, Dv=36)), capi.EUNSUPPORTED),           # (72-byte rows are not whole vectors)
         (_bwd(dict(impl=capi.IMPL_MFMA, dtype=capi.F32, D=160, Dv=160)), capi.EUNSUPPORTED),
-        (_bwd(dict(impl=capi.IMPL_MFMA, add_mask=0x20000)), capi.EUNSUPPORTED),
+        (_bwd(dict(impl=capi.IMPL_MFMA, dtype=capi.F32, add_mask=0x20000)), capi.EUNSUPPORTED),      # (the 16-bit kernels take a mask, the f32 ones do not)
         (_bwd(dict(impl=capi.IMPL_SPLITKV)), capi.EUNSUPPORTED),
         (_bwd(dict(D=320, Dv=320)), capi.EUNSUPPORTED),
         (_bwd(dict(Hq=6, Hkv=4)), capi.ESHAPE),

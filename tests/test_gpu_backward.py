@@ -161,6 +161,46 @@ def test_generic_backward_f32_against_the_oracle(gpu, shape):
     compare("dv", dv, rv.reshape(B, Hkv, Skv, Dv), tol=1e-5)
 
 
+@pytest.mark.parametrize("dtype", [capi.BF16, capi.F16], ids=lambda x: dtypes.NAMES[x])
+@pytest.mark.parametrize("shape", [
+    # B, Hq, Hkv, Sq, Skv, D, Dv, causal, kv_lens, mask kind
+    (2, 2, 2, 150, 200, 128, 128, False, None, "full"),            # values with -inf holes, a mask of its own per batch entry and head
+    (2, 4, 2, 130, 130, 64, 64, True, None, "head"),               # grouped queries: [1, Hq, Sq, Skv] on top of the causal flag
+    (2, 3, 3, 100, 260, 128, 128, False, [260, 90], "row"),        # [1, 1, 1, Skv]: one row for everybody, with key counts
+    (1, 2, 2, 200, 200, 96, 72, False, None, "causal_tensor"),     # the causal mask as a tensor (no flag), padded head dimensions
+    (2, 2, 1, 70, 333, 128, 128, False, None, "batch"),            # [B, 1, Sq, Skv]; 333 keys: rows of the mask are not 8-byte aligned
+], ids=["full", "gqa_head_causal", "row_lens", "causal_tensor", "batch_unaligned"])
+def test_matrix_core_backward_with_a_dense_mask(gpu, dtype, shape):
+    """16-bit gradients with a dense additive mask run on the matrix-core kernels (instances that add the mask's values to
+    the scores before the exponential): against the f64 oracle, AUTO picks them, and the generic kernels agree."""
+    B, Hq, Hkv, Sq, Skv, D, Dv, causal, lens, mk = shape
+    G = Hq // Hkv
+    say("matrix-core backward with a mask: %s %s" % (dtypes.NAMES[dtype], shape))
+    q, k, v, go = make_d(71 + Sq, B, Hq, Hkv, Sq, Skv, D, Dv, dtype)
+    r = np.random.Generator(np.random.PCG64(72))
+    if mk == "causal_tensor":
+        mask = np.triu(np.full((Sq, Skv), -np.inf, np.float32), 1 + Skv - Sq).reshape(1, 1, Sq, Skv)
+    else:
+        mshape = {"full": (B, Hq, Sq, Skv), "row": (1, 1, 1, Skv), "head": (1, Hq, Sq, Skv), "batch": (B, 1, Sq, Skv)}[mk]
+        mask = r.standard_normal(mshape, dtype=np.float32)
+        mask[r.random(mshape) < 0.25] = -np.inf
+        mask[..., 0] = 0.0                                       # every row keeps a visible key
+    mask = dtypes.round_to(mask, dtype)
+    lens_a = None if lens is None else np.asarray(lens, np.int32)
+    kw = dict(causal=causal, kv_lens=lens_a, mask=mask)
+    out, dq, dk, dv = host.sdpa_backward(q, k, v, go, dtype, impl=capi.IMPL_MFMA, **kw)
+    auto = host.sdpa_backward(q, k, v, go, dtype, **kw)
+    gen = host.sdpa_backward(q, k, v, go, dtype, impl=capi.IMPL_GENERIC, **kw)
+    m5 = np.broadcast_to(mask, (B, Hq, Sq, Skv)).reshape(B, Hkv, G, Sq, Skv)
+    rq, rk, rv = BW.sdpa_backward(q.reshape(B, Hkv, G, Sq, D), k[:, :, None], v[:, :, None], go.reshape(B, Hkv, G, Sq, Dv),
+                                  mask=m5, causal=causal, kv_lens=None if lens is None else lens_a.reshape(B, 1, 1))
+    for name, x, a, gx, r_ in zip(("dq", "dk", "dv"), (dq, dk, dv), auto[1:], gen[1:],
+                                  (rq.reshape(B, Hq, Sq, D), rk.reshape(B, Hkv, Skv, D), rv.reshape(B, Hkv, Skv, Dv))):
+        compare(name, x, r_, tol=2e-2)
+        assert np.array_equal(x, a), name + ": AUTO takes the same kernels"
+        compare(name + " generic vs matrix-core", gx, x, tol=1e-2)
+
+
 @pytest.mark.parametrize("dtype,dims", [(capi.BF16, (96, 96)), (capi.BF16, (40, 72)), (capi.F16, (128, 64)), (capi.BF16, (8, 8)), (capi.F16, (80, 80)),
                                         (capi.F32, (96, 96)), (capi.F32, (20, 36)), (capi.F32, (128, 64)), (capi.F32, (4, 4))],
                          ids=lambda x: dtypes.NAMES[x] if isinstance(x, int) else "D%d_Dv%d" % x)
