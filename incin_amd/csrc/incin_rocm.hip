@@ -938,18 +938,31 @@ static int check_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, bool* empty, int* kin
     const int64_t big = f32 ? (1 << 22) : (1 << 24);
     ok = ok && d->q_stride[2] >= 0 && d->q_stride[2] < big && d->k_stride[2] >= 0 && d->k_stride[2] < big && d->v_stride[2] >= 0 &&
          d->v_stride[2] < big && bd->d_o_stride[2] >= 0 && bd->d_o_stride[2] < big;
+    if (d->add_mask)      // a tile's mask values are addressed with 32-bit byte offsets from the tile's first row
+        ok = ok && d->mask_stride[2] >= 0 && d->mask_stride[3] >= 0 &&
+             (64 * d->mask_stride[2] + (d->Skv > 0 ? d->Skv - 1 : 0) * d->mask_stride[3] + 1) * 2 < (int64_t)0x7fffffff;
     const int fast = f32 ? 2 : 1;
     if (d->impl == INCIN_ROCM_IMPL_AUTO) *kind = ok ? fast : 0;
     else if (d->impl == INCIN_ROCM_IMPL_GENERIC) *kind = 0;
     else if (d->impl == INCIN_ROCM_IMPL_MFMA) {
         if (!ok)
             return fail(INCIN_ROCM_EUNSUPPORTED, "%s: the MFMA kernels need D and Dv <= 128 in whole 16-byte vectors, a finite scale (f16 / bf16: "
-                        "positive), no dense mask in f32, and rows 16-byte aligned with strides that are multiples of 16 bytes below 2^%d elements",
+                        "positive), no dense mask in f32 (f16 / bf16: 64 rows of the mask within 2 GiB), and rows 16-byte aligned with strides that are multiples of 16 bytes below 2^%d elements",
                         OP, f32 ? 22 : 24);
         *kind = fast;
     } else
         return fail(INCIN_ROCM_EUNSUPPORTED, "%s: impl is one of AUTO, GENERIC, MFMA", OP);
     return 0;
+}
+
+// Workspace of a backward call: two f32 per query row; with a dense mask on the 16-bit matrix-core kernels also the mask's
+// block flags (one byte per 32 rows x 32 keys, as the forward's: hidden blocks are skipped), behind them.
+static size_t bwd_rows_bytes(const incin_rocm_sdpa_desc_t* d) { return (2 * (size_t)(d->B * d->Hq * d->Sq) * sizeof(float) + 255) / 256 * 256; }
+static size_t bwd_flags_bytes(const incin_rocm_sdpa_desc_t* d, int kind)
+{
+    if (kind != 1 || !d->add_mask) return 0;
+    const int64_t nbh = (d->mask_stride[0] ? d->B : 1) * (d->mask_stride[1] ? d->Hq : 1);
+    return (size_t)(nbh * ((d->Sq + 31) / 32) * ((d->Skv + 31) / 32) + 255) / 256 * 256;
 }
 
 int incin_rocm_sdpa_bwd_workspace(const incin_rocm_sdpa_bwd_desc_t* bd, size_t* bytes)
@@ -959,7 +972,10 @@ int incin_rocm_sdpa_bwd_workspace(const incin_rocm_sdpa_bwd_desc_t* bd, size_t* 
     bool empty = false;
     int kind = 0;
     if (int rc = check_bwd(bd, &empty, &kind)) return rc;
-    if (!empty) *bytes = 2 * (size_t)(bd->fwd.B * bd->fwd.Hq * bd->fwd.Sq) * sizeof(float);
+    if (!empty) {
+        const size_t flags = bwd_flags_bytes(&bd->fwd, kind);
+        *bytes = flags ? bwd_rows_bytes(&bd->fwd) + flags : 2 * (size_t)(bd->fwd.B * bd->fwd.Hq * bd->fwd.Sq) * sizeof(float);
+    }
     return 0;
 }
 
@@ -981,7 +997,9 @@ int incin_rocm_sdpa_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, void* stream)
         }
         return 0;
     }
-    const size_t need = 2 * (size_t)(bd->fwd.B * bd->fwd.Hq * bd->fwd.Sq) * sizeof(float);      // two f32 per query row
+    const size_t flag_bytes = bwd_flags_bytes(&bd->fwd, kind);
+    const size_t need = flag_bytes ? bwd_rows_bytes(&bd->fwd) + flag_bytes
+                                   : 2 * (size_t)(bd->fwd.B * bd->fwd.Hq * bd->fwd.Sq) * sizeof(float);      // two f32 per query row (+ the mask's block flags)
     if (!bd->workspace || bd->workspace_bytes < need || !aligned16(bd->workspace))
         return fail(INCIN_ROCM_EWORKSPACE, "scaled_dot_product_attention backward: %zu workspace bytes needed (16-byte aligned), %zu given",
                     need, bd->workspace ? bd->workspace_bytes : (size_t)0);
@@ -1000,6 +1018,15 @@ int incin_rocm_sdpa_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, void* stream)
     bp.dq_sb = bd->d_q_stride[0]; bp.dq_sh = bd->d_q_stride[1]; bp.dq_ss = bd->d_q_stride[2];
     bp.dk_sb = bd->d_k_stride[0]; bp.dk_sh = bd->d_k_stride[1]; bp.dk_ss = bd->d_k_stride[2];
     bp.dv_sb = bd->d_v_stride[0]; bp.dv_sh = bd->d_v_stride[1]; bp.dv_ss = bd->d_v_stride[2];
+    bp.f.mask_flags = nullptr;
+    bp.f.mask_lims = nullptr;
+    if (flag_bytes) {
+        if (((bd->fwd.Sq + 31) / 32) > 65535 || (bd->fwd.mask_stride[0] ? bd->fwd.B : 1) * (bd->fwd.mask_stride[1] ? bd->fwd.Hq : 1) > 65535)
+            return fail(INCIN_ROCM_ESHAPE, "scaled_dot_product_attention backward: mask too large for one launch of the matrix-core kernels");
+        bp.f.mask_flags = (const uint8_t*)bd->workspace + bwd_rows_bytes(&bd->fwd);
+        hipError_t ec = incin_rocm::launch_mask_classify(bp.f, bd->fwd.dtype, (hipStream_t)stream);
+        if (ec != hipSuccess) return hip_fail(ec, "mask classification launch");
+    }
     hipError_t e = kind == 2   ? incin_rocm::launch_sdpa_bwd_f32(bp, (hipStream_t)stream)
                    : kind == 1 ? incin_rocm::launch_sdpa_bwd_mfma(bp, bd->fwd.dtype, (hipStream_t)stream)
                                : incin_rocm::launch_sdpa_bwd_generic(bp, bd->fwd.dtype, (hipStream_t)stream);

@@ -174,8 +174,32 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
     }
     if (q0 >= rows_b) j_end = 0;
     if (q0 + wave * 32 >= rows_b) lim_wave_max = 0;
-    const int n_tiles = (j_end + PF_BN - 1) / PF_BN;
+    int n_tiles = (j_end + PF_BN - 1) / PF_BN, t_first = 0;
     const int n_act = lim_wave_max > 0 ? (lim_wave_max + PF_BN - 1) / PF_BN : 0;
+    // DENSE: the block flags of this wavefront's 32 rows, one per 32 keys (1 all zero, 2 all -inf: no values to fetch), and
+    // the tiles between the first and the last key block that some row of the workgroup sees (a causal mask or a window
+    // given as a tensor hides the rest of the row of tiles: those are not even copied)
+    [[maybe_unused]] const uint8_t* mflags = nullptr;
+    [[maybe_unused]] const int nkb32 = (Skv + 31) >> 5;
+    if (DENSE && p.mask_flags) {
+        __shared__ int s_seen[2];
+        const int nrb32 = (Sq + 31) >> 5;
+        const uint8_t* fl = mask_flags_of(p, b, hq);
+        mflags = fl + (int64_t)min((q0 >> 5) + wave, nrb32 - 1) * nkb32;
+        if (tid == 0) { s_seen[0] = 0x7fffffff; s_seen[1] = -1; }
+        __syncthreads();
+        int lo = 0x7fffffff, hi = -1;
+        for (int c = tid; c < min(2 * n_tiles, nkb32); c += 256) {
+            bool seen = false;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) seen = seen || fl[(int64_t)min((q0 >> 5) + w, nrb32 - 1) * nkb32 + c] != 2;
+            if (seen) { lo = min(lo, c); hi = max(hi, c); }
+        }
+        if (hi >= 0) { atomicMin(&s_seen[0], lo); atomicMax(&s_seen[1], hi); }
+        __syncthreads();
+        t_first = s_seen[1] < 0 ? 0 : __builtin_amdgcn_readfirstlane(s_seen[0]) >> 1;
+        n_tiles = s_seen[1] < 0 ? 0 : min(n_tiles, (__builtin_amdgcn_readfirstlane(s_seen[1]) >> 1) + 1);
+    }
 
     BwdTiles<T, D, 4, NDB> tl;
     tl.init(wave, lane, p.k_ss, p.v_ss, p.D, p.Dv, 0);
@@ -186,7 +210,7 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
     vec8 qreg[NSTEP], greg[NSTEP];
     const int qi = min(my_i, Sq - 1);
     const unsigned lds0 = lds_address(smem);
-    if (n_tiles > 0) tl.issue(0, kp, p.k_ss, Skv, 0, lds0, wave);
+    if (t_first < n_tiles) tl.issue(0, kp, p.k_ss, Skv, t_first * PF_BN, lds0 + (t_first & 1) * L::TILE_BYTES, wave);
     {
         static_assert(2 * L::TILE_BYTES >= 4 * 4096, "the V buffers hold a 4 KiB staging area per wavefront");
         char* stage = smem + 2 * L::TILE_BYTES + wave * 4096;
@@ -202,7 +226,7 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
             for (int e = 0; e < 8; ++e) qreg[s][e] = (T)((float)qreg[s][e] * c2);
     }
     __syncthreads();      // every wavefront has its rows out of the V buffers
-    if (n_tiles > 0) tl.issue(1, vp, p.v_ss, Skv, 0, lds0 + 2 * L::TILE_BYTES, wave);
+    if (t_first < n_tiles) tl.issue(1, vp, p.v_ss, Skv, t_first * PF_BN, lds0 + (2 + (t_first & 1)) * L::TILE_BYTES, wave);
     const int64_t stat = ((int64_t)b * p.Hq + hq) * Sq + qi;
     [[maybe_unused]] const T* mrow = nullptr;      // DENSE: this lane's row of the mask
     if (DENSE) mrow = (const T*)p.mask + (int64_t)b * p.m_sb + (int64_t)hq * p.m_sh + (int64_t)qi * p.m_si;
@@ -223,13 +247,25 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
     int lim_wave_min = kv_len;
     if (p.causal) lim_wave_min = clampi(q0 + wave * 32 + coff + 1, 0, kv_len);
 
-    for (int t = 0; t < n_tiles; ++t) {
+    [[maybe_unused]] int fv[2] = {0, 0};      // DENSE: the two flags of the tile about to start, as loaded (asked for a tile ahead)
+    [[maybe_unused]] auto tile_flags = [&](int t) __attribute__((always_inline)) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) fv[kb] = 2 * t + kb < nkb32 ? (int)mflags[2 * t + kb] : 2;
+    };
+    if (DENSE && mflags && t_first < n_tiles) tile_flags(t_first);
+    for (int t = t_first; t < n_tiles; ++t) {
         // K(t), V(t) have landed for everyone and everyone is done with tile t-1: the other pair of buffers is free
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         if (t + 1 < n_tiles) {
             tl.issue(0, kp, p.k_ss, Skv, (t + 1) * PF_BN, lds0 + ((t + 1) & 1) * L::TILE_BYTES, wave);
             tl.issue(1, vp, p.v_ss, Skv, (t + 1) * PF_BN, lds0 + (2 + ((t + 1) & 1)) * L::TILE_BYTES, wave);
+        }
+        [[maybe_unused]] int flags_t[2] = {0, 0};
+        if (DENSE && mflags) {
+            flags_t[0] = __builtin_amdgcn_readfirstlane(fv[0]);
+            flags_t[1] = __builtin_amdgcn_readfirstlane(fv[1]);
+            if (t + 1 < n_tiles) tile_flags(t + 1);
         }
         if (t >= n_act) continue;
         const char* kt = smem + (t & 1) * L::TILE_BYTES;
@@ -248,7 +284,17 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
             }
             typedef T vec4 __attribute__((ext_vector_type(4)));
             [[maybe_unused]] vec4 mv[4];
-            if (DENSE) {      // the mask's values of this lane's 16 keys, asked for ahead of the products
+            [[maybe_unused]] int flag = 0;
+            if (DENSE && mflags) {
+                flag = flags_t[kb];
+                if (flag == 2) {      // the mask hides the block from all 32 rows: S starts from -inf, as at the causal edge (the
+                                      // products run all the same: branches around them cost every tile more than these blocks save)
+                    asm volatile("" ::: "memory");
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) s_acc[r] = -INFINITY;
+                }
+            }
+            if (DENSE && flag == 0) {      // the mask's values of this lane's 16 keys, asked for ahead of the products
 #pragma unroll
                 for (int r4 = 0; r4 < 4; ++r4) {
                     const int j = j0 + 32 * kb + 8 * r4 + 4 * g;
@@ -264,7 +310,7 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
                 s_acc = Mma<T>::run(tl.rows_op(kt, kb, s), qreg[s], s_acc);
                 dp_acc = Mma<T>::run(tl.rows_op(vt, kb, s), greg[s], dp_acc);
             }
-            if (DENSE) {
+            if (DENSE && flag == 0) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) s_acc[r] = __builtin_fmaf((float)mv[r / 4][r % 4], 1.4426950408889634f, s_acc[r]);
             }
@@ -289,7 +335,7 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
     }
     {
         constexpr int PER_BUF = L::TILE_BYTES / 4096;      // staging areas per buffer: 4 (D = 128) or 2
-        char* stage = smem + ((wave / PER_BUF) * 2 + (n_tiles & 1)) * L::TILE_BYTES + (wave % PER_BUF) * 4096;
+        char* stage = smem + ((wave / PER_BUF) * 2 + (max(n_tiles, t_first) & 1)) * L::TILE_BYTES + (wave % PER_BUF) * 4096;
         store_o_rows(dq_acc, p.scale, stage, dqp, q0 + wave * 32, Sq, bp.dq_ss, p.D, lane);
     }
 #endif
@@ -313,7 +359,9 @@ constexpr int BWD_RING = 4;        // matrix operands in flight from LDS (reads 
 // t after a barrier.  Tiles t - 1 and t stay resident while tile t + 1 is copied: three stages.  The S and dP
 // accumulators do not start from zero but from -L_i log2(e) and -D_i (staged per tile next to the Q and dO rows), so
 // P = exp2(S) and dS = P * dP need no subtraction.
-// DENSE: a dense additive mask - a lane holds one key and 16 query rows of a block, so its mask values are 16 loads down a
+// DENSE: a dense additive mask, with one flag per block of 32 rows x 32 keys (mask_classify_kernel ran before).  Tiles before
+// the first and after the last block that shows this workgroup any key are left out; inside that range a block of zeros or
+// of -inf needs no values.  Otherwise: a lane holds one key and 16 query rows of a block, so its mask values are 16 loads down a
 // column of the mask, asked for at the start of a step and added (times log2 e) to the scores where P is taken.
 template <typename T, int D, bool DENSE = false>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
@@ -371,11 +419,36 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
     const int i_begin_wg = p.causal ? clampi(j0 - coff, 0, Sq) : 0;
     // first query row that sees every key of this wavefront: tiles from there on need no mask
     const int i_all_wave = p.causal ? max(j0 + kb * 32 + 31 - coff, 0) : 0;
-    const int t_begin = i_begin_wg / PF_BN;
+    int t_begin = i_begin_wg / PF_BN;
     // query rows at and beyond rows_b are padding (q_lens): the tiles end there, and the rows between there and the end of
     // the last tile arrive as zeros like rows past Sq (Q, dO and the per-row values), which leaves dS and P^T dO at zero
     const int rows_b = p.q_lens ? clampi(p.q_lens[b], 0, Sq) : Sq;
-    const int n_qt = (rows_b + PF_BN - 1) / PF_BN;
+    int n_qt = (rows_b + PF_BN - 1) / PF_BN;
+    if (DENSE && p.mask_flags) {
+        // The tiles between the first and the last block of 32 query rows, over the group's heads, from which the mask does not
+        // hide all of this workgroup's keys: a causal mask or a window given as a tensor leaves the others out altogether.
+        __shared__ int s_seen[2];
+        const int nkb = (Skv + 31) >> 5, nrb = (Sq + 31) >> 5, c0 = kblk * 4;
+        if (tid == 0) { s_seen[0] = 0x7fffffff; s_seen[1] = -1; }
+        __syncthreads();
+        int lo = 0x7fffffff, hi = -1;
+        const int r_lo = 2 * t_begin, r_n = min(2 * n_qt, nrb) - r_lo;
+        for (int x = tid; x < r_n * p.G; x += 512) {
+            const int rb = r_lo + x % r_n;
+            const uint8_t* fl = mask_flags_of(p, b, hkv * p.G + x / r_n) + (int64_t)rb * nkb;
+            bool seen = false;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) seen = seen || fl[min(c0 + c, nkb - 1)] != 2;
+            if (seen) { lo = min(lo, rb); hi = max(hi, rb); }
+        }
+        if (hi >= 0) { atomicMin(&s_seen[0], lo); atomicMax(&s_seen[1], hi); }
+        __syncthreads();
+        if (s_seen[1] < 0) n_qt = t_begin;
+        else {
+            t_begin = __builtin_amdgcn_readfirstlane(s_seen[0]) >> 1;
+            n_qt = (__builtin_amdgcn_readfirstlane(s_seen[1]) >> 1) + 1;
+        }
+    }
     const int tiles_per_head = j0 < kv_len ? max(n_qt - t_begin, 0) : 0;
     const int n_tiles = tiles_per_head * p.G;           // the group's query heads one after another
 
@@ -454,9 +527,21 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
     // that tile's stage and from the exchange buffer) with P and dS of tile t computed on the vector ALU between them, then
     // - after a barrier, when everyone has read tile t - 1's P and dS - this wavefront's P and dS of tile t into the buffer.
     // WITH_A = false is the step after the last tile: only the second half.
-    // DENSE: the mask's column of this lane's key, for the query head in hand
-    [[maybe_unused]] const int64_t m_col = (int64_t)min(my_j, Skv - 1) * p.m_sj;
-    auto step = [&](int stage, int pstage, int i0, bool has_prev, [[maybe_unused]] int head, auto WITH_A_) __attribute__((always_inline)) {
+    // DENSE: the mask's column of this lane's key, for the query head in hand; and the flags of this wavefront's 32 keys -
+    // per block of 32 query rows: 1 says the mask is zero there, 2 that it hides the keys from all of the rows (neither needs
+    // the mask's values)
+    // (the values are fetched with one lane offset - the key's column and the lane's first row - plus a scalar offset per
+    // register, from a descriptor that starts at the tile's first row and ends with the head's last row: rows past Sq read
+    // zeros; the host has checked that 64 rows fit 32-bit offsets)
+    [[maybe_unused]] const int m_lane = (int)(((int64_t)min(my_j, Skv - 1) * p.m_sj + (int64_t)(4 * g) * p.m_si) * 2);
+    [[maybe_unused]] const int m_row2 = (int)(p.m_si * 2);
+    [[maybe_unused]] const int nkb32 = (Skv + 31) >> 5, nrb32 = (Sq + 31) >> 5;
+    [[maybe_unused]] const int my_kb32 = min(kblk * 4 + kb, nkb32 - 1);
+    // (the flag of a tile - this wavefront's query block of it - is asked for one tile ahead: tile_flag)
+    [[maybe_unused]] auto tile_flag = [&](int i0, int head) __attribute__((always_inline)) {
+        return (int)mask_flags_of(p, b, hkv * p.G + head)[(int64_t)min((i0 >> 5) + role, nrb32 - 1) * nkb32 + my_kb32];
+    };
+    auto step = [&](int stage, int pstage, int i0, bool has_prev, [[maybe_unused]] int head, [[maybe_unused]] int f_own, auto WITH_A_) __attribute__((always_inline)) {
         constexpr bool WITH_A = decltype(WITH_A_)::value;
         const char* qt = smem + stage * STAGE;
         const char* gt = qt + L::TILE_BYTES;
@@ -466,12 +551,22 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
         vec8 ring[R];
         floatx16 sa, da;
         vec8 pp[2], ds[2];
-        [[maybe_unused]] T mval[16];
-        if (WITH_A && DENSE) {      // register r is row i0 + 32 * role + 8 * (r / 4) + 4 * g + (r % 4); rows past the last repeat it
-            const T* mc = (const T*)p.mask + (int64_t)b * p.m_sb + (int64_t)(hkv * p.G + head) * p.m_sh + m_col;
+        typedef T vec2 __attribute__((ext_vector_type(2)));
+        [[maybe_unused]] vec2 mval[8];       // (pairs: two 16-bit loads fill one register)
+        [[maybe_unused]] bool own_hidden = false, own_zero = false;
+        if (WITH_A && DENSE) {
+            own_hidden = f_own == 2;
+            own_zero = f_own == 1;
+        }
+        [[maybe_unused]] const bool own_values = WITH_A && DENSE && !own_zero && !own_hidden;
+        if (own_values) {      // register r is row i0 + 32 * role + 8 * (r / 4) + 4 * g + (r % 4); rows past the last repeat it
+            const int row0 = i0 + 32 * role;
+            const T* mc = (const T*)p.mask + (int64_t)b * p.m_sb + (int64_t)(hkv * p.G + head) * p.m_sh + (int64_t)row0 * p.m_si;
+            const int64_t left = row0 < Sq ? ((int64_t)(Sq - 1 - row0) * p.m_si + (int64_t)(Skv - 1) * p.m_sj + 1) * 2 : 0;
+            const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)mc, 0, (int)min(left, (int64_t)0x7fffffff), 0x00020000);
 #pragma unroll
             for (int r = 0; r < 16; ++r)
-                mval[r] = mc[(int64_t)min(i0 + 32 * role + 8 * (r / 4) + 4 * g + (r % 4), Sq - 1) * p.m_si];
+                mval[r / 2][r % 2] = __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b16(rs, m_lane, (8 * (r / 4) + (r % 4)) * m_row2, 0));
         }
         if (WITH_A) {
             // The accumulators start from -L_i log2(e) and -D_i.  What the mask hides starts from -inf instead and ends as
@@ -490,6 +585,12 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
             };
 #pragma unroll
             for (int i = 0; i < R; ++i) fetch_a(i);
+            if (DENSE && own_hidden) {      // (as at the causal edge: S starts from -inf; the products run all the same - branches
+                                            //  around them cost every tile more than these tiles save)
+                asm volatile("" ::: "memory");
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sa[r] = -INFINITY;
+            }
             if (i0 < i_all_wave) {          // some row of the tile does not see every key of this wavefront
                 asm volatile("" ::: "memory");      // (a real branch: as selects this would cost every tile 32 vector instructions)
                 const int rel = lo_i - i0 - 4 * g - 32 * role;      // register r is row i0 + 32*role + 8*(r/4) + 4*g + (r%4)
@@ -503,11 +604,15 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
                 else da = Mma<T>::run(ring[i % R], vreg[i / 2], da);
                 if (i + R < NA) fetch_a(i + R);
             }
+            if (own_values) {       // (the mask's values are no longer needed past this point: the second half has no room for them)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sa[r] = __builtin_fmaf((float)mval[r / 2][r % 2], 1.4426950408889634f, sa[r]);
+            }
         }
         // P and dS of register r of the own query block, rounded for the next products
         auto soft = [&](int r) __attribute__((always_inline)) {
             if (!WITH_A) return;
-            const float pr = __builtin_amdgcn_exp2f(DENSE ? __builtin_fmaf((float)mval[r], 1.4426950408889634f, sa[r]) : sa[r]);
+            const float pr = __builtin_amdgcn_exp2f(sa[r]);
             pp[r / 8][r % 8] = (T)pr;
             ds[r / 8][r % 8] = (T)(pr * da[r]);
         };
@@ -557,6 +662,8 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
         issue(0);
     }
     int i0 = t_begin * PF_BN, stage = 0, pstage = 0, head = 0;
+    [[maybe_unused]] int fv_own = 0;      // the flag of the tile about to start, as loaded
+    if (DENSE && p.mask_flags && n_tiles > 0) fv_own = tile_flag(i0, 0);
     for (int t = 0; t < n_tiles; ++t) {
         // Tile t has landed for everyone, tile t - 1's P and dS are in the exchange buffer, and everyone is done with tile
         // t - 2: its stage is free for tile t + 1.
@@ -565,17 +672,24 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
         __syncthreads();
         const int nstage = stage == 2 ? 0 : stage + 1;
         if (t + 1 < n_tiles) issue(nstage);
+        const int i0_next = i0 + PF_BN >= n_qt * PF_BN ? t_begin * PF_BN : i0 + PF_BN;      // (then: next head of the group)
+        const int head_next = i0 + PF_BN >= n_qt * PF_BN ? head + 1 : head;
+        int f_own = 0;
+        if (DENSE && p.mask_flags) {
+            f_own = __builtin_amdgcn_readfirstlane(fv_own);
+            if (t + 1 < n_tiles) fv_own = tile_flag(i0_next, head_next);
+        }
         // Every wavefront computes every tile: one whose keys no row of the tile sees (the first tile or two under a
         // causal mask) works on -inf, and would wait at the barriers for the others anyway.
-        step(stage, pstage, i0, t > 0, head, std::true_type{});
+        step(stage, pstage, i0, t > 0, head, f_own, std::true_type{});
         pstage = stage;
         stage = nstage;
-        i0 += PF_BN;
-        if (i0 >= n_qt * PF_BN) { i0 = t_begin * PF_BN; ++head; }      // next head of the group
+        i0 = i0_next;
+        head = head_next;
     }
     if (n_tiles > 0) {
         __syncthreads();
-        step(stage, pstage, i0, true, head, std::false_type{});
+        step(stage, pstage, i0, true, head, 0, std::false_type{});
     }
 
     if (my_j < Skv) {
@@ -610,7 +724,7 @@ static hipError_t launch_bwd_t(const SdpaBwdParams& bp, hipStream_t stream)
         const int nqb = (p.Sq + PF_BM - 1) / PF_BM;
         const int64_t total = (int64_t)nqb * p.Hq * p.B;
         SdpaBwdParams bq = bp;      // two workgroups per CU, an eighth of the CUs per XCD
-        bq.f.interleave = work_interleave(p.causal != 0, 2 * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
+        bq.f.interleave = work_interleave(p.causal != 0 || p.mask != nullptr, 2 * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
         bq.f.deal_groups = (total & 7) == 0 ? work_deal(bq.f.interleave, p.G, nqb, total >> 3) : 0;
         hipLaunchKernelGGL((sdpa_bwd_dq_kernel<T, D, DENSE>), dim3((unsigned)total), dim3(256), 0, stream, bq);
     }

@@ -257,7 +257,8 @@ int incin_rocm_sdpa_fwd_static(const incin_rocm_sdpa_desc_t* desc, void* stream)
  * scale; both without a dense mask and with 16-byte aligned rows - and generic f32-arithmetic kernels otherwise; GENERIC and MFMA pin one or
  * the other.  A query row with no visible key (NaN in the forward) gets a zero gradient and
  * contributes nothing to d_k and d_v, where the reference's tape would spread NaN over the whole head.
- * The workspace holds two floats per query row (2 x [B, Hq, Sq]; ask incin_rocm_sdpa_bwd_workspace for the size);
+ * The workspace holds two floats per query row (2 x [B, Hq, Sq]) and, for a dense mask on the 16-bit matrix-core kernels, a byte
+ * per 32 rows x 32 keys of the mask behind them (ask incin_rocm_sdpa_bwd_workspace for the size);
  * d_q, d_k, d_v are fully overwritten. */
 typedef struct {
     incin_rocm_sdpa_desc_t fwd;

@@ -269,7 +269,11 @@ def test_backward_validation_and_workspace_size():
     # two f32 per query row, whichever kernels take the request
     assert capi.sdpa_bwd_workspace(_bwd()) == 2 * 2 * 4 * 128 * 4
     assert capi.sdpa_bwd_workspace(_bwd(dict(dtype=capi.F32))) == 2 * 2 * 4 * 128 * 4
-    assert capi.sdpa_bwd_workspace(_bwd(dict(add_mask=0x20000))) == 2 * 2 * 4 * 128 * 4
+    # ... plus, for a dense mask on the 16-bit matrix-core kernels, the mask's block flags (a byte per 32 rows x 32 keys, in 256s)
+    assert capi.sdpa_bwd_workspace(_bwd(dict(add_mask=0x20000))) == 2 * 2 * 4 * 128 * 4 + 256
+    assert capi.sdpa_bwd_workspace(_bwd(dict(add_mask=0x20000, mask_stride=(4 * 128 * 128, 128 * 128, 128, 1)))) == 2 * 2 * 4 * 128 * 4 + 256      # 8 mask planes x 16 flags, rounded up
+    assert capi.sdpa_bwd_workspace(_bwd(dict(add_mask=0x20000, impl=capi.IMPL_GENERIC))) == 2 * 2 * 4 * 128 * 4
+    assert capi.sdpa_bwd_workspace(_bwd(dict(add_mask=0x20000, dtype=capi.F32))) == 2 * 2 * 4 * 128 * 4
     assert capi.sdpa_bwd_workspace(_bwd(dict(Sq=0))) == 0            # nothing to compute
     for bd, code in [
         (_bwd(dict(lse=None)), capi.EINVAL),                          # the forward's normalisers are an input

@@ -169,7 +169,10 @@ def test_generic_backward_f32_against_the_oracle(gpu, shape):
     (2, 3, 3, 100, 260, 128, 128, False, [260, 90], "row"),        # [1, 1, 1, Skv]: one row for everybody, with key counts
     (1, 2, 2, 200, 200, 96, 72, False, None, "causal_tensor"),     # the causal mask as a tensor (no flag), padded head dimensions
     (2, 2, 1, 70, 333, 128, 128, False, None, "batch"),            # [B, 1, Sq, Skv]; 333 keys: rows of the mask are not 8-byte aligned
-], ids=["full", "gqa_head_causal", "row_lens", "causal_tensor", "batch_unaligned"])
+    (1, 4, 2, 330, 400, 128, 128, False, None, "causal_bias"),     # per-head distance bias under the causal triangle: blocks of all kinds
+    (2, 2, 2, 300, 300, 64, 64, False, None, "window"),            # a band of 70 keys: hidden blocks on both sides, zeros between
+    (1, 2, 1, 257, 290, 128, 128, True, None, "blocks"),           # random 32 x 32 blocks hidden / zero / values, under the causal flag
+], ids=["full", "gqa_head_causal", "row_lens", "causal_tensor", "batch_unaligned", "causal_bias", "window", "blocks"])
 def test_matrix_core_backward_with_a_dense_mask(gpu, dtype, shape):
     """16-bit gradients with a dense additive mask run on the matrix-core kernels (instances that add the mask's values to
     the scores before the exponential): against the f64 oracle, AUTO picks them, and the generic kernels agree."""
@@ -180,6 +183,17 @@ def test_matrix_core_backward_with_a_dense_mask(gpu, dtype, shape):
     r = np.random.Generator(np.random.PCG64(72))
     if mk == "causal_tensor":
         mask = np.triu(np.full((Sq, Skv), -np.inf, np.float32), 1 + Skv - Sq).reshape(1, 1, Sq, Skv)
+    elif mk == "causal_bias":
+        dist = (np.arange(Sq)[:, None] + (Skv - Sq) - np.arange(Skv)[None, :]).astype(np.float32)
+        mask = np.where(dist >= 0, -dist[None] * (0.5 ** np.arange(1, Hq + 1, dtype=np.float32))[:, None, None], -np.inf)[None].astype(np.float32)
+    elif mk == "window":
+        dist = np.arange(Sq)[:, None] - np.arange(Skv)[None, :]
+        mask = np.where((dist >= 0) & (dist < 70), 0.0, -np.inf).astype(np.float32).reshape(1, 1, Sq, Skv)
+    elif mk == "blocks":
+        kinds = r.integers(0, 3, size=(B, Hq, (Sq + 31) // 32, (Skv + 31) // 32))
+        kinds[..., 0] = 1                                        # every row keeps visible keys
+        big = np.repeat(np.repeat(kinds, 32, axis=2), 32, axis=3)[:, :, :Sq, :Skv]
+        mask = np.where(big == 0, -np.inf, np.where(big == 1, 0.0, r.standard_normal((B, Hq, Sq, Skv), dtype=np.float32))).astype(np.float32)
     else:
         mshape = {"full": (B, Hq, Sq, Skv), "row": (1, 1, 1, Skv), "head": (1, Hq, Sq, Skv), "batch": (B, 1, Sq, Skv)}[mk]
         mask = r.standard_normal(mshape, dtype=np.float32)
