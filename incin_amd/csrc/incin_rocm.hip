@@ -931,7 +931,7 @@ static int check_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, bool* empty, int* kin
     const bool f32 = d->dtype == INCIN_ROCM_F32;
     const int vec = f32 ? 4 : 8;
     // (head dimensions up to 128 in whole 16-byte vectors, D and Dv not necessarily equal: zero-padded into the 64 / 128 instances)
-    bool ok = d->D > 0 && d->D <= 128 && d->Dv <= 128 && d->D % vec == 0 && d->Dv % vec == 0 && (!d->add_mask || !f32) && std::isfinite(d->scale) && (f32 || d->scale > 0.0f);
+    bool ok = d->D > 0 && d->D <= 128 && d->Dv <= 128 && d->D % vec == 0 && d->Dv % vec == 0 && std::isfinite(d->scale) && (f32 || d->scale > 0.0f);
     ok = ok && fast_layout_ok(d, vec) && aligned16(bd->d_o) && aligned16(bd->d_q) && aligned16(bd->d_k) && aligned16(bd->d_v);
     for (int a = 0; a < 3; ++a)
         ok = ok && bd->d_o_stride[a] % vec == 0 && bd->d_q_stride[a] % vec == 0 && bd->d_k_stride[a] % vec == 0 && bd->d_v_stride[a] % vec == 0;
@@ -940,14 +940,14 @@ static int check_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, bool* empty, int* kin
          d->v_stride[2] < big && bd->d_o_stride[2] >= 0 && bd->d_o_stride[2] < big;
     if (d->add_mask)      // a tile's mask values are addressed with 32-bit byte offsets from the tile's first row
         ok = ok && d->mask_stride[2] >= 0 && d->mask_stride[3] >= 0 &&
-             (64 * d->mask_stride[2] + (d->Skv > 0 ? d->Skv - 1 : 0) * d->mask_stride[3] + 1) * 2 < (int64_t)0x7fffffff;
+             (64 * d->mask_stride[2] + (d->Skv > 0 ? d->Skv - 1 : 0) * d->mask_stride[3] + 1) * (f32 ? 4 : 2) < (int64_t)0x7fffffff;
     const int fast = f32 ? 2 : 1;
     if (d->impl == INCIN_ROCM_IMPL_AUTO) *kind = ok ? fast : 0;
     else if (d->impl == INCIN_ROCM_IMPL_GENERIC) *kind = 0;
     else if (d->impl == INCIN_ROCM_IMPL_MFMA) {
         if (!ok)
             return fail(INCIN_ROCM_EUNSUPPORTED, "%s: the MFMA kernels need D and Dv <= 128 in whole 16-byte vectors, a finite scale (f16 / bf16: "
-                        "positive), no dense mask in f32 (f16 / bf16: 64 rows of the mask within 2 GiB), and rows 16-byte aligned with strides that are multiples of 16 bytes below 2^%d elements",
+                        "positive), 64 rows of a dense mask within 2 GiB, and rows 16-byte aligned with strides that are multiples of 16 bytes below 2^%d elements",
                         OP, f32 ? 22 : 24);
         *kind = fast;
     } else
@@ -955,12 +955,12 @@ static int check_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, bool* empty, int* kin
     return 0;
 }
 
-// Workspace of a backward call: two f32 per query row; with a dense mask on the 16-bit matrix-core kernels also the mask's
+// Workspace of a backward call: two f32 per query row; with a dense mask on the matrix-core kernels also the mask's
 // block flags (one byte per 32 rows x 32 keys, as the forward's: hidden blocks are skipped), behind them.
 static size_t bwd_rows_bytes(const incin_rocm_sdpa_desc_t* d) { return (2 * (size_t)(d->B * d->Hq * d->Sq) * sizeof(float) + 255) / 256 * 256; }
 static size_t bwd_flags_bytes(const incin_rocm_sdpa_desc_t* d, int kind)
 {
-    if (kind != 1 || !d->add_mask) return 0;
+    if (kind == 0 || !d->add_mask) return 0;
     const int64_t nbh = (d->mask_stride[0] ? d->B : 1) * (d->mask_stride[1] ? d->Hq : 1);
     return (size_t)(nbh * ((d->Sq + 31) / 32) * ((d->Skv + 31) / 32) + 255) / 256 * 256;
 }

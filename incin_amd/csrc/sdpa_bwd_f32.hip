@@ -110,7 +110,12 @@ __global__ __launch_bounds__(256) void bwd_f32_delta_kernel(SdpaBwdParams p)
 }
 
 // ---- dQ ----------------------------------------------------------------------------------------------------------------
-template <int D>
+// DENSE: a dense additive mask - its values (times log2 e) are added to the scores before the exponential; what it hides
+// (-inf) ends as P = 0 like the causal edge.  A lane owns a query: the 16 keys of a block are four 16-byte loads of its row
+// of the mask, asked for one tile ahead (right after the next tile's copies are issued) so that they arrive with that
+// tile.  The mask's block flags (mask_classify_kernel ran before) give the first and the last tile in which any row of the
+// workgroup sees a key: the tiles outside are left out.
+template <int D, bool DENSE = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 128 ? 1 : 2, D == 128 ? 1 : 2)))
 void bwd_f32_dq_kernel(SdpaBwdParams bp)
 {
@@ -156,8 +161,26 @@ void bwd_f32_dq_kernel(SdpaBwdParams bp)
     }
     if (q0 >= rows_b) j_end = 0;
     if (q0 + wave * 32 >= rows_b) lim_wave_min = lim_wave_max = 0;
-    const int n_tiles = (j_end + KT - 1) / KT;
+    int n_tiles = (j_end + KT - 1) / KT, t_first = 0;
     const int n_act = lim_wave_max > 0 ? (lim_wave_max + KT - 1) / KT : 0;
+    if (DENSE && p.mask_flags) {
+        __shared__ int s_seen[2];
+        const int nkb32 = (Skv + 31) >> 5, nrb32 = (Sq + 31) >> 5;
+        const uint8_t* fl = mask_flags_of(p, b, hq);
+        if (tid == 0) { s_seen[0] = 0x7fffffff; s_seen[1] = -1; }
+        __syncthreads();
+        int lo = 0x7fffffff, hi = -1;
+        for (int c = tid; c < min(NB * n_tiles, nkb32); c += 256) {
+            bool seen = false;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) seen = seen || fl[(int64_t)min((q0 >> 5) + w, nrb32 - 1) * nkb32 + c] != 2;
+            if (seen) { lo = min(lo, c); hi = max(hi, c); }
+        }
+        if (hi >= 0) { atomicMin(&s_seen[0], lo); atomicMax(&s_seen[1], hi); }
+        __syncthreads();
+        t_first = s_seen[1] < 0 ? 0 : __builtin_amdgcn_readfirstlane(s_seen[0]) / NB;
+        n_tiles = s_seen[1] < 0 ? 0 : min(n_tiles, __builtin_amdgcn_readfirstlane(s_seen[1]) / NB + 1);
+    }
 
     F32Addr<D> ad;
     ad.init(wave, lane, p.k_ss, p.v_ss, p.D, p.Dv);
@@ -203,11 +226,48 @@ void bwd_f32_dq_kernel(SdpaBwdParams bp)
 #pragma unroll
         for (int r = 0; r < 16; ++r) dq_acc[db][r] = 0.0f;
 
-    if (n_tiles > 0) issue_kv(0);
-    for (int t = 0; t < n_tiles; ++t) {
+    // DENSE: this lane's row of the mask; the values of a tile's keys, register r of block kb being key
+    // t * KT + 32 * kb + 8 * (r / 4) + 4 * g + r % 4
+    [[maybe_unused]] float4v m_next[NB][4], m_cur[NB][4];
+    [[maybe_unused]] const float* mrow = nullptr;
+    [[maybe_unused]] bool m_vec = false;
+    if (DENSE) {
+        mrow = (const float*)p.mask + (int64_t)b * p.m_sb + (int64_t)hq * p.m_sh + (int64_t)min(my_i, Sq - 1) * p.m_si;
+        m_vec = p.mask_vec && (reinterpret_cast<uintptr_t>(p.mask) & 15u) == 0;
+    }
+    [[maybe_unused]] auto load_mask = [&](int t) __attribute__((always_inline)) {
+#pragma unroll
+        for (int kb = 0; kb < NB; ++kb)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                const int j = t * KT + 32 * kb + 8 * r4 + 4 * g;
+                if (m_vec && j + 3 < Skv) m_next[kb][r4] = *(const float4v*)(mrow + j);
+                else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) m_next[kb][r4][e] = mrow[(int64_t)min(j + e, Skv - 1) * p.m_sj];
+                }
+            }
+    };
+    if (t_first < n_tiles) {
+        issue_kv(t_first);
+        if (DENSE) load_mask(t_first);
+    }
+    for (int t = t_first; t < n_tiles; ++t) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if (t + 1 < n_tiles) issue_kv(t + 1);
+        if (DENSE) {      // (arrived: a wait the compiler places for them is placed here, before the next copies are issued)
+#pragma unroll
+            for (int kb = 0; kb < NB; ++kb)
+#pragma unroll
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    m_cur[kb][r4] = m_next[kb][r4];
+                    asm volatile("" : "+v"(m_cur[kb][r4]));
+                }
+        }
+        if (t + 1 < n_tiles) {
+            issue_kv(t + 1);
+            if (DENSE) load_mask(t + 1);
+        }
         if (t >= n_act) continue;
         const char* kt = smem + (t & 1) * L::TILE_BYTES;
         const char* vt = smem + (2 + (t & 1)) * L::TILE_BYTES;
@@ -250,6 +310,10 @@ void bwd_f32_dq_kernel(SdpaBwdParams bp)
                 for (int r = 0; r < 16; ++r)
                     if (8 * (r / 4) + (r % 4) >= rel) s[r] = -INFINITY;
             }
+            if (DENSE) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) s[r] = __builtin_fmaf(m_cur[kb][r / 4][r % 4], 1.4426950408889634f, s[r]);
+            }
             // dS^T = P^T (dP^T - D); a masked pair has P = 0 and a finite second factor
 #pragma unroll
             for (int r = 0; r < 16; ++r) s[r] = __builtin_amdgcn_exp2f(s[r]) * dp[r];
@@ -286,7 +350,12 @@ void bwd_f32_dq_kernel(SdpaBwdParams bp)
 // ---- dK, dV ------------------------------------------------------------------------------------------------------------
 constexpr int BWD32_KEYS = 128;      // keys per workgroup: 32 per wavefront
 
-template <int D>
+// DENSE: a dense additive mask.  A lane owns a key and holds 16 query rows of a block: its values are 16 loads down a column
+// of the mask (one buffer descriptor per tile that starts at the tile's first row and ends with the head's last - rows past
+// Sq read zeros - one lane offset for the key's column and the lane's first row, a scalar offset per register; the host has
+// checked that a tile's rows fit 32-bit offsets), asked for one tile ahead like the dQ kernel's.  The block flags trim the
+// tiles to those between the first and the last block of rows, over the group's heads, that see any key of the workgroup.
+template <int D, bool DENSE = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(D == 128 ? 1 : 2, D == 128 ? 1 : 2)))
 void bwd_f32_dkv_kernel(SdpaBwdParams bp)
 {
@@ -331,11 +400,34 @@ void bwd_f32_dkv_kernel(SdpaBwdParams bp)
     const int i_begin_wg = p.causal ? clampi(j0 - coff, 0, Sq) : 0;
     // first query row that sees every key of this wavefront: tiles from there on need no mask
     const int i_all_wave = p.causal ? max(j0 + wave * 32 + 31 - coff, 0) : 0;
-    const int t_begin = i_begin_wg / QT;
+    int t_begin = i_begin_wg / QT;
     // query rows at and beyond rows_b are padding (q_lens): the tiles end there, and the rows between there and the end of
     // the last tile arrive as zeros like rows past Sq
     const int rows_b = p.q_lens ? clampi(p.q_lens[b], 0, Sq) : Sq;
-    const int n_qt = (rows_b + QT - 1) / QT;
+    int n_qt = (rows_b + QT - 1) / QT;
+    if (DENSE && p.mask_flags) {
+        __shared__ int s_seen[2];
+        const int nkb32 = (Skv + 31) >> 5, nrb32 = (Sq + 31) >> 5, c0 = kblk * 4;
+        if (tid == 0) { s_seen[0] = 0x7fffffff; s_seen[1] = -1; }
+        __syncthreads();
+        int lo = 0x7fffffff, hi = -1;
+        const int r_lo = NB * t_begin, r_n = min(NB * n_qt, nrb32) - r_lo;
+        for (int x = tid; x < r_n * p.G; x += 256) {
+            const int rb = r_lo + x % r_n;
+            const uint8_t* fl = mask_flags_of(p, b, hkv * p.G + x / r_n) + (int64_t)rb * nkb32;
+            bool seen = false;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) seen = seen || fl[min(c0 + c, nkb32 - 1)] != 2;
+            if (seen) { lo = min(lo, rb); hi = max(hi, rb); }
+        }
+        if (hi >= 0) { atomicMin(&s_seen[0], lo); atomicMax(&s_seen[1], hi); }
+        __syncthreads();
+        if (s_seen[1] < 0) n_qt = t_begin;
+        else {
+            t_begin = __builtin_amdgcn_readfirstlane(s_seen[0]) / NB;
+            n_qt = __builtin_amdgcn_readfirstlane(s_seen[1]) / NB + 1;
+        }
+    }
     const int tiles_per_head = j0 < kv_len ? max(n_qt - t_begin, 0) : 0;
     const int n_tiles = tiles_per_head * p.G;           // the group's query heads one after another
 
@@ -387,11 +479,41 @@ void bwd_f32_dkv_kernel(SdpaBwdParams bp)
         }
     };
 
-    if (n_tiles > 0) issue(0, 0);
+    // DENSE: the mask's values of a tile, register r of block qb being query row r0 + 32 * qb + 8 * (r / 4) + 4 * g + r % 4
+    [[maybe_unused]] float m_next[NB][16], m_cur[NB][16];
+    [[maybe_unused]] const int m_lane = (int)(((int64_t)min(my_j, Skv - 1) * p.m_sj + (int64_t)(4 * g) * p.m_si) * 4);
+    [[maybe_unused]] const int m_row4 = (int)(p.m_si * 4);
+    [[maybe_unused]] auto load_mask = [&](int n) __attribute__((always_inline)) {
+        const int h = n / tiles_per_head, r0 = (t_begin + n % tiles_per_head) * QT;
+        const float* mc = (const float*)p.mask + (int64_t)b * p.m_sb + (int64_t)(hkv * p.G + h) * p.m_sh + (int64_t)r0 * p.m_si;
+        const int64_t left = r0 < Sq ? ((int64_t)(Sq - 1 - r0) * p.m_si + (int64_t)(Skv - 1) * p.m_sj + 1) * 4 : 0;
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)mc, 0, (int)min(left, (int64_t)0x7fffffff), 0x00020000);
+#pragma unroll
+        for (int qb = 0; qb < NB; ++qb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                m_next[qb][r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, m_lane, (32 * qb + 8 * (r / 4) + (r % 4)) * m_row4, 0));
+    };
+    if (n_tiles > 0) {
+        issue(0, 0);
+        if (DENSE) load_mask(0);
+    }
     for (int n = 0; n < n_tiles; ++n) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if (n + 1 < n_tiles) issue(n + 1, (n + 1) & 1);
+        if (DENSE) {      // (arrived: a wait the compiler places for them is placed here, before the next copies are issued)
+#pragma unroll
+            for (int qb = 0; qb < NB; ++qb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    m_cur[qb][r] = m_next[qb][r];
+                    asm volatile("" : "+v"(m_cur[qb][r]));
+                }
+        }
+        if (n + 1 < n_tiles) {
+            issue(n + 1, (n + 1) & 1);
+            if (DENSE) load_mask(n + 1);
+        }
         const char* qt = smem + (n & 1) * STAGE;
         const char* gt = qt + L::TILE_BYTES;
         const char* nl = gt + L::TILE_BYTES;
@@ -438,6 +560,10 @@ void bwd_f32_dkv_kernel(SdpaBwdParams bp)
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
                     if (8 * (r / 4) + (r % 4) < rel) s[r] = -INFINITY;
+            }
+            if (DENSE) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) s[r] = __builtin_fmaf(m_cur[qb][r], 1.4426950408889634f, s[r]);
             }
             // rows past Sq arrive as zeros throughout (L' = 0, dO = 0: P = exp2(q.k) finite times dP = 0 for dS, and their
             // P meets dO = 0 in dV); rows without any visible key carry -inf already
@@ -489,7 +615,7 @@ void bwd_f32_dkv_kernel(SdpaBwdParams bp)
 #endif
 }
 
-template <int D>
+template <int D, bool DENSE = false>
 static hipError_t launch_bwd_f32_t(const SdpaBwdParams& bp, hipStream_t stream)
 {
     const SdpaParams& p = bp.f;
@@ -500,20 +626,22 @@ static hipError_t launch_bwd_f32_t(const SdpaBwdParams& bp, hipStream_t stream)
         const int64_t total = (int64_t)nqb * p.Hq * p.B;
         if (total > 0x7fffffffLL) return hipErrorInvalidValue;
         SdpaBwdParams bq = bp;
-        bq.f.interleave = work_interleave(p.causal != 0, (D == 128 ? 1 : 2) * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
+        bq.f.interleave = work_interleave(p.causal != 0 || p.mask != nullptr, (D == 128 ? 1 : 2) * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
         bq.f.deal_groups = (total & 7) == 0 ? work_deal(bq.f.interleave, p.G, nqb, total >> 3) : 0;
-        hipLaunchKernelGGL((bwd_f32_dq_kernel<D>), dim3((unsigned)total), dim3(256), 0, stream, bq);
+        hipLaunchKernelGGL((bwd_f32_dq_kernel<D, DENSE>), dim3((unsigned)total), dim3(256), 0, stream, bq);
     }
     const int nkb = (p.Skv + BWD32_KEYS - 1) / BWD32_KEYS;
     if ((int64_t)nkb * p.Hkv * p.B > 0)
-        hipLaunchKernelGGL((bwd_f32_dkv_kernel<D>), dim3((unsigned)((int64_t)nkb * p.Hkv * p.B)), dim3(256), 0, stream, bp);
+        hipLaunchKernelGGL((bwd_f32_dkv_kernel<D, DENSE>), dim3((unsigned)((int64_t)nkb * p.Hkv * p.B)), dim3(256), 0, stream, bp);
     return hipGetLastError();
 }
 
-// Host has validated: f32, D and Dv <= 128 in whole 16-byte vectors (bp.f.Dp = the instance: 64 or 128), no dense mask, finite scale, unit last-axis strides, 16-byte aligned rows,
-// row strides below 2^22 elements, lse and the workspace present.
+// Host has validated: f32, D and Dv <= 128 in whole 16-byte vectors (bp.f.Dp = the instance: 64 or 128), finite scale, unit last-axis strides, 16-byte aligned rows,
+// row strides below 2^22 elements, lse and the workspace present; a dense mask (the DENSE instances) of any non-negative strides
+// of which 64 rows fit 32-bit byte offsets, its block flags computed.
 hipError_t launch_sdpa_bwd_f32(const SdpaBwdParams& bp, hipStream_t stream)
 {
+    if (bp.f.mask) return bp.f.Dp == 128 ? launch_bwd_f32_t<128, true>(bp, stream) : launch_bwd_f32_t<64, true>(bp, stream);
     return bp.f.Dp == 128 ? launch_bwd_f32_t<128>(bp, stream) : launch_bwd_f32_t<64>(bp, stream);
 }
 

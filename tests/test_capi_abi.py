@@ -269,11 +269,11 @@ def test_backward_validation_and_workspace_size():
     # two f32 per query row, whichever kernels take the request
     assert capi.sdpa_bwd_workspace(_bwd()) == 2 * 2 * 4 * 128 * 4
     assert capi.sdpa_bwd_workspace(_bwd(dict(dtype=capi.F32))) == 2 * 2 * 4 * 128 * 4
-    # ... plus, for a dense mask on the 16-bit matrix-core kernels, the mask's block flags (a byte per 32 rows x 32 keys, in 256s)
+    # ... plus, for a dense mask on the matrix-core kernels, the mask's block flags (a byte per 32 rows x 32 keys, in 256s)
     assert capi.sdpa_bwd_workspace(_bwd(dict(add_mask=0x20000))) == 2 * 2 * 4 * 128 * 4 + 256
     assert capi.sdpa_bwd_workspace(_bwd(dict(add_mask=0x20000, mask_stride=(4 * 128 * 128, 128 * 128, 128, 1)))) == 2 * 2 * 4 * 128 * 4 + 256      # 8 mask planes x 16 flags, rounded up
     assert capi.sdpa_bwd_workspace(_bwd(dict(add_mask=0x20000, impl=capi.IMPL_GENERIC))) == 2 * 2 * 4 * 128 * 4
-    assert capi.sdpa_bwd_workspace(_bwd(dict(add_mask=0x20000, dtype=capi.F32))) == 2 * 2 * 4 * 128 * 4
+    assert capi.sdpa_bwd_workspace(_bwd(dict(add_mask=0x20000, dtype=capi.F32))) == 2 * 2 * 4 * 128 * 4 + 256
     assert capi.sdpa_bwd_workspace(_bwd(dict(Sq=0))) == 0            # nothing to compute
     for bd, code in [
         (_bwd(dict(lse=None)), capi.EINVAL),                          # the forward's normalisers are an input
@@ -281,7 +281,7 @@ def test_backward_validation_and_workspace_size():
         (_bwd(dict(impl=capi.IMPL_MFMA, D=160, Dv=160)), capi.EUNSUPPORTED),         # pinned to kernels that do not take it
         (_bwd(dict(impl=capi.IMPL_MFMA, D=36, Dv=36)), capi.EUNSUPPORTED),           # (72-byte rows are not whole vectors)
         (_bwd(dict(impl=capi.IMPL_MFMA, dtype=capi.F32, D=160, Dv=160)), capi.EUNSUPPORTED),
-        (_bwd(dict(impl=capi.IMPL_MFMA, dtype=capi.F32, add_mask=0x20000)), capi.EUNSUPPORTED),      # (the 16-bit kernels take a mask, the f32 ones do not)
+        (_bwd(dict(impl=capi.IMPL_MFMA, add_mask=0x20000, mask_stride=(0, 0, 1 << 25, 1))), capi.EUNSUPPORTED),      # (64 rows of the mask do not fit 32-bit offsets)
         (_bwd(dict(impl=capi.IMPL_SPLITKV)), capi.EUNSUPPORTED),
         (_bwd(dict(D=320, Dv=320)), capi.EUNSUPPORTED),
         (_bwd(dict(Hq=6, Hkv=4)), capi.ESHAPE),
