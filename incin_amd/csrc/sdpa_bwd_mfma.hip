@@ -247,7 +247,13 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
     int lim_wave_min = kv_len;
     if (p.causal) lim_wave_min = clampi(q0 + wave * 32 + coff + 1, 0, kv_len);
 
-    [[maybe_unused]] int fv[2] = {0, 0};      // DENSE: the two flags of the tile about to start, as loaded (asked for a tile ahead)
+    // DENSE: the two flags of a tile are asked for one tile ahead, after the copies of that tile are issued, and taken
+    // behind the tile barrier, before the next copies are issued: a load that is issued and consumed inside one tile makes
+    // the compiler wait for everything in flight - the next tile's copies, which it does not know of, included.  The values
+    // of a block that has any are such loads (there are no registers to hold them a tile ahead): a tile with values pays a
+    // memory latency that the second workgroup of the compute unit has to cover.
+    typedef T vec4 __attribute__((ext_vector_type(4)));
+    [[maybe_unused]] int fv[2] = {0, 0};
     [[maybe_unused]] auto tile_flags = [&](int t) __attribute__((always_inline)) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) fv[kb] = 2 * t + kb < nkb32 ? (int)mflags[2 * t + kb] : 2;
@@ -257,15 +263,18 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
         // K(t), V(t) have landed for everyone and everyone is done with tile t-1: the other pair of buffers is free
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
+        [[maybe_unused]] int flags_t[2] = {0, 0};
+        if (DENSE && mflags) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                asm volatile("" : "+v"(fv[kb]));
+                flags_t[kb] = __builtin_amdgcn_readfirstlane(fv[kb]);
+            }
+        }
         if (t + 1 < n_tiles) {
             tl.issue(0, kp, p.k_ss, Skv, (t + 1) * PF_BN, lds0 + ((t + 1) & 1) * L::TILE_BYTES, wave);
             tl.issue(1, vp, p.v_ss, Skv, (t + 1) * PF_BN, lds0 + (2 + ((t + 1) & 1)) * L::TILE_BYTES, wave);
-        }
-        [[maybe_unused]] int flags_t[2] = {0, 0};
-        if (DENSE && mflags) {
-            flags_t[0] = __builtin_amdgcn_readfirstlane(fv[0]);
-            flags_t[1] = __builtin_amdgcn_readfirstlane(fv[1]);
-            if (t + 1 < n_tiles) tile_flags(t + 1);
+            if (DENSE && mflags) tile_flags(t + 1);
         }
         if (t >= n_act) continue;
         const char* kt = smem + (t & 1) * L::TILE_BYTES;
@@ -282,7 +291,6 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
                 for (int r = 0; r < 16; ++r)
                     if (8 * (r / 4) + (r % 4) >= rel) s_acc[r] = -INFINITY;
             }
-            typedef T vec4 __attribute__((ext_vector_type(4)));
             [[maybe_unused]] vec4 mv[4];
             [[maybe_unused]] int flag = 0;
             if (DENSE && mflags) {
@@ -537,11 +545,36 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
     [[maybe_unused]] const int m_row2 = (int)(p.m_si * 2);
     [[maybe_unused]] const int nkb32 = (Skv + 31) >> 5, nrb32 = (Sq + 31) >> 5;
     [[maybe_unused]] const int my_kb32 = min(kblk * 4 + kb, nkb32 - 1);
-    // (the flag of a tile - this wavefront's query block of it - is asked for one tile ahead: tile_flag)
-    [[maybe_unused]] auto tile_flag = [&](int i0, int head) __attribute__((always_inline)) {
+    // The flag of a tile (this wavefront's query block of it) is asked for two tiles ahead and the values of a block that has
+    // any one tile ahead, right after the copies of that tile are issued, into registers of their own that are handed over
+    // behind the tile barrier: a load that is issued and consumed inside one step makes the compiler wait for everything in
+    // flight - the next tile's copies, which it does not know of, included: a memory latency in every step.
+    typedef T vec2 __attribute__((ext_vector_type(2)));
+    // (each value arrives in a register of its own - a 16-bit load into half a register would have to wait for the load
+    // of the other half - and two are packed into one at the hand-over)
+    [[maybe_unused]] vec2 mval[8];
+    [[maybe_unused]] unsigned mnext[16];
+    [[maybe_unused]] auto tile_of = [&](int n, int* i0, int* head) __attribute__((always_inline)) {       // n-th tile of the walk
+        *head = n / tiles_per_head;
+        *i0 = (t_begin + n % tiles_per_head) * PF_BN;
+    };
+    [[maybe_unused]] auto tile_flag = [&](int n) __attribute__((always_inline)) {
+        int i0, head;
+        tile_of(n, &i0, &head);
         return (int)mask_flags_of(p, b, hkv * p.G + head)[(int64_t)min((i0 >> 5) + role, nrb32 - 1) * nkb32 + my_kb32];
     };
-    auto step = [&](int stage, int pstage, int i0, bool has_prev, [[maybe_unused]] int head, [[maybe_unused]] int f_own, auto WITH_A_) __attribute__((always_inline)) {
+    [[maybe_unused]] auto tile_values = [&](int n) __attribute__((always_inline)) {      // register r is row i0 + 32 * role + 8 * (r / 4) + 4 * g + (r % 4)
+        int i0, head;
+        tile_of(n, &i0, &head);
+        const int row0 = i0 + 32 * role;
+        const T* mc = (const T*)p.mask + (int64_t)b * p.m_sb + (int64_t)(hkv * p.G + head) * p.m_sh + (int64_t)row0 * p.m_si;
+        const int64_t left = row0 < Sq ? ((int64_t)(Sq - 1 - row0) * p.m_si + (int64_t)(Skv - 1) * p.m_sj + 1) * 2 : 0;
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)mc, 0, (int)min(left, (int64_t)0x7fffffff), 0x00020000);
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            mnext[r] = (unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rs, m_lane, (8 * (r / 4) + (r % 4)) * m_row2, 0);
+    };
+    auto step = [&](int stage, int pstage, int i0, bool has_prev, [[maybe_unused]] int f_own, auto WITH_A_) __attribute__((always_inline)) {
         constexpr bool WITH_A = decltype(WITH_A_)::value;
         const char* qt = smem + stage * STAGE;
         const char* gt = qt + L::TILE_BYTES;
@@ -551,23 +584,12 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
         vec8 ring[R];
         floatx16 sa, da;
         vec8 pp[2], ds[2];
-        typedef T vec2 __attribute__((ext_vector_type(2)));
-        [[maybe_unused]] vec2 mval[8];       // (pairs: two 16-bit loads fill one register)
         [[maybe_unused]] bool own_hidden = false, own_zero = false;
         if (WITH_A && DENSE) {
             own_hidden = f_own == 2;
             own_zero = f_own == 1;
         }
         [[maybe_unused]] const bool own_values = WITH_A && DENSE && !own_zero && !own_hidden;
-        if (own_values) {      // register r is row i0 + 32 * role + 8 * (r / 4) + 4 * g + (r % 4); rows past the last repeat it
-            const int row0 = i0 + 32 * role;
-            const T* mc = (const T*)p.mask + (int64_t)b * p.m_sb + (int64_t)(hkv * p.G + head) * p.m_sh + (int64_t)row0 * p.m_si;
-            const int64_t left = row0 < Sq ? ((int64_t)(Sq - 1 - row0) * p.m_si + (int64_t)(Skv - 1) * p.m_sj + 1) * 2 : 0;
-            const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)mc, 0, (int)min(left, (int64_t)0x7fffffff), 0x00020000);
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-                mval[r / 2][r % 2] = __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b16(rs, m_lane, (8 * (r / 4) + (r % 4)) * m_row2, 0));
-        }
         if (WITH_A) {
             // The accumulators start from -L_i log2(e) and -D_i.  What the mask hides starts from -inf instead and ends as
             // P = 0, dS = 0 * (finite): only the causal edge needs that here, rows past Sq arrive as zeros throughout (dO = 0,
@@ -661,35 +683,47 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
         to_head(0);
         issue(0);
     }
-    int i0 = t_begin * PF_BN, stage = 0, pstage = 0, head = 0;
-    [[maybe_unused]] int fv_own = 0;      // the flag of the tile about to start, as loaded
-    if (DENSE && p.mask_flags && n_tiles > 0) fv_own = tile_flag(i0, 0);
+    int i0 = t_begin * PF_BN, stage = 0, pstage = 0;
+    // DENSE: the flags of tiles t and t + 1 (known), of tile t + 2 (asked for); without flags every block counts as one with values
+    [[maybe_unused]] int f_cur = 0, f_next = 0, fv_next2 = 0;
+    if (DENSE && n_tiles > 0) {
+        if (p.mask_flags) {
+            f_cur = __builtin_amdgcn_readfirstlane(tile_flag(0));
+            if (n_tiles > 1) fv_next2 = tile_flag(1);
+        }
+        if (f_cur == 0) tile_values(0);
+    }
     for (int t = 0; t < n_tiles; ++t) {
         // Tile t has landed for everyone, tile t - 1's P and dS are in the exchange buffer, and everyone is done with tile
         // t - 2: its stage is free for tile t + 1.
         __builtin_amdgcn_s_waitcnt(0x0F70);             // vmcnt(0)
         asm volatile("" ::: "memory");
         __syncthreads();
+        if (DENSE) {      // (arrived: waits the compiler places for these are placed here, before the next copies are issued)
+            asm volatile("" : "+v"(fv_next2));
+            f_next = t + 1 < n_tiles && p.mask_flags ? __builtin_amdgcn_readfirstlane(fv_next2) : 0;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) asm volatile("" : "+v"(mnext[i]));
+#pragma unroll
+            for (int i = 0; i < 8; ++i) mval[i] = __builtin_bit_cast(vec2, mnext[2 * i] | (mnext[2 * i + 1] << 16));
+        }
         const int nstage = stage == 2 ? 0 : stage + 1;
         if (t + 1 < n_tiles) issue(nstage);
-        const int i0_next = i0 + PF_BN >= n_qt * PF_BN ? t_begin * PF_BN : i0 + PF_BN;      // (then: next head of the group)
-        const int head_next = i0 + PF_BN >= n_qt * PF_BN ? head + 1 : head;
-        int f_own = 0;
-        if (DENSE && p.mask_flags) {
-            f_own = __builtin_amdgcn_readfirstlane(fv_own);
-            if (t + 1 < n_tiles) fv_own = tile_flag(i0_next, head_next);
+        if (DENSE) {
+            if (p.mask_flags && t + 2 < n_tiles) fv_next2 = tile_flag(t + 2);
+            if (t + 1 < n_tiles && f_next == 0) tile_values(t + 1);
         }
         // Every wavefront computes every tile: one whose keys no row of the tile sees (the first tile or two under a
         // causal mask) works on -inf, and would wait at the barriers for the others anyway.
-        step(stage, pstage, i0, t > 0, head, f_own, std::true_type{});
+        step(stage, pstage, i0, t > 0, f_cur, std::true_type{});
         pstage = stage;
         stage = nstage;
-        i0 = i0_next;
-        head = head_next;
+        i0 = i0 + PF_BN >= n_qt * PF_BN ? t_begin * PF_BN : i0 + PF_BN;      // (then: next head of the group)
+        f_cur = f_next;
     }
     if (n_tiles > 0) {
         __syncthreads();
-        step(stage, pstage, i0, true, head, 0, std::false_type{});
+        step(stage, pstage, i0, true, 0, std::false_type{});
     }
 
     if (my_j < Skv) {
