@@ -147,6 +147,17 @@ bool mask_rows_chunk_copyable(const incin_rocm_sdpa_desc_t* d)
     return extent < (1LL << 29);
 }
 
+// A 16-bit dense mask whose values the prefill kernel can bring into LDS by 16-byte copies, 32 rows x 64 keys at a time from a
+// descriptor that starts at the first of the 32 rows: unit key stride, a key count that is a multiple of 8 (no copy straddles
+// the end of the last row), every row 16-byte aligned, non-negative strides, 32 rows within the copies' 32-bit offsets.
+bool mask_rows_stageable(const incin_rocm_sdpa_desc_t* d)
+{
+    if (!d->add_mask || d->mask_stride[3] != 1 || d->Skv % 8 != 0 || (reinterpret_cast<uintptr_t>(d->add_mask) & 15u) != 0) return false;
+    for (int a = 0; a < 3; ++a)
+        if (d->mask_stride[a] < 0 || d->mask_stride[a] % 8 != 0) return false;
+    return (32 * d->mask_stride[2] + d->Skv) < (1LL << 29);
+}
+
 int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
 {
     if (!d) return fail(INCIN_ROCM_EINVAL, "scaled_dot_product_attention: null descriptor");
@@ -424,6 +435,7 @@ void fill_params(const incin_rocm_sdpa_desc_t* d, const Plan& plan, SdpaParams* 
     p->o_sb = d->o_stride[0]; p->o_sh = d->o_stride[1]; p->o_ss = d->o_stride[2];
     p->m_sb = d->mask_stride[0]; p->m_sh = d->mask_stride[1]; p->m_si = d->mask_stride[2]; p->m_sj = d->mask_stride[3];
     p->mask_vec = mask_rows_vector_loadable(d);
+    p->mask_chunks = d->dtype != INCIN_ROCM_F32 && mask_rows_stageable(d);
     p->B = (int)d->B; p->Hq = (int)d->Hq; p->Hkv = (int)d->Hkv; p->G = (int)(d->Hq / d->Hkv);
     p->Sq = (int)d->Sq; p->Skv = (int)d->Skv; p->D = (int)d->D; p->Dv = (int)d->Dv;
     p->Dp = std::max(d->D, d->Dv) <= 64 ? 64 : std::max(d->D, d->Dv) <= 128 ? 128 : 256;      // (means something to the matrix-core and split-KV kernels only)

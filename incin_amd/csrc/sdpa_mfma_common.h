@@ -106,14 +106,17 @@ __device__ __forceinline__ unsigned lds_address(const void* p)
 }
 __device__ __forceinline__ void dma_copy16(uint4v desc, unsigned lds_addr, int byte_offset)
 {
-    // (one wait state between the write of m0 and the copy that reads it)
-    asm volatile("s_nop 0\n\tbuffer_load_dwordx4 %0, %1, 0 offen lds" ::"v"(byte_offset), "s"(desc), "{m0}"(lds_addr) : "memory");
+    // (five wait states ahead of the copy: one is what a write of m0 needs before the copy that reads it, five what a vector
+    // instruction that wrote one of the descriptor's or the offset's scalar registers needs - the compiler brings spilled scalar
+    // registers back with v_readlane, may do so right in front of this statement, and does not see the memory instruction
+    // inside it, so it adds none itself; a copy that read a stale descriptor has fetched from wherever that pointed)
+    asm volatile("s_nop 4\n\tbuffer_load_dwordx4 %0, %1, 0 offen lds" ::"v"(byte_offset), "s"(desc), "{m0}"(lds_addr) : "memory");
 }
 // The same with a wavefront-uniform byte offset added to every lane's (the instruction's scalar offset operand): copies that
 // differ only by such an offset share one register of lane offsets.
 __device__ __forceinline__ void dma_copy16_at(uint4v desc, unsigned lds_addr, int byte_offset, int uniform_offset)
 {
-    asm volatile("s_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds" ::"v"(byte_offset), "s"(desc), "s"(uniform_offset), "{m0}"(lds_addr) : "memory");
+    asm volatile("s_nop 4\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds" ::"v"(byte_offset), "s"(desc), "s"(uniform_offset), "{m0}"(lds_addr) : "memory");
 }
 // Offset for the lane of such a copy that fetches 16-byte chunk `chunk` of row `row` (rows `row_bytes` apart in memory,
 // `data_bytes` of data each): a chunk at or beyond the row's data gets an offset that no descriptor covers, so that lane
@@ -126,7 +129,7 @@ __device__ __forceinline__ int dma_chunk_offset(int row, int row_bytes, int chun
 // The same for 64 lanes x 4 bytes (256 bytes of LDS).
 __device__ __forceinline__ void dma_copy4(uint4v desc, unsigned lds_addr, int byte_offset)
 {
-    asm volatile("s_nop 0\n\tbuffer_load_dword %0, %1, 0 offen lds" ::"v"(byte_offset), "s"(desc), "{m0}"(lds_addr) : "memory");
+    asm volatile("s_nop 4\n\tbuffer_load_dword %0, %1, 0 offen lds" ::"v"(byte_offset), "s"(desc), "{m0}"(lds_addr) : "memory");
 }
 
 // CU count of the current device (256 if the query fails: only launch geometry depends on it).

@@ -42,6 +42,7 @@ struct SdpaParams {
     const int32_t* mask_lims;
     int32_t lims_rows;         // rows per block of the launch that takes the blocks whose rows all have a limit (128 or 256; set by the launcher)
     int32_t mask_vec;          // 16-bit MFMA kernel: the mask's rows allow 8-byte loads of 4 consecutive keys
+    int32_t mask_chunks;       // 16-bit MFMA prefill kernel: the mask's rows can be copied into LDS 16 bytes (8 keys) at a time
 };
 
 typedef __bf16 bf16_t;

@@ -93,12 +93,17 @@ namespace incin_rocm {
 // the workgroups all of whose rows the mask gives n zeros and then -inf (mask_row_limits_kernel wrote n per row: a causal mask,
 // key padding, both): to them the tensor says nothing their limits do not, and they run exactly as without one.  A masked
 // request is two launches, LIMS then DENSE, and every block of p.lims_rows rows is computed by one of them: by LIMS if all
-// its rows have a limit, else by DENSE (whose 128-row workgroups look at the limits of the LIMS block that holds them).
+// its rows have a limit, else by DENSE (whose workgroups look at the limits of the LIMS block, or blocks, that hold their rows).
+// 3 (STAGED) is DENSE with the mask's values brought into LDS: every wavefront copies the 32 rows x 64 keys of its own rows a
+// tile ahead, with the K and V copies of that tile, into one of two 4 KiB buffers of its own (16-byte chunks XOR-swizzled by
+// row so that the 8-byte reads of a wavefront meet no bank conflict), and takes them from there.  A value loaded from memory
+// inside a tile would make the compiler wait for everything in flight - the next tiles' copies, which it does not know of,
+// included - a memory latency in every tile; and there are no registers to hold a tile's values a tile ahead.
 template <typename T, int D, int MASK, int NW, bool SPLIT = false, int KS = D / 16, int NB = D / 32>
 __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void sdpa_prefill_mfma_kernel(SdpaParams p)
 {
-    constexpr bool DENSE = MASK == 1, LIMS = MASK == 2;
+    constexpr bool STAGED = MASK == 3, DENSE = MASK == 1 || STAGED, LIMS = MASK == 2;
 #if defined(__HIP_DEVICE_COMPILE__)   // the body uses device-only types (buffer descriptors); the host pass needs only the stub
     typedef typename Mma<T>::vec8 vec8;
     typedef PfLayout<D> L;
@@ -178,7 +183,9 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     // the flags of this wavefront's tiles, two per tile, kept in LDS when they fit (up to 32768 keys): a flag is on
     // the path of every tile, and a global load there costs a memory latency per tile
     constexpr int FLAG_TILES = 512;
-    __shared__ uint8_t s_flags[DENSE ? NW * 2 * FLAG_TILES : 4];
+    __shared__ __attribute__((aligned(16))) uint8_t s_flags[DENSE ? NW * 2 * FLAG_TILES : 4];
+    __shared__ __attribute__((aligned(1024))) char s_mzone[STAGED ? NW * 2 * 4096 : 16];
+    [[maybe_unused]] bool wave_done = false;      // DENSE: this wavefront's rows were computed by the launch before (it keeps the barriers company)
     if ((DENSE || LIMS) && p.mask_lims != nullptr) {
         // does every row of the block of lims_rows rows around this workgroup's have a limit?  (uniform over the workgroup)
         const int32_t* lims = mask_lims_of(p, b, hq);
@@ -206,7 +213,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
             if (__builtin_amdgcn_readfirstlane(all ? 1 : 0) == 0) return;      // the dense-mask launch computes this block
             j_end = __builtin_amdgcn_readfirstlane(je);
             n_tiles = (j_end + PF_BN - 1) / PF_BN;
-        } else {
+        } else if (p.lims_rows >= BM) {
             const int blk0 = (q0 / p.lims_rows) * p.lims_rows, blk1 = min(blk0 + p.lims_rows, rows_b);
             bool ok = true;
             for (int i = blk0 + tid; i < blk1; i += 64 * NW) ok = ok && lims[p.m_si ? i : 0] >= 0;
@@ -218,6 +225,22 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
             for (int w2 = 0; w2 < NW; ++w2) all = all && s_range[w2] != 0;
             if (__builtin_amdgcn_readfirstlane(all ? 1 : 0) != 0) return;      // the launch before this one computed the block from its limits
             __syncthreads();                                                   // (s_range is used again below)
+        } else {
+            // blocks of 128 rows under a workgroup of 256: the launch before computed those of them whose rows all have a limit
+            const bool ok = my_i >= rows_b || lims[p.m_si ? my_i : 0] >= 0;
+            const bool wave_ok = __builtin_amdgcn_ballot_w64(!ok) == 0;
+            if (lane == 0) s_range[wave] = wave_ok ? 1 : 0;
+            __syncthreads();
+            bool all = true, mine_ok = true;
+#pragma unroll
+            for (int w2 = 0; w2 < NW; ++w2) {
+                all = all && s_range[w2] != 0;
+                if (w2 / 4 == wave / 4) mine_ok = mine_ok && s_range[w2] != 0;
+            }
+            if (__builtin_amdgcn_readfirstlane(all ? 1 : 0) != 0) return;
+            wave_done = __builtin_amdgcn_readfirstlane(mine_ok ? 1 : 0) != 0;
+            if (wave_done) lim_wave_min = lim_wave_max = 0;
+            __syncthreads();
         }
     }
     const bool flags_in_lds = DENSE && n_tiles <= FLAG_TILES;
@@ -225,7 +248,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
         mflags = mask_flags_of(p, b, hq) + (int64_t)((q0 >> 5) + wave) * nkb32;
         mrow = (const T*)p.mask + (int64_t)b * p.m_sb + (int64_t)hq * p.m_sh + (int64_t)min(my_i, Sq - 1) * p.m_si;
         int lo = 0x7fffffff, hi = -1;
-        if (q0 + wave * 32 < rows_b)
+        if (q0 + wave * 32 < rows_b && !wave_done)
             for (int t = lane; t < n_tiles; t += 64) {
                 const int f0 = mflags[2 * t], f1 = 2 * t + 1 < nkb32 ? mflags[2 * t + 1] : 2;
                 if (f0 != 2 || f1 != 2) { lo = min(lo, t); hi = max(hi, t); }
@@ -255,6 +278,43 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
         for (int off = 32; off >= 1; off >>= 1) z = min(z, __shfl_xor(z, off, 64));
         z_end = __builtin_amdgcn_readfirstlane(z);
     }
+
+    // flag of 32-key block blk (= 2 * tile + half) for this wavefront's rows; past the last block: hidden
+    [[maybe_unused]] auto flag_of = [&](int blk) __attribute__((always_inline)) -> int {
+        if (blk >= nkb32) return 2;
+        const int f = flags_in_lds ? (int)s_flags[wave * FLAG_TILES * 2 + blk] : (int)mflags[blk];
+        return __builtin_amdgcn_readfirstlane(f);
+    };
+    // STAGED: the copies of this wavefront's 32 rows x 64 keys of the mask for tile t into its buffer t % 2.  Copy c, lane l:
+    // row 8 c + l / 8, position l % 8 of the row's eight 16-byte chunks, which takes chunk (l % 8) ^ ((row / 2) % 8).  The
+    // descriptor starts at the wavefront's first row and ends with the head's last row (rows past Sq deliver zeros).
+    // ((row / 2) % 8 = (l / 16) ^ 4 (c % 2): two lane offsets serve the four copies, the rows' 8 c go into the scalar offset)
+    [[maybe_unused]] int m_voff[2];
+    [[maybe_unused]] int m_rd = 0;                 // this lane's read position in a buffer, before the XOR with the chunk it wants
+    [[maybe_unused]] uint4v m_desc = {0u, 0u, 0u, 0u};
+    [[maybe_unused]] unsigned m_lds = 0;
+    if (STAGED) {
+        const int row0 = q0 + wave * 32;
+#pragma unroll
+        for (int c = 0; c < 2; ++c) m_voff[c] = (int)((int64_t)(lane >> 3) * p.m_si * 2) + (((lane & 7) ^ (lane >> 4) ^ (4 * c)) << 4);
+        m_rd = ql * 128 + g * 8 + (((ql >> 1) & 7) << 4);
+        const int64_t left = row0 < Sq ? ((int64_t)(Sq - 1 - row0) * p.m_si + Skv) * 2 : 0;
+        m_desc = dma_descriptor((const T*)p.mask + (int64_t)b * p.m_sb + (int64_t)hq * p.m_sh + (int64_t)row0 * p.m_si,
+                                (int)(left > 0x7fffffffLL ? 0x7fffffffLL : left));
+        m_lds = lds_address(s_mzone) + wave * 2 * 4096;
+    }
+    [[maybe_unused]] auto issue_m = [&](int t) __attribute__((always_inline)) {
+        if (t >= n_tiles) return;
+        bool values;                                // does a block of the tile have any?
+        if (flags_in_lds) {                         // (both flags in one LDS read: this sits in front of every tile's copies)
+            const unsigned f2 = *(const unsigned short*)&s_flags[(wave * FLAG_TILES + t) * 2];
+            values = (f2 & 0xffu) == 0 || (f2 >> 8) == 0;
+        } else
+            values = flag_of(2 * t) == 0 || flag_of(2 * t + 1) == 0;
+        if (__builtin_amdgcn_readfirstlane(values ? 1 : 0) == 0) return;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) dma_copy16_at(m_desc, m_lds + (t & 1) * 4096 + c * 1024, m_voff[c % 2], t * PF_BN * 2 + c * 8 * (int)p.m_si * 2);
+    };
 
     // ---- global -> LDS copy plan ---------------------------------------------------
     // wavefront-wide load number ii = wave*LPW + c fills LDS bytes [ii*1024, ii*1024 + 1024)
@@ -306,6 +366,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     if (n_tiles > t_first) {
         issue_k(t_first, t_first & 1);
         if (t_first + 1 < n_tiles) issue_k(t_first + 1, (t_first + 1) & 1);
+        if (STAGED) { issue_m(t_first); issue_m(t_first + 1); }
     }
 
     // ---- LDS read addresses (bytes inside a tile buffer) ------------------------------------
@@ -455,6 +516,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
         __syncthreads();
     };
     auto turn_issue = [&](int t) __attribute__((always_inline)) {
+        if (STAGED) issue_m(t + 2);      // (into the buffer of tile t, whose values were taken before this turn; first: it reads a flag)
         if (t + 2 < n_tiles) issue_k(t + 2, t & 1);
         if (t + 1 < n_tiles) issue_v(t + 1, (t + 1) & 1);
     };
@@ -630,12 +692,6 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     // Dense mask on the scores of the tile that starts at key j0 (scores are in log2 units): per 32-key half, nothing
     // where the flag says zeros, -inf where it says hidden, else the values themselves - 4 consecutive keys per load
     // where the mask's layout allows (unit key stride, 8-byte aligned rows), element by element otherwise.
-    // flag of 32-key block blk (= 2 * tile + half) for this wavefront's rows; past the last block: hidden
-    auto flag_of = [&](int blk) __attribute__((always_inline)) -> int {
-        if (blk >= nkb32) return 2;
-        const int f = flags_in_lds ? (int)s_flags[wave * FLAG_TILES * 2 + blk] : (int)mflags[blk];
-        return __builtin_amdgcn_readfirstlane(f);
-    };
     auto add_dense_mask = [&](floatx16 (&sx)[2], int j0) __attribute__((always_inline)) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
@@ -651,7 +707,8 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
                 const int j = j0 + 32 * kb + 8 * r4 + 4 * g;
                 typedef T vec4 __attribute__((ext_vector_type(4)));
                 vec4 mv;
-                if (p.mask_vec && j + 3 < Skv) mv = *(const vec4*)(mrow + j);
+                if (STAGED) mv = *(const vec4*)(s_mzone + (wave * 2 + ((j0 / PF_BN) & 1)) * 4096 + (m_rd ^ ((4 * kb + r4) << 4)));
+                else if (p.mask_vec && j + 3 < Skv) mv = *(const vec4*)(mrow + j);
                 else {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) mv[e] = mrow[(int64_t)min(j + e, Skv - 1) * p.m_sj];
@@ -804,6 +861,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
 #undef SGB
 
     // ---- normalise and store ------------------------------------------------------------------
+    if (DENSE && wave_done) return;      // (every barrier is behind)
     const float l_tot = xor32_sum(l_run);
     if constexpr (SPLIT) {
         // partial result of this split: unnormalised O, and (reference, sum) in the log2 units the combine kernel takes for
@@ -847,7 +905,7 @@ static hipError_t launch_prefill_nw(const SdpaParams& p0, hipStream_t stream)
     // of the compute units per XCD
     p.interleave = work_interleave(p.causal != 0 || p.mask != nullptr, (8 / NW) * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
     p.deal_groups = (total & 7) == 0 ? work_deal(p.interleave, p.G, nqb, total >> 3) : 0;
-    constexpr bool DENSE = MASK == 1;
+    constexpr bool DENSE = MASK == 1 || MASK == 3;
     if constexpr (MASK == 0 && NW == 4) {
         if (p.num_splits > 1) {          // split launch: partial results, then the split-KV kernels' combine pass
             hipLaunchKernelGGL((sdpa_prefill_mfma_kernel<T, D, 0, 4, true>), dim3((unsigned)total, (unsigned)p.num_splits), dim3(256), 0, stream, p);
@@ -885,6 +943,9 @@ static hipError_t launch_prefill_t(const SdpaParams& p0, hipStream_t stream)
             const int64_t blocks256 = (int64_t)((p.Sq + 255) / 256) * p.Hq * p.B;
             p.lims_rows = D == 128 && (rows == 256 || (rows != 128 && p.Skv >= 4096 && blocks256 >= 6 * (int64_t)device_cus())) ? 256 : 128;
         }
+        // the mask's values through LDS where its layout allows the copies; at D = 128 in workgroups of 256 rows (the buffers
+        // of two workgroups of 128 would not fit a compute unit beside their K and V tiles)
+        if (p.mask_chunks) return launch_prefill_nw<T, D, 3, D == 128 ? 8 : 4>(p, stream);
     }
     if constexpr (D == 128 && MASK != 1) {
         // INCIN_ROCM_PREFILL_BLOCK_ROWS = 128 or 256 overrides the rule (for tests: small shapes through the 256-row form)
