@@ -185,6 +185,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     constexpr int FLAG_TILES = 512;
     __shared__ __attribute__((aligned(16))) uint8_t s_flags[DENSE ? NW * 2 * FLAG_TILES : 4];
     __shared__ __attribute__((aligned(1024))) char s_mzone[STAGED ? NW * 2 * 4096 : 16];
+    __shared__ __attribute__((aligned(1024))) char s_zero[STAGED ? 4096 : 16];      // zeros: what a tile of two all-zero blocks reads instead of a copy
     [[maybe_unused]] bool wave_done = false;      // DENSE: this wavefront's rows were computed by the launch before (it keeps the barriers company)
     if ((DENSE || LIMS) && p.mask_lims != nullptr) {
         // does every row of the block of lims_rows rows around this workgroup's have a limit?  (uniform over the workgroup)
@@ -262,6 +263,7 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
         w_first = __builtin_amdgcn_readfirstlane(lo);
         w_last = __builtin_amdgcn_readfirstlane(hi);
         if (lane == 0) { s_range[wave] = lo; s_range[NW + wave] = hi; }
+        if (STAGED && tid < 256) *(uint4v*)(s_zero + tid * 16) = uint4v{0u, 0u, 0u, 0u};
         __syncthreads();
         int g_lo = s_range[0], g_hi = s_range[NW];
 #pragma unroll
@@ -270,10 +272,14 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
         t_first = __builtin_amdgcn_readfirstlane(g_hi < 0 ? 0 : g_lo);
         n_tiles = __builtin_amdgcn_readfirstlane(g_hi + 1);      // (0 when the mask hides everything from these 128 rows)
         // z_end: the first tile after t_first in which the mask does something to this wavefront's rows; the tiles
-        // t_first + 1 .. z_end - 1 run through the pipelined loop like tiles of a launch without a mask
+        // t_first + 1 .. z_end - 1 run through the pipelined loop like tiles of a launch without a mask.  (STAGED: the first
+        // tile that the mask hides from this wavefront altogether, which it skips - every other tile has its values in LDS,
+        // zeros and -inf included, and goes through the pipelined loop)
         int z = n_tiles;
-        for (int t = t_first + 1 + lane; t < n_tiles; t += 64)
-            if (mflags[2 * t] != 1 || (2 * t + 1 < nkb32 ? mflags[2 * t + 1] : 2) != 1) { z = t; break; }
+        for (int t = t_first + 1 + lane; t < n_tiles; t += 64) {
+            const int f0 = mflags[2 * t], f1 = 2 * t + 1 < nkb32 ? mflags[2 * t + 1] : 2;
+            if (STAGED ? (f0 == 2 && f1 == 2) : (f0 != 1 || f1 != 1)) { z = t; break; }
+        }
 #pragma unroll
         for (int off = 32; off >= 1; off >>= 1) z = min(z, __shfl_xor(z, off, 64));
         z_end = __builtin_amdgcn_readfirstlane(z);
@@ -284,6 +290,14 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
         if (blk >= nkb32) return 2;
         const int f = flags_in_lds ? (int)s_flags[wave * FLAG_TILES * 2 + blk] : (int)mflags[blk];
         return __builtin_amdgcn_readfirstlane(f);
+    };
+    // both flags of tile t in one value: the second block's in bits 8 - 15 (one LDS read where the flags are there: this sits
+    // in front of every tile's copies and in every pipelined iteration)
+    [[maybe_unused]] auto tile_flags = [&](int t) __attribute__((always_inline)) -> unsigned {
+        unsigned f2;
+        if (flags_in_lds) f2 = *(const unsigned short*)&s_flags[(wave * FLAG_TILES + t) * 2];
+        else f2 = (unsigned)flag_of(2 * t) | ((unsigned)flag_of(2 * t + 1) << 8);
+        return (unsigned)__builtin_amdgcn_readfirstlane((int)f2);
     };
     // STAGED: the copies of this wavefront's 32 rows x 64 keys of the mask for tile t into its buffer t % 2.  Copy c, lane l:
     // row 8 c + l / 8, position l % 8 of the row's eight 16-byte chunks, which takes chunk (l % 8) ^ ((row / 2) % 8).  The
@@ -305,13 +319,9 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     }
     [[maybe_unused]] auto issue_m = [&](int t) __attribute__((always_inline)) {
         if (t >= n_tiles) return;
-        bool values;                                // does a block of the tile have any?
-        if (flags_in_lds) {                         // (both flags in one LDS read: this sits in front of every tile's copies)
-            const unsigned f2 = *(const unsigned short*)&s_flags[(wave * FLAG_TILES + t) * 2];
-            values = (f2 & 0xffu) == 0 || (f2 >> 8) == 0;
-        } else
-            values = flag_of(2 * t) == 0 || flag_of(2 * t + 1) == 0;
-        if (__builtin_amdgcn_readfirstlane(values ? 1 : 0) == 0) return;
+        // not for a tile the mask hides from this wavefront altogether (it skips the tile), nor for one of two all-zero blocks
+        // (it reads the zeros of s_zero instead)
+        if (tile_flags(t) == 0x0202u || tile_flags(t) == 0x0101u) return;
 #pragma unroll
         for (int c = 0; c < 4; ++c) dma_copy16_at(m_desc, m_lds + (t & 1) * 4096 + c * 1024, m_voff[c % 2], t * PF_BN * 2 + c * 8 * (int)p.m_si * 2);
     };
@@ -528,8 +538,11 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     // Hot iteration (tiles t and t+1 both computed by this wavefront, tile t+1 needs no mask):
     // probabilities of tile t (scores in sacc[par], their maximum in tmax) on the vector ALU while the matrix
     // pipe computes the scores of tile t+1; then O^T += V(t)^T P(t)^T with the maximum of S^T(t+1) underneath.
-    auto iter = [&](int t, auto PAR_) __attribute__((always_inline)) {
+    // WITH_M (STAGED): the mask's 32 values for this lane's scores of tile t + 1 are taken from the wavefront's buffer (zeros,
+    // -inf and values alike) and added on the way into the maximum, under the matrix instructions of the O^T update.
+    auto iter = [&](int t, auto PAR_, auto WITH_M_) __attribute__((always_inline)) {
         constexpr int par = decltype(PAR_)::value;
+        constexpr bool WITH_M = decltype(WITH_M_)::value;
         floatx16 (&sc)[2] = sacc[par];
         floatx16 (&sn)[2] = sacc[1 - par];
         const char* k_nxt = smem + (1 - par) * L::TILE_BYTES;        // K(t+1)
@@ -563,13 +576,27 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
         }
         __builtin_amdgcn_sched_barrier(0);
         l_run += rsum;
-        float m0 = sn[0][0], m1 = sn[1][0];
+        float m0 = WITH_M ? -INFINITY : sn[0][0], m1 = WITH_M ? -INFINITY : sn[1][0];
+        typedef T vec4 __attribute__((ext_vector_type(4)));
+        [[maybe_unused]] vec4 mv[2][2];      // the values of registers 4 r4 .. 4 r4 + 3 of both key blocks, read one group of four ahead
+        [[maybe_unused]] const char* mz = s_mzone + (wave * 2 + 1 - par) * 4096;      // (t + 1 has the parity 1 - par)
+        if (WITH_M && tile_flags(t + 1) == 0x0101u) mz = s_zero;
+        [[maybe_unused]] auto read_m = [&](int r4) __attribute__((always_inline)) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) mv[r4 % 2][kb] = *(const vec4*)(mz + (m_rd ^ ((4 * kb + r4) << 4)));
+        };
+        if (WITH_M) read_m(0);
 #pragma unroll
         for (int i = 0; i < NPV; ++i) {
             o_acc[i % NDB] = Mma<T>::run(vbuf[i % VD], pb[i / NDB], o_acc[i % NDB]);
             if (i + VD < NPV) read_v(v_cur, i + VD);
 #pragma unroll
             for (int r = pair_lo(i); r < pair_lo(i + 1); ++r) {
+                if (WITH_M) {
+                    if (r % 4 == 0 && r + 4 < 16) read_m(r / 4 + 1);
+                    sn[0][r] = __builtin_fmaf((float)mv[(r / 4) % 2][0][r % 4], 1.4426950408889634f, sn[0][r]);
+                    sn[1][r] = __builtin_fmaf((float)mv[(r / 4) % 2][1][r % 4], 1.4426950408889634f, sn[1][r]);
+                }
                 m0 = fmaxf(m0, sn[0][r]);
                 m1 = fmaxf(m1, sn[1][r]);
             }
@@ -582,8 +609,11 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
     // a score of tile t passed the reference by more than 2^SHIFT.  Only then (rare: the reference is the maximum of
     // an earlier tile) the exact path runs: maximum of tile t, reference moved, O^T and the row sum rescaled, both score
     // tiles shifted and the probabilities of tile t taken again - before anything of tile t has been accumulated.
-    auto iter_or = [&](int t, auto PAR_) __attribute__((always_inline)) {
+    // (WITH_M as in iter: the mask's values for tile t + 1 go onto its scores under the O^T update; the check of the next
+    // iteration then sees probabilities of scores that carry them)
+    auto iter_or = [&](int t, auto PAR_, auto WITH_M_) __attribute__((always_inline)) {
         constexpr int par = decltype(PAR_)::value;
+        constexpr bool WITH_M = decltype(WITH_M_)::value;
         floatx16 (&sc)[2] = sacc[par];
         floatx16 (&sn)[2] = sacc[1 - par];
         const char* k_nxt = smem + (1 - par) * L::TILE_BYTES;        // K(t+1)
@@ -666,6 +696,15 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
         }
         __builtin_amdgcn_sched_barrier(0);
         float rs[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        typedef T vec4 __attribute__((ext_vector_type(4)));
+        [[maybe_unused]] vec4 mv[2][2];      // the values of registers 4 r4 .. 4 r4 + 3 of both key blocks, read one group of four ahead
+        [[maybe_unused]] const char* mz = s_mzone + (wave * 2 + 1 - par) * 4096;      // (t + 1 has the parity 1 - par)
+        if (WITH_M && tile_flags(t + 1) == 0x0101u) mz = s_zero;
+        [[maybe_unused]] auto read_m = [&](int r4) __attribute__((always_inline)) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) mv[r4 % 2][kb] = *(const vec4*)(mz + (m_rd ^ ((4 * kb + r4) << 4)));
+        };
+        if (WITH_M) read_m(0);
 #pragma unroll
         for (int i = 0; i < NPV; ++i) {
             o_acc[i % NDB] = Mma<T>::run(vbuf[i % VD], pb[i / NDB], o_acc[i % NDB]);
@@ -675,13 +714,21 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
             for (int ii = pair_lo(i); ii < pair_lo(i + 1); ++ii) {
                 typename Mma<T>::vec2 pr = {pb[ii / 4][2 * (ii % 4)], pb[ii / 4][2 * (ii % 4) + 1]};
                 rs[ii % 4] = Mma<T>::add2(pr, rs[ii % 4]);
+                if (WITH_M) {
+                    const int r = ii;
+                    if (r % 4 == 0 && r + 4 < 16) read_m(r / 4 + 1);
+                    sn[0][r] = __builtin_fmaf((float)mv[(r / 4) % 2][0][r % 4], 1.4426950408889634f, sn[0][r]);
+                    sn[1][r] = __builtin_fmaf((float)mv[(r / 4) % 2][1][r % 4], 1.4426950408889634f, sn[1][r]);
+                }
             }
         }
+        if (!WITH_M) {
 #pragma unroll
-        for (int i = 0; i < NPV; ++i) {
-            SGB(SG_MFMA, 1);
-            if (pair_lo(i + 1) - pair_lo(i) == 1) SGB(SG_VALU, 1); else SGB(SG_VALU, 2);
-            if (i + VD < NPV) SGB(SG_DSR, 2);
+            for (int i = 0; i < NPV; ++i) {
+                SGB(SG_MFMA, 1);
+                if (pair_lo(i + 1) - pair_lo(i) == 1) SGB(SG_VALU, 1); else SGB(SG_VALU, 2);
+                if (i + VD < NPV) SGB(SG_DSR, 2);
+            }
         }
         asm volatile("" : "+v"(rs[0]), "+v"(rs[1]), "+v"(rs[2]), "+v"(rs[3]));      // (keeps the sums from being sunk below the next barrier)
         __builtin_amdgcn_sched_barrier(0);
@@ -764,15 +811,15 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
                         for (int r = 0; r < 16; ++r) sacc[0][kb][r] -= delta;
                 }
                 for (; t + 2 < n_hot; t += 2) {
-                    iter_or(t, std::integral_constant<int, 0>{});
-                    iter_or(t + 1, std::integral_constant<int, 1>{});
+                    iter_or(t, std::integral_constant<int, 0>{}, std::integral_constant<bool, STAGED>{});
+                    iter_or(t + 1, std::integral_constant<int, 1>{}, std::integral_constant<bool, STAGED>{});
                 }
                 tmax = max_of(sacc[0]);           // the masked loop below decides by maxima
             }
         } else {
             for (; t + 2 < n_hot; t += 2) {
-                iter(t, std::integral_constant<int, 0>{});
-                iter(t + 1, std::integral_constant<int, 1>{});
+                iter(t, std::integral_constant<int, 0>{}, std::false_type{});
+                iter(t + 1, std::integral_constant<int, 1>{}, std::false_type{});
             }
         }
         // the rest, one tile at a time without overlap; the pending scores are in sacc[0]
@@ -841,19 +888,20 @@ void sdpa_prefill_mfma_kernel(SdpaParams p)
                 if (pending && !(t & 1) && t + 2 < hot_end && __builtin_amdgcn_ballot_w64(!inited) == 0) {
                     adjust_reference(sacc[0]);
                     for (; t + 2 < hot_end; t += 2) {
-                        iter_or(t, std::integral_constant<int, 0>{});
-                        iter_or(t + 1, std::integral_constant<int, 1>{});
+                        iter_or(t, std::integral_constant<int, 0>{}, std::integral_constant<bool, STAGED>{});
+                        iter_or(t + 1, std::integral_constant<int, 1>{}, std::integral_constant<bool, STAGED>{});
                     }
                     tmax = max_of(sacc[0]);
                 }
                 plain_step();
             }
         } else {
+            // (STAGED: every tile's values are in LDS, zeros and -inf included, and the pipelined iteration adds them all: one code path)
             if ((t & 1) && t < n_tiles) plain_step();
             if (pending)
                 for (; t + 2 < hot_end; t += 2) {
-                    iter(t, std::integral_constant<int, 0>{});
-                    iter(t + 1, std::integral_constant<int, 1>{});
+                    iter(t, std::integral_constant<int, 0>{}, std::integral_constant<bool, STAGED>{});
+                    iter(t + 1, std::integral_constant<int, 1>{}, std::integral_constant<bool, STAGED>{});
                 }
             while (t < n_tiles) plain_step();
         }

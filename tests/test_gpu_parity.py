@@ -440,6 +440,52 @@ def test_auto_splits_the_keys_of_a_wide_prefill_launch_that_fills_the_device(gpu
 
 @pytest.mark.parametrize("dtype", [capi.BF16, capi.F16], ids=lambda x: dtypes.NAMES[x])
 @pytest.mark.parametrize("rows", ["128", "256"])
+@pytest.mark.parametrize("D", [128, 64])
+def test_mask_values_through_lds(gpu, dtype, rows, D, monkeypatch):
+    """A 16-bit mask whose rows can be copied 16 bytes at a time (unit key stride, a key count that is a multiple of 8, aligned
+    rows) reaches the prefill kernel's scores through LDS, a tile ahead of its use; tiles with values, tiles of zeros and
+    tiles with hidden blocks all go through the pipelined loop.  Against the oracle: values everywhere, a distance bias under
+    the causal triangle, a band, blocks of all three kinds at random, rows broadcast over queries, masks in which some blocks
+    of 128 rows are all limits (computed by the launch before, so that half of a 256-row workgroup has nothing to do) and
+    others carry values, on top of the causal flag and key counts, S_q not a multiple of the blocks; both workgroup forms."""
+    monkeypatch.setenv("INCIN_ROCM_PREFILL_BLOCK_ROWS", rows)
+    tol = TOL[dtype]
+    r = rng(SEED0 + 140 + D)
+    B, Hq, Hkv, Sq, Skv = 2, 4, 2, 600, 704
+    q, k, v = inputs(3200 + D, B, Hq, Hkv, Sq, Skv, D, D, dtype)
+    NEG = -np.inf
+    causal = O.causal_additive_mask(Sq, Skv).reshape(1, 1, Sq, Skv)
+    dist = (np.arange(Sq)[:, None] + (Skv - Sq) - np.arange(Skv)[None, :]).astype(np.float32)
+    cases = []
+    cases.append(("values everywhere [B,Hq,Sq,Skv]", r.standard_normal((B, Hq, Sq, Skv), dtype=np.float32), {}))
+    slopes = (0.5 ** np.arange(1, Hq + 1, dtype=np.float32))[:, None, None]
+    cases.append(("distance bias under the causal triangle [1,Hq,Sq,Skv]", np.where(dist >= 0, -dist[None] * slopes, NEG)[None].astype(np.float32), {}))
+    cases.append(("a band of 150 keys with a bias inside [Sq,Skv]", np.where((dist >= 0) & (dist < 150), -0.01 * dist, NEG).astype(np.float32), {}))
+    kinds = r.integers(0, 3, size=(1, Hq, (Sq + 31) // 32, (Skv + 31) // 32))
+    kinds[..., 0] = 1                                                                      # every row keeps visible keys
+    big = np.repeat(np.repeat(kinds, 32, axis=2), 32, axis=3)[:, :, :Sq, :Skv]
+    cases.append(("blocks hidden / zero / valued at random [1,Hq,Sq,Skv]", np.where(big == 0, NEG, np.where(big == 1, 0.0, r.standard_normal((1, Hq, Sq, Skv), dtype=np.float32))).astype(np.float32), {}))
+    cases.append(("one row of values for every query [B,1,1,Skv]", r.standard_normal((B, 1, 1, Skv), dtype=np.float32), {}))
+    mixed = np.broadcast_to(causal, (1, Hq, Sq, Skv)).copy()
+    mixed[0, :, 128:256] += r.standard_normal((Hq, 128, Skv), dtype=np.float32)           # rows 128..255 carry values, the blocks around them are limits
+    mixed[0, 1, 384:512, :40] = -2.0
+    cases.append(("causal, with blocks of 128 rows that carry values [1,Hq,Sq,Skv]", mixed, {}))
+    cases.append(("values under a causal flag and key counts", r.standard_normal((Sq, Skv), dtype=np.float32), dict(causal=True, kv_lens=np.array([704, 68], np.int32))))
+    for what, m, kw in cases:
+        say("mask values through LDS: %s, %s rows, D=%d, %s" % (dtypes.NAMES[dtype], rows, D, what))
+        m = dtypes.round_to(np.ascontiguousarray(m), dtype)
+        got, info = host.sdpa(q, k, v, dtype, mask=m, impl=capi.IMPL_MFMA, return_info=True, **kw)
+        assert info["impl"] == capi.IMPL_MFMA
+        full = np.broadcast_to(m, (B, Hq, Sq, Skv)).copy()             # (the oracle takes one mask: the flag and the counts folded in)
+        if kw.get("causal"):
+            full += causal
+        if kw.get("kv_lens") is not None:
+            full += np.where(np.arange(Skv)[None, :] < kw["kv_lens"][:, None], 0.0, NEG).astype(np.float32)[:, None, None, :]
+        check(got, oracle_full(q, k, v, G=Hq // Hkv, mask=full), tol, what)
+
+
+@pytest.mark.parametrize("dtype", [capi.BF16, capi.F16], ids=lambda x: dtypes.NAMES[x])
+@pytest.mark.parametrize("rows", ["128", "256"])
 @pytest.mark.parametrize("D", [128, 64, 256])
 def test_mask_tensors_whose_rows_are_zeros_then_minus_infinity(gpu, dtype, rows, D, monkeypatch):
     """A mask tensor whose every row is n zeros followed by -inf - the causal mask as the reference's callers build it, a
