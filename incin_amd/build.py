@@ -4,6 +4,7 @@ The library is built in-tree (incin_amd/lib/) so that it travels with the
 source tree; nothing is installed.  `python -m incin_amd.build` rebuilds it.
 """
 import os
+import shutil
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -31,11 +32,33 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-u
 
 
 def _compile(src):
-    obj = os.path.join(LIBDIR, os.path.splitext(src)[0] + ".o")
-    cmd = [HIPCC] + FLAGS + EXTRA_FLAGS.get(src, []) + ["-c", os.path.join(CSRC, src), "-o", obj]
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, r.stdout, r.stderr))
+    """One source to one object.  The compiler's intermediate files are kept for the duration (in a directory of their own,
+    removed afterwards) because one of them is the GPU assembly the object was made from: hazards.scan_asm reads it for
+    inline copies that sit too close behind a vector write of one of their scalar operands - something the compiler cannot
+    check, since it does not see the memory instruction inside the inline assembly."""
+    from . import hazards
+    name = os.path.splitext(src)[0]
+    obj = os.path.join(LIBDIR, name + ".o")
+    tmp = os.path.join(LIBDIR, "tmp_" + name)
+    shutil.rmtree(tmp, ignore_errors=True)
+    os.makedirs(tmp)
+    try:
+        tmp_obj = os.path.join(tmp, name + ".o")
+        cmd = [HIPCC] + FLAGS + EXTRA_FLAGS.get(src, []) + ["-save-temps=obj", "-c", os.path.join(CSRC, src), "-o", tmp_obj]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, r.stdout, r.stderr))
+        asm = [f for f in os.listdir(tmp) if f.endswith(".s") and "amdgcn" in f]
+        if not asm:
+            raise RuntimeError("no GPU assembly found for %s in %s" % (src, tmp))
+        for f in asm:
+            bad = hazards.check_file(os.path.join(tmp, f))
+            if bad:
+                raise RuntimeError("%s: inline copies fewer than %d wait states behind a vector write of a scalar operand:\n%s" % (
+                    src, hazards.NEEDED, "\n".join("  %s line %d: %s  <-  %s  (%d wait states)" % b for b in bad)))
+        os.replace(tmp_obj, obj)
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
     return obj
 
 

@@ -104,13 +104,20 @@ __device__ __forceinline__ unsigned lds_address(const void* p)
 {
     return (unsigned)(unsigned long long)(const __attribute__((address_space(3))) char*)p;
 }
+// Wait states in front of a copy.  One is what a write of m0 needs before the copy that reads it.  Five is what a vector
+// instruction that wrote one of the copy's scalar operands needs: the compiler brings spilled scalar registers back with
+// v_readlane_b32, may do so right in front of the statement, does not see the memory instruction inside it and so adds no
+// wait states itself - and a copy that read a stale descriptor has fetched from wherever that pointed (wrong values, or a
+// memory fault).  The copies of the K / V / Q / dO tiles, whose descriptors are put together by scalar instructions right
+// in front of them, keep one wait state (five cost the prefill kernel 0.5 - 1 %), and the build checks the code the compiler
+// wrote for every such copy (incin_amd/hazards.py: it fails if a vector write of an operand is nearer than five wait states);
+// the others (descriptors that live across a kernel and may come back from a spill) take five.
+#ifndef INCIN_DMA_WAIT
+#define INCIN_DMA_WAIT "s_nop 0"
+#endif
 __device__ __forceinline__ void dma_copy16(uint4v desc, unsigned lds_addr, int byte_offset)
 {
-    // (five wait states ahead of the copy: one is what a write of m0 needs before the copy that reads it, five what a vector
-    // instruction that wrote one of the descriptor's or the offset's scalar registers needs - the compiler brings spilled scalar
-    // registers back with v_readlane, may do so right in front of this statement, and does not see the memory instruction
-    // inside it, so it adds none itself; a copy that read a stale descriptor has fetched from wherever that pointed)
-    asm volatile("s_nop 4\n\tbuffer_load_dwordx4 %0, %1, 0 offen lds" ::"v"(byte_offset), "s"(desc), "{m0}"(lds_addr) : "memory");
+    asm volatile(INCIN_DMA_WAIT "\n\tbuffer_load_dwordx4 %0, %1, 0 offen lds" ::"v"(byte_offset), "s"(desc), "{m0}"(lds_addr) : "memory");
 }
 // The same with a wavefront-uniform byte offset added to every lane's (the instruction's scalar offset operand): copies that
 // differ only by such an offset share one register of lane offsets.
