@@ -784,6 +784,30 @@ def main():
                 "unit": "TFLOP/s", "ratio_to_causal_flag": wall / wall_m, "parity_max_abs_err": w.parity()}
             tm.free()
             mws.free()
+            # and with a mask that has values: a distance bias under the causal triangle (-0.01 per key of distance, -inf above
+            # the diagonal) - no row limit describes it; the kernel takes the values through LDS, a tile ahead
+            dist = np.arange(S, dtype=np.float32)[:, None] - np.arange(S, dtype=np.float32)[None, :]
+            bias = np.where(dist >= 0, -0.01 * dist, -np.inf).astype(np.float32)
+            tm = capi.DeviceBuffer.from_numpy(dtypes.encode(bias, capi.BF16))
+            w.desc.add_mask = tm.ptr
+            w.desc.workspace, w.desc.workspace_bytes = None, 0
+            mws = capi.DeviceBuffer(capi.sdpa_workspace(w.desc)[0])
+            w.desc.workspace, w.desc.workspace_bytes = mws.ptr, mws.nbytes
+            wall_b = w.time(args.steps, args.warmup)[0]
+            # (parity on sampled rows, against the oracle given the same tensor: the workload's own check knows the causal flag only)
+            qh, kh, vh = (dtypes.round_to(x, capi.BF16) for x in w.host)
+            rr = rng(98)
+            rows = np.stack([rr.integers(0, B * H, 48), rr.integers(0, S, 48)], axis=1)
+            rows[0], rows[1] = (0, 0), (B * H - 1, S - 1)
+            ref = O.sdpa_rows(qh.reshape(B, H, 1, S, D), kh[:, :, None], vh[:, :, None], rows, mask=dtypes.round_to(bias, capi.BF16).reshape(1, 1, 1, S, S))
+            got = w.to.to_f32().reshape(B * H, S, D)[rows[:, 0], rows[:, 1]]
+            result["prefill_with_bias_tensor"] = {
+                "what": "config 3 with a distance bias under the causal triangle as a bf16 [S, S] additive tensor (values: no "
+                        "row limit describes it); same FLOP count", "ms_per_step": wall_b, "value": flops / (wall_b * 1e-3) / 1e12,
+                "unit": "TFLOP/s", "ratio_to_causal_flag": wall / wall_b, "parity_max_abs_err": float(np.abs(got - ref).max()),
+                "parity_sample": "48 sampled rows against the oracle given the same tensor"}
+            tm.free()
+            mws.free()
         w.free()
         if not args.no_cpu_baseline:
             slices = 12
