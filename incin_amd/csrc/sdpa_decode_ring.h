@@ -22,7 +22,9 @@ constexpr int DM_SLOT_BYTES = 8192;      // a block of K or of V: 16-bit storage
 #endif
 __device__ __forceinline__ void dm_copy16(uint4v desc, unsigned lds_addr, int byte_offset)
 {
-    asm volatile("s_nop 4\n\tbuffer_load_dwordx4 %0, %1, 0 offen" DM_CACHE " lds" ::"v"(byte_offset), "s"(desc), "{m0}"(lds_addr) : "memory");
+    // (one wait state, as dma_copy16: the descriptors of these copies are put together right in front of them, and the build
+    // checks the generated code)
+    asm volatile(INCIN_DMA_WAIT "\n\tbuffer_load_dwordx4 %0, %1, 0 offen" DM_CACHE " lds" ::"v"(byte_offset), "s"(desc), "{m0}"(lds_addr) : "memory");
 }
 
 // All but the newest NSLOT - 1 copies of this wavefront (CPB instructions each: 8 for an 8 KiB slot) have landed.
