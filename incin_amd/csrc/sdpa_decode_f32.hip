@@ -180,27 +180,33 @@ __global__ __launch_bounds__(256) void sdpa_decode_f32_kernel(SdpaParams p)
         ++issued;
         slot_in = slot_in + 1 == NSLOT ? 0 : slot_in + 1;
     };
-    for (int u = 0; u < NSLOT; ++u) issue_next();
-
     // ---- operands ----------------------------------------------------------------------------------------------
-    // Q'^T = (Q * scale * log2 e)^T (B operand, resident): this lane's row, floats 16 j + 4 g .. + 3 of it per group j
+    // Q'^T = (Q * scale * log2 e)^T (B operand, resident): this lane's row, floats 16 j + 4 g .. + 3 of it per group j.  All of
+    // its loads are asked for first, every lane from an address that exists (a lane beyond the head dimension reads the row's
+    // start, a row that does not exist is row 0 of the group's first head), and nothing looks at them until the first copies
+    // are on their way too: a load that is scaled right behind its issue waits for itself, one after the other, and behind
+    // the copies for all of those as well.
     floatx4 qreg[NRB][NJ];
+#pragma unroll
+    for (int rb = 0; rb < NRB; ++rb) {
+        const float* qrow = (const float*)p.q + (int64_t)b * p.q_sb + (int64_t)hq[rb] * p.q_sh + (int64_t)qi[rb] * p.q_ss;
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) qreg[rb][j] = *(const floatx4*)(qrow + (j * 16 + g * 4 < p.D ? j * 16 + g * 4 : 0));
+    }
+    for (int u = 0; u < NSLOT; ++u) issue_next();
+    __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0), told to the compiler too: the Q rows (and the first copies) have arrived
+    asm volatile("" ::: "memory");
     {
         const float c2 = p.scale * 1.4426950408889634f;      // scores in log2 units
 #pragma unroll
-        for (int rb = 0; rb < NRB; ++rb) {
-            const float* qrow = (const float*)p.q + (int64_t)b * p.q_sb + (int64_t)hq[rb] * p.q_sh + (int64_t)qi[rb] * p.q_ss + g * 4;
+        for (int rb = 0; rb < NRB; ++rb)
 #pragma unroll
             for (int j = 0; j < NJ; ++j) {
                 const bool in = valid[rb] && j * 16 + g * 4 < p.D;      // (rows that do not exist, and beyond the head dimension: zeros, like K's)
-                if (j * 16 + g * 4 < p.D) qreg[rb][j] = *(const floatx4*)(qrow + j * 16);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) qreg[rb][j][e] = in ? qreg[rb][j][e] * c2 : 0.0f;
             }
-        }
     }
-    __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0), told to the compiler too: the Q rows (and the first copies) have arrived
-    asm volatile("" ::: "memory");
     // K operand of group j: row n of the sub-block, logical chunk 4 j + g, stored at chunk (4 j + g) ^ f(n) = (g ^ f(n)) ^ 4 j;
     // the row's offset, the chunk bits of g ^ f and those of 4 j share no bits, so the address is k_base ^ (j << 6).
     const int k_base = ql * L::ROWB + ((g ^ L::f(ql)) << 4);

@@ -147,24 +147,29 @@ __global__ __launch_bounds__(256) void sdpa_decode_mfma_kernel(SdpaParams p)
         ++issued;
         slot_in = slot_in + 1 == NSLOT ? 0 : slot_in + 1;
     };
-    for (int u = 0; u < NSLOT; ++u) issue_next();
-
     // ---- operands ----------------------------------------------------------------------------------------------
-    // Q^T (B operand, resident): this lane's row, elements 16 s + 8 g .. + 7 of it per k-step s
+    // Q^T (B operand, resident): this lane's row, elements 16 s + 8 g .. + 7 of it per k-step s.  All of its loads are asked
+    // for first, every lane from an address that exists (a lane beyond the head dimension reads the row's start, a row that
+    // does not exist is row 0 of the group's first head), and nothing looks at them until the first copies are on their way
+    // too: a load that is looked at right behind its issue waits for itself, eight of them one after the other, and behind
+    // the copies for all of those as well.
     vec8 qreg[NRB][NSTEP];
 #pragma unroll
     for (int rb = 0; rb < NRB; ++rb) {
-        const T* qrow = (const T*)p.q + (int64_t)b * p.q_sb + (int64_t)hq[rb] * p.q_sh + (int64_t)qi[rb] * p.q_ss + g * 8;
+        const T* qrow = (const T*)p.q + (int64_t)b * p.q_sb + (int64_t)hq[rb] * p.q_sh + (int64_t)qi[rb] * p.q_ss;
 #pragma unroll
-        for (int s = 0; s < NSTEP; ++s) {
-            if (s * 16 + g * 8 < p.D) qreg[rb][s] = *(const vec8*)(qrow + s * 16);
+        for (int s = 0; s < NSTEP; ++s) qreg[rb][s] = *(const vec8*)(qrow + (s * 16 + g * 8 < p.D ? s * 16 + g * 8 : 0));
+    }
+    for (int u = 0; u < NSLOT; ++u) issue_next();
+    __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0), told to the compiler too: the Q rows (and the first copies) have arrived
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int rb = 0; rb < NRB; ++rb)
+#pragma unroll
+        for (int s = 0; s < NSTEP; ++s)
             if (!valid[rb] || s * 16 + g * 8 >= p.D)      // (rows that do not exist, and beyond the head dimension: zeros, like K's)
 #pragma unroll
                 for (int e = 0; e < 8; ++e) qreg[rb][s][e] = (T)0.0f;
-        }
-    }
-    __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0), told to the compiler too: the Q rows (and the first copies) have arrived
-    asm volatile("" ::: "memory");
     // K operand: lane (ql, g) reads row ql, logical chunk 2 s + g
     int k_addr[NSTEP];
     {
