@@ -52,7 +52,7 @@ TRAFFIC_KIB = {   # leg/shape/variant: (FETCH_SIZE, WRITE_SIZE)
     "decode_gqa/f32_gqa4_b32_kv8192/auto": (1048910, 512), "decode_gqa/f32_gqa4_b32_kv8192/vector_alu": (1050700 + 2152, 4352 + 512),
     "decode_gqa/f32_gqa8_sq4_b8_kv8192/auto": (266342 + 4264, 8704.3 + 1024),
     "head_dims/prefill_d96": (109157, 62546.7), "head_dims/prefill_d256": (556912, 131083), "head_dims/chunk_d256": (68960.5 + 33320.5, 67438.4 + 4096),
-    "head_dims/decode_d96": (393400, 192), "head_dims/decode_d256": (1048960, 512),
+    "head_dims/decode_d96": (393400, 192), "head_dims/decode_d256": (1048960, 512), "head_dims/prefill_d96_s4096": (206387, 123320),
     "prefill_chunk/bf16_sq128_kv32768/auto": (66326.4 + 16680.5, 33392.9 + 1024), "prefill_chunk/bf16_sq128_kv32768/unsplit": (66199.5, 1024),
     "prefill_chunk/bf16_sq512_kv32768/auto": (67708 + 17448.5, 33677.2 + 4096), "prefill_chunk/bf16_sq512_kv32768/unsplit": (67735.5, 4096),
     "prefill_chunk/f32_sq128_kv32768/auto": (132204 + 16680, 33316.9 + 2048), "prefill_chunk/f32_sq128_kv32768/unsplit": (132192, 2048),
@@ -358,7 +358,8 @@ def head_dims_leg(steps, warmup, only_shape=None):
     names = {capi.IMPL_SPLITKV_MFMA: "sdpa_decode_mfma_kernel", capi.IMPL_MFMA: "sdpa_prefill_mfma_kernel", capi.IMPL_GENERIC: "sdpa_generic_kernel"}
     for i, (name, B, Hq, Hkv, Sq, Skv, D, causal) in enumerate((("prefill_d96", 8, 16, 16, 2048, 2048, 96, True), ("prefill_d256", 4, 16, 16, 4096, 4096, 256, True),
                                                                  ("chunk_d256", 1, 32, 8, 256, 16384, 256, True),
-                                                                 ("decode_d96", 32, 32, 8, 1, 8192, 96, False), ("decode_d256", 32, 32, 8, 1, 8192, 256, False))):
+                                                                 ("decode_d96", 32, 32, 8, 1, 8192, 96, False), ("decode_d256", 32, 32, 8, 1, 8192, 256, False),
+                                                                 ("prefill_d96_s4096", 8, 16, 16, 4096, 4096, 96, True))):      # (config 3's shape at D = 96)
         if only_shape is not None and name != only_shape:
             continue
         w = Workload("head_dims_" + name, SEED0 + 80 + i, B, Hq, Hkv, Sq, Skv, D, capi.BF16, causal)
