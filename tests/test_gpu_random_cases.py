@@ -157,3 +157,42 @@ def test_random_cases_over_head_dimensions(gpu):
     say("kernels exercised: %s" % used)
     for impl in (capi.IMPL_GENERIC, capi.IMPL_MFMA, capi.IMPL_SPLITKV_MFMA):
         assert used.get(impl, 0) >= 5, "kernel %d was hardly reached: %s" % (impl, used)
+
+
+def test_random_cases_with_masks_whose_rows_can_be_copied(gpu):
+    """The same differential draw aimed at the path that takes a 16-bit mask's values through LDS (key counts that are
+    multiples of 8, so that the mask's rows are 16-byte aligned): every case has a mask - values with holes, or blocks of 32 x 32
+    that are hidden, zero or valued at random, or a band - with any of its leading axes broadcast, under the causal flag and key
+    counts or not, query counts that do not fill the workgroups, grouped queries, head dimensions the instances take whole and
+    padded; every kernel the planner accepts for each case."""
+    r = np.random.Generator(np.random.PCG64(20261127))
+    used = {}
+    for i in range(60):
+        dtype = int(r.choice([capi.F16, capi.BF16]))
+        D = int(r.choice([64, 128, 128, 80, 32]))
+        Dv = D if r.random() < 0.8 else int(r.choice([64, 128]))
+        Hkv, G, B = int(r.integers(1, 4)), int(r.choice([1, 1, 2, 4])), int(r.integers(1, 4))
+        Skv = 8 * int(r.integers(1, 90))
+        Sq = Skv if r.random() < 0.5 else int(r.integers(1, 700))
+        causal = bool(r.random() < 0.4)
+        lens = r.integers(0, Skv + 1, B).astype(np.int32) if r.random() < 0.3 else None
+        shp = [B if r.random() < 0.5 else 1, Hkv * G if r.random() < 0.5 else 1, Sq if r.random() < 0.8 else 1, Skv]
+        kind = r.choice(["holes", "blocks", "band", "values"])
+        mask = r.standard_normal(shp, dtype=np.float32)
+        if kind == "holes":
+            mask[r.random(shp) < 0.2] = -np.inf
+        elif kind == "blocks":
+            kinds = r.integers(0, 3, size=(shp[0], shp[1], (shp[2] + 31) // 32, (Skv + 31) // 32))
+            big = np.repeat(np.repeat(kinds, 32, axis=2), 32, axis=3)[:, :, :shp[2], :Skv]
+            mask = np.where(big == 0, -np.inf, np.where(big == 1, 0.0, mask)).astype(np.float32)
+        elif kind == "band" and shp[2] > 1:
+            dist = np.arange(Sq)[:, None] + (Skv - Sq) - np.arange(Skv)[None, :]
+            mask = np.where((np.abs(dist) <= int(r.integers(8, 200)))[None, None], 0.1 * mask, -np.inf).astype(np.float32)
+        c = dict(dtype=dtype, B=B, Hkv=Hkv, G=G, Sq=Sq, Skv=Skv, D=D, Dv=Dv, causal=causal, lens=lens, mask=mask,
+                 scale=None if r.random() < 0.6 else float(r.uniform(0.02, 0.4)))
+        if i % 20 == 0:
+            say("random case (copyable masks) %d/60" % i)
+        for impl in run_case(2000 + i, c, r):
+            used[impl] = used.get(impl, 0) + 1
+    say("kernels exercised: %s" % used)
+    assert used.get(capi.IMPL_MFMA, 0) >= 40, "the prefill kernels were hardly reached: %s" % used
