@@ -219,6 +219,49 @@ def test_matrix_core_backward_with_a_dense_mask(gpu, dtype, shape):
         compare(name + " generic vs matrix-core", gx, x, tol=1e-5 if f32 else 1e-2)
 
 
+def test_backward_random_cases_with_a_dense_mask(gpu):
+    """Seeded random shapes with a mask tensor on the matrix-core backward kernels, all three dtypes: values with holes, blocks
+    of 32 x 32 hidden / zero / valued at random, a band; any leading axis of the mask broadcast; lengths on either side of the
+    tiles; with and without the causal flag and key counts.  Column 0 of every mask row stays visible (and row 0 sees key 0
+    under the causal alignment with Sq <= Skv), so the oracle has no NaN.  Each case is printed before it runs."""
+    r = np.random.Generator(np.random.PCG64(2027))
+    for case in range(30):
+        dtype = (capi.BF16, capi.F16, capi.F32)[case % 3]
+        D = 128 if case % 2 else 64
+        B, Hkv, G = int(r.integers(1, 3)), int(r.integers(1, 3)), int(r.choice([1, 2, 4]))
+        Skv = int(r.choice([r.integers(1, 70), r.integers(60, 140), r.integers(120, 420)]))
+        causal = bool(r.integers(0, 2))
+        Sq = int(r.integers(1, Skv + 1)) if causal else int(r.integers(1, 300))
+        lens = r.integers(1, Skv + 1, B).astype(np.int32) if r.integers(0, 2) else None
+        Hq = Hkv * G
+        shp = [B if r.random() < 0.5 else 1, Hq if r.random() < 0.5 else 1, Sq if r.random() < 0.8 else 1, Skv]
+        kind = str(r.choice(["holes", "blocks", "band"]))
+        mask = r.standard_normal(shp, dtype=np.float32)
+        if kind == "holes":
+            mask[r.random(shp) < 0.25] = -np.inf
+        elif kind == "blocks":
+            kinds = r.integers(0, 3, size=(shp[0], shp[1], (shp[2] + 31) // 32, (Skv + 31) // 32))
+            big = np.repeat(np.repeat(kinds, 32, axis=2), 32, axis=3)[:, :, :shp[2], :Skv]
+            mask = np.where(big == 0, -np.inf, np.where(big == 1, 0.0, mask)).astype(np.float32)
+        elif shp[2] > 1:
+            dist = np.arange(Sq)[:, None] + (Skv - Sq) - np.arange(Skv)[None, :]
+            mask = np.where((np.abs(dist) <= int(r.integers(8, 120)))[None, None], 0.1 * mask, -np.inf).astype(np.float32)
+        mask[..., 0] = 0.0
+        mask = dtypes.round_to(mask, dtype)
+        say("masked backward random case %d: dtype=%d D=%d B=%d Hq=%d Hkv=%d Sq=%d Skv=%d causal=%s lens=%s mask %s %r"
+            % (case, dtype, D, B, Hq, Hkv, Sq, Skv, causal, None if lens is None else lens.tolist(), kind, tuple(shp)))
+        q, k, v, go = make(300 + case, B, Hq, Hkv, Sq, Skv, D, dtype)
+        out, dq, dk, dv = host.sdpa_backward(q, k, v, go, dtype, causal=causal, kv_lens=lens, mask=mask, impl=capi.IMPL_MFMA)
+        m5 = np.broadcast_to(mask, (B, Hq, Sq, Skv)).reshape(B, Hkv, G, Sq, Skv)
+        rq, rk, rv = BW.sdpa_backward(q.reshape(B, Hkv, G, Sq, D), k[:, :, None], v[:, :, None], go.reshape(B, Hkv, G, Sq, D),
+                                      mask=m5, causal=causal, kv_lens=None if lens is None else lens.reshape(B, 1, 1))
+        assert not np.isnan(rq).any(), "case construction: a row without keys"
+        tol = 1e-5 if dtype == capi.F32 else 2e-2
+        compare("dq", dq, rq.reshape(B, Hq, Sq, D), tol=tol)
+        compare("dk", dk, rk.reshape(B, Hkv, Skv, D), tol=tol)
+        compare("dv", dv, rv.reshape(B, Hkv, Skv, D), tol=tol)
+
+
 @pytest.mark.parametrize("dtype,dims", [(capi.BF16, (96, 96)), (capi.BF16, (40, 72)), (capi.F16, (128, 64)), (capi.BF16, (8, 8)), (capi.F16, (80, 80)),
                                         (capi.F32, (96, 96)), (capi.F32, (20, 36)), (capi.F32, (128, 64)), (capi.F32, (4, 4))],
                          ids=lambda x: dtypes.NAMES[x] if isinstance(x, int) else "D%d_Dv%d" % x)
