@@ -9,18 +9,20 @@ sees, and restores spilled scalar registers with exactly such v_readlane_b32 ins
 reads a stale descriptor fetches from wherever that pointed: wrong values, or a memory fault.
 
 `scan_asm` walks the assembly the compiler wrote for a source file (kept with -save-temps while building) and reports every
-inline copy with fewer than five wait states between it and a vector write of one of its scalar operands.  The build fails
+inline copy with fewer than five wait states between it and a vector write of one of its scalar operands (m0, which holds
+the copy's LDS address, among them).  The build fails
 on a report; the remedy is a longer `s_nop` in front of the copy in question (sdpa_mfma_common.h, sdpa_decode_ring.h).
 """
 import re
 
 NEEDED = 5
 _SREG = re.compile(r"\bs(\d+)\b|\bs\[(\d+):(\d+)\]")
-_VALU_SGPR_WRITE = re.compile(r"^\s*(v_readlane_b32|v_readfirstlane_b32|v_cmp\w*_e64|v_cmpx\w*_e64)\s+(s\[\d+:\d+\]|s\d+)")
+_VALU_SGPR_WRITE = re.compile(r"^\s*(v_readlane_b32|v_readfirstlane_b32|v_cmp\w*_e64|v_cmpx\w*_e64)\s+(s\[\d+:\d+\]|s\d+|m0)")
+M0 = -1          # (m0, which every copy into LDS reads for its LDS address, stands in the register sets as -1)
 
 
 def _sregs(text):
-    regs = set()
+    regs = {M0} if re.search(r"\bm0\b", text) else set()
     for m in _SREG.finditer(text):
         if m.group(1) is not None:
             regs.add(int(m.group(1)))
@@ -47,7 +49,7 @@ def scan_asm(text):
         if not (t.startswith("buffer_load") and t.endswith("lds")):
             continue
         operands = t.split(None, 1)[1]
-        regs = _sregs(operands.replace("m0", ""))
+        regs = _sregs(operands) | {M0}
         waits = 0
         k = n - 1
         while k >= 0 and waits < NEEDED:

@@ -32,6 +32,13 @@ def test_only_the_copys_own_operands_count():
     assert len(hazards.scan_asm(text)) == 1
 
 
+def test_a_vector_write_of_m0_counts_too():
+    text = HEAD + "\tv_readfirstlane_b32 m0, v7\n" + COPY % "s_nop 0"
+    assert len(hazards.scan_asm(text)) == 1
+    text = HEAD + "\tv_readfirstlane_b32 s9, v7\n\ts_mov_b32 m0, s9\n" + COPY % "s_nop 0"          # through a scalar move: fine
+    assert hazards.scan_asm(text) == []
+
+
 def test_scalar_writes_and_the_second_copy_of_a_group_are_fine():
     text = (HEAD + "\tv_readlane_b32 s27, v177, 33\n" + COPY % "s_nop 4" + "\ts_add_i32 m0, s4, 0x8400\n\ts_mov_b32 s24, s76\n" + COPY % "s_nop 0")
     assert hazards.scan_asm(text) == []
