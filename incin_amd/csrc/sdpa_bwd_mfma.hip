@@ -371,10 +371,15 @@ constexpr int BWD_RING = 4;        // matrix operands in flight from LDS (reads 
 // the first and after the last block that shows this workgroup any key are left out; inside that range a block of zeros or
 // of -inf needs no values.  Otherwise: a lane holds one key and 16 query rows of a block, so its mask values are 16 loads down a
 // column of the mask, asked for at the start of a step and added (times log2 e) to the scores where P is taken.
-template <typename T, int D, bool DENSE = false>
+// MASK: 0 none, 1 (DENSE) as described, 2 (STAGED) DENSE with the values through LDS where the mask's rows can be copied 16 bytes
+// at a time: every wavefront copies the 32 rows x 32 keys of its own block of the next tile (two copies, rows of 64 bytes) into
+// 2 KiB of its own and takes its column of them with four transposing reads - 8 bytes per lane, four rows of four keys,
+// handed round among 16 lanes so that each ends with four rows of its own key - instead of 16 two-byte loads.
+template <typename T, int D, int MASK = 0>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
 {
+    constexpr bool DENSE = MASK != 0, STAGED = MASK == 2;
 #if defined(__HIP_DEVICE_COMPILE__)
     typedef typename Mma<T>::vec8 vec8;
     typedef PfLayout<D> L;
@@ -387,7 +392,8 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
     constexpr int XCHG = 4 * 2 * 4 * 1024;              // [key block][query block][P lo, P hi, dS lo, dS hi]: 64 lanes x 16 bytes
     const SdpaParams& p = bp.f;
     constexpr int NS = 3;                               // stages: tiles t - 1 and t in use, tile t + 1 arriving
-    __shared__ __attribute__((aligned(1024))) char smem[NS * STAGE + XCHG];
+    constexpr int MZONE = STAGED ? 8 * 2048 : 0;        // STAGED: 32 rows x 64 bytes of mask values per wavefront
+    __shared__ __attribute__((aligned(1024))) char smem[NS * STAGE + XCHG + MZONE];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -563,6 +569,23 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
         tile_of(n, &i0, &head);
         return (int)mask_flags_of(p, b, hkv * p.G + head)[(int64_t)min((i0 >> 5) + role, nrb32 - 1) * nkb32 + my_kb32];
     };
+    // STAGED: copy c of a tile's two brings rows 16 c + lane / 4, 16-byte chunk lane % 4 of the 64 bytes this wavefront's 32 keys
+    // take in a row (the rows' 16 c into the scalar offset); the descriptor starts at the block's first row and first key and
+    // ends with the head's last row, so rows past Sq deliver zeros.  A lane's transposing read r4 takes 8 bytes of row
+    // 8 r4 + 4 g + (lane % 16) / 4, keys 16 (lane / 16 % 2) + 4 (lane % 4) .. + 3, and returns rows 8 r4 + 4 g .. + 3 of key lane % 32.
+    [[maybe_unused]] const unsigned m_zone = lds_address(smem) + NS * STAGE + XCHG + wave * 2048;
+    [[maybe_unused]] const int m_cp = (int)((int64_t)(lane >> 2) * p.m_si * 2) + (lane & 3) * 16;
+    [[maybe_unused]] const int m_tr = (4 * g + ((lane & 15) >> 2)) * 64 + ((lane >> 4) & 1) * 32 + (lane & 3) * 8;
+    [[maybe_unused]] auto tile_copy = [&](int n) __attribute__((always_inline)) {
+        int i0, head;
+        tile_of(n, &i0, &head);
+        const int row0 = i0 + 32 * role, key0 = j0 + kb * 32;
+        const T* mc = (const T*)p.mask + (int64_t)b * p.m_sb + (int64_t)(hkv * p.G + head) * p.m_sh + (int64_t)row0 * p.m_si + key0;
+        const int64_t left = row0 < Sq && key0 < Skv ? ((int64_t)(Sq - 1 - row0) * p.m_si + (Skv - key0)) * 2 : 0;
+        const uint4v md = dma_descriptor(mc, (int)min(left, (int64_t)0x7fffffff));
+#pragma unroll
+        for (int c = 0; c < 2; ++c) dma_copy16_at(md, m_zone + c * 1024, m_cp, c * 16 * (int)p.m_si * 2);
+    };
     [[maybe_unused]] auto tile_values = [&](int n) __attribute__((always_inline)) {      // register r is row i0 + 32 * role + 8 * (r / 4) + 4 * g + (r % 4)
         int i0, head;
         tile_of(n, &i0, &head);
@@ -691,7 +714,7 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
             f_cur = __builtin_amdgcn_readfirstlane(tile_flag(0));
             if (n_tiles > 1) fv_next2 = tile_flag(1);
         }
-        if (f_cur == 0) tile_values(0);
+        if (f_cur == 0) { if (STAGED) tile_copy(0); else tile_values(0); }
     }
     for (int t = 0; t < n_tiles; ++t) {
         // Tile t has landed for everyone, tile t - 1's P and dS are in the exchange buffer, and everyone is done with tile
@@ -702,16 +725,33 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
         if (DENSE) {      // (arrived: waits the compiler places for these are placed here, before the next copies are issued)
             asm volatile("" : "+v"(fv_next2));
             f_next = t + 1 < n_tiles && p.mask_flags ? __builtin_amdgcn_readfirstlane(fv_next2) : 0;
+            if (STAGED) {
+                if (f_cur == 0) {      // this tile's values out of the wavefront's buffer, which the next tile's copies may then take
 #pragma unroll
-            for (int i = 0; i < 16; ++i) asm volatile("" : "+v"(mnext[i]));
+                    for (int r4 = 0; r4 < 4; ++r4) {
+                        const short4v x = __builtin_amdgcn_ds_read_tr16_b64_v4i16((short4v __attribute__((address_space(3)))*)(smem + NS * STAGE + XCHG + wave * 2048 + m_tr + r4 * 512));
 #pragma unroll
-            for (int i = 0; i < 8; ++i) mval[i] = __builtin_bit_cast(vec2, mnext[2 * i] | (mnext[2 * i + 1] << 16));
+                        for (int e = 0; e < 4; ++e) mval[2 * r4 + e / 2][e % 2] = __builtin_bit_cast(T, (short)x[e]);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) asm volatile("" : "+v"(mnext[i]));
+#pragma unroll
+                for (int i = 0; i < 8; ++i) mval[i] = __builtin_bit_cast(vec2, mnext[2 * i] | (mnext[2 * i + 1] << 16));
+            }
         }
         const int nstage = stage == 2 ? 0 : stage + 1;
         if (t + 1 < n_tiles) issue(nstage);
         if (DENSE) {
             if (p.mask_flags && t + 2 < n_tiles) fv_next2 = tile_flag(t + 2);
-            if (t + 1 < n_tiles && f_next == 0) tile_values(t + 1);
+            if (t + 1 < n_tiles && f_next == 0) {
+                if (STAGED) {
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");      // (the reads above have delivered: the buffer is free)
+                    tile_copy(t + 1);
+                } else
+                    tile_values(t + 1);
+            }
         }
         // Every wavefront computes every tile: one whose keys no row of the tile sees (the first tile or two under a
         // causal mask) works on -inf, and would wait at the barriers for the others anyway.
@@ -764,7 +804,11 @@ static hipError_t launch_bwd_t(const SdpaBwdParams& bp, hipStream_t stream)
     }
     const int nkb = (p.Skv + BWD_KEYS - 1) / BWD_KEYS;
     if ((int64_t)nkb * p.Hkv * p.B > 0)
-        hipLaunchKernelGGL((sdpa_bwd_dkv_kernel<T, D, DENSE>), dim3((unsigned)((int64_t)nkb * p.Hkv * p.B)), dim3(512), 0, stream, bp);
+    {
+        const dim3 grid((unsigned)((int64_t)nkb * p.Hkv * p.B));
+        if (DENSE && p.mask_chunks) hipLaunchKernelGGL((sdpa_bwd_dkv_kernel<T, D, DENSE ? 2 : 0>), grid, dim3(512), 0, stream, bp);
+        else hipLaunchKernelGGL((sdpa_bwd_dkv_kernel<T, D, DENSE ? 1 : 0>), grid, dim3(512), 0, stream, bp);
+    }
     return hipGetLastError();
 }
 

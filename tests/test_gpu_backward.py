@@ -170,8 +170,8 @@ def test_generic_backward_f32_against_the_oracle(gpu, shape):
     (1, 2, 2, 200, 200, 96, 72, False, None, "causal_tensor"),     # the causal mask as a tensor (no flag), padded head dimensions
     (2, 2, 1, 70, 333, 128, 128, False, None, "batch"),            # [B, 1, Sq, Skv]; 333 keys: rows of the mask are not 8-byte aligned
     (1, 4, 2, 330, 400, 128, 128, False, None, "causal_bias"),     # per-head distance bias under the causal triangle: blocks of all kinds
-    (2, 2, 2, 300, 300, 64, 64, False, None, "window"),            # a band of 70 keys: hidden blocks on both sides, zeros between
-    (1, 2, 1, 257, 290, 128, 128, True, None, "blocks"),           # random 32 x 32 blocks hidden / zero / values, under the causal flag
+    (2, 2, 2, 300, 304, 64, 64, False, None, "window"),            # a band of 70 keys: hidden blocks on both sides, zeros between
+    (1, 2, 1, 257, 296, 128, 128, True, None, "blocks"),           # random 32 x 32 blocks hidden / zero / values, under the causal flag
 ], ids=["full", "gqa_head_causal", "row_lens", "causal_tensor", "batch_unaligned", "causal_bias", "window", "blocks"])
 def test_matrix_core_backward_with_a_dense_mask(gpu, dtype, shape):
     """Gradients with a dense additive mask run on the matrix-core kernels, 16-bit and f32 (instances that add the mask's values
@@ -187,7 +187,7 @@ def test_matrix_core_backward_with_a_dense_mask(gpu, dtype, shape):
         dist = (np.arange(Sq)[:, None] + (Skv - Sq) - np.arange(Skv)[None, :]).astype(np.float32)
         mask = np.where(dist >= 0, -dist[None] * (0.5 ** np.arange(1, Hq + 1, dtype=np.float32))[:, None, None], -np.inf)[None].astype(np.float32)
     elif mk == "window":
-        dist = np.arange(Sq)[:, None] - np.arange(Skv)[None, :]
+        dist = np.arange(Sq)[:, None] + (Skv - Sq) - np.arange(Skv)[None, :]
         mask = np.where((dist >= 0) & (dist < 70), 0.0, -np.inf).astype(np.float32).reshape(1, 1, Sq, Skv)
     elif mk == "blocks":
         kinds = r.integers(0, 3, size=(B, Hq, (Sq + 31) // 32, (Skv + 31) // 32))
@@ -230,6 +230,8 @@ def test_backward_random_cases_with_a_dense_mask(gpu):
         D = 128 if case % 2 else 64
         B, Hkv, G = int(r.integers(1, 3)), int(r.integers(1, 3)), int(r.choice([1, 2, 4]))
         Skv = int(r.choice([r.integers(1, 70), r.integers(60, 140), r.integers(120, 420)]))
+        if case % 4 < 2:
+            Skv = (Skv + 7) // 8 * 8          # (rows the 16-bit dK/dV kernel can copy into LDS)
         causal = bool(r.integers(0, 2))
         Sq = int(r.integers(1, Skv + 1)) if causal else int(r.integers(1, 300))
         lens = r.integers(1, Skv + 1, B).astype(np.int32) if r.integers(0, 2) else None
