@@ -127,16 +127,23 @@ struct BwdTiles {
 // ---- dQ ----------------------------------------------------------------------------------------------------------------
 // DENSE: a dense additive mask - its values (times log2 e) are added to the scores before the exponential, fetched while
 // the matrix instructions of the scores run; what the mask hides (-inf) ends as P = 0 like the causal edge.
-template <typename T, int D, bool DENSE = false>
+// MASK: 0 none, 1 (DENSE) as described, 2 (STAGED) DENSE with the values through LDS where the mask's rows can be copied 16 bytes
+// at a time: a wavefront owns 4 KiB behind the tiles - 32 rows x 32 keys for each half of a tile, rows of 64 bytes, their four
+// 16-byte chunks XOR-swizzled by row - reads a half's values from there (four 8-byte reads per lane) and, once they are
+// on the scores, copies the same half of the next tile into the place they left: the copy has most of a tile's time to
+// land and no load sits inside the tile.  (The buffers of two workgroups and their tiles fill a compute unit's LDS to the
+// byte: the two words of the tile-range search live in the buffers before the first copy.)
+template <typename T, int D, int MASK = 0>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
 {
+    constexpr bool DENSE = MASK != 0, STAGED = MASK == 2;
 #if defined(__HIP_DEVICE_COMPILE__)
     typedef typename Mma<T>::vec8 vec8;
     typedef PfLayout<D> L;
     constexpr int NSTEP = D / 16, NDB = D / 32;
     const SdpaParams& p = bp.f;
-    __shared__ __attribute__((aligned(1024))) char smem[4 * L::TILE_BYTES];      // K buffers 0, 1, V buffers 0, 1
+    __shared__ __attribute__((aligned(1024))) char smem[4 * L::TILE_BYTES + (STAGED ? 4 * 4096 : 0)];      // K buffers 0, 1, V buffers 0, 1 (, mask values)
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -182,7 +189,12 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
     [[maybe_unused]] const uint8_t* mflags = nullptr;
     [[maybe_unused]] const int nkb32 = (Skv + 31) >> 5;
     if (DENSE && p.mask_flags) {
-        __shared__ int s_seen[2];
+        int* s_seen;
+        if constexpr (STAGED) s_seen = (int*)(smem + 4 * L::TILE_BYTES);
+        else {
+            __shared__ int s_seen_words[2];
+            s_seen = s_seen_words;
+        }
         const int nrb32 = (Sq + 31) >> 5;
         const uint8_t* fl = mask_flags_of(p, b, hq);
         mflags = fl + (int64_t)min((q0 >> 5) + wave, nrb32 - 1) * nkb32;
@@ -247,18 +259,50 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
     int lim_wave_min = kv_len;
     if (p.causal) lim_wave_min = clampi(q0 + wave * 32 + coff + 1, 0, kv_len);
 
-    // DENSE: the two flags of a tile are asked for one tile ahead, after the copies of that tile are issued, and taken
-    // behind the tile barrier, before the next copies are issued: a load that is issued and consumed inside one tile makes
-    // the compiler wait for everything in flight - the next tile's copies, which it does not know of, included.  The values
-    // of a block that has any are such loads (there are no registers to hold them a tile ahead): a tile with values pays a
-    // memory latency that the second workgroup of the compute unit has to cover.
+    // DENSE: the flags of a tile are asked for ahead of it (two tiles ahead for STAGED, which decides a tile ahead what to copy),
+    // after the copies of a tile are issued, and taken behind the tile barrier, before the next copies are issued: a load that
+    // is issued and consumed inside one tile makes the compiler wait for everything in flight - the next tile's copies,
+    // which it does not know of, included.  Without STAGED the values of a block that has any are such loads (there are no
+    // registers to hold them a tile ahead): a tile with values pays a memory latency that the second workgroup of the
+    // compute unit has to cover.
     typedef T vec4 __attribute__((ext_vector_type(4)));
     [[maybe_unused]] int fv[2] = {0, 0};
+    [[maybe_unused]] int f_cur[2] = {0, 0}, f_nxt[2] = {0, 0};      // STAGED: the flags of tiles t and t + 1 (fv: of t + 2, as loaded)
     [[maybe_unused]] auto tile_flags = [&](int t) __attribute__((always_inline)) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) fv[kb] = 2 * t + kb < nkb32 ? (int)mflags[2 * t + kb] : 2;
     };
+    // STAGED: copy c of a half's two brings rows 16 c + lane / 4, and into position lane % 4 of the row's four chunks the chunk
+    // (lane % 4) ^ (row / 4 % 4) (= (lane / 16) % 4 for both copies); the rows' 16 c, the half and the tile go into the scalar
+    // offset.  The descriptor starts at the wavefront's first row and ends with the head's last row (rows past Sq deliver zeros).
+    [[maybe_unused]] const unsigned m_zone = lds_address(smem) + 4 * L::TILE_BYTES + wave * 4096;
+    [[maybe_unused]] const int m_cp = (int)((int64_t)(lane >> 2) * p.m_si * 2) + (((lane & 3) ^ ((lane >> 4) & 3)) << 4);
+    [[maybe_unused]] const int m_rd = ql * 64 + g * 8 + (((ql >> 2) & 3) << 4);      // this lane's read position in a half, before the XOR with the chunk
+    [[maybe_unused]] uint4v m_desc = {0u, 0u, 0u, 0u};
+    if (STAGED) {
+        const int row0 = q0 + wave * 32;
+        const int64_t left = row0 < Sq ? ((int64_t)(Sq - 1 - row0) * p.m_si + Skv) * 2 : 0;
+        m_desc = dma_descriptor((const T*)p.mask + (int64_t)b * p.m_sb + (int64_t)hq * p.m_sh + (int64_t)row0 * p.m_si,
+                                (int)(left > 0x7fffffffLL ? 0x7fffffffLL : left));
+    }
+    [[maybe_unused]] auto half_copy = [&](int t, int kb) __attribute__((always_inline)) {
+#pragma unroll
+        for (int c = 0; c < 2; ++c) dma_copy16_at(m_desc, m_zone + kb * 2048 + c * 1024, m_cp, (t * PF_BN + kb * 32) * 2 + c * 16 * (int)p.m_si * 2);
+    };
     if (DENSE && mflags && t_first < n_tiles) tile_flags(t_first);
+    if (STAGED && t_first < n_tiles) {
+        // (the prologue's barrier is behind: the words of the tile-range search in the first buffer are done with)
+        if (mflags) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) f_cur[kb] = __builtin_amdgcn_readfirstlane(fv[kb]);
+            if (t_first + 1 < n_tiles) tile_flags(t_first + 1);
+        }
+        if (t_first < n_act) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+                if (f_cur[kb] == 0) half_copy(t_first, kb);
+        }
+    }
     for (int t = t_first; t < n_tiles; ++t) {
         // K(t), V(t) have landed for everyone and everyone is done with tile t-1: the other pair of buffers is free
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -268,13 +312,22 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
                 asm volatile("" : "+v"(fv[kb]));
-                flags_t[kb] = __builtin_amdgcn_readfirstlane(fv[kb]);
+                if (STAGED) {
+                    flags_t[kb] = f_cur[kb];
+                    f_nxt[kb] = t + 1 < n_tiles ? __builtin_amdgcn_readfirstlane(fv[kb]) : 2;
+                } else
+                    flags_t[kb] = __builtin_amdgcn_readfirstlane(fv[kb]);
             }
         }
         if (t + 1 < n_tiles) {
             tl.issue(0, kp, p.k_ss, Skv, (t + 1) * PF_BN, lds0 + ((t + 1) & 1) * L::TILE_BYTES, wave);
             tl.issue(1, vp, p.v_ss, Skv, (t + 1) * PF_BN, lds0 + (2 + ((t + 1) & 1)) * L::TILE_BYTES, wave);
-            if (DENSE && mflags) tile_flags(t + 1);
+            if (DENSE && mflags && !STAGED) tile_flags(t + 1);
+        }
+        if (STAGED && mflags) {
+            if (t + 2 < n_tiles) tile_flags(t + 2);
+            f_cur[0] = f_nxt[0];
+            f_cur[1] = f_nxt[1];
         }
         if (t >= n_act) continue;
         const char* kt = smem + (t & 1) * L::TILE_BYTES;
@@ -306,7 +359,8 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
 #pragma unroll
                 for (int r4 = 0; r4 < 4; ++r4) {
                     const int j = j0 + 32 * kb + 8 * r4 + 4 * g;
-                    if (p.mask_vec && j + 3 < Skv) mv[r4] = *(const vec4*)(mrow + j);
+                    if (STAGED) mv[r4] = *(const vec4*)(smem + 4 * L::TILE_BYTES + wave * 4096 + kb * 2048 + (m_rd ^ (r4 << 4)));
+                    else if (p.mask_vec && j + 3 < Skv) mv[r4] = *(const vec4*)(mrow + j);
                     else {
 #pragma unroll
                         for (int e = 0; e < 4; ++e) mv[r4][e] = mrow[(int64_t)min(j + e, Skv - 1) * p.m_sj];
@@ -321,6 +375,13 @@ void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
             if (DENSE && flag == 0) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) s_acc[r] = __builtin_fmaf((float)mv[r / 4][r % 4], 1.4426950408889634f, s_acc[r]);
+            }
+            if (STAGED) {      // (this half's values are on the scores: its place is free for the same half of the next tile)
+                const int fn = mflags ? f_cur[kb] : 0;      // (f_cur holds the next tile's flags by now)
+                if (t + 1 < n_tiles && t + 1 < n_act && fn == 0) {
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    half_copy(t + 1, kb);
+                }
             }
             vec8 ds[2];
 #pragma unroll
@@ -800,7 +861,8 @@ static hipError_t launch_bwd_t(const SdpaBwdParams& bp, hipStream_t stream)
         SdpaBwdParams bq = bp;      // two workgroups per CU, an eighth of the CUs per XCD
         bq.f.interleave = work_interleave(p.causal != 0 || p.mask != nullptr, 2 * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
         bq.f.deal_groups = (total & 7) == 0 ? work_deal(bq.f.interleave, p.G, nqb, total >> 3) : 0;
-        hipLaunchKernelGGL((sdpa_bwd_dq_kernel<T, D, DENSE>), dim3((unsigned)total), dim3(256), 0, stream, bq);
+        if (DENSE && p.mask_chunks) hipLaunchKernelGGL((sdpa_bwd_dq_kernel<T, D, DENSE ? 2 : 0>), dim3((unsigned)total), dim3(256), 0, stream, bq);
+        else hipLaunchKernelGGL((sdpa_bwd_dq_kernel<T, D, DENSE ? 1 : 0>), dim3((unsigned)total), dim3(256), 0, stream, bq);
     }
     const int nkb = (p.Skv + BWD_KEYS - 1) / BWD_KEYS;
     if ((int64_t)nkb * p.Hkv * p.B > 0)
