@@ -133,11 +133,13 @@ struct BwdTiles {
 // on the scores, copies the same half of the next tile into the place they left: the copy has most of a tile's time to
 // land and no load sits inside the tile.  (The buffers of two workgroups and their tiles fill a compute unit's LDS to the
 // byte: the two words of the tile-range search live in the buffers before the first copy.)
+// Wavefronts per SIMD: two; three for D = 64 without a mask tensor, which fits 168 registers without a spill (48 KiB of LDS
+// per workgroup: three workgroups per compute unit) - the masked instances would spill 11 - 42 registers there.
 template <typename T, int D, int MASK = 0>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((D == 64 && MASK == 0) ? 3 : 2, (D == 64 && MASK == 0) ? 3 : 2)))
 void sdpa_bwd_dq_kernel(SdpaBwdParams bp)
 {
-    constexpr bool DENSE = MASK != 0, STAGED = MASK == 2;
+    [[maybe_unused]] constexpr bool DENSE = MASK != 0, STAGED = MASK == 2;
 #if defined(__HIP_DEVICE_COMPILE__)
     typedef typename Mma<T>::vec8 vec8;
     typedef PfLayout<D> L;
@@ -440,7 +442,7 @@ template <typename T, int D, int MASK = 0>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
 {
-    constexpr bool DENSE = MASK != 0, STAGED = MASK == 2;
+    [[maybe_unused]] constexpr bool DENSE = MASK != 0, STAGED = MASK == 2;
 #if defined(__HIP_DEVICE_COMPILE__)
     typedef typename Mma<T>::vec8 vec8;
     typedef PfLayout<D> L;
