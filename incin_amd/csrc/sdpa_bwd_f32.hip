@@ -24,6 +24,7 @@
 
 #include "sdpa_bwd.h"
 #include "sdpa_mfma_common.h"
+#include "side_stream.h"
 
 namespace incin_rocm {
 
@@ -620,20 +621,36 @@ static hipError_t launch_bwd_f32_t(const SdpaBwdParams& bp, hipStream_t stream)
 {
     const SdpaParams& p = bp.f;
     const int64_t rows = (int64_t)p.B * p.Hq * p.Sq;
+    const int nqb = (p.Sq + PF_BM - 1) / PF_BM;
+    const int64_t total = (int64_t)nqb * p.Hq * p.B;
+    if (total > 0x7fffffffLL) return hipErrorInvalidValue;
+    const int nkb = (p.Skv + BWD32_KEYS - 1) / BWD32_KEYS;
+    const bool with_dkv = (int64_t)nkb * p.Hkv * p.B > 0;
+    // the dQ kernel on a side stream where one is to be had (side_stream.h) - it and the dK/dV kernel read the same inputs and
+    // the row dots, and write different outputs - when the call is short of work: at most two rounds of dQ workgroups (one
+    // per compute unit at a time at D = 128, two at 64).  Measured, whole call, forked against one stream (causal): 8 heads x
+    // 1024 0.60 (D = 128) / 0.76 (64), 32 heads x 1024 0.82 / 0.97, 32 heads x 2048 0.87 / 0.71, 8 heads x 8192 1.03 / 0.73; with
+    // more work than that 0.95 - 1.06 (128 heads x 2048 0.95 / 1.02, 64 heads x 4096 without a mask 1.02 / 1.06): not forked.
+    SideStreamLease side(stream, rows > 0 && with_dkv && total <= 2 * (int64_t)(D == 128 ? 1 : 2) * device_cus());
+    bool forked = false;
     if (rows > 0) {
         hipLaunchKernelGGL(bwd_f32_delta_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, bp);
-        const int nqb = (p.Sq + PF_BM - 1) / PF_BM;
-        const int64_t total = (int64_t)nqb * p.Hq * p.B;
-        if (total > 0x7fffffffLL) return hipErrorInvalidValue;
+        forked = with_dkv && side.active() && side.fork() == hipSuccess;
+    }
+    if (with_dkv)
+        hipLaunchKernelGGL((bwd_f32_dkv_kernel<D, DENSE>), dim3((unsigned)((int64_t)nkb * p.Hkv * p.B)), dim3(256), 0, stream, bp);
+    if (rows > 0) {
         SdpaBwdParams bq = bp;
         bq.f.interleave = work_interleave(p.causal != 0 || p.mask != nullptr, (D == 128 ? 1 : 2) * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
         bq.f.deal_groups = (total & 7) == 0 ? work_deal(bq.f.interleave, p.G, nqb, total >> 3) : 0;
-        hipLaunchKernelGGL((bwd_f32_dq_kernel<D, DENSE>), dim3((unsigned)total), dim3(256), 0, stream, bq);
+        hipLaunchKernelGGL((bwd_f32_dq_kernel<D, DENSE>), dim3((unsigned)total), dim3(256), 0, forked ? side.stream() : stream, bq);
     }
-    const int nkb = (p.Skv + BWD32_KEYS - 1) / BWD32_KEYS;
-    if ((int64_t)nkb * p.Hkv * p.B > 0)
-        hipLaunchKernelGGL((bwd_f32_dkv_kernel<D, DENSE>), dim3((unsigned)((int64_t)nkb * p.Hkv * p.B)), dim3(256), 0, stream, bp);
-    return hipGetLastError();
+    const hipError_t launched = hipGetLastError();
+    if (forked) {
+        const hipError_t e = side.join();      // (also after a failed launch: whatever did reach the side stream is ordered before the caller's next work)
+        if (e != hipSuccess) return e;
+    }
+    return launched;
 }
 
 // Host has validated: f32, D and Dv <= 128 in whole 16-byte vectors (bp.f.Dp = the instance: 64 or 128), finite scale, unit last-axis strides, 16-byte aligned rows,

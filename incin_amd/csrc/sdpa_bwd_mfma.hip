@@ -20,6 +20,7 @@
 
 #include "sdpa_bwd.h"
 #include "sdpa_mfma_common.h"
+#include "side_stream.h"
 
 namespace incin_rocm {
 
@@ -851,29 +852,48 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
 #endif
 }
 
+// The dQ kernel goes to a side stream where one is to be had (side_stream.h) - it and the dK/dV kernel read the same inputs
+// and the row dots, and write different outputs - when the call is short of work: at most two rounds of dQ workgroups (two
+// per compute unit at a time), or D = 64.  Measured, whole call, forked against one stream (bf16, causal): 8 heads x 1024
+// 0.80 (D = 128) / 0.91 (64), 8 heads x 8192 0.875 / 0.98, 32 heads x 2048 0.98 / 0.89, 128 heads x 4096 1.00 - 1.03 / 0.96,
+// 32 heads x 8192 1.01 / 0.94: at D = 128 two launches that each fill the device only disturb each other's longest-first
+// order, at D = 64 the dQ kernel's workgroups still fill the dK/dV kernel's tail.  (The fork and join cost about 5 us: 32
+// heads x 1024, 256 workgroups in a call of 52 - 74 us, is 8 - 9 % slower forked.)
 template <typename T, int D, bool DENSE = false>
 static hipError_t launch_bwd_t(const SdpaBwdParams& bp, hipStream_t stream)
 {
     const SdpaParams& p = bp.f;
     const int64_t rows = (int64_t)p.B * p.Hq * p.Sq;
+    const int nkb = (p.Skv + BWD_KEYS - 1) / BWD_KEYS;
+    const bool with_dkv = (int64_t)nkb * p.Hkv * p.B > 0;
+    const int64_t dq_total = (int64_t)((p.Sq + PF_BM - 1) / PF_BM) * p.Hq * p.B;
+    SideStreamLease side(stream, rows > 0 && with_dkv && (D == 64 || dq_total <= 4 * (int64_t)device_cus()));
+    bool forked = false;
     if (rows > 0) {
         hipLaunchKernelGGL((sdpa_bwd_delta_kernel<T>), dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, stream, bp);
+        forked = with_dkv && side.active() && side.fork() == hipSuccess;
+    }
+    if (with_dkv) {
+        const dim3 grid((unsigned)((int64_t)nkb * p.Hkv * p.B));
+        if (DENSE && p.mask_chunks) hipLaunchKernelGGL((sdpa_bwd_dkv_kernel<T, D, DENSE ? 2 : 0>), grid, dim3(512), 0, stream, bp);
+        else hipLaunchKernelGGL((sdpa_bwd_dkv_kernel<T, D, DENSE ? 1 : 0>), grid, dim3(512), 0, stream, bp);
+    }
+    if (rows > 0) {
+        hipStream_t sq = forked ? side.stream() : stream;
         const int nqb = (p.Sq + PF_BM - 1) / PF_BM;
         const int64_t total = (int64_t)nqb * p.Hq * p.B;
         SdpaBwdParams bq = bp;      // two workgroups per CU, an eighth of the CUs per XCD
         bq.f.interleave = work_interleave(p.causal != 0 || p.mask != nullptr, 2 * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
         bq.f.deal_groups = (total & 7) == 0 ? work_deal(bq.f.interleave, p.G, nqb, total >> 3) : 0;
-        if (DENSE && p.mask_chunks) hipLaunchKernelGGL((sdpa_bwd_dq_kernel<T, D, DENSE ? 2 : 0>), dim3((unsigned)total), dim3(256), 0, stream, bq);
-        else hipLaunchKernelGGL((sdpa_bwd_dq_kernel<T, D, DENSE ? 1 : 0>), dim3((unsigned)total), dim3(256), 0, stream, bq);
+        if (DENSE && p.mask_chunks) hipLaunchKernelGGL((sdpa_bwd_dq_kernel<T, D, DENSE ? 2 : 0>), dim3((unsigned)total), dim3(256), 0, sq, bq);
+        else hipLaunchKernelGGL((sdpa_bwd_dq_kernel<T, D, DENSE ? 1 : 0>), dim3((unsigned)total), dim3(256), 0, sq, bq);
     }
-    const int nkb = (p.Skv + BWD_KEYS - 1) / BWD_KEYS;
-    if ((int64_t)nkb * p.Hkv * p.B > 0)
-    {
-        const dim3 grid((unsigned)((int64_t)nkb * p.Hkv * p.B));
-        if (DENSE && p.mask_chunks) hipLaunchKernelGGL((sdpa_bwd_dkv_kernel<T, D, DENSE ? 2 : 0>), grid, dim3(512), 0, stream, bp);
-        else hipLaunchKernelGGL((sdpa_bwd_dkv_kernel<T, D, DENSE ? 1 : 0>), grid, dim3(512), 0, stream, bp);
+    const hipError_t launched = hipGetLastError();
+    if (forked) {
+        const hipError_t e = side.join();      // (also after a failed launch: whatever did reach the side stream is ordered before the caller's next work)
+        if (e != hipSuccess) return e;
     }
-    return hipGetLastError();
+    return launched;
 }
 
 // Host has validated: dtype f16/bf16, D and Dv <= 128 in whole 16-byte vectors (bp.f.Dp = the instance: 64 or 128; smaller

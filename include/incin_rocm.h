@@ -254,12 +254,17 @@ int incin_rocm_sdpa_fwd_static(const incin_rocm_sdpa_desc_t* desc, void* stream)
  * O, lse and d_o rows are never read, their d_q rows are written as zero and they add nothing to d_k and d_v).
  * fwd.impl picks the kernels: AUTO = matrix-core kernels where they apply - D and Dv up to 128 in whole 16-byte vectors (zero-padded
  * into instances for 64 and 128); f16 / bf16 with a positive scale, f32 (IEEE single-precision matrix instructions) with any finite
- * scale; both without a dense mask and with 16-byte aligned rows - and generic f32-arithmetic kernels otherwise; GENERIC and MFMA pin one or
- * the other.  A query row with no visible key (NaN in the forward) gets a zero gradient and
+ * scale; both with 16-byte aligned rows, and a dense mask of non-negative strides of which 64 rows fit 32-bit byte offsets
+ * - and generic f32-arithmetic kernels otherwise; GENERIC and MFMA pin one or the other.  A query row with no visible key (NaN in the forward) gets a zero gradient and
  * contributes nothing to d_k and d_v, where the reference's tape would spread NaN over the whole head.
- * The workspace holds two floats per query row (2 x [B, Hq, Sq]) and, for a dense mask on the 16-bit matrix-core kernels, a byte
+ * The workspace holds two floats per query row (2 x [B, Hq, Sq]) and, for a dense mask on the matrix-core kernels, a byte
  * per 32 rows x 32 keys of the mask behind them (ask incin_rocm_sdpa_bwd_workspace for the size);
- * d_q, d_k, d_v are fully overwritten. */
+ * d_q, d_k, d_v are fully overwritten.
+ * Streams: everything the call launches is ordered behind the work already on `stream` and ahead of whatever `stream` gets
+ * next.  A call of the matrix-core kernels that is short of work may run its dQ kernel on a stream of the library's own
+ * beside the dK/dV kernel (forked from and joined to `stream` with events; the library's streams have the default priority,
+ * are created on demand, shared by all calls on a device and kept until the process ends).  Never while `stream` is being
+ * captured into a graph, and never with INCIN_ROCM_BWD_STREAMS=1 in the environment (read at every call). */
 typedef struct {
     incin_rocm_sdpa_desc_t fwd;
     const void* d_o;               /* [B, Hq, Sq, D], dtype of the operands */

@@ -202,3 +202,103 @@ def test_overlapping_launches_with_workspaces_of_their_own(gpu):
         assert np.array_equal(c.to.to_f32(), expect), "party %d" % i
     graph.destroy()
     gstream.destroy()
+
+
+class BackwardPair:
+    """Two dependent backward calls: the second takes the first's dQ as its dO, so it is right only if the first call's
+    kernels - whichever stream the library put them on - are ordered before it on the caller's stream."""
+
+    def __init__(self, seed, dtype, D, B=2, Hq=4, Hkv=2, S=300):
+        r = np.random.Generator(np.random.PCG64(seed))
+        mk = lambda *s: r.standard_normal(s, dtype=np.float32)
+        self.keep = []
+        tq, tk, tv, tg = (host.DeviceTensor.from_f32(x, dtype) for x in (mk(B, Hq, S, D), mk(B, Hkv, S, D), mk(B, Hkv, S, D), mk(B, Hq, S, D)))
+        to = host.DeviceTensor((B, Hq, S, D), dtype)
+        lse = capi.DeviceBuffer(B * Hq * S * 4)
+        fwd = host.make_desc(tq, tk, tv, to, causal=True, lse=lse)
+        nbytes, _, _ = capi.sdpa_workspace(fwd)
+        fws = capi.DeviceBuffer(max(nbytes, 256))
+        fwd.workspace, fwd.workspace_bytes = fws.ptr, fws.nbytes
+        capi.sdpa_fwd(fwd)
+        capi.sync()
+        self.keep += [tq, tk, tv, tg, to, lse, fws]
+        self.outs, self.descs = [], []
+        d_o = tg
+        for _ in range(2):
+            tdq = host.DeviceTensor((B, Hq, S, D), dtype)
+            tdk, tdv = host.DeviceTensor((B, Hkv, S, D), dtype), host.DeviceTensor((B, Hkv, S, D), dtype)
+            bd = capi.SdpaBwdDesc()
+            bd.fwd = fwd
+            for name, t in (("d_o", d_o), ("d_q", tdq), ("d_k", tdk), ("d_v", tdv)):
+                setattr(bd, name, t.ptr)
+                st = host._strides3(t.shape)
+                for i in range(3):
+                    getattr(bd, name + "_stride")[i] = st[i]
+            ws = capi.DeviceBuffer(capi.sdpa_bwd_workspace(bd))
+            bd.workspace, bd.workspace_bytes = ws.ptr, ws.nbytes
+            self.keep.append(ws)
+            self.descs.append(bd)
+            self.outs += [tdq, tdk, tdv]
+            d_o = tdq
+
+    def run(self, stream=None):
+        for bd in self.descs:
+            capi.sdpa_bwd(bd, stream)
+
+    def clear(self):
+        for t in self.outs:
+            capi.check(capi.load().incin_rocm_memset(0, t.ptr, 0x7f, t.buf.nbytes))
+        capi.sync()
+
+    def read(self):
+        return [t.to_f32() for t in self.outs]
+
+
+@pytest.mark.parametrize("dtype, D", [(capi.BF16, 128), (capi.BF16, 64), (capi.F32, 128), (capi.F32, 64)],
+                         ids=["bf16_d128", "bf16_d64", "f32_d128", "f32_d64"])
+def test_backward_with_its_dq_kernel_on_a_side_stream(gpu, dtype, D, monkeypatch):
+    """A backward call short of work puts its dQ kernel on a stream of the library's own beside the dK/dV kernel and joins
+    the caller's stream afterwards.  Against the same calls held to one stream (INCIN_ROCM_BWD_STREAMS=1): bit-identical
+    gradients of two dependent calls, back to back on a stream of the caller's, and from three host threads at once, each on
+    a stream of its own with problems of its own (the library's streams come out of a shared pool)."""
+    pairs = [BackwardPair(500 + i, dtype, D) for i in range(3)]
+    monkeypatch.setenv("INCIN_ROCM_BWD_STREAMS", "1")
+    expect = []
+    for p in pairs:
+        p.run()
+        capi.sync()
+        expect.append(p.read())
+        p.clear()
+    monkeypatch.delenv("INCIN_ROCM_BWD_STREAMS")
+    say("backward on two streams: dtype %d, D %d, one thread" % (dtype, D))
+    stream = capi.Stream()
+    for rep in range(5):
+        pairs[0].run(stream.ptr)
+        stream.sync()
+        for name, got, e in zip(("dq1", "dk1", "dv1", "dq2", "dk2", "dv2"), pairs[0].read(), expect[0]):
+            assert np.array_equal(got, e), "%s, repetition %d" % (name, rep)
+        pairs[0].clear()
+    stream.destroy()
+    errors = []
+
+    def worker(p):
+        try:
+            s = capi.Stream()
+            for _ in range(15):
+                p.run(s.ptr)
+            s.sync()
+            s.destroy()
+        except Exception as e:      # noqa: BLE001 - reported below
+            errors.append(e)
+
+    say("backward on two streams: dtype %d, D %d, three threads" % (dtype, D))
+    threads = [threading.Thread(target=worker, args=(p,)) for p in pairs]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    capi.sync()
+    for i, (p, exp) in enumerate(zip(pairs, expect)):
+        for name, got, e in zip(("dq1", "dk1", "dv1", "dq2", "dk2", "dv2"), p.read(), exp):
+            assert np.array_equal(got, e), "thread %d, %s" % (i, name)
