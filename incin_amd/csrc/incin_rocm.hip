@@ -9,6 +9,7 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 
@@ -977,6 +978,36 @@ static size_t bwd_flags_bytes(const incin_rocm_sdpa_desc_t* d, int kind)
     return (size_t)(nbh * ((d->Sq + 31) / 32) * ((d->Skv + 31) / 32) + 255) / 256 * 256;
 }
 
+// f32 matrix-core kernels: into how many workgroups the key tiles of a block of 128 rows (dQ kernel, which = 0) or the query
+// tiles of a block of 128 keys (dK/dV kernel, which = 1) are dealt.  A launch of half a round of workgroups or less leaves
+// most of the device idle - under a causal mask every SIMD has one wavefront and all wait for the one with the longest
+// walk - so its tiles go to 2 workgroups (up to half a round) or 4 (up to a quarter), each with at least four tiles of 64 to
+// walk; the sums of parts 1 .. meet in planes of the workspace and a pass adds them (sdpa_bwd.h).  Measured, whole call,
+// against one workgroup per block (causal, with the dQ kernel on its side stream either way): 8 heads x 1024 keys 0.36 (D =
+// 64, 4 parts) / 0.56 (128); 32 heads x 1024 0.86 (D = 64, 2 parts: config 2's shape) and 0.99 at D = 128 (a full round:
+// not split); 16 query heads on 4 KV heads x 2048 0.38 / 0.41; from a full round on 1.0 - 1.13: not split.
+static int bwd_f32_parts(const incin_rocm_sdpa_desc_t* d, int kind, int which)
+{
+    if (kind != 2) return 1;
+    const char* forced = getenv("INCIN_ROCM_BWD_PARTS");      // (1, 2 or 4 for both kernels: a test knob)
+    const int64_t blocks = which == 0 ? ((d->Sq + 127) / 128) * d->Hq * d->B : ((d->Skv + 127) / 128) * d->Hkv * d->B;
+    const int64_t slots = (int64_t)((d->D > 64 || d->Dv > 64) ? 1 : 2) * compute_units_of(d->device);
+    const int64_t walk = (which == 0 ? d->Skv : d->Sq * (d->Hq / d->Hkv)) / 64;
+    int parts = 1;
+    if (forced && (atoi(forced) == 1 || atoi(forced) == 2 || atoi(forced) == 4)) parts = atoi(forced);
+    else if (2 * blocks <= slots) parts = 4 * blocks <= slots ? 4 : 2;
+    while (parts > 1 && walk < 4 * parts) parts >>= 1;
+    return parts;
+}
+static size_t round256(size_t n) { return (n + 255) / 256 * 256; }
+static size_t bwd_planes_bytes(const incin_rocm_sdpa_desc_t* d, int parts_q, int parts_kv)
+{
+    const size_t q = round256((size_t)(d->B * d->Hq * d->Sq * d->D) * sizeof(float));
+    const size_t k = round256((size_t)(d->B * d->Hkv * d->Skv * d->D) * sizeof(float));
+    const size_t v = round256((size_t)(d->B * d->Hkv * d->Skv * d->Dv) * sizeof(float));
+    return (size_t)(parts_q - 1) * q + (size_t)(parts_kv - 1) * (k + v);
+}
+
 int incin_rocm_sdpa_bwd_workspace(const incin_rocm_sdpa_bwd_desc_t* bd, size_t* bytes)
 {
     if (!bytes) return fail(INCIN_ROCM_EINVAL, "scaled_dot_product_attention backward: null output");
@@ -986,7 +1017,8 @@ int incin_rocm_sdpa_bwd_workspace(const incin_rocm_sdpa_bwd_desc_t* bd, size_t* 
     if (int rc = check_bwd(bd, &empty, &kind)) return rc;
     if (!empty) {
         const size_t flags = bwd_flags_bytes(&bd->fwd, kind);
-        *bytes = flags ? bwd_rows_bytes(&bd->fwd) + flags : 2 * (size_t)(bd->fwd.B * bd->fwd.Hq * bd->fwd.Sq) * sizeof(float);
+        const size_t planes = bwd_planes_bytes(&bd->fwd, bwd_f32_parts(&bd->fwd, kind, 0), bwd_f32_parts(&bd->fwd, kind, 1));
+        *bytes = flags || planes ? bwd_rows_bytes(&bd->fwd) + flags + planes : 2 * (size_t)(bd->fwd.B * bd->fwd.Hq * bd->fwd.Sq) * sizeof(float);
     }
     return 0;
 }
@@ -1010,8 +1042,10 @@ int incin_rocm_sdpa_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, void* stream)
         return 0;
     }
     const size_t flag_bytes = bwd_flags_bytes(&bd->fwd, kind);
-    const size_t need = flag_bytes ? bwd_rows_bytes(&bd->fwd) + flag_bytes
-                                   : 2 * (size_t)(bd->fwd.B * bd->fwd.Hq * bd->fwd.Sq) * sizeof(float);      // two f32 per query row (+ the mask's block flags)
+    const int parts_q = bwd_f32_parts(&bd->fwd, kind, 0), parts_kv = bwd_f32_parts(&bd->fwd, kind, 1);
+    const size_t plane_bytes = bwd_planes_bytes(&bd->fwd, parts_q, parts_kv);
+    const size_t need = flag_bytes || plane_bytes ? bwd_rows_bytes(&bd->fwd) + flag_bytes + plane_bytes
+                                   : 2 * (size_t)(bd->fwd.B * bd->fwd.Hq * bd->fwd.Sq) * sizeof(float);      // two f32 per query row (+ the mask's block flags, + the planes of a split call)
     if (!bd->workspace || bd->workspace_bytes < need || !aligned16(bd->workspace))
         return fail(INCIN_ROCM_EWORKSPACE, "scaled_dot_product_attention backward: %zu workspace bytes needed (16-byte aligned), %zu given",
                     need, bd->workspace ? bd->workspace_bytes : (size_t)0);
@@ -1032,6 +1066,17 @@ int incin_rocm_sdpa_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, void* stream)
     bp.dv_sb = bd->d_v_stride[0]; bp.dv_sh = bd->d_v_stride[1]; bp.dv_ss = bd->d_v_stride[2];
     bp.f.mask_flags = nullptr;
     bp.f.mask_lims = nullptr;
+    bp.parts_q = parts_q;
+    bp.parts_kv = parts_kv;
+    if (plane_bytes) {
+        const incin_rocm_sdpa_desc_t* d = &bd->fwd;
+        char* at = (char*)bd->workspace + bwd_rows_bytes(d) + flag_bytes;
+        bp.part_dq = (float*)at;
+        at += (size_t)(parts_q - 1) * round256((size_t)(d->B * d->Hq * d->Sq * d->D) * sizeof(float));
+        bp.part_dk = (float*)at;
+        at += (size_t)(parts_kv - 1) * round256((size_t)(d->B * d->Hkv * d->Skv * d->D) * sizeof(float));
+        bp.part_dv = (float*)at;
+    }
     if (flag_bytes) {
         if (((bd->fwd.Sq + 31) / 32) > 65535 || (bd->fwd.mask_stride[0] ? bd->fwd.B : 1) * (bd->fwd.mask_stride[1] ? bd->fwd.Hq : 1) > 65535)
             return fail(INCIN_ROCM_ESHAPE, "scaled_dot_product_attention backward: mask too large for one launch of the matrix-core kernels");

@@ -183,6 +183,15 @@ void bwd_f32_dq_kernel(SdpaBwdParams bp)
         n_tiles = s_seen[1] < 0 ? 0 : min(n_tiles, __builtin_amdgcn_readfirstlane(s_seen[1]) / NB + 1);
     }
 
+    // this workgroup's share of the tiles (bp.parts_q workgroups per block of rows: blockIdx.y says which)
+    const int part = blockIdx.y;
+    if (gridDim.y > 1) {
+        const int span = max(n_tiles - t_first, 0), parts = gridDim.y;
+        const int lo = t_first + (int)((int64_t)span * part / parts), hi = t_first + (int)((int64_t)span * (part + 1) / parts);
+        t_first = lo;
+        n_tiles = hi;
+    }
+
     F32Addr<D> ad;
     ad.init(wave, lane, p.k_ss, p.v_ss, p.D, p.Dv);
     const unsigned lds0 = lds_address(smem);
@@ -335,6 +344,8 @@ void bwd_f32_dq_kernel(SdpaBwdParams bp)
     }
     if (my_i < Sq) {
         float* row = dqp + (int64_t)my_i * bp.dq_ss;
+        if (part > 0)      // (a plane of the workspace: contiguous rows of D floats)
+            row = bp.part_dq + ((((int64_t)(part - 1) * p.B + b) * p.Hq + hq) * Sq + my_i) * p.D;
 #pragma unroll
         for (int db = 0; db < NDB; ++db)
 #pragma unroll
@@ -430,7 +441,10 @@ void bwd_f32_dkv_kernel(SdpaBwdParams bp)
         }
     }
     const int tiles_per_head = j0 < kv_len ? max(n_qt - t_begin, 0) : 0;
-    const int n_tiles = tiles_per_head * p.G;           // the group's query heads one after another
+    const int n_all = tiles_per_head * p.G;             // the group's query heads one after another
+    // this workgroup's share of the walk (bp.parts_kv workgroups per key block: blockIdx.y says which)
+    const int part = blockIdx.y;
+    const int n_lo = (int)((int64_t)n_all * part / (int)gridDim.y), n_tiles = (int)((int64_t)n_all * (part + 1) / (int)gridDim.y);
 
     F32Addr<D> ad;
     ad.init(wave, lane, p.q_ss, bp.do_ss, p.D, p.Dv);
@@ -495,11 +509,11 @@ void bwd_f32_dkv_kernel(SdpaBwdParams bp)
             for (int r = 0; r < 16; ++r)
                 m_next[qb][r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, m_lane, (32 * qb + 8 * (r / 4) + (r % 4)) * m_row4, 0));
     };
-    if (n_tiles > 0) {
-        issue(0, 0);
-        if (DENSE) load_mask(0);
+    if (n_lo < n_tiles) {
+        issue(n_lo, n_lo & 1);
+        if (DENSE) load_mask(n_lo);
     }
-    for (int n = 0; n < n_tiles; ++n) {
+    for (int n = n_lo; n < n_tiles; ++n) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         if (DENSE) {      // (arrived: a wait the compiler places for them is placed here, before the next copies are issued)
@@ -598,6 +612,11 @@ void bwd_f32_dkv_kernel(SdpaBwdParams bp)
     if (my_j < Skv) {
         float* krow = dkp + (int64_t)my_j * bp.dk_ss;
         float* vrow = dvp + (int64_t)my_j * bp.dv_ss;
+        if (part > 0) {      // (planes of the workspace: contiguous rows of D and Dv floats)
+            const int64_t r = (((int64_t)(part - 1) * p.B + b) * p.Hkv + hkv) * Skv + my_j;
+            krow = bp.part_dk + r * p.D;
+            vrow = bp.part_dv + r * p.Dv;
+        }
         const bool live = my_j < kv_len;               // (a key past kv_len met no mask above: its sums are not gradients)
 #pragma unroll
         for (int db = 0; db < NDB; ++db)
@@ -614,6 +633,38 @@ void bwd_f32_dkv_kernel(SdpaBwdParams bp)
             }
     }
 #endif
+}
+
+// dst rows [B, H, S, D] by strides += planes 0 .. nplanes - 1 of src ([nplanes][B, H, S, D] contiguous), in that order; blockIdx.y
+// picks one of two such jobs (dK and dV share a launch).  A thread takes four floats.
+struct AddPlanesJob {
+    float* dst;
+    const float* src;
+    int64_t sb, sh, ss;
+    int B, H, S, D;
+};
+__global__ __launch_bounds__(256) void bwd_f32_add_planes_kernel(AddPlanesJob j0, AddPlanesJob j1, int nplanes)
+{
+    const AddPlanesJob& j = blockIdx.y == 0 ? j0 : j1;
+    const int d4 = j.D >> 2;
+    const int64_t n = (int64_t)j.B * j.H * j.S * d4;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    const int64_t row = idx / d4;
+    const int c = (int)(idx - row * d4) * 4;
+    const int s = (int)(row % j.S);
+    const int64_t bh = row / j.S;
+    const int h = (int)(bh % j.H);
+    const int64_t b = bh / j.H;
+    float* d = j.dst + b * j.sb + h * j.sh + (int64_t)s * j.ss + c;
+    float4v acc = *(const float4v*)d;
+    const int64_t plane = (int64_t)j.B * j.H * j.S * j.D;
+    for (int k = 0; k < nplanes; ++k) {
+        const float4v x = *(const float4v*)(j.src + k * plane + row * j.D + c);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] += x[e];
+    }
+    *(float4v*)d = acc;
 }
 
 template <int D, bool DENSE = false>
@@ -637,13 +688,29 @@ static hipError_t launch_bwd_f32_t(const SdpaBwdParams& bp, hipStream_t stream)
         hipLaunchKernelGGL(bwd_f32_delta_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, bp);
         forked = with_dkv && side.active() && side.fork() == hipSuccess;
     }
-    if (with_dkv)
-        hipLaunchKernelGGL((bwd_f32_dkv_kernel<D, DENSE>), dim3((unsigned)((int64_t)nkb * p.Hkv * p.B)), dim3(256), 0, stream, bp);
+    const unsigned parts_q = bp.parts_q > 1 ? (unsigned)bp.parts_q : 1u, parts_kv = bp.parts_kv > 1 ? (unsigned)bp.parts_kv : 1u;
+    if (with_dkv) {
+        const unsigned parts = parts_kv;
+        hipLaunchKernelGGL((bwd_f32_dkv_kernel<D, DENSE>), dim3((unsigned)((int64_t)nkb * p.Hkv * p.B), parts), dim3(256), 0, stream, bp);
+        if (parts > 1) {
+            const AddPlanesJob jk = {(float*)bp.d_k, bp.part_dk, bp.dk_sb, bp.dk_sh, bp.dk_ss, p.B, p.Hkv, p.Skv, p.D};
+            const AddPlanesJob jv = {(float*)bp.d_v, bp.part_dv, bp.dv_sb, bp.dv_sh, bp.dv_ss, p.B, p.Hkv, p.Skv, p.Dv};
+            const int64_t n4 = (int64_t)p.B * p.Hkv * p.Skv * (max(p.D, p.Dv) >> 2);
+            hipLaunchKernelGGL(bwd_f32_add_planes_kernel, dim3((unsigned)((n4 + 255) / 256), 2), dim3(256), 0, stream, jk, jv, (int)parts - 1);
+        }
+    }
     if (rows > 0) {
+        hipStream_t sq = forked ? side.stream() : stream;
+        const unsigned parts = parts_q;
         SdpaBwdParams bq = bp;
         bq.f.interleave = work_interleave(p.causal != 0 || p.mask != nullptr, (D == 128 ? 1 : 2) * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
         bq.f.deal_groups = (total & 7) == 0 ? work_deal(bq.f.interleave, p.G, nqb, total >> 3) : 0;
-        hipLaunchKernelGGL((bwd_f32_dq_kernel<D, DENSE>), dim3((unsigned)total), dim3(256), 0, forked ? side.stream() : stream, bq);
+        hipLaunchKernelGGL((bwd_f32_dq_kernel<D, DENSE>), dim3((unsigned)total, parts), dim3(256), 0, sq, bq);
+        if (parts > 1) {
+            const AddPlanesJob jq = {(float*)bp.d_q, bp.part_dq, bp.dq_sb, bp.dq_sh, bp.dq_ss, p.B, p.Hq, p.Sq, p.D};
+            const int64_t n4 = (int64_t)p.B * p.Hq * p.Sq * (p.D >> 2);
+            hipLaunchKernelGGL(bwd_f32_add_planes_kernel, dim3((unsigned)((n4 + 255) / 256), 1), dim3(256), 0, sq, jq, jq, (int)parts - 1);
+        }
     }
     const hipError_t launched = hipGetLastError();
     if (forked) {

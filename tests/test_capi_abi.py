@@ -275,6 +275,21 @@ def test_backward_validation_and_workspace_size():
     assert capi.sdpa_bwd_workspace(_bwd(dict(add_mask=0x20000, impl=capi.IMPL_GENERIC))) == 2 * 2 * 4 * 128 * 4
     assert capi.sdpa_bwd_workspace(_bwd(dict(add_mask=0x20000, dtype=capi.F32))) == 2 * 2 * 4 * 128 * 4 + 256
     assert capi.sdpa_bwd_workspace(_bwd(dict(Sq=0))) == 0            # nothing to compute
+    # ... plus, for an f32 call on the matrix-core kernels that does not fill the device, the planes that the parts of a
+    # block sum into: 2 x 4 heads x 1024 rows are 64 blocks of 128 for either kernel, a quarter of the 256 workgroups a device
+    # of 256 compute units (no device to ask here) holds at D = 128 - four parts, three planes per gradient
+    def long(**fwd_kw):
+        bd = _bwd(dict(Sq=1024, Skv=1024, **fwd_kw))
+        for st in (bd.fwd.q_stride, bd.fwd.k_stride, bd.fwd.v_stride, bd.fwd.o_stride, bd.d_o_stride, bd.d_q_stride, bd.d_k_stride, bd.d_v_stride):
+            st[0], st[1], st[2] = 4 * 1024 * 128, 1024 * 128, 128
+        return bd
+    rows, plane = 2 * 2 * 4 * 1024 * 4, 2 * 4 * 1024 * 128 * 4
+    assert capi.sdpa_bwd_workspace(long()) == rows                                          # (16-bit storage: no planes)
+    assert capi.sdpa_bwd_workspace(long(dtype=capi.F32)) == rows + 3 * 3 * plane
+    assert capi.sdpa_bwd_workspace(long(dtype=capi.F32, impl=capi.IMPL_GENERIC)) == rows
+    assert capi.sdpa_bwd_workspace(long(dtype=capi.F32, D=64, Dv=64)) == rows + 3 * 3 * plane // 2      # (512 workgroups at a time at D = 64)
+    assert capi.sdpa_bwd_workspace(long(dtype=capi.F32, B=8)) == 4 * rows                     # a full round of blocks: not dealt
+    assert capi.sdpa_bwd_workspace(long(dtype=capi.F32, B=4)) == 2 * rows + 3 * 2 * plane     # half a round: two parts
     for bd, code in [
         (_bwd(dict(lse=None)), capi.EINVAL),                          # the forward's normalisers are an input
         (_bwd(d_k=None), capi.EINVAL),
