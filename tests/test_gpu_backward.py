@@ -91,6 +91,35 @@ def test_backward_random_cases(gpu):
         compare("dv", dv, rv)
 
 
+def test_backward_random_cases_f32(gpu):
+    """The same draw in f32 over longer sequences: key and query counts up to 1600, where a call this small has the walks of
+    its blocks dealt to 2 or 4 workgroups and its dQ kernel on a second stream - by the library's own rule, nothing forced.
+    1e-5 of the largest gradient magnitude against the f64 oracle."""
+    r = np.random.Generator(np.random.PCG64(2027))
+    for case in range(18):
+        D = 128 if case % 3 else 64
+        B, Hkv, G = int(r.integers(1, 3)), int(r.integers(1, 4)), int(r.choice([1, 2, 4]))
+        Skv = int(r.choice([r.integers(1, 140), r.integers(120, 700), r.integers(500, 1600), r.integers(1000, 1600)]))
+        causal = bool(r.integers(0, 2))
+        Sq = int(r.integers(1, Skv + 1)) if causal else int(r.choice([r.integers(1, 300), r.integers(500, 1300)]))
+        lens = None
+        if r.integers(0, 2):
+            lens = r.integers(1, Skv + 1, B).astype(np.int32)
+        scale = float(r.choice([1.0 / np.sqrt(D), 0.05, 0.2]))
+        Hq = Hkv * G
+        say("backward random case %d (f32): B=%d Hq=%d Hkv=%d Sq=%d Skv=%d D=%d causal=%s lens=%s scale=%g"
+            % (case, B, Hq, Hkv, Sq, Skv, D, causal, None if lens is None else lens.tolist(), scale))
+        q, k, v, go = make(300 + case, B, Hq, Hkv, Sq, Skv, D, capi.F32)
+        out, dq, dk, dv = host.sdpa_backward(q, k, v, go, capi.F32, scale=scale, causal=causal, kv_lens=lens)
+        rq, rk, rv = BW.sdpa_backward(q.reshape(B, Hkv, G, Sq, D), k[:, :, None], v[:, :, None], go.reshape(B, Hkv, G, Sq, D),
+                                      scale=scale, causal=causal, kv_lens=None if lens is None else lens.reshape(B, 1, 1))
+        rq, rk, rv = rq.reshape(B, Hq, Sq, D), rk.reshape(B, Hkv, Skv, D), rv.reshape(B, Hkv, Skv, D)
+        assert not np.isnan(rq).any(), "case construction: a row without keys"
+        compare("dq", dq, rq, tol=1e-5)
+        compare("dk", dk, rk, tol=1e-5)
+        compare("dv", dv, rv, tol=1e-5)
+
+
 def test_rows_without_visible_keys_get_zero_gradients(gpu):
     # Sq > Skv under causal alignment: the first Sq - Skv rows see nothing (NaN in the forward).  They get a zero dq
     # and contribute nothing to dk, dv; the other rows are what the oracle gives for them alone.
