@@ -248,6 +248,46 @@ def test_matrix_core_backward_with_a_dense_mask(gpu, dtype, shape):
         compare(name + " generic vs matrix-core", gx, x, tol=1e-5 if f32 else 1e-2)
 
 
+@pytest.mark.parametrize("dtype", [capi.BF16, capi.F16, capi.F32], ids=lambda x: dtypes.NAMES[x])
+@pytest.mark.parametrize("shape", [
+    # B, Hq, Hkv, Sq, Skv, D, causal, mask kind
+    (1, 4, 2, 1100, 1400, 128, True, "blocks"),
+    (1, 2, 2, 1300, 1304, 64, False, "band"),
+    (2, 2, 1, 900, 1600, 128, False, "values"),
+    (1, 2, 2, 1027, 1501, 64, True, "blocks"),          # rows of the mask that cannot be copied 16 bytes at a time
+], ids=["blocks_gqa128", "band64", "values128", "blocks_unaligned64"])
+def test_matrix_core_backward_with_a_dense_mask_over_many_tiles(gpu, dtype, shape):
+    """Masks over 14 - 25 tiles of keys and of query rows, where the kernels' look-ahead (flags two tiles ahead, values or their
+    copies into LDS one ahead, tile ranges trimmed by the flags) runs at length: random blocks of 32 x 32 that are hidden, zero or
+    valued (runs of each), a band of values around the diagonal with -inf away from it, values with holes everywhere."""
+    B, Hq, Hkv, Sq, Skv, D, causal, mk = shape
+    G = Hq // Hkv
+    say("matrix-core backward with a mask over many tiles: %s %s" % (dtypes.NAMES[dtype], shape))
+    q, k, v, go = make(81 + Sq, B, Hq, Hkv, Sq, Skv, D, dtype)
+    r = np.random.Generator(np.random.PCG64(82))
+    if mk == "blocks":
+        kinds = r.integers(0, 3, size=(1, Hq, (Sq + 31) // 32, (Skv + 31) // 32))
+        kinds[..., 0] = 1                                        # every row keeps visible keys
+        big = np.repeat(np.repeat(kinds, 32, axis=2), 32, axis=3)[:, :, :Sq, :Skv]
+        mask = np.where(big == 0, -np.inf, np.where(big == 1, 0.0, r.standard_normal((1, Hq, Sq, Skv), dtype=np.float32))).astype(np.float32)
+    elif mk == "band":
+        dist = np.abs(np.arange(Sq)[:, None] - np.arange(Skv)[None, :])
+        mask = np.where(dist > 300, -np.inf, np.where(dist < 100, r.standard_normal((Sq, Skv)), 0.0)).astype(np.float32).reshape(1, 1, Sq, Skv)
+    else:
+        mask = r.standard_normal((B, 1, Sq, Skv), dtype=np.float32)
+        mask[r.random(mask.shape) < 0.25] = -np.inf
+        mask[..., 0] = 0.0
+    mask = dtypes.round_to(mask, dtype)
+    out, dq, dk, dv = host.sdpa_backward(q, k, v, go, dtype, causal=causal, mask=mask)
+    m5 = np.broadcast_to(mask, (B, Hq, Sq, Skv)).reshape(B, Hkv, G, Sq, Skv)
+    rq, rk, rv = BW.sdpa_backward(q.reshape(B, Hkv, G, Sq, D), k[:, :, None], v[:, :, None], go.reshape(B, Hkv, G, Sq, D), mask=m5, causal=causal)
+    assert not np.isnan(rq).any(), "case construction: a row without keys"
+    tol = 1e-5 if dtype == capi.F32 else 2e-2
+    compare("dq", dq, rq.reshape(B, Hq, Sq, D), tol=tol)
+    compare("dk", dk, rk.reshape(B, Hkv, Skv, D), tol=tol)
+    compare("dv", dv, rv.reshape(B, Hkv, Skv, D), tol=tol)
+
+
 def test_backward_random_cases_with_a_dense_mask(gpu):
     """Seeded random shapes with a mask tensor on the matrix-core backward kernels, all three dtypes: values with holes, blocks
     of 32 x 32 hidden / zero / valued at random, a band; any leading axis of the mask broadcast; lengths on either side of the
