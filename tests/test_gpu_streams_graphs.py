@@ -103,12 +103,16 @@ def test_graph_capture_and_replay(gpu, name, kw):
     graph.destroy()
 
 
-@pytest.mark.parametrize("dtype, impl", [(capi.BF16, capi.IMPL_AUTO), (capi.F32, capi.IMPL_AUTO)], ids=["bf16_matrix_core", "f32_generic"])
-def test_training_step_in_a_graph(gpu, dtype, impl):
+@pytest.mark.parametrize("dtype, impl, S", [(capi.BF16, capi.IMPL_AUTO, 300), (capi.F32, capi.IMPL_AUTO, 300), (capi.F32, capi.IMPL_AUTO, 1100),
+                                            (capi.F32, capi.IMPL_GENERIC, 300)],
+                         ids=["bf16_matrix_core", "f32_matrix_core", "f32_matrix_core_dealt_blocks", "f32_generic"])
+def test_training_step_in_a_graph(gpu, dtype, impl, S):
     """Forward (keeping the row normalisers) and backward recorded into one launch graph and replayed: every replay gives
     the bytes the eager calls gave, with the program's own eager work between replays.  The backward launches three kernels
-    and neither allocates nor clears memory."""
-    B, Hq, Hkv, S, D = 2, 4, 2, 300, 128
+    (five at 1100 tokens in f32, where the walks of a block are dealt to several workgroups and a pass adds their sums) on
+    the captured stream alone - eagerly a call this small puts one of them on a second stream - and neither allocates nor
+    clears memory."""
+    B, Hq, Hkv, D = 2, 4, 2, 128
     r = np.random.Generator(np.random.PCG64(300))
     mk = lambda *s: r.standard_normal(s, dtype=np.float32)
     tq, tk, tv, tg = (host.DeviceTensor.from_f32(x, dtype) for x in (mk(B, Hq, S, D), mk(B, Hkv, S, D), mk(B, Hkv, S, D), mk(B, Hq, S, D)))
@@ -117,6 +121,8 @@ def test_training_step_in_a_graph(gpu, dtype, impl):
     lse = capi.DeviceBuffer(B * Hq * S * 4)
     bd = capi.SdpaBwdDesc()
     bd.fwd = host.make_desc(tq, tk, tv, to, causal=True, impl=impl, lse=lse)
+    fws = capi.DeviceBuffer(max(capi.sdpa_workspace(bd.fwd)[0], 256))
+    bd.fwd.workspace, bd.fwd.workspace_bytes = fws.ptr, fws.nbytes
     for name, t in (("d_o", tg), ("d_q", tdq), ("d_k", tdk), ("d_v", tdv)):
         setattr(bd, name, t.ptr)
         st = host._strides3(t.shape)
