@@ -57,9 +57,12 @@ TRAFFIC_KIB = {   # leg/shape/variant: (FETCH_SIZE, WRITE_SIZE)
     "prefill_chunk/bf16_sq512_kv32768/auto": (67708 + 17448.5, 33677.2 + 4096), "prefill_chunk/bf16_sq512_kv32768/unsplit": (67735.5, 4096),
     "prefill_chunk/f32_sq128_kv32768/auto": (132204 + 16680, 33316.9 + 2048), "prefill_chunk/f32_sq128_kv32768/unsplit": (132192, 2048),
     "f32/f32_c1": (187.2, 32), "f32/f32_c2": (12378.4, 8192), "f32/f32_large": (1523050, 262144),
-    "backward/bf16_d128": (133146 + 368971 + 264723, 4096 + 131072 + 262358),          # (row dots + dQ + dK/dV kernels)
-    "backward/bf16_d64": (135194 + 302550 + 266323, 8192 + 131072 + 262144),
-    "backward/f32_d64": (8735 + 16600 + 16607.5, 512 + 8192 + 16423.3), "backward/f32_d128": (270367 + 885089 + 932720, 8192 + 262144 + 524288),
+    "backward/bf16_d128": (133150 + 367216 + 264788, 4096 + 131072 + 262324),          # (row dots + dQ + dK/dV kernels)
+    "backward/bf16_d64": (135199 + 309173 + 266324, 8192 + 131072 + 262152),
+    # (config 2's shape in f32: blocks dealt to two workgroups - the kernels write a plane each beside the gradients, and the two
+    #  passes that add the planes follow)
+    "backward/f32_d64": (8735 + 16613 + 16883 + 8219 + 16411, 512 + 16384 + 32778.2 + 8192 + 16384),
+    "backward/f32_d128": (270367 + 875814 + 924203, 8192 + 262144 + 524288),
 }
 TRAFFIC_PROFILE = "profiles/fetch_write_size_bench_legs.txt"
 
