@@ -185,3 +185,66 @@ def test_config3_backward_full(gpu):
         lse_row = BW.logsumexp(q[b, h], k[b, h], causal=True)[-1]
         p_last = np.exp(x_last[b, h] - lse_row)
         assert np.abs(dv[b, h, -1] - p_last * go[b, h, -1]).max() <= 2e-2 * max(1.0, float(np.abs(p_last * go[b, h, -1]).max()))
+
+
+def test_one_long_sequence_forward_and_backward(gpu):
+    """131072 tokens, two query heads on one KV head, bf16, causal: byte offsets inside a head reach 2^25, a head's scores
+    2^34 pairs, a workgroup walks up to 2048 tiles.  In float64 on the host, from what a row or a key needs alone: output and dQ
+    of sampled rows; dK and dV of sampled keys among the last 2048 (their rows' normalisers cost a 2048 x 131072 product).  For
+    all of it, identities that need no oracle: the column sums of dV are those of dO (every probability row sums to one), and
+    sum_j <dK_j, k_j> = sum_i <dQ_i, q_i> (both are scale * sum_ij dS_ij <q_i, k_j>)."""
+    B, Hq, Hkv, S, D = 1, 2, 1, 131072, 128
+    dt = capi.BF16
+    say("one long sequence: bf16 causal S=131072, 2 query heads on 1 KV head, D=128")
+    q, go = gen(70, (B, Hq, S, D), dt), gen(73, (B, Hq, S, D), dt)
+    k, v = gen(71, (B, Hkv, S, D), dt), gen(72, (B, Hkv, S, D), dt)
+    out, dq, dk, dv = host.sdpa_backward(q, k, v, go, dt, causal=True)
+    scale = 1.0 / np.sqrt(D)
+    k64, v64 = k[0, 0].astype(np.float64), v[0, 0].astype(np.float64)
+    q64, go64 = q[0].astype(np.float64), go[0].astype(np.float64)
+    worst = {"o": 0.0, "dq": 0.0, "dk": 0.0, "dv": 0.0}          # (gradients: largest error over the sampled rows or keys ...
+    largest = {"dq": 0.0, "dk": 0.0, "dv": 0.0}                # ... against the largest reference magnitude among them)
+    for h in range(Hq):
+        for i in [0, 1, 63, 64, 255, 256, 4097, 65535, 65536, 100003, S - 2, S - 1]:
+            s = (k64[:i + 1] @ q64[h, i]) * scale
+            p = np.exp(s - s.max())
+            p /= p.sum()
+            o_ref = p @ v64[:i + 1]
+            worst["o"] = max(worst["o"], float(np.abs(out[0, h, i] - o_ref).max()))
+            ds = p * (v64[:i + 1] @ go64[h, i] - float(o_ref @ go64[h, i]))
+            dq_ref = (ds @ k64[:i + 1]) * scale
+            worst["dq"], largest["dq"] = max(worst["dq"], float(np.abs(dq[0, h, i] - dq_ref).max())), max(largest["dq"], float(np.abs(dq_ref).max()))
+    T = 2048                                   # the last T rows: normalisers and D_i = <dO_i, O_i> in float64
+    lse, delta = np.empty((Hq, T)), np.empty((Hq, T))
+    for h in range(Hq):
+        s = (q64[h, S - T:] @ k64.T) * scale
+        s[np.arange(S - T, S)[:, None] < np.arange(S)[None, :]] = -np.inf
+        m = s.max(axis=1)
+        e = np.exp(s - m[:, None])
+        lse[h] = m + np.log(e.sum(axis=1))
+        delta[h] = np.einsum("id,id->i", (e / e.sum(axis=1)[:, None]) @ v64, go64[h, S - T:])
+    for j in [S - T, S - 1500, S - 129, S - 128, S - 33, S - 1]:
+        dk_ref, dv_ref = np.zeros(D), np.zeros(D)
+        for h in range(Hq):
+            r = j - (S - T)
+            p = np.exp((q64[h, j:] @ k64[j]) * scale - lse[h, r:])
+            dv_ref += p @ go64[h, j:]
+            dk_ref += ((p * (go64[h, j:] @ v64[j] - delta[h, r:])) @ q64[h, j:]) * scale
+        worst["dk"], largest["dk"] = max(worst["dk"], float(np.abs(dk[0, 0, j] - dk_ref).max())), max(largest["dk"], float(np.abs(dk_ref).max()))
+        worst["dv"], largest["dv"] = max(worst["dv"], float(np.abs(dv[0, 0, j] - dv_ref).max())), max(largest["dv"], float(np.abs(dv_ref).max()))
+    for name in largest:
+        worst[name] /= largest[name]
+    say("one long sequence: worst output error %.3e; gradients relative to the largest among the sampled rows or keys: dq %.3e dk %.3e dv %.3e"
+        % (worst["o"], worst["dq"], worst["dk"], worst["dv"]))
+    assert worst["o"] <= TOL[dt]
+    assert max(worst["dq"], worst["dk"], worst["dv"]) <= 2e-2
+    # the identities, with room for the roundings of 131072 bf16 rows adding up like a random walk
+    dv64, dk64, dq64 = dv[0, 0].astype(np.float64), dk[0, 0].astype(np.float64), dq[0].astype(np.float64)
+    sums, want = dv64.sum(axis=0), go64.sum(axis=(0, 1))
+    say("one long sequence: column sums of dV against those of dO: worst %.3e" % np.abs(sums - want).max())
+    # (a row's probabilities are rounded to bf16 before the product with dO: they sum to one within 2^-9, and the rows' errors,
+    #  each times a dO of order one, add up like a random walk)
+    assert np.abs(sums - want).max() <= 2.0 ** -9 * np.sqrt(Hq * S) * np.abs(go64).max()
+    tk, tq = np.einsum("jd,jd->j", dk64, k64), np.einsum("hid,hid->hi", dq64, q64)
+    say("one long sequence: sum <dK, k> = %.6e, sum <dQ, q> = %.6e" % (tk.sum(), tq.sum()))
+    assert abs(tk.sum() - tq.sum()) <= 2.0 ** -8 * 4 * (np.sqrt((tk ** 2).sum()) + np.sqrt((tq ** 2).sum()))
