@@ -187,15 +187,16 @@ def test_config3_backward_full(gpu):
         assert np.abs(dv[b, h, -1] - p_last * go[b, h, -1]).max() <= 2e-2 * max(1.0, float(np.abs(p_last * go[b, h, -1]).max()))
 
 
-def test_one_long_sequence_forward_and_backward(gpu):
-    """131072 tokens, two query heads on one KV head, bf16, causal: byte offsets inside a head reach 2^25, a head's scores
+@pytest.mark.parametrize("dt", [capi.BF16, capi.F32], ids=["bf16", "f32"])
+def test_one_long_sequence_forward_and_backward(gpu, dt):
+    """131072 tokens, two query heads on one KV head, bf16 and f32, causal: byte offsets inside a head reach 2^25 (f32: 2^26), a head's scores
     2^34 pairs, a workgroup walks up to 2048 tiles.  In float64 on the host, from what a row or a key needs alone: output and dQ
     of sampled rows; dK and dV of sampled keys among the last 2048 (their rows' normalisers cost a 2048 x 131072 product).  For
     all of it, identities that need no oracle: the column sums of dV are those of dO (every probability row sums to one), and
     sum_j <dK_j, k_j> = sum_i <dQ_i, q_i> (both are scale * sum_ij dS_ij <q_i, k_j>)."""
     B, Hq, Hkv, S, D = 1, 2, 1, 131072, 128
-    dt = capi.BF16
-    say("one long sequence: bf16 causal S=131072, 2 query heads on 1 KV head, D=128")
+    eps = 2.0 ** -9 if dt == capi.BF16 else 2.0 ** -18          # (f32: roundings of sums of up to 131072 terms)
+    say("one long sequence: %s causal S=131072, 2 query heads on 1 KV head, D=128" % dtypes.NAMES[dt])
     q, go = gen(70, (B, Hq, S, D), dt), gen(73, (B, Hq, S, D), dt)
     k, v = gen(71, (B, Hkv, S, D), dt), gen(72, (B, Hkv, S, D), dt)
     out, dq, dk, dv = host.sdpa_backward(q, k, v, go, dt, causal=True)
@@ -237,14 +238,14 @@ def test_one_long_sequence_forward_and_backward(gpu):
     say("one long sequence: worst output error %.3e; gradients relative to the largest among the sampled rows or keys: dq %.3e dk %.3e dv %.3e"
         % (worst["o"], worst["dq"], worst["dk"], worst["dv"]))
     assert worst["o"] <= TOL[dt]
-    assert max(worst["dq"], worst["dk"], worst["dv"]) <= 2e-2
+    assert max(worst["dq"], worst["dk"], worst["dv"]) <= TOL[dt]
     # the identities, with room for the roundings of 131072 bf16 rows adding up like a random walk
     dv64, dk64, dq64 = dv[0, 0].astype(np.float64), dk[0, 0].astype(np.float64), dq[0].astype(np.float64)
     sums, want = dv64.sum(axis=0), go64.sum(axis=(0, 1))
     say("one long sequence: column sums of dV against those of dO: worst %.3e" % np.abs(sums - want).max())
-    # (a row's probabilities are rounded to bf16 before the product with dO: they sum to one within 2^-9, and the rows' errors,
+    # (bf16: a row's probabilities are rounded before the product with dO: they sum to one within 2^-9, and the rows' errors,
     #  each times a dO of order one, add up like a random walk)
-    assert np.abs(sums - want).max() <= 2.0 ** -9 * np.sqrt(Hq * S) * np.abs(go64).max()
+    assert np.abs(sums - want).max() <= eps * np.sqrt(Hq * S) * np.abs(go64).max()
     tk, tq = np.einsum("jd,jd->j", dk64, k64), np.einsum("hid,hid->hi", dq64, q64)
     say("one long sequence: sum <dK, k> = %.6e, sum <dQ, q> = %.6e" % (tk.sum(), tq.sum()))
-    assert abs(tk.sum() - tq.sum()) <= 2.0 ** -8 * 4 * (np.sqrt((tk ** 2).sum()) + np.sqrt((tq ** 2).sum()))
+    assert abs(tk.sum() - tq.sum()) <= 8 * eps * (np.sqrt((tk ** 2).sum()) + np.sqrt((tq ** 2).sum()))
