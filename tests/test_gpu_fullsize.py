@@ -249,3 +249,24 @@ def test_one_long_sequence_forward_and_backward(gpu, dt):
     tk, tq = np.einsum("jd,jd->j", dk64, k64), np.einsum("hid,hid->hi", dq64, q64)
     say("one long sequence: sum <dK, k> = %.6e, sum <dQ, q> = %.6e" % (tk.sum(), tq.sum()))
     assert abs(tk.sum() - tq.sum()) <= 8 * eps * (np.sqrt((tk ** 2).sum()) + np.sqrt((tq ** 2).sum()))
+
+
+@pytest.mark.parametrize("dt", [capi.BF16, capi.F32], ids=["bf16", "f32"])
+@pytest.mark.parametrize("shape", [(4096, 8, 49, 32, False), (60000, 1, 40, 64, True)], ids=["windows_49x32", "batch_60000"])
+def test_very_many_small_heads(gpu, dt, shape):
+    """Tens of thousands of small heads (window attention: 4096 windows x 8 heads of 49 tokens, head dimension 32; a batch of
+    60000, just under the limit of a launch): work lists of 32768 - 60000 items on every kernel, forward and backward, with
+    sampled heads - first, last, middle, random - against the oracles."""
+    from oracle import sdpa_backward as BW
+    B, H, S, D, causal = shape
+    say("very many small heads: %s B=%d H=%d S=%d D=%d causal=%s" % (dtypes.NAMES[dt], B, H, S, D, causal))
+    r = np.random.Generator(np.random.PCG64(75))
+    q, k, v, go = (dtypes.round_to(r.standard_normal((B, H, S, D), dtype=np.float32), dt) for _ in range(4))
+    out, dq, dk, dv = host.sdpa_backward(q, k, v, go, dt, causal=causal)
+    for b, h in ((0, 0), (B - 1, H - 1), (B // 2, H // 2), (int(r.integers(0, B)), int(r.integers(0, H))), (B - 9, 0), (7, H - 1)):
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        ref = O.sdpa(q[sl], k[sl], v[sl], causal=causal)
+        assert float(np.abs(out[sl] - ref).max()) <= TOL[dt], "output of head (%d, %d)" % (b, h)
+        for name, g, r_ in zip(("dq", "dk", "dv"), (dq, dk, dv), BW.sdpa_backward(q[sl], k[sl], v[sl], go[sl], causal=causal)):
+            err = float(np.abs(g[sl] - r_).max() / np.abs(r_).max())
+            assert err <= TOL[dt], "%s of head (%d, %d): %.3e" % (name, b, h, err)
