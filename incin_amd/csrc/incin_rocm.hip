@@ -978,34 +978,50 @@ static size_t bwd_flags_bytes(const incin_rocm_sdpa_desc_t* d, int kind)
     return (size_t)(nbh * ((d->Sq + 31) / 32) * ((d->Skv + 31) / 32) + 255) / 256 * 256;
 }
 
-// f32 matrix-core kernels: into how many workgroups the key tiles of a block of 128 rows (dQ kernel, which = 0) or the query
+// Matrix-core kernels: into how many workgroups the key tiles of a block of 128 rows (dQ kernel, which = 0) or the query
 // tiles of a block of 128 keys (dK/dV kernel, which = 1) are dealt.  A launch of half a round of workgroups or less leaves
 // most of the device idle - under a causal mask every SIMD has one wavefront and all wait for the one with the longest
 // walk - so its tiles go to 2 workgroups (up to half a round) or 4 (up to a quarter), each with at least four tiles of 64 to
-// walk; the sums of parts 1 .. meet in planes of the workspace and a pass adds them (sdpa_bwd.h).  Measured, whole call,
-// against one workgroup per block (causal, with the dQ kernel on its side stream either way): 8 heads x 1024 keys 0.36 (D =
-// 64, 4 parts) / 0.56 (128); 32 heads x 1024 0.86 (D = 64, 2 parts: config 2's shape) and 0.99 at D = 128 (a full round:
-// not split); 16 query heads on 4 KV heads x 2048 0.38 / 0.41; from a full round on 1.0 - 1.13: not split.
-static int bwd_f32_parts(const incin_rocm_sdpa_desc_t* d, int kind, int which)
+// walk; the sums meet in planes of the workspace and a pass adds them (sdpa_bwd.h).
+// f32 (kind 2), both kernels.  Measured, whole call, against one workgroup per block (causal, with the dQ kernel on its side
+// stream either way): 8 heads x 1024 keys 0.36 (D = 64, 4 parts) / 0.56 (128); 32 heads x 1024 0.86 (D = 64, 2 parts: config
+// 2's shape) and 0.99 at D = 128 (a full round: not split); 16 query heads on 4 KV heads x 2048 0.38 / 0.41; from a full round
+// on 1.0 - 1.13: not split.
+// 16-bit storage (kind 1), the dK/dV kernel only - a workgroup of it fills a compute unit, a round is one per compute unit,
+// and with grouped queries a key block walks every head of its group: few KV heads on a device (a model's KV heads
+// divided over devices) leave most compute units without a block.  Measured, whole call, bf16 causal D = 128: 8 query heads on
+// 1 KV head x 8192 keys 1.66 -> 0.73 ms (4 parts; 2: 0.54 of the time, 8: 0.46), x 4096 0.84 -> 0.25 (8 parts: 0.28); 16 on 2
+// x 8192 0.72 (2 parts; 4: 0.85); 32 on 4 x 4096 0.80 (2); D = 64 8 on 1 x 8192 0.40; not worth it for short walks (8 heads x
+// 2048 keys without groups, 32 tiles per block: 1.19 in 2 parts) - a part keeps at least 64 tiles.  The kernel takes up to 8
+// parts, the rule stops at 4.
+static int bwd_parts(const incin_rocm_sdpa_desc_t* d, int kind, int which)
 {
-    if (kind != 2) return 1;
-    const char* forced = getenv("INCIN_ROCM_BWD_PARTS");      // (1, 2 or 4 for both kernels: a test knob)
+    if (kind == 0 || (kind == 1 && which == 0)) return 1;
+    const char* forced = getenv("INCIN_ROCM_BWD_PARTS");      // (1, 2, 4 or 8 for every kernel that takes parts: a test knob)
     const int64_t blocks = which == 0 ? ((d->Sq + 127) / 128) * d->Hq * d->B : ((d->Skv + 127) / 128) * d->Hkv * d->B;
-    const int64_t slots = (int64_t)((d->D > 64 || d->Dv > 64) ? 1 : 2) * compute_units_of(d->device);
+    const int64_t slots = (int64_t)(kind == 1 || d->D > 64 || d->Dv > 64 ? 1 : 2) * compute_units_of(d->device);
     const int64_t walk = (which == 0 ? d->Skv : d->Sq * (d->Hq / d->Hkv)) / 64;
     int parts = 1;
-    if (forced && (atoi(forced) == 1 || atoi(forced) == 2 || atoi(forced) == 4)) parts = atoi(forced);
-    else if (2 * blocks <= slots) parts = 4 * blocks <= slots ? 4 : 2;
-    while (parts > 1 && walk < 4 * parts) parts >>= 1;
+    const int f = forced ? atoi(forced) : 0;
+    if (f == 1 || f == 2 || f == 4 || f == 8) {
+        parts = std::min(f, kind == 1 ? 8 : 4);
+        while (parts > 1 && walk < 4 * parts) parts >>= 1;
+        return parts;
+    }
+    while (parts < 4 && 2 * parts * blocks <= slots) parts *= 2;
+    // (f32: four tiles per part are enough to pay for the planes; 16-bit storage, whose tiles take an eighth of the time: 64)
+    while (parts > 1 && walk < (kind == 1 ? 64 : 4) * parts) parts >>= 1;
     return parts;
 }
 static size_t round256(size_t n) { return (n + 255) / 256 * 256; }
-static size_t bwd_planes_bytes(const incin_rocm_sdpa_desc_t* d, int parts_q, int parts_kv)
+static size_t bwd_planes_bytes(const incin_rocm_sdpa_desc_t* d, int kind, int parts_q, int parts_kv)
 {
     const size_t q = round256((size_t)(d->B * d->Hq * d->Sq * d->D) * sizeof(float));
     const size_t k = round256((size_t)(d->B * d->Hkv * d->Skv * d->D) * sizeof(float));
     const size_t v = round256((size_t)(d->B * d->Hkv * d->Skv * d->Dv) * sizeof(float));
-    return (size_t)(parts_q - 1) * q + (size_t)(parts_kv - 1) * (k + v);
+    // (f32: part 0 writes the gradient itself; 16-bit storage: every part of a divided walk writes a plane)
+    const int planes_kv = kind == 1 ? (parts_kv > 1 ? parts_kv : 0) : parts_kv - 1;
+    return (size_t)(parts_q - 1) * q + (size_t)planes_kv * (k + v);
 }
 
 int incin_rocm_sdpa_bwd_workspace(const incin_rocm_sdpa_bwd_desc_t* bd, size_t* bytes)
@@ -1017,7 +1033,7 @@ int incin_rocm_sdpa_bwd_workspace(const incin_rocm_sdpa_bwd_desc_t* bd, size_t* 
     if (int rc = check_bwd(bd, &empty, &kind)) return rc;
     if (!empty) {
         const size_t flags = bwd_flags_bytes(&bd->fwd, kind);
-        const size_t planes = bwd_planes_bytes(&bd->fwd, bwd_f32_parts(&bd->fwd, kind, 0), bwd_f32_parts(&bd->fwd, kind, 1));
+        const size_t planes = bwd_planes_bytes(&bd->fwd, kind, bwd_parts(&bd->fwd, kind, 0), bwd_parts(&bd->fwd, kind, 1));
         *bytes = flags || planes ? bwd_rows_bytes(&bd->fwd) + flags + planes : 2 * (size_t)(bd->fwd.B * bd->fwd.Hq * bd->fwd.Sq) * sizeof(float);
     }
     return 0;
@@ -1042,8 +1058,8 @@ int incin_rocm_sdpa_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, void* stream)
         return 0;
     }
     const size_t flag_bytes = bwd_flags_bytes(&bd->fwd, kind);
-    const int parts_q = bwd_f32_parts(&bd->fwd, kind, 0), parts_kv = bwd_f32_parts(&bd->fwd, kind, 1);
-    const size_t plane_bytes = bwd_planes_bytes(&bd->fwd, parts_q, parts_kv);
+    const int parts_q = bwd_parts(&bd->fwd, kind, 0), parts_kv = bwd_parts(&bd->fwd, kind, 1);
+    const size_t plane_bytes = bwd_planes_bytes(&bd->fwd, kind, parts_q, parts_kv);
     const size_t need = flag_bytes || plane_bytes ? bwd_rows_bytes(&bd->fwd) + flag_bytes + plane_bytes
                                    : 2 * (size_t)(bd->fwd.B * bd->fwd.Hq * bd->fwd.Sq) * sizeof(float);      // two f32 per query row (+ the mask's block flags, + the planes of a split call)
     if (!bd->workspace || bd->workspace_bytes < need || !aligned16(bd->workspace))
@@ -1074,7 +1090,7 @@ int incin_rocm_sdpa_bwd(const incin_rocm_sdpa_bwd_desc_t* bd, void* stream)
         bp.part_dq = (float*)at;
         at += (size_t)(parts_q - 1) * round256((size_t)(d->B * d->Hq * d->Sq * d->D) * sizeof(float));
         bp.part_dk = (float*)at;
-        at += (size_t)(parts_kv - 1) * round256((size_t)(d->B * d->Hkv * d->Skv * d->D) * sizeof(float));
+        at += (size_t)(kind == 1 ? parts_kv : parts_kv - 1) * round256((size_t)(d->B * d->Hkv * d->Skv * d->D) * sizeof(float));
         bp.part_dv = (float*)at;
     }
     if (flag_bytes) {

@@ -18,14 +18,15 @@ struct SdpaBwdParams {
     int64_t dq_sb, dq_sh, dq_ss;
     int64_t dk_sb, dk_sh, dk_ss;
     int64_t dv_sb, dv_sh, dv_ss;
-    // f32 matrix-core kernels on a launch that does not fill the device: the key tiles of a dQ workgroup are dealt to parts_q
-    // workgroups, the query tiles of a dK/dV workgroup to parts_kv (1, 2 or 4 each).  Part 0 writes the gradient's rows; part
-    // k > 0 writes its sums into plane k - 1 of a contiguous f32 copy of the gradient's shape in the workspace, and a pass
-    // after the kernel adds the planes to the rows in order.
+    // Matrix-core kernels on a launch that does not fill the device: the key tiles of a dQ workgroup are dealt to parts_q
+    // workgroups (f32 only), the query tiles of a dK/dV workgroup to parts_kv (1, 2, 4; 16-bit storage also 8).  The sums meet in
+    // planes of the workspace - contiguous f32 copies of the gradient's shape - and a pass behind the kernel adds them in
+    // order.  f32: part 0 writes the gradient's rows itself and part k > 0 plane k - 1, which the pass adds to the rows; 16-bit
+    // storage: every part writes a plane, and the pass rounds their sum into the rows.
     int32_t parts_q, parts_kv;
-    float* part_dq;                // workspace, [parts_q - 1][B, Hq, Sq, D]
-    float* part_dk;                // workspace, [parts_kv - 1][B, Hkv, Skv, D]
-    float* part_dv;                // workspace, [parts_kv - 1][B, Hkv, Skv, Dv]
+    float* part_dq;                // workspace, f32: [parts_q - 1][B, Hq, Sq, D]
+    float* part_dk;                // workspace, f32: [parts_kv - 1][B, Hkv, Skv, D]; 16-bit storage: [parts_kv][...]
+    float* part_dv;                // workspace, likewise [..][B, Hkv, Skv, Dv]
 };
 
 hipError_t launch_sdpa_bwd_mfma(const SdpaBwdParams& bp, int dtype, hipStream_t stream);

@@ -528,7 +528,12 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
         }
     }
     const int tiles_per_head = j0 < kv_len ? max(n_qt - t_begin, 0) : 0;
-    const int n_tiles = tiles_per_head * p.G;           // the group's query heads one after another
+    const int n_all = tiles_per_head * p.G;             // the group's query heads one after another
+    // bp.parts_kv workgroups share a key block: each walks a stretch n_lo .. n_tiles - 1 of the tiles and leaves its sums in a
+    // plane of the workspace (blockIdx.y says which stretch; one workgroup: the whole walk, and the gradients' rows directly)
+    const int part = blockIdx.y, parts = gridDim.y;
+    const int n_lo = parts > 1 ? (int)((int64_t)n_all * part / parts) : 0;
+    const int n_tiles = parts > 1 ? (int)((int64_t)n_all * (part + 1) / parts) : n_all;
 
     BwdTiles<T, D, 8, NCB> tl;
     tl.init(wave, lane, p.q_ss, bp.do_ss, p.D, p.Dv, NCB * role);
@@ -578,6 +583,13 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
         nx_grem = (int64_t)(nx_rows - 1) * bp.do_ss * 2 + p.Dv * 2;
         nx_r = 0;
         nx_h = h;
+    };
+    auto seek = [&](int n) __attribute__((always_inline)) {      // the copies start at tile n of the walk
+        const int h = n / tiles_per_head, r = n - h * tiles_per_head;
+        to_head(h);
+        nx_q += r * q_step; nx_g += r * g_step; nx_s += (int64_t)r * PF_BN * 4;
+        nx_qrem -= r * q_step; nx_grem -= r * g_step; nx_rows -= r * PF_BN;
+        nx_r = r;
     };
     auto clamp31 = [](int64_t x) { return (x >> 31) ? 0x7fffffff : (int)x; };       // (x is never negative here)
     auto issue = [&](int stage) __attribute__((always_inline)) {
@@ -766,21 +778,21 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
         }
     };
 
-    if (n_tiles > 0) {
-        to_head(0);
+    if (n_lo < n_tiles) {
+        seek(n_lo);
         issue(0);
     }
-    int i0 = t_begin * PF_BN, stage = 0, pstage = 0;
+    int i0 = (t_begin + (n_lo < n_tiles ? n_lo % tiles_per_head : 0)) * PF_BN, stage = 0, pstage = 0;
     // DENSE: the flags of tiles t and t + 1 (known), of tile t + 2 (asked for); without flags every block counts as one with values
     [[maybe_unused]] int f_cur = 0, f_next = 0, fv_next2 = 0;
-    if (DENSE && n_tiles > 0) {
+    if (DENSE && n_lo < n_tiles) {
         if (p.mask_flags) {
-            f_cur = __builtin_amdgcn_readfirstlane(tile_flag(0));
-            if (n_tiles > 1) fv_next2 = tile_flag(1);
+            f_cur = __builtin_amdgcn_readfirstlane(tile_flag(n_lo));
+            if (n_lo + 1 < n_tiles) fv_next2 = tile_flag(n_lo + 1);
         }
-        if (f_cur == 0) { if (STAGED) tile_copy(0); else tile_values(0); }
+        if (f_cur == 0) { if (STAGED) tile_copy(n_lo); else tile_values(n_lo); }
     }
-    for (int t = 0; t < n_tiles; ++t) {
+    for (int t = n_lo; t < n_tiles; ++t) {
         // Tile t has landed for everyone, tile t - 1's P and dS are in the exchange buffer, and everyone is done with tile
         // t - 2: its stage is free for tile t + 1.
         __builtin_amdgcn_s_waitcnt(0x0F70);             // vmcnt(0)
@@ -819,17 +831,41 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
         }
         // Every wavefront computes every tile: one whose keys no row of the tile sees (the first tile or two under a
         // causal mask) works on -inf, and would wait at the barriers for the others anyway.
-        step(stage, pstage, i0, t > 0, f_cur, std::true_type{});
+        step(stage, pstage, i0, t > n_lo, f_cur, std::true_type{});
         pstage = stage;
         stage = nstage;
         i0 = i0 + PF_BN >= n_qt * PF_BN ? t_begin * PF_BN : i0 + PF_BN;      // (then: next head of the group)
         f_cur = f_next;
     }
-    if (n_tiles > 0) {
+    if (n_lo < n_tiles) {
         __syncthreads();
         step(stage, pstage, i0, true, 0, std::false_type{});
     }
 
+    if (parts > 1) {
+        // this stretch's sums as f32 into its plane of the workspace (contiguous rows of D and Dv floats); the pass behind
+        // the kernel adds the planes in order and writes the gradients' rows
+        if (my_j < Skv) {
+            const int64_t r = (((int64_t)part * p.B + b) * p.Hkv + hkv) * Skv + my_j;
+            float* krow = bp.part_dk + r * p.D + role * (D / 2);
+            float* vrow = bp.part_dv + r * p.Dv + role * (D / 2);
+#pragma unroll
+            for (int d = 0; d < NCB; ++d)
+#pragma unroll
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    float4v wk, wv;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        wk[e] = my_j < kv_len ? dk_acc[d][r4 * 4 + e] * p.scale : 0.0f;
+                        wv[e] = my_j < kv_len ? dv_acc[d][r4 * 4 + e] : 0.0f;
+                    }
+                    const int col = role * (D / 2) + d * 32 + r4 * 8 + g * 4;
+                    if (col < p.D) *(float4v*)(krow + d * 32 + r4 * 8 + g * 4) = wk;
+                    if (col < p.Dv) *(float4v*)(vrow + d * 32 + r4 * 8 + g * 4) = wv;
+                }
+        }
+        return;
+    }
     if (my_j < Skv) {
         T* krow = dkp + (int64_t)my_j * bp.dk_ss + role * (D / 2);
         T* vrow = dvp + (int64_t)my_j * bp.dv_ss + role * (D / 2);
@@ -850,6 +886,43 @@ void sdpa_bwd_dkv_kernel(SdpaBwdParams bp)
             }
     }
 #endif
+}
+
+// dst rows [B, H, S, D] of T by strides = the sum of planes 0 .. nplanes - 1 of src ([nplanes][B, H, S, D] f32, contiguous), added
+// in that order; blockIdx.y picks one of two such jobs (dK and dV share a launch).  A thread takes four elements.
+template <typename T> struct SumPlanesJob {
+    T* dst;
+    const float* src;
+    int64_t sb, sh, ss;
+    int B, H, S, D;
+};
+template <typename T>
+__global__ __launch_bounds__(256) void sdpa_bwd_sum_planes_kernel(SumPlanesJob<T> j0, SumPlanesJob<T> j1, int nplanes)
+{
+    typedef float float4v __attribute__((ext_vector_type(4)));
+    const SumPlanesJob<T>& j = blockIdx.y == 0 ? j0 : j1;
+    const int d4 = j.D >> 2;
+    const int64_t n = (int64_t)j.B * j.H * j.S * d4;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n) return;
+    const int64_t row = idx / d4;
+    const int c = (int)(idx - row * d4) * 4;
+    const int s = (int)(row % j.S);
+    const int64_t bh = row / j.S;
+    const int h = (int)(bh % j.H);
+    const int64_t b = bh / j.H;
+    const int64_t plane = (int64_t)j.B * j.H * j.S * j.D;
+    float4v acc = *(const float4v*)(j.src + row * j.D + c);
+    for (int k = 1; k < nplanes; ++k) {
+        const float4v x = *(const float4v*)(j.src + k * plane + row * j.D + c);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] += x[e];
+    }
+    typedef T vec4 __attribute__((ext_vector_type(4)));
+    vec4 w;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) w[e] = (T)acc[e];
+    *(vec4*)(j.dst + b * j.sb + h * j.sh + (int64_t)s * j.ss + c) = w;
 }
 
 // The dQ kernel goes to a side stream where one is to be had (side_stream.h) - it and the dK/dV kernel read the same inputs
@@ -874,9 +947,16 @@ static hipError_t launch_bwd_t(const SdpaBwdParams& bp, hipStream_t stream)
         forked = with_dkv && side.active() && side.fork() == hipSuccess;
     }
     if (with_dkv) {
-        const dim3 grid((unsigned)((int64_t)nkb * p.Hkv * p.B));
+        const unsigned parts = bp.parts_kv > 1 ? (unsigned)bp.parts_kv : 1u;
+        const dim3 grid((unsigned)((int64_t)nkb * p.Hkv * p.B), parts);
         if (DENSE && p.mask_chunks) hipLaunchKernelGGL((sdpa_bwd_dkv_kernel<T, D, DENSE ? 2 : 0>), grid, dim3(512), 0, stream, bp);
         else hipLaunchKernelGGL((sdpa_bwd_dkv_kernel<T, D, DENSE ? 1 : 0>), grid, dim3(512), 0, stream, bp);
+        if (parts > 1) {
+            const SumPlanesJob<T> jk = {(T*)bp.d_k, bp.part_dk, bp.dk_sb, bp.dk_sh, bp.dk_ss, p.B, p.Hkv, p.Skv, p.D};
+            const SumPlanesJob<T> jv = {(T*)bp.d_v, bp.part_dv, bp.dv_sb, bp.dv_sh, bp.dv_ss, p.B, p.Hkv, p.Skv, p.Dv};
+            const int64_t n4 = (int64_t)p.B * p.Hkv * p.Skv * (max(p.D, p.Dv) >> 2);
+            hipLaunchKernelGGL((sdpa_bwd_sum_planes_kernel<T>), dim3((unsigned)((n4 + 255) / 256), 2), dim3(256), 0, stream, jk, jv, (int)parts);
+        }
     }
     if (rows > 0) {
         hipStream_t sq = forked ? side.stream() : stream;

@@ -258,9 +258,9 @@ int incin_rocm_sdpa_fwd_static(const incin_rocm_sdpa_desc_t* desc, void* stream)
  * - and generic f32-arithmetic kernels otherwise; GENERIC and MFMA pin one or the other.  A query row with no visible key (NaN in the forward) gets a zero gradient and
  * contributes nothing to d_k and d_v, where the reference's tape would spread NaN over the whole head.
  * The workspace holds two floats per query row (2 x [B, Hq, Sq]) and, for a dense mask on the matrix-core kernels, a byte
- * per 32 rows x 32 keys of the mask behind them, and for an f32 call on the matrix-core kernels that does not fill the device
- * one to three f32 copies of the gradients' shapes, which workgroups that share a block of rows or keys sum into (ask
- * incin_rocm_sdpa_bwd_workspace for the size: it depends on the device's compute-unit count);
+ * per 32 rows x 32 keys of the mask behind them, and for a call on the matrix-core kernels that does not fill the device
+ * (f32; 16-bit storage with few KV heads) up to four f32 copies of the gradients' shapes, which workgroups that share a block
+ * of rows or keys sum into (ask incin_rocm_sdpa_bwd_workspace for the size: it depends on the device's compute-unit count);
  * d_q, d_k, d_v are fully overwritten.
  * Streams: everything the call launches is ordered behind the work already on `stream` and ahead of whatever `stream` gets
  * next.  A call of the matrix-core kernels that is short of work may run its dQ kernel on a stream of the library's own

@@ -278,13 +278,17 @@ def test_backward_validation_and_workspace_size():
     # ... plus, for an f32 call on the matrix-core kernels that does not fill the device, the planes that the parts of a
     # block sum into: 2 x 4 heads x 1024 rows are 64 blocks of 128 for either kernel, a quarter of the 256 workgroups a device
     # of 256 compute units (no device to ask here) holds at D = 128 - four parts, three planes per gradient
-    def long(**fwd_kw):
-        bd = _bwd(dict(Sq=1024, Skv=1024, **fwd_kw))
+    def long(S=1024, **fwd_kw):
+        bd = _bwd(dict(Sq=S, Skv=S, **fwd_kw))
         for st in (bd.fwd.q_stride, bd.fwd.k_stride, bd.fwd.v_stride, bd.fwd.o_stride, bd.d_o_stride, bd.d_q_stride, bd.d_k_stride, bd.d_v_stride):
-            st[0], st[1], st[2] = 4 * 1024 * 128, 1024 * 128, 128
+            st[0], st[1], st[2] = 4 * S * 128, S * 128, 128
         return bd
     rows, plane = 2 * 2 * 4 * 1024 * 4, 2 * 4 * 1024 * 128 * 4
-    assert capi.sdpa_bwd_workspace(long()) == rows                                          # (16-bit storage: no planes)
+    assert capi.sdpa_bwd_workspace(long()) == rows                                          # (16-bit storage: walks of 16 tiles are not dealt)
+    # 16-bit storage, four query heads on one KV head x 4096 keys: 64 key blocks whose walks of 256 tiles go to four workgroups
+    # each, every one with a plane for dK and one for dV
+    assert capi.sdpa_bwd_workspace(long(S=4096, Hkv=1)) == 4 * rows + 4 * 2 * (2 * 4096 * 128 * 4)
+    assert capi.sdpa_bwd_workspace(long(S=4096, Hkv=1, B=8)) == 16 * rows                    # (a full round of key blocks: not dealt)
     assert capi.sdpa_bwd_workspace(long(dtype=capi.F32)) == rows + 3 * 3 * plane
     assert capi.sdpa_bwd_workspace(long(dtype=capi.F32, impl=capi.IMPL_GENERIC)) == rows
     assert capi.sdpa_bwd_workspace(long(dtype=capi.F32, D=64, Dv=64)) == rows + 3 * 3 * plane // 2      # (512 workgroups at a time at D = 64)

@@ -448,6 +448,59 @@ def test_matrix_core_backward_f32_in_parts(gpu, monkeypatch, parts, shape):
         assert not dq[b, :, nq:].any() and not dk[b, :, nk:].any() and not dv[b, :, nk:].any()
 
 
+@pytest.mark.parametrize("parts", ["1", "2", "4", "8"])
+@pytest.mark.parametrize("dtype", [capi.BF16, capi.F16], ids=lambda x: dtypes.NAMES[x])
+@pytest.mark.parametrize("shape", [
+    # B, Hq, Hkv, Sq, Skv, D, Dv, causal, kv_lens, q_lens, mask
+    (1, 8, 1, 1024, 1024, 128, 128, True, None, None, None),                # eight query heads walking one KV head's key blocks
+    (2, 4, 2, 600, 1100, 64, 64, True, [1100, 300], None, None),
+    (1, 2, 2, 2100, 520, 128, 64, False, None, None, None),                 # D != Dv: planes of different widths
+    (1, 8, 2, 520, 1504, 128, 128, True, None, None, "window"),             # a mask whose values go through LDS; its flags trim the walk before it is dealt
+    (2, 2, 2, 1024, 1024, 64, 64, True, [1024, 700], [1024, 700], None),    # padding rows and keys: zero in every plane
+    (1, 4, 1, 700, 333, 128, 128, False, None, None, "values"),             # a mask whose rows cannot be copied
+], ids=["gqa8", "ragged_gqa64", "rect_d_dv", "window_gqa", "padded", "values_unaligned"])
+def test_matrix_core_backward_16bit_in_parts(gpu, monkeypatch, parts, dtype, shape):
+    """The 16-bit dK/dV kernel with the walk of a key block - the query tiles of every head of its group - dealt to 1, 2, 4 and 8
+    workgroups whose sums meet as f32 in planes of the workspace (what a call with few key blocks gets by itself;
+    INCIN_ROCM_BWD_PARTS forces it): against the f64 oracle each, exact zeros where padding is."""
+    B, Hq, Hkv, Sq, Skv, D, Dv, causal, lens, qlens, mk = shape
+    G = Hq // Hkv
+    monkeypatch.setenv("INCIN_ROCM_BWD_PARTS", parts)
+    say("matrix-core backward %s in %s parts: %s" % (dtypes.NAMES[dtype], parts, shape))
+    q, k, v, go = make_d(95 + Sq, B, Hq, Hkv, Sq, Skv, D, Dv, dtype)
+    r = np.random.Generator(np.random.PCG64(96))
+    mask = None
+    if mk == "window":
+        dist = np.arange(Sq)[:, None] + (Skv - Sq) - np.arange(Skv)[None, :]
+        mask = np.where((dist >= 0) & (dist < 400), -0.01 * dist, -np.inf).astype(np.float32).reshape(1, 1, Sq, Skv)
+    elif mk == "values":
+        mask = r.standard_normal((1, Hq, Sq, Skv), dtype=np.float32)
+        mask[r.random(mask.shape) < 0.25] = -np.inf
+        mask[..., 0] = 0.0
+    if mask is not None:
+        mask = dtypes.round_to(mask, dtype)
+    lens_a = None if lens is None else np.asarray(lens, np.int32)
+    qlens_a = None if qlens is None else np.asarray(qlens, np.int32)
+    out, dq, dk, dv = host.sdpa_backward(q, k, v, go, dtype, impl=capi.IMPL_MFMA, causal=causal, kv_lens=lens_a, q_lens=qlens_a, mask=mask,
+                                         poison_padding=qlens is not None)
+    for b in range(B):
+        nq = Sq if qlens is None else int(qlens[b])
+        nk = Skv if lens is None else int(lens[b])
+        m5 = None if mask is None else np.broadcast_to(mask, (B, Hq, Sq, Skv))[b:b + 1, :, :nq, :nk].reshape(1, Hkv, G, nq, nk)
+        if causal and nk - nq != Skv - Sq:      # (a sequence cut to its lengths: the causal diagonal stays anchored at the full extents)
+            tri = np.triu(np.full((Sq, Skv), -np.inf, np.float32), 1 + Skv - Sq)[:nq, :nk].reshape(1, 1, 1, nq, nk)
+            m5 = tri if m5 is None else m5 + tri
+            cz = False
+        else:
+            cz = causal
+        rq, rk, rv = BW.sdpa_backward(q[b:b + 1, :, :nq].reshape(1, Hkv, G, nq, D), k[b:b + 1, :, None, :nk], v[b:b + 1, :, None, :nk],
+                                      go[b:b + 1, :, :nq].reshape(1, Hkv, G, nq, Dv), mask=m5, causal=cz)
+        compare("dq[%d]" % b, dq[b:b + 1, :, :nq], rq.reshape(1, Hq, nq, D))
+        compare("dk[%d]" % b, dk[b:b + 1, :, :nk], rk.reshape(1, Hkv, nk, D))
+        compare("dv[%d]" % b, dv[b:b + 1, :, :nk], rv.reshape(1, Hkv, nk, Dv))
+        assert not dq[b, :, nq:].any() and not dk[b, :, nk:].any() and not dv[b, :, nk:].any()
+
+
 def test_matrix_core_backward_f32_rows_without_keys(gpu):
     # Sq > Skv under causal alignment: the first Sq - Skv rows see nothing; they get a zero dq and add nothing to dk, dv
     B, H, Sq, Skv, D = 1, 2, 96, 40, 64
