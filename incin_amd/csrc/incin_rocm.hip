@@ -1011,6 +1011,10 @@ static int bwd_parts(const incin_rocm_sdpa_desc_t* d, int kind, int which)
     while (parts < 4 && 2 * parts * blocks <= slots) parts *= 2;
     // (f32: four tiles per part are enough to pay for the planes; 16-bit storage, whose tiles take an eighth of the time: 64)
     while (parts > 1 && walk < (kind == 1 ? 64 : 4) * parts) parts >>= 1;
+    // 16-bit storage, up to a full round of key blocks with very long walks (8 query heads on 1 KV head x 32768 keys: 256 blocks
+    // of up to 4096 tiles): under a causal mask the longest walk is twice the average and the round ends with it - four parts
+    // make four rounds of shorter items (10.2 -> 7.3 ms there; 16 heads on 2 x 16384, 2048 tiles: 0.84; at 512 tiles 1.05)
+    if (kind == 1 && parts == 1 && blocks <= slots && walk >= 2048 && (d->causal || d->add_mask)) parts = 4;
     return parts;
 }
 static size_t round256(size_t n) { return (n + 255) / 256 * 256; }

@@ -704,7 +704,7 @@ static hipError_t launch_bwd_f32_t(const SdpaBwdParams& bp, hipStream_t stream)
         const unsigned parts = parts_q;
         SdpaBwdParams bq = bp;
         bq.f.interleave = work_interleave(p.causal != 0 || p.mask != nullptr, (D == 128 ? 1 : 2) * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
-        bq.f.deal_groups = (total & 7) == 0 ? work_deal(bq.f.interleave, p.G, nqb, total >> 3) : 0;
+        bq.f.deal_groups = (total & 7) == 0 ? work_deal(bq.f.interleave, p.G, nqb, total >> 3, p.causal != 0 || p.mask != nullptr) : 0;
         hipLaunchKernelGGL((bwd_f32_dq_kernel<D, DENSE>), dim3((unsigned)total, parts), dim3(256), 0, sq, bq);
         if (parts > 1) {
             const AddPlanesJob jq = {(float*)bp.d_q, bp.part_dq, bp.dq_sb, bp.dq_sh, bp.dq_ss, p.B, p.Hq, p.Sq, p.D};

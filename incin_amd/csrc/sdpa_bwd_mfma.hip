@@ -964,7 +964,7 @@ static hipError_t launch_bwd_t(const SdpaBwdParams& bp, hipStream_t stream)
         const int64_t total = (int64_t)nqb * p.Hq * p.B;
         SdpaBwdParams bq = bp;      // two workgroups per CU, an eighth of the CUs per XCD
         bq.f.interleave = work_interleave(p.causal != 0 || p.mask != nullptr, 2 * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
-        bq.f.deal_groups = (total & 7) == 0 ? work_deal(bq.f.interleave, p.G, nqb, total >> 3) : 0;
+        bq.f.deal_groups = (total & 7) == 0 ? work_deal(bq.f.interleave, p.G, nqb, total >> 3, p.causal != 0 || p.mask != nullptr) : 0;
         if (DENSE && p.mask_chunks) hipLaunchKernelGGL((sdpa_bwd_dq_kernel<T, D, DENSE ? 2 : 0>), dim3((unsigned)total), dim3(256), 0, sq, bq);
         else hipLaunchKernelGGL((sdpa_bwd_dq_kernel<T, D, DENSE ? 1 : 0>), dim3((unsigned)total), dim3(256), 0, sq, bq);
     }

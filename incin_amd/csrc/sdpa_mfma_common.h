@@ -177,9 +177,14 @@ __device__ __forceinline__ WorkItem work_item(int vid, int F, int G, int nqb)
 // Item `item` of XCD `xcd`'s share of the work list (a share holds share_len items).  When a share holds whole
 // groups, (batch, KV head) pairs are dealt to the XCDs in turn - pair h goes to XCD h % 8, and an XCD groups the
 // pairs it holds F at a time - so the sequences of a ragged batch spread over all XCDs instead of one long sequence
-// filling the shares of two of them.  Otherwise a share is a contiguous eighth of the list.
+// filling the shares of two of them.  Otherwise a share is a contiguous eighth of the list - unless (deal = 2) a share is
+// less than one group and the group's blocks differ in length (a causal mask): a contiguous piece of a list that runs
+// longest-first would give one XCD the long blocks of every head and another the short ones (8 query heads on one KV head,
+// 64 blocks each: the first XCD would get 1.9 times the average), so the list is dealt item by item - item i of the list to
+// XCD i % 8, which is the order workgroups reach the XCDs in anyway.
 __device__ __forceinline__ WorkItem work_item_of_share(int xcd, int item, int share_len, int F, int G, int nqb, int deal)
 {
+    if (deal == 2) return work_item(item * 8 + xcd, F, G, nqb);
     if (!deal) return work_item(xcd * share_len + item, F, G, nqb);
     const int per_group = F * G * nqb;
     const int g_local = item / per_group, r = item - g_local * per_group;
@@ -190,9 +195,10 @@ __device__ __forceinline__ WorkItem work_item_of_share(int xcd, int item, int sh
     w.qblk = nqb - 1 - rank;
     return w;
 }
-inline int work_deal(int F, int G, int nqb, long long share_items)
+inline int work_deal(int F, int G, int nqb, long long share_items, bool uneven)
 {
-    return share_items % ((long long)F * G * nqb) == 0 ? 1 : 0;
+    const long long group = (long long)F * G * nqb;
+    return share_items % group == 0 ? 1 : (uneven && share_items < group ? 2 : 0);
 }
 
 // F for a launch: `slots` workgroups run on an XCD at a time, a range of the list (the whole list, or an eighth of it

@@ -307,7 +307,7 @@ static hipError_t launch_prefill_f32_t(const SdpaParams& p0, hipStream_t stream)
     if (total <= 0) return hipSuccess;
     if (total > 0x7fffffffLL) return hipErrorInvalidValue;
     p.interleave = work_interleave(p.causal != 0 || p.mask != nullptr, 2 * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
-    p.deal_groups = (total & 7) == 0 ? work_deal(p.interleave, p.G, nqb, total >> 3) : 0;
+    p.deal_groups = (total & 7) == 0 ? work_deal(p.interleave, p.G, nqb, total >> 3, p.causal != 0 || p.mask != nullptr) : 0;
     if constexpr (!DENSE) {
         if (p.num_splits > 1) {          // split launch: partial results, then the split-KV kernels' combine pass
             hipLaunchKernelGGL((sdpa_prefill_f32_kernel<D, false, true>), dim3((unsigned)total, (unsigned)p.num_splits), dim3(256), 0, stream, p);

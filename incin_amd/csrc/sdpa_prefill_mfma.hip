@@ -952,7 +952,7 @@ static hipError_t launch_prefill_nw(const SdpaParams& p0, hipStream_t stream)
     // 256 registers per lane: eight wavefronts per compute unit, i.e. two workgroups of four or one of eight; an eighth
     // of the compute units per XCD
     p.interleave = work_interleave(p.causal != 0 || p.mask != nullptr, (8 / NW) * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
-    p.deal_groups = (total & 7) == 0 ? work_deal(p.interleave, p.G, nqb, total >> 3) : 0;
+    p.deal_groups = (total & 7) == 0 ? work_deal(p.interleave, p.G, nqb, total >> 3, p.causal != 0 || p.mask != nullptr) : 0;
     constexpr bool DENSE = MASK == 1 || MASK == 3;
     if constexpr (MASK == 0 && NW == 4) {
         if (p.num_splits > 1) {          // split launch: partial results, then the split-KV kernels' combine pass

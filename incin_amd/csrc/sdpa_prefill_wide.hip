@@ -370,7 +370,7 @@ hipError_t launch_sdpa_prefill_wide(const SdpaParams& p0, int dtype, hipStream_t
     if (total > 0x7fffffffLL) return hipErrorInvalidValue;
     // two workgroups per compute unit, an eighth of the compute units per XCD
     p.interleave = work_interleave(p.causal != 0 || p.mask != nullptr, 2 * device_cus() / 8, p.G, nqb, (total & 7) == 0 ? total >> 3 : total);
-    p.deal_groups = (total & 7) == 0 ? work_deal(p.interleave, p.G, nqb, total >> 3) : 0;
+    p.deal_groups = (total & 7) == 0 ? work_deal(p.interleave, p.G, nqb, total >> 3, p.causal != 0 || p.mask != nullptr) : 0;
     if (p.mask && p.mask_lims) {       // the blocks whose rows all have a limit; then, below, the others
         if (dtype == 1) hipLaunchKernelGGL((sdpa_prefill_wide_kernel<f16_t, 2>), dim3((unsigned)total), dim3(256), 0, stream, p);
         else hipLaunchKernelGGL((sdpa_prefill_wide_kernel<bf16_t, 2>), dim3((unsigned)total), dim3(256), 0, stream, p);
