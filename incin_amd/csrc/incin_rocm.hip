@@ -1015,6 +1015,12 @@ static int bwd_parts(const incin_rocm_sdpa_desc_t* d, int kind, int which)
     // of up to 4096 tiles): under a causal mask the longest walk is twice the average and the round ends with it - four parts
     // make four rounds of shorter items (10.2 -> 7.3 ms there; 16 heads on 2 x 16384, 2048 tiles: 0.84; at 512 tiles 1.05)
     if (kind == 1 && parts == 1 && blocks <= slots && walk >= 2048 && (d->causal || d->add_mask)) parts = 4;
+    // ... and two parts already from 256 tiles on when the dQ kernel is not running beside this one to fill the compute units the
+    // short walks leave idle (the launcher's rule: D = 64, or at most four dQ blocks per compute unit).  One sequence of 4096
+    // tokens, D = 128: 64 query heads on 8 KV heads 1.28 -> 1.01 ms, 128 on 8 2.62 -> 1.91, 48 on 8 0.97 -> 0.79, 2 x 32 on 4 1.29 ->
+    // 1.02; with the dQ kernel beside it (2 x 8 on 2 x 8192) two parts cost 19 %.
+    const bool dq_beside = (d->D <= 64 && d->Dv <= 64) || ((d->Sq + 127) / 128) * d->Hq * d->B <= 4 * (int64_t)compute_units_of(d->device);
+    if (kind == 1 && parts == 1 && blocks <= slots && walk >= 256 && !dq_beside && (d->causal || d->add_mask)) parts = 2;
     return parts;
 }
 static size_t round256(size_t n) { return (n + 255) / 256 * 256; }
