@@ -352,7 +352,11 @@ int make_plan(const incin_rocm_sdpa_desc_t* d, Plan* plan)
         int64_t splits = d->num_splits;
         if (splits == 0) {
             const int64_t cus = compute_units_of(d->device);
-            const int64_t max_by_len = d->Skv / 256 > 0 ? d->Skv / 256 : 1;
+            // (from 65536 keys on a split keeps at least 1024: with one or two groups the filling alone would ask for 512 splits of
+            //  256 keys, each hardly past its ring's start-up, and a combine pass over 512 partial results per row - one sequence
+            //  of 131072 keys on one KV head: 35.9 us in 512 splits, 26.5 in 256, 24.1 in 128, 30.6 in 64)
+            const int64_t min_len = d->Skv >= 65536 ? 1024 : 256;
+            const int64_t max_by_len = d->Skv / min_len > 0 ? d->Skv / min_len : 1;
             const int64_t max_splits = std::min<int64_t>(max_by_len, std::max<int64_t>(1, 4 * cus / groups));
             auto fill = [&](int64_t s) {           // (with the split length, and so the count, s really leads to)
                 const int64_t len = ((d->Skv + s - 1) / s + 255) / 256 * 256;
