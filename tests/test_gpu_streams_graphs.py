@@ -103,16 +103,18 @@ def test_graph_capture_and_replay(gpu, name, kw):
     graph.destroy()
 
 
-@pytest.mark.parametrize("dtype, impl, S", [(capi.BF16, capi.IMPL_AUTO, 300), (capi.F32, capi.IMPL_AUTO, 300), (capi.F32, capi.IMPL_AUTO, 1100),
-                                            (capi.F32, capi.IMPL_GENERIC, 300)],
-                         ids=["bf16_matrix_core", "f32_matrix_core", "f32_matrix_core_dealt_blocks", "f32_generic"])
-def test_training_step_in_a_graph(gpu, dtype, impl, S):
+@pytest.mark.parametrize("dtype, impl, S, heads", [(capi.BF16, capi.IMPL_AUTO, 300, (4, 2)), (capi.F32, capi.IMPL_AUTO, 300, (4, 2)),
+                                                   (capi.F32, capi.IMPL_AUTO, 1100, (4, 2)), (capi.F32, capi.IMPL_GENERIC, 300, (4, 2)),
+                                                   (capi.BF16, capi.IMPL_AUTO, 1100, (8, 1))],
+                         ids=["bf16_matrix_core", "f32_matrix_core", "f32_matrix_core_dealt_blocks", "f32_generic", "bf16_one_kv_head_dealt_walks"])
+def test_training_step_in_a_graph(gpu, dtype, impl, S, heads):
     """Forward (keeping the row normalisers) and backward recorded into one launch graph and replayed: every replay gives
     the bytes the eager calls gave, with the program's own eager work between replays.  The backward launches three kernels
-    (five at 1100 tokens in f32, where the walks of a block are dealt to several workgroups and a pass adds their sums) on
+    (up to five at 1100 tokens, where the walks of a block - in f32, and in bf16 with eight query heads on one KV head - are dealt to
+    several workgroups and a pass adds their sums) on
     the captured stream alone - eagerly a call this small puts one of them on a second stream - and neither allocates nor
     clears memory."""
-    B, Hq, Hkv, D = 2, 4, 2, 128
+    (Hq, Hkv), B, D = heads, 2, 128
     r = np.random.Generator(np.random.PCG64(300))
     mk = lambda *s: r.standard_normal(s, dtype=np.float32)
     tq, tk, tv, tg = (host.DeviceTensor.from_f32(x, dtype) for x in (mk(B, Hq, S, D), mk(B, Hkv, S, D), mk(B, Hkv, S, D), mk(B, Hq, S, D)))
